@@ -1,0 +1,1244 @@
+// CPU restatement of the VSAG search-core arithmetic (k-means assignment, FP32 / SQ8 / SQ4 /
+// SQ4-uniform / SQ8-uniform / RaBitQ distance computers, bounded-heap top-k, IVF route/scan/rerank).
+//
+// THIS FILE IS TEST INFRASTRUCTURE.  It is the checker that the HIP library is compared with, and the
+// CPU baseline that bench.py times beside the GPU.  Nothing in the product path links, loads or
+// calls it; the shipped library fails loudly when its HIP code object is missing instead of coming
+// here.  Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may load it.
+//
+// Every function cites the reference file:line (relative to the VSAG source tree) whose arithmetic
+// it restates.  How each one is pinned (known answers of the reference's own tests, the compiled
+// reference scalar kernels, closed forms, brute force) is listed beside the tests that do it:
+//   pinned by reference known answers ... sq_encode (NaN->0, 0.5->127/7), squ_encode byte images,
+//                                          rabitq 4-bit query planes, rabitq_binary_ip 0/36/32
+//   pinned by compiled reference kernels . fp32/sq8/sq4 distances, sq4u/sq8u code IP, binary IPs,
+//                                          normalize-with-centroid
+//   pinned by closed form / brute force .. sq_train (sorted order statistics), kmeans_assign (fp64
+//                                          argmin), heaps (sort), ivf composition (nprobe=nlist)
+//   parity unpinned ...................... rabitq_dist op order and kmeans inertia are fixed only by
+//                                          their formulas (no executable reference, no golden value
+//                                          in the reference tests); tolerance 1e-4 relative covers it
+#include <algorithm>
+#include <cfloat>
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <limits>
+#include <queue>
+#include <random>
+#include <utility>
+#include <vector>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORC_API extern "C" __attribute__((visibility("default")))
+
+namespace {
+
+enum Metric { kL2 = 0, kIP = 1, kCosine = 2 };
+
+inline uint64_t
+align_up(uint64_t v, uint64_t a) {
+    return (v + a - 1) / a * a;
+}
+
+// ---------------------------------------------------------------- FP32 primitives
+// src/simd/generic.cpp:99-107 with the Width=1 traits (src/simd/traits/simd_traits_generic.h:42-96):
+// one running fp32 sum, sub then multiply-add per element, element order 0..dim-1.
+inline float
+fp32_l2sqr(const float* q, const float* x, uint64_t dim) {
+    float s = 0.0F;
+    for (uint64_t i = 0; i < dim; ++i) {
+        float t = q[i] - x[i];
+        s = t * t + s;
+    }
+    return s;
+}
+
+inline float
+fp32_ip(const float* q, const float* x, uint64_t dim) {
+    float s = 0.0F;
+    for (uint64_t i = 0; i < dim; ++i) {
+        s = q[i] * x[i] + s;
+    }
+    return s;
+}
+
+// src/simd/generic.cpp:874-878: norm = sqrt(<x,x>), to = from / norm (a zero norm divides by 1).
+inline float
+normalize(const float* from, float* to, uint64_t dim) {
+    float norm = std::sqrt(fp32_ip(from, from, dim));
+    float scalar = norm == 0 ? 1.0F : norm;  // DivScalarImpl, src/simd/kernels/scalar_op.h:40-42
+    for (uint64_t i = 0; i < dim; ++i) {
+        to[i] = from[i] / scalar;
+    }
+    return norm;
+}
+
+// src/simd/kernels/normalize.h:35-83: norm of (from - centroid); norm_sq < 1e-5 -> norm = 1.
+inline float
+normalize_with_centroid(const float* from, const float* centroid, float* to, uint64_t dim) {
+    float norm_sq = 0.0F;
+    for (uint64_t i = 0; i < dim; ++i) {
+        float d = from[i] - centroid[i];
+        norm_sq = d * d + norm_sq;
+    }
+    float norm = (norm_sq < 1e-5F) ? 1.0F : std::sqrt(norm_sq);
+    for (uint64_t i = 0; i < dim; ++i) {
+        to[i] = (from[i] - centroid[i]) / norm;
+    }
+    return norm;
+}
+
+// ---------------------------------------------------------------- scalar quantization
+// src/quantization/scalar_quantization/scalar_quantization_utils.h:19-30
+inline float
+clamp_delta(float delta) {
+    if (!(delta >= 0.0F)) {
+        return 0.0F;
+    }
+    if (delta > 0.999F) {
+        return 1.0F;
+    }
+    return delta;
+}
+
+// src/simd/kernels/sq8_compute.h:44-137 (Width=1): code/255 then *diff+lb, fp32.
+inline float
+sq8_ip(const float* q, const uint8_t* c, const float* lb, const float* diff, uint64_t dim) {
+    float s = 0.0F;
+    const float inv255 = 1.0F / 255.0F;
+    for (uint64_t i = 0; i < dim; ++i) {
+        float normalized = static_cast<float>(c[i]) * inv255;
+        float adjusted = normalized * diff[i] + lb[i];
+        s = q[i] * adjusted + s;
+    }
+    return s;
+}
+
+inline float
+sq8_l2sqr(const float* q, const uint8_t* c, const float* lb, const float* diff, uint64_t dim) {
+    float s = 0.0F;
+    const float inv255 = 1.0F / 255.0F;
+    for (uint64_t i = 0; i < dim; ++i) {
+        float normalized = static_cast<float>(c[i]) * inv255;
+        float adjusted = normalized * diff[i] + lb[i];
+        float d = q[i] - adjusted;
+        s = d * d + s;
+    }
+    return s;
+}
+
+// src/simd/generic.cpp:316-340 (scalar SQ4): nibble * (1/15) * diff + lb, low nibble = even dim.
+inline float
+sq4_value(const uint8_t* c, const float* lb, const float* diff, uint64_t i) {
+    uint8_t nibble = (i & 1) ? (c[i >> 1] >> 4) : (c[i >> 1] & 0x0f);
+    return nibble * (1.0F / 15.0F) * diff[i] + lb[i];
+}
+
+inline float
+sq4_ip(const float* q, const uint8_t* c, const float* lb, const float* diff, uint64_t dim) {
+    float s = 0.0F;
+    for (uint64_t i = 0; i < dim; ++i) {
+        s += q[i] * sq4_value(c, lb, diff, i);
+    }
+    return s;
+}
+
+inline float
+sq4_l2sqr(const float* q, const uint8_t* c, const float* lb, const float* diff, uint64_t dim) {
+    float s = 0.0F;
+    for (uint64_t i = 0; i < dim; ++i) {
+        float d = q[i] - sq4_value(c, lb, diff, i);
+        s += d * d;
+    }
+    return s;
+}
+
+// src/simd/generic.cpp:406-431: integer code x code inner products.
+inline int32_t
+sq4u_codes_ip(const uint8_t* a, const uint8_t* b, uint64_t dim) {
+    int32_t r = 0;
+    for (uint64_t d = 0; d < dim; d += 2) {
+        int32_t x_lo = a[d >> 1] & 0x0f;
+        int32_t x_hi = (a[d >> 1] & 0xf0) >> 4;
+        int32_t y_lo = b[d >> 1] & 0x0f;
+        int32_t y_hi = (b[d >> 1] & 0xf0) >> 4;
+        r += x_lo * y_lo + x_hi * y_hi;
+    }
+    return r;
+}
+
+inline int32_t
+sq8u_codes_ip(const uint8_t* a, const uint8_t* b, uint64_t dim) {
+    int32_t r = 0;
+    for (uint64_t d = 0; d < dim; ++d) {
+        r += static_cast<int32_t>(a[d]) * static_cast<int32_t>(b[d]);
+    }
+    return r;
+}
+
+// Byte layout of the uniform codes.
+// sq4_uniform_quantizer.cpp:33-72 ; sq8_uniform_quantizer.cpp:30-62.
+struct UniformLayout {
+    uint64_t code_bytes;        // bytes holding nibbles / bytes (before alignment)
+    uint64_t offset_norm;       // u64 sum code^2 (L2; SQ4U also for cosine)
+    uint64_t offset_sum;        // f32 sum of raw values (IP / cosine)
+    uint64_t offset_codes_sum;  // f32 sum of codes (SQ4U IP / cosine only)
+    uint64_t code_size;
+    bool has_norm, has_sum, has_codes_sum;
+};
+
+inline UniformLayout
+uniform_layout(uint64_t dim, int bits, int metric) {
+    UniformLayout l{};
+    uint64_t align = 1;
+    bool norm = (metric == kL2) || (bits == 4 && metric == kCosine);
+    bool sum = (metric == kIP || metric == kCosine);
+    if (norm) {
+        align = std::max<uint64_t>(align, 8);
+    }
+    if (sum) {
+        align = std::max<uint64_t>(align, 4);
+    }
+    l.code_bytes = (bits == 4) ? (dim + 1) / 2 : dim;
+    l.code_size = align_up(l.code_bytes, align);
+    l.has_norm = norm;
+    l.has_sum = sum;
+    l.has_codes_sum = sum && bits == 4;
+    if (norm) {
+        l.offset_norm = l.code_size;
+        l.code_size += align_up(8, align);
+    }
+    if (sum) {
+        l.offset_sum = l.code_size;
+        l.code_size += align_up(4, align);
+        if (bits == 4) {
+            l.offset_codes_sum = l.code_size;
+            l.code_size += align_up(4, align);
+        }
+    }
+    return l;
+}
+
+// ---------------------------------------------------------------- RaBitQ (1-bit base)
+// rabitq_quantizer.cpp:102-176: field offsets of the base code and of the processed query.
+struct RabitqLayout {
+    uint64_t dim;
+    uint64_t offset_norm, offset_error, offset_sum, offset_raw_norm, code_size;
+    bool has_sum, has_raw_norm;
+    uint64_t aligned_dim, plane_bytes;
+    uint64_t q_offset_lb, q_offset_delta, q_offset_sum, q_offset_norm, q_offset_raw_norm, query_code_size;
+};
+
+inline RabitqLayout
+rabitq_layout(uint64_t dim, int metric, int query_bits) {
+    RabitqLayout l{};
+    l.dim = dim;
+    const uint64_t a = 4;
+    uint64_t cs = align_up((dim + 7) / 8, a);
+    l.offset_norm = cs;
+    cs += 4;
+    l.offset_error = cs;
+    cs += 4;
+    l.has_sum = query_bits != 32;
+    if (l.has_sum) {
+        l.offset_sum = cs;
+        cs += 4;
+    }
+    l.has_raw_norm = (metric == kIP || metric == kCosine);
+    if (l.has_raw_norm) {
+        l.offset_raw_norm = cs;
+        cs += 4;
+    }
+    l.code_size = cs;
+    uint64_t qs = 0;
+    if (query_bits == 4) {
+        l.aligned_dim = (dim + 511) / 512 * 512;
+        l.plane_bytes = l.aligned_dim / 8;
+        qs = l.aligned_dim / 8 * 4;
+        l.q_offset_lb = qs;
+        qs += 4;
+        l.q_offset_delta = qs;
+        qs += 4;
+        l.q_offset_sum = qs;
+        qs += 4;
+    } else {
+        qs = align_up(4 * dim, a);
+    }
+    l.q_offset_norm = qs;
+    qs += 4;
+    if (l.has_raw_norm) {
+        l.q_offset_raw_norm = qs;
+        qs += 4;
+    }
+    l.query_code_size = qs;
+    return l;
+}
+
+// src/simd/generic.cpp:447-471
+inline float
+rabitq_float_binary_ip(const float* v, const uint8_t* bits, uint64_t dim, float inv_sqrt_d) {
+    if (dim == 0) {
+        return 0.0F;
+    }
+    float pos, neg;
+    if (inv_sqrt_d > 1e-3) {
+        pos = inv_sqrt_d;
+        neg = -inv_sqrt_d;
+    } else {
+        pos = 1.0F;
+        neg = 0;
+    }
+    float r = 0.0F;
+    for (uint64_t d = 0; d < dim; ++d) {
+        bool bit = ((bits[d / 8] >> (d % 8)) & 1) != 0;
+        r += (bit ? pos : neg) * v[d];
+    }
+    return r;
+}
+
+// src/simd/generic.cpp:832-872: sum_b popcount(plane_b & bits) << b; planes are ceil(dim/8) bytes apart.
+inline uint32_t
+rabitq_sq4u_binary_ip(const uint8_t* planes, const uint8_t* bits, uint64_t dim) {
+    if (dim == 0) {
+        return 0;
+    }
+    uint64_t num_bytes = (dim + 7) / 8;
+    uint32_t r = 0;
+    for (uint64_t b = 0; b < 4; ++b) {
+        uint32_t cnt = 0;
+        for (uint64_t i = 0; i < num_bytes; ++i) {
+            cnt += __builtin_popcount(static_cast<unsigned>(planes[b * num_bytes + i] & bits[i]));
+        }
+        r += cnt << b;
+    }
+    return r;
+}
+
+inline float
+rd_f32(const uint8_t* p) {
+    float v;
+    std::memcpy(&v, p, 4);
+    return v;
+}
+inline void
+wr_f32(uint8_t* p, float v) {
+    std::memcpy(p, &v, 4);
+}
+
+// y = Q x, Q row-major (random_orthogonal_transformer.cpp:58-77; cblas_sgemv RowMajor NoTrans).
+inline void
+rotate(const float* rot, const float* x, float* y, uint64_t dim) {
+    for (uint64_t i = 0; i < dim; ++i) {
+        y[i] = fp32_ip(rot + i * dim, x, dim);
+    }
+}
+
+// rabitq_quantizer.cpp:915-939
+inline float
+l2_ube(float nb, float nq, float est_ip_norm) {
+    float p1 = nb * nb;
+    float p2 = nq * nq;
+    float p3 = -2 * nb * nq * est_ip_norm;
+    return p1 + p2 + p3;
+}
+
+inline float
+recover_sq4u(uint32_t ip, float base_sum, float query_sum, float lb, float delta, float inv_sqrt_d,
+             uint64_t dim) {
+    float p1 = inv_sqrt_d * delta * 2 * static_cast<float>(ip);
+    float p2 = inv_sqrt_d * lb * 2 * base_sum;
+    float p3 = inv_sqrt_d * delta * query_sum;
+    float p4 = inv_sqrt_d * lb * static_cast<float>(dim);
+    return p1 + p2 - p3 - p4;
+}
+
+// ---------------------------------------------------------------- bounded heaps
+using Rec = std::pair<float, uint32_t>;
+struct CmpMax {
+    bool
+    operator()(const Rec& a, const Rec& b) const {
+        return a.first < b.first;
+    }
+};
+
+// impl/heap/standard_heap.cpp:24-53 (max_heap, fixed_size): when full, dist > top is dropped,
+// dist == top is pushed and one maximum popped.
+struct FixedMaxHeap {
+    std::vector<Rec> q;
+    uint64_t cap;
+    explicit FixedMaxHeap(uint64_t k) : cap(k) {
+        q.reserve(k + 1);
+    }
+    void
+    push(float d, uint32_t id) {
+        if (q.size() == cap && !q.empty()) {
+            if (d > q.front().first) {
+                return;
+            }
+        }
+        q.emplace_back(d, id);
+        std::push_heap(q.begin(), q.end(), CmpMax());
+        if (q.size() > cap) {
+            pop();
+        }
+    }
+    void
+    pop() {
+        std::pop_heap(q.begin(), q.end(), CmpMax());
+        q.pop_back();
+    }
+    // inner_index_interface.cpp:1141-1145: pop into slots count-1 .. 0 -> ascending.
+    uint64_t
+    drain(uint32_t* ids, float* dists) {
+        uint64_t n = q.size();
+        for (int64_t j = static_cast<int64_t>(n) - 1; j >= 0; --j) {
+            dists[j] = q.front().first;
+            ids[j] = q.front().second;
+            pop();
+        }
+        return n;
+    }
+};
+
+// algorithm/ivf/flat_bucket_searcher.cpp:62-104 and impl/reorder/flatten_reorder.cpp:99-110: push only
+// when the heap is not full or dist < cached top (strict), then pop down to topk.
+struct StrictMaxHeap {
+    std::vector<Rec> q;
+    uint64_t cap;
+    float top = std::numeric_limits<float>::max();
+    explicit StrictMaxHeap(uint64_t k) : cap(k) {
+        q.reserve(k + 1);
+    }
+    void
+    push(float d, uint32_t id) {
+        if (q.size() < cap || d < top) {
+            q.emplace_back(d, id);
+            std::push_heap(q.begin(), q.end(), CmpMax());
+        }
+        while (q.size() > cap) {
+            std::pop_heap(q.begin(), q.end(), CmpMax());
+            q.pop_back();
+        }
+        if (!q.empty() && q.size() == cap) {
+            top = q.front().first;
+        }
+    }
+    uint64_t
+    drain(uint32_t* ids, float* dists) {
+        uint64_t n = q.size();
+        for (int64_t j = static_cast<int64_t>(n) - 1; j >= 0; --j) {
+            dists[j] = q.front().first;
+            ids[j] = q.front().second;
+            std::pop_heap(q.begin(), q.end(), CmpMax());
+            q.pop_back();
+        }
+        return n;
+    }
+};
+
+// One (query, code) distance of the chosen store kind, as the quantizers' ComputeDistImpl return it:
+// L2 -> squared L2, IP/cosine -> 1 - ip (fp32_quantizer.cpp:164-188, scalar_quantizer.cpp:180-196).
+enum Kind { kFP32 = 0, kSQ8 = 1, kSQ4 = 2, kSQ4U = 3, kSQ8U = 4, kRaBitQ = 5 };
+
+struct Store {
+    int kind;
+    int metric;
+    uint64_t dim;
+    uint64_t code_size;
+    const uint8_t* codes;
+    const float* lb;    // per-dim (sq8/sq4) or &scalar (uniform)
+    const float* diff;  // per-dim (sq8/sq4) or &scalar (uniform)
+    int query_bits;     // rabitq only
+};
+
+inline float
+uniform_dist(const Store& s, const uint8_t* qcode, const uint8_t* code) {
+    // sq4_uniform_quantizer.cpp:166-201 ; sq8_uniform_quantizer.cpp:141-170
+    int bits = s.kind == kSQ4U ? 4 : 8;
+    UniformLayout l = uniform_layout(s.dim, bits, s.metric);
+    float levels = bits == 4 ? 15.0F : 255.0F;
+    float diff = *s.diff;
+    float lb = *s.lb;
+    float scalar_rate = static_cast<float>((diff / static_cast<double>(levels)) * (diff / static_cast<double>(levels)));
+    float result = static_cast<float>(bits == 4 ? sq4u_codes_ip(qcode, code, s.dim) : sq8u_codes_ip(qcode, code, s.dim));
+    if (s.metric == kL2) {
+        uint64_t n1, n2;
+        std::memcpy(&n1, qcode + l.offset_norm, 8);
+        std::memcpy(&n2, code + l.offset_norm, 8);
+        return (static_cast<float>(n1) + static_cast<float>(n2) - 2 * result) * scalar_rate;
+    }
+    float s1 = rd_f32(qcode + l.offset_sum);
+    float s2 = rd_f32(code + l.offset_sum);
+    result = lb * (s1 + s2) + scalar_rate * result + lb * lb;
+    return 1 - result;
+}
+
+// rabitq_quantizer.cpp:1775-1860, 1-bit base and 4-bit or 32-bit query.
+inline float
+rabitq_dist(const RabitqLayout& l, int metric, int query_bits, const uint8_t* qcode, const uint8_t* code) {
+    float inv_sqrt_d = 1.0F / std::sqrt(static_cast<float>(l.dim));
+    float ip_bq;
+    if (query_bits == 4) {
+        std::vector<uint8_t> tmp(l.aligned_dim / 8, 0);
+        std::memcpy(tmp.data(), code, l.offset_norm);
+        uint32_t ip = rabitq_sq4u_binary_ip(qcode, tmp.data(), l.aligned_dim);
+        float base_sum = rd_f32(code + l.offset_sum);
+        float query_sum = rd_f32(qcode + l.q_offset_sum);
+        float lb = rd_f32(qcode + l.q_offset_lb);
+        float delta = rd_f32(qcode + l.q_offset_delta);
+        ip_bq = recover_sq4u(ip, base_sum, query_sum, lb, delta, inv_sqrt_d, l.dim);
+    } else {
+        ip_bq = rabitq_float_binary_ip(reinterpret_cast<const float*>(qcode), code, l.dim, inv_sqrt_d);
+    }
+    float query_norm = rd_f32(qcode + l.q_offset_norm);
+    float base_norm = rd_f32(code + l.offset_norm);
+    float query_raw_norm = 0, base_raw_norm = 0;
+    if (l.has_raw_norm) {
+        query_raw_norm = rd_f32(qcode + l.q_offset_raw_norm);
+        base_raw_norm = rd_f32(code + l.offset_raw_norm);
+    }
+    float base_error = rd_f32(code + l.offset_error);
+    if (std::abs(base_error) < 1e-5) {
+        base_error = (base_error >= 0) ? 1.0F : -1.0F;
+    }
+    float ip_est = ip_bq / base_error;
+    float result = l2_ube(base_norm, query_norm, ip_est);
+    auto approx_zero = [](float v) { return std::abs(v) < 1e-5; };
+    if (metric == kCosine) {
+        if (approx_zero(query_raw_norm) || approx_zero(base_raw_norm)) {
+            result = 1;
+        } else {
+            result = 1 - (query_raw_norm * query_raw_norm + base_raw_norm * base_raw_norm - result) * 0.5F /
+                             (query_raw_norm * base_raw_norm);
+        }
+    }
+    if (metric == kIP) {
+        if (approx_zero(query_raw_norm) || approx_zero(base_raw_norm)) {
+            result = 1;
+        } else {
+            result = 1 - (query_raw_norm * query_raw_norm + base_raw_norm * base_raw_norm - result) * 0.5F;
+        }
+    }
+    return result;
+}
+
+inline float
+store_dist(const Store& s, const RabitqLayout* rl, const uint8_t* q, const uint8_t* code) {
+    const float* qf = reinterpret_cast<const float*>(q);
+    switch (s.kind) {
+        case kFP32: {
+            const float* x = reinterpret_cast<const float*>(code);
+            return s.metric == kL2 ? fp32_l2sqr(qf, x, s.dim) : 1 - fp32_ip(qf, x, s.dim);
+        }
+        case kSQ8:
+            return s.metric == kL2 ? sq8_l2sqr(qf, code, s.lb, s.diff, s.dim)
+                                   : 1 - sq8_ip(qf, code, s.lb, s.diff, s.dim);
+        case kSQ4:
+            return s.metric == kL2 ? sq4_l2sqr(qf, code, s.lb, s.diff, s.dim)
+                                   : 1 - sq4_ip(qf, code, s.lb, s.diff, s.dim);
+        case kSQ4U:
+        case kSQ8U:
+            return uniform_dist(s, q, code);
+        case kRaBitQ:
+            return rabitq_dist(*rl, s.metric, s.query_bits, q, code);
+    }
+    return 0;
+}
+
+}  // namespace
+
+// ================================================================= exported C entry points
+
+ORC_API float
+orc_fp32_l2sqr(const float* q, const float* x, uint64_t dim) {
+    return fp32_l2sqr(q, x, dim);
+}
+ORC_API float
+orc_fp32_ip(const float* q, const float* x, uint64_t dim) {
+    return fp32_ip(q, x, dim);
+}
+ORC_API float
+orc_normalize(const float* from, float* to, uint64_t dim) {
+    return normalize(from, to, dim);
+}
+ORC_API float
+orc_normalize_with_centroid(const float* from, const float* c, float* to, uint64_t dim) {
+    return normalize_with_centroid(from, c, to, dim);
+}
+ORC_API float
+orc_sq8_ip(const float* q, const uint8_t* c, const float* lb, const float* diff, uint64_t dim) {
+    return sq8_ip(q, c, lb, diff, dim);
+}
+ORC_API float
+orc_sq8_l2sqr(const float* q, const uint8_t* c, const float* lb, const float* diff, uint64_t dim) {
+    return sq8_l2sqr(q, c, lb, diff, dim);
+}
+ORC_API float
+orc_sq4_ip(const float* q, const uint8_t* c, const float* lb, const float* diff, uint64_t dim) {
+    return sq4_ip(q, c, lb, diff, dim);
+}
+ORC_API float
+orc_sq4_l2sqr(const float* q, const uint8_t* c, const float* lb, const float* diff, uint64_t dim) {
+    return sq4_l2sqr(q, c, lb, diff, dim);
+}
+ORC_API int32_t
+orc_sq4u_codes_ip(const uint8_t* a, const uint8_t* b, uint64_t dim) {
+    return sq4u_codes_ip(a, b, dim);
+}
+ORC_API int32_t
+orc_sq8u_codes_ip(const uint8_t* a, const uint8_t* b, uint64_t dim) {
+    return sq8u_codes_ip(a, b, dim);
+}
+ORC_API uint32_t
+orc_rabitq_sq4u_binary_ip(const uint8_t* planes, const uint8_t* bits, uint64_t dim) {
+    return rabitq_sq4u_binary_ip(planes, bits, dim);
+}
+ORC_API float
+orc_rabitq_float_binary_ip(const float* v, const uint8_t* bits, uint64_t dim, float inv_sqrt_d) {
+    return rabitq_float_binary_ip(v, bits, dim, inv_sqrt_d);
+}
+
+// ---- scalar-quantization trainer --------------------------------------------------------------
+// scalar_quantization_trainer.cpp:125-146: deterministic strided sample, at most max_sample rows.
+static uint64_t
+sq_sample(const float* data, uint64_t count, uint64_t dim, bool need_normalize, uint64_t max_sample,
+          std::vector<float>& out) {
+    uint64_t step = 2147483647UL % count;
+    uint64_t sample_count = max_sample;
+    if (count <= max_sample) {
+        step = 1;
+        sample_count = count;
+    }
+    out.resize(sample_count * dim);
+    for (uint64_t j = 0; j < sample_count; ++j) {
+        uint64_t idx = (j * step) % count;
+        if (need_normalize) {
+            normalize(data + idx * dim, out.data() + j * dim, dim);
+        } else {
+            std::memcpy(out.data() + j * dim, data + idx * dim, dim * sizeof(float));
+        }
+    }
+    return sample_count;
+}
+
+// scalar_quantization_trainer.cpp:72-122.  mode 1 = CLASSIC (min/max), 3 = TRUNC_BOUND (the default):
+// two bounded heaps per dimension, seeded with a sentinel, keep the ignore_count largest / smallest.
+static void
+sq_train_bounds(const float* s, uint64_t count, uint64_t dim, int bits, float trunc_rate, int mode, float* upper,
+                float* lower) {
+    if (mode == 1) {
+        for (uint64_t i = 0; i < dim; ++i) {
+            upper[i] = std::numeric_limits<float>::lowest();
+            lower[i] = std::numeric_limits<float>::max();
+            for (uint64_t j = 0; j < count; ++j) {
+                float v = s[j * dim + i];
+                upper[i] = std::max(upper[i], v);
+                lower[i] = std::min(lower[i], v);
+            }
+        }
+        return;
+    }
+    double ignore_rate = 0.001;
+    if (bits == 4) {
+        ignore_rate = trunc_rate;
+    }
+    auto ignore_count = static_cast<uint64_t>(static_cast<double>(count - 1) * ignore_rate);
+    ignore_count = ignore_count < 1 ? 1 : ignore_count;
+    for (uint64_t i = 0; i < dim; ++i) {
+        std::priority_queue<float, std::vector<float>, std::greater<>> heap_max;
+        std::priority_queue<float, std::vector<float>, std::less<>> heap_min;
+        heap_max.emplace(std::numeric_limits<float>::lowest());
+        heap_min.emplace(std::numeric_limits<float>::max());
+        for (uint64_t j = 0; j < count; ++j) {
+            float v = s[j * dim + i];
+            if (v > heap_max.top() || heap_max.size() < ignore_count) {
+                heap_max.emplace(v);
+            }
+            if (heap_max.size() > ignore_count) {
+                heap_max.pop();
+            }
+            if (v < heap_min.top() || heap_min.size() < ignore_count) {
+                heap_min.emplace(v);
+            }
+            if (heap_min.size() > ignore_count) {
+                heap_min.pop();
+            }
+        }
+        upper[i] = heap_max.top();
+        lower[i] = heap_min.top();
+    }
+}
+
+// ScalarQuantizationTrainer::Train (scalar_quantization_trainer.cpp:30-45) + ScalarQuantizer::TrainImpl
+// (scalar_quantizer.cpp:52-73): returns lower_bound[d] and diff[d] = upper - lower.
+ORC_API void
+orc_sq_train(const float* data, uint64_t count, uint64_t dim, int bits, int metric, int mode, float trunc_rate,
+             uint64_t max_sample, float* lb, float* diff) {
+    std::vector<float> sample;
+    uint64_t sc = sq_sample(data, count, dim, metric == kCosine, max_sample ? max_sample : 100000, sample);
+    sq_train_bounds(sample.data(), sc, dim, bits, trunc_rate, mode, diff, lb);
+    for (uint64_t i = 0; i < dim; ++i) {
+        diff[i] -= lb[i];
+    }
+}
+
+// ScalarQuantizationTrainer::TrainUniform (scalar_quantization_trainer.cpp:47-70) + the uniform
+// quantizers' TrainImpl (sq4_uniform_quantizer.cpp:86-108: TRUNC_BOUND; sq8_uniform_quantizer.cpp:76-98:
+// CLASSIC).  Returns scalar lower bound and diff.
+ORC_API void
+orc_sq_train_uniform(const float* data, uint64_t count, uint64_t dim, int bits, int metric, int mode, float trunc_rate,
+                     uint64_t max_sample, float* lb_out, float* diff_out) {
+    std::vector<float> sample;
+    uint64_t sc = sq_sample(data, count, dim, metric == kCosine, max_sample ? max_sample : 100000, sample);
+    std::vector<float> upper(dim), lower(dim);
+    sq_train_bounds(sample.data(), sc, dim, bits, trunc_rate, mode, upper.data(), lower.data());
+    float ub, lb;
+    if (mode == 1) {
+        ub = *std::max_element(upper.begin(), upper.end());
+        lb = *std::min_element(lower.begin(), lower.end());
+    } else {
+        ub = *std::min_element(upper.begin(), upper.end());
+        lb = *std::max_element(lower.begin(), lower.end());
+        if (lb > ub) {
+            std::swap(lb, ub);
+        }
+    }
+    *lb_out = lb;
+    *diff_out = ub - lb;
+}
+
+// ScalarQuantizer::EncodeOneImpl (scalar_quantizer.cpp:85-112): divide by diff[d], clamp, truncate.
+ORC_API void
+orc_sq_encode(const float* data, uint64_t n, uint64_t dim, int bits, int metric, const float* lb, const float* diff,
+              uint8_t* codes) {
+    uint64_t code_size = align_up(dim * bits, 8) / 8;
+    float levels = static_cast<float>((1 << bits) - 1);
+    std::vector<float> tmp(dim);
+    for (uint64_t i = 0; i < n; ++i) {
+        const float* cur = data + i * dim;
+        if (metric == kCosine) {
+            normalize(cur, tmp.data(), dim);
+            cur = tmp.data();
+        }
+        uint8_t* c = codes + i * code_size;
+        std::memset(c, 0, code_size);
+        for (uint64_t d = 0; d < dim; ++d) {
+            float delta;
+            if (diff[d] < std::numeric_limits<float>::epsilon()) {
+                delta = 1.0F;
+            } else {
+                delta = 1.0F * (cur[d] - lb[d]) / diff[d];
+            }
+            delta = clamp_delta(delta);
+            auto scaled = static_cast<uint8_t>(levels * delta);
+            uint64_t idx = (d * bits) / 8;
+            uint64_t off = (d * bits) % 8;
+            c[idx] |= scaled << off;
+        }
+    }
+}
+
+// ScalarQuantizer::DecodeOneImpl (scalar_quantizer.cpp:114-125).
+ORC_API void
+orc_sq_decode(const uint8_t* codes, uint64_t n, uint64_t dim, int bits, const float* lb, const float* diff,
+              float* data) {
+    uint64_t code_size = align_up(dim * bits, 8) / 8;
+    float levels = static_cast<float>(1 << bits) - 1.0F;
+    for (uint64_t i = 0; i < n; ++i) {
+        for (uint64_t d = 0; d < dim; ++d) {
+            uint64_t idx = (d * bits) / 8, off = (d * bits) % 8;
+            data[i * dim + d] =
+                static_cast<float>((codes[i * code_size + idx] >> off) & ((1 << bits) - 1)) / levels * diff[d] + lb[d];
+        }
+    }
+}
+
+ORC_API uint64_t
+orc_squ_code_size(uint64_t dim, int bits, int metric) {
+    return uniform_layout(dim, bits, metric).code_size;
+}
+
+// SQ4UniformQuantizer::EncodeOneImpl (sq4_uniform_quantizer.cpp:110-152) and SQ8UniformQuantizer::
+// EncodeOneImpl (sq8_uniform_quantizer.cpp:100-132): multiply by 1/diff, clamp, truncate.  Padding
+// bytes (which the reference leaves untouched) are written as zero.
+ORC_API void
+orc_squ_encode(const float* data, uint64_t n, uint64_t dim, int bits, int metric, float lb, float diff,
+               uint8_t* codes) {
+    UniformLayout l = uniform_layout(dim, bits, metric);
+    float levels = bits == 4 ? 15.0F : 255.0F;
+    std::vector<float> tmp(dim);
+    float inv_diff = diff == 0.0F ? 0.0F : 1.0F / diff;
+    for (uint64_t i = 0; i < n; ++i) {
+        const float* cur = data + i * dim;
+        if (metric == kCosine) {
+            normalize(cur, tmp.data(), dim);
+            cur = tmp.data();
+        }
+        uint8_t* c = codes + i * l.code_size;
+        std::memset(c, 0, l.code_size);
+        uint64_t norm = 0;
+        float sum = 0, codes_sum = 0;
+        for (uint64_t d = 0; d < dim; ++d) {
+            float delta = (cur[d] - lb) * inv_diff;
+            delta = clamp_delta(delta);
+            auto scaled = static_cast<uint8_t>(levels * delta);
+            if (bits == 4) {
+                if (d & 1) {
+                    c[d >> 1] |= scaled << 4;
+                } else {
+                    c[d >> 1] = scaled;
+                }
+            } else {
+                c[d] = scaled;
+            }
+            norm += static_cast<uint64_t>(scaled) * static_cast<uint64_t>(scaled);
+            sum += cur[d];
+            codes_sum += static_cast<float>(scaled);
+        }
+        if (metric == kL2) {
+            std::memcpy(c + l.offset_norm, &norm, 8);
+        }
+        if (l.has_sum) {
+            wr_f32(c + l.offset_sum, sum);
+            if (l.has_codes_sum) {
+                wr_f32(c + l.offset_codes_sum, codes_sum);
+            }
+        }
+    }
+}
+
+ORC_API float
+orc_squ_dist(const uint8_t* qcode, const uint8_t* code, uint64_t dim, int bits, int metric, float lb, float diff) {
+    Store s{bits == 4 ? kSQ4U : kSQ8U, metric, dim, 0, nullptr, &lb, &diff, 0};
+    return uniform_dist(s, qcode, code);
+}
+
+// ---- RaBitQ -----------------------------------------------------------------------------------
+ORC_API uint64_t
+orc_rabitq_code_size(uint64_t dim, int metric, int query_bits) {
+    return rabitq_layout(dim, metric, query_bits).code_size;
+}
+ORC_API uint64_t
+orc_rabitq_query_code_size(uint64_t dim, int metric, int query_bits) {
+    return rabitq_layout(dim, metric, query_bits).query_code_size;
+}
+
+// RaBitQuantizer::TrainImpl (rabitq_quantizer.cpp:209-254): centroid = rotation applied to the
+// fp32 running-sum mean of the data.  The rotation itself is an input (the reference draws it from
+// std::random_device, random_orthogonal_transformer.cpp:101-102).
+ORC_API void
+orc_rabitq_train(const float* data, uint64_t n, uint64_t dim, const float* rot, float* centroid) {
+    std::vector<float> mean(dim, 0.0F);
+    for (uint64_t i = 0; i < n; ++i) {
+        for (uint64_t d = 0; d < dim; ++d) {
+            mean[d] += data[i * dim + d];
+        }
+    }
+    for (uint64_t d = 0; d < dim; ++d) {
+        mean[d] = mean[d] / static_cast<float>(n);
+    }
+    rotate(rot, mean.data(), centroid, dim);
+}
+
+// RaBitQuantizer::EncodeOneInternal, 1-bit branch (rabitq_quantizer.cpp:724-856).
+ORC_API void
+orc_rabitq_encode(const float* data, uint64_t n, uint64_t dim, const float* rot, const float* centroid, int metric,
+                  int query_bits, uint8_t* codes) {
+    RabitqLayout l = rabitq_layout(dim, metric, query_bits);
+    float inv_sqrt_d = 1.0F / std::sqrt(static_cast<float>(dim));
+#pragma omp parallel
+    {
+        std::vector<float> t(dim), nd(dim);
+#pragma omp for schedule(static)
+        for (int64_t i = 0; i < static_cast<int64_t>(n); ++i) {
+            const float* x = data + i * dim;
+            uint8_t* c = codes + i * l.code_size;
+            std::memset(c, 0, l.code_size);
+            float raw_norm = 0;
+            if (l.has_raw_norm) {
+                for (uint64_t d = 0; d < dim; ++d) {
+                    raw_norm += x[d] * x[d];
+                }
+            }
+            raw_norm = std::sqrt(raw_norm);
+            rotate(rot, x, t.data(), dim);
+            float norm = normalize_with_centroid(t.data(), centroid, nd.data(), dim);
+            uint64_t binary_sum = 0;
+            for (uint64_t d = 0; d < dim; ++d) {
+                if (nd[d] >= 0.0F) {
+                    ++binary_sum;
+                    c[d / 8] |= static_cast<uint8_t>(1U << (d % 8));
+                }
+            }
+            float error = rabitq_float_binary_ip(nd.data(), c, dim, inv_sqrt_d);
+            wr_f32(c + l.offset_norm, norm);
+            wr_f32(c + l.offset_error, error);
+            if (l.has_sum) {
+                wr_f32(c + l.offset_sum, static_cast<float>(binary_sum));
+            }
+            if (l.has_raw_norm) {
+                wr_f32(c + l.offset_raw_norm, raw_norm);
+            }
+        }
+    }
+}
+
+// RaBitQuantizer::EncodeSQ + ReOrderSQ (rabitq_quantizer.cpp:2049-2088): per-query min/max, round to
+// nearest of 15 levels, then bit b of every dim goes to plane b (planes aligned_dim/8 bytes apart).
+ORC_API void
+orc_rabitq_encode_sq(const float* normed, uint64_t dim, uint8_t* quantized, float* upper, float* lower, float* delta,
+                     float* query_sum) {
+    float lb = std::numeric_limits<float>::max();
+    float ub = std::numeric_limits<float>::lowest();
+    for (uint64_t i = 0; i < dim; ++i) {
+        float v = normed[i];
+        if (v < lb) {
+            lb = v;
+        }
+        if (v > ub) {
+            ub = v;
+        }
+    }
+    float dl = (ub - lb) / 15;
+    float inv_delta = (std::abs(dl) < 1e-5) ? 0.0F : 1.0F / dl;
+    float qs = 0;
+    for (uint64_t i = 0; i < dim; ++i) {
+        auto val = std::round((normed[i] - lb) * inv_delta);
+        quantized[i] = static_cast<uint8_t>(val);
+        qs += static_cast<float>(val);
+    }
+    *upper = ub;
+    *lower = lb;
+    *delta = dl;
+    *query_sum = qs;
+}
+
+ORC_API void
+orc_rabitq_reorder_sq(const uint8_t* quantized, uint64_t dim, uint8_t* planes /* zeroed, 4*aligned_dim/8 */) {
+    uint64_t offset = ((dim + 511) / 512 * 512) / 8;
+    for (uint64_t d = 0; d < dim; ++d) {
+        for (uint64_t b = 0; b < 4; ++b) {
+            bool bit = (quantized[d] & (1 << b)) != 0;
+            planes[b * offset + d / 8] |= (static_cast<int32_t>(bit) * (1 << (d % 8)));
+        }
+    }
+}
+
+// RaBitQuantizer::ProcessQueryImpl (rabitq_quantizer.cpp:2130-2217).
+ORC_API void
+orc_rabitq_process_query(const float* query, uint64_t dim, const float* rot, const float* centroid, int metric,
+                         int query_bits, uint8_t* qcode) {
+    RabitqLayout l = rabitq_layout(dim, metric, query_bits);
+    std::memset(qcode, 0, l.query_code_size);
+    std::vector<float> t(dim), nd(dim);
+    float raw = 0;
+    if (l.has_raw_norm) {
+        for (uint64_t d = 0; d < dim; ++d) {
+            raw += query[d] * query[d];
+        }
+    }
+    raw = std::sqrt(raw);
+    rotate(rot, query, t.data(), dim);
+    float qnorm = normalize_with_centroid(t.data(), centroid, nd.data(), dim);
+    if (query_bits == 4) {
+        std::vector<uint8_t> quant(dim, 0);
+        float ub, lb, delta, qsum;
+        orc_rabitq_encode_sq(nd.data(), dim, quant.data(), &ub, &lb, &delta, &qsum);
+        orc_rabitq_reorder_sq(quant.data(), dim, qcode);
+        wr_f32(qcode + l.q_offset_lb, lb);
+        wr_f32(qcode + l.q_offset_delta, delta);
+        wr_f32(qcode + l.q_offset_sum, qsum);
+    } else {
+        std::memcpy(qcode, nd.data(), dim * sizeof(float));
+    }
+    wr_f32(qcode + l.q_offset_norm, qnorm);
+    if (l.has_raw_norm) {
+        wr_f32(qcode + l.q_offset_raw_norm, raw);
+    }
+}
+
+ORC_API float
+orc_rabitq_dist(const uint8_t* qcode, const uint8_t* code, uint64_t dim, int metric, int query_bits) {
+    RabitqLayout l = rabitq_layout(dim, metric, query_bits);
+    return rabitq_dist(l, metric, query_bits, qcode, code);
+}
+
+// ---- k-means ----------------------------------------------------------------------------------
+// KMeansCluster::find_nearest_one_with_blas (impl/cluster/kmeans_cluster.cpp:193-305).
+// distances[m] = -2 <c_m, x> (the SGEMM; OpenBLAS 0.3.24 is absent, so the contraction is a plain fp32
+// dot in element order), += y_sqr[m], first minimum, err += double(float(min + x_sqr)); returns err/n.
+ORC_API double
+orc_kmeans_assign(const float* x, uint64_t n, uint64_t dim, const float* cent, uint64_t k, int32_t* labels,
+                  float* min_dist /* may be null: min_m(||c||^2 - 2<c,x>) */) {
+    std::vector<float> y_sqr(k);
+    for (uint64_t j = 0; j < k; ++j) {
+        y_sqr[j] = fp32_ip(cent + j * dim, cent + j * dim, dim);
+    }
+    double error = 0.0;
+#pragma omp parallel
+    {
+        std::vector<float> dist(k);
+        double local = 0.0;
+#pragma omp for schedule(static)
+        for (int64_t i = 0; i < static_cast<int64_t>(n); ++i) {
+            const float* xi = x + i * dim;
+            for (uint64_t j = 0; j < k; ++j) {
+                dist[j] = -2.0F * fp32_ip(cent + j * dim, xi, dim);
+                dist[j] = 1.0F * y_sqr[j] + dist[j];
+            }
+            auto* me = std::min_element(dist.data(), dist.data() + k);
+            float x_sqr = fp32_ip(xi, xi, dim);
+            labels[i] = static_cast<int32_t>(me - dist.data());
+            if (min_dist != nullptr) {
+                min_dist[i] = *me;
+            }
+            local += static_cast<double>(*me + x_sqr);
+        }
+#pragma omp critical
+        error += local;
+    }
+    return error / static_cast<float>(n);
+}
+
+// Centroid update of KMeansCluster::Run (kmeans_cluster.cpp:108-172): fp32 sums of member rows in
+// blocks of 1024 rows (merged here in block order; the reference merges in thread-completion order),
+// scaled by 1/count.  Empty clusters are left untouched and reported through counts[j] == 0 (the
+// reference re-seeds them from std::random_device, :156-171 — the caller does that with its own RNG).
+ORC_API void
+orc_kmeans_update(const float* x, const int32_t* labels, uint64_t n, uint64_t dim, uint64_t k, float* cent,
+                  int32_t* counts) {
+    std::vector<float> sums(k * dim, 0.0F), local(k * dim);
+    std::vector<int32_t> lc(k);
+    std::fill(counts, counts + k, 0);
+    for (uint64_t s = 0; s < n; s += 1024) {
+        uint64_t e = std::min(s + 1024, n);
+        std::fill(local.begin(), local.end(), 0.0F);
+        std::fill(lc.begin(), lc.end(), 0);
+        for (uint64_t i = s; i < e; ++i) {
+            int32_t l = labels[i];
+            if (l >= 0 && l < static_cast<int32_t>(k)) {
+                lc[l]++;
+                for (uint64_t d = 0; d < dim; ++d) {
+                    local[l * dim + d] += x[i * dim + d];
+                }
+            }
+        }
+        for (uint64_t j = 0; j < k; ++j) {
+            if (lc[j] > 0) {
+                counts[j] += lc[j];
+                for (uint64_t d = 0; d < dim; ++d) {
+                    sums[j * dim + d] += local[j * dim + d];
+                }
+            }
+        }
+    }
+    for (uint64_t j = 0; j < k; ++j) {
+        if (counts[j] > 0) {
+            float inv = 1.0F / static_cast<float>(counts[j]);
+            for (uint64_t d = 0; d < dim; ++d) {
+                cent[j * dim + d] = sums[j * dim + d] * inv;
+            }
+        }
+    }
+}
+
+// Lloyd driver (kmeans_cluster.cpp:46-190) with the initial centroids given and empty clusters
+// re-seeded from mt19937(seed) + uniform_int_distribution<uint64_t>(0, n-1), drawn in cluster order.
+// Returns the loss of the last assignment (err / n).
+ORC_API double
+orc_kmeans_run(const float* x, uint64_t n, uint64_t dim, float* cent /* in: init, out: final */, uint64_t k, int iters,
+               uint64_t seed, int32_t* labels) {
+    std::mt19937 gen(static_cast<uint32_t>(seed));
+    std::vector<int32_t> counts(k);
+    double err = 0;
+    for (int it = 0; it < iters; ++it) {
+        err = orc_kmeans_assign(x, n, dim, cent, k, labels, nullptr);
+        orc_kmeans_update(x, labels, n, dim, k, cent, counts.data());
+        std::uniform_int_distribution<uint64_t> dis(0, n - 1);
+        for (uint64_t j = 0; j < k; ++j) {
+            if (counts[j] == 0) {
+                uint64_t idx = dis(gen);
+                std::memcpy(cent + j * dim, x + idx * dim, dim * sizeof(float));
+            }
+        }
+    }
+    return err;
+}
+
+// ---- flat scan with bounded heap (BruteForce::SearchWithRequest hot loop) ----------------------
+// algorithm/bruteforce/bruteforce.cpp:518-551: every inner id in order, dist -> fixed-size max-heap;
+// result packed ascending (inner_index_interface.cpp:1171-1200).  `queries` holds processed queries:
+// fp32 rows for fp32/sq8/sq4, encoded query codes for the uniform kinds and RaBitQ.  Rows with fewer
+// than k results are padded with id 0xFFFFFFFF / +inf.  OpenMP over queries mirrors the reference
+// evaluator (tools/eval/case/search_eval_case.cpp:233-248).
+ORC_API void
+orc_flat_scan_topk(int kind, int metric, uint64_t dim, const uint8_t* codes, uint64_t n, uint64_t code_size,
+                   const float* lb, const float* diff, int query_bits, const uint8_t* queries, uint64_t nq,
+                   uint64_t query_stride, uint64_t k, int strict_heap, uint32_t* out_ids, float* out_dists,
+                   int threads) {
+    Store s{kind, metric, dim, code_size, codes, lb, diff, query_bits};
+    RabitqLayout rl = rabitq_layout(dim, metric, query_bits ? query_bits : 4);
+#ifdef _OPENMP
+    if (threads > 0) {
+        omp_set_num_threads(threads);
+    }
+#endif
+#pragma omp parallel for schedule(dynamic)
+    for (int64_t qi = 0; qi < static_cast<int64_t>(nq); ++qi) {
+        const uint8_t* q = queries + qi * query_stride;
+        uint32_t* ids = out_ids + qi * k;
+        float* ds = out_dists + qi * k;
+        uint64_t cnt;
+        if (strict_heap) {
+            StrictMaxHeap h(k);
+            for (uint64_t i = 0; i < n; ++i) {
+                h.push(store_dist(s, &rl, q, codes + i * code_size), static_cast<uint32_t>(i));
+            }
+            cnt = h.drain(ids, ds);
+        } else {
+            FixedMaxHeap h(k);
+            for (uint64_t i = 0; i < n; ++i) {
+                h.push(store_dist(s, &rl, q, codes + i * code_size), static_cast<uint32_t>(i));
+            }
+            cnt = h.drain(ids, ds);
+        }
+        for (uint64_t j = cnt; j < k; ++j) {
+            ids[j] = 0xFFFFFFFFU;
+            ds[j] = std::numeric_limits<float>::infinity();
+        }
+    }
+}
+
+// All (query, code) distances, for small parity cases.
+ORC_API void
+orc_flat_dists(int kind, int metric, uint64_t dim, const uint8_t* codes, uint64_t n, uint64_t code_size,
+               const float* lb, const float* diff, int query_bits, const uint8_t* queries, uint64_t nq,
+               uint64_t query_stride, float* out /* nq x n */) {
+    Store s{kind, metric, dim, code_size, codes, lb, diff, query_bits};
+    RabitqLayout rl = rabitq_layout(dim, metric, query_bits ? query_bits : 4);
+#pragma omp parallel for schedule(static)
+    for (int64_t qi = 0; qi < static_cast<int64_t>(nq); ++qi) {
+        for (uint64_t i = 0; i < n; ++i) {
+            out[qi * n + i] = store_dist(s, &rl, queries + qi * query_stride, codes + i * code_size);
+        }
+    }
+}
+
+// ---- IVF --------------------------------------------------------------------------------------
+// Exact routing: the nprobe nearest centroids by fp32 distance (the reference routes through an HGraph
+// over the centroids, ivf_nearest_partition.cpp:99-147; its exact form is what `disable_bucket_scan`
+// reports, ivf.cpp:1589-1660).  Ascending distance, ties by heap order.
+ORC_API void
+orc_ivf_route(const float* cent, uint64_t nlist, uint64_t dim, int metric, const float* queries, uint64_t nq,
+              uint64_t nprobe, int32_t* out_buckets, float* out_dists) {
+    Store s{kFP32, metric == kCosine ? kIP : metric, dim, dim * 4, reinterpret_cast<const uint8_t*>(cent), nullptr,
+            nullptr, 0};
+#pragma omp parallel for schedule(dynamic)
+    for (int64_t qi = 0; qi < static_cast<int64_t>(nq); ++qi) {
+        FixedMaxHeap h(nprobe);
+        const auto* q = reinterpret_cast<const uint8_t*>(queries + qi * dim);
+        for (uint64_t j = 0; j < nlist; ++j) {
+            h.push(store_dist(s, nullptr, q, s.codes + j * s.code_size), static_cast<uint32_t>(j));
+        }
+        std::vector<uint32_t> ids(nprobe);
+        std::vector<float> ds(nprobe);
+        uint64_t cnt = h.drain(ids.data(), ds.data());
+        for (uint64_t j = 0; j < nprobe; ++j) {
+            out_buckets[qi * nprobe + j] = j < cnt ? static_cast<int32_t>(ids[j]) : -1;
+            out_dists[qi * nprobe + j] = j < cnt ? ds[j] : std::numeric_limits<float>::infinity();
+        }
+    }
+}
+
+// Posting lists as the reference fills them without a thread pool (ivf.cpp:590-724,
+// bucket_datacell.h:670-709): vectors appended to their bucket in input order -> a stable counting
+// sort by label.  offsets has nlist+1 entries; order[p] is the inner id at posting position p.
+ORC_API void
+orc_ivf_build_lists(const int32_t* labels, uint64_t n, uint64_t nlist, uint64_t* offsets, uint32_t* order) {
+    std::fill(offsets, offsets + nlist + 1, 0);
+    for (uint64_t i = 0; i < n; ++i) {
+        offsets[labels[i] + 1]++;
+    }
+    for (uint64_t j = 0; j < nlist; ++j) {
+        offsets[j + 1] += offsets[j];
+    }
+    std::vector<uint64_t> cur(offsets, offsets + nlist);
+    for (uint64_t i = 0; i < n; ++i) {
+        order[cur[labels[i]]++] = static_cast<uint32_t>(i);
+    }
+}
+
+// IVF::search<KNN> for one batch with routing injected (ivf.cpp:1693-1828): for each probed bucket in
+// the given order, scan the list (bucket_datacell.h:527-572) and feed (dist, inner id) to one
+// strict-`<` heap of size kcand (flat_bucket_searcher.cpp:62-104).  codes are in posting order.
+ORC_API void
+orc_ivf_scan(int kind, int metric, uint64_t dim, const uint8_t* codes, uint64_t code_size, const float* lb,
+             const float* diff, int query_bits, const uint64_t* offsets, const uint32_t* order,
+             const uint8_t* queries, uint64_t nq, uint64_t query_stride, const int32_t* buckets, uint64_t nprobe,
+             uint64_t kcand, uint32_t* out_ids, float* out_dists, int threads) {
+    Store s{kind, metric, dim, code_size, codes, lb, diff, query_bits};
+    RabitqLayout rl = rabitq_layout(dim, metric, query_bits ? query_bits : 4);
+#ifdef _OPENMP
+    if (threads > 0) {
+        omp_set_num_threads(threads);
+    }
+#endif
+#pragma omp parallel for schedule(dynamic)
+    for (int64_t qi = 0; qi < static_cast<int64_t>(nq); ++qi) {
+        StrictMaxHeap h(kcand);
+        const uint8_t* q = queries + qi * query_stride;
+        for (uint64_t p = 0; p < nprobe; ++p) {
+            int32_t b = buckets[qi * nprobe + p];
+            if (b < 0) {
+                continue;
+            }
+            for (uint64_t pos = offsets[b]; pos < offsets[b + 1]; ++pos) {
+                h.push(store_dist(s, &rl, q, codes + pos * code_size), order[pos]);
+            }
+        }
+        uint64_t cnt = h.drain(out_ids + qi * kcand, out_dists + qi * kcand);
+        for (uint64_t j = cnt; j < kcand; ++j) {
+            out_ids[qi * kcand + j] = 0xFFFFFFFFU;
+            out_dists[qi * kcand + j] = std::numeric_limits<float>::infinity();
+        }
+    }
+}
+
+// FlattenReorder::Reorder (impl/reorder/flatten_reorder.cpp:52-114): exact fp32 distance of every
+// candidate (in candidate order) into a strict-`<` heap of size k, packed ascending.
+ORC_API void
+orc_rerank_fp32(const float* raw, uint64_t dim, int metric, const float* queries, uint64_t nq, const uint32_t* cand,
+                uint64_t kcand, uint64_t k, uint32_t* out_ids, float* out_dists) {
+#pragma omp parallel for schedule(dynamic)
+    for (int64_t qi = 0; qi < static_cast<int64_t>(nq); ++qi) {
+        StrictMaxHeap h(k);
+        const float* q = queries + qi * dim;
+        for (uint64_t j = 0; j < kcand; ++j) {
+            uint32_t id = cand[qi * kcand + j];
+            if (id == 0xFFFFFFFFU) {
+                continue;
+            }
+            const float* x = raw + static_cast<uint64_t>(id) * dim;
+            float d = metric == kL2 ? fp32_l2sqr(q, x, dim) : 1 - fp32_ip(q, x, dim);
+            h.push(d, id);
+        }
+        uint64_t cnt = h.drain(out_ids + qi * k, out_dists + qi * k);
+        for (uint64_t j = cnt; j < k; ++j) {
+            out_ids[qi * k + j] = 0xFFFFFFFFU;
+            out_dists[qi * k + j] = std::numeric_limits<float>::infinity();
+        }
+    }
+}
+
+ORC_API int
+orc_max_threads() {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}

@@ -1,0 +1,290 @@
+"""ctypes access to the CPU checker (oracle/liboracle.so) and, when built, to the reference's own scalar
+kernels compiled from its sources (oracle/_ref/libvsag_generic.so).  Test infrastructure only."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+LIB = os.path.join(ORACLE_DIR, "liboracle.so")
+REF_GENERIC = os.path.join(ORACLE_DIR, "_ref", "libvsag_generic.so")
+
+L2, IP, COSINE = 0, 1, 2
+FP32, SQ8, SQ4, SQ4U, SQ8U, RABITQ = range(6)
+KIND_BITS = {SQ8: 8, SQ4: 4, SQ4U: 4, SQ8U: 8}
+
+_f32p = C.POINTER(C.c_float)
+_u8p = C.POINTER(C.c_uint8)
+_lib = None
+
+
+def build():
+    subprocess.run(["make", "-C", ORACLE_DIR, "liboracle.so"], check=True, stdout=subprocess.DEVNULL)
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB):
+            build()
+        _lib = C.CDLL(LIB)
+        _lib.orc_kmeans_assign.restype = C.c_double
+        _lib.orc_kmeans_run.restype = C.c_double
+        for name in ("orc_fp32_l2sqr", "orc_fp32_ip", "orc_sq8_ip", "orc_sq8_l2sqr", "orc_sq4_ip", "orc_sq4_l2sqr",
+                     "orc_squ_dist", "orc_rabitq_dist", "orc_normalize", "orc_normalize_with_centroid",
+                     "orc_rabitq_float_binary_ip"):
+            getattr(_lib, name).restype = C.c_float
+        for name in ("orc_squ_code_size", "orc_rabitq_code_size", "orc_rabitq_query_code_size"):
+            getattr(_lib, name).restype = C.c_uint64
+        _lib.orc_rabitq_sq4u_binary_ip.restype = C.c_uint32
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def u64(v):
+    return C.c_uint64(int(v))
+
+
+def sq_train(x, bits, metric=L2, mode=3, trunc_rate=0.05, max_sample=0):
+    x = f32(x)
+    n, d = x.shape
+    lb = np.empty(d, np.float32)
+    diff = np.empty(d, np.float32)
+    lib().orc_sq_train(_p(x), u64(n), u64(d), bits, metric, mode, C.c_float(trunc_rate), u64(max_sample), _p(lb),
+                       _p(diff))
+    return lb, diff
+
+
+def sq_train_uniform(x, bits, metric=L2, mode=3, trunc_rate=0.05, max_sample=0):
+    x = f32(x)
+    n, d = x.shape
+    lb = C.c_float()
+    diff = C.c_float()
+    lib().orc_sq_train_uniform(_p(x), u64(n), u64(d), bits, metric, mode, C.c_float(trunc_rate), u64(max_sample),
+                               C.byref(lb), C.byref(diff))
+    return np.float32(lb.value), np.float32(diff.value)
+
+
+def sq_encode(x, bits, lb, diff, metric=L2):
+    x = f32(x)
+    n, d = x.shape
+    cs = (d * bits + 7) // 8
+    codes = np.zeros((n, cs), np.uint8)
+    lib().orc_sq_encode(_p(x), u64(n), u64(d), bits, metric, _p(f32(lb)), _p(f32(diff)), _p(codes))
+    return codes
+
+
+def sq_decode(codes, d, bits, lb, diff):
+    n = codes.shape[0]
+    out = np.empty((n, d), np.float32)
+    lib().orc_sq_decode(_p(np.ascontiguousarray(codes)), u64(n), u64(d), bits, _p(f32(lb)), _p(f32(diff)), _p(out))
+    return out
+
+
+def squ_code_size(d, bits, metric):
+    return int(lib().orc_squ_code_size(u64(d), bits, metric))
+
+
+def squ_encode(x, bits, lb, diff, metric=L2):
+    x = f32(x)
+    n, d = x.shape
+    cs = squ_code_size(d, bits, metric)
+    codes = np.zeros((n, cs), np.uint8)
+    lib().orc_squ_encode(_p(x), u64(n), u64(d), bits, metric, C.c_float(lb), C.c_float(diff), _p(codes))
+    return codes
+
+
+def rabitq_code_size(d, metric, qbits=4):
+    return int(lib().orc_rabitq_code_size(u64(d), metric, qbits))
+
+
+def rabitq_query_code_size(d, metric, qbits=4):
+    return int(lib().orc_rabitq_query_code_size(u64(d), metric, qbits))
+
+
+def rabitq_train(x, rot):
+    x = f32(x)
+    n, d = x.shape
+    c = np.empty(d, np.float32)
+    lib().orc_rabitq_train(_p(x), u64(n), u64(d), _p(f32(rot)), _p(c))
+    return c
+
+
+def rabitq_encode(x, rot, centroid, metric, qbits=4):
+    x = f32(x)
+    n, d = x.shape
+    codes = np.zeros((n, rabitq_code_size(d, metric, qbits)), np.uint8)
+    lib().orc_rabitq_encode(_p(x), u64(n), u64(d), _p(f32(rot)), _p(f32(centroid)), metric, qbits, _p(codes))
+    return codes
+
+
+def rabitq_process_query(q, rot, centroid, metric, qbits=4):
+    q = f32(q)
+    nq, d = q.shape
+    qs = rabitq_query_code_size(d, metric, qbits)
+    out = np.zeros((nq, qs), np.uint8)
+    rot = f32(rot)
+    centroid = f32(centroid)
+    for i in range(nq):
+        lib().orc_rabitq_process_query(_p(q[i]), u64(d), _p(rot), _p(centroid), metric, qbits,
+                                       C.c_void_p(out.ctypes.data + i * qs))
+    return out
+
+
+def flat_scan_topk(kind, metric, d, codes, queries, k, lb=None, diff=None, qbits=4, strict=False, threads=0):
+    """codes: (n, code_size) uint8 (fp32 rows viewed as bytes); queries: processed queries, 2-D."""
+    codes = np.ascontiguousarray(codes)
+    queries = np.ascontiguousarray(queries)
+    n = codes.shape[0]
+    cs = codes.shape[1] * codes.itemsize
+    nq = queries.shape[0]
+    qstride = queries.shape[1] * queries.itemsize
+    ids = np.empty((nq, k), np.uint32)
+    dists = np.empty((nq, k), np.float32)
+    lbp = _p(f32(np.atleast_1d(lb))) if lb is not None else None
+    dfp = _p(f32(np.atleast_1d(diff))) if diff is not None else None
+    lib().orc_flat_scan_topk(kind, metric, u64(d), _p(codes), u64(n), u64(cs), lbp, dfp, qbits, _p(queries), u64(nq),
+                             u64(qstride), u64(k), int(strict), _p(ids), _p(dists), threads)
+    return ids, dists
+
+
+def flat_dists(kind, metric, d, codes, queries, lb=None, diff=None, qbits=4):
+    codes = np.ascontiguousarray(codes)
+    queries = np.ascontiguousarray(queries)
+    n = codes.shape[0]
+    cs = codes.shape[1] * codes.itemsize
+    nq = queries.shape[0]
+    qstride = queries.shape[1] * queries.itemsize
+    out = np.empty((nq, n), np.float32)
+    lbp = _p(f32(np.atleast_1d(lb))) if lb is not None else None
+    dfp = _p(f32(np.atleast_1d(diff))) if diff is not None else None
+    lib().orc_flat_dists(kind, metric, u64(d), _p(codes), u64(n), u64(cs), lbp, dfp, qbits, _p(queries), u64(nq),
+                         u64(qstride), _p(out))
+    return out
+
+
+def kmeans_assign(x, cent):
+    x = f32(x)
+    cent = f32(cent)
+    n, d = x.shape
+    k = cent.shape[0]
+    labels = np.empty(n, np.int32)
+    mind = np.empty(n, np.float32)
+    loss = lib().orc_kmeans_assign(_p(x), u64(n), u64(d), _p(cent), u64(k), _p(labels), _p(mind))
+    return labels, mind, loss
+
+
+def kmeans_update(x, labels, cent):
+    x = f32(x)
+    cent = f32(cent).copy()
+    n, d = x.shape
+    k = cent.shape[0]
+    counts = np.empty(k, np.int32)
+    lib().orc_kmeans_update(_p(x), _p(np.ascontiguousarray(labels, np.int32)), u64(n), u64(d), u64(k), _p(cent),
+                            _p(counts))
+    return cent, counts
+
+
+def kmeans_run(x, cent0, iters, seed):
+    x = f32(x)
+    cent = f32(cent0).copy()
+    n, d = x.shape
+    k = cent.shape[0]
+    labels = np.empty(n, np.int32)
+    loss = lib().orc_kmeans_run(_p(x), u64(n), u64(d), _p(cent), u64(k), iters, u64(seed), _p(labels))
+    return cent, labels, loss
+
+
+def ivf_route(cent, queries, nprobe, metric=L2):
+    cent = f32(cent)
+    queries = f32(queries)
+    nlist, d = cent.shape
+    nq = queries.shape[0]
+    b = np.empty((nq, nprobe), np.int32)
+    ds = np.empty((nq, nprobe), np.float32)
+    lib().orc_ivf_route(_p(cent), u64(nlist), u64(d), metric, _p(queries), u64(nq), u64(nprobe), _p(b), _p(ds))
+    return b, ds
+
+
+def ivf_build_lists(labels, nlist):
+    labels = np.ascontiguousarray(labels, np.int32)
+    n = labels.shape[0]
+    offsets = np.empty(nlist + 1, np.uint64)
+    order = np.empty(n, np.uint32)
+    lib().orc_ivf_build_lists(_p(labels), u64(n), u64(nlist), _p(offsets), _p(order))
+    return offsets, order
+
+
+def ivf_scan(kind, metric, d, codes_posting, offsets, order, queries, buckets, kcand, lb=None, diff=None, qbits=4,
+             threads=0):
+    codes = np.ascontiguousarray(codes_posting)
+    queries = np.ascontiguousarray(queries)
+    buckets = np.ascontiguousarray(buckets, np.int32)
+    cs = codes.shape[1] * codes.itemsize
+    nq, nprobe = buckets.shape
+    qstride = queries.shape[1] * queries.itemsize
+    ids = np.empty((nq, kcand), np.uint32)
+    dists = np.empty((nq, kcand), np.float32)
+    lbp = _p(f32(np.atleast_1d(lb))) if lb is not None else None
+    dfp = _p(f32(np.atleast_1d(diff))) if diff is not None else None
+    lib().orc_ivf_scan(kind, metric, u64(d), _p(codes), u64(cs), lbp, dfp, qbits,
+                       _p(np.ascontiguousarray(offsets, np.uint64)), _p(np.ascontiguousarray(order, np.uint32)),
+                       _p(queries), u64(nq), u64(qstride), _p(buckets), u64(nprobe), u64(kcand), _p(ids), _p(dists),
+                       threads)
+    return ids, dists
+
+
+def rerank_fp32(raw, queries, cand, k, metric=L2):
+    raw = f32(raw)
+    queries = f32(queries)
+    cand = np.ascontiguousarray(cand, np.uint32)
+    nq, kcand = cand.shape
+    d = raw.shape[1]
+    ids = np.empty((nq, k), np.uint32)
+    dists = np.empty((nq, k), np.float32)
+    lib().orc_rerank_fp32(_p(raw), u64(d), metric, _p(queries), u64(nq), _p(cand), u64(kcand), u64(k), _p(ids),
+                          _p(dists))
+    return ids, dists
+
+
+# ---- the reference's own scalar kernels, compiled from its sources (when oracle/_ref was built) ----------
+_ref = None
+_REF_SYMBOLS = {
+    "FP32ComputeIP": "_ZN4vsag7generic13FP32ComputeIPEPKfS2_m",
+    "FP32ComputeL2Sqr": "_ZN4vsag7generic16FP32ComputeL2SqrEPKfS2_m",
+    "SQ8ComputeIP": "_ZN4vsag7generic12SQ8ComputeIPEPKfPKhS2_S2_m",
+    "SQ8ComputeL2Sqr": "_ZN4vsag7generic15SQ8ComputeL2SqrEPKfPKhS2_S2_m",
+    "SQ4ComputeIP": "_ZN4vsag7generic12SQ4ComputeIPEPKfPKhS2_S2_m",
+    "SQ4ComputeL2Sqr": "_ZN4vsag7generic15SQ4ComputeL2SqrEPKfPKhS2_S2_m",
+    "SQ4UniformComputeCodesIP": "_ZN4vsag7generic24SQ4UniformComputeCodesIPEPKhS2_m",
+    "SQ8UniformComputeCodesIP": "_ZN4vsag7generic24SQ8UniformComputeCodesIPEPKhS2_m",
+    "RaBitQSQ4UBinaryIP": "_ZN4vsag7generic18RaBitQSQ4UBinaryIPEPKhS2_m",
+    "RaBitQFloatBinaryIP": "_ZN4vsag7generic19RaBitQFloatBinaryIPEPKfPKhmf",
+    "NormalizeWithCentroid": "_ZN4vsag7generic21NormalizeWithCentroidEPKfS2_Pfm",
+    "Normalize": "_ZN4vsag7generic9NormalizeEPKfPfm",
+}
+
+
+def ref():
+    """dict name -> ctypes function of vsag::generic, or None when oracle/_ref is not built."""
+    global _ref
+    if _ref is None:
+        if not os.path.exists(REF_GENERIC):
+            return None
+        dll = C.CDLL(REF_GENERIC)
+        fns = {}
+        for name, sym in _REF_SYMBOLS.items():
+            fn = getattr(dll, sym)
+            fn.restype = C.c_uint32 if name == "RaBitQSQ4UBinaryIP" else C.c_float
+            fns[name] = fn
+        _ref = fns
+    return _ref

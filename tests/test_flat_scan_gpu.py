@@ -1,0 +1,119 @@
+"""Parity of the HIP flat scan + fused top-k against the CPU checker, through the C ABI.
+
+Tolerances (stated by the task): float distances within 1e-4 relative; top-k ids identical where distance
+gaps exceed the tie band; integer paths (uniform codes) produce bit-identical distances."""
+import numpy as np
+import pytest
+
+import oracle as orc
+from gpu_helpers import Store, assert_topk_close, gaussian_mixture
+
+pytestmark = pytest.mark.gpu
+
+METRICS = [(orc.L2, "l2"), (orc.IP, "ip")]
+
+
+def _sq_case(rng, n, d, nq, bits):
+    x, means = gaussian_mixture(rng, n, d, 20, 0.05)
+    q, _ = gaussian_mixture(rng, nq, d, 20, 0.05, means=means)
+    lb, diff = orc.sq_train(x, bits)
+    codes = orc.sq_encode(x, bits, lb, diff)
+    return x, q, lb, diff, codes
+
+
+@pytest.mark.parametrize("metric,mname", METRICS)
+@pytest.mark.parametrize("n,d,nq,k", [(20000, 128, 37, 10), (1000, 33, 5, 10), (63, 7, 3, 4), (1, 16, 2, 3),
+                                      (5000, 960, 9, 100)])
+def test_sq8_flat_scan(lib, metric, mname, n, d, nq, k):
+    rng = np.random.default_rng(47 + n + d)
+    x, q, lb, diff, codes = _sq_case(rng, n, d, nq, 8)
+    st = Store(lib.KIND_SQ8, metric, d, lb=lb, diff=diff)
+    st.append(codes)
+    assert st.size() == n
+    ids, ds = st.flat_scan(q, k)
+    rids, rds = orc.flat_scan_topk(orc.SQ8, metric, d, codes, q, k, lb=lb, diff=diff)
+    assert_topk_close(ids, ds, rids, rds, label="sq8 %s n=%d d=%d" % (mname, n, d))
+    st.destroy()
+
+
+@pytest.mark.parametrize("metric,mname", METRICS)
+@pytest.mark.parametrize("n,d,nq,k", [(8000, 128, 17, 10), (500, 65, 4, 7)])
+def test_sq4_flat_scan(lib, metric, mname, n, d, nq, k):
+    rng = np.random.default_rng(48 + n + d)
+    x, q, lb, diff, codes = _sq_case(rng, n, d, nq, 4)
+    st = Store(lib.KIND_SQ4, metric, d, lb=lb, diff=diff)
+    st.append(codes)
+    ids, ds = st.flat_scan(q, k)
+    rids, rds = orc.flat_scan_topk(orc.SQ4, metric, d, codes, q, k, lb=lb, diff=diff)
+    assert_topk_close(ids, ds, rids, rds, label="sq4 %s n=%d d=%d" % (mname, n, d))
+    st.destroy()
+
+
+@pytest.mark.parametrize("metric,mname", METRICS + [(orc.COSINE, "cosine")])
+@pytest.mark.parametrize("n,d,nq,k", [(10000, 128, 21, 10), (300, 9, 3, 5), (4000, 960, 6, 64)])
+def test_fp32_flat_scan(lib, metric, mname, n, d, nq, k):
+    rng = np.random.default_rng(49 + n + d)
+    x = rng.random((n, d), dtype=np.float32)
+    q = rng.random((nq, d), dtype=np.float32)
+    st = Store(lib.KIND_FP32, metric, d)
+    st.append(x.view(np.uint8).reshape(n, 4 * d))
+    ids, ds = st.flat_scan(q, k)
+    if metric == orc.COSINE:
+        xn = x / np.sqrt((x.astype(np.float64) ** 2).sum(1, keepdims=True)).astype(np.float32)
+        qn = q / np.sqrt((q.astype(np.float64) ** 2).sum(1, keepdims=True)).astype(np.float32)
+        rids, rds = orc.flat_scan_topk(orc.FP32, orc.IP, d, xn.view(np.uint8).reshape(n, 4 * d), qn, k)
+        assert_topk_close(ids, ds, rids, rds, atol=2e-6, label="fp32 cosine")
+    else:
+        rids, rds = orc.flat_scan_topk(orc.FP32, metric, d, x.view(np.uint8).reshape(n, 4 * d), q, k)
+        assert_topk_close(ids, ds, rids, rds, atol=2e-6, label="fp32 %s n=%d d=%d" % (mname, n, d))
+    st.destroy()
+
+
+@pytest.mark.parametrize("metric,mname", METRICS)
+@pytest.mark.parametrize("bits,kind", [(4, "sq4u"), (8, "sq8u")])
+@pytest.mark.parametrize("n,d,nq,k", [(12000, 128, 19, 10), (700, 33, 4, 100)])
+def test_uniform_flat_scan_bit_exact(lib, metric, mname, bits, kind, n, d, nq, k):
+    rng = np.random.default_rng(50 + n + d + bits)
+    x, means = gaussian_mixture(rng, n, d, 20, 0.05)
+    q, _ = gaussian_mixture(rng, nq, d, 20, 0.05, means=means)
+    okind = orc.SQ4U if bits == 4 else orc.SQ8U
+    lkind = lib.KIND_SQ4_UNIFORM if bits == 4 else lib.KIND_SQ8_UNIFORM
+    lb, diff = orc.sq_train_uniform(x, bits, metric, mode=3 if bits == 4 else 1)
+    codes = orc.squ_encode(x, bits, lb, diff, metric)
+    qcodes = orc.squ_encode(q, bits, lb, diff, metric)
+    st = Store(lkind, metric, d, bounds=[lb, diff])
+    st.append(codes)
+    ids, ds = st.flat_scan(q, k)
+    rids, rds = orc.flat_scan_topk(okind, metric, d, codes, qcodes, k, lb=lb, diff=diff)
+    # integer inner products: the distance multiset must be identical bit for bit for L2; the IP form has
+    # three float operations whose order is kept, so it is bit-exact as well.
+    assert np.array_equal(ds.view(np.uint32), rds.view(np.uint32)), "%s %s distances differ" % (kind, mname)
+    assert_topk_close(ids, ds, rids, rds, rtol=0, atol=0, tie_rtol=0, label=kind)
+    st.destroy()
+
+
+def test_append_in_pieces_equals_one_append(lib):
+    rng = np.random.default_rng(7)
+    n, d = 3000, 48
+    x, q, lb, diff, codes = _sq_case(rng, n, d, 6, 8)
+    a = Store(lib.KIND_SQ8, orc.L2, d, lb=lb, diff=diff)
+    a.append(codes)
+    b = Store(lib.KIND_SQ8, orc.L2, d, lb=lb, diff=diff)
+    for s, e in [(0, 1), (1, 64), (64, 1000), (1000, 1001), (1001, 3000)]:
+        b.append(codes[s:e])
+    ia, da = a.flat_scan(q, 10)
+    ib, db = b.flat_scan(q, 10)
+    assert np.array_equal(ia, ib) and np.array_equal(da, db)
+    a.destroy()
+    b.destroy()
+
+
+def test_empty_store_and_bad_arguments(lib):
+    st = Store(lib.KIND_FP32, orc.L2, 8)
+    ids, ds = st.flat_scan(np.zeros((2, 8), np.float32), 3)
+    assert np.all(ids == 0xFFFFFFFF) and np.all(np.isinf(ds))
+    import ctypes as C
+    rc = lib.load_library().vsag_amd_flat_scan_topk(st.handle, None, 1, 0, None, None, None, 0, None)
+    assert rc == lib.INVALID_ARGUMENT
+    assert b"k must be" in lib.load_library().vsag_amd_last_error()
+    st.destroy()

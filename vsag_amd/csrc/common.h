@@ -1,0 +1,121 @@
+// Shared host/device helpers of the gfx950 search core: error plumbing, key encoding, tile geometry.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/vsag_amd.h"
+
+namespace vsag_amd {
+
+constexpr int kWave = 64;          // gfx950 wavefront width; one code tile holds 64 codes
+constexpr int kGranule = 16;       // bytes per lane per tile row (one dwordx4)
+constexpr uint32_t kMaxTopK = 1024;
+constexpr uint64_t kInfKey = 0xFFFFFFFFFFFFFFFFull;
+
+// ---- error plumbing -----------------------------------------------------------------------------
+char* last_error_buffer();  // thread-local, 1024 bytes
+
+inline int
+fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(last_error_buffer(), 1024, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+#define VA_HIP(expr)                                                                                     \
+    do {                                                                                                 \
+        hipError_t err__ = (expr);                                                                       \
+        if (err__ != hipSuccess) {                                                                       \
+            return ::vsag_amd::fail(err__ == hipErrorOutOfMemory ? VSAG_AMD_NO_ENOUGH_MEMORY            \
+                                                                 : VSAG_AMD_INTERNAL_ERROR,             \
+                                    "%s failed: %s (%s:%d)", #expr, hipGetErrorString(err__), __FILE__, \
+                                    __LINE__);                                                           \
+        }                                                                                                \
+    } while (0)
+
+#define VA_CHECK_ARG(cond, ...)                                              \
+    do {                                                                     \
+        if (!(cond)) {                                                       \
+            return ::vsag_amd::fail(VSAG_AMD_INVALID_ARGUMENT, __VA_ARGS__); \
+        }                                                                    \
+    } while (0)
+
+#define VA_TRY(expr)          \
+    do {                      \
+        int rc__ = (expr);    \
+        if (rc__ != 0) {      \
+            return rc__;      \
+        }                     \
+    } while (0)
+
+int ensure_init();  // VSAG_AMD_INTERNAL_ERROR when no gfx950 device is usable
+int device_cu_count();
+
+inline uint64_t
+round_up(uint64_t v, uint64_t a) {
+    return (v + a - 1) / a * a;
+}
+inline uint64_t
+div_up(uint64_t v, uint64_t a) {
+    return (v + a - 1) / a;
+}
+
+// Carves 256-byte aligned pieces out of a caller-supplied workspace.
+struct Carver {
+    uint8_t* base;
+    size_t size;
+    size_t used = 0;
+    Carver(void* p, size_t n) : base(static_cast<uint8_t*>(p)), size(n) {
+    }
+    template <typename T>
+    T*
+    take(size_t count) {
+        size_t bytes = round_up(count * sizeof(T), 256);
+        T* r = reinterpret_cast<T*>(base + used);
+        used += bytes;
+        return r;
+    }
+    bool
+    ok() const {
+        return used <= size && (base != nullptr || used == 0);
+    }
+};
+
+// ---- (distance, id) keys --------------------------------------------------------------------------
+// A key orders by distance first and inner id second when compared as an unsigned 64-bit integer.
+__host__ __device__ inline uint32_t
+float_to_ordered(float f) {
+#ifdef __HIP_DEVICE_COMPILE__
+    uint32_t u = __float_as_uint(f);
+#else
+    uint32_t u;
+    memcpy(&u, &f, 4);
+#endif
+    return u ^ ((u >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+}
+
+__host__ __device__ inline float
+ordered_to_float(uint32_t u) {
+    u ^= (u >> 31) ? 0x80000000u : 0xFFFFFFFFu;
+#ifdef __HIP_DEVICE_COMPILE__
+    return __uint_as_float(u);
+#else
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+#endif
+}
+
+__host__ __device__ inline uint64_t
+make_key(float dist, uint32_t id) {
+    return (static_cast<uint64_t>(float_to_ordered(dist)) << 32) | id;
+}
+
+}  // namespace vsag_amd

@@ -1,0 +1,278 @@
+// Per-tile distance loops of every store kind: 64 codes (one per lane) against T queries at once.
+//
+// Every lane owns one code of the tile, so no cross-lane reduction is needed, and everything that is
+// the same for all codes (per-dimension scales, the T processed queries) is read through the constant
+// address space with wave-uniform addresses: the compiler turns those into s_load_dwordx16 and feeds
+// the values to the VALU as SGPR operands, which costs no vector instruction and no LDS bandwidth.
+//
+// Reference arithmetic restated here (one query x one code each):
+//   FP32   src/simd/kernels/compute_l2.h:27-76, compute_ip.h:38-90      (fp32_quantizer.cpp:164-188)
+//   SQ8    src/simd/kernels/sq8_compute.h:44-137                        (scalar_quantizer.cpp:180-196)
+//   SQ4    src/simd/generic.cpp:316-340, kernels/sq4_compute.h:21-95
+//   SQ4U   src/simd/generic.cpp:406-422 + sq4_uniform_quantizer.cpp:166-201
+//   SQ8U   src/simd/generic.cpp:424-431 + sq8_uniform_quantizer.cpp:141-170
+//   RaBitQ src/simd/generic.cpp:832-872 + rabitq_quantizer.cpp:915-939,1775-1860
+#pragma once
+
+#include "common.h"
+
+namespace vsag_amd {
+
+typedef const float __attribute__((address_space(4))) * cfloat_p;
+typedef const uint32_t __attribute__((address_space(4))) * cu32_p;
+
+__device__ inline cfloat_p
+as_const(const float* p) {
+    return (cfloat_p)(uintptr_t)p;
+}
+__device__ inline cu32_p
+as_const(const uint32_t* p) {
+    return (cu32_p)(uintptr_t)p;
+}
+
+struct ScanArgs {
+    const uint4* tiles;
+    const uint32_t* meta;   // nmeta arrays of meta_stride words
+    uint64_t meta_stride;
+    const float* scale;     // sq8/sq4: per-dim scale, dpad floats
+    const uint32_t* qtab;   // processed queries, qstride words each
+    const float* qmeta;     // per-query scalars, qmeta_stride floats each
+    uint32_t qstride;
+    uint32_t qmeta_stride;
+    uint32_t G;
+    uint32_t dim;
+    float f0, f1, f2;       // uniform kinds: lb, scalar_rate, lb*lb
+};
+
+template <int KIND, int METRIC, int T>
+__device__ inline void
+tile_distances(const ScanArgs& a, uint64_t tile, const uint32_t (&qidx)[T], uint32_t lane, float (&out)[T]) {
+    const uint4* tp = a.tiles + tile * a.G * kWave + lane;
+    const uint64_t slot = tile * kWave + lane;
+
+    if constexpr (KIND == VSAG_AMD_KIND_FP32) {
+        float acc[T];
+        cfloat_p qrow[T];
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            acc[t] = 0.0F;
+            qrow[t] = as_const(reinterpret_cast<const float*>(a.qtab) + static_cast<size_t>(qidx[t]) * a.qstride);
+        }
+        for (uint32_t j = 0; j < a.G; ++j) {
+            uint4 c = tp[j * kWave];
+            float x[4] = {__uint_as_float(c.x), __uint_as_float(c.y), __uint_as_float(c.z), __uint_as_float(c.w)};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+#pragma unroll
+                for (int t = 0; t < T; ++t) {
+                    float qv = qrow[t][4 * j + e];
+                    if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                        float d = x[e] - qv;
+                        acc[t] = fmaf(d, d, acc[t]);
+                    } else {
+                        acc[t] = fmaf(x[e], qv, acc[t]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            out[t] = METRIC == VSAG_AMD_METRIC_L2 ? acc[t] : 1.0F - acc[t];
+        }
+    } else if constexpr (KIND == VSAG_AMD_KIND_SQ8) {
+        // qtab row: L2 -> q[d] - lb[d];  IP -> q[d] * scale[d], qmeta[0] = sum q[d] * lb[d].
+        float acc[T];
+        cfloat_p qrow[T];
+        cfloat_p sc = as_const(a.scale);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            acc[t] = 0.0F;
+            qrow[t] = as_const(reinterpret_cast<const float*>(a.qtab) + static_cast<size_t>(qidx[t]) * a.qstride);
+        }
+        for (uint32_t j = 0; j < a.G; ++j) {
+            uint4 c = tp[j * kWave];
+            uint32_t w[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                float cf = static_cast<float>((w[e >> 2] >> (8 * (e & 3))) & 0xffU);
+                if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                    float y = cf * sc[16 * j + e];
+#pragma unroll
+                    for (int t = 0; t < T; ++t) {
+                        float d = y - qrow[t][16 * j + e];
+                        acc[t] = fmaf(d, d, acc[t]);
+                    }
+                } else {
+#pragma unroll
+                    for (int t = 0; t < T; ++t) {
+                        acc[t] = fmaf(cf, qrow[t][16 * j + e], acc[t]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                out[t] = acc[t];
+            } else {
+                out[t] = 1.0F - (acc[t] + a.qmeta[static_cast<size_t>(qidx[t]) * a.qmeta_stride]);
+            }
+        }
+    } else if constexpr (KIND == VSAG_AMD_KIND_SQ4) {
+        // Byte b of a code holds dim 2b in its low nibble and dim 2b+1 in its high nibble.
+        float acc[T];
+        cfloat_p qrow[T];
+        cfloat_p sc = as_const(a.scale);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            acc[t] = 0.0F;
+            qrow[t] = as_const(reinterpret_cast<const float*>(a.qtab) + static_cast<size_t>(qidx[t]) * a.qstride);
+        }
+        for (uint32_t j = 0; j < a.G; ++j) {
+            uint4 c = tp[j * kWave];
+            uint32_t w[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                uint32_t lo = w[m] & 0x0F0F0F0FU;
+                uint32_t hi = (w[m] >> 4) & 0x0F0F0F0FU;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    uint32_t src = (e & 1) ? hi : lo;
+                    float cf = static_cast<float>((src >> (8 * (e >> 1))) & 0xffU);
+                    uint32_t d = 32 * j + 8 * m + e;
+                    if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                        float y = cf * sc[d];
+#pragma unroll
+                        for (int t = 0; t < T; ++t) {
+                            float df = y - qrow[t][d];
+                            acc[t] = fmaf(df, df, acc[t]);
+                        }
+                    } else {
+#pragma unroll
+                        for (int t = 0; t < T; ++t) {
+                            acc[t] = fmaf(cf, qrow[t][d], acc[t]);
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                out[t] = acc[t];
+            } else {
+                out[t] = 1.0F - (acc[t] + a.qmeta[static_cast<size_t>(qidx[t]) * a.qmeta_stride]);
+            }
+        }
+    } else if constexpr (KIND == VSAG_AMD_KIND_SQ4_UNIFORM || KIND == VSAG_AMD_KIND_SQ8_UNIFORM) {
+        // Integer code x code inner product.  SQ4U qtab row: per code dword {low nibbles, high nibbles
+        // << 4 kept in place}; the high-nibble products come out 16x too large and are shifted back.
+        uint32_t acc_lo[T], acc_hi[T];
+        cu32_p qrow[T];
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            acc_lo[t] = 0;
+            acc_hi[t] = 0;
+            qrow[t] = as_const(a.qtab + static_cast<size_t>(qidx[t]) * a.qstride);
+        }
+        for (uint32_t j = 0; j < a.G; ++j) {
+            uint4 c = tp[j * kWave];
+            uint32_t w[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                if constexpr (KIND == VSAG_AMD_KIND_SQ4_UNIFORM) {
+                    uint32_t lo = w[m] & 0x0F0F0F0FU;
+                    uint32_t hi = w[m] & 0xF0F0F0F0U;
+#pragma unroll
+                    for (int t = 0; t < T; ++t) {
+                        acc_lo[t] = __builtin_amdgcn_udot4(lo, qrow[t][2 * (4 * j + m)], acc_lo[t], false);
+                        acc_hi[t] = __builtin_amdgcn_udot4(hi, qrow[t][2 * (4 * j + m) + 1], acc_hi[t], false);
+                    }
+                } else {
+#pragma unroll
+                    for (int t = 0; t < T; ++t) {
+                        acc_lo[t] = __builtin_amdgcn_udot4(w[m], qrow[t][4 * j + m], acc_lo[t], false);
+                    }
+                }
+            }
+        }
+        float m0 = __uint_as_float(a.meta[slot]);
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            uint32_t ip = KIND == VSAG_AMD_KIND_SQ4_UNIFORM ? acc_lo[t] + (acc_hi[t] >> 4) : acc_lo[t];
+            float result = static_cast<float>(static_cast<int32_t>(ip));
+            float qm = a.qmeta[static_cast<size_t>(qidx[t]) * a.qmeta_stride];
+            if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                // (float(norm_q) + float(norm_o) - 2 ip) * scalar_rate
+                out[t] = (qm + m0 - 2 * result) * a.f1;
+            } else {
+                // 1 - (lb (sum_q + sum_o) + scalar_rate ip + lb^2)
+                float r = a.f0 * (qm + m0) + a.f1 * result + a.f2;
+                out[t] = 1 - r;
+            }
+        }
+    } else if constexpr (KIND == VSAG_AMD_KIND_RABITQ) {
+        // qtab row: per code dword the four query bit planes.  qmeta: {2 delta/sqrt(d), 2 lb/sqrt(d),
+        // delta sum_q/sqrt(d), lb d/sqrt(d), ||Rq - c||, ||q||}.
+        uint32_t acc[T][4];
+        cu32_p qrow[T];
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            acc[t][0] = acc[t][1] = acc[t][2] = acc[t][3] = 0;
+            qrow[t] = as_const(a.qtab + static_cast<size_t>(qidx[t]) * a.qstride);
+        }
+        for (uint32_t j = 0; j < a.G; ++j) {
+            uint4 c = tp[j * kWave];
+            uint32_t w[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+#pragma unroll
+                for (int t = 0; t < T; ++t) {
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) {
+                        acc[t][b] += __builtin_popcount(w[m] & qrow[t][4 * (4 * j + m) + b]);
+                    }
+                }
+            }
+        }
+        float base_norm = __uint_as_float(a.meta[slot]);
+        float base_error = __uint_as_float(a.meta[a.meta_stride + slot]);
+        float base_sum = __uint_as_float(a.meta[2 * a.meta_stride + slot]);
+        float base_raw = METRIC == VSAG_AMD_METRIC_L2 ? 0.0F : __uint_as_float(a.meta[3 * a.meta_stride + slot]);
+        if (fabsf(base_error) < 1e-5F) {
+            base_error = (base_error >= 0) ? 1.0F : -1.0F;
+        }
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const float* qm = a.qmeta + static_cast<size_t>(qidx[t]) * a.qmeta_stride;
+            uint32_t ip = acc[t][0] + (acc[t][1] << 1) + (acc[t][2] << 2) + (acc[t][3] << 3);
+            float p1 = qm[0] * static_cast<float>(ip);
+            float p2 = qm[1] * base_sum;
+            float ip_bq = p1 + p2 - qm[2] - qm[3];
+            float ip_est = ip_bq / base_error;
+            float qn = qm[4];
+            float e1 = base_norm * base_norm;
+            float e2 = qn * qn;
+            float e3 = -2 * base_norm * qn * ip_est;
+            float result = e1 + e2 + e3;
+            if constexpr (METRIC == VSAG_AMD_METRIC_IP) {
+                float qr = qm[5];
+                if (fabsf(qr) < 1e-5F || fabsf(base_raw) < 1e-5F) {
+                    result = 1;
+                } else {
+                    result = 1 - (qr * qr + base_raw * base_raw - result) * 0.5F;
+                }
+            } else if constexpr (METRIC == VSAG_AMD_METRIC_COSINE) {
+                float qr = qm[5];
+                if (fabsf(qr) < 1e-5F || fabsf(base_raw) < 1e-5F) {
+                    result = 1;
+                } else {
+                    result = 1 - (qr * qr + base_raw * base_raw - result) * 0.5F / (qr * base_raw);
+                }
+            }
+            out[t] = result;
+        }
+    }
+}
+
+}  // namespace vsag_amd

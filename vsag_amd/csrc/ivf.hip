@@ -1,0 +1,599 @@
+// Batched IVF search: exact routing, posting-list scan with a fused per-(query, list) top-k, per-query
+// merge, fp32 rerank (IVF::search<KNN_SEARCH>, src/algorithm/ivf/ivf.cpp:1693-1828; BucketDataCell::
+// ScanBucketById, src/datacell/bucket_datacell.h:527-572; FlatBucketSearcher::Search,
+// src/algorithm/ivf/flat_bucket_searcher.cpp:26-138; FlattenReorder::Reorder,
+// src/impl/reorder/flatten_reorder.cpp:52-114).
+//
+// The reference walks "for each query, for each probed list".  Here the (query, list) pairs of the whole
+// batch are regrouped by list on the device, so that one wave streams a posting list once for up to T
+// queries that probe it.  A pair keeps its own LDS selector; what it cannot beat is cut off early by a
+// per-query bound shared through global memory: the first probed list of every query is scanned in a
+// first launch and its kcand-th distance seeds the bound for the remaining lists.  The bound only ever
+// drops candidates that cannot be in the final kcand, so the result does not depend on scheduling.
+#include "distance.h"
+#include "store.h"
+#include "topk.h"
+
+namespace vsag_amd {
+
+struct ScanPlanIvf {
+    int T;
+    uint32_t S;
+    QueryLayout ql;
+    size_t qcode_bytes;
+    uint64_t npairs;
+    uint64_t max_items;
+};
+
+uint64_t rabitq_query_code_size(uint32_t dim, int metric, int query_bits);
+int prepare_queries(const vsag_amd_store* s, const float* queries, uint64_t nq, uint64_t nq_pad, const QueryLayout& ql,
+                    uint32_t* qtab, float* qmeta, uint8_t* qcodes, hipStream_t st);
+ScanArgs make_scan_args(const vsag_amd_store* s, const QueryLayout& ql, const uint32_t* qtab, const float* qmeta);
+void timing_begin(hipStream_t st);
+void timing_end(hipStream_t st);
+
+__global__ void
+fill32_kernel(uint32_t* p, uint32_t v, uint64_t n) {
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) {
+        p[i] = v;
+    }
+}
+
+// Pairs of probe columns [p0, p1): how many queries probe each list.
+__global__ void
+count_pairs_kernel(const int32_t* buckets, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t p1, uint32_t nlist,
+                   uint32_t* counts) {
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    uint32_t w = p1 - p0;
+    if (i >= nq * w) {
+        return;
+    }
+    uint64_t q = i / w;
+    uint32_t p = p0 + static_cast<uint32_t>(i % w);
+    int32_t b = buckets[q * nprobe + p];
+    if (b >= 0 && static_cast<uint32_t>(b) < nlist) {
+        atomicAdd(&counts[b], 1U);
+    }
+}
+
+// One workgroup: exclusive prefix sums of the pair counts and of the work items ceil(count / T).
+__global__ void __launch_bounds__(1024)
+offsets_kernel(const uint32_t* counts, uint32_t nlist, uint32_t T, uint32_t* pair_off, uint32_t* item_off) {
+    __shared__ uint32_t s_pairs[1024];
+    __shared__ uint32_t s_items[1024];
+    uint32_t per = (nlist + blockDim.x - 1) / blockDim.x;
+    uint32_t begin = threadIdx.x * per;
+    uint32_t end = begin + per < nlist ? begin + per : nlist;
+    uint32_t sp = 0, si = 0;
+    for (uint32_t i = begin; i < end; ++i) {
+        sp += counts[i];
+        si += (counts[i] + T - 1) / T;
+    }
+    s_pairs[threadIdx.x] = sp;
+    s_items[threadIdx.x] = si;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t rp = 0, ri = 0;
+        for (uint32_t i = 0; i < blockDim.x; ++i) {
+            uint32_t tp = s_pairs[i], ti = s_items[i];
+            s_pairs[i] = rp;
+            s_items[i] = ri;
+            rp += tp;
+            ri += ti;
+        }
+        pair_off[nlist] = rp;
+        item_off[nlist] = ri;
+    }
+    __syncthreads();
+    uint32_t rp = s_pairs[threadIdx.x], ri = s_items[threadIdx.x];
+    for (uint32_t i = begin; i < end; ++i) {
+        pair_off[i] = rp;
+        item_off[i] = ri;
+        rp += counts[i];
+        ri += (counts[i] + T - 1) / T;
+    }
+}
+
+__global__ void
+scatter_pairs_kernel(const int32_t* buckets, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t p1, uint32_t nlist,
+                     const uint32_t* pair_off, uint32_t* cursor, uint32_t* sorted_pair) {
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    uint32_t w = p1 - p0;
+    if (i >= nq * w) {
+        return;
+    }
+    uint64_t q = i / w;
+    uint32_t p = p0 + static_cast<uint32_t>(i % w);
+    int32_t b = buckets[q * nprobe + p];
+    if (b >= 0 && static_cast<uint32_t>(b) < nlist) {
+        uint32_t pos = pair_off[b] + atomicAdd(&cursor[b], 1U);
+        sorted_pair[pos] = static_cast<uint32_t>(q * nprobe + p);
+    }
+}
+
+struct IvfArgs {
+    const uint32_t* ids;         // inner id per tile slot
+    const uint32_t* list_tile;   // nlist+1
+    const uint32_t* pair_off;    // nlist+1
+    const uint32_t* item_off;    // nlist+1
+    const uint32_t* sorted_pair; // pair index (q * nprobe + p) grouped by list
+    uint32_t nlist;
+    uint32_t nprobe;
+    uint32_t dummy_query;        // index of an all-zero query row
+    uint32_t k;
+    uint32_t S;
+    uint32_t* bound;             // per query: ordered distance no final candidate can exceed
+    uint64_t* partial;           // npairs_total x k keys
+    uint32_t* partial_cnt;       // npairs_total
+};
+
+template <int KIND, int METRIC, int T>
+__global__ void __launch_bounds__(256)
+ivf_scan_kernel(ScanArgs a, IvfArgs v) {
+    extern __shared__ uint64_t lds[];
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t item = blockIdx.x * (blockDim.x >> 6) + wave;
+    const uint32_t total = as_const(v.item_off)[v.nlist];
+    if (item >= total) {
+        return;
+    }
+    // Which list: last b with item_off[b] <= item.
+    cu32_p ioff = as_const(v.item_off);
+    uint32_t lo = 0, hi = v.nlist;
+    while (hi - lo > 1) {
+        uint32_t mid = (lo + hi) >> 1;
+        if (ioff[mid] <= item) {
+            lo = mid;
+        } else {
+            hi = mid;
+        }
+    }
+    const uint32_t b = lo;
+    const uint32_t group = item - ioff[b];
+    const uint32_t pbeg = as_const(v.pair_off)[b] + group * T;
+    const uint32_t pend = as_const(v.pair_off)[b + 1];
+
+    const uint32_t S = v.S, k = v.k;
+    uint64_t* sel = lds + static_cast<size_t>(wave) * T * S;
+    uint32_t qidx[T], pair[T];
+    uint64_t tau[T];
+    uint32_t cnt[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        bool live = pbeg + t < pend;
+        pair[t] = live ? as_const(v.sorted_pair)[pbeg + t] : 0xFFFFFFFFU;
+        qidx[t] = live ? pair[t] / v.nprobe : v.dummy_query;
+        cnt[t] = 0;
+        uint32_t bound = live ? __builtin_amdgcn_readfirstlane(__atomic_load_n(&v.bound[qidx[t]], __ATOMIC_RELAXED))
+                              : 0U;
+        // Everything at or below the bound passes, whatever its id.
+        tau[t] = (static_cast<uint64_t>(bound) << 32) | 0xFFFFFFFFULL;
+    }
+    for (uint32_t i = lane; i < T * S; i += kWave) {
+        sel[i] = kInfKey;
+    }
+    wave_lds_fence();
+
+    const uint32_t tbeg = as_const(v.list_tile)[b], tend = as_const(v.list_tile)[b + 1];
+    for (uint32_t tile = tbeg; tile < tend; ++tile) {
+        float d[T];
+        tile_distances<KIND, METRIC, T>(a, tile, qidx, lane, d);
+        const uint32_t id = v.ids[static_cast<uint64_t>(tile) * kWave + lane];
+        const bool valid = id != VSAG_AMD_INVALID_ID;
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            uint64_t key = make_key(d[t], id);
+            bool pass = valid && key < tau[t];
+            uint64_t* keys = sel + t * S;
+            cnt[t] = selector_append(keys, k, cnt[t], pass, key);
+            if (cnt[t] + kWave > S - k) {
+                uint64_t th = selector_flush(keys, S, k, cnt[t], lane);
+                cnt[t] = 0;
+                if (pair[t] != 0xFFFFFFFFU) {
+                    uint32_t bound;
+                    if (th != kInfKey) {
+                        // This pair alone already holds k candidates at or below th.
+                        uint32_t mine = static_cast<uint32_t>(th >> 32);
+                        uint32_t old = lane == 0 ? atomicMin(&v.bound[qidx[t]], mine) : 0U;
+                        old = __builtin_amdgcn_readfirstlane(old);
+                        bound = old < mine ? old : mine;
+                    } else {
+                        bound = __builtin_amdgcn_readfirstlane(__atomic_load_n(&v.bound[qidx[t]], __ATOMIC_RELAXED));
+                    }
+                    uint64_t shared_tau = (static_cast<uint64_t>(bound) << 32) | 0xFFFFFFFFULL;
+                    tau[t] = th < shared_tau ? th : shared_tau;
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        if (pair[t] == 0xFFFFFFFFU) {
+            continue;
+        }
+        uint64_t* keys = sel + t * S;
+        uint64_t th = selector_flush(keys, S, k, cnt[t], lane);
+        if (th != kInfKey && lane == 0) {
+            atomicMin(&v.bound[qidx[t]], static_cast<uint32_t>(th >> 32));
+        }
+        uint64_t* dst = v.partial + static_cast<uint64_t>(pair[t]) * k;
+        uint32_t valid_count = 0;
+        for (uint32_t i0 = 0; i0 < k; i0 += kWave) {
+            uint32_t i = i0 + lane;
+            uint64_t key = i < k ? keys[i] : kInfKey;
+            bool ok = key != kInfKey;
+            if (ok) {
+                dst[i] = key;
+            }
+            valid_count += __popcll(__ballot(ok));
+        }
+        if (lane == 0) {
+            v.partial_cnt[pair[t]] = valid_count;
+        }
+    }
+}
+
+// One wave per query: best k keys over the partial lists of its nprobe pairs.
+__global__ void __launch_bounds__(64)
+ivf_merge_kernel(const uint64_t* partial, const uint32_t* partial_cnt, uint32_t nprobe, uint32_t k, uint32_t S,
+                 uint32_t* ids, float* dists) {
+    extern __shared__ uint64_t lds[];
+    const uint32_t lane = threadIdx.x;
+    const uint64_t q = blockIdx.x;
+    selector_init(lds, S, lane);
+    uint32_t cnt = 0;
+    uint64_t tau = kInfKey;
+    for (uint32_t p = 0; p < nprobe; ++p) {
+        uint64_t pair = q * nprobe + p;
+        uint32_t c = as_const(partial_cnt)[pair];
+        const uint64_t* src = partial + pair * k;
+        for (uint32_t base = 0; base < c; base += kWave) {
+            uint32_t i = base + lane;
+            uint64_t key = i < c ? src[i] : kInfKey;
+            bool pass = key < tau;
+            cnt = selector_append(lds, k, cnt, pass, key);
+            if (cnt + kWave > S - k) {
+                tau = selector_flush(lds, S, k, cnt, lane);
+                cnt = 0;
+            }
+        }
+    }
+    selector_flush(lds, S, k, cnt, lane);
+    for (uint32_t i = lane; i < k; i += kWave) {
+        uint64_t key = lds[i];
+        if (key == kInfKey) {
+            ids[q * k + i] = VSAG_AMD_INVALID_ID;
+            dists[q * k + i] = __builtin_inff();
+        } else {
+            ids[q * k + i] = static_cast<uint32_t>(key);
+            dists[q * k + i] = ordered_to_float(static_cast<uint32_t>(key >> 32));
+        }
+    }
+}
+
+// Exact fp32 distances of the candidates of one query (one wave per query), best k kept.
+__global__ void __launch_bounds__(64)
+rerank_kernel(const float* raw, uint64_t n, uint32_t dim, int metric, const float* queries, const uint32_t* cand,
+              uint32_t kcand, uint32_t k, uint32_t S, uint32_t* ids, float* dists) {
+    extern __shared__ uint64_t lds[];
+    const uint32_t lane = threadIdx.x;
+    const uint64_t q = blockIdx.x;
+    const float* qv = queries + q * dim;
+    for (uint32_t i = lane; i < S; i += kWave) {
+        lds[i] = kInfKey;
+    }
+    wave_lds_fence();
+    float inv_norm = 1.0F;
+    if (metric == VSAG_AMD_METRIC_COSINE) {
+        float s = 0.0F;
+        for (uint32_t d = lane; d < dim; d += kWave) {
+            s = fmaf(qv[d], qv[d], s);
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            s += __shfl_xor(s, off);
+        }
+        inv_norm = s > 0.0F ? 1.0F / sqrtf(s) : 1.0F;
+    }
+    for (uint32_t j = 0; j < kcand; ++j) {
+        uint32_t id = as_const(cand)[q * kcand + j];
+        if (id == VSAG_AMD_INVALID_ID || id >= n) {
+            continue;
+        }
+        const float* x = raw + static_cast<uint64_t>(id) * dim;
+        float s = 0.0F, xx = 0.0F;
+        for (uint32_t d = lane; d < dim; d += kWave) {
+            float xv = x[d];
+            if (metric == VSAG_AMD_METRIC_L2) {
+                float t = qv[d] - xv;
+                s = fmaf(t, t, s);
+            } else {
+                s = fmaf(qv[d], xv, s);
+                xx = fmaf(xv, xv, xx);
+            }
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            s += __shfl_xor(s, off);
+            xx += __shfl_xor(xx, off);
+        }
+        float dist;
+        if (metric == VSAG_AMD_METRIC_L2) {
+            dist = s;
+        } else if (metric == VSAG_AMD_METRIC_IP) {
+            dist = 1.0F - s;
+        } else {
+            float xn = xx > 0.0F ? 1.0F / sqrtf(xx) : 1.0F;
+            dist = 1.0F - s * inv_norm * xn;
+        }
+        if (lane == 0) {
+            lds[j] = make_key(dist, id);
+        }
+    }
+    wave_lds_fence();
+    wave_bitonic_sort(lds, S, lane);
+    for (uint32_t i = lane; i < k; i += kWave) {
+        uint64_t key = lds[i];
+        if (key == kInfKey) {
+            ids[q * k + i] = VSAG_AMD_INVALID_ID;
+            dists[q * k + i] = __builtin_inff();
+        } else {
+            ids[q * k + i] = static_cast<uint32_t>(key);
+            dists[q * k + i] = ordered_to_float(static_cast<uint32_t>(key >> 32));
+        }
+    }
+}
+
+template <int KIND, int METRIC>
+static void
+launch_ivf_t(int T, dim3 grid, dim3 block, size_t lds, hipStream_t st, const ScanArgs& a, const IvfArgs& v) {
+    switch (T) {
+        case 1:
+            hipLaunchKernelGGL((ivf_scan_kernel<KIND, METRIC, 1>), grid, block, lds, st, a, v);
+            break;
+        case 2:
+            hipLaunchKernelGGL((ivf_scan_kernel<KIND, METRIC, 2>), grid, block, lds, st, a, v);
+            break;
+        default:
+            hipLaunchKernelGGL((ivf_scan_kernel<KIND, METRIC, 4>), grid, block, lds, st, a, v);
+            break;
+    }
+}
+
+template <int KIND>
+static void
+launch_ivf_m(int metric, int T, dim3 grid, dim3 block, size_t lds, hipStream_t st, const ScanArgs& a,
+             const IvfArgs& v) {
+    if (metric == VSAG_AMD_METRIC_L2) {
+        launch_ivf_t<KIND, VSAG_AMD_METRIC_L2>(T, grid, block, lds, st, a, v);
+    } else if (metric == VSAG_AMD_METRIC_COSINE && KIND == VSAG_AMD_KIND_RABITQ) {
+        launch_ivf_t<KIND, VSAG_AMD_METRIC_COSINE>(T, grid, block, lds, st, a, v);
+    } else {
+        launch_ivf_t<KIND, VSAG_AMD_METRIC_IP>(T, grid, block, lds, st, a, v);
+    }
+}
+
+static int
+launch_ivf(const vsag_amd_store* s, int T, dim3 grid, dim3 block, size_t lds, hipStream_t st, const ScanArgs& a,
+           const IvfArgs& v) {
+    switch (s->kind) {
+        case VSAG_AMD_KIND_FP32:
+            launch_ivf_m<VSAG_AMD_KIND_FP32>(s->metric, T, grid, block, lds, st, a, v);
+            break;
+        case VSAG_AMD_KIND_SQ8:
+            launch_ivf_m<VSAG_AMD_KIND_SQ8>(s->metric, T, grid, block, lds, st, a, v);
+            break;
+        case VSAG_AMD_KIND_SQ4:
+            launch_ivf_m<VSAG_AMD_KIND_SQ4>(s->metric, T, grid, block, lds, st, a, v);
+            break;
+        case VSAG_AMD_KIND_SQ4_UNIFORM:
+            launch_ivf_m<VSAG_AMD_KIND_SQ4_UNIFORM>(s->metric, T, grid, block, lds, st, a, v);
+            break;
+        case VSAG_AMD_KIND_SQ8_UNIFORM:
+            launch_ivf_m<VSAG_AMD_KIND_SQ8_UNIFORM>(s->metric, T, grid, block, lds, st, a, v);
+            break;
+        case VSAG_AMD_KIND_RABITQ:
+            launch_ivf_m<VSAG_AMD_KIND_RABITQ>(s->metric, T, grid, block, lds, st, a, v);
+            break;
+        default:
+            return fail(VSAG_AMD_INVALID_ARGUMENT, "unknown store kind %d", s->kind);
+    }
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
+struct IvfBuffers {
+    uint32_t* qtab;
+    float* qmeta;
+    uint8_t* qcodes;
+    uint32_t* counts;     // nlist + 1
+    uint32_t* cursor;     // nlist + 1
+    uint32_t* pair_off;   // nlist + 1
+    uint32_t* item_off;   // nlist + 1
+    uint32_t* sorted_pair;
+    uint32_t* bound;
+    uint32_t* partial_cnt;
+    uint64_t* partial;
+};
+
+static void
+plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, ScanPlanIvf* p) {
+    p->S = selector_slots(kcand);
+    uint64_t npairs = nq * nprobe;
+    uint64_t avg = s->nlist ? npairs / s->nlist : 1;
+    int t = 4;
+    if (s->kind == VSAG_AMD_KIND_RABITQ || ((s->kind == VSAG_AMD_KIND_SQ8 || s->kind == VSAG_AMD_KIND_SQ4) &&
+                                            s->metric == VSAG_AMD_METRIC_L2)) {
+        t = 2;
+    }
+    while (t > 1 && static_cast<uint64_t>(t) > avg) {
+        t >>= 1;
+    }
+    while (t > 1 && static_cast<size_t>(t) * p->S * 8 > 65536) {
+        t >>= 1;
+    }
+    p->T = t;
+    p->ql = query_layout(s);
+    p->qcode_bytes = 0;
+    if (s->kind == VSAG_AMD_KIND_SQ4_UNIFORM || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
+        p->qcode_bytes = nq * s->code_size;
+    } else if (s->kind == VSAG_AMD_KIND_RABITQ) {
+        p->qcode_bytes = nq * rabitq_query_code_size(s->dim, s->metric, s->query_bits);
+    }
+    p->npairs = npairs;
+    p->max_items = div_up(npairs, t) + s->nlist;
+}
+
+static size_t
+carve_ivf(Carver& c, const vsag_amd_store* s, const ScanPlanIvf& p, uint64_t nq, uint32_t kcand, IvfBuffers* b) {
+    b->qtab = c.take<uint32_t>((nq + 1) * p.ql.qstride);
+    b->qmeta = c.take<float>((nq + 1) * p.ql.qmeta);
+    b->qcodes = c.take<uint8_t>(p.qcode_bytes);
+    b->counts = c.take<uint32_t>(s->nlist + 1);
+    b->cursor = c.take<uint32_t>(s->nlist + 1);
+    b->pair_off = c.take<uint32_t>(s->nlist + 1);
+    b->item_off = c.take<uint32_t>(s->nlist + 1);
+    b->sorted_pair = c.take<uint32_t>(p.npairs);
+    b->bound = c.take<uint32_t>(nq);
+    b->partial_cnt = c.take<uint32_t>(p.npairs);
+    b->partial = c.take<uint64_t>(p.npairs * kcand);
+    return c.used;
+}
+
+static int
+check_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand) {
+    VA_CHECK_ARG(s != nullptr, "store is null");
+    VA_CHECK_ARG(s->nlist > 0, "ivf scan on a flat store");
+    VA_CHECK_ARG(kcand >= 1 && kcand <= kMaxTopK, "kcand must be in [1, %u], got %u", kMaxTopK, kcand);
+    VA_CHECK_ARG(nprobe >= 1 && nprobe <= 65536, "nprobe must be in [1, 65536], got %u", nprobe);
+    VA_CHECK_ARG(nq >= 1 && nq * nprobe < 0xFFFFFFFFull, "nq * nprobe must be below 2^32 - 1");
+    return 0;
+}
+
+static inline uint32_t
+blocks_for(uint64_t n) {
+    return static_cast<uint32_t>(div_up(n ? n : 1, 256));
+}
+
+}  // namespace vsag_amd
+
+using namespace vsag_amd;
+
+extern "C" size_t
+vsag_amd_ivf_route_workspace_bytes(const vsag_amd_store_t* centroids, uint64_t nq, uint32_t nprobe) {
+    return vsag_amd_flat_scan_workspace_bytes(centroids, nq, nprobe);
+}
+
+extern "C" int
+vsag_amd_ivf_route(const vsag_amd_store_t* centroids, const float* queries_dev, uint64_t nq, uint32_t nprobe,
+                   int32_t* buckets_dev, float* dists_dev, void* workspace_dev, size_t workspace_bytes, void* stream) {
+    VA_CHECK_ARG(centroids != nullptr && centroids->kind == VSAG_AMD_KIND_FP32,
+                 "routing needs an fp32 store of centroids");
+    // VSAG_AMD_INVALID_ID and -1 are the same 32 bits, so the id buffer is the bucket buffer.
+    return vsag_amd_flat_scan_topk(centroids, queries_dev, nq, nprobe, reinterpret_cast<uint32_t*>(buckets_dev),
+                                   dists_dev, workspace_dev, workspace_bytes, stream);
+}
+
+extern "C" size_t
+vsag_amd_ivf_scan_workspace_bytes(const vsag_amd_store_t* s, uint64_t nq, uint32_t nprobe, uint32_t kcand) {
+    if (check_ivf(s, nq, nprobe, kcand) != 0) {
+        return 0;
+    }
+    ScanPlanIvf p;
+    plan_ivf(s, nq, nprobe, kcand, &p);
+    Carver c(nullptr, 0);
+    IvfBuffers b;
+    return carve_ivf(c, s, p, nq, kcand, &b) + 256;
+}
+
+extern "C" int
+vsag_amd_ivf_scan_topk(const vsag_amd_store_t* s, const float* queries_dev, uint64_t nq, const int32_t* buckets_dev,
+                       uint32_t nprobe, uint32_t kcand, uint32_t* ids_dev, float* dists_dev, void* workspace_dev,
+                       size_t workspace_bytes, void* stream) {
+    VA_TRY(ensure_init());
+    VA_TRY(check_ivf(s, nq, nprobe, kcand));
+    VA_CHECK_ARG(queries_dev && buckets_dev && ids_dev && dists_dev, "null pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    ScanPlanIvf p;
+    plan_ivf(s, nq, nprobe, kcand, &p);
+    Carver c(workspace_dev, workspace_bytes);
+    IvfBuffers b;
+    carve_ivf(c, s, p, nq, kcand, &b);
+    VA_CHECK_ARG(c.ok(), "workspace too small: need %zu bytes, got %zu", c.used, workspace_bytes);
+
+    // Row nq of the query tables is the all-zero row that idle slots of a query tile point at.
+    VA_TRY(prepare_queries(s, queries_dev, nq, nq + 1, p.ql, b.qtab, b.qmeta, b.qcodes, st));
+    ScanArgs a = make_scan_args(s, p.ql, b.qtab, b.qmeta);
+    hipLaunchKernelGGL(fill32_kernel, dim3(blocks_for(nq)), dim3(256), 0, st, b.bound, 0xFFFFFFFFU, nq);
+    hipLaunchKernelGGL(fill32_kernel, dim3(blocks_for(p.npairs)), dim3(256), 0, st, b.partial_cnt, 0U, p.npairs);
+
+    IvfArgs v{};
+    v.ids = s->ids_dev;
+    v.list_tile = s->list_tile_dev;
+    v.pair_off = b.pair_off;
+    v.item_off = b.item_off;
+    v.sorted_pair = b.sorted_pair;
+    v.nlist = s->nlist;
+    v.nprobe = nprobe;
+    v.dummy_query = static_cast<uint32_t>(nq);
+    v.k = kcand;
+    v.S = p.S;
+    v.bound = b.bound;
+    v.partial = b.partial;
+    v.partial_cnt = b.partial_cnt;
+
+    uint32_t waves = 4;
+    while (waves > 1 && static_cast<size_t>(waves) * p.T * p.S * 8 > 65536) {
+        waves >>= 1;
+    }
+    size_t lds = static_cast<size_t>(waves) * p.T * p.S * 8;
+    // Two passes: the nearest list of every query first (it seeds the per-query bound), then the rest.
+    uint32_t cols[3] = {0, 1, nprobe};
+    timing_begin(st);
+    for (int pass = 0; pass < 2; ++pass) {
+        uint32_t p0 = cols[pass], p1 = cols[pass + 1];
+        if (p1 <= p0) {
+            continue;
+        }
+        uint64_t pairs = nq * (p1 - p0);
+        hipLaunchKernelGGL(fill32_kernel, dim3(blocks_for(s->nlist + 1)), dim3(256), 0, st, b.counts, 0U,
+                           static_cast<uint64_t>(s->nlist + 1));
+        hipLaunchKernelGGL(fill32_kernel, dim3(blocks_for(s->nlist + 1)), dim3(256), 0, st, b.cursor, 0U,
+                           static_cast<uint64_t>(s->nlist + 1));
+        hipLaunchKernelGGL(count_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq, nprobe, p0,
+                           p1, s->nlist, b.counts);
+        hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, st, b.counts, s->nlist,
+                           static_cast<uint32_t>(p.T), b.pair_off, b.item_off);
+        hipLaunchKernelGGL(scatter_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq, nprobe,
+                           p0, p1, s->nlist, b.pair_off, b.cursor, b.sorted_pair);
+        uint64_t max_items = div_up(pairs, p.T) + s->nlist;
+        dim3 grid(static_cast<uint32_t>(div_up(max_items, waves)));
+        VA_TRY(launch_ivf(s, p.T, grid, dim3(waves * kWave), lds, st, a, v));
+    }
+    timing_end(st);
+    hipLaunchKernelGGL(ivf_merge_kernel, dim3(static_cast<uint32_t>(nq)), dim3(kWave), p.S * 8, st, b.partial,
+                       b.partial_cnt, nprobe, kcand, p.S, ids_dev, dists_dev);
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
+extern "C" int
+vsag_amd_rerank_fp32(const float* raw_dev, uint64_t n, uint32_t dim, int metric, const float* queries_dev, uint64_t nq,
+                     const uint32_t* cand_ids_dev, uint32_t kcand, uint32_t k, uint32_t* ids_dev, float* dists_dev,
+                     void* stream) {
+    VA_TRY(ensure_init());
+    VA_CHECK_ARG(raw_dev && queries_dev && cand_ids_dev && ids_dev && dists_dev, "null pointer");
+    VA_CHECK_ARG(kcand >= 1 && kcand <= 4096, "kcand must be in [1, 4096], got %u", kcand);
+    VA_CHECK_ARG(k >= 1 && k <= kcand, "k must be in [1, kcand], got %u", k);
+    VA_CHECK_ARG(metric >= VSAG_AMD_METRIC_L2 && metric <= VSAG_AMD_METRIC_COSINE, "unknown metric %d", metric);
+    VA_CHECK_ARG(nq >= 1 && nq < (1ull << 31), "nq must be in [1, 2^31)");
+    uint32_t S = 64;
+    while (S < kcand) {
+        S <<= 1;
+    }
+    hipLaunchKernelGGL(rerank_kernel, dim3(static_cast<uint32_t>(nq)), dim3(kWave), S * 8,
+                       static_cast<hipStream_t>(stream), raw_dev, n, dim, metric, queries_dev, cand_ids_dev, kcand, k,
+                       S, ids_dev, dists_dev);
+    VA_HIP(hipGetLastError());
+    return 0;
+}

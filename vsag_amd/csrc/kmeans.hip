@@ -1,0 +1,594 @@
+// k-means assignment as an fp32 MFMA contraction with a fused argmin, centroid update and Lloyd driver
+// (KMeansCluster::find_nearest_one_with_blas / Run, src/impl/cluster/kmeans_cluster.cpp:46-305).
+//
+// The reference forms distances = -2 C X^T with SGEMM into a k x 65536 buffer, then makes a second pass
+// adding ||c||^2 and taking std::min_element per row.  Here one kernel does both: a workgroup owns a
+// 128-row tile of X and walks the centroid tiles of its group; v_mfma_f32_32x32x2_f32 accumulates
+// <c_m, x_n> with centroids as the M side and data rows as the N side, so that after the K loop every
+// lane holds 16 centroid values of ONE data row and the argmin needs no cross-lane traffic until the
+// very end.  Candidates are (ordered distance, centroid index) keys, so the smallest index wins ties
+// exactly like std::min_element.
+//
+// Grid: x = centroid group (tile t belongs to group t % groups, groups <= 8), y = row tile.  Workgroups
+// are dealt round-robin to the eight XCDs in x-major order, so one XCD always works on the same
+// quarter-to-eighth of the centroids and keeps them in its own L2, while the X tile is what streams.
+#include <hipcub/hipcub.hpp>
+
+#include <random>
+#include <vector>
+
+#include "common.h"
+
+namespace vsag_amd {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128;  // centroids per tile
+constexpr int BN = 128;  // data rows per tile
+constexpr int BK = 32;   // contraction depth per stage
+constexpr int kPlane = BM;  // float4 slots per (parity, chunk) plane
+
+// LDS operand layout for one stage: [parity h = k & 1][chunk c = (k >> 1) / 4][row] of float4, element e
+// of the float4 is k = 2 (4 c + e) + h.  A lane of the MFMA (row = lane % 32, h = lane / 32) then reads
+// its operand for four consecutive k-steps with one conflict-free ds_read_b128.
+struct Stage {
+    float4 a[2 * 4 * kPlane];
+    float4 b[2 * 4 * kPlane];
+};
+
+__device__ inline float4
+load_row_chunk(const float* base, uint64_t row, uint64_t rows, uint32_t k0, uint32_t dim, bool aligned) {
+    float4 v = make_float4(0.0F, 0.0F, 0.0F, 0.0F);
+    if (row < rows) {
+        const float* p = base + row * dim + k0;
+        if (aligned && k0 + 4 <= dim) {
+            v = *reinterpret_cast<const float4*>(p);
+        } else {
+            if (k0 < dim) {
+                v.x = p[0];
+            }
+            if (k0 + 1 < dim) {
+                v.y = p[1];
+            }
+            if (k0 + 2 < dim) {
+                v.z = p[2];
+            }
+            if (k0 + 3 < dim) {
+                v.w = p[3];
+            }
+        }
+    }
+    return v;
+}
+
+// Scatter one global float4 (k = 4g .. 4g+3 of `row`) into the parity planes.
+__device__ inline void
+stage_store(float4* plane, uint32_t row, uint32_t g, float4 v) {
+    uint32_t c = g >> 1, e = (g & 1) * 2;
+    float* even = reinterpret_cast<float*>(&plane[(0 * 4 + c) * kPlane + row]) + e;
+    float* odd = reinterpret_cast<float*>(&plane[(1 * 4 + c) * kPlane + row]) + e;
+    *reinterpret_cast<float2*>(even) = make_float2(v.x, v.z);
+    *reinterpret_cast<float2*>(odd) = make_float2(v.y, v.w);
+}
+
+__global__ void __launch_bounds__(256, 2)
+kmeans_assign_kernel(const float* __restrict__ X, uint64_t n, const float* __restrict__ C, uint32_t k, uint32_t dim,
+                     const float* __restrict__ ynorm, unsigned long long* __restrict__ best, uint32_t groups) {
+    __shared__ Stage stage[2];  // 64 KiB: two workgroups fit the 160 KiB of a gfx950 CU
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    const uint32_t wave = tid >> 6;
+    const uint32_t wm = wave & 1;   // which 64 centroids of the tile
+    const uint32_t wn = wave >> 1;  // which 64 data rows of the tile
+    const uint32_t half = lane >> 5;
+    const uint32_t l32 = lane & 31;
+    const uint64_t row0 = static_cast<uint64_t>(blockIdx.y) * BN;
+    const bool aligned = (dim & 3) == 0;
+    const uint32_t ktiles = (dim + BK - 1) / BK;
+    const uint32_t ctiles = (k + BM - 1) / BM;
+
+    // Loader roles: 1024 float4 per operand per stage, four per thread.
+    uint32_t ld_row[4], ld_g[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        uint32_t idx = tid + 256 * r;
+        ld_row[r] = idx >> 3;
+        ld_g[r] = idx & 7;
+    }
+
+    unsigned long long my_best[2] = {~0ull, ~0ull};  // per n-block of this wave, for row l32
+
+    for (uint32_t ct = blockIdx.x; ct < ctiles; ct += groups) {
+        const uint64_t c0 = static_cast<uint64_t>(ct) * BM;
+        floatx16 acc[2][2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    acc[i][j][e] = 0.0F;
+                }
+            }
+        }
+        __syncthreads();  // the previous tile's readers of the stages are done
+        float4 ra[4], rb[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            ra[r] = load_row_chunk(C, c0 + ld_row[r], k, 4 * ld_g[r], dim, aligned);
+            rb[r] = load_row_chunk(X, row0 + ld_row[r], n, 4 * ld_g[r], dim, aligned);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            stage_store(stage[0].a, ld_row[r], ld_g[r], ra[r]);
+            stage_store(stage[0].b, ld_row[r], ld_g[r], rb[r]);
+        }
+        __syncthreads();
+        for (uint32_t kt = 0; kt < ktiles; ++kt) {
+            const uint32_t cur = kt & 1;
+            if (kt + 1 < ktiles) {
+                uint32_t k0 = (kt + 1) * BK;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    ra[r] = load_row_chunk(C, c0 + ld_row[r], k, k0 + 4 * ld_g[r], dim, aligned);
+                    rb[r] = load_row_chunk(X, row0 + ld_row[r], n, k0 + 4 * ld_g[r], dim, aligned);
+                }
+            }
+            const float4* pa = stage[cur].a + half * 4 * kPlane + wm * 64 + l32;
+            const float4* pb = stage[cur].b + half * 4 * kPlane + wn * 64 + l32;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                float4 a0 = pa[c * kPlane];
+                float4 a1 = pa[c * kPlane + 32];
+                float4 b0 = pb[c * kPlane];
+                float4 b1 = pb[c * kPlane + 32];
+                const float av0[4] = {a0.x, a0.y, a0.z, a0.w};
+                const float av1[4] = {a1.x, a1.y, a1.z, a1.w};
+                const float bv0[4] = {b0.x, b0.y, b0.z, b0.w};
+                const float bv1[4] = {b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[e], bv0[e], acc[0][0], 0, 0, 0);
+                    acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[e], bv1[e], acc[0][1], 0, 0, 0);
+                    acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[e], bv0[e], acc[1][0], 0, 0, 0);
+                    acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[e], bv1[e], acc[1][1], 0, 0, 0);
+                }
+            }
+            if (kt + 1 < ktiles) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    stage_store(stage[cur ^ 1].a, ld_row[r], ld_g[r], ra[r]);
+                    stage_store(stage[cur ^ 1].b, ld_row[r], ld_g[r], rb[r]);
+                }
+            }
+            __syncthreads();
+        }
+        // Fused argmin: acc[i][j][e] = <c_m, x_n> with m = c0 + wm*64 + i*32 + 8*(e/4) + 4*half + e%4 and
+        // n = row0 + wn*64 + j*32 + l32.  m grows with (i, e), so a strict `<` keeps the first minimum.
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            float bd = __builtin_inff();
+            uint32_t bi = 0xFFFFFFFFU;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    uint32_t ml = wm * 64 + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+                    bool ok = c0 + ml < k;
+                    float dist = (ok ? ynorm[c0 + ml] : 0.0F) + (-2.0F * acc[i][j][e]);
+                    if (ok && dist < bd) {
+                        bd = dist;
+                        bi = static_cast<uint32_t>(c0) + ml;
+                    }
+                }
+            }
+            if (bi != 0xFFFFFFFFU) {
+                unsigned long long key = make_key(bd, bi);
+                if (key < my_best[j]) {
+                    my_best[j] = key;
+                }
+            }
+        }
+    }
+    // Combine the two halves of the wave (they hold different centroids of the same data row), then
+    // publish with one 64-bit atomic per row and wave.
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        unsigned long long other = __shfl_xor(my_best[j], 32);
+        unsigned long long key = other < my_best[j] ? other : my_best[j];
+        uint64_t row = row0 + wn * 64 + j * 32 + l32;
+        if (half == 0 && row < n && key != ~0ull) {
+            atomicMin(&best[row], key);
+        }
+    }
+}
+
+__global__ void
+fill_u64_kernel(unsigned long long* p, unsigned long long v, uint64_t n) {
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) {
+        p[i] = v;
+    }
+}
+
+// ||row||^2 for every row; one wave per row.
+__global__ void __launch_bounds__(256)
+row_sqnorm_kernel(const float* x, uint64_t n, uint32_t dim, float* out) {
+    uint64_t row = static_cast<uint64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    uint32_t lane = threadIdx.x & 63;
+    if (row >= n) {
+        return;
+    }
+    const float* r = x + row * dim;
+    float s = 0.0F;
+    for (uint32_t d = lane; d < dim; d += 64) {
+        s = fmaf(r[d], r[d], s);
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        s += __shfl_down(s, off);
+    }
+    if (lane == 0) {
+        out[row] = s;
+    }
+}
+
+// labels / min distances out of the keys, and the loss: sum over rows of double(float(min + ||x||^2))
+// (kmeans_cluster.cpp:279-304).  Block partial sums go to `partial` and are added in block order by the
+// last kernel, so the result does not depend on scheduling.
+__global__ void __launch_bounds__(256)
+kmeans_finalize_kernel(const unsigned long long* best, const float* xnorm, uint64_t n, int32_t* labels,
+                       float* min_dist, double* partial) {
+    __shared__ double red[4];
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    double v = 0.0;
+    if (i < n) {
+        unsigned long long key = best[i];
+        float md = ordered_to_float(static_cast<uint32_t>(key >> 32));
+        labels[i] = static_cast<int32_t>(static_cast<uint32_t>(key));
+        if (min_dist != nullptr) {
+            min_dist[i] = md;
+        }
+        v = static_cast<double>(md + xnorm[i]);
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        v += __shfl_down(v, off);
+    }
+    if ((threadIdx.x & 63) == 0) {
+        red[threadIdx.x >> 6] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        partial[blockIdx.x] = red[0] + red[1] + red[2] + red[3];
+    }
+}
+
+__global__ void
+loss_reduce_kernel(const double* partial, uint64_t count, uint64_t n, double* loss) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        double s = 0.0;
+        for (uint64_t i = 0; i < count; ++i) {
+            s += partial[i];
+        }
+        *loss = s / static_cast<float>(n);
+    }
+}
+
+// ------------------------------------------------------------------ centroid update
+__global__ void
+iota_u32_kernel(uint32_t* p, uint64_t n) {
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) {
+        p[i] = static_cast<uint32_t>(i);
+    }
+}
+
+__global__ void
+count_labels_kernel(const int32_t* labels, uint64_t n, uint32_t k, uint32_t* counts) {
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) {
+        int32_t l = labels[i];
+        if (l >= 0 && static_cast<uint32_t>(l) < k) {
+            atomicAdd(&counts[l], 1U);
+        }
+    }
+}
+
+// Exclusive prefix sum of k counts by one workgroup (k is a few thousand).
+__global__ void __launch_bounds__(1024)
+exclusive_scan_kernel(const uint32_t* counts, uint32_t k, uint32_t* offsets) {
+    __shared__ uint32_t sums[1024];
+    uint32_t per = (k + blockDim.x - 1) / blockDim.x;
+    uint32_t begin = threadIdx.x * per;
+    uint32_t end = begin + per < k ? begin + per : k;
+    uint32_t s = 0;
+    for (uint32_t i = begin; i < end; ++i) {
+        s += counts[i];
+    }
+    sums[threadIdx.x] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t run = 0;
+        for (uint32_t i = 0; i < blockDim.x; ++i) {
+            uint32_t t = sums[i];
+            sums[i] = run;
+            run += t;
+        }
+        offsets[k] = run;
+    }
+    __syncthreads();
+    uint32_t run = sums[threadIdx.x];
+    for (uint32_t i = begin; i < end; ++i) {
+        offsets[i] = run;
+        run += counts[i];
+    }
+}
+
+// One workgroup per centroid: mean of its member rows (rows sorted by label, in row order), fp32 running
+// sums per dimension.  Empty clusters keep their centroid.
+__global__ void __launch_bounds__(256)
+centroid_mean_kernel(const float* x, uint32_t dim, const uint32_t* sorted_rows, const uint32_t* offsets,
+                     float* centroids, int32_t* counts_out) {
+    uint32_t j = blockIdx.x;
+    uint32_t begin = offsets[j], end = offsets[j + 1];
+    if (threadIdx.x == 0) {
+        counts_out[j] = static_cast<int32_t>(end - begin);
+    }
+    if (end == begin) {
+        return;
+    }
+    float inv = 1.0F / static_cast<float>(end - begin);
+    for (uint32_t d0 = 0; d0 < dim; d0 += blockDim.x * 4) {
+        uint32_t d = d0 + threadIdx.x * 4;
+        float s[4] = {0.0F, 0.0F, 0.0F, 0.0F};
+        if (d + 4 <= dim && (dim & 3) == 0) {
+            for (uint32_t p = begin; p < end; ++p) {
+                float4 v = *reinterpret_cast<const float4*>(x + static_cast<uint64_t>(sorted_rows[p]) * dim + d);
+                s[0] += v.x;
+                s[1] += v.y;
+                s[2] += v.z;
+                s[3] += v.w;
+            }
+        } else {
+            for (uint32_t p = begin; p < end; ++p) {
+                const float* r = x + static_cast<uint64_t>(sorted_rows[p]) * dim;
+                for (int e = 0; e < 4; ++e) {
+                    if (d + e < dim) {
+                        s[e] += r[d + e];
+                    }
+                }
+            }
+        }
+        for (int e = 0; e < 4; ++e) {
+            if (d + e < dim) {
+                centroids[static_cast<uint64_t>(j) * dim + d + e] = s[e] * inv;
+            }
+        }
+    }
+}
+
+void timing_begin(hipStream_t st);
+void timing_end(hipStream_t st);
+
+struct AssignBuffers {
+    float* ynorm;
+    float* xnorm;
+    unsigned long long* best;
+    double* partial;
+    double* loss_tmp;
+};
+
+static size_t
+carve_assign(Carver& c, uint64_t n, uint32_t k, AssignBuffers* b) {
+    b->ynorm = c.take<float>(k);
+    b->xnorm = c.take<float>(n);
+    b->best = c.take<unsigned long long>(n);
+    b->partial = c.take<double>(div_up(n, 256));
+    b->loss_tmp = c.take<double>(1);
+    return c.used;
+}
+
+static int
+assign_launch(const float* x, uint64_t n, uint32_t dim, const float* cent, uint32_t k, int32_t* labels,
+              float* min_dist, double* loss_dev, const AssignBuffers& b, bool have_xnorm, hipStream_t st) {
+    hipLaunchKernelGGL(row_sqnorm_kernel, dim3(static_cast<uint32_t>(div_up(k, 4))), dim3(256), 0, st, cent,
+                       static_cast<uint64_t>(k), dim, b.ynorm);
+    if (!have_xnorm) {
+        hipLaunchKernelGGL(row_sqnorm_kernel, dim3(static_cast<uint32_t>(div_up(n, 4))), dim3(256), 0, st, x, n, dim,
+                           b.xnorm);
+    }
+    hipLaunchKernelGGL(fill_u64_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, b.best, ~0ull,
+                       n);
+    uint32_t ctiles = (k + BM - 1) / BM;
+    uint32_t groups = ctiles < 8 ? ctiles : 8;
+    // grid.y is limited to 65535 row tiles: larger inputs go slab by slab.
+    const uint64_t slab_rows = 65535ull * BN;
+    timing_begin(st);
+    for (uint64_t r0 = 0; r0 < n; r0 += slab_rows) {
+        uint64_t rows = n - r0 < slab_rows ? n - r0 : slab_rows;
+        dim3 grid(groups, static_cast<uint32_t>(div_up(rows, BN)));
+        hipLaunchKernelGGL(kmeans_assign_kernel, grid, dim3(256), 0, st, x + r0 * dim, rows, cent, k, dim, b.ynorm,
+                           b.best + r0, groups);
+    }
+    timing_end(st);
+    hipLaunchKernelGGL(kmeans_finalize_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, b.best,
+                       b.xnorm, n, labels, min_dist, b.partial);
+    hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(64), 0, st, b.partial, div_up(n, 256), n,
+                       loss_dev ? loss_dev : b.loss_tmp);
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
+struct UpdateBuffers {
+    uint32_t* counts;
+    uint32_t* offsets;
+    uint32_t* rows_in;
+    uint32_t* rows_out;
+    int32_t* keys_out;
+    void* sort_tmp;
+    size_t sort_tmp_bytes;
+};
+
+static size_t
+sort_temp_bytes(uint64_t n) {
+    size_t bytes = 0;
+    hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, static_cast<const int32_t*>(nullptr),
+                                       static_cast<int32_t*>(nullptr), static_cast<const uint32_t*>(nullptr),
+                                       static_cast<uint32_t*>(nullptr), static_cast<int>(n), 0, 32, nullptr);
+    return bytes;
+}
+
+static size_t
+carve_update(Carver& c, uint64_t n, uint32_t k, UpdateBuffers* b) {
+    b->counts = c.take<uint32_t>(k + 1);
+    b->offsets = c.take<uint32_t>(k + 1);
+    b->rows_in = c.take<uint32_t>(n);
+    b->rows_out = c.take<uint32_t>(n);
+    b->keys_out = c.take<int32_t>(n);
+    b->sort_tmp_bytes = sort_temp_bytes(n);
+    b->sort_tmp = c.take<uint8_t>(b->sort_tmp_bytes);
+    return c.used;
+}
+
+static int
+update_launch(const float* x, const int32_t* labels, uint64_t n, uint32_t dim, uint32_t k, float* cent,
+              int32_t* counts_dev, const UpdateBuffers& b, hipStream_t st) {
+    uint32_t blocks = static_cast<uint32_t>(div_up(n, 256));
+    hipLaunchKernelGGL(fill_u64_kernel, dim3((k / 2 + 1 + 255) / 256), dim3(256), 0, st,
+                       reinterpret_cast<unsigned long long*>(b.counts), 0ull, static_cast<uint64_t>(k / 2 + 1));
+    hipLaunchKernelGGL(count_labels_kernel, dim3(blocks), dim3(256), 0, st, labels, n, k, b.counts);
+    hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, st, b.counts, k, b.offsets);
+    hipLaunchKernelGGL(iota_u32_kernel, dim3(blocks), dim3(256), 0, st, b.rows_in, n);
+    int end_bit = 1;
+    while ((1ull << end_bit) < k) {
+        ++end_bit;
+    }
+    size_t tmp_bytes = b.sort_tmp_bytes;
+    VA_HIP(hipcub::DeviceRadixSort::SortPairs(b.sort_tmp, tmp_bytes, labels, b.keys_out, b.rows_in, b.rows_out,
+                                              static_cast<int>(n), 0, end_bit, st));
+    hipLaunchKernelGGL(centroid_mean_kernel, dim3(k), dim3(256), 0, st, x, dim, b.rows_out, b.offsets, cent,
+                       counts_dev);
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
+static int
+check_kmeans(const void* x, uint64_t n, uint32_t dim, const void* cent, uint32_t k) {
+    VA_CHECK_ARG(k >= 1, "k must be positive");
+    VA_CHECK_ARG(n >= 1, "count must be positive");
+    VA_CHECK_ARG(x != nullptr && cent != nullptr, "datas cannot be null");
+    VA_CHECK_ARG(dim >= 1 && dim <= 65536, "dim must be in [1, 65536], got %u", dim);
+    VA_CHECK_ARG(n < (1ull << 31), "n must be below 2^31");
+    return 0;
+}
+
+}  // namespace vsag_amd
+
+using namespace vsag_amd;
+
+extern "C" size_t
+vsag_amd_kmeans_assign_workspace_bytes(uint64_t n, uint32_t dim, uint32_t k) {
+    (void)dim;
+    Carver c(nullptr, 0);
+    AssignBuffers b;
+    return carve_assign(c, n, k, &b) + 256;
+}
+
+extern "C" int
+vsag_amd_kmeans_assign(const float* x_dev, uint64_t n, uint32_t dim, const float* centroids_dev, uint32_t k,
+                       int32_t* labels_dev, float* min_dist_dev, double* loss_dev, void* workspace_dev,
+                       size_t workspace_bytes, void* stream) {
+    VA_TRY(ensure_init());
+    VA_TRY(check_kmeans(x_dev, n, dim, centroids_dev, k));
+    VA_CHECK_ARG(labels_dev != nullptr, "labels_dev is null");
+    Carver c(workspace_dev, workspace_bytes);
+    AssignBuffers b;
+    carve_assign(c, n, k, &b);
+    VA_CHECK_ARG(c.ok(), "workspace too small: need %zu bytes, got %zu", c.used, workspace_bytes);
+    return assign_launch(x_dev, n, dim, centroids_dev, k, labels_dev, min_dist_dev, loss_dev, b, false,
+                         static_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t
+vsag_amd_kmeans_update_workspace_bytes(uint64_t n, uint32_t dim, uint32_t k) {
+    (void)dim;
+    if (ensure_init() != 0) {
+        return 0;
+    }
+    Carver c(nullptr, 0);
+    UpdateBuffers b;
+    return carve_update(c, n, k, &b) + 256;
+}
+
+extern "C" int
+vsag_amd_kmeans_update(const float* x_dev, const int32_t* labels_dev, uint64_t n, uint32_t dim, uint32_t k,
+                       float* centroids_dev, int32_t* counts_dev, void* workspace_dev, size_t workspace_bytes,
+                       void* stream) {
+    VA_TRY(ensure_init());
+    VA_TRY(check_kmeans(x_dev, n, dim, centroids_dev, k));
+    VA_CHECK_ARG(labels_dev != nullptr && counts_dev != nullptr, "null labels / counts");
+    Carver c(workspace_dev, workspace_bytes);
+    UpdateBuffers b;
+    carve_update(c, n, k, &b);
+    VA_CHECK_ARG(c.ok(), "workspace too small: need %zu bytes, got %zu", c.used, workspace_bytes);
+    return update_launch(x_dev, labels_dev, n, dim, k, centroids_dev, counts_dev, b, static_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t
+vsag_amd_kmeans_run_workspace_bytes(uint64_t n, uint32_t dim, uint32_t k) {
+    (void)dim;
+    if (ensure_init() != 0) {
+        return 0;
+    }
+    Carver c(nullptr, 0);
+    AssignBuffers a;
+    UpdateBuffers u;
+    carve_assign(c, n, k, &a);
+    carve_update(c, n, k, &u);
+    c.take<int32_t>(k);
+    return c.used + 256;
+}
+
+extern "C" int
+vsag_amd_kmeans_run(const float* x_dev, uint64_t n, uint32_t dim, float* centroids_dev, uint32_t k, int iters,
+                    uint64_t seed, int32_t* labels_dev, double* loss, void* workspace_dev, size_t workspace_bytes,
+                    void* stream) {
+    VA_TRY(ensure_init());
+    VA_TRY(check_kmeans(x_dev, n, dim, centroids_dev, k));
+    VA_CHECK_ARG(k <= n, "k cannot be larger than count");
+    VA_CHECK_ARG(labels_dev != nullptr, "labels_dev is null");
+    VA_CHECK_ARG(iters >= 0, "iters must not be negative");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    Carver c(workspace_dev, workspace_bytes);
+    AssignBuffers a;
+    UpdateBuffers u;
+    carve_assign(c, n, k, &a);
+    carve_update(c, n, k, &u);
+    int32_t* counts_dev = c.take<int32_t>(k);
+    VA_CHECK_ARG(c.ok(), "workspace too small: need %zu bytes, got %zu", c.used, workspace_bytes);
+
+    std::mt19937 gen(static_cast<uint32_t>(seed));
+    std::vector<int32_t> counts(k);
+    double last = 0.0;
+    for (int it = 0; it < iters; ++it) {
+        VA_TRY(assign_launch(x_dev, n, dim, centroids_dev, k, labels_dev, nullptr, a.loss_tmp, a, it > 0, st));
+        VA_TRY(update_launch(x_dev, labels_dev, n, dim, k, centroids_dev, counts_dev, u, st));
+        VA_HIP(hipMemcpyAsync(counts.data(), counts_dev, k * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+        VA_HIP(hipMemcpyAsync(&last, a.loss_tmp, sizeof(double), hipMemcpyDeviceToHost, st));
+        VA_HIP(hipStreamSynchronize(st));
+        // Empty clusters restart from a random data row (kmeans_cluster.cpp:156-171).
+        std::uniform_int_distribution<uint64_t> dis(0, n - 1);
+        for (uint32_t j = 0; j < k; ++j) {
+            if (counts[j] == 0) {
+                uint64_t idx = dis(gen);
+                VA_HIP(hipMemcpyAsync(centroids_dev + static_cast<uint64_t>(j) * dim, x_dev + idx * dim,
+                                      dim * sizeof(float), hipMemcpyDeviceToDevice, st));
+            }
+        }
+    }
+    VA_HIP(hipStreamSynchronize(st));
+    if (loss != nullptr) {
+        *loss = last;
+    }
+    return 0;
+}

@@ -1,0 +1,791 @@
+// Quantizer training and encoding on the device: scalar-quantization bounds, sq8/sq4 codes, uniform
+// codes, RaBitQ 1-bit codes and processed queries.  These are build-time and per-batch steps, not the
+// scan; they are written so that their results equal the reference's scalar arithmetic bit for bit where
+// that arithmetic is order-dependent (running fp32 sums are kept in element order, products and sums are
+// not fused: this translation unit is compiled with -ffp-contract=off).
+#include <cfloat>
+
+#include "common.h"
+#include "topk.h"
+
+namespace vsag_amd {
+
+// ------------------------------------------------------------------ helpers
+// generic::Normalize (src/simd/generic.cpp:874-878, kernels/scalar_op.h:32-60): ||x|| as a running sum in
+// element order; a zero norm divides by one.
+__global__ void
+row_norm_kernel(const float* x, uint64_t n, uint32_t dim, float* norms) {
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) {
+        return;
+    }
+    const float* r = x + i * dim;
+    float s = 0.0F;
+    for (uint32_t d = 0; d < dim; ++d) {
+        s = r[d] * r[d] + s;
+    }
+    float norm = sqrtf(s);
+    norms[i] = norm == 0.0F ? 1.0F : norm;
+}
+
+// ClampScalarQuantizationDelta (scalar_quantization_utils.h:19-30).
+__device__ inline float
+clamp_delta(float delta) {
+    if (!(delta >= 0.0F)) {
+        return 0.0F;
+    }
+    if (delta > 0.999F) {
+        return 1.0F;
+    }
+    return delta;
+}
+
+// ------------------------------------------------------------------ sq8 / sq4 encode
+// ScalarQuantizer::EncodeOneImpl (scalar_quantizer.cpp:85-112).  One thread per code byte.
+__global__ void __launch_bounds__(256)
+sq_encode_kernel(const float* x, uint64_t n, uint32_t dim, int bits, const float* lb, const float* diff,
+                 const float* norms, uint32_t code_size, uint8_t* codes) {
+    uint64_t gid = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    uint64_t i = gid / code_size;
+    uint32_t b = static_cast<uint32_t>(gid % code_size);
+    if (i >= n) {
+        return;
+    }
+    const float* r = x + i * dim;
+    float inv = norms ? norms[i] : 1.0F;
+    float levels = static_cast<float>((1 << bits) - 1);
+    uint32_t per_byte = 8 / bits;
+    uint32_t byte = 0;
+    for (uint32_t e = 0; e < per_byte; ++e) {
+        uint32_t d = b * per_byte + e;
+        if (d >= dim) {
+            break;
+        }
+        float v = norms ? r[d] / inv : r[d];
+        float delta;
+        if (diff[d] < FLT_EPSILON) {
+            delta = 1.0F;
+        } else {
+            delta = 1.0F * (v - lb[d]) / diff[d];
+        }
+        delta = clamp_delta(delta);
+        uint32_t scaled = static_cast<uint8_t>(levels * delta);
+        byte |= scaled << (e * bits);
+    }
+    codes[i * code_size + b] = static_cast<uint8_t>(byte);
+}
+
+// ------------------------------------------------------------------ uniform encode
+// SQ4UniformQuantizer::EncodeOneImpl / SQ8UniformQuantizer::EncodeOneImpl.  One wave per row; the integer
+// norm is order-free, the two fp32 sums are accumulated by lane 0 in element order.
+__global__ void __launch_bounds__(256)
+squ_encode_kernel(const float* x, uint64_t n, uint32_t dim, int bits, int metric, const float* bounds,
+                  const float* norms, uint32_t code_size, uint32_t payload, uint32_t off_norm, uint32_t off_sum,
+                  uint32_t off_codes_sum, uint8_t* codes) {
+    uint64_t row = static_cast<uint64_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    uint32_t lane = threadIdx.x & 63;
+    if (row >= n) {
+        return;
+    }
+    const float* r = x + row * dim;
+    uint8_t* c = codes + row * code_size;
+    float lb = bounds[0], diff = bounds[1];
+    float inv_diff = diff == 0.0F ? 0.0F : 1.0F / diff;
+    float levels = bits == 4 ? 15.0F : 255.0F;
+    float nrm = norms ? norms[row] : 1.0F;
+    uint32_t per_byte = 8 / bits;
+    uint32_t norm_part = 0;
+    for (uint32_t b = lane; b < code_size; b += kWave) {
+        uint32_t byte = 0;
+        if (b < payload) {
+            for (uint32_t e = 0; e < per_byte; ++e) {
+                uint32_t d = b * per_byte + e;
+                if (d >= dim) {
+                    break;
+                }
+                float v = norms ? r[d] / nrm : r[d];
+                float delta = clamp_delta((v - lb) * inv_diff);
+                uint32_t scaled = static_cast<uint8_t>(levels * delta);
+                byte |= scaled << (e * bits);
+                norm_part += scaled * scaled;
+            }
+        }
+        c[b] = static_cast<uint8_t>(byte);
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        norm_part += __shfl_down(norm_part, off);
+    }
+    // All lanes have written their bytes; lane 0 overwrites the trailing fields.
+    wave_lds_fence();
+    if (lane == 0) {
+        if (metric == VSAG_AMD_METRIC_L2) {
+            uint64_t v = norm_part;
+            for (int b = 0; b < 8; ++b) {
+                c[off_norm + b] = static_cast<uint8_t>(v >> (8 * b));
+            }
+        } else {
+            float sum = 0.0F, codes_sum = 0.0F;
+            for (uint32_t d = 0; d < dim; ++d) {
+                float v = norms ? r[d] / nrm : r[d];
+                float delta = clamp_delta((v - lb) * inv_diff);
+                uint32_t scaled = static_cast<uint8_t>(levels * delta);
+                sum += v;
+                codes_sum += static_cast<float>(scaled);
+            }
+            uint32_t u = __float_as_uint(sum);
+            for (int b = 0; b < 4; ++b) {
+                c[off_sum + b] = static_cast<uint8_t>(u >> (8 * b));
+            }
+            if (bits == 4) {
+                u = __float_as_uint(codes_sum);
+                for (int b = 0; b < 4; ++b) {
+                    c[off_codes_sum + b] = static_cast<uint8_t>(u >> (8 * b));
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ C = A * B^T, k in element order
+// C[i][j] = sum_k A[i][k] * B[j][k], one unfused multiply and add per k in increasing k, so every output
+// equals a scalar running-sum dot product (the RowMajor sgemv of random_orthogonal_transformer.cpp:58-77
+// restated in element order).  64 x 64 output tile per workgroup, 4 x 4 outputs per thread.
+__global__ void __launch_bounds__(256)
+gemm_nt_seq_kernel(const float* A, const float* B, float* C, uint64_t M, uint32_t N, uint32_t K) {
+    __shared__ float As[16][65];
+    __shared__ float Bs[16][65];
+    const uint32_t tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const uint64_t row0 = static_cast<uint64_t>(blockIdx.y) * 64;
+    const uint32_t col0 = blockIdx.x * 64;
+    float acc[4][4] = {};
+    for (uint32_t k0 = 0; k0 < K; k0 += 16) {
+        for (uint32_t idx = threadIdx.x; idx < 64 * 16; idx += 256) {
+            uint32_t r = idx >> 4, kk = idx & 15;
+            uint64_t ar = row0 + r;
+            uint32_t br = col0 + r;
+            As[kk][r] = (ar < M && k0 + kk < K) ? A[ar * K + k0 + kk] : 0.0F;
+            Bs[kk][r] = (br < N && k0 + kk < K) ? B[static_cast<uint64_t>(br) * K + k0 + kk] : 0.0F;
+        }
+        __syncthreads();
+        uint32_t kmax = K - k0 < 16 ? K - k0 : 16;
+        for (uint32_t kk = 0; kk < kmax; ++kk) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                a[i] = As[kk][ty * 4 + i];
+                b[i] = Bs[kk][tx * 4 + i];
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    acc[i][j] = a[i] * b[j] + acc[i][j];
+                }
+            }
+        }
+        __syncthreads();
+    }
+    for (int i = 0; i < 4; ++i) {
+        uint64_t r = row0 + ty * 4 + i;
+        if (r >= M) {
+            continue;
+        }
+        for (int j = 0; j < 4; ++j) {
+            uint32_t cidx = col0 + tx * 4 + j;
+            if (cidx < N) {
+                C[r * N + cidx] = acc[i][j];
+            }
+        }
+    }
+}
+
+static int
+gemm_nt_seq(const float* A, const float* B, float* C, uint64_t M, uint32_t N, uint32_t K, hipStream_t st) {
+    dim3 grid((N + 63) / 64, static_cast<uint32_t>(div_up(M, 64)));
+    hipLaunchKernelGGL(gemm_nt_seq_kernel, grid, dim3(256), 0, st, A, B, C, M, N, K);
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
+// ------------------------------------------------------------------ RaBitQ
+struct RabitqLayout {
+    uint32_t dim, code_bytes;
+    uint32_t offset_norm, offset_error, offset_sum, offset_raw_norm, code_size;
+    int has_sum, has_raw_norm;
+    uint32_t aligned_dim, plane_bytes;
+    uint32_t q_offset_lb, q_offset_delta, q_offset_sum, q_offset_norm, q_offset_raw_norm, query_code_size;
+};
+
+// rabitq_quantizer.cpp:102-176 (1-bit base, standard version, no PCA / MRQ / split storage).
+__host__ __device__ inline RabitqLayout
+rabitq_layout(uint32_t dim, int metric, int query_bits) {
+    RabitqLayout l{};
+    l.dim = dim;
+    l.code_bytes = (dim + 7) / 8;
+    uint32_t cs = (l.code_bytes + 3) / 4 * 4;
+    l.offset_norm = cs;
+    cs += 4;
+    l.offset_error = cs;
+    cs += 4;
+    l.has_sum = query_bits != 32;
+    if (l.has_sum) {
+        l.offset_sum = cs;
+        cs += 4;
+    }
+    l.has_raw_norm = metric != VSAG_AMD_METRIC_L2;
+    if (l.has_raw_norm) {
+        l.offset_raw_norm = cs;
+        cs += 4;
+    }
+    l.code_size = cs;
+    uint32_t qs;
+    if (query_bits == 4) {
+        l.aligned_dim = (dim + 511) / 512 * 512;
+        l.plane_bytes = l.aligned_dim / 8;
+        qs = l.plane_bytes * 4;
+        l.q_offset_lb = qs;
+        qs += 4;
+        l.q_offset_delta = qs;
+        qs += 4;
+        l.q_offset_sum = qs;
+        qs += 4;
+    } else {
+        qs = 4 * dim;
+    }
+    l.q_offset_norm = qs;
+    qs += 4;
+    if (l.has_raw_norm) {
+        l.q_offset_raw_norm = qs;
+        qs += 4;
+    }
+    l.query_code_size = qs;
+    return l;
+}
+
+uint64_t
+rabitq_code_size(uint32_t dim, int metric, int query_bits) {
+    return rabitq_layout(dim, metric, query_bits).code_size;
+}
+uint64_t
+rabitq_query_code_size(uint32_t dim, int metric, int query_bits) {
+    return rabitq_layout(dim, metric, query_bits).query_code_size;
+}
+
+__device__ inline void
+store_f32(uint8_t* p, float v) {
+    uint32_t u = __float_as_uint(v);
+    for (int b = 0; b < 4; ++b) {
+        p[b] = static_cast<uint8_t>(u >> (8 * b));
+    }
+}
+
+// Column means as running fp32 sums over the rows in order (rabitq_quantizer.cpp:224-241).
+__global__ void
+column_mean_seq_kernel(const float* x, uint64_t n, uint32_t dim, float* mean) {
+    uint32_t d = blockIdx.x * blockDim.x + threadIdx.x;
+    if (d >= dim) {
+        return;
+    }
+    float s = 0.0F;
+    for (uint64_t i = 0; i < n; ++i) {
+        s += x[i * dim + d];
+    }
+    mean[d] = s / static_cast<float>(n);
+}
+
+// Second half of RaBitQuantizer::EncodeOneInternal (rabitq_quantizer.cpp:749-856) for rows already rotated:
+// raw norm of the input row, NormalizeWithCentroid (kernels/normalize.h:35-83), sign bits, error =
+// RaBitQFloatBinaryIP(normed, bits) (generic.cpp:447-471), bit count.  One thread per row, element order.
+__global__ void __launch_bounds__(64)
+rabitq_finish_encode_kernel(const float* raw, const float* rotated, uint64_t n, uint32_t dim, const float* centroid,
+                            int metric, int query_bits, uint8_t* codes) {
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) {
+        return;
+    }
+    RabitqLayout l = rabitq_layout(dim, metric, query_bits);
+    const float* y = rotated + i * dim;
+    uint8_t* c = codes + i * l.code_size;
+    float raw_norm = 0.0F;
+    if (l.has_raw_norm) {
+        const float* x = raw + i * dim;
+        for (uint32_t d = 0; d < dim; ++d) {
+            raw_norm += x[d] * x[d];
+        }
+    }
+    raw_norm = sqrtf(raw_norm);
+    float norm_sq = 0.0F;
+    for (uint32_t d = 0; d < dim; ++d) {
+        float t = y[d] - centroid[d];
+        norm_sq = t * t + norm_sq;
+    }
+    float norm = norm_sq < 1e-5F ? 1.0F : sqrtf(norm_sq);
+    float inv_sqrt_d = 1.0F / sqrtf(static_cast<float>(dim));
+    float pos, neg;
+    if (inv_sqrt_d > 1e-3F) {
+        pos = inv_sqrt_d;
+        neg = -inv_sqrt_d;
+    } else {
+        pos = 1.0F;
+        neg = 0.0F;
+    }
+    float error = 0.0F;
+    uint32_t binary_sum = 0;
+    for (uint32_t b = 0; b < l.offset_norm; ++b) {
+        uint32_t byte = 0;
+        for (uint32_t e = 0; e < 8; ++e) {
+            uint32_t d = b * 8 + e;
+            if (d >= dim) {
+                break;
+            }
+            float nd = (y[d] - centroid[d]) / norm;
+            bool bit = nd >= 0.0F;
+            if (bit) {
+                byte |= 1U << e;
+                ++binary_sum;
+            }
+            error += (bit ? pos : neg) * nd;
+        }
+        c[b] = static_cast<uint8_t>(byte);
+    }
+    store_f32(c + l.offset_norm, norm);
+    store_f32(c + l.offset_error, error);
+    if (l.has_sum) {
+        store_f32(c + l.offset_sum, static_cast<float>(binary_sum));
+    }
+    if (l.has_raw_norm) {
+        store_f32(c + l.offset_raw_norm, raw_norm);
+    }
+}
+
+// Second half of RaBitQuantizer::ProcessQueryImpl (rabitq_quantizer.cpp:2130-2217) with EncodeSQ and
+// ReOrderSQ (:2049-2088) for queries already rotated.  One thread per query.
+__global__ void __launch_bounds__(64)
+rabitq_finish_query_kernel(const float* raw, const float* rotated, uint64_t nq, uint32_t dim, const float* centroid,
+                           int metric, int query_bits, uint8_t* qcodes) {
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= nq) {
+        return;
+    }
+    RabitqLayout l = rabitq_layout(dim, metric, query_bits);
+    const float* y = rotated + i * dim;
+    uint8_t* qc = qcodes + i * l.query_code_size;
+    float raw_norm = 0.0F;
+    if (l.has_raw_norm) {
+        const float* x = raw + i * dim;
+        for (uint32_t d = 0; d < dim; ++d) {
+            raw_norm += x[d] * x[d];
+        }
+    }
+    raw_norm = sqrtf(raw_norm);
+    float norm_sq = 0.0F;
+    for (uint32_t d = 0; d < dim; ++d) {
+        float t = y[d] - centroid[d];
+        norm_sq = t * t + norm_sq;
+    }
+    float norm = norm_sq < 1e-5F ? 1.0F : sqrtf(norm_sq);
+    if (query_bits == 4) {
+        float lb = FLT_MAX, ub = -FLT_MAX;
+        for (uint32_t d = 0; d < dim; ++d) {
+            float v = (y[d] - centroid[d]) / norm;
+            if (v < lb) {
+                lb = v;
+            }
+            if (v > ub) {
+                ub = v;
+            }
+        }
+        float delta = (ub - lb) / 15;
+        float inv_delta = fabsf(delta) < 1e-5F ? 0.0F : 1.0F / delta;
+        float qsum = 0.0F;
+        for (uint32_t b = 0; b < l.plane_bytes; ++b) {
+            uint32_t plane[4] = {0, 0, 0, 0};
+            for (uint32_t e = 0; e < 8; ++e) {
+                uint32_t d = b * 8 + e;
+                if (d >= dim) {
+                    break;
+                }
+                float v = (y[d] - centroid[d]) / norm;
+                float val = roundf((v - lb) * inv_delta);
+                uint32_t q = static_cast<uint8_t>(val);
+                qsum += static_cast<float>(val);
+                for (uint32_t p = 0; p < 4; ++p) {
+                    plane[p] |= ((q >> p) & 1U) << e;
+                }
+            }
+            for (uint32_t p = 0; p < 4; ++p) {
+                qc[p * l.plane_bytes + b] = static_cast<uint8_t>(plane[p]);
+            }
+        }
+        store_f32(qc + l.q_offset_lb, lb);
+        store_f32(qc + l.q_offset_delta, delta);
+        store_f32(qc + l.q_offset_sum, qsum);
+    } else {
+        for (uint32_t d = 0; d < dim; ++d) {
+            store_f32(qc + 4 * d, (y[d] - centroid[d]) / norm);
+        }
+    }
+    store_f32(qc + l.q_offset_norm, norm);
+    if (l.has_raw_norm) {
+        store_f32(qc + l.q_offset_raw_norm, raw_norm);
+    }
+}
+
+int
+squ_encode_launch(const float* x, uint64_t n, uint32_t dim, int bits, int metric, const float* bounds, uint8_t* codes,
+                  hipStream_t st) {
+    if (n == 0) {
+        return 0;
+    }
+    int kind = bits == 4 ? VSAG_AMD_KIND_SQ4_UNIFORM : VSAG_AMD_KIND_SQ8_UNIFORM;
+    uint32_t code_size = static_cast<uint32_t>(vsag_amd_code_size(kind, metric, dim, 0));
+    uint32_t payload = bits == 4 ? (dim + 1) / 2 : dim;
+    bool norm = metric == VSAG_AMD_METRIC_L2 || (bits == 4 && metric == VSAG_AMD_METRIC_COSINE);
+    uint32_t align = norm ? 8 : 4;
+    uint32_t off = static_cast<uint32_t>(round_up(payload, align));
+    uint32_t off_norm = off;
+    uint32_t off_sum = off + (norm ? 8 : 0);
+    uint32_t off_codes_sum = off_sum + align;
+    float* norms = nullptr;
+    if (metric == VSAG_AMD_METRIC_COSINE) {
+        VA_HIP(hipMallocAsync(reinterpret_cast<void**>(&norms), n * 4, st));
+        hipLaunchKernelGGL(row_norm_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, x, n, dim,
+                           norms);
+    }
+    hipLaunchKernelGGL(squ_encode_kernel, dim3(static_cast<uint32_t>(div_up(n, 4))), dim3(256), 0, st, x, n, dim, bits,
+                       metric, bounds, norms, code_size, payload, off_norm, off_sum, off_codes_sum, codes);
+    VA_HIP(hipGetLastError());
+    if (norms != nullptr) {
+        VA_HIP(hipFreeAsync(norms, st));
+    }
+    return 0;
+}
+
+// Rotates rows in slabs so that the temporary stays bounded, then runs `finish` on each slab.
+template <typename Finish>
+static int
+rabitq_rotate_slabs(const float* x, uint64_t n, uint32_t dim, const float* rot, hipStream_t st, Finish finish) {
+    const uint64_t slab = 1ull << 18;
+    uint64_t rows = n < slab ? n : slab;
+    float* tmp = nullptr;
+    VA_HIP(hipMallocAsync(reinterpret_cast<void**>(&tmp), rows * dim * 4, st));
+    int rc = 0;
+    for (uint64_t s = 0; s < n && rc == 0; s += slab) {
+        uint64_t m = n - s < slab ? n - s : slab;
+        rc = gemm_nt_seq(x + s * dim, rot, tmp, m, dim, dim, st);
+        if (rc == 0) {
+            rc = finish(s, m, tmp);
+        }
+    }
+    hipError_t e = hipFreeAsync(tmp, st);
+    if (rc == 0 && e != hipSuccess) {
+        return fail(VSAG_AMD_INTERNAL_ERROR, "hipFreeAsync failed: %s", hipGetErrorString(e));
+    }
+    return rc;
+}
+
+int
+rabitq_process_query_launch(const float* q, uint64_t nq, uint32_t dim, const float* rot, const float* centroid,
+                            int metric, int query_bits, uint8_t* qcodes, hipStream_t st) {
+    if (nq == 0) {
+        return 0;
+    }
+    uint64_t qsize = rabitq_query_code_size(dim, metric, query_bits);
+    return rabitq_rotate_slabs(q, nq, dim, rot, st, [&](uint64_t s, uint64_t m, const float* rotated) {
+        hipLaunchKernelGGL(rabitq_finish_query_kernel, dim3(static_cast<uint32_t>(div_up(m, 64))), dim3(64), 0, st,
+                           q + s * dim, rotated, m, dim, centroid, metric, query_bits, qcodes + s * qsize);
+        VA_HIP(hipGetLastError());
+        return 0;
+    });
+}
+
+// ------------------------------------------------------------------ scalar-quantization trainer
+// Sample gather (scalar_quantization_trainer.cpp:125-146): row j of the sample is row (j * step) % n,
+// written transposed (sample_t[d][j]) so that the per-dimension selection reads contiguously.
+__global__ void __launch_bounds__(256)
+sq_sample_kernel(const float* x, uint64_t n, uint32_t dim, uint64_t step, uint64_t sample_count, const float* norms,
+                 float* sample_t) {
+    uint64_t gid = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    uint64_t j = gid / dim;
+    uint32_t d = static_cast<uint32_t>(gid % dim);
+    if (j >= sample_count) {
+        return;
+    }
+    uint64_t idx = (j * step) % n;
+    float v = x[idx * dim + d];
+    if (norms != nullptr) {
+        v = v / norms[idx];
+    }
+    sample_t[static_cast<uint64_t>(d) * sample_count + j] = v;
+}
+
+// k-th smallest (1-based) of vals[0,count) by an 8-bit radix descent over order-preserving keys.
+// One workgroup per call site; hist is a 256-entry LDS array.
+__device__ inline float
+block_kth_smallest(const float* vals, uint64_t count, uint64_t kth, uint32_t* hist, uint32_t* shared) {
+    uint32_t prefix = 0, mask = 0;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) {
+            hist[i] = 0;
+        }
+        __syncthreads();
+        for (uint64_t i = threadIdx.x; i < count; i += blockDim.x) {
+            uint32_t key = float_to_ordered(vals[i]);
+            if ((key & mask) == prefix) {
+                atomicAdd(&hist[(key >> shift) & 0xff], 1U);
+            }
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            uint64_t acc = 0;
+            uint32_t bin = 0;
+            for (; bin < 256; ++bin) {
+                if (acc + hist[bin] >= kth) {
+                    break;
+                }
+                acc += hist[bin];
+            }
+            shared[0] = bin;
+            shared[1] = static_cast<uint32_t>(acc);
+        }
+        __syncthreads();
+        prefix |= shared[0] << shift;
+        mask |= 0xffU << shift;
+        kth -= shared[1];
+        __syncthreads();
+    }
+    return ordered_to_float(prefix);
+}
+
+// trunc_bound_train / classic_train (scalar_quantization_trainer.cpp:72-122): the bounded heaps keep the
+// ignore_count largest and smallest sample values of a dimension; their tops are the ignore_count-th
+// largest and smallest.  CLASSIC is the same with ignore_count = 1.  Writes lower bound and diff.
+__global__ void __launch_bounds__(256)
+sq_bounds_kernel(const float* sample_t, uint64_t count, uint32_t dim, uint64_t ignore_count, float* lb, float* diff,
+                 float* upper_out, float* lower_out) {
+    __shared__ uint32_t hist[256];
+    __shared__ uint32_t shared[2];
+    uint32_t d = blockIdx.x;
+    const float* col = sample_t + static_cast<uint64_t>(d) * count;
+    uint64_t k = ignore_count < count ? ignore_count : count;
+    float lower = block_kth_smallest(col, count, k, hist, shared);
+    float upper = block_kth_smallest(col, count, count - k + 1, hist, shared);
+    if (threadIdx.x == 0) {
+        if (lb != nullptr) {
+            lb[d] = lower;
+            diff[d] = upper - lower;
+        }
+        if (upper_out != nullptr) {
+            upper_out[d] = upper;
+            lower_out[d] = lower;
+        }
+    }
+}
+
+// TrainUniform (scalar_quantization_trainer.cpp:47-70): CLASSIC -> max of uppers / min of lowers;
+// TRUNC_BOUND -> min of uppers / max of lowers, swapped when inverted.  out = {lb, diff}.
+__global__ void
+sq_uniform_reduce_kernel(const float* upper, const float* lower, uint32_t dim, int mode, float* out) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) {
+        return;
+    }
+    float ub = upper[0], lb = lower[0];
+    for (uint32_t d = 1; d < dim; ++d) {
+        if (mode == VSAG_AMD_SQ_TRAIN_CLASSIC) {
+            ub = fmaxf(ub, upper[d]);
+            lb = fminf(lb, lower[d]);
+        } else {
+            ub = fminf(ub, upper[d]);
+            lb = fmaxf(lb, lower[d]);
+        }
+    }
+    if (mode != VSAG_AMD_SQ_TRAIN_CLASSIC && lb > ub) {
+        float t = lb;
+        lb = ub;
+        ub = t;
+    }
+    out[0] = lb;
+    out[1] = ub - lb;
+}
+
+struct TrainPlan {
+    uint64_t sample_count, step, ignore_count;
+};
+
+static TrainPlan
+train_plan(uint64_t n, int bits, int mode, float trunc_rate, uint64_t max_sample) {
+    TrainPlan p{};
+    if (max_sample == 0) {
+        max_sample = 100000;
+    }
+    p.step = 2147483647ULL % n;
+    p.sample_count = max_sample;
+    if (n <= max_sample) {
+        p.step = 1;
+        p.sample_count = n;
+    }
+    if (mode == VSAG_AMD_SQ_TRAIN_CLASSIC) {
+        p.ignore_count = 1;
+    } else {
+        double rate = bits == 4 ? static_cast<double>(trunc_rate) : 0.001;
+        auto ic = static_cast<uint64_t>(static_cast<double>(p.sample_count - 1) * rate);
+        p.ignore_count = ic < 1 ? 1 : ic;
+    }
+    return p;
+}
+
+static int
+sq_train_common(const float* x, uint64_t n, uint32_t dim, int bits, int metric, int mode, float trunc_rate,
+                uint64_t max_sample, float* lb, float* diff, float* uniform_out, void* ws, size_t ws_bytes,
+                hipStream_t st) {
+    VA_TRY(ensure_init());
+    VA_CHECK_ARG(x != nullptr && n >= 1, "sq_train needs at least one row");
+    VA_CHECK_ARG(dim >= 1 && dim <= 65536, "dim must be in [1, 65536], got %u", dim);
+    VA_CHECK_ARG(bits == 4 || bits == 8, "bits must be 4 or 8, got %d", bits);
+    VA_CHECK_ARG(mode == VSAG_AMD_SQ_TRAIN_CLASSIC || mode == VSAG_AMD_SQ_TRAIN_TRUNC_BOUND, "unknown train mode %d",
+                 mode);
+    TrainPlan p = train_plan(n, bits, mode, trunc_rate, max_sample);
+    Carver c(ws, ws_bytes);
+    float* sample_t = c.take<float>(p.sample_count * dim);
+    float* norms = c.take<float>(metric == VSAG_AMD_METRIC_COSINE ? n : 0);
+    float* upper = c.take<float>(dim);
+    float* lower = c.take<float>(dim);
+    VA_CHECK_ARG(c.ok(), "workspace too small: need %zu bytes, got %zu", c.used, ws_bytes);
+    if (metric == VSAG_AMD_METRIC_COSINE) {
+        hipLaunchKernelGGL(row_norm_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, x, n, dim,
+                           norms);
+    } else {
+        norms = nullptr;
+    }
+    hipLaunchKernelGGL(sq_sample_kernel, dim3(static_cast<uint32_t>(div_up(p.sample_count * dim, 256))), dim3(256), 0,
+                       st, x, n, dim, p.step, p.sample_count, norms, sample_t);
+    hipLaunchKernelGGL(sq_bounds_kernel, dim3(dim), dim3(256), 0, st, sample_t, p.sample_count, dim, p.ignore_count,
+                       lb, diff, upper, lower);
+    if (uniform_out != nullptr) {
+        hipLaunchKernelGGL(sq_uniform_reduce_kernel, dim3(1), dim3(64), 0, st, upper, lower, dim, mode, uniform_out);
+    }
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
+}  // namespace vsag_amd
+
+using namespace vsag_amd;
+
+extern "C" size_t
+vsag_amd_sq_train_workspace_bytes(uint64_t n, uint32_t dim, uint64_t max_sample) {
+    if (n == 0) {
+        return 0;
+    }
+    TrainPlan p = train_plan(n, 8, VSAG_AMD_SQ_TRAIN_TRUNC_BOUND, 0.05F, max_sample);
+    return round_up(p.sample_count * dim * 4, 256) + round_up(n * 4, 256) + 2 * round_up(dim * 4ull, 256) + 256;
+}
+
+extern "C" int
+vsag_amd_sq_train(const float* x_dev, uint64_t n, uint32_t dim, int bits, int metric, int mode, float trunc_rate,
+                  uint64_t max_sample, float* lower_bound_dev, float* diff_dev, void* workspace_dev,
+                  size_t workspace_bytes, void* stream) {
+    VA_CHECK_ARG(lower_bound_dev && diff_dev, "null output");
+    return sq_train_common(x_dev, n, dim, bits, metric, mode, trunc_rate, max_sample, lower_bound_dev, diff_dev,
+                           nullptr, workspace_dev, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int
+vsag_amd_sq_train_uniform(const float* x_dev, uint64_t n, uint32_t dim, int bits, int metric, int mode,
+                          float trunc_rate, uint64_t max_sample, float* out_dev, void* workspace_dev,
+                          size_t workspace_bytes, void* stream) {
+    VA_CHECK_ARG(out_dev, "null output");
+    return sq_train_common(x_dev, n, dim, bits, metric, mode, trunc_rate, max_sample, nullptr, nullptr, out_dev,
+                           workspace_dev, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int
+vsag_amd_sq_encode(const float* x_dev, uint64_t n, uint32_t dim, int bits, int metric, const float* lower_bound_dev,
+                   const float* diff_dev, uint8_t* codes_dev, void* stream) {
+    VA_TRY(ensure_init());
+    VA_CHECK_ARG(bits == 4 || bits == 8, "bits must be 4 or 8, got %d", bits);
+    VA_CHECK_ARG(dim >= 1 && dim <= 65536, "dim must be in [1, 65536], got %u", dim);
+    if (n == 0) {
+        return 0;
+    }
+    VA_CHECK_ARG(x_dev && lower_bound_dev && diff_dev && codes_dev, "null pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    uint32_t code_size = (dim * bits + 7) / 8;
+    float* norms = nullptr;
+    if (metric == VSAG_AMD_METRIC_COSINE) {
+        VA_HIP(hipMallocAsync(reinterpret_cast<void**>(&norms), n * 4, st));
+        hipLaunchKernelGGL(row_norm_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, x_dev, n,
+                           dim, norms);
+    }
+    uint64_t threads = n * code_size;
+    VA_CHECK_ARG(div_up(threads, 256) < (1ull << 31), "too many rows for one encode call");
+    hipLaunchKernelGGL(sq_encode_kernel, dim3(static_cast<uint32_t>(div_up(threads, 256))), dim3(256), 0, st, x_dev, n,
+                       dim, bits, lower_bound_dev, diff_dev, norms, code_size, codes_dev);
+    VA_HIP(hipGetLastError());
+    if (norms != nullptr) {
+        VA_HIP(hipFreeAsync(norms, st));
+    }
+    return 0;
+}
+
+extern "C" int
+vsag_amd_squ_encode(const float* x_dev, uint64_t n, uint32_t dim, int bits, int metric, const float* bounds_dev,
+                    uint8_t* codes_dev, void* stream) {
+    VA_TRY(ensure_init());
+    VA_CHECK_ARG(bits == 4 || bits == 8, "bits must be 4 or 8, got %d", bits);
+    VA_CHECK_ARG(dim >= 1 && dim <= 65536, "dim must be in [1, 65536], got %u", dim);
+    VA_CHECK_ARG(n == 0 || (x_dev && bounds_dev && codes_dev), "null pointer");
+    return squ_encode_launch(x_dev, n, dim, bits, metric, bounds_dev, codes_dev, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int
+vsag_amd_rabitq_train(const float* x_dev, uint64_t n, uint32_t dim, const float* rotation_dev, float* centroid_dev,
+                      void* stream) {
+    VA_TRY(ensure_init());
+    VA_CHECK_ARG(x_dev && rotation_dev && centroid_dev && n >= 1, "null pointer or empty data");
+    VA_CHECK_ARG(dim >= 1 && dim <= 65536, "dim must be in [1, 65536], got %u", dim);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    float* mean = nullptr;
+    VA_HIP(hipMallocAsync(reinterpret_cast<void**>(&mean), dim * 4, st));
+    hipLaunchKernelGGL(column_mean_seq_kernel, dim3((dim + 63) / 64), dim3(64), 0, st, x_dev, n, dim, mean);
+    int rc = gemm_nt_seq(mean, rotation_dev, centroid_dev, 1, dim, dim, st);
+    VA_HIP(hipFreeAsync(mean, st));
+    return rc;
+}
+
+extern "C" int
+vsag_amd_rabitq_encode(const float* x_dev, uint64_t n, uint32_t dim, const float* rotation_dev,
+                       const float* centroid_dev, int metric, int query_bits, uint8_t* codes_dev, void* stream) {
+    VA_TRY(ensure_init());
+    VA_CHECK_ARG(query_bits == 4 || query_bits == 32, "query_bits must be 4 or 32, got %d", query_bits);
+    VA_CHECK_ARG(dim >= 1 && dim <= 65536, "dim must be in [1, 65536], got %u", dim);
+    if (n == 0) {
+        return 0;
+    }
+    VA_CHECK_ARG(x_dev && rotation_dev && centroid_dev && codes_dev, "null pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    uint64_t csize = rabitq_code_size(dim, metric, query_bits);
+    return rabitq_rotate_slabs(x_dev, n, dim, rotation_dev, st, [&](uint64_t s, uint64_t m, const float* rotated) {
+        hipLaunchKernelGGL(rabitq_finish_encode_kernel, dim3(static_cast<uint32_t>(div_up(m, 64))), dim3(64), 0, st,
+                           x_dev + s * dim, rotated, m, dim, centroid_dev, metric, query_bits, codes_dev + s * csize);
+        VA_HIP(hipGetLastError());
+        return 0;
+    });
+}
+
+extern "C" uint64_t
+vsag_amd_rabitq_query_code_size(uint32_t dim, int metric, int query_bits) {
+    return rabitq_query_code_size(dim, metric, query_bits);
+}
+
+extern "C" int
+vsag_amd_rabitq_process_query(const float* q_dev, uint64_t nq, uint32_t dim, const float* rotation_dev,
+                              const float* centroid_dev, int metric, int query_bits, uint8_t* qcodes_dev,
+                              void* stream) {
+    VA_TRY(ensure_init());
+    VA_CHECK_ARG(query_bits == 4 || query_bits == 32, "query_bits must be 4 or 32, got %d", query_bits);
+    VA_CHECK_ARG(dim >= 1 && dim <= 65536, "dim must be in [1, 65536], got %u", dim);
+    VA_CHECK_ARG(nq == 0 || (q_dev && rotation_dev && centroid_dev && qcodes_dev), "null pointer");
+    return rabitq_process_query_launch(q_dev, nq, dim, rotation_dev, centroid_dev, metric, query_bits, qcodes_dev,
+                                       static_cast<hipStream_t>(stream));
+}

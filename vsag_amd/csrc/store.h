@@ -1,0 +1,64 @@
+// Device-resident code store: quantizer state + codes re-tiled for wave64 streaming.
+//
+// HBM layout.  Codes are grouped into tiles of 64.  A tile is G rows of 1 KiB; row j holds bytes
+// [16j, 16j+16) of each of the 64 codes, lane-major, so one global_load_dwordx4 per lane reads a whole
+// row fully coalesced and every lane ends up with the bytes of "its" code.  Only the leading
+// payload_bytes of a reference code (the part the distance loop consumes) go into the tiles; trailing
+// per-code scalars (norms, sums, RaBitQ factors) are kept as structure-of-arrays words in `meta`.
+// A flat store maps tile t, lane l to inner id 64 t + l.  A posting-list store pads every list to whole
+// tiles and keeps an explicit inner-id array in the same tile order.
+#pragma once
+
+#include <vector>
+
+#include "common.h"
+
+struct vsag_amd_store {
+    int kind = 0;
+    int metric = 0;
+    uint32_t dim = 0;
+    int query_bits = 4;
+
+    uint32_t code_size = 0;      // bytes per code in the reference layout
+    uint32_t payload_bytes = 0;  // leading bytes consumed by the distance loop
+    uint32_t G = 0;              // 16-byte granules per code
+    uint32_t dpad = 0;           // dims covered by G granules (per-dim tables are this long)
+    uint32_t nmeta = 0;          // 4-byte metadata words per code
+    uint32_t meta_offset[4] = {0, 0, 0, 0};  // byte offsets of those words in the reference code
+    uint32_t meta_is_u64 = 0;    // bit m set: word m is a u64 in the reference code, kept as float
+
+    // quantizer state
+    float* scale_dev = nullptr;  // sq8/sq4: diff[d]/levels, zero beyond dim
+    float* lb_dev = nullptr;     // sq8/sq4: lower bound, zero beyond dim
+    float* diff_dev = nullptr;   // sq8/sq4: diff (kept for encoders)
+    float ulb = 0, udiff = 0, scalar_rate = 0;  // uniform kinds
+    float* bounds_dev = nullptr;                // uniform kinds: {lb, diff}
+    float* rotation_dev = nullptr;              // rabitq
+    float* centroid_dev = nullptr;              // rabitq
+
+    // codes
+    uint4* tiles = nullptr;
+    uint32_t* meta = nullptr;    // nmeta arrays of cap_tiles*64 words
+    uint64_t cap_tiles = 0;
+    uint64_t ntiles = 0;
+    uint64_t n = 0;
+
+    // posting lists (nlist == 0: flat store)
+    uint32_t nlist = 0;
+    uint32_t* ids_dev = nullptr;         // inner id per tile slot, VSAG_AMD_INVALID_ID in padding
+    uint32_t* list_tile_dev = nullptr;   // nlist+1 tile offsets
+    std::vector<uint32_t> list_sizes;    // host copy
+    std::vector<uint32_t> list_tile;     // host copy, nlist+1
+};
+
+namespace vsag_amd {
+
+// Query-side table geometry of one store kind (what the prepare kernel writes per query).
+struct QueryLayout {
+    uint32_t qstride;  // 4-byte words per query in the main table
+    uint32_t qmeta;    // floats per query in the scalar table
+};
+
+QueryLayout query_layout(const vsag_amd_store* s);
+
+}  // namespace vsag_amd

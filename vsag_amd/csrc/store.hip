@@ -1,0 +1,529 @@
+// Code stores: creation, growth, and re-tiling of reference-layout codes into the wave64 tile layout
+// (the device-side counterpart of FlattenDataCell::BatchInsertVector, src/datacell/flatten_datacell.h:279-314,
+// and of BucketDataCell::InsertVector, src/datacell/bucket_datacell.h:670-709).
+#include <hipcub/hipcub.hpp>
+
+#include <cmath>
+#include <new>
+
+#include "store.h"
+
+namespace vsag_amd {
+
+uint64_t rabitq_code_size(uint32_t dim, int metric, int query_bits);
+
+// dst_slot[i] = tile slot (tile * 64 + lane) of source code i; src_index[i] = row of the source code.
+// One thread per (code, granule): gathers up to 16 payload bytes and writes one uint4; the thread of
+// granule 0 also moves the per-code metadata words.
+struct RetileArgs {
+    const uint8_t* codes;
+    uint64_t n;
+    uint32_t code_size;
+    uint32_t payload_bytes;
+    uint32_t G;
+    uint32_t nmeta;
+    uint32_t meta_offset[4];
+    uint32_t meta_is_u64;
+    uint4* tiles;
+    uint32_t* meta;
+    uint64_t meta_stride;
+    uint64_t first_slot;          // flat append: slot of source code 0
+    const uint32_t* src_index;    // list form: sorted position -> source row (may be null)
+    const uint32_t* dst_slot;     // list form: sorted position -> tile slot (may be null)
+    uint32_t* ids;                // list form: inner id per slot
+    int normalize;                // fp32 + cosine: store x / ||x||
+    uint32_t dim;
+};
+
+__global__ void __launch_bounds__(256)
+retile_kernel(RetileArgs a) {
+    uint64_t gid = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    uint64_t i = gid / a.G;
+    uint32_t j = static_cast<uint32_t>(gid % a.G);
+    if (i >= a.n) {
+        return;
+    }
+    uint64_t row = a.src_index ? a.src_index[i] : i;
+    uint64_t slot = a.dst_slot ? a.dst_slot[i] : a.first_slot + i;
+    const uint8_t* src = a.codes + row * a.code_size;
+    uint32_t w[4] = {0, 0, 0, 0};
+    if (a.normalize) {
+        const float* x = reinterpret_cast<const float*>(src);
+        float s = 0.0F;
+        for (uint32_t d = 0; d < a.dim; ++d) {
+            s = fmaf(x[d], x[d], s);
+        }
+        float norm = sqrtf(s);
+        for (uint32_t e = 0; e < 4; ++e) {
+            uint32_t d = 4 * j + e;
+            if (d < a.dim) {
+                w[e] = __float_as_uint(x[d] / norm);
+            }
+        }
+    } else {
+        for (uint32_t b = 0; b < 16; ++b) {
+            uint32_t off = 16 * j + b;
+            if (off < a.payload_bytes) {
+                w[b >> 2] |= static_cast<uint32_t>(src[off]) << (8 * (b & 3));
+            }
+        }
+    }
+    uint64_t tile = slot / kWave;
+    uint32_t lane = static_cast<uint32_t>(slot % kWave);
+    a.tiles[(tile * a.G + j) * kWave + lane] = make_uint4(w[0], w[1], w[2], w[3]);
+    if (j == 0) {
+        for (uint32_t m = 0; m < a.nmeta; ++m) {
+            const uint8_t* p = src + a.meta_offset[m];
+            uint32_t word;
+            if ((a.meta_is_u64 >> m) & 1) {
+                uint64_t v = 0;
+                for (int b = 0; b < 8; ++b) {
+                    v |= static_cast<uint64_t>(p[b]) << (8 * b);
+                }
+                word = __float_as_uint(static_cast<float>(v));
+            } else {
+                word = 0;
+                for (int b = 0; b < 4; ++b) {
+                    word |= static_cast<uint32_t>(p[b]) << (8 * b);
+                }
+            }
+            a.meta[m * a.meta_stride + slot] = word;
+        }
+        if (a.ids != nullptr) {
+            a.ids[slot] = static_cast<uint32_t>(row);
+        }
+    }
+}
+
+__global__ void
+fill_u32_kernel(uint32_t* p, uint32_t v, uint64_t n) {
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) {
+        p[i] = v;
+    }
+}
+
+__global__ void
+scale_table_kernel(const float* lb, const float* diff, uint32_t dim, uint32_t dpad, float levels, float* scale,
+                   float* lb_out, float* diff_out) {
+    uint32_t d = blockIdx.x * blockDim.x + threadIdx.x;
+    if (d < dpad) {
+        scale[d] = d < dim ? diff[d] / levels : 0.0F;
+        lb_out[d] = d < dim ? lb[d] : 0.0F;
+        diff_out[d] = d < dim ? diff[d] : 0.0F;
+    }
+}
+
+__global__ void
+histogram_kernel(const int32_t* labels, uint64_t n, uint32_t nlist, uint32_t* counts, uint32_t* bad) {
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) {
+        int32_t l = labels[i];
+        if (l < 0 || static_cast<uint32_t>(l) >= nlist) {
+            atomicAdd(bad, 1U);
+        } else {
+            atomicAdd(&counts[l], 1U);
+        }
+    }
+}
+
+__global__ void
+iota_kernel(uint32_t* p, uint64_t n) {
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) {
+        p[i] = static_cast<uint32_t>(i);
+    }
+}
+
+// sorted position p (codes ordered by label, stable) -> tile slot inside its list.
+__global__ void
+list_slot_kernel(const int32_t* sorted_labels, uint64_t n, const uint32_t* list_start /* prefix of sizes */,
+                 const uint32_t* list_tile, uint32_t* dst_slot) {
+    uint64_t p = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (p < n) {
+        uint32_t l = static_cast<uint32_t>(sorted_labels[p]);
+        uint32_t rank = static_cast<uint32_t>(p) - list_start[l];
+        dst_slot[p] = list_tile[l] * kWave + rank;
+    }
+}
+
+static int
+grow(vsag_amd_store* s, uint64_t need_tiles, hipStream_t st) {
+    if (need_tiles <= s->cap_tiles) {
+        return 0;
+    }
+    uint64_t cap = s->cap_tiles ? s->cap_tiles : 16;
+    while (cap < need_tiles) {
+        cap *= 2;
+    }
+    uint4* tiles = nullptr;
+    uint32_t* meta = nullptr;
+    size_t tile_bytes = cap * s->G * kWave * sizeof(uint4);
+    VA_HIP(hipMalloc(&tiles, tile_bytes));
+    VA_HIP(hipMemsetAsync(tiles, 0, tile_bytes, st));
+    if (s->nmeta > 0) {
+        VA_HIP(hipMalloc(&meta, cap * kWave * s->nmeta * sizeof(uint32_t)));
+        VA_HIP(hipMemsetAsync(meta, 0, cap * kWave * s->nmeta * sizeof(uint32_t), st));
+    }
+    if (s->ntiles > 0) {
+        VA_HIP(hipMemcpyAsync(tiles, s->tiles, s->ntiles * s->G * kWave * sizeof(uint4), hipMemcpyDeviceToDevice, st));
+        for (uint32_t m = 0; m < s->nmeta; ++m) {
+            VA_HIP(hipMemcpyAsync(meta + m * cap * kWave, s->meta + m * s->cap_tiles * kWave,
+                                  s->ntiles * kWave * sizeof(uint32_t), hipMemcpyDeviceToDevice, st));
+        }
+    }
+    VA_HIP(hipStreamSynchronize(st));
+    if (s->tiles) {
+        VA_HIP(hipFree(s->tiles));
+    }
+    if (s->meta) {
+        VA_HIP(hipFree(s->meta));
+    }
+    s->tiles = tiles;
+    s->meta = meta;
+    s->cap_tiles = cap;
+    return 0;
+}
+
+static RetileArgs
+retile_args(const vsag_amd_store* s, const uint8_t* codes, uint64_t n) {
+    RetileArgs a{};
+    a.codes = codes;
+    a.n = n;
+    a.code_size = s->code_size;
+    a.payload_bytes = s->payload_bytes;
+    a.G = s->G;
+    a.nmeta = s->nmeta;
+    for (int m = 0; m < 4; ++m) {
+        a.meta_offset[m] = s->meta_offset[m];
+    }
+    a.meta_is_u64 = s->meta_is_u64;
+    a.tiles = s->tiles;
+    a.meta = s->meta;
+    a.meta_stride = s->cap_tiles * kWave;
+    a.normalize = (s->kind == VSAG_AMD_KIND_FP32 && s->metric == VSAG_AMD_METRIC_COSINE) ? 1 : 0;
+    a.dim = s->dim;
+    return a;
+}
+
+}  // namespace vsag_amd
+
+using namespace vsag_amd;
+
+extern "C" uint64_t
+vsag_amd_code_size(int kind, int metric, uint32_t dim, int rabitq_query_bits) {
+    auto up = [](uint64_t v, uint64_t a) { return (v + a - 1) / a * a; };
+    switch (kind) {
+        case VSAG_AMD_KIND_FP32:
+            return 4ull * dim;
+        case VSAG_AMD_KIND_SQ8:
+            return dim;
+        case VSAG_AMD_KIND_SQ4:
+            return (static_cast<uint64_t>(dim) * 4 + 7) / 8;
+        case VSAG_AMD_KIND_SQ4_UNIFORM: {
+            // sq4_uniform_quantizer.cpp:33-72: norm (u64) for l2 and cosine, two f32 sums for ip and cosine.
+            bool norm = metric == VSAG_AMD_METRIC_L2 || metric == VSAG_AMD_METRIC_COSINE;
+            bool sum = metric != VSAG_AMD_METRIC_L2;
+            uint64_t align = norm ? 8 : 4;
+            uint64_t size = up((dim + 1) / 2, align);
+            if (norm) {
+                size += up(8, align);
+            }
+            if (sum) {
+                size += 2 * up(4, align);
+            }
+            return size;
+        }
+        case VSAG_AMD_KIND_SQ8_UNIFORM: {
+            // sq8_uniform_quantizer.cpp:30-62: norm (u64) for l2, one f32 sum for ip and cosine.
+            bool norm = metric == VSAG_AMD_METRIC_L2;
+            uint64_t align = norm ? 8 : 4;
+            return up(dim, align) + (norm ? 8 : 4);
+        }
+        case VSAG_AMD_KIND_RABITQ:
+            return rabitq_code_size(dim, metric, rabitq_query_bits ? rabitq_query_bits : 4);
+        default:
+            return 0;
+    }
+}
+
+extern "C" int
+vsag_amd_store_create(const vsag_amd_store_params_t* p, vsag_amd_store_t** out) {
+    VA_TRY(ensure_init());
+    VA_CHECK_ARG(p != nullptr && out != nullptr, "null params / output");
+    *out = nullptr;
+    VA_CHECK_ARG(p->kind >= VSAG_AMD_KIND_FP32 && p->kind <= VSAG_AMD_KIND_RABITQ, "unknown store kind %d", p->kind);
+    VA_CHECK_ARG(p->metric >= VSAG_AMD_METRIC_L2 && p->metric <= VSAG_AMD_METRIC_COSINE, "unknown metric %d",
+                 p->metric);
+    VA_CHECK_ARG(p->dim >= 1 && p->dim <= 65536, "dim must be in [1, 65536], got %u", p->dim);
+    vsag_amd_store* s = new (std::nothrow) vsag_amd_store();
+    if (s == nullptr) {
+        return fail(VSAG_AMD_NO_ENOUGH_MEMORY, "host allocation failed");
+    }
+    s->kind = p->kind;
+    s->metric = p->metric;
+    s->dim = p->dim;
+    s->query_bits = p->rabitq_query_bits ? p->rabitq_query_bits : 4;
+    s->code_size = static_cast<uint32_t>(vsag_amd_code_size(p->kind, p->metric, p->dim, s->query_bits));
+    uint32_t dims_per_granule = 16;
+    auto up = [](uint64_t v, uint64_t a) { return (v + a - 1) / a * a; };
+    int rc = 0;
+    switch (p->kind) {
+        case VSAG_AMD_KIND_FP32:
+            s->payload_bytes = 4 * p->dim;
+            dims_per_granule = 4;
+            break;
+        case VSAG_AMD_KIND_SQ8:
+            s->payload_bytes = p->dim;
+            dims_per_granule = 16;
+            break;
+        case VSAG_AMD_KIND_SQ4:
+            s->payload_bytes = (p->dim + 1) / 2;
+            dims_per_granule = 32;
+            break;
+        case VSAG_AMD_KIND_SQ4_UNIFORM: {
+            s->payload_bytes = (p->dim + 1) / 2;
+            dims_per_granule = 32;
+            bool norm = p->metric == VSAG_AMD_METRIC_L2 || p->metric == VSAG_AMD_METRIC_COSINE;
+            uint64_t align = norm ? 8 : 4;
+            uint64_t off = up(s->payload_bytes, align);
+            s->nmeta = 1;
+            if (p->metric == VSAG_AMD_METRIC_L2) {
+                s->meta_offset[0] = static_cast<uint32_t>(off);
+                s->meta_is_u64 = 1;
+            } else {
+                s->meta_offset[0] = static_cast<uint32_t>(off + (norm ? up(8, align) : 0));
+            }
+            break;
+        }
+        case VSAG_AMD_KIND_SQ8_UNIFORM: {
+            s->payload_bytes = p->dim;
+            dims_per_granule = 16;
+            uint64_t align = p->metric == VSAG_AMD_METRIC_L2 ? 8 : 4;
+            s->nmeta = 1;
+            s->meta_offset[0] = static_cast<uint32_t>(up(p->dim, align));
+            s->meta_is_u64 = p->metric == VSAG_AMD_METRIC_L2 ? 1 : 0;
+            break;
+        }
+        case VSAG_AMD_KIND_RABITQ: {
+            s->payload_bytes = (p->dim + 7) / 8;
+            dims_per_granule = 128;
+            uint32_t off = static_cast<uint32_t>(up(s->payload_bytes, 4));
+            // norm, error, sum, raw norm (rabitq_quantizer.cpp:102-133); sum exists for query_bits != 32.
+            s->nmeta = 4;
+            s->meta_offset[0] = off;
+            s->meta_offset[1] = off + 4;
+            s->meta_offset[2] = s->query_bits != 32 ? off + 8 : off + 4;
+            s->meta_offset[3] = p->metric != VSAG_AMD_METRIC_L2 ? s->code_size - 4 : off + 4;
+            break;
+        }
+    }
+    s->G = static_cast<uint32_t>((s->payload_bytes + kGranule - 1) / kGranule);
+    s->dpad = s->G * dims_per_granule;
+
+    auto fail_free = [&](int code) {
+        vsag_amd_store_destroy(s);
+        return code;
+    };
+    if (p->kind == VSAG_AMD_KIND_SQ8 || p->kind == VSAG_AMD_KIND_SQ4) {
+        if (p->lower_bound_dev == nullptr || p->diff_dev == nullptr) {
+            return fail_free(fail(VSAG_AMD_INVALID_ARGUMENT, "sq8/sq4 store needs lower_bound_dev and diff_dev"));
+        }
+        if (hipMalloc(&s->scale_dev, s->dpad * 4) != hipSuccess || hipMalloc(&s->lb_dev, s->dpad * 4) != hipSuccess ||
+            hipMalloc(&s->diff_dev, s->dpad * 4) != hipSuccess) {
+            return fail_free(fail(VSAG_AMD_NO_ENOUGH_MEMORY, "hipMalloc of quantizer tables failed"));
+        }
+        float levels = p->kind == VSAG_AMD_KIND_SQ8 ? 255.0F : 15.0F;
+        hipLaunchKernelGGL(scale_table_kernel, dim3((s->dpad + 255) / 256), dim3(256), 0, nullptr, p->lower_bound_dev,
+                           p->diff_dev, p->dim, s->dpad, levels, s->scale_dev, s->lb_dev, s->diff_dev);
+        if (hipStreamSynchronize(nullptr) != hipSuccess) {
+            return fail_free(fail(VSAG_AMD_INTERNAL_ERROR, "building the scale table failed"));
+        }
+    } else if (p->kind == VSAG_AMD_KIND_SQ4_UNIFORM || p->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
+        if (p->lower_bound_dev == nullptr) {
+            return fail_free(fail(VSAG_AMD_INVALID_ARGUMENT, "uniform store needs lower_bound_dev = {lb, diff}"));
+        }
+        float b[2];
+        if (hipMalloc(&s->bounds_dev, 8) != hipSuccess ||
+            hipMemcpy(s->bounds_dev, p->lower_bound_dev, 8, hipMemcpyDeviceToDevice) != hipSuccess ||
+            hipMemcpy(b, p->lower_bound_dev, 8, hipMemcpyDeviceToHost) != hipSuccess) {
+            return fail_free(fail(VSAG_AMD_INTERNAL_ERROR, "copying the uniform bounds failed"));
+        }
+        s->ulb = b[0];
+        s->udiff = b[1];
+        // sq4_uniform_quantizer.cpp:104 / sq8_uniform_quantizer.cpp:94: (diff / L) * (diff / L) in double.
+        double levels = p->kind == VSAG_AMD_KIND_SQ4_UNIFORM ? 15.0 : 255.0;
+        s->scalar_rate = static_cast<float>((s->udiff / levels) * (s->udiff / levels));
+    } else if (p->kind == VSAG_AMD_KIND_RABITQ) {
+        if (p->rotation_dev == nullptr || p->centroid_dev == nullptr) {
+            return fail_free(fail(VSAG_AMD_INVALID_ARGUMENT, "rabitq store needs rotation_dev and centroid_dev"));
+        }
+        size_t rb = static_cast<size_t>(p->dim) * p->dim * 4;
+        if (hipMalloc(&s->rotation_dev, rb) != hipSuccess || hipMalloc(&s->centroid_dev, p->dim * 4) != hipSuccess ||
+            hipMemcpy(s->rotation_dev, p->rotation_dev, rb, hipMemcpyDeviceToDevice) != hipSuccess ||
+            hipMemcpy(s->centroid_dev, p->centroid_dev, p->dim * 4, hipMemcpyDeviceToDevice) != hipSuccess) {
+            return fail_free(fail(VSAG_AMD_NO_ENOUGH_MEMORY, "copying the rabitq rotation failed"));
+        }
+    }
+    (void)rc;
+    *out = s;
+    return 0;
+}
+
+extern "C" int
+vsag_amd_store_destroy(vsag_amd_store_t* s) {
+    if (s == nullptr) {
+        return 0;
+    }
+    void* ptrs[] = {s->scale_dev, s->lb_dev,  s->diff_dev, s->bounds_dev,    s->rotation_dev, s->centroid_dev,
+                    s->tiles,     s->meta,    s->ids_dev,  s->list_tile_dev};
+    for (void* p : ptrs) {
+        if (p != nullptr) {
+            (void)hipFree(p);
+        }
+    }
+    delete s;
+    return 0;
+}
+
+extern "C" uint64_t
+vsag_amd_store_size(const vsag_amd_store_t* s) {
+    return s ? s->n : 0;
+}
+
+extern "C" int
+vsag_amd_store_append(vsag_amd_store_t* s, const uint8_t* codes_dev, uint64_t n, void* stream) {
+    VA_TRY(ensure_init());
+    VA_CHECK_ARG(s != nullptr, "store is null");
+    VA_CHECK_ARG(s->nlist == 0, "append on a posting-list store");
+    if (n == 0) {
+        return 0;
+    }
+    VA_CHECK_ARG(codes_dev != nullptr, "codes_dev is null");
+    VA_CHECK_ARG(s->n + n < 0xFFFFFFFFull, "a store holds fewer than 2^32 - 1 codes");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    uint64_t need = div_up(s->n + n, kWave);
+    VA_TRY(grow(s, need, st));
+    RetileArgs a = retile_args(s, codes_dev, n);
+    a.first_slot = s->n;
+    uint64_t threads = n * s->G;
+    hipLaunchKernelGGL(retile_kernel, dim3(static_cast<uint32_t>(div_up(threads, 256))), dim3(256), 0, st, a);
+    VA_HIP(hipGetLastError());
+    s->n += n;
+    s->ntiles = need;
+    return 0;
+}
+
+extern "C" int
+vsag_amd_store_set_lists(vsag_amd_store_t* s, const uint8_t* codes_dev, const int32_t* labels_dev, uint64_t n,
+                         uint32_t nlist, void* stream) {
+    VA_TRY(ensure_init());
+    VA_CHECK_ARG(s != nullptr, "store is null");
+    VA_CHECK_ARG(nlist >= 1 && nlist <= (1u << 24), "nlist must be in [1, 2^24], got %u", nlist);
+    VA_CHECK_ARG(n < 0xFFFFFFFFull, "a store holds fewer than 2^32 - 1 codes");
+    VA_CHECK_ARG(n == 0 || (codes_dev && labels_dev), "null codes / labels");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+
+    // 1. list sizes
+    uint32_t* counts = nullptr;
+    VA_HIP(hipMalloc(&counts, (nlist + 1) * sizeof(uint32_t)));
+    VA_HIP(hipMemsetAsync(counts, 0, (nlist + 1) * sizeof(uint32_t), st));
+    if (n > 0) {
+        hipLaunchKernelGGL(histogram_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, labels_dev,
+                           n, nlist, counts, counts + nlist);
+    }
+    std::vector<uint32_t> sizes(nlist + 1);
+    VA_HIP(hipMemcpyAsync(sizes.data(), counts, (nlist + 1) * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    VA_HIP(hipStreamSynchronize(st));
+    VA_HIP(hipFree(counts));
+    VA_CHECK_ARG(sizes[nlist] == 0, "%u labels are outside [0, %u)", sizes[nlist], nlist);
+
+    // 2. tile offsets (each list padded to whole tiles) and code offsets
+    std::vector<uint32_t> list_tile(nlist + 1, 0), list_start(nlist + 1, 0);
+    for (uint32_t l = 0; l < nlist; ++l) {
+        list_tile[l + 1] = list_tile[l] + static_cast<uint32_t>(div_up(sizes[l], kWave));
+        list_start[l + 1] = list_start[l] + sizes[l];
+    }
+    uint64_t ntiles = list_tile[nlist];
+
+    // 3. fresh storage
+    for (void* p : {static_cast<void*>(s->tiles), static_cast<void*>(s->meta), static_cast<void*>(s->ids_dev),
+                    static_cast<void*>(s->list_tile_dev)}) {
+        if (p != nullptr) {
+            VA_HIP(hipFree(p));
+        }
+    }
+    s->tiles = nullptr;
+    s->meta = nullptr;
+    s->ids_dev = nullptr;
+    s->list_tile_dev = nullptr;
+    s->cap_tiles = 0;
+    s->ntiles = 0;
+    s->n = 0;
+    uint64_t cap = ntiles > 0 ? ntiles : 1;
+    VA_HIP(hipMalloc(&s->tiles, cap * s->G * kWave * sizeof(uint4)));
+    VA_HIP(hipMemsetAsync(s->tiles, 0, cap * s->G * kWave * sizeof(uint4), st));
+    if (s->nmeta > 0) {
+        VA_HIP(hipMalloc(&s->meta, cap * kWave * s->nmeta * sizeof(uint32_t)));
+        VA_HIP(hipMemsetAsync(s->meta, 0, cap * kWave * s->nmeta * sizeof(uint32_t), st));
+    }
+    VA_HIP(hipMalloc(&s->ids_dev, cap * kWave * sizeof(uint32_t)));
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(static_cast<uint32_t>(div_up(cap * kWave, 256))), dim3(256), 0, st,
+                       s->ids_dev, VSAG_AMD_INVALID_ID, cap * kWave);
+    VA_HIP(hipMalloc(&s->list_tile_dev, (nlist + 1) * sizeof(uint32_t)));
+    VA_HIP(hipMemcpyAsync(s->list_tile_dev, list_tile.data(), (nlist + 1) * sizeof(uint32_t), hipMemcpyHostToDevice,
+                          st));
+    s->cap_tiles = cap;
+    s->ntiles = ntiles;
+    s->nlist = nlist;
+    s->list_sizes.assign(sizes.begin(), sizes.begin() + nlist);
+    s->list_tile = list_tile;
+
+    if (n > 0) {
+        // 4. stable sort of inner ids by label: the order the reference gets by appending vectors to their
+        // bucket one after another (ivf.cpp:661-675 without a thread pool).
+        int32_t* keys_out = nullptr;
+        uint32_t *vals_in = nullptr, *vals_out = nullptr, *start_dev = nullptr, *dst_slot = nullptr;
+        void* tmp = nullptr;
+        size_t tmp_bytes = 0;
+        VA_HIP(hipMalloc(&keys_out, n * 4));
+        VA_HIP(hipMalloc(&vals_in, n * 4));
+        VA_HIP(hipMalloc(&vals_out, n * 4));
+        VA_HIP(hipMalloc(&dst_slot, n * 4));
+        VA_HIP(hipMalloc(&start_dev, (nlist + 1) * 4));
+        VA_HIP(hipMemcpyAsync(start_dev, list_start.data(), (nlist + 1) * 4, hipMemcpyHostToDevice, st));
+        hipLaunchKernelGGL(iota_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, vals_in, n);
+        int end_bit = 1;
+        while ((1u << end_bit) < nlist) {
+            ++end_bit;
+        }
+        VA_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, labels_dev, keys_out, vals_in, vals_out,
+                                                  static_cast<int>(n), 0, end_bit, st));
+        VA_HIP(hipMalloc(&tmp, tmp_bytes));
+        VA_HIP(hipcub::DeviceRadixSort::SortPairs(tmp, tmp_bytes, labels_dev, keys_out, vals_in, vals_out,
+                                                  static_cast<int>(n), 0, end_bit, st));
+        hipLaunchKernelGGL(list_slot_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, keys_out, n,
+                           start_dev, s->list_tile_dev, dst_slot);
+        RetileArgs a = retile_args(s, codes_dev, n);
+        a.src_index = vals_out;
+        a.dst_slot = dst_slot;
+        a.ids = s->ids_dev;
+        hipLaunchKernelGGL(retile_kernel, dim3(static_cast<uint32_t>(div_up(n * s->G, 256))), dim3(256), 0, st, a);
+        VA_HIP(hipGetLastError());
+        VA_HIP(hipStreamSynchronize(st));
+        for (void* p : {static_cast<void*>(keys_out), static_cast<void*>(vals_in), static_cast<void*>(vals_out),
+                        static_cast<void*>(dst_slot), static_cast<void*>(start_dev), tmp}) {
+            VA_HIP(hipFree(p));
+        }
+    }
+    s->n = n;
+    return 0;
+}
+
+extern "C" int
+vsag_amd_store_list_sizes(const vsag_amd_store_t* s, uint32_t* sizes, uint32_t nlist) {
+    VA_CHECK_ARG(s != nullptr && sizes != nullptr, "null store / output");
+    VA_CHECK_ARG(s->nlist == nlist, "store has %u lists, asked for %u", s->nlist, nlist);
+    memcpy(sizes, s->list_sizes.data(), nlist * sizeof(uint32_t));
+    return 0;
+}

@@ -1,0 +1,108 @@
+// Wave-level streaming top-k selector kept in LDS.
+//
+// One wavefront owns one selector per query it serves.  A selector is an array of S 64-bit keys
+// (S a power of two, S >= k + 128): slots [0,k) hold the best keys found so far, slots [k,k+cnt) hold
+// pending candidates that passed the current threshold.  When the pending region could overflow on the
+// next 64-wide append, the wave sorts the whole array (bitonic, in LDS) which leaves the k best in
+// front and yields the new threshold keys[k-1].  No workgroup barrier is involved: only the owning
+// wave touches a selector, and LDS operations of one wave complete in program order.
+//
+// This replaces the reference's per-query bounded max-heap (src/impl/heap/standard_heap.cpp:24-53,
+// src/algorithm/ivf/flat_bucket_searcher.cpp:89-100): same k smallest distances, with ties ordered by
+// inner id (the reference leaves the order of equal distances unspecified).
+#pragma once
+
+#include "common.h"
+
+namespace vsag_amd {
+
+__device__ inline void
+wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+__device__ inline uint32_t
+lane_id() {
+    return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+}
+
+// Number of set bits of `mask` below this lane.
+__device__ inline uint32_t
+mask_rank(uint64_t mask) {
+    return __builtin_amdgcn_mbcnt_hi(static_cast<uint32_t>(mask >> 32),
+                                     __builtin_amdgcn_mbcnt_lo(static_cast<uint32_t>(mask), 0u));
+}
+
+__device__ inline uint64_t
+wave_uniform_u64(uint64_t v) {
+    uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+    uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+    return (static_cast<uint64_t>(hi) << 32) | lo;
+}
+
+// Selector size for a given k.
+__host__ __device__ inline uint32_t
+selector_slots(uint32_t k) {
+    uint32_t s = 256;
+    while (s < k + 128) {
+        s <<= 1;
+    }
+    return s;
+}
+
+__device__ inline void
+selector_init(uint64_t* keys, uint32_t S, uint32_t lane) {
+    for (uint32_t i = lane; i < S; i += kWave) {
+        keys[i] = kInfKey;
+    }
+    wave_lds_fence();
+}
+
+// Ascending bitonic sort of keys[0,S) by one wavefront.
+__device__ inline void
+wave_bitonic_sort(uint64_t* keys, uint32_t S, uint32_t lane) {
+    for (uint32_t size = 2; size <= S; size <<= 1) {
+        for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+            for (uint32_t i = lane; i < (S >> 1); i += kWave) {
+                uint32_t pos = 2 * i - (i & (stride - 1));
+                uint64_t a = keys[pos];
+                uint64_t b = keys[pos + stride];
+                bool up = (pos & size) == 0;
+                if ((a > b) == up) {
+                    keys[pos] = b;
+                    keys[pos + stride] = a;
+                }
+            }
+            wave_lds_fence();
+        }
+    }
+}
+
+// Sorts, keeps the k best in front, returns the new threshold key (wave-uniform).
+__device__ inline uint64_t
+selector_flush(uint64_t* keys, uint32_t S, uint32_t k, uint32_t cnt, uint32_t lane) {
+    for (uint32_t i = k + cnt + lane; i < S; i += kWave) {
+        keys[i] = kInfKey;
+    }
+    wave_lds_fence();
+    wave_bitonic_sort(keys, S, lane);
+    return wave_uniform_u64(keys[k - 1]);
+}
+
+// Appends the keys of the lanes with `pass` set behind the pending region; returns the new count.
+// The caller guarantees k + cnt + 64 <= S.
+__device__ inline uint32_t
+selector_append(uint64_t* keys, uint32_t k, uint32_t cnt, bool pass, uint64_t key) {
+    uint64_t mask = __ballot(pass);
+    if (mask != 0) {
+        if (pass) {
+            keys[k + cnt + mask_rank(mask)] = key;
+        }
+        cnt += __popcll(mask);
+    }
+    return cnt;
+}
+
+}  // namespace vsag_amd
