@@ -1113,6 +1113,37 @@ orc_flat_scan_topk(int kind, int metric, uint64_t dim, const uint8_t* codes, uin
     }
 }
 
+// The same loop with the per-code distance supplied by the caller: used to time the reference's own
+// compiled SIMD kernels (oracle/_ref, e.g. vsag::avx512::SQ8ComputeL2Sqr) under the BruteForce loop and
+// heap restated above.  fn has the SQ8 / SQ4 signature (query, code, lower_bound, diff, dim); the value it
+// returns is turned into a distance as scalar_quantizer.cpp:180-196 does (IP -> 1 - ip).
+typedef float (*sq_dist_fn)(const float*, const uint8_t*, const float*, const float*, uint64_t);
+ORC_API void
+orc_flat_scan_topk_fn(void* fn_ptr, int metric, uint64_t dim, const uint8_t* codes, uint64_t n, uint64_t code_size,
+                      const float* lb, const float* diff, const float* queries, uint64_t nq, uint64_t k,
+                      uint32_t* out_ids, float* out_dists, int threads) {
+    auto fn = reinterpret_cast<sq_dist_fn>(fn_ptr);
+#ifdef _OPENMP
+    if (threads > 0) {
+        omp_set_num_threads(threads);
+    }
+#endif
+#pragma omp parallel for schedule(dynamic)
+    for (int64_t qi = 0; qi < static_cast<int64_t>(nq); ++qi) {
+        const float* q = queries + qi * dim;
+        FixedMaxHeap h(k);
+        for (uint64_t i = 0; i < n; ++i) {
+            float v = fn(q, codes + i * code_size, lb, diff, dim);
+            h.push(metric == kL2 ? v : 1 - v, static_cast<uint32_t>(i));
+        }
+        uint64_t cnt = h.drain(out_ids + qi * k, out_dists + qi * k);
+        for (uint64_t j = cnt; j < k; ++j) {
+            out_ids[qi * k + j] = 0xFFFFFFFFU;
+            out_dists[qi * k + j] = std::numeric_limits<float>::infinity();
+        }
+    }
+}
+
 // All (query, code) distances, for small parity cases.
 ORC_API void
 orc_flat_dists(int kind, int metric, uint64_t dim, const uint8_t* codes, uint64_t n, uint64_t code_size,
@@ -1232,6 +1263,19 @@ orc_rerank_fp32(const float* raw, uint64_t dim, int metric, const float* queries
             out_dists[qi * k + j] = std::numeric_limits<float>::infinity();
         }
     }
+}
+
+// 1 when the host CPU can run the reference's avx512 kernels (flags of src/simd/CMakeLists.txt:57).
+ORC_API int
+orc_cpu_has_avx512() {
+    return __builtin_cpu_supports("avx512f") && __builtin_cpu_supports("avx512bw") &&
+           __builtin_cpu_supports("avx512dq") && __builtin_cpu_supports("avx512vl") &&
+           __builtin_cpu_supports("avx512cd") && __builtin_cpu_supports("avx512ifma") &&
+           __builtin_cpu_supports("avx512vbmi");
+}
+ORC_API int
+orc_cpu_has_avx2() {
+    return __builtin_cpu_supports("avx2") && __builtin_cpu_supports("fma");
 }
 
 ORC_API int

@@ -1,5 +1,5 @@
 """ctypes access to the CPU checker (oracle/liboracle.so) and, when built, to the reference's own scalar
-kernels compiled from its sources (oracle/_ref/libvsag_generic.so).  Test infrastructure only."""
+kernels compiled from its sources (oracle/_ref/libvsag_simd.so).  Test infrastructure only."""
 import ctypes as C
 import os
 import subprocess
@@ -9,7 +9,7 @@ import numpy as np
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_DIR = os.path.join(ROOT, "oracle")
 LIB = os.path.join(ORACLE_DIR, "liboracle.so")
-REF_GENERIC = os.path.join(ORACLE_DIR, "_ref", "libvsag_generic.so")
+REF_SIMD = os.path.join(ORACLE_DIR, "_ref", "libvsag_simd.so")
 
 L2, IP, COSINE = 0, 1, 2
 FP32, SQ8, SQ4, SQ4U, SQ8U, RABITQ = range(6)
@@ -278,9 +278,9 @@ def ref():
     """dict name -> ctypes function of vsag::generic, or None when oracle/_ref is not built."""
     global _ref
     if _ref is None:
-        if not os.path.exists(REF_GENERIC):
+        if not os.path.exists(REF_SIMD):
             return None
-        dll = C.CDLL(REF_GENERIC)
+        dll = C.CDLL(REF_SIMD)
         fns = {}
         for name, sym in _REF_SYMBOLS.items():
             fn = getattr(dll, sym)
@@ -288,3 +288,34 @@ def ref():
             fns[name] = fn
         _ref = fns
     return _ref
+
+
+def ref_best_isa():
+    """Highest ISA tier of the reference's kernels this host can execute: 'avx512', 'avx2' or 'generic'."""
+    if lib().orc_cpu_has_avx512():
+        return "avx512"
+    if lib().orc_cpu_has_avx2():
+        return "avx2"
+    return "generic"
+
+
+def ref_sq8_fn(metric, isa):
+    """Address of vsag::<isa>::SQ8ComputeL2Sqr / SQ8ComputeIP in oracle/_ref, or None."""
+    if not os.path.exists(REF_SIMD):
+        return None
+    dll = C.CDLL(REF_SIMD)
+    name = "SQ8ComputeL2Sqr" if metric == L2 else "SQ8ComputeIP"
+    sym = "_ZN4vsag%d%s%d%sEPKfPKhS2_S2_m" % (len(isa), isa, len(name), name)
+    return C.cast(getattr(dll, sym), C.c_void_p)
+
+
+def flat_scan_topk_fn(fn, metric, d, codes, queries, k, lb, diff, threads=0):
+    codes = np.ascontiguousarray(codes)
+    queries = f32(queries)
+    n, cs = codes.shape
+    nq = queries.shape[0]
+    ids = np.empty((nq, k), np.uint32)
+    dists = np.empty((nq, k), np.float32)
+    lib().orc_flat_scan_topk_fn(fn, metric, u64(d), _p(codes), u64(n), u64(cs), _p(f32(lb)), _p(f32(diff)),
+                                _p(queries), u64(nq), u64(k), _p(ids), _p(dists), threads)
+    return ids, dists

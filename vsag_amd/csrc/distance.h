@@ -44,162 +44,175 @@ struct ScanArgs {
     float f0, f1, f2;       // uniform kinds: lb, scalar_rate, lb*lb
 };
 
+// Tile rows are consumed in groups of kGroup granules so that the loads of the next group can be in flight
+// while the current one is being multiplied (see TileStream below).
+constexpr int kGroup = 4;
+
+// Running sums of T queries against the code owned by this lane.
+template <int KIND, int T>
+struct Acc {
+    float f[T];         // fp32 / sq8 / sq4
+    uint32_t lo[T];     // uniform kinds (and plane 0 of rabitq)
+    uint32_t hi[T];     // sq4_uniform high nibbles (x16); rabitq plane 1
+    uint32_t p2[T];     // rabitq plane 2
+    uint32_t p3[T];     // rabitq plane 3
+};
+
+template <int KIND, int T>
+__device__ inline void
+acc_reset(Acc<KIND, T>& a) {
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        a.f[t] = 0.0F;
+        a.lo[t] = a.hi[t] = a.p2[t] = a.p3[t] = 0;
+    }
+}
+
+// Wave-uniform row pointers of the T processed queries (constant address space -> scalar loads).
+template <int T>
+struct QueryRows {
+    cu32_p row[T];
+};
+
+template <int T>
+__device__ inline QueryRows<T>
+query_rows(const ScanArgs& a, const uint32_t (&qidx)[T]) {
+    QueryRows<T> r;
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        r.row[t] = as_const(a.qtab + static_cast<size_t>(qidx[t]) * a.qstride);
+    }
+    return r;
+}
+
+// One granule (16 bytes of this lane's code, granule index j) against the T queries.
 template <int KIND, int METRIC, int T>
 __device__ inline void
-tile_distances(const ScanArgs& a, uint64_t tile, const uint32_t (&qidx)[T], uint32_t lane, float (&out)[T]) {
-    const uint4* tp = a.tiles + tile * a.G * kWave + lane;
-    const uint64_t slot = tile * kWave + lane;
-
+accumulate_granule(const ScanArgs& a, const QueryRows<T>& q, uint32_t j, uint4 c, Acc<KIND, T>& acc) {
+    const uint32_t w[4] = {c.x, c.y, c.z, c.w};
     if constexpr (KIND == VSAG_AMD_KIND_FP32) {
-        float acc[T];
-        cfloat_p qrow[T];
 #pragma unroll
-        for (int t = 0; t < T; ++t) {
-            acc[t] = 0.0F;
-            qrow[t] = as_const(reinterpret_cast<const float*>(a.qtab) + static_cast<size_t>(qidx[t]) * a.qstride);
-        }
-        for (uint32_t j = 0; j < a.G; ++j) {
-            uint4 c = tp[j * kWave];
-            float x[4] = {__uint_as_float(c.x), __uint_as_float(c.y), __uint_as_float(c.z), __uint_as_float(c.w)};
+        for (int e = 0; e < 4; ++e) {
+            float x = __uint_as_float(w[e]);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-#pragma unroll
-                for (int t = 0; t < T; ++t) {
-                    float qv = qrow[t][4 * j + e];
-                    if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
-                        float d = x[e] - qv;
-                        acc[t] = fmaf(d, d, acc[t]);
-                    } else {
-                        acc[t] = fmaf(x[e], qv, acc[t]);
-                    }
+            for (int t = 0; t < T; ++t) {
+                float qv = __uint_as_float(q.row[t][4 * j + e]);
+                if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                    float d = x - qv;
+                    acc.f[t] = fmaf(d, d, acc.f[t]);
+                } else {
+                    acc.f[t] = fmaf(x, qv, acc.f[t]);
                 }
             }
-        }
-#pragma unroll
-        for (int t = 0; t < T; ++t) {
-            out[t] = METRIC == VSAG_AMD_METRIC_L2 ? acc[t] : 1.0F - acc[t];
         }
     } else if constexpr (KIND == VSAG_AMD_KIND_SQ8) {
         // qtab row: L2 -> q[d] - lb[d];  IP -> q[d] * scale[d], qmeta[0] = sum q[d] * lb[d].
-        float acc[T];
-        cfloat_p qrow[T];
         cfloat_p sc = as_const(a.scale);
 #pragma unroll
-        for (int t = 0; t < T; ++t) {
-            acc[t] = 0.0F;
-            qrow[t] = as_const(reinterpret_cast<const float*>(a.qtab) + static_cast<size_t>(qidx[t]) * a.qstride);
-        }
-        for (uint32_t j = 0; j < a.G; ++j) {
-            uint4 c = tp[j * kWave];
-            uint32_t w[4] = {c.x, c.y, c.z, c.w};
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                float cf = static_cast<float>((w[e >> 2] >> (8 * (e & 3))) & 0xffU);
-                if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
-                    float y = cf * sc[16 * j + e];
-#pragma unroll
-                    for (int t = 0; t < T; ++t) {
-                        float d = y - qrow[t][16 * j + e];
-                        acc[t] = fmaf(d, d, acc[t]);
-                    }
-                } else {
-#pragma unroll
-                    for (int t = 0; t < T; ++t) {
-                        acc[t] = fmaf(cf, qrow[t][16 * j + e], acc[t]);
-                    }
-                }
-            }
-        }
-#pragma unroll
-        for (int t = 0; t < T; ++t) {
+        for (int e = 0; e < 16; ++e) {
+            float cf = static_cast<float>((w[e >> 2] >> (8 * (e & 3))) & 0xffU);
             if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
-                out[t] = acc[t];
+                float y = cf * sc[16 * j + e];
+#pragma unroll
+                for (int t = 0; t < T; ++t) {
+                    float d = y - __uint_as_float(q.row[t][16 * j + e]);
+                    acc.f[t] = fmaf(d, d, acc.f[t]);
+                }
             } else {
-                out[t] = 1.0F - (acc[t] + a.qmeta[static_cast<size_t>(qidx[t]) * a.qmeta_stride]);
+#pragma unroll
+                for (int t = 0; t < T; ++t) {
+                    acc.f[t] = fmaf(cf, __uint_as_float(q.row[t][16 * j + e]), acc.f[t]);
+                }
             }
         }
     } else if constexpr (KIND == VSAG_AMD_KIND_SQ4) {
         // Byte b of a code holds dim 2b in its low nibble and dim 2b+1 in its high nibble.
-        float acc[T];
-        cfloat_p qrow[T];
         cfloat_p sc = as_const(a.scale);
 #pragma unroll
-        for (int t = 0; t < T; ++t) {
-            acc[t] = 0.0F;
-            qrow[t] = as_const(reinterpret_cast<const float*>(a.qtab) + static_cast<size_t>(qidx[t]) * a.qstride);
-        }
-        for (uint32_t j = 0; j < a.G; ++j) {
-            uint4 c = tp[j * kWave];
-            uint32_t w[4] = {c.x, c.y, c.z, c.w};
+        for (int m = 0; m < 4; ++m) {
+            uint32_t lo = w[m] & 0x0F0F0F0FU;
+            uint32_t hi = (w[m] >> 4) & 0x0F0F0F0FU;
 #pragma unroll
-            for (int m = 0; m < 4; ++m) {
-                uint32_t lo = w[m] & 0x0F0F0F0FU;
-                uint32_t hi = (w[m] >> 4) & 0x0F0F0F0FU;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    uint32_t src = (e & 1) ? hi : lo;
-                    float cf = static_cast<float>((src >> (8 * (e >> 1))) & 0xffU);
-                    uint32_t d = 32 * j + 8 * m + e;
-                    if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
-                        float y = cf * sc[d];
-#pragma unroll
-                        for (int t = 0; t < T; ++t) {
-                            float df = y - qrow[t][d];
-                            acc[t] = fmaf(df, df, acc[t]);
-                        }
-                    } else {
-#pragma unroll
-                        for (int t = 0; t < T; ++t) {
-                            acc[t] = fmaf(cf, qrow[t][d], acc[t]);
-                        }
-                    }
-                }
-            }
-        }
-#pragma unroll
-        for (int t = 0; t < T; ++t) {
-            if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
-                out[t] = acc[t];
-            } else {
-                out[t] = 1.0F - (acc[t] + a.qmeta[static_cast<size_t>(qidx[t]) * a.qmeta_stride]);
-            }
-        }
-    } else if constexpr (KIND == VSAG_AMD_KIND_SQ4_UNIFORM || KIND == VSAG_AMD_KIND_SQ8_UNIFORM) {
-        // Integer code x code inner product.  SQ4U qtab row: per code dword {low nibbles, high nibbles
-        // << 4 kept in place}; the high-nibble products come out 16x too large and are shifted back.
-        uint32_t acc_lo[T], acc_hi[T];
-        cu32_p qrow[T];
-#pragma unroll
-        for (int t = 0; t < T; ++t) {
-            acc_lo[t] = 0;
-            acc_hi[t] = 0;
-            qrow[t] = as_const(a.qtab + static_cast<size_t>(qidx[t]) * a.qstride);
-        }
-        for (uint32_t j = 0; j < a.G; ++j) {
-            uint4 c = tp[j * kWave];
-            uint32_t w[4] = {c.x, c.y, c.z, c.w};
-#pragma unroll
-            for (int m = 0; m < 4; ++m) {
-                if constexpr (KIND == VSAG_AMD_KIND_SQ4_UNIFORM) {
-                    uint32_t lo = w[m] & 0x0F0F0F0FU;
-                    uint32_t hi = w[m] & 0xF0F0F0F0U;
+            for (int e = 0; e < 8; ++e) {
+                uint32_t src = (e & 1) ? hi : lo;
+                float cf = static_cast<float>((src >> (8 * (e >> 1))) & 0xffU);
+                uint32_t d = 32 * j + 8 * m + e;
+                if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                    float y = cf * sc[d];
 #pragma unroll
                     for (int t = 0; t < T; ++t) {
-                        acc_lo[t] = __builtin_amdgcn_udot4(lo, qrow[t][2 * (4 * j + m)], acc_lo[t], false);
-                        acc_hi[t] = __builtin_amdgcn_udot4(hi, qrow[t][2 * (4 * j + m) + 1], acc_hi[t], false);
+                        float df = y - __uint_as_float(q.row[t][d]);
+                        acc.f[t] = fmaf(df, df, acc.f[t]);
                     }
                 } else {
 #pragma unroll
                     for (int t = 0; t < T; ++t) {
-                        acc_lo[t] = __builtin_amdgcn_udot4(w[m], qrow[t][4 * j + m], acc_lo[t], false);
+                        acc.f[t] = fmaf(cf, __uint_as_float(q.row[t][d]), acc.f[t]);
                     }
                 }
             }
         }
+    } else if constexpr (KIND == VSAG_AMD_KIND_SQ4_UNIFORM) {
+        // qtab row: per code dword {low nibbles, high nibbles}.  The code's high nibbles stay in place
+        // (x16), so their products come out 16 times too large and are shifted back at the end.
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            uint32_t lo = w[m] & 0x0F0F0F0FU;
+            uint32_t hi = w[m] & 0xF0F0F0F0U;
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                acc.lo[t] = __builtin_amdgcn_udot4(lo, q.row[t][2 * (4 * j + m)], acc.lo[t], false);
+                acc.hi[t] = __builtin_amdgcn_udot4(hi, q.row[t][2 * (4 * j + m) + 1], acc.hi[t], false);
+            }
+        }
+    } else if constexpr (KIND == VSAG_AMD_KIND_SQ8_UNIFORM) {
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                acc.lo[t] = __builtin_amdgcn_udot4(w[m], q.row[t][4 * j + m], acc.lo[t], false);
+            }
+        }
+    } else if constexpr (KIND == VSAG_AMD_KIND_RABITQ) {
+        // qtab row: per code dword the four query bit planes.
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                cu32_p qp = q.row[t] + 4 * (4 * j + m);
+                acc.lo[t] += __builtin_popcount(w[m] & qp[0]);
+                acc.hi[t] += __builtin_popcount(w[m] & qp[1]);
+                acc.p2[t] += __builtin_popcount(w[m] & qp[2]);
+                acc.p3[t] += __builtin_popcount(w[m] & qp[3]);
+            }
+        }
+    }
+}
+
+// Distances of the finished code (tile slot `slot`) to the T queries.
+template <int KIND, int METRIC, int T>
+__device__ inline void
+finish_distances(const ScanArgs& a, const uint32_t (&qidx)[T], uint64_t slot, const Acc<KIND, T>& acc,
+                 float (&out)[T]) {
+    if constexpr (KIND == VSAG_AMD_KIND_FP32) {
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            out[t] = METRIC == VSAG_AMD_METRIC_L2 ? acc.f[t] : 1.0F - acc.f[t];
+        }
+    } else if constexpr (KIND == VSAG_AMD_KIND_SQ8 || KIND == VSAG_AMD_KIND_SQ4) {
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                out[t] = acc.f[t];
+            } else {
+                out[t] = 1.0F - (acc.f[t] + a.qmeta[static_cast<size_t>(qidx[t]) * a.qmeta_stride]);
+            }
+        }
+    } else if constexpr (KIND == VSAG_AMD_KIND_SQ4_UNIFORM || KIND == VSAG_AMD_KIND_SQ8_UNIFORM) {
         float m0 = __uint_as_float(a.meta[slot]);
 #pragma unroll
         for (int t = 0; t < T; ++t) {
-            uint32_t ip = KIND == VSAG_AMD_KIND_SQ4_UNIFORM ? acc_lo[t] + (acc_hi[t] >> 4) : acc_lo[t];
+            uint32_t ip = KIND == VSAG_AMD_KIND_SQ4_UNIFORM ? acc.lo[t] + (acc.hi[t] >> 4) : acc.lo[t];
             float result = static_cast<float>(static_cast<int32_t>(ip));
             float qm = a.qmeta[static_cast<size_t>(qidx[t]) * a.qmeta_stride];
             if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
@@ -212,40 +225,18 @@ tile_distances(const ScanArgs& a, uint64_t tile, const uint32_t (&qidx)[T], uint
             }
         }
     } else if constexpr (KIND == VSAG_AMD_KIND_RABITQ) {
-        // qtab row: per code dword the four query bit planes.  qmeta: {2 delta/sqrt(d), 2 lb/sqrt(d),
-        // delta sum_q/sqrt(d), lb d/sqrt(d), ||Rq - c||, ||q||}.
-        uint32_t acc[T][4];
-        cu32_p qrow[T];
-#pragma unroll
-        for (int t = 0; t < T; ++t) {
-            acc[t][0] = acc[t][1] = acc[t][2] = acc[t][3] = 0;
-            qrow[t] = as_const(a.qtab + static_cast<size_t>(qidx[t]) * a.qstride);
-        }
-        for (uint32_t j = 0; j < a.G; ++j) {
-            uint4 c = tp[j * kWave];
-            uint32_t w[4] = {c.x, c.y, c.z, c.w};
-#pragma unroll
-            for (int m = 0; m < 4; ++m) {
-#pragma unroll
-                for (int t = 0; t < T; ++t) {
-#pragma unroll
-                    for (int b = 0; b < 4; ++b) {
-                        acc[t][b] += __builtin_popcount(w[m] & qrow[t][4 * (4 * j + m) + b]);
-                    }
-                }
-            }
-        }
+        // qmeta: {2 delta/sqrt(d), 2 lb/sqrt(d), delta sum_q/sqrt(d), lb d/sqrt(d), ||Rq - c||, ||q||}.
         float base_norm = __uint_as_float(a.meta[slot]);
         float base_error = __uint_as_float(a.meta[a.meta_stride + slot]);
         float base_sum = __uint_as_float(a.meta[2 * a.meta_stride + slot]);
         float base_raw = METRIC == VSAG_AMD_METRIC_L2 ? 0.0F : __uint_as_float(a.meta[3 * a.meta_stride + slot]);
-        if (fabsf(base_error) < 1e-5F) {
+        if (static_cast<double>(fabsf(base_error)) < 1e-5) {
             base_error = (base_error >= 0) ? 1.0F : -1.0F;
         }
 #pragma unroll
         for (int t = 0; t < T; ++t) {
             const float* qm = a.qmeta + static_cast<size_t>(qidx[t]) * a.qmeta_stride;
-            uint32_t ip = acc[t][0] + (acc[t][1] << 1) + (acc[t][2] << 2) + (acc[t][3] << 3);
+            uint32_t ip = acc.lo[t] + (acc.hi[t] << 1) + (acc.p2[t] << 2) + (acc.p3[t] << 3);
             float p1 = qm[0] * static_cast<float>(ip);
             float p2 = qm[1] * base_sum;
             float ip_bq = p1 + p2 - qm[2] - qm[3];
@@ -257,14 +248,14 @@ tile_distances(const ScanArgs& a, uint64_t tile, const uint32_t (&qidx)[T], uint
             float result = e1 + e2 + e3;
             if constexpr (METRIC == VSAG_AMD_METRIC_IP) {
                 float qr = qm[5];
-                if (fabsf(qr) < 1e-5F || fabsf(base_raw) < 1e-5F) {
+                if (static_cast<double>(fabsf(qr)) < 1e-5 || static_cast<double>(fabsf(base_raw)) < 1e-5) {
                     result = 1;
                 } else {
                     result = 1 - (qr * qr + base_raw * base_raw - result) * 0.5F;
                 }
             } else if constexpr (METRIC == VSAG_AMD_METRIC_COSINE) {
                 float qr = qm[5];
-                if (fabsf(qr) < 1e-5F || fabsf(base_raw) < 1e-5F) {
+                if (static_cast<double>(fabsf(qr)) < 1e-5 || static_cast<double>(fabsf(base_raw)) < 1e-5) {
                     result = 1;
                 } else {
                     result = 1 - (qr * qr + base_raw * base_raw - result) * 0.5F / (qr * base_raw);
@@ -274,5 +265,36 @@ tile_distances(const ScanArgs& a, uint64_t tile, const uint32_t (&qidx)[T], uint
         }
     }
 }
+
+// The sequence of granule groups one wave walks: tiles first, first + stride, ... below end; inside a tile
+// groups j0 = 0, kGroup, ...  `load` fetches a group into registers, `advance` steps to the next one.
+struct TileStream {
+    const uint4* base;   // tiles + lane
+    uint64_t tile, end, stride;
+    uint32_t j0, G;
+
+    __device__ inline bool
+    valid() const {
+        return tile < end;
+    }
+    __device__ inline void
+    load(uint4 (&regs)[kGroup]) const {
+        const uint4* tp = base + (tile * G + j0) * kWave;
+#pragma unroll
+        for (int u = 0; u < kGroup; ++u) {
+            if (j0 + u < G) {
+                regs[u] = tp[u * kWave];
+            }
+        }
+    }
+    __device__ inline void
+    advance() {
+        j0 += kGroup;
+        if (j0 >= G) {
+            j0 = 0;
+            tile += stride;
+        }
+    }
+};
 
 }  // namespace vsag_amd

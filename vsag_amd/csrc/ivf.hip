@@ -177,10 +177,31 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
     wave_lds_fence();
 
     const uint32_t tbeg = as_const(v.list_tile)[b], tend = as_const(v.list_tile)[b + 1];
-    for (uint32_t tile = tbeg; tile < tend; ++tile) {
+    const QueryRows<T> qrows = query_rows<T>(a, qidx);
+    TileStream cur{a.tiles + lane, tbeg, tend, 1, 0, a.G};
+    TileStream nxt = cur;
+    uint4 buf_a[kGroup], buf_b[kGroup];
+    if (cur.valid()) {
+        cur.load(buf_a);
+    }
+    Acc<KIND, T> acc;
+    acc_reset(acc);
+
+    auto consume = [&](const uint4(&regs)[kGroup]) {
+#pragma unroll
+        for (int u = 0; u < kGroup; ++u) {
+            if (cur.j0 + u < a.G) {
+                accumulate_granule<KIND, METRIC, T>(a, qrows, cur.j0 + u, regs[u], acc);
+            }
+        }
+        if (cur.j0 + kGroup < a.G) {
+            return;
+        }
+        const uint64_t slot = cur.tile * kWave + lane;
         float d[T];
-        tile_distances<KIND, METRIC, T>(a, tile, qidx, lane, d);
-        const uint32_t id = v.ids[static_cast<uint64_t>(tile) * kWave + lane];
+        finish_distances<KIND, METRIC, T>(a, qidx, slot, acc, d);
+        acc_reset(acc);
+        const uint32_t id = v.ids[slot];
         const bool valid = id != VSAG_AMD_INVALID_ID;
 #pragma unroll
         for (int t = 0; t < T; ++t) {
@@ -207,6 +228,24 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
                 }
             }
         }
+    };
+
+    while (cur.valid()) {
+        nxt.advance();
+        if (nxt.valid()) {
+            nxt.load(buf_b);
+        }
+        consume(buf_a);
+        cur = nxt;
+        if (!cur.valid()) {
+            break;
+        }
+        nxt.advance();
+        if (nxt.valid()) {
+            nxt.load(buf_a);
+        }
+        consume(buf_b);
+        cur = nxt;
     }
 #pragma unroll
     for (int t = 0; t < T; ++t) {

@@ -1,202 +1,30 @@
 // Flat scan with fused per-query top-k (BruteForce::SearchWithRequest hot loop,
-// src/algorithm/bruteforce/bruteforce.cpp:481-597), batched over queries.
+// src/algorithm/bruteforce/bruteforce.cpp:481-597; FlattenDataCell::query,
+// src/datacell/flatten_datacell.h:334-440), batched over queries.
 //
-// Grid: x = query tile (T queries), y = chunk of code tiles.  A workgroup has up to four waves; wave w
-// walks tiles chunk_begin + w, + W, ... and keeps one LDS selector per query of the tile.  Workgroups
-// that are resident together have consecutive x and the same y, so they stream the same chunk of codes
-// at the same time and share it through each XCD's L2.  Every wave leaves its k best keys in a partial
-// buffer; a second kernel merges the partials of a query.
+// Work decomposition.  Grid x = query tile (T queries), y = chunk of code tiles.  A workgroup has up to
+// four waves; wave w walks tiles chunk_begin + w, + W, ... with the next granule group already in flight,
+// and keeps one LDS selector per query of the tile.  Workgroups that are resident together have
+// consecutive x and the same y, so they stream the same chunk of codes at about the same time.
+//
+// Selection.  Every (wave, query) has a selector in LDS (topk.h).  Chunks and waves of one query share a
+// per-query bound in global memory (the k-th best distance any of them has proven so far), so later
+// work drops almost everything with one compare.  Each (chunk, wave) leaves a short sorted list of
+// survivors; a merge kernel picks the k best per query.
 #include "distance.h"
 #include "store.h"
 #include "topk.h"
 
 namespace vsag_amd {
 
-// ------------------------------------------------------------------ query preparation
-// One workgroup (256 threads) per query row; rows >= nq are written as zeros so that a partly filled
-// query tile computes harmless values.
-__device__ inline float
-block_sum(float v, float* red) {
-    for (int off = 32; off > 0; off >>= 1) {
-        v += __shfl_down(v, off);
-    }
-    uint32_t wave = threadIdx.x >> 6;
-    if ((threadIdx.x & 63) == 0) {
-        red[wave] = v;
-    }
-    __syncthreads();
-    float s = 0;
-    for (uint32_t i = 0; i < (blockDim.x >> 6); ++i) {
-        s += red[i];
-    }
-    __syncthreads();
-    return s;
-}
+void timing_begin(hipStream_t st);
+void timing_end(hipStream_t st);
+int prepare_queries(const vsag_amd_store* s, const float* queries, uint64_t nq, uint64_t nq_pad, const QueryLayout& ql,
+                    uint32_t* qtab, float* qmeta, uint8_t* qcodes, hipStream_t st);
+ScanArgs make_scan_args(const vsag_amd_store* s, const QueryLayout& ql, const uint32_t* qtab, const float* qmeta);
+uint64_t rabitq_query_code_size(uint32_t dim, int metric, int query_bits);
 
-// fp32 / sq8 / sq4 tables (ProcessQueryImpl of fp32_quantizer.cpp:216-233 and scalar_quantizer.cpp:154-171
-// keep the query in fp32, normalised for cosine; the per-dimension constants are folded in here).
-__global__ void __launch_bounds__(256)
-prepare_float_queries(const float* q, uint64_t nq, uint32_t dim, int kind, int metric, const float* scale,
-                      const float* lb, float* qtab, uint32_t qstride, float* qmeta, uint32_t qmeta_stride) {
-    __shared__ float red[4];
-    uint64_t row = blockIdx.x;
-    float* out = qtab + row * qstride;
-    if (row >= nq) {
-        for (uint32_t d = threadIdx.x; d < qstride; d += blockDim.x) {
-            out[d] = 0.0F;
-        }
-        if (threadIdx.x < qmeta_stride) {
-            qmeta[row * qmeta_stride + threadIdx.x] = 0.0F;
-        }
-        return;
-    }
-    const float* src = q + row * dim;
-    float inv_norm = 1.0F;
-    bool cosine = metric == VSAG_AMD_METRIC_COSINE;
-    if (cosine) {
-        float s = 0;
-        for (uint32_t d = threadIdx.x; d < dim; d += blockDim.x) {
-            s += src[d] * src[d];
-        }
-        s = block_sum(s, red);
-        inv_norm = sqrtf(s);
-    }
-    float bias = 0;
-    for (uint32_t d = threadIdx.x; d < qstride; d += blockDim.x) {
-        float v = 0.0F;
-        if (d < dim) {
-            float x = cosine ? src[d] / inv_norm : src[d];
-            if (kind == VSAG_AMD_KIND_FP32) {
-                v = x;
-            } else if (metric == VSAG_AMD_METRIC_L2) {
-                v = x - lb[d];
-            } else {
-                v = x * scale[d];
-                bias += x * lb[d];
-            }
-        }
-        out[d] = v;
-    }
-    if (kind != VSAG_AMD_KIND_FP32 && metric != VSAG_AMD_METRIC_L2) {
-        bias = block_sum(bias, red);
-        if (threadIdx.x == 0) {
-            qmeta[row * qmeta_stride] = bias;
-        }
-    } else if (threadIdx.x < qmeta_stride) {
-        qmeta[row * qmeta_stride + threadIdx.x] = 0.0F;
-    }
-}
-
-// Uniform kinds: the query has been encoded with the base encoder (ProcessQueryImpl = EncodeOneImpl,
-// sq4_uniform_quantizer.cpp:204-215, sq8_uniform_quantizer.cpp:178-190); split it into the dwords the
-// scan consumes.  meta_off = byte offset of the query's norm (u64, L2) or sum (f32, IP / cosine).
-__global__ void __launch_bounds__(256)
-prepare_uniform_queries(const uint8_t* qcodes, uint64_t nq, uint32_t code_size, uint32_t payload, int bits,
-                        uint32_t meta_off, int meta_u64, uint32_t ndw, uint32_t* qtab, uint32_t qstride,
-                        float* qmeta, uint32_t qmeta_stride) {
-    uint64_t row = blockIdx.x;
-    uint32_t* out = qtab + row * qstride;
-    if (row >= nq) {
-        for (uint32_t d = threadIdx.x; d < qstride; d += blockDim.x) {
-            out[d] = 0;
-        }
-        if (threadIdx.x < qmeta_stride) {
-            qmeta[row * qmeta_stride + threadIdx.x] = 0.0F;
-        }
-        return;
-    }
-    const uint8_t* c = qcodes + row * code_size;
-    for (uint32_t w = threadIdx.x; w < ndw; w += blockDim.x) {
-        uint32_t v = 0;
-        for (uint32_t b = 0; b < 4; ++b) {
-            uint32_t idx = 4 * w + b;
-            if (idx < payload) {
-                v |= static_cast<uint32_t>(c[idx]) << (8 * b);
-            }
-        }
-        if (bits == 4) {
-            out[2 * w] = v & 0x0F0F0F0FU;
-            out[2 * w + 1] = (v >> 4) & 0x0F0F0F0FU;
-        } else {
-            out[w] = v;
-        }
-    }
-    if (threadIdx.x == 0) {
-        float m;
-        if (meta_u64) {
-            uint64_t nrm = 0;
-            for (int b = 0; b < 8; ++b) {
-                nrm |= static_cast<uint64_t>(c[meta_off + b]) << (8 * b);
-            }
-            m = static_cast<float>(nrm);
-        } else {
-            uint32_t u = 0;
-            for (int b = 0; b < 4; ++b) {
-                u |= static_cast<uint32_t>(c[meta_off + b]) << (8 * b);
-            }
-            m = __uint_as_float(u);
-        }
-        qmeta[row * qmeta_stride] = m;
-        for (uint32_t i = 1; i < qmeta_stride; ++i) {
-            qmeta[row * qmeta_stride + i] = 0.0F;
-        }
-    }
-}
-
-// RaBitQ: processed queries in the reference layout (four planes aligned_dim/8 bytes apart, then lb,
-// delta, code sum, norm, raw norm: rabitq_quantizer.cpp:135-176) -> plane-interleaved dwords + the
-// per-query factors of recover_dist_between_sq4u_and_fp32 (rabitq_quantizer.cpp:924-939).
-__global__ void __launch_bounds__(256)
-prepare_rabitq_queries(const uint8_t* qcodes, uint64_t nq, uint32_t qcode_size, uint32_t plane_bytes, uint32_t dim,
-                       int has_raw_norm, uint32_t ndw, uint32_t* qtab, uint32_t qstride, float* qmeta,
-                       uint32_t qmeta_stride) {
-    uint64_t row = blockIdx.x;
-    uint32_t* out = qtab + row * qstride;
-    if (row >= nq) {
-        for (uint32_t d = threadIdx.x; d < qstride; d += blockDim.x) {
-            out[d] = 0;
-        }
-        if (threadIdx.x < qmeta_stride) {
-            qmeta[row * qmeta_stride + threadIdx.x] = 0.0F;
-        }
-        return;
-    }
-    const uint8_t* c = qcodes + row * qcode_size;
-    uint32_t code_bytes = (dim + 7) / 8;
-    for (uint32_t i = threadIdx.x; i < ndw * 4; i += blockDim.x) {
-        uint32_t w = i >> 2, b = i & 3;
-        uint32_t v = 0;
-        for (uint32_t k = 0; k < 4; ++k) {
-            uint32_t idx = 4 * w + k;
-            if (idx < code_bytes) {
-                v |= static_cast<uint32_t>(c[b * plane_bytes + idx]) << (8 * k);
-            }
-        }
-        out[i] = v;
-    }
-    if (threadIdx.x == 0) {
-        const uint8_t* tail = c + 4 * static_cast<uint64_t>(plane_bytes);
-        auto rd = [&](uint32_t off) {
-            uint32_t u = 0;
-            for (int b = 0; b < 4; ++b) {
-                u |= static_cast<uint32_t>(tail[off + b]) << (8 * b);
-            }
-            return __uint_as_float(u);
-        };
-        float lb = rd(0), delta = rd(4), qsum = rd(8), qnorm = rd(12);
-        float qraw = has_raw_norm ? rd(16) : 0.0F;
-        float inv_sqrt_d = 1.0F / sqrtf(static_cast<float>(dim));
-        float* m = qmeta + row * qmeta_stride;
-        m[0] = inv_sqrt_d * delta * 2;
-        m[1] = inv_sqrt_d * lb * 2;
-        m[2] = inv_sqrt_d * delta * qsum;
-        m[3] = inv_sqrt_d * lb * static_cast<float>(dim);
-        m[4] = qnorm;
-        m[5] = qraw;
-        m[6] = 0;
-        m[7] = 0;
-    }
-}
+constexpr uint32_t kMaxWaves = 4;
 
 __global__ void
 fill_words_kernel(uint32_t* p, uint32_t v, uint64_t n) {
@@ -206,7 +34,6 @@ fill_words_kernel(uint32_t* p, uint32_t v, uint64_t n) {
     }
 }
 
-// ------------------------------------------------------------------ flat scan
 struct FlatArgs {
     uint64_t n;
     uint64_t ntiles;
@@ -214,8 +41,10 @@ struct FlatArgs {
     uint64_t nq;
     uint32_t k;
     uint32_t S;
-    uint32_t nslots;   // partial lists per query = chunks * waves
-    uint64_t* partial; // nq x nslots x k keys
+    uint32_t nslots;        // partial lists per query = chunks * waves
+    uint32_t* bound;        // per query: ordered distance that k candidates are known to reach
+    uint64_t* partial;      // nq x nslots x k keys
+    uint32_t* partial_cnt;  // nq x nslots
 };
 
 template <int KIND, int METRIC, int T>
@@ -229,82 +58,152 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
     uint64_t* sel = lds + static_cast<size_t>(wave) * T * S;
 
     uint32_t qidx[T];
+    uint32_t thr[T];  // a candidate passes when its ordered distance is below thr
+    uint32_t cnt[T];
 #pragma unroll
     for (int t = 0; t < T; ++t) {
         qidx[t] = blockIdx.x * T + t;
+        cnt[t] = 0;
+        uint32_t bs = qidx[t] < f.nq ? __builtin_amdgcn_readfirstlane(__atomic_load_n(&f.bound[qidx[t]], __ATOMIC_RELAXED))
+                                     : 0xFFFFFFFFU;
+        thr[t] = bs == 0xFFFFFFFFU ? bs : bs + 1;
     }
     for (uint32_t i = lane; i < T * S; i += kWave) {
         sel[i] = kInfKey;
     }
     wave_lds_fence();
 
-    uint32_t cnt[T];
-    float tau[T];
-    bool open[T];
-#pragma unroll
-    for (int t = 0; t < T; ++t) {
-        cnt[t] = 0;
-        tau[t] = __builtin_inff();
-        open[t] = true;
-    }
-
     const uint64_t tile_begin = static_cast<uint64_t>(blockIdx.y) * f.tiles_per_chunk;
     uint64_t tile_end = tile_begin + f.tiles_per_chunk;
     if (tile_end > f.ntiles) {
         tile_end = f.ntiles;
     }
-    for (uint64_t tile = tile_begin + wave; tile < tile_end; tile += nwaves) {
+    // Software pipeline over granule groups: the loads of group g+1 (possibly of the next tile) are
+    // issued before group g is consumed, so every wave keeps kGroup KiB in flight.  Two register buffers
+    // alternate; the loop body is written out twice so that both are addressed statically.
+    const QueryRows<T> qrows = query_rows<T>(a, qidx);
+    TileStream cur{a.tiles + lane, tile_begin + wave, tile_end, nwaves, 0, a.G};
+    TileStream nxt = cur;
+    uint4 buf_a[kGroup], buf_b[kGroup];
+    if (cur.valid()) {
+        cur.load(buf_a);
+    }
+    Acc<KIND, T> acc;
+    acc_reset(acc);
+
+    auto consume = [&](const uint4(&regs)[kGroup]) {
+#pragma unroll
+        for (int u = 0; u < kGroup; ++u) {
+            if (cur.j0 + u < a.G) {
+                accumulate_granule<KIND, METRIC, T>(a, qrows, cur.j0 + u, regs[u], acc);
+            }
+        }
+        if (cur.j0 + kGroup < a.G) {
+            return;
+        }
+        const uint64_t id = cur.tile * kWave + lane;
         float d[T];
-        tile_distances<KIND, METRIC, T>(a, tile, qidx, lane, d);
-        const uint64_t id = tile * kWave + lane;
+        finish_distances<KIND, METRIC, T>(a, qidx, id, acc, d);
+        acc_reset(acc);
         const bool valid = id < f.n;
 #pragma unroll
         for (int t = 0; t < T; ++t) {
-            // Inner ids grow along the scan, so `d < tau` is the (distance, id) order exactly.
-            bool pass = valid && (open[t] || d[t] < tau[t]);
+            // Inner ids grow along the scan, so "ordered distance < thr" is exactly the (distance, id)
+            // order against the wave's own k-th key, and "<= bound" against the shared bound.
+            uint32_t od = float_to_ordered(d[t]);
+            bool pass = valid && od < thr[t];
             uint64_t* keys = sel + t * S;
-            cnt[t] = selector_append(keys, k, cnt[t], pass, make_key(d[t], static_cast<uint32_t>(id)));
+            cnt[t] = selector_append(keys, k, cnt[t], pass,
+                                     (static_cast<uint64_t>(od) << 32) | static_cast<uint32_t>(id));
             if (cnt[t] + kWave > S - k) {
                 uint64_t th = selector_flush(keys, S, k, cnt[t], lane);
                 cnt[t] = 0;
-                open[t] = th == kInfKey;
-                tau[t] = open[t] ? __builtin_inff() : ordered_to_float(static_cast<uint32_t>(th >> 32));
+                uint32_t tl = static_cast<uint32_t>(th >> 32);  // 0xFFFFFFFF while fewer than k seen
+                uint32_t bs = 0xFFFFFFFFU;
+                if (qidx[t] < f.nq) {
+                    if (th != kInfKey) {
+                        uint32_t old = lane == 0 ? atomicMin(&f.bound[qidx[t]], tl) : 0U;
+                        bs = __builtin_amdgcn_readfirstlane(old);
+                    } else {
+                        bs = __builtin_amdgcn_readfirstlane(__atomic_load_n(&f.bound[qidx[t]], __ATOMIC_RELAXED));
+                    }
+                }
+                uint32_t tb = bs == 0xFFFFFFFFU ? bs : bs + 1;
+                thr[t] = tl < tb ? tl : tb;
             }
         }
+    };
+
+    while (cur.valid()) {
+        nxt.advance();
+        if (nxt.valid()) {
+            nxt.load(buf_b);
+        }
+        consume(buf_a);
+        cur = nxt;
+        if (!cur.valid()) {
+            break;
+        }
+        nxt.advance();
+        if (nxt.valid()) {
+            nxt.load(buf_a);
+        }
+        consume(buf_b);
+        cur = nxt;
     }
+
     const uint32_t slot = blockIdx.y * nwaves + wave;
 #pragma unroll
     for (int t = 0; t < T; ++t) {
+        if (qidx[t] >= f.nq) {
+            continue;
+        }
         uint64_t* keys = sel + t * S;
-        selector_flush(keys, S, k, cnt[t], lane);
-        if (qidx[t] < f.nq) {
-            uint64_t* dst = f.partial + (static_cast<uint64_t>(qidx[t]) * f.nslots + slot) * k;
-            for (uint32_t i = lane; i < k; i += kWave) {
-                dst[i] = keys[i];
+        uint64_t th = selector_flush(keys, S, k, cnt[t], lane);
+        if (th != kInfKey && lane == 0) {
+            atomicMin(&f.bound[qidx[t]], static_cast<uint32_t>(th >> 32));
+        }
+        const uint64_t list = static_cast<uint64_t>(qidx[t]) * f.nslots + slot;
+        uint64_t* dst = f.partial + list * k;
+        uint32_t valid_count = 0;
+        for (uint32_t i0 = 0; i0 < k; i0 += kWave) {
+            uint32_t i = i0 + lane;
+            uint64_t key = i < k ? keys[i] : kInfKey;
+            bool ok = key != kInfKey;
+            if (ok) {
+                dst[i] = key;
             }
+            valid_count += __popcll(__ballot(ok));
+        }
+        if (lane == 0) {
+            f.partial_cnt[list] = valid_count;
         }
     }
 }
 
-// One wave per query: k best keys of `count` partial keys, written as ids / distances (ascending).
+// One wave per query: the k best keys over its partial lists, written as ids / distances (ascending).
 __global__ void __launch_bounds__(64)
-merge_partials_kernel(const uint64_t* partial, uint64_t per_query, uint32_t k, uint32_t S, uint32_t* ids,
-                      float* dists) {
+merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, uint32_t nslots, uint32_t k, uint32_t S,
+                      uint32_t* ids, float* dists) {
     extern __shared__ uint64_t lds[];
     const uint32_t lane = threadIdx.x;
     const uint64_t q = blockIdx.x;
     selector_init(lds, S, lane);
-    const uint64_t* src = partial + q * per_query;
     uint32_t cnt = 0;
     uint64_t tau = kInfKey;
-    for (uint64_t base = 0; base < per_query; base += kWave) {
-        uint64_t idx = base + lane;
-        uint64_t key = idx < per_query ? src[idx] : kInfKey;
-        bool pass = key < tau;
-        cnt = selector_append(lds, k, cnt, pass, key);
-        if (cnt + kWave > S - k) {
-            tau = selector_flush(lds, S, k, cnt, lane);
-            cnt = 0;
+    for (uint32_t slot = 0; slot < nslots; ++slot) {
+        const uint64_t list = q * nslots + slot;
+        const uint32_t c = as_const(partial_cnt)[list];
+        const uint64_t* src = partial + list * k;
+        for (uint32_t base = 0; base < c; base += kWave) {
+            uint32_t i = base + lane;
+            uint64_t key = i < c ? src[i] : kInfKey;
+            bool pass = key < tau;
+            cnt = selector_append(lds, k, cnt, pass, key);
+            if (cnt + kWave > S - k) {
+                tau = selector_flush(lds, S, k, cnt, lane);
+                cnt = 0;
+            }
         }
     }
     selector_flush(lds, S, k, cnt, lane);
@@ -327,115 +226,73 @@ static thread_local int tl_last_tile = 0;
 static thread_local uint64_t tl_last_passes = 0;
 static thread_local uint64_t tl_last_bytes = 0;
 
-QueryLayout
-query_layout(const vsag_amd_store* s) {
-    QueryLayout l{};
-    uint32_t ndw = s->G * 4;
-    switch (s->kind) {
-        case VSAG_AMD_KIND_FP32:
-            l.qstride = s->dpad;
-            l.qmeta = 1;
-            break;
-        case VSAG_AMD_KIND_SQ8:
-        case VSAG_AMD_KIND_SQ4:
-            l.qstride = s->dpad;
-            l.qmeta = 1;
-            break;
-        case VSAG_AMD_KIND_SQ4_UNIFORM:
-            l.qstride = ndw * 2;
-            l.qmeta = 1;
-            break;
-        case VSAG_AMD_KIND_SQ8_UNIFORM:
-            l.qstride = ndw;
-            l.qmeta = 1;
-            break;
-        case VSAG_AMD_KIND_RABITQ:
-            l.qstride = ndw * 4;
-            l.qmeta = 8;
-            break;
-    }
-    // Rows start on a 64-byte boundary so that scalar dwordx16 loads stay aligned.
-    l.qstride = static_cast<uint32_t>(round_up(l.qstride, 16));
-    return l;
-}
-
-// Largest query tile the kind supports without spilling SGPRs / registers.
+// Queries per wave.  More queries per pass means fewer passes over the codes but more scalar registers;
+// these are the largest tiles that still compile without spilling.
 static int
-default_query_tile(const vsag_amd_store* s, uint64_t nq) {
-    int t;
+default_query_tile(const vsag_amd_store* s) {
     switch (s->kind) {
-        case VSAG_AMD_KIND_FP32:
-            t = 4;
-            break;
         case VSAG_AMD_KIND_SQ8:
         case VSAG_AMD_KIND_SQ4:
-            t = s->metric == VSAG_AMD_METRIC_L2 ? 2 : 4;
-            break;
+            return 4;
         case VSAG_AMD_KIND_RABITQ:
-            t = 2;
-            break;
+            return 2;
         default:
-            t = 4;
+            return 4;
     }
-    while (t > 1 && static_cast<uint64_t>(t) > nq) {
-        t >>= 1;
-    }
-    return t;
 }
 
 struct ScanPlan {
     int T;
     uint32_t S;
     uint32_t waves;
+    uint64_t groups;     // grid x
     uint64_t nq_pad;
-    uint64_t chunks;
+    uint64_t chunks;     // grid y
     uint64_t tiles_per_chunk;
-    uint32_t nslots;
+    size_t lds_bytes;
     QueryLayout ql;
     size_t qcode_bytes;  // staging for encoded queries (uniform kinds, rabitq)
 };
 
-uint64_t rabitq_query_code_size(uint32_t dim, int metric, int query_bits);
-
-static int
+static void
 make_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, uint64_t ntiles, ScanPlan* p) {
-    p->T = g_tile_override > 0 ? g_tile_override : default_query_tile(s, nq);
     p->S = selector_slots(k);
-    // Selectors of one workgroup must fit 64 KiB of LDS.
-    while (p->T > 1 && static_cast<size_t>(p->T) * p->S * 8 > 65536) {
-        p->T >>= 1;
+    int T = g_tile_override > 0 ? g_tile_override : default_query_tile(s);
+    while (T > 1 && static_cast<uint64_t>(T) > nq) {
+        T >>= 1;
     }
-    uint32_t waves = 4;
-    while (waves > 1 && static_cast<size_t>(waves) * p->T * p->S * 8 > 65536) {
+    const size_t lds_budget = 65536;
+    while (T > 1 && static_cast<size_t>(T) * p->S * 8 > lds_budget) {
+        T >>= 1;
+    }
+    uint32_t waves = kMaxWaves;
+    while (waves > 1 && static_cast<size_t>(waves) * T * p->S * 8 > lds_budget) {
         waves >>= 1;
     }
+    p->T = T;
     p->waves = waves;
-    p->nq_pad = round_up(nq, p->T);
-    uint64_t qtiles = p->nq_pad / p->T;
+    p->lds_bytes = static_cast<size_t>(waves) * T * p->S * 8;
+    p->groups = div_up(nq, static_cast<uint64_t>(T));
+    p->nq_pad = p->groups * T;
     uint64_t chunks;
     if (g_chunk_override > 0) {
         chunks = g_chunk_override;
     } else {
-        // Enough workgroups for about eight rounds over the machine, but at least 16 tiles per wave.
-        uint64_t target = static_cast<uint64_t>(device_cu_count()) * 8 * 8;
-        chunks = div_up(target, qtiles);
+        // About eight rounds of workgroups over the machine (eight workgroups fit a CU).
+        chunks = div_up(static_cast<uint64_t>(device_cu_count()) * 8 * 8, p->groups);
     }
-    uint64_t max_chunks = ntiles / (16 * waves);
+    uint64_t max_chunks = ntiles / (16 * waves);  // at least 16 tiles per wave
     if (max_chunks < 1) {
         max_chunks = 1;
     }
     if (chunks > max_chunks) {
         chunks = max_chunks;
     }
-    if (chunks < 1) {
-        chunks = 1;
-    }
     if (chunks > 65535) {
         chunks = 65535;
     }
     p->tiles_per_chunk = div_up(ntiles > 0 ? ntiles : 1, chunks);
     p->chunks = div_up(ntiles > 0 ? ntiles : 1, p->tiles_per_chunk);
-    p->nslots = static_cast<uint32_t>(p->chunks * waves);
     p->ql = query_layout(s);
     p->qcode_bytes = 0;
     if (s->kind == VSAG_AMD_KIND_SQ4_UNIFORM || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
@@ -443,88 +300,26 @@ make_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, uint64_t ntiles, Sca
     } else if (s->kind == VSAG_AMD_KIND_RABITQ) {
         p->qcode_bytes = nq * rabitq_query_code_size(s->dim, s->metric, s->query_bits);
     }
-    return 0;
 }
 
 struct ScanBuffers {
     uint32_t* qtab;
     float* qmeta;
     uint8_t* qcodes;
+    uint32_t* bound;
+    uint32_t* partial_cnt;
     uint64_t* partial;
 };
 
 static size_t
-carve_scan(Carver& c, const ScanPlan& p, uint64_t partial_keys, ScanBuffers* b) {
+carve_scan(Carver& c, const ScanPlan& p, uint64_t nq, uint32_t k, ScanBuffers* b) {
     b->qtab = c.take<uint32_t>(p.nq_pad * p.ql.qstride);
     b->qmeta = c.take<float>(p.nq_pad * p.ql.qmeta);
     b->qcodes = c.take<uint8_t>(p.qcode_bytes);
-    b->partial = c.take<uint64_t>(partial_keys);
+    b->bound = c.take<uint32_t>(nq);
+    b->partial_cnt = c.take<uint32_t>(nq * p.chunks * p.waves);
+    b->partial = c.take<uint64_t>(nq * p.chunks * p.waves * k);
     return c.used;
-}
-
-void timing_begin(hipStream_t st);
-void timing_end(hipStream_t st);
-int squ_encode_launch(const float* x, uint64_t n, uint32_t dim, int bits, int metric, const float* bounds,
-                      uint8_t* codes, hipStream_t st);
-int rabitq_process_query_launch(const float* q, uint64_t nq, uint32_t dim, const float* rot, const float* centroid,
-                                int metric, int query_bits, uint8_t* qcodes, hipStream_t st);
-
-// Runs ProcessQueryImpl of the store's quantizer for nq raw queries and fills the scan tables.
-int
-prepare_queries(const vsag_amd_store* s, const float* queries, uint64_t nq, uint64_t nq_pad, const QueryLayout& ql,
-                uint32_t* qtab, float* qmeta, uint8_t* qcodes, hipStream_t st) {
-    dim3 grid(static_cast<uint32_t>(nq_pad));
-    switch (s->kind) {
-        case VSAG_AMD_KIND_FP32:
-        case VSAG_AMD_KIND_SQ8:
-        case VSAG_AMD_KIND_SQ4:
-            hipLaunchKernelGGL(prepare_float_queries, grid, dim3(256), 0, st, queries, nq, s->dim, s->kind, s->metric,
-                               s->scale_dev, s->lb_dev, reinterpret_cast<float*>(qtab), ql.qstride, qmeta, ql.qmeta);
-            break;
-        case VSAG_AMD_KIND_SQ4_UNIFORM:
-        case VSAG_AMD_KIND_SQ8_UNIFORM: {
-            int bits = s->kind == VSAG_AMD_KIND_SQ4_UNIFORM ? 4 : 8;
-            VA_TRY(squ_encode_launch(queries, nq, s->dim, bits, s->metric, s->bounds_dev, qcodes, st));
-            hipLaunchKernelGGL(prepare_uniform_queries, grid, dim3(256), 0, st, qcodes, nq, s->code_size,
-                               s->payload_bytes, bits, s->meta_offset[0], static_cast<int>(s->meta_is_u64 & 1),
-                               s->G * 4, qtab, ql.qstride, qmeta, ql.qmeta);
-            break;
-        }
-        case VSAG_AMD_KIND_RABITQ: {
-            VA_CHECK_ARG(s->query_bits == 4, "rabitq scan supports 4-bit queries only");
-            VA_TRY(rabitq_process_query_launch(queries, nq, s->dim, s->rotation_dev, s->centroid_dev, s->metric,
-                                               s->query_bits, qcodes, st));
-            uint32_t aligned_dim = (s->dim + 511) / 512 * 512;
-            hipLaunchKernelGGL(prepare_rabitq_queries, grid, dim3(256), 0, st, qcodes, nq,
-                               static_cast<uint32_t>(rabitq_query_code_size(s->dim, s->metric, s->query_bits)),
-                               aligned_dim / 8, s->dim, s->metric != VSAG_AMD_METRIC_L2 ? 1 : 0, s->G * 4, qtab,
-                               ql.qstride, qmeta, ql.qmeta);
-            break;
-        }
-        default:
-            return fail(VSAG_AMD_INVALID_ARGUMENT, "unknown store kind %d", s->kind);
-    }
-    VA_HIP(hipGetLastError());
-    return 0;
-}
-
-ScanArgs
-make_scan_args(const vsag_amd_store* s, const QueryLayout& ql, const uint32_t* qtab, const float* qmeta) {
-    ScanArgs a{};
-    a.tiles = s->tiles;
-    a.meta = s->meta;
-    a.meta_stride = s->cap_tiles * kWave;
-    a.scale = s->scale_dev;
-    a.qtab = qtab;
-    a.qmeta = qmeta;
-    a.qstride = ql.qstride;
-    a.qmeta_stride = ql.qmeta;
-    a.G = s->G;
-    a.dim = s->dim;
-    a.f0 = s->ulb;
-    a.f1 = s->scalar_rate;
-    a.f2 = s->ulb * s->ulb;
-    return a;
 }
 
 template <int KIND, int METRIC>
@@ -562,9 +357,9 @@ launch_flat_m(int metric, int T, dim3 grid, dim3 block, size_t lds, hipStream_t 
 
 static int
 launch_flat(const vsag_amd_store* s, const ScanPlan& p, const ScanArgs& a, const FlatArgs& f, hipStream_t st) {
-    dim3 grid(static_cast<uint32_t>(p.nq_pad / p.T), static_cast<uint32_t>(p.chunks));
+    dim3 grid(static_cast<uint32_t>(p.groups), static_cast<uint32_t>(p.chunks));
     dim3 block(p.waves * kWave);
-    size_t lds = static_cast<size_t>(p.waves) * p.T * p.S * 8;
+    size_t lds = p.lds_bytes;
     switch (s->kind) {
         case VSAG_AMD_KIND_FP32:
             launch_flat_m<VSAG_AMD_KIND_FP32>(s->metric, p.T, grid, block, lds, st, a, f);
@@ -613,7 +408,7 @@ vsag_amd_flat_scan_workspace_bytes(const vsag_amd_store_t* s, uint64_t nq, uint3
     make_plan(s, nq, k, s->ntiles, &p);
     Carver c(nullptr, 0);
     ScanBuffers b;
-    return carve_scan(c, p, nq * p.nslots * k, &b) + 256;
+    return carve_scan(c, p, nq, k, &b) + 256;
 }
 
 extern "C" int
@@ -629,10 +424,12 @@ vsag_amd_flat_scan_topk(const vsag_amd_store_t* s, const float* queries_dev, uin
     make_plan(s, nq, k, s->ntiles, &p);
     Carver c(workspace_dev, workspace_bytes);
     ScanBuffers b;
-    carve_scan(c, p, nq * p.nslots * k, &b);
+    carve_scan(c, p, nq, k, &b);
     VA_CHECK_ARG(c.ok(), "workspace too small: need %zu bytes, got %zu", c.used, workspace_bytes);
 
     VA_TRY(prepare_queries(s, queries_dev, nq, p.nq_pad, p.ql, b.qtab, b.qmeta, b.qcodes, st));
+    hipLaunchKernelGGL(fill_words_kernel, dim3(static_cast<uint32_t>(div_up(nq, 256))), dim3(256), 0, st, b.bound,
+                       0xFFFFFFFFU, nq);
     ScanArgs a = make_scan_args(s, p.ql, b.qtab, b.qmeta);
     FlatArgs f{};
     f.n = s->n;
@@ -641,23 +438,24 @@ vsag_amd_flat_scan_topk(const vsag_amd_store_t* s, const float* queries_dev, uin
     f.nq = nq;
     f.k = k;
     f.S = p.S;
-    f.nslots = p.nslots;
+    f.nslots = static_cast<uint32_t>(p.chunks * p.waves);
+    f.bound = b.bound;
     f.partial = b.partial;
+    f.partial_cnt = b.partial_cnt;
     if (s->ntiles == 0) {
-        // Empty store: every slot of the partial buffer must still read as "no candidate".
-        uint64_t words = nq * p.nslots * k * 2;
-        hipLaunchKernelGGL(fill_words_kernel, dim3(static_cast<uint32_t>(div_up(words, 256))), dim3(256), 0, st,
-                           reinterpret_cast<uint32_t*>(b.partial), 0xFFFFFFFFU, words);
+        // Empty store: every partial list must still read as empty.
+        hipLaunchKernelGGL(fill_words_kernel, dim3(static_cast<uint32_t>(div_up(nq * f.nslots, 256))), dim3(256), 0,
+                           st, b.partial_cnt, 0U, nq * f.nslots);
     } else {
         timing_begin(st);
         VA_TRY(launch_flat(s, p, a, f, st));
         timing_end(st);
     }
     hipLaunchKernelGGL(merge_partials_kernel, dim3(static_cast<uint32_t>(nq)), dim3(kWave), p.S * 8, st, b.partial,
-                       static_cast<uint64_t>(p.nslots) * k, k, p.S, ids_dev, dists_dev);
+                       b.partial_cnt, f.nslots, k, p.S, ids_dev, dists_dev);
     VA_HIP(hipGetLastError());
     tl_last_tile = p.T;
-    tl_last_passes = p.nq_pad / p.T;
+    tl_last_passes = p.groups;
     tl_last_bytes = s->ntiles * s->G * kWave * kGranule;
     return 0;
 }

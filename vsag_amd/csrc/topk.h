@@ -1,7 +1,7 @@
 // Wave-level streaming top-k selector kept in LDS.
 //
 // One wavefront owns one selector per query it serves.  A selector is an array of S 64-bit keys
-// (S a power of two, S >= k + 128): slots [0,k) hold the best keys found so far, slots [k,k+cnt) hold
+// (S a power of two, S >= k + 96): slots [0,k) hold the best keys found so far, slots [k,k+cnt) hold
 // pending candidates that passed the current threshold.  When the pending region could overflow on the
 // next 64-wide append, the wave sorts the whole array (bitonic, in LDS) which leaves the k best in
 // front and yields the new threshold keys[k-1].  No workgroup barrier is involved: only the owning
@@ -45,8 +45,8 @@ wave_uniform_u64(uint64_t v) {
 // Selector size for a given k.
 __host__ __device__ inline uint32_t
 selector_slots(uint32_t k) {
-    uint32_t s = 256;
-    while (s < k + 128) {
+    uint32_t s = 128;
+    while (s < k + 96) {
         s <<= 1;
     }
     return s;
