@@ -21,6 +21,9 @@
 extern "C" {
 #endif
 
+/* Exported entry points; everything else in the library has hidden visibility. */
+#define VSAG_AMD_API __attribute__((visibility("default")))
+
 #define VSAG_AMD_SUCCESS 0
 #define VSAG_AMD_UNKNOWN_ERROR (-1)
 #define VSAG_AMD_INTERNAL_ERROR (-2)
@@ -55,21 +58,21 @@ extern "C" {
 
 /* Selects `device`, checks that it is a gfx950 part and that the library's code object loads.
  * Fails (VSAG_AMD_INTERNAL_ERROR) when there is no usable GPU: there is no CPU fallback. */
-int vsag_amd_init(int device);
-const char* vsag_amd_last_error(void);
+VSAG_AMD_API int vsag_amd_init(int device);
+VSAG_AMD_API const char* vsag_amd_last_error(void);
 /* Name of the device selected by vsag_amd_init, its CU count and memory (bytes). */
-int vsag_amd_device_info(char* name, size_t name_bytes, int* compute_units, uint64_t* hbm_bytes);
+VSAG_AMD_API int vsag_amd_device_info(char* name, size_t name_bytes, int* compute_units, uint64_t* hbm_bytes);
 
 /* Thin wrappers over hipMalloc / hipFree / hipMemcpyAsync / hipStreamSynchronize so that a host
  * with no HIP headers (cgo, ctypes, a C++ index class) can own device buffers.  The two copies that
  * touch host memory return after the copy has finished; d2d and memset are asynchronous. */
-int vsag_amd_malloc(void** ptr_dev, size_t bytes);
-int vsag_amd_free(void* ptr_dev);
-int vsag_amd_memcpy_h2d(void* dst_dev, const void* src, size_t bytes, void* stream);
-int vsag_amd_memcpy_d2h(void* dst, const void* src_dev, size_t bytes, void* stream);
-int vsag_amd_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
-int vsag_amd_memset(void* dst_dev, int value, size_t bytes, void* stream);
-int vsag_amd_stream_synchronize(void* stream);
+VSAG_AMD_API int vsag_amd_malloc(void** ptr_dev, size_t bytes);
+VSAG_AMD_API int vsag_amd_free(void* ptr_dev);
+VSAG_AMD_API int vsag_amd_memcpy_h2d(void* dst_dev, const void* src, size_t bytes, void* stream);
+VSAG_AMD_API int vsag_amd_memcpy_d2h(void* dst, const void* src_dev, size_t bytes, void* stream);
+VSAG_AMD_API int vsag_amd_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
+VSAG_AMD_API int vsag_amd_memset(void* dst_dev, int value, size_t bytes, void* stream);
+VSAG_AMD_API int vsag_amd_stream_synchronize(void* stream);
 
 /* ------------------------------------------------------------------ quantizer training ------- */
 
@@ -78,15 +81,15 @@ int vsag_amd_stream_synchronize(void* stream);
  * and diff = upper - lower from at most max_sample (0 = 100000) strided sample rows.  TRUNC_BOUND keeps
  * the ignore_count-th largest / smallest value per dimension; cosine normalises the sample rows first.
  * bits = 8 or 4.  Workspace: vsag_amd_sq_train_workspace_bytes(). */
-size_t vsag_amd_sq_train_workspace_bytes(uint64_t n, uint32_t dim, uint64_t max_sample);
-int vsag_amd_sq_train(const float* x_dev, uint64_t n, uint32_t dim, int bits, int metric, int mode,
+VSAG_AMD_API size_t vsag_amd_sq_train_workspace_bytes(uint64_t n, uint32_t dim, uint64_t max_sample);
+VSAG_AMD_API int vsag_amd_sq_train(const float* x_dev, uint64_t n, uint32_t dim, int bits, int metric, int mode,
                       float trunc_rate, uint64_t max_sample, float* lower_bound_dev, float* diff_dev,
                       void* workspace_dev, size_t workspace_bytes, void* stream);
 
 /* ScalarQuantizationTrainer::TrainUniform + SQ4UniformQuantizer::TrainImpl / SQ8UniformQuantizer::
  * TrainImpl (scalar_quantization_trainer.cpp:47-70; sq4_uniform_quantizer.cpp:86-108;
  * sq8_uniform_quantizer.cpp:76-98).  Writes two floats: out_dev[0] = lower bound, out_dev[1] = diff. */
-int vsag_amd_sq_train_uniform(const float* x_dev, uint64_t n, uint32_t dim, int bits, int metric,
+VSAG_AMD_API int vsag_amd_sq_train_uniform(const float* x_dev, uint64_t n, uint32_t dim, int bits, int metric,
                               int mode, float trunc_rate, uint64_t max_sample, float* out_dev,
                               void* workspace_dev, size_t workspace_bytes, void* stream);
 
@@ -95,11 +98,11 @@ int vsag_amd_sq_train_uniform(const float* x_dev, uint64_t n, uint32_t dim, int 
 /* Bytes per code in the reference's layout (Quantizer::GetCodeSize): fp32 4*dim; sq8 dim; sq4
  * ceil(dim/2) (scalar_quantizer.cpp:28-36); uniform kinds sq4_uniform_quantizer.cpp:33-72 and
  * sq8_uniform_quantizer.cpp:30-62; rabitq 1-bit base rabitq_quantizer.cpp:102-133. */
-uint64_t vsag_amd_code_size(int kind, int metric, uint32_t dim, int rabitq_query_bits);
+VSAG_AMD_API uint64_t vsag_amd_code_size(int kind, int metric, uint32_t dim, int rabitq_query_bits);
 
 /* ScalarQuantizer::EncodeBatch (scalar_quantizer.cpp:85-112): fp32 rows -> sq8 / sq4 codes in the
  * reference byte layout, n x code_size.  Cosine normalises each row first. */
-int vsag_amd_sq_encode(const float* x_dev, uint64_t n, uint32_t dim, int bits, int metric,
+VSAG_AMD_API int vsag_amd_sq_encode(const float* x_dev, uint64_t n, uint32_t dim, int bits, int metric,
                        const float* lower_bound_dev, const float* diff_dev, uint8_t* codes_dev,
                        void* stream);
 
@@ -107,22 +110,22 @@ int vsag_amd_sq_encode(const float* x_dev, uint64_t n, uint32_t dim, int bits, i
  * (sq4_uniform_quantizer.cpp:110-152, sq8_uniform_quantizer.cpp:100-132): codes plus the trailing
  * u64 sum of squared codes (L2) or f32 sums (IP / cosine).  bounds_dev = {lower bound, diff}.
  * Also used for queries (ProcessQueryImpl encodes the query with the same routine). */
-int vsag_amd_squ_encode(const float* x_dev, uint64_t n, uint32_t dim, int bits, int metric,
+VSAG_AMD_API int vsag_amd_squ_encode(const float* x_dev, uint64_t n, uint32_t dim, int bits, int metric,
                         const float* bounds_dev, uint8_t* codes_dev, void* stream);
 
 /* RaBitQuantizer::TrainImpl (rabitq_quantizer.cpp:209-254) with the rotation supplied by the caller
  * (row-major dim x dim, y = R x): centroid = R * mean(x). */
-int vsag_amd_rabitq_train(const float* x_dev, uint64_t n, uint32_t dim, const float* rotation_dev,
+VSAG_AMD_API int vsag_amd_rabitq_train(const float* x_dev, uint64_t n, uint32_t dim, const float* rotation_dev,
                           float* centroid_dev, void* stream);
 /* RaBitQuantizer::EncodeOneInternal, 1-bit base (rabitq_quantizer.cpp:724-856): n x code_size codes
  * [bits | norm | error | sum (query_bits != 32) | raw norm (ip, cosine)]. */
-int vsag_amd_rabitq_encode(const float* x_dev, uint64_t n, uint32_t dim, const float* rotation_dev,
+VSAG_AMD_API int vsag_amd_rabitq_encode(const float* x_dev, uint64_t n, uint32_t dim, const float* rotation_dev,
                            const float* centroid_dev, int metric, int query_bits, uint8_t* codes_dev,
                            void* stream);
 /* RaBitQuantizer::ProcessQueryImpl (rabitq_quantizer.cpp:2130-2217): nq x query_code_size processed
  * queries (4-bit: four bit planes of aligned_dim/8 bytes, lb, delta, code sum, norm, raw norm). */
-uint64_t vsag_amd_rabitq_query_code_size(uint32_t dim, int metric, int query_bits);
-int vsag_amd_rabitq_process_query(const float* q_dev, uint64_t nq, uint32_t dim,
+VSAG_AMD_API uint64_t vsag_amd_rabitq_query_code_size(uint32_t dim, int metric, int query_bits);
+VSAG_AMD_API int vsag_amd_rabitq_process_query(const float* q_dev, uint64_t nq, uint32_t dim,
                                   const float* rotation_dev, const float* centroid_dev, int metric,
                                   int query_bits, uint8_t* qcodes_dev, void* stream);
 
@@ -145,23 +148,23 @@ typedef struct vsag_amd_store_params {
     int rabitq_query_bits;        /* rabitq: 4 or 32 (only 4 is scanned on the device). */
 } vsag_amd_store_params_t;
 
-int vsag_amd_store_create(const vsag_amd_store_params_t* params, vsag_amd_store_t** store);
-int vsag_amd_store_destroy(vsag_amd_store_t* store);
-uint64_t vsag_amd_store_size(const vsag_amd_store_t* store);
+VSAG_AMD_API int vsag_amd_store_create(const vsag_amd_store_params_t* params, vsag_amd_store_t** store);
+VSAG_AMD_API int vsag_amd_store_destroy(vsag_amd_store_t* store);
+VSAG_AMD_API uint64_t vsag_amd_store_size(const vsag_amd_store_t* store);
 
 /* FlattenDataCell::BatchInsertVector (flatten_datacell.h:279-314): append n codes given in the
  * reference byte layout (n x code_size, device memory); inner ids continue from the current size.
  * Synchronises `stream` when the store has to grow. */
-int vsag_amd_store_append(vsag_amd_store_t* store, const uint8_t* codes_dev, uint64_t n, void* stream);
+VSAG_AMD_API int vsag_amd_store_append(vsag_amd_store_t* store, const uint8_t* codes_dev, uint64_t n, void* stream);
 
 /* Posting-list form (BucketDataCell, bucket_datacell.h:670-709 + IVF::Add, ivf.cpp:590-724): codes in
  * the reference byte layout in inner-id order plus one bucket label per code.  Lists are laid out
  * contiguously, each padded to whole tiles, in stable (input) order inside a bucket.  Replaces any
  * previous content. */
-int vsag_amd_store_set_lists(vsag_amd_store_t* store, const uint8_t* codes_dev, const int32_t* labels_dev,
+VSAG_AMD_API int vsag_amd_store_set_lists(vsag_amd_store_t* store, const uint8_t* codes_dev, const int32_t* labels_dev,
                              uint64_t n, uint32_t nlist, void* stream);
 /* Sizes of the posting lists (nlist values) copied to host memory. */
-int vsag_amd_store_list_sizes(const vsag_amd_store_t* store, uint32_t* sizes, uint32_t nlist);
+VSAG_AMD_API int vsag_amd_store_list_sizes(const vsag_amd_store_t* store, uint32_t* sizes, uint32_t nlist);
 
 /* ------------------------------------------------------------------ flat scan + top-k -------- */
 
@@ -170,44 +173,44 @@ int vsag_amd_store_list_sizes(const vsag_amd_store_t* store, uint32_t* sizes, ui
  * queries.  queries_dev: nq x dim fp32 raw queries (the library applies ProcessQueryImpl of the store's
  * quantizer itself).  Output: nq x k inner ids / distances, ascending by (distance, id); rows shorter
  * than k are padded with VSAG_AMD_INVALID_ID / +inf.  1 <= k <= 1024. */
-size_t vsag_amd_flat_scan_workspace_bytes(const vsag_amd_store_t* store, uint64_t nq, uint32_t k);
-int vsag_amd_flat_scan_topk(const vsag_amd_store_t* store, const float* queries_dev, uint64_t nq,
+VSAG_AMD_API size_t vsag_amd_flat_scan_workspace_bytes(const vsag_amd_store_t* store, uint64_t nq, uint32_t k);
+VSAG_AMD_API int vsag_amd_flat_scan_topk(const vsag_amd_store_t* store, const float* queries_dev, uint64_t nq,
                             uint32_t k, uint32_t* ids_dev, float* dists_dev, void* workspace_dev,
                             size_t workspace_bytes, void* stream);
 
 /* Tuning knobs of the scan (query tile T in {1,2,4,8}, 0 = automatic; number of base chunks, 0 =
  * automatic).  Process-wide; meant for benchmarks. */
-int vsag_amd_set_scan_tuning(int query_tile, int base_chunks);
+VSAG_AMD_API int vsag_amd_set_scan_tuning(int query_tile, int base_chunks);
 /* What the last flat scan on this thread used: query tile, passes over the code array, bytes of codes
  * one pass reads. */
-int vsag_amd_last_scan_info(int* query_tile, uint64_t* passes, uint64_t* bytes_per_pass);
+VSAG_AMD_API int vsag_amd_last_scan_info(int* query_tile, uint64_t* passes, uint64_t* bytes_per_pass);
 
 /* Measurement hook: when enabled, a call records HIP events on its stream around the launch of its
  * dominant kernel (flat scan, posting-list scan, k-means assignment); vsag_amd_last_kernel_ms() waits
  * for the last such launch of the calling thread and returns its duration. */
-int vsag_amd_set_kernel_timing(int enable);
-int vsag_amd_last_kernel_ms(float* ms);
+VSAG_AMD_API int vsag_amd_set_kernel_timing(int enable);
+VSAG_AMD_API int vsag_amd_last_kernel_ms(float* ms);
 
 /* ------------------------------------------------------------------ k-means ------------------ */
 
 /* KMeansCluster::find_nearest_one_with_blas (impl/cluster/kmeans_cluster.cpp:193-305):
  * labels[i] = first argmin_j (||c_j||^2 - 2<c_j, x_i>), min_dist[i] = that minimum (may be NULL),
  * *loss_dev (double, may be NULL) = sum_i (min + ||x_i||^2) / n. */
-size_t vsag_amd_kmeans_assign_workspace_bytes(uint64_t n, uint32_t dim, uint32_t k);
-int vsag_amd_kmeans_assign(const float* x_dev, uint64_t n, uint32_t dim, const float* centroids_dev,
+VSAG_AMD_API size_t vsag_amd_kmeans_assign_workspace_bytes(uint64_t n, uint32_t dim, uint32_t k);
+VSAG_AMD_API int vsag_amd_kmeans_assign(const float* x_dev, uint64_t n, uint32_t dim, const float* centroids_dev,
                            uint32_t k, int32_t* labels_dev, float* min_dist_dev, double* loss_dev,
                            void* workspace_dev, size_t workspace_bytes, void* stream);
 /* Centroid update of KMeansCluster::Run (kmeans_cluster.cpp:108-172): mean of member rows; clusters
  * with no member keep their centroid and report counts_dev[j] = 0 (the caller re-seeds them). */
-size_t vsag_amd_kmeans_update_workspace_bytes(uint64_t n, uint32_t dim, uint32_t k);
-int vsag_amd_kmeans_update(const float* x_dev, const int32_t* labels_dev, uint64_t n, uint32_t dim,
+VSAG_AMD_API size_t vsag_amd_kmeans_update_workspace_bytes(uint64_t n, uint32_t dim, uint32_t k);
+VSAG_AMD_API int vsag_amd_kmeans_update(const float* x_dev, const int32_t* labels_dev, uint64_t n, uint32_t dim,
                            uint32_t k, float* centroids_dev, int32_t* counts_dev, void* workspace_dev,
                            size_t workspace_bytes, void* stream);
 /* KMeansCluster::Run (kmeans_cluster.cpp:46-190) with the initial centroids given in centroids_dev
  * and empty clusters re-seeded from mt19937(seed) (the reference draws both from std::random_device).
  * Runs `iters` Lloyd iterations; *loss receives the loss of the last assignment.  Blocking. */
-size_t vsag_amd_kmeans_run_workspace_bytes(uint64_t n, uint32_t dim, uint32_t k);
-int vsag_amd_kmeans_run(const float* x_dev, uint64_t n, uint32_t dim, float* centroids_dev, uint32_t k,
+VSAG_AMD_API size_t vsag_amd_kmeans_run_workspace_bytes(uint64_t n, uint32_t dim, uint32_t k);
+VSAG_AMD_API int vsag_amd_kmeans_run(const float* x_dev, uint64_t n, uint32_t dim, float* centroids_dev, uint32_t k,
                         int iters, uint64_t seed, int32_t* labels_dev, double* loss,
                         void* workspace_dev, size_t workspace_bytes, void* stream);
 
@@ -216,8 +219,8 @@ int vsag_amd_kmeans_run(const float* x_dev, uint64_t n, uint32_t dim, float* cen
 /* Routing (IVFNearestPartition::ClassifyDatasForSearch, ivf_nearest_partition.cpp:99-147, done exactly
  * instead of through the reference's HGraph): the nprobe nearest centroids of every query, ascending.
  * centroids are an fp32 store created with vsag_amd_store_create + append. */
-size_t vsag_amd_ivf_route_workspace_bytes(const vsag_amd_store_t* centroids, uint64_t nq, uint32_t nprobe);
-int vsag_amd_ivf_route(const vsag_amd_store_t* centroids, const float* queries_dev, uint64_t nq,
+VSAG_AMD_API size_t vsag_amd_ivf_route_workspace_bytes(const vsag_amd_store_t* centroids, uint64_t nq, uint32_t nprobe);
+VSAG_AMD_API int vsag_amd_ivf_route(const vsag_amd_store_t* centroids, const float* queries_dev, uint64_t nq,
                        uint32_t nprobe, int32_t* buckets_dev, float* dists_dev, void* workspace_dev,
                        size_t workspace_bytes, void* stream);
 
@@ -225,16 +228,16 @@ int vsag_amd_ivf_route(const vsag_amd_store_t* centroids, const float* queries_d
  * (bucket_datacell.h:527-572) + FlatBucketSearcher::Search (flat_bucket_searcher.cpp:26-138) for a
  * batch: every query scans the nprobe lists named in buckets_dev (nq x nprobe, -1 = skip) and keeps the
  * kcand best (distance, inner id), ascending, padded with VSAG_AMD_INVALID_ID / +inf. */
-size_t vsag_amd_ivf_scan_workspace_bytes(const vsag_amd_store_t* lists, uint64_t nq, uint32_t nprobe,
+VSAG_AMD_API size_t vsag_amd_ivf_scan_workspace_bytes(const vsag_amd_store_t* lists, uint64_t nq, uint32_t nprobe,
                                          uint32_t kcand);
-int vsag_amd_ivf_scan_topk(const vsag_amd_store_t* lists, const float* queries_dev, uint64_t nq,
+VSAG_AMD_API int vsag_amd_ivf_scan_topk(const vsag_amd_store_t* lists, const float* queries_dev, uint64_t nq,
                            const int32_t* buckets_dev, uint32_t nprobe, uint32_t kcand, uint32_t* ids_dev,
                            float* dists_dev, void* workspace_dev, size_t workspace_bytes, void* stream);
 
 /* FlattenReorder::Reorder (impl/reorder/flatten_reorder.cpp:52-114): exact fp32 distances of the
  * candidates (nq x kcand inner ids into raw_dev, n x dim fp32 row-major; VSAG_AMD_INVALID_ID skipped),
  * best k kept, ascending. */
-int vsag_amd_rerank_fp32(const float* raw_dev, uint64_t n, uint32_t dim, int metric,
+VSAG_AMD_API int vsag_amd_rerank_fp32(const float* raw_dev, uint64_t n, uint32_t dim, int metric,
                          const float* queries_dev, uint64_t nq, const uint32_t* cand_ids_dev,
                          uint32_t kcand, uint32_t k, uint32_t* ids_dev, float* dists_dev, void* stream);
 

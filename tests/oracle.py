@@ -319,3 +319,22 @@ def flat_scan_topk_fn(fn, metric, d, codes, queries, k, lb, diff, threads=0):
     lib().orc_flat_scan_topk_fn(fn, metric, u64(d), _p(codes), u64(n), u64(cs), _p(f32(lb)), _p(f32(diff)),
                                 _p(queries), u64(nq), u64(k), _p(ids), _p(dists), threads)
     return ids, dists
+
+
+def rabitq_encode_sq(normed):
+    normed = f32(normed)
+    d = normed.shape[0]
+    quant = np.zeros(d, np.uint8)
+    ub, lb, delta, qsum = C.c_float(), C.c_float(), C.c_float(), C.c_float()
+    lib().orc_rabitq_encode_sq(_p(normed), u64(d), _p(quant), C.byref(ub), C.byref(lb), C.byref(delta),
+                               C.byref(qsum))
+    return quant, ub.value, lb.value, delta.value, qsum.value
+
+
+def rabitq_reorder_sq(quant):
+    quant = np.ascontiguousarray(quant, np.uint8)
+    d = quant.shape[0]
+    plane_bytes = (d + 511) // 512 * 512 // 8
+    planes = np.zeros(4 * plane_bytes, np.uint8)
+    lib().orc_rabitq_reorder_sq(_p(quant), u64(d), _p(planes))
+    return planes, plane_bytes

@@ -1,0 +1,426 @@
+"""Pins the CPU checker (oracle/) itself, on the CPU:
+  * against the known answers the reference's own unit tests hold (cited per test),
+  * against the reference's scalar kernels compiled from its sources (oracle/_ref, when built),
+  * against closed forms / brute force chosen so that a dropped term, a wrong index or a swapped operand fails.
+The same vectors are committed under tests/golden/ so that the checks also run where the reference sources
+are not mounted."""
+import ctypes as C
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle as orc
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+# get_common_used_dims() of the reference fixtures (tests/fixtures/core/common.cpp:59-65)
+DIMS = [7, 8, 9, 32, 33, 48, 64, 65, 70, 96, 97, 109, 128, 129, 160, 161, 192, 193, 224, 225, 256, 512, 784, 960,
+        1024, 1536]
+
+
+# ------------------------------------------------------------------ reference known answers
+def test_sq8_sq4_nan_and_half_known_answers():
+    # scalar_quantizer_test.cpp:101-135: train on {0,0},{1,1}; encode {NaN, 0.5}
+    train = np.array([[0, 0], [1, 1]], np.float32)
+    query = np.array([[np.nan, 0.5]], np.float32)
+    lb, diff = orc.sq_train(train, 8)
+    assert np.array_equal(lb, [0, 0]) and np.array_equal(diff, [1, 1])
+    c8 = orc.sq_encode(query, 8, lb, diff)
+    assert c8[0, 0] == 0 and c8[0, 1] == int(np.float32(255.0) * np.float32(0.5)) == 127
+    dec = orc.sq_decode(c8, 2, 8, lb, diff)
+    assert abs(dec[0, 0]) <= 1e-6 and abs(dec[0, 1] - 127.0 / 255.0) <= 1e-6
+    lb4, diff4 = orc.sq_train(train, 4)
+    c4 = orc.sq_encode(query, 4, lb4, diff4)
+    assert (c4[0, 0] & 0x0F) == 0 and ((c4[0, 0] >> 4) & 0x0F) == 7
+    dec = orc.sq_decode(c4, 2, 4, lb4, diff4)
+    assert abs(dec[0, 0]) <= 1e-6 and abs(dec[0, 1] - 7.0 / 15.0) <= 1e-6
+
+
+def test_sq4_uniform_byte_images():
+    # rabitq_quantizer_test.cpp:1012-1024: trunc_rate 0, one training vector, IP layout [nibbles|sum|code sum]
+    data = np.array([[1, 2, 4, 8, 15, 0]], np.float32)
+    lb, diff = orc.sq_train_uniform(data, 4, orc.IP, mode=3, trunc_rate=0.0)
+    assert lb == 0 and diff == 15
+    code = orc.squ_encode(data, 4, lb, diff, orc.IP)[0]
+    assert code.shape[0] == 4 + 4 + 4
+    assert bytes(code[:3]) == bytes([0x21, 0x84, 0x0F])
+    assert abs(code[4:8].view(np.float32)[0] - 30) < 1e-5 and abs(code[8:12].view(np.float32)[0] - 30) < 1e-5
+    # :1069-1081, dim 15
+    data = np.array([[1, 2, 4, 8, 0, 3, 11, 15, 9, 13, 10, 6, 7, 12, 14]], np.float32)
+    lb, diff = orc.sq_train_uniform(data, 4, orc.IP, mode=3, trunc_rate=0.0)
+    code = orc.squ_encode(data, 4, lb, diff, orc.IP)[0]
+    assert bytes(code[:8]) == bytes([0x21, 0x84, 0x30, 0xFB, 0xD9, 0x6A, 0xC7, 0x0E])
+
+
+def test_uniform_zero_range_gives_zero_codes():
+    # sq4_uniform_quantizer_test.cpp:82, sq8_uniform_quantizer_test.cpp:51
+    data = np.full((10, 12), 0.25, np.float32)
+    for bits in (4, 8):
+        lb, diff = orc.sq_train_uniform(data, bits, orc.L2, mode=3 if bits == 4 else 1)
+        assert diff == 0
+        codes = orc.squ_encode(data, bits, lb, diff, orc.L2)
+        assert not codes.any()
+
+
+def test_rabitq_query_sq_and_planes_known_answers():
+    # rabitq_quantizer_test.cpp:1126-1175 (dim 6) and :1190-1243 (dim 15): EncodeSQ keeps integer inputs,
+    # ReOrderSQ puts bit b of every dim into plane b, planes 64 bytes apart.
+    quant, ub, lb, delta, qsum = orc.rabitq_encode_sq(np.array([1, 2, 4, 8, 15, 0], np.float32))
+    assert list(quant) == [1, 2, 4, 8, 15, 0] and lb == 0 and ub == 15 and delta == 1 and qsum == 30
+    planes, pb = orc.rabitq_reorder_sq(quant)
+    assert pb == 64
+    expect = np.zeros(256, np.uint8)
+    expect[0], expect[64], expect[128], expect[192] = 0x11, 0x12, 0x14, 0x18
+    assert np.array_equal(planes, expect)
+    data15 = np.array([1, 2, 4, 8, 0, 3, 11, 15, 9, 13, 10, 6, 7, 12, 14], np.float32)
+    quant, *_ = orc.rabitq_encode_sq(data15)
+    assert list(quant) == list(data15.astype(np.uint8))
+    planes, pb = orc.rabitq_reorder_sq(quant)
+    expect = np.zeros(256, np.uint8)
+    expect[0:2] = [0xE1, 0x13]
+    expect[64:66] = [0xE2, 0x5C]
+    expect[128:130] = [0x84, 0x7A]
+    expect[192:194] = [0xC8, 0x67]
+    assert np.array_equal(planes, expect)
+    # :1245-1272: an all-equal vector has delta 0 -> all-zero codes
+    quant, ub, lb, delta, qsum = orc.rabitq_encode_sq(np.full(9, 0.5, np.float32))
+    assert delta == 0 and not quant.any() and qsum == 0
+
+
+def test_rabitq_binary_ip_known_answers():
+    # simd/rabitq_simd_test.cpp:118-144
+    codes = np.zeros(64, np.uint8)
+    codes[:8] = [0xFF, 0xFF, 0x0F, 0x0F, 0xF0, 0xF0, 0x00, 0x00]
+    bits = np.zeros(64, np.uint8)
+    bits[:2] = [0xAA, 0x55]
+    L = orc.lib()
+    for dim in range(17):
+        r = L.orc_rabitq_sq4u_binary_ip(codes.ctypes.data_as(C.c_void_p), bits.ctypes.data_as(C.c_void_p),
+                                        C.c_uint64(dim))
+        assert r == (0 if dim == 0 else 36 if dim <= 8 else 32), (dim, r)
+
+
+def test_code_sizes_of_the_benchmark_configs():
+    # SURVEY-independent arithmetic from the constructors: sq4_uniform_quantizer.cpp:33-72 (d=128, l2 -> 64+8),
+    # rabitq_quantizer.cpp:102-133 (d=768, ip, 4-bit query -> 96 + 4*4), query 4 planes of 128 B + 5 floats.
+    assert orc.squ_code_size(128, 4, orc.L2) == 72
+    assert orc.squ_code_size(128, 8, orc.L2) == 136 and orc.squ_code_size(128, 8, orc.IP) == 132
+    assert orc.squ_code_size(6, 4, orc.IP) == 12 and orc.squ_code_size(15, 4, orc.IP) == 16
+    assert orc.rabitq_code_size(768, orc.IP) == 112 and orc.rabitq_code_size(768, orc.L2) == 108
+    assert orc.rabitq_query_code_size(768, orc.IP) == 4 * 128 + 20
+
+
+# ------------------------------------------------------------------ compiled reference kernels
+def _vec_cases():
+    rng = np.random.default_rng(47)
+    for d in DIMS:
+        q = rng.uniform(0.1, 0.9, d).astype(np.float32)
+        x = rng.uniform(0.1, 0.9, d).astype(np.float32)
+        lb = rng.uniform(-0.2, 0.1, d).astype(np.float32)
+        diff = rng.uniform(0.5, 1.5, d).astype(np.float32)
+        c8 = rng.integers(0, 256, d).astype(np.uint8)
+        c8b = rng.integers(0, 256, d).astype(np.uint8)
+        c4 = rng.integers(0, 256, (d + 1) // 2).astype(np.uint8)
+        c4b = rng.integers(0, 256, (d + 1) // 2).astype(np.uint8)
+        if d % 2:
+            c4[-1] &= 0x0F
+            c4b[-1] &= 0x0F
+        yield d, q, x, lb, diff, c8, c8b, c4, c4b
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _primitive_values(fns):
+    """name -> list of values over DIMS, computed with `fns` (oracle or reference symbols)."""
+    out = {}
+    for d, q, x, lb, diff, c8, c8b, c4, c4b in _vec_cases():
+        n = C.c_uint64(d)
+        vals = {
+            "fp32_ip": fns["fp32_ip"](_p(q), _p(x), n),
+            "fp32_l2": fns["fp32_l2"](_p(q), _p(x), n),
+            "sq8_ip": fns["sq8_ip"](_p(q), _p(c8), _p(lb), _p(diff), n),
+            "sq8_l2": fns["sq8_l2"](_p(q), _p(c8), _p(lb), _p(diff), n),
+            "sq4_ip": fns["sq4_ip"](_p(q), _p(c4), _p(lb), _p(diff), n),
+            "sq4_l2": fns["sq4_l2"](_p(q), _p(c4), _p(lb), _p(diff), n),
+            "sq4u_ip": float(fns["sq4u_ip"](_p(c4), _p(c4b), n)),
+            "sq8u_ip": float(fns["sq8u_ip"](_p(c8), _p(c8b), n)),
+        }
+        for k, v in vals.items():
+            out.setdefault(k, []).append(float(v))
+    return out
+
+
+def _oracle_fns():
+    L = orc.lib()
+    L.orc_sq4u_codes_ip.restype = C.c_int32
+    L.orc_sq8u_codes_ip.restype = C.c_int32
+    return {"fp32_ip": L.orc_fp32_ip, "fp32_l2": L.orc_fp32_l2sqr, "sq8_ip": L.orc_sq8_ip, "sq8_l2": L.orc_sq8_l2sqr,
+            "sq4_ip": L.orc_sq4_ip, "sq4_l2": L.orc_sq4_l2sqr, "sq4u_ip": L.orc_sq4u_codes_ip,
+            "sq8u_ip": L.orc_sq8u_codes_ip}
+
+
+def test_primitives_match_compiled_reference_kernels():
+    ref = orc.ref()
+    if ref is None:
+        pytest.skip("oracle/_ref is not built (reference sources not mounted)")
+    rfns = {"fp32_ip": ref["FP32ComputeIP"], "fp32_l2": ref["FP32ComputeL2Sqr"], "sq8_ip": ref["SQ8ComputeIP"],
+            "sq8_l2": ref["SQ8ComputeL2Sqr"], "sq4_ip": ref["SQ4ComputeIP"], "sq4_l2": ref["SQ4ComputeL2Sqr"],
+            "sq4u_ip": ref["SQ4UniformComputeCodesIP"], "sq8u_ip": ref["SQ8UniformComputeCodesIP"]}
+    a, b = _primitive_values(_oracle_fns()), _primitive_values(rfns)
+    for name in a:
+        va, vb = np.array(a[name]), np.array(b[name])
+        if name.endswith("u_ip"):
+            assert np.array_equal(va, vb), name
+        else:
+            # same scalar arithmetic; the reference build may contract a*b+c into an fma
+            assert np.allclose(va, vb, rtol=2e-6, atol=1e-6), (name, np.abs(va - vb).max())
+
+
+def test_primitives_match_committed_golden_vectors():
+    """tests/golden/simd_generic.json holds the values of vsag::generic::* on the seeded vectors above
+    (written by tests/golden/make_simd_golden.py from the compiled reference)."""
+    path = os.path.join(GOLDEN, "simd_generic.json")
+    gold = json.load(open(path))
+    a = _primitive_values(_oracle_fns())
+    for name, vals in gold["values"].items():
+        va, vb = np.array(a[name]), np.array(vals)
+        if name.endswith("u_ip"):
+            assert np.array_equal(va, vb), name
+        else:
+            assert np.allclose(va, vb, rtol=2e-6, atol=1e-6), (name, np.abs(va - vb).max())
+
+
+def test_rabitq_bit_kernels_match_reference():
+    ref = orc.ref()
+    if ref is None:
+        pytest.skip("oracle/_ref is not built (reference sources not mounted)")
+    rng = np.random.default_rng(165)
+    L = orc.lib()
+    for d in DIMS:
+        nb = (d + 7) // 8
+        planes = rng.integers(0, 256, 4 * nb).astype(np.uint8)
+        bits = rng.integers(0, 256, nb).astype(np.uint8)
+        if d % 8:  # the kernels require zero padding bits
+            mask = (1 << (d % 8)) - 1
+            bits[-1] &= mask
+            for b in range(4):
+                planes[b * nb + nb - 1] &= mask
+        assert L.orc_rabitq_sq4u_binary_ip(_p(planes), _p(bits), C.c_uint64(d)) == \
+            ref["RaBitQSQ4UBinaryIP"](_p(planes), _p(bits), C.c_uint64(d))
+        v = rng.standard_normal(d).astype(np.float32)
+        inv = C.c_float(1.0 / np.sqrt(np.float32(d)))
+        a = L.orc_rabitq_float_binary_ip(_p(v), _p(bits), C.c_uint64(d), inv)
+        b = ref["RaBitQFloatBinaryIP"](_p(v), _p(bits), C.c_uint64(d), inv)
+        assert abs(a - b) <= 2e-6 * max(1.0, abs(b))
+        cen = rng.standard_normal(d).astype(np.float32)
+        o1, o2 = np.empty(d, np.float32), np.empty(d, np.float32)
+        n1 = L.orc_normalize_with_centroid(_p(v), _p(cen), _p(o1), C.c_uint64(d))
+        n2 = ref["NormalizeWithCentroid"](_p(v), _p(cen), _p(o2), C.c_uint64(d))
+        assert abs(n1 - n2) <= 2e-6 * n2 and np.allclose(o1, o2, rtol=2e-6, atol=1e-7)
+
+
+# ------------------------------------------------------------------ closed forms and brute force
+def test_popcount_identity_of_the_binary_ip():
+    # sum_b 2^b popcount(plane_b & bits) == sum over set bits of the 4-bit code
+    rng = np.random.default_rng(1)
+    L = orc.lib()
+    for d in (6, 15, 64, 127, 768):
+        code = rng.integers(0, 16, d).astype(np.uint8)
+        bit = rng.integers(0, 2, d).astype(np.uint8)
+        planes, pb = orc.rabitq_reorder_sq(code)
+        bits = np.zeros(pb, np.uint8)
+        for i in range(d):
+            bits[i // 8] |= bit[i] << (i % 8)
+        got = L.orc_rabitq_sq4u_binary_ip(_p(planes), _p(bits), C.c_uint64(pb * 8))
+        assert got == int((code.astype(np.int64) * bit).sum())
+
+
+def test_sq_train_is_the_order_statistic():
+    rng = np.random.default_rng(2)
+    for n, d, bits, rate in [(5000, 5, 8, 0.001), (5000, 5, 4, 0.05), (120000, 3, 8, 0.001), (10, 2, 4, 0.05)]:
+        x = rng.standard_normal((n, d)).astype(np.float32)
+        x[:, 0] = np.round(x[:, 0] * 3) / 3
+        lb, diff = orc.sq_train(x, bits, trunc_rate=rate)
+        if n <= 100000:
+            sample = x
+        else:
+            step = 2147483647 % n
+            sample = x[(np.arange(100000, dtype=np.int64) * step) % n]
+        cnt = sample.shape[0]
+        ignore = max(1, int((cnt - 1) * (rate if bits == 4 else 0.001)))
+        s = np.sort(sample, axis=0)
+        assert np.array_equal(lb, s[ignore - 1]) and np.array_equal(lb + diff, (s[cnt - ignore] - lb) + lb)
+        assert np.array_equal(diff, s[cnt - ignore] - s[ignore - 1])
+    # uniform: TRUNC_BOUND takes min of uppers / max of lowers; CLASSIC the global extremes
+    x = rng.random((3000, 6), dtype=np.float32)
+    lb, diff = orc.sq_train_uniform(x, 8, mode=1)
+    assert lb == x.min() and np.float32(lb + diff) == np.float32(x.min() + (x.max() - x.min()))
+    lb4, diff4 = orc.sq_train_uniform(x, 4, mode=3, trunc_rate=0.05)
+    s = np.sort(x, axis=0)
+    ignore = int(2999 * 0.05)
+    assert lb4 == s[ignore - 1].max() and diff4 == np.float32(s[3000 - ignore].min() - s[ignore - 1].max())
+
+
+def test_sq_codes_round_trip_on_the_integer_grid():
+    # quantizer_test.h:134-175: values on the code grid come back exactly
+    rng = np.random.default_rng(3)
+    for bits in (8, 4):
+        levels = (1 << bits) - 1
+        d = 40
+        grid = rng.integers(0, levels + 1, (200, d)).astype(np.float32)
+        lb = np.zeros(d, np.float32)
+        diff = np.full(d, levels, np.float32)
+        codes = orc.sq_encode(grid, bits, lb, diff)
+        dec = orc.sq_decode(codes, d, bits, lb, diff)
+        # delta > 0.999 is clamped to 1 (scalar_quantization_utils.h:19-30): the top level maps to itself too
+        assert np.array_equal(dec, grid)
+
+
+def test_sq_distance_is_distance_to_the_decoded_vector():
+    rng = np.random.default_rng(4)
+    d, n = 96, 50
+    x = rng.random((n, d), dtype=np.float32)
+    q = rng.random((3, d), dtype=np.float32)
+    for bits, kind in ((8, orc.SQ8), (4, orc.SQ4)):
+        lb, diff = orc.sq_train(x, bits)
+        codes = orc.sq_encode(x, bits, lb, diff)
+        dec = orc.sq_decode(codes, d, bits, lb, diff).astype(np.float64)
+        l2 = orc.flat_dists(kind, orc.L2, d, codes, q, lb=lb, diff=diff)
+        ip = orc.flat_dists(kind, orc.IP, d, codes, q, lb=lb, diff=diff)
+        assert np.allclose(l2, ((q[:, None, :].astype(np.float64) - dec[None]) ** 2).sum(2), rtol=1e-5)
+        assert np.allclose(ip, 1.0 - q.astype(np.float64) @ dec.T, rtol=1e-5, atol=1e-5)
+
+
+def test_uniform_l2_closed_form_and_ip_quirk():
+    rng = np.random.default_rng(5)
+    d, n = 33, 40
+    x = rng.random((n, d), dtype=np.float32)
+    for bits, kind in ((4, orc.SQ4U), (8, orc.SQ8U)):
+        levels = (1 << bits) - 1
+        lb, diff = orc.sq_train_uniform(x, bits, orc.L2, mode=3 if bits == 4 else 1)
+        codes = orc.squ_encode(x, bits, lb, diff, orc.L2)
+        dists = orc.flat_dists(kind, orc.L2, d, codes, codes[:5], lb=lb, diff=diff)
+        # integer codes: unpack and compare with (n1 + n2 - 2 ip) (diff / L)^2
+        if bits == 4:
+            raw = np.zeros((n, d), np.int64)
+            for i in range(d):
+                raw[:, i] = (codes[:, i // 2] >> (4 * (i % 2))) & 0xF
+        else:
+            raw = codes[:, :d].astype(np.int64)
+        norms = codes[:, -8:].view(np.uint64)[:, 0].astype(np.int64)
+        assert np.array_equal(norms, (raw ** 2).sum(1))
+        expect = ((raw[:5, None, :] - raw[None]) ** 2).sum(2) * (float(diff) / levels) ** 2
+        assert np.allclose(dists, expect, rtol=1e-5, atol=1e-7)
+        assert np.allclose(np.diag(dists[:, :5]), 0, atol=1e-7)
+        # IP keeps the reference's form lb (sum_q + sum_o) + rate <c_q, c_o> + lb^2 with raw-value sums
+        codes_ip = orc.squ_encode(x, bits, lb, diff, orc.IP)
+        got = orc.flat_dists(kind, orc.IP, d, codes_ip, codes_ip[:5], lb=lb, diff=diff)
+        sums = x.astype(np.float64).sum(1)
+        rate = (float(diff) / levels) ** 2
+        expect = 1.0 - (lb * (sums[:5, None] + sums[None]) + rate * (raw[:5] @ raw.T) + float(lb) ** 2)
+        assert np.allclose(got, expect, rtol=1e-4, atol=1e-4)
+
+
+def _rotation(rng, d):
+    q, r = np.linalg.qr(rng.standard_normal((d, d)))
+    return (q * np.sign(np.diag(r))).astype(np.float32)
+
+
+def test_rabitq_encode_invariants_and_estimator():
+    rng = np.random.default_rng(6)
+    d, n = 128, 400
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    x /= np.linalg.norm(x, axis=1, keepdims=True)
+    rot = _rotation(rng, d)
+    cen = orc.rabitq_train(x, rot)
+    assert np.allclose(cen, rot.astype(np.float64) @ x.astype(np.float64).mean(0), atol=1e-5)
+    codes = orc.rabitq_encode(x, rot, cen, orc.IP)
+    nb = d // 8
+    y = (x.astype(np.float64) @ rot.astype(np.float64).T) - cen
+    norm = np.linalg.norm(y, axis=1)
+    o = y / norm[:, None]
+    bits = np.unpackbits(codes[:, :nb], axis=1, bitorder="little")[:, :d]
+    near_zero = np.abs(o) < 1e-6
+    assert np.all((bits == (o >= 0)) | near_zero)
+    f = codes[:, nb:].view(np.float32)  # norm, error, sum, raw norm
+    assert np.allclose(f[:, 0], norm, rtol=1e-5)
+    assert np.allclose(f[:, 1], np.abs(o).sum(1) / np.sqrt(d), rtol=1e-4)  # error = <o_bar, o> = sum|o_d| / sqrt(d)
+    assert np.array_equal(f[:, 2], bits.sum(1).astype(np.float32))
+    assert np.allclose(f[:, 3], 1.0, rtol=1e-5)
+    # estimator: the 4-bit and the fp32 query forms agree within the query quantisation error, and both
+    # estimate the true inner-product distance with the error RaBitQ promises at this dimension
+    q = rng.standard_normal((20, d)).astype(np.float32)
+    q /= np.linalg.norm(q, axis=1, keepdims=True)
+    d4 = orc.flat_dists(orc.RABITQ, orc.IP, d, codes, orc.rabitq_process_query(q, rot, cen, orc.IP, 4), qbits=4)
+    codes32 = orc.rabitq_encode(x, rot, cen, orc.IP, qbits=32)
+    d32 = orc.flat_dists(orc.RABITQ, orc.IP, d, codes32, orc.rabitq_process_query(q, rot, cen, orc.IP, 32), qbits=32)
+    true = 1.0 - q.astype(np.float64) @ x.astype(np.float64).T
+    assert np.abs(d4 - d32).max() < 0.05
+    assert np.abs(d32 - true).mean() < 0.08 and np.abs(d4 - true).mean() < 0.08
+    assert np.corrcoef(d4.ravel(), true.ravel())[0, 1] > 0.7
+
+
+def test_kmeans_assign_is_the_exact_argmin():
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((800, 24)).astype(np.float32)
+    cent = rng.standard_normal((37, 24)).astype(np.float32)
+    cent[20] = cent[5]  # a tie: the first minimum wins
+    labels, mind, loss = orc.kmeans_assign(x, cent)
+    d2 = ((x[:, None, :].astype(np.float64) - cent[None].astype(np.float64)) ** 2).sum(2)
+    assert np.array_equal(labels, d2.argmin(1)) and 20 not in labels
+    xn = (x.astype(np.float64) ** 2).sum(1)
+    assert np.allclose(mind + xn, d2.min(1), atol=1e-4)
+    assert abs(loss - d2.min(1).mean()) < 1e-4
+    # update = mean of members, empty clusters reported
+    newc, counts = orc.kmeans_update(x, labels, cent)
+    for j in range(37):
+        m = labels == j
+        assert counts[j] == m.sum()
+        if m.any():
+            assert np.allclose(newc[j], x[m].mean(0), atol=1e-5)
+        else:
+            assert np.array_equal(newc[j], cent[j])
+
+
+def test_heaps_equal_sorting():
+    rng = np.random.default_rng(8)
+    n, d, k = 700, 10, 13
+    x = rng.random((n, d), dtype=np.float32)
+    q = rng.random((6, d), dtype=np.float32)
+    codes = x.view(np.uint8).reshape(n, 4 * d)
+    all_d = orc.flat_dists(orc.FP32, orc.L2, d, codes, q)
+    for strict in (False, True):
+        ids, ds = orc.flat_scan_topk(orc.FP32, orc.L2, d, codes, q, k, strict=strict)
+        order = np.argsort(all_d, axis=1, kind="stable")[:, :k]
+        assert np.array_equal(ds, np.take_along_axis(all_d, order, 1))
+        assert np.array_equal(ids, order.astype(np.uint32))
+    ids, ds = orc.flat_scan_topk(orc.FP32, orc.L2, d, codes[:5], q, k)
+    assert np.all(ids[:, 5:] == 0xFFFFFFFF) and np.all(np.isinf(ds[:, 5:]))
+
+
+def test_ivf_probing_every_list_equals_the_flat_scan():
+    rng = np.random.default_rng(9)
+    n, d, nlist, nq, k = 1500, 16, 12, 9, 10
+    x = rng.random((n, d), dtype=np.float32)
+    q = rng.random((nq, d), dtype=np.float32)
+    cent = x[:nlist].copy()
+    labels, _, _ = orc.kmeans_assign(x, cent)
+    offsets, order = orc.ivf_build_lists(labels, nlist)
+    # stable counting sort: inside a list inner ids ascend; lists are contiguous in label order
+    for j in range(nlist):
+        seg = order[int(offsets[j]):int(offsets[j + 1])]
+        assert np.all(labels[seg] == j) and np.all(np.diff(seg.astype(np.int64)) > 0)
+    codes = x.view(np.uint8).reshape(n, 4 * d)
+    buckets = np.tile(np.arange(nlist, dtype=np.int32), (nq, 1))
+    ids, ds = orc.ivf_scan(orc.FP32, orc.L2, d, codes[order], offsets, order, q, buckets, k)
+    fids, fds = orc.flat_scan_topk(orc.FP32, orc.L2, d, codes, q, k, strict=True)
+    assert np.array_equal(ds, fds) and np.array_equal(np.sort(ids, 1), np.sort(fids, 1))
+    # routing is the exact centroid top-nprobe; rerank of exact candidates returns them sorted
+    b, bd = orc.ivf_route(cent, q, 4)
+    dc = ((q[:, None, :].astype(np.float64) - cent[None].astype(np.float64)) ** 2).sum(2)
+    assert np.array_equal(b, np.argsort(dc, 1, kind="stable")[:, :4].astype(np.int32))
+    rids, rds = orc.rerank_fp32(x, q, ids, 5)
+    assert np.array_equal(rds, fds[:, :5])
