@@ -1,0 +1,206 @@
+"""brute_force / ivf through the kept API (CreateIndex -> Build -> KnnSearch with the reference's JSON), modelled on
+the reference's functional tests: recall floors (tests/test_ivf.cpp:94-102 with RECALL_THRESHOLD 0.85,
+tests/test_index.h:373), result shape (tests/test_index/test_index_search.cpp:60-99), batch == serial
+(tests/test_ivf.cpp:3283-3341), exact self-distance after fp32 reorder (tests/test_ivf.cpp:340-367), error paths."""
+import json
+
+import numpy as np
+import pytest
+
+import oracle as orc
+from vsag_amd import pyvsag
+
+pytestmark = pytest.mark.gpu
+RECALL_THRESHOLD = 0.85
+
+
+def vectors(count, dim, seed=47, normalize=True):
+    """generate_vectors of the reference fixtures (tests/fixtures/data/vector_generator.cpp:121-124)."""
+    rng = np.random.Generator(np.random.MT19937(seed))
+    x = rng.uniform(0.1, 0.9, (count, dim)).astype(np.float32)
+    if normalize:
+        x /= np.linalg.norm(x, axis=1, keepdims=True)
+    return x
+
+
+def ground_truth(x, q, k, metric):
+    x64, q64 = x.astype(np.float64), q.astype(np.float64)
+    if metric == "l2":
+        d = ((q64[:, None, :] - x64[None]) ** 2).sum(2)
+    elif metric == "ip":
+        d = 1 - q64 @ x64.T
+    else:
+        d = 1 - (q64 / np.linalg.norm(q64, axis=1, keepdims=True)) @ (x64 / np.linalg.norm(x64, axis=1, keepdims=True)).T
+    idx = np.argsort(d, 1, kind="stable")[:, :k]
+    return idx, np.take_along_axis(d, idx, 1)
+
+
+def recall(ids, gt_ids, labels):
+    hit = sum(len(set(a.tolist()) & set(labels[b].tolist())) for a, b in zip(ids, gt_ids))
+    return hit / float(gt_ids.size)
+
+
+def make(name, dim, metric, **index_param):
+    return pyvsag.Index(name, json.dumps({"dtype": "float32", "metric_type": metric, "dim": dim,
+                                         "index_param": index_param}))
+
+
+@pytest.mark.parametrize("metric", ["l2", "ip", "cosine"])
+@pytest.mark.parametrize("quant,floor", [("fp32", 0.99), ("sq8", 0.84), ("sq4_uniform", 0.5), ("sq8_uniform", 0.84)])
+def test_brute_force_build_and_search(lib, metric, quant, floor):
+    n, d, nq, k = 2000, 64, 50, 10
+    x = vectors(n, d)
+    q = vectors(nq, d, seed=165)
+    labels = np.arange(n, dtype=np.int64) * 3 + 7
+    idx = make("brute_force", d, metric, base_quantization_type=quant)
+    assert idx.build(x, labels, n, d) == 0
+    assert idx.get_num_elements() == n
+    gt, gt_d = ground_truth(x, q, k, metric)
+    ids, dists = idx.knn_search_batch(q, k, "{}")
+    assert ids.shape == (nq, k)
+    assert recall(ids, gt, labels) >= floor * RECALL_THRESHOLD
+    assert np.all(np.diff(dists, axis=1) >= 0)
+    # one query per call, as the reference's KnnSearch is used: same result as the batch row
+    for i in range(5):
+        sid, sd = idx.knn_search(q[i], k, "{}")
+        assert sid.shape == (k,) and np.array_equal(sid, ids[i]) and np.array_equal(sd, dists[i])
+    if quant == "fp32":
+        assert np.allclose(dists, gt_d, rtol=1e-4, atol=2e-6)
+        assert recall(ids, gt, labels) == 1.0
+    idx.close()
+
+
+def test_brute_force_conventions(lib):
+    d = 16
+    idx = make("brute_force", d, "l2")
+    # empty index -> empty result, not an error
+    ids, dists = idx.knn_search(np.zeros(d, np.float32), 5, "{}")
+    assert ids.size == 0
+    x = vectors(7, d)
+    labels = np.array([10, 11, 12, 13, 14, 15, 10], np.int64)  # one duplicate id
+    assert idx.build(x, labels, 7, d) == 1
+    assert idx.get_num_elements() == 6
+    # fewer results than k -> short result
+    ids, dists = idx.knn_search(x[2], 20, "{}")
+    assert ids.size == 6 and ids[0] == 12 and dists[0] <= 2e-6
+    # adding more, duplicates are reported
+    assert idx.add(vectors(3, d, seed=5), np.array([15, 16, 17], np.int64), 3, d) == 1
+    assert idx.get_num_elements() == 8
+    with pytest.raises(pyvsag.VsagError) as e:
+        idx.build(x, labels, 7, d)
+    assert e.value.code == -5  # BUILD_TWICE
+    with pytest.raises(pyvsag.VsagError) as e:
+        idx.knn_search(np.zeros(d + 1, np.float32), 5, "{}")
+    assert e.value.code == -3
+    with pytest.raises(pyvsag.VsagError) as e:
+        idx.knn_search(np.zeros(d, np.float32), 0, "{}")
+    assert e.value.code == -3
+    with pytest.raises(pyvsag.VsagError) as e:
+        idx.knn_search(np.zeros(d, np.float32), 3, "{bad")
+    assert e.value.code == -3
+    with pytest.raises(pyvsag.VsagError) as e:
+        idx.add(vectors(2, d + 2), np.array([100, 101], np.int64), 2, d + 2)
+    assert e.value.code == -3
+    idx.close()
+
+
+IVF_SEARCH = json.dumps({"ivf": {"scan_buckets_count": 30}})
+
+
+@pytest.mark.parametrize("metric", ["l2", "ip", "cosine"])
+@pytest.mark.parametrize("quant,reorder,floor", [("fp32", False, 0.90), ("sq8", False, 0.84),
+                                                 ("sq8_uniform", True, 0.89), ("sq4_uniform", True, 0.80)])
+def test_ivf_recall_floors(lib, metric, quant, reorder, floor):
+    n, d, nq, k = 2400, 64, 100, 10
+    x = vectors(n, d)
+    q = vectors(nq, d, seed=165)
+    labels = np.arange(n, dtype=np.int64) + 1000
+    params = {"buckets_count": 50, "base_quantization_type": quant, "train_sample_count": 2400}
+    if reorder:
+        params.update(use_reorder=True, precise_quantization_type="fp32")
+    idx = make("ivf", d, metric, **params)
+    assert idx.build(x, labels, n, d) == 0
+    gt, _ = ground_truth(x, q, k, metric)
+    search = json.dumps({"ivf": {"scan_buckets_count": 30, "factor": 4.0}})
+    ids, dists = idx.knn_search_batch(q, k, search)
+    r = recall(ids, gt, labels)
+    assert r >= floor * RECALL_THRESHOLD, r
+    assert np.all(np.diff(dists, axis=1) >= 0)
+    # batch == serial, bit for bit
+    for i in range(8):
+        sid, sd = idx.knn_search(q[i], k, search)
+        assert np.array_equal(sid, ids[i]) and np.array_equal(sd, dists[i])
+    idx.close()
+
+
+def test_ivf_self_query_is_exact_after_fp32_reorder(lib):
+    n, d = 2000, 32
+    x = vectors(n, d)
+    labels = np.arange(n, dtype=np.int64)
+    idx = make("ivf", d, "l2", buckets_count=20, base_quantization_type="sq8", use_reorder=True,
+               precise_quantization_type="fp32", train_sample_count=2000)
+    idx.build(x, labels, n, d)
+    search = json.dumps({"ivf": {"scan_buckets_count": 20, "factor": 5.0}})
+    ids, dists = idx.knn_search_batch(x[:200], 1, search)
+    assert np.array_equal(ids[:, 0], labels[:200])
+    assert np.all(np.abs(dists[:, 0]) < 2e-6)
+    idx.close()
+
+
+def test_ivf_probing_every_bucket_equals_brute_force(lib):
+    n, d, nq, k = 3000, 48, 40, 10
+    x = vectors(n, d, normalize=False)
+    q = vectors(nq, d, seed=165, normalize=False)
+    labels = np.arange(n, dtype=np.int64)
+    bf = make("brute_force", d, "l2", base_quantization_type="fp32")
+    bf.build(x, labels, n, d)
+    ivf = make("ivf", d, "l2", buckets_count=64, base_quantization_type="fp32", train_sample_count=3000)
+    ivf.build(x, labels, n, d)
+    a_ids, a_d = bf.knn_search_batch(q, k, "{}")
+    b_ids, b_d = ivf.knn_search_batch(q, k, json.dumps({"ivf": {"scan_buckets_count": 1000}}))
+    assert np.array_equal(a_ids, b_ids) and np.array_equal(a_d, b_d)
+    # incremental add keeps the lists consistent
+    x2 = vectors(500, d, seed=9, normalize=False)
+    l2 = np.arange(500, dtype=np.int64) + n
+    assert bf.add(x2, l2, 500, d) == 0 and ivf.add(x2, l2, 500, d) == 0
+    a_ids, a_d = bf.knn_search_batch(q, k, "{}")
+    b_ids, b_d = ivf.knn_search_batch(q, k, json.dumps({"ivf": {"scan_buckets_count": 64}}))
+    assert np.array_equal(a_ids, b_ids) and np.array_equal(a_d, b_d)
+    bf.close()
+    ivf.close()
+
+
+def test_ivf_routing_only_and_errors(lib):
+    n, d = 1500, 24
+    x = vectors(n, d)
+    idx = make("ivf", d, "l2", buckets_count=16, train_sample_count=1500)
+    idx.build(x, np.arange(n, dtype=np.int64), n, d)
+    ids, dists = idx.knn_search(x[0], 4, json.dumps({"ivf": {"scan_buckets_count": 4, "disable_bucket_scan": True}}))
+    assert ids.size == 4 and np.all((ids >= 0) & (ids < 16)) and np.all(np.diff(dists) >= 0)
+    with pytest.raises(pyvsag.VsagError) as e:
+        idx.knn_search(x[0], 4, "{}")
+    assert e.value.code == -3 and "ivf" in e.value.message
+    with pytest.raises(pyvsag.VsagError) as e:
+        idx.knn_search(x[0], 4, json.dumps({"ivf": {"factor": 2.0}}))
+    assert e.value.code == -3 and "scan_buckets_count" in e.value.message
+    small = make("ivf", d, "l2", buckets_count=64, train_sample_count=512)
+    with pytest.raises(pyvsag.VsagError) as e:
+        small.build(x[:10], np.arange(10, dtype=np.int64), 10, d)
+    assert e.value.code == -3 and "k cannot be larger than count" in e.value.message
+    idx.close()
+    small.close()
+
+
+def test_ivf_rabitq_with_reorder(lib):
+    # tests/test_ivf.cpp:1212-1230: rabitq base codes, fp32 reorder
+    n, d, nq, k = 3000, 128, 50, 10
+    x = vectors(n, d)
+    q = vectors(nq, d, seed=165)
+    labels = np.arange(n, dtype=np.int64)
+    idx = make("ivf", d, "l2", buckets_count=10, base_quantization_type="rabitq", rabitq_bits_per_dim_query=4,
+               use_reorder=True, precise_quantization_type="fp32", train_sample_count=3000)
+    idx.build(x, labels, n, d)
+    gt, _ = ground_truth(x, q, k, "l2")
+    ids, _ = idx.knn_search_batch(q, k, json.dumps({"ivf": {"scan_buckets_count": 10, "factor": 20.0}}))
+    assert recall(ids, gt, labels) >= 0.85
+    idx.close()

@@ -59,7 +59,8 @@ def build_host(verbose=True):
     if not sources:
         return None
     lib = os.path.join(LIB, "libvsag_amd_host.so")
-    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-I" + os.path.join(ROOT, "..", "include"),
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-fvisibility=hidden",
+           "-I" + os.path.join(ROOT, "..", "include"),
            "-o", lib] + [os.path.join(HOST, s) for s in sources] + [
                "-L" + LIB, "-lvsag_amd", "-Wl,-rpath,$ORIGIN", "-lpthread"]
     out = _run(cmd)

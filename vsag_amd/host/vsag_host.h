@@ -1,0 +1,205 @@
+// Host-side mirror of the part of VSAG's public API that drives the search core:
+//   vsag::Factory::CreateIndex("brute_force" | "ivf", json)  (include/vsag/factory.h:47-50)
+//   vsag::Index::{Build, Add, KnnSearch, GetNumElements}       (include/vsag/index.h:126,150,284-374)
+//   vsag::Dataset builder                                       (include/vsag/dataset.h:134-511)
+//   vsag::Error / ErrorType                                     (include/vsag/errors.h:26-56)
+// Same names, argument meaning, JSON keys and error behaviour; the arithmetic behind it runs in the HIP
+// library (include/vsag_amd.h).  The reference returns tl::expected<T, Error>; Expected<T> below has the
+// same has_value() / value() / error() surface.
+#pragma once
+
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <utility>
+#include <vector>
+
+namespace vsag {
+
+#define VSAG_HOST_EXPORT __attribute__((visibility("default")))
+
+enum class ErrorType {
+    UNKNOWN_ERROR = 1,
+    INTERNAL_ERROR,
+    INVALID_ARGUMENT,
+    WRONG_STATUS,
+    BUILD_TWICE,
+    INDEX_NOT_EMPTY,
+    UNSUPPORTED_INDEX,
+    UNSUPPORTED_INDEX_OPERATION,
+    DIMENSION_NOT_EQUAL,
+    INDEX_EMPTY,
+    NO_ENOUGH_MEMORY,
+    READ_ERROR,
+    MISSING_FILE,
+    INVALID_BINARY,
+};
+
+struct Error {
+    Error(ErrorType t, std::string msg) : type(t), message(std::move(msg)) {
+    }
+    ErrorType type;
+    std::string message;
+};
+
+template <typename T>
+class Expected {
+public:
+    Expected(T value) : has_(true), value_(std::move(value)), error_(ErrorType::UNKNOWN_ERROR, "") {
+    }
+    Expected(Error error) : has_(false), value_(), error_(std::move(error)) {
+    }
+    bool
+    has_value() const {
+        return has_;
+    }
+    explicit operator bool() const {
+        return has_;
+    }
+    T&
+    value() {
+        return value_;
+    }
+    const T&
+    value() const {
+        return value_;
+    }
+    T&
+    operator*() {
+        return value_;
+    }
+    T*
+    operator->() {
+        return &value_;
+    }
+    const Error&
+    error() const {
+        return error_;
+    }
+
+private:
+    bool has_;
+    T value_;
+    Error error_;
+};
+
+class Dataset;
+using DatasetPtr = std::shared_ptr<Dataset>;
+
+// Column container with the reference's builder style.  An owning dataset frees ids / distances / vectors
+// with delete[] when it dies (results of a search are owning).
+class VSAG_HOST_EXPORT Dataset : public std::enable_shared_from_this<Dataset> {
+public:
+    static DatasetPtr
+    Make() {
+        return DatasetPtr(new Dataset());
+    }
+    ~Dataset() {
+        if (owner_) {
+            delete[] ids_;
+            delete[] distances_;
+            delete[] vectors_;
+        }
+    }
+    DatasetPtr
+    Owner(bool is_owner) {
+        owner_ = is_owner;
+        return shared_from_this();
+    }
+    DatasetPtr
+    NumElements(int64_t n) {
+        num_elements_ = n;
+        return shared_from_this();
+    }
+    DatasetPtr
+    Dim(int64_t d) {
+        dim_ = d;
+        return shared_from_this();
+    }
+    DatasetPtr
+    Ids(const int64_t* ids) {
+        ids_ = ids;
+        return shared_from_this();
+    }
+    DatasetPtr
+    Distances(const float* d) {
+        distances_ = d;
+        return shared_from_this();
+    }
+    DatasetPtr
+    Float32Vectors(const float* v) {
+        vectors_ = v;
+        return shared_from_this();
+    }
+    DatasetPtr
+    Statistics(std::string s) {
+        statistics_ = std::move(s);
+        return shared_from_this();
+    }
+    int64_t
+    GetNumElements() const {
+        return num_elements_;
+    }
+    int64_t
+    GetDim() const {
+        return dim_;
+    }
+    const int64_t*
+    GetIds() const {
+        return ids_;
+    }
+    const float*
+    GetDistances() const {
+        return distances_;
+    }
+    const float*
+    GetFloat32Vectors() const {
+        return vectors_;
+    }
+    const std::string&
+    GetStatistics() const {
+        return statistics_;
+    }
+
+private:
+    Dataset() = default;
+    bool owner_ = true;
+    int64_t num_elements_ = 0;
+    int64_t dim_ = 0;
+    const int64_t* ids_ = nullptr;
+    const float* distances_ = nullptr;
+    const float* vectors_ = nullptr;
+    std::string statistics_;
+};
+
+class VSAG_HOST_EXPORT Index {
+public:
+    virtual ~Index() = default;
+
+    // Train + Add.  Returns the ids that could not be inserted (duplicates of ids already present).
+    virtual Expected<std::vector<int64_t>>
+    Build(const DatasetPtr& base) = 0;
+
+    virtual Expected<std::vector<int64_t>>
+    Add(const DatasetPtr& base) = 0;
+
+    // query: NumElements rows of Dim floats.  One row -> result NumElements(1), Dim(count <= k), ascending
+    // distances, ids are the user labels.  Several rows -> NumElements(nq), Dim(k), short rows padded with
+    // id -1 / distance +inf (the batch convention of IVF::SearchWithRequest, src/algorithm/ivf/ivf.cpp:2137-2210).
+    virtual Expected<DatasetPtr>
+    KnnSearch(const DatasetPtr& query, int64_t k, const std::string& parameters) const = 0;
+
+    virtual int64_t
+    GetNumElements() const = 0;
+};
+
+class VSAG_HOST_EXPORT Factory {
+public:
+    // name: "brute_force" or "ivf".  parameters: {"dtype":"float32","metric_type":"l2"|"ip"|"cosine","dim":N,
+    // "index_param":{...}} with the reference's keys (src/constants.cpp:195-216,255-265); unknown index_param
+    // keys are INVALID_ARGUMENT "invalid config param: <key>" (src/utils/util_functions.cpp:45-66).
+    static Expected<std::shared_ptr<Index>>
+    CreateIndex(const std::string& name, const std::string& parameters);
+};
+
+}  // namespace vsag

@@ -1,0 +1,127 @@
+"""Python view of the GPU-backed index classes with the call shapes of the reference's pyvsag.Index
+(python_bindings/index_binding.cpp:641-716): Index(name, parameters), build(vectors, ids, num_elements, dim),
+add(...), knn_search(vector, k, parameters) -> (ids, dists), get_num_elements().  knn_search_batch is the
+addition (many queries per call).  Everything goes through libvsag_amd_host.so's C API; errors raise
+VsagError with the reference's error code."""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+HOST_LIB_PATH = os.path.join(_HERE, "lib", "libvsag_amd_host.so")
+
+ERROR_NAMES = {0: "SUCCESS", -1: "UNKNOWN_ERROR", -2: "INTERNAL_ERROR", -3: "INVALID_ARGUMENT", -4: "WRONG_STATUS",
+               -5: "BUILD_TWICE", -6: "INDEX_NOT_EMPTY", -7: "UNSUPPORTED_INDEX", -8: "UNSUPPORTED_INDEX_OPERATION",
+               -9: "DIMENSION_NOT_EQUAL", -10: "INDEX_EMPTY", -11: "NO_ENOUGH_MEMORY"}
+
+
+class ErrorT(C.Structure):
+    _fields_ = [("code", C.c_int), ("message", C.c_char * 1024)]
+
+
+class SearchResult(C.Structure):
+    _fields_ = [("dists", C.POINTER(C.c_float)), ("ids", C.POINTER(C.c_int64)), ("count", C.c_int64),
+                ("other_result", C.c_void_p)]
+
+
+class VsagError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("%s: %s" % (ERROR_NAMES.get(code, str(code)), message))
+        self.code = code
+        self.message = message
+
+
+_lib = None
+
+
+def _load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(HOST_LIB_PATH):
+            raise FileNotFoundError("%s is not built: run `python -m vsag_amd.build`" % HOST_LIB_PATH)
+        # the kernels' library first, so that the host library's dependency resolves to the in-tree build
+        C.CDLL(os.path.join(_HERE, "lib", "libvsag_amd.so"), mode=C.RTLD_GLOBAL)
+        lib = C.CDLL(HOST_LIB_PATH)
+        lib.vsag_index_factory.restype = C.c_void_p
+        lib.vsag_index_factory.argtypes = [C.c_char_p, C.c_char_p]
+        lib.vsag_last_factory_error.restype = ErrorT
+        lib.vsag_index_destroy.restype = ErrorT
+        lib.vsag_index_destroy.argtypes = [C.c_void_p]
+        for name in ("vsag_index_build", "vsag_index_add"):
+            fn = getattr(lib, name)
+            fn.restype = ErrorT
+            fn.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint64]
+        lib.vsag_index_knn_search.restype = ErrorT
+        lib.vsag_index_knn_search.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int64, C.c_char_p,
+                                              C.POINTER(SearchResult)]
+        lib.vsag_index_knn_search_batch.restype = ErrorT
+        lib.vsag_index_knn_search_batch.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint64, C.c_int64,
+                                                    C.c_char_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_int64)]
+        lib.vsag_index_get_num_elements.restype = C.c_int64
+        lib.vsag_index_get_num_elements.argtypes = [C.c_void_p]
+        lib.vsag_last_failed_id_count.restype = C.c_int64
+        _lib = lib
+    return _lib
+
+
+def _check(err):
+    if err.code != 0:
+        raise VsagError(err.code, err.message.decode("utf-8", "replace"))
+
+
+class Index:
+    def __init__(self, name, parameters):
+        lib = _load()
+        self._h = lib.vsag_index_factory(name.encode(), parameters.encode())
+        if not self._h:
+            _check(lib.vsag_last_factory_error())
+            raise VsagError(-1, "index creation failed")
+
+    def _insert(self, fn, vectors, ids, num_elements, dim):
+        v = np.ascontiguousarray(vectors, np.float32).reshape(-1)
+        i = np.ascontiguousarray(ids, np.int64).reshape(-1)
+        assert v.size >= num_elements * dim and i.size >= num_elements
+        _check(fn(self._h, v.ctypes.data, i.ctypes.data, dim, num_elements))
+        return int(_load().vsag_last_failed_id_count())
+
+    def build(self, vectors, ids, num_elements, dim):
+        """Returns the number of ids that could not be inserted."""
+        return self._insert(_load().vsag_index_build, vectors, ids, num_elements, dim)
+
+    def add(self, vectors, ids, num_elements, dim):
+        return self._insert(_load().vsag_index_add, vectors, ids, num_elements, dim)
+
+    def knn_search(self, vector, k, parameters):
+        q = np.ascontiguousarray(vector, np.float32).reshape(-1)
+        kk = max(int(k), 1)
+        ids = np.empty(kk, np.int64)
+        dists = np.empty(kk, np.float32)
+        res = SearchResult(dists.ctypes.data_as(C.POINTER(C.c_float)), ids.ctypes.data_as(C.POINTER(C.c_int64)), 0,
+                           None)
+        _check(_load().vsag_index_knn_search(self._h, q.ctypes.data, q.size, k, parameters.encode(), C.byref(res)))
+        return ids[:res.count].copy(), dists[:res.count].copy()
+
+    def knn_search_batch(self, vectors, k, parameters):
+        q = np.ascontiguousarray(vectors, np.float32)
+        nq, dim = q.shape
+        ids = np.empty((nq, k), np.int64)
+        dists = np.empty((nq, k), np.float32)
+        rdim = C.c_int64()
+        _check(_load().vsag_index_knn_search_batch(self._h, q.ctypes.data, nq, dim, k, parameters.encode(),
+                                                   ids.ctypes.data, dists.ctypes.data, C.byref(rdim)))
+        return ids, dists
+
+    def get_num_elements(self):
+        return int(_load().vsag_index_get_num_elements(self._h))
+
+    def close(self):
+        if self._h:
+            _load().vsag_index_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
