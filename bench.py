@@ -1,11 +1,15 @@
 #!/usr/bin/env python3
-"""Headline benchmark: QPS @ recall@10 of the flat SQ8 scan (1M x 128 codes, 10 000 queries, k = 10).
+"""Benchmarks of the MI355X search core on the reference's five configurations.
 
-One step = one pass of the hot path (query preparation + scan with fused top-k + merge) over the whole
+Default (what the driver runs): --config c2, the headline metric "QPS @ recall@10 (1M x 128 SQ8 scan)":
+one step = one pass of the hot path (query preparation + scan with fused top-k + merge) over the whole
 query batch, inputs resident in HBM.  Prints ONE JSON line with the metric, the roofline of the dominant
 kernel (HIP events recorded by the library around that kernel on its own stream) and the CPU baseline
 (the reference's own SIMD kernel compiled from its sources when oracle/_ref is present, else the CPU
 restatement), timed on this host's cores on a bounded sample of the same workload.
+
+Other configs (--config c1 | c3 | c4 | c5) print one line each in the same shape for the fp32 brute-force
+scan, k-means assignment, the IVF SQ4-uniform search and the RaBitQ scan + rerank.
 """
 import argparse
 import ctypes as C
@@ -21,19 +25,30 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
+MFMA_F32_PEAK_TFLOPS = 157.3
 
 
-def mixture(seed_means, seed_rows, n, d, components, sigma, means=None):
-    """Gaussian mixture drawn from MT19937 streams (means uniform[0,1)^d, isotropic sigma)."""
-    if means is None:
-        means = np.random.Generator(np.random.MT19937(seed_means)).random((components, d), dtype=np.float32)
-    rng = np.random.Generator(np.random.MT19937(seed_rows))
-    out = np.empty((n, d), np.float32)
-    step = 1 << 17
+def mt(seed):
+    return np.random.Generator(np.random.MT19937(seed))
+
+
+def mixture_chunks(seed_rows, n, d, means, sigma, step=1 << 17):
+    """Gaussian-mixture rows in chunks, drawn from one MT19937 stream."""
+    rng = mt(seed_rows)
     for s in range(0, n, step):
         e = min(n, s + step)
-        which = rng.integers(0, components, e - s)
-        out[s:e] = means[which] + np.float32(sigma) * rng.standard_normal((e - s, d), dtype=np.float32)
+        which = rng.integers(0, means.shape[0], e - s)
+        yield s, means[which] + np.float32(sigma) * rng.standard_normal((e - s, d), dtype=np.float32)
+
+
+def mixture(seed_means, seed_rows, n, d, components, sigma, means=None, normal_means=False):
+    if means is None:
+        g = mt(seed_means)
+        means = g.standard_normal((components, d), dtype=np.float32) if normal_means else \
+            g.random((components, d), dtype=np.float32)
+    out = np.empty((n, d), np.float32)
+    for s, blk in mixture_chunks(seed_rows, n, d, means, sigma):
+        out[s:s + blk.shape[0]] = blk
     return out, means
 
 
@@ -44,16 +59,11 @@ def exact_topk_host(x, q, k, metric):
     pre = min(n, 8 * k)
     cand_d = np.full((q.shape[0], 0), np.inf, np.float32)
     cand_i = np.zeros((q.shape[0], 0), np.int64)
-    xn = None
     chunk = 1 << 17
     for s in range(0, n, chunk):
         xb = x[s:s + chunk]
         ip = q @ xb.T
-        if metric == "l2":
-            xn = np.einsum("ij,ij->i", xb, xb)
-            dist = xn[None, :] - 2.0 * ip
-        else:
-            dist = -ip
+        dist = np.einsum("ij,ij->i", xb, xb)[None, :] - 2.0 * ip if metric == "l2" else -ip
         m = min(pre, dist.shape[1])
         part = np.argpartition(dist, m - 1, axis=1)[:, :m]
         cand_d = np.concatenate([cand_d, np.take_along_axis(dist, part, 1)], 1)
@@ -79,95 +89,127 @@ def recall_at_k(ids, gt):
     return hits / float(gt.size)
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--n", type=int, default=1000000)
-    ap.add_argument("--dim", type=int, default=128)
-    ap.add_argument("--nq", type=int, default=10000)
-    ap.add_argument("--k", type=int, default=10)
-    ap.add_argument("--tile", type=int, default=0, help="query tile override (0 = library default)")
-    ap.add_argument("--chunks", type=int, default=0, help="base chunk override (0 = library default)")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-recall", action="store_true", help="skip the recall check")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: the search core is single-GPU by design (see DESIGN.md); "
-              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
-        sys.exit(2)
+class Env:
+    def __init__(self, args):
+        from vsag_amd import capi
+        self.capi = capi
+        self.lib = capi.load_library()
+        capi.init(0)
+        self.dev_name, self.cus, self.hbm = capi.device_info()
+        self.args = args
+        capi.check(self.lib.vsag_amd_set_kernel_timing(1))
 
-    from vsag_amd import capi
-    lib = capi.load_library()
-    capi.init(0)
-    dev_name, cus, hbm = capi.device_info()
-    n, d, nq, k = args.n, args.dim, args.nq, args.k
+    def buf(self, nbytes):
+        return self.capi.DeviceBuffer(nbytes)
 
+    def upload(self, arr):
+        return self.capi.DeviceBuffer.from_numpy(arr)
+
+    def kernel_ms(self):
+        ms = C.c_float()
+        self.capi.check(self.lib.vsag_amd_last_kernel_ms(C.byref(ms)))
+        return ms.value
+
+    def make_store(self, kind, metric, dim, lb=None, diff=None, bounds=None, rot=None, cen=None, qbits=4):
+        p = self.capi.StoreParams()
+        p.kind, p.metric, p.dim, p.rabitq_query_bits = kind, metric, dim, qbits
+        if lb is not None:
+            p.lower_bound_dev, p.diff_dev = lb.ptr, diff.ptr
+        if bounds is not None:
+            p.lower_bound_dev = bounds.ptr
+        if rot is not None:
+            p.rotation_dev, p.centroid_dev = rot.ptr, cen.ptr
+        h = C.c_void_p()
+        self.capi.check(self.lib.vsag_amd_store_create(C.byref(p), C.byref(h)))
+        return h
+
+    def timed(self, step, steps, warmup):
+        for _ in range(warmup):
+            step()
+        self.capi.synchronize()
+        kms = []
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+            kms.append(self.kernel_ms())
+        self.capi.synchronize()
+        wall = time.perf_counter() - t0
+        return wall / steps, float(np.mean(kms))
+
+    def flat_scan_fn(self, store, q_dev, nq, k, ids_dev, ds_dev):
+        wsb = self.lib.vsag_amd_flat_scan_workspace_bytes(store, nq, k)
+        ws = self.buf(wsb)
+
+        def step():
+            self.capi.check(self.lib.vsag_amd_flat_scan_topk(store, q_dev.ptr, nq, k, ids_dev.ptr, ds_dev.ptr, ws.ptr,
+                                                             wsb, None))
+        return step, ws
+
+    def scan_info(self):
+        tile, passes, bpp = C.c_int(), C.c_uint64(), C.c_uint64()
+        self.lib.vsag_amd_last_scan_info(C.byref(tile), C.byref(passes), C.byref(bpp))
+        return tile.value, passes.value, bpp.value
+
+    def base_line(self, metric, unit, value, sec_per_step, dtype, workload, extra, roofline, cpu):
+        cfg = {"workload": workload, "device": self.dev_name, "compute_units": self.cus}
+        cfg.update(extra)
+        return {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": self.args.steps,
+                "warmup": self.args.warmup, "ms_per_step": 1e3 * sec_per_step, "higher_is_better": True,
+                "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic", "config": cfg,
+                "roofline": roofline, "cpu_baseline": cpu}
+
+
+# ------------------------------------------------------------------------------------------- C2 (headline)
+def run_c2(env):
+    args, capi, lib = env.args, env.capi, env.lib
+    n, d, nq, k = args.n or 1000000, args.dim or 128, args.nq or 10000, args.k
     t0 = time.time()
     x, means = mixture(315, 47, n, d, 1000, 0.05)
     q, _ = mixture(315, 165, nq, d, 1000, 0.05, means=means)
     t_gen = time.time() - t0
 
     # Build on the device: train bounds, encode, re-tile (Index::Build of the reference's brute_force).
-    x_dev = capi.DeviceBuffer.from_numpy(x)
-    lb_dev, diff_dev = capi.DeviceBuffer(d * 4), capi.DeviceBuffer(d * 4)
+    x_dev = env.upload(x)
+    lb_dev, diff_dev = env.buf(d * 4), env.buf(d * 4)
     wsb = lib.vsag_amd_sq_train_workspace_bytes(n, d, 0)
-    ws = capi.DeviceBuffer(wsb)
+    ws = env.buf(wsb)
     t0 = time.time()
     capi.check(lib.vsag_amd_sq_train(x_dev.ptr, n, d, 8, capi.METRIC_L2, capi.SQ_TRAIN_TRUNC_BOUND, 0.05, 0,
                                      lb_dev.ptr, diff_dev.ptr, ws.ptr, wsb, None))
-    codes_dev = capi.DeviceBuffer(n * d)
+    codes_dev = env.buf(n * d)
     capi.check(lib.vsag_amd_sq_encode(x_dev.ptr, n, d, 8, capi.METRIC_L2, lb_dev.ptr, diff_dev.ptr, codes_dev.ptr,
                                       None))
     stores = {}
     for name, metric in (("l2", capi.METRIC_L2), ("ip", capi.METRIC_IP)):
-        p = capi.StoreParams()
-        p.kind, p.metric, p.dim = capi.KIND_SQ8, metric, d
-        p.lower_bound_dev, p.diff_dev = lb_dev.ptr, diff_dev.ptr
-        h = C.c_void_p()
-        capi.check(lib.vsag_amd_store_create(C.byref(p), C.byref(h)))
-        capi.check(lib.vsag_amd_store_append(h, codes_dev.ptr, n, None))
-        stores[name] = h
+        stores[name] = env.make_store(capi.KIND_SQ8, metric, d, lb=lb_dev, diff=diff_dev)
+        capi.check(lib.vsag_amd_store_append(stores[name], codes_dev.ptr, n, None))
     capi.synchronize()
     t_build = time.time() - t0
     ws.free()
+    x_dev.free()
 
-    q_dev = capi.DeviceBuffer.from_numpy(q)
-    ids_dev, ds_dev = capi.DeviceBuffer(nq * k * 4), capi.DeviceBuffer(nq * k * 4)
+    q_dev = env.upload(q)
+    ids_dev, ds_dev = env.buf(nq * k * 4), env.buf(nq * k * 4)
     capi.check(lib.vsag_amd_set_scan_tuning(args.tile, args.chunks))
-    capi.check(lib.vsag_amd_set_kernel_timing(1))
-
     results = {}
     for name in ("ip", "l2"):  # l2 last: it is the headline line
-        h = stores[name]
-        wsb = lib.vsag_amd_flat_scan_workspace_bytes(h, nq, k)
-        ws = capi.DeviceBuffer(wsb)
-
-        def step():
-            capi.check(lib.vsag_amd_flat_scan_topk(h, q_dev.ptr, nq, k, ids_dev.ptr, ds_dev.ptr, ws.ptr, wsb, None))
-
-        for _ in range(args.warmup):
-            step()
-        capi.synchronize()
-        kernel_ms = []
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-            ms = C.c_float()
-            capi.check(lib.vsag_amd_last_kernel_ms(C.byref(ms)))
-            kernel_ms.append(ms.value)
-        capi.synchronize()
-        wall = time.perf_counter() - t0
-        tile, passes, bytes_per_pass = C.c_int(), C.c_uint64(), C.c_uint64()
-        lib.vsag_amd_last_scan_info(C.byref(tile), C.byref(passes), C.byref(bytes_per_pass))
-        ids = ids_dev.to_numpy(np.uint32, (nq, k))
-        results[name] = dict(ms_per_step=1e3 * wall / args.steps, qps=nq * args.steps / wall,
-                             kernel_ms=float(np.mean(kernel_ms)), tile=tile.value, passes=passes.value,
-                             bytes_per_pass=bytes_per_pass.value, ids=ids)
+        step, ws = env.flat_scan_fn(stores[name], q_dev, nq, k, ids_dev, ds_dev)
+        sec, kms = env.timed(step, args.steps, args.warmup)
+        tile, passes, bpp = env.scan_info()
+        results[name] = dict(sec=sec, qps=nq / sec, kernel_ms=kms, tile=tile, passes=passes, bytes_per_pass=bpp,
+                             ids=ids_dev.to_numpy(np.uint32, (nq, k)))
         ws.free()
 
-    # recall@10 against exact brute force on the raw fp32 vectors (host, fp64 distances) on the first queries
+    # one query per call (the reference's own call pattern): a single streaming pass over the codes
+    single = None
+    if not args.no_single:
+        step, ws = env.flat_scan_fn(stores["l2"], q_dev, 1, k, ids_dev, ds_dev)
+        sec, kms = env.timed(step, 50, 5)
+        _, _, bpp = env.scan_info()
+        single = {"latency_us": 1e6 * sec, "kernel_us": 1e3 * kms, "hbm_gbs": bpp / (kms * 1e-3) / 1e9,
+                  "hbm_frac": bpp / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        ws.free()
+
     recall = {}
     if not args.no_recall:
         nrec = min(nq, 500)
@@ -175,7 +217,6 @@ def main():
             gt = exact_topk_host(x, q[:nrec], k, name)
             recall[name] = recall_at_k(results[name]["ids"][:nrec], gt)
 
-    # CPU baseline on a bounded sample of the same workload
     cpu = None
     if not args.no_cpu:
         import oracle as orc
@@ -186,7 +227,6 @@ def main():
         isa = orc.ref_best_isa()
         fn = orc.ref_sq8_fn(orc.L2, isa)
         sample = min(nq, 8 * threads)
-        kind = "reference" if fn is not None else "port"
 
         def run_cpu(qs, th):
             if fn is not None:
@@ -201,46 +241,317 @@ def main():
         run_cpu(q[:2], 1)
         t_one = (time.perf_counter() - t0) / 2
         same = float(np.mean([len(set(a) & set(b)) / float(k) for a, b in zip(cids, results["l2"]["ids"][:sample])]))
-        cpu = {"value": sample / t_all, "unit": "queries/s", "cores": threads, "kind": kind,
+        cpu = {"value": sample / t_all, "unit": "queries/s", "cores": threads,
+               "kind": "reference" if fn is not None else "port",
                "sample": "%d of the %d queries over all %d codes, one query per call, OpenMP dynamic over queries; "
                          "distance = %s, loop and heap = restated BruteForce::SearchWithRequest" %
                          (sample, nq, n, ("vsag::%s::SQ8ComputeL2Sqr compiled from the reference sources" % isa)
                           if fn is not None else "CPU restatement (oracle)"),
                "single_thread_qps": 1.0 / t_one, "topk_overlap_with_gpu": same}
 
-    r = results["l2"]
+    r, ri = results["l2"], results["ip"]
     algo_bytes = r["passes"] * r["bytes_per_pass"]
     achieved = algo_bytes / (r["kernel_ms"] * 1e-3) / 1e9
-    ri = results["ip"]
-    out = {
-        "metric": "QPS @ recall@10 (1M x 128 SQ8 scan)",
-        "value": r["qps"],
-        "unit": "queries/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": r["ms_per_step"],
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "u8 codes, f32 accumulate",
-        "data": "synthetic",
-        "config": {
-            "workload": "configs[1]: flat SQ8 scan, N=%d, d=%d, %d queries, k=%d, L2 (headline) and IP" % (n, d, nq, k),
-            "recall_at_10_l2": recall.get("l2"), "recall_at_10_ip": recall.get("ip"),
-            "ip_qps": ri["qps"], "ip_ms_per_step": ri["ms_per_step"], "ip_query_tile": ri["tile"],
-            "ip_kernel_ms": ri["kernel_ms"],
-            "ip_algorithmic_gbs": ri["passes"] * ri["bytes_per_pass"] / (ri["kernel_ms"] * 1e-3) / 1e9,
-            "query_tile": r["tile"], "passes_per_step": r["passes"], "bytes_per_pass": r["bytes_per_pass"],
-            "build_seconds": t_build, "datagen_seconds": t_gen, "device": dev_name, "compute_units": cus,
-        },
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "flat_scan_kernel<sq8, l2, T=%d>" % r["tile"], "kernel_ms": r["kernel_ms"],
-                     "algorithmic_bytes_per_launch": algo_bytes},
-        "cpu_baseline": cpu,
-    }
-    print(json.dumps(out))
+    extra = {"recall_at_10_l2": recall.get("l2"), "recall_at_10_ip": recall.get("ip"),
+             "ip_qps": ri["qps"], "ip_ms_per_step": 1e3 * ri["sec"], "ip_query_tile": ri["tile"],
+             "ip_kernel_ms": ri["kernel_ms"],
+             "ip_algorithmic_gbs": ri["passes"] * ri["bytes_per_pass"] / (ri["kernel_ms"] * 1e-3) / 1e9,
+             "query_tile": r["tile"], "passes_per_step": r["passes"], "bytes_per_pass": r["bytes_per_pass"],
+             "single_query_l2": single, "build_seconds": t_build, "datagen_seconds": t_gen}
+    roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+            "kernel": "flat_scan_kernel<sq8, l2, T=%d>" % r["tile"], "kernel_ms": r["kernel_ms"],
+            "algorithmic_bytes_per_launch": algo_bytes}
+    return env.base_line("QPS @ recall@10 (1M x 128 SQ8 scan)", "queries/s", r["qps"], r["sec"],
+                         "u8 codes, f32 accumulate",
+                         "configs[1]: flat SQ8 scan, N=%d, d=%d, %d queries, k=%d, L2 (headline) and IP" % (n, d, nq, k),
+                         extra, roof, cpu)
+
+
+# ------------------------------------------------------------------------------------------- C1
+def run_c1(env):
+    args, capi, lib = env.args, env.capi, env.lib
+    n, d, nq, k = args.n or 100000, args.dim or 128, args.nq or 1000, args.k
+    x = mt(47).random((n, d), dtype=np.float32)
+    q = mt(165).random((nq, d), dtype=np.float32)
+    store = env.make_store(capi.KIND_FP32, capi.METRIC_L2, d)
+    x_dev = env.upload(x)
+    capi.check(lib.vsag_amd_store_append(store, x_dev.ptr, n, None))
+    q_dev = env.upload(q)
+    ids_dev, ds_dev = env.buf(nq * k * 4), env.buf(nq * k * 4)
+    capi.check(lib.vsag_amd_set_scan_tuning(args.tile, args.chunks))
+    step, ws = env.flat_scan_fn(store, q_dev, nq, k, ids_dev, ds_dev)
+    sec, kms = env.timed(step, args.steps, args.warmup)
+    tile, passes, bpp = env.scan_info()
+    ids = ids_dev.to_numpy(np.uint32, (nq, k))
+    rec = None if args.no_recall else recall_at_k(ids[:200], exact_topk_host(x, q[:200], k, "l2"))
+    cpu = None
+    if not args.no_cpu:
+        import oracle as orc
+        threads = min(os.cpu_count() or 1, 16)
+        sample = min(nq, 16 * threads)
+        codes = x.view(np.uint8).reshape(n, 4 * d)
+        orc.flat_scan_topk(orc.FP32, orc.L2, d, codes, q[:threads], k, threads=threads)
+        t0 = time.perf_counter()
+        orc.flat_scan_topk(orc.FP32, orc.L2, d, codes, q[:sample], k, threads=threads)
+        cpu = {"value": sample / (time.perf_counter() - t0), "unit": "queries/s", "cores": threads, "kind": "port",
+               "sample": "%d of the %d queries over all %d vectors, CPU restatement of generic::FP32ComputeL2Sqr + "
+                         "BruteForce loop, OpenMP over queries" % (sample, nq, n)}
+    algo = passes * bpp
+    achieved = algo / (kms * 1e-3) / 1e9
+    roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+            "traffic": None, "kernel": "flat_scan_kernel<fp32, l2, T=%d>" % tile, "kernel_ms": kms,
+            "algorithmic_bytes_per_launch": algo, "flops_per_launch": 2.0 * n * d * nq,
+            "tflops": 2.0 * n * d * nq / (kms * 1e-3) / 1e12}
+    return env.base_line("QPS @ recall@10 (100k x 128 fp32 brute force)", "queries/s", nq / sec, sec, "f32",
+                         "configs[0]: brute_force fp32 L2, N=%d, d=%d, %d queries, k=%d" % (n, d, nq, k),
+                         {"recall_at_10": rec, "query_tile": tile, "passes_per_step": passes, "bytes_per_pass": bpp},
+                         roof, cpu)
+
+
+# ------------------------------------------------------------------------------------------- C3
+def run_c3(env):
+    args, capi, lib = env.args, env.capi, env.lib
+    n, d, k, iters = args.n or 1000000, args.dim or 960, args.nlist or 4096, 10
+    means = mt(315).standard_normal((k, d), dtype=np.float32)
+    x_dev = env.buf(n * d * 4)
+    pick = np.sort(mt(7).choice(n, k, replace=False))  # seeded random-sample initial centroids
+    init = np.empty((k, d), np.float32)
+    sample_rows = []
+    t0 = time.time()
+    for s, blk in mixture_chunks(47, n, d, means, 0.2, step=1 << 15):
+        capi.check(lib.vsag_amd_memcpy_h2d(x_dev.ptr + s * d * 4, blk.ctypes.data, blk.nbytes, None))
+        lo, hi = np.searchsorted(pick, [s, s + blk.shape[0]])
+        init[lo:hi] = blk[pick[lo:hi] - s]
+        if s < (1 << 15):
+            sample_rows.append(blk[:8192].copy())
+    t_gen = time.time() - t0
+    cent = env.upload(init)
+    labels, loss = env.buf(n * 4), env.buf(8)
+    wsb = lib.vsag_amd_kmeans_assign_workspace_bytes(n, d, k)
+    ws = env.buf(wsb)
+
+    def step():
+        capi.check(lib.vsag_amd_kmeans_assign(x_dev.ptr, n, d, cent.ptr, k, labels.ptr, None, loss.ptr, ws.ptr, wsb,
+                                              None))
+    sec, kms = env.timed(step, args.steps, args.warmup)
+    ws.free()
+    # the full Lloyd run: 10 iterations from the same initial centroids
+    cent2 = env.upload(init)
+    wsb = lib.vsag_amd_kmeans_run_workspace_bytes(n, d, k)
+    ws = env.buf(wsb)
+    final = C.c_double()
+    t0 = time.perf_counter()
+    capi.check(lib.vsag_amd_kmeans_run(x_dev.ptr, n, d, cent2.ptr, k, iters, 7, labels.ptr, C.byref(final), ws.ptr, wsb,
+                                       None))
+    t_run = time.perf_counter() - t0
+    cpu = None
+    if not args.no_cpu:
+        import oracle as orc
+        xs = sample_rows[0]
+        threads = min(os.cpu_count() or 1, 16)
+        orc.kmeans_assign(xs[:256], init)
+        t0 = time.perf_counter()
+        ol, _, oloss = orc.kmeans_assign(xs, init)
+        t_cpu = time.perf_counter() - t0
+        gl = labels  # noqa: F841
+        step()
+        capi.synchronize()
+        glabels = labels.to_numpy(np.int32, (n,))[:xs.shape[0]]
+        cpu = {"value": xs.shape[0] / t_cpu, "unit": "rows/s", "cores": threads, "kind": "port",
+               "sample": "first %d of the %d rows against all %d centroids, CPU restatement of "
+                         "find_nearest_one_with_blas (scalar dot instead of OpenBLAS SGEMM), OpenMP over rows" %
+                         (xs.shape[0], n, k),
+               "label_agreement_with_gpu": float((ol == glabels).mean())}
+    flops = 2.0 * n * k * d
+    tf = flops / (kms * 1e-3) / 1e12
+    roof = {"bound": "mfma", "achieved": tf, "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": tf / MFMA_F32_PEAK_TFLOPS, "traffic": None, "kernel": "kmeans_assign_kernel", "kernel_ms": kms,
+            "flops_per_launch": flops}
+    return env.base_line("k-means assign rows/s", "rows/s", n / sec, sec, "f32",
+                         "configs[2]: k-means assignment, N=%d, d=%d, k=%d (one step = one assignment pass)" % (n, d, k),
+                         {"lloyd_iterations": iters, "lloyd_seconds": t_run, "final_loss": final.value,
+                          "datagen_seconds": t_gen}, roof, cpu)
+
+
+# ------------------------------------------------------------------------------------------- C4
+def run_c4(env):
+    args, capi, lib = env.args, env.capi, env.lib
+    n, d, nq, k = args.n or 10000000, args.dim or 128, args.nq or 10000, args.k
+    nlist, nprobe, kcand = args.nlist or 4096, 64, 100
+    means = mt(315).random((10000, d), dtype=np.float32)
+    x_dev = env.buf(n * d * 4)
+    pick = np.sort(mt(7).choice(n, nlist, replace=False))
+    init = np.empty((nlist, d), np.float32)
+    for s, blk in mixture_chunks(47, n, d, means, 0.05):
+        capi.check(lib.vsag_amd_memcpy_h2d(x_dev.ptr + s * d * 4, blk.ctypes.data, blk.nbytes, None))
+        lo, hi = np.searchsorted(pick, [s, s + blk.shape[0]])
+        init[lo:hi] = blk[pick[lo:hi] - s]
+    q, _ = mixture(315, 165, nq, d, 10000, 0.05, means=means)
+    t0 = time.perf_counter()
+    # train on a sample (the first 262144 rows), assign everything, encode, build the lists
+    ns = min(n, 64 * nlist)
+    cent = env.upload(init)
+    slabels = env.buf(ns * 4)
+    wsb = lib.vsag_amd_kmeans_run_workspace_bytes(ns, d, nlist)
+    ws = env.buf(wsb)
+    capi.check(lib.vsag_amd_kmeans_run(x_dev.ptr, ns, d, cent.ptr, nlist, 10, 7, slabels.ptr, None, ws.ptr, wsb, None))
+    ws.free()
+    labels = env.buf(n * 4)
+    wsb = lib.vsag_amd_kmeans_assign_workspace_bytes(n, d, nlist)
+    ws = env.buf(wsb)
+    capi.check(lib.vsag_amd_kmeans_assign(x_dev.ptr, n, d, cent.ptr, nlist, labels.ptr, None, None, ws.ptr, wsb, None))
+    ws.free()
+    bounds = env.buf(8)
+    wsb = lib.vsag_amd_sq_train_workspace_bytes(ns, d, 0)
+    ws = env.buf(wsb)
+    capi.check(lib.vsag_amd_sq_train_uniform(x_dev.ptr, ns, d, 4, capi.METRIC_L2, capi.SQ_TRAIN_TRUNC_BOUND, 0.05, 0,
+                                             bounds.ptr, ws.ptr, wsb, None))
+    ws.free()
+    cs = int(lib.vsag_amd_code_size(capi.KIND_SQ4_UNIFORM, capi.METRIC_L2, d, 0))
+    codes = env.buf(n * cs)
+    capi.check(lib.vsag_amd_squ_encode(x_dev.ptr, n, d, 4, capi.METRIC_L2, bounds.ptr, codes.ptr, None))
+    lists = env.make_store(capi.KIND_SQ4_UNIFORM, capi.METRIC_L2, d, bounds=bounds)
+    capi.check(lib.vsag_amd_store_set_lists(lists, codes.ptr, labels.ptr, n, nlist, None))
+    cstore = env.make_store(capi.KIND_FP32, capi.METRIC_L2, d)
+    capi.check(lib.vsag_amd_store_append(cstore, cent.ptr, nlist, None))
+    capi.synchronize()
+    t_build = time.perf_counter() - t0
+    codes.free()
+    sizes = np.zeros(nlist, np.uint32)
+    capi.check(lib.vsag_amd_store_list_sizes(lists, sizes.ctypes.data, nlist))
+
+    q_dev = env.upload(q)
+    buckets, bd = env.buf(nq * nprobe * 4), env.buf(nq * nprobe * 4)
+    cand, cand_d = env.buf(nq * kcand * 4), env.buf(nq * kcand * 4)
+    out_i, out_d = env.buf(nq * k * 4), env.buf(nq * k * 4)
+    wr = lib.vsag_amd_ivf_route_workspace_bytes(cstore, nq, nprobe)
+    wsc = lib.vsag_amd_ivf_scan_workspace_bytes(lists, nq, nprobe, kcand)
+    ws = env.buf(max(wr, wsc))
+
+    def step():
+        capi.check(lib.vsag_amd_ivf_route(cstore, q_dev.ptr, nq, nprobe, buckets.ptr, bd.ptr, ws.ptr, wr, None))
+        capi.check(lib.vsag_amd_ivf_scan_topk(lists, q_dev.ptr, nq, buckets.ptr, nprobe, kcand, cand.ptr, cand_d.ptr,
+                                              ws.ptr, wsc, None))
+        capi.check(lib.vsag_amd_rerank_fp32(x_dev.ptr, n, d, capi.METRIC_L2, q_dev.ptr, nq, cand.ptr, kcand, k,
+                                            out_i.ptr, out_d.ptr, None))
+    sec, kms = env.timed(step, args.steps, args.warmup)
+    ids = out_i.to_numpy(np.uint32, (nq, k))
+    b = buckets.to_numpy(np.int32, (nq, nprobe))
+    scanned = sizes[b.clip(0)].astype(np.int64).sum()  # codes scanned per step, summed over queries
+    algo = float(scanned) * (cs + 4)
+    rec = None
+    if not args.no_recall:
+        # exact fp32 ground truth from the library's own fp32 flat scan (checked against the CPU checker in tests)
+        flat = env.make_store(capi.KIND_FP32, capi.METRIC_L2, d)
+        capi.check(lib.vsag_amd_store_append(flat, x_dev.ptr, n, None))
+        nrec = min(nq, 1000)
+        gi, gd = env.buf(nrec * k * 4), env.buf(nrec * k * 4)
+        st, w2 = env.flat_scan_fn(flat, q_dev, nrec, k, gi, gd)
+        st()
+        rec = recall_at_k(ids[:nrec], gi.to_numpy(np.uint32, (nrec, k)))
+        w2.free()
+        lib.vsag_amd_store_destroy(flat)
+    achieved = algo / (kms * 1e-3) / 1e9
+    roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+            "traffic": None, "kernel": "ivf_scan_kernel<sq4_uniform, l2>", "kernel_ms": kms,
+            "algorithmic_bytes_per_launch": algo}
+    return env.base_line("QPS @ recall@10 (IVF SQ4-uniform, 10M x 128)", "queries/s", nq / sec, sec,
+                         "u4 codes, i32 dot", "configs[3]: IVF search, N=%d, d=%d, nlist=%d, nprobe=%d, rerank %d, "
+                         "%d queries, k=%d" % (n, d, nlist, nprobe, kcand, nq, k),
+                         {"recall_at_10": rec, "build_seconds": t_build, "scanned_codes_per_query": float(scanned) / nq,
+                          "bytes_per_scanned_code": cs + 4}, roof, None)
+
+
+# ------------------------------------------------------------------------------------------- C5
+def run_c5(env):
+    args, capi, lib = env.args, env.capi, env.lib
+    n, d, nq, k, kcand = args.n or 5000000, args.dim or 768, args.nq or 10000, args.k, 200
+    x_dev = env.buf(n * d * 4)
+    rng = mt(47)
+    step_rows = 1 << 15
+    for s in range(0, n, step_rows):
+        blk = rng.standard_normal((min(step_rows, n - s), d), dtype=np.float32)
+        blk /= np.linalg.norm(blk, axis=1, keepdims=True)
+        capi.check(lib.vsag_amd_memcpy_h2d(x_dev.ptr + s * d * 4, blk.ctypes.data, blk.nbytes, None))
+    q = mt(165).standard_normal((nq, d), dtype=np.float32)
+    q /= np.linalg.norm(q, axis=1, keepdims=True)
+    g = mt(315).standard_normal((d, d))
+    rot, r = np.linalg.qr(g)
+    rot = (rot * np.sign(np.diag(r))).astype(np.float32)  # seeded Gaussian -> QR, passed to CPU and GPU alike
+    t0 = time.perf_counter()
+    rot_dev = env.upload(rot)
+    cen = env.buf(d * 4)
+    capi.check(lib.vsag_amd_rabitq_train(x_dev.ptr, n, d, rot_dev.ptr, cen.ptr, None))
+    cs = int(lib.vsag_amd_code_size(capi.KIND_RABITQ, capi.METRIC_IP, d, 4))
+    codes = env.buf(n * cs)
+    capi.check(lib.vsag_amd_rabitq_encode(x_dev.ptr, n, d, rot_dev.ptr, cen.ptr, capi.METRIC_IP, 4, codes.ptr, None))
+    store = env.make_store(capi.KIND_RABITQ, capi.METRIC_IP, d, rot=rot_dev, cen=cen, qbits=4)
+    capi.check(lib.vsag_amd_store_append(store, codes.ptr, n, None))
+    capi.synchronize()
+    t_build = time.perf_counter() - t0
+    codes.free()
+    q_dev = env.upload(q)
+    cand, cand_d = env.buf(nq * kcand * 4), env.buf(nq * kcand * 4)
+    out_i, out_d = env.buf(nq * k * 4), env.buf(nq * k * 4)
+    capi.check(lib.vsag_amd_set_scan_tuning(args.tile, args.chunks))
+    scan, ws = env.flat_scan_fn(store, q_dev, nq, kcand, cand, cand_d)
+
+    def step():
+        scan()
+        capi.check(lib.vsag_amd_rerank_fp32(x_dev.ptr, n, d, capi.METRIC_IP, q_dev.ptr, nq, cand.ptr, kcand, k,
+                                            out_i.ptr, out_d.ptr, None))
+    sec, kms = env.timed(step, args.steps, args.warmup)
+    tile, passes, bpp = env.scan_info()
+    ids = out_i.to_numpy(np.uint32, (nq, k))
+    rec = None
+    if not args.no_recall:
+        flat = env.make_store(capi.KIND_FP32, capi.METRIC_IP, d)
+        capi.check(lib.vsag_amd_store_append(flat, x_dev.ptr, n, None))
+        nrec = min(nq, 500)
+        gi, gd = env.buf(nrec * k * 4), env.buf(nrec * k * 4)
+        st, w2 = env.flat_scan_fn(flat, q_dev, nrec, k, gi, gd)
+        st()
+        rec = recall_at_k(ids[:nrec], gi.to_numpy(np.uint32, (nrec, k)))
+        w2.free()
+        lib.vsag_amd_store_destroy(flat)
+    algo = passes * n * float(cs)
+    achieved = algo / (kms * 1e-3) / 1e9
+    roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+            "traffic": None, "kernel": "flat_scan_kernel<rabitq, ip, T=%d>" % tile, "kernel_ms": kms,
+            "algorithmic_bytes_per_launch": algo}
+    return env.base_line("QPS @ recall@10 (RaBitQ 1-bit scan + rerank 200, 5M x 768)", "queries/s", nq / sec, sec,
+                         "1-bit codes x 4-bit queries, u32 popcount",
+                         "configs[4]: RaBitQ full scan + fp32 rerank of %d, N=%d, d=%d, %d queries, k=%d, IP" %
+                         (kcand, n, d, nq, k),
+                         {"recall_at_10": rec, "build_seconds": t_build, "query_tile": tile, "passes_per_step": passes,
+                          "bytes_per_code": cs}, roof, None)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--n", type=int, default=0)
+    ap.add_argument("--dim", type=int, default=0)
+    ap.add_argument("--nq", type=int, default=0)
+    ap.add_argument("--nlist", type=int, default=0)
+    ap.add_argument("--k", type=int, default=10)
+    ap.add_argument("--tile", type=int, default=0, help="query tile override (0 = library default)")
+    ap.add_argument("--chunks", type=int, default=0, help="base chunk override (0 = library default)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-recall", action="store_true", help="skip the recall check")
+    ap.add_argument("--no-single", action="store_true", help="skip the one-query-per-call measurement")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the search core is single-GPU by design (DESIGN.md says how it would "
+              "shard); --gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    env = Env(args)
+    line = {"c1": run_c1, "c2": run_c2, "c3": run_c3, "c4": run_c4, "c5": run_c5}[args.config](env)
+    print(json.dumps(line))
 
 
 if __name__ == "__main__":
