@@ -258,8 +258,13 @@ def run_c2(env):
              "ip_algorithmic_gbs": ri["passes"] * ri["bytes_per_pass"] / (ri["kernel_ms"] * 1e-3) / 1e9,
              "query_tile": r["tile"], "passes_per_step": r["passes"], "bytes_per_pass": r["bytes_per_pass"],
              "single_query_l2": single, "build_seconds": t_build, "datagen_seconds": t_gen}
+    # HBM/fabric bytes of one launch of this exact configuration, from rocprofv3 --pmc FETCH_SIZE (x 2.00, the
+    # factor that makes kernels of known size read their size) + WRITE_SIZE (x 1.00): profiles/flat_scan_sq8_c2.md.
+    traffic = None
+    if (n, d, nq, k, r["tile"]) == (1000000, 128, 10000, 10, 4):
+        traffic = 111504620 * 2.00 * 1024 + 32254 * 1024
     roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+            "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
             "kernel": "flat_scan_kernel<sq8, l2, T=%d>" % r["tile"], "kernel_ms": r["kernel_ms"],
             "algorithmic_bytes_per_launch": algo_bytes}
     return env.base_line("QPS @ recall@10 (1M x 128 SQ8 scan)", "queries/s", r["qps"], r["sec"],
