@@ -82,6 +82,15 @@ def exact_topk_host(x, q, k, metric):
     return out
 
 
+def device_rows(env, x_dev, rows, d):
+    """Rows of a device-resident n x d fp32 matrix, copied one by one (a few thousand at most)."""
+    rows = np.asarray(rows, np.int64)
+    out = np.empty((rows.size, d), np.float32)
+    for i, r in enumerate(rows):
+        env.capi.check(env.lib.vsag_amd_memcpy_d2h(out[i].ctypes.data, x_dev.ptr + int(r) * d * 4, d * 4, None))
+    return out
+
+
 def recall_at_k(ids, gt):
     hits = 0
     for a, b in zip(ids, gt):
@@ -422,7 +431,6 @@ def run_c4(env):
     capi.check(lib.vsag_amd_store_append(cstore, cent.ptr, nlist, None))
     capi.synchronize()
     t_build = time.perf_counter() - t0
-    codes.free()
     sizes = np.zeros(nlist, np.uint32)
     capi.check(lib.vsag_amd_store_list_sizes(lists, sizes.ctypes.data, nlist))
 
@@ -446,6 +454,7 @@ def run_c4(env):
     scanned = sizes[b.clip(0)].astype(np.int64).sum()  # codes scanned per step, summed over queries
     algo = float(scanned) * (cs + 4)
     rec = None
+    gt_ids = None
     if not args.no_recall:
         # exact fp32 ground truth from the library's own fp32 flat scan (checked against the CPU checker in tests)
         flat = env.make_store(capi.KIND_FP32, capi.METRIC_L2, d)
@@ -454,18 +463,69 @@ def run_c4(env):
         gi, gd = env.buf(nrec * k * 4), env.buf(nrec * k * 4)
         st, w2 = env.flat_scan_fn(flat, q_dev, nrec, k, gi, gd)
         st()
-        rec = recall_at_k(ids[:nrec], gi.to_numpy(np.uint32, (nrec, k)))
+        gt_ids = gi.to_numpy(np.uint32, (nrec, k))
+        rec = recall_at_k(ids[:nrec], gt_ids)
         w2.free()
         lib.vsag_amd_store_destroy(flat)
+    cpu = None
+    if not args.no_cpu:
+        # CPU restatement of IVF::search + reorder on a sample of the same queries, routing injected (the GPU's
+        # exact routing), same codes and lists: candidates, reranked ids and recall must agree.
+        import oracle as orc
+        threads = min(os.cpu_count() or 1, 16)
+        sample = min(nq, 16 * threads)
+        hcodes = codes.to_numpy(np.uint8, (n, cs))
+        hlabels = labels.to_numpy(np.int32, (n,))
+        hb = bounds.to_numpy(np.float32, (2,))
+        offsets, order = orc.ivf_build_lists(hlabels, nlist)
+        posting = hcodes[order]
+        qcodes = orc.squ_encode(q[:sample], 4, hb[0], hb[1], orc.L2)
+        orc.ivf_scan(orc.SQ4U, orc.L2, d, posting, offsets, order, qcodes[:threads], b[:threads], kcand,
+                     lb=hb[0], diff=hb[1], threads=threads)
+        t0 = time.perf_counter()
+        cids, cds = orc.ivf_scan(orc.SQ4U, orc.L2, d, posting, offsets, order, qcodes, b[:sample], kcand,
+                                 lb=hb[0], diff=hb[1], threads=threads)
+        t_cpu = time.perf_counter() - t0
+        gcand = cand.to_numpy(np.uint32, (nq, kcand))[:sample]
+        gcd = cand_d.to_numpy(np.float32, (nq, kcand))[:sample]
+        uniq = np.unique(cids[cids != 0xFFFFFFFF])
+        raw = device_rows(env, x_dev, uniq, d)
+        pos = {int(v): i for i, v in enumerate(uniq)}
+        rids = np.empty((sample, k), np.uint32)
+        for i in range(sample):
+            rows = raw[[pos[int(v)] for v in cids[i]]]
+            dd = ((rows.astype(np.float64) - q[i].astype(np.float64)) ** 2).sum(1)
+            rids[i] = cids[i][np.lexsort((cids[i], dd))[:k]]
+        cpu = {"value": sample / t_cpu, "unit": "queries/s", "cores": threads, "kind": "port",
+               "sample": "%d of the %d queries, CPU restatement of IVF::search (scan of the same %d probed lists per "
+                         "query with the strict-< heap) on the same SQ4-uniform codes, OpenMP over queries; rerank in "
+                         "fp64 on the host" % (sample, nq, nprobe),
+               "candidate_distances_bit_equal": bool(np.array_equal(cds.view(np.uint32), gcd.view(np.uint32))),
+               "candidate_overlap_with_gpu": float(np.mean([len(set(a) & set(bb)) / float(kcand)
+                                                            for a, bb in zip(cids, gcand)])),
+               "topk_overlap_with_gpu": float(np.mean([len(set(a) & set(bb)) / float(k)
+                                                       for a, bb in zip(rids, ids[:sample])])),
+               "recall_at_10": None if gt_ids is None else recall_at_k(rids, gt_ids[:sample]),
+               "gpu_recall_at_10_same_queries": None if gt_ids is None else recall_at_k(ids[:sample], gt_ids[:sample])}
+    codes.free()
     achieved = algo / (kms * 1e-3) / 1e9
+    # One step launches the scan kernel twice (nearest list of every query first, then the other lists); kernel_ms,
+    # the algorithmic bytes (76 B per (query, scanned code), the reference's per-query list reads) and the traffic
+    # are the sums over both launches.  Traffic: rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this exact
+    # configuration, profiles/ivf_scan_sq4u_c4.md.  Work items that share a list are co-scheduled and read it
+    # through L2 once per <= 4 queries, so the fraction against HBM exceeds 1: this kernel is bound by VALU issue.
+    traffic = None
+    if (n, d, nq, k, nlist) == (10000000, 128, 10000, 10, 4096):
+        traffic = (471200.19 + 1633918.44) * 2.00 * 1024 + (10050.06 + 19932.66) * 1024
     roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None, "kernel": "ivf_scan_kernel<sq4_uniform, l2>", "kernel_ms": kms,
-            "algorithmic_bytes_per_launch": algo}
+            "traffic": traffic, "kernel": "ivf_scan_kernel<sq4_uniform, l2> (2 launches per step)", "kernel_ms": kms,
+            "algorithmic_bytes_per_launch": algo,
+            "distance_evaluations_per_second": float(scanned) / (kms * 1e-3)}
     return env.base_line("QPS @ recall@10 (IVF SQ4-uniform, 10M x 128)", "queries/s", nq / sec, sec,
                          "u4 codes, i32 dot", "configs[3]: IVF search, N=%d, d=%d, nlist=%d, nprobe=%d, rerank %d, "
                          "%d queries, k=%d" % (n, d, nlist, nprobe, kcand, nq, k),
                          {"recall_at_10": rec, "build_seconds": t_build, "scanned_codes_per_query": float(scanned) / nq,
-                          "bytes_per_scanned_code": cs + 4}, roof, None)
+                          "bytes_per_scanned_code": cs + 4}, roof, cpu)
 
 
 # ------------------------------------------------------------------------------------------- C5
@@ -495,7 +555,6 @@ def run_c5(env):
     capi.check(lib.vsag_amd_store_append(store, codes.ptr, n, None))
     capi.synchronize()
     t_build = time.perf_counter() - t0
-    codes.free()
     q_dev = env.upload(q)
     cand, cand_d = env.buf(nq * kcand * 4), env.buf(nq * kcand * 4)
     out_i, out_d = env.buf(nq * k * 4), env.buf(nq * k * 4)
@@ -510,6 +569,7 @@ def run_c5(env):
     tile, passes, bpp = env.scan_info()
     ids = out_i.to_numpy(np.uint32, (nq, k))
     rec = None
+    gt_ids = None
     if not args.no_recall:
         flat = env.make_store(capi.KIND_FP32, capi.METRIC_IP, d)
         capi.check(lib.vsag_amd_store_append(flat, x_dev.ptr, n, None))
@@ -517,20 +577,58 @@ def run_c5(env):
         gi, gd = env.buf(nrec * k * 4), env.buf(nrec * k * 4)
         st, w2 = env.flat_scan_fn(flat, q_dev, nrec, k, gi, gd)
         st()
-        rec = recall_at_k(ids[:nrec], gi.to_numpy(np.uint32, (nrec, k)))
+        gt_ids = gi.to_numpy(np.uint32, (nrec, k))
+        rec = recall_at_k(ids[:nrec], gt_ids)
         w2.free()
         lib.vsag_amd_store_destroy(flat)
+    cpu = None
+    if not args.no_cpu:
+        # CPU restatement of the RaBitQ scan (ProcessQueryImpl + ComputeQueryBaseImpl + heap) on a sample of the same
+        # queries against the same codes, then fp64 rerank of its 200 candidates.
+        import oracle as orc
+        threads = min(os.cpu_count() or 1, 16)
+        sample = min(nq, 2 * threads)
+        hcodes = codes.to_numpy(np.uint8, (n, cs))
+        hcen = cen.to_numpy(np.float32, (d,))
+        qcodes = orc.rabitq_process_query(q[:sample], rot, hcen, orc.IP, 4)
+        t0 = time.perf_counter()
+        cids, cds = orc.flat_scan_topk(orc.RABITQ, orc.IP, d, hcodes, qcodes, kcand, qbits=4, threads=threads)
+        t_cpu = time.perf_counter() - t0
+        gcand = cand.to_numpy(np.uint32, (nq, kcand))[:sample]
+        uniq = np.unique(cids)
+        raw = device_rows(env, x_dev, uniq, d)
+        pos = {int(v): i for i, v in enumerate(uniq)}
+        rids = np.empty((sample, k), np.uint32)
+        for i in range(sample):
+            rows = raw[[pos[int(v)] for v in cids[i]]]
+            dd = 1.0 - rows.astype(np.float64) @ q[i].astype(np.float64)
+            rids[i] = cids[i][np.lexsort((cids[i], dd))[:k]]
+        cpu = {"value": sample / t_cpu, "unit": "queries/s", "cores": threads, "kind": "port",
+               "sample": "%d of the %d queries over all %d codes, CPU restatement of RaBitQuantizer::ProcessQueryImpl + "
+                         "ComputeQueryBaseImpl + BruteForce heap, OpenMP over queries; rerank in fp64 on the host" %
+                         (sample, nq, n),
+               "candidate_overlap_with_gpu": float(np.mean([len(set(a) & set(bb)) / float(kcand)
+                                                            for a, bb in zip(cids, gcand)])),
+               "topk_overlap_with_gpu": float(np.mean([len(set(a) & set(bb)) / float(k)
+                                                       for a, bb in zip(rids, ids[:sample])])),
+               "recall_at_10": None if gt_ids is None else recall_at_k(rids, gt_ids[:sample]),
+               "gpu_recall_at_10_same_queries": None if gt_ids is None else recall_at_k(ids[:sample], gt_ids[:sample])}
+    codes.free()
     algo = passes * n * float(cs)
     achieved = algo / (kms * 1e-3) / 1e9
+    # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this exact configuration, profiles/flat_scan_rabitq_c5.md
+    traffic = None
+    if (n, d, nq, k, tile) == (5000000, 768, 10000, 10, 2):
+        traffic = 1051929650.94 * 2.00 * 1024 + 250734.91 * 1024
     roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None, "kernel": "flat_scan_kernel<rabitq, ip, T=%d>" % tile, "kernel_ms": kms,
+            "traffic": traffic, "kernel": "flat_scan_kernel<rabitq, ip, T=%d>" % tile, "kernel_ms": kms,
             "algorithmic_bytes_per_launch": algo}
     return env.base_line("QPS @ recall@10 (RaBitQ 1-bit scan + rerank 200, 5M x 768)", "queries/s", nq / sec, sec,
                          "1-bit codes x 4-bit queries, u32 popcount",
                          "configs[4]: RaBitQ full scan + fp32 rerank of %d, N=%d, d=%d, %d queries, k=%d, IP" %
                          (kcand, n, d, nq, k),
                          {"recall_at_10": rec, "build_seconds": t_build, "query_tile": tile, "passes_per_step": passes,
-                          "bytes_per_code": cs}, roof, None)
+                          "bytes_per_code": cs}, roof, cpu)
 
 
 def main():
