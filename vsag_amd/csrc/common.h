@@ -14,6 +14,16 @@ namespace vsag_amd {
 
 constexpr int kWave = 64;          // gfx950 wavefront width; one code tile holds 64 codes
 constexpr int kGranule = 16;       // bytes per lane per tile row (one dwordx4)
+constexpr int kMaxGroup = 8;       // most granule rows the scans fetch together
+// Readable bytes past the last tile of every tile buffer: the last group of a tile is fetched whole.
+constexpr size_t kTileSlackBytes = static_cast<size_t>(kMaxGroup - 1) * kWave * kGranule;
+
+// Granule rows fetched together by a wave that serves T queries: one query leaves registers for a deeper
+// prefetch, which a wave needs when few waves share the memory latency.
+template <int T>
+struct GroupOf {
+    static constexpr int value = T == 1 ? 8 : 4;
+};
 constexpr uint32_t kMaxTopK = 1024;
 constexpr uint64_t kInfKey = 0xFFFFFFFFFFFFFFFFull;
 

@@ -44,9 +44,8 @@ struct ScanArgs {
     float f0, f1, f2;       // uniform kinds: lb, scalar_rate, lb*lb
 };
 
-// Tile rows are consumed in groups of kGroup granules so that the loads of the next group can be in flight
+// Tile rows are consumed in groups of GROUP granules so that the loads of the next group can be in flight
 // while the current one is being multiplied (see TileStream below).
-constexpr int kGroup = 4;
 
 // Running sums of T queries against the code owned by this lane.
 template <int KIND, int T>
@@ -267,9 +266,11 @@ finish_distances(const ScanArgs& a, const uint32_t (&qidx)[T], uint64_t slot, co
 }
 
 // The sequence of granule groups one wave walks: tiles first, first + stride, ... below end; inside a tile
-// groups j0 = 0, kGroup, ...  `load` fetches a group into registers, `advance` steps to the next one.
+// groups j0 = 0, GROUP, ...  `load` fetches a group into registers, `advance` steps to the next one.
+template <int GROUP>
 struct TileStream {
-    const uint4* base;   // tiles + lane
+    const uint4* tiles;  // wave-uniform; a lane reads element `lane` of a 64-element granule row
+    uint32_t lane;
     uint64_t tile, end, stride;
     uint32_t j0, G;
 
@@ -277,19 +278,23 @@ struct TileStream {
     valid() const {
         return tile < end;
     }
+    // Always issues GROUP loads at fixed offsets from one row address, with no branch around any of them,
+    // so that the consumer can wait for this group alone while the next one stays in flight.  A stream that
+    // has run out reads `fallback` (any tile the caller knows to exist); the last group of a tile may run up
+    // to GROUP - 1 granules past it, into the next tile or the slack that every tile buffer ends with
+    // (kTileSlackBytes) -- those registers are never consumed.
     __device__ inline void
-    load(uint4 (&regs)[kGroup]) const {
-        const uint4* tp = base + (tile * G + j0) * kWave;
+    load(uint4 (&regs)[GROUP], uint64_t fallback) const {
+        const uint64_t t = tile < end ? tile : fallback;
+        const uint4* tp = tiles + (t * G + j0) * kWave + lane;
 #pragma unroll
-        for (int u = 0; u < kGroup; ++u) {
-            if (j0 + u < G) {
-                regs[u] = tp[u * kWave];
-            }
+        for (int u = 0; u < GROUP; ++u) {
+            regs[u] = tp[u * kWave];
         }
     }
     __device__ inline void
     advance() {
-        j0 += kGroup;
+        j0 += GROUP;
         if (j0 >= G) {
             j0 = 0;
             tile += stride;

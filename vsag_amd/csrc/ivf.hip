@@ -178,23 +178,24 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
 
     const uint32_t tbeg = as_const(v.list_tile)[b], tend = as_const(v.list_tile)[b + 1];
     const QueryRows<T> qrows = query_rows<T>(a, qidx);
-    TileStream cur{a.tiles + lane, tbeg, tend, 1, 0, a.G};
-    TileStream nxt = cur;
-    uint4 buf_a[kGroup], buf_b[kGroup];
+    constexpr int GROUP = GroupOf<T>::value;
+    TileStream<GROUP> cur{a.tiles, lane, tbeg, tend, 1, 0, a.G};
+    TileStream<GROUP> nxt = cur;
+    uint4 buf_a[GROUP], buf_b[GROUP];
     if (cur.valid()) {
-        cur.load(buf_a);
+        cur.load(buf_a, cur.tile);
     }
     Acc<KIND, T> acc;
     acc_reset(acc);
 
-    auto consume = [&](const uint4(&regs)[kGroup]) {
+    auto consume = [&](const uint4(&regs)[GROUP]) {
 #pragma unroll
-        for (int u = 0; u < kGroup; ++u) {
+        for (int u = 0; u < GROUP; ++u) {
             if (cur.j0 + u < a.G) {
                 accumulate_granule<KIND, METRIC, T>(a, qrows, cur.j0 + u, regs[u], acc);
             }
         }
-        if (cur.j0 + kGroup < a.G) {
+        if (cur.j0 + GROUP < a.G) {
             return;
         }
         const uint64_t slot = cur.tile * kWave + lane;
@@ -207,43 +208,39 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
         for (int t = 0; t < T; ++t) {
             uint64_t key = make_key(d[t], id);
             bool pass = valid && key < tau[t];
+            uint64_t mask = __ballot(pass);
+            if (mask == 0) {
+                continue;
+            }
             uint64_t* keys = sel + t * S;
-            cnt[t] = selector_append(keys, k, cnt[t], pass, key);
-            if (cnt[t] + kWave > S - k) {
+            uint32_t np = __popcll(mask);
+            if (k + cnt[t] + np > S) {
                 uint64_t th = selector_flush(keys, S, k, cnt[t], lane);
                 cnt[t] = 0;
                 if (pair[t] != 0xFFFFFFFFU) {
-                    uint32_t bound;
-                    if (th != kInfKey) {
-                        // This pair alone already holds k candidates at or below th.
-                        uint32_t mine = static_cast<uint32_t>(th >> 32);
-                        uint32_t old = lane == 0 ? atomicMin(&v.bound[qidx[t]], mine) : 0U;
-                        old = __builtin_amdgcn_readfirstlane(old);
-                        bound = old < mine ? old : mine;
-                    } else {
-                        bound = __builtin_amdgcn_readfirstlane(__atomic_load_n(&v.bound[qidx[t]], __ATOMIC_RELAXED));
-                    }
+                    // th finite: this pair alone already holds k candidates at or below th.
+                    uint32_t bound = lower_shared(&v.bound[qidx[t]], static_cast<uint32_t>(th >> 32), lane);
                     uint64_t shared_tau = (static_cast<uint64_t>(bound) << 32) | 0xFFFFFFFFULL;
                     tau[t] = th < shared_tau ? th : shared_tau;
                 }
             }
+            if (pass) {
+                keys[k + cnt[t] + mask_rank(mask)] = key;
+            }
+            cnt[t] += np;
         }
     };
 
     while (cur.valid()) {
         nxt.advance();
-        if (nxt.valid()) {
-            nxt.load(buf_b);
-        }
+        nxt.load(buf_b, cur.tile);
         consume(buf_a);
         cur = nxt;
         if (!cur.valid()) {
             break;
         }
         nxt.advance();
-        if (nxt.valid()) {
-            nxt.load(buf_a);
-        }
+        nxt.load(buf_a, cur.tile);
         consume(buf_b);
         cur = nxt;
     }
@@ -252,24 +249,33 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
         if (pair[t] == 0xFFFFFFFFU) {
             continue;
         }
+        // What the shared bound still admits is usually less than k keys, which go out unsorted; only a
+        // pair left with more sorts once more (and then has a k-th key to lower the bound with).
         uint64_t* keys = sel + t * S;
-        uint64_t th = selector_flush(keys, S, k, cnt[t], lane);
-        if (th != kInfKey && lane == 0) {
-            atomicMin(&v.bound[qidx[t]], static_cast<uint32_t>(th >> 32));
-        }
-        uint64_t* dst = v.partial + static_cast<uint64_t>(pair[t]) * k;
-        uint32_t valid_count = 0;
-        for (uint32_t i0 = 0; i0 < k; i0 += kWave) {
-            uint32_t i = i0 + lane;
-            uint64_t key = i < k ? keys[i] : kInfKey;
-            bool ok = key != kInfKey;
-            if (ok) {
-                dst[i] = key;
+        wave_lds_fence();
+        uint32_t bs = __builtin_amdgcn_readfirstlane(__atomic_load_n(&v.bound[qidx[t]], __ATOMIC_RELAXED));
+        uint32_t total = k + cnt[t];
+        uint32_t admitted = selector_count_admitted(keys, total, bs, lane);
+        if (admitted > k) {
+            uint64_t th = selector_flush(keys, S, k, cnt[t], lane);
+            bs = lower_shared(&v.bound[qidx[t]], static_cast<uint32_t>(th >> 32), lane);
+            total = k;
+            admitted = selector_count_admitted(keys, total, bs, lane);
+        } else if (admitted == k) {
+            // Exactly k admitted keys: their largest distance is a bound other pairs can use.
+            uint32_t mx = 0;
+            for (uint32_t i = lane; i < total; i += kWave) {
+                uint64_t key = keys[i];
+                uint32_t od = static_cast<uint32_t>(key >> 32);
+                mx = key != kInfKey && od <= bs && od > mx ? od : mx;
             }
-            valid_count += __popcll(__ballot(ok));
+            lower_shared(&v.bound[qidx[t]], wave_max_u32(mx), lane);  // bs itself must stay what was counted with
         }
         if (lane == 0) {
-            v.partial_cnt[pair[t]] = valid_count;
+            v.partial_cnt[pair[t]] = admitted;
+        }
+        if (admitted != 0) {
+            selector_copy_admitted(keys, total, bs, v.partial + static_cast<uint64_t>(pair[t]) * k, lane);
         }
     }
 }

@@ -279,18 +279,57 @@ store_f32(uint8_t* p, float v) {
     }
 }
 
-// Column means as running fp32 sums over the rows in order (rabitq_quantizer.cpp:224-241).
-__global__ void
+// Column means as running fp32 sums over the rows in order (rabitq_quantizer.cpp:224-241).  A workgroup owns 32
+// columns: all 1024 threads stage the next 256 rows of those columns in LDS while the first 32 threads add the
+// current 256 rows, one column each, in row order -- the additions stay sequential, the loads do not.
+constexpr uint32_t kMeanCols = 32;
+constexpr uint32_t kMeanRows = 256;
+
+__global__ void __launch_bounds__(1024)
 column_mean_seq_kernel(const float* x, uint64_t n, uint32_t dim, float* mean) {
-    uint32_t d = blockIdx.x * blockDim.x + threadIdx.x;
-    if (d >= dim) {
-        return;
-    }
+    __shared__ float stage[2][kMeanRows][kMeanCols];
+    const uint32_t col = threadIdx.x & (kMeanCols - 1);
+    const uint32_t slot = threadIdx.x / kMeanCols;  // 0..31
+    const uint32_t d = blockIdx.x * kMeanCols + col;
+    const bool live = d < dim;
+    float regs[kMeanRows / 32];
+    auto fetch = [&](uint64_t row0) {
+#pragma unroll
+        for (uint32_t u = 0; u < kMeanRows / 32; ++u) {
+            uint64_t r = row0 + u * 32 + slot;
+            regs[u] = live && r < n ? x[r * dim + d] : 0.0F;
+        }
+    };
+    auto park = [&](uint32_t b) {
+#pragma unroll
+        for (uint32_t u = 0; u < kMeanRows / 32; ++u) {
+            stage[b][u * 32 + slot][col] = regs[u];
+        }
+    };
+    fetch(0);
+    park(0);
+    __syncthreads();
     float s = 0.0F;
-    for (uint64_t i = 0; i < n; ++i) {
-        s += x[i * dim + d];
+    uint32_t b = 0;
+    for (uint64_t row0 = 0; row0 < n; row0 += kMeanRows, b ^= 1) {
+        const bool more = row0 + kMeanRows < n;
+        if (more) {
+            fetch(row0 + kMeanRows);
+        }
+        if (slot == 0) {
+            uint32_t m = n - row0 < kMeanRows ? static_cast<uint32_t>(n - row0) : kMeanRows;
+            for (uint32_t r = 0; r < m; ++r) {
+                s += stage[b][r][col];
+            }
+        }
+        if (more) {
+            park(b ^ 1);
+        }
+        __syncthreads();
     }
-    mean[d] = s / static_cast<float>(n);
+    if (slot == 0 && live) {
+        mean[d] = s / static_cast<float>(n);
+    }
 }
 
 // Second half of RaBitQuantizer::EncodeOneInternal (rabitq_quantizer.cpp:749-856) for rows already rotated:
@@ -747,7 +786,8 @@ vsag_amd_rabitq_train(const float* x_dev, uint64_t n, uint32_t dim, const float*
     hipStream_t st = static_cast<hipStream_t>(stream);
     float* mean = nullptr;
     VA_HIP(hipMallocAsync(reinterpret_cast<void**>(&mean), dim * 4, st));
-    hipLaunchKernelGGL(column_mean_seq_kernel, dim3((dim + 63) / 64), dim3(64), 0, st, x_dev, n, dim, mean);
+    hipLaunchKernelGGL(column_mean_seq_kernel, dim3((dim + kMeanCols - 1) / kMeanCols), dim3(1024), 0, st, x_dev, n, dim,
+                       mean);
     int rc = gemm_nt_seq(mean, rotation_dev, centroid_dev, 1, dim, dim, st);
     VA_HIP(hipFreeAsync(mean, st));
     return rc;

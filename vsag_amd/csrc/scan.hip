@@ -9,8 +9,10 @@
 //
 // Selection.  Every (wave, query) has a selector in LDS (topk.h).  Chunks and waves of one query share a
 // per-query bound in global memory (the k-th best distance any of them has proven so far), so later
-// work drops almost everything with one compare.  Each (chunk, wave) leaves a short sorted list of
-// survivors; a merge kernel picks the k best per query.
+// work drops almost everything with one compare.  Each (chunk, wave) leaves a short counted list of the
+// survivors that the bound still admits; a merge kernel picks the k best per query.  All waves of a query
+// share a handful of addresses (its bound, its seed row), and atomics on one address serialise in L2, so
+// every atomicMin is preceded by a plain load and issued only when it would lower the value.
 #include "distance.h"
 #include "store.h"
 #include "topk.h"
@@ -26,11 +28,15 @@ uint64_t rabitq_query_code_size(uint32_t dim, int metric, int query_bits);
 
 constexpr uint32_t kMaxWaves = 4;
 
+// Per query: no bound yet, no seeds yet.
 __global__ void
-fill_words_kernel(uint32_t* p, uint32_t v, uint64_t n) {
+reset_queries_kernel(uint32_t* bound, uint64_t nq, uint32_t* seed, uint64_t nseed) {
     uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (i < n) {
-        p[i] = v;
+    if (i < nq) {
+        bound[i] = 0xFFFFFFFFU;
+    }
+    if (i < nseed) {
+        seed[i] = 0xFFFFFFFFU;
     }
 }
 
@@ -45,9 +51,18 @@ struct FlatArgs {
     uint32_t* bound;        // per query: ordered distance that k candidates are known to reach
     uint64_t* partial;      // nq x nslots x k keys
     uint32_t* partial_cnt;  // nq x nslots
+    uint32_t* seed;         // nq x k smallest first-tile distances by wave class, or null (see kSeedTiles)
 };
 
-template <int KIND, int METRIC, int T>
+// Cold start.  A wave that begins without a bound would have to sort its first tiles just to learn a
+// threshold.  Instead every such wave publishes the smallest distance of its first tile into slot
+// (global wave index mod k) of its query's seed row; waves own disjoint codes, so once all k slots are
+// filled their maximum is a distance that k different codes reach -- a valid bound, usually far tighter
+// than anything one wave could find alone.  A cold wave re-reads the row after each of its first
+// kSeedTiles tiles; the host enables seeding only when there are at least 2k waves per query.
+constexpr uint32_t kSeedTiles = 6;
+
+template <int KIND, int METRIC, int T, bool SEED>
 __global__ void __launch_bounds__(256)
 flat_scan_kernel(ScanArgs a, FlatArgs f) {
     extern __shared__ uint64_t lds[];
@@ -58,8 +73,9 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
     uint64_t* sel = lds + static_cast<size_t>(wave) * T * S;
 
     uint32_t qidx[T];
-    uint32_t thr[T];  // a candidate passes when its ordered distance is below thr
+    uint32_t thr[T];   // a candidate passes when its ordered distance is below thr
     uint32_t cnt[T];
+    uint32_t cold[T];  // tiles after which this wave still looks at the seed row
 #pragma unroll
     for (int t = 0; t < T; ++t) {
         qidx[t] = blockIdx.x * T + t;
@@ -67,11 +83,13 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
         uint32_t bs = qidx[t] < f.nq ? __builtin_amdgcn_readfirstlane(__atomic_load_n(&f.bound[qidx[t]], __ATOMIC_RELAXED))
                                      : 0xFFFFFFFFU;
         thr[t] = bs == 0xFFFFFFFFU ? bs : bs + 1;
+        cold[t] = SEED && qidx[t] < f.nq && bs == 0xFFFFFFFFU ? kSeedTiles : 0;
     }
     for (uint32_t i = lane; i < T * S; i += kWave) {
         sel[i] = kInfKey;
     }
     wave_lds_fence();
+    const uint32_t seed_slot = (blockIdx.y * nwaves + wave) % k;
 
     const uint64_t tile_begin = static_cast<uint64_t>(blockIdx.y) * f.tiles_per_chunk;
     uint64_t tile_end = tile_begin + f.tiles_per_chunk;
@@ -79,26 +97,42 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
         tile_end = f.ntiles;
     }
     // Software pipeline over granule groups: the loads of group g+1 (possibly of the next tile) are
-    // issued before group g is consumed, so every wave keeps kGroup KiB in flight.  Two register buffers
+    // issued before group g is consumed, so every wave keeps GROUP KiB in flight.  Two register buffers
     // alternate; the loop body is written out twice so that both are addressed statically.
     const QueryRows<T> qrows = query_rows<T>(a, qidx);
-    TileStream cur{a.tiles + lane, tile_begin + wave, tile_end, nwaves, 0, a.G};
-    TileStream nxt = cur;
-    uint4 buf_a[kGroup], buf_b[kGroup];
+    constexpr int GROUP = GroupOf<T>::value;
+    TileStream<GROUP> cur{a.tiles, lane, tile_begin + wave, tile_end, nwaves, 0, a.G};
+    TileStream<GROUP> nxt = cur;
+    uint4 buf_a[GROUP], buf_b[GROUP];
     if (cur.valid()) {
-        cur.load(buf_a);
+        cur.load(buf_a, cur.tile);
     }
     Acc<KIND, T> acc;
     acc_reset(acc);
 
-    auto consume = [&](const uint4(&regs)[kGroup]) {
+    // Sorts selector t and folds its k-th key and the shared bound into thr[t].
+    auto flush = [&](int t) {
+        uint64_t* keys = sel + t * S;
+        uint64_t th = selector_flush(keys, S, k, cnt[t], lane);
+        cnt[t] = 0;
+        cold[t] = 0;
+        uint32_t tl = static_cast<uint32_t>(th >> 32);  // 0xFFFFFFFF while fewer than k seen
+        uint32_t bs = 0xFFFFFFFFU;
+        if (qidx[t] < f.nq) {
+            bs = lower_shared(&f.bound[qidx[t]], tl, lane);  // tl = 0xFFFFFFFF lowers nothing
+        }
+        uint32_t tb = bs == 0xFFFFFFFFU ? bs : bs + 1;
+        thr[t] = tl < tb ? tl : tb;
+    };
+
+    auto consume = [&](const uint4(&regs)[GROUP]) {
 #pragma unroll
-        for (int u = 0; u < kGroup; ++u) {
+        for (int u = 0; u < GROUP; ++u) {
             if (cur.j0 + u < a.G) {
                 accumulate_granule<KIND, METRIC, T>(a, qrows, cur.j0 + u, regs[u], acc);
             }
         }
-        if (cur.j0 + kGroup < a.G) {
+        if (cur.j0 + GROUP < a.G) {
             return;
         }
         const uint64_t id = cur.tile * kWave + lane;
@@ -111,43 +145,50 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
             // Inner ids grow along the scan, so "ordered distance < thr" is exactly the (distance, id)
             // order against the wave's own k-th key, and "<= bound" against the shared bound.
             uint32_t od = float_to_ordered(d[t]);
-            bool pass = valid && od < thr[t];
-            uint64_t* keys = sel + t * S;
-            cnt[t] = selector_append(keys, k, cnt[t], pass,
-                                     (static_cast<uint64_t>(od) << 32) | static_cast<uint32_t>(id));
-            if (cnt[t] + kWave > S - k) {
-                uint64_t th = selector_flush(keys, S, k, cnt[t], lane);
-                cnt[t] = 0;
-                uint32_t tl = static_cast<uint32_t>(th >> 32);  // 0xFFFFFFFF while fewer than k seen
-                uint32_t bs = 0xFFFFFFFFU;
-                if (qidx[t] < f.nq) {
-                    if (th != kInfKey) {
-                        uint32_t old = lane == 0 ? atomicMin(&f.bound[qidx[t]], tl) : 0U;
-                        bs = __builtin_amdgcn_readfirstlane(old);
-                    } else {
-                        bs = __builtin_amdgcn_readfirstlane(__atomic_load_n(&f.bound[qidx[t]], __ATOMIC_RELAXED));
-                    }
+            if (SEED && cold[t] != 0) {
+                uint32_t* row = f.seed + static_cast<uint64_t>(qidx[t]) * k;
+                if (cold[t] == kSeedTiles) {
+                    uint32_t m = wave_min_u32(valid ? od : 0xFFFFFFFFU);
+                    lower_shared(&row[seed_slot], m, lane);
                 }
-                uint32_t tb = bs == 0xFFFFFFFFU ? bs : bs + 1;
-                thr[t] = tl < tb ? tl : tb;
+                --cold[t];
+                uint32_t mx = 0;
+                for (uint32_t i = lane; i < k; i += kWave) {
+                    uint32_t v = __atomic_load_n(&row[i], __ATOMIC_RELAXED);
+                    mx = v > mx ? v : mx;
+                }
+                mx = wave_max_u32(mx);
+                if (mx != 0xFFFFFFFFU) {
+                    cold[t] = 0;
+                    mx = lower_shared(&f.bound[qidx[t]], mx, lane);
+                    thr[t] = mx + 1 < thr[t] ? mx + 1 : thr[t];
+                }
+            }
+            bool pass = valid && od < thr[t];
+            uint64_t mask = __ballot(pass);
+            if (mask != 0) {
+                uint32_t np = __popcll(mask);
+                if (k + cnt[t] + np > S) {
+                    flush(t);
+                }
+                if (pass) {
+                    sel[t * S + k + cnt[t] + mask_rank(mask)] = (static_cast<uint64_t>(od) << 32) | static_cast<uint32_t>(id);
+                }
+                cnt[t] += np;
             }
         }
     };
 
     while (cur.valid()) {
         nxt.advance();
-        if (nxt.valid()) {
-            nxt.load(buf_b);
-        }
+        nxt.load(buf_b, cur.tile);
         consume(buf_a);
         cur = nxt;
         if (!cur.valid()) {
             break;
         }
         nxt.advance();
-        if (nxt.valid()) {
-            nxt.load(buf_a);
-        }
+        nxt.load(buf_a, cur.tile);
         consume(buf_b);
         cur = nxt;
     }
@@ -158,52 +199,90 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
         if (qidx[t] >= f.nq) {
             continue;
         }
+        // Whatever lies above the shared bound is beaten by k candidates of other waves.  What remains is
+        // usually less than k keys, which go out as they are; only a wave left with more sorts once more.
         uint64_t* keys = sel + t * S;
-        uint64_t th = selector_flush(keys, S, k, cnt[t], lane);
-        if (th != kInfKey && lane == 0) {
-            atomicMin(&f.bound[qidx[t]], static_cast<uint32_t>(th >> 32));
+        wave_lds_fence();
+        uint32_t bs = __builtin_amdgcn_readfirstlane(__atomic_load_n(&f.bound[qidx[t]], __ATOMIC_RELAXED));
+        uint32_t total = k + cnt[t];
+        uint32_t admitted = selector_count_admitted(keys, total, bs, lane);
+        if (admitted > k) {
+            uint64_t th = selector_flush(keys, S, k, cnt[t], lane);
+            bs = lower_shared(&f.bound[qidx[t]], static_cast<uint32_t>(th >> 32), lane);
+            total = k;
+            admitted = selector_count_admitted(keys, total, bs, lane);
         }
         const uint64_t list = static_cast<uint64_t>(qidx[t]) * f.nslots + slot;
-        uint64_t* dst = f.partial + list * k;
-        uint32_t valid_count = 0;
-        for (uint32_t i0 = 0; i0 < k; i0 += kWave) {
-            uint32_t i = i0 + lane;
-            uint64_t key = i < k ? keys[i] : kInfKey;
-            bool ok = key != kInfKey;
-            if (ok) {
-                dst[i] = key;
-            }
-            valid_count += __popcll(__ballot(ok));
-        }
         if (lane == 0) {
-            f.partial_cnt[list] = valid_count;
+            f.partial_cnt[list] = admitted;
+        }
+        if (admitted != 0) {
+            selector_copy_admitted(keys, total, bs, f.partial + list * k, lane);
         }
     }
 }
 
-// One wave per query: the k best keys over its partial lists, written as ids / distances (ascending).
-__global__ void __launch_bounds__(64)
-merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, uint32_t nslots, uint32_t k, uint32_t S,
-                      uint32_t* ids, float* dists) {
-    extern __shared__ uint64_t lds[];
-    const uint32_t lane = threadIdx.x;
+// One workgroup per query: the k best keys over its counted partial lists, written as ids / distances
+// (ascending).  All threads first keep what the final shared bound admits (at least k keys when k exist) in
+// an LDS pool; wave 0 then selects from the pool -- or straight from the lists when the pool overflowed
+// (long runs of equal distances).
+constexpr uint32_t kPoolKeys = 2048;
+
+__global__ void __launch_bounds__(1024)
+merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, const uint32_t* bound, uint32_t nslots,
+                      uint32_t k, uint32_t S, uint32_t* ids, float* dists) {
+    extern __shared__ uint64_t lds[];  // S selector keys, then the pool
+    __shared__ uint32_t npool;
+    uint64_t* pool = lds + S;
     const uint64_t q = blockIdx.x;
+    const uint32_t* cnts = partial_cnt + q * nslots;
+    const uint64_t* src = partial + q * nslots * k;
+    const uint32_t total = nslots * k;  // list entries, most of them beyond their list's count
+    const uint64_t admit = (static_cast<uint64_t>(as_const(bound)[q]) << 32) | 0xFFFFFFFFULL;
+    if (threadIdx.x == 0) {
+        npool = 0;
+    }
+    __syncthreads();
+    for (uint32_t e = threadIdx.x; e < total; e += blockDim.x) {
+        uint32_t slot = e / k;
+        if (e - slot * k < cnts[slot]) {
+            uint64_t key = src[e];
+            if (key <= admit) {
+                uint32_t pos = atomicAdd(&npool, 1U);
+                if (pos < kPoolKeys) {
+                    pool[pos] = key;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x >= kWave) {
+        return;
+    }
+    const uint32_t lane = threadIdx.x;
+    const bool pooled = npool <= kPoolKeys;
+    const uint32_t count = pooled ? npool : total;
     selector_init(lds, S, lane);
     uint32_t cnt = 0;
     uint64_t tau = kInfKey;
-    for (uint32_t slot = 0; slot < nslots; ++slot) {
-        const uint64_t list = q * nslots + slot;
-        const uint32_t c = as_const(partial_cnt)[list];
-        const uint64_t* src = partial + list * k;
-        for (uint32_t base = 0; base < c; base += kWave) {
-            uint32_t i = base + lane;
-            uint64_t key = i < c ? src[i] : kInfKey;
-            bool pass = key < tau;
-            cnt = selector_append(lds, k, cnt, pass, key);
-            if (cnt + kWave > S - k) {
-                tau = selector_flush(lds, S, k, cnt, lane);
-                cnt = 0;
+    for (uint32_t base = 0; base < count; base += kWave) {
+        uint32_t e = base + lane;
+        uint64_t key = kInfKey;
+        if (e < count) {
+            if (pooled) {
+                key = pool[e];
+            } else {
+                uint32_t slot = e / k;
+                if (e - slot * k < cnts[slot]) {
+                    key = src[e];
+                }
             }
+        }
+        bool pass = key < tau;
+        cnt = selector_append(lds, k, cnt, pass, key);
+        if (cnt + kWave > S - k) {
+            tau = selector_flush(lds, S, k, cnt, lane);
+            cnt = 0;
         }
     }
     selector_flush(lds, S, k, cnt, lane);
@@ -252,6 +331,7 @@ struct ScanPlan {
     size_t lds_bytes;
     QueryLayout ql;
     size_t qcode_bytes;  // staging for encoded queries (uniform kinds, rabitq)
+    bool seeded;         // cold waves learn a bound from each other's first tiles (kSeedTiles)
 };
 
 static void
@@ -278,8 +358,13 @@ make_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, uint64_t ntiles, Sca
     if (g_chunk_override > 0) {
         chunks = g_chunk_override;
     } else {
-        // About eight rounds of workgroups over the machine (eight workgroups fit a CU).
-        chunks = div_up(static_cast<uint64_t>(device_cu_count()) * 8 * 8, p->groups);
+        // Workgroups in the grid: about 64 per query group, but at least two per compute unit (few queries:
+        // every wave still has a long run of tiles behind its cold start) and at most eight rounds of
+        // workgroups over the machine (eight fit a compute unit).
+        uint64_t want = 64 * p->groups;
+        const uint64_t lo = static_cast<uint64_t>(device_cu_count()) * 2, hi = static_cast<uint64_t>(device_cu_count()) * 64;
+        want = want < lo ? lo : want > hi ? hi : want;
+        chunks = div_up(want, p->groups);
     }
     uint64_t max_chunks = ntiles / (16 * waves);  // at least 16 tiles per wave
     if (max_chunks < 1) {
@@ -293,6 +378,8 @@ make_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, uint64_t ntiles, Sca
     }
     p->tiles_per_chunk = div_up(ntiles > 0 ? ntiles : 1, chunks);
     p->chunks = div_up(ntiles > 0 ? ntiles : 1, p->tiles_per_chunk);
+    // Seeding pays when a query's waves all start cold together, i.e. when the whole grid is resident at once.
+    p->seeded = p->chunks * waves >= 2ull * k && k <= 256 && p->groups * p->chunks * waves <= 8192;
     p->ql = query_layout(s);
     p->qcode_bytes = 0;
     if (s->kind == VSAG_AMD_KIND_SQ4_UNIFORM || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
@@ -309,6 +396,7 @@ struct ScanBuffers {
     uint32_t* bound;
     uint32_t* partial_cnt;
     uint64_t* partial;
+    uint32_t* seed;  // null when the plan does not seed
 };
 
 static size_t
@@ -318,8 +406,22 @@ carve_scan(Carver& c, const ScanPlan& p, uint64_t nq, uint32_t k, ScanBuffers* b
     b->qcodes = c.take<uint8_t>(p.qcode_bytes);
     b->bound = c.take<uint32_t>(nq);
     b->partial_cnt = c.take<uint32_t>(nq * p.chunks * p.waves);
+    b->seed = c.take<uint32_t>(p.seeded ? nq * k : 0);
+    if (!p.seeded) {
+        b->seed = nullptr;
+    }
     b->partial = c.take<uint64_t>(nq * p.chunks * p.waves * k);
     return c.used;
+}
+
+template <int KIND, int METRIC, int T>
+static void
+launch_flat_s(dim3 grid, dim3 block, size_t lds, hipStream_t st, const ScanArgs& a, const FlatArgs& f) {
+    if (f.seed != nullptr) {
+        hipLaunchKernelGGL((flat_scan_kernel<KIND, METRIC, T, true>), grid, block, lds, st, a, f);
+    } else {
+        hipLaunchKernelGGL((flat_scan_kernel<KIND, METRIC, T, false>), grid, block, lds, st, a, f);
+    }
 }
 
 template <int KIND, int METRIC>
@@ -327,16 +429,16 @@ static void
 launch_flat_t(int T, dim3 grid, dim3 block, size_t lds, hipStream_t st, const ScanArgs& a, const FlatArgs& f) {
     switch (T) {
         case 1:
-            hipLaunchKernelGGL((flat_scan_kernel<KIND, METRIC, 1>), grid, block, lds, st, a, f);
+            launch_flat_s<KIND, METRIC, 1>(grid, block, lds, st, a, f);
             break;
         case 2:
-            hipLaunchKernelGGL((flat_scan_kernel<KIND, METRIC, 2>), grid, block, lds, st, a, f);
+            launch_flat_s<KIND, METRIC, 2>(grid, block, lds, st, a, f);
             break;
         case 4:
-            hipLaunchKernelGGL((flat_scan_kernel<KIND, METRIC, 4>), grid, block, lds, st, a, f);
+            launch_flat_s<KIND, METRIC, 4>(grid, block, lds, st, a, f);
             break;
         default:
-            hipLaunchKernelGGL((flat_scan_kernel<KIND, METRIC, 8>), grid, block, lds, st, a, f);
+            launch_flat_s<KIND, METRIC, 8>(grid, block, lds, st, a, f);
             break;
     }
 }
@@ -428,8 +530,9 @@ vsag_amd_flat_scan_topk(const vsag_amd_store_t* s, const float* queries_dev, uin
     VA_CHECK_ARG(c.ok(), "workspace too small: need %zu bytes, got %zu", c.used, workspace_bytes);
 
     VA_TRY(prepare_queries(s, queries_dev, nq, p.nq_pad, p.ql, b.qtab, b.qmeta, b.qcodes, st));
-    hipLaunchKernelGGL(fill_words_kernel, dim3(static_cast<uint32_t>(div_up(nq, 256))), dim3(256), 0, st, b.bound,
-                       0xFFFFFFFFU, nq);
+    const uint64_t nseed = p.seeded ? nq * k : 0;
+    hipLaunchKernelGGL(reset_queries_kernel, dim3(static_cast<uint32_t>(div_up(nq > nseed ? nq : nseed, 256))), dim3(256),
+                       0, st, b.bound, nq, b.seed, nseed);
     ScanArgs a = make_scan_args(s, p.ql, b.qtab, b.qmeta);
     FlatArgs f{};
     f.n = s->n;
@@ -442,17 +545,18 @@ vsag_amd_flat_scan_topk(const vsag_amd_store_t* s, const float* queries_dev, uin
     f.bound = b.bound;
     f.partial = b.partial;
     f.partial_cnt = b.partial_cnt;
-    if (s->ntiles == 0) {
-        // Empty store: every partial list must still read as empty.
-        hipLaunchKernelGGL(fill_words_kernel, dim3(static_cast<uint32_t>(div_up(nq * f.nslots, 256))), dim3(256), 0,
-                           st, b.partial_cnt, 0U, nq * f.nslots);
-    } else {
+    f.seed = b.seed;
+    if (s->ntiles != 0) {
         timing_begin(st);
         VA_TRY(launch_flat(s, p, a, f, st));
         timing_end(st);
     }
-    hipLaunchKernelGGL(merge_partials_kernel, dim3(static_cast<uint32_t>(nq)), dim3(kWave), p.S * 8, st, b.partial,
-                       b.partial_cnt, f.nslots, k, p.S, ids_dev, dists_dev);
+    // Few queries: many candidates each (every wave starts without a bound), so give each merge more threads.
+    const uint32_t merge_threads = nq <= 256 ? 1024 : 256;
+    // An empty store has no lists to read.
+    hipLaunchKernelGGL(merge_partials_kernel, dim3(static_cast<uint32_t>(nq)), dim3(merge_threads),
+                       (p.S + kPoolKeys) * 8, st, b.partial, b.partial_cnt, b.bound, s->ntiles != 0 ? f.nslots : 0U, k,
+                       p.S, ids_dev, dists_dev);
     VA_HIP(hipGetLastError());
     tl_last_tile = p.T;
     tl_last_passes = p.groups;

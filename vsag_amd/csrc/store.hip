@@ -158,7 +158,7 @@ grow(vsag_amd_store* s, uint64_t need_tiles, hipStream_t st) {
     }
     uint4* tiles = nullptr;
     uint32_t* meta = nullptr;
-    size_t tile_bytes = cap * s->G * kWave * sizeof(uint4);
+    size_t tile_bytes = cap * s->G * kWave * sizeof(uint4) + kTileSlackBytes;
     VA_HIP(hipMalloc(&tiles, tile_bytes));
     VA_HIP(hipMemsetAsync(tiles, 0, tile_bytes, st));
     if (s->nmeta > 0) {
@@ -461,7 +461,7 @@ vsag_amd_store_set_lists(vsag_amd_store_t* s, const uint8_t* codes_dev, const in
     s->ntiles = 0;
     s->n = 0;
     uint64_t cap = ntiles > 0 ? ntiles : 1;
-    VA_HIP(hipMalloc(&s->tiles, cap * s->G * kWave * sizeof(uint4)));
+    VA_HIP(hipMalloc(&s->tiles, cap * s->G * kWave * sizeof(uint4) + kTileSlackBytes));
     VA_HIP(hipMemsetAsync(s->tiles, 0, cap * s->G * kWave * sizeof(uint4), st));
     if (s->nmeta > 0) {
         VA_HIP(hipMalloc(&s->meta, cap * kWave * s->nmeta * sizeof(uint32_t)));

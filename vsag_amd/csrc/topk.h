@@ -2,9 +2,9 @@
 //
 // One wavefront owns one selector per query it serves.  A selector is an array of S 64-bit keys
 // (S a power of two, S >= k + 96): slots [0,k) hold the best keys found so far, slots [k,k+cnt) hold
-// pending candidates that passed the current threshold.  When the pending region could overflow on the
-// next 64-wide append, the wave sorts the whole array (bitonic, in LDS) which leaves the k best in
-// front and yields the new threshold keys[k-1].  No workgroup barrier is involved: only the owning
+// pending candidates that passed the current threshold.  When an append would overflow the pending
+// region, the wave first sorts the whole array (bitonic, in LDS) which leaves the k best in front and
+// yields the new threshold keys[k-1].  No workgroup barrier is involved: only the owning
 // wave touches a selector, and LDS operations of one wave complete in program order.
 //
 // This replaces the reference's per-query bounded max-heap (src/impl/heap/standard_heap.cpp:24-53,
@@ -103,6 +103,65 @@ selector_append(uint64_t* keys, uint32_t k, uint32_t cnt, bool pass, uint64_t ke
         cnt += __popcll(mask);
     }
     return cnt;
+}
+
+// How many of keys[0,total) are real and have an ordered distance of at most `bound` (wave-uniform).
+__device__ inline uint32_t
+selector_count_admitted(const uint64_t* keys, uint32_t total, uint32_t bound, uint32_t lane) {
+    uint32_t n = 0;
+    for (uint32_t i0 = 0; i0 < total; i0 += kWave) {
+        uint32_t i = i0 + lane;
+        uint64_t key = i < total ? keys[i] : kInfKey;
+        bool ok = key != kInfKey && static_cast<uint32_t>(key >> 32) <= bound;
+        n += __popcll(__ballot(ok));
+    }
+    return n;
+}
+
+// Copies those keys to dst[0, count), in selector order.
+__device__ inline void
+selector_copy_admitted(const uint64_t* keys, uint32_t total, uint32_t bound, uint64_t* dst, uint32_t lane) {
+    uint32_t n = 0;
+    for (uint32_t i0 = 0; i0 < total; i0 += kWave) {
+        uint32_t i = i0 + lane;
+        uint64_t key = i < total ? keys[i] : kInfKey;
+        bool ok = key != kInfKey && static_cast<uint32_t>(key >> 32) <= bound;
+        uint64_t mask = __ballot(ok);
+        if (ok) {
+            dst[n + mask_rank(mask)] = key;
+        }
+        n += __popcll(mask);
+    }
+}
+
+__device__ inline uint32_t
+wave_min_u32(uint32_t v) {
+    for (int off = 32; off > 0; off >>= 1) {
+        uint32_t o = __shfl_xor(v, off);
+        v = o < v ? o : v;
+    }
+    return __builtin_amdgcn_readfirstlane(v);
+}
+
+__device__ inline uint32_t
+wave_max_u32(uint32_t v) {
+    for (int off = 32; off > 0; off >>= 1) {
+        uint32_t o = __shfl_xor(v, off);
+        v = o > v ? o : v;
+    }
+    return __builtin_amdgcn_readfirstlane(v);
+}
+
+// Lowers *p to v if v is smaller; returns the smaller of v and the value seen (wave-uniform).  The atomic
+// is skipped when a plain load already shows a value that is not larger.
+__device__ inline uint32_t
+lower_shared(uint32_t* p, uint32_t v, uint32_t lane) {
+    uint32_t seen = __builtin_amdgcn_readfirstlane(__atomic_load_n(p, __ATOMIC_RELAXED));
+    if (v < seen) {
+        uint32_t old = lane == 0 ? atomicMin(p, v) : 0U;
+        seen = __builtin_amdgcn_readfirstlane(old);
+    }
+    return seen < v ? seen : v;
 }
 
 }  // namespace vsag_amd

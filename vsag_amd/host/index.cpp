@@ -355,6 +355,12 @@ check_query(const DatasetPtr& query, int64_t k, uint32_t dim) {
 DatasetPtr
 pack_results(const std::vector<uint32_t>& ids, const std::vector<float>& dists, int64_t nq, int64_t k,
              const std::vector<int64_t>& labels, const std::string& stats) {
+    for (int64_t i = 0; i < nq * k; ++i) {
+        if (ids[i] != VSAG_AMD_INVALID_ID && ids[i] >= labels.size()) {
+            throw VsagException(ErrorType::INTERNAL_ERROR,
+                                "search returned inner id " + std::to_string(ids[i]) + " of " + std::to_string(labels.size()));
+        }
+    }
     auto result = Dataset::Make();
     if (nq == 1) {
         int64_t count = 0;
