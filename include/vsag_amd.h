@@ -178,6 +178,22 @@ VSAG_AMD_API int vsag_amd_flat_scan_topk(const vsag_amd_store_t* store, const fl
                             uint32_t k, uint32_t* ids_dev, float* dists_dev, void* workspace_dev,
                             size_t workspace_bytes, void* stream);
 
+/* Pre-filter and range limit of a search (BruteForce::SearchWithRequest with a Filter and in RANGE_SEARCH mode,
+ * bruteforce.cpp:519-545; FlatBucketSearcher::Search, flat_bucket_searcher.cpp:61-137).
+ * deny_bits_dev: bit (id & 31) of word (id >> 5) set = inner id `id` is filtered out, ceil(n / 32) words of
+ * device memory, or NULL.  The caller maps labels to inner ids (InnerIdWrapperFilter,
+ * impl/filter/inner_id_wrapper_filter.h:23-57).  use_radius != 0: only distances <= radius are returned. */
+typedef struct vsag_amd_search_options {
+    const uint32_t* deny_bits_dev;
+    int use_radius;
+    float radius;
+} vsag_amd_search_options_t;
+
+/* vsag_amd_flat_scan_topk under the given options (NULL = none).  Same workspace size. */
+VSAG_AMD_API int vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* store, const float* queries_dev, uint64_t nq,
+                               uint32_t k, const vsag_amd_search_options_t* options, uint32_t* ids_dev,
+                               float* dists_dev, void* workspace_dev, size_t workspace_bytes, void* stream);
+
 /* Tuning knobs of the scan (query tile T in {1,2,4,8}, 0 = automatic; number of base chunks, 0 =
  * automatic).  Process-wide; meant for benchmarks. */
 VSAG_AMD_API int vsag_amd_set_scan_tuning(int query_tile, int base_chunks);
@@ -233,6 +249,12 @@ VSAG_AMD_API size_t vsag_amd_ivf_scan_workspace_bytes(const vsag_amd_store_t* li
 VSAG_AMD_API int vsag_amd_ivf_scan_topk(const vsag_amd_store_t* lists, const float* queries_dev, uint64_t nq,
                            const int32_t* buckets_dev, uint32_t nprobe, uint32_t kcand, uint32_t* ids_dev,
                            float* dists_dev, void* workspace_dev, size_t workspace_bytes, void* stream);
+
+/* vsag_amd_ivf_scan_topk under the given options (NULL = none).  Same workspace size. */
+VSAG_AMD_API int vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* lists, const float* queries_dev, uint64_t nq,
+                              const int32_t* buckets_dev, uint32_t nprobe, uint32_t kcand,
+                              const vsag_amd_search_options_t* options, uint32_t* ids_dev, float* dists_dev,
+                              void* workspace_dev, size_t workspace_bytes, void* stream);
 
 /* FlattenReorder::Reorder (impl/reorder/flatten_reorder.cpp:52-114): exact fp32 distances of the
  * candidates (nq x kcand inner ids into raw_dev, n x dim fp32 row-major; VSAG_AMD_INVALID_ID skipped),

@@ -59,10 +59,39 @@ class Store:
     def size(self):
         return int(self.lib.vsag_amd_store_size(self.handle))
 
-    def flat_scan(self, queries, k):
+    def _options(self, deny, radius):
+        """(options pointer or None, buffers to free).  deny: boolean array over inner ids (True = filtered out)."""
+        if deny is None and radius is None:
+            return None, []
+        opt = capi.SearchOptions()
+        keep = []
+        if deny is not None:
+            bits = np.packbits(np.asarray(deny, bool), bitorder="little")
+            words = np.zeros((bits.size + 3) // 4 * 4, np.uint8)
+            words[:bits.size] = bits
+            buf = dev(words.view(np.uint32))
+            keep.append(buf)
+            opt.deny_bits_dev = buf.ptr
+        if radius is not None:
+            opt.use_radius, opt.radius = 1, float(radius)
+        return opt, keep
+
+    def flat_scan(self, queries, k, deny=None, radius=None):
         q = np.ascontiguousarray(queries, np.float32)
         nq = q.shape[0]
         qb = dev(q)
+        opt, keep = self._options(deny, radius)
+        if opt is not None:
+            ids = capi.DeviceBuffer(nq * k * 4)
+            ds = capi.DeviceBuffer(nq * k * 4)
+            wsb = self.lib.vsag_amd_flat_scan_workspace_bytes(self.handle, nq, k)
+            ws = capi.DeviceBuffer(wsb)
+            capi.check(self.lib.vsag_amd_flat_scan_topk_ex(self.handle, qb.ptr, nq, k, C.byref(opt), ids.ptr, ds.ptr,
+                                                          ws.ptr, wsb, None))
+            out = ids.to_numpy(np.uint32, (nq, k)), ds.to_numpy(np.float32, (nq, k))
+            for b in [qb, ids, ds, ws] + keep:
+                b.free()
+            return out
         ids = capi.DeviceBuffer(nq * k * 4)
         ds = capi.DeviceBuffer(nq * k * 4)
         wsb = self.lib.vsag_amd_flat_scan_workspace_bytes(self.handle, nq, k)
@@ -73,11 +102,23 @@ class Store:
             b.free()
         return out
 
-    def ivf_scan(self, queries, buckets, kcand):
+    def ivf_scan(self, queries, buckets, kcand, deny=None, radius=None):
         q = np.ascontiguousarray(queries, np.float32)
         b = np.ascontiguousarray(buckets, np.int32)
         nq, nprobe = b.shape
         qb, bb = dev(q), dev(b)
+        opt, keep = self._options(deny, radius)
+        if opt is not None:
+            ids = capi.DeviceBuffer(nq * kcand * 4)
+            ds = capi.DeviceBuffer(nq * kcand * 4)
+            wsb = self.lib.vsag_amd_ivf_scan_workspace_bytes(self.handle, nq, nprobe, kcand)
+            ws = capi.DeviceBuffer(wsb)
+            capi.check(self.lib.vsag_amd_ivf_scan_topk_ex(self.handle, qb.ptr, nq, bb.ptr, nprobe, kcand, C.byref(opt),
+                                                         ids.ptr, ds.ptr, ws.ptr, wsb, None))
+            out = ids.to_numpy(np.uint32, (nq, kcand)), ds.to_numpy(np.float32, (nq, kcand))
+            for x in [qb, bb, ids, ds, ws] + keep:
+                x.free()
+            return out
         ids = capi.DeviceBuffer(nq * kcand * 4)
         ds = capi.DeviceBuffer(nq * kcand * 4)
         wsb = self.lib.vsag_amd_ivf_scan_workspace_bytes(self.handle, nq, nprobe, kcand)

@@ -204,3 +204,89 @@ def test_ivf_rabitq_with_reorder(lib):
     ids, _ = idx.knn_search_batch(q, k, json.dumps({"ivf": {"scan_buckets_count": 10, "factor": 20.0}}))
     assert recall(ids, gt, labels) >= 0.85
     idx.close()
+
+
+# ------------------------------------------------------------------------------------------------------------------
+# Pre-filters and range search, after TestIndex::TestFilterSearch / TestRangeSearch
+# (tests/test_index/test_index_search.cpp:100-160,263-350): filter(label) == True filters the vector out; the range
+# radius sits between the (k-1)-th and k-th exact distances; results never contain a filtered label.
+def _filtered_truth(x, q, labels, k, metric, keep):
+    allowed = np.nonzero(keep)[0]
+    gt, gt_d = ground_truth(x[allowed], q, k, metric)
+    return labels[allowed][gt], gt_d
+
+
+@pytest.mark.parametrize("name,params,search", [
+    ("brute_force", {"base_quantization_type": "fp32"}, "{}"),
+    ("brute_force", {"base_quantization_type": "sq8"}, "{}"),
+    ("ivf", {"buckets_count": 20, "base_quantization_type": "fp32"}, json.dumps({"ivf": {"scan_buckets_count": 20}})),
+    ("ivf", {"buckets_count": 20, "base_quantization_type": "sq8", "use_reorder": True,
+             "precise_quantization_type": "fp32"}, json.dumps({"ivf": {"scan_buckets_count": 20, "factor": 4.0}})),
+])
+def test_filter_search(lib, name, params, search):
+    n, d, nq, k = 3000, 32, 20, 10
+    x = vectors(n, d)
+    q = vectors(nq, d, seed=165)
+    labels = np.arange(n, dtype=np.int64) * 5 + 3
+    idx = make(name, d, "l2", **params)
+    assert idx.build(x, labels, n, d) == 0
+    flt = lambda label: label % 3 != 0  # noqa: E731  (keeps a third, like the fixtures' valid_ratio cases)
+    keep = np.array([not flt(int(v)) for v in labels])
+    gt_labels, gt_d = _filtered_truth(x, q, labels, k, "l2", keep)
+    hits = range_hits = 0
+    for i in range(nq):
+        ids, dists = idx.knn_search(q[i], k, search, filter=flt)
+        assert ids.size == k and np.all(np.diff(dists) >= 0)
+        assert not any(flt(int(v)) for v in ids)
+        hits += len(set(ids.tolist()) & set(gt_labels[i].tolist()))
+        threshold = 0.5 * float(gt_d[i][k - 2] + gt_d[i][k - 1])
+        rids, rd = idx.range_search(q[i], threshold, search, filter=flt)
+        assert not any(flt(int(v)) for v in rids)
+        assert np.all(rd <= threshold + 2e-6) or params["base_quantization_type"] != "fp32"
+        range_hits += len(set(rids.tolist()) & set(gt_labels[i][:k - 1].tolist()))
+    floor = 0.99 if params["base_quantization_type"] == "fp32" else 0.8
+    assert hits / float(nq * k) > floor * RECALL_THRESHOLD
+    assert range_hits / float(nq * (k - 1)) > floor * RECALL_THRESHOLD
+    # nothing survives the filter: empty result, not an error
+    ids, dists = idx.knn_search(q[0], k, search, filter=lambda label: True)
+    assert ids.size == 0
+    idx.close()
+
+
+@pytest.mark.parametrize("name,params,search", [
+    ("brute_force", {"base_quantization_type": "fp32"}, "{}"),
+    ("ivf", {"buckets_count": 16, "base_quantization_type": "fp32"}, json.dumps({"ivf": {"scan_buckets_count": 16}})),
+])
+def test_range_search(lib, name, params, search):
+    n, d, nq = 5000, 16, 12
+    x = vectors(n, d)
+    q = vectors(nq, d, seed=165)
+    labels = np.arange(n, dtype=np.int64) + 100
+    idx = make(name, d, "l2", **params)
+    assert idx.build(x, labels, n, d) == 0
+    x64 = x.astype(np.float64)
+    for i in range(nq):
+        dd = ((x64 - q[i].astype(np.float64)) ** 2).sum(1)
+        order = np.argsort(dd, kind="stable")
+        # a radius that takes in 1500 vectors: more than one device scan of 1024
+        for count in (7, 1500):
+            radius = 0.5 * float(dd[order[count - 1]] + dd[order[count]])
+            ids, dists = idx.range_search(q[i], radius, search)
+            # the bucket searcher admits radius + 2e-6 (THRESHOLD_ERROR, impl/searcher/basic_searcher.h:39)
+            slack = 2e-6 if name == "ivf" else 0.0
+            extra = int(np.sum((dd > radius) & (dd <= radius + slack + 1e-7)))
+            assert count <= ids.size <= count + extra, (i, count, ids.size)
+            assert np.all(np.diff(dists) >= 0) and dists[-1] <= radius + slack + 1e-7
+            assert set(ids[:count].tolist()) == set(labels[order[:count]].tolist())
+            np.testing.assert_allclose(dists[:count], dd[order[:count]], rtol=1e-4, atol=1e-6)
+            lim_ids, lim_d = idx.range_search(q[i], radius, search, limit=5)
+            assert lim_ids.size == 5 and set(lim_ids.tolist()) == set(labels[order[:5]].tolist())
+        ids, _ = idx.range_search(q[i], 0.0, search)  # nothing that close
+        assert ids.size == 0
+    with pytest.raises(pyvsag.VsagError) as e:
+        idx.range_search(q[0], -1.0, search)
+    assert e.value.code == -3
+    with pytest.raises(pyvsag.VsagError) as e:
+        idx.range_search(q[0], 1.0, search, limit=0)
+    assert e.value.code == -3
+    idx.close()

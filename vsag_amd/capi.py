@@ -36,6 +36,10 @@ class StoreParams(C.Structure):
                 ("centroid_dev", C.c_void_p), ("rabitq_query_bits", C.c_int)]
 
 
+class SearchOptions(C.Structure):
+    _fields_ = [("deny_bits_dev", C.c_void_p), ("use_radius", C.c_int), ("radius", C.c_float)]
+
+
 _u64, _u32, _i32, _sz, _vp, _f32 = C.c_uint64, C.c_uint32, C.c_int, C.c_size_t, C.c_void_p, C.c_float
 
 # name -> (restype, argtypes); the list is also what the export test checks against the header.
@@ -68,6 +72,7 @@ PROTOTYPES = {
     "vsag_amd_store_list_sizes": (C.c_int, [_vp, _vp, _u32]),
     "vsag_amd_flat_scan_workspace_bytes": (_sz, [_vp, _u64, _u32]),
     "vsag_amd_flat_scan_topk": (C.c_int, [_vp, _vp, _u64, _u32, _vp, _vp, _vp, _sz, _vp]),
+    "vsag_amd_flat_scan_topk_ex": (C.c_int, [_vp, _vp, _u64, _u32, _vp, _vp, _vp, _vp, _sz, _vp]),
     "vsag_amd_set_scan_tuning": (C.c_int, [_i32, _i32]),
     "vsag_amd_last_scan_info": (C.c_int, [C.POINTER(C.c_int), C.POINTER(_u64), C.POINTER(_u64)]),
     "vsag_amd_set_kernel_timing": (C.c_int, [_i32]),
@@ -83,6 +88,7 @@ PROTOTYPES = {
     "vsag_amd_ivf_route": (C.c_int, [_vp, _vp, _u64, _u32, _vp, _vp, _vp, _sz, _vp]),
     "vsag_amd_ivf_scan_workspace_bytes": (_sz, [_vp, _u64, _u32, _u32]),
     "vsag_amd_ivf_scan_topk": (C.c_int, [_vp, _vp, _u64, _vp, _u32, _u32, _vp, _vp, _vp, _sz, _vp]),
+    "vsag_amd_ivf_scan_topk_ex": (C.c_int, [_vp, _vp, _u64, _vp, _u32, _u32, _vp, _vp, _vp, _vp, _sz, _vp]),
     "vsag_amd_rerank_fp32": (C.c_int, [_vp, _u64, _u32, _i32, _vp, _u64, _vp, _u32, _u32, _vp, _vp, _vp]),
 }
 

@@ -128,4 +128,16 @@ make_key(float dist, uint32_t id) {
     return (static_cast<uint64_t>(float_to_ordered(dist)) << 32) | id;
 }
 
+// Bit `id` of a deny mask (vsag_amd_search_options_t::deny_bits_dev); a null mask denies nothing.
+__device__ inline bool
+denied(const uint32_t* deny, uint64_t id) {
+    return deny != nullptr && ((deny[id >> 5] >> (id & 31)) & 1U) != 0;
+}
+
+// The per-query bound a search starts from: nothing known, or the radius of a range search.
+inline uint32_t
+initial_bound(const vsag_amd_search_options_t* options) {
+    return options != nullptr && options->use_radius ? float_to_ordered(options->radius) : 0xFFFFFFFFU;
+}
+
 }  // namespace vsag_amd

@@ -123,6 +123,7 @@ struct IvfArgs {
     uint32_t dummy_query;        // index of an all-zero query row
     uint32_t k;
     uint32_t S;
+    const uint32_t* deny;        // filtered-out inner ids as a bit mask, or null
     uint32_t* bound;             // per query: ordered distance no final candidate can exceed
     uint64_t* partial;           // npairs_total x k keys
     uint32_t* partial_cnt;       // npairs_total
@@ -203,7 +204,7 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
         finish_distances<KIND, METRIC, T>(a, qidx, slot, acc, d);
         acc_reset(acc);
         const uint32_t id = v.ids[slot];
-        const bool valid = id != VSAG_AMD_INVALID_ID;
+        const bool valid = id != VSAG_AMD_INVALID_ID && !denied(v.deny, id);
 #pragma unroll
         for (int t = 0; t < T; ++t) {
             uint64_t key = make_key(d[t], id);
@@ -555,6 +556,14 @@ extern "C" int
 vsag_amd_ivf_scan_topk(const vsag_amd_store_t* s, const float* queries_dev, uint64_t nq, const int32_t* buckets_dev,
                        uint32_t nprobe, uint32_t kcand, uint32_t* ids_dev, float* dists_dev, void* workspace_dev,
                        size_t workspace_bytes, void* stream) {
+    return vsag_amd_ivf_scan_topk_ex(s, queries_dev, nq, buckets_dev, nprobe, kcand, nullptr, ids_dev, dists_dev,
+                                     workspace_dev, workspace_bytes, stream);
+}
+
+extern "C" int
+vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, uint64_t nq, const int32_t* buckets_dev,
+                          uint32_t nprobe, uint32_t kcand, const vsag_amd_search_options_t* options, uint32_t* ids_dev,
+                          float* dists_dev, void* workspace_dev, size_t workspace_bytes, void* stream) {
     VA_TRY(ensure_init());
     VA_TRY(check_ivf(s, nq, nprobe, kcand));
     VA_CHECK_ARG(queries_dev && buckets_dev && ids_dev && dists_dev, "null pointer");
@@ -569,7 +578,7 @@ vsag_amd_ivf_scan_topk(const vsag_amd_store_t* s, const float* queries_dev, uint
     // Row nq of the query tables is the all-zero row that idle slots of a query tile point at.
     VA_TRY(prepare_queries(s, queries_dev, nq, nq + 1, p.ql, b.qtab, b.qmeta, b.qcodes, st));
     ScanArgs a = make_scan_args(s, p.ql, b.qtab, b.qmeta);
-    hipLaunchKernelGGL(fill32_kernel, dim3(blocks_for(nq)), dim3(256), 0, st, b.bound, 0xFFFFFFFFU, nq);
+    hipLaunchKernelGGL(fill32_kernel, dim3(blocks_for(nq)), dim3(256), 0, st, b.bound, initial_bound(options), nq);
     hipLaunchKernelGGL(fill32_kernel, dim3(blocks_for(p.npairs)), dim3(256), 0, st, b.partial_cnt, 0U, p.npairs);
 
     IvfArgs v{};
@@ -583,6 +592,7 @@ vsag_amd_ivf_scan_topk(const vsag_amd_store_t* s, const float* queries_dev, uint
     v.dummy_query = static_cast<uint32_t>(nq);
     v.k = kcand;
     v.S = p.S;
+    v.deny = options != nullptr ? options->deny_bits_dev : nullptr;
     v.bound = b.bound;
     v.partial = b.partial;
     v.partial_cnt = b.partial_cnt;

@@ -30,10 +30,10 @@ constexpr uint32_t kMaxWaves = 4;
 
 // Per query: no bound yet, no seeds yet.
 __global__ void
-reset_queries_kernel(uint32_t* bound, uint64_t nq, uint32_t* seed, uint64_t nseed) {
+reset_queries_kernel(uint32_t* bound, uint32_t bound0, uint64_t nq, uint32_t* seed, uint64_t nseed) {
     uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i < nq) {
-        bound[i] = 0xFFFFFFFFU;
+        bound[i] = bound0;
     }
     if (i < nseed) {
         seed[i] = 0xFFFFFFFFU;
@@ -52,6 +52,7 @@ struct FlatArgs {
     uint64_t* partial;      // nq x nslots x k keys
     uint32_t* partial_cnt;  // nq x nslots
     uint32_t* seed;         // nq x k smallest first-tile distances by wave class, or null (see kSeedTiles)
+    const uint32_t* deny;   // filtered-out inner ids as a bit mask, or null
 };
 
 // Cold start.  A wave that begins without a bound would have to sort its first tiles just to learn a
@@ -139,7 +140,7 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
         float d[T];
         finish_distances<KIND, METRIC, T>(a, qidx, id, acc, d);
         acc_reset(acc);
-        const bool valid = id < f.n;
+        const bool valid = id < f.n && !denied(f.deny, id);
 #pragma unroll
         for (int t = 0; t < T; ++t) {
             // Inner ids grow along the scan, so "ordered distance < thr" is exactly the (distance, id)
@@ -517,6 +518,14 @@ extern "C" int
 vsag_amd_flat_scan_topk(const vsag_amd_store_t* s, const float* queries_dev, uint64_t nq, uint32_t k,
                         uint32_t* ids_dev, float* dists_dev, void* workspace_dev, size_t workspace_bytes,
                         void* stream) {
+    return vsag_amd_flat_scan_topk_ex(s, queries_dev, nq, k, nullptr, ids_dev, dists_dev, workspace_dev,
+                                      workspace_bytes, stream);
+}
+
+extern "C" int
+vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, uint64_t nq, uint32_t k,
+                           const vsag_amd_search_options_t* options, uint32_t* ids_dev, float* dists_dev,
+                           void* workspace_dev, size_t workspace_bytes, void* stream) {
     VA_TRY(ensure_init());
     VA_TRY(check_scan_call(s, nq, k));
     VA_CHECK_ARG(s->nlist == 0, "flat scan on a posting-list store");
@@ -532,7 +541,7 @@ vsag_amd_flat_scan_topk(const vsag_amd_store_t* s, const float* queries_dev, uin
     VA_TRY(prepare_queries(s, queries_dev, nq, p.nq_pad, p.ql, b.qtab, b.qmeta, b.qcodes, st));
     const uint64_t nseed = p.seeded ? nq * k : 0;
     hipLaunchKernelGGL(reset_queries_kernel, dim3(static_cast<uint32_t>(div_up(nq > nseed ? nq : nseed, 256))), dim3(256),
-                       0, st, b.bound, nq, b.seed, nseed);
+                       0, st, b.bound, initial_bound(options), nq, b.seed, nseed);
     ScanArgs a = make_scan_args(s, p.ql, b.qtab, b.qmeta);
     FlatArgs f{};
     f.n = s->n;
@@ -546,6 +555,7 @@ vsag_amd_flat_scan_topk(const vsag_amd_store_t* s, const float* queries_dev, uin
     f.partial = b.partial;
     f.partial_cnt = b.partial_cnt;
     f.seed = b.seed;
+    f.deny = options != nullptr ? options->deny_bits_dev : nullptr;
     if (s->ntiles != 0) {
         timing_begin(st);
         VA_TRY(launch_flat(s, p, a, f, st));

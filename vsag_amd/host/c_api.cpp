@@ -2,6 +2,7 @@
 #include "vsag_host_c_api.h"
 
 #include <algorithm>
+#include <functional>
 #include <cstdio>
 #include <cstring>
 #include <limits>
@@ -106,9 +107,12 @@ vsag_index_add(vsag_index_t index, const float* data, const int64_t* ids, uint64
     return success();
 }
 
-extern "C" Error_t
-vsag_index_knn_search(vsag_index_t index, const float* query, uint64_t dim, int64_t k, const char* parameters,
-                      SearchResult_t* search_result) {
+namespace {
+
+// Shared body of the four single-query searches: `range` selects RangeSearch(radius, limited_size = k).
+Error_t
+search_one(vsag_index_t index, const float* query, uint64_t dim, bool range, float radius, int64_t k,
+           const char* parameters, FilterFunc_t filter, SearchResult_t* search_result) {
     if (search_result == nullptr) {
         return make_error(VSAG_UNKNOWN_ERROR, "search result is NULL");
     }
@@ -117,11 +121,18 @@ vsag_index_knn_search(vsag_index_t index, const float* query, uint64_t dim, int6
         return make_error(VSAG_UNKNOWN_ERROR, "index is NULL");
     }
     if (k <= 0) {
-        return make_error(VSAG_INVALID_ARGUMENT, "knn_search requires k >= 1");
+        return make_error(VSAG_INVALID_ARGUMENT, range ? "range_search requires k >= 1" : "knn_search requires k >= 1");
     }
     auto q = vsag::Dataset::Make();
     q->Owner(false)->Dim(static_cast<int64_t>(dim))->NumElements(1)->Float32Vectors(query);
-    auto result = vi->index_->KnnSearch(q, k, parameters ? parameters : "");
+    const std::string params = parameters ? parameters : "";
+    std::function<bool(int64_t)> fn;
+    if (filter != nullptr) {
+        fn = [filter](int64_t id) { return filter(id); };
+    }
+    auto result = range ? (fn ? vi->index_->RangeSearch(q, radius, params, fn, k)
+                              : vi->index_->RangeSearch(q, radius, params, k))
+                        : (fn ? vi->index_->KnnSearch(q, k, params, fn) : vi->index_->KnnSearch(q, k, params));
     if (!result.has_value()) {
         return make_error(result.error());
     }
@@ -132,6 +143,32 @@ vsag_index_knn_search(vsag_index_t index, const float* query, uint64_t dim, int6
     }
     search_result->count = to_write;
     return success();
+}
+
+}  // namespace
+
+extern "C" Error_t
+vsag_index_knn_search(vsag_index_t index, const float* query, uint64_t dim, int64_t k, const char* parameters,
+                      SearchResult_t* search_result) {
+    return search_one(index, query, dim, false, 0.0F, k, parameters, nullptr, search_result);
+}
+
+extern "C" Error_t
+vsag_index_knn_search_with_filter(vsag_index_t index, const float* query, uint64_t dim, int64_t k,
+                                  const char* parameters, FilterFunc_t filter, SearchResult_t* search_result) {
+    return search_one(index, query, dim, false, 0.0F, k, parameters, filter, search_result);
+}
+
+extern "C" Error_t
+vsag_index_range_search(vsag_index_t index, const float* query, uint64_t dim, float radius, int64_t k,
+                        const char* parameters, SearchResult_t* search_result) {
+    return search_one(index, query, dim, true, radius, k, parameters, nullptr, search_result);
+}
+
+extern "C" Error_t
+vsag_index_range_search_with_filter(vsag_index_t index, const float* query, uint64_t dim, float radius, int64_t k,
+                                    const char* parameters, FilterFunc_t filter, SearchResult_t* search_result) {
+    return search_one(index, query, dim, true, radius, k, parameters, filter, search_result);
 }
 
 extern "C" Error_t

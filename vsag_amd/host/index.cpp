@@ -7,6 +7,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <functional>
 #include <limits>
 #include <mutex>
 #include <random>
@@ -433,8 +434,164 @@ reject_unknown_keys(const Json& index_param, const std::set<std::string>& known)
     }
 }
 
+// What a search asks for beyond (query, k): a pre-filter on labels and / or a radius.
+struct SearchSpec {
+    bool range = false;
+    float radius = 0.0F;
+    int64_t limited_size = -1;
+    std::function<bool(int64_t)> valid;  // empty = every label is kept
+};
+
+// Deny mask over inner ids for the device scans (bit set = filtered out), kept on the host as well so that
+// a range search can add the ids it has already returned.
+struct DenyMask {
+    std::vector<uint32_t> words;
+    DevBuf dev_words;
+    bool active = false;
+
+    void
+    init(const std::vector<int64_t>& labels, const std::function<bool(int64_t)>& valid, bool force) {
+        active = static_cast<bool>(valid) || force;
+        if (!active) {
+            return;
+        }
+        words.assign((labels.size() + 31) / 32, 0U);
+        if (valid) {
+            for (size_t i = 0; i < labels.size(); ++i) {
+                if (!valid(labels[i])) {
+                    words[i >> 5] |= 1U << (i & 31);
+                }
+            }
+        }
+        upload();
+    }
+    void
+    deny(uint32_t id) {
+        words[id >> 5] |= 1U << (id & 31);
+    }
+    void
+    upload() {
+        dev_words.reserve(std::max<size_t>(words.size() * 4, 4));
+        dev(vsag_amd_memcpy_h2d(dev_words.p, words.data(), words.size() * 4, nullptr));
+    }
+    vsag_amd_search_options_t
+    options(const SearchSpec& spec, float radius_slack) const {
+        vsag_amd_search_options_t o{};
+        o.deny_bits_dev = active ? dev_words.as<uint32_t>() : nullptr;
+        o.use_radius = spec.range ? 1 : 0;
+        o.radius = spec.radius + radius_slack;
+        return o;
+    }
+};
+
+constexpr int64_t kMaxDeviceK = 1024;  // largest k of one device scan
+
+// One ascending row of (distance, inner id) as a single-query result dataset.
+DatasetPtr
+pack_row(const std::vector<std::pair<float, uint32_t>>& row, const std::vector<int64_t>& labels,
+         const std::string& stats) {
+    std::vector<uint32_t> ids(std::max<size_t>(row.size(), 1), VSAG_AMD_INVALID_ID);
+    std::vector<float> dists(ids.size(), std::numeric_limits<float>::infinity());
+    for (size_t i = 0; i < row.size(); ++i) {
+        dists[i] = row[i].first;
+        ids[i] = row[i].second;
+    }
+    return pack_results(ids, dists, 1, static_cast<int64_t>(ids.size()), labels, stats);
+}
+
+// The search overloads of the public interface, reduced to one virtual search().
+class GpuIndex : public Index {
+public:
+    Expected<DatasetPtr>
+    KnnSearch(const DatasetPtr& query, int64_t k, const std::string& parameters) const override {
+        return run(query, k, parameters, SearchSpec{});
+    }
+    Expected<DatasetPtr>
+    KnnSearch(const DatasetPtr& query, int64_t k, const std::string& parameters, BitsetPtr invalid) const override {
+        return run(query, k, parameters, with_bitset(SearchSpec{}, invalid));
+    }
+    Expected<DatasetPtr>
+    KnnSearch(const DatasetPtr& query, int64_t k, const std::string& parameters,
+              const std::function<bool(int64_t)>& filter) const override {
+        return run(query, k, parameters, with_function(SearchSpec{}, filter));
+    }
+    Expected<DatasetPtr>
+    KnnSearch(const DatasetPtr& query, int64_t k, const std::string& parameters,
+              const FilterPtr& filter) const override {
+        return run(query, k, parameters, with_filter(SearchSpec{}, filter));
+    }
+    Expected<DatasetPtr>
+    RangeSearch(const DatasetPtr& query, float radius, const std::string& parameters,
+                int64_t limited_size) const override {
+        return run(query, 1, parameters, range_spec(radius, limited_size));
+    }
+    Expected<DatasetPtr>
+    RangeSearch(const DatasetPtr& query, float radius, const std::string& parameters, BitsetPtr invalid,
+                int64_t limited_size) const override {
+        return run(query, 1, parameters, with_bitset(range_spec(radius, limited_size), invalid));
+    }
+    Expected<DatasetPtr>
+    RangeSearch(const DatasetPtr& query, float radius, const std::string& parameters,
+                const std::function<bool(int64_t)>& filter, int64_t limited_size) const override {
+        return run(query, 1, parameters, with_function(range_spec(radius, limited_size), filter));
+    }
+    Expected<DatasetPtr>
+    RangeSearch(const DatasetPtr& query, float radius, const std::string& parameters, const FilterPtr& filter,
+                int64_t limited_size) const override {
+        return run(query, 1, parameters, with_filter(range_spec(radius, limited_size), filter));
+    }
+
+protected:
+    virtual DatasetPtr
+    search(const DatasetPtr& query, int64_t k, const std::string& parameters, const SearchSpec& spec) const = 0;
+
+private:
+    Expected<DatasetPtr>
+    run(const DatasetPtr& query, int64_t k, const std::string& parameters, const SearchSpec& spec) const {
+        return safe_call<DatasetPtr>([&]() {
+            if (spec.range) {
+                // InnerIndexInterface::validate_range_args (inner_index_interface.cpp:1252-1259)
+                CHECK_ARGUMENT(std::isfinite(spec.radius), "radius must be finite");
+                CHECK_ARGUMENT(spec.radius >= 0.0F,
+                               "radius(" + std::to_string(spec.radius) + ") must be greater equal than 0");
+                CHECK_ARGUMENT(spec.limited_size != 0, "limited_size(0) must not be equal to 0");
+            }
+            return search(query, k, parameters, spec);
+        });
+    }
+    static SearchSpec
+    range_spec(float radius, int64_t limited_size) {
+        SearchSpec s;
+        s.range = true;
+        s.radius = radius;
+        s.limited_size = limited_size;
+        return s;
+    }
+    static SearchSpec
+    with_bitset(SearchSpec s, const BitsetPtr& invalid) {
+        if (invalid != nullptr) {
+            s.valid = [invalid](int64_t label) { return !invalid->Test(label & 0xFFFFFFFFLL); };
+        }
+        return s;
+    }
+    static SearchSpec
+    with_function(SearchSpec s, const std::function<bool(int64_t)>& filter) {
+        if (filter) {
+            s.valid = [filter](int64_t label) { return !filter(label); };
+        }
+        return s;
+    }
+    static SearchSpec
+    with_filter(SearchSpec s, const FilterPtr& filter) {
+        if (filter != nullptr) {
+            s.valid = [filter](int64_t label) { return filter->CheckValid(label); };
+        }
+        return s;
+    }
+};
+
 // ------------------------------------------------------------------------------------------- brute_force
-class BruteForce : public Index {
+class BruteForce : public GpuIndex {
 public:
     BruteForce(const CommonParam& common, const Json& index_param) {
         static const std::set<std::string> known = {
@@ -483,42 +640,68 @@ public:
         });
     }
 
-    Expected<DatasetPtr>
-    KnnSearch(const DatasetPtr& query, int64_t k, const std::string& parameters) const override {
-        return safe_call<DatasetPtr>([&]() {
-            check_query(query, k, q_.dim);
-            if (!parameters.empty()) {
-                Json p = Json::Parse(parameters);  // {"parallelism": p}, optionally under "brute_force"
-                CHECK_ARGUMENT(p.IsObject(), "search parameters must be a JSON object");
-            }
-            std::lock_guard<std::mutex> lock(mutex_);
-            const int64_t nq = query->GetNumElements();
-            if (labels_.empty()) {
-                auto empty = Dataset::Make();
-                empty->NumElements(1)->Dim(0);
-                return empty;
-            }
-            CHECK_ARGUMENT(k <= 1024, "the GPU path supports k <= 1024, got " + std::to_string(k));
+protected:
+    DatasetPtr
+    search(const DatasetPtr& query, int64_t k, const std::string& parameters, const SearchSpec& spec) const override {
+        check_query(query, k, q_.dim);
+        if (!parameters.empty()) {
+            Json p = Json::Parse(parameters);  // {"parallelism": p}, optionally under "brute_force"
+            CHECK_ARGUMENT(p.IsObject(), "search parameters must be a JSON object");
+        }
+        std::lock_guard<std::mutex> lock(mutex_);
+        const int64_t nq = query->GetNumElements();
+        if (labels_.empty()) {
+            auto empty = Dataset::Make();
+            empty->NumElements(1)->Dim(0);
+            return empty;
+        }
+        CHECK_ARGUMENT(!spec.range || nq == 1, "range search takes one query");
+        CHECK_ARGUMENT(spec.range || k <= kMaxDeviceK, "the GPU path supports k <= 1024, got " + std::to_string(k));
+        queries_.reserve(static_cast<size_t>(nq) * q_.dim * 4);
+        dev(vsag_amd_memcpy_h2d(queries_.p, query->GetFloat32Vectors(), static_cast<size_t>(nq) * q_.dim * 4, nullptr));
+        DenyMask mask;
+        mask.init(labels_, spec.valid, spec.range);
+        const vsag_amd_search_options_t opt = mask.options(spec, 0.0F);
+        // distance_evaluations as the reference counts them: every stored vector once per query
+        const std::string stats = "{\"dist_cmp\":" + std::to_string(labels_.size() * static_cast<size_t>(nq)) + "}";
+        const auto n = static_cast<int64_t>(labels_.size());
+        if (!spec.range) {
             const auto kk = static_cast<uint32_t>(k);
-            queries_.reserve(static_cast<size_t>(nq) * q_.dim * 4);
-            dev(vsag_amd_memcpy_h2d(queries_.p, query->GetFloat32Vectors(), static_cast<size_t>(nq) * q_.dim * 4,
-                                    nullptr));
-            out_ids_.reserve(static_cast<size_t>(nq) * kk * 4);
-            out_d_.reserve(static_cast<size_t>(nq) * kk * 4);
-            size_t wsb = vsag_amd_flat_scan_workspace_bytes(store_.s, nq, kk);
-            workspace_.reserve(wsb);
-            dev(vsag_amd_flat_scan_topk(store_.s, queries_.as<float>(), nq, kk, out_ids_.as<uint32_t>(),
-                                        out_d_.as<float>(), workspace_.p, wsb, nullptr));
-            std::vector<uint32_t> ids(static_cast<size_t>(nq) * kk);
-            std::vector<float> dists(static_cast<size_t>(nq) * kk);
-            dev(vsag_amd_memcpy_d2h(ids.data(), out_ids_.p, ids.size() * 4, nullptr));
-            dev(vsag_amd_memcpy_d2h(dists.data(), out_d_.p, dists.size() * 4, nullptr));
-            // distance_evaluations as the reference counts them: every stored vector once per query
-            std::string stats = "{\"dist_cmp\":" + std::to_string(labels_.size() * static_cast<size_t>(nq)) + "}";
+            std::vector<uint32_t> ids;
+            std::vector<float> dists;
+            scan(nq, kk, opt, ids, dists);
             return pack_results(ids, dists, nq, k, labels_, stats);
-        });
+        }
+        // Range: the nearest candidates within the radius, a device scan of at most 1024 at a time; what a
+        // scan returned is denied to the next one, so the rows come out in ascending order.
+        std::vector<std::pair<float, uint32_t>> row;
+        int64_t remaining = spec.limited_size > 0 ? spec.limited_size : n;
+        while (remaining > 0) {
+            const auto kk = static_cast<uint32_t>(std::min<int64_t>({remaining, kMaxDeviceK, n}));
+            std::vector<uint32_t> ids;
+            std::vector<float> dists;
+            scan(1, kk, opt, ids, dists);
+            uint32_t got = 0;
+            while (got < kk && ids[got] != VSAG_AMD_INVALID_ID) {
+                row.emplace_back(dists[got], ids[got]);
+                mask.deny(ids[got]);
+                ++got;
+            }
+            remaining -= got;
+            if (got < kk) {
+                break;
+            }
+            mask.upload();
+        }
+        if (row.empty()) {
+            auto empty = Dataset::Make();
+            empty->NumElements(1)->Dim(0)->Statistics(stats);
+            return empty;
+        }
+        return pack_row(row, labels_, stats);
     }
 
+public:
     int64_t
     GetNumElements() const override {
         std::lock_guard<std::mutex> lock(mutex_);
@@ -526,6 +709,22 @@ public:
     }
 
 private:
+    // One device scan of the uploaded queries; results copied to the host.
+    void
+    scan(int64_t nq, uint32_t kk, const vsag_amd_search_options_t& opt, std::vector<uint32_t>& ids,
+         std::vector<float>& dists) const {
+        out_ids_.reserve(static_cast<size_t>(nq) * kk * 4);
+        out_d_.reserve(static_cast<size_t>(nq) * kk * 4);
+        size_t wsb = vsag_amd_flat_scan_workspace_bytes(store_.s, nq, kk);
+        workspace_.reserve(wsb);
+        dev(vsag_amd_flat_scan_topk_ex(store_.s, queries_.as<float>(), nq, kk, &opt, out_ids_.as<uint32_t>(),
+                                       out_d_.as<float>(), workspace_.p, wsb, nullptr));
+        ids.resize(static_cast<size_t>(nq) * kk);
+        dists.resize(ids.size());
+        dev(vsag_amd_memcpy_d2h(ids.data(), out_ids_.p, ids.size() * 4, nullptr));
+        dev(vsag_amd_memcpy_d2h(dists.data(), out_d_.p, dists.size() * 4, nullptr));
+    }
+
     std::vector<int64_t>
     add_locked(const DatasetPtr& base) {
         check_base(base, q_.dim);
@@ -565,7 +764,7 @@ private:
 };
 
 // ------------------------------------------------------------------------------------------- ivf
-class IVF : public Index {
+class IVF : public GpuIndex {
 public:
     IVF(const CommonParam& common, const Json& index_param) : common_(common) {
         static const std::set<std::string> known = {
@@ -644,97 +843,127 @@ public:
         });
     }
 
-    Expected<DatasetPtr>
-    KnnSearch(const DatasetPtr& query, int64_t k, const std::string& parameters) const override {
-        return safe_call<DatasetPtr>([&]() {
-            check_query(query, k, q_.dim);
-            // IVFSearchParameters::FromJson (src/algorithm/ivf/ivf_parameter.cpp:150-187)
-            Json params = Json::Parse(parameters);
-            CHECK_ARGUMENT(params.IsObject() && params.Contains("ivf"), "parameters must contains ivf");
-            const Json& ivf = params["ivf"];
-            CHECK_ARGUMENT(ivf.IsObject() && ivf.Contains("scan_buckets_count"),
-                           "parameters[ivf] must contains scan_buckets_count");
-            int64_t scan = ivf["scan_buckets_count"].GetInt();
-            CHECK_ARGUMENT(scan >= 1, "scan_buckets_count must be positive");
-            float factor = 2.0F;
-            if (ivf.Contains("factor")) {
-                factor = static_cast<float>(ivf["factor"].GetFloat());
-            }
-            bool enable_reorder = true;
-            if (ivf.Contains("enable_reorder")) {
-                enable_reorder = ivf["enable_reorder"].GetBool();
-            }
-            bool disable_scan = ivf.Contains("disable_bucket_scan") && ivf["disable_bucket_scan"].GetBool();
+protected:
+    DatasetPtr
+    search(const DatasetPtr& query, int64_t k, const std::string& parameters, const SearchSpec& spec) const override {
+        check_query(query, k, q_.dim);
+        // IVFSearchParameters::FromJson (src/algorithm/ivf/ivf_parameter.cpp:150-187)
+        Json params = Json::Parse(parameters);
+        CHECK_ARGUMENT(params.IsObject() && params.Contains("ivf"), "parameters must contains ivf");
+        const Json& ivf = params["ivf"];
+        CHECK_ARGUMENT(ivf.IsObject() && ivf.Contains("scan_buckets_count"),
+                       "parameters[ivf] must contains scan_buckets_count");
+        int64_t scan = ivf["scan_buckets_count"].GetInt();
+        CHECK_ARGUMENT(scan >= 1, "scan_buckets_count must be positive");
+        float factor = 2.0F;
+        if (ivf.Contains("factor")) {
+            factor = static_cast<float>(ivf["factor"].GetFloat());
+        }
+        bool enable_reorder = true;
+        if (ivf.Contains("enable_reorder")) {
+            enable_reorder = ivf["enable_reorder"].GetBool();
+        }
+        bool disable_scan = ivf.Contains("disable_bucket_scan") && ivf["disable_bucket_scan"].GetBool();
 
-            std::lock_guard<std::mutex> lock(mutex_);
-            const int64_t nq = query->GetNumElements();
-            if (labels_.empty()) {
-                auto empty = Dataset::Make();
-                empty->NumElements(1)->Dim(0);
-                return empty;
+        std::lock_guard<std::mutex> lock(mutex_);
+        const int64_t nq = query->GetNumElements();
+        if (labels_.empty()) {
+            auto empty = Dataset::Make();
+            empty->NumElements(1)->Dim(0);
+            return empty;
+        }
+        CHECK_ARGUMENT(!spec.range || nq == 1, "range search takes one query");
+        const auto n = static_cast<int64_t>(labels_.size());
+        const auto nprobe = static_cast<uint32_t>(std::min<int64_t>(scan, nlist_));  // ivf.cpp:1573-1574
+        const bool reorder = use_reorder_ && enable_reorder;
+        if (reorder) {
+            CHECK_ARGUMENT(factor > 0.0F, "factor must be positive when use_reorder is true");
+        }
+
+        queries_.reserve(static_cast<size_t>(nq) * q_.dim * 4);
+        dev(vsag_amd_memcpy_h2d(queries_.p, query->GetFloat32Vectors(), static_cast<size_t>(nq) * q_.dim * 4, nullptr));
+        // 1. route (exact nearest centroids)
+        buckets_.reserve(static_cast<size_t>(nq) * nprobe * 4);
+        bucket_d_.reserve(static_cast<size_t>(nq) * nprobe * 4);
+        size_t wsb = vsag_amd_ivf_route_workspace_bytes(centroid_store_.s, nq, nprobe);
+        workspace_.reserve(wsb);
+        dev(vsag_amd_ivf_route(centroid_store_.s, queries_.as<float>(), nq, nprobe, buckets_.as<int32_t>(),
+                               bucket_d_.as<float>(), workspace_.p, wsb, nullptr));
+        if (disable_scan && !spec.range) {
+            // routing only: bucket ids + centroid distances (ivf.cpp:1589-1660)
+            std::vector<uint32_t> ids(static_cast<size_t>(nq) * nprobe);
+            std::vector<float> dists(ids.size());
+            dev(vsag_amd_memcpy_d2h(ids.data(), buckets_.p, ids.size() * 4, nullptr));
+            dev(vsag_amd_memcpy_d2h(dists.data(), bucket_d_.p, dists.size() * 4, nullptr));
+            std::vector<int64_t> identity(nlist_);
+            for (uint32_t i = 0; i < nlist_; ++i) {
+                identity[i] = i;
             }
-            const auto nprobe = static_cast<uint32_t>(std::min<int64_t>(scan, nlist_));  // ivf.cpp:1573-1574
-            const bool reorder = use_reorder_ && enable_reorder;
+            return pack_results(ids, dists, nq, nprobe, identity, "{}");
+        }
+        DenyMask mask;
+        mask.init(labels_, spec.valid, spec.range);
+        // FlatBucketSearcher compares against radius + THRESHOLD_ERROR (flat_bucket_searcher.cpp:121,
+        // impl/searcher/basic_searcher.h:39).
+        const vsag_amd_search_options_t opt = mask.options(spec, 2e-6F);
+
+        if (!spec.range) {
             int64_t kcand = k;
             if (reorder) {
-                CHECK_ARGUMENT(factor > 0.0F, "factor must be positive when use_reorder is true");
-                kcand = static_cast<int64_t>(factor * static_cast<float>(k));  // ivf.cpp:2316
-                kcand = std::max<int64_t>(kcand, 1);
+                kcand = std::max<int64_t>(static_cast<int64_t>(factor * static_cast<float>(k)), 1);  // ivf.cpp:2316
             }
-            CHECK_ARGUMENT(kcand <= 1024 && k <= 1024, "the GPU path supports factor * k <= 1024");
-
-            queries_.reserve(static_cast<size_t>(nq) * q_.dim * 4);
-            dev(vsag_amd_memcpy_h2d(queries_.p, query->GetFloat32Vectors(), static_cast<size_t>(nq) * q_.dim * 4,
-                                    nullptr));
-            // 1. route (exact nearest centroids)
-            buckets_.reserve(static_cast<size_t>(nq) * nprobe * 4);
-            bucket_d_.reserve(static_cast<size_t>(nq) * nprobe * 4);
-            size_t wsb = vsag_amd_ivf_route_workspace_bytes(centroid_store_.s, nq, nprobe);
-            workspace_.reserve(wsb);
-            dev(vsag_amd_ivf_route(centroid_store_.s, queries_.as<float>(), nq, nprobe, buckets_.as<int32_t>(),
-                                   bucket_d_.as<float>(), workspace_.p, wsb, nullptr));
-            if (disable_scan) {
-                // routing only: bucket ids + centroid distances (ivf.cpp:1589-1660)
-                std::vector<uint32_t> ids(static_cast<size_t>(nq) * nprobe);
-                std::vector<float> dists(ids.size());
-                dev(vsag_amd_memcpy_d2h(ids.data(), buckets_.p, ids.size() * 4, nullptr));
-                dev(vsag_amd_memcpy_d2h(dists.data(), bucket_d_.p, dists.size() * 4, nullptr));
-                std::vector<int64_t> identity(nlist_);
-                for (uint32_t i = 0; i < nlist_; ++i) {
-                    identity[i] = i;
-                }
-                return pack_results(ids, dists, nq, nprobe, identity, "{}");
-            }
-            // 2. scan the probed lists
-            const auto kc = static_cast<uint32_t>(kcand);
-            cand_ids_.reserve(static_cast<size_t>(nq) * kc * 4);
-            cand_d_.reserve(static_cast<size_t>(nq) * kc * 4);
-            wsb = vsag_amd_ivf_scan_workspace_bytes(lists_.s, nq, nprobe, kc);
-            workspace_.reserve(wsb);
-            dev(vsag_amd_ivf_scan_topk(lists_.s, queries_.as<float>(), nq, buckets_.as<int32_t>(), nprobe, kc,
-                                       cand_ids_.as<uint32_t>(), cand_d_.as<float>(), workspace_.p, wsb, nullptr));
-            const DevBuf* final_ids = &cand_ids_;
-            const DevBuf* final_d = &cand_d_;
-            int64_t kout = kcand;
-            if (reorder) {
-                // 3. exact rerank, best min(k, candidates) kept (flatten_reorder.cpp:77)
-                kout = std::min<int64_t>(k, kcand);
-                out_ids_.reserve(static_cast<size_t>(nq) * kout * 4);
-                out_d_.reserve(static_cast<size_t>(nq) * kout * 4);
-                dev(vsag_amd_rerank_fp32(raw_.as<float>(), labels_.size(), q_.dim, q_.metric, queries_.as<float>(), nq,
-                                         cand_ids_.as<uint32_t>(), kc, static_cast<uint32_t>(kout),
-                                         out_ids_.as<uint32_t>(), out_d_.as<float>(), nullptr));
-                final_ids = &out_ids_;
-                final_d = &out_d_;
-            }
-            std::vector<uint32_t> ids(static_cast<size_t>(nq) * kout);
-            std::vector<float> dists(ids.size());
-            dev(vsag_amd_memcpy_d2h(ids.data(), final_ids->p, ids.size() * 4, nullptr));
-            dev(vsag_amd_memcpy_d2h(dists.data(), final_d->p, dists.size() * 4, nullptr));
+            CHECK_ARGUMENT(kcand <= kMaxDeviceK && k <= kMaxDeviceK, "the GPU path supports factor * k <= 1024");
+            // 2. scan the probed lists; 3. exact rerank, best min(k, candidates) kept (flatten_reorder.cpp:77)
+            const int64_t kout = reorder ? std::min<int64_t>(k, kcand) : kcand;
+            std::vector<uint32_t> ids;
+            std::vector<float> dists;
+            scan_lists(nq, nprobe, static_cast<uint32_t>(kcand), opt, reorder ? static_cast<uint32_t>(kout) : 0U, ids,
+                       dists);
             return pack_results(ids, dists, nq, kout, labels_, "{}");
-        });
+        }
+        // Range (ivf.cpp:2282-2307): candidates within the radius by the list codes, at most factor *
+        // limited_size of them when a rerank follows; the rerank keeps the nearest limited_size (all of them
+        // when unlimited).  A device scan returns at most 1024 candidates; what it returned is denied to the
+        // next scan.
+        int64_t want = spec.limited_size > 0 ? spec.limited_size : n;
+        if (reorder && spec.limited_size > 0) {
+            want = std::max<int64_t>(static_cast<int64_t>(factor * static_cast<float>(spec.limited_size)), 1);
+        }
+        std::vector<std::pair<float, uint32_t>> row;
+        int64_t remaining = want;
+        while (remaining > 0) {
+            const auto kc = static_cast<uint32_t>(std::min<int64_t>({remaining, kMaxDeviceK, n}));
+            std::vector<uint32_t> ids;
+            std::vector<float> dists;
+            scan_lists(1, nprobe, kc, opt, reorder ? kc : 0U, ids, dists);
+            uint32_t got = 0;
+            while (got < kc && ids[got] != VSAG_AMD_INVALID_ID) {
+                row.emplace_back(dists[got], ids[got]);
+                mask.deny(ids[got]);
+                ++got;
+            }
+            remaining -= got;
+            if (got < kc) {
+                break;
+            }
+            mask.upload();
+        }
+        if (reorder) {
+            // batches were reranked one by one: order the whole row by exact distance
+            std::sort(row.begin(), row.end());
+            if (spec.limited_size > 0 && static_cast<int64_t>(row.size()) > spec.limited_size) {
+                row.resize(static_cast<size_t>(spec.limited_size));
+            }
+        }
+        if (row.empty()) {
+            auto empty = Dataset::Make();
+            empty->NumElements(1)->Dim(0)->Statistics("{}");
+            return empty;
+        }
+        return pack_row(row, labels_, "{}");
     }
 
+public:
     int64_t
     GetNumElements() const override {
         std::lock_guard<std::mutex> lock(mutex_);
@@ -742,6 +971,36 @@ public:
     }
 
 private:
+    // Scan of the routed lists for the uploaded queries, then (rerank_k > 0) the exact fp32 rerank that keeps
+    // rerank_k; results copied to the host, kcand or rerank_k per query.
+    void
+    scan_lists(int64_t nq, uint32_t nprobe, uint32_t kcand, const vsag_amd_search_options_t& opt, uint32_t rerank_k,
+               std::vector<uint32_t>& ids, std::vector<float>& dists) const {
+        cand_ids_.reserve(static_cast<size_t>(nq) * kcand * 4);
+        cand_d_.reserve(static_cast<size_t>(nq) * kcand * 4);
+        size_t wsb = vsag_amd_ivf_scan_workspace_bytes(lists_.s, nq, nprobe, kcand);
+        workspace_.reserve(wsb);
+        dev(vsag_amd_ivf_scan_topk_ex(lists_.s, queries_.as<float>(), nq, buckets_.as<int32_t>(), nprobe, kcand, &opt,
+                                      cand_ids_.as<uint32_t>(), cand_d_.as<float>(), workspace_.p, wsb, nullptr));
+        const DevBuf* final_ids = &cand_ids_;
+        const DevBuf* final_d = &cand_d_;
+        uint32_t kout = kcand;
+        if (rerank_k > 0) {
+            kout = rerank_k;
+            out_ids_.reserve(static_cast<size_t>(nq) * kout * 4);
+            out_d_.reserve(static_cast<size_t>(nq) * kout * 4);
+            dev(vsag_amd_rerank_fp32(raw_.as<float>(), labels_.size(), q_.dim, q_.metric, queries_.as<float>(), nq,
+                                     cand_ids_.as<uint32_t>(), kcand, kout, out_ids_.as<uint32_t>(), out_d_.as<float>(),
+                                     nullptr));
+            final_ids = &out_ids_;
+            final_d = &out_d_;
+        }
+        ids.resize(static_cast<size_t>(nq) * kout);
+        dists.resize(ids.size());
+        dev(vsag_amd_memcpy_d2h(ids.data(), final_ids->p, ids.size() * 4, nullptr));
+        dev(vsag_amd_memcpy_d2h(dists.data(), final_d->p, dists.size() * 4, nullptr));
+    }
+
     // IVF::Train (ivf.cpp:564-588): sample, k-means (25 iterations, hard-coded in
     // ivf_nearest_partition.cpp:65-70), quantizer training on the same sample.
     void

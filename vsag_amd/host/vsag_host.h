@@ -3,12 +3,14 @@
 //   vsag::Index::{Build, Add, KnnSearch, GetNumElements}       (include/vsag/index.h:126,150,284-374)
 //   vsag::Dataset builder                                       (include/vsag/dataset.h:134-511)
 //   vsag::Error / ErrorType                                     (include/vsag/errors.h:26-56)
+//   vsag::Bitset, vsag::Filter                                  (include/vsag/bitset.h:27-101, filter.h:24-80)
 // Same names, argument meaning, JSON keys and error behaviour; the arithmetic behind it runs in the HIP
 // library (include/vsag_amd.h).  The reference returns tl::expected<T, Error>; Expected<T> below has the
 // same has_value() / value() / error() surface.
 #pragma once
 
 #include <cstdint>
+#include <functional>
 #include <memory>
 #include <string>
 #include <utility>
@@ -172,6 +174,56 @@ private:
     std::string statistics_;
 };
 
+// Pre-filter by bit mask: bit (label & 0xFFFFFFFF) set = the vector with that label is filtered OUT
+// (BlackListFilter::CheckValid, src/impl/filter/black_list_filter.cpp:24-31).
+class Bitset;
+using BitsetPtr = std::shared_ptr<Bitset>;
+class VSAG_HOST_EXPORT Bitset {
+public:
+    static BitsetPtr
+    Make() {
+        return BitsetPtr(new Bitset());
+    }
+    void
+    Set(int64_t pos, bool value = true) {
+        auto word = static_cast<size_t>(pos >> 6);
+        if (word >= words_.size()) {
+            if (!value) {
+                return;
+            }
+            words_.resize(word + 1, 0);
+        }
+        const uint64_t bit = 1ULL << (pos & 63);
+        words_[word] = value ? words_[word] | bit : words_[word] & ~bit;
+    }
+    bool
+    Test(int64_t pos) const {
+        auto word = static_cast<size_t>(pos >> 6);
+        return word < words_.size() && ((words_[word] >> (pos & 63)) & 1ULL) != 0;
+    }
+    uint64_t
+    Count() const {
+        uint64_t c = 0;
+        for (uint64_t w : words_) {
+            c += static_cast<uint64_t>(__builtin_popcountll(w));
+        }
+        return c;
+    }
+
+private:
+    Bitset() = default;
+    std::vector<uint64_t> words_;
+};
+
+// Pre-filter by callback object: CheckValid(label) == true keeps the vector.
+class Filter {
+public:
+    virtual ~Filter() = default;
+    virtual bool
+    CheckValid(int64_t id) const = 0;
+};
+using FilterPtr = std::shared_ptr<Filter>;
+
 class VSAG_HOST_EXPORT Index {
 public:
     virtual ~Index() = default;
@@ -188,6 +240,31 @@ public:
     // id -1 / distance +inf (the batch convention of IVF::SearchWithRequest, src/algorithm/ivf/ivf.cpp:2137-2210).
     virtual Expected<DatasetPtr>
     KnnSearch(const DatasetPtr& query, int64_t k, const std::string& parameters) const = 0;
+
+    // Pre-filtered searches (include/vsag/index.h:284-322).  invalid: see Bitset.  filter(label) == true
+    // filters the vector OUT (BlackListFilter); a FilterPtr keeps what CheckValid accepts.
+    virtual Expected<DatasetPtr>
+    KnnSearch(const DatasetPtr& query, int64_t k, const std::string& parameters, BitsetPtr invalid) const = 0;
+    virtual Expected<DatasetPtr>
+    KnnSearch(const DatasetPtr& query, int64_t k, const std::string& parameters,
+              const std::function<bool(int64_t)>& filter) const = 0;
+    virtual Expected<DatasetPtr>
+    KnnSearch(const DatasetPtr& query, int64_t k, const std::string& parameters, const FilterPtr& filter) const = 0;
+
+    // Everything within `radius` (distance <= radius), ascending; limited_size > 0 keeps the nearest
+    // limited_size, -1 keeps all, 0 is INVALID_ARGUMENT (include/vsag/index.h:394-466).
+    virtual Expected<DatasetPtr>
+    RangeSearch(const DatasetPtr& query, float radius, const std::string& parameters,
+                int64_t limited_size = -1) const = 0;
+    virtual Expected<DatasetPtr>
+    RangeSearch(const DatasetPtr& query, float radius, const std::string& parameters, BitsetPtr invalid,
+                int64_t limited_size = -1) const = 0;
+    virtual Expected<DatasetPtr>
+    RangeSearch(const DatasetPtr& query, float radius, const std::string& parameters,
+                const std::function<bool(int64_t)>& filter, int64_t limited_size = -1) const = 0;
+    virtual Expected<DatasetPtr>
+    RangeSearch(const DatasetPtr& query, float radius, const std::string& parameters, const FilterPtr& filter,
+                int64_t limited_size = -1) const = 0;
 
     virtual int64_t
     GetNumElements() const = 0;

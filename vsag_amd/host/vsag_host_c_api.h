@@ -53,6 +53,17 @@ VSAG_HOST_API Error_t vsag_index_add(vsag_index_t index, const float* data, cons
                                      uint64_t count);
 VSAG_HOST_API Error_t vsag_index_knn_search(vsag_index_t index, const float* query, uint64_t dim, int64_t k,
                                             const char* parameters, SearchResult_t* search_result);
+/* filter(label) == true filters the vector out (include/vsag/vsag_c_api.h:43,165-172). */
+typedef bool (*FilterFunc_t)(int64_t id);
+VSAG_HOST_API Error_t vsag_index_knn_search_with_filter(vsag_index_t index, const float* query, uint64_t dim, int64_t k,
+                                                        const char* parameters, FilterFunc_t filter,
+                                                        SearchResult_t* search_result);
+/* Everything within radius, at most k (>= 1) results, nearest first (vsag_c_api.h:186-216). */
+VSAG_HOST_API Error_t vsag_index_range_search(vsag_index_t index, const float* query, uint64_t dim, float radius,
+                                              int64_t k, const char* parameters, SearchResult_t* search_result);
+VSAG_HOST_API Error_t vsag_index_range_search_with_filter(vsag_index_t index, const float* query, uint64_t dim,
+                                                          float radius, int64_t k, const char* parameters,
+                                                          FilterFunc_t filter, SearchResult_t* search_result);
 /* nq queries at once; ids / dists have room for nq * k values, rows padded with -1 / +inf. */
 VSAG_HOST_API Error_t vsag_index_knn_search_batch(vsag_index_t index, const float* queries, uint64_t nq, uint64_t dim,
                                                   int64_t k, const char* parameters, int64_t* ids, float* dists,

@@ -1,7 +1,8 @@
 """Python view of the GPU-backed index classes with the call shapes of the reference's pyvsag.Index
 (python_bindings/index_binding.cpp:641-716): Index(name, parameters), build(vectors, ids, num_elements, dim),
-add(...), knn_search(vector, k, parameters) -> (ids, dists), get_num_elements().  knn_search_batch is the
-addition (many queries per call).  Everything goes through libvsag_amd_host.so's C API; errors raise
+add(...), knn_search(vector, k, parameters) -> (ids, dists), range_search(point, threshold, parameters),
+get_num_elements().  Additions: knn_search_batch (many queries per call) and the `filter` / `limit` keywords
+(the C API's *_with_filter entry points: filter(label) == True filters the vector out).  Everything goes through libvsag_amd_host.so's C API; errors raise
 VsagError with the reference's error code."""
 import ctypes as C
 import os
@@ -23,6 +24,9 @@ class ErrorT(C.Structure):
 class SearchResult(C.Structure):
     _fields_ = [("dists", C.POINTER(C.c_float)), ("ids", C.POINTER(C.c_int64)), ("count", C.c_int64),
                 ("other_result", C.c_void_p)]
+
+
+FILTER_FUNC = C.CFUNCTYPE(C.c_bool, C.c_int64)
 
 
 class VsagError(RuntimeError):
@@ -55,6 +59,15 @@ def _load():
         lib.vsag_index_knn_search.restype = ErrorT
         lib.vsag_index_knn_search.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int64, C.c_char_p,
                                               C.POINTER(SearchResult)]
+        lib.vsag_index_knn_search_with_filter.restype = ErrorT
+        lib.vsag_index_knn_search_with_filter.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_int64, C.c_char_p,
+                                                          FILTER_FUNC, C.POINTER(SearchResult)]
+        lib.vsag_index_range_search.restype = ErrorT
+        lib.vsag_index_range_search.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_float, C.c_int64, C.c_char_p,
+                                                C.POINTER(SearchResult)]
+        lib.vsag_index_range_search_with_filter.restype = ErrorT
+        lib.vsag_index_range_search_with_filter.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_float, C.c_int64,
+                                                            C.c_char_p, FILTER_FUNC, C.POINTER(SearchResult)]
         lib.vsag_index_knn_search_batch.restype = ErrorT
         lib.vsag_index_knn_search_batch.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint64, C.c_int64,
                                                     C.c_char_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_int64)]
@@ -92,14 +105,37 @@ class Index:
     def add(self, vectors, ids, num_elements, dim):
         return self._insert(_load().vsag_index_add, vectors, ids, num_elements, dim)
 
-    def knn_search(self, vector, k, parameters):
+    def knn_search(self, vector, k, parameters, filter=None):
         q = np.ascontiguousarray(vector, np.float32).reshape(-1)
         kk = max(int(k), 1)
         ids = np.empty(kk, np.int64)
         dists = np.empty(kk, np.float32)
         res = SearchResult(dists.ctypes.data_as(C.POINTER(C.c_float)), ids.ctypes.data_as(C.POINTER(C.c_int64)), 0,
                            None)
-        _check(_load().vsag_index_knn_search(self._h, q.ctypes.data, q.size, k, parameters.encode(), C.byref(res)))
+        if filter is None:
+            _check(_load().vsag_index_knn_search(self._h, q.ctypes.data, q.size, k, parameters.encode(), C.byref(res)))
+        else:
+            cb = FILTER_FUNC(lambda label: bool(filter(label)))
+            _check(_load().vsag_index_knn_search_with_filter(self._h, q.ctypes.data, q.size, k, parameters.encode(), cb,
+                                                             C.byref(res)))
+        return ids[:res.count].copy(), dists[:res.count].copy()
+
+    def range_search(self, point, threshold, parameters, limit=None, filter=None):
+        """Everything within `threshold`, nearest first; at most `limit` results (default: every vector)."""
+        q = np.ascontiguousarray(point, np.float32).reshape(-1)
+        kk = max(int(limit) if limit is not None else self.get_num_elements(), 1)
+        ids = np.empty(kk, np.int64)
+        dists = np.empty(kk, np.float32)
+        res = SearchResult(dists.ctypes.data_as(C.POINTER(C.c_float)), ids.ctypes.data_as(C.POINTER(C.c_int64)), 0,
+                           None)
+        lim = int(limit) if limit is not None else kk
+        if filter is None:
+            _check(_load().vsag_index_range_search(self._h, q.ctypes.data, q.size, threshold, lim, parameters.encode(),
+                                                   C.byref(res)))
+        else:
+            cb = FILTER_FUNC(lambda label: bool(filter(label)))
+            _check(_load().vsag_index_range_search_with_filter(self._h, q.ctypes.data, q.size, threshold, lim,
+                                                               parameters.encode(), cb, C.byref(res)))
         return ids[:res.count].copy(), dists[:res.count].copy()
 
     def knn_search_batch(self, vectors, k, parameters):
