@@ -10,6 +10,11 @@
 // per-query bound shared through global memory: the first probed list of every query is scanned in a
 // first launch and its kcand-th distance seeds the bound for the remaining lists.  The bound only ever
 // drops candidates that cannot be in the final kcand, so the result does not depend on scheduling.
+//
+// Few queries make few (query, list) pairs, and a wave per pair would leave the machine idle while each
+// wave walks a whole list.  Then lists are cut into chunks of a few tiles, a work item is (list, query
+// group, chunk), all probe columns go in one launch, and the cold waves learn a bound from each other's
+// first tiles as in the flat scan.
 #include "distance.h"
 #include "store.h"
 #include "topk.h"
@@ -22,7 +27,10 @@ struct ScanPlanIvf {
     QueryLayout ql;
     size_t qcode_bytes;
     uint64_t npairs;
-    uint64_t max_items;
+    uint32_t tiles_per_item;  // 0xFFFFFFFF: a work item walks its whole list
+    uint32_t chunks_max;      // partial lists per (query, list) pair
+    bool chunked;             // one launch over all probe columns, seeded cold start
+    bool seeded;
 };
 
 uint64_t rabitq_query_code_size(uint32_t dim, int metric, int query_bits);
@@ -31,12 +39,24 @@ int prepare_queries(const vsag_amd_store* s, const float* queries, uint64_t nq, 
 ScanArgs make_scan_args(const vsag_amd_store* s, const QueryLayout& ql, const uint32_t* qtab, const float* qmeta);
 void timing_begin(hipStream_t st);
 void timing_end(hipStream_t st);
+int launch_merge_partials(const uint64_t* partial, const uint32_t* partial_cnt, const uint32_t* bound, uint32_t nslots,
+                          uint32_t k, uint32_t S, uint64_t nq, uint32_t* ids, float* dists, hipStream_t st);
+
+// Up to five word arrays set in one launch.
+struct FillJob {
+    uint32_t* p[5];
+    uint32_t v[5];
+    uint64_t n[5];
+};
 
 __global__ void
-fill32_kernel(uint32_t* p, uint32_t v, uint64_t n) {
+fill_jobs_kernel(FillJob j) {
     uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (i < n) {
-        p[i] = v;
+#pragma unroll
+    for (int a = 0; a < 5; ++a) {
+        if (i < j.n[a]) {
+            j.p[a][i] = j.v[a];
+        }
     }
 }
 
@@ -57,9 +77,17 @@ count_pairs_kernel(const int32_t* buckets, uint64_t nq, uint32_t nprobe, uint32_
     }
 }
 
-// One workgroup: exclusive prefix sums of the pair counts and of the work items ceil(count / T).
+// Work items of a list: query groups x tile chunks.
+__device__ inline uint32_t
+list_items(uint32_t pairs, uint32_t T, uint32_t tiles, uint32_t tiles_per_item) {
+    uint32_t chunks = tiles_per_item == 0xFFFFFFFFU ? (tiles != 0 ? 1U : 0U) : (tiles + tiles_per_item - 1) / tiles_per_item;
+    return ((pairs + T - 1) / T) * chunks;
+}
+
+// One workgroup: exclusive prefix sums of the pair counts and of the work items.
 __global__ void __launch_bounds__(1024)
-offsets_kernel(const uint32_t* counts, uint32_t nlist, uint32_t T, uint32_t* pair_off, uint32_t* item_off) {
+offsets_kernel(const uint32_t* counts, const uint32_t* list_tile, uint32_t nlist, uint32_t T, uint32_t tiles_per_item,
+               uint32_t* pair_off, uint32_t* item_off) {
     __shared__ uint32_t s_pairs[1024];
     __shared__ uint32_t s_items[1024];
     uint32_t per = (nlist + blockDim.x - 1) / blockDim.x;
@@ -68,7 +96,7 @@ offsets_kernel(const uint32_t* counts, uint32_t nlist, uint32_t T, uint32_t* pai
     uint32_t sp = 0, si = 0;
     for (uint32_t i = begin; i < end; ++i) {
         sp += counts[i];
-        si += (counts[i] + T - 1) / T;
+        si += list_items(counts[i], T, list_tile[i + 1] - list_tile[i], tiles_per_item);
     }
     s_pairs[threadIdx.x] = sp;
     s_items[threadIdx.x] = si;
@@ -91,7 +119,7 @@ offsets_kernel(const uint32_t* counts, uint32_t nlist, uint32_t T, uint32_t* pai
         pair_off[i] = rp;
         item_off[i] = ri;
         rp += counts[i];
-        ri += (counts[i] + T - 1) / T;
+        ri += list_items(counts[i], T, list_tile[i + 1] - list_tile[i], tiles_per_item);
     }
 }
 
@@ -124,12 +152,18 @@ struct IvfArgs {
     uint32_t k;
     uint32_t S;
     const uint32_t* deny;        // filtered-out inner ids as a bit mask, or null
+    uint32_t tiles_per_item;     // 0xFFFFFFFF: whole lists
+    uint32_t chunks_max;         // partial lists per pair
     uint32_t* bound;             // per query: ordered distance no final candidate can exceed
-    uint64_t* partial;           // npairs_total x k keys
-    uint32_t* partial_cnt;       // npairs_total
+    uint32_t* seed;              // nq x k first-tile minima by work-item class, or null (flat scan's cold start)
+    uint64_t* partial;           // npairs_total x chunks_max x k keys
+    uint32_t* partial_cnt;       // npairs_total x chunks_max
 };
 
-template <int KIND, int METRIC, int T>
+constexpr uint32_t kIvfSeedTiles = 4;
+
+// CHUNKED: work items are chunks of lists and start cold together (few queries); otherwise whole lists.
+template <int KIND, int METRIC, int T, bool CHUNKED>
 __global__ void __launch_bounds__(256)
 ivf_scan_kernel(ScanArgs a, IvfArgs v) {
     extern __shared__ uint64_t lds[];
@@ -152,7 +186,16 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
         }
     }
     const uint32_t b = lo;
-    const uint32_t group = item - ioff[b];
+    const uint32_t list_begin = as_const(v.list_tile)[b], list_end = as_const(v.list_tile)[b + 1];
+    uint32_t group = item - ioff[b], chunk = 0;
+    uint32_t tbeg = list_begin, tend = list_end;
+    if (CHUNKED) {
+        const uint32_t chunks = (list_end - list_begin + v.tiles_per_item - 1) / v.tiles_per_item;
+        chunk = group % chunks;
+        group = group / chunks;
+        tbeg = list_begin + chunk * v.tiles_per_item;
+        tend = tbeg + v.tiles_per_item < list_end ? tbeg + v.tiles_per_item : list_end;
+    }
     const uint32_t pbeg = as_const(v.pair_off)[b] + group * T;
     const uint32_t pend = as_const(v.pair_off)[b + 1];
 
@@ -161,6 +204,7 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
     uint32_t qidx[T], pair[T];
     uint64_t tau[T];
     uint32_t cnt[T];
+    uint32_t cold[T];  // tiles after which this item still looks at the seed row (see the flat scan)
 #pragma unroll
     for (int t = 0; t < T; ++t) {
         bool live = pbeg + t < pend;
@@ -171,13 +215,14 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
                               : 0U;
         // Everything at or below the bound passes, whatever its id.
         tau[t] = (static_cast<uint64_t>(bound) << 32) | 0xFFFFFFFFULL;
+        cold[t] = CHUNKED && v.seed != nullptr && live && bound == 0xFFFFFFFFU ? kIvfSeedTiles : 0;
     }
+    const uint32_t seed_slot = item % k;
     for (uint32_t i = lane; i < T * S; i += kWave) {
         sel[i] = kInfKey;
     }
     wave_lds_fence();
 
-    const uint32_t tbeg = as_const(v.list_tile)[b], tend = as_const(v.list_tile)[b + 1];
     const QueryRows<T> qrows = query_rows<T>(a, qidx);
     constexpr int GROUP = GroupOf<T>::value;
     TileStream<GROUP> cur{a.tiles, lane, tbeg, tend, 1, 0, a.G};
@@ -208,6 +253,26 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
 #pragma unroll
         for (int t = 0; t < T; ++t) {
             uint64_t key = make_key(d[t], id);
+            if (CHUNKED && cold[t] != 0) {
+                uint32_t* row = v.seed + static_cast<uint64_t>(qidx[t]) * k;
+                if (cold[t] == kIvfSeedTiles) {
+                    uint32_t m = wave_min_u32(valid ? static_cast<uint32_t>(key >> 32) : 0xFFFFFFFFU);
+                    lower_shared(&row[seed_slot], m, lane);
+                }
+                --cold[t];
+                uint32_t mx = 0;
+                for (uint32_t i = lane; i < k; i += kWave) {
+                    uint32_t sv = __atomic_load_n(&row[i], __ATOMIC_RELAXED);
+                    mx = sv > mx ? sv : mx;
+                }
+                mx = wave_max_u32(mx);
+                if (mx != 0xFFFFFFFFU) {
+                    cold[t] = 0;
+                    mx = lower_shared(&v.bound[qidx[t]], mx, lane);
+                    uint64_t shared_tau = (static_cast<uint64_t>(mx) << 32) | 0xFFFFFFFFULL;
+                    tau[t] = tau[t] < shared_tau ? tau[t] : shared_tau;
+                }
+            }
             bool pass = valid && key < tau[t];
             uint64_t mask = __ballot(pass);
             if (mask == 0) {
@@ -218,6 +283,7 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
             if (k + cnt[t] + np > S) {
                 uint64_t th = selector_flush(keys, S, k, cnt[t], lane);
                 cnt[t] = 0;
+                cold[t] = 0;
                 if (pair[t] != 0xFFFFFFFFU) {
                     // th finite: this pair alone already holds k candidates at or below th.
                     uint32_t bound = lower_shared(&v.bound[qidx[t]], static_cast<uint32_t>(th >> 32), lane);
@@ -272,113 +338,108 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
             }
             lower_shared(&v.bound[qidx[t]], wave_max_u32(mx), lane);  // bs itself must stay what was counted with
         }
+        const uint64_t list = static_cast<uint64_t>(pair[t]) * v.chunks_max + chunk;
         if (lane == 0) {
-            v.partial_cnt[pair[t]] = admitted;
+            v.partial_cnt[list] = admitted;
         }
         if (admitted != 0) {
-            selector_copy_admitted(keys, total, bs, v.partial + static_cast<uint64_t>(pair[t]) * k, lane);
+            selector_copy_admitted(keys, total, bs, v.partial + list * k, lane);
         }
     }
 }
 
-// One wave per query: best k keys over the partial lists of its nprobe pairs.
-__global__ void __launch_bounds__(64)
-ivf_merge_kernel(const uint64_t* partial, const uint32_t* partial_cnt, uint32_t nprobe, uint32_t k, uint32_t S,
-                 uint32_t* ids, float* dists) {
-    extern __shared__ uint64_t lds[];
-    const uint32_t lane = threadIdx.x;
-    const uint64_t q = blockIdx.x;
-    selector_init(lds, S, lane);
-    uint32_t cnt = 0;
-    uint64_t tau = kInfKey;
-    for (uint32_t p = 0; p < nprobe; ++p) {
-        uint64_t pair = q * nprobe + p;
-        uint32_t c = as_const(partial_cnt)[pair];
-        const uint64_t* src = partial + pair * k;
-        for (uint32_t base = 0; base < c; base += kWave) {
-            uint32_t i = base + lane;
-            uint64_t key = i < c ? src[i] : kInfKey;
-            bool pass = key < tau;
-            cnt = selector_append(lds, k, cnt, pass, key);
-            if (cnt + kWave > S - k) {
-                tau = selector_flush(lds, S, k, cnt, lane);
-                cnt = 0;
-            }
-        }
-    }
-    selector_flush(lds, S, k, cnt, lane);
-    for (uint32_t i = lane; i < k; i += kWave) {
-        uint64_t key = lds[i];
-        if (key == kInfKey) {
-            ids[q * k + i] = VSAG_AMD_INVALID_ID;
-            dists[q * k + i] = __builtin_inff();
-        } else {
-            ids[q * k + i] = static_cast<uint32_t>(key);
-            dists[q * k + i] = ordered_to_float(static_cast<uint32_t>(key >> 32));
-        }
-    }
-}
+// Exact fp32 distances of the candidates of one query, best k kept.  One workgroup of four waves per query;
+// sixteen lanes share a candidate, so a workgroup has sixteen gathered rows in flight.
+constexpr uint32_t kRerankThreads = 256;
 
-// Exact fp32 distances of the candidates of one query (one wave per query), best k kept.
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(kRerankThreads)
 rerank_kernel(const float* raw, uint64_t n, uint32_t dim, int metric, const float* queries, const uint32_t* cand,
               uint32_t kcand, uint32_t k, uint32_t S, uint32_t* ids, float* dists) {
     extern __shared__ uint64_t lds[];
-    const uint32_t lane = threadIdx.x;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t sub = tid >> 4, l = tid & 15;  // candidate slot of this step, lane within it
     const uint64_t q = blockIdx.x;
     const float* qv = queries + q * dim;
-    for (uint32_t i = lane; i < S; i += kWave) {
+    for (uint32_t i = tid; i < S; i += kRerankThreads) {
         lds[i] = kInfKey;
     }
-    wave_lds_fence();
     float inv_norm = 1.0F;
     if (metric == VSAG_AMD_METRIC_COSINE) {
         float s = 0.0F;
-        for (uint32_t d = lane; d < dim; d += kWave) {
+        for (uint32_t d = l; d < dim; d += 16) {
             s = fmaf(qv[d], qv[d], s);
         }
-        for (int off = 32; off > 0; off >>= 1) {
+        for (int off = 8; off > 0; off >>= 1) {
             s += __shfl_xor(s, off);
         }
         inv_norm = s > 0.0F ? 1.0F / sqrtf(s) : 1.0F;
     }
-    for (uint32_t j = 0; j < kcand; ++j) {
-        uint32_t id = as_const(cand)[q * kcand + j];
-        if (id == VSAG_AMD_INVALID_ID || id >= n) {
-            continue;
-        }
-        const float* x = raw + static_cast<uint64_t>(id) * dim;
+    __syncthreads();
+    const bool vec4 = (dim & 3) == 0;
+    for (uint32_t j0 = 0; j0 < kcand; j0 += kRerankThreads / 16) {
+        const uint32_t j = j0 + sub;
+        uint32_t id = j < kcand ? as_const(cand)[q * kcand + j] : VSAG_AMD_INVALID_ID;
+        const bool live = id != VSAG_AMD_INVALID_ID && id < n;
+        const float* x = raw + static_cast<uint64_t>(live ? id : 0) * dim;
         float s = 0.0F, xx = 0.0F;
-        for (uint32_t d = lane; d < dim; d += kWave) {
-            float xv = x[d];
-            if (metric == VSAG_AMD_METRIC_L2) {
-                float t = qv[d] - xv;
-                s = fmaf(t, t, s);
+        if (live) {
+            if (vec4) {
+                for (uint32_t d = l * 4; d < dim; d += 64) {
+                    float4 xv = *reinterpret_cast<const float4*>(x + d);
+                    float4 qq = *reinterpret_cast<const float4*>(qv + d);
+                    if (metric == VSAG_AMD_METRIC_L2) {
+                        float t0 = qq.x - xv.x, t1 = qq.y - xv.y, t2 = qq.z - xv.z, t3 = qq.w - xv.w;
+                        s = fmaf(t0, t0, s);
+                        s = fmaf(t1, t1, s);
+                        s = fmaf(t2, t2, s);
+                        s = fmaf(t3, t3, s);
+                    } else {
+                        s = fmaf(qq.x, xv.x, s);
+                        s = fmaf(qq.y, xv.y, s);
+                        s = fmaf(qq.z, xv.z, s);
+                        s = fmaf(qq.w, xv.w, s);
+                        xx = fmaf(xv.x, xv.x, xx);
+                        xx = fmaf(xv.y, xv.y, xx);
+                        xx = fmaf(xv.z, xv.z, xx);
+                        xx = fmaf(xv.w, xv.w, xx);
+                    }
+                }
             } else {
-                s = fmaf(qv[d], xv, s);
-                xx = fmaf(xv, xv, xx);
+                for (uint32_t d = l; d < dim; d += 16) {
+                    float xv = x[d];
+                    if (metric == VSAG_AMD_METRIC_L2) {
+                        float t = qv[d] - xv;
+                        s = fmaf(t, t, s);
+                    } else {
+                        s = fmaf(qv[d], xv, s);
+                        xx = fmaf(xv, xv, xx);
+                    }
+                }
             }
         }
-        for (int off = 32; off > 0; off >>= 1) {
+        for (int off = 8; off > 0; off >>= 1) {
             s += __shfl_xor(s, off);
             xx += __shfl_xor(xx, off);
         }
-        float dist;
-        if (metric == VSAG_AMD_METRIC_L2) {
-            dist = s;
-        } else if (metric == VSAG_AMD_METRIC_IP) {
-            dist = 1.0F - s;
-        } else {
-            float xn = xx > 0.0F ? 1.0F / sqrtf(xx) : 1.0F;
-            dist = 1.0F - s * inv_norm * xn;
-        }
-        if (lane == 0) {
+        if (live && l == 0) {
+            float dist;
+            if (metric == VSAG_AMD_METRIC_L2) {
+                dist = s;
+            } else if (metric == VSAG_AMD_METRIC_IP) {
+                dist = 1.0F - s;
+            } else {
+                float xn = xx > 0.0F ? 1.0F / sqrtf(xx) : 1.0F;
+                dist = 1.0F - s * inv_norm * xn;
+            }
             lds[j] = make_key(dist, id);
         }
     }
-    wave_lds_fence();
-    wave_bitonic_sort(lds, S, lane);
-    for (uint32_t i = lane; i < k; i += kWave) {
+    __syncthreads();
+    if (tid >= kWave) {
+        return;
+    }
+    wave_bitonic_sort(lds, S, tid);
+    for (uint32_t i = tid; i < k; i += kWave) {
         uint64_t key = lds[i];
         if (key == kInfKey) {
             ids[q * k + i] = VSAG_AMD_INVALID_ID;
@@ -387,6 +448,16 @@ rerank_kernel(const float* raw, uint64_t n, uint32_t dim, int metric, const floa
             ids[q * k + i] = static_cast<uint32_t>(key);
             dists[q * k + i] = ordered_to_float(static_cast<uint32_t>(key >> 32));
         }
+    }
+}
+
+template <int KIND, int METRIC, int T>
+static void
+launch_ivf_c(dim3 grid, dim3 block, size_t lds, hipStream_t st, const ScanArgs& a, const IvfArgs& v) {
+    if (v.tiles_per_item != 0xFFFFFFFFU) {
+        hipLaunchKernelGGL((ivf_scan_kernel<KIND, METRIC, T, true>), grid, block, lds, st, a, v);
+    } else {
+        hipLaunchKernelGGL((ivf_scan_kernel<KIND, METRIC, T, false>), grid, block, lds, st, a, v);
     }
 }
 
@@ -395,13 +466,13 @@ static void
 launch_ivf_t(int T, dim3 grid, dim3 block, size_t lds, hipStream_t st, const ScanArgs& a, const IvfArgs& v) {
     switch (T) {
         case 1:
-            hipLaunchKernelGGL((ivf_scan_kernel<KIND, METRIC, 1>), grid, block, lds, st, a, v);
+            launch_ivf_c<KIND, METRIC, 1>(grid, block, lds, st, a, v);
             break;
         case 2:
-            hipLaunchKernelGGL((ivf_scan_kernel<KIND, METRIC, 2>), grid, block, lds, st, a, v);
+            launch_ivf_c<KIND, METRIC, 2>(grid, block, lds, st, a, v);
             break;
         default:
-            hipLaunchKernelGGL((ivf_scan_kernel<KIND, METRIC, 4>), grid, block, lds, st, a, v);
+            launch_ivf_c<KIND, METRIC, 4>(grid, block, lds, st, a, v);
             break;
     }
 }
@@ -458,6 +529,7 @@ struct IvfBuffers {
     uint32_t* item_off;   // nlist + 1
     uint32_t* sorted_pair;
     uint32_t* bound;
+    uint32_t* seed;
     uint32_t* partial_cnt;
     uint64_t* partial;
 };
@@ -487,7 +559,23 @@ plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, 
         p->qcode_bytes = nq * rabitq_query_code_size(s->dim, s->metric, s->query_bits);
     }
     p->npairs = npairs;
-    p->max_items = div_up(npairs, t) + s->nlist;
+    // Enough (list, query group) items to fill the machine: every item walks its whole list, the nearest list
+    // of every query goes first.  Otherwise lists are cut into chunks for about 8192 items in all (a probed
+    // list is taken as twice the average length), within 256 MiB of partial lists.
+    const uint64_t groups = div_up(npairs, static_cast<uint64_t>(t));
+    p->chunked = groups < 8192 && s->max_list_tiles > 2;
+    p->tiles_per_item = 0xFFFFFFFFU;
+    p->chunks_max = 1;
+    if (p->chunked) {
+        const uint64_t avg_tiles = std::max<uint64_t>(1, s->nlist ? s->ntiles / s->nlist : 1);
+        uint64_t tpi = std::max<uint64_t>(2, div_up(groups * avg_tiles * 2, 8192));
+        while (npairs * div_up(s->max_list_tiles, tpi) * kcand * 8 > (256ull << 20)) {
+            tpi *= 2;
+        }
+        p->tiles_per_item = static_cast<uint32_t>(std::min<uint64_t>(tpi, 0x7FFFFFFFU));
+        p->chunks_max = static_cast<uint32_t>(div_up(s->max_list_tiles, tpi));
+    }
+    p->seeded = p->chunked && kcand <= 256;
 }
 
 static size_t
@@ -501,8 +589,9 @@ carve_ivf(Carver& c, const vsag_amd_store* s, const ScanPlanIvf& p, uint64_t nq,
     b->item_off = c.take<uint32_t>(s->nlist + 1);
     b->sorted_pair = c.take<uint32_t>(p.npairs);
     b->bound = c.take<uint32_t>(nq);
-    b->partial_cnt = c.take<uint32_t>(p.npairs);
-    b->partial = c.take<uint64_t>(p.npairs * kcand);
+    b->seed = c.take<uint32_t>(p.seeded ? nq * kcand : 0);
+    b->partial_cnt = c.take<uint32_t>(p.npairs * p.chunks_max);
+    b->partial = c.take<uint64_t>(p.npairs * p.chunks_max * kcand);
     return c.used;
 }
 
@@ -578,8 +667,19 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
     // Row nq of the query tables is the all-zero row that idle slots of a query tile point at.
     VA_TRY(prepare_queries(s, queries_dev, nq, nq + 1, p.ql, b.qtab, b.qmeta, b.qcodes, st));
     ScanArgs a = make_scan_args(s, p.ql, b.qtab, b.qmeta);
-    hipLaunchKernelGGL(fill32_kernel, dim3(blocks_for(nq)), dim3(256), 0, st, b.bound, initial_bound(options), nq);
-    hipLaunchKernelGGL(fill32_kernel, dim3(blocks_for(p.npairs)), dim3(256), 0, st, b.partial_cnt, 0U, p.npairs);
+    const uint64_t nlists1 = static_cast<uint64_t>(s->nlist) + 1;
+    const uint64_t nslots_all = p.npairs * p.chunks_max;
+    const uint64_t nseed = p.seeded ? nq * kcand : 0;
+    auto fill = [&](const FillJob& job) {
+        uint64_t most = 0;
+        for (uint64_t n : job.n) {
+            most = std::max(most, n);
+        }
+        hipLaunchKernelGGL(fill_jobs_kernel, dim3(blocks_for(most)), dim3(256), 0, st, job);
+    };
+    fill(FillJob{{b.bound, b.partial_cnt, b.counts, b.cursor, b.seed},
+                 {initial_bound(options), 0U, 0U, 0U, 0xFFFFFFFFU},
+                 {nq, nslots_all, nlists1, nlists1, nseed}});
 
     IvfArgs v{};
     v.ids = s->ids_dev;
@@ -593,7 +693,10 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
     v.k = kcand;
     v.S = p.S;
     v.deny = options != nullptr ? options->deny_bits_dev : nullptr;
+    v.tiles_per_item = p.tiles_per_item;
+    v.chunks_max = p.chunks_max;
     v.bound = b.bound;
+    v.seed = p.seeded ? b.seed : nullptr;
     v.partial = b.partial;
     v.partial_cnt = b.partial_cnt;
 
@@ -602,8 +705,9 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
         waves >>= 1;
     }
     size_t lds = static_cast<size_t>(waves) * p.T * p.S * 8;
-    // Two passes: the nearest list of every query first (it seeds the per-query bound), then the rest.
-    uint32_t cols[3] = {0, 1, nprobe};
+    // Whole lists: two passes, the nearest list of every query first (it seeds the per-query bound), then the
+    // rest.  Chunked lists: all probe columns at once.
+    uint32_t cols[3] = {0, p.chunked ? nprobe : 1, nprobe};
     timing_begin(st);
     for (int pass = 0; pass < 2; ++pass) {
         uint32_t p0 = cols[pass], p1 = cols[pass + 1];
@@ -611,25 +715,23 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
             continue;
         }
         uint64_t pairs = nq * (p1 - p0);
-        hipLaunchKernelGGL(fill32_kernel, dim3(blocks_for(s->nlist + 1)), dim3(256), 0, st, b.counts, 0U,
-                           static_cast<uint64_t>(s->nlist + 1));
-        hipLaunchKernelGGL(fill32_kernel, dim3(blocks_for(s->nlist + 1)), dim3(256), 0, st, b.cursor, 0U,
-                           static_cast<uint64_t>(s->nlist + 1));
+        if (pass == 1) {
+            fill(FillJob{{b.counts, b.cursor, nullptr, nullptr, nullptr}, {0U, 0U, 0U, 0U, 0U}, {nlists1, nlists1, 0, 0, 0}});
+        }
         hipLaunchKernelGGL(count_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq, nprobe, p0,
                            p1, s->nlist, b.counts);
-        hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, st, b.counts, s->nlist,
-                           static_cast<uint32_t>(p.T), b.pair_off, b.item_off);
+        hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, st, b.counts, s->list_tile_dev, s->nlist,
+                           static_cast<uint32_t>(p.T), p.tiles_per_item, b.pair_off, b.item_off);
         hipLaunchKernelGGL(scatter_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq, nprobe,
                            p0, p1, s->nlist, b.pair_off, b.cursor, b.sorted_pair);
-        uint64_t max_items = div_up(pairs, p.T) + s->nlist;
+        // At most one partly filled query group per probed list, each cut into at most chunks_max items.
+        uint64_t max_items = (div_up(pairs, p.T) + std::min<uint64_t>(s->nlist, pairs)) * p.chunks_max;
         dim3 grid(static_cast<uint32_t>(div_up(max_items, waves)));
         VA_TRY(launch_ivf(s, p.T, grid, dim3(waves * kWave), lds, st, a, v));
     }
     timing_end(st);
-    hipLaunchKernelGGL(ivf_merge_kernel, dim3(static_cast<uint32_t>(nq)), dim3(kWave), p.S * 8, st, b.partial,
-                       b.partial_cnt, nprobe, kcand, p.S, ids_dev, dists_dev);
-    VA_HIP(hipGetLastError());
-    return 0;
+    return launch_merge_partials(b.partial, b.partial_cnt, b.bound, nprobe * p.chunks_max, kcand, p.S, nq, ids_dev,
+                                 dists_dev, st);
 }
 
 extern "C" int
@@ -646,7 +748,7 @@ vsag_amd_rerank_fp32(const float* raw_dev, uint64_t n, uint32_t dim, int metric,
     while (S < kcand) {
         S <<= 1;
     }
-    hipLaunchKernelGGL(rerank_kernel, dim3(static_cast<uint32_t>(nq)), dim3(kWave), S * 8,
+    hipLaunchKernelGGL(rerank_kernel, dim3(static_cast<uint32_t>(nq)), dim3(kRerankThreads), S * 8,
                        static_cast<hipStream_t>(stream), raw_dev, n, dim, metric, queries_dev, cand_ids_dev, kcand, k,
                        S, ids_dev, dists_dev);
     VA_HIP(hipGetLastError());

@@ -227,7 +227,7 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
 // (ascending).  All threads first keep what the final shared bound admits (at least k keys when k exist) in
 // an LDS pool; wave 0 then selects from the pool -- or straight from the lists when the pool overflowed
 // (long runs of equal distances).
-constexpr uint32_t kPoolKeys = 2048;
+constexpr uint32_t kPoolKeys = 4096;
 
 __global__ void __launch_bounds__(1024)
 merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, const uint32_t* bound, uint32_t nslots,
@@ -238,52 +238,79 @@ merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, cons
     const uint64_t q = blockIdx.x;
     const uint32_t* cnts = partial_cnt + q * nslots;
     const uint64_t* src = partial + q * nslots * k;
-    const uint32_t total = nslots * k;  // list entries, most of them beyond their list's count
-    const uint64_t admit = (static_cast<uint64_t>(as_const(bound)[q]) << 32) | 0xFFFFFFFFULL;
-    if (threadIdx.x == 0) {
-        npool = 0;
-    }
-    __syncthreads();
-    for (uint32_t e = threadIdx.x; e < total; e += blockDim.x) {
-        uint32_t slot = e / k;
-        if (e - slot * k < cnts[slot]) {
-            uint64_t key = src[e];
-            if (key <= admit) {
-                uint32_t pos = atomicAdd(&npool, 1U);
-                if (pos < kPoolKeys) {
-                    pool[pos] = key;
-                }
-            }
-        }
-    }
-    __syncthreads();
-    if (threadIdx.x >= kWave) {
-        return;
-    }
-    const uint32_t lane = threadIdx.x;
-    const bool pooled = npool <= kPoolKeys;
-    const uint32_t count = pooled ? npool : total;
-    selector_init(lds, S, lane);
+    __shared__ uint64_t admit_s;
+    uint64_t admit = (static_cast<uint64_t>(as_const(bound)[q]) << 32) | 0xFFFFFFFFULL;
+    const uint32_t lane = threadIdx.x & (kWave - 1);
     uint32_t cnt = 0;
     uint64_t tau = kInfKey;
-    for (uint32_t base = 0; base < count; base += kWave) {
-        uint32_t e = base + lane;
-        uint64_t key = kInfKey;
-        if (e < count) {
-            if (pooled) {
-                key = pool[e];
-            } else {
-                uint32_t slot = e / k;
-                if (e - slot * k < cnts[slot]) {
-                    key = src[e];
-                }
-            }
-        }
+    auto offer = [&](uint64_t key) {
         bool pass = key < tau;
         cnt = selector_append(lds, k, cnt, pass, key);
         if (cnt + kWave > S - k) {
             tau = selector_flush(lds, S, k, cnt, lane);
             cnt = 0;
+        }
+    };
+    bool pooled = false;
+    for (int round = 0; round < 4 && !pooled; ++round) {
+        if (threadIdx.x == 0) {
+            npool = 0;
+        }
+        __syncthreads();
+        // A thread per list: most lists are empty or nearly so once the bound is known.
+        for (uint32_t slot = threadIdx.x; slot < nslots; slot += blockDim.x) {
+            const uint32_t c = cnts[slot];
+            const uint64_t* list = src + static_cast<uint64_t>(slot) * k;
+            for (uint32_t i = 0; i < c; ++i) {
+                uint64_t key = list[i];
+                if (key <= admit) {
+                    uint32_t pos = atomicAdd(&npool, 1U);
+                    if (pos < kPoolKeys) {
+                        pool[pos] = key;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        pooled = npool <= kPoolKeys;
+        if (!pooled) {
+            // Too many for the pool: the k-th smallest of the keys that did fit bounds the k-th smallest of
+            // all, so it is a valid, much tighter admission key for another round.
+            if (threadIdx.x < kWave) {
+                selector_init(lds, S, lane);
+                cnt = 0;
+                tau = kInfKey;
+                for (uint32_t base = 0; base < kPoolKeys; base += kWave) {
+                    offer(pool[base + lane]);
+                }
+                uint64_t kth = selector_flush(lds, S, k, cnt, lane);
+                if (lane == 0) {
+                    admit_s = kth;
+                }
+            }
+            __syncthreads();
+            admit = admit_s;
+        }
+    }
+    if (threadIdx.x >= kWave) {
+        return;
+    }
+    selector_init(lds, S, lane);
+    cnt = 0;
+    tau = kInfKey;
+    if (pooled) {
+        const uint32_t count = npool;
+        for (uint32_t base = 0; base < count; base += kWave) {
+            offer(base + lane < count ? pool[base + lane] : kInfKey);
+        }
+    } else {
+        // Pool overflow: wave 0 walks the lists themselves, 64 entries at a time.
+        for (uint32_t slot = 0; slot < nslots; ++slot) {
+            const uint32_t c = cnts[slot];
+            const uint64_t* list = src + static_cast<uint64_t>(slot) * k;
+            for (uint32_t base = 0; base < c; base += kWave) {
+                offer(base + lane < c ? list[base + lane] : kInfKey);
+            }
         }
     }
     selector_flush(lds, S, k, cnt, lane);
@@ -300,6 +327,17 @@ merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, cons
 }
 
 // ------------------------------------------------------------------ host side
+int
+launch_merge_partials(const uint64_t* partial, const uint32_t* partial_cnt, const uint32_t* bound, uint32_t nslots,
+                      uint32_t k, uint32_t S, uint64_t nq, uint32_t* ids, float* dists, hipStream_t st) {
+    // Few queries: many candidates each (every wave starts without a bound), so give each merge more threads.
+    const uint32_t threads = nq <= 256 ? 1024 : 256;
+    hipLaunchKernelGGL(merge_partials_kernel, dim3(static_cast<uint32_t>(nq)), dim3(threads), (S + kPoolKeys) * 8, st,
+                       partial, partial_cnt, bound, nslots, k, S, ids, dists);
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
 static int g_tile_override = 0;
 static int g_chunk_override = 0;
 static thread_local int tl_last_tile = 0;
@@ -367,7 +405,13 @@ make_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, uint64_t ntiles, Sca
         want = want < lo ? lo : want > hi ? hi : want;
         chunks = div_up(want, p->groups);
     }
-    uint64_t max_chunks = ntiles / (16 * waves);  // at least 16 tiles per wave
+    // At least 16 tiles per wave -- fewer (down to one) when the store is so small that this would leave
+    // most of the machine without a workgroup (centroid routing, small indexes).
+    uint64_t tiles_min = 16;
+    while (tiles_min > 1 && p->groups * (ntiles / (tiles_min * waves)) < static_cast<uint64_t>(device_cu_count())) {
+        tiles_min >>= 1;
+    }
+    uint64_t max_chunks = ntiles / (tiles_min * waves);
     if (max_chunks < 1) {
         max_chunks = 1;
     }
@@ -561,13 +605,9 @@ vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, 
         VA_TRY(launch_flat(s, p, a, f, st));
         timing_end(st);
     }
-    // Few queries: many candidates each (every wave starts without a bound), so give each merge more threads.
-    const uint32_t merge_threads = nq <= 256 ? 1024 : 256;
     // An empty store has no lists to read.
-    hipLaunchKernelGGL(merge_partials_kernel, dim3(static_cast<uint32_t>(nq)), dim3(merge_threads),
-                       (p.S + kPoolKeys) * 8, st, b.partial, b.partial_cnt, b.bound, s->ntiles != 0 ? f.nslots : 0U, k,
-                       p.S, ids_dev, dists_dev);
-    VA_HIP(hipGetLastError());
+    VA_TRY(launch_merge_partials(b.partial, b.partial_cnt, b.bound, s->ntiles != 0 ? f.nslots : 0U, k, p.S, nq, ids_dev,
+                                 dists_dev, st));
     tl_last_tile = p.T;
     tl_last_passes = p.groups;
     tl_last_bytes = s->ntiles * s->G * kWave * kGranule;

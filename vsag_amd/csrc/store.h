@@ -49,6 +49,7 @@ struct vsag_amd_store {
     uint32_t* list_tile_dev = nullptr;   // nlist+1 tile offsets
     std::vector<uint32_t> list_sizes;    // host copy
     std::vector<uint32_t> list_tile;     // host copy, nlist+1
+    uint32_t max_list_tiles = 0;         // tiles of the longest list
 };
 
 namespace vsag_amd {

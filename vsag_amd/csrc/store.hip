@@ -478,6 +478,10 @@ vsag_amd_store_set_lists(vsag_amd_store_t* s, const uint8_t* codes_dev, const in
     s->nlist = nlist;
     s->list_sizes.assign(sizes.begin(), sizes.begin() + nlist);
     s->list_tile = list_tile;
+    s->max_list_tiles = 0;
+    for (uint32_t b = 0; b < nlist; ++b) {
+        s->max_list_tiles = std::max(s->max_list_tiles, list_tile[b + 1] - list_tile[b]);
+    }
 
     if (n > 0) {
         // 4. stable sort of inner ids by label: the order the reference gets by appending vectors to their
