@@ -77,17 +77,27 @@ count_pairs_kernel(const int32_t* buckets, uint64_t nq, uint32_t nprobe, uint32_
     }
 }
 
+// Chunks a list of `tiles` tiles is cut into: about tiles_per_item tiles each, at most chunks_max chunks
+// (longer lists get longer chunks); 0xFFFFFFFF = never cut.
+__device__ inline uint32_t
+list_chunks(uint32_t tiles, uint32_t tiles_per_item, uint32_t chunks_max) {
+    if (tiles_per_item == 0xFFFFFFFFU) {
+        return tiles != 0 ? 1U : 0U;
+    }
+    uint32_t chunks = (tiles + tiles_per_item - 1) / tiles_per_item;
+    return chunks < chunks_max ? chunks : chunks_max;
+}
+
 // Work items of a list: query groups x tile chunks.
 __device__ inline uint32_t
-list_items(uint32_t pairs, uint32_t T, uint32_t tiles, uint32_t tiles_per_item) {
-    uint32_t chunks = tiles_per_item == 0xFFFFFFFFU ? (tiles != 0 ? 1U : 0U) : (tiles + tiles_per_item - 1) / tiles_per_item;
-    return ((pairs + T - 1) / T) * chunks;
+list_items(uint32_t pairs, uint32_t T, uint32_t tiles, uint32_t tiles_per_item, uint32_t chunks_max) {
+    return ((pairs + T - 1) / T) * list_chunks(tiles, tiles_per_item, chunks_max);
 }
 
 // One workgroup: exclusive prefix sums of the pair counts and of the work items.
 __global__ void __launch_bounds__(1024)
 offsets_kernel(const uint32_t* counts, const uint32_t* list_tile, uint32_t nlist, uint32_t T, uint32_t tiles_per_item,
-               uint32_t* pair_off, uint32_t* item_off) {
+               uint32_t chunks_max, uint32_t* pair_off, uint32_t* item_off) {
     __shared__ uint32_t s_pairs[1024];
     __shared__ uint32_t s_items[1024];
     uint32_t per = (nlist + blockDim.x - 1) / blockDim.x;
@@ -96,7 +106,7 @@ offsets_kernel(const uint32_t* counts, const uint32_t* list_tile, uint32_t nlist
     uint32_t sp = 0, si = 0;
     for (uint32_t i = begin; i < end; ++i) {
         sp += counts[i];
-        si += list_items(counts[i], T, list_tile[i + 1] - list_tile[i], tiles_per_item);
+        si += list_items(counts[i], T, list_tile[i + 1] - list_tile[i], tiles_per_item, chunks_max);
     }
     s_pairs[threadIdx.x] = sp;
     s_items[threadIdx.x] = si;
@@ -119,7 +129,7 @@ offsets_kernel(const uint32_t* counts, const uint32_t* list_tile, uint32_t nlist
         pair_off[i] = rp;
         item_off[i] = ri;
         rp += counts[i];
-        ri += list_items(counts[i], T, list_tile[i + 1] - list_tile[i], tiles_per_item);
+        ri += list_items(counts[i], T, list_tile[i + 1] - list_tile[i], tiles_per_item, chunks_max);
     }
 }
 
@@ -137,6 +147,70 @@ scatter_pairs_kernel(const int32_t* buckets, uint64_t nq, uint32_t nprobe, uint3
     if (b >= 0 && static_cast<uint32_t>(b) < nlist) {
         uint32_t pos = pair_off[b] + atomicAdd(&cursor[b], 1U);
         sorted_pair[pos] = static_cast<uint32_t>(q * nprobe + p);
+    }
+}
+
+// The three regrouping steps above for a small batch (all probe columns) in one workgroup.
+__global__ void __launch_bounds__(1024)
+regroup_small_kernel(const int32_t* buckets, uint64_t nq, uint32_t nprobe, const uint32_t* list_tile, uint32_t nlist,
+                     uint32_t T, uint32_t tiles_per_item, uint32_t chunks_max, uint32_t* counts, uint32_t* cursor,
+                     uint32_t* pair_off, uint32_t* item_off, uint32_t* sorted_pair) {
+    __shared__ uint32_t s_pairs[1024];
+    __shared__ uint32_t s_items[1024];
+    const uint64_t npairs = nq * nprobe;
+    for (uint32_t i = threadIdx.x; i <= nlist; i += blockDim.x) {
+        counts[i] = 0;
+        cursor[i] = 0;
+    }
+    __syncthreads();
+    for (uint64_t i = threadIdx.x; i < npairs; i += blockDim.x) {
+        int32_t b = buckets[i];
+        if (b >= 0 && static_cast<uint32_t>(b) < nlist) {
+            atomicAdd(&counts[b], 1U);
+        }
+    }
+    // The counts were made by atomics in L2; the fences keep the plain loads below from an older cached line.
+    __threadfence();
+    __syncthreads();
+    __threadfence();
+    uint32_t per = (nlist + blockDim.x - 1) / blockDim.x;
+    uint32_t begin = threadIdx.x * per;
+    uint32_t end = begin + per < nlist ? begin + per : nlist;
+    uint32_t sp = 0, si = 0;
+    for (uint32_t i = begin; i < end; ++i) {
+        sp += counts[i];
+        si += list_items(counts[i], T, list_tile[i + 1] - list_tile[i], tiles_per_item, chunks_max);
+    }
+    s_pairs[threadIdx.x] = sp;
+    s_items[threadIdx.x] = si;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t rp = 0, ri = 0;
+        for (uint32_t i = 0; i < blockDim.x; ++i) {
+            uint32_t tp = s_pairs[i], ti = s_items[i];
+            s_pairs[i] = rp;
+            s_items[i] = ri;
+            rp += tp;
+            ri += ti;
+        }
+        pair_off[nlist] = rp;
+        item_off[nlist] = ri;
+    }
+    __syncthreads();
+    uint32_t rp = s_pairs[threadIdx.x], ri = s_items[threadIdx.x];
+    for (uint32_t i = begin; i < end; ++i) {
+        pair_off[i] = rp;
+        item_off[i] = ri;
+        rp += counts[i];
+        ri += list_items(counts[i], T, list_tile[i + 1] - list_tile[i], tiles_per_item, chunks_max);
+    }
+    __syncthreads();
+    for (uint64_t i = threadIdx.x; i < npairs; i += blockDim.x) {
+        int32_t b = buckets[i];
+        if (b >= 0 && static_cast<uint32_t>(b) < nlist) {
+            uint32_t pos = pair_off[b] + atomicAdd(&cursor[b], 1U);
+            sorted_pair[pos] = static_cast<uint32_t>(i);
+        }
     }
 }
 
@@ -190,11 +264,14 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
     uint32_t group = item - ioff[b], chunk = 0;
     uint32_t tbeg = list_begin, tend = list_end;
     if (CHUNKED) {
-        const uint32_t chunks = (list_end - list_begin + v.tiles_per_item - 1) / v.tiles_per_item;
+        const uint32_t tiles = list_end - list_begin;
+        const uint32_t chunks = list_chunks(tiles, v.tiles_per_item, v.chunks_max);
+        const uint32_t per = (tiles + chunks - 1) / chunks;
         chunk = group % chunks;
         group = group / chunks;
-        tbeg = list_begin + chunk * v.tiles_per_item;
-        tend = tbeg + v.tiles_per_item < list_end ? tbeg + v.tiles_per_item : list_end;
+        tbeg = list_begin + chunk * per;
+        tbeg = tbeg < list_end ? tbeg : list_end;
+        tend = tbeg + per < list_end ? tbeg + per : list_end;
     }
     const uint32_t pbeg = as_const(v.pair_off)[b] + group * T;
     const uint32_t pend = as_const(v.pair_off)[b + 1];
@@ -561,19 +638,20 @@ plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, 
     p->npairs = npairs;
     // Enough (list, query group) items to fill the machine: every item walks its whole list, the nearest list
     // of every query goes first.  Otherwise lists are cut into chunks for about 8192 items in all (a probed
-    // list is taken as twice the average length), within 256 MiB of partial lists.
+    // list is taken as twice the average length), at most 64 chunks per list and 256 MiB of partial lists.
     const uint64_t groups = div_up(npairs, static_cast<uint64_t>(t));
     p->chunked = groups < 8192 && s->max_list_tiles > 2;
     p->tiles_per_item = 0xFFFFFFFFU;
     p->chunks_max = 1;
     if (p->chunked) {
         const uint64_t avg_tiles = std::max<uint64_t>(1, s->nlist ? s->ntiles / s->nlist : 1);
-        uint64_t tpi = std::max<uint64_t>(2, div_up(groups * avg_tiles * 2, 8192));
-        while (npairs * div_up(s->max_list_tiles, tpi) * kcand * 8 > (256ull << 20)) {
-            tpi *= 2;
+        const uint64_t tpi = std::max<uint64_t>(2, div_up(groups * avg_tiles * 2, 8192));
+        uint64_t cap = std::min<uint64_t>(64, div_up(s->max_list_tiles, tpi));
+        while (cap > 1 && npairs * cap * kcand * 8 > (256ull << 20)) {
+            cap /= 2;
         }
         p->tiles_per_item = static_cast<uint32_t>(std::min<uint64_t>(tpi, 0x7FFFFFFFU));
-        p->chunks_max = static_cast<uint32_t>(div_up(s->max_list_tiles, tpi));
+        p->chunks_max = static_cast<uint32_t>(cap);
     }
     p->seeded = p->chunked && kcand <= 256;
 }
@@ -679,7 +757,7 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
     };
     fill(FillJob{{b.bound, b.partial_cnt, b.counts, b.cursor, b.seed},
                  {initial_bound(options), 0U, 0U, 0U, 0xFFFFFFFFU},
-                 {nq, nslots_all, nlists1, nlists1, nseed}});
+                 {nq, nslots_all, p.chunked ? 0 : nlists1, p.chunked ? 0 : nlists1, nseed}});
 
     IvfArgs v{};
     v.ids = s->ids_dev;
@@ -718,12 +796,18 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
         if (pass == 1) {
             fill(FillJob{{b.counts, b.cursor, nullptr, nullptr, nullptr}, {0U, 0U, 0U, 0U, 0U}, {nlists1, nlists1, 0, 0, 0}});
         }
-        hipLaunchKernelGGL(count_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq, nprobe, p0,
-                           p1, s->nlist, b.counts);
-        hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, st, b.counts, s->list_tile_dev, s->nlist,
-                           static_cast<uint32_t>(p.T), p.tiles_per_item, b.pair_off, b.item_off);
-        hipLaunchKernelGGL(scatter_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq, nprobe,
-                           p0, p1, s->nlist, b.pair_off, b.cursor, b.sorted_pair);
+        if (p.chunked) {
+            hipLaunchKernelGGL(regroup_small_kernel, dim3(1), dim3(1024), 0, st, buckets_dev, nq, nprobe,
+                               s->list_tile_dev, s->nlist, static_cast<uint32_t>(p.T), p.tiles_per_item, p.chunks_max,
+                               b.counts, b.cursor, b.pair_off, b.item_off, b.sorted_pair);
+        } else {
+            hipLaunchKernelGGL(count_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq, nprobe,
+                               p0, p1, s->nlist, b.counts);
+            hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, st, b.counts, s->list_tile_dev, s->nlist,
+                               static_cast<uint32_t>(p.T), p.tiles_per_item, p.chunks_max, b.pair_off, b.item_off);
+            hipLaunchKernelGGL(scatter_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq,
+                               nprobe, p0, p1, s->nlist, b.pair_off, b.cursor, b.sorted_pair);
+        }
         // At most one partly filled query group per probed list, each cut into at most chunks_max items.
         uint64_t max_items = (div_up(pairs, p.T) + std::min<uint64_t>(s->nlist, pairs)) * p.chunks_max;
         dim3 grid(static_cast<uint32_t>(div_up(max_items, waves)));

@@ -223,38 +223,116 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
     }
 }
 
+// Block-wide selection: the k-th smallest of keys[0, n) (all different), found by an 8-bit radix descent
+// with LDS histograms; kInfKey when n < k.  Every thread of the workgroup calls it and gets the same value.
+struct SelectScratch {
+    uint32_t hist[256];
+    uint32_t bin;
+    uint32_t before;
+};
+
+__device__ inline uint64_t
+block_kth_smallest(const uint64_t* keys, uint32_t n, uint32_t k, SelectScratch& sc) {
+    if (n < k) {
+        return kInfKey;
+    }
+    uint64_t prefix = 0;
+    uint32_t want = k;  // rank of the wanted key among those that share the prefix
+    for (int shift = 56; shift >= 0; shift -= 8) {
+        const uint64_t hi_mask = shift == 56 ? 0ULL : ~0ULL << (shift + 8);
+        for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) {
+            sc.hist[i] = 0;
+        }
+        __syncthreads();
+        for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
+            uint64_t key = keys[i];
+            if (((key ^ prefix) & hi_mask) == 0) {
+                atomicAdd(&sc.hist[(key >> shift) & 255U], 1U);
+            }
+        }
+        __syncthreads();
+        if (threadIdx.x < kWave) {
+            const uint32_t lane = threadIdx.x;
+            uint32_t h0 = sc.hist[4 * lane], h1 = sc.hist[4 * lane + 1], h2 = sc.hist[4 * lane + 2],
+                     h3 = sc.hist[4 * lane + 3];
+            uint32_t incl = h0 + h1 + h2 + h3;
+            for (int off = 1; off < kWave; off <<= 1) {
+                uint32_t o = __shfl_up(incl, off);
+                if (static_cast<int>(lane) >= off) {
+                    incl += o;
+                }
+            }
+            uint32_t before = incl - (h0 + h1 + h2 + h3);
+            if (before < want && want <= incl) {
+                uint32_t b = 0;
+                if (before + h0 < want) {
+                    before += h0;
+                    b = 1;
+                    if (before + h1 < want) {
+                        before += h1;
+                        b = 2;
+                        if (before + h2 < want) {
+                            before += h2;
+                            b = 3;
+                        }
+                    }
+                }
+                sc.bin = 4 * lane + b;
+                sc.before = before;
+            }
+        }
+        __syncthreads();
+        prefix |= static_cast<uint64_t>(sc.bin) << shift;
+        want -= sc.before;
+        __syncthreads();
+    }
+    return prefix;
+}
+
+// Ascending bitonic sort of keys[0, P) (P a power of two) by the whole workgroup.
+__device__ inline void
+block_bitonic_sort(uint64_t* keys, uint32_t P) {
+    for (uint32_t size = 2; size <= P; size <<= 1) {
+        for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+            for (uint32_t i = threadIdx.x; i < (P >> 1); i += blockDim.x) {
+                uint32_t pos = 2 * i - (i & (stride - 1));
+                uint64_t a = keys[pos];
+                uint64_t b = keys[pos + stride];
+                bool up = (pos & size) == 0;
+                if ((a > b) == up) {
+                    keys[pos] = b;
+                    keys[pos + stride] = a;
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
 // One workgroup per query: the k best keys over its counted partial lists, written as ids / distances
 // (ascending).  All threads first keep what the final shared bound admits (at least k keys when k exist) in
-// an LDS pool; wave 0 then selects from the pool -- or straight from the lists when the pool overflowed
-// (long runs of equal distances).
+// an LDS pool; a radix selection finds the k-th smallest of the pool, the keys up to it are compacted and
+// sorted.  When the pool overflows (long runs of nearly equal distances), the k-th smallest of what did fit
+// -- an upper bound of the k-th smallest of all -- becomes the admission key of another round.
 constexpr uint32_t kPoolKeys = 4096;
 
 __global__ void __launch_bounds__(1024)
 merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, const uint32_t* bound, uint32_t nslots,
                       uint32_t k, uint32_t S, uint32_t* ids, float* dists) {
-    extern __shared__ uint64_t lds[];  // S selector keys, then the pool
+    extern __shared__ uint64_t lds[];  // S output keys, then the pool
     __shared__ uint32_t npool;
+    __shared__ uint32_t nout;
+    __shared__ SelectScratch scratch;
     uint64_t* pool = lds + S;
     const uint64_t q = blockIdx.x;
     const uint32_t* cnts = partial_cnt + q * nslots;
     const uint64_t* src = partial + q * nslots * k;
-    __shared__ uint64_t admit_s;
     uint64_t admit = (static_cast<uint64_t>(as_const(bound)[q]) << 32) | 0xFFFFFFFFULL;
-    const uint32_t lane = threadIdx.x & (kWave - 1);
-    uint32_t cnt = 0;
-    uint64_t tau = kInfKey;
-    auto offer = [&](uint64_t key) {
-        bool pass = key < tau;
-        cnt = selector_append(lds, k, cnt, pass, key);
-        if (cnt + kWave > S - k) {
-            tau = selector_flush(lds, S, k, cnt, lane);
-            cnt = 0;
-        }
-    };
-    bool pooled = false;
-    for (int round = 0; round < 4 && !pooled; ++round) {
+    // Finitely many rounds: every round that overflows lowers `admit` below at least one pooled key.
+    for (;;) {
         if (threadIdx.x == 0) {
             npool = 0;
+            nout = 0;
         }
         __syncthreads();
         // A thread per list: most lists are empty or nearly so once the bound is known.
@@ -272,49 +350,33 @@ merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, cons
             }
         }
         __syncthreads();
-        pooled = npool <= kPoolKeys;
-        if (!pooled) {
-            // Too many for the pool: the k-th smallest of the keys that did fit bounds the k-th smallest of
-            // all, so it is a valid, much tighter admission key for another round.
-            if (threadIdx.x < kWave) {
-                selector_init(lds, S, lane);
-                cnt = 0;
-                tau = kInfKey;
-                for (uint32_t base = 0; base < kPoolKeys; base += kWave) {
-                    offer(pool[base + lane]);
-                }
-                uint64_t kth = selector_flush(lds, S, k, cnt, lane);
-                if (lane == 0) {
-                    admit_s = kth;
+        const uint32_t total = npool;
+        const uint32_t n = total < kPoolKeys ? total : kPoolKeys;
+        const uint64_t kth = block_kth_smallest(pool, n, k, scratch);
+        if (total <= kPoolKeys) {
+            // The k smallest (all of them when fewer than k) go to the front of the output area.
+            for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
+                uint64_t key = pool[i];
+                if (key <= kth) {
+                    lds[atomicAdd(&nout, 1U)] = key;
                 }
             }
-            __syncthreads();
-            admit = admit_s;
+            break;
         }
+        admit = kth;
+        __syncthreads();
     }
-    if (threadIdx.x >= kWave) {
-        return;
+    __syncthreads();
+    uint32_t P = 2;
+    while (P < k) {
+        P <<= 1;
     }
-    selector_init(lds, S, lane);
-    cnt = 0;
-    tau = kInfKey;
-    if (pooled) {
-        const uint32_t count = npool;
-        for (uint32_t base = 0; base < count; base += kWave) {
-            offer(base + lane < count ? pool[base + lane] : kInfKey);
-        }
-    } else {
-        // Pool overflow: wave 0 walks the lists themselves, 64 entries at a time.
-        for (uint32_t slot = 0; slot < nslots; ++slot) {
-            const uint32_t c = cnts[slot];
-            const uint64_t* list = src + static_cast<uint64_t>(slot) * k;
-            for (uint32_t base = 0; base < c; base += kWave) {
-                offer(base + lane < c ? list[base + lane] : kInfKey);
-            }
-        }
+    for (uint32_t i = nout + threadIdx.x; i < P; i += blockDim.x) {
+        lds[i] = kInfKey;
     }
-    selector_flush(lds, S, k, cnt, lane);
-    for (uint32_t i = lane; i < k; i += kWave) {
+    __syncthreads();
+    block_bitonic_sort(lds, P);
+    for (uint32_t i = threadIdx.x; i < k; i += blockDim.x) {
         uint64_t key = lds[i];
         if (key == kInfKey) {
             ids[q * k + i] = VSAG_AMD_INVALID_ID;
