@@ -94,12 +94,45 @@ list_items(uint32_t pairs, uint32_t T, uint32_t tiles, uint32_t tiles_per_item, 
     return ((pairs + T - 1) / T) * list_chunks(tiles, tiles_per_item, chunks_max);
 }
 
+// Exclusive prefix sums of two per-thread values over a workgroup of up to 1024 threads; wave totals go
+// through `wave_sums` (2 x 16 words of LDS).  Returns the grand totals.
+__device__ inline void
+block_exclusive_scan2(uint32_t& a, uint32_t& b, uint32_t (*wave_sums)[16], uint32_t& total_a, uint32_t& total_b) {
+    const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6, nwaves = (blockDim.x + kWave - 1) >> 6;
+    uint32_t ia = a, ib = b;
+    for (int off = 1; off < kWave; off <<= 1) {
+        uint32_t oa = __shfl_up(ia, off), ob = __shfl_up(ib, off);
+        if (static_cast<int>(lane) >= off) {
+            ia += oa;
+            ib += ob;
+        }
+    }
+    if (lane == kWave - 1) {
+        wave_sums[0][wave] = ia;
+        wave_sums[1][wave] = ib;
+    }
+    __syncthreads();
+    uint32_t ba = 0, bb = 0;
+    total_a = 0;
+    total_b = 0;
+    for (uint32_t w = 0; w < nwaves; ++w) {
+        uint32_t sa = wave_sums[0][w], sb = wave_sums[1][w];
+        if (w < wave) {
+            ba += sa;
+            bb += sb;
+        }
+        total_a += sa;
+        total_b += sb;
+    }
+    a = ba + ia - a;
+    b = bb + ib - b;
+}
+
 // One workgroup: exclusive prefix sums of the pair counts and of the work items.
 __global__ void __launch_bounds__(1024)
 offsets_kernel(const uint32_t* counts, const uint32_t* list_tile, uint32_t nlist, uint32_t T, uint32_t tiles_per_item,
                uint32_t chunks_max, uint32_t* pair_off, uint32_t* item_off) {
-    __shared__ uint32_t s_pairs[1024];
-    __shared__ uint32_t s_items[1024];
+    __shared__ uint32_t wave_sums[2][16];
     uint32_t per = (nlist + blockDim.x - 1) / blockDim.x;
     uint32_t begin = threadIdx.x * per;
     uint32_t end = begin + per < nlist ? begin + per : nlist;
@@ -108,23 +141,12 @@ offsets_kernel(const uint32_t* counts, const uint32_t* list_tile, uint32_t nlist
         sp += counts[i];
         si += list_items(counts[i], T, list_tile[i + 1] - list_tile[i], tiles_per_item, chunks_max);
     }
-    s_pairs[threadIdx.x] = sp;
-    s_items[threadIdx.x] = si;
-    __syncthreads();
+    uint32_t rp = sp, ri = si, all_pairs, all_items;
+    block_exclusive_scan2(rp, ri, wave_sums, all_pairs, all_items);
     if (threadIdx.x == 0) {
-        uint32_t rp = 0, ri = 0;
-        for (uint32_t i = 0; i < blockDim.x; ++i) {
-            uint32_t tp = s_pairs[i], ti = s_items[i];
-            s_pairs[i] = rp;
-            s_items[i] = ri;
-            rp += tp;
-            ri += ti;
-        }
-        pair_off[nlist] = rp;
-        item_off[nlist] = ri;
+        pair_off[nlist] = all_pairs;
+        item_off[nlist] = all_items;
     }
-    __syncthreads();
-    uint32_t rp = s_pairs[threadIdx.x], ri = s_items[threadIdx.x];
     for (uint32_t i = begin; i < end; ++i) {
         pair_off[i] = rp;
         item_off[i] = ri;
@@ -155,8 +177,7 @@ __global__ void __launch_bounds__(1024)
 regroup_small_kernel(const int32_t* buckets, uint64_t nq, uint32_t nprobe, const uint32_t* list_tile, uint32_t nlist,
                      uint32_t T, uint32_t tiles_per_item, uint32_t chunks_max, uint32_t* counts, uint32_t* cursor,
                      uint32_t* pair_off, uint32_t* item_off, uint32_t* sorted_pair) {
-    __shared__ uint32_t s_pairs[1024];
-    __shared__ uint32_t s_items[1024];
+    __shared__ uint32_t wave_sums[2][16];
     const uint64_t npairs = nq * nprobe;
     for (uint32_t i = threadIdx.x; i <= nlist; i += blockDim.x) {
         counts[i] = 0;
@@ -181,23 +202,12 @@ regroup_small_kernel(const int32_t* buckets, uint64_t nq, uint32_t nprobe, const
         sp += counts[i];
         si += list_items(counts[i], T, list_tile[i + 1] - list_tile[i], tiles_per_item, chunks_max);
     }
-    s_pairs[threadIdx.x] = sp;
-    s_items[threadIdx.x] = si;
-    __syncthreads();
+    uint32_t rp = sp, ri = si, all_pairs, all_items;
+    block_exclusive_scan2(rp, ri, wave_sums, all_pairs, all_items);
     if (threadIdx.x == 0) {
-        uint32_t rp = 0, ri = 0;
-        for (uint32_t i = 0; i < blockDim.x; ++i) {
-            uint32_t tp = s_pairs[i], ti = s_items[i];
-            s_pairs[i] = rp;
-            s_items[i] = ri;
-            rp += tp;
-            ri += ti;
-        }
-        pair_off[nlist] = rp;
-        item_off[nlist] = ri;
+        pair_off[nlist] = all_pairs;
+        item_off[nlist] = all_items;
     }
-    __syncthreads();
-    uint32_t rp = s_pairs[threadIdx.x], ri = s_items[threadIdx.x];
     for (uint32_t i = begin; i < end; ++i) {
         pair_off[i] = rp;
         item_off[i] = ri;
@@ -637,7 +647,7 @@ plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, 
     }
     p->npairs = npairs;
     // Enough (list, query group) items to fill the machine: every item walks its whole list, the nearest list
-    // of every query goes first.  Otherwise lists are cut into chunks for about 8192 items in all (a probed
+    // of every query goes first.  Otherwise lists are cut into chunks of at least four tiles for about 4096 items in all (a probed
     // list is taken as twice the average length), at most 64 chunks per list and 256 MiB of partial lists.
     const uint64_t groups = div_up(npairs, static_cast<uint64_t>(t));
     p->chunked = groups < 8192 && s->max_list_tiles > 2;
@@ -645,7 +655,7 @@ plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, 
     p->chunks_max = 1;
     if (p->chunked) {
         const uint64_t avg_tiles = std::max<uint64_t>(1, s->nlist ? s->ntiles / s->nlist : 1);
-        const uint64_t tpi = std::max<uint64_t>(2, div_up(groups * avg_tiles * 2, 8192));
+        const uint64_t tpi = std::max<uint64_t>(4, div_up(groups * avg_tiles * 2, 4096));
         uint64_t cap = std::min<uint64_t>(64, div_up(s->max_list_tiles, tpi));
         while (cap > 1 && npairs * cap * kcand * 8 > (256ull << 20)) {
             cap /= 2;

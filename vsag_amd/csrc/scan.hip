@@ -225,10 +225,15 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
 
 // Block-wide selection: the k-th smallest of keys[0, n) (all different), found by an 8-bit radix descent
 // with LDS histograms; kInfKey when n < k.  Every thread of the workgroup calls it and gets the same value.
+// Bytes that all keys share are skipped (the leading bytes of distances from one neighbourhood are equal, and
+// a histogram with one occupied bin is 4096 atomics on one address); the descent stops as soon as the wanted
+// key is alone in its bin.
 struct SelectScratch {
     uint32_t hist[256];
     uint32_t bin;
     uint32_t before;
+    uint32_t count;
+    unsigned long long lo, hi, found;
 };
 
 __device__ inline uint64_t
@@ -236,9 +241,37 @@ block_kth_smallest(const uint64_t* keys, uint32_t n, uint32_t k, SelectScratch& 
     if (n < k) {
         return kInfKey;
     }
+    if (threadIdx.x == 0) {
+        sc.lo = ~0ULL;
+        sc.hi = 0ULL;
+    }
+    __syncthreads();
+    {
+        unsigned long long lo = ~0ULL, hi = 0ULL;
+        for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
+            unsigned long long key = keys[i];
+            lo = key < lo ? key : lo;
+            hi = key > hi ? key : hi;
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            unsigned long long ol = __shfl_xor(lo, off), oh = __shfl_xor(hi, off);
+            lo = ol < lo ? ol : lo;
+            hi = oh > hi ? oh : hi;
+        }
+        if ((threadIdx.x & (kWave - 1)) == 0) {
+            atomicMin(&sc.lo, lo);
+            atomicMax(&sc.hi, hi);
+        }
+    }
+    __syncthreads();
+    const uint64_t spread = sc.lo ^ sc.hi;
     uint64_t prefix = 0;
     uint32_t want = k;  // rank of the wanted key among those that share the prefix
     for (int shift = 56; shift >= 0; shift -= 8) {
+        if ((spread >> shift) == 0) {
+            prefix |= sc.lo & (0xFFULL << shift);  // every key has this byte
+            continue;
+        }
         const uint64_t hi_mask = shift == 56 ? 0ULL : ~0ULL << (shift + 8);
         for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) {
             sc.hist[i] = 0;
@@ -253,38 +286,44 @@ block_kth_smallest(const uint64_t* keys, uint32_t n, uint32_t k, SelectScratch& 
         __syncthreads();
         if (threadIdx.x < kWave) {
             const uint32_t lane = threadIdx.x;
-            uint32_t h0 = sc.hist[4 * lane], h1 = sc.hist[4 * lane + 1], h2 = sc.hist[4 * lane + 2],
-                     h3 = sc.hist[4 * lane + 3];
-            uint32_t incl = h0 + h1 + h2 + h3;
+            uint32_t h[4] = {sc.hist[4 * lane], sc.hist[4 * lane + 1], sc.hist[4 * lane + 2], sc.hist[4 * lane + 3]};
+            uint32_t sum = h[0] + h[1] + h[2] + h[3];
+            uint32_t incl = sum;
             for (int off = 1; off < kWave; off <<= 1) {
                 uint32_t o = __shfl_up(incl, off);
                 if (static_cast<int>(lane) >= off) {
                     incl += o;
                 }
             }
-            uint32_t before = incl - (h0 + h1 + h2 + h3);
+            uint32_t before = incl - sum;
             if (before < want && want <= incl) {
                 uint32_t b = 0;
-                if (before + h0 < want) {
-                    before += h0;
-                    b = 1;
-                    if (before + h1 < want) {
-                        before += h1;
-                        b = 2;
-                        if (before + h2 < want) {
-                            before += h2;
-                            b = 3;
-                        }
-                    }
+                while (before + h[b] < want) {
+                    before += h[b];
+                    ++b;
                 }
                 sc.bin = 4 * lane + b;
                 sc.before = before;
+                sc.count = h[b];
             }
         }
         __syncthreads();
         prefix |= static_cast<uint64_t>(sc.bin) << shift;
         want -= sc.before;
+        const bool alone = sc.count == 1;
         __syncthreads();
+        if (alone) {
+            // One key left under this prefix: it is the answer.
+            const uint64_t known = ~0ULL << shift;
+            for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
+                uint64_t key = keys[i];
+                if (((key ^ prefix) & known) == 0) {
+                    sc.found = key;
+                }
+            }
+            __syncthreads();
+            return sc.found;
+        }
     }
     return prefix;
 }
