@@ -448,6 +448,22 @@ def run_c4(env):
                                               ws.ptr, wsc, None))
         capi.check(lib.vsag_amd_rerank_fp32(x_dev.ptr, n, d, capi.METRIC_L2, q_dev.ptr, nq, cand.ptr, kcand, k,
                                             out_i.ptr, out_d.ptr, None))
+    # one query per call (the reference's own call pattern): route + scan of 64 lists + rerank, synchronised per query
+    single = None
+    if not args.no_single:
+        t_one = []
+        for i in range(5 + 50):
+            qp = q_dev.ptr + (i % nq) * d * 4
+            t0 = time.perf_counter()
+            capi.check(lib.vsag_amd_ivf_route(cstore, qp, 1, nprobe, buckets.ptr, bd.ptr, ws.ptr, wr, None))
+            capi.check(lib.vsag_amd_ivf_scan_topk(lists, qp, 1, buckets.ptr, nprobe, kcand, cand.ptr, cand_d.ptr, ws.ptr,
+                                                  wsc, None))
+            capi.check(lib.vsag_amd_rerank_fp32(x_dev.ptr, n, d, capi.METRIC_L2, qp, 1, cand.ptr, kcand, k, out_i.ptr,
+                                                out_d.ptr, None))
+            capi.synchronize()
+            if i >= 5:
+                t_one.append(time.perf_counter() - t0)
+        single = {"latency_us": 1e6 * float(np.mean(t_one)), "queries_per_second_one_at_a_time": 1.0 / float(np.mean(t_one))}
     sec, kms = env.timed(step, args.steps, args.warmup)
     ids = out_i.to_numpy(np.uint32, (nq, k))
     b = buckets.to_numpy(np.int32, (nq, nprobe))
@@ -525,7 +541,7 @@ def run_c4(env):
                          "u4 codes, i32 dot", "configs[3]: IVF search, N=%d, d=%d, nlist=%d, nprobe=%d, rerank %d, "
                          "%d queries, k=%d" % (n, d, nlist, nprobe, kcand, nq, k),
                          {"recall_at_10": rec, "build_seconds": t_build, "scanned_codes_per_query": float(scanned) / nq,
-                          "bytes_per_scanned_code": cs + 4}, roof, cpu)
+                          "bytes_per_scanned_code": cs + 4, "single_query": single}, roof, cpu)
 
 
 # ------------------------------------------------------------------------------------------- C5

@@ -191,14 +191,16 @@ def test_ivf_routing_only_and_errors(lib):
     small.close()
 
 
-def test_ivf_rabitq_with_reorder(lib):
+@pytest.mark.parametrize("query_bits", [4, 32, None])  # None: the reference's default, fp32 queries
+def test_ivf_rabitq_with_reorder(lib, query_bits):
     # tests/test_ivf.cpp:1212-1230: rabitq base codes, fp32 reorder
     n, d, nq, k = 3000, 128, 50, 10
     x = vectors(n, d)
     q = vectors(nq, d, seed=165)
     labels = np.arange(n, dtype=np.int64)
-    idx = make("ivf", d, "l2", buckets_count=10, base_quantization_type="rabitq", rabitq_bits_per_dim_query=4,
-               use_reorder=True, precise_quantization_type="fp32", train_sample_count=3000)
+    extra = {} if query_bits is None else {"rabitq_bits_per_dim_query": query_bits}
+    idx = make("ivf", d, "l2", buckets_count=10, base_quantization_type="rabitq",
+               use_reorder=True, precise_quantization_type="fp32", train_sample_count=3000, **extra)
     idx.build(x, labels, n, d)
     gt, _ = ground_truth(x, q, k, "l2")
     ids, _ = idx.knn_search_batch(q, k, json.dumps({"ivf": {"scan_buckets_count": 10, "factor": 20.0}}))

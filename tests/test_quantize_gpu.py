@@ -164,3 +164,25 @@ def test_rabitq_flat_scan(lib, metric, mname, n, d, nq, k):
     # Integer inner products are exact and the float estimator keeps the checker's operation order.
     assert_topk_close(ids, ds, rids, rds, rtol=1e-5, atol=1e-6, label="rabitq " + mname)
     st.destroy()
+
+
+@pytest.mark.parametrize("metric,mname", [(orc.L2, "l2"), (orc.IP, "ip"), (orc.COSINE, "cosine")])
+@pytest.mark.parametrize("n,d,nq,k", [(6000, 128, 11, 10), (900, 768, 5, 100), (300, 15, 3, 7), (2000, 200, 1, 10)])
+def test_rabitq_flat_scan_fp32_queries(lib, metric, mname, n, d, nq, k):
+    """rabitq_bits_per_dim_query = 32: the query stays fp32 (RaBitQFloatBinaryIP, src/simd/generic.cpp:447-471)."""
+    from gpu_helpers import Store, assert_topk_close
+    rng = np.random.default_rng(n + d + 32)
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    q = rng.standard_normal((nq, d)).astype(np.float32)
+    rot = _rotation(rng, d)
+    cen = orc.rabitq_train(x, rot)
+    codes = orc.rabitq_encode(x, rot, cen, metric, 32)
+    qcodes = orc.rabitq_process_query(q, rot, cen, metric, 32)
+    st = Store(capi.KIND_RABITQ, metric, d, rot=rot, centroid=cen, qbits=32)
+    assert st.code_size() == codes.shape[1]
+    st.append(codes)
+    ids, ds = st.flat_scan(q, k)
+    rids, rds = orc.flat_scan_topk(orc.RABITQ, metric, d, codes, qcodes, k, qbits=32)
+    # the sum over set bits is taken in another order than the checker's running sum
+    assert_topk_close(ids, ds, rids, rds, rtol=1e-4, atol=2e-5, tie_rtol=2e-4, label="rabitq fp32 query " + mname)
+    st.destroy()

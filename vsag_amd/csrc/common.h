@@ -14,6 +14,9 @@ namespace vsag_amd {
 
 constexpr int kWave = 64;          // gfx950 wavefront width; one code tile holds 64 codes
 constexpr int kGranule = 16;       // bytes per lane per tile row (one dwordx4)
+// Scan-kernel variant of VSAG_AMD_KIND_RABITQ for stores whose queries stay fp32 (rabitq_bits_per_dim_query = 32);
+// only the kernel templates and their dispatch know it.
+constexpr int kKindRabitqF32 = VSAG_AMD_KIND_RABITQ + 1;
 constexpr int kMaxGroup = 8;       // most granule rows the scans fetch together
 // Readable bytes past the last tile of every tile buffer: the last group of a tile is fetched whole.
 constexpr size_t kTileSlackBytes = static_cast<size_t>(kMaxGroup - 1) * kWave * kGranule;

@@ -172,6 +172,21 @@ accumulate_granule(const ScanArgs& a, const QueryRows<T>& q, uint32_t j, uint4 c
                 acc.lo[t] = __builtin_amdgcn_udot4(w[m], q.row[t][4 * j + m], acc.lo[t], false);
             }
         }
+    } else if constexpr (KIND == kKindRabitqF32) {
+        // qtab row: the rotated, centred, normalised query as fp32; a granule holds the bits of 128 dimensions.
+        // Sum of the query values under set bits: a sign-extended one-bit extract is an all-ones / all-zeros
+        // mask for the value.
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+#pragma unroll
+            for (int e = 0; e < 32; ++e) {
+                uint32_t mask = static_cast<uint32_t>(__builtin_amdgcn_sbfe(static_cast<int32_t>(w[m]), e, 1));
+#pragma unroll
+                for (int t = 0; t < T; ++t) {
+                    acc.f[t] += __uint_as_float(mask & q.row[t][128 * j + 32 * m + e]);
+                }
+            }
+        }
     } else if constexpr (KIND == VSAG_AMD_KIND_RABITQ) {
         // qtab row: per code dword the four query bit planes.
 #pragma unroll
@@ -223,11 +238,13 @@ finish_distances(const ScanArgs& a, const uint32_t (&qidx)[T], uint64_t slot, co
                 out[t] = 1 - r;
             }
         }
-    } else if constexpr (KIND == VSAG_AMD_KIND_RABITQ) {
-        // qmeta: {2 delta/sqrt(d), 2 lb/sqrt(d), delta sum_q/sqrt(d), lb d/sqrt(d), ||Rq - c||, ||q||}.
+    } else if constexpr (KIND == VSAG_AMD_KIND_RABITQ || KIND == kKindRabitqF32) {
+        // qmeta, 4-bit queries: {2 delta/sqrt(d), 2 lb/sqrt(d), delta sum_q/sqrt(d), lb d/sqrt(d), ||Rq - c||, ||q||};
+        // fp32 queries: {2/sqrt(d), -, sum_q/sqrt(d), -, ||Rq - c||, ||q||} (RaBitQFloatBinaryIP, generic.cpp:447-471:
+        // +q/sqrt(d) under a set bit, -q/sqrt(d) under a clear one).
         float base_norm = __uint_as_float(a.meta[slot]);
         float base_error = __uint_as_float(a.meta[a.meta_stride + slot]);
-        float base_sum = __uint_as_float(a.meta[2 * a.meta_stride + slot]);
+        float base_sum = KIND == VSAG_AMD_KIND_RABITQ ? __uint_as_float(a.meta[2 * a.meta_stride + slot]) : 0.0F;
         float base_raw = METRIC == VSAG_AMD_METRIC_L2 ? 0.0F : __uint_as_float(a.meta[3 * a.meta_stride + slot]);
         if (static_cast<double>(fabsf(base_error)) < 1e-5) {
             base_error = (base_error >= 0) ? 1.0F : -1.0F;
@@ -235,10 +252,15 @@ finish_distances(const ScanArgs& a, const uint32_t (&qidx)[T], uint64_t slot, co
 #pragma unroll
         for (int t = 0; t < T; ++t) {
             const float* qm = a.qmeta + static_cast<size_t>(qidx[t]) * a.qmeta_stride;
-            uint32_t ip = acc.lo[t] + (acc.hi[t] << 1) + (acc.p2[t] << 2) + (acc.p3[t] << 3);
-            float p1 = qm[0] * static_cast<float>(ip);
-            float p2 = qm[1] * base_sum;
-            float ip_bq = p1 + p2 - qm[2] - qm[3];
+            float ip_bq;
+            if constexpr (KIND == VSAG_AMD_KIND_RABITQ) {
+                uint32_t ip = acc.lo[t] + (acc.hi[t] << 1) + (acc.p2[t] << 2) + (acc.p3[t] << 3);
+                float p1 = qm[0] * static_cast<float>(ip);
+                float p2 = qm[1] * base_sum;
+                ip_bq = p1 + p2 - qm[2] - qm[3];
+            } else {
+                ip_bq = qm[0] * acc.f[t] - qm[2];
+            }
             float ip_est = ip_bq / base_error;
             float qn = qm[4];
             float e1 = base_norm * base_norm;

@@ -570,7 +570,7 @@ launch_ivf_m(int metric, int T, dim3 grid, dim3 block, size_t lds, hipStream_t s
              const IvfArgs& v) {
     if (metric == VSAG_AMD_METRIC_L2) {
         launch_ivf_t<KIND, VSAG_AMD_METRIC_L2>(T, grid, block, lds, st, a, v);
-    } else if (metric == VSAG_AMD_METRIC_COSINE && KIND == VSAG_AMD_KIND_RABITQ) {
+    } else if (metric == VSAG_AMD_METRIC_COSINE && (KIND == VSAG_AMD_KIND_RABITQ || KIND == kKindRabitqF32)) {
         launch_ivf_t<KIND, VSAG_AMD_METRIC_COSINE>(T, grid, block, lds, st, a, v);
     } else {
         launch_ivf_t<KIND, VSAG_AMD_METRIC_IP>(T, grid, block, lds, st, a, v);
@@ -597,7 +597,11 @@ launch_ivf(const vsag_amd_store* s, int T, dim3 grid, dim3 block, size_t lds, hi
             launch_ivf_m<VSAG_AMD_KIND_SQ8_UNIFORM>(s->metric, T, grid, block, lds, st, a, v);
             break;
         case VSAG_AMD_KIND_RABITQ:
-            launch_ivf_m<VSAG_AMD_KIND_RABITQ>(s->metric, T, grid, block, lds, st, a, v);
+            if (s->query_bits == 32) {
+                launch_ivf_m<kKindRabitqF32>(s->metric, T, grid, block, lds, st, a, v);
+            } else {
+                launch_ivf_m<VSAG_AMD_KIND_RABITQ>(s->metric, T, grid, block, lds, st, a, v);
+            }
             break;
         default:
             return fail(VSAG_AMD_INVALID_ARGUMENT, "unknown store kind %d", s->kind);

@@ -220,13 +220,63 @@ query_layout(const vsag_amd_store* s) {
             l.qmeta = 1;
             break;
         case VSAG_AMD_KIND_RABITQ:
-            l.qstride = ndw * 4;
+            l.qstride = s->query_bits == 32 ? s->dpad : ndw * 4;
             l.qmeta = 8;
             break;
     }
     // Rows start on a 64-byte boundary so that scalar dwordx16 loads stay aligned.
     l.qstride = static_cast<uint32_t>(round_up(l.qstride, 16));
     return l;
+}
+
+// Processed fp32 queries of a RaBitQ store (the normalised rotated residual, its norm, the raw norm:
+// rabitq_quantizer.cpp:2049-2088) -> table row padded with zeros + the factors of the estimator.
+__global__ void __launch_bounds__(256)
+prepare_rabitq_f32_queries(const uint8_t* qcodes, uint64_t nq, uint32_t qcode_size, uint32_t dim, int has_raw_norm,
+                           uint32_t* qtab, uint32_t qstride, float* qmeta, uint32_t qmeta_stride) {
+    __shared__ float partial[256];
+    uint64_t row = blockIdx.x;
+    uint32_t* out = qtab + row * qstride;
+    if (row >= nq) {
+        for (uint32_t d = threadIdx.x; d < qstride; d += blockDim.x) {
+            out[d] = 0;
+        }
+        if (threadIdx.x < qmeta_stride) {
+            qmeta[row * qmeta_stride + threadIdx.x] = 0.0F;
+        }
+        return;
+    }
+    const uint8_t* c = qcodes + row * qcode_size;
+    auto rd = [&](uint32_t off) {
+        uint32_t u = 0;
+        for (int b = 0; b < 4; ++b) {
+            u |= static_cast<uint32_t>(c[off + b]) << (8 * b);
+        }
+        return u;
+    };
+    float s = 0.0F;
+    for (uint32_t d = threadIdx.x; d < qstride; d += blockDim.x) {
+        uint32_t u = d < dim ? rd(4 * d) : 0U;
+        out[d] = u;
+        s += __uint_as_float(u);
+    }
+    partial[threadIdx.x] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float total = 0.0F;
+        for (uint32_t i = 0; i < blockDim.x; ++i) {
+            total += partial[i];
+        }
+        uint32_t tail = (4 * dim + 3) / 4 * 4;
+        float inv_sqrt_d = 1.0F / sqrtf(static_cast<float>(dim));
+        float* m = qmeta + row * qmeta_stride;
+        m[0] = 2.0F * inv_sqrt_d;
+        m[1] = 0.0F;
+        m[2] = inv_sqrt_d * total;
+        m[3] = 0.0F;
+        m[4] = __uint_as_float(rd(tail));
+        m[5] = has_raw_norm ? __uint_as_float(rd(tail + 4)) : 0.0F;
+    }
 }
 
 // Runs ProcessQueryImpl of the store's quantizer for nq raw queries and fills the scan tables.
@@ -251,9 +301,15 @@ prepare_queries(const vsag_amd_store* s, const float* queries, uint64_t nq, uint
             break;
         }
         case VSAG_AMD_KIND_RABITQ: {
-            VA_CHECK_ARG(s->query_bits == 4, "rabitq scan supports 4-bit queries only");
+            VA_CHECK_ARG(s->query_bits == 4 || s->query_bits == 32, "rabitq scan supports 4-bit and fp32 queries");
             VA_TRY(rabitq_process_query_launch(queries, nq, s->dim, s->rotation_dev, s->centroid_dev, s->metric,
                                                s->query_bits, qcodes, st));
+            if (s->query_bits == 32) {
+                hipLaunchKernelGGL(prepare_rabitq_f32_queries, grid, dim3(256), 0, st, qcodes, nq,
+                                   static_cast<uint32_t>(rabitq_query_code_size(s->dim, s->metric, 32)), s->dim,
+                                   s->metric != VSAG_AMD_METRIC_L2 ? 1 : 0, qtab, ql.qstride, qmeta, ql.qmeta);
+                break;
+            }
             uint32_t aligned_dim = (s->dim + 511) / 512 * 512;
             hipLaunchKernelGGL(prepare_rabitq_queries, grid, dim3(256), 0, st, qcodes, nq,
                                static_cast<uint32_t>(rabitq_query_code_size(s->dim, s->metric, s->query_bits)),

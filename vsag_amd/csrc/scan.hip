@@ -596,7 +596,7 @@ launch_flat_m(int metric, int T, dim3 grid, dim3 block, size_t lds, hipStream_t 
     // Cosine stores hold normalised vectors and scan as inner product (RaBitQ has its own formula).
     if (metric == VSAG_AMD_METRIC_L2) {
         launch_flat_t<KIND, VSAG_AMD_METRIC_L2>(T, grid, block, lds, st, a, f);
-    } else if (metric == VSAG_AMD_METRIC_COSINE && KIND == VSAG_AMD_KIND_RABITQ) {
+    } else if (metric == VSAG_AMD_METRIC_COSINE && (KIND == VSAG_AMD_KIND_RABITQ || KIND == kKindRabitqF32)) {
         launch_flat_t<KIND, VSAG_AMD_METRIC_COSINE>(T, grid, block, lds, st, a, f);
     } else {
         launch_flat_t<KIND, VSAG_AMD_METRIC_IP>(T, grid, block, lds, st, a, f);
@@ -625,7 +625,11 @@ launch_flat(const vsag_amd_store* s, const ScanPlan& p, const ScanArgs& a, const
             launch_flat_m<VSAG_AMD_KIND_SQ8_UNIFORM>(s->metric, p.T, grid, block, lds, st, a, f);
             break;
         case VSAG_AMD_KIND_RABITQ:
-            launch_flat_m<VSAG_AMD_KIND_RABITQ>(s->metric, p.T, grid, block, lds, st, a, f);
+            if (s->query_bits == 32) {
+                launch_flat_m<kKindRabitqF32>(s->metric, p.T, grid, block, lds, st, a, f);
+            } else {
+                launch_flat_m<VSAG_AMD_KIND_RABITQ>(s->metric, p.T, grid, block, lds, st, a, f);
+            }
             break;
         default:
             return fail(VSAG_AMD_INVALID_ARGUMENT, "unknown store kind %d", s->kind);

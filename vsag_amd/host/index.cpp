@@ -609,8 +609,8 @@ public:
             q_.rabitq_query_bits = static_cast<int>(index_param["rabitq_bits_per_dim_query"].GetInt());
         }
         if (q_.kind == VSAG_AMD_KIND_RABITQ) {
-            CHECK_ARGUMENT(q_.rabitq_query_bits == 4,
-                           "the GPU path scans rabitq with rabitq_bits_per_dim_query = 4 only");
+            CHECK_ARGUMENT(q_.rabitq_query_bits == 4 || q_.rabitq_query_bits == 32,
+                           "rabitq_bits_per_dim_query must be 4 or 32");
             if (index_param.Contains("rabitq_bits_per_dim_base")) {
                 CHECK_ARGUMENT(index_param["rabitq_bits_per_dim_base"].GetInt() == 1,
                                "the GPU path supports rabitq_bits_per_dim_base = 1 only");
@@ -785,8 +785,8 @@ public:
             q_.rabitq_query_bits = static_cast<int>(index_param["rabitq_bits_per_dim_query"].GetInt());
         }
         if (q_.kind == VSAG_AMD_KIND_RABITQ) {
-            CHECK_ARGUMENT(q_.rabitq_query_bits == 4,
-                           "the GPU path scans rabitq with rabitq_bits_per_dim_query = 4 only");
+            CHECK_ARGUMENT(q_.rabitq_query_bits == 4 || q_.rabitq_query_bits == 32,
+                           "rabitq_bits_per_dim_query must be 4 or 32");
         }
         if (index_param.Contains("buckets_count")) {
             int64_t b = index_param["buckets_count"].GetInt();
