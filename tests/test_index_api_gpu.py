@@ -292,3 +292,34 @@ def test_range_search(lib, name, params, search):
         idx.range_search(q[0], 1.0, search, limit=0)
     assert e.value.code == -3
     idx.close()
+
+
+@pytest.mark.parametrize("name,params,search", [
+    ("brute_force", {"base_quantization_type": "fp32"}, "{}"),
+    ("ivf", {"buckets_count": 16, "base_quantization_type": "fp32"}, json.dumps({"ivf": {"scan_buckets_count": 16}})),
+    ("ivf", {"buckets_count": 16, "base_quantization_type": "sq8", "use_reorder": True,
+             "precise_quantization_type": "fp32"}, json.dumps({"ivf": {"scan_buckets_count": 16, "factor": 1.5}})),
+])
+def test_k_above_one_device_scan(lib, name, params, search):
+    """k larger than the 1024 results of one device scan: one query per call, several scans."""
+    n, d, k = 6000, 16, 2500
+    x = vectors(n, d)
+    q = vectors(3, d, seed=165)
+    labels = np.arange(n, dtype=np.int64) * 2
+    idx = make(name, d, "l2", **params)
+    assert idx.build(x, labels, n, d) == 0
+    gt, gt_d = ground_truth(x, q, k, "l2")
+    for i in range(3):
+        ids, dists = idx.knn_search(q[i], k, search)
+        assert ids.size == k and np.unique(ids).size == k
+        assert np.all(np.diff(dists) >= 0)
+        hit = len(set(ids.tolist()) & set(labels[gt[i]].tolist())) / float(k)
+        if params["base_quantization_type"] == "fp32":
+            assert hit >= 0.999
+            np.testing.assert_allclose(dists, gt_d[i], rtol=1e-4, atol=1e-6)
+        else:
+            assert hit >= 0.9
+    with pytest.raises(pyvsag.VsagError) as e:
+        idx.knn_search_batch(q, k, search)
+    assert e.value.code == -3
+    idx.close()

@@ -655,27 +655,29 @@ protected:
             empty->NumElements(1)->Dim(0);
             return empty;
         }
-        CHECK_ARGUMENT(!spec.range || nq == 1, "range search takes one query");
-        CHECK_ARGUMENT(spec.range || k <= kMaxDeviceK, "the GPU path supports k <= 1024, got " + std::to_string(k));
+        // One device scan returns at most 1024 results per query.  A range search, and a KnnSearch with a larger
+        // k, run scan after scan for one query: what a scan returned is denied to the next one, so the rows come
+        // out in ascending order.
+        const bool looped = spec.range || k > kMaxDeviceK;
+        CHECK_ARGUMENT(!looped || nq == 1, spec.range ? "range search takes one query"
+                                                      : "k above 1024 is supported for one query per call");
         queries_.reserve(static_cast<size_t>(nq) * q_.dim * 4);
         dev(vsag_amd_memcpy_h2d(queries_.p, query->GetFloat32Vectors(), static_cast<size_t>(nq) * q_.dim * 4, nullptr));
         DenyMask mask;
-        mask.init(labels_, spec.valid, spec.range);
+        mask.init(labels_, spec.valid, looped);
         const vsag_amd_search_options_t opt = mask.options(spec, 0.0F);
         // distance_evaluations as the reference counts them: every stored vector once per query
         const std::string stats = "{\"dist_cmp\":" + std::to_string(labels_.size() * static_cast<size_t>(nq)) + "}";
         const auto n = static_cast<int64_t>(labels_.size());
-        if (!spec.range) {
+        if (!looped) {
             const auto kk = static_cast<uint32_t>(k);
             std::vector<uint32_t> ids;
             std::vector<float> dists;
             scan(nq, kk, opt, ids, dists);
             return pack_results(ids, dists, nq, k, labels_, stats);
         }
-        // Range: the nearest candidates within the radius, a device scan of at most 1024 at a time; what a
-        // scan returned is denied to the next one, so the rows come out in ascending order.
         std::vector<std::pair<float, uint32_t>> row;
-        int64_t remaining = spec.limited_size > 0 ? spec.limited_size : n;
+        int64_t remaining = spec.range ? (spec.limited_size > 0 ? spec.limited_size : n) : k;
         while (remaining > 0) {
             const auto kk = static_cast<uint32_t>(std::min<int64_t>({remaining, kMaxDeviceK, n}));
             std::vector<uint32_t> ids;
@@ -872,13 +874,21 @@ protected:
             empty->NumElements(1)->Dim(0);
             return empty;
         }
-        CHECK_ARGUMENT(!spec.range || nq == 1, "range search takes one query");
         const auto n = static_cast<int64_t>(labels_.size());
         const auto nprobe = static_cast<uint32_t>(std::min<int64_t>(scan, nlist_));  // ivf.cpp:1573-1574
         const bool reorder = use_reorder_ && enable_reorder;
         if (reorder) {
             CHECK_ARGUMENT(factor > 0.0F, "factor must be positive when use_reorder is true");
         }
+        int64_t kcand = k;
+        if (reorder && !spec.range) {
+            kcand = std::max<int64_t>(static_cast<int64_t>(factor * static_cast<float>(k)), 1);  // ivf.cpp:2316
+        }
+        // One device scan returns at most 1024 candidates per query; more (and every range search) run scan
+        // after scan for one query, each denied what the earlier ones returned.
+        const bool looped = spec.range || kcand > kMaxDeviceK;
+        CHECK_ARGUMENT(!looped || nq == 1, spec.range ? "range search takes one query"
+                                                      : "factor * k above 1024 is supported for one query per call");
 
         queries_.reserve(static_cast<size_t>(nq) * q_.dim * 4);
         dev(vsag_amd_memcpy_h2d(queries_.p, query->GetFloat32Vectors(), static_cast<size_t>(nq) * q_.dim * 4, nullptr));
@@ -902,17 +912,12 @@ protected:
             return pack_results(ids, dists, nq, nprobe, identity, "{}");
         }
         DenyMask mask;
-        mask.init(labels_, spec.valid, spec.range);
+        mask.init(labels_, spec.valid, looped);
         // FlatBucketSearcher compares against radius + THRESHOLD_ERROR (flat_bucket_searcher.cpp:121,
         // impl/searcher/basic_searcher.h:39).
         const vsag_amd_search_options_t opt = mask.options(spec, 2e-6F);
 
-        if (!spec.range) {
-            int64_t kcand = k;
-            if (reorder) {
-                kcand = std::max<int64_t>(static_cast<int64_t>(factor * static_cast<float>(k)), 1);  // ivf.cpp:2316
-            }
-            CHECK_ARGUMENT(kcand <= kMaxDeviceK && k <= kMaxDeviceK, "the GPU path supports factor * k <= 1024");
+        if (!looped) {
             // 2. scan the probed lists; 3. exact rerank, best min(k, candidates) kept (flatten_reorder.cpp:77)
             const int64_t kout = reorder ? std::min<int64_t>(k, kcand) : kcand;
             std::vector<uint32_t> ids;
@@ -923,11 +928,15 @@ protected:
         }
         // Range (ivf.cpp:2282-2307): candidates within the radius by the list codes, at most factor *
         // limited_size of them when a rerank follows; the rerank keeps the nearest limited_size (all of them
-        // when unlimited).  A device scan returns at most 1024 candidates; what it returned is denied to the
-        // next scan.
-        int64_t want = spec.limited_size > 0 ? spec.limited_size : n;
-        if (reorder && spec.limited_size > 0) {
-            want = std::max<int64_t>(static_cast<int64_t>(factor * static_cast<float>(spec.limited_size)), 1);
+        // when unlimited).  Large k: kcand candidates, the rerank keeps k.
+        int64_t want = kcand;
+        int64_t keep = k;
+        if (spec.range) {
+            want = spec.limited_size > 0 ? spec.limited_size : n;
+            keep = want;
+            if (reorder && spec.limited_size > 0) {
+                want = std::max<int64_t>(static_cast<int64_t>(factor * static_cast<float>(spec.limited_size)), 1);
+            }
         }
         std::vector<std::pair<float, uint32_t>> row;
         int64_t remaining = want;
@@ -951,8 +960,8 @@ protected:
         if (reorder) {
             // batches were reranked one by one: order the whole row by exact distance
             std::sort(row.begin(), row.end());
-            if (spec.limited_size > 0 && static_cast<int64_t>(row.size()) > spec.limited_size) {
-                row.resize(static_cast<size_t>(spec.limited_size));
+            if (static_cast<int64_t>(row.size()) > keep) {
+                row.resize(static_cast<size_t>(keep));
             }
         }
         if (row.empty()) {
