@@ -276,6 +276,15 @@ def run_c2(env):
             "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
             "kernel": "flat_scan_kernel<sq8, l2, T=%d>" % r["tile"], "kernel_ms": r["kernel_ms"],
             "algorithmic_bytes_per_launch": algo_bytes}
+    if r["tile"] >= 64:
+        # The batch went through the matrix-core contraction (query tile 128): the dominant kernel multiplies
+        # every code of the store but the exactly scanned prefix with every query, 2 d flops per pair.
+        flops = 2.0 * n * d * nq
+        tf = flops / (r["kernel_ms"] * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": tf, "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": tf / MFMA_F32_PEAK_TFLOPS, "traffic": None, "kernel": "prefilter_kernel<sq8> (fp32 MFMA)",
+                "kernel_ms": r["kernel_ms"], "flops_per_launch": flops,
+                "algorithmic_bytes_per_launch": algo_bytes, "algorithmic_gbs": achieved}
     return env.base_line("QPS @ recall@10 (1M x 128 SQ8 scan)", "queries/s", r["qps"], r["sec"],
                          "u8 codes, f32 accumulate",
                          "configs[1]: flat SQ8 scan, N=%d, d=%d, %d queries, k=%d, L2 (headline) and IP" % (n, d, nq, k),
@@ -317,6 +326,11 @@ def run_c1(env):
             "traffic": None, "kernel": "flat_scan_kernel<fp32, l2, T=%d>" % tile, "kernel_ms": kms,
             "algorithmic_bytes_per_launch": algo, "flops_per_launch": 2.0 * n * d * nq,
             "tflops": 2.0 * n * d * nq / (kms * 1e-3) / 1e12}
+    if tile >= 64:
+        tf = 2.0 * n * d * nq / (kms * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": tf, "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": tf / MFMA_F32_PEAK_TFLOPS, "traffic": None, "kernel": "prefilter_kernel<fp32> (fp32 MFMA)",
+                "kernel_ms": kms, "flops_per_launch": 2.0 * n * d * nq}
     return env.base_line("QPS @ recall@10 (100k x 128 fp32 brute force)", "queries/s", nq / sec, sec, "f32",
                          "configs[0]: brute_force fp32 L2, N=%d, d=%d, %d queries, k=%d" % (n, d, nq, k),
                          {"recall_at_10": rec, "query_tile": tile, "passes_per_step": passes, "bytes_per_pass": bpp},
@@ -660,6 +674,8 @@ def main():
     ap.add_argument("--k", type=int, default=10)
     ap.add_argument("--tile", type=int, default=0, help="query tile override (0 = library default)")
     ap.add_argument("--chunks", type=int, default=0, help="base chunk override (0 = library default)")
+    ap.add_argument("--contraction", type=int, default=0, choices=[-1, 0, 1],
+                    help="matrix-core path of the flat scans: -1 never, 0 library default, 1 whenever supported")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-recall", action="store_true", help="skip the recall check")
     ap.add_argument("--no-single", action="store_true", help="skip the one-query-per-call measurement")
@@ -669,6 +685,7 @@ def main():
               "shard); --gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
     env = Env(args)
+    env.capi.check(env.lib.vsag_amd_set_scan_contraction(args.contraction))
     line = {"c1": run_c1, "c2": run_c2, "c3": run_c3, "c4": run_c4, "c5": run_c5}[args.config](env)
     print(json.dumps(line))
 

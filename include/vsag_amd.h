@@ -194,6 +194,13 @@ VSAG_AMD_API int vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* store, const
                                uint32_t k, const vsag_amd_search_options_t* options, uint32_t* ids_dev,
                                float* dists_dev, void* workspace_dev, size_t workspace_bytes, void* stream);
 
+/* Large batches on flat fp32 / sq8 stores are served by a matrix-core contraction that pre-selects candidates,
+ * which are then recomputed and selected exactly as the streaming scan does (same results, bit for bit).
+ * mode: 0 = when it pays (default: >= 1024 queries, k <= 128, >= 4096 tiles), 1 = whenever the store and k
+ * allow it, -1 = never.  Process-wide; affects vsag_amd_flat_scan_workspace_bytes as well.  No counterpart in the
+ * reference (it scans one query at a time). */
+VSAG_AMD_API int vsag_amd_set_scan_contraction(int mode);
+
 /* Tuning knobs of the scan (query tile T in {1,2,4,8}, 0 = automatic; number of base chunks, 0 =
  * automatic).  Process-wide; meant for benchmarks. */
 VSAG_AMD_API int vsag_amd_set_scan_tuning(int query_tile, int base_chunks);

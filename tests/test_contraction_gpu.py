@@ -1,0 +1,89 @@
+"""Large batches on flat fp32 / sq8 stores: the matrix-core contraction pre-selects, the streaming arithmetic
+decides.  Its results must equal the streaming scan's bit for bit (and therefore the checker's within the usual
+tolerance), including when candidates overflow and the streaming kernel takes over."""
+import numpy as np
+import pytest
+
+import oracle as orc
+from gpu_helpers import Store, assert_topk_close, gaussian_mixture
+from vsag_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture()
+def modes(lib):
+    L = capi.load_library()
+
+    def both(store, q, k):
+        capi.check(L.vsag_amd_set_scan_contraction(-1))
+        plain = store.flat_scan(q, k)
+        capi.check(L.vsag_amd_set_scan_contraction(1))
+        fast = store.flat_scan(q, k)
+        tile = capi.C.c_int()
+        L.vsag_amd_last_scan_info(capi.C.byref(tile), None, None)
+        capi.check(L.vsag_amd_set_scan_contraction(0))
+        return plain, fast, tile.value
+    yield both
+    capi.check(L.vsag_amd_set_scan_contraction(0))
+
+
+def same(a, b):
+    return np.array_equal(a[0], b[0]) and np.array_equal(a[1].view(np.uint32), b[1].view(np.uint32))
+
+
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP])
+@pytest.mark.parametrize("n,d,nq,k", [(40000, 128, 300, 10), (20001, 100, 129, 100), (9000, 960, 64, 10),
+                                      (5000, 33, 1000, 7)])
+def test_sq8_contraction_equals_streaming(lib, modes, metric, n, d, nq, k):
+    rng = np.random.default_rng(n + d + k)
+    x, means = gaussian_mixture(rng, n, d, 30, 0.05)
+    q, _ = gaussian_mixture(rng, nq, d, 30, 0.05, means=means)
+    lb, diff = orc.sq_train(x, 8, metric)
+    codes = orc.sq_encode(x, 8, lb, diff, metric)
+    st = Store(capi.KIND_SQ8, metric, d, lb=lb, diff=diff)
+    st.append(codes[:n // 3])
+    st.append(codes[n // 3:])  # the per-code terms follow appends
+    plain, fast, tile = modes(st, q, k)
+    assert tile == 128, "the contraction path did not run"
+    assert same(plain, fast)
+    ri, rd = orc.flat_scan_topk(orc.SQ8, metric, d, codes, q[:16], k, lb=lb, diff=diff)
+    assert_topk_close(fast[0][:16], fast[1][:16], ri, rd, label="sq8 contraction")
+    st.destroy()
+
+
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
+@pytest.mark.parametrize("n,d,nq,k", [(30000, 128, 200, 10), (7000, 65, 77, 32)])
+def test_fp32_contraction_equals_streaming(lib, modes, metric, n, d, nq, k):
+    rng = np.random.default_rng(n + d + k + metric)
+    x = rng.random((n, d), dtype=np.float32)
+    q = rng.random((nq, d), dtype=np.float32)
+    x[5] = q[3]  # an exact duplicate of a query: distance 0 must come out as 0
+    st = Store(capi.KIND_FP32, metric, d)
+    st.append(x.view(np.uint8).reshape(n, 4 * d))
+    plain, fast, tile = modes(st, q, k)
+    assert tile == 128
+    assert same(plain, fast)
+    if metric == orc.L2:
+        assert fast[0][3, 0] == 5 and fast[1][3, 0] == 0.0
+    st.destroy()
+
+
+def test_contraction_overflow_falls_back_to_streaming(lib, modes):
+    """Thousands of equal distances per query: the candidate buffers overflow, the streaming kernel serves the query."""
+    rng = np.random.default_rng(8)
+    n, d, nq, k = 30000, 32, 150, 10
+    base = rng.integers(0, 256, (40, d), dtype=np.uint8)
+    codes = base[rng.integers(0, 40, n)]  # 40 distinct codes, 750 copies each
+    lb, diff = np.zeros(d, np.float32), np.ones(d, np.float32)
+    q = rng.random((nq, d), dtype=np.float32)
+    st = Store(capi.KIND_SQ8, orc.L2, d, lb=lb, diff=diff)
+    st.append(codes)
+    plain, fast, tile = modes(st, q, k)
+    assert tile == 128
+    assert same(plain, fast)
+    ri, rd = orc.flat_scan_topk(orc.SQ8, orc.L2, d, codes, q[:8], k, lb=lb, diff=diff)
+    # which of the equal distances the checker keeps is its heap's business; the distances must agree
+    np.testing.assert_allclose(fast[1][:8], rd, rtol=1e-5)
+    assert np.all(np.diff(fast[0], axis=1)[np.diff(fast[1], axis=1) == 0] > 0), "ties are ordered by id"
+    st.destroy()

@@ -21,7 +21,8 @@ HIP_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
 ]
-KERNEL_SOURCES = ["runtime.hip", "store.hip", "quantize.hip", "prepare.hip", "scan.hip", "ivf.hip", "kmeans.hip"]
+KERNEL_SOURCES = ["runtime.hip", "store.hip", "quantize.hip", "prepare.hip", "scan.hip", "prefilter.hip", "ivf.hip",
+                  "kmeans.hip"]
 
 
 def _run(cmd):

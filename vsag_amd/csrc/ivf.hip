@@ -40,7 +40,8 @@ ScanArgs make_scan_args(const vsag_amd_store* s, const QueryLayout& ql, const ui
 void timing_begin(hipStream_t st);
 void timing_end(hipStream_t st);
 int launch_merge_partials(const uint64_t* partial, const uint32_t* partial_cnt, const uint32_t* bound, uint32_t nslots,
-                          uint32_t k, uint32_t S, uint64_t nq, uint32_t* ids, float* dists, hipStream_t st);
+                          uint32_t stride, uint32_t k, uint32_t S, uint64_t nq, uint32_t* ids, float* dists,
+                          hipStream_t st);
 
 // Up to five word arrays set in one launch.
 struct FillJob {
@@ -828,8 +829,8 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
         VA_TRY(launch_ivf(s, p.T, grid, dim3(waves * kWave), lds, st, a, v));
     }
     timing_end(st);
-    return launch_merge_partials(b.partial, b.partial_cnt, b.bound, nprobe * p.chunks_max, kcand, p.S, nq, ids_dev,
-                                 dists_dev, st);
+    return launch_merge_partials(b.partial, b.partial_cnt, b.bound, nprobe * p.chunks_max, nprobe * p.chunks_max, kcand,
+                                 p.S, nq, ids_dev, dists_dev, st);
 }
 
 extern "C" int

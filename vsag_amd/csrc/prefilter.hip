@@ -1,0 +1,547 @@
+// Large query batches against a flat fp32 / sq8 store: the scan becomes a contraction on the matrix cores.
+//
+// With thousands of queries the streaming scan (scan.hip) is bound by vector-ALU issue, not by memory: every
+// (query, code) pair costs d multiply-adds on the VALU.  The same inner products are an (N x d) * (d x nq)
+// matrix product, which v_mfma_f32_32x32x2_f32 delivers several times faster -- but a product in the form
+// |a|^2 - 2<a, y> + |y|^2 does not reproduce the reference's sum of (a_d - y_d)^2 bit for bit, and cancels badly
+// for near-duplicates.  So the matrix product only pre-selects:
+//
+//   1. the streaming kernel scans a prefix of the store exactly; its k-th distance is a bound per query;
+//   2. prefilter_kernel forms all inner products of the remaining codes with all queries tile by tile and
+//      keeps the (query, code) pairs whose distance, minus a rigorous bound of the rounding error of the
+//      product form, does not exceed the query's bound -- a few hundred candidates per query;
+//   3. rescore_kernel recomputes these candidates with the streaming kernel's own arithmetic (the same
+//      accumulate_granule in the same order) and selects from them as the streaming kernel would.
+//
+// The result is therefore the streaming result, bit for bit.  A query whose candidates overflow their buffer
+// (no bound yet, masses of equal distances) is flagged and served by the streaming kernel over the remaining
+// tiles instead.
+#include "distance.h"
+#include "store.h"
+#include "topk.h"
+
+namespace vsag_amd {
+
+void timing_begin(hipStream_t st);
+void timing_end(hipStream_t st);
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int PM = 128;  // codes per tile (two storage tiles)
+constexpr int PN = 128;  // queries per tile
+constexpr int PK = 32;   // contraction depth per stage
+constexpr int kPfPlane = PM;
+
+// LDS operand layout of one stage: [parity h = k & 1][chunk c = (k >> 1) / 4][row] of float4, element e of the
+// float4 is k = 2 (4 c + e) + h, so that a lane of the MFMA (row = lane % 32, h = lane / 32) reads its operand
+// for four consecutive k-steps with one conflict-free ds_read_b128.
+struct PfStage {
+    float4 a[2 * 4 * kPfPlane];
+    float4 b[2 * 4 * kPfPlane];
+};
+
+// Scatter four consecutive k (k = 4g .. 4g+3 of `row`) into the parity planes.
+__device__ inline void
+pf_stage_store(float4* plane, uint32_t row, uint32_t g, float4 v) {
+    uint32_t c = g >> 1, e = (g & 1) * 2;
+    float* even = reinterpret_cast<float*>(&plane[(0 * 4 + c) * kPfPlane + row]) + e;
+    float* odd = reinterpret_cast<float*>(&plane[(1 * 4 + c) * kPfPlane + row]) + e;
+    *reinterpret_cast<float2*>(even) = make_float2(v.x, v.z);
+    *reinterpret_cast<float2*>(odd) = make_float2(v.y, v.w);
+}
+
+struct PrefilterArgs {
+    const uint4* tiles;
+    uint32_t G;
+    uint64_t tile_begin, tile_end;  // storage tiles covered
+    uint64_t n;                     // codes in the store (slots at or beyond are padding)
+    const float* scale;             // sq8, l2: y_d = c_d * scale_d; null: y_d = c_d
+    const float* qtab;              // processed queries, qstride floats per row, zero beyond the dimension
+    uint32_t qstride;
+    uint64_t nq;
+    uint32_t kdim;                  // contraction length
+    const float* term;              // per slot |y|^2
+    float term_factor;              // 1 (l2) or 0 (ip)
+    float dot_factor;               // -2 (l2) or -1 (ip)
+    const float* tau;               // per query: keep a pair when term_factor |y|^2 + dot_factor <a, y> <= tau
+    uint32_t* cand;                 // nq x cap slots
+    uint32_t* cand_cnt;             // nq
+    uint32_t cap;
+    uint32_t groups;                // grid x; code tile t is walked by group t % groups
+};
+
+__device__ inline float4
+pf_query_chunk(const float* qtab, uint64_t row, uint64_t rows, uint32_t k0, uint32_t stride) {
+    if (row < rows && k0 + 4 <= stride) {
+        return *reinterpret_cast<const float4*>(qtab + row * stride + k0);
+    }
+    return make_float4(0.0F, 0.0F, 0.0F, 0.0F);
+}
+
+template <int KIND>
+__global__ void __launch_bounds__(256, 2)
+prefilter_kernel(PrefilterArgs p) {
+    __shared__ PfStage stage[2];  // 64 KiB
+    // The per-code terms of a tile's epilogue live in stage 1, which the next tile does not write before its
+    // first barrier inside the contraction loop.
+    float* code_term = reinterpret_cast<float*>(stage[1].a);
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    const uint32_t wave = tid >> 6;
+    const uint32_t wm = wave & 1;   // which 64 codes of the tile
+    const uint32_t wn = wave >> 1;  // which 64 queries of the tile
+    const uint32_t half = lane >> 5;
+    const uint32_t l32 = lane & 31;
+    const uint64_t q0 = static_cast<uint64_t>(blockIdx.y) * PN;
+    const uint32_t ktiles = (p.kdim + PK - 1) / PK;
+    const uint64_t span = p.tile_end - p.tile_begin;
+    const uint64_t mtiles = (span + 1) / 2;
+
+    // Query loader roles: 1024 float4 per stage, four per thread (row = idx / 8, chunk = idx % 8).
+    uint32_t qrow[4], qg[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        uint32_t idx = tid + 256 * r;
+        qrow[r] = idx >> 3;
+        qg[r] = idx & 7;
+    }
+    float tau_n[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        uint64_t q = q0 + wn * 64 + j * 32 + l32;
+        tau_n[j] = q < p.nq ? p.tau[q] : -__builtin_inff();
+    }
+
+    // Code loader: a thread fetches granules of code `crow` of the tile (storage tile crow / 64, lane crow % 64).
+    const uint32_t crow = tid & 127;
+    const uint32_t cpart = tid >> 7;  // 0 / 1
+    auto code_granule = [&](uint64_t mt, uint32_t j) {
+        uint64_t tile = p.tile_begin + 2 * mt + (crow >> 6);
+        if (tile < p.tile_end && j < p.G) {
+            return p.tiles[(tile * p.G + j) * kWave + (crow & 63)];
+        }
+        return make_uint4(0, 0, 0, 0);
+    };
+    // sq8: a stage is 32 dimensions = granules 2 kt and 2 kt + 1, one per thread.
+    // fp32: a stage is 32 dimensions = granules 8 kt .. 8 kt + 7, four per thread (cpart, cpart + 2, ...).
+    constexpr int kCodeRegs = KIND == VSAG_AMD_KIND_SQ8 ? 1 : 4;
+    auto fetch_codes = [&](uint64_t mt, uint32_t kt, uint4 (&regs)[kCodeRegs]) {
+        if constexpr (KIND == VSAG_AMD_KIND_SQ8) {
+            regs[0] = code_granule(mt, 2 * kt + cpart);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                regs[r] = code_granule(mt, 8 * kt + cpart + 2 * r);
+            }
+        }
+    };
+    auto park_codes = [&](float4* plane, uint32_t kt, const uint4 (&regs)[kCodeRegs]) {
+        if constexpr (KIND == VSAG_AMD_KIND_SQ8) {
+            const uint32_t w[4] = {regs[0].x, regs[0].y, regs[0].z, regs[0].w};
+            const uint32_t d0 = PK * kt + 16 * cpart;
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                float4 v = make_float4(static_cast<float>(w[m] & 0xffU), static_cast<float>((w[m] >> 8) & 0xffU),
+                                       static_cast<float>((w[m] >> 16) & 0xffU), static_cast<float>(w[m] >> 24));
+                if (p.scale != nullptr && d0 + 16 <= p.kdim) {
+                    float4 sc = *reinterpret_cast<const float4*>(p.scale + d0 + 4 * m);
+                    v.x *= sc.x;
+                    v.y *= sc.y;
+                    v.z *= sc.z;
+                    v.w *= sc.w;
+                }
+                pf_stage_store(plane, crow, 4 * cpart + m, v);
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float4 v = make_float4(__uint_as_float(regs[r].x), __uint_as_float(regs[r].y),
+                                       __uint_as_float(regs[r].z), __uint_as_float(regs[r].w));
+                pf_stage_store(plane, crow, cpart + 2 * r, v);
+            }
+        }
+    };
+
+    // Operands of stage 0 of the first tile; from then on the next tile's stage 0 is fetched while the last
+    // stage of the current tile is multiplied, so that no tile starts by waiting for memory.
+    uint4 rc[kCodeRegs];
+    float4 rq[4];
+    float my_term = 0.0F;
+    auto fetch_stage0 = [&](uint64_t mt) {
+        fetch_codes(mt, 0, rc);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            rq[r] = pf_query_chunk(p.qtab, q0 + qrow[r], p.nq, 4 * qg[r], p.qstride);
+        }
+    };
+    if (blockIdx.x < mtiles) {
+        fetch_stage0(blockIdx.x);
+    }
+    for (uint64_t mt = blockIdx.x; mt < mtiles; mt += p.groups) {
+        floatx16 acc[2][2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    acc[i][j][e] = 0.0F;
+                }
+            }
+        }
+        const uint64_t slot0 = (p.tile_begin + 2 * mt) * kWave;
+        // Stage 0 is free: the previous tile's contraction ended with a barrier, its epilogue reads stage 1.
+        park_codes(stage[0].a, 0, rc);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            pf_stage_store(stage[0].b, qrow[r], qg[r], rq[r]);
+        }
+        if (tid < PM) {
+            uint64_t slot = slot0 + tid;
+            bool real = slot < p.n && p.tile_begin + 2 * mt + (tid >> 6) < p.tile_end;
+            my_term = real ? p.term_factor * p.term[slot] : __builtin_inff();
+        }
+        __syncthreads();  // also: every wave has left the previous epilogue, stage 1 may be written
+        for (uint32_t kt = 0; kt < ktiles; ++kt) {
+            const uint32_t cur = kt & 1;
+            if (kt + 1 < ktiles) {
+                fetch_codes(mt, kt + 1, rc);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    rq[r] = pf_query_chunk(p.qtab, q0 + qrow[r], p.nq, PK * (kt + 1) + 4 * qg[r], p.qstride);
+                }
+            } else if (mt + p.groups < mtiles) {
+                fetch_stage0(mt + p.groups);
+            }
+            const float4* pa = stage[cur].a + half * 4 * kPfPlane + wm * 64 + l32;
+            const float4* pb = stage[cur].b + half * 4 * kPfPlane + wn * 64 + l32;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                float4 a0 = pa[c * kPfPlane];
+                float4 a1 = pa[c * kPfPlane + 32];
+                float4 b0 = pb[c * kPfPlane];
+                float4 b1 = pb[c * kPfPlane + 32];
+                const float av0[4] = {a0.x, a0.y, a0.z, a0.w};
+                const float av1[4] = {a1.x, a1.y, a1.z, a1.w};
+                const float bv0[4] = {b0.x, b0.y, b0.z, b0.w};
+                const float bv1[4] = {b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[e], bv0[e], acc[0][0], 0, 0, 0);
+                    acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[e], bv1[e], acc[0][1], 0, 0, 0);
+                    acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[e], bv0[e], acc[1][0], 0, 0, 0);
+                    acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[e], bv1[e], acc[1][1], 0, 0, 0);
+                }
+            }
+            if (kt + 1 < ktiles) {
+                park_codes(stage[cur ^ 1].a, kt + 1, rc);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    pf_stage_store(stage[cur ^ 1].b, qrow[r], qg[r], rq[r]);
+                }
+            }
+            __syncthreads();
+        }
+        if (tid < PM) {
+            code_term[tid] = my_term;
+        }
+        __syncthreads();
+        // acc[i][j][e] = <y_m, a_n> with m = wm*64 + i*32 + 8*(e/4) + 4*half + e%4 (code of the tile) and
+        // n = wn*64 + j*32 + l32 (query of the tile).
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint64_t q = q0 + wn * 64 + j * 32 + l32;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const uint32_t ml = wm * 64 + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+                    const float v = code_term[ml] + p.dot_factor * acc[i][j][e];
+                    if (v <= tau_n[j]) {
+                        uint32_t pos = atomicAdd(&p.cand_cnt[q], 1U);
+                        if (pos < p.cap) {
+                            p.cand[q * p.cap + pos] = static_cast<uint32_t>(slot0 + ml);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// |y|^2 of the codes in slots [first, first + count) and the running maximum of |y| (as float bits; norms are
+// not negative, so the bits order like the values).  One lane per code, dimensions in order.
+template <int KIND>
+__global__ void __launch_bounds__(256)
+code_term_kernel(const uint4* tiles, uint32_t G, const float* scale, uint64_t first, uint64_t count, float* term,
+                 uint32_t* ymax_bits) {
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    float s = 0.0F;
+    if (i < count) {
+        uint64_t slot = first + i;
+        uint64_t tile = slot >> 6;
+        uint32_t ln = static_cast<uint32_t>(slot & 63);
+        for (uint32_t j = 0; j < G; ++j) {
+            uint4 c = tiles[(tile * G + j) * kWave + ln];
+            const uint32_t w[4] = {c.x, c.y, c.z, c.w};
+            if constexpr (KIND == VSAG_AMD_KIND_SQ8) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    float y = static_cast<float>((w[e >> 2] >> (8 * (e & 3))) & 0xffU);
+                    if (scale != nullptr) {
+                        y *= scale[16 * j + e];
+                    }
+                    s = fmaf(y, y, s);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float y = __uint_as_float(w[e]);
+                    s = fmaf(y, y, s);
+                }
+            }
+        }
+        term[slot] = s;
+    }
+    float m = sqrtf(s);
+    for (int off = 32; off > 0; off >>= 1) {
+        float o = __shfl_xor(m, off);
+        m = o > m ? o : m;
+    }
+    if ((threadIdx.x & 63) == 0 && m > 0.0F) {
+        atomicMax(ymax_bits, __float_as_uint(m));
+    }
+}
+
+// Per query: the admission threshold of the prefilter.  With dist = C_q + B <a, y> + F |y|^2 (l2: C = |a|^2,
+// B = -2, F = 1; ip: C = 1 - qmeta, B = -1, F = 0) and the fp32 contraction of kdim terms off by at most
+// kdim * 2^-22 * |a| * |y| (twice the worst case of sequential fp32 accumulation), a pair can only belong to the
+// result when B <a, y> + F |y|^2 <= bound - C + |B| * err, plus the rounding of these few terms themselves.
+__global__ void __launch_bounds__(64)
+prefilter_tau_kernel(const float* qtab, uint32_t qstride, uint32_t kdim, const float* qmeta, uint32_t qmeta_stride,
+                     int is_l2, const uint32_t* bound, const uint32_t* ymax_bits, uint64_t nq, float* tau) {
+    uint64_t q = blockIdx.x;
+    uint32_t lane = threadIdx.x;
+    const float* row = qtab + q * qstride;
+    float a2 = 0.0F;
+    for (uint32_t d = lane; d < kdim; d += kWave) {
+        a2 = fmaf(row[d], row[d], a2);
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        a2 += __shfl_xor(a2, off);
+    }
+    if (lane != 0) {
+        return;
+    }
+    uint32_t b = bound[q];
+    if (b == 0xFFFFFFFFU) {
+        tau[q] = 3.0e38F;  // no bound yet: everything is a candidate (and the query will overflow)
+        return;
+    }
+    float bd = ordered_to_float(b);
+    float ymax = __uint_as_float(*ymax_bits);
+    float cq = is_l2 ? a2 : 1.0F - (qmeta != nullptr ? qmeta[q * qmeta_stride] : 0.0F);
+    float factor = is_l2 ? 2.0F : 1.0F;
+    float err = factor * static_cast<float>(kdim) * 2.4e-7F * sqrtf(a2) * ymax;
+    float magnitude = fabsf(bd) + fabsf(cq) + (is_l2 ? ymax * ymax : 0.0F) + factor * sqrtf(a2) * ymax;
+    float t = bd - cq + err + 1.0e-6F * magnitude;
+    tau[q] = t < 3.0e38F ? t : 3.0e38F;
+}
+
+struct RescoreArgs {
+    const uint32_t* cand;
+    const uint32_t* cand_cnt;
+    uint32_t cap;
+    uint64_t n;
+    uint32_t k, S;
+    uint32_t* bound;
+    uint64_t* partial;
+    uint32_t* partial_cnt;
+    uint32_t nslots;
+    uint32_t out_slot;
+    uint32_t* gate;  // per query: 1 = candidates overflowed, the streaming kernel must serve the query
+};
+
+// One wave per query: exact distances of its candidates by the streaming kernel's arithmetic, best k kept.
+template <int KIND, int METRIC>
+__global__ void __launch_bounds__(64)
+rescore_kernel(ScanArgs a, RescoreArgs r) {
+    extern __shared__ uint64_t keys[];
+    const uint32_t lane = threadIdx.x;
+    const uint32_t q = blockIdx.x;
+    const uint32_t total = as_const(r.cand_cnt)[q];
+    const uint64_t list = static_cast<uint64_t>(q) * r.nslots + r.out_slot;
+    if (total > r.cap) {
+        if (lane == 0) {
+            r.gate[q] = 1;
+            r.partial_cnt[list] = 0;
+        }
+        return;
+    }
+    if (lane == 0) {
+        r.gate[q] = 0;
+    }
+    const uint32_t S = r.S, k = r.k;
+    selector_init(keys, S, lane);
+    uint32_t cnt = 0;
+    uint32_t bs = __builtin_amdgcn_readfirstlane(__atomic_load_n(&r.bound[q], __ATOMIC_RELAXED));
+    // Candidates arrive in no particular order, so ties are decided on whole (distance, id) keys.
+    uint64_t tau = (static_cast<uint64_t>(bs) << 32) | 0xFFFFFFFFULL;
+    const uint32_t qidx[1] = {q};
+    const QueryRows<1> qrows = query_rows<1>(a, qidx);
+    const uint32_t* mine = r.cand + static_cast<uint64_t>(q) * r.cap;
+    for (uint32_t base = 0; base < total; base += kWave) {
+        const bool have = base + lane < total;
+        const uint32_t slot = have ? mine[base + lane] : 0U;
+        const uint64_t tile = slot >> 6;
+        const uint32_t ln = slot & 63;
+        Acc<KIND, 1> acc;
+        acc_reset(acc);
+        for (uint32_t j = 0; j < a.G; ++j) {
+            uint4 c = a.tiles[(tile * a.G + j) * kWave + ln];
+            accumulate_granule<KIND, METRIC, 1>(a, qrows, j, c, acc);
+        }
+        float d[1];
+        finish_distances<KIND, METRIC, 1>(a, qidx, slot, acc, d);
+        const uint64_t key = make_key(d[0], slot);
+        bool pass = have && slot < r.n && key <= tau;
+        uint64_t mask = __ballot(pass);
+        if (mask != 0) {
+            uint32_t np = __popcll(mask);
+            if (k + cnt + np > S) {
+                uint64_t th = selector_flush(keys, S, k, cnt, lane);
+                cnt = 0;
+                uint32_t b = lower_shared(&r.bound[q], static_cast<uint32_t>(th >> 32), lane);
+                uint64_t shared_tau = (static_cast<uint64_t>(b) << 32) | 0xFFFFFFFFULL;
+                tau = th < shared_tau ? th : shared_tau;
+            }
+            if (pass) {
+                keys[k + cnt + mask_rank(mask)] = key;
+            }
+            cnt += np;
+        }
+    }
+    wave_lds_fence();
+    bs = __builtin_amdgcn_readfirstlane(__atomic_load_n(&r.bound[q], __ATOMIC_RELAXED));
+    uint32_t kept = k + cnt;
+    uint32_t admitted = selector_count_admitted(keys, kept, bs, lane);
+    if (admitted > k) {
+        uint64_t th = selector_flush(keys, S, k, cnt, lane);
+        bs = lower_shared(&r.bound[q], static_cast<uint32_t>(th >> 32), lane);
+        kept = k;
+        admitted = selector_count_admitted(keys, kept, bs, lane);
+    }
+    if (lane == 0) {
+        r.partial_cnt[list] = admitted;
+    }
+    if (admitted != 0) {
+        selector_copy_admitted(keys, kept, bs, r.partial + list * k, lane);
+    }
+}
+
+// ------------------------------------------------------------------ host side
+bool
+prefilter_supports(const vsag_amd_store* s) {
+    return s->nlist == 0 && (s->kind == VSAG_AMD_KIND_FP32 || s->kind == VSAG_AMD_KIND_SQ8) && s->pf_term != nullptr;
+}
+
+// |y|^2 for freshly appended codes (y as the contraction sees it: scaled codes for sq8 l2, raw code values
+// for sq8 ip, the stored vector for fp32).
+int
+launch_code_terms(vsag_amd_store* s, uint64_t first, uint64_t count, hipStream_t st) {
+    if (count == 0 || s->pf_term == nullptr) {
+        return 0;
+    }
+    dim3 grid(static_cast<uint32_t>(div_up(count, 256)));
+    if (s->kind == VSAG_AMD_KIND_SQ8) {
+        const float* scale = s->metric == VSAG_AMD_METRIC_L2 ? s->scale_dev : nullptr;
+        hipLaunchKernelGGL(code_term_kernel<VSAG_AMD_KIND_SQ8>, grid, dim3(256), 0, st, s->tiles, s->G, scale, first,
+                           count, s->pf_term, s->pf_ymax);
+    } else {
+        hipLaunchKernelGGL(code_term_kernel<VSAG_AMD_KIND_FP32>, grid, dim3(256), 0, st, s->tiles, s->G,
+                           static_cast<const float*>(nullptr), first, count, s->pf_term, s->pf_ymax);
+    }
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
+template <int KIND>
+static void
+launch_rescore_m(int metric, dim3 grid, size_t lds, hipStream_t st, const ScanArgs& a, const RescoreArgs& r) {
+    if (metric == VSAG_AMD_METRIC_L2) {
+        hipLaunchKernelGGL((rescore_kernel<KIND, VSAG_AMD_METRIC_L2>), grid, dim3(kWave), lds, st, a, r);
+    } else {
+        hipLaunchKernelGGL((rescore_kernel<KIND, VSAG_AMD_METRIC_IP>), grid, dim3(kWave), lds, st, a, r);
+    }
+}
+
+// Steps 2 and 3 of the header comment for tiles [tile_begin, tile_end); the exact prefix scan has already
+// left its bounds in `bound`.  Writes one partial list per query (out_slot) and the overflow flags.
+int
+launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t k, uint32_t S, uint64_t tile_begin,
+                 uint64_t tile_end, uint32_t* bound, float* tau, uint32_t* cand, uint32_t* cand_cnt, uint32_t cap,
+                 uint64_t* partial, uint32_t* partial_cnt, uint32_t nslots, uint32_t out_slot, uint32_t* gate,
+                 hipStream_t st) {
+    const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
+    const bool sq8 = s->kind == VSAG_AMD_KIND_SQ8;
+    hipLaunchKernelGGL(prefilter_tau_kernel, dim3(static_cast<uint32_t>(nq)), dim3(kWave), 0, st,
+                       reinterpret_cast<const float*>(a.qtab), a.qstride, s->dpad, sq8 && !l2 ? a.qmeta : nullptr,
+                       a.qmeta_stride, l2 ? 1 : 0, bound, s->pf_ymax, nq, tau);
+    PrefilterArgs p{};
+    p.tiles = s->tiles;
+    p.G = s->G;
+    p.tile_begin = tile_begin;
+    p.tile_end = tile_end;
+    p.n = s->n;
+    p.scale = sq8 && l2 ? s->scale_dev : nullptr;
+    p.qtab = reinterpret_cast<const float*>(a.qtab);
+    p.qstride = a.qstride;
+    p.nq = nq;
+    p.kdim = s->dpad;
+    p.term = s->pf_term;
+    p.term_factor = l2 ? 1.0F : 0.0F;
+    p.dot_factor = l2 ? -2.0F : -1.0F;
+    p.tau = tau;
+    p.cand = cand;
+    p.cand_cnt = cand_cnt;
+    p.cap = cap;
+    const uint64_t mtiles = (tile_end - tile_begin + 1) / 2;
+    const uint64_t qtiles = div_up(nq, static_cast<uint64_t>(PN));
+    // About four workgroups per compute unit in flight; a group walks every groups-th code tile.
+    uint64_t groups = div_up(static_cast<uint64_t>(device_cu_count()) * 4, qtiles);
+    groups = std::max<uint64_t>(1, std::min<uint64_t>(groups, mtiles));
+    p.groups = static_cast<uint32_t>(groups);
+    dim3 grid(p.groups, static_cast<uint32_t>(qtiles));
+    timing_begin(st);
+    if (sq8) {
+        hipLaunchKernelGGL(prefilter_kernel<VSAG_AMD_KIND_SQ8>, grid, dim3(256), 0, st, p);
+    } else {
+        hipLaunchKernelGGL(prefilter_kernel<VSAG_AMD_KIND_FP32>, grid, dim3(256), 0, st, p);
+    }
+    timing_end(st);
+    VA_HIP(hipGetLastError());
+    RescoreArgs r{};
+    r.cand = cand;
+    r.cand_cnt = cand_cnt;
+    r.cap = cap;
+    r.n = s->n;
+    r.k = k;
+    r.S = S;
+    r.bound = bound;
+    r.partial = partial;
+    r.partial_cnt = partial_cnt;
+    r.nslots = nslots;
+    r.out_slot = out_slot;
+    r.gate = gate;
+    dim3 rgrid(static_cast<uint32_t>(nq));
+    if (sq8) {
+        launch_rescore_m<VSAG_AMD_KIND_SQ8>(s->metric, rgrid, S * 8, st, a, r);
+    } else {
+        launch_rescore_m<VSAG_AMD_KIND_FP32>(s->metric, rgrid, S * 8, st, a, r);
+    }
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
+}  // namespace vsag_amd

@@ -28,6 +28,33 @@ uint64_t rabitq_query_code_size(uint32_t dim, int metric, int query_bits);
 
 constexpr uint32_t kMaxWaves = 4;
 
+// Zeroes two word arrays.
+__global__ void
+fill_words2_kernel(uint32_t* a, uint64_t na, uint32_t* b, uint64_t nb) {
+    uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < na) {
+        a[i] = 0;
+    }
+    if (i < nb) {
+        b[i] = 0;
+    }
+}
+
+// bound[q] = the k-th distance of a merged result, when there is one.
+__global__ void
+tighten_bound_kernel(const float* dists, uint32_t k, uint64_t nq, uint32_t* bound) {
+    uint64_t q = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (q < nq) {
+        float kth = dists[q * k + k - 1];
+        if (kth < __builtin_inff()) {
+            uint32_t o = float_to_ordered(kth);
+            if (o < bound[q]) {
+                bound[q] = o;
+            }
+        }
+    }
+}
+
 // Per query: no bound yet, no seeds yet.
 __global__ void
 reset_queries_kernel(uint32_t* bound, uint32_t bound0, uint64_t nq, uint32_t* seed, uint64_t nseed) {
@@ -42,12 +69,15 @@ reset_queries_kernel(uint32_t* bound, uint32_t bound0, uint64_t nq, uint32_t* se
 
 struct FlatArgs {
     uint64_t n;
-    uint64_t ntiles;
+    uint64_t tile0;         // the launch covers tiles [tile0, tile_end)
+    uint64_t tile_end;
     uint64_t tiles_per_chunk;
     uint64_t nq;
     uint32_t k;
     uint32_t S;
-    uint32_t nslots;        // partial lists per query = chunks * waves
+    uint32_t nslots;        // partial lists per query (all launches of the call)
+    uint32_t slot0;         // first list of this launch
+    const uint32_t* gate;   // per query: 0 = this launch leaves the query alone; null = every query
     uint32_t* bound;        // per query: ordered distance that k candidates are known to reach
     uint64_t* partial;      // nq x nslots x k keys
     uint32_t* partial_cnt;  // nq x nslots
@@ -77,14 +107,21 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
     uint32_t thr[T];   // a candidate passes when its ordered distance is below thr
     uint32_t cnt[T];
     uint32_t cold[T];  // tiles after which this wave still looks at the seed row
+    bool live[T];      // a real query that this launch serves
+    bool any_live = false;
 #pragma unroll
     for (int t = 0; t < T; ++t) {
         qidx[t] = blockIdx.x * T + t;
         cnt[t] = 0;
-        uint32_t bs = qidx[t] < f.nq ? __builtin_amdgcn_readfirstlane(__atomic_load_n(&f.bound[qidx[t]], __ATOMIC_RELAXED))
-                                     : 0xFFFFFFFFU;
-        thr[t] = bs == 0xFFFFFFFFU ? bs : bs + 1;
-        cold[t] = SEED && qidx[t] < f.nq && bs == 0xFFFFFFFFU ? kSeedTiles : 0;
+        live[t] = qidx[t] < f.nq && (f.gate == nullptr || as_const(f.gate)[qidx[t]] != 0);
+        any_live = any_live || live[t];
+        uint32_t bs = live[t] ? __builtin_amdgcn_readfirstlane(__atomic_load_n(&f.bound[qidx[t]], __ATOMIC_RELAXED))
+                              : 0xFFFFFFFFU;
+        thr[t] = !live[t] ? 0U : bs == 0xFFFFFFFFU ? bs : bs + 1;
+        cold[t] = SEED && live[t] && bs == 0xFFFFFFFFU ? kSeedTiles : 0;
+    }
+    if (!any_live) {
+        return;
     }
     for (uint32_t i = lane; i < T * S; i += kWave) {
         sel[i] = kInfKey;
@@ -92,10 +129,10 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
     wave_lds_fence();
     const uint32_t seed_slot = (blockIdx.y * nwaves + wave) % k;
 
-    const uint64_t tile_begin = static_cast<uint64_t>(blockIdx.y) * f.tiles_per_chunk;
+    const uint64_t tile_begin = f.tile0 + static_cast<uint64_t>(blockIdx.y) * f.tiles_per_chunk;
     uint64_t tile_end = tile_begin + f.tiles_per_chunk;
-    if (tile_end > f.ntiles) {
-        tile_end = f.ntiles;
+    if (tile_end > f.tile_end) {
+        tile_end = f.tile_end;
     }
     // Software pipeline over granule groups: the loads of group g+1 (possibly of the next tile) are
     // issued before group g is consumed, so every wave keeps GROUP KiB in flight.  Two register buffers
@@ -119,7 +156,7 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
         cold[t] = 0;
         uint32_t tl = static_cast<uint32_t>(th >> 32);  // 0xFFFFFFFF while fewer than k seen
         uint32_t bs = 0xFFFFFFFFU;
-        if (qidx[t] < f.nq) {
+        if (live[t]) {
             bs = lower_shared(&f.bound[qidx[t]], tl, lane);  // tl = 0xFFFFFFFF lowers nothing
         }
         uint32_t tb = bs == 0xFFFFFFFFU ? bs : bs + 1;
@@ -194,10 +231,10 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
         cur = nxt;
     }
 
-    const uint32_t slot = blockIdx.y * nwaves + wave;
+    const uint32_t slot = f.slot0 + blockIdx.y * nwaves + wave;
 #pragma unroll
     for (int t = 0; t < T; ++t) {
-        if (qidx[t] >= f.nq) {
+        if (!live[t]) {
             continue;
         }
         // Whatever lies above the shared bound is beaten by k candidates of other waves.  What remains is
@@ -357,15 +394,15 @@ constexpr uint32_t kPoolKeys = 4096;
 
 __global__ void __launch_bounds__(1024)
 merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, const uint32_t* bound, uint32_t nslots,
-                      uint32_t k, uint32_t S, uint32_t* ids, float* dists) {
+                      uint32_t stride, uint32_t k, uint32_t S, uint32_t* ids, float* dists) {
     extern __shared__ uint64_t lds[];  // S output keys, then the pool
     __shared__ uint32_t npool;
     __shared__ uint32_t nout;
     __shared__ SelectScratch scratch;
     uint64_t* pool = lds + S;
     const uint64_t q = blockIdx.x;
-    const uint32_t* cnts = partial_cnt + q * nslots;
-    const uint64_t* src = partial + q * nslots * k;
+    const uint32_t* cnts = partial_cnt + q * stride;  // the first nslots of the query's `stride` lists
+    const uint64_t* src = partial + q * stride * k;
     uint64_t admit = (static_cast<uint64_t>(as_const(bound)[q]) << 32) | 0xFFFFFFFFULL;
     // Finitely many rounds: every round that overflows lowers `admit` below at least one pooled key.
     for (;;) {
@@ -430,11 +467,12 @@ merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, cons
 // ------------------------------------------------------------------ host side
 int
 launch_merge_partials(const uint64_t* partial, const uint32_t* partial_cnt, const uint32_t* bound, uint32_t nslots,
-                      uint32_t k, uint32_t S, uint64_t nq, uint32_t* ids, float* dists, hipStream_t st) {
+                      uint32_t stride, uint32_t k, uint32_t S, uint64_t nq, uint32_t* ids, float* dists,
+                      hipStream_t st) {
     // Few queries: many candidates each (every wave starts without a bound), so give each merge more threads.
     const uint32_t threads = nq <= 256 ? 1024 : 256;
     hipLaunchKernelGGL(merge_partials_kernel, dim3(static_cast<uint32_t>(nq)), dim3(threads), (S + kPoolKeys) * 8, st,
-                       partial, partial_cnt, bound, nslots, k, S, ids, dists);
+                       partial, partial_cnt, bound, nslots, stride, k, S, ids, dists);
     VA_HIP(hipGetLastError());
     return 0;
 }
@@ -535,6 +573,65 @@ make_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, uint64_t ntiles, Sca
     }
 }
 
+// A call is served either by one streaming launch over all tiles, or -- large batches on fp32 / sq8 stores
+// (prefilter.hip) -- by a streaming launch over a prefix, the matrix-core prefilter with exact rescoring over the
+// rest, and a streaming launch over the rest for the queries whose candidates overflowed.
+struct CallPlan {
+    ScanPlan all;
+    bool contraction = false;
+    ScanPlan prefix, rest;
+    uint64_t prefix_tiles = 0;
+    uint32_t cap = 0;          // candidates per query
+    uint32_t nslots = 0;       // partial lists per query
+    bool any_seeded = false;
+};
+
+static int g_prefilter_mode = 0;  // -1 never, 0 when it pays, 1 whenever the store supports it
+
+bool prefilter_supports(const vsag_amd_store* s);
+int launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t k, uint32_t S, uint64_t tile_begin,
+                     uint64_t tile_end, uint32_t* bound, float* tau, uint32_t* cand, uint32_t* cand_cnt, uint32_t cap,
+                     uint64_t* partial, uint32_t* partial_cnt, uint32_t nslots, uint32_t out_slot, uint32_t* gate,
+                     hipStream_t st);
+
+static void
+make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
+    make_plan(s, nq, k, s->ntiles, &c->all);
+    c->nslots = static_cast<uint32_t>(c->all.chunks * c->all.waves);
+    c->any_seeded = c->all.seeded;
+    c->contraction = false;
+    if (g_prefilter_mode < 0 || !prefilter_supports(s)) {
+        return;
+    }
+    const bool forced = g_prefilter_mode > 0;
+    if (!forced && (nq < 1024 || k > 128 || s->ntiles < 4096)) {
+        return;
+    }
+    // Candidate buffers: at most 2 GiB in all, 1024 to 4096 candidates per query.
+    uint64_t cap = 4096;
+    while (cap > 1024 && nq * cap * 4 > (2ull << 30)) {
+        cap /= 2;
+    }
+    if (nq * cap * 4 > (2ull << 30)) {
+        return;
+    }
+    // The prefix is scanned exactly; its k-th distance admits about k * (rest / prefix) codes of the rest.
+    // Keep that below an eighth of the buffer.
+    uint64_t prefix = std::max<uint64_t>(forced ? 2 : 256, div_up(8ull * k * s->ntiles, cap));
+    prefix += prefix & 1;  // the contraction walks pairs of tiles
+    if (prefix > s->ntiles / (forced ? 2 : 4) || prefix >= s->ntiles) {
+        return;
+    }
+    c->contraction = true;
+    c->prefix_tiles = prefix;
+    c->cap = static_cast<uint32_t>(cap);
+    make_plan(s, nq, k, prefix, &c->prefix);
+    make_plan(s, nq, k, s->ntiles - prefix, &c->rest);
+    uint32_t pf_slots = static_cast<uint32_t>(c->prefix.chunks * c->prefix.waves + 1 + c->rest.chunks * c->rest.waves);
+    c->nslots = std::max(c->nslots, pf_slots);
+    c->any_seeded = c->any_seeded || c->prefix.seeded || c->rest.seeded;
+}
+
 struct ScanBuffers {
     uint32_t* qtab;
     float* qmeta;
@@ -542,21 +639,31 @@ struct ScanBuffers {
     uint32_t* bound;
     uint32_t* partial_cnt;
     uint64_t* partial;
-    uint32_t* seed;  // null when the plan does not seed
+    uint32_t* seed;  // null when no launch of the plan seeds
+    // contraction only
+    float* tau;
+    uint32_t* cand_cnt;
+    uint32_t* gate;
+    uint32_t* cand;
 };
 
 static size_t
-carve_scan(Carver& c, const ScanPlan& p, uint64_t nq, uint32_t k, ScanBuffers* b) {
+carve_scan(Carver& c, const CallPlan& cp, uint64_t nq, uint32_t k, ScanBuffers* b) {
+    const ScanPlan& p = cp.all;
     b->qtab = c.take<uint32_t>(p.nq_pad * p.ql.qstride);
     b->qmeta = c.take<float>(p.nq_pad * p.ql.qmeta);
     b->qcodes = c.take<uint8_t>(p.qcode_bytes);
     b->bound = c.take<uint32_t>(nq);
-    b->partial_cnt = c.take<uint32_t>(nq * p.chunks * p.waves);
-    b->seed = c.take<uint32_t>(p.seeded ? nq * k : 0);
-    if (!p.seeded) {
+    b->partial_cnt = c.take<uint32_t>(nq * cp.nslots);
+    b->seed = c.take<uint32_t>(cp.any_seeded ? nq * k : 0);
+    if (!cp.any_seeded) {
         b->seed = nullptr;
     }
-    b->partial = c.take<uint64_t>(nq * p.chunks * p.waves * k);
+    b->partial = c.take<uint64_t>(nq * cp.nslots * k);
+    b->tau = c.take<float>(cp.contraction ? nq : 0);
+    b->cand_cnt = c.take<uint32_t>(cp.contraction ? nq : 0);
+    b->gate = c.take<uint32_t>(cp.contraction ? nq : 0);
+    b->cand = c.take<uint32_t>(cp.contraction ? nq * cp.cap : 0);
     return c.used;
 }
 
@@ -656,11 +763,11 @@ vsag_amd_flat_scan_workspace_bytes(const vsag_amd_store_t* s, uint64_t nq, uint3
     if (check_scan_call(s, nq, k) != 0 || ensure_init() != 0) {
         return 0;
     }
-    ScanPlan p;
-    make_plan(s, nq, k, s->ntiles, &p);
+    CallPlan cp;
+    make_call_plan(s, nq, k, &cp);
     Carver c(nullptr, 0);
     ScanBuffers b;
-    return carve_scan(c, p, nq, k, &b) + 256;
+    return carve_scan(c, cp, nq, k, &b) + 256;
 }
 
 extern "C" int
@@ -671,6 +778,34 @@ vsag_amd_flat_scan_topk(const vsag_amd_store_t* s, const float* queries_dev, uin
                                       workspace_bytes, stream);
 }
 
+namespace {
+
+// One streaming launch over tiles [tile0, tile_end), writing partial lists slot0, slot0 + 1, ...
+int
+run_streaming(const vsag_amd_store* s, const ScanPlan& p, const ScanArgs& a, const ScanBuffers& b, uint64_t nq,
+              uint32_t k, const vsag_amd_search_options_t* options, uint64_t tile0, uint64_t tile_end, uint32_t slot0,
+              uint32_t nslots, const uint32_t* gate, hipStream_t st) {
+    FlatArgs f{};
+    f.n = s->n;
+    f.tile0 = tile0;
+    f.tile_end = tile_end;
+    f.tiles_per_chunk = p.tiles_per_chunk;
+    f.nq = nq;
+    f.k = k;
+    f.S = p.S;
+    f.nslots = nslots;
+    f.slot0 = slot0;
+    f.gate = gate;
+    f.bound = b.bound;
+    f.partial = b.partial;
+    f.partial_cnt = b.partial_cnt;
+    f.seed = p.seeded ? b.seed : nullptr;
+    f.deny = options != nullptr ? options->deny_bits_dev : nullptr;
+    return launch_flat(s, p, a, f, st);
+}
+
+}  // namespace
+
 extern "C" int
 vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, uint64_t nq, uint32_t k,
                            const vsag_amd_search_options_t* options, uint32_t* ids_dev, float* dists_dev,
@@ -680,42 +815,61 @@ vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, 
     VA_CHECK_ARG(s->nlist == 0, "flat scan on a posting-list store");
     VA_CHECK_ARG(queries_dev && ids_dev && dists_dev, "null query / output pointer");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    ScanPlan p;
-    make_plan(s, nq, k, s->ntiles, &p);
+    CallPlan cp;
+    make_call_plan(s, nq, k, &cp);
     Carver c(workspace_dev, workspace_bytes);
     ScanBuffers b;
-    carve_scan(c, p, nq, k, &b);
+    carve_scan(c, cp, nq, k, &b);
     VA_CHECK_ARG(c.ok(), "workspace too small: need %zu bytes, got %zu", c.used, workspace_bytes);
+    // A pre-filter or a radius goes the streaming way (the prefilter knows neither).
+    const bool contraction = cp.contraction && options == nullptr;
+    const ScanPlan& p = cp.all;
 
     VA_TRY(prepare_queries(s, queries_dev, nq, p.nq_pad, p.ql, b.qtab, b.qmeta, b.qcodes, st));
-    const uint64_t nseed = p.seeded ? nq * k : 0;
+    const uint64_t nseed = b.seed != nullptr ? nq * k : 0;
     hipLaunchKernelGGL(reset_queries_kernel, dim3(static_cast<uint32_t>(div_up(nq > nseed ? nq : nseed, 256))), dim3(256),
                        0, st, b.bound, initial_bound(options), nq, b.seed, nseed);
     ScanArgs a = make_scan_args(s, p.ql, b.qtab, b.qmeta);
-    FlatArgs f{};
-    f.n = s->n;
-    f.ntiles = s->ntiles;
-    f.tiles_per_chunk = p.tiles_per_chunk;
-    f.nq = nq;
-    f.k = k;
-    f.S = p.S;
-    f.nslots = static_cast<uint32_t>(p.chunks * p.waves);
-    f.bound = b.bound;
-    f.partial = b.partial;
-    f.partial_cnt = b.partial_cnt;
-    f.seed = b.seed;
-    f.deny = options != nullptr ? options->deny_bits_dev : nullptr;
-    if (s->ntiles != 0) {
+    uint32_t nslots = 0;
+    if (s->ntiles == 0) {
+        // An empty store has no lists to read.
+    } else if (!contraction) {
+        nslots = static_cast<uint32_t>(p.chunks * p.waves);
         timing_begin(st);
-        VA_TRY(launch_flat(s, p, a, f, st));
+        VA_TRY(run_streaming(s, p, a, b, nq, k, options, 0, s->ntiles, 0, nslots, nullptr, st));
         timing_end(st);
+        tl_last_tile = p.T;
+        tl_last_passes = p.groups;
+    } else {
+        const uint32_t slots_prefix = static_cast<uint32_t>(cp.prefix.chunks * cp.prefix.waves);
+        const uint32_t slots_rest = static_cast<uint32_t>(cp.rest.chunks * cp.rest.waves);
+        nslots = slots_prefix + 1 + slots_rest;
+        // The gated launch leaves the lists of most queries untouched: they must read as empty.  No candidates yet.
+        hipLaunchKernelGGL(fill_words2_kernel, dim3(static_cast<uint32_t>(div_up(nq * nslots, 256))), dim3(256), 0, st,
+                           b.partial_cnt, nq * nslots, b.cand_cnt, nq);
+        VA_TRY(run_streaming(s, cp.prefix, a, b, nq, k, nullptr, 0, cp.prefix_tiles, 0, nslots, nullptr, st));
+        // The waves of the prefix each know the k-th distance of their own tiles only; the k-th of the whole
+        // prefix (a merge into the output arrays, which the final merge overwrites) is the bound to filter with.
+        VA_TRY(launch_merge_partials(b.partial, b.partial_cnt, b.bound, slots_prefix, nslots, k, p.S, nq, ids_dev,
+                                     dists_dev, st));
+        hipLaunchKernelGGL(tighten_bound_kernel, dim3(static_cast<uint32_t>(div_up(nq, 256))), dim3(256), 0, st,
+                           dists_dev, k, nq, b.bound);
+        VA_TRY(launch_prefilter(s, a, nq, k, p.S, cp.prefix_tiles, s->ntiles, b.bound, b.tau, b.cand, b.cand_cnt, cp.cap,
+                                b.partial, b.partial_cnt, nslots, slots_prefix, b.gate, st));
+        VA_TRY(run_streaming(s, cp.rest, a, b, nq, k, nullptr, cp.prefix_tiles, s->ntiles, slots_prefix + 1, nslots,
+                             b.gate, st));
+        tl_last_tile = 128;  // queries per pass of the contraction
+        tl_last_passes = div_up(nq, 128);
     }
-    // An empty store has no lists to read.
-    VA_TRY(launch_merge_partials(b.partial, b.partial_cnt, b.bound, s->ntiles != 0 ? f.nslots : 0U, k, p.S, nq, ids_dev,
-                                 dists_dev, st));
-    tl_last_tile = p.T;
-    tl_last_passes = p.groups;
+    VA_TRY(launch_merge_partials(b.partial, b.partial_cnt, b.bound, nslots, nslots, k, p.S, nq, ids_dev, dists_dev, st));
     tl_last_bytes = s->ntiles * s->G * kWave * kGranule;
+    return 0;
+}
+
+extern "C" int
+vsag_amd_set_scan_contraction(int mode) {
+    VA_CHECK_ARG(mode >= -1 && mode <= 1, "mode must be -1 (never), 0 (when it pays) or 1 (whenever supported)");
+    g_prefilter_mode = mode;
     return 0;
 }
 

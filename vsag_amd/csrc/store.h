@@ -50,6 +50,11 @@ struct vsag_amd_store {
     std::vector<uint32_t> list_sizes;    // host copy
     std::vector<uint32_t> list_tile;     // host copy, nlist+1
     uint32_t max_list_tiles = 0;         // tiles of the longest list
+
+    // flat fp32 / sq8 stores: per slot |y|^2 and the largest |y| (float bits) of the code as the batched
+    // contraction sees it, kept up to date by append
+    float* pf_term = nullptr;
+    uint32_t* pf_ymax = nullptr;
 };
 
 namespace vsag_amd {
@@ -61,5 +66,6 @@ struct QueryLayout {
 };
 
 QueryLayout query_layout(const vsag_amd_store* s);
+int launch_code_terms(vsag_amd_store* s, uint64_t first, uint64_t count, hipStream_t st);
 
 }  // namespace vsag_amd

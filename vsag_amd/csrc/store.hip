@@ -172,6 +172,13 @@ grow(vsag_amd_store* s, uint64_t need_tiles, hipStream_t st) {
                                   s->ntiles * kWave * sizeof(uint32_t), hipMemcpyDeviceToDevice, st));
         }
     }
+    float* term = nullptr;
+    if (s->pf_ymax != nullptr) {
+        VA_HIP(hipMalloc(&term, cap * kWave * sizeof(float)));
+        if (s->ntiles > 0) {
+            VA_HIP(hipMemcpyAsync(term, s->pf_term, s->ntiles * kWave * sizeof(float), hipMemcpyDeviceToDevice, st));
+        }
+    }
     VA_HIP(hipStreamSynchronize(st));
     if (s->tiles) {
         VA_HIP(hipFree(s->tiles));
@@ -179,8 +186,12 @@ grow(vsag_amd_store* s, uint64_t need_tiles, hipStream_t st) {
     if (s->meta) {
         VA_HIP(hipFree(s->meta));
     }
+    if (s->pf_term) {
+        VA_HIP(hipFree(s->pf_term));
+    }
     s->tiles = tiles;
     s->meta = meta;
+    s->pf_term = term;
     s->cap_tiles = cap;
     return 0;
 }
@@ -365,6 +376,11 @@ vsag_amd_store_create(const vsag_amd_store_params_t* p, vsag_amd_store_t** out) 
             return fail_free(fail(VSAG_AMD_NO_ENOUGH_MEMORY, "copying the rabitq rotation failed"));
         }
     }
+    if (p->kind == VSAG_AMD_KIND_FP32 || p->kind == VSAG_AMD_KIND_SQ8) {
+        if (hipMalloc(&s->pf_ymax, 4) != hipSuccess || hipMemset(s->pf_ymax, 0, 4) != hipSuccess) {
+            return fail_free(fail(VSAG_AMD_NO_ENOUGH_MEMORY, "hipMalloc of the norm scalar failed"));
+        }
+    }
     (void)rc;
     *out = s;
     return 0;
@@ -376,7 +392,7 @@ vsag_amd_store_destroy(vsag_amd_store_t* s) {
         return 0;
     }
     void* ptrs[] = {s->scale_dev, s->lb_dev,  s->diff_dev, s->bounds_dev,    s->rotation_dev, s->centroid_dev,
-                    s->tiles,     s->meta,    s->ids_dev,  s->list_tile_dev};
+                    s->tiles,     s->meta,    s->ids_dev,  s->list_tile_dev, s->pf_term,      s->pf_ymax};
     for (void* p : ptrs) {
         if (p != nullptr) {
             (void)hipFree(p);
@@ -409,6 +425,7 @@ vsag_amd_store_append(vsag_amd_store_t* s, const uint8_t* codes_dev, uint64_t n,
     uint64_t threads = n * s->G;
     hipLaunchKernelGGL(retile_kernel, dim3(static_cast<uint32_t>(div_up(threads, 256))), dim3(256), 0, st, a);
     VA_HIP(hipGetLastError());
+    VA_TRY(launch_code_terms(s, s->n, n, st));
     s->n += n;
     s->ntiles = need;
     return 0;
