@@ -196,7 +196,7 @@ VSAG_AMD_API int vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* store, const
 
 /* Large batches on flat fp32 / sq8 stores are served by a matrix-core contraction that pre-selects candidates,
  * which are then recomputed and selected exactly as the streaming scan does (same results, bit for bit).
- * mode: 0 = when it pays (default: >= 1024 queries, k <= 128, >= 4096 tiles), 1 = whenever the store and k
+ * mode: 0 = when it pays (default: >= 512 queries, k <= 128, >= 65536 codes), 1 = whenever the store and k
  * allow it, -1 = never.  Process-wide; affects vsag_amd_flat_scan_workspace_bytes as well.  No counterpart in the
  * reference (it scans one query at a time). */
 VSAG_AMD_API int vsag_amd_set_scan_contraction(int mode);

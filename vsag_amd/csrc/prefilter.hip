@@ -79,12 +79,12 @@ pf_query_chunk(const float* qtab, uint64_t row, uint64_t rows, uint32_t k0, uint
 }
 
 template <int KIND>
-__global__ void __launch_bounds__(256, 2)
+__global__ void __launch_bounds__(256, 3)
 prefilter_kernel(PrefilterArgs p) {
-    __shared__ PfStage stage[2];  // 64 KiB
-    // The per-code terms of a tile's epilogue live in stage 1, which the next tile does not write before its
-    // first barrier inside the contraction loop.
-    float* code_term = reinterpret_cast<float*>(stage[1].a);
+    // One 32 KiB stage: three workgroups (twelve waves, as many as the 170 registers of a wave allow) per compute
+    // unit fill each other's barriers and loader phases, which pays more than double buffering with fewer waves.
+    __shared__ PfStage stage[1];
+    __shared__ float code_term[PM];
 
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
@@ -191,7 +191,7 @@ prefilter_kernel(PrefilterArgs p) {
             }
         }
         const uint64_t slot0 = (p.tile_begin + 2 * mt) * kWave;
-        // Stage 0 is free: the previous tile's contraction ended with a barrier, its epilogue reads stage 1.
+        // The stage is free: the previous tile's contraction ended with a barrier.
         park_codes(stage[0].a, 0, rc);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -200,11 +200,10 @@ prefilter_kernel(PrefilterArgs p) {
         if (tid < PM) {
             uint64_t slot = slot0 + tid;
             bool real = slot < p.n && p.tile_begin + 2 * mt + (tid >> 6) < p.tile_end;
-            my_term = real ? p.term_factor * p.term[slot] : __builtin_inff();
+            code_term[tid] = real ? p.term_factor * p.term[slot] : __builtin_inff();
         }
-        __syncthreads();  // also: every wave has left the previous epilogue, stage 1 may be written
+        __syncthreads();  // also: every wave has left the previous epilogue (code_term)
         for (uint32_t kt = 0; kt < ktiles; ++kt) {
-            const uint32_t cur = kt & 1;
             if (kt + 1 < ktiles) {
                 fetch_codes(mt, kt + 1, rc);
 #pragma unroll
@@ -214,8 +213,8 @@ prefilter_kernel(PrefilterArgs p) {
             } else if (mt + p.groups < mtiles) {
                 fetch_stage0(mt + p.groups);
             }
-            const float4* pa = stage[cur].a + half * 4 * kPfPlane + wm * 64 + l32;
-            const float4* pb = stage[cur].b + half * 4 * kPfPlane + wn * 64 + l32;
+            const float4* pa = stage[0].a + half * 4 * kPfPlane + wm * 64 + l32;
+            const float4* pb = stage[0].b + half * 4 * kPfPlane + wn * 64 + l32;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 float4 a0 = pa[c * kPfPlane];
@@ -234,35 +233,40 @@ prefilter_kernel(PrefilterArgs p) {
                     acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[e], bv1[e], acc[1][1], 0, 0, 0);
                 }
             }
+            __syncthreads();  // every wave has read the stage
             if (kt + 1 < ktiles) {
-                park_codes(stage[cur ^ 1].a, kt + 1, rc);
+                park_codes(stage[0].a, kt + 1, rc);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    pf_stage_store(stage[cur ^ 1].b, qrow[r], qg[r], rq[r]);
+                    pf_stage_store(stage[0].b, qrow[r], qg[r], rq[r]);
                 }
+                __syncthreads();
             }
-            __syncthreads();
         }
-        if (tid < PM) {
-            code_term[tid] = my_term;
-        }
-        __syncthreads();
-        // acc[i][j][e] = <y_m, a_n> with m = wm*64 + i*32 + 8*(e/4) + 4*half + e%4 (code of the tile) and
-        // n = wn*64 + j*32 + l32 (query of the tile).
+        // Nearly nothing passes: first collect the verdicts of all 64 products of this lane branch-free, then
+        // let the rare lanes with a hit append.
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            const uint64_t q = q0 + wn * 64 + j * 32 + l32;
+            uint32_t hits = 0;
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const uint32_t ml = wm * 64 + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
                     const float v = code_term[ml] + p.dot_factor * acc[i][j][e];
-                    if (v <= tau_n[j]) {
-                        uint32_t pos = atomicAdd(&p.cand_cnt[q], 1U);
-                        if (pos < p.cap) {
-                            p.cand[q * p.cap + pos] = static_cast<uint32_t>(slot0 + ml);
-                        }
+                    hits |= (v <= tau_n[j] ? 1U : 0U) << (16 * i + e);
+                }
+            }
+            if (hits != 0) {
+                const uint64_t q = q0 + wn * 64 + j * 32 + l32;
+                while (hits != 0) {
+                    const uint32_t bit = static_cast<uint32_t>(__builtin_ctz(hits));
+                    hits &= hits - 1;
+                    const uint32_t i = bit >> 4, e = bit & 15;
+                    const uint32_t ml = wm * 64 + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+                    uint32_t pos = atomicAdd(&p.cand_cnt[q], 1U);
+                    if (pos < p.cap) {
+                        p.cand[q * p.cap + pos] = static_cast<uint32_t>(slot0 + ml);
                     }
                 }
             }
@@ -508,8 +512,9 @@ launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32
     p.cap = cap;
     const uint64_t mtiles = (tile_end - tile_begin + 1) / 2;
     const uint64_t qtiles = div_up(nq, static_cast<uint64_t>(PN));
-    // About four workgroups per compute unit in flight; a group walks every groups-th code tile.
-    uint64_t groups = div_up(static_cast<uint64_t>(device_cu_count()) * 4, qtiles);
+    // About six workgroups per compute unit (two rounds of the three that fit); a group walks every groups-th
+    // code tile.
+    uint64_t groups = div_up(static_cast<uint64_t>(device_cu_count()) * 6, qtiles);
     groups = std::max<uint64_t>(1, std::min<uint64_t>(groups, mtiles));
     p.groups = static_cast<uint32_t>(groups);
     dim3 grid(p.groups, static_cast<uint32_t>(qtiles));

@@ -604,7 +604,7 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
         return;
     }
     const bool forced = g_prefilter_mode > 0;
-    if (!forced && (nq < 1024 || k > 128 || s->ntiles < 4096)) {
+    if (!forced && (nq < 512 || k > 128 || s->ntiles < 1024)) {
         return;
     }
     // Candidate buffers: at most 2 GiB in all, 1024 to 4096 candidates per query.
