@@ -323,3 +323,22 @@ def test_k_above_one_device_scan(lib, name, params, search):
         idx.knn_search_batch(q, k, search)
     assert e.value.code == -3
     idx.close()
+
+
+@pytest.mark.parametrize("quant", ["fp32", "sq8"])
+def test_large_batch_equals_one_by_one(lib, quant):
+    """A batch large enough for the matrix-core path of the flat scan returns what single queries return."""
+    n, d, nq, k = 70000, 32, 600, 10
+    x = vectors(n, d, normalize=False)
+    q = vectors(nq, d, seed=165, normalize=False)
+    labels = np.arange(n, dtype=np.int64) + 5
+    idx = make("brute_force", d, "l2", base_quantization_type=quant)
+    assert idx.build(x, labels, n, d) == 0
+    ids, dists = idx.knn_search_batch(q, k, "{}")
+    for i in range(0, nq, 37):
+        si, sd = idx.knn_search(q[i], k, "{}")
+        assert np.array_equal(si, ids[i]) and np.array_equal(sd.view(np.uint32), dists[i].view(np.uint32)), i
+    if quant == "fp32":
+        gt, _ = ground_truth(x, q[:50], k, "l2")
+        assert recall(ids[:50], gt, labels) >= 0.999
+    idx.close()

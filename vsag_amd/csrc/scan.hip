@@ -822,7 +822,8 @@ vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, 
     carve_scan(c, cp, nq, k, &b);
     VA_CHECK_ARG(c.ok(), "workspace too small: need %zu bytes, got %zu", c.used, workspace_bytes);
     // A pre-filter or a radius goes the streaming way (the prefilter knows neither).
-    const bool contraction = cp.contraction && options == nullptr;
+    const bool plain = options == nullptr || (options->deny_bits_dev == nullptr && options->use_radius == 0);
+    const bool contraction = cp.contraction && plain;
     const ScanPlan& p = cp.all;
 
     VA_TRY(prepare_queries(s, queries_dev, nq, p.nq_pad, p.ql, b.qtab, b.qmeta, b.qcodes, st));
