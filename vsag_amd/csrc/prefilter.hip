@@ -30,24 +30,24 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 constexpr int PM = 128;  // codes per tile (two storage tiles)
 constexpr int PN = 128;  // queries per tile
 constexpr int PK = 32;   // contraction depth per stage
-constexpr int kPfPlane = PM;
+// Rows of a (parity, chunk) plane are PM float4; four more pad the plane so that the four chunks of one row
+// start sixteen banks apart: a loader wave writes whole float4 slots of four rows x four chunks (or of 64
+// consecutive rows of one chunk) without a bank conflict, and the MFMA lanes read 64 consecutive rows.
+constexpr int kPfPlane = PM + 4;
 
-// LDS operand layout of one stage: [parity h = k & 1][chunk c = (k >> 1) / 4][row] of float4, element e of the
-// float4 is k = 2 (4 c + e) + h, so that a lane of the MFMA (row = lane % 32, h = lane / 32) reads its operand
-// for four consecutive k-steps with one conflict-free ds_read_b128.
+// LDS operand layout of one stage: [parity h = k & 1][chunk c = k / 8][row] of float4, element e of the float4
+// is k = 8 c + 2 e + h, so that a lane of the MFMA (row = lane % 32, h = lane / 32) reads its operand for four
+// consecutive k-steps with one ds_read_b128.
 struct PfStage {
     float4 a[2 * 4 * kPfPlane];
     float4 b[2 * 4 * kPfPlane];
 };
 
-// Scatter four consecutive k (k = 4g .. 4g+3 of `row`) into the parity planes.
+// Eight consecutive k (k = 8c .. 8c+7 of `row`, lo = the first four) as the two float4 slots of chunk c.
 __device__ inline void
-pf_stage_store(float4* plane, uint32_t row, uint32_t g, float4 v) {
-    uint32_t c = g >> 1, e = (g & 1) * 2;
-    float* even = reinterpret_cast<float*>(&plane[(0 * 4 + c) * kPfPlane + row]) + e;
-    float* odd = reinterpret_cast<float*>(&plane[(1 * 4 + c) * kPfPlane + row]) + e;
-    *reinterpret_cast<float2*>(even) = make_float2(v.x, v.z);
-    *reinterpret_cast<float2*>(odd) = make_float2(v.y, v.w);
+pf_stage_store8(float4* plane, uint32_t row, uint32_t c, float4 lo, float4 hi) {
+    plane[(0 * 4 + c) * kPfPlane + row] = make_float4(lo.x, lo.z, hi.x, hi.z);
+    plane[(1 * 4 + c) * kPfPlane + row] = make_float4(lo.y, lo.w, hi.y, hi.w);
 }
 
 struct PrefilterArgs {
@@ -98,13 +98,14 @@ prefilter_kernel(PrefilterArgs p) {
     const uint64_t span = p.tile_end - p.tile_begin;
     const uint64_t mtiles = (span + 1) / 2;
 
-    // Query loader roles: 1024 float4 per stage, four per thread (row = idx / 8, chunk = idx % 8).
-    uint32_t qrow[4], qg[4];
+    // Query loader roles: 512 (row, chunk) pairs of eight floats per stage, two per thread; four lanes cover the
+    // 128 contiguous bytes of a row.
+    uint32_t qrow[2], qc[2];
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
+    for (int r = 0; r < 2; ++r) {
         uint32_t idx = tid + 256 * r;
-        qrow[r] = idx >> 3;
-        qg[r] = idx & 7;
+        qrow[r] = idx >> 2;
+        qc[r] = idx & 3;
     }
     float tau_n[2];
 #pragma unroll
@@ -123,42 +124,47 @@ prefilter_kernel(PrefilterArgs p) {
         }
         return make_uint4(0, 0, 0, 0);
     };
-    // sq8: a stage is 32 dimensions = granules 2 kt and 2 kt + 1, one per thread.
-    // fp32: a stage is 32 dimensions = granules 8 kt .. 8 kt + 7, four per thread (cpart, cpart + 2, ...).
+    // sq8: a stage is 32 dimensions = granules 2 kt and 2 kt + 1, one per thread (chunks 2 cpart, 2 cpart + 1).
+    // fp32: a stage is 32 dimensions = granules 8 kt .. 8 kt + 7; a thread takes chunks cpart and cpart + 2, two
+    // granules each.
     constexpr int kCodeRegs = KIND == VSAG_AMD_KIND_SQ8 ? 1 : 4;
     auto fetch_codes = [&](uint64_t mt, uint32_t kt, uint4 (&regs)[kCodeRegs]) {
         if constexpr (KIND == VSAG_AMD_KIND_SQ8) {
             regs[0] = code_granule(mt, 2 * kt + cpart);
         } else {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                regs[r] = code_granule(mt, 8 * kt + cpart + 2 * r);
+            for (int r = 0; r < 2; ++r) {
+                regs[2 * r] = code_granule(mt, 8 * kt + 2 * (cpart + 2 * r));
+                regs[2 * r + 1] = code_granule(mt, 8 * kt + 2 * (cpart + 2 * r) + 1);
             }
         }
+    };
+    auto as_floats = [](uint4 v) {
+        return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
     };
     auto park_codes = [&](float4* plane, uint32_t kt, const uint4 (&regs)[kCodeRegs]) {
         if constexpr (KIND == VSAG_AMD_KIND_SQ8) {
             const uint32_t w[4] = {regs[0].x, regs[0].y, regs[0].z, regs[0].w};
             const uint32_t d0 = PK * kt + 16 * cpart;
+            float4 v[4];
 #pragma unroll
             for (int m = 0; m < 4; ++m) {
-                float4 v = make_float4(static_cast<float>(w[m] & 0xffU), static_cast<float>((w[m] >> 8) & 0xffU),
-                                       static_cast<float>((w[m] >> 16) & 0xffU), static_cast<float>(w[m] >> 24));
+                v[m] = make_float4(static_cast<float>(w[m] & 0xffU), static_cast<float>((w[m] >> 8) & 0xffU),
+                                   static_cast<float>((w[m] >> 16) & 0xffU), static_cast<float>(w[m] >> 24));
                 if (p.scale != nullptr && d0 + 16 <= p.kdim) {
                     float4 sc = *reinterpret_cast<const float4*>(p.scale + d0 + 4 * m);
-                    v.x *= sc.x;
-                    v.y *= sc.y;
-                    v.z *= sc.z;
-                    v.w *= sc.w;
+                    v[m].x *= sc.x;
+                    v[m].y *= sc.y;
+                    v[m].z *= sc.z;
+                    v[m].w *= sc.w;
                 }
-                pf_stage_store(plane, crow, 4 * cpart + m, v);
             }
+            pf_stage_store8(plane, crow, 2 * cpart, v[0], v[1]);
+            pf_stage_store8(plane, crow, 2 * cpart + 1, v[2], v[3]);
         } else {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                float4 v = make_float4(__uint_as_float(regs[r].x), __uint_as_float(regs[r].y),
-                                       __uint_as_float(regs[r].z), __uint_as_float(regs[r].w));
-                pf_stage_store(plane, crow, cpart + 2 * r, v);
+            for (int r = 0; r < 2; ++r) {
+                pf_stage_store8(plane, crow, cpart + 2 * r, as_floats(regs[2 * r]), as_floats(regs[2 * r + 1]));
             }
         }
     };
@@ -167,13 +173,22 @@ prefilter_kernel(PrefilterArgs p) {
     // stage of the current tile is multiplied, so that no tile starts by waiting for memory.
     uint4 rc[kCodeRegs];
     float4 rq[4];
-    float my_term = 0.0F;
+    auto fetch_queries = [&](uint32_t kt) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            rq[2 * r] = pf_query_chunk(p.qtab, q0 + qrow[r], p.nq, PK * kt + 8 * qc[r], p.qstride);
+            rq[2 * r + 1] = pf_query_chunk(p.qtab, q0 + qrow[r], p.nq, PK * kt + 8 * qc[r] + 4, p.qstride);
+        }
+    };
+    auto park_queries = [&](float4* plane) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            pf_stage_store8(plane, qrow[r], qc[r], rq[2 * r], rq[2 * r + 1]);
+        }
+    };
     auto fetch_stage0 = [&](uint64_t mt) {
         fetch_codes(mt, 0, rc);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            rq[r] = pf_query_chunk(p.qtab, q0 + qrow[r], p.nq, 4 * qg[r], p.qstride);
-        }
+        fetch_queries(0);
     };
     if (blockIdx.x < mtiles) {
         fetch_stage0(blockIdx.x);
@@ -193,10 +208,7 @@ prefilter_kernel(PrefilterArgs p) {
         const uint64_t slot0 = (p.tile_begin + 2 * mt) * kWave;
         // The stage is free: the previous tile's contraction ended with a barrier.
         park_codes(stage[0].a, 0, rc);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            pf_stage_store(stage[0].b, qrow[r], qg[r], rq[r]);
-        }
+        park_queries(stage[0].b);
         if (tid < PM) {
             uint64_t slot = slot0 + tid;
             bool real = slot < p.n && p.tile_begin + 2 * mt + (tid >> 6) < p.tile_end;
@@ -206,10 +218,7 @@ prefilter_kernel(PrefilterArgs p) {
         for (uint32_t kt = 0; kt < ktiles; ++kt) {
             if (kt + 1 < ktiles) {
                 fetch_codes(mt, kt + 1, rc);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    rq[r] = pf_query_chunk(p.qtab, q0 + qrow[r], p.nq, PK * (kt + 1) + 4 * qg[r], p.qstride);
-                }
+                fetch_queries(kt + 1);
             } else if (mt + p.groups < mtiles) {
                 fetch_stage0(mt + p.groups);
             }
@@ -236,10 +245,7 @@ prefilter_kernel(PrefilterArgs p) {
             __syncthreads();  // every wave has read the stage
             if (kt + 1 < ktiles) {
                 park_codes(stage[0].a, kt + 1, rc);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    pf_stage_store(stage[0].b, qrow[r], qg[r], rq[r]);
-                }
+                park_queries(stage[0].b);
                 __syncthreads();
             }
         }
