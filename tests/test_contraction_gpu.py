@@ -69,6 +69,28 @@ def test_fp32_contraction_equals_streaming(lib, modes, metric, n, d, nq, k):
     st.destroy()
 
 
+@pytest.mark.parametrize("kind", ["fp32", "sq8"])
+def test_many_short_tiles_per_workgroup(lib, modes, kind):
+    """100000 x 128 against 1000 queries: every workgroup walks many code tiles with a short contraction each, so
+    the epilogue of one tile runs next to the start of the following one."""
+    rng = np.random.default_rng(77)
+    n, d, nq, k = 100000, 128, 1000, 10
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    q = rng.standard_normal((nq, d)).astype(np.float32)
+    if kind == "fp32":
+        st = Store(capi.KIND_FP32, orc.L2, d)
+        st.append(x.view(np.uint8).reshape(n, 4 * d))
+    else:
+        lb, diff = orc.sq_train(x, 8, orc.L2)
+        st = Store(capi.KIND_SQ8, orc.L2, d, lb=lb, diff=diff)
+        st.append(orc.sq_encode(x, 8, lb, diff, orc.L2))
+    for _ in range(3):
+        plain, fast, tile = modes(st, q, k)
+        assert tile == 128
+        assert same(plain, fast)
+    st.destroy()
+
+
 def test_contraction_overflow_falls_back_to_streaming(lib, modes):
     """Thousands of equal distances per query: the candidate buffers overflow, the streaming kernel serves the query."""
     rng = np.random.default_rng(8)

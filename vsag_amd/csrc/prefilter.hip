@@ -209,12 +209,13 @@ prefilter_kernel(PrefilterArgs p) {
         // The stage is free: the previous tile's contraction ended with a barrier.
         park_codes(stage[0].a, 0, rc);
         park_queries(stage[0].b);
+        float my_term = 0.0F;  // parked in LDS late: slower waves may still be reading the previous tile's terms
         if (tid < PM) {
             uint64_t slot = slot0 + tid;
             bool real = slot < p.n && p.tile_begin + 2 * mt + (tid >> 6) < p.tile_end;
-            code_term[tid] = real ? p.term_factor * p.term[slot] : __builtin_inff();
+            my_term = real ? p.term_factor * p.term[slot] : __builtin_inff();
         }
-        __syncthreads();  // also: every wave has left the previous epilogue (code_term)
+        __syncthreads();
         for (uint32_t kt = 0; kt < ktiles; ++kt) {
             if (kt + 1 < ktiles) {
                 fetch_codes(mt, kt + 1, rc);
@@ -241,6 +242,10 @@ prefilter_kernel(PrefilterArgs p) {
                     acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[e], bv0[e], acc[1][0], 0, 0, 0);
                     acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[e], bv1[e], acc[1][1], 0, 0, 0);
                 }
+            }
+            if (kt + 1 == ktiles && tid < PM) {
+                // Every wave is past this tile's first barrier, hence out of the previous tile's epilogue.
+                code_term[tid] = my_term;
             }
             __syncthreads();  // every wave has read the stage
             if (kt + 1 < ktiles) {
