@@ -196,9 +196,11 @@ VSAG_AMD_API int vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* store, const
 
 /* Large batches on flat fp32 / sq8 stores are served by a matrix-core contraction that pre-selects candidates,
  * which are then recomputed and selected exactly as the streaming scan does (same results, bit for bit).
+ * sq8 stores of at most 128 dimensions pre-select on the int8 matrix cores (queries split into two int8 planes
+ * with a rigorous bound on the remainder), the others on the fp32 matrix cores.
  * mode: 0 = when it pays (default: >= 512 queries, k <= 128, >= 65536 codes), 1 = whenever the store and k
- * allow it, -1 = never.  Process-wide; affects vsag_amd_flat_scan_workspace_bytes as well.  No counterpart in the
- * reference (it scans one query at a time). */
+ * allow it, 2 = like 1 but always on the fp32 matrix cores, -1 = never.  Process-wide; affects
+ * vsag_amd_flat_scan_workspace_bytes as well.  No counterpart in the reference (it scans one query at a time). */
 VSAG_AMD_API int vsag_amd_set_scan_contraction(int mode);
 
 /* Tuning knobs of the scan (query tile T in {1,2,4,8}, 0 = automatic; number of base chunks, 0 =

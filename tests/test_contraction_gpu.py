@@ -15,10 +15,10 @@ pytestmark = pytest.mark.gpu
 def modes(lib):
     L = capi.load_library()
 
-    def both(store, q, k):
+    def both(store, q, k, mode=1):
         capi.check(L.vsag_amd_set_scan_contraction(-1))
         plain = store.flat_scan(q, k)
-        capi.check(L.vsag_amd_set_scan_contraction(1))
+        capi.check(L.vsag_amd_set_scan_contraction(mode))
         fast = store.flat_scan(q, k)
         tile = capi.C.c_int()
         L.vsag_amd_last_scan_info(capi.C.byref(tile), None, None)
@@ -44,11 +44,43 @@ def test_sq8_contraction_equals_streaming(lib, modes, metric, n, d, nq, k):
     st = Store(capi.KIND_SQ8, metric, d, lb=lb, diff=diff)
     st.append(codes[:n // 3])
     st.append(codes[n // 3:])  # the per-code terms follow appends
-    plain, fast, tile = modes(st, q, k)
-    assert tile == 128, "the contraction path did not run"
-    assert same(plain, fast)
+    # mode 1: the int8 matrix cores up to 128 dimensions (256 queries per pass); mode 2: always the fp32 ones
+    for mode, tile_expected in ((1, 256 if d <= 128 else 128), (2, 128)):
+        plain, fast, tile = modes(st, q, k, mode)
+        assert tile == tile_expected, "the contraction path did not run"
+        assert same(plain, fast)
     ri, rd = orc.flat_scan_topk(orc.SQ8, metric, d, codes, q[:16], k, lb=lb, diff=diff)
     assert_topk_close(fast[0][:16], fast[1][:16], ri, rd, label="sq8 contraction")
+    st.destroy()
+
+
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
+@pytest.mark.parametrize("d", [16, 100, 128])
+def test_sq8_int8_planes_hold_for_awkward_queries(lib, modes, metric, d):
+    """Queries the two int8 planes represent badly or trivially: one dominant dimension, tiny and huge magnitudes,
+    all zeros, copies of stored vectors, far outside the trained range."""
+    rng = np.random.default_rng(1000 + d + metric)
+    n, nq, k = 30000, 320, 10
+    x, means = gaussian_mixture(rng, n, d, 20, 0.05)
+    q, _ = gaussian_mixture(rng, nq, d, 20, 0.05, means=means)
+    if metric != orc.COSINE:  # no direction to normalise
+        q[0] = 0.0
+        q[1] = 1e-20
+    q[2] *= 1e6
+    q[3] *= 1e-6
+    q[4] = 0.0
+    q[4, d // 2] = 1e4
+    q[5:40] = x[5:40]          # duplicates of stored vectors
+    q[40:60] = -q[40:60]
+    q[60:80] += 100.0          # far outside [lb, lb + diff]
+    q[80, :] = np.where(np.arange(d) % 2 == 0, 1e-3, 1e3)
+    lb, diff = orc.sq_train(x, 8, metric)
+    codes = orc.sq_encode(x, 8, lb, diff, metric)
+    st = Store(capi.KIND_SQ8, metric, d, lb=lb, diff=diff)
+    st.append(codes)
+    plain, fast, tile = modes(st, q, k)
+    assert tile == 256
+    assert same(plain, fast)
     st.destroy()
 
 
@@ -86,7 +118,7 @@ def test_many_short_tiles_per_workgroup(lib, modes, kind):
         st.append(orc.sq_encode(x, 8, lb, diff, orc.L2))
     for _ in range(3):
         plain, fast, tile = modes(st, q, k)
-        assert tile == 128
+        assert tile == (128 if kind == "fp32" else 256)
         assert same(plain, fast)
     st.destroy()
 
@@ -101,9 +133,10 @@ def test_contraction_overflow_falls_back_to_streaming(lib, modes):
     q = rng.random((nq, d), dtype=np.float32)
     st = Store(capi.KIND_SQ8, orc.L2, d, lb=lb, diff=diff)
     st.append(codes)
-    plain, fast, tile = modes(st, q, k)
-    assert tile == 128
-    assert same(plain, fast)
+    for mode, tile_expected in ((1, 256), (2, 128)):
+        plain, fast, tile = modes(st, q, k, mode)
+        assert tile == tile_expected
+        assert same(plain, fast)
     ri, rd = orc.flat_scan_topk(orc.SQ8, orc.L2, d, codes, q[:8], k, lb=lb, diff=diff)
     # which of the equal distances the checker keeps is its heap's business; the distances must agree
     np.testing.assert_allclose(fast[1][:8], rd, rtol=1e-5)

@@ -292,7 +292,8 @@ __global__ void __launch_bounds__(256)
 code_term_kernel(const uint4* tiles, uint32_t G, const float* scale, uint64_t first, uint64_t count, float* term,
                  uint32_t* ymax_bits) {
     uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    float s = 0.0F;
+    // Summed in double and rounded once: the int8 prefilter budgets two fp32 roundoffs for this term.
+    double s = 0.0;
     if (i < count) {
         uint64_t slot = first + i;
         uint64_t tile = slot >> 6;
@@ -303,23 +304,23 @@ code_term_kernel(const uint4* tiles, uint32_t G, const float* scale, uint64_t fi
             if constexpr (KIND == VSAG_AMD_KIND_SQ8) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    float y = static_cast<float>((w[e >> 2] >> (8 * (e & 3))) & 0xffU);
+                    double y = static_cast<double>((w[e >> 2] >> (8 * (e & 3))) & 0xffU);
                     if (scale != nullptr) {
-                        y *= scale[16 * j + e];
+                        y *= static_cast<double>(scale[16 * j + e]);
                     }
-                    s = fmaf(y, y, s);
+                    s = fma(y, y, s);
                 }
             } else {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    float y = __uint_as_float(w[e]);
-                    s = fmaf(y, y, s);
+                    double y = static_cast<double>(__uint_as_float(w[e]));
+                    s = fma(y, y, s);
                 }
             }
         }
-        term[slot] = s;
+        term[slot] = static_cast<float>(s);
     }
-    float m = sqrtf(s);
+    float m = static_cast<float>(sqrt(s)) * (1.0F + 2.0e-7F);
     for (int off = 32; off > 0; off >>= 1) {
         float o = __shfl_xor(m, off);
         m = o > m ? o : m;
@@ -376,7 +377,12 @@ struct RescoreArgs {
     uint32_t nslots;
     uint32_t out_slot;
     uint32_t* gate;  // per query: 1 = candidates overflowed, the streaming kernel must serve the query
+    // sub_lists != 0: the candidates of a query sit in sub_lists lists of sub_cap slots with a count each (a count
+    // above sub_cap = that list overflowed); they are gathered into LDS first (at most kRescoreGather of them).
+    uint32_t sub_lists, sub_cap;
 };
+
+constexpr uint32_t kRescoreGather = 4096;
 
 // One wave per query: exact distances of its candidates by the streaming kernel's arithmetic, best k kept.
 template <int KIND, int METRIC>
@@ -385,9 +391,40 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
     extern __shared__ uint64_t keys[];
     const uint32_t lane = threadIdx.x;
     const uint32_t q = blockIdx.x;
-    const uint32_t total = as_const(r.cand_cnt)[q];
     const uint64_t list = static_cast<uint64_t>(q) * r.nslots + r.out_slot;
-    if (total > r.cap) {
+    uint32_t total = 0;
+    bool overflow = false;
+    const uint32_t* mine = r.cand + static_cast<uint64_t>(q) * r.cap;
+    if (r.sub_lists == 0) {
+        total = as_const(r.cand_cnt)[q];
+        overflow = total > r.cap;
+    } else {
+        // Gather the private lists of the query behind the selector: a lane per list, offsets by a wave scan.
+        uint32_t* flat = reinterpret_cast<uint32_t*>(keys + r.S);
+        const uint32_t* counts = r.cand_cnt + static_cast<uint64_t>(q) * r.sub_lists;
+        const uint32_t* lists = r.cand + static_cast<uint64_t>(q) * r.sub_lists * r.sub_cap;
+        for (uint32_t g0 = 0; g0 < r.sub_lists && !overflow; g0 += kWave) {
+            const uint32_t g = g0 + lane;
+            const uint32_t c = g < r.sub_lists ? as_const(counts)[g] : 0U;
+            uint32_t incl = c;
+            for (int off = 1; off < 64; off <<= 1) {
+                uint32_t o = __shfl_up(incl, off);
+                incl += lane >= static_cast<uint32_t>(off) ? o : 0U;
+            }
+            const uint32_t sum = __shfl(incl, 63);
+            overflow = __ballot(c > r.sub_cap) != 0 || total + sum > kRescoreGather;
+            if (!overflow) {
+                const uint32_t at = total + incl - c;
+                for (uint32_t i = 0; i < c; ++i) {
+                    flat[at + i] = as_const(lists)[static_cast<uint64_t>(g) * r.sub_cap + i];
+                }
+                total += sum;
+            }
+        }
+        wave_lds_fence();
+        mine = flat;
+    }
+    if (overflow) {
         if (lane == 0) {
             r.gate[q] = 1;
             r.partial_cnt[list] = 0;
@@ -405,7 +442,6 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
     uint64_t tau = (static_cast<uint64_t>(bs) << 32) | 0xFFFFFFFFULL;
     const uint32_t qidx[1] = {q};
     const QueryRows<1> qrows = query_rows<1>(a, qidx);
-    const uint32_t* mine = r.cand + static_cast<uint64_t>(q) * r.cap;
     for (uint32_t base = 0; base < total; base += kWave) {
         const bool have = base + lane < total;
         const uint32_t slot = have ? mine[base + lane] : 0U;
@@ -491,15 +527,62 @@ launch_rescore_m(int metric, dim3 grid, size_t lds, hipStream_t st, const ScanAr
     }
 }
 
+int launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride, const float* qmeta,
+                        uint32_t qmeta_stride, uint64_t nq, uint64_t tile_begin, uint64_t tile_end,
+                        const uint32_t* bound, uint8_t* q8, float* u, uint32_t* tau, uint32_t* cand, uint32_t* cand_cnt,
+                        uint32_t sub_lists, uint32_t sub_cap, hipStream_t st);
+
+// Step 3 of the header comment: exact distances of the collected candidates.
+static int
+launch_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t k, uint32_t S, uint32_t* bound,
+               const uint32_t* cand, const uint32_t* cand_cnt, uint32_t cap, uint32_t sub_lists, uint32_t sub_cap,
+               uint64_t* partial, uint32_t* partial_cnt, uint32_t nslots, uint32_t out_slot, uint32_t* gate,
+               hipStream_t st) {
+    const bool sq8 = s->kind == VSAG_AMD_KIND_SQ8;
+    RescoreArgs r{};
+    r.cand = cand;
+    r.cand_cnt = cand_cnt;
+    r.cap = cap;
+    r.n = s->n;
+    r.k = k;
+    r.S = S;
+    r.bound = bound;
+    r.partial = partial;
+    r.partial_cnt = partial_cnt;
+    r.nslots = nslots;
+    r.out_slot = out_slot;
+    r.gate = gate;
+    r.sub_lists = sub_lists;
+    r.sub_cap = sub_cap;
+    dim3 rgrid(static_cast<uint32_t>(nq));
+    const size_t lds = S * 8 + (sub_lists != 0 ? kRescoreGather * 4 : 0);
+    if (sq8) {
+        launch_rescore_m<VSAG_AMD_KIND_SQ8>(s->metric, rgrid, lds, st, a, r);
+    } else {
+        launch_rescore_m<VSAG_AMD_KIND_FP32>(s->metric, rgrid, lds, st, a, r);
+    }
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
+
 // Steps 2 and 3 of the header comment for tiles [tile_begin, tile_end); the exact prefix scan has already
 // left its bounds in `bound`.  Writes one partial list per query (out_slot) and the overflow flags.
 int
 launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t k, uint32_t S, uint64_t tile_begin,
                  uint64_t tile_end, uint32_t* bound, float* tau, uint32_t* cand, uint32_t* cand_cnt, uint32_t cap,
                  uint64_t* partial, uint32_t* partial_cnt, uint32_t nslots, uint32_t out_slot, uint32_t* gate,
-                 hipStream_t st) {
+                 uint8_t* q8, float* q8_u, uint32_t sub_lists, uint32_t sub_cap, hipStream_t st) {
     const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
     const bool sq8 = s->kind == VSAG_AMD_KIND_SQ8;
+    if (q8 != nullptr) {
+        // At most 128 dimensions of sq8: the int8 matrix cores pre-select (prefilter_i8.hip).
+        VA_TRY(launch_prefilter_i8(s, reinterpret_cast<const float*>(a.qtab), a.qstride, a.qmeta, a.qmeta_stride, nq,
+                                   tile_begin, tile_end, bound, q8, q8_u, reinterpret_cast<uint32_t*>(tau), cand,
+                                   cand_cnt, sub_lists, sub_cap, st));
+        return launch_rescore(s, a, nq, k, S, bound, cand, cand_cnt, 0, sub_lists, sub_cap, partial, partial_cnt, nslots,
+                              out_slot, gate, st);
+    }
     hipLaunchKernelGGL(prefilter_tau_kernel, dim3(static_cast<uint32_t>(nq)), dim3(kWave), 0, st,
                        reinterpret_cast<const float*>(a.qtab), a.qstride, s->dpad, sq8 && !l2 ? a.qmeta : nullptr,
                        a.qmeta_stride, l2 ? 1 : 0, bound, s->pf_ymax, nq, tau);
@@ -537,27 +620,8 @@ launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32
     }
     timing_end(st);
     VA_HIP(hipGetLastError());
-    RescoreArgs r{};
-    r.cand = cand;
-    r.cand_cnt = cand_cnt;
-    r.cap = cap;
-    r.n = s->n;
-    r.k = k;
-    r.S = S;
-    r.bound = bound;
-    r.partial = partial;
-    r.partial_cnt = partial_cnt;
-    r.nslots = nslots;
-    r.out_slot = out_slot;
-    r.gate = gate;
-    dim3 rgrid(static_cast<uint32_t>(nq));
-    if (sq8) {
-        launch_rescore_m<VSAG_AMD_KIND_SQ8>(s->metric, rgrid, S * 8, st, a, r);
-    } else {
-        launch_rescore_m<VSAG_AMD_KIND_FP32>(s->metric, rgrid, S * 8, st, a, r);
-    }
-    VA_HIP(hipGetLastError());
-    return 0;
+    return launch_rescore(s, a, nq, k, S, bound, cand, cand_cnt, cap, 0, 0, partial, partial_cnt, nslots, out_slot, gate,
+                          st);
 }
 
 }  // namespace vsag_amd

@@ -1,0 +1,450 @@
+// Pre-selection for large query batches on a flat sq8 store of at most 128 dimensions, on the int8 matrix cores.
+//
+// The streaming distance of an sq8 code is a function of <b, c>: c the code bytes (0..255), b the query folded
+// with the per-dimension scale (l2: b_d = (q_d - lb_d) scale_d, ip: b_d = q_d scale_d).  Each query row b is split
+// once, in double precision, into two int8 planes and a remainder,
+//
+//      b_d = s2 (256 h_d + l_d) + e_d,      h_d, l_d in [-128, 127],   s2 = max|b| / (127 * 256),
+//
+// so that <b, c> = s2 (256 <h, c> + <l, c>) + <e, c>.  The two integer products come out of
+// v_mfma_i32_32x32x32_i8 exactly; the remainder is bounded rigorously per query by 255 max(sum of positive e_d,
+// sum of negative e_d), because every c_d lies in [0, 255].  The matrix cores take signed bytes: the staged codes
+// are c_d - 128 (one xor per word), and 128 sum_d (256 h_d + l_d) moves into the per-query threshold.
+//
+// A (query, code) pair is kept when its distance, lowered by every error term (the remainder above, the rounding
+// of the streaming kernel's own fp32 arithmetic, the rounding of the per-code |y|^2 and of the test itself), does
+// not exceed the query's bound.  The kept pairs are rescored exactly (rescore_kernel, prefilter.hip), so the
+// result equals the streaming scan's bit for bit.
+//
+// Work split: a workgroup is four waves; each wave keeps the operands of 64 queries (both planes, 64 registers)
+// for the whole kernel and meets every 64-code storage tile the workgroup walks, which is staged in LDS in the
+// tile's own granule-major order -- that order is the operand order of the matrix instruction (lane % 32 = code,
+// lane / 32 = which 16 of the 32 dimensions of a step), so staging is a plain copy.
+#include "store.h"
+#include "topk.h"
+
+namespace vsag_amd {
+
+void timing_begin(hipStream_t st);
+void timing_end(hipStream_t st);
+
+typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef int intx16 __attribute__((ext_vector_type(16)));
+
+constexpr uint32_t kI8Dims = 128;       // dimensions the kernel covers (eight granules, four matrix steps)
+constexpr uint32_t kI8QueryBytes = 256;  // two planes of 128 bytes per query
+constexpr uint32_t kI8Group = 256;       // queries per workgroup
+
+struct QuantizeArgs {
+    const float* qtab;  // processed queries (distance.h): l2 q - lb, ip q * scale; zero beyond the dimension
+    uint32_t qstride;
+    uint32_t kdim;        // <= 128
+    const float* scale;   // l2: per-dimension scale folded into b; ip: null
+    const float* qmeta;   // ip: sum q_d lb_d per query
+    uint32_t qmeta_stride;
+    int is_l2;
+    const uint32_t* bound;      // per query, ordered-float bits; 0xFFFFFFFF = none yet
+    const uint32_t* ymax_bits;  // largest |y| of the store (l2: scaled codes, ip: raw codes)
+    uint64_t nq, nq_pad;
+    uint8_t* q8;     // nq_pad x 256 bytes
+    float* u;        // l2: -2 s2
+    uint32_t* tau;   // l2: float bits of the threshold on |y|^2 + u T; ip: smallest T that passes (int32)
+};
+
+__device__ inline double
+wave_sum_f64(double v) {
+    for (int off = 32; off > 0; off >>= 1) {
+        v += __shfl_xor(v, off);
+    }
+    return v;
+}
+
+__device__ inline double
+wave_max_f64(double v) {
+    for (int off = 32; off > 0; off >>= 1) {
+        double o = __shfl_xor(v, off);
+        v = o > v ? o : v;
+    }
+    return v;
+}
+
+// One wave per query; lane l owns dimensions l and l + 64.
+__global__ void __launch_bounds__(64)
+quantize_queries_i8_kernel(QuantizeArgs p) {
+    const uint64_t q = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    uint8_t* out = p.q8 + q * kI8QueryBytes;
+    if (q >= p.nq) {
+        // Padding rows: zero operands and a threshold nothing meets.
+        out[lane] = 0;
+        out[64 + lane] = 0;
+        out[128 + lane] = 0;
+        out[192 + lane] = 0;
+        if (lane == 0) {
+            p.u[q] = 0.0F;
+            p.tau[q] = p.is_l2 ? __float_as_uint(-__builtin_inff()) : 0x7FFFFFFFU;
+        }
+        return;
+    }
+    const float* row = p.qtab + q * p.qstride;
+    double a[2], b[2];
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+        const uint32_t d = lane + 64 * r;
+        a[r] = d < p.kdim ? static_cast<double>(row[d]) : 0.0;
+        // The product of two floats is exact in double.
+        b[r] = p.scale != nullptr && d < p.kdim ? a[r] * static_cast<double>(p.scale[d]) : a[r];
+    }
+    const double amax = wave_max_f64(fmax(fabs(b[0]), fabs(b[1])));
+    const double s1 = amax / 127.0;
+    const double s2 = s1 / 256.0;
+    double e_pos = 0.0, e_neg = 0.0, w = 0.0;
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+        double h = 0.0, l = 0.0;
+        if (amax > 0.0) {
+            h = fmin(fmax(rint(b[r] / s1), -127.0), 127.0);
+            l = fmin(fmax(rint((b[r] - s1 * h) / s2), -128.0), 127.0);
+        }
+        const double whole = 256.0 * h + l;  // an integer below 2^16: exact
+        const double e = b[r] - s2 * whole;
+        e_pos += e > 0.0 ? e : 0.0;
+        e_neg += e < 0.0 ? -e : 0.0;
+        w += whole;
+        out[lane + 64 * r] = static_cast<uint8_t>(static_cast<int8_t>(h));
+        out[128 + lane + 64 * r] = static_cast<uint8_t>(static_cast<int8_t>(l));
+    }
+    e_pos = wave_sum_f64(e_pos);
+    e_neg = wave_sum_f64(e_neg);
+    w = wave_sum_f64(w);  // exact: integers
+    const double a2 = wave_sum_f64(a[0] * a[0] + a[1] * a[1]);
+    const double b1 = wave_sum_f64(fabs(b[0]) + fabs(b[1]));
+    if (lane != 0) {
+        return;
+    }
+    const uint32_t bbits = p.bound[q];
+    const float u = static_cast<float>(-2.0 * s2);
+    p.u[q] = u;
+    if (bbits == 0xFFFFFFFFU || !(b1 < 1.0e300) || !(a2 < 1.0e300)) {
+        // No bound yet, or a query with NaN / infinite entries: everything is a candidate (and the query will
+        // overflow into the streaming kernel).
+        p.tau[q] = p.is_l2 ? __float_as_uint(3.0e38F) : 0x80000000U;
+        return;
+    }
+    constexpr double kU = 5.9604644775390625e-8;  // 2^-24, the unit roundoff of fp32
+    const double bd = static_cast<double>(ordered_to_float(bbits));
+    const double ymax = static_cast<double>(__uint_as_float(*p.ymax_bits)) * (1.0 + 1.0e-6);
+    // |<e, c>| for any code, plus the rounding of the double arithmetic above.
+    const double q_err = 255.0 * fmax(e_pos, e_neg) + 1.0e-12 * 255.0 * b1;
+    if (p.is_l2) {
+        // The streaming kernel sums fl(fl(c s) - a)^2 in fp32: off from the real sum S by at most
+        // 2u sum |y - a| |y| + (n + 2) u S <= 2u sqrt(S) |y| + (n + 2) u S to first order; twice that is allowed for.
+        const double s_abs = fabs(bd);
+        const double e_stream = 4.0 * kU * sqrt(s_abs) * ymax + 2.0 * (p.kdim + 4) * kU * s_abs;
+        // |y|^2 per code is accumulated in double and rounded once.
+        const double e_term = 2.0 * kU * ymax * ymax;
+        // dist = a2 + |y|^2 - 2 s2 (T + 128 w) - 2 <e, c>, T the integer the matrix cores deliver.
+        const double t_real = bd - a2 + 256.0 * s2 * w + 2.0 * q_err + e_stream + e_term;
+        // The test itself runs in fp32: fl(T) u + |y|^2 in one fma against the rounded threshold.
+        const double reach = 2.0 * (255.0 + 129.0) * b1;  // bounds |2 s2 T|
+        const double slack = 4.0 * kU * (reach + ymax * ymax + fabs(t_real));
+        const double t = t_real + slack;
+        p.tau[q] = __float_as_uint(t < 3.0e38 ? static_cast<float>(t) : 3.0e38F);
+    } else {
+        // dist = 1 - (fl(sum c a) + qmeta): the fp32 sum is off by at most n u sum |c a|, the two closing
+        // operations by u of their results; twice that is allowed for.
+        const double qm = p.qmeta != nullptr ? static_cast<double>(p.qmeta[q * p.qmeta_stride]) : 0.0;
+        const double m = fmin(255.0 * b1, sqrt(a2) * ymax * (1.0 + 1.0e-6));
+        const double e_stream = 2.0 * (p.kdim + 2) * kU * m + 4.0 * kU * (m + fabs(qm) + 1.0 + fabs(bd));
+        // 1 - qm - s2 (T + 128 w) - <e, c> <= bd   <=>   T >= -(bd - 1 + qm + errors) / s2 - 128 w.
+        const double rhs = bd - 1.0 + qm + q_err + e_stream;
+        int32_t ti;
+        if (s2 > 0.0) {
+            const double x = floor(-rhs / s2 - 128.0 * w) - 2.0;
+            ti = x >= 2147483647.0 ? 0x7FFFFFFF : (x <= -2147483648.0 ? static_cast<int32_t>(0x80000000U)
+                                                                      : static_cast<int32_t>(x));
+        } else {
+            ti = rhs >= 0.0 ? static_cast<int32_t>(0x80000000U) : 0x7FFFFFFF;
+        }
+        p.tau[q] = static_cast<uint32_t>(ti);
+    }
+}
+
+struct PrefilterI8Args {
+    const uint4* tiles;
+    uint32_t G;
+    uint64_t tile_begin, tile_end;
+    uint64_t n;
+    const uint4* q8;      // [query][plane][granule]
+    uint64_t nq;
+    const float* term;    // per slot |y|^2 (l2)
+    const float* u;       // per query (l2)
+    const uint32_t* tau;  // per query
+    // Candidates go to private lists: list (group, lane / 32) of a query belongs to one lane of one wave for the
+    // whole kernel, so appending needs no atomic and nobody waits for one.
+    uint32_t* cand;       // [query][2 groups][sub_cap]
+    uint32_t* cand_cnt;   // [query][2 groups]; a count above sub_cap means the list overflowed
+    uint32_t sub_cap;
+    uint32_t groups;      // grid x; tile t of the span is walked by group t % groups
+};
+
+struct I8Stage {
+    uint4 codes[8 * kWave];  // granule-major, as in the store; bytes are c - 128
+    float term[kWave];
+};
+
+template <int METRIC>
+__global__ void __launch_bounds__(256, 2)
+prefilter_i8_kernel(PrefilterI8Args p) {
+    __shared__ I8Stage stage[2];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    const uint32_t wave = tid >> 6;
+    const uint32_t half = lane >> 5;
+    const uint32_t l32 = lane & 31;
+    const uint64_t q_base = (static_cast<uint64_t>(blockIdx.y) * 4 + wave) * kWave;
+    const bool active = q_base < p.nq;  // the query table is padded to whole workgroups
+    const uint64_t span = p.tile_end - p.tile_begin;
+
+    // Query operands: block j = queries q_base + 32 j + lane % 32; step s = dimensions 32 s + 16 (lane / 32) ...
+    intx4 qh[2][4], ql[2][4];
+    float uq[2];
+    uint32_t tau[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint64_t q = q_base + 32 * j + l32;
+        const uint4* rowp = p.q8 + q * (kI8QueryBytes / 16);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const uint4 hv = rowp[2 * s + half];
+            const uint4 lv = rowp[8 + 2 * s + half];
+            qh[j][s] = intx4{static_cast<int>(hv.x), static_cast<int>(hv.y), static_cast<int>(hv.z),
+                             static_cast<int>(hv.w)};
+            ql[j][s] = intx4{static_cast<int>(lv.x), static_cast<int>(lv.y), static_cast<int>(lv.z),
+                             static_cast<int>(lv.w)};
+        }
+        uq[j] = p.u[q];
+        tau[j] = p.tau[q];
+    }
+
+    uint32_t ncand[2] = {0, 0};
+    uint32_t* my_list[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint64_t q = q_base + 32 * j + l32;
+        my_list[j] = p.cand + ((q < p.nq ? q : 0) * 2 * p.groups + 2 * blockIdx.x + half) * p.sub_cap;
+    }
+
+    // Staging: wave w copies granules w and w + 4 of the tile, a lane per code.
+    uint4 regs[2];
+    float my_term = 0.0F;
+    auto fetch = [&](uint64_t t) {
+        const uint64_t tile = p.tile_begin + t;
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const uint32_t j = wave + 4 * r;
+            uint4 v = make_uint4(0x80808080U, 0x80808080U, 0x80808080U, 0x80808080U);
+            if (j < p.G) {
+                v = p.tiles[(tile * p.G + j) * kWave + lane];
+            }
+            regs[r] = make_uint4(v.x ^ 0x80808080U, v.y ^ 0x80808080U, v.z ^ 0x80808080U, v.w ^ 0x80808080U);
+        }
+        if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+            if (wave == 0) {
+                const uint64_t slot = tile * kWave + lane;
+                my_term = slot < p.n ? p.term[slot] : __builtin_inff();
+            }
+        }
+    };
+    auto park = [&](I8Stage& st) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            st.codes[(wave + 4 * r) * kWave + lane] = regs[r];
+        }
+        if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+            if (wave == 0) {
+                st.term[lane] = my_term;
+            }
+        }
+    };
+
+    uint64_t t = blockIdx.x;
+    if (t < span) {
+        fetch(t);
+        park(stage[0]);
+    }
+    __syncthreads();
+    uint32_t cur = 0;
+    for (; t < span; t += p.groups) {
+        const uint64_t tn = t + p.groups;
+        if (tn < span) {
+            fetch(tn);
+        }
+        if (active) {
+            const I8Stage& st = stage[cur];
+            const uint64_t slot0 = (p.tile_begin + t) * kWave;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                intx4 av[4];
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const uint4 c = st.codes[(2 * s + half) * kWave + 32 * i + l32];
+                    av[s] = intx4{static_cast<int>(c.x), static_cast<int>(c.y), static_cast<int>(c.z),
+                                  static_cast<int>(c.w)};
+                }
+                intx16 hi[2], lo[2];
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        hi[j][e] = 0;
+                        lo[j][e] = 0;
+                    }
+                }
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        hi[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s], qh[j][s], hi[j], 0, 0, 0);
+                        lo[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s], ql[j][s], lo[j], 0, 0, 0);
+                    }
+                }
+                // Element e of a lane is code 32 i + 8 (e / 4) + 4 (lane / 32) + e % 4 against query l32 of block j.
+                float tm[16];
+                if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const float4 v = *reinterpret_cast<const float4*>(&st.term[32 * i + 8 * g + 4 * half]);
+                        tm[4 * g] = v.x;
+                        tm[4 * g + 1] = v.y;
+                        tm[4 * g + 2] = v.z;
+                        tm[4 * g + 3] = v.w;
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    uint64_t hit[16];
+                    uint64_t any = 0;
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int32_t tt = (hi[j][e] << 8) + lo[j][e];
+                        bool pass;
+                        if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                            pass = fmaf(static_cast<float>(tt), uq[j], tm[e]) <= __uint_as_float(tau[j]);
+                        } else {
+                            pass = tt >= static_cast<int32_t>(tau[j]);
+                        }
+                        hit[e] = __ballot(pass);
+                        any |= hit[e];
+                    }
+                    if (any != 0) {
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) {
+                            if (hit[e] != 0 && ((hit[e] >> lane) & 1ULL) != 0) {
+                                const uint64_t slot = slot0 + 32 * i + 8 * (e >> 2) + 4 * half + (e & 3);
+                                if (slot < p.n) {
+                                    if (ncand[j] < p.sub_cap) {
+                                        my_list[j][ncand[j]] = static_cast<uint32_t>(slot);
+                                    }
+                                    ++ncand[j];
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        if (tn < span) {
+            park(stage[cur ^ 1]);
+        }
+        __syncthreads();  // the next stage is complete, and every wave is done with this one
+        cur ^= 1;
+    }
+    if (active) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint64_t q = q_base + 32 * j + l32;
+            if (q < p.nq) {
+                p.cand_cnt[q * 2 * p.groups + 2 * blockIdx.x + half] = ncand[j];
+            }
+        }
+    }
+}
+
+bool
+prefilter_i8_supports(const vsag_amd_store* s) {
+    return s->kind == VSAG_AMD_KIND_SQ8 && s->dpad <= kI8Dims && s->G <= 8;
+}
+
+// Bytes of the quantized query table for nq queries.
+size_t
+prefilter_i8_query_bytes(uint64_t nq) {
+    return static_cast<size_t>(div_up(nq, static_cast<uint64_t>(kI8Group)) * kI8Group) * kI8QueryBytes;
+}
+
+// Candidate lists per query (two per workgroup column) for nq queries over `span` tiles.
+uint32_t
+prefilter_i8_sub_lists(uint64_t nq, uint64_t span) {
+    const uint64_t qgroups = div_up(nq, static_cast<uint64_t>(kI8Group));
+    // Two workgroups fit a compute unit; three rounds of them even out the tail.
+    uint64_t groups = div_up(static_cast<uint64_t>(device_cu_count()) * 6, qgroups);
+    groups = std::max<uint64_t>(1, std::min<uint64_t>(groups, span));
+    return static_cast<uint32_t>(2 * groups);
+}
+
+// Quantizes the queries against their current bounds and collects the candidates of tiles [tile_begin, tile_end)
+// into sub_lists lists of sub_cap slots per query (sub_lists as prefilter_i8_sub_lists gives it).
+int
+launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride, const float* qmeta,
+                    uint32_t qmeta_stride, uint64_t nq, uint64_t tile_begin, uint64_t tile_end, const uint32_t* bound,
+                    uint8_t* q8, float* u, uint32_t* tau, uint32_t* cand, uint32_t* cand_cnt, uint32_t sub_lists,
+                    uint32_t sub_cap, hipStream_t st) {
+    const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
+    const uint64_t nq_pad = div_up(nq, static_cast<uint64_t>(kI8Group)) * kI8Group;
+    QuantizeArgs z{};
+    z.qtab = qtab;
+    z.qstride = qstride;
+    z.kdim = s->dpad;
+    z.scale = l2 ? s->scale_dev : nullptr;
+    z.qmeta = l2 ? nullptr : qmeta;
+    z.qmeta_stride = qmeta_stride;
+    z.is_l2 = l2 ? 1 : 0;
+    z.bound = bound;
+    z.ymax_bits = s->pf_ymax;
+    z.nq = nq;
+    z.nq_pad = nq_pad;
+    z.q8 = q8;
+    z.u = u;
+    z.tau = tau;
+    hipLaunchKernelGGL(quantize_queries_i8_kernel, dim3(static_cast<uint32_t>(nq_pad)), dim3(kWave), 0, st, z);
+    VA_HIP(hipGetLastError());
+
+    PrefilterI8Args p{};
+    p.tiles = s->tiles;
+    p.G = s->G;
+    p.tile_begin = tile_begin;
+    p.tile_end = tile_end;
+    p.n = s->n;
+    p.q8 = reinterpret_cast<const uint4*>(q8);
+    p.nq = nq;
+    p.term = s->pf_term;
+    p.u = u;
+    p.tau = tau;
+    p.cand = cand;
+    p.cand_cnt = cand_cnt;
+    p.sub_cap = sub_cap;
+    p.groups = sub_lists / 2;
+    VA_CHECK_ARG(sub_lists == prefilter_i8_sub_lists(nq, tile_end - tile_begin), "candidate lists do not match the grid");
+    dim3 grid(p.groups, static_cast<uint32_t>(nq_pad / kI8Group));
+    timing_begin(st);
+    if (l2) {
+        hipLaunchKernelGGL(prefilter_i8_kernel<VSAG_AMD_METRIC_L2>, grid, dim3(256), 0, st, p);
+    } else {
+        hipLaunchKernelGGL(prefilter_i8_kernel<VSAG_AMD_METRIC_IP>, grid, dim3(256), 0, st, p);
+    }
+    timing_end(st);
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
+}  // namespace vsag_amd

@@ -581,18 +581,25 @@ struct CallPlan {
     bool contraction = false;
     ScanPlan prefix, rest;
     uint64_t prefix_tiles = 0;
+    bool int8 = false;         // the int8 matrix cores pre-select (sq8, at most 128 dimensions)
     uint32_t cap = 0;          // candidates per query
+    uint32_t sub_lists = 0;    // int8: private candidate lists per query ...
+    uint32_t sub_cap = 0;      // ... of this many slots; cap = sub_lists * sub_cap
     uint32_t nslots = 0;       // partial lists per query
     bool any_seeded = false;
 };
 
-static int g_prefilter_mode = 0;  // -1 never, 0 when it pays, 1 whenever the store supports it
+// -1 never, 0 when it pays, 1 whenever the store supports it, 2 like 1 but on the fp32 matrix cores only
+static int g_prefilter_mode = 0;
 
 bool prefilter_supports(const vsag_amd_store* s);
 int launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t k, uint32_t S, uint64_t tile_begin,
                      uint64_t tile_end, uint32_t* bound, float* tau, uint32_t* cand, uint32_t* cand_cnt, uint32_t cap,
                      uint64_t* partial, uint32_t* partial_cnt, uint32_t nslots, uint32_t out_slot, uint32_t* gate,
-                     hipStream_t st);
+                     uint8_t* q8, float* q8_u, uint32_t sub_lists, uint32_t sub_cap, hipStream_t st);
+bool prefilter_i8_supports(const vsag_amd_store* s);
+size_t prefilter_i8_query_bytes(uint64_t nq);
+uint32_t prefilter_i8_sub_lists(uint64_t nq, uint64_t span);
 
 static void
 make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
@@ -623,8 +630,16 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
         return;
     }
     c->contraction = true;
+    c->int8 = g_prefilter_mode != 2 && prefilter_i8_supports(s);
     c->prefix_tiles = prefix;
     c->cap = static_cast<uint32_t>(cap);
+    if (c->int8) {
+        // The expected load of a list is an eighth of its share of the buffer; short lists get room for the tail
+        // of that distribution.
+        c->sub_lists = prefilter_i8_sub_lists(nq, s->ntiles - prefix);
+        c->sub_cap = std::max<uint32_t>(16, static_cast<uint32_t>(div_up(cap, static_cast<uint64_t>(c->sub_lists))));
+        c->cap = c->sub_lists * c->sub_cap;
+    }
     make_plan(s, nq, k, prefix, &c->prefix);
     make_plan(s, nq, k, s->ntiles - prefix, &c->rest);
     uint32_t pf_slots = static_cast<uint32_t>(c->prefix.chunks * c->prefix.waves + 1 + c->rest.chunks * c->rest.waves);
@@ -645,6 +660,8 @@ struct ScanBuffers {
     uint32_t* cand_cnt;
     uint32_t* gate;
     uint32_t* cand;
+    uint8_t* q8;   // int8 planes of the queries, null on the fp32 matrix cores
+    float* q8_u;
 };
 
 static size_t
@@ -660,8 +677,14 @@ carve_scan(Carver& c, const CallPlan& cp, uint64_t nq, uint32_t k, ScanBuffers* 
         b->seed = nullptr;
     }
     b->partial = c.take<uint64_t>(nq * cp.nslots * k);
-    b->tau = c.take<float>(cp.contraction ? nq : 0);
-    b->cand_cnt = c.take<uint32_t>(cp.contraction ? nq : 0);
+    const uint64_t nq_pad8 = prefilter_i8_query_bytes(nq) / 256;  // whole workgroups of the int8 prefilter
+    b->tau = c.take<float>(cp.contraction ? nq_pad8 : 0);
+    b->q8_u = c.take<float>(cp.int8 ? nq_pad8 : 0);
+    b->q8 = c.take<uint8_t>(cp.int8 ? prefilter_i8_query_bytes(nq) : 0);
+    if (!cp.int8) {
+        b->q8 = nullptr;
+    }
+    b->cand_cnt = c.take<uint32_t>(cp.contraction ? nq * std::max<uint32_t>(1, cp.sub_lists) : 0);
     b->gate = c.take<uint32_t>(cp.contraction ? nq : 0);
     b->cand = c.take<uint32_t>(cp.contraction ? nq * cp.cap : 0);
     return c.used;
@@ -856,11 +879,12 @@ vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, 
         hipLaunchKernelGGL(tighten_bound_kernel, dim3(static_cast<uint32_t>(div_up(nq, 256))), dim3(256), 0, st,
                            dists_dev, k, nq, b.bound);
         VA_TRY(launch_prefilter(s, a, nq, k, p.S, cp.prefix_tiles, s->ntiles, b.bound, b.tau, b.cand, b.cand_cnt, cp.cap,
-                                b.partial, b.partial_cnt, nslots, slots_prefix, b.gate, st));
+                                b.partial, b.partial_cnt, nslots, slots_prefix, b.gate, b.q8, b.q8_u, cp.sub_lists,
+                                cp.sub_cap, st));
         VA_TRY(run_streaming(s, cp.rest, a, b, nq, k, nullptr, cp.prefix_tiles, s->ntiles, slots_prefix + 1, nslots,
                              b.gate, st));
-        tl_last_tile = 128;  // queries per pass of the contraction
-        tl_last_passes = div_up(nq, 128);
+        tl_last_tile = cp.int8 ? 256 : 128;  // queries per pass of the contraction
+        tl_last_passes = div_up(nq, cp.int8 ? 256 : 128);
     }
     VA_TRY(launch_merge_partials(b.partial, b.partial_cnt, b.bound, nslots, nslots, k, p.S, nq, ids_dev, dists_dev, st));
     tl_last_bytes = s->ntiles * s->G * kWave * kGranule;
@@ -869,7 +893,8 @@ vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, 
 
 extern "C" int
 vsag_amd_set_scan_contraction(int mode) {
-    VA_CHECK_ARG(mode >= -1 && mode <= 1, "mode must be -1 (never), 0 (when it pays) or 1 (whenever supported)");
+    VA_CHECK_ARG(mode >= -1 && mode <= 2,
+                 "mode must be -1 (never), 0 (when it pays), 1 (whenever supported) or 2 (1 on the fp32 matrix cores)");
     g_prefilter_mode = mode;
     return 0;
 }
