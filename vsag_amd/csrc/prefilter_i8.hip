@@ -185,13 +185,33 @@ struct PrefilterI8Args {
     uint32_t* cand;       // [query][2 groups][sub_cap]
     uint32_t* cand_cnt;   // [query][2 groups]; a count above sub_cap means the list overflowed
     uint32_t sub_cap;
-    uint32_t groups;      // grid x; tile t of the span is walked by group t % groups
+    uint32_t groups;      // grid x; stage g of the span (kI8StageTiles tiles) is walked by group g % groups
 };
 
+constexpr int kI8StageTiles = 2;  // storage tiles per LDS stage (one barrier per stage)
+
 struct I8Stage {
-    uint4 codes[8 * kWave];  // granule-major, as in the store; bytes are c - 128
-    float term[kWave];
+    uint4 codes[kI8StageTiles][8 * kWave];  // granule-major, as in the store; bytes are c - 128
+    float term[kI8StageTiles][kWave];
 };
+
+// The sixteen verdicts of one 32 x 32 block for this lane's query; returns the lanes with any verdict set.
+template <int METRIC>
+__device__ inline uint64_t
+i8_verdicts(const intx16& hi, const intx16& lo, const float (&tm)[16], float uq, uint32_t tau, bool (&pass)[16]) {
+    uint64_t any = 0;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        const int32_t tt = (hi[e] << 8) + lo[e];
+        if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+            pass[e] = fmaf(static_cast<float>(tt), uq, tm[e]) <= __uint_as_float(tau);
+        } else {
+            pass[e] = tt >= static_cast<int32_t>(tau);
+        }
+        any |= __ballot(pass[e]);
+    }
+    return any;
+}
 
 template <int METRIC>
 __global__ void __launch_bounds__(256, 2)
@@ -205,11 +225,14 @@ prefilter_i8_kernel(PrefilterI8Args p) {
     const uint64_t q_base = (static_cast<uint64_t>(blockIdx.y) * 4 + wave) * kWave;
     const bool active = q_base < p.nq;  // the query table is padded to whole workgroups
     const uint64_t span = p.tile_end - p.tile_begin;
+    const uint64_t nstages = (span + kI8StageTiles - 1) / kI8StageTiles;
 
     // Query operands: block j = queries q_base + 32 j + lane % 32; step s = dimensions 32 s + 16 (lane / 32) ...
     intx4 qh[2][4], ql[2][4];
     float uq[2];
     uint32_t tau[2];
+    uint32_t ncand[2] = {0, 0};
+    uint32_t* my_list[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const uint64_t q = q_base + 32 * j + l32;
@@ -225,136 +248,141 @@ prefilter_i8_kernel(PrefilterI8Args p) {
         }
         uq[j] = p.u[q];
         tau[j] = p.tau[q];
-    }
-
-    uint32_t ncand[2] = {0, 0};
-    uint32_t* my_list[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const uint64_t q = q_base + 32 * j + l32;
         my_list[j] = p.cand + ((q < p.nq ? q : 0) * 2 * p.groups + 2 * blockIdx.x + half) * p.sub_cap;
     }
 
-    // Staging: wave w copies granules w and w + 4 of the tile, a lane per code.
-    uint4 regs[2];
-    float my_term = 0.0F;
-    auto fetch = [&](uint64_t t) {
-        const uint64_t tile = p.tile_begin + t;
+    // Staging: wave w copies granules w and w + 4 of each tile of the stage, a lane per code.
+    uint4 regs[kI8StageTiles][2];
+    float my_term[kI8StageTiles];
+    auto fetch = [&](uint64_t sg) {
 #pragma unroll
-        for (int r = 0; r < 2; ++r) {
-            const uint32_t j = wave + 4 * r;
-            uint4 v = make_uint4(0x80808080U, 0x80808080U, 0x80808080U, 0x80808080U);
-            if (j < p.G) {
-                v = p.tiles[(tile * p.G + j) * kWave + lane];
+        for (int tt = 0; tt < kI8StageTiles; ++tt) {
+            const uint64_t tile = p.tile_begin + sg * kI8StageTiles + tt;
+            const bool real = tile < p.tile_end;
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const uint32_t j = wave + 4 * r;
+                // Raw bytes; they turn into c - 128 when parked, so that nothing waits for the load here.
+                regs[tt][r] = make_uint4(0x80808080U, 0x80808080U, 0x80808080U, 0x80808080U);
+                if (real && j < p.G) {
+                    regs[tt][r] = p.tiles[(tile * p.G + j) * kWave + lane];
+                }
             }
-            regs[r] = make_uint4(v.x ^ 0x80808080U, v.y ^ 0x80808080U, v.z ^ 0x80808080U, v.w ^ 0x80808080U);
-        }
-        if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
-            if (wave == 0) {
-                const uint64_t slot = tile * kWave + lane;
-                my_term = slot < p.n ? p.term[slot] : __builtin_inff();
+            if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                my_term[tt] = 0.0F;
+                if (wave == 0) {
+                    const uint64_t slot = tile * kWave + lane;
+                    my_term[tt] = real && slot < p.n ? p.term[slot] : __builtin_inff();
+                }
             }
         }
     };
     auto park = [&](I8Stage& st) {
 #pragma unroll
-        for (int r = 0; r < 2; ++r) {
-            st.codes[(wave + 4 * r) * kWave + lane] = regs[r];
-        }
-        if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
-            if (wave == 0) {
-                st.term[lane] = my_term;
+        for (int tt = 0; tt < kI8StageTiles; ++tt) {
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const uint4 v = regs[tt][r];
+                st.codes[tt][(wave + 4 * r) * kWave + lane] =
+                    make_uint4(v.x ^ 0x80808080U, v.y ^ 0x80808080U, v.z ^ 0x80808080U, v.w ^ 0x80808080U);
+            }
+            if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                if (wave == 0) {
+                    st.term[tt][lane] = my_term[tt];
+                }
             }
         }
     };
 
-    uint64_t t = blockIdx.x;
-    if (t < span) {
-        fetch(t);
-        park(stage[0]);
-    }
+    // A stage is a run of 32 x 32 blocks: block b = (tile b / 4 of the stage, codes 32 ((b / 2) % 2) ..., queries
+    // 32 (b % 2) ...).  The matrix instructions of block b + 1 are issued among the verdicts of block b, so that
+    // the matrix pipe and the vector ALU of the wave run side by side.
+    constexpr int kBlocks = 4 * kI8StageTiles;
+    // The grid never has more columns than there are stages, so the first stage exists.  Fetching it without a
+    // condition also lets every load issued so far (the query operands) complete here, once, instead of being
+    // waited for inside the loop, where that wait would hold up the prefetch of the next stage.
+    uint64_t sg = blockIdx.x;
+    fetch(sg);
+    park(stage[0]);
     __syncthreads();
     uint32_t cur = 0;
-    for (; t < span; t += p.groups) {
-        const uint64_t tn = t + p.groups;
-        if (tn < span) {
-            fetch(tn);
+    for (; sg < nstages; sg += p.groups) {
+        const uint64_t sn = sg + p.groups;
+        if (sn < nstages) {
+            fetch(sn);
         }
         if (active) {
             const I8Stage& st = stage[cur];
-            const uint64_t slot0 = (p.tile_begin + t) * kWave;
+            const uint64_t slot0 = (p.tile_begin + sg * kI8StageTiles) * kWave;
+            intx16 hi[2], lo[2];  // two sets: one being filled, one being judged
+            auto multiply = [&](int b, intx16& h, intx16& l) {
+                const int tt = b >> 2, i = (b >> 1) & 1, j = b & 1;
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                intx4 av[4];
-#pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    const uint4 c = st.codes[(2 * s + half) * kWave + 32 * i + l32];
-                    av[s] = intx4{static_cast<int>(c.x), static_cast<int>(c.y), static_cast<int>(c.z),
-                                  static_cast<int>(c.w)};
-                }
-                intx16 hi[2], lo[2];
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        hi[j][e] = 0;
-                        lo[j][e] = 0;
-                    }
+                for (int e = 0; e < 16; ++e) {
+                    h[e] = 0;
+                    l[e] = 0;
                 }
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
-#pragma unroll
-                    for (int j = 0; j < 2; ++j) {
-                        hi[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s], qh[j][s], hi[j], 0, 0, 0);
-                        lo[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[s], ql[j][s], lo[j], 0, 0, 0);
-                    }
+                    const uint4 c = st.codes[tt][(2 * s + half) * kWave + 32 * i + l32];
+                    const intx4 av = intx4{static_cast<int>(c.x), static_cast<int>(c.y), static_cast<int>(c.z),
+                                           static_cast<int>(c.w)};
+                    h = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, qh[j][s], h, 0, 0, 0);
+                    l = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, ql[j][s], l, 0, 0, 0);
                 }
+            };
+            multiply(0, hi[0], lo[0]);
+#pragma unroll
+            for (int b = 0; b < kBlocks; ++b) {
+                const int tt = b >> 2, i = (b >> 1) & 1, j = b & 1;
                 // Element e of a lane is code 32 i + 8 (e / 4) + 4 (lane / 32) + e % 4 against query l32 of block j.
                 float tm[16];
                 if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
 #pragma unroll
                     for (int g = 0; g < 4; ++g) {
-                        const float4 v = *reinterpret_cast<const float4*>(&st.term[32 * i + 8 * g + 4 * half]);
+                        const float4 v = *reinterpret_cast<const float4*>(&st.term[tt][32 * i + 8 * g + 4 * half]);
                         tm[4 * g] = v.x;
                         tm[4 * g + 1] = v.y;
                         tm[4 * g + 2] = v.z;
                         tm[4 * g + 3] = v.w;
                     }
                 }
+                if (b + 1 < kBlocks) {
+                    multiply(b + 1, hi[(b + 1) & 1], lo[(b + 1) & 1]);
+                }
+                // Nearly nothing passes: the sixteen verdicts stay in scalar registers, and only when one of them
+                // has a bit set does the wave turn them into a bit mask per lane.
+                bool pass[16];
+                const uint64_t any = i8_verdicts<METRIC>(hi[b & 1], lo[b & 1], tm, uq[j], tau[j], pass);
+                if (b + 1 < kBlocks) {
+                    // One matrix instruction (32 cycles of the pipe), then its share of the 64 verdict instructions.
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    uint64_t hit[16];
-                    uint64_t any = 0;
+                    for (int m = 0; m < 8; ++m) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, METRIC == VSAG_AMD_METRIC_L2 ? 8 : 4, 0);
+                    }
+                }
+                if (any != 0) {
+                    uint32_t bits = 0;
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
-                        const int32_t tt = (hi[j][e] << 8) + lo[j][e];
-                        bool pass;
-                        if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
-                            pass = fmaf(static_cast<float>(tt), uq[j], tm[e]) <= __uint_as_float(tau[j]);
-                        } else {
-                            pass = tt >= static_cast<int32_t>(tau[j]);
-                        }
-                        hit[e] = __ballot(pass);
-                        any |= hit[e];
+                        bits |= pass[e] ? 1U << e : 0U;
                     }
-                    if (any != 0) {
-#pragma unroll
-                        for (int e = 0; e < 16; ++e) {
-                            if (hit[e] != 0 && ((hit[e] >> lane) & 1ULL) != 0) {
-                                const uint64_t slot = slot0 + 32 * i + 8 * (e >> 2) + 4 * half + (e & 3);
-                                if (slot < p.n) {
-                                    if (ncand[j] < p.sub_cap) {
-                                        my_list[j][ncand[j]] = static_cast<uint32_t>(slot);
-                                    }
-                                    ++ncand[j];
-                                }
+                    while (bits != 0) {
+                        const uint32_t e = static_cast<uint32_t>(__builtin_ctz(bits));
+                        bits &= bits - 1;
+                        const uint64_t slot = slot0 + 64 * tt + 32 * i + 8 * (e >> 2) + 4 * half + (e & 3);
+                        if (slot < p.n) {
+                            if (ncand[j] < p.sub_cap) {
+                                my_list[j][ncand[j]] = static_cast<uint32_t>(slot);
                             }
+                            ++ncand[j];
                         }
                     }
                 }
             }
         }
-        if (tn < span) {
+        if (sn < nstages) {
             park(stage[cur ^ 1]);
         }
         __syncthreads();  // the next stage is complete, and every wave is done with this one
@@ -386,9 +414,9 @@ prefilter_i8_query_bytes(uint64_t nq) {
 uint32_t
 prefilter_i8_sub_lists(uint64_t nq, uint64_t span) {
     const uint64_t qgroups = div_up(nq, static_cast<uint64_t>(kI8Group));
-    // Two workgroups fit a compute unit; three rounds of them even out the tail.
-    uint64_t groups = div_up(static_cast<uint64_t>(device_cu_count()) * 6, qgroups);
-    groups = std::max<uint64_t>(1, std::min<uint64_t>(groups, span));
+    // Two workgroups fit a compute unit; just under four full rounds of them (never a nearly empty last round).
+    uint64_t groups = static_cast<uint64_t>(device_cu_count()) * 8 / qgroups;
+    groups = std::max<uint64_t>(1, std::min<uint64_t>(groups, div_up(span, static_cast<uint64_t>(kI8StageTiles))));
     return static_cast<uint32_t>(2 * groups);
 }
 
