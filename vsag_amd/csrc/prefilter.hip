@@ -375,8 +375,9 @@ struct RescoreArgs {
     uint64_t* partial;
     uint32_t* partial_cnt;
     uint32_t nslots;
+    uint32_t first_slot;  // the list of the first level of this call; out_slot - first_slot levels came before
     uint32_t out_slot;
-    uint32_t* gate;  // per query: 1 = candidates overflowed, the streaming kernel must serve the query
+    uint32_t* gate;  // per query: 1 = candidates overflowed at some level, the streaming kernel must serve the query
     // sub_lists != 0: the candidates of a query sit in sub_lists lists of sub_cap slots with a count each (a count
     // above sub_cap = that list overflowed); they are gathered into LDS first (at most kRescoreGather of them).
     uint32_t sub_lists, sub_cap;
@@ -424,15 +425,17 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
         wave_lds_fence();
         mine = flat;
     }
-    if (overflow) {
+    if (overflow || as_const(r.gate)[q] != 0) {
+        // The streaming kernel will scan every tile behind the prefix for this query: the lists of the levels so
+        // far must not contribute the same codes a second time.
+        const uint32_t nlev = r.out_slot - r.first_slot + 1;
+        if (lane < nlev) {
+            r.partial_cnt[static_cast<uint64_t>(q) * r.nslots + r.first_slot + lane] = 0;
+        }
         if (lane == 0) {
             r.gate[q] = 1;
-            r.partial_cnt[list] = 0;
         }
         return;
-    }
-    if (lane == 0) {
-        r.gate[q] = 0;
     }
     const uint32_t S = r.S, k = r.k;
     selector_init(keys, S, lane);
@@ -536,10 +539,11 @@ int launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qst
 static int
 launch_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t k, uint32_t S, uint32_t* bound,
                const uint32_t* cand, const uint32_t* cand_cnt, uint32_t cap, uint32_t sub_lists, uint32_t sub_cap,
-               uint64_t* partial, uint32_t* partial_cnt, uint32_t nslots, uint32_t out_slot, uint32_t* gate,
-               hipStream_t st) {
+               uint64_t* partial, uint32_t* partial_cnt, uint32_t nslots, uint32_t first_slot, uint32_t out_slot,
+               uint32_t* gate, hipStream_t st) {
     const bool sq8 = s->kind == VSAG_AMD_KIND_SQ8;
     RescoreArgs r{};
+    r.first_slot = first_slot;
     r.cand = cand;
     r.cand_cnt = cand_cnt;
     r.cap = cap;
@@ -567,12 +571,12 @@ launch_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t
 
 
 // Steps 2 and 3 of the header comment for tiles [tile_begin, tile_end); the exact prefix scan has already
-// left its bounds in `bound`.  Writes one partial list per query (out_slot) and the overflow flags.
+// left its bounds in `bound`.  Writes one partial list per query (out_slot) and raises the overflow flags.
 int
 launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t k, uint32_t S, uint64_t tile_begin,
                  uint64_t tile_end, uint32_t* bound, float* tau, uint32_t* cand, uint32_t* cand_cnt, uint32_t cap,
-                 uint64_t* partial, uint32_t* partial_cnt, uint32_t nslots, uint32_t out_slot, uint32_t* gate,
-                 uint8_t* q8, float* q8_u, uint32_t sub_lists, uint32_t sub_cap, hipStream_t st) {
+                 uint64_t* partial, uint32_t* partial_cnt, uint32_t nslots, uint32_t first_slot, uint32_t out_slot,
+                 uint32_t* gate, uint8_t* q8, float* q8_u, uint32_t sub_lists, uint32_t sub_cap, hipStream_t st) {
     const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
     const bool sq8 = s->kind == VSAG_AMD_KIND_SQ8;
     if (q8 != nullptr) {
@@ -581,7 +585,7 @@ launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32
                                    tile_begin, tile_end, bound, q8, q8_u, reinterpret_cast<uint32_t*>(tau), cand,
                                    cand_cnt, sub_lists, sub_cap, st));
         return launch_rescore(s, a, nq, k, S, bound, cand, cand_cnt, 0, sub_lists, sub_cap, partial, partial_cnt, nslots,
-                              out_slot, gate, st);
+                              first_slot, out_slot, gate, st);
     }
     hipLaunchKernelGGL(prefilter_tau_kernel, dim3(static_cast<uint32_t>(nq)), dim3(kWave), 0, st,
                        reinterpret_cast<const float*>(a.qtab), a.qstride, s->dpad, sq8 && !l2 ? a.qmeta : nullptr,
@@ -620,8 +624,8 @@ launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32
     }
     timing_end(st);
     VA_HIP(hipGetLastError());
-    return launch_rescore(s, a, nq, k, S, bound, cand, cand_cnt, cap, 0, 0, partial, partial_cnt, nslots, out_slot, gate,
-                          st);
+    return launch_rescore(s, a, nq, k, S, bound, cand, cand_cnt, cap, 0, 0, partial, partial_cnt, nslots, first_slot,
+                          out_slot, gate, st);
 }
 
 }  // namespace vsag_amd

@@ -581,10 +581,16 @@ struct CallPlan {
     bool contraction = false;
     ScanPlan prefix, rest;
     uint64_t prefix_tiles = 0;
+    // The tiles behind the prefix are pre-selected level by level, each level against the k-th distance of
+    // everything before it: level l covers tiles [level_begin[l], level_begin[l + 1]).
+    static constexpr int kMaxLevels = 3;
+    int levels = 0;
+    uint64_t level_begin[kMaxLevels + 1] = {0, 0, 0, 0};
     bool int8 = false;         // the int8 matrix cores pre-select (sq8, at most 128 dimensions)
-    uint32_t cap = 0;          // candidates per query
-    uint32_t sub_lists = 0;    // int8: private candidate lists per query ...
-    uint32_t sub_cap = 0;      // ... of this many slots; cap = sub_lists * sub_cap
+    uint32_t cap = 0;          // candidates per query and level
+    uint32_t sub_lists[kMaxLevels] = {0, 0, 0};  // int8: private candidate lists per query ...
+    uint32_t sub_cap[kMaxLevels] = {0, 0, 0};    // ... of this many slots
+    uint32_t max_lists = 0;    // the largest sub_lists
     uint32_t nslots = 0;       // partial lists per query
     bool any_seeded = false;
 };
@@ -595,8 +601,8 @@ static int g_prefilter_mode = 0;
 bool prefilter_supports(const vsag_amd_store* s);
 int launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t k, uint32_t S, uint64_t tile_begin,
                      uint64_t tile_end, uint32_t* bound, float* tau, uint32_t* cand, uint32_t* cand_cnt, uint32_t cap,
-                     uint64_t* partial, uint32_t* partial_cnt, uint32_t nslots, uint32_t out_slot, uint32_t* gate,
-                     uint8_t* q8, float* q8_u, uint32_t sub_lists, uint32_t sub_cap, hipStream_t st);
+                     uint64_t* partial, uint32_t* partial_cnt, uint32_t nslots, uint32_t first_slot, uint32_t out_slot,
+                     uint32_t* gate, uint8_t* q8, float* q8_u, uint32_t sub_lists, uint32_t sub_cap, hipStream_t st);
 bool prefilter_i8_supports(const vsag_amd_store* s);
 size_t prefilter_i8_query_bytes(uint64_t nq);
 uint32_t prefilter_i8_sub_lists(uint64_t nq, uint64_t span);
@@ -622,27 +628,53 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
     if (nq * cap * 4 > (2ull << 30)) {
         return;
     }
-    // The prefix is scanned exactly; its k-th distance admits about k * (rest / prefix) codes of the rest.
-    // Keep that below an eighth of the buffer.
-    uint64_t prefix = std::max<uint64_t>(forced ? 2 : 256, div_up(8ull * k * s->ntiles, cap));
-    prefix += prefix & 1;  // the contraction walks pairs of tiles
-    if (prefix > s->ntiles / (forced ? 2 : 4) || prefix >= s->ntiles) {
+    // A level behind b tiles admits about k * (its tiles / b) codes per query: with every boundary a factor r
+    // behind the next one that is k * r, kept below an eighth of the buffer.  The prefix in front of the first
+    // level is scanned exactly by the streaming kernel.
+    const uint64_t r = std::min<uint64_t>(16, std::max<uint64_t>(2, cap / (8ull * k)));
+    const uint64_t min_prefix = forced ? 2 : 64;
+    uint64_t bounds[CallPlan::kMaxLevels + 1];
+    int nb = 0;
+    bounds[nb++] = s->ntiles;
+    uint64_t cur = s->ntiles;
+    while (nb <= CallPlan::kMaxLevels) {
+        uint64_t next = std::max(min_prefix, div_up(cur, r));
+        next += next & 1;
+        if (nb > 1 && cur < 4 * next) {
+            break;  // too thin a level to be worth its launches
+        }
+        bounds[nb++] = next;
+        cur = next;
+        if (next == min_prefix) {
+            break;
+        }
+    }
+    const uint64_t prefix = bounds[nb - 1];
+    if (nb < 2 || prefix > s->ntiles / (forced ? 2 : 4) || prefix >= s->ntiles) {
         return;
     }
     c->contraction = true;
     c->int8 = g_prefilter_mode != 2 && prefilter_i8_supports(s);
     c->prefix_tiles = prefix;
     c->cap = static_cast<uint32_t>(cap);
+    c->levels = nb - 1;
+    for (int l = 0; l <= c->levels; ++l) {
+        c->level_begin[l] = bounds[nb - 1 - l];
+    }
+    c->max_lists = 0;
     if (c->int8) {
-        // The expected load of a list is an eighth of its share of the buffer; short lists get room for the tail
-        // of that distribution.
-        c->sub_lists = prefilter_i8_sub_lists(nq, s->ntiles - prefix);
-        c->sub_cap = std::max<uint32_t>(16, static_cast<uint32_t>(div_up(cap, static_cast<uint64_t>(c->sub_lists))));
-        c->cap = c->sub_lists * c->sub_cap;
+        for (int l = 0; l < c->levels; ++l) {
+            // The expected load of a list is an eighth of its share of the buffer; short lists get room for the
+            // tail of that distribution.
+            c->sub_lists[l] = prefilter_i8_sub_lists(nq, c->level_begin[l + 1] - c->level_begin[l]);
+            c->sub_cap[l] = std::max<uint32_t>(16, static_cast<uint32_t>(div_up(cap, static_cast<uint64_t>(c->sub_lists[l]))));
+            c->cap = std::max(c->cap, c->sub_lists[l] * c->sub_cap[l]);
+            c->max_lists = std::max(c->max_lists, c->sub_lists[l]);
+        }
     }
     make_plan(s, nq, k, prefix, &c->prefix);
     make_plan(s, nq, k, s->ntiles - prefix, &c->rest);
-    uint32_t pf_slots = static_cast<uint32_t>(c->prefix.chunks * c->prefix.waves + 1 + c->rest.chunks * c->rest.waves);
+    uint32_t pf_slots = static_cast<uint32_t>(c->prefix.chunks * c->prefix.waves + c->levels + c->rest.chunks * c->rest.waves);
     c->nslots = std::max(c->nslots, pf_slots);
     c->any_seeded = c->any_seeded || c->prefix.seeded || c->rest.seeded;
 }
@@ -684,7 +716,7 @@ carve_scan(Carver& c, const CallPlan& cp, uint64_t nq, uint32_t k, ScanBuffers* 
     if (!cp.int8) {
         b->q8 = nullptr;
     }
-    b->cand_cnt = c.take<uint32_t>(cp.contraction ? nq * std::max<uint32_t>(1, cp.sub_lists) : 0);
+    b->cand_cnt = c.take<uint32_t>(cp.contraction ? nq * std::max<uint32_t>(1, cp.max_lists) : 0);
     b->gate = c.take<uint32_t>(cp.contraction ? nq : 0);
     b->cand = c.take<uint32_t>(cp.contraction ? nq * cp.cap : 0);
     return c.used;
@@ -867,21 +899,30 @@ vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, 
     } else {
         const uint32_t slots_prefix = static_cast<uint32_t>(cp.prefix.chunks * cp.prefix.waves);
         const uint32_t slots_rest = static_cast<uint32_t>(cp.rest.chunks * cp.rest.waves);
-        nslots = slots_prefix + 1 + slots_rest;
-        // The gated launch leaves the lists of most queries untouched: they must read as empty.  No candidates yet.
+        const uint32_t levels = static_cast<uint32_t>(cp.levels);
+        nslots = slots_prefix + levels + slots_rest;
+        // The gated launch leaves the lists of most queries untouched: they must read as empty.  No query has
+        // overflowed yet.
         hipLaunchKernelGGL(fill_words2_kernel, dim3(static_cast<uint32_t>(div_up(nq * nslots, 256))), dim3(256), 0, st,
-                           b.partial_cnt, nq * nslots, b.cand_cnt, nq);
+                           b.partial_cnt, nq * nslots, b.gate, nq);
         VA_TRY(run_streaming(s, cp.prefix, a, b, nq, k, nullptr, 0, cp.prefix_tiles, 0, nslots, nullptr, st));
-        // The waves of the prefix each know the k-th distance of their own tiles only; the k-th of the whole
-        // prefix (a merge into the output arrays, which the final merge overwrites) is the bound to filter with.
-        VA_TRY(launch_merge_partials(b.partial, b.partial_cnt, b.bound, slots_prefix, nslots, k, p.S, nq, ids_dev,
-                                     dists_dev, st));
-        hipLaunchKernelGGL(tighten_bound_kernel, dim3(static_cast<uint32_t>(div_up(nq, 256))), dim3(256), 0, st,
-                           dists_dev, k, nq, b.bound);
-        VA_TRY(launch_prefilter(s, a, nq, k, p.S, cp.prefix_tiles, s->ntiles, b.bound, b.tau, b.cand, b.cand_cnt, cp.cap,
-                                b.partial, b.partial_cnt, nslots, slots_prefix, b.gate, b.q8, b.q8_u, cp.sub_lists,
-                                cp.sub_cap, st));
-        VA_TRY(run_streaming(s, cp.rest, a, b, nq, k, nullptr, cp.prefix_tiles, s->ntiles, slots_prefix + 1, nslots,
+        for (uint32_t l = 0; l < levels; ++l) {
+            // The lists so far each know the k-th distance of their own part only; the k-th of everything before
+            // this level (a merge into the output arrays, which the final merge overwrites) is the bound to
+            // filter it with.
+            VA_TRY(launch_merge_partials(b.partial, b.partial_cnt, b.bound, slots_prefix + l, nslots, k, p.S, nq, ids_dev,
+                                         dists_dev, st));
+            hipLaunchKernelGGL(tighten_bound_kernel, dim3(static_cast<uint32_t>(div_up(nq, 256))), dim3(256), 0, st,
+                               dists_dev, k, nq, b.bound);
+            if (!cp.int8) {
+                hipLaunchKernelGGL(fill_words2_kernel, dim3(static_cast<uint32_t>(div_up(nq, 256))), dim3(256), 0, st,
+                                   b.cand_cnt, nq, static_cast<uint32_t*>(nullptr), 0);
+            }
+            VA_TRY(launch_prefilter(s, a, nq, k, p.S, cp.level_begin[l], cp.level_begin[l + 1], b.bound, b.tau, b.cand,
+                                    b.cand_cnt, cp.cap, b.partial, b.partial_cnt, nslots, slots_prefix, slots_prefix + l,
+                                    b.gate, b.q8, b.q8_u, cp.sub_lists[l], cp.sub_cap[l], st));
+        }
+        VA_TRY(run_streaming(s, cp.rest, a, b, nq, k, nullptr, cp.prefix_tiles, s->ntiles, slots_prefix + levels, nslots,
                              b.gate, st));
         tl_last_tile = cp.int8 ? 256 : 128;  // queries per pass of the contraction
         tl_last_passes = div_up(nq, cp.int8 ? 256 : 128);
