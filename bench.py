@@ -26,6 +26,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
 MFMA_F32_PEAK_TFLOPS = 157.3
+MFMA_I8_PEAK_TOPS = 5000.0  # dense int8, published
 
 
 def mt(seed):
@@ -270,16 +271,29 @@ def run_c2(env):
     # HBM/fabric bytes of one launch of this exact configuration, from rocprofv3 --pmc FETCH_SIZE (x 2.00, the
     # factor that makes kernels of known size read their size) + WRITE_SIZE (x 1.00): profiles/flat_scan_sq8_c2.md.
     traffic = None
+    traffic_i8 = None  # filled from the rocprofv3 --pmc runs of the int8 kernel (profiles/)
     if (n, d, nq, k, r["tile"]) == (1000000, 128, 10000, 10, 4):
         traffic = 111504620 * 2.00 * 1024 + 32254 * 1024
     roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
             "kernel": "flat_scan_kernel<sq8, l2, T=%d>" % r["tile"], "kernel_ms": r["kernel_ms"],
             "algorithmic_bytes_per_launch": algo_bytes}
-    if r["tile"] >= 64:
-        # The batch went through the matrix-core contraction (query tile 128): the dominant kernel multiplies
-        # every code of the store but the exactly scanned prefix with every query, 2 d flops per pair.
-        flops = 2.0 * n * d * nq
+    if r["tile"] == 256:
+        # The batch went through the int8 matrix cores (256 queries per workgroup): the timed kernel multiplies
+        # every code of the last level (bytes_per_pass / d of them) with two int8 planes of every query.
+        codes = r["bytes_per_pass"] / float(-(-d // 16) * 16)
+        ops = 2.0 * 2.0 * codes * (-(-d // 32) * 32) * nq
+        tops = ops / (r["kernel_ms"] * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": tops, "peak": MFMA_I8_PEAK_TOPS, "unit": "TOP/s",
+                "frac": tops / MFMA_I8_PEAK_TOPS, "traffic": traffic_i8 if (n, d, nq, k) == (1000000, 128, 10000, 10)
+                else None, "kernel": "prefilter_i8_kernel<l2> (int8 MFMA, last level)", "kernel_ms": r["kernel_ms"],
+                "ops_per_launch": ops, "codes_per_launch": codes,
+                "algorithmic_bytes_per_launch": algo_bytes, "algorithmic_gbs": achieved}
+    elif r["tile"] >= 64:
+        # The batch went through the fp32 matrix-core contraction (query tile 128): the timed kernel multiplies
+        # every code of the last level with every query, 2 d flops per pair.
+        codes = r["bytes_per_pass"] / float(-(-d // 16) * 16)
+        flops = 2.0 * codes * d * nq
         tf = flops / (r["kernel_ms"] * 1e-3) / 1e12
         roof = {"bound": "mfma", "achieved": tf, "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": tf / MFMA_F32_PEAK_TFLOPS, "traffic": None, "kernel": "prefilter_kernel<sq8> (fp32 MFMA)",
@@ -327,10 +341,13 @@ def run_c1(env):
             "algorithmic_bytes_per_launch": algo, "flops_per_launch": 2.0 * n * d * nq,
             "tflops": 2.0 * n * d * nq / (kms * 1e-3) / 1e12}
     if tile >= 64:
-        tf = 2.0 * n * d * nq / (kms * 1e-3) / 1e12
+        # The timed kernel is the last level of the contraction: bpp bytes of fp32 codes against every query.
+        codes = bpp / (4.0 * d)
+        tf = 2.0 * codes * d * nq / (kms * 1e-3) / 1e12
         roof = {"bound": "mfma", "achieved": tf, "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": tf / MFMA_F32_PEAK_TFLOPS, "traffic": None, "kernel": "prefilter_kernel<fp32> (fp32 MFMA)",
-                "kernel_ms": kms, "flops_per_launch": 2.0 * n * d * nq}
+                "frac": tf / MFMA_F32_PEAK_TFLOPS, "traffic": None,
+                "kernel": "prefilter_kernel<fp32> (fp32 MFMA, last level)", "kernel_ms": kms,
+                "flops_per_launch": 2.0 * codes * d * nq, "codes_per_launch": codes}
     return env.base_line("QPS @ recall@10 (100k x 128 fp32 brute force)", "queries/s", nq / sec, sec, "f32",
                          "configs[0]: brute_force fp32 L2, N=%d, d=%d, %d queries, k=%d" % (n, d, nq, k),
                          {"recall_at_10": rec, "query_tile": tile, "passes_per_step": passes, "bytes_per_pass": bpp},

@@ -315,8 +315,33 @@ prefilter_i8_kernel(PrefilterI8Args p) {
             const I8Stage& st = stage[cur];
             const uint64_t slot0 = (p.tile_begin + sg * kI8StageTiles) * kWave;
             intx16 hi[2], lo[2];  // two sets: one being filled, one being judged
+            // Row r of the stage = codes 32 (r % 2) ... of its tile r / 2; blocks 2 r and 2 r + 1 are its two query
+            // halves.  Code operands and |y|^2 terms of a row are read from LDS one block before their first use
+            // (two register sets each), so that no matrix instruction and no verdict waits for LDS.
+            intx4 av[2][4];
+            float tm[2][16];
+            auto read_row = [&](int r) {
+                const int tt = r >> 1, i = r & 1;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const uint4 c = st.codes[tt][(2 * s + half) * kWave + 32 * i + l32];
+                    av[r & 1][s] = intx4{static_cast<int>(c.x), static_cast<int>(c.y), static_cast<int>(c.z),
+                                         static_cast<int>(c.w)};
+                }
+                if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                    // Element e of a lane is code 32 i + 8 (e / 4) + 4 (lane / 32) + e % 4 of the tile.
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const float4 v = *reinterpret_cast<const float4*>(&st.term[tt][32 * i + 8 * g + 4 * half]);
+                        tm[r & 1][4 * g] = v.x;
+                        tm[r & 1][4 * g + 1] = v.y;
+                        tm[r & 1][4 * g + 2] = v.z;
+                        tm[r & 1][4 * g + 3] = v.w;
+                    }
+                }
+            };
             auto multiply = [&](int b, intx16& h, intx16& l) {
-                const int tt = b >> 2, i = (b >> 1) & 1, j = b & 1;
+                const int r = b >> 1, j = b & 1;
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     h[e] = 0;
@@ -324,28 +349,19 @@ prefilter_i8_kernel(PrefilterI8Args p) {
                 }
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
-                    const uint4 c = st.codes[tt][(2 * s + half) * kWave + 32 * i + l32];
-                    const intx4 av = intx4{static_cast<int>(c.x), static_cast<int>(c.y), static_cast<int>(c.z),
-                                           static_cast<int>(c.w)};
-                    h = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, qh[j][s], h, 0, 0, 0);
-                    l = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, ql[j][s], l, 0, 0, 0);
+                    h = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[r & 1][s], qh[j][s], h, 0, 0, 0);
+                    l = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[r & 1][s], ql[j][s], l, 0, 0, 0);
                 }
             };
+            read_row(0);
             multiply(0, hi[0], lo[0]);
 #pragma unroll
             for (int b = 0; b < kBlocks; ++b) {
-                const int tt = b >> 2, i = (b >> 1) & 1, j = b & 1;
-                // Element e of a lane is code 32 i + 8 (e / 4) + 4 (lane / 32) + e % 4 against query l32 of block j.
-                float tm[16];
-                if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const float4 v = *reinterpret_cast<const float4*>(&st.term[tt][32 * i + 8 * g + 4 * half]);
-                        tm[4 * g] = v.x;
-                        tm[4 * g + 1] = v.y;
-                        tm[4 * g + 2] = v.z;
-                        tm[4 * g + 3] = v.w;
-                    }
+                const int r = b >> 1, j = b & 1;
+                constexpr int kDsReads = METRIC == VSAG_AMD_METRIC_L2 ? 8 : 4;
+                const bool reads = j == 0 && b + 2 < kBlocks;
+                if (reads) {
+                    read_row(r + 1);
                 }
                 if (b + 1 < kBlocks) {
                     multiply(b + 1, hi[(b + 1) & 1], lo[(b + 1) & 1]);
@@ -353,9 +369,13 @@ prefilter_i8_kernel(PrefilterI8Args p) {
                 // Nearly nothing passes: the sixteen verdicts stay in scalar registers, and only when one of them
                 // has a bit set does the wave turn them into a bit mask per lane.
                 bool pass[16];
-                const uint64_t any = i8_verdicts<METRIC>(hi[b & 1], lo[b & 1], tm, uq[j], tau[j], pass);
+                const uint64_t any = i8_verdicts<METRIC>(hi[b & 1], lo[b & 1], tm[r & 1], uq[j], tau[j], pass);
                 if (b + 1 < kBlocks) {
-                    // One matrix instruction (32 cycles of the pipe), then its share of the 64 verdict instructions.
+                    // The LDS reads first; then one matrix instruction (32 cycles of the pipe) at a time, each
+                    // followed by its share of the verdict instructions.
+                    if (reads) {
+                        __builtin_amdgcn_sched_group_barrier(0x100, kDsReads, 0);
+                    }
 #pragma unroll
                     for (int m = 0; m < 8; ++m) {
                         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -371,7 +391,7 @@ prefilter_i8_kernel(PrefilterI8Args p) {
                     while (bits != 0) {
                         const uint32_t e = static_cast<uint32_t>(__builtin_ctz(bits));
                         bits &= bits - 1;
-                        const uint64_t slot = slot0 + 64 * tt + 32 * i + 8 * (e >> 2) + 4 * half + (e & 3);
+                        const uint64_t slot = slot0 + 32 * r + 8 * (e >> 2) + 4 * half + (e & 3);
                         if (slot < p.n) {
                             if (ncand[j] < p.sub_cap) {
                                 my_list[j][ncand[j]] = static_cast<uint32_t>(slot);

@@ -928,7 +928,9 @@ vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, 
         tl_last_passes = div_up(nq, cp.int8 ? 256 : 128);
     }
     VA_TRY(launch_merge_partials(b.partial, b.partial_cnt, b.bound, nslots, nslots, k, p.S, nq, ids_dev, dists_dev, st));
-    tl_last_bytes = s->ntiles * s->G * kWave * kGranule;
+    // Code bytes under the timed kernel: the whole store, or the last (by far the largest) level of the contraction.
+    const uint64_t timed_tiles = contraction ? s->ntiles - cp.level_begin[cp.levels - 1] : s->ntiles;
+    tl_last_bytes = timed_tiles * s->G * kWave * kGranule;
     return 0;
 }
 
