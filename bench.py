@@ -271,9 +271,10 @@ def run_c2(env):
     # HBM/fabric bytes of one launch of this exact configuration, from rocprofv3 --pmc FETCH_SIZE (x 2.00, the
     # factor that makes kernels of known size read their size) + WRITE_SIZE (x 1.00): profiles/flat_scan_sq8_c2.md.
     traffic = None
-    traffic_i8 = None  # filled from the rocprofv3 --pmc runs of the int8 kernel (profiles/)
+    # the same two counters for the last-level launch of the int8 kernel: profiles/prefilter_i8_sq8_c2.md
+    traffic_i8 = 2422324.4 * 2.00 * 1024 + 68345.8 * 1024
     if (n, d, nq, k, r["tile"]) == (1000000, 128, 10000, 10, 4):
-        traffic = 111504620 * 2.00 * 1024 + 32254 * 1024
+        traffic = 115043826 * 2.00 * 1024 + 28593 * 1024
     roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
             "kernel": "flat_scan_kernel<sq8, l2, T=%d>" % r["tile"], "kernel_ms": r["kernel_ms"],
@@ -345,7 +346,9 @@ def run_c1(env):
         codes = bpp / (4.0 * d)
         tf = 2.0 * codes * d * nq / (kms * 1e-3) / 1e12
         roof = {"bound": "mfma", "achieved": tf, "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": tf / MFMA_F32_PEAK_TFLOPS, "traffic": None,
+                "frac": tf / MFMA_F32_PEAK_TFLOPS,
+                # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this launch: profiles/prefilter_fp32_c1.md
+                "traffic": 87735.7 * 2.00 * 1024 + 23281.8 * 1024 if (n, d, nq, k) == (100000, 128, 1000, 10) else None,
                 "kernel": "prefilter_kernel<fp32> (fp32 MFMA, last level)", "kernel_ms": kms,
                 "flops_per_launch": 2.0 * codes * d * nq, "codes_per_launch": codes}
     return env.base_line("QPS @ recall@10 (100k x 128 fp32 brute force)", "queries/s", nq / sec, sec, "f32",
@@ -411,7 +414,12 @@ def run_c3(env):
     flops = 2.0 * n * k * d
     tf = flops / (kms * 1e-3) / 1e12
     roof = {"bound": "mfma", "achieved": tf, "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": tf / MFMA_F32_PEAK_TFLOPS, "traffic": None, "kernel": "kmeans_assign_kernel", "kernel_ms": kms,
+            "frac": tf / MFMA_F32_PEAK_TFLOPS,
+            # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of one launch: profiles/kmeans_assign_c3.md.  Far above
+            # the 3.9 GB of inputs: every row tile re-reads the centroids from beyond the L2 (they come from the
+            # last-level cache, the kernel stays bound by the matrix cores).
+            "traffic": 65124676.8 * 2.00 * 1024 + 125000.0 * 1024 if (n, d, k) == (1000000, 960, 4096) else None,
+            "kernel": "kmeans_assign_kernel", "kernel_ms": kms,
             "flops_per_launch": flops}
     return env.base_line("k-means assign rows/s", "rows/s", n / sec, sec, "f32",
                          "configs[2]: k-means assignment, N=%d, d=%d, k=%d (one step = one assignment pass)" % (n, d, k),
@@ -563,7 +571,7 @@ def run_c4(env):
     # through L2 once per <= 4 queries, so the fraction against HBM exceeds 1: this kernel is bound by VALU issue.
     traffic = None
     if (n, d, nq, k, nlist) == (10000000, 128, 10000, 10, 4096):
-        traffic = (471200.19 + 1633918.44) * 2.00 * 1024 + (10050.06 + 19932.66) * 1024
+        traffic = (483541.75 + 1699620.5) * 2.00 * 1024 + (9817.03 + 19921.13) * 1024
     roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
             "traffic": traffic, "kernel": "ivf_scan_kernel<sq4_uniform, l2> (2 launches per step)", "kernel_ms": kms,
             "algorithmic_bytes_per_launch": algo,
@@ -666,7 +674,7 @@ def run_c5(env):
     # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this exact configuration, profiles/flat_scan_rabitq_c5.md
     traffic = None
     if (n, d, nq, k, tile) == (5000000, 768, 10000, 10, 2):
-        traffic = 1051929650.94 * 2.00 * 1024 + 250734.91 * 1024
+        traffic = 1432385046.4 * 2.00 * 1024 + 242731.1 * 1024
     roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
             "traffic": traffic, "kernel": "flat_scan_kernel<rabitq, ip, T=%d>" % tile, "kernel_ms": kms,
             "algorithmic_bytes_per_launch": algo}
