@@ -196,6 +196,8 @@ VSAG_AMD_API int vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* store, const
 
 /* Large batches on flat fp32 / sq8 stores are served by a matrix-core contraction that pre-selects candidates,
  * which are then recomputed and selected exactly as the streaming scan does (same results, bit for bit).
+ * Posting lists of sq4_uniform / L2 codes of at most 128 dimensions scan the probe columns behind the first on the
+ * int8 matrix cores when a batch has at least 8192 (query, list) groups (same results; off with mode -1).
  * sq8 stores of at most 128 dimensions pre-select on the int8 matrix cores (queries split into two int8 planes
  * with a rigorous bound on the remainder), the others on the fp32 matrix cores.
  * mode: 0 = when it pays (default: >= 512 queries, k <= 128, >= 65536 codes), 1 = whenever the store and k
@@ -206,8 +208,9 @@ VSAG_AMD_API int vsag_amd_set_scan_contraction(int mode);
 /* Tuning knobs of the scan (query tile T in {1,2,4,8}, 0 = automatic; number of base chunks, 0 =
  * automatic).  Process-wide; meant for benchmarks. */
 VSAG_AMD_API int vsag_amd_set_scan_tuning(int query_tile, int base_chunks);
-/* What the last flat scan on this thread used: query tile, passes over the code array, bytes of codes
- * one pass reads. */
+/* What the last flat scan on this thread used: query tile (128 / 256: the batch went through the fp32 / int8
+ * matrix cores), passes over the code array, bytes of codes one pass reads.  After a posting-list scan: query tile
+ * only (256: the columns behind the first went through the int8 matrix cores). */
 VSAG_AMD_API int vsag_amd_last_scan_info(int* query_tile, uint64_t* passes, uint64_t* bytes_per_pass);
 
 /* Measurement hook: when enabled, a call records HIP events on its stream around the launch of its

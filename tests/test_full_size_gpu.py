@@ -93,6 +93,16 @@ def test_sq8_scan_1m(lib, metric, ometric):
     check_result_shape(ids, dists, n)
     oi, od = orc.flat_scan_topk(orc.SQ8, ometric, d, codes, q[:32], k, lb=lb, diff=diff)
     assert_topk_close(ids[:32], dists[:32], oi, od, label="sq8 1M")
+    # 512 queries go through the int8 matrix-core pre-selection; the streaming kernel alone must return the same bits
+    info = capi.C.c_int()
+    lib.vsag_amd_last_scan_info(capi.C.byref(info), None, None)
+    assert info.value == 256, "the int8 pre-selection did not run"
+    capi.check(lib.vsag_amd_set_scan_contraction(-1))
+    try:
+        si, sd = store.flat_scan(q, k)
+    finally:
+        capi.check(lib.vsag_amd_set_scan_contraction(0))
+    assert np.array_equal(si, ids) and np.array_equal(sd.view(np.uint32), dists.view(np.uint32))
     # the same answer whatever the query tile, and one query per call (a different grid and cold start)
     for tile in (1, 2):
         ti, td = scan_with_tile(lib, store, q[:256], k, tile)

@@ -1,0 +1,81 @@
+"""Large batches on sq4_uniform / L2 posting lists: the probe columns behind the first go through the int8 matrix
+cores.  The integer test selects exactly what the streaming kernel would admit and the distances are formed by the
+same operations, so ids and distance bits must equal the streaming scan's (and the checker's distances)."""
+import numpy as np
+import pytest
+
+import oracle as orc
+from gpu_helpers import Store, gaussian_mixture
+from vsag_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(seed, n, d, nlist, nq, components=40, sigma=0.05):
+    rng = np.random.default_rng(seed)
+    x, means = gaussian_mixture(rng, n, d, components, sigma)
+    q, _ = gaussian_mixture(rng, nq, d, components, sigma, means=means)
+    cent = x[rng.choice(n, nlist, replace=False)].copy()
+    labels, _, _ = orc.kmeans_assign(x, cent)
+    l, dd = orc.sq_train_uniform(x, 4, orc.L2, mode=3)
+    codes = orc.squ_encode(x, 4, l, dd, orc.L2)
+    st = Store(capi.KIND_SQ4_UNIFORM, orc.L2, d, bounds=[l, dd])
+    st.set_lists(codes, labels, nlist)
+    return x, q, cent, labels, codes, (l, dd), st
+
+
+def _both(lib, st, q, buckets, kcand):
+    L = lib.load_library()
+    capi.check(L.vsag_amd_set_scan_contraction(-1))
+    try:
+        plain = st.ivf_scan(q, buckets, kcand)
+    finally:
+        capi.check(L.vsag_amd_set_scan_contraction(0))
+    fast = st.ivf_scan(q, buckets, kcand)
+    tile = capi.C.c_int()
+    L.vsag_amd_last_scan_info(capi.C.byref(tile), None, None)
+    assert tile.value == 256, "the matrix-core pass did not run"
+    return plain, fast
+
+
+def _same(a, b):
+    return np.array_equal(a[0], b[0]) and np.array_equal(a[1].view(np.uint32), b[1].view(np.uint32))
+
+
+@pytest.mark.parametrize("n,d,nlist,nq,nprobe,kcand", [(60000, 128, 64, 2100, 16, 100), (30000, 100, 37, 4500, 8, 10),
+                                                       (20000, 32, 16, 9000, 4, 32)])
+def test_matrix_core_columns_equal_streaming(lib, n, d, nlist, nq, nprobe, kcand):
+    x, q, cent, labels, codes, (l, dd), st = _case(n + d, n, d, nlist, nq)
+    buckets, _ = orc.ivf_route(cent, q, nprobe)
+    plain, fast = _both(lib, st, q, buckets, kcand)
+    assert _same(plain, fast)
+    # and the checker's distances, bit for bit, on a sample
+    offsets, order = orc.ivf_build_lists(labels, nlist)
+    qproc = orc.squ_encode(q[:64], 4, l, dd, orc.L2)
+    _, rds = orc.ivf_scan(orc.SQ4U, orc.L2, d, codes[order], offsets, order, qproc, buckets[:64], kcand, lb=l, diff=dd)
+    assert np.array_equal(fast[1][:64].view(np.uint32), rds.view(np.uint32))
+    st.destroy()
+
+
+def test_overflowing_lists_fall_back_to_streaming(lib):
+    """Queries routed to a far list first: the bound the first column leaves is so loose that the other lists hold
+    hundreds of better codes, more than a private list takes; those queries go back to the streaming kernel."""
+    n, d, nlist, nq, nprobe, kcand = 40000, 64, 8, 9000, 4, 10
+    x, q, cent, labels, codes, (l, dd), st = _case(11, n, d, nlist, nq, components=8, sigma=0.02)
+    routed, _ = orc.ivf_route(cent, q, nlist)
+    buckets = np.ascontiguousarray(routed[:, [nlist - 1, 0, 1, 2]])  # farthest list first, then the nearest three
+    plain, fast = _both(lib, st, q, buckets, kcand)
+    assert _same(plain, fast)
+    st.destroy()
+
+
+def test_missing_buckets_and_ragged_lists(lib):
+    n, d, nlist, nq, nprobe, kcand = 30000, 128, 50, 3000, 12, 20
+    x, q, cent, labels, codes, (l, dd), st = _case(5, n, d, nlist, nq)
+    buckets, _ = orc.ivf_route(cent, q, nprobe)
+    buckets = buckets.copy()
+    buckets[::3, 5:] = -1       # fewer lists than columns
+    buckets[1::7, 0] = -1       # no first list at all: no bound, everything overflows
+    plain, fast = _both(lib, st, q, buckets, kcand)
+    assert _same(plain, fast)
+    st.destroy()

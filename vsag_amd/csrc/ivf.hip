@@ -31,9 +31,16 @@ struct ScanPlanIvf {
     uint32_t chunks_max;      // partial lists per (query, list) pair
     bool chunked;             // one launch over all probe columns, seeded cold start
     bool seeded;
+    bool mfma;                // probe columns behind the first go through the int8 matrix cores (ivf_i8.hip)
 };
 
 uint64_t rabitq_query_code_size(uint32_t dim, int metric, int query_bits);
+int scan_contraction_mode();
+void note_last_scan(int query_tile, uint64_t passes, uint64_t bytes_per_pass);
+bool ivf_i8_supports(const vsag_amd_store* s);
+int launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
+                  const uint32_t* pair_off, const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound,
+                  int32_t* tq, uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st);
 int prepare_queries(const vsag_amd_store* s, const float* queries, uint64_t nq, uint64_t nq_pad, const QueryLayout& ql,
                     uint32_t* qtab, float* qmeta, uint8_t* qcodes, hipStream_t st);
 ScanArgs make_scan_args(const vsag_amd_store* s, const QueryLayout& ql, const uint32_t* qtab, const float* qmeta);
@@ -243,6 +250,7 @@ struct IvfArgs {
     uint32_t* seed;              // nq x k first-tile minima by work-item class, or null (flat scan's cold start)
     uint64_t* partial;           // npairs_total x chunks_max x k keys
     uint32_t* partial_cnt;       // npairs_total x chunks_max
+    const uint32_t* gate;        // per query, or null: only queries with a raised gate are served
 };
 
 constexpr uint32_t kIvfSeedTiles = 4;
@@ -293,10 +301,16 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
     uint64_t tau[T];
     uint32_t cnt[T];
     uint32_t cold[T];  // tiles after which this item still looks at the seed row (see the flat scan)
+    bool any_live = false;
 #pragma unroll
     for (int t = 0; t < T; ++t) {
         bool live = pbeg + t < pend;
         pair[t] = live ? as_const(v.sorted_pair)[pbeg + t] : 0xFFFFFFFFU;
+        if (live && v.gate != nullptr && as_const(v.gate)[pair[t] / v.nprobe] == 0) {
+            live = false;
+            pair[t] = 0xFFFFFFFFU;
+        }
+        any_live = any_live || live;
         qidx[t] = live ? pair[t] / v.nprobe : v.dummy_query;
         cnt[t] = 0;
         uint32_t bound = live ? __builtin_amdgcn_readfirstlane(__atomic_load_n(&v.bound[qidx[t]], __ATOMIC_RELAXED))
@@ -304,6 +318,9 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
         // Everything at or below the bound passes, whatever its id.
         tau[t] = (static_cast<uint64_t>(bound) << 32) | 0xFFFFFFFFULL;
         cold[t] = CHUNKED && v.seed != nullptr && live && bound == 0xFFFFFFFFU ? kIvfSeedTiles : 0;
+    }
+    if (!any_live) {
+        return;  // nothing but gated-off queries
     }
     const uint32_t seed_slot = item % k;
     for (uint32_t i = lane; i < T * S; i += kWave) {
@@ -624,6 +641,8 @@ struct IvfBuffers {
     uint32_t* seed;
     uint32_t* partial_cnt;
     uint64_t* partial;
+    uint32_t* gate;       // mfma: nq
+    int32_t* tq;          // mfma: nq + 1
 };
 
 static void
@@ -669,6 +688,13 @@ plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, 
         p->chunks_max = static_cast<uint32_t>(cap);
     }
     p->seeded = p->chunked && kcand <= 256;
+    // Large batches on sq4_uniform / L2 lists: the streaming kernel scans the nearest list of every query, the int8
+    // matrix cores the other columns, into two private lists per (query, list) pair.
+    p->mfma = !p->chunked && nprobe > 1 && scan_contraction_mode() >= 0 && ivf_i8_supports(s) &&
+              npairs * 2 * kcand * 8 <= (8ull << 30);
+    if (p->mfma) {
+        p->chunks_max = 2;
+    }
 }
 
 static size_t
@@ -685,6 +711,8 @@ carve_ivf(Carver& c, const vsag_amd_store* s, const ScanPlanIvf& p, uint64_t nq,
     b->seed = c.take<uint32_t>(p.seeded ? nq * kcand : 0);
     b->partial_cnt = c.take<uint32_t>(p.npairs * p.chunks_max);
     b->partial = c.take<uint64_t>(p.npairs * p.chunks_max * kcand);
+    b->gate = c.take<uint32_t>(p.mfma ? nq : 0);
+    b->tq = c.take<int32_t>(p.mfma ? nq + 1 : 0);
     return c.used;
 }
 
@@ -801,6 +829,8 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
     // Whole lists: two passes, the nearest list of every query first (it seeds the per-query bound), then the
     // rest.  Chunked lists: all probe columns at once.
     uint32_t cols[3] = {0, p.chunked ? nprobe : 1, nprobe};
+    // A pre-filter or a radius goes the streaming way (the matrix-core pass knows neither).
+    const bool mfma = p.mfma && (options == nullptr || (options->deny_bits_dev == nullptr && options->use_radius == 0));
     timing_begin(st);
     for (int pass = 0; pass < 2; ++pass) {
         uint32_t p0 = cols[pass], p1 = cols[pass + 1];
@@ -809,7 +839,27 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
         }
         uint64_t pairs = nq * (p1 - p0);
         if (pass == 1) {
-            fill(FillJob{{b.counts, b.cursor, nullptr, nullptr, nullptr}, {0U, 0U, 0U, 0U, 0U}, {nlists1, nlists1, 0, 0, 0}});
+            fill(FillJob{{b.counts, b.cursor, mfma ? b.gate : nullptr, nullptr, nullptr}, {0U, 0U, 0U, 0U, 0U},
+                         {nlists1, nlists1, mfma ? nq : 0, 0, 0}});
+        }
+        if (pass == 1 && mfma) {
+            // Pairs grouped by list once; workgroups of 256 pairs for the matrix cores, then -- for the queries whose
+            // lists overflowed -- the streaming kernel's items over the same grouping.
+            hipLaunchKernelGGL(count_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq, nprobe,
+                               p0, p1, s->nlist, b.counts);
+            hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, st, b.counts, s->list_tile_dev, s->nlist, 256U,
+                               0xFFFFFFFFU, 1U, b.pair_off, b.item_off);
+            hipLaunchKernelGGL(scatter_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq,
+                               nprobe, p0, p1, s->nlist, b.pair_off, b.cursor, b.sorted_pair);
+            VA_TRY(launch_ivf_i8(s, a, nq, nprobe, p0, kcand, b.pair_off, b.item_off, b.sorted_pair, b.bound, b.tq,
+                                 b.partial, b.partial_cnt, b.gate, st));
+            hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, st, b.counts, s->list_tile_dev, s->nlist,
+                               static_cast<uint32_t>(p.T), 0xFFFFFFFFU, 1U, b.pair_off, b.item_off);
+            v.gate = b.gate;
+            uint64_t max_items = div_up(pairs, p.T) + std::min<uint64_t>(s->nlist, pairs);
+            dim3 grid(static_cast<uint32_t>(div_up(max_items, waves)));
+            VA_TRY(launch_ivf(s, p.T, grid, dim3(waves * kWave), lds, st, a, v));
+            continue;
         }
         if (p.chunked) {
             hipLaunchKernelGGL(regroup_small_kernel, dim3(1), dim3(1024), 0, st, buckets_dev, nq, nprobe,
@@ -829,6 +879,7 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
         VA_TRY(launch_ivf(s, p.T, grid, dim3(waves * kWave), lds, st, a, v));
     }
     timing_end(st);
+    note_last_scan(mfma ? 256 : p.T, 0, 0);
     return launch_merge_partials(b.partial, b.partial_cnt, b.bound, nprobe * p.chunks_max, nprobe * p.chunks_max, kcand,
                                  p.S, nq, ids_dev, dists_dev, st);
 }

@@ -1,0 +1,375 @@
+// Posting lists of sq4_uniform codes (L2, at most 128 dimensions) against large query batches, on the int8 matrix
+// cores.
+//
+// The streaming IVF kernel (ivf.hip) is bound by vector-ALU issue: every (query, code) pair costs sixteen dot4
+// instructions.  The distance of this quantizer is a function of integers only,
+//
+//      dist = fl((Nq + No - 2 <q, o>) * scalar_rate),      Nq, No the squared norms of the 4-bit codes,
+//
+// (distance.h, finish_distances; sq4_uniform_quantizer.cpp:168-223 of the reference), and v_mfma_i32_32x32x32_i8
+// delivers <q, o> exactly.  "dist <= bound" is therefore the integer test 2 <q, o> - No >= Nq - tmax(bound), where
+// tmax is the largest integer t with fl(t * scalar_rate) <= bound; the pairs that pass are exactly the ones the
+// streaming kernel would admit under the same bound, and their distances are formed by the same three fp32
+// operations.  The kernel serves the probe columns behind the first one: the nearest list of every query has been
+// scanned by the streaming kernel, which leaves the bound.
+//
+// Work split: the (query, list) pairs are grouped by list as for the streaming kernel; a workgroup is a list and up
+// to 256 of its pairs, four waves of 64.  It walks the whole list, two tiles per LDS stage; staging splits the
+// nibbles, so a staged tile looks like eight 16-byte granules per code in the operand order of the instruction.
+// What passes goes into the private list of (pair, lane / 32): no atomics.  A list that overflows raises the
+// query's gate; gated queries drop these lists and are served by the streaming kernel.
+#include "distance.h"
+#include "store.h"
+#include "topk.h"
+
+namespace vsag_amd {
+
+typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef int intx16 __attribute__((ext_vector_type(16)));
+
+constexpr uint32_t kIvfI8Pairs = 256;  // pairs per workgroup
+constexpr int kIvfI8StageTiles = 2;
+
+// Per query: Tq = Nq - tmax(bound) (see the header), widened by one level; the slow path re-checks exactly.
+__global__ void __launch_bounds__(256)
+ivf_i8_threshold_kernel(const uint32_t* bound, const float* qmeta, uint32_t qmeta_stride, float rate, uint64_t nq,
+                        int32_t* tq) {
+    const uint64_t q = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (q > nq) {
+        return;
+    }
+    if (q == nq) {
+        tq[q] = 0x7FFFFFFF;  // the all-zero query row idle lanes point at: nothing passes
+        return;
+    }
+    const uint32_t b = bound[q];
+    if (b == 0xFFFFFFFFU || !(rate > 0.0F)) {
+        tq[q] = static_cast<int32_t>(0x80000000U);  // no bound: everything passes (and the query will overflow)
+        return;
+    }
+    const float bd = ordered_to_float(b);
+    const double t0 = floor(static_cast<double>(bd) / static_cast<double>(rate));
+    int64_t t = t0 > 1.0e9 ? 1000000000LL : (t0 < -1.0e9 ? -1000000000LL : static_cast<int64_t>(t0));
+    for (int i = 0; i < 4 && static_cast<float>(t + 1) * rate <= bd; ++i) {
+        ++t;
+    }
+    for (int i = 0; i < 4 && static_cast<float>(t) * rate > bd; ++i) {
+        --t;
+    }
+    const int64_t nqv = static_cast<int64_t>(qmeta[q * qmeta_stride]);
+    int64_t v = nqv - (t + 1);
+    v = v > 0x7FFFFFFELL ? 0x7FFFFFFELL : (v < -0x7FFFFFFFLL ? -0x7FFFFFFFLL : v);
+    tq[q] = static_cast<int32_t>(v);
+}
+
+struct IvfI8Args {
+    const uint4* tiles;
+    uint32_t G;                  // granules per code (<= 4)
+    const uint32_t* meta;        // per slot: No as float bits
+    const uint32_t* ids;         // inner id per tile slot
+    const uint32_t* list_tile;   // nlist + 1
+    const uint32_t* pair_off;    // nlist + 1
+    const uint32_t* item_off;    // nlist + 1: workgroups per list (256 pairs each), prefix sums
+    const uint32_t* sorted_pair; // pair index (q * nprobe + p) grouped by list
+    uint32_t nlist, nprobe;
+    uint32_t dummy_query;        // index of the all-zero query row
+    const uint32_t* qtab;        // processed queries (distance.h): per code dword {low nibbles, high nibbles}
+    uint32_t qstride;
+    const float* qmeta;
+    uint32_t qmeta_stride;
+    float rate;
+    const int32_t* tq;           // per query (+ the dummy row)
+    const uint32_t* bound;       // per query, ordered distance
+    uint32_t k;                  // capacity of a private list
+    uint64_t* partial;           // [pair][2][k] keys
+    uint32_t* partial_cnt;       // [pair][2]
+    uint32_t* gate;              // per query: raised when one of its lists overflowed
+};
+
+struct IvfI8Stage {
+    uint4 codes[kIvfI8StageTiles][8 * kWave];  // [2 granule + nibble half][code]: one nibble per byte
+    int32_t term[kIvfI8StageTiles][kWave];     // -No per code
+};
+
+__global__ void __launch_bounds__(256, 2)
+ivf_i8_kernel(IvfI8Args p) {
+    __shared__ IvfI8Stage stage[2];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    const uint32_t wave = tid >> 6;
+    const uint32_t half = lane >> 5;
+    const uint32_t l32 = lane & 31;
+    const uint32_t item = blockIdx.x;
+    cu32_p ioff = as_const(p.item_off);
+    if (item >= ioff[p.nlist]) {
+        return;  // the whole workgroup
+    }
+    // Which list: last b with item_off[b] <= item.
+    uint32_t lo_b = 0, hi_b = p.nlist;
+    while (hi_b - lo_b > 1) {
+        const uint32_t mid = (lo_b + hi_b) >> 1;
+        if (ioff[mid] <= item) {
+            lo_b = mid;
+        } else {
+            hi_b = mid;
+        }
+    }
+    const uint32_t b = lo_b;
+    const uint32_t tile_begin = as_const(p.list_tile)[b], tile_end = as_const(p.list_tile)[b + 1];
+    const uint32_t pbeg = as_const(p.pair_off)[b] + (item - ioff[b]) * kIvfI8Pairs + wave * kWave;
+    const uint32_t pend = as_const(p.pair_off)[b + 1];
+    const bool active = pbeg < pend;
+    const uint32_t span = tile_end - tile_begin;
+    const uint32_t nstages = (span + kIvfI8StageTiles - 1) / kIvfI8StageTiles;
+    if (nstages == 0) {
+        return;  // an empty list: its pairs keep their zero counts
+    }
+
+    // Query operands: block j = pairs pbeg + 32 j + lane % 32; step s = granule s, this lane's nibble half.
+    intx4 qv[2][4];
+    int32_t tq[2];
+    uint32_t pair[2], qidx[2];
+    uint32_t ncand[2] = {0, 0};
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint32_t idx = pbeg + 32 * j + l32;
+        const bool live = idx < pend;
+        pair[j] = live ? as_const(p.sorted_pair)[idx] : 0xFFFFFFFFU;
+        qidx[j] = live ? pair[j] / p.nprobe : p.dummy_query;
+        const uint4* rowp = reinterpret_cast<const uint4*>(p.qtab + static_cast<uint64_t>(qidx[j]) * p.qstride);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            uint4 x0 = make_uint4(0, 0, 0, 0), x1 = make_uint4(0, 0, 0, 0);
+            if (static_cast<uint32_t>(s) < p.G) {
+                x0 = rowp[2 * s];
+                x1 = rowp[2 * s + 1];
+            }
+            qv[j][s] = half == 0 ? intx4{static_cast<int>(x0.x), static_cast<int>(x0.z), static_cast<int>(x1.x),
+                                         static_cast<int>(x1.z)}
+                                 : intx4{static_cast<int>(x0.y), static_cast<int>(x0.w), static_cast<int>(x1.y),
+                                         static_cast<int>(x1.w)};
+        }
+        tq[j] = p.tq[qidx[j]];
+    }
+
+    // Staging: wave w copies granule w of both tiles of the stage, a lane per code; the nibbles are split on the
+    // way into LDS.  Wave t also brings the -No terms of tile t.
+    uint4 regs[kIvfI8StageTiles];
+    int32_t my_term = 0;
+    auto fetch = [&](uint32_t sg) {
+#pragma unroll
+        for (int tt = 0; tt < kIvfI8StageTiles; ++tt) {
+            const uint32_t tile = tile_begin + sg * kIvfI8StageTiles + tt;
+            regs[tt] = make_uint4(0, 0, 0, 0);
+            if (tile < tile_end && wave < p.G) {
+                regs[tt] = p.tiles[(static_cast<uint64_t>(tile) * p.G + wave) * kWave + lane];
+            }
+            if (wave == static_cast<uint32_t>(tt)) {
+                my_term = static_cast<int32_t>(0xC0000000U);  // padding tiles: far below any threshold
+                if (tile < tile_end) {
+                    my_term = -static_cast<int32_t>(__uint_as_float(p.meta[static_cast<uint64_t>(tile) * kWave + lane]));
+                }
+            }
+        }
+    };
+    auto park = [&](IvfI8Stage& st) {
+#pragma unroll
+        for (int tt = 0; tt < kIvfI8StageTiles; ++tt) {
+            const uint4 v = regs[tt];
+            st.codes[tt][(2 * wave) * kWave + lane] =
+                make_uint4(v.x & 0x0F0F0F0FU, v.y & 0x0F0F0F0FU, v.z & 0x0F0F0F0FU, v.w & 0x0F0F0F0FU);
+            st.codes[tt][(2 * wave + 1) * kWave + lane] = make_uint4((v.x >> 4) & 0x0F0F0F0FU, (v.y >> 4) & 0x0F0F0F0FU,
+                                                                       (v.z >> 4) & 0x0F0F0F0FU, (v.w >> 4) & 0x0F0F0F0FU);
+            if (wave == static_cast<uint32_t>(tt)) {
+                st.term[tt][lane] = my_term;
+            }
+        }
+    };
+
+    constexpr int kBlocks = 4 * kIvfI8StageTiles;
+    fetch(0);
+    park(stage[0]);
+    __syncthreads();
+    uint32_t cur = 0;
+    for (uint32_t sg = 0; sg < nstages; ++sg) {
+        if (sg + 1 < nstages) {
+            fetch(sg + 1);
+        }
+        if (active) {
+            const IvfI8Stage& st = stage[cur];
+            const uint64_t slot0 = (static_cast<uint64_t>(tile_begin) + sg * kIvfI8StageTiles) * kWave;
+            intx16 acc[2];  // one being filled, one being judged
+            intx4 av[2][4];
+            int32_t tm[2][16];
+            auto read_row = [&](int r) {
+                const int tt = r >> 1, i = r & 1;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const uint4 c = st.codes[tt][(2 * s + half) * kWave + 32 * i + l32];
+                    av[r & 1][s] = intx4{static_cast<int>(c.x), static_cast<int>(c.y), static_cast<int>(c.z),
+                                         static_cast<int>(c.w)};
+                }
+                // Element e of a lane is code 32 i + 8 (e / 4) + 4 (lane / 32) + e % 4 of the tile.
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int4 v = *reinterpret_cast<const int4*>(&st.term[tt][32 * i + 8 * g + 4 * half]);
+                    tm[r & 1][4 * g] = v.x;
+                    tm[r & 1][4 * g + 1] = v.y;
+                    tm[r & 1][4 * g + 2] = v.z;
+                    tm[r & 1][4 * g + 3] = v.w;
+                }
+            };
+            auto multiply = [&](int blk, intx16& c) {
+                const int r = blk >> 1, j = blk & 1;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    c[e] = 0;
+                }
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[r & 1][s], qv[j][s], c, 0, 0, 0);
+                }
+            };
+            read_row(0);
+            multiply(0, acc[0]);
+#pragma unroll
+            for (int blk = 0; blk < kBlocks; ++blk) {
+                const int r = blk >> 1, j = blk & 1;
+                const bool reads = j == 0 && blk + 2 < kBlocks;
+                if (reads) {
+                    read_row(r + 1);
+                }
+                if (blk + 1 < kBlocks) {
+                    multiply(blk + 1, acc[(blk + 1) & 1]);
+                }
+                // The sixteen verdicts stay in scalar registers; only a block with a hit builds a mask per lane.
+                bool pass[16];
+                uint64_t any = 0;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    pass[e] = (acc[blk & 1][e] << 1) + tm[r & 1][e] >= tq[j];
+                    any |= __ballot(pass[e]);
+                }
+                if (blk + 1 < kBlocks) {
+                    if (reads) {
+                        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+                    }
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+                    }
+                }
+                if (any != 0) {
+                    uint32_t bits = 0;
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        bits |= pass[e] ? 1U << e : 0U;
+                    }
+                    while (bits != 0) {
+                        const uint32_t e = static_cast<uint32_t>(__builtin_ctz(bits));
+                        bits &= bits - 1;
+                        const uint64_t slot = slot0 + 32 * r + 8 * (e >> 2) + 4 * half + (e & 3);
+                        const uint32_t id = p.ids[slot];
+                        if (id != VSAG_AMD_INVALID_ID && pair[j] != 0xFFFFFFFFU) {
+                            // The streaming kernel's own three operations on the same integers.
+                            const float result = static_cast<float>(acc[blk & 1][e]);
+                            const float qm = p.qmeta[static_cast<uint64_t>(qidx[j]) * p.qmeta_stride];
+                            const float m0 = __uint_as_float(p.meta[slot]);
+                            const float dist = (qm + m0 - 2 * result) * p.rate;
+                            if (float_to_ordered(dist) <= as_const(p.bound)[qidx[j]]) {
+                                if (ncand[j] < p.k) {
+                                    p.partial[(static_cast<uint64_t>(pair[j]) * 2 + half) * p.k + ncand[j]] =
+                                        make_key(dist, id);
+                                }
+                                ++ncand[j];
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        if (sg + 1 < nstages) {
+            park(stage[cur ^ 1]);
+        }
+        __syncthreads();  // the next stage is complete, and every wave is done with this one
+        cur ^= 1;
+    }
+    if (active) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            if (pair[j] != 0xFFFFFFFFU) {
+                p.partial_cnt[static_cast<uint64_t>(pair[j]) * 2 + half] = ncand[j] < p.k ? ncand[j] : p.k;
+                if (ncand[j] > p.k) {
+                    p.gate[qidx[j]] = 1;
+                }
+            }
+        }
+    }
+}
+
+// Gated queries: the streaming kernel rescans their lists, so what the matrix-core pass left must not count.
+__global__ void __launch_bounds__(256)
+ivf_i8_clear_gated_kernel(const uint32_t* gate, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t* partial_cnt) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const uint64_t per = nprobe - p0;
+    if (i >= nq * per) {
+        return;
+    }
+    const uint64_t q = i / per;
+    if (gate[q] != 0) {
+        const uint64_t pair = q * nprobe + p0 + i % per;
+        partial_cnt[2 * pair] = 0;
+        partial_cnt[2 * pair + 1] = 0;
+    }
+}
+
+bool
+ivf_i8_supports(const vsag_amd_store* s) {
+    return s->kind == VSAG_AMD_KIND_SQ4_UNIFORM && s->metric == VSAG_AMD_METRIC_L2 && s->G <= 4 && s->nlist > 0 &&
+           s->scalar_rate > 0.0F;
+}
+
+// The pairs of probe columns [p0, nprobe) are grouped by list (pair_off, sorted_pair) and item_off counts
+// workgroups of 256 pairs per list; `bound` holds what the first columns left.  tq: nq + 1 words of scratch.
+int
+launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
+              const uint32_t* pair_off, const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound,
+              int32_t* tq, uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st) {
+    hipLaunchKernelGGL(ivf_i8_threshold_kernel, dim3(static_cast<uint32_t>(div_up(nq + 1, 256))), dim3(256), 0, st, bound,
+                       a.qmeta, a.qmeta_stride, a.f1, nq, tq);
+    IvfI8Args p{};
+    p.tiles = s->tiles;
+    p.G = s->G;
+    p.meta = a.meta;
+    p.ids = s->ids_dev;
+    p.list_tile = s->list_tile_dev;
+    p.pair_off = pair_off;
+    p.item_off = item_off;
+    p.sorted_pair = sorted_pair;
+    p.nlist = s->nlist;
+    p.nprobe = nprobe;
+    p.dummy_query = static_cast<uint32_t>(nq);
+    p.qtab = a.qtab;
+    p.qstride = a.qstride;
+    p.qmeta = a.qmeta;
+    p.qmeta_stride = a.qmeta_stride;
+    p.rate = a.f1;
+    p.tq = tq;
+    p.bound = bound;
+    p.k = kcand;
+    p.partial = partial;
+    p.partial_cnt = partial_cnt;
+    p.gate = gate;
+    // At most one partly filled workgroup per probed list.
+    const uint64_t pairs = nq * (nprobe - p0);
+    const uint64_t max_items = div_up(pairs, static_cast<uint64_t>(kIvfI8Pairs)) + std::min<uint64_t>(s->nlist, pairs);
+    hipLaunchKernelGGL(ivf_i8_kernel, dim3(static_cast<uint32_t>(max_items)), dim3(256), 0, st, p);
+    VA_HIP(hipGetLastError());
+    hipLaunchKernelGGL(ivf_i8_clear_gated_kernel, dim3(static_cast<uint32_t>(div_up(pairs, 256))), dim3(256), 0, st, gate,
+                       nq, nprobe, p0, partial_cnt);
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
+}  // namespace vsag_amd

@@ -934,6 +934,21 @@ vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, 
     return 0;
 }
 
+namespace vsag_amd {
+int
+scan_contraction_mode() {
+    return g_prefilter_mode;
+}
+
+// What vsag_amd_last_scan_info reports, for the posting-list scan.
+void
+note_last_scan(int query_tile, uint64_t passes, uint64_t bytes_per_pass) {
+    tl_last_tile = query_tile;
+    tl_last_passes = passes;
+    tl_last_bytes = bytes_per_pass;
+}
+}  // namespace vsag_amd
+
 extern "C" int
 vsag_amd_set_scan_contraction(int mode) {
     VA_CHECK_ARG(mode >= -1 && mode <= 2,
