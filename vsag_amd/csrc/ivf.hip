@@ -38,6 +38,7 @@ uint64_t rabitq_query_code_size(uint32_t dim, int metric, int query_bits);
 int scan_contraction_mode();
 void note_last_scan(int query_tile, uint64_t passes, uint64_t bytes_per_pass);
 bool ivf_i8_supports(const vsag_amd_store* s);
+uint32_t ivf_i8_lists_per_pair();
 int launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
                   const uint32_t* pair_off, const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound,
                   int32_t* tq, uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st);
@@ -267,6 +268,9 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
     if (item >= total) {
         return;
     }
+    if (v.gate != nullptr && as_const(v.gate)[v.dummy_query] == 0) {
+        return;  // word nq of the gate array counts the raised gates: none, nothing to serve
+    }
     // Which list: last b with item_off[b] <= item.
     cu32_p ioff = as_const(v.item_off);
     uint32_t lo = 0, hi = v.nlist;
@@ -306,7 +310,7 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
     for (int t = 0; t < T; ++t) {
         bool live = pbeg + t < pend;
         pair[t] = live ? as_const(v.sorted_pair)[pbeg + t] : 0xFFFFFFFFU;
-        if (live && v.gate != nullptr && as_const(v.gate)[pair[t] / v.nprobe] == 0) {
+        if (live && v.gate != nullptr && as_const(v.gate)[pair[t] / v.nprobe] == 0) {  // (gate[dummy_query] != 0 here)
             live = false;
             pair[t] = 0xFFFFFFFFU;
         }
@@ -691,9 +695,9 @@ plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, 
     // Large batches on sq4_uniform / L2 lists: the streaming kernel scans the nearest list of every query, the int8
     // matrix cores the other columns, into two private lists per (query, list) pair.
     p->mfma = !p->chunked && nprobe > 1 && scan_contraction_mode() >= 0 && ivf_i8_supports(s) &&
-              npairs * 2 * kcand * 8 <= (8ull << 30);
+              npairs * ivf_i8_lists_per_pair() * kcand * 8 <= (8ull << 30);
     if (p->mfma) {
-        p->chunks_max = 2;
+        p->chunks_max = ivf_i8_lists_per_pair();
     }
 }
 
@@ -711,7 +715,7 @@ carve_ivf(Carver& c, const vsag_amd_store* s, const ScanPlanIvf& p, uint64_t nq,
     b->seed = c.take<uint32_t>(p.seeded ? nq * kcand : 0);
     b->partial_cnt = c.take<uint32_t>(p.npairs * p.chunks_max);
     b->partial = c.take<uint64_t>(p.npairs * p.chunks_max * kcand);
-    b->gate = c.take<uint32_t>(p.mfma ? nq : 0);
+    b->gate = c.take<uint32_t>(p.mfma ? nq + 1 : 0);
     b->tq = c.take<int32_t>(p.mfma ? nq + 1 : 0);
     return c.used;
 }
@@ -840,7 +844,7 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
         uint64_t pairs = nq * (p1 - p0);
         if (pass == 1) {
             fill(FillJob{{b.counts, b.cursor, mfma ? b.gate : nullptr, nullptr, nullptr}, {0U, 0U, 0U, 0U, 0U},
-                         {nlists1, nlists1, mfma ? nq : 0, 0, 0}});
+                         {nlists1, nlists1, mfma ? nq + 1 : 0, 0, 0}});
         }
         if (pass == 1 && mfma) {
             // Pairs grouped by list once; workgroups of 256 pairs for the matrix cores, then -- for the queries whose
@@ -848,7 +852,7 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
             hipLaunchKernelGGL(count_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq, nprobe,
                                p0, p1, s->nlist, b.counts);
             hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, st, b.counts, s->list_tile_dev, s->nlist, 256U,
-                               0xFFFFFFFFU, 1U, b.pair_off, b.item_off);
+                               64U, 4U, b.pair_off, b.item_off);  // ivf_i8.hip: kIvfI8ChunkTiles, kIvfI8Chunks
             hipLaunchKernelGGL(scatter_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq,
                                nprobe, p0, p1, s->nlist, b.pair_off, b.cursor, b.sorted_pair);
             VA_TRY(launch_ivf_i8(s, a, nq, nprobe, p0, kcand, b.pair_off, b.item_off, b.sorted_pair, b.bound, b.tq,
@@ -874,7 +878,7 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
                                nprobe, p0, p1, s->nlist, b.pair_off, b.cursor, b.sorted_pair);
         }
         // At most one partly filled query group per probed list, each cut into at most chunks_max items.
-        uint64_t max_items = (div_up(pairs, p.T) + std::min<uint64_t>(s->nlist, pairs)) * p.chunks_max;
+        uint64_t max_items = (div_up(pairs, p.T) + std::min<uint64_t>(s->nlist, pairs)) * (p.chunked ? p.chunks_max : 1);
         dim3 grid(static_cast<uint32_t>(div_up(max_items, waves)));
         VA_TRY(launch_ivf(s, p.T, grid, dim3(waves * kWave), lds, st, a, v));
     }

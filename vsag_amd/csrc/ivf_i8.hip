@@ -29,6 +29,16 @@ typedef int intx16 __attribute__((ext_vector_type(16)));
 
 constexpr uint32_t kIvfI8Pairs = 256;  // pairs per workgroup
 constexpr int kIvfI8StageTiles = 2;
+// Lists are cut into chunks of about kIvfI8ChunkTiles tiles, at most kIvfI8Chunks per list (longer lists get longer
+// chunks), so that one long list does not outlast the rest of the grid.
+constexpr uint32_t kIvfI8ChunkTiles = 64;
+constexpr uint32_t kIvfI8Chunks = 4;
+
+__host__ __device__ inline uint32_t
+ivf_i8_list_chunks(uint32_t tiles) {
+    const uint32_t chunks = (tiles + kIvfI8ChunkTiles - 1) / kIvfI8ChunkTiles;
+    return chunks < kIvfI8Chunks ? chunks : kIvfI8Chunks;
+}
 
 // Per query: Tq = Nq - tmax(bound) (see the header), widened by one level; the slow path re-checks exactly.
 __global__ void __launch_bounds__(256)
@@ -81,9 +91,9 @@ struct IvfI8Args {
     const int32_t* tq;           // per query (+ the dummy row)
     const uint32_t* bound;       // per query, ordered distance
     uint32_t k;                  // capacity of a private list
-    uint64_t* partial;           // [pair][2][k] keys
-    uint32_t* partial_cnt;       // [pair][2]
-    uint32_t* gate;              // per query: raised when one of its lists overflowed
+    uint64_t* partial;           // [pair][chunk][lane / 32][k] keys
+    uint32_t* partial_cnt;       // [pair][chunk][lane / 32]
+    uint32_t* gate;              // per query: raised when one of its lists overflowed; gate[nq] counts them
 };
 
 struct IvfI8Stage {
@@ -115,14 +125,22 @@ ivf_i8_kernel(IvfI8Args p) {
         }
     }
     const uint32_t b = lo_b;
-    const uint32_t tile_begin = as_const(p.list_tile)[b], tile_end = as_const(p.list_tile)[b + 1];
-    const uint32_t pbeg = as_const(p.pair_off)[b] + (item - ioff[b]) * kIvfI8Pairs + wave * kWave;
+    // Items of a list: (block of 256 pairs) x (tile chunk), chunk fastest.
+    const uint32_t list_begin = as_const(p.list_tile)[b], list_end = as_const(p.list_tile)[b + 1];
+    const uint32_t chunks = ivf_i8_list_chunks(list_end - list_begin);
+    const uint32_t per = chunks != 0 ? (list_end - list_begin + chunks - 1) / chunks : 0;
+    const uint32_t chunk = chunks != 0 ? (item - ioff[b]) % chunks : 0;
+    const uint32_t group = chunks != 0 ? (item - ioff[b]) / chunks : 0;
+    uint32_t tile_begin = list_begin + chunk * per;
+    tile_begin = tile_begin < list_end ? tile_begin : list_end;
+    const uint32_t tile_end = tile_begin + per < list_end ? tile_begin + per : list_end;
+    const uint32_t pbeg = as_const(p.pair_off)[b] + group * kIvfI8Pairs + wave * kWave;
     const uint32_t pend = as_const(p.pair_off)[b + 1];
     const bool active = pbeg < pend;
     const uint32_t span = tile_end - tile_begin;
     const uint32_t nstages = (span + kIvfI8StageTiles - 1) / kIvfI8StageTiles;
     if (nstages == 0) {
-        return;  // an empty list: its pairs keep their zero counts
+        return;  // an empty chunk: its lists keep their zero counts
     }
 
     // Query operands: block j = pairs pbeg + 32 j + lane % 32; step s = granule s, this lane's nibble half.
@@ -130,6 +148,7 @@ ivf_i8_kernel(IvfI8Args p) {
     int32_t tq[2];
     uint32_t pair[2], qidx[2];
     uint32_t ncand[2] = {0, 0};
+    uint64_t my_list[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const uint32_t idx = pbeg + 32 * j + l32;
@@ -150,6 +169,7 @@ ivf_i8_kernel(IvfI8Args p) {
                                          static_cast<int>(x1.w)};
         }
         tq[j] = p.tq[qidx[j]];
+        my_list[j] = (static_cast<uint64_t>(live ? pair[j] : 0) * kIvfI8Chunks + chunk) * 2 + half;
     }
 
     // Staging: wave w copies granule w of both tiles of the stage, a lane per code; the nibbles are split on the
@@ -279,8 +299,7 @@ ivf_i8_kernel(IvfI8Args p) {
                             const float dist = (qm + m0 - 2 * result) * p.rate;
                             if (float_to_ordered(dist) <= as_const(p.bound)[qidx[j]]) {
                                 if (ncand[j] < p.k) {
-                                    p.partial[(static_cast<uint64_t>(pair[j]) * 2 + half) * p.k + ncand[j]] =
-                                        make_key(dist, id);
+                                    p.partial[my_list[j] * p.k + ncand[j]] = make_key(dist, id);
                                 }
                                 ++ncand[j];
                             }
@@ -299,9 +318,11 @@ ivf_i8_kernel(IvfI8Args p) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             if (pair[j] != 0xFFFFFFFFU) {
-                p.partial_cnt[static_cast<uint64_t>(pair[j]) * 2 + half] = ncand[j] < p.k ? ncand[j] : p.k;
+                p.partial_cnt[my_list[j]] = ncand[j] < p.k ? ncand[j] : p.k;
                 if (ncand[j] > p.k) {
-                    p.gate[qidx[j]] = 1;
+                    if (atomicExch(&p.gate[qidx[j]], 1U) == 0U) {
+                        atomicAdd(&p.gate[p.dummy_query], 1U);
+                    }
                 }
             }
         }
@@ -317,11 +338,18 @@ ivf_i8_clear_gated_kernel(const uint32_t* gate, uint64_t nq, uint32_t nprobe, ui
         return;
     }
     const uint64_t q = i / per;
-    if (gate[q] != 0) {
+    if (gate[nq] != 0 && gate[q] != 0) {
         const uint64_t pair = q * nprobe + p0 + i % per;
-        partial_cnt[2 * pair] = 0;
-        partial_cnt[2 * pair + 1] = 0;
+        for (uint32_t l = 0; l < 2 * kIvfI8Chunks; ++l) {
+            partial_cnt[2 * kIvfI8Chunks * pair + l] = 0;
+        }
     }
+}
+
+// Private lists per (query, list) pair.
+uint32_t
+ivf_i8_lists_per_pair() {
+    return 2 * kIvfI8Chunks;
 }
 
 bool
@@ -331,7 +359,8 @@ ivf_i8_supports(const vsag_amd_store* s) {
 }
 
 // The pairs of probe columns [p0, nprobe) are grouped by list (pair_off, sorted_pair) and item_off counts
-// workgroups of 256 pairs per list; `bound` holds what the first columns left.  tq: nq + 1 words of scratch.
+// workgroups per list (blocks of 256 pairs x tile chunks: offsets_kernel with T = 256, kIvfI8ChunkTiles,
+// kIvfI8Chunks); `bound` holds what the first columns left.  tq, gate: nq + 1 words each, gate zeroed.
 int
 launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
               const uint32_t* pair_off, const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound,
@@ -361,9 +390,10 @@ launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     p.partial = partial;
     p.partial_cnt = partial_cnt;
     p.gate = gate;
-    // At most one partly filled workgroup per probed list.
+    // At most one partly filled block of pairs per probed list, each cut into at most kIvfI8Chunks items.
     const uint64_t pairs = nq * (nprobe - p0);
-    const uint64_t max_items = div_up(pairs, static_cast<uint64_t>(kIvfI8Pairs)) + std::min<uint64_t>(s->nlist, pairs);
+    const uint64_t max_items =
+        (div_up(pairs, static_cast<uint64_t>(kIvfI8Pairs)) + std::min<uint64_t>(s->nlist, pairs)) * kIvfI8Chunks;
     hipLaunchKernelGGL(ivf_i8_kernel, dim3(static_cast<uint32_t>(max_items)), dim3(256), 0, st, p);
     VA_HIP(hipGetLastError());
     hipLaunchKernelGGL(ivf_i8_clear_gated_kernel, dim3(static_cast<uint32_t>(div_up(pairs, 256))), dim3(256), 0, st, gate,
