@@ -852,7 +852,7 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
             hipLaunchKernelGGL(count_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq, nprobe,
                                p0, p1, s->nlist, b.counts);
             hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, st, b.counts, s->list_tile_dev, s->nlist, 256U,
-                               64U, 4U, b.pair_off, b.item_off);  // ivf_i8.hip: kIvfI8ChunkTiles, kIvfI8Chunks
+                               32U, 4U, b.pair_off, b.item_off);  // ivf_i8.hip: kIvfI8ChunkTiles, kIvfI8Chunks
             hipLaunchKernelGGL(scatter_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq,
                                nprobe, p0, p1, s->nlist, b.pair_off, b.cursor, b.sorted_pair);
             VA_TRY(launch_ivf_i8(s, a, nq, nprobe, p0, kcand, b.pair_off, b.item_off, b.sorted_pair, b.bound, b.tq,

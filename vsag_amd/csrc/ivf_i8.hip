@@ -13,11 +13,11 @@
 // operations.  The kernel serves the probe columns behind the first one: the nearest list of every query has been
 // scanned by the streaming kernel, which leaves the bound.
 //
-// Work split: the (query, list) pairs are grouped by list as for the streaming kernel; a workgroup is a list and up
-// to 256 of its pairs, four waves of 64.  It walks the whole list, two tiles per LDS stage; staging splits the
-// nibbles, so a staged tile looks like eight 16-byte granules per code in the operand order of the instruction.
-// What passes goes into the private list of (pair, lane / 32): no atomics.  A list that overflows raises the
-// query's gate; gated queries drop these lists and are served by the streaming kernel.
+// Work split: the (query, list) pairs are grouped by list as for the streaming kernel; a workgroup is a chunk of a
+// list's tiles and up to 256 of its pairs, four waves of 64.  It walks the chunk two tiles per LDS stage; staging
+// splits the nibbles, so a staged tile looks like eight 16-byte granules per code in the operand order of the
+// instruction.  What passes goes into the private list of (pair, chunk, lane / 32): no atomics.  A list that
+// overflows raises the query's gate; gated queries drop these lists and are served by the streaming kernel.
 #include "distance.h"
 #include "store.h"
 #include "topk.h"
@@ -31,7 +31,7 @@ constexpr uint32_t kIvfI8Pairs = 256;  // pairs per workgroup
 constexpr int kIvfI8StageTiles = 2;
 // Lists are cut into chunks of about kIvfI8ChunkTiles tiles, at most kIvfI8Chunks per list (longer lists get longer
 // chunks), so that one long list does not outlast the rest of the grid.
-constexpr uint32_t kIvfI8ChunkTiles = 64;
+constexpr uint32_t kIvfI8ChunkTiles = 32;
 constexpr uint32_t kIvfI8Chunks = 4;
 
 __host__ __device__ inline uint32_t
