@@ -47,6 +47,9 @@ def _same(a, b):
 def test_matrix_core_columns_equal_streaming(lib, n, d, nlist, nq, nprobe, kcand):
     x, q, cent, labels, codes, (l, dd), st = _case(n + d, n, d, nlist, nq)
     buckets, _ = orc.ivf_route(cent, q, nprobe)
+    buckets = buckets.copy()
+    buckets[70:73, 0] = -1      # three queries without a first list: no bound, served by the direct fallback launch
+    buckets[80, 0] = buckets[80, nprobe - 1]  # a far list first (and probed twice): a loose bound
     plain, fast = _both(lib, st, q, buckets, kcand)
     assert _same(plain, fast)
     # and the checker's distances, bit for bit, on a sample

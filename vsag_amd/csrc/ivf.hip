@@ -41,7 +41,8 @@ bool ivf_i8_supports(const vsag_amd_store* s);
 uint32_t ivf_i8_lists_per_pair();
 int launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
                   const uint32_t* pair_off, const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound,
-                  int32_t* tq, uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st);
+                  int32_t* tq, uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, const int32_t* buckets,
+                  uint32_t* gpairs, uint32_t gpairs_cap, hipStream_t st);
 int prepare_queries(const vsag_amd_store* s, const float* queries, uint64_t nq, uint64_t nq_pad, const QueryLayout& ql,
                     uint32_t* qtab, float* qmeta, uint8_t* qcodes, hipStream_t st);
 ScanArgs make_scan_args(const vsag_amd_store* s, const QueryLayout& ql, const uint32_t* qtab, const float* qmeta);
@@ -252,6 +253,13 @@ struct IvfArgs {
     uint64_t* partial;           // npairs_total x chunks_max x k keys
     uint32_t* partial_cnt;       // npairs_total x chunks_max
     const uint32_t* gate;        // per query, or null: only queries with a raised gate are served
+    // Direct mode (non-null `direct`): the work is a short array of pairs instead of the per-list grouping;
+    // direct_count[0] of them, each worth chunks_max consecutive items.  More than direct_cap pairs are left to a
+    // launch over the grouping (which in turn stands back when direct mode can take them).
+    const uint32_t* direct;
+    const uint32_t* direct_count;
+    uint32_t direct_cap;
+    const int32_t* buckets;      // direct mode: list of a pair
 };
 
 constexpr uint32_t kIvfSeedTiles = 4;
@@ -264,31 +272,59 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t item = blockIdx.x * (blockDim.x >> 6) + wave;
-    const uint32_t total = as_const(v.item_off)[v.nlist];
-    if (item >= total) {
-        return;
-    }
-    if (v.gate != nullptr && as_const(v.gate)[v.dummy_query] == 0) {
-        return;  // word nq of the gate array counts the raised gates: none, nothing to serve
-    }
-    // Which list: last b with item_off[b] <= item.
-    cu32_p ioff = as_const(v.item_off);
-    uint32_t lo = 0, hi = v.nlist;
-    while (hi - lo > 1) {
-        uint32_t mid = (lo + hi) >> 1;
-        if (ioff[mid] <= item) {
-            lo = mid;
-        } else {
-            hi = mid;
+    uint32_t list_begin, list_end, local, pfirst, plast;
+    cu32_p pairs_src = as_const(v.sorted_pair);
+    if (v.direct != nullptr) {
+        const uint32_t count = as_const(v.direct_count)[0];
+        const uint32_t vi = item / v.chunks_max;
+        if (count > v.direct_cap || vi >= count) {
+            return;
         }
+        pairs_src = as_const(v.direct);
+        const int32_t bk = v.buckets[pairs_src[vi]];  // a real list: pairs without one are never queued
+        list_begin = as_const(v.list_tile)[bk];
+        list_end = as_const(v.list_tile)[bk + 1];
+        local = item % v.chunks_max;
+        pfirst = vi;
+        plast = vi + 1;
+    } else {
+        const uint32_t total = as_const(v.item_off)[v.nlist];
+        if (item >= total) {
+            return;
+        }
+        if (v.gate != nullptr) {
+            // Words nq and nq + 1 of the gate array count the raised gates and their pairs: nothing to serve, or
+            // few enough for the direct launch.
+            const uint32_t raised = as_const(v.gate)[v.dummy_query];
+            if (raised == 0 || (v.direct_cap != 0 && as_const(v.gate)[v.dummy_query + 1] <= v.direct_cap)) {
+                return;
+            }
+        }
+        // Which list: last b with item_off[b] <= item.
+        cu32_p ioff = as_const(v.item_off);
+        uint32_t lo = 0, hi = v.nlist;
+        while (hi - lo > 1) {
+            uint32_t mid = (lo + hi) >> 1;
+            if (ioff[mid] <= item) {
+                lo = mid;
+            } else {
+                hi = mid;
+            }
+        }
+        list_begin = as_const(v.list_tile)[lo];
+        list_end = as_const(v.list_tile)[lo + 1];
+        local = item - ioff[lo];
+        pfirst = as_const(v.pair_off)[lo];
+        plast = as_const(v.pair_off)[lo + 1];
     }
-    const uint32_t b = lo;
-    const uint32_t list_begin = as_const(v.list_tile)[b], list_end = as_const(v.list_tile)[b + 1];
-    uint32_t group = item - ioff[b], chunk = 0;
+    uint32_t group = local, chunk = 0;
     uint32_t tbeg = list_begin, tend = list_end;
     if (CHUNKED) {
         const uint32_t tiles = list_end - list_begin;
         const uint32_t chunks = list_chunks(tiles, v.tiles_per_item, v.chunks_max);
+        if (chunks == 0) {
+            return;
+        }
         const uint32_t per = (tiles + chunks - 1) / chunks;
         chunk = group % chunks;
         group = group / chunks;
@@ -296,8 +332,8 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
         tbeg = tbeg < list_end ? tbeg : list_end;
         tend = tbeg + per < list_end ? tbeg + per : list_end;
     }
-    const uint32_t pbeg = as_const(v.pair_off)[b] + group * T;
-    const uint32_t pend = as_const(v.pair_off)[b + 1];
+    const uint32_t pbeg = pfirst + group * T;
+    const uint32_t pend = plast;
 
     const uint32_t S = v.S, k = v.k;
     uint64_t* sel = lds + static_cast<size_t>(wave) * T * S;
@@ -309,8 +345,8 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
 #pragma unroll
     for (int t = 0; t < T; ++t) {
         bool live = pbeg + t < pend;
-        pair[t] = live ? as_const(v.sorted_pair)[pbeg + t] : 0xFFFFFFFFU;
-        if (live && v.gate != nullptr && as_const(v.gate)[pair[t] / v.nprobe] == 0) {  // (gate[dummy_query] != 0 here)
+        pair[t] = live ? pairs_src[pbeg + t] : 0xFFFFFFFFU;
+        if (live && v.gate != nullptr && as_const(v.gate)[pair[t] / v.nprobe] == 0) {
             live = false;
             pair[t] = 0xFFFFFFFFU;
         }
@@ -645,9 +681,13 @@ struct IvfBuffers {
     uint32_t* seed;
     uint32_t* partial_cnt;
     uint64_t* partial;
-    uint32_t* gate;       // mfma: nq
+    uint32_t* gate;       // mfma: nq + 2 (flags, raised gates, their pairs)
     int32_t* tq;          // mfma: nq + 1
+    uint32_t* gpairs;     // mfma: pairs of gated queries, kGatedPairsCap
 };
+
+// Pairs of gated queries the direct fallback launch takes; more go through the per-list grouping.
+constexpr uint32_t kGatedPairsCap = 4096;
 
 static void
 plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, ScanPlanIvf* p) {
@@ -715,7 +755,8 @@ carve_ivf(Carver& c, const vsag_amd_store* s, const ScanPlanIvf& p, uint64_t nq,
     b->seed = c.take<uint32_t>(p.seeded ? nq * kcand : 0);
     b->partial_cnt = c.take<uint32_t>(p.npairs * p.chunks_max);
     b->partial = c.take<uint64_t>(p.npairs * p.chunks_max * kcand);
-    b->gate = c.take<uint32_t>(p.mfma ? nq + 1 : 0);
+    b->gate = c.take<uint32_t>(p.mfma ? nq + 2 : 0);
+    b->gpairs = c.take<uint32_t>(p.mfma ? kGatedPairsCap : 0);
     b->tq = c.take<int32_t>(p.mfma ? nq + 1 : 0);
     return c.used;
 }
@@ -844,7 +885,7 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
         uint64_t pairs = nq * (p1 - p0);
         if (pass == 1) {
             fill(FillJob{{b.counts, b.cursor, mfma ? b.gate : nullptr, nullptr, nullptr}, {0U, 0U, 0U, 0U, 0U},
-                         {nlists1, nlists1, mfma ? nq + 1 : 0, 0, 0}});
+                         {nlists1, nlists1, mfma ? nq + 2 : 0, 0, 0}});
         }
         if (pass == 1 && mfma) {
             // Pairs grouped by list once; workgroups of 256 pairs for the matrix cores, then -- for the queries whose
@@ -856,10 +897,25 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
             hipLaunchKernelGGL(scatter_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq,
                                nprobe, p0, p1, s->nlist, b.pair_off, b.cursor, b.sorted_pair);
             VA_TRY(launch_ivf_i8(s, a, nq, nprobe, p0, kcand, b.pair_off, b.item_off, b.sorted_pair, b.bound, b.tq,
-                                 b.partial, b.partial_cnt, b.gate, st));
+                                 b.partial, b.partial_cnt, b.gate, buckets_dev, b.gpairs, kGatedPairsCap, st));
+            // Few gated pairs (the usual case): one wave per pair and chunk of its list.
+            IvfArgs d = v;
+            d.direct = b.gpairs;
+            d.direct_count = b.gate + nq + 1;
+            d.direct_cap = kGatedPairsCap;
+            d.buckets = buckets_dev;
+            d.tiles_per_item = 16;
+            uint32_t dwaves = 4;
+            while (dwaves > 1 && static_cast<size_t>(dwaves) * p.S * 8 > 65536) {
+                dwaves >>= 1;
+            }
+            dim3 dgrid(static_cast<uint32_t>(div_up(static_cast<uint64_t>(kGatedPairsCap) * d.chunks_max, dwaves)));
+            VA_TRY(launch_ivf(s, 1, dgrid, dim3(dwaves * kWave), static_cast<size_t>(dwaves) * p.S * 8, st, a, d));
+            // Many: the streaming kernel's items over the same grouping (stands back otherwise).
             hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, st, b.counts, s->list_tile_dev, s->nlist,
                                static_cast<uint32_t>(p.T), 0xFFFFFFFFU, 1U, b.pair_off, b.item_off);
             v.gate = b.gate;
+            v.direct_cap = kGatedPairsCap;
             uint64_t max_items = div_up(pairs, p.T) + std::min<uint64_t>(s->nlist, pairs);
             dim3 grid(static_cast<uint32_t>(div_up(max_items, waves)));
             VA_TRY(launch_ivf(s, p.T, grid, dim3(waves * kWave), lds, st, a, v));

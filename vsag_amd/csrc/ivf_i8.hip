@@ -329,19 +329,27 @@ ivf_i8_kernel(IvfI8Args p) {
     }
 }
 
-// Gated queries: the streaming kernel rescans their lists, so what the matrix-core pass left must not count.
+// Gated queries: the streaming kernel rescans their lists, so what the matrix-core pass left must not count.  Their
+// pairs with a list are queued for that rescan (gate[nq + 1] counts them, also beyond the queue's capacity).
 __global__ void __launch_bounds__(256)
-ivf_i8_clear_gated_kernel(const uint32_t* gate, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t* partial_cnt) {
+ivf_i8_clear_gated_kernel(uint32_t* gate, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t* partial_cnt,
+                          const int32_t* buckets, uint32_t* gpairs, uint32_t gpairs_cap) {
     const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     const uint64_t per = nprobe - p0;
-    if (i >= nq * per) {
+    if (i >= nq * per || gate[nq] == 0) {
         return;
     }
     const uint64_t q = i / per;
-    if (gate[nq] != 0 && gate[q] != 0) {
+    if (gate[q] != 0) {
         const uint64_t pair = q * nprobe + p0 + i % per;
         for (uint32_t l = 0; l < 2 * kIvfI8Chunks; ++l) {
             partial_cnt[2 * kIvfI8Chunks * pair + l] = 0;
+        }
+        if (buckets[pair] >= 0) {
+            const uint32_t pos = atomicAdd(&gate[nq + 1], 1U);
+            if (pos < gpairs_cap) {
+                gpairs[pos] = static_cast<uint32_t>(pair);
+            }
         }
     }
 }
@@ -360,11 +368,12 @@ ivf_i8_supports(const vsag_amd_store* s) {
 
 // The pairs of probe columns [p0, nprobe) are grouped by list (pair_off, sorted_pair) and item_off counts
 // workgroups per list (blocks of 256 pairs x tile chunks: offsets_kernel with T = 256, kIvfI8ChunkTiles,
-// kIvfI8Chunks); `bound` holds what the first columns left.  tq, gate: nq + 1 words each, gate zeroed.
+// kIvfI8Chunks); `bound` holds what the first columns left.  tq: nq + 1 words; gate: nq + 2 words, zeroed.
 int
 launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
               const uint32_t* pair_off, const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound,
-              int32_t* tq, uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st) {
+              int32_t* tq, uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, const int32_t* buckets,
+              uint32_t* gpairs, uint32_t gpairs_cap, hipStream_t st) {
     hipLaunchKernelGGL(ivf_i8_threshold_kernel, dim3(static_cast<uint32_t>(div_up(nq + 1, 256))), dim3(256), 0, st, bound,
                        a.qmeta, a.qmeta_stride, a.f1, nq, tq);
     IvfI8Args p{};
@@ -397,7 +406,7 @@ launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     hipLaunchKernelGGL(ivf_i8_kernel, dim3(static_cast<uint32_t>(max_items)), dim3(256), 0, st, p);
     VA_HIP(hipGetLastError());
     hipLaunchKernelGGL(ivf_i8_clear_gated_kernel, dim3(static_cast<uint32_t>(div_up(pairs, 256))), dim3(256), 0, st, gate,
-                       nq, nprobe, p0, partial_cnt);
+                       nq, nprobe, p0, partial_cnt, buckets, gpairs, gpairs_cap);
     VA_HIP(hipGetLastError());
     return 0;
 }
