@@ -504,6 +504,8 @@ def run_c4(env):
                 t_one.append(time.perf_counter() - t0)
         single = {"latency_us": 1e6 * float(np.mean(t_one)), "queries_per_second_one_at_a_time": 1.0 / float(np.mean(t_one))}
     sec, kms = env.timed(step, args.steps, args.warmup)
+    tile = C.c_int()
+    lib.vsag_amd_last_scan_info(C.byref(tile), None, None)  # 256: the int8 matrix cores took columns 1..nprobe-1
     ids = out_i.to_numpy(np.uint32, (nq, k))
     b = buckets.to_numpy(np.int32, (nq, nprobe))
     scanned = sizes[b.clip(0)].astype(np.int64).sum()  # codes scanned per step, summed over queries
@@ -570,12 +572,26 @@ def run_c4(env):
     # configuration, profiles/ivf_scan_sq4u_c4.md.  Work items that share a list are co-scheduled and read it
     # through L2 once per <= 4 queries, so the fraction against HBM exceeds 1: this kernel is bound by VALU issue.
     traffic = None
-    if (n, d, nq, k, nlist) == (10000000, 128, 10000, 10, 4096):
-        traffic = (483541.75 + 1699620.5) * 2.00 * 1024 + (9817.03 + 19921.13) * 1024
+    if (n, d, nq, k, nlist) == (10000000, 128, 10000, 10, 4096) and tile.value != 256:
+        traffic = (482513.06 + 1698762.06) * 2.00 * 1024 + (9817.03 + 19915.53) * 1024
     roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
             "traffic": traffic, "kernel": "ivf_scan_kernel<sq4_uniform, l2> (2 launches per step)", "kernel_ms": kms,
             "algorithmic_bytes_per_launch": algo,
             "distance_evaluations_per_second": float(scanned) / (kms * 1e-3)}
+    if tile.value == 256:
+        # The probe columns behind the first went through the int8 matrix cores; the timed kernel is that pass alone:
+        # every code of those lists against every query probing them, 2 x 128 integer operations per pair.
+        rest = sizes[b[:, 1:].clip(0)].astype(np.int64).sum() - (b[:, 1:] < 0).sum() * int(sizes[0])
+        ops = 2.0 * (-(-d // 32) * 32) * float(rest)
+        tops = ops / (kms * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": tops, "peak": MFMA_I8_PEAK_TOPS, "unit": "TOP/s",
+                "frac": tops / MFMA_I8_PEAK_TOPS,
+                # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this launch: profiles/ivf_i8_sq4u_c4.md
+                "traffic": 493403.25 * 2.00 * 1024 + 73485.56 * 1024
+                if (n, d, nq, k, nlist) == (10000000, 128, 10000, 10, 4096) else None,
+                "kernel": "ivf_i8_kernel (int8 MFMA, probe columns 1..%d)" % (nprobe - 1), "kernel_ms": kms,
+                "ops_per_launch": ops, "distance_evaluations_per_launch": float(rest),
+                "distance_evaluations_per_second": float(rest) / (kms * 1e-3)}
     return env.base_line("QPS @ recall@10 (IVF SQ4-uniform, 10M x 128)", "queries/s", nq / sec, sec,
                          "u4 codes, i32 dot", "configs[3]: IVF search, N=%d, d=%d, nlist=%d, nprobe=%d, rerank %d, "
                          "%d queries, k=%d" % (n, d, nlist, nprobe, kcand, nq, k),

@@ -938,7 +938,9 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
         dim3 grid(static_cast<uint32_t>(div_up(max_items, waves)));
         VA_TRY(launch_ivf(s, p.T, grid, dim3(waves * kWave), lds, st, a, v));
     }
-    timing_end(st);
+    if (!mfma) {
+        timing_end(st);  // the matrix-core pass is timed on its own (ivf_i8.hip)
+    }
     note_last_scan(mfma ? 256 : p.T, 0, 0);
     return launch_merge_partials(b.partial, b.partial_cnt, b.bound, nprobe * p.chunks_max, nprobe * p.chunks_max, kcand,
                                  p.S, nq, ids_dev, dists_dev, st);

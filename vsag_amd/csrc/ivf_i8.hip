@@ -24,6 +24,9 @@
 
 namespace vsag_amd {
 
+void timing_begin(hipStream_t st);
+void timing_end(hipStream_t st);
+
 typedef int intx4 __attribute__((ext_vector_type(4)));
 typedef int intx16 __attribute__((ext_vector_type(16)));
 
@@ -403,7 +406,9 @@ launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     const uint64_t pairs = nq * (nprobe - p0);
     const uint64_t max_items =
         (div_up(pairs, static_cast<uint64_t>(kIvfI8Pairs)) + std::min<uint64_t>(s->nlist, pairs)) * kIvfI8Chunks;
+    timing_begin(st);
     hipLaunchKernelGGL(ivf_i8_kernel, dim3(static_cast<uint32_t>(max_items)), dim3(256), 0, st, p);
+    timing_end(st);
     VA_HIP(hipGetLastError());
     hipLaunchKernelGGL(ivf_i8_clear_gated_kernel, dim3(static_cast<uint32_t>(div_up(pairs, 256))), dim3(256), 0, st, gate,
                        nq, nprobe, p0, partial_cnt, buckets, gpairs, gpairs_cap);
