@@ -722,8 +722,9 @@ def main():
     ap.add_argument("--no-single", action="store_true", help="skip the one-query-per-call measurement")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py measures one GPU: the search core is single-GPU by design (DESIGN.md says how it would "
-              "shard); --gpus %d is not supported" % args.gpus, file=sys.stderr)
+        print("bench.py measures one GPU: the search core is single-GPU by design (sharding it means splitting "
+              "the base rows or posting lists and merging nq x k results); --gpus %d is not supported" % args.gpus,
+              file=sys.stderr)
         sys.exit(2)
     env = Env(args)
     env.capi.check(env.lib.vsag_amd_set_scan_contraction(args.contraction))

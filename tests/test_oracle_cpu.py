@@ -102,7 +102,7 @@ def test_rabitq_binary_ip_known_answers():
 
 
 def test_code_sizes_of_the_benchmark_configs():
-    # SURVEY-independent arithmetic from the constructors: sq4_uniform_quantizer.cpp:33-72 (d=128, l2 -> 64+8),
+    # the arithmetic of the constructors: sq4_uniform_quantizer.cpp:33-72 (d=128, l2 -> 64+8),
     # rabitq_quantizer.cpp:102-133 (d=768, ip, 4-bit query -> 96 + 4*4), query 4 planes of 128 B + 5 floats.
     assert orc.squ_code_size(128, 4, orc.L2) == 72
     assert orc.squ_code_size(128, 8, orc.L2) == 136 and orc.squ_code_size(128, 8, orc.IP) == 132
