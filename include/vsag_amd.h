@@ -196,7 +196,7 @@ VSAG_AMD_API int vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* store, const
 
 /* Large batches on flat fp32 / sq8 stores are served by a matrix-core contraction that pre-selects candidates,
  * which are then recomputed and selected exactly as the streaming scan does (same results, bit for bit).
- * Posting lists of sq4_uniform / L2 codes of at most 128 dimensions scan the probe columns behind the first on the
+ * Posting lists of sq4_uniform codes of at most 128 dimensions (any metric) scan the probe columns behind the first on the
  * int8 matrix cores when a batch has at least 8192 (query, list) groups (same results; off with mode -1).
  * sq8 stores of at most 128 dimensions pre-select on the int8 matrix cores (queries split into two int8 planes
  * with a rigorous bound on the remainder), the others on the fp32 matrix cores.

@@ -11,15 +11,15 @@ from vsag_amd import capi
 pytestmark = pytest.mark.gpu
 
 
-def _case(seed, n, d, nlist, nq, components=40, sigma=0.05):
+def _case(seed, n, d, nlist, nq, components=40, sigma=0.05, metric=orc.L2):
     rng = np.random.default_rng(seed)
     x, means = gaussian_mixture(rng, n, d, components, sigma)
     q, _ = gaussian_mixture(rng, nq, d, components, sigma, means=means)
     cent = x[rng.choice(n, nlist, replace=False)].copy()
     labels, _, _ = orc.kmeans_assign(x, cent)
-    l, dd = orc.sq_train_uniform(x, 4, orc.L2, mode=3)
-    codes = orc.squ_encode(x, 4, l, dd, orc.L2)
-    st = Store(capi.KIND_SQ4_UNIFORM, orc.L2, d, bounds=[l, dd])
+    l, dd = orc.sq_train_uniform(x, 4, metric, mode=3)
+    codes = orc.squ_encode(x, 4, l, dd, metric)
+    st = Store(capi.KIND_SQ4_UNIFORM, metric, d, bounds=[l, dd])
     st.set_lists(codes, labels, nlist)
     return x, q, cent, labels, codes, (l, dd), st
 
@@ -81,4 +81,22 @@ def test_missing_buckets_and_ragged_lists(lib):
     buckets[1::7, 0] = -1       # no first list at all: no bound, everything overflows
     plain, fast = _both(lib, st, q, buckets, kcand)
     assert _same(plain, fast)
+    st.destroy()
+
+
+@pytest.mark.parametrize("metric", [orc.IP, orc.COSINE])
+@pytest.mark.parametrize("n,d,nlist,nq,nprobe,kcand", [(60000, 128, 64, 2100, 16, 100), (30000, 100, 37, 4500, 8, 10)])
+def test_inner_product_and_cosine_columns_equal_streaming(lib, metric, n, d, nlist, nq, nprobe, kcand):
+    """No integer form for these metrics: a float threshold with every rounding charged against it, then the
+    streaming kernel's own operations on what passes."""
+    x, q, cent, labels, codes, (l, dd), st = _case(n + d + metric, n, d, nlist, nq, metric=metric)
+    buckets, _ = orc.ivf_route(cent, q, nprobe)
+    buckets = buckets.copy()
+    buckets[70:73, 0] = -1
+    plain, fast = _both(lib, st, q, buckets, kcand)
+    assert _same(plain, fast)
+    offsets, order = orc.ivf_build_lists(labels, nlist)
+    qproc = orc.squ_encode(q[:64], 4, l, dd, metric)
+    _, rds = orc.ivf_scan(orc.SQ4U, metric, d, codes[order], offsets, order, qproc, buckets[:64], kcand, lb=l, diff=dd)
+    assert np.array_equal(fast[1][:64].view(np.uint32), rds.view(np.uint32))
     st.destroy()

@@ -1,5 +1,4 @@
-// Posting lists of sq4_uniform codes (L2, at most 128 dimensions) against large query batches, on the int8 matrix
-// cores.
+// Posting lists of sq4_uniform codes (at most 128 dimensions) against large query batches, on the int8 matrix cores.
 //
 // The streaming IVF kernel (ivf.hip) is bound by vector-ALU issue: every (query, code) pair costs sixteen dot4
 // instructions.  The distance of this quantizer is a function of integers only,
@@ -10,7 +9,10 @@
 // delivers <q, o> exactly.  "dist <= bound" is therefore the integer test 2 <q, o> - No >= Nq - tmax(bound), where
 // tmax is the largest integer t with fl(t * scalar_rate) <= bound; the pairs that pass are exactly the ones the
 // streaming kernel would admit under the same bound, and their distances are formed by the same three fp32
-// operations.  The kernel serves the probe columns behind the first one: the nearest list of every query has been
+// operations.  Inner product and cosine, dist = 1 - (lb (sum_q + sum_o) + rate <q, o> + lb^2), have no integer form:
+// there the test is float(<q, o>) >= A_q + g * sum_o with every rounding of the streaming formula (and of the test)
+// charged against A_q, and what passes is re-checked with the streaming kernel's own operations.
+// The kernel serves the probe columns behind the first one: the nearest list of every query has been
 // scanned by the streaming kernel, which leaves the bound.
 //
 // Work split: the (query, list) pairs are grouped by list as for the streaming kernel; a workgroup is a chunk of a
@@ -45,22 +47,43 @@ ivf_i8_list_chunks(uint32_t tiles) {
 
 // Per query: Tq = Nq - tmax(bound) (see the header), widened by one level; the slow path re-checks exactly.
 __global__ void __launch_bounds__(256)
-ivf_i8_threshold_kernel(const uint32_t* bound, const float* qmeta, uint32_t qmeta_stride, float rate, uint64_t nq,
-                        int32_t* tq) {
+ivf_i8_threshold_kernel(const uint32_t* bound, const float* qmeta, uint32_t qmeta_stride, int is_l2, float lb, float rate,
+                        float lb2, uint32_t dpad, uint64_t nq, int32_t* tq) {
     const uint64_t q = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (q > nq) {
         return;
     }
+    // Inner product: tq holds the bits of the float A_q.
+    const int32_t never = is_l2 ? 0x7FFFFFFF : 0x7F800000, always = static_cast<int32_t>(is_l2 ? 0x80000000U : 0xFF800000U);
     if (q == nq) {
-        tq[q] = 0x7FFFFFFF;  // the all-zero query row idle lanes point at: nothing passes
+        tq[q] = never;  // the all-zero query row idle lanes point at: nothing passes
         return;
     }
     const uint32_t b = bound[q];
     if (b == 0xFFFFFFFFU || !(rate > 0.0F)) {
-        tq[q] = static_cast<int32_t>(0x80000000U);  // no bound: everything passes (and the query will overflow)
+        tq[q] = always;  // no bound: everything passes (and the query will overflow)
         return;
     }
     const float bd = ordered_to_float(b);
+    if (!is_l2) {
+        // out = fl(1 - fl(fl(fl(lb fl(qm + m0)) + fl(rate ip)) + lb2)) <= bd.  With the real r* = lb (qm + m0) +
+        // rate ip + lb2: |r - r*| and the rounding of 1 - r stay below 8u of the magnitudes involved, so
+        // out <= bd implies rate ip >= 1 - bd - lb2 - lb qm - lb m0 - eps.
+        constexpr double kU = 5.9604644775390625e-8;
+        const double qm = static_cast<double>(qmeta[q * qmeta_stride]);
+        const double m0_max = 15.0 * dpad, ip_max = 225.0 * dpad;
+        const double mag = fabs(static_cast<double>(lb)) * (fabs(qm) + m0_max) + static_cast<double>(rate) * ip_max +
+                           fabs(static_cast<double>(lb2)) + 1.0 + fabs(static_cast<double>(bd));
+        double aq = (1.0 - bd - lb2 - static_cast<double>(lb) * qm - 16.0 * kU * mag) / static_cast<double>(rate);
+        // the test adds fl(g m0) to A_q in fp32
+        aq -= 8.0 * kU * (fabs(aq) + fabs(static_cast<double>(lb) / rate) * m0_max + ip_max);
+        float f = static_cast<float>(aq);
+        if (static_cast<double>(f) > aq) {
+            f = nextafterf(f, -__builtin_inff());
+        }
+        tq[q] = __float_as_int(f);
+        return;
+    }
     const double t0 = floor(static_cast<double>(bd) / static_cast<double>(rate));
     int64_t t = t0 > 1.0e9 ? 1000000000LL : (t0 < -1.0e9 ? -1000000000LL : static_cast<int64_t>(t0));
     for (int i = 0; i < 4 && static_cast<float>(t + 1) * rate <= bd; ++i) {
@@ -90,7 +113,7 @@ struct IvfI8Args {
     uint32_t qstride;
     const float* qmeta;
     uint32_t qmeta_stride;
-    float rate;
+    float lb, rate, lb2;         // the quantizer's constants (distance.h: f0, f1, f2)
     const int32_t* tq;           // per query (+ the dummy row)
     const uint32_t* bound;       // per query, ordered distance
     uint32_t k;                  // capacity of a private list
@@ -104,6 +127,7 @@ struct IvfI8Stage {
     int32_t term[kIvfI8StageTiles][kWave];     // -No per code
 };
 
+template <int METRIC>
 __global__ void __launch_bounds__(256, 2)
 ivf_i8_kernel(IvfI8Args p) {
     __shared__ IvfI8Stage stage[2];
@@ -188,9 +212,12 @@ ivf_i8_kernel(IvfI8Args p) {
                 regs[tt] = p.tiles[(static_cast<uint64_t>(tile) * p.G + wave) * kWave + lane];
             }
             if (wave == static_cast<uint32_t>(tt)) {
-                my_term = static_cast<int32_t>(0xC0000000U);  // padding tiles: far below any threshold
+                // l2: -No; inner product: the bits of g * sum_o, g = -lb / rate.  Padding tiles never pass.
+                my_term = METRIC == VSAG_AMD_METRIC_L2 ? static_cast<int32_t>(0xC0000000U) : 0x7F800000;
                 if (tile < tile_end) {
-                    my_term = -static_cast<int32_t>(__uint_as_float(p.meta[static_cast<uint64_t>(tile) * kWave + lane]));
+                    const float m0 = __uint_as_float(p.meta[static_cast<uint64_t>(tile) * kWave + lane]);
+                    my_term = METRIC == VSAG_AMD_METRIC_L2 ? -static_cast<int32_t>(m0)
+                                                           : __float_as_int(m0 * (-p.lb / p.rate));
                 }
             }
         }
@@ -270,7 +297,12 @@ ivf_i8_kernel(IvfI8Args p) {
                 uint64_t any = 0;
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    pass[e] = (acc[blk & 1][e] << 1) + tm[r & 1][e] >= tq[j];
+                    if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                        pass[e] = (acc[blk & 1][e] << 1) + tm[r & 1][e] >= tq[j];
+                    } else {
+                        pass[e] = static_cast<float>(acc[blk & 1][e]) >=
+                                  __int_as_float(tm[r & 1][e]) + __int_as_float(tq[j]);
+                    }
                     any |= __ballot(pass[e]);
                 }
                 if (blk + 1 < kBlocks) {
@@ -280,7 +312,7 @@ ivf_i8_kernel(IvfI8Args p) {
 #pragma unroll
                     for (int m = 0; m < 4; ++m) {
                         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, METRIC == VSAG_AMD_METRIC_L2 ? 8 : 12, 0);
                     }
                 }
                 if (any != 0) {
@@ -299,7 +331,13 @@ ivf_i8_kernel(IvfI8Args p) {
                             const float result = static_cast<float>(acc[blk & 1][e]);
                             const float qm = p.qmeta[static_cast<uint64_t>(qidx[j]) * p.qmeta_stride];
                             const float m0 = __uint_as_float(p.meta[slot]);
-                            const float dist = (qm + m0 - 2 * result) * p.rate;
+                            float dist;
+                            if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                                dist = (qm + m0 - 2 * result) * p.rate;
+                            } else {
+                                const float rr = p.lb * (qm + m0) + p.rate * result + p.lb2;
+                                dist = 1 - rr;
+                            }
                             if (float_to_ordered(dist) <= as_const(p.bound)[qidx[j]]) {
                                 if (ncand[j] < p.k) {
                                     p.partial[my_list[j] * p.k + ncand[j]] = make_key(dist, id);
@@ -365,8 +403,7 @@ ivf_i8_lists_per_pair() {
 
 bool
 ivf_i8_supports(const vsag_amd_store* s) {
-    return s->kind == VSAG_AMD_KIND_SQ4_UNIFORM && s->metric == VSAG_AMD_METRIC_L2 && s->G <= 4 && s->nlist > 0 &&
-           s->scalar_rate > 0.0F;
+    return s->kind == VSAG_AMD_KIND_SQ4_UNIFORM && s->G <= 4 && s->nlist > 0 && s->scalar_rate > 0.0F;
 }
 
 // The pairs of probe columns [p0, nprobe) are grouped by list (pair_off, sorted_pair) and item_off counts
@@ -377,8 +414,9 @@ launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
               const uint32_t* pair_off, const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound,
               int32_t* tq, uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, const int32_t* buckets,
               uint32_t* gpairs, uint32_t gpairs_cap, hipStream_t st) {
+    const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
     hipLaunchKernelGGL(ivf_i8_threshold_kernel, dim3(static_cast<uint32_t>(div_up(nq + 1, 256))), dim3(256), 0, st, bound,
-                       a.qmeta, a.qmeta_stride, a.f1, nq, tq);
+                       a.qmeta, a.qmeta_stride, l2 ? 1 : 0, a.f0, a.f1, a.f2, s->dpad, nq, tq);
     IvfI8Args p{};
     p.tiles = s->tiles;
     p.G = s->G;
@@ -395,7 +433,9 @@ launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     p.qstride = a.qstride;
     p.qmeta = a.qmeta;
     p.qmeta_stride = a.qmeta_stride;
+    p.lb = a.f0;
     p.rate = a.f1;
+    p.lb2 = a.f2;
     p.tq = tq;
     p.bound = bound;
     p.k = kcand;
@@ -407,7 +447,11 @@ launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     const uint64_t max_items =
         (div_up(pairs, static_cast<uint64_t>(kIvfI8Pairs)) + std::min<uint64_t>(s->nlist, pairs)) * kIvfI8Chunks;
     timing_begin(st);
-    hipLaunchKernelGGL(ivf_i8_kernel, dim3(static_cast<uint32_t>(max_items)), dim3(256), 0, st, p);
+    if (l2) {
+        hipLaunchKernelGGL(ivf_i8_kernel<VSAG_AMD_METRIC_L2>, dim3(static_cast<uint32_t>(max_items)), dim3(256), 0, st, p);
+    } else {
+        hipLaunchKernelGGL(ivf_i8_kernel<VSAG_AMD_METRIC_IP>, dim3(static_cast<uint32_t>(max_items)), dim3(256), 0, st, p);
+    }
     timing_end(st);
     VA_HIP(hipGetLastError());
     hipLaunchKernelGGL(ivf_i8_clear_gated_kernel, dim3(static_cast<uint32_t>(div_up(pairs, 256))), dim3(256), 0, st, gate,
