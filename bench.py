@@ -301,6 +301,7 @@ def run_c2(env):
                 "kernel_ms": r["kernel_ms"], "flops_per_launch": flops,
                 "algorithmic_bytes_per_launch": algo_bytes, "algorithmic_gbs": achieved}
     return env.base_line("QPS @ recall@10 (1M x 128 SQ8 scan)", "queries/s", r["qps"], r["sec"],
+                         "u8 codes; i8 x i8 -> i32 pre-selection, f32 results" if r["tile"] == 256 else
                          "u8 codes, f32 accumulate",
                          "configs[1]: flat SQ8 scan, N=%d, d=%d, %d queries, k=%d, L2 (headline) and IP" % (n, d, nq, k),
                          extra, roof, cpu)

@@ -1,0 +1,66 @@
+"""Seeded random configurations (sizes, dimensions, k, metrics, cluster structure, duplicated queries): the matrix-core
+routes of the flat scan (int8 / fp32 pre-selection) and of the posting-list scan (int8 pass) against the streaming
+kernels, ids and distance bits."""
+import numpy as np
+import pytest
+
+import oracle as orc
+from gpu_helpers import Store, gaussian_mixture
+from vsag_amd import capi
+
+pytestmark = pytest.mark.gpu
+
+
+def _same(a, b):
+    return np.array_equal(a[0], b[0]) and np.array_equal(a[1].view(np.uint32), b[1].view(np.uint32))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_configuration(lib, seed):
+    L = lib.load_library()
+    rng = np.random.default_rng(1000 + seed)
+    kind = ["sq8", "fp32", "ivf"][seed % 3]
+    d = int(rng.choice([16, 24, 32, 48, 64, 96, 100, 128] + ([200, 256] if kind != "ivf" else [])))
+    n = int(rng.integers(20000, 200000))
+    nq = int(rng.integers(512, 2500))
+    k = int(rng.choice([1, 5, 10, 32, 100]))
+    metric = int(rng.choice([orc.L2, orc.IP, orc.COSINE]))
+    comps = int(rng.choice([1, 5, 50, 500]))
+    sigma = float(rng.choice([0.01, 0.05, 0.3]))
+    x, means = gaussian_mixture(rng, n, d, comps, sigma)
+    q, _ = gaussian_mixture(rng, nq, d, comps, sigma, means=means)
+    if rng.random() < 0.4:
+        q[: nq // 4] = x[rng.integers(0, n, nq // 4)]  # copies of stored vectors
+    buckets = None
+    if kind == "sq8":
+        lb, diff = orc.sq_train(x, 8, metric)
+        st = Store(capi.KIND_SQ8, metric, d, lb=lb, diff=diff)
+        st.append(orc.sq_encode(x, 8, lb, diff, metric))
+    elif kind == "fp32":
+        st = Store(capi.KIND_FP32, metric, d)
+        st.append(x.view(np.uint8).reshape(n, 4 * d))
+    else:
+        nlist = int(rng.choice([16, 64, 200]))
+        nprobe = min(int(rng.choice([4, 8, 16])), nlist)
+        nq = max(nq, 8192 * 4 // (nprobe - 1) + 64)  # enough (list, query group) items for the matrix-core pass
+        q = np.tile(q, (nq // q.shape[0] + 1, 1))[:nq] + 1e-3 * rng.standard_normal((nq, d)).astype(np.float32)
+        cent = x[rng.choice(n, nlist, replace=False)].copy()
+        labels, _, _ = orc.kmeans_assign(x, cent)
+        l, dd = orc.sq_train_uniform(x, 4, metric, mode=3)
+        st = Store(capi.KIND_SQ4_UNIFORM, metric, d, bounds=[l, dd])
+        st.set_lists(orc.squ_encode(x, 4, l, dd, metric), labels, nlist)
+        buckets, _ = orc.ivf_route(cent, q, nprobe)
+    res = {}
+    try:
+        for mode in ((-1, 0) if kind == "ivf" else (-1, 1, 2)):
+            capi.check(L.vsag_amd_set_scan_contraction(mode))
+            res[mode] = st.ivf_scan(q, buckets, max(k, 10)) if kind == "ivf" else st.flat_scan(q, k)
+            if mode != -1:
+                tile = capi.C.c_int()
+                L.vsag_amd_last_scan_info(capi.C.byref(tile), None, None)
+                assert tile.value >= 128, "the matrix-core route did not run"
+    finally:
+        capi.check(L.vsag_amd_set_scan_contraction(0))
+    for mode, r in res.items():
+        assert _same(res[-1], r), (kind, n, d, nq, k, metric, mode)
+    st.destroy()
