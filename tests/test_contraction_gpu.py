@@ -142,3 +142,40 @@ def test_contraction_overflow_falls_back_to_streaming(lib, modes):
     np.testing.assert_allclose(fast[1][:8], rd, rtol=1e-5)
     assert np.all(np.diff(fast[0], axis=1)[np.diff(fast[1], axis=1) == 0] > 0), "ties are ordered by id"
     st.destroy()
+
+
+def _rabitq_store(rng, n, d, metric, centered=True):
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    if centered:
+        x /= np.linalg.norm(x, axis=1, keepdims=True)
+    else:
+        x = x * 0.1 + 1.0  # far from the origin: large raw norms, small residuals
+    g = rng.standard_normal((d, d))
+    rot, r = np.linalg.qr(g)
+    rot = (rot * np.sign(np.diag(r))).astype(np.float32)
+    cen = orc.rabitq_train(x, rot)
+    st = Store(capi.KIND_RABITQ, metric, d, rot=rot, centroid=cen)
+    st.append(orc.rabitq_encode(x, rot, cen, metric))
+    return x, st
+
+
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP])
+@pytest.mark.parametrize("n,d,nq,k,centered", [(30000, 128, 300, 10, True), (20000, 768, 260, 200, True),
+                                               (9000, 100, 129, 50, False), (70000, 256, 700, 100, True)])
+def test_rabitq_contraction_equals_streaming(lib, modes, metric, n, d, nq, k, centered):
+    """1-bit codes against 4-bit queries on the int8 matrix cores: the estimator is affine in the integer inner
+    product, so the pre-selection is a threshold on it; the rescored result must equal the streaming scan's bits."""
+    rng = np.random.default_rng(n + d + k + metric)
+    x, st = _rabitq_store(rng, n, d, metric, centered)
+    q = rng.standard_normal((nq, d)).astype(np.float32)
+    if centered:
+        q /= np.linalg.norm(q, axis=1, keepdims=True)
+    else:
+        q = q * 0.1 + 1.0
+    q[3] = x[17]                 # a stored vector
+    q[4] = 0.0                   # no direction at all
+    q[5] = 1.0                   # constant coordinates before the rotation
+    plain, fast, tile = modes(st, q, k)
+    assert tile == 128, "the contraction path did not run"
+    assert same(plain, fast)
+    st.destroy()

@@ -289,7 +289,10 @@ finish_distances(const ScanArgs& a, const uint32_t (&qidx)[T], uint64_t slot, co
 
 // The sequence of granule groups one wave walks: tiles first, first + stride, ... below end; inside a tile
 // groups j0 = 0, GROUP, ...  `load` fetches a group into registers, `advance` steps to the next one.
-template <int GROUP>
+// OVERLAP: when the granules of a tile are not a multiple of GROUP, the last group of a tile starts GROUP granules
+// before the tile's end instead of running past it: it re-reads granules the previous group has just fetched
+// (cache hits) rather than granules of the next tile (memory traffic), and only its new granules are consumed.
+template <int GROUP, bool OVERLAP = false>
 struct TileStream {
     const uint4* tiles;  // wave-uniform; a lane reads element `lane` of a 64-element granule row
     uint32_t lane;
@@ -308,11 +311,19 @@ struct TileStream {
     __device__ inline void
     load(uint4 (&regs)[GROUP], uint64_t fallback) const {
         const uint64_t t = tile < end ? tile : fallback;
-        const uint4* tp = tiles + (t * G + j0) * kWave + lane;
+        const uint4* tp = tiles + (t * G + first()) * kWave + lane;
 #pragma unroll
         for (int u = 0; u < GROUP; ++u) {
             regs[u] = tp[u * kWave];
         }
+    }
+    // Granule held by register 0 of the group at j0.
+    __device__ inline uint32_t
+    first() const {
+        if constexpr (OVERLAP) {
+            return G >= GROUP && j0 + GROUP > G ? G - GROUP : j0;
+        }
+        return j0;
     }
     __device__ inline void
     advance() {

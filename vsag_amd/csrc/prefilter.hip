@@ -378,8 +378,8 @@ struct RescoreArgs {
     uint32_t first_slot;  // the list of the first level of this call; out_slot - first_slot levels came before
     uint32_t out_slot;
     uint32_t* gate;  // per query: 1 = candidates overflowed at some level, the streaming kernel must serve the query
-    // sub_lists != 0: the candidates of a query sit in sub_lists lists of sub_cap slots with a count each (a count
-    // above sub_cap = that list overflowed); they are gathered into LDS first (at most kRescoreGather of them).
+    // sub_lists != 0: the candidates of a query sit in sub_lists lists of sub_cap (<= kRescoreGather) slots with a
+    // count each (a count above sub_cap = that list overflowed); they are gathered into LDS a few lists at a time.
     uint32_t sub_lists, sub_cap;
 };
 
@@ -393,37 +393,15 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
     const uint32_t lane = threadIdx.x;
     const uint32_t q = blockIdx.x;
     const uint64_t list = static_cast<uint64_t>(q) * r.nslots + r.out_slot;
-    uint32_t total = 0;
     bool overflow = false;
-    const uint32_t* mine = r.cand + static_cast<uint64_t>(q) * r.cap;
+    const uint32_t* counts = r.cand_cnt + static_cast<uint64_t>(q) * (r.sub_lists != 0 ? r.sub_lists : 1);
     if (r.sub_lists == 0) {
-        total = as_const(r.cand_cnt)[q];
-        overflow = total > r.cap;
+        overflow = as_const(counts)[0] > r.cap;
     } else {
-        // Gather the private lists of the query behind the selector: a lane per list, offsets by a wave scan.
-        uint32_t* flat = reinterpret_cast<uint32_t*>(keys + r.S);
-        const uint32_t* counts = r.cand_cnt + static_cast<uint64_t>(q) * r.sub_lists;
-        const uint32_t* lists = r.cand + static_cast<uint64_t>(q) * r.sub_lists * r.sub_cap;
-        for (uint32_t g0 = 0; g0 < r.sub_lists && !overflow; g0 += kWave) {
+        for (uint32_t g0 = 0; g0 < r.sub_lists; g0 += kWave) {
             const uint32_t g = g0 + lane;
-            const uint32_t c = g < r.sub_lists ? as_const(counts)[g] : 0U;
-            uint32_t incl = c;
-            for (int off = 1; off < 64; off <<= 1) {
-                uint32_t o = __shfl_up(incl, off);
-                incl += lane >= static_cast<uint32_t>(off) ? o : 0U;
-            }
-            const uint32_t sum = __shfl(incl, 63);
-            overflow = __ballot(c > r.sub_cap) != 0 || total + sum > kRescoreGather;
-            if (!overflow) {
-                const uint32_t at = total + incl - c;
-                for (uint32_t i = 0; i < c; ++i) {
-                    flat[at + i] = as_const(lists)[static_cast<uint64_t>(g) * r.sub_cap + i];
-                }
-                total += sum;
-            }
+            overflow = overflow || __ballot(g < r.sub_lists && as_const(counts)[g] > r.sub_cap) != 0;
         }
-        wave_lds_fence();
-        mine = flat;
     }
     if (overflow || as_const(r.gate)[q] != 0) {
         // The streaming kernel will scan every tile behind the prefix for this query: the lists of the levels so
@@ -445,35 +423,67 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
     uint64_t tau = (static_cast<uint64_t>(bs) << 32) | 0xFFFFFFFFULL;
     const uint32_t qidx[1] = {q};
     const QueryRows<1> qrows = query_rows<1>(a, qidx);
-    for (uint32_t base = 0; base < total; base += kWave) {
-        const bool have = base + lane < total;
-        const uint32_t slot = have ? mine[base + lane] : 0U;
-        const uint64_t tile = slot >> 6;
-        const uint32_t ln = slot & 63;
-        Acc<KIND, 1> acc;
-        acc_reset(acc);
-        for (uint32_t j = 0; j < a.G; ++j) {
-            uint4 c = a.tiles[(tile * a.G + j) * kWave + ln];
-            accumulate_granule<KIND, METRIC, 1>(a, qrows, j, c, acc);
+    auto rescore = [&](const uint32_t* mine, uint32_t total) {
+        for (uint32_t base = 0; base < total; base += kWave) {
+            const bool have = base + lane < total;
+            const uint32_t slot = have ? mine[base + lane] : 0U;
+            const uint64_t tile = slot >> 6;
+            const uint32_t ln = slot & 63;
+            Acc<KIND, 1> acc;
+            acc_reset(acc);
+            for (uint32_t j = 0; j < a.G; ++j) {
+                uint4 c = a.tiles[(tile * a.G + j) * kWave + ln];
+                accumulate_granule<KIND, METRIC, 1>(a, qrows, j, c, acc);
+            }
+            float d[1];
+            finish_distances<KIND, METRIC, 1>(a, qidx, slot, acc, d);
+            const uint64_t key = make_key(d[0], slot);
+            bool pass = have && slot < r.n && key <= tau;
+            uint64_t mask = __ballot(pass);
+            if (mask != 0) {
+                uint32_t np = __popcll(mask);
+                if (k + cnt + np > S) {
+                    uint64_t th = selector_flush(keys, S, k, cnt, lane);
+                    cnt = 0;
+                    uint32_t b = lower_shared(&r.bound[q], static_cast<uint32_t>(th >> 32), lane);
+                    uint64_t shared_tau = (static_cast<uint64_t>(b) << 32) | 0xFFFFFFFFULL;
+                    tau = th < shared_tau ? th : shared_tau;
+                }
+                if (pass) {
+                    keys[k + cnt + mask_rank(mask)] = key;
+                }
+                cnt += np;
+            }
         }
-        float d[1];
-        finish_distances<KIND, METRIC, 1>(a, qidx, slot, acc, d);
-        const uint64_t key = make_key(d[0], slot);
-        bool pass = have && slot < r.n && key <= tau;
-        uint64_t mask = __ballot(pass);
-        if (mask != 0) {
-            uint32_t np = __popcll(mask);
-            if (k + cnt + np > S) {
-                uint64_t th = selector_flush(keys, S, k, cnt, lane);
-                cnt = 0;
-                uint32_t b = lower_shared(&r.bound[q], static_cast<uint32_t>(th >> 32), lane);
-                uint64_t shared_tau = (static_cast<uint64_t>(b) << 32) | 0xFFFFFFFFULL;
-                tau = th < shared_tau ? th : shared_tau;
+    };
+    if (r.sub_lists == 0) {
+        rescore(r.cand + static_cast<uint64_t>(q) * r.cap, as_const(counts)[0]);
+    } else {
+        // Gather the private lists of the query behind the selector, as many at a time as are sure to fit: a lane
+        // per list, offsets by a wave scan.
+        uint32_t* flat = reinterpret_cast<uint32_t*>(keys + r.S);
+        const uint32_t* lists = r.cand + static_cast<uint64_t>(q) * r.sub_lists * r.sub_cap;
+        uint32_t batch = kRescoreGather / r.sub_cap;
+        batch = batch > kWave ? kWave : (batch == 0 ? 1 : batch);
+        for (uint32_t g0 = 0; g0 < r.sub_lists; g0 += batch) {
+            const uint32_t g = g0 + lane;
+            const uint32_t c = lane < batch && g < r.sub_lists ? as_const(counts)[g] : 0U;
+            uint32_t incl = c;
+            for (int off = 1; off < 64; off <<= 1) {
+                uint32_t o = __shfl_up(incl, off);
+                incl += lane >= static_cast<uint32_t>(off) ? o : 0U;
             }
-            if (pass) {
-                keys[k + cnt + mask_rank(mask)] = key;
+            const uint32_t sum = __shfl(incl, 63);
+            if (sum == 0) {
+                continue;
             }
-            cnt += np;
+            wave_lds_fence();  // the previous batch has been read
+            const uint32_t at = incl - c;
+            for (uint32_t i = 0; i < c; ++i) {
+                flat[at + i] = as_const(lists)[static_cast<uint64_t>(g) * r.sub_cap + i];
+            }
+            wave_lds_fence();
+            rescore(flat, sum);
         }
     }
     wave_lds_fence();
@@ -495,8 +505,16 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
 }
 
 // ------------------------------------------------------------------ host side
+bool prefilter_rb_supports(const vsag_amd_store* s);
+int launch_prefilter_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint64_t tile_begin, uint64_t tile_end,
+                        const uint32_t* bound, uint8_t* scratch, uint32_t* cand, uint32_t* cand_cnt, uint32_t sub_lists,
+                        uint32_t sub_cap, hipStream_t st);
+
 bool
 prefilter_supports(const vsag_amd_store* s) {
+    if (prefilter_rb_supports(s)) {
+        return true;
+    }
     return s->nlist == 0 && (s->kind == VSAG_AMD_KIND_FP32 || s->kind == VSAG_AMD_KIND_SQ8) && s->pf_term != nullptr;
 }
 
@@ -541,7 +559,6 @@ launch_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t
                const uint32_t* cand, const uint32_t* cand_cnt, uint32_t cap, uint32_t sub_lists, uint32_t sub_cap,
                uint64_t* partial, uint32_t* partial_cnt, uint32_t nslots, uint32_t first_slot, uint32_t out_slot,
                uint32_t* gate, hipStream_t st) {
-    const bool sq8 = s->kind == VSAG_AMD_KIND_SQ8;
     RescoreArgs r{};
     r.first_slot = first_slot;
     r.cand = cand;
@@ -560,8 +577,10 @@ launch_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t
     r.sub_cap = sub_cap;
     dim3 rgrid(static_cast<uint32_t>(nq));
     const size_t lds = S * 8 + (sub_lists != 0 ? kRescoreGather * 4 : 0);
-    if (sq8) {
+    if (s->kind == VSAG_AMD_KIND_SQ8) {
         launch_rescore_m<VSAG_AMD_KIND_SQ8>(s->metric, rgrid, lds, st, a, r);
+    } else if (s->kind == VSAG_AMD_KIND_RABITQ) {
+        launch_rescore_m<VSAG_AMD_KIND_RABITQ>(s->metric, rgrid, lds, st, a, r);
     } else {
         launch_rescore_m<VSAG_AMD_KIND_FP32>(s->metric, rgrid, lds, st, a, r);
     }
@@ -579,6 +598,12 @@ launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32
                  uint32_t* gate, uint8_t* q8, float* q8_u, uint32_t sub_lists, uint32_t sub_cap, hipStream_t st) {
     const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
     const bool sq8 = s->kind == VSAG_AMD_KIND_SQ8;
+    if (s->kind == VSAG_AMD_KIND_RABITQ) {
+        // 1-bit codes against 4-bit queries on the int8 matrix cores (prefilter_rb.hip); q8 is its scratch.
+        VA_TRY(launch_prefilter_rb(s, a, nq, tile_begin, tile_end, bound, q8, cand, cand_cnt, sub_lists, sub_cap, st));
+        return launch_rescore(s, a, nq, k, S, bound, cand, cand_cnt, 0, sub_lists, sub_cap, partial, partial_cnt, nslots,
+                              first_slot, out_slot, gate, st);
+    }
     if (q8 != nullptr) {
         // At most 128 dimensions of sq8: the int8 matrix cores pre-select (prefilter_i8.hip).
         VA_TRY(launch_prefilter_i8(s, reinterpret_cast<const float*>(a.qtab), a.qstride, a.qmeta, a.qmeta_stride, nq,

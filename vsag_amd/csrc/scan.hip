@@ -139,8 +139,10 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
     // alternate; the loop body is written out twice so that both are addressed statically.
     const QueryRows<T> qrows = query_rows<T>(a, qidx);
     constexpr int GROUP = GroupOf<T>::value;
-    TileStream<GROUP> cur{a.tiles, lane, tile_begin + wave, tile_end, nwaves, 0, a.G};
-    TileStream<GROUP> nxt = cur;
+    // RaBitQ codes have G = dim / 128 granules, often no multiple of the group (768 dimensions: 6).
+    constexpr bool OVERLAP = KIND == VSAG_AMD_KIND_RABITQ || KIND == kKindRabitqF32;
+    TileStream<GROUP, OVERLAP> cur{a.tiles, lane, tile_begin + wave, tile_end, nwaves, 0, a.G};
+    TileStream<GROUP, OVERLAP> nxt = cur;
     uint4 buf_a[GROUP], buf_b[GROUP];
     if (cur.valid()) {
         cur.load(buf_a, cur.tile);
@@ -164,10 +166,12 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
     };
 
     auto consume = [&](const uint4(&regs)[GROUP]) {
+        const uint32_t first = cur.first();
 #pragma unroll
         for (int u = 0; u < GROUP; ++u) {
-            if (cur.j0 + u < a.G) {
-                accumulate_granule<KIND, METRIC, T>(a, qrows, cur.j0 + u, regs[u], acc);
+            const uint32_t g = first + u;
+            if (g >= cur.j0 && g < a.G) {
+                accumulate_granule<KIND, METRIC, T>(a, qrows, g, regs[u], acc);
             }
         }
         if (cur.j0 + GROUP < a.G) {
@@ -587,10 +591,12 @@ struct CallPlan {
     int levels = 0;
     uint64_t level_begin[kMaxLevels + 1] = {0, 0, 0, 0};
     bool int8 = false;         // the int8 matrix cores pre-select (sq8, at most 128 dimensions)
+    bool rb = false;           // RaBitQ store: 1-bit codes x 4-bit queries on the int8 matrix cores
     uint32_t cap = 0;          // candidates per query and level
     uint32_t sub_lists[kMaxLevels] = {0, 0, 0};  // int8: private candidate lists per query ...
     uint32_t sub_cap[kMaxLevels] = {0, 0, 0};    // ... of this many slots
     uint32_t max_lists = 0;    // the largest sub_lists
+    size_t rb_scratch = 0;     // rb: bytes of the expanded queries and per-query factors
     uint32_t nslots = 0;       // partial lists per query
     bool any_seeded = false;
 };
@@ -606,6 +612,9 @@ int launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, ui
 bool prefilter_i8_supports(const vsag_amd_store* s);
 size_t prefilter_i8_query_bytes(uint64_t nq);
 uint32_t prefilter_i8_sub_lists(uint64_t nq, uint64_t span);
+bool prefilter_rb_supports(const vsag_amd_store* s);
+size_t prefilter_rb_scratch_bytes(const vsag_amd_store* s, uint64_t nq);
+uint32_t prefilter_rb_sub_lists(uint64_t nq, uint64_t span);
 
 static void
 make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
@@ -617,11 +626,13 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
         return;
     }
     const bool forced = g_prefilter_mode > 0;
-    if (!forced && (nq < 512 || k > 128 || s->ntiles < 1024)) {
+    const bool rb = prefilter_rb_supports(s);
+    if (!forced && (nq < 512 || k > (rb ? 256U : 128U) || s->ntiles < 1024)) {
         return;
     }
-    // Candidate buffers: at most 2 GiB in all, 1024 to 4096 candidates per query.
-    uint64_t cap = 4096;
+    // Candidate buffers: at most 2 GiB in all, 1024 to 4096 candidates per query (RaBitQ stores are searched with
+    // hundreds of candidates for a later rerank: eight times as many).
+    uint64_t cap = rb ? 32768 : 4096;
     while (cap > 1024 && nq * cap * 4 > (2ull << 30)) {
         cap /= 2;
     }
@@ -655,6 +666,8 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
     }
     c->contraction = true;
     c->int8 = g_prefilter_mode != 2 && prefilter_i8_supports(s);
+    c->rb = rb;
+    c->rb_scratch = rb ? prefilter_rb_scratch_bytes(s, nq) : 0;
     c->prefix_tiles = prefix;
     c->cap = static_cast<uint32_t>(cap);
     c->levels = nb - 1;
@@ -662,6 +675,15 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
         c->level_begin[l] = bounds[nb - 1 - l];
     }
     c->max_lists = 0;
+    if (c->rb) {
+        for (int l = 0; l < c->levels; ++l) {
+            c->sub_lists[l] = prefilter_rb_sub_lists(nq, c->level_begin[l + 1] - c->level_begin[l]);
+            c->sub_cap[l] = std::max<uint32_t>(16, static_cast<uint32_t>(div_up(cap, static_cast<uint64_t>(c->sub_lists[l]))));
+            c->sub_cap[l] = std::min<uint32_t>(c->sub_cap[l], 4096);  // what the rescoring gathers at a time
+            c->cap = std::max(c->cap, c->sub_lists[l] * c->sub_cap[l]);
+            c->max_lists = std::max(c->max_lists, c->sub_lists[l]);
+        }
+    }
     if (c->int8) {
         for (int l = 0; l < c->levels; ++l) {
             // The expected load of a list is an eighth of its share of the buffer; short lists get room for the
@@ -712,8 +734,8 @@ carve_scan(Carver& c, const CallPlan& cp, uint64_t nq, uint32_t k, ScanBuffers* 
     const uint64_t nq_pad8 = prefilter_i8_query_bytes(nq) / 256;  // whole workgroups of the int8 prefilter
     b->tau = c.take<float>(cp.contraction ? nq_pad8 : 0);
     b->q8_u = c.take<float>(cp.int8 ? nq_pad8 : 0);
-    b->q8 = c.take<uint8_t>(cp.int8 ? prefilter_i8_query_bytes(nq) : 0);
-    if (!cp.int8) {
+    b->q8 = c.take<uint8_t>(cp.int8 ? prefilter_i8_query_bytes(nq) : (cp.rb ? cp.rb_scratch : 0));
+    if (!cp.int8 && !cp.rb) {
         b->q8 = nullptr;
     }
     b->cand_cnt = c.take<uint32_t>(cp.contraction ? nq * std::max<uint32_t>(1, cp.max_lists) : 0);
@@ -914,7 +936,7 @@ vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, 
                                          dists_dev, st));
             hipLaunchKernelGGL(tighten_bound_kernel, dim3(static_cast<uint32_t>(div_up(nq, 256))), dim3(256), 0, st,
                                dists_dev, k, nq, b.bound);
-            if (!cp.int8) {
+            if (!cp.int8 && !cp.rb) {
                 hipLaunchKernelGGL(fill_words2_kernel, dim3(static_cast<uint32_t>(div_up(nq, 256))), dim3(256), 0, st,
                                    b.cand_cnt, nq, static_cast<uint32_t*>(nullptr), 0);
             }
