@@ -695,8 +695,21 @@ def run_c5(env):
     roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
             "traffic": traffic, "kernel": "flat_scan_kernel<rabitq, ip, T=%d>" % tile, "kernel_ms": kms,
             "algorithmic_bytes_per_launch": algo}
+    dtype = "1-bit codes x 4-bit queries, u32 popcount"
+    if tile >= 64:
+        # The batch was pre-selected on the int8 matrix cores (1-bit codes and 4-bit queries expanded to bytes) and
+        # the survivors rescored with the popcount arithmetic.  The timed kernel is the last level: bpp bytes of
+        # d / 8-byte codes against every query.
+        lcodes = bpp / (d / 8.0)
+        ops = 2.0 * lcodes * d * nq
+        tops = ops / (kms * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": tops, "peak": MFMA_I8_PEAK_TOPS, "unit": "TOP/s",
+                "frac": tops / MFMA_I8_PEAK_TOPS, "traffic": None,
+                "kernel": "prefilter_rb_kernel<ip> (int8 MFMA, last level)", "kernel_ms": kms, "ops_per_launch": ops,
+                "codes_per_launch": lcodes}
+        dtype = "1-bit codes x 4-bit queries: int8 MFMA pre-selection, u32 popcount rescoring"
     return env.base_line("QPS @ recall@10 (RaBitQ 1-bit scan + rerank 200, 5M x 768)", "queries/s", nq / sec, sec,
-                         "1-bit codes x 4-bit queries, u32 popcount",
+                         dtype,
                          "configs[4]: RaBitQ full scan + fp32 rerank of %d, N=%d, d=%d, %d queries, k=%d, IP" %
                          (kcand, n, d, nq, k),
                          {"recall_at_10": rec, "build_seconds": t_build, "query_tile": tile, "passes_per_step": passes,

@@ -34,7 +34,9 @@ typedef int intx4 __attribute__((ext_vector_type(4)));
 typedef int intx16 __attribute__((ext_vector_type(16)));
 
 constexpr uint32_t kRbQueries = 128;  // queries per workgroup
-constexpr uint32_t kRbMaxG = 8;       // granules per code the kernel holds in registers (1024 dimensions)
+constexpr uint32_t kRbMaxG = 8;       // granules per code (1024 dimensions): the query group has to fit the LDS
+constexpr uint32_t kRbWaves = 8;      // waves per workgroup, two per SIMD: one multiplies while the other decides
+constexpr uint32_t kRbThreads = kRbWaves * kWave;
 
 // 4-bit queries as bytes: row q holds, per code dword w, the 32 values of dimensions 32 w ... (dpad bytes per row).
 __global__ void __launch_bounds__(256)
@@ -133,7 +135,7 @@ struct PrefilterRbArgs {
     uint32_t* cand;        // [query][sub_lists][sub_cap]
     uint32_t* cand_cnt;    // [query][sub_lists]
     uint32_t sub_cap;
-    uint32_t groups;       // grid x; the grid has groups * 4 waves per query group
+    uint32_t groups;       // grid x; the grid has groups * kRbWaves waves per query group
 };
 
 __device__ inline int
@@ -143,7 +145,7 @@ rb_spread(uint32_t nibble) {
 }
 
 template <int METRIC>
-__global__ void __launch_bounds__(256, 1)
+__global__ void __launch_bounds__(kRbThreads, 2)
 prefilter_rb_kernel(PrefilterRbArgs p) {
     extern __shared__ uint4 rb_lds[];
     const uint32_t tid = threadIdx.x;
@@ -163,10 +165,8 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
     }
     float u1[4], u2[4], u3[4], u4[4];
     uint32_t ncand[4] = {0, 0, 0, 0};
-    uint32_t* my_list[4];
-    bool q_real[4];
-    const uint32_t sub_lists = p.groups * 8;
-    const uint32_t my_sub = (blockIdx.x * 4 + wave) * 2 + half;
+    const uint32_t sub_lists = p.groups * 2 * kRbWaves;
+    const uint32_t my_sub = (blockIdx.x * kRbWaves + wave) * 2 + half;
 #pragma unroll
     for (int qb = 0; qb < 4; ++qb) {
         const uint64_t q = q0 + 32 * qb + l32;
@@ -174,26 +174,18 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
         u2[qb] = p.u[p.nq_pad + q];
         u3[qb] = p.u[2 * p.nq_pad + q];
         u4[qb] = p.u[3 * p.nq_pad + q];
-        q_real[qb] = q < p.nq;
-        my_list[qb] = p.cand + ((q_real[qb] ? q : 0) * sub_lists + my_sub) * p.sub_cap;
     }
     __syncthreads();
 
     const uint64_t span = p.tile_end - p.tile_begin;
-    for (uint64_t t = static_cast<uint64_t>(blockIdx.x) * 4 + wave; t < span; t += static_cast<uint64_t>(p.groups) * 4) {
+    for (uint64_t t = static_cast<uint64_t>(blockIdx.x) * kRbWaves + wave; t < span;
+         t += static_cast<uint64_t>(p.groups) * kRbWaves) {
         const uint64_t tile = p.tile_begin + t;
-        // The bits of this lane's two codes (rows l32 and 32 + l32 of the tile).
-        uint4 bits[2][kRbMaxG];
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-#pragma unroll
-            for (uint32_t g = 0; g < kRbMaxG; ++g) {
-                bits[i][g] = make_uint4(0, 0, 0, 0);
-                if (g < p.G) {
-                    bits[i][g] = p.tiles[(tile * p.G + g) * kWave + 32 * i + l32];
-                }
-            }
-        }
+        // The bits of this lane's two codes (rows l32 and 32 + l32 of the tile), a granule at a time and one ahead.
+        const uint4* code_rows = p.tiles + tile * p.G * kWave + l32;
+        uint4 bits[2], ahead[2];
+        bits[0] = code_rows[0];
+        bits[1] = code_rows[32];
         // Per-code constants, a lane per code.
         const uint64_t my_slot = tile * kWave + lane;
         const float bn = __uint_as_float(p.meta[my_slot]);
@@ -235,13 +227,17 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
 #pragma unroll
         for (uint32_t g = 0; g < kRbMaxG; ++g) {
             if (g < p.G) {
+                if (g + 1 < p.G) {
+                    ahead[0] = code_rows[(g + 1) * kWave];
+                    ahead[1] = code_rows[(g + 1) * kWave + 32];
+                }
 #pragma unroll
                 for (int m = 0; m < 4; ++m) {
                     const uint32_t s = 4 * g + m;
                     intx4 av[2];
 #pragma unroll
                     for (int i = 0; i < 2; ++i) {
-                        const uint32_t dw = m == 0 ? bits[i][g].x : (m == 1 ? bits[i][g].y : (m == 2 ? bits[i][g].z : bits[i][g].w));
+                        const uint32_t dw = m == 0 ? bits[i].x : (m == 1 ? bits[i].y : (m == 2 ? bits[i].z : bits[i].w));
                         const uint32_t hb = dw >> (16 * half);
                         av[i] = intx4{rb_spread(hb & 15U), rb_spread((hb >> 4) & 15U), rb_spread((hb >> 8) & 15U),
                                       rb_spread((hb >> 12) & 15U)};
@@ -255,50 +251,54 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
                         acc[qb][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[1], bv, acc[qb][1], 0, 0, 0);
                     }
                 }
+                bits[0] = ahead[0];
+                bits[1] = ahead[1];
             }
         }
 
         // Element e of a lane is code 32 i + 8 (e / 4) + 4 (lane / 32) + e % 4 of the tile against query l32 of block qb.
+        // Four elements (one float4 of each per-code constant) at a time keeps the registers of two waves per SIMD.
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
-            float ca[16], cb[16], cs[16];
 #pragma unroll
             for (int gq = 0; gq < 4; ++gq) {
                 const uint32_t row = 32 * i + 8 * gq + 4 * half;
                 const float4 va = *reinterpret_cast<const float4*>(&cc[row]);
                 const float4 vb = *reinterpret_cast<const float4*>(&cc[kWave + row]);
                 const float4 vs = *reinterpret_cast<const float4*>(&cc[2 * kWave + row]);
-                ca[4 * gq] = va.x, ca[4 * gq + 1] = va.y, ca[4 * gq + 2] = va.z, ca[4 * gq + 3] = va.w;
-                cb[4 * gq] = vb.x, cb[4 * gq + 1] = vb.y, cb[4 * gq + 2] = vb.z, cb[4 * gq + 3] = vb.w;
-                cs[4 * gq] = vs.x, cs[4 * gq + 1] = vs.y, cs[4 * gq + 2] = vs.z, cs[4 * gq + 3] = vs.w;
-            }
+                const float ca[4] = {va.x, va.y, va.z, va.w};
+                const float cb[4] = {vb.x, vb.y, vb.z, vb.w};
+                const float cs[4] = {vs.x, vs.y, vs.z, vs.w};
 #pragma unroll
-            for (int qb = 0; qb < 4; ++qb) {
-                bool pass[16];
-                uint64_t any = 0;
+                for (int qb = 0; qb < 4; ++qb) {
+                    bool pass[4];
+                    uint64_t any = 0;
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    float thr = fmaf(cs[e], u3[qb], fmaf(cb[e], u2[qb], fmaf(ca[e], u1[qb], u4[qb])));
-                    thr = fmaf(fabsf(thr), -1.0e-4F, thr);
-                    pass[e] = static_cast<float>(acc[qb][i][e]) >= thr;
-                    any |= __ballot(pass[e]);
-                }
-                if (any != 0) {
-                    uint32_t hits = 0;
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        hits |= pass[e] ? 1U << e : 0U;
+                    for (int j = 0; j < 4; ++j) {
+                        float thr = fmaf(cs[j], u3[qb], fmaf(cb[j], u2[qb], fmaf(ca[j], u1[qb], u4[qb])));
+                        thr = fmaf(fabsf(thr), -1.0e-4F, thr);
+                        pass[j] = static_cast<float>(acc[qb][i][4 * gq + j]) >= thr;
+                        any |= __ballot(pass[j]);
                     }
-                    while (hits != 0) {
-                        const uint32_t e = static_cast<uint32_t>(__builtin_ctz(hits));
-                        hits &= hits - 1;
-                        const uint32_t code = 32 * i + 8 * (e >> 2) + 4 * half + (e & 3);
-                        const uint64_t slot = tile * kWave + code;
-                        if (slot < p.n && ((special_mask >> code) & 1ULL) == 0) {
-                            if (ncand[qb] < p.sub_cap) {
-                                my_list[qb][ncand[qb]] = static_cast<uint32_t>(slot);
+                    if (any != 0) {
+                        uint32_t hits = 0;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            hits |= pass[j] ? 1U << j : 0U;
+                        }
+                        const uint64_t q = q0 + 32 * qb + l32;
+                        uint32_t* list = p.cand + ((q < p.nq ? q : 0) * sub_lists + my_sub) * p.sub_cap;
+                        while (hits != 0) {
+                            const uint32_t j = static_cast<uint32_t>(__builtin_ctz(hits));
+                            hits &= hits - 1;
+                            const uint32_t code = row + j;
+                            const uint64_t slot = tile * kWave + code;
+                            if (slot < p.n && ((special_mask >> code) & 1ULL) == 0) {
+                                if (ncand[qb] < p.sub_cap) {
+                                    list[ncand[qb]] = static_cast<uint32_t>(slot);
+                                }
+                                ++ncand[qb];
                             }
-                            ++ncand[qb];
                         }
                     }
                 }
@@ -312,9 +312,10 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
                 rest &= rest - 1;
 #pragma unroll
                 for (int qb = 0; qb < 4; ++qb) {
-                    if (q_real[qb]) {
+                    const uint64_t q = q0 + 32 * qb + l32;
+                    if (q < p.nq) {
                         if (ncand[qb] < p.sub_cap) {
-                            my_list[qb][ncand[qb]] = static_cast<uint32_t>(tile * kWave + code);
+                            p.cand[(q * sub_lists + my_sub) * p.sub_cap + ncand[qb]] = static_cast<uint32_t>(tile * kWave + code);
                         }
                         ++ncand[qb];
                     }
@@ -355,8 +356,8 @@ prefilter_rb_sub_lists(uint64_t nq, uint64_t span) {
     const uint64_t qgroups = div_up(nq, static_cast<uint64_t>(kRbQueries));
     // One workgroup fits a compute unit (its query group fills the LDS); just under four rounds of them.
     uint64_t groups = static_cast<uint64_t>(device_cu_count()) * 4 / qgroups;
-    groups = std::max<uint64_t>(1, std::min<uint64_t>(groups, div_up(span, 4)));
-    return static_cast<uint32_t>(8 * groups);
+    groups = std::max<uint64_t>(1, std::min<uint64_t>(groups, div_up(span, static_cast<uint64_t>(kRbWaves))));
+    return static_cast<uint32_t>(2 * kRbWaves * groups);
 }
 
 int
@@ -388,19 +389,19 @@ launch_prefilter_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uin
     p.cand = cand;
     p.cand_cnt = cand_cnt;
     p.sub_cap = sub_cap;
-    p.groups = sub_lists / 8;
+    p.groups = sub_lists / (2 * kRbWaves);
     VA_CHECK_ARG(sub_lists == prefilter_rb_sub_lists(nq, tile_end - tile_begin), "candidate lists do not match the grid");
-    const size_t lds = static_cast<size_t>(8 * s->G) * kRbQueries * 16 + 4 * 3 * kWave * sizeof(float);
+    const size_t lds = static_cast<size_t>(8 * s->G) * kRbQueries * 16 + kRbWaves * 3 * kWave * sizeof(float);
     dim3 grid(p.groups, static_cast<uint32_t>(nq_pad / kRbQueries));
     timing_begin(st);
     if (l2) {
         VA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(prefilter_rb_kernel<VSAG_AMD_METRIC_L2>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        hipLaunchKernelGGL(prefilter_rb_kernel<VSAG_AMD_METRIC_L2>, grid, dim3(256), lds, st, p);
+        hipLaunchKernelGGL(prefilter_rb_kernel<VSAG_AMD_METRIC_L2>, grid, dim3(kRbThreads), lds, st, p);
     } else {
         VA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(prefilter_rb_kernel<VSAG_AMD_METRIC_IP>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        hipLaunchKernelGGL(prefilter_rb_kernel<VSAG_AMD_METRIC_IP>, grid, dim3(256), lds, st, p);
+        hipLaunchKernelGGL(prefilter_rb_kernel<VSAG_AMD_METRIC_IP>, grid, dim3(kRbThreads), lds, st, p);
     }
     timing_end(st);
     VA_HIP(hipGetLastError());
