@@ -354,8 +354,19 @@ prefilter_rb_scratch_bytes(const vsag_amd_store* s, uint64_t nq) {
 uint32_t
 prefilter_rb_sub_lists(uint64_t nq, uint64_t span) {
     const uint64_t qgroups = div_up(nq, static_cast<uint64_t>(kRbQueries));
-    // One workgroup fits a compute unit (its query group fills the LDS); just under four rounds of them.
-    uint64_t groups = static_cast<uint64_t>(device_cu_count()) * 4 / qgroups;
+    // One workgroup fits a compute unit (its query group fills the LDS) and all of them take equally long: three to
+    // six rounds of them, whichever leaves the last round fullest.
+    const uint64_t cus = static_cast<uint64_t>(device_cu_count());
+    uint64_t groups = 1;
+    double best = 0.0;
+    for (uint64_t rounds = 3; rounds <= 6; ++rounds) {
+        const uint64_t g = std::max<uint64_t>(1, cus * rounds / qgroups);
+        const double fill = static_cast<double>(g * qgroups) / static_cast<double>(cus * div_up(g * qgroups, cus));
+        if (fill > best + 1e-9) {
+            best = fill;
+            groups = g;
+        }
+    }
     groups = std::max<uint64_t>(1, std::min<uint64_t>(groups, div_up(span, static_cast<uint64_t>(kRbWaves))));
     return static_cast<uint32_t>(2 * kRbWaves * groups);
 }

@@ -587,14 +587,14 @@ struct CallPlan {
     uint64_t prefix_tiles = 0;
     // The tiles behind the prefix are pre-selected level by level, each level against the k-th distance of
     // everything before it: level l covers tiles [level_begin[l], level_begin[l + 1]).
-    static constexpr int kMaxLevels = 3;
+    static constexpr int kMaxLevels = 6;
     int levels = 0;
-    uint64_t level_begin[kMaxLevels + 1] = {0, 0, 0, 0};
+    uint64_t level_begin[kMaxLevels + 1] = {};
     bool int8 = false;         // the int8 matrix cores pre-select (sq8, at most 128 dimensions)
     bool rb = false;           // RaBitQ store: 1-bit codes x 4-bit queries on the int8 matrix cores
     uint32_t cap = 0;          // candidates per query and level
-    uint32_t sub_lists[kMaxLevels] = {0, 0, 0};  // int8: private candidate lists per query ...
-    uint32_t sub_cap[kMaxLevels] = {0, 0, 0};    // ... of this many slots
+    uint32_t sub_lists[kMaxLevels] = {};  // int8: private candidate lists per query ...
+    uint32_t sub_cap[kMaxLevels] = {};    // ... of this many slots
     uint32_t max_lists = 0;    // the largest sub_lists
     size_t rb_scratch = 0;     // rb: bytes of the expanded queries and per-query factors
     uint32_t nslots = 0;       // partial lists per query
@@ -642,7 +642,13 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
     // A level behind b tiles admits about k * (its tiles / b) codes per query: with every boundary a factor r
     // behind the next one that is k * r, kept below an eighth of the buffer.  The prefix in front of the first
     // level is scanned exactly by the streaming kernel.
-    const uint64_t r = std::min<uint64_t>(16, std::max<uint64_t>(2, cap / (8ull * k)));
+    // Every level also costs a merge of the lists so far, every admitted code an exact rescoring: with the hundreds
+    // of candidates a RaBitQ search keeps, the rescoring of k * r codes per query and level outweighs the merges
+    // unless r is small.
+    uint64_t r = std::min<uint64_t>(16, std::max<uint64_t>(2, cap / (8ull * k)));
+    if (rb) {
+        r = std::min<uint64_t>(r, std::max<uint64_t>(4, 800 / k));
+    }
     const uint64_t min_prefix = forced ? 2 : 64;
     uint64_t bounds[CallPlan::kMaxLevels + 1];
     int nb = 0;
@@ -651,7 +657,7 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
     while (nb <= CallPlan::kMaxLevels) {
         uint64_t next = std::max(min_prefix, div_up(cur, r));
         next += next & 1;
-        if (nb > 1 && cur < 4 * next) {
+        if (nb > 1 && cur < std::min<uint64_t>(4, r / 2) * next) {
             break;  // too thin a level to be worth its launches
         }
         bounds[nb++] = next;
