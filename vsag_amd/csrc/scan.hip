@@ -415,16 +415,43 @@ merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, cons
             nout = 0;
         }
         __syncthreads();
-        // A thread per list: most lists are empty or nearly so once the bound is known.
-        for (uint32_t slot = threadIdx.x; slot < nslots; slot += blockDim.x) {
-            const uint32_t c = cnts[slot];
-            const uint64_t* list = src + static_cast<uint64_t>(slot) * k;
-            for (uint32_t i = 0; i < c; ++i) {
-                uint64_t key = list[i];
-                if (key <= admit) {
-                    uint32_t pos = atomicAdd(&npool, 1U);
-                    if (pos < kPoolKeys) {
+        if (nslots * 4 <= blockDim.x) {
+            // Few lists (the levels of a pre-selected batch): a wave per list, a lane per key.
+            const uint32_t lane = threadIdx.x & (kWave - 1);
+            for (uint32_t slot = threadIdx.x / kWave; slot < nslots; slot += blockDim.x / kWave) {
+                const uint32_t c = cnts[slot];
+                const uint64_t* list = src + static_cast<uint64_t>(slot) * k;
+                for (uint32_t i0 = 0; i0 < c; i0 += kWave) {
+                    const uint32_t i = i0 + lane;
+                    const uint64_t key = i < c ? list[i] : kInfKey;
+                    const bool keep = i < c && key <= admit;
+                    const uint64_t votes = __ballot(keep);
+                    if (votes == 0) {
+                        continue;
+                    }
+                    uint32_t base = 0;
+                    if (lane == 0) {
+                        base = atomicAdd(&npool, static_cast<uint32_t>(__popcll(votes)));
+                    }
+                    base = __shfl(base, 0);
+                    const uint32_t pos = base + static_cast<uint32_t>(__popcll(votes & ((1ULL << lane) - 1)));
+                    if (keep && pos < kPoolKeys) {
                         pool[pos] = key;
+                    }
+                }
+            }
+        } else {
+            // A thread per list: most lists are empty or nearly so once the bound is known.
+            for (uint32_t slot = threadIdx.x; slot < nslots; slot += blockDim.x) {
+                const uint32_t c = cnts[slot];
+                const uint64_t* list = src + static_cast<uint64_t>(slot) * k;
+                for (uint32_t i = 0; i < c; ++i) {
+                    uint64_t key = list[i];
+                    if (key <= admit) {
+                        uint32_t pos = atomicAdd(&npool, 1U);
+                        if (pos < kPoolKeys) {
+                            pool[pos] = key;
+                        }
                     }
                 }
             }
