@@ -691,7 +691,7 @@ def run_c5(env):
     # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this exact configuration, profiles/flat_scan_rabitq_c5.md
     traffic = None
     if (n, d, nq, k, tile) == (5000000, 768, 10000, 10, 2):
-        traffic = 1432385046.4 * 2.00 * 1024 + 242731.1 * 1024
+        traffic = 1142603761.9 * 2.00 * 1024 + 242555.2 * 1024
     roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
             "traffic": traffic, "kernel": "flat_scan_kernel<rabitq, ip, T=%d>" % tile, "kernel_ms": kms,
             "algorithmic_bytes_per_launch": algo}
@@ -704,7 +704,9 @@ def run_c5(env):
         ops = 2.0 * lcodes * d * nq
         tops = ops / (kms * 1e-3) / 1e12
         roof = {"bound": "mfma", "achieved": tops, "peak": MFMA_I8_PEAK_TOPS, "unit": "TOP/s",
-                "frac": tops / MFMA_I8_PEAK_TOPS, "traffic": None,
+                # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this launch: profiles/prefilter_rb_rabitq_c5.md
+                "frac": tops / MFMA_I8_PEAK_TOPS,
+                "traffic": 1056540.5 * 2.00 * 1024 + 212990.6 * 1024 if (n, d, nq, k) == (5000000, 768, 10000, 10) else None,
                 "kernel": "prefilter_rb_kernel<ip> (int8 MFMA, last level)", "kernel_ms": kms, "ops_per_launch": ops,
                 "codes_per_launch": lcodes}
         dtype = "1-bit codes x 4-bit queries: int8 MFMA pre-selection, u32 popcount rescoring"

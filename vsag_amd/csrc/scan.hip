@@ -394,11 +394,12 @@ block_bitonic_sort(uint64_t* keys, uint32_t P) {
 // an LDS pool; a radix selection finds the k-th smallest of the pool, the keys up to it are compacted and
 // sorted.  When the pool overflows (long runs of nearly equal distances), the k-th smallest of what did fit
 // -- an upper bound of the k-th smallest of all -- becomes the admission key of another round.
-constexpr uint32_t kPoolKeys = 4096;
+constexpr uint32_t kPoolKeys = 4096;       // few queries per call: every wave started without a bound
+constexpr uint32_t kPoolKeysBatch = 2048;  // batches: the bound is known, and twice the workgroups fit a compute unit
 
 __global__ void __launch_bounds__(1024)
 merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, const uint32_t* bound, uint32_t nslots,
-                      uint32_t stride, uint32_t k, uint32_t S, uint32_t* ids, float* dists) {
+                      uint32_t stride, uint32_t k, uint32_t S, uint32_t pool_keys, uint32_t* ids, float* dists) {
     extern __shared__ uint64_t lds[];  // S output keys, then the pool
     __shared__ uint32_t npool;
     __shared__ uint32_t nout;
@@ -435,7 +436,7 @@ merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, cons
                     }
                     base = __shfl(base, 0);
                     const uint32_t pos = base + static_cast<uint32_t>(__popcll(votes & ((1ULL << lane) - 1)));
-                    if (keep && pos < kPoolKeys) {
+                    if (keep && pos < pool_keys) {
                         pool[pos] = key;
                     }
                 }
@@ -445,12 +446,20 @@ merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, cons
             for (uint32_t slot = threadIdx.x; slot < nslots; slot += blockDim.x) {
                 const uint32_t c = cnts[slot];
                 const uint64_t* list = src + static_cast<uint64_t>(slot) * k;
-                for (uint32_t i = 0; i < c; ++i) {
-                    uint64_t key = list[i];
-                    if (key <= admit) {
-                        uint32_t pos = atomicAdd(&npool, 1U);
-                        if (pos < kPoolKeys) {
-                            pool[pos] = key;
+                // Four loads in flight at a time: the pool's atomics would otherwise serialise them.
+                for (uint32_t i = 0; i < c; i += 4) {
+                    uint64_t key[4];
+#pragma unroll
+                    for (uint32_t j = 0; j < 4; ++j) {
+                        key[j] = i + j < c ? list[i + j] : kInfKey;
+                    }
+#pragma unroll
+                    for (uint32_t j = 0; j < 4; ++j) {
+                        if (i + j < c && key[j] <= admit) {
+                            uint32_t pos = atomicAdd(&npool, 1U);
+                            if (pos < pool_keys) {
+                                pool[pos] = key[j];
+                            }
                         }
                     }
                 }
@@ -458,9 +467,9 @@ merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, cons
         }
         __syncthreads();
         const uint32_t total = npool;
-        const uint32_t n = total < kPoolKeys ? total : kPoolKeys;
+        const uint32_t n = total < pool_keys ? total : pool_keys;
         const uint64_t kth = block_kth_smallest(pool, n, k, scratch);
-        if (total <= kPoolKeys) {
+        if (total <= pool_keys) {
             // The k smallest (all of them when fewer than k) go to the front of the output area.
             for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
                 uint64_t key = pool[i];
@@ -502,8 +511,9 @@ launch_merge_partials(const uint64_t* partial, const uint32_t* partial_cnt, cons
                       hipStream_t st) {
     // Few queries: many candidates each (every wave starts without a bound), so give each merge more threads.
     const uint32_t threads = nq <= 256 ? 1024 : 256;
-    hipLaunchKernelGGL(merge_partials_kernel, dim3(static_cast<uint32_t>(nq)), dim3(threads), (S + kPoolKeys) * 8, st,
-                       partial, partial_cnt, bound, nslots, stride, k, S, ids, dists);
+    const uint32_t pool_keys = nq <= 256 ? kPoolKeys : kPoolKeysBatch;
+    hipLaunchKernelGGL(merge_partials_kernel, dim3(static_cast<uint32_t>(nq)), dim3(threads), (S + pool_keys) * 8, st,
+                       partial, partial_cnt, bound, nslots, stride, k, S, pool_keys, ids, dists);
     VA_HIP(hipGetLastError());
     return 0;
 }
