@@ -194,8 +194,10 @@ VSAG_AMD_API int vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* store, const
                                uint32_t k, const vsag_amd_search_options_t* options, uint32_t* ids_dev,
                                float* dists_dev, void* workspace_dev, size_t workspace_bytes, void* stream);
 
-/* Large batches on flat fp32 / sq8 stores are served by a matrix-core contraction that pre-selects candidates,
- * which are then recomputed and selected exactly as the streaming scan does (same results, bit for bit).
+/* Large batches on flat fp32 / sq8 / rabitq stores are served by a matrix-core contraction that pre-selects
+ * candidates, which are then recomputed and selected exactly as the streaming scan does (same results, bit for bit).
+ * rabitq stores with 4-bit queries and at most 1024 dimensions (L2, inner product) expand code bits and query nibbles to
+ * bytes for the int8 matrix cores (the integer product is exact; k up to 256 by default).
  * Posting lists of sq4_uniform codes of at most 128 dimensions (any metric) scan the probe columns behind the first on the
  * int8 matrix cores when a batch has at least 8192 (query, list) groups (same results; off with mode -1).
  * sq8 stores of at most 128 dimensions pre-select on the int8 matrix cores (queries split into two int8 planes

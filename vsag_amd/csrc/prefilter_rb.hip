@@ -17,10 +17,11 @@
 // query.
 //
 // Work split: the 4-bit queries of a group of 128 are expanded to bytes once and stay in LDS (96 KB for 768
-// dimensions) in the operand order of the instruction; a wave owns storage tiles (64 codes, their bits in registers,
-// expanded to 0/1 bytes per step with three vector instructions per dword nibble) and meets all 128 queries of the
-// group: 8 accumulators, 8 matrix instructions per expanded step.  No barrier inside the loop.  What passes goes into
-// the private list of (query, wave of the grid, lane / 32).
+// dimensions) in the operand order of the instruction; a wave owns storage tiles (64 codes; their bits come a granule
+// at a time, one granule ahead, and are expanded to 0/1 bytes with three vector instructions per nibble) and meets all
+// 128 queries of the group: 8 accumulators, 8 matrix instructions per expanded step.  A workgroup is eight waves,
+// two per SIMD, so that one wave's verdicts run under the other's matrix instructions; no barrier inside the loop.
+// What passes goes into the private list of (query, wave of the grid, lane / 32).
 #include "distance.h"
 #include "store.h"
 #include "topk.h"
