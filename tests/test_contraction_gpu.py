@@ -161,7 +161,8 @@ def _rabitq_store(rng, n, d, metric, centered=True):
 
 @pytest.mark.parametrize("metric", [orc.L2, orc.IP])
 @pytest.mark.parametrize("n,d,nq,k,centered", [(30000, 128, 300, 10, True), (20000, 768, 260, 200, True),
-                                               (9000, 100, 129, 50, False), (70000, 256, 700, 100, True)])
+                                               (9000, 100, 129, 50, False), (70000, 256, 700, 100, True),
+                                               (12000, 1024, 150, 20, True)])
 def test_rabitq_contraction_equals_streaming(lib, modes, metric, n, d, nq, k, centered):
     """1-bit codes against 4-bit queries on the int8 matrix cores: the estimator is affine in the integer inner
     product, so the pre-selection is a threshold on it; the rescored result must equal the streaming scan's bits."""
