@@ -2,13 +2,14 @@
 the reference's functional tests: recall floors (tests/test_ivf.cpp:94-102 with RECALL_THRESHOLD 0.85,
 tests/test_index.h:373), result shape (tests/test_index/test_index_search.cpp:60-99), batch == serial
 (tests/test_ivf.cpp:3283-3341), exact self-distance after fp32 reorder (tests/test_ivf.cpp:340-367), error paths."""
+import ctypes as C
 import json
 
 import numpy as np
 import pytest
 
 import oracle as orc
-from vsag_amd import pyvsag
+from vsag_amd import capi, pyvsag
 
 pytestmark = pytest.mark.gpu
 RECALL_THRESHOLD = 0.85
@@ -342,6 +343,25 @@ def test_ivf_large_batch_equals_one_by_one(lib, reorder):
     ids, dists = idx.knn_search_batch(q, k, search)
     for i in range(0, nq, 61):
         si, sd = idx.knn_search(q[i], k, search)
+        assert np.array_equal(si, ids[i]) and np.array_equal(sd.view(np.uint32), dists[i].view(np.uint32)), i
+    idx.close()
+
+
+def test_rabitq_large_batch_equals_one_by_one(lib):
+    """brute_force over 1-bit RaBitQ codes with 4-bit queries: a batch served by the int8 matrix cores returns what
+    single queries (streaming popcount scan) return."""
+    n, d, nq, k = 70000, 256, 600, 50
+    x = vectors(n, d)
+    q = vectors(nq, d, seed=165)
+    labels = np.arange(n, dtype=np.int64) * 3 + 2
+    idx = make("brute_force", d, "ip", base_quantization_type="rabitq", rabitq_bits_per_dim_query=4)
+    assert idx.build(x, labels, n, d) == 0
+    ids, dists = idx.knn_search_batch(q, k, "{}")
+    tile, passes, nbytes = C.c_int(), C.c_uint64(), C.c_uint64()
+    capi.load_library().vsag_amd_last_scan_info(C.byref(tile), C.byref(passes), C.byref(nbytes))
+    assert tile.value == 128, "the batch did not take the matrix-core route"
+    for i in range(0, nq, 41):
+        si, sd = idx.knn_search(q[i], k, "{}")
         assert np.array_equal(si, ids[i]) and np.array_equal(sd.view(np.uint32), dists[i].view(np.uint32)), i
     idx.close()
 
