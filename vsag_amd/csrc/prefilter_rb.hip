@@ -11,7 +11,8 @@
 //      A_c = err / (2 norm), B_c = (norm^2 [- raw^2]) A_c, S_c = set bits            (per code)
 //      u1 = K_q / (qn qm0), u2 = 1 / (qn qm0), u3 = -qm1 / qm0, u4 = (qm2 + qm3) / qm0  (per query; K_q holds the bound)
 //
-// evaluated in fp32 and lowered by 1 + 1e-4 |thr| (several orders above the rounding of either form).  The pairs that
+// evaluated in fp32 and lowered by 1 + 1e-4 thr (several orders above the rounding of either form; the product is
+// never negative, so a negative threshold needs no margin).  The pairs that
 // pass are rescored by rescore_kernel with the streaming arithmetic, so the result is the streaming scan's bit for bit.
 // Codes the derivation does not cover (zero norm, non-positive error factor, zero raw norm) are candidates of every
 // query.
@@ -109,10 +110,13 @@ rabitq_tau_kernel(const float* qmeta, uint32_t qmeta_stride, const uint32_t* bou
                 const double v1 = kq * inv, v3 = -qm1 / qm0, v4 = qm23 / qm0 - 1.0;
                 // Factors so large that the fp32 threshold would lose its margin: everything passes instead.
                 if (fabs(v1) <= 1.0e4 && inv <= 1.0e4 && fabs(v3) <= 64.0 && fabs(v4) <= 1.0e5) {
-                    u1 = static_cast<float>(v1);
-                    u2 = static_cast<float>(inv);
-                    u3 = static_cast<float>(v3);
-                    u4 = static_cast<float>(v4);
+                    // The relative margin rides on the factors: a positive threshold comes out 1e-4 lower, a
+                    // negative one is passed by every (non-negative) product anyway.
+                    const double lower = 1.0 - 1.0e-4;
+                    u1 = static_cast<float>(v1 * lower);
+                    u2 = static_cast<float>(inv * lower);
+                    u3 = static_cast<float>(v3 * lower);
+                    u4 = static_cast<float>(v4 * lower);
                 }
             }
         }
@@ -276,8 +280,7 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
                     uint64_t any = 0;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        float thr = fmaf(cs[j], u3[qb], fmaf(cb[j], u2[qb], fmaf(ca[j], u1[qb], u4[qb])));
-                        thr = fmaf(fabsf(thr), -1.0e-4F, thr);
+                        const float thr = fmaf(cs[j], u3[qb], fmaf(cb[j], u2[qb], fmaf(ca[j], u1[qb], u4[qb])));
                         pass[j] = static_cast<float>(acc[qb][i][4 * gq + j]) >= thr;
                         any |= __ballot(pass[j]);
                     }
