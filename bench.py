@@ -706,7 +706,7 @@ def run_c5(env):
         roof = {"bound": "mfma", "achieved": tops, "peak": MFMA_I8_PEAK_TOPS, "unit": "TOP/s",
                 # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this launch: profiles/prefilter_rb_rabitq_c5.md
                 "frac": tops / MFMA_I8_PEAK_TOPS,
-                "traffic": 1056540.5 * 2.00 * 1024 + 212990.6 * 1024 if (n, d, nq, k) == (5000000, 768, 10000, 10) else None,
+                "traffic": 1056537.4 * 2.00 * 1024 + 213139.2 * 1024 if (n, d, nq, k) == (5000000, 768, 10000, 10) else None,
                 "kernel": "prefilter_rb_kernel<ip> (int8 MFMA, last level)", "kernel_ms": kms, "ops_per_launch": ops,
                 "codes_per_launch": lcodes}
         dtype = "1-bit codes x 4-bit queries: int8 MFMA pre-selection, u32 popcount rescoring"
