@@ -64,3 +64,46 @@ def test_random_configuration(lib, seed):
     for mode, r in res.items():
         assert _same(res[-1], r), (kind, n, d, nq, k, metric, mode)
     st.destroy()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_rabitq_configuration(lib, seed):
+    """1-bit RaBitQ codes against 4-bit queries: the int8 pre-selection against the streaming popcount kernel on seeded
+    random sizes, dimensions (padded and unpadded), k, metrics, centred and far-off data, duplicated queries."""
+    L = lib.load_library()
+    rng = np.random.default_rng(2000 + seed)
+    d = int(rng.choice([32, 64, 100, 128, 200, 256, 384, 512, 960]))
+    n = int(rng.integers(8000, 60000))
+    nq = int(rng.integers(130, 900))
+    k = int(rng.choice([1, 10, 50, 100, 200, 256]))
+    metric = int(rng.choice([orc.L2, orc.IP]))
+    comps = int(rng.choice([1, 5, 50]))
+    sigma = float(rng.choice([0.05, 0.3, 1.0]))
+    x, means = gaussian_mixture(rng, n, d, comps, sigma)
+    q, _ = gaussian_mixture(rng, nq, d, comps, sigma, means=means)
+    if seed % 2 == 0:
+        x /= np.linalg.norm(x, axis=1, keepdims=True)
+        q /= np.linalg.norm(q, axis=1, keepdims=True)
+    if rng.random() < 0.5:
+        q[: nq // 4] = x[rng.integers(0, n, nq // 4)]  # copies of stored vectors
+    if seed % 3 == 0:
+        x[rng.integers(0, n, 40)] = x[0]               # a clump of equal vectors
+    g = rng.standard_normal((d, d))
+    rot, r = np.linalg.qr(g)
+    rot = (rot * np.sign(np.diag(r))).astype(np.float32)
+    cen = orc.rabitq_train(x, rot)
+    st = Store(capi.KIND_RABITQ, metric, d, rot=rot, centroid=cen)
+    st.append(orc.rabitq_encode(x, rot, cen, metric))
+    res = {}
+    try:
+        for mode in (-1, 1):
+            capi.check(L.vsag_amd_set_scan_contraction(mode))
+            res[mode] = st.flat_scan(q, k)
+            if mode != -1:
+                tile = capi.C.c_int()
+                L.vsag_amd_last_scan_info(capi.C.byref(tile), None, None)
+                assert tile.value == 128, "the matrix-core route did not run"
+    finally:
+        capi.check(L.vsag_amd_set_scan_contraction(0))
+    assert _same(res[-1], res[1]), (n, d, nq, k, metric)
+    st.destroy()
