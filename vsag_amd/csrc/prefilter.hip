@@ -378,12 +378,14 @@ struct RescoreArgs {
     uint32_t first_slot;  // the list of the first level of this call; out_slot - first_slot levels came before
     uint32_t out_slot;
     uint32_t* gate;  // per query: 1 = candidates overflowed at some level, the streaming kernel must serve the query
-    // sub_lists != 0: the candidates of a query sit in sub_lists lists of sub_cap (<= kRescoreGather) slots with a
-    // count each (a count above sub_cap = that list overflowed); they are gathered into LDS a few lists at a time.
-    uint32_t sub_lists, sub_cap;
+    // sub_lists != 0: the candidates of a query sit in sub_lists lists of sub_cap (<= gather) slots with a count each
+    // (a count above sub_cap = that list overflowed); they are gathered into `gather` words of LDS.
+    uint32_t sub_lists, sub_cap, gather;
 };
 
-constexpr uint32_t kRescoreGather = 4096;
+// Words of LDS for gathered candidates: small, so that many of these one-wave workgroups share a compute unit (the
+// kernel lives on memory latency), but never less than one private list.
+constexpr uint32_t kRescoreGather = 1024;
 
 // One wave per query: exact distances of its candidates by the streaming kernel's arithmetic, best k kept.
 template <int KIND, int METRIC>
@@ -459,12 +461,13 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
     if (r.sub_lists == 0) {
         rescore(r.cand + static_cast<uint64_t>(q) * r.cap, as_const(counts)[0]);
     } else {
-        // Gather the private lists of the query behind the selector, as many at a time as are sure to fit: a lane
-        // per list, offsets by a wave scan.
+        // Gather the private lists of the query behind the selector -- a lane per list, offsets by a wave scan -- and
+        // rescore whenever the next round of lists might not fit (usually once, at the end: full waves of candidates).
         uint32_t* flat = reinterpret_cast<uint32_t*>(keys + r.S);
         const uint32_t* lists = r.cand + static_cast<uint64_t>(q) * r.sub_lists * r.sub_cap;
-        uint32_t batch = kRescoreGather / r.sub_cap;
+        uint32_t batch = r.gather / r.sub_cap;
         batch = batch > kWave ? kWave : (batch == 0 ? 1 : batch);
+        uint32_t fill = 0;
         for (uint32_t g0 = 0; g0 < r.sub_lists; g0 += batch) {
             const uint32_t g = g0 + lane;
             const uint32_t c = lane < batch && g < r.sub_lists ? as_const(counts)[g] : 0U;
@@ -477,14 +480,20 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
             if (sum == 0) {
                 continue;
             }
-            wave_lds_fence();  // the previous batch has been read
-            const uint32_t at = incl - c;
+            if (fill + sum > r.gather) {
+                wave_lds_fence();
+                rescore(flat, fill);
+                fill = 0;
+                wave_lds_fence();  // what was gathered has been read
+            }
+            const uint32_t at = fill + incl - c;
             for (uint32_t i = 0; i < c; ++i) {
                 flat[at + i] = as_const(lists)[static_cast<uint64_t>(g) * r.sub_cap + i];
             }
-            wave_lds_fence();
-            rescore(flat, sum);
+            fill += sum;
         }
+        wave_lds_fence();
+        rescore(flat, fill);
     }
     wave_lds_fence();
     bs = __builtin_amdgcn_readfirstlane(__atomic_load_n(&r.bound[q], __ATOMIC_RELAXED));
@@ -575,8 +584,9 @@ launch_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t
     r.gate = gate;
     r.sub_lists = sub_lists;
     r.sub_cap = sub_cap;
+    r.gather = std::max(kRescoreGather, sub_cap);
     dim3 rgrid(static_cast<uint32_t>(nq));
-    const size_t lds = S * 8 + (sub_lists != 0 ? kRescoreGather * 4 : 0);
+    const size_t lds = S * 8 + (sub_lists != 0 ? r.gather * 4 : 0);
     if (s->kind == VSAG_AMD_KIND_SQ8) {
         launch_rescore_m<VSAG_AMD_KIND_SQ8>(s->metric, rgrid, lds, st, a, r);
     } else if (s->kind == VSAG_AMD_KIND_RABITQ) {
