@@ -470,6 +470,104 @@ rabitq_finish_query_kernel(const float* raw, const float* rotated, uint64_t nq, 
     }
 }
 
+// The same, one wave per query: the loads are coalesced and everything but the two sums whose order matters (the
+// squared norms, added dimension by dimension like the reference does) is spread over the lanes.  The sum of the
+// quantised values is a sum of small integers, exact in any order.  LDS: dim floats, twice that with a raw norm.
+__global__ void __launch_bounds__(64)
+rabitq_finish_query_wave_kernel(const float* raw, const float* rotated, uint64_t nq, uint32_t dim, const float* centroid,
+                                int metric, int query_bits, uint8_t* qcodes) {
+    extern __shared__ float fq_lds[];
+    const uint64_t i = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    RabitqLayout l = rabitq_layout(dim, metric, query_bits);
+    const float* y = rotated + i * dim;
+    uint8_t* qc = qcodes + i * l.query_code_size;
+    float* t = fq_lds;        // y - centroid
+    float* xx = fq_lds + dim;  // squares of the raw query
+    for (uint32_t d = lane; d < dim; d += kWave) {
+        t[d] = y[d] - centroid[d];
+        if (l.has_raw_norm) {
+            const float x = raw[i * dim + d];
+            xx[d] = x * x;
+        }
+    }
+    wave_lds_fence();
+    float raw_norm = 0.0F, norm_sq = 0.0F;
+    if (lane == 0) {
+        for (uint32_t d = 0; d < dim; ++d) {
+            const float v = t[d];
+            norm_sq = v * v + norm_sq;
+            if (l.has_raw_norm) {
+                raw_norm += xx[d];
+            }
+        }
+    }
+    raw_norm = sqrtf(__shfl(raw_norm, 0));
+    norm_sq = __shfl(norm_sq, 0);
+    const float norm = norm_sq < 1e-5F ? 1.0F : sqrtf(norm_sq);
+    if (query_bits == 4) {
+        float lb = FLT_MAX, ub = -FLT_MAX;
+        for (uint32_t d = lane; d < dim; d += kWave) {
+            const float v = t[d] / norm;
+            if (v < lb) {
+                lb = v;
+            }
+            if (v > ub) {
+                ub = v;
+            }
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ol = __shfl_xor(lb, off), ou = __shfl_xor(ub, off);
+            if (ol < lb) {
+                lb = ol;
+            }
+            if (ou > ub) {
+                ub = ou;
+            }
+        }
+        const float delta = (ub - lb) / 15;
+        const float inv_delta = fabsf(delta) < 1e-5F ? 0.0F : 1.0F / delta;
+        float qsum = 0.0F;
+        for (uint32_t b = lane; b < l.plane_bytes; b += kWave) {
+            uint32_t plane[4] = {0, 0, 0, 0};
+            for (uint32_t e = 0; e < 8; ++e) {
+                const uint32_t d = b * 8 + e;
+                if (d >= dim) {
+                    break;
+                }
+                const float v = t[d] / norm;
+                const float val = roundf((v - lb) * inv_delta);
+                const uint32_t q = static_cast<uint8_t>(val);
+                qsum += static_cast<float>(val);
+                for (uint32_t p = 0; p < 4; ++p) {
+                    plane[p] |= ((q >> p) & 1U) << e;
+                }
+            }
+            for (uint32_t p = 0; p < 4; ++p) {
+                qc[p * l.plane_bytes + b] = static_cast<uint8_t>(plane[p]);
+            }
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            qsum += __shfl_xor(qsum, off);
+        }
+        if (lane == 0) {
+            store_f32(qc + l.q_offset_lb, lb);
+            store_f32(qc + l.q_offset_delta, delta);
+            store_f32(qc + l.q_offset_sum, qsum);
+        }
+    } else {
+        for (uint32_t d = lane; d < dim; d += kWave) {
+            store_f32(qc + 4 * d, t[d] / norm);
+        }
+    }
+    if (lane == 0) {
+        store_f32(qc + l.q_offset_norm, norm);
+        if (l.has_raw_norm) {
+            store_f32(qc + l.q_offset_raw_norm, raw_norm);
+        }
+    }
+}
+
 int
 squ_encode_launch(const float* x, uint64_t n, uint32_t dim, int bits, int metric, const float* bounds, uint8_t* codes,
                   hipStream_t st) {
@@ -531,8 +629,14 @@ rabitq_process_query_launch(const float* q, uint64_t nq, uint32_t dim, const flo
     }
     uint64_t qsize = rabitq_query_code_size(dim, metric, query_bits);
     return rabitq_rotate_slabs(q, nq, dim, rot, st, [&](uint64_t s, uint64_t m, const float* rotated) {
-        hipLaunchKernelGGL(rabitq_finish_query_kernel, dim3(static_cast<uint32_t>(div_up(m, 64))), dim3(64), 0, st,
-                           q + s * dim, rotated, m, dim, centroid, metric, query_bits, qcodes + s * qsize);
+        const size_t lds = static_cast<size_t>(dim) * 4 * (rabitq_layout(dim, metric, query_bits).has_raw_norm ? 2 : 1);
+        if (lds <= 48 * 1024) {
+            hipLaunchKernelGGL(rabitq_finish_query_wave_kernel, dim3(static_cast<uint32_t>(m)), dim3(64), lds, st,
+                               q + s * dim, rotated, m, dim, centroid, metric, query_bits, qcodes + s * qsize);
+        } else {
+            hipLaunchKernelGGL(rabitq_finish_query_kernel, dim3(static_cast<uint32_t>(div_up(m, 64))), dim3(64), 0, st,
+                               q + s * dim, rotated, m, dim, centroid, metric, query_bits, qcodes + s * qsize);
+        }
         VA_HIP(hipGetLastError());
         return 0;
     });
