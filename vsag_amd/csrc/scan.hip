@@ -557,6 +557,11 @@ static void
 make_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, uint64_t ntiles, ScanPlan* p) {
     p->S = selector_slots(k);
     int T = g_tile_override > 0 ? g_tile_override : default_query_tile(s);
+    if (g_tile_override <= 0 && s->kind == VSAG_AMD_KIND_FP32 && ntiles >= 1024) {
+        // 512 bytes per code and pass: on a long scan the passes are what costs (100k x 128: a quarter faster than 4);
+        // short scans (centroid routing, the exact prefix of a pre-selected batch) live on their selectors instead.
+        T = 8;
+    }
     while (T > 1 && static_cast<uint64_t>(T) > nq) {
         T >>= 1;
     }
