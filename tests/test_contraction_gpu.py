@@ -180,3 +180,28 @@ def test_rabitq_contraction_equals_streaming(lib, modes, metric, n, d, nq, k, ce
     assert tile == 128, "the contraction path did not run"
     assert same(plain, fast)
     st.destroy()
+
+
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
+@pytest.mark.parametrize("n,d,nq,k", [(40000, 128, 300, 10), (20001, 100, 129, 100), (5000, 33, 1000, 7),
+                                      (70000, 64, 600, 1)])
+def test_sq8_uniform_contraction_equals_streaming(lib, modes, metric, n, d, nq, k):
+    """sq8_uniform: code and query are both rows of bytes, the product is an integer the int8 matrix cores deliver
+    exactly; distances are integers scaled once, so ties abound and must come out in id order on both routes."""
+    rng = np.random.default_rng(n + d + k + 3 * metric)
+    x, means = gaussian_mixture(rng, n, d, 30, 0.05)
+    q, _ = gaussian_mixture(rng, nq, d, 30, 0.05, means=means)
+    q[3] = x[17]          # a stored vector
+    q[4] = 0.0            # clamps to the lower bound everywhere
+    q[5] = 10.0           # clamps to the upper bound everywhere
+    lb, diff = orc.sq_train_uniform(x, 8, metric, mode=1)
+    codes = orc.squ_encode(x, 8, lb, diff, metric)
+    st = Store(capi.KIND_SQ8_UNIFORM, metric, d, bounds=[lb, diff])
+    st.append(codes[:n // 3])
+    st.append(codes[n // 3:])
+    plain, fast, tile = modes(st, q, k)
+    assert tile == 256, "the int8 route did not run"
+    assert same(plain, fast)
+    plain, fast, tile = modes(st, q, k, mode=2)  # no fp32 route for this kind: still the int8 matrix cores
+    assert tile == 256 and same(plain, fast)
+    st.destroy()

@@ -107,3 +107,38 @@ def test_random_rabitq_configuration(lib, seed):
         capi.check(L.vsag_amd_set_scan_contraction(0))
     assert _same(res[-1], res[1]), (n, d, nq, k, metric)
     st.destroy()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_sq8_uniform_configuration(lib, seed):
+    """sq8_uniform flat stores: the int8 pre-selection (exact integer products, the l2 form of the test for every
+    metric) against the streaming kernel on seeded random configurations."""
+    L = lib.load_library()
+    rng = np.random.default_rng(3000 + seed)
+    d = int(rng.choice([16, 24, 32, 48, 64, 96, 100, 128]))
+    n = int(rng.integers(20000, 200000))
+    nq = int(rng.integers(512, 2500))
+    k = int(rng.choice([1, 5, 10, 32, 100]))
+    metric = int(rng.choice([orc.L2, orc.IP, orc.COSINE]))
+    comps = int(rng.choice([1, 5, 50, 500]))
+    sigma = float(rng.choice([0.01, 0.05, 0.3]))
+    x, means = gaussian_mixture(rng, n, d, comps, sigma)
+    q, _ = gaussian_mixture(rng, nq, d, comps, sigma, means=means)
+    if rng.random() < 0.4:
+        q[: nq // 4] = x[rng.integers(0, n, nq // 4)]
+    lb, diff = orc.sq_train_uniform(x, 8, metric, mode=int(rng.choice([1, 3])))
+    st = Store(capi.KIND_SQ8_UNIFORM, metric, d, bounds=[lb, diff])
+    st.append(orc.squ_encode(x, 8, lb, diff, metric))
+    res = {}
+    try:
+        for mode in (-1, 1):
+            capi.check(L.vsag_amd_set_scan_contraction(mode))
+            res[mode] = st.flat_scan(q, k)
+            if mode != -1:
+                tile = capi.C.c_int()
+                L.vsag_amd_last_scan_info(capi.C.byref(tile), None, None)
+                assert tile.value == 256, "the int8 route did not run"
+    finally:
+        capi.check(L.vsag_amd_set_scan_contraction(0))
+    assert _same(res[-1], res[1]), (n, d, nq, k, metric)
+    st.destroy()

@@ -519,12 +519,27 @@ int launch_prefilter_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq,
                         const uint32_t* bound, uint8_t* scratch, uint32_t* cand, uint32_t* cand_cnt, uint32_t sub_lists,
                         uint32_t sub_cap, hipStream_t st);
 
+bool prefilter_i8_supports(const vsag_amd_store* s);
+
 bool
 prefilter_supports(const vsag_amd_store* s) {
     if (prefilter_rb_supports(s)) {
         return true;
     }
+    if (s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
+        return prefilter_i8_supports(s);  // the int8 matrix cores or nothing
+    }
     return s->nlist == 0 && (s->kind == VSAG_AMD_KIND_FP32 || s->kind == VSAG_AMD_KIND_SQ8) && s->pf_term != nullptr;
+}
+
+// sq8_uniform: the per-code term of the int8 test, from the code's stored scalar (prefilter_i8.hip).
+__global__ void __launch_bounds__(256)
+uniform_term_kernel(const uint32_t* meta, uint64_t first, uint64_t count, int is_l2, float lb, float* term) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < count) {
+        const float m = __uint_as_float(meta[first + i]);
+        term[first + i] = is_l2 ? m : -(lb * m);
+    }
 }
 
 // |y|^2 for freshly appended codes (y as the contraction sees it: scaled codes for sq8 l2, raw code values
@@ -535,7 +550,10 @@ launch_code_terms(vsag_amd_store* s, uint64_t first, uint64_t count, hipStream_t
         return 0;
     }
     dim3 grid(static_cast<uint32_t>(div_up(count, 256)));
-    if (s->kind == VSAG_AMD_KIND_SQ8) {
+    if (s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
+        hipLaunchKernelGGL(uniform_term_kernel, grid, dim3(256), 0, st, s->meta, first, count,
+                           s->metric == VSAG_AMD_METRIC_L2 ? 1 : 0, s->ulb, s->pf_term);
+    } else if (s->kind == VSAG_AMD_KIND_SQ8) {
         const float* scale = s->metric == VSAG_AMD_METRIC_L2 ? s->scale_dev : nullptr;
         hipLaunchKernelGGL(code_term_kernel<VSAG_AMD_KIND_SQ8>, grid, dim3(256), 0, st, s->tiles, s->G, scale, first,
                            count, s->pf_term, s->pf_ymax);
@@ -589,6 +607,8 @@ launch_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t
     const size_t lds = S * 8 + (sub_lists != 0 ? r.gather * 4 : 0);
     if (s->kind == VSAG_AMD_KIND_SQ8) {
         launch_rescore_m<VSAG_AMD_KIND_SQ8>(s->metric, rgrid, lds, st, a, r);
+    } else if (s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
+        launch_rescore_m<VSAG_AMD_KIND_SQ8_UNIFORM>(s->metric, rgrid, lds, st, a, r);
     } else if (s->kind == VSAG_AMD_KIND_RABITQ) {
         launch_rescore_m<VSAG_AMD_KIND_RABITQ>(s->metric, rgrid, lds, st, a, r);
     } else {

@@ -1,4 +1,5 @@
-// Pre-selection for large query batches on a flat sq8 store of at most 128 dimensions, on the int8 matrix cores.
+// Pre-selection for large query batches on a flat sq8 (or sq8_uniform, see UniformQuantizeArgs) store of at most 128
+// dimensions, on the int8 matrix cores.
 //
 // The streaming distance of an sq8 code is a function of <b, c>: c the code bytes (0..255), b the query folded
 // with the per-dimension scale (l2: b_d = (q_d - lb_d) scale_d, ip: b_d = q_d scale_d).  Each query row b is split
@@ -168,6 +169,100 @@ quantize_queries_i8_kernel(QuantizeArgs p) {
         }
         p.tau[q] = static_cast<uint32_t>(ti);
     }
+}
+
+// sq8_uniform stores: the query is a row of bytes itself (its uniform code, 0..255), so the product with the code is
+// an integer the matrix cores deliver exactly.  A byte q splits as 256 h + l with h in {0, 1} and l in [-128, 127];
+// with the codes staged as c - 128 the kernel's T = 256 H + L is <code, query> - 128 sum(query).  The streaming
+// distance is a short fp32 expression of that integer and two scalars (distance.h, finish_distances):
+//      l2:       ((norm_q + norm_o) - 2 ip) rate            ip/cosine:  1 - (lb (sum_q + sum_o) + rate ip + lb^2)
+// so "distance <= bound" becomes the kernel's test fma(T, u, term_o) <= tau with (u, term_o) = (-2, norm_o) or
+// (-rate, -lb sum_o), and tau carrying the bound, the query's scalars and every rounding of both forms.
+struct UniformQuantizeArgs {
+    const uint32_t* qtab;  // the queries' uniform codes, qstride words each
+    uint32_t qstride;
+    uint32_t kdim;         // <= 128
+    const float* qmeta;    // per query: norm (l2) or sum (ip, cosine) of its code
+    uint32_t qmeta_stride;
+    int is_l2;
+    float lb, rate, lb2;
+    const uint32_t* bound;
+    uint64_t nq, nq_pad;
+    uint8_t* q8;
+    float* u;
+    uint32_t* tau;
+};
+
+// One wave per query; lane l owns dimensions l and l + 64.
+__global__ void __launch_bounds__(64)
+quantize_uniform_i8_kernel(UniformQuantizeArgs p) {
+    const uint64_t q = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    uint8_t* out = p.q8 + q * kI8QueryBytes;
+    if (q >= p.nq) {
+        out[lane] = 0;
+        out[64 + lane] = 0;
+        out[128 + lane] = 0;
+        out[192 + lane] = 0;
+        if (lane == 0) {
+            p.u[q] = 0.0F;
+            p.tau[q] = __float_as_uint(-__builtin_inff());
+        }
+        return;
+    }
+    const uint32_t* row = p.qtab + q * p.qstride;
+    double sum = 0.0;
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+        const uint32_t d = lane + 64 * r;
+        const uint32_t v = d < p.kdim ? (row[d >> 2] >> (8 * (d & 3))) & 255U : 0U;
+        const uint32_t h = v >> 7;
+        out[d] = static_cast<uint8_t>(h);
+        out[128 + d] = static_cast<uint8_t>(v - 256U * h);  // the low byte of the two's complement of v - 256 h
+        sum += static_cast<double>(v);
+    }
+    sum = wave_sum_f64(sum);  // exact: integers
+    if (lane != 0) {
+        return;
+    }
+    const uint32_t bbits = p.bound[q];
+    const double rate = static_cast<double>(p.rate);
+    p.u[q] = p.is_l2 ? -2.0F : -p.rate;
+    if (bbits == 0xFFFFFFFFU) {
+        p.tau[q] = __float_as_uint(3.0e38F);  // no bound yet: everything is a candidate
+        return;
+    }
+    constexpr double kU = 5.9604644775390625e-8;  // 2^-24
+    const double bd = static_cast<double>(ordered_to_float(bbits));
+    const double qm = static_cast<double>(p.qmeta[q * p.qmeta_stride]);
+    const double ip_max = 255.0 * sum;                 // <code, query> of any code
+    const double t_max = 128.0 * 256.0 * p.kdim;       // |T| of any code
+    const double m_max = p.is_l2 ? 255.0 * 255.0 * p.kdim : 255.0 * p.kdim;  // norm_o, sum_o of any code
+    double t;
+    if (p.is_l2) {
+        // Streaming: fl(fl(fl(qm + m) - 2 R) rate), R the integer as a float (exact below 2^24).  The two sums round
+        // by at most u of their magnitude each, the product by u of itself.
+        if (!(rate > 0.0)) {
+            p.tau[q] = __float_as_uint(3.0e38F);
+            return;
+        }
+        const double reach = fabs(qm) + m_max + 2.0 * ip_max;
+        const double x_max = bd / rate * (1.0 + 4.0 * kU) + 4.0 * kU * reach;  // what qm + m - 2 ip may reach
+        // qm + m - 2 (T + 128 sum) <= x_max   <=>   m - 2 T <= x_max - qm + 256 sum
+        t = x_max - qm + 256.0 * sum;
+        // The test itself: fl(m - 2 T) in one fma against the rounded threshold.
+        t += 4.0 * kU * (m_max + 2.0 * t_max + fabs(t));
+    } else {
+        // Streaming: r = fl(fl(fl(lb fl(qm + m)) + fl(rate R)) + lb2), distance fl(1 - r).
+        const double lb = fabs(static_cast<double>(p.lb)), lb2 = fabs(static_cast<double>(p.lb2));
+        const double reach = lb * (fabs(qm) + m_max) + rate * ip_max + lb2 + 1.0 + fabs(bd);
+        const double e_stream = 8.0 * kU * reach;
+        // 1 - lb (qm + m) - rate (T + 128 sum) - lb2 <= bd + e   <=>   -rate T - lb m <= bd + e - 1 + lb qm + 128 rate sum + lb2
+        t = bd + e_stream - 1.0 + static_cast<double>(p.lb) * qm + 128.0 * rate * sum + static_cast<double>(p.lb2);
+        // term_o = fl(-lb m) and the fma of the test.
+        t += 4.0 * kU * (2.0 * lb * m_max + rate * t_max + fabs(t));
+    }
+    p.tau[q] = __float_as_uint(t < 3.0e38 ? (t > -3.0e38 ? static_cast<float>(t) : -3.0e38F) : 3.0e38F);
 }
 
 struct PrefilterI8Args {
@@ -421,7 +516,8 @@ prefilter_i8_kernel(PrefilterI8Args p) {
 
 bool
 prefilter_i8_supports(const vsag_amd_store* s) {
-    return s->kind == VSAG_AMD_KIND_SQ8 && s->dpad <= kI8Dims && s->G <= 8;
+    return (s->kind == VSAG_AMD_KIND_SQ8 || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) && s->nlist == 0 && s->pf_term != nullptr &&
+           s->dpad <= kI8Dims && s->G <= 8;
 }
 
 // Bytes of the quantized query table for nq queries.
@@ -447,8 +543,29 @@ launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride
                     uint32_t qmeta_stride, uint64_t nq, uint64_t tile_begin, uint64_t tile_end, const uint32_t* bound,
                     uint8_t* q8, float* u, uint32_t* tau, uint32_t* cand, uint32_t* cand_cnt, uint32_t sub_lists,
                     uint32_t sub_cap, hipStream_t st) {
-    const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
+    const bool uniform = s->kind == VSAG_AMD_KIND_SQ8_UNIFORM;
+    // The uniform kinds use the l2 form of the test (fma of the integer and a per-code term) for every metric.
+    const bool l2 = s->metric == VSAG_AMD_METRIC_L2 || uniform;
     const uint64_t nq_pad = div_up(nq, static_cast<uint64_t>(kI8Group)) * kI8Group;
+    if (uniform) {
+        UniformQuantizeArgs z{};
+        z.qtab = reinterpret_cast<const uint32_t*>(qtab);
+        z.qstride = qstride;
+        z.kdim = s->dpad;
+        z.qmeta = qmeta;
+        z.qmeta_stride = qmeta_stride;
+        z.is_l2 = s->metric == VSAG_AMD_METRIC_L2 ? 1 : 0;
+        z.lb = s->ulb;
+        z.rate = s->scalar_rate;
+        z.lb2 = s->ulb * s->ulb;
+        z.bound = bound;
+        z.nq = nq;
+        z.nq_pad = nq_pad;
+        z.q8 = q8;
+        z.u = u;
+        z.tau = tau;
+        hipLaunchKernelGGL(quantize_uniform_i8_kernel, dim3(static_cast<uint32_t>(nq_pad)), dim3(kWave), 0, st, z);
+    }
     QuantizeArgs z{};
     z.qtab = qtab;
     z.qstride = qstride;
@@ -464,7 +581,9 @@ launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride
     z.q8 = q8;
     z.u = u;
     z.tau = tau;
-    hipLaunchKernelGGL(quantize_queries_i8_kernel, dim3(static_cast<uint32_t>(nq_pad)), dim3(kWave), 0, st, z);
+    if (!uniform) {
+        hipLaunchKernelGGL(quantize_queries_i8_kernel, dim3(static_cast<uint32_t>(nq_pad)), dim3(kWave), 0, st, z);
+    }
     VA_HIP(hipGetLastError());
 
     PrefilterI8Args p{};

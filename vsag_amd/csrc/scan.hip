@@ -713,7 +713,8 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
         return;
     }
     c->contraction = true;
-    c->int8 = g_prefilter_mode != 2 && prefilter_i8_supports(s);
+    // Mode 2 asks for the fp32 matrix cores, which sq8_uniform stores have no route for.
+    c->int8 = prefilter_i8_supports(s) && (g_prefilter_mode != 2 || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM);
     c->rb = rb;
     c->rb_scratch = rb ? prefilter_rb_scratch_bytes(s, nq) : 0;
     c->prefix_tiles = prefix;
