@@ -194,7 +194,7 @@ VSAG_AMD_API int vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* store, const
                                uint32_t k, const vsag_amd_search_options_t* options, uint32_t* ids_dev,
                                float* dists_dev, void* workspace_dev, size_t workspace_bytes, void* stream);
 
-/* Large batches on flat fp32 / sq8 / sq8_uniform (at most 128 dimensions) / rabitq stores are served by a matrix-core contraction that pre-selects
+/* Large batches on flat fp32 / sq8 / sq8_uniform / sq4_uniform (the uniform kinds: at most 128 dimensions) / rabitq stores are served by a matrix-core contraction that pre-selects
  * candidates, which are then recomputed and selected exactly as the streaming scan does (same results, bit for bit).
  * rabitq stores with 4-bit queries and at most 1024 dimensions (L2, inner product) expand code bits and query nibbles to
  * bytes for the int8 matrix cores (the integer product is exact; k up to 256 by default).

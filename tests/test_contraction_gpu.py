@@ -205,3 +205,25 @@ def test_sq8_uniform_contraction_equals_streaming(lib, modes, metric, n, d, nq, 
     plain, fast, tile = modes(st, q, k, mode=2)  # no fp32 route for this kind: still the int8 matrix cores
     assert tile == 256 and same(plain, fast)
     st.destroy()
+
+
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
+@pytest.mark.parametrize("n,d,nq,k", [(40000, 128, 300, 10), (20001, 100, 129, 100), (5000, 33, 1000, 7),
+                                      (70000, 64, 600, 1)])
+def test_sq4_uniform_contraction_equals_streaming(lib, modes, metric, n, d, nq, k):
+    """sq4_uniform: two 4-bit values per byte, split into low- and high-nibble granules when staged."""
+    rng = np.random.default_rng(n + d + k + 5 * metric)
+    x, means = gaussian_mixture(rng, n, d, 30, 0.05)
+    q, _ = gaussian_mixture(rng, nq, d, 30, 0.05, means=means)
+    q[3] = x[17]
+    q[4] = 0.0
+    q[5] = 10.0
+    lb, diff = orc.sq_train_uniform(x, 4, metric, mode=3)
+    codes = orc.squ_encode(x, 4, lb, diff, metric)
+    st = Store(capi.KIND_SQ4_UNIFORM, metric, d, bounds=[lb, diff])
+    st.append(codes[:n // 3])
+    st.append(codes[n // 3:])
+    plain, fast, tile = modes(st, q, k)
+    assert tile == 256, "the int8 route did not run"
+    assert same(plain, fast)
+    st.destroy()

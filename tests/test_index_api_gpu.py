@@ -366,7 +366,7 @@ def test_rabitq_large_batch_equals_one_by_one(lib):
     idx.close()
 
 
-@pytest.mark.parametrize("quant", ["fp32", "sq8", "sq8_uniform"])
+@pytest.mark.parametrize("quant", ["fp32", "sq8", "sq8_uniform", "sq4_uniform"])
 def test_large_batch_equals_one_by_one(lib, quant):
     """A batch large enough for the matrix-core path of the flat scan returns what single queries return."""
     n, d, nq, k = 70000, 32, 600, 10

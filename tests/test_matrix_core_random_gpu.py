@@ -110,9 +110,10 @@ def test_random_rabitq_configuration(lib, seed):
 
 
 @pytest.mark.parametrize("seed", range(8))
-def test_random_sq8_uniform_configuration(lib, seed):
-    """sq8_uniform flat stores: the int8 pre-selection (exact integer products, the l2 form of the test for every
-    metric) against the streaming kernel on seeded random configurations."""
+def test_random_uniform_configuration(lib, seed):
+    """sq8_uniform and sq4_uniform flat stores: the int8 pre-selection (exact integer products, the l2 form of the test
+    for every metric) against the streaming kernel on seeded random configurations."""
+    bits = 8 if seed % 2 == 0 else 4
     L = lib.load_library()
     rng = np.random.default_rng(3000 + seed)
     d = int(rng.choice([16, 24, 32, 48, 64, 96, 100, 128]))
@@ -126,9 +127,9 @@ def test_random_sq8_uniform_configuration(lib, seed):
     q, _ = gaussian_mixture(rng, nq, d, comps, sigma, means=means)
     if rng.random() < 0.4:
         q[: nq // 4] = x[rng.integers(0, n, nq // 4)]
-    lb, diff = orc.sq_train_uniform(x, 8, metric, mode=int(rng.choice([1, 3])))
-    st = Store(capi.KIND_SQ8_UNIFORM, metric, d, bounds=[lb, diff])
-    st.append(orc.squ_encode(x, 8, lb, diff, metric))
+    lb, diff = orc.sq_train_uniform(x, bits, metric, mode=int(rng.choice([1, 3])))
+    st = Store(capi.KIND_SQ8_UNIFORM if bits == 8 else capi.KIND_SQ4_UNIFORM, metric, d, bounds=[lb, diff])
+    st.append(orc.squ_encode(x, bits, lb, diff, metric))
     res = {}
     try:
         for mode in (-1, 1):
@@ -140,5 +141,5 @@ def test_random_sq8_uniform_configuration(lib, seed):
                 assert tile.value == 256, "the int8 route did not run"
     finally:
         capi.check(L.vsag_amd_set_scan_contraction(0))
-    assert _same(res[-1], res[1]), (n, d, nq, k, metric)
+    assert _same(res[-1], res[1]), (bits, n, d, nq, k, metric)
     st.destroy()

@@ -526,7 +526,7 @@ prefilter_supports(const vsag_amd_store* s) {
     if (prefilter_rb_supports(s)) {
         return true;
     }
-    if (s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
+    if (s->kind == VSAG_AMD_KIND_SQ8_UNIFORM || s->kind == VSAG_AMD_KIND_SQ4_UNIFORM) {
         return prefilter_i8_supports(s);  // the int8 matrix cores or nothing
     }
     return s->nlist == 0 && (s->kind == VSAG_AMD_KIND_FP32 || s->kind == VSAG_AMD_KIND_SQ8) && s->pf_term != nullptr;
@@ -550,7 +550,7 @@ launch_code_terms(vsag_amd_store* s, uint64_t first, uint64_t count, hipStream_t
         return 0;
     }
     dim3 grid(static_cast<uint32_t>(div_up(count, 256)));
-    if (s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
+    if (s->kind == VSAG_AMD_KIND_SQ8_UNIFORM || s->kind == VSAG_AMD_KIND_SQ4_UNIFORM) {
         hipLaunchKernelGGL(uniform_term_kernel, grid, dim3(256), 0, st, s->meta, first, count,
                            s->metric == VSAG_AMD_METRIC_L2 ? 1 : 0, s->ulb, s->pf_term);
     } else if (s->kind == VSAG_AMD_KIND_SQ8) {
@@ -609,6 +609,8 @@ launch_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t
         launch_rescore_m<VSAG_AMD_KIND_SQ8>(s->metric, rgrid, lds, st, a, r);
     } else if (s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
         launch_rescore_m<VSAG_AMD_KIND_SQ8_UNIFORM>(s->metric, rgrid, lds, st, a, r);
+    } else if (s->kind == VSAG_AMD_KIND_SQ4_UNIFORM) {
+        launch_rescore_m<VSAG_AMD_KIND_SQ4_UNIFORM>(s->metric, rgrid, lds, st, a, r);
     } else if (s->kind == VSAG_AMD_KIND_RABITQ) {
         launch_rescore_m<VSAG_AMD_KIND_RABITQ>(s->metric, rgrid, lds, st, a, r);
     } else {

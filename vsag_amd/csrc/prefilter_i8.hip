@@ -171,7 +171,7 @@ quantize_queries_i8_kernel(QuantizeArgs p) {
     }
 }
 
-// sq8_uniform stores: the query is a row of bytes itself (its uniform code, 0..255), so the product with the code is
+// sq8_uniform (and, with 4-bit values, sq4_uniform) stores: the query is a row of bytes itself (its uniform code, 0..255), so the product with the code is
 // an integer the matrix cores deliver exactly.  A byte q splits as 256 h + l with h in {0, 1} and l in [-128, 127];
 // with the codes staged as c - 128 the kernel's T = 256 H + L is <code, query> - 128 sum(query).  The streaming
 // distance is a short fp32 expression of that integer and two scalars (distance.h, finish_distances):
@@ -185,6 +185,7 @@ struct UniformQuantizeArgs {
     const float* qmeta;    // per query: norm (l2) or sum (ip, cosine) of its code
     uint32_t qmeta_stride;
     int is_l2;
+    int nibbles;           // sq4_uniform: qtab holds, per code dword, a word of low-nibble and one of high-nibble values
     float lb, rate, lb2;
     const uint32_t* bound;
     uint64_t nq, nq_pad;
@@ -214,8 +215,15 @@ quantize_uniform_i8_kernel(UniformQuantizeArgs p) {
     double sum = 0.0;
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
-        const uint32_t d = lane + 64 * r;
-        const uint32_t v = d < p.kdim ? (row[d >> 2] >> (8 * (d & 3))) & 255U : 0U;
+        const uint32_t d = lane + 64 * r;  // operand position: staged granule d / 16, byte d % 16
+        uint32_t v = 0;
+        if (p.nibbles) {
+            // Staged granule g holds the low (g even) or high (g odd) nibbles of code bytes 16 (g / 2) ...
+            const uint32_t g = d >> 4, b = 16 * (g >> 1) + (d & 15);
+            v = 2 * b + (g & 1) < p.kdim ? (row[2 * (b >> 2) + (g & 1)] >> (8 * (b & 3))) & 255U : 0U;
+        } else {
+            v = d < p.kdim ? (row[d >> 2] >> (8 * (d & 3))) & 255U : 0U;
+        }
         const uint32_t h = v >> 7;
         out[d] = static_cast<uint8_t>(h);
         out[128 + d] = static_cast<uint8_t>(v - 256U * h);  // the low byte of the two's complement of v - 256 h
@@ -235,9 +243,11 @@ quantize_uniform_i8_kernel(UniformQuantizeArgs p) {
     constexpr double kU = 5.9604644775390625e-8;  // 2^-24
     const double bd = static_cast<double>(ordered_to_float(bbits));
     const double qm = static_cast<double>(p.qmeta[q * p.qmeta_stride]);
-    const double ip_max = 255.0 * sum;                 // <code, query> of any code
+    const double cmax = p.nibbles ? 15.0 : 255.0;      // largest code value
+    const double shift = p.nibbles ? 0.0 : 128.0;      // the codes are staged as c - shift
+    const double ip_max = cmax * sum;                  // <code, query> of any code
     const double t_max = 128.0 * 256.0 * p.kdim;       // |T| of any code
-    const double m_max = p.is_l2 ? 255.0 * 255.0 * p.kdim : 255.0 * p.kdim;  // norm_o, sum_o of any code
+    const double m_max = p.is_l2 ? cmax * cmax * p.kdim : cmax * p.kdim;  // norm_o, sum_o of any code
     double t;
     if (p.is_l2) {
         // Streaming: fl(fl(fl(qm + m) - 2 R) rate), R the integer as a float (exact below 2^24).  The two sums round
@@ -248,8 +258,8 @@ quantize_uniform_i8_kernel(UniformQuantizeArgs p) {
         }
         const double reach = fabs(qm) + m_max + 2.0 * ip_max;
         const double x_max = bd / rate * (1.0 + 4.0 * kU) + 4.0 * kU * reach;  // what qm + m - 2 ip may reach
-        // qm + m - 2 (T + 128 sum) <= x_max   <=>   m - 2 T <= x_max - qm + 256 sum
-        t = x_max - qm + 256.0 * sum;
+        // qm + m - 2 (T + shift sum) <= x_max   <=>   m - 2 T <= x_max - qm + 2 shift sum
+        t = x_max - qm + 2.0 * shift * sum;
         // The test itself: fl(m - 2 T) in one fma against the rounded threshold.
         t += 4.0 * kU * (m_max + 2.0 * t_max + fabs(t));
     } else {
@@ -257,8 +267,9 @@ quantize_uniform_i8_kernel(UniformQuantizeArgs p) {
         const double lb = fabs(static_cast<double>(p.lb)), lb2 = fabs(static_cast<double>(p.lb2));
         const double reach = lb * (fabs(qm) + m_max) + rate * ip_max + lb2 + 1.0 + fabs(bd);
         const double e_stream = 8.0 * kU * reach;
-        // 1 - lb (qm + m) - rate (T + 128 sum) - lb2 <= bd + e   <=>   -rate T - lb m <= bd + e - 1 + lb qm + 128 rate sum + lb2
-        t = bd + e_stream - 1.0 + static_cast<double>(p.lb) * qm + 128.0 * rate * sum + static_cast<double>(p.lb2);
+        // 1 - lb (qm + m) - rate (T + shift sum) - lb2 <= bd + e
+        //     <=>   -rate T - lb m <= bd + e - 1 + lb qm + shift rate sum + lb2
+        t = bd + e_stream - 1.0 + static_cast<double>(p.lb) * qm + shift * rate * sum + static_cast<double>(p.lb2);
         // term_o = fl(-lb m) and the fma of the test.
         t += 4.0 * kU * (2.0 * lb * m_max + rate * t_max + fabs(t));
     }
@@ -308,7 +319,9 @@ i8_verdicts(const intx16& hi, const intx16& lo, const float (&tm)[16], float uq,
     return any;
 }
 
-template <int METRIC>
+// NIBBLE: the codes hold two 4-bit values per byte (sq4_uniform, at most four granules per code): a granule is staged
+// as two, its low nibbles and its high nibbles, as they are (0..15 needs no shift to fit a signed byte).
+template <int METRIC, bool NIBBLE = false>
 __global__ void __launch_bounds__(256, 2)
 prefilter_i8_kernel(PrefilterI8Args p) {
     __shared__ I8Stage stage[2];
@@ -355,10 +368,11 @@ prefilter_i8_kernel(PrefilterI8Args p) {
             const uint64_t tile = p.tile_begin + sg * kI8StageTiles + tt;
             const bool real = tile < p.tile_end;
 #pragma unroll
-            for (int r = 0; r < 2; ++r) {
+            for (int r = 0; r < (NIBBLE ? 1 : 2); ++r) {
                 const uint32_t j = wave + 4 * r;
                 // Raw bytes; they turn into c - 128 when parked, so that nothing waits for the load here.
-                regs[tt][r] = make_uint4(0x80808080U, 0x80808080U, 0x80808080U, 0x80808080U);
+                const uint32_t none = NIBBLE ? 0U : 0x80808080U;
+                regs[tt][r] = make_uint4(none, none, none, none);
                 if (real && j < p.G) {
                     regs[tt][r] = p.tiles[(tile * p.G + j) * kWave + lane];
                 }
@@ -375,11 +389,19 @@ prefilter_i8_kernel(PrefilterI8Args p) {
     auto park = [&](I8Stage& st) {
 #pragma unroll
         for (int tt = 0; tt < kI8StageTiles; ++tt) {
+            if constexpr (NIBBLE) {
+                const uint4 v = regs[tt][0];
+                const uint32_t m = 0x0F0F0F0FU;
+                st.codes[tt][(2 * wave) * kWave + lane] = make_uint4(v.x & m, v.y & m, v.z & m, v.w & m);
+                st.codes[tt][(2 * wave + 1) * kWave + lane] =
+                    make_uint4((v.x >> 4) & m, (v.y >> 4) & m, (v.z >> 4) & m, (v.w >> 4) & m);
+            } else {
 #pragma unroll
-            for (int r = 0; r < 2; ++r) {
-                const uint4 v = regs[tt][r];
-                st.codes[tt][(wave + 4 * r) * kWave + lane] =
-                    make_uint4(v.x ^ 0x80808080U, v.y ^ 0x80808080U, v.z ^ 0x80808080U, v.w ^ 0x80808080U);
+                for (int r = 0; r < 2; ++r) {
+                    const uint4 v = regs[tt][r];
+                    st.codes[tt][(wave + 4 * r) * kWave + lane] =
+                        make_uint4(v.x ^ 0x80808080U, v.y ^ 0x80808080U, v.z ^ 0x80808080U, v.w ^ 0x80808080U);
+                }
             }
             if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
                 if (wave == 0) {
@@ -516,6 +538,9 @@ prefilter_i8_kernel(PrefilterI8Args p) {
 
 bool
 prefilter_i8_supports(const vsag_amd_store* s) {
+    if (s->kind == VSAG_AMD_KIND_SQ4_UNIFORM) {
+        return s->nlist == 0 && s->pf_term != nullptr && s->dpad <= kI8Dims && s->G <= 4;
+    }
     return (s->kind == VSAG_AMD_KIND_SQ8 || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) && s->nlist == 0 && s->pf_term != nullptr &&
            s->dpad <= kI8Dims && s->G <= 8;
 }
@@ -543,7 +568,8 @@ launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride
                     uint32_t qmeta_stride, uint64_t nq, uint64_t tile_begin, uint64_t tile_end, const uint32_t* bound,
                     uint8_t* q8, float* u, uint32_t* tau, uint32_t* cand, uint32_t* cand_cnt, uint32_t sub_lists,
                     uint32_t sub_cap, hipStream_t st) {
-    const bool uniform = s->kind == VSAG_AMD_KIND_SQ8_UNIFORM;
+    const bool nibbles = s->kind == VSAG_AMD_KIND_SQ4_UNIFORM;
+    const bool uniform = s->kind == VSAG_AMD_KIND_SQ8_UNIFORM || nibbles;
     // The uniform kinds use the l2 form of the test (fma of the integer and a per-code term) for every metric.
     const bool l2 = s->metric == VSAG_AMD_METRIC_L2 || uniform;
     const uint64_t nq_pad = div_up(nq, static_cast<uint64_t>(kI8Group)) * kI8Group;
@@ -555,6 +581,7 @@ launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride
         z.qmeta = qmeta;
         z.qmeta_stride = qmeta_stride;
         z.is_l2 = s->metric == VSAG_AMD_METRIC_L2 ? 1 : 0;
+        z.nibbles = nibbles ? 1 : 0;
         z.lb = s->ulb;
         z.rate = s->scalar_rate;
         z.lb2 = s->ulb * s->ulb;
@@ -604,7 +631,9 @@ launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride
     VA_CHECK_ARG(sub_lists == prefilter_i8_sub_lists(nq, tile_end - tile_begin), "candidate lists do not match the grid");
     dim3 grid(p.groups, static_cast<uint32_t>(nq_pad / kI8Group));
     timing_begin(st);
-    if (l2) {
+    if (nibbles) {
+        hipLaunchKernelGGL((prefilter_i8_kernel<VSAG_AMD_METRIC_L2, true>), grid, dim3(256), 0, st, p);
+    } else if (l2) {
         hipLaunchKernelGGL(prefilter_i8_kernel<VSAG_AMD_METRIC_L2>, grid, dim3(256), 0, st, p);
     } else {
         hipLaunchKernelGGL(prefilter_i8_kernel<VSAG_AMD_METRIC_IP>, grid, dim3(256), 0, st, p);

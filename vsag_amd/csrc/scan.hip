@@ -713,8 +713,9 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
         return;
     }
     c->contraction = true;
-    // Mode 2 asks for the fp32 matrix cores, which sq8_uniform stores have no route for.
-    c->int8 = prefilter_i8_supports(s) && (g_prefilter_mode != 2 || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM);
+    // Mode 2 asks for the fp32 matrix cores, which the uniform kinds have no route for.
+    c->int8 = prefilter_i8_supports(s) && (g_prefilter_mode != 2 || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM ||
+                                           s->kind == VSAG_AMD_KIND_SQ4_UNIFORM);
     c->rb = rb;
     c->rb_scratch = rb ? prefilter_rb_scratch_bytes(s, nq) : 0;
     c->prefix_tiles = prefix;

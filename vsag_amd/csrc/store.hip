@@ -378,7 +378,7 @@ vsag_amd_store_create(const vsag_amd_store_params_t* p, vsag_amd_store_t** out) 
     }
     // Stores the matrix cores can pre-select on keep a per-code term (and the largest norm, where a threshold needs it).
     if (p->kind == VSAG_AMD_KIND_FP32 || p->kind == VSAG_AMD_KIND_SQ8 ||
-        (p->kind == VSAG_AMD_KIND_SQ8_UNIFORM && s->dpad <= 128)) {
+        ((p->kind == VSAG_AMD_KIND_SQ8_UNIFORM || p->kind == VSAG_AMD_KIND_SQ4_UNIFORM) && s->dpad <= 128)) {
         if (hipMalloc(&s->pf_ymax, 4) != hipSuccess || hipMemset(s->pf_ymax, 0, 4) != hipSuccess) {
             return fail_free(fail(VSAG_AMD_NO_ENOUGH_MEMORY, "hipMalloc of the norm scalar failed"));
         }
