@@ -444,9 +444,13 @@ struct UpdateBuffers {
 static size_t
 sort_temp_bytes(uint64_t n) {
     size_t bytes = 0;
-    hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, static_cast<const int32_t*>(nullptr),
-                                       static_cast<int32_t*>(nullptr), static_cast<const uint32_t*>(nullptr),
-                                       static_cast<uint32_t*>(nullptr), static_cast<int>(n), 0, 32, nullptr);
+    // A size query only; a failure leaves 0 and the sort that follows reports it.
+    if (hipcub::DeviceRadixSort::SortPairs(nullptr, bytes, static_cast<const int32_t*>(nullptr),
+                                           static_cast<int32_t*>(nullptr), static_cast<const uint32_t*>(nullptr),
+                                           static_cast<uint32_t*>(nullptr), static_cast<int>(n), 0, 32,
+                                           nullptr) != hipSuccess) {
+        bytes = 0;
+    }
     return bytes;
 }
 
