@@ -462,15 +462,15 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
         rescore(r.cand + static_cast<uint64_t>(q) * r.cap, as_const(counts)[0]);
     } else {
         // Gather the private lists of the query behind the selector -- a lane per list, offsets by a wave scan -- and
-        // rescore whenever the next round of lists might not fit (usually once, at the end: full waves of candidates).
+        // rescore whenever the next lists might not fit (usually once, at the end: full waves of candidates).  64 lists
+        // go in one round when what they hold fits; a round of fuller lists goes in pieces that fit even when full.
         uint32_t* flat = reinterpret_cast<uint32_t*>(keys + r.S);
         const uint32_t* lists = r.cand + static_cast<uint64_t>(q) * r.sub_lists * r.sub_cap;
-        uint32_t batch = r.gather / r.sub_cap;
-        batch = batch > kWave ? kWave : (batch == 0 ? 1 : batch);
+        uint32_t piece = r.gather / r.sub_cap;
+        piece = piece > kWave ? kWave : (piece == 0 ? 1 : piece);
         uint32_t fill = 0;
-        for (uint32_t g0 = 0; g0 < r.sub_lists; g0 += batch) {
-            const uint32_t g = g0 + lane;
-            const uint32_t c = lane < batch && g < r.sub_lists ? as_const(counts)[g] : 0U;
+        auto gather = [&](uint32_t g, uint32_t c) {
+            // c = this lane's share (0: none); returns after the lanes' entries are in flat[fill ...].
             uint32_t incl = c;
             for (int off = 1; off < 64; off <<= 1) {
                 uint32_t o = __shfl_up(incl, off);
@@ -478,7 +478,7 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
             }
             const uint32_t sum = __shfl(incl, 63);
             if (sum == 0) {
-                continue;
+                return;
             }
             if (fill + sum > r.gather) {
                 wave_lds_fence();
@@ -487,10 +487,37 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
                 wave_lds_fence();  // what was gathered has been read
             }
             const uint32_t at = fill + incl - c;
-            for (uint32_t i = 0; i < c; ++i) {
-                flat[at + i] = as_const(lists)[static_cast<uint64_t>(g) * r.sub_cap + i];
+            const uint32_t* mine = lists + static_cast<uint64_t>(g) * r.sub_cap;
+            // Four loads in flight per lane.
+            for (uint32_t i = 0; i < c; i += 4) {
+                uint32_t v[4];
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j) {
+                    v[j] = i + j < c ? as_const(mine)[i + j] : 0U;
+                }
+#pragma unroll
+                for (uint32_t j = 0; j < 4; ++j) {
+                    if (i + j < c) {
+                        flat[at + i + j] = v[j];
+                    }
+                }
             }
             fill += sum;
+        };
+        for (uint32_t g0 = 0; g0 < r.sub_lists; g0 += kWave) {
+            const uint32_t g = g0 + lane;
+            const uint32_t c = g < r.sub_lists ? as_const(counts)[g] : 0U;
+            uint32_t total = c;
+            for (int off = 32; off > 0; off >>= 1) {
+                total += __shfl_xor(total, off);
+            }
+            if (total <= r.gather) {
+                gather(g, c);
+            } else {
+                for (uint32_t b0 = 0; b0 < kWave; b0 += piece) {
+                    gather(g, lane >= b0 && lane < b0 + piece ? c : 0U);
+                }
+            }
         }
         wave_lds_fence();
         rescore(flat, fill);
