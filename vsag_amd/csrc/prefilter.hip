@@ -381,6 +381,7 @@ struct RescoreArgs {
     // sub_lists != 0: the candidates of a query sit in sub_lists lists of sub_cap (<= gather) slots with a count each
     // (a count above sub_cap = that list overflowed); they are gathered into `gather` words of LDS.
     uint32_t sub_lists, sub_cap, gather;
+    const uint4* rows;  // the codes a row per code (store.h), or null: read the tiles
 };
 
 // Words of LDS for gathered candidates: small, so that many of these one-wave workgroups share a compute unit (the
@@ -433,8 +434,9 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
             const uint32_t ln = slot & 63;
             Acc<KIND, 1> acc;
             acc_reset(acc);
+            const uint4* row = r.rows != nullptr ? r.rows + static_cast<uint64_t>(slot) * a.G : nullptr;
             for (uint32_t j = 0; j < a.G; ++j) {
-                uint4 c = a.tiles[(tile * a.G + j) * kWave + ln];
+                const uint4 c = row != nullptr ? row[j] : a.tiles[(tile * a.G + j) * kWave + ln];
                 accumulate_granule<KIND, METRIC, 1>(a, qrows, j, c, acc);
             }
             float d[1];
@@ -630,6 +632,7 @@ launch_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t
     r.sub_lists = sub_lists;
     r.sub_cap = sub_cap;
     r.gather = std::max(kRescoreGather, sub_cap);
+    r.rows = s->rows;
     dim3 rgrid(static_cast<uint32_t>(nq));
     const size_t lds = S * 8 + (sub_lists != 0 ? r.gather * 4 : 0);
     if (s->kind == VSAG_AMD_KIND_SQ8) {

@@ -53,6 +53,9 @@ struct vsag_amd_store {
 
     // flat fp32 / sq8 stores: per slot |y|^2 and the largest |y| (float bits) of the code as the batched
     // contraction sees it, kept up to date by append
+    // Flat stores the matrix cores pre-select on: the codes once more, a row per code (G granules in a run), for the
+    // rescoring of scattered candidates -- one or two memory lines per candidate instead of one per granule.
+    uint4* rows = nullptr;
     float* pf_term = nullptr;
     uint32_t* pf_ymax = nullptr;
 };

@@ -147,6 +147,26 @@ list_slot_kernel(const int32_t* sorted_labels, uint64_t n, const uint32_t* list_
     }
 }
 
+// Stores whose large batches are pre-selected on the matrix cores and rescored (prefilter.hip).
+static bool
+keeps_rows(const vsag_amd_store* s) {
+    // Not fp32 stores: the copy would double the largest of all stores for the smallest gain.
+    return (s->pf_ymax != nullptr && s->kind != VSAG_AMD_KIND_FP32) ||
+           (s->kind == VSAG_AMD_KIND_RABITQ && s->query_bits == 4);
+}
+
+// rows[slot][j] = granule j of the code in `slot`, from the tiles.
+__global__ void __launch_bounds__(256)
+rows_from_tiles_kernel(const uint4* tiles, uint32_t G, uint64_t first_slot, uint64_t count, uint4* rows) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= count * G) {
+        return;
+    }
+    const uint64_t slot = first_slot + i / G;
+    const uint32_t j = static_cast<uint32_t>(i % G);
+    rows[slot * G + j] = tiles[((slot / kWave) * G + j) * kWave + slot % kWave];
+}
+
 static int
 grow(vsag_amd_store* s, uint64_t need_tiles, hipStream_t st) {
     if (need_tiles <= s->cap_tiles) {
@@ -179,6 +199,13 @@ grow(vsag_amd_store* s, uint64_t need_tiles, hipStream_t st) {
             VA_HIP(hipMemcpyAsync(term, s->pf_term, s->ntiles * kWave * sizeof(float), hipMemcpyDeviceToDevice, st));
         }
     }
+    uint4* rows = nullptr;
+    if (keeps_rows(s)) {
+        VA_HIP(hipMalloc(&rows, cap * kWave * s->G * sizeof(uint4)));
+        if (s->ntiles > 0) {
+            VA_HIP(hipMemcpyAsync(rows, s->rows, s->ntiles * kWave * s->G * sizeof(uint4), hipMemcpyDeviceToDevice, st));
+        }
+    }
     VA_HIP(hipStreamSynchronize(st));
     if (s->tiles) {
         VA_HIP(hipFree(s->tiles));
@@ -189,6 +216,10 @@ grow(vsag_amd_store* s, uint64_t need_tiles, hipStream_t st) {
     if (s->pf_term) {
         VA_HIP(hipFree(s->pf_term));
     }
+    if (s->rows) {
+        VA_HIP(hipFree(s->rows));
+    }
+    s->rows = rows;
     s->tiles = tiles;
     s->meta = meta;
     s->pf_term = term;
@@ -394,7 +425,8 @@ vsag_amd_store_destroy(vsag_amd_store_t* s) {
         return 0;
     }
     void* ptrs[] = {s->scale_dev, s->lb_dev,  s->diff_dev, s->bounds_dev,    s->rotation_dev, s->centroid_dev,
-                    s->tiles,     s->meta,    s->ids_dev,  s->list_tile_dev, s->pf_term,      s->pf_ymax};
+                    s->tiles,     s->meta,    s->ids_dev,  s->list_tile_dev, s->pf_term,      s->pf_ymax,
+                    s->rows};
     for (void* p : ptrs) {
         if (p != nullptr) {
             (void)hipFree(p);
@@ -427,6 +459,11 @@ vsag_amd_store_append(vsag_amd_store_t* s, const uint8_t* codes_dev, uint64_t n,
     uint64_t threads = n * s->G;
     hipLaunchKernelGGL(retile_kernel, dim3(static_cast<uint32_t>(div_up(threads, 256))), dim3(256), 0, st, a);
     VA_HIP(hipGetLastError());
+    if (s->rows != nullptr) {
+        hipLaunchKernelGGL(rows_from_tiles_kernel, dim3(static_cast<uint32_t>(div_up(threads, 256))), dim3(256), 0, st,
+                           s->tiles, s->G, s->n, n, s->rows);
+        VA_HIP(hipGetLastError());
+    }
     VA_TRY(launch_code_terms(s, s->n, n, st));
     s->n += n;
     s->ntiles = need;
