@@ -435,9 +435,22 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
             Acc<KIND, 1> acc;
             acc_reset(acc);
             const uint4* row = r.rows != nullptr ? r.rows + static_cast<uint64_t>(slot) * a.G : nullptr;
-            for (uint32_t j = 0; j < a.G; ++j) {
-                const uint4 c = row != nullptr ? row[j] : a.tiles[(tile * a.G + j) * kWave + ln];
-                accumulate_granule<KIND, METRIC, 1>(a, qrows, j, c, acc);
+            // A few granules are fetched before the first is used: a candidate's loads wait for memory together.
+            // (sq8 l2 holds scale and query of every dimension in flight in scalar registers: two granules' worth.)
+            constexpr uint32_t kAhead = KIND == VSAG_AMD_KIND_SQ8 && METRIC == VSAG_AMD_METRIC_L2 ? 2 : 4;
+            for (uint32_t j0 = 0; j0 < a.G; j0 += kAhead) {
+                uint4 c[kAhead];
+#pragma unroll
+                for (uint32_t u = 0; u < kAhead; ++u) {
+                    const uint32_t j = j0 + u < a.G ? j0 + u : a.G - 1;
+                    c[u] = row != nullptr ? row[j] : a.tiles[(tile * a.G + j) * kWave + ln];
+                }
+#pragma unroll
+                for (uint32_t u = 0; u < kAhead; ++u) {
+                    if (j0 + u < a.G) {
+                        accumulate_granule<KIND, METRIC, 1>(a, qrows, j0 + u, c[u], acc);
+                    }
+                }
             }
             float d[1];
             finish_distances<KIND, METRIC, 1>(a, qidx, slot, acc, d);
