@@ -504,11 +504,84 @@ merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, cons
     }
 }
 
+// The same for a handful of short lists (the levels of a pre-selected batch with a small k): one wave per query, the
+// admitted keys sorted in LDS.  Every list holds at most k keys, so nslots * k keys of room never overflow.
+constexpr uint32_t kSmallMergeKeys = 512;
+
+__global__ void __launch_bounds__(64)
+merge_small_kernel(const uint64_t* partial, const uint32_t* partial_cnt, const uint32_t* bound, uint32_t nslots,
+                   uint32_t stride, uint32_t k, uint32_t* ids, float* dists) {
+    __shared__ uint64_t pool[kSmallMergeKeys];
+    const uint32_t lane = threadIdx.x;
+    const uint64_t q = blockIdx.x;
+    const uint32_t* cnts = partial_cnt + q * stride;
+    const uint64_t* src = partial + q * stride * k;
+    const uint64_t admit = (static_cast<uint64_t>(as_const(bound)[q]) << 32) | 0xFFFFFFFFULL;
+    const uint32_t mine = lane < nslots ? cnts[lane] : 0U;  // nslots <= 64
+    uint32_t fill = 0;
+    uint64_t lists = __ballot(mine != 0);
+    while (lists != 0) {
+        const uint32_t slot = static_cast<uint32_t>(__builtin_ctzll(lists));
+        lists &= lists - 1;
+        const uint32_t c = __shfl(mine, static_cast<int>(slot));
+        const uint64_t* list = src + static_cast<uint64_t>(slot) * k;
+        for (uint32_t i0 = 0; i0 < c; i0 += kWave) {
+            const uint32_t i = i0 + lane;
+            const uint64_t key = i < c ? list[i] : kInfKey;
+            const bool keep = i < c && key <= admit;
+            const uint64_t votes = __ballot(keep);
+            if (keep) {
+                pool[fill + static_cast<uint32_t>(__popcll(votes & ((1ULL << lane) - 1)))] = key;
+            }
+            fill += static_cast<uint32_t>(__popcll(votes));
+        }
+    }
+    uint32_t P = 2;
+    while (P < fill || P < k) {
+        P <<= 1;
+    }
+    P = P > kSmallMergeKeys ? kSmallMergeKeys : P;  // k <= nslots * k <= kSmallMergeKeys, a power of two
+    for (uint32_t i = fill + lane; i < P; i += kWave) {
+        pool[i] = kInfKey;
+    }
+    wave_lds_fence();
+    for (uint32_t size = 2; size <= P; size <<= 1) {
+        for (uint32_t step = size >> 1; step > 0; step >>= 1) {
+            for (uint32_t t = lane; t < P / 2; t += kWave) {
+                const uint32_t pos = 2 * t - (t & (step - 1));
+                const uint64_t x = pool[pos], y = pool[pos + step];
+                const bool up = (pos & size) == 0;
+                if ((x > y) == up) {
+                    pool[pos] = y;
+                    pool[pos + step] = x;
+                }
+            }
+            wave_lds_fence();
+        }
+    }
+    for (uint32_t i = lane; i < k; i += kWave) {
+        const uint64_t key = pool[i];
+        if (key == kInfKey) {
+            ids[q * k + i] = VSAG_AMD_INVALID_ID;
+            dists[q * k + i] = __builtin_inff();
+        } else {
+            ids[q * k + i] = static_cast<uint32_t>(key);
+            dists[q * k + i] = ordered_to_float(static_cast<uint32_t>(key >> 32));
+        }
+    }
+}
+
 // ------------------------------------------------------------------ host side
 int
 launch_merge_partials(const uint64_t* partial, const uint32_t* partial_cnt, const uint32_t* bound, uint32_t nslots,
                       uint32_t stride, uint32_t k, uint32_t S, uint64_t nq, uint32_t* ids, float* dists,
                       hipStream_t st) {
+    if (nslots <= kWave && static_cast<uint64_t>(nslots) * k <= kSmallMergeKeys && nq > 256) {
+        hipLaunchKernelGGL(merge_small_kernel, dim3(static_cast<uint32_t>(nq)), dim3(kWave), 0, st, partial, partial_cnt,
+                           bound, nslots, stride, k, ids, dists);
+        VA_HIP(hipGetLastError());
+        return 0;
+    }
     // Few queries: many candidates each (every wave starts without a bound), so give each merge more threads.
     const uint32_t threads = nq <= 256 ? 1024 : 256;
     const uint32_t pool_keys = nq <= 256 ? kPoolKeys : kPoolKeysBatch;
