@@ -409,6 +409,10 @@ merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, cons
     const uint32_t* cnts = partial_cnt + q * stride;  // the first nslots of the query's `stride` lists
     const uint64_t* src = partial + q * stride * k;
     uint64_t admit = (static_cast<uint64_t>(as_const(bound)[q]) << 32) | 0xFFFFFFFFULL;
+    uint32_t sort_room = 2;  // keys the closing sort takes: the power of two from k on
+    while (sort_room < k) {
+        sort_room <<= 1;
+    }
     // Finitely many rounds: every round that overflows lowers `admit` below at least one pooled key.
     for (;;) {
         if (threadIdx.x == 0) {
@@ -468,6 +472,17 @@ merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, cons
         __syncthreads();
         const uint32_t total = npool;
         const uint32_t n = total < pool_keys ? total : pool_keys;
+        if (total <= sort_room) {
+            // The usual case once the bound is tight: hardly more than k keys are admitted, and the sort that follows
+            // orders them all without a selection first.
+            for (uint32_t i = threadIdx.x; i < total; i += blockDim.x) {
+                lds[i] = pool[i];
+            }
+            if (threadIdx.x == 0) {
+                nout = total;
+            }
+            break;
+        }
         const uint64_t kth = block_kth_smallest(pool, n, k, scratch);
         if (total <= pool_keys) {
             // The k smallest (all of them when fewer than k) go to the front of the output area.
