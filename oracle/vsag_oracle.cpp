@@ -13,11 +13,16 @@
 //                                          rabitq 4-bit query planes, rabitq_binary_ip 0/36/32
 //   pinned by compiled reference kernels . fp32/sq8/sq4 distances, sq4u/sq8u code IP, binary IPs,
 //                                          normalize-with-centroid
-//   pinned by closed form / brute force .. sq_train (sorted order statistics), kmeans_assign (fp64
-//                                          argmin), heaps (sort), ivf composition (nprobe=nlist)
-//   parity unpinned ...................... rabitq_dist op order and kmeans inertia are fixed only by
-//                                          their formulas (no executable reference, no golden value
-//                                          in the reference tests); tolerance 1e-4 relative covers it
+//   pinned by closed form / brute force .. sq_train (sorted order statistics), kmeans_assign and its
+//                                          loss (fp64 argmin and mean of the minima), heaps (sort), ivf
+//                                          composition (nprobe=nlist), rabitq_dist (a stored vector as
+//                                          32-bit query: estimate exactly 0 / 1 - |x|^2; the +-1 clamp of
+//                                          a tiny error field; zero raw norms -> 1; the 4-bit branch
+//                                          against the fp32 branch on the dequantised query)
+//   parity unpinned ...................... nothing; what the formulas leave open is the order of fp32
+//                                          operations inside rabitq_dist and the k-means loss (no
+//                                          executable reference class), which the 1e-4 relative
+//                                          tolerance of the comparisons covers
 #include <algorithm>
 #include <cfloat>
 #include <cmath>

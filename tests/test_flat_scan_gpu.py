@@ -117,3 +117,46 @@ def test_empty_store_and_bad_arguments(lib):
     assert rc == lib.INVALID_ARGUMENT
     assert b"k must be" in lib.load_library().vsag_amd_last_error()
     st.destroy()
+
+
+def _unit_rows(a):
+    """Rows divided by their norm; a zero row divides by 1 (DivScalarImpl, simd/kernels/scalar_op.h:40-42)."""
+    norm = np.sqrt((a.astype(np.float64) ** 2).sum(1, keepdims=True)).astype(np.float32)
+    norm[norm == 0] = 1.0
+    return (a / norm).astype(np.float32)
+
+
+@pytest.mark.parametrize("kind", ["fp32", "sq8"])
+@pytest.mark.parametrize("contraction", [0, 1])
+def test_cosine_with_zero_rows_and_a_zero_query(lib, kind, contraction):
+    """A zero base row and a zero query under cosine: the reference divides by 1 instead of by the zero norm, so the
+    distance is 1 - 0 = 1 and nothing turns into NaN; the other queries' results do not change."""
+    rng = np.random.default_rng(91)
+    n, d, nq, k = 70000 if contraction else 3000, 64, 6, 10
+    x = (rng.random((n, d), dtype=np.float32) - 0.3).astype(np.float32)
+    x[17] = 0.0
+    x[n - 5] = 0.0
+    q = (rng.random((nq, d), dtype=np.float32) - 0.3).astype(np.float32)
+    q[2] = 0.0
+    l = lib.load_library()
+    if kind == "fp32":
+        st = Store(lib.KIND_FP32, orc.COSINE, d)
+        st.append(x.view(np.uint8).reshape(n, 4 * d))
+        ref = lambda qq: orc.flat_scan_topk(orc.FP32, orc.IP, d, _unit_rows(x).view(np.uint8).reshape(n, 4 * d), qq, k)
+    else:
+        lb, diff = orc.sq_train(x, 8, orc.COSINE)
+        codes = orc.sq_encode(x, 8, lb, diff, orc.COSINE)
+        st = Store(lib.KIND_SQ8, orc.COSINE, d, lb=lb, diff=diff)
+        st.append(codes)
+        ref = lambda qq: orc.flat_scan_topk(orc.SQ8, orc.IP, d, codes, qq, k, lb=lb, diff=diff)
+    lib.check(l.vsag_amd_set_scan_contraction(contraction))
+    try:
+        ids, ds = st.flat_scan(q, k)
+    finally:
+        lib.check(l.vsag_amd_set_scan_contraction(0))
+    assert not np.isnan(ds).any(), "a zero norm must not produce NaN distances"
+    rids, rds = ref(_unit_rows(q))
+    assert_topk_close(ids, ds, rids, rds, atol=2e-6, label="%s cosine with zero rows" % kind)
+    if kind == "fp32":
+        assert np.all(ds[2] == 1.0), "a zero query is at distance 1 from everything"
+    st.destroy()

@@ -363,6 +363,127 @@ def test_rabitq_encode_invariants_and_estimator():
     assert np.corrcoef(d4.ravel(), true.ravel())[0, 1] > 0.7
 
 
+def _rabitq_dist(qcode, code, d, metric, qbits):
+    L = orc.lib()
+    return float(L.orc_rabitq_dist(_p(np.ascontiguousarray(qcode)), _p(np.ascontiguousarray(code)), C.c_uint64(d), metric,
+                                   qbits))
+
+
+def _rabitq_case(seed, d, n, metric, unit):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    if unit:
+        x /= np.linalg.norm(x, axis=1, keepdims=True)
+    rot = _rotation(rng, d)
+    cen = orc.rabitq_train(x, rot)
+    return rng, x, rot, cen
+
+
+@pytest.mark.parametrize("d", [64, 128, 200, 768])
+def test_rabitq_estimator_self_distance_is_exact(d):
+    """A 32-bit query equal to a stored vector: <o, o_bar> of the query IS the code's error field (the same
+    RaBitQFloatBinaryIP over the same normalised vector), so ip_est = error / error = 1 and the estimate collapses to
+    (|o| - |q|)^2 = 0 exactly, the inner-product distance to 1 - |x|^2 and cosine to 0.  Dropping the division by the
+    error, dividing by the norm instead, or a wrong sign in l2_ube all leave 2 n^2 (1 - error) or worse here.  The
+    reference tests self-distances the same way (rabitq_quantizer_test.cpp:72-103)."""
+    rng, x, rot, cen = _rabitq_case(60 + d, d, 50, orc.L2, unit=False)
+    for metric in (orc.L2, orc.IP, orc.COSINE):
+        codes = orc.rabitq_encode(x, rot, cen, metric, qbits=32)
+        qcodes = orc.rabitq_process_query(x, rot, cen, metric, 32)
+        nb = (d + 7) // 8
+        nb4 = (nb + 3) // 4 * 4
+        for i in range(x.shape[0]):
+            f = codes[i, nb4:].view(np.float32)  # norm, error, (raw norm)
+            assert 0.5 < f[1] < 1.0  # the error factor is far from 1, so a dropped division would show
+            got = _rabitq_dist(qcodes[i], codes[i], d, metric, 32)
+            if metric == orc.L2:
+                assert got == 0.0
+            elif metric == orc.IP:
+                r = np.float32(f[2])
+                assert got == float(np.float32(1) - (r * r + r * r - np.float32(0)) * np.float32(0.5))
+                assert abs(got - (1.0 - float((x[i].astype(np.float64) ** 2).sum()))) < 1e-4 * d
+            else:
+                assert abs(got) < 1e-6
+
+
+def test_rabitq_estimator_error_clamp_and_zero_norms():
+    """|error| < 1e-5 is replaced by +1 / -1 by its sign (rabitq_quantizer.cpp:1824-1827); a raw norm below 1e-5 on
+    either side makes the inner-product and cosine distance 1 (:1838-1857)."""
+    d = 128
+    rng, x, rot, cen = _rabitq_case(71, d, 8, orc.IP, unit=True)
+    nb = d // 8
+    L = orc.lib()
+    q = rng.standard_normal((1, d)).astype(np.float32)
+    q32 = orc.rabitq_process_query(q, rot, cen, orc.L2, 32)[0]
+    codes = orc.rabitq_encode(x, rot, cen, orc.L2, qbits=32)
+    inv = C.c_float(1.0 / np.sqrt(np.float32(d)))
+    for i in range(4):
+        code = codes[i].copy()
+        f = code[nb:].view(np.float32)  # norm, error
+        ip_bq = np.float32(L.orc_rabitq_float_binary_ip(_p(q32), _p(code), C.c_uint64(d), inv))
+        n_o, n_q = np.float32(f[0]), q32[4 * d:].view(np.float32)[0]
+        for forced, divisor in ((1e-6, 1.0), (-1e-6, -1.0), (0.0, 1.0), (9.9e-6, 1.0), (-9.9e-6, -1.0), (2e-5, 2e-5),
+                                (-2e-5, -2e-5)):
+            f[1] = forced
+            est = np.float32(ip_bq / np.float32(divisor))
+            expect = n_o * n_o + n_q * n_q + np.float32(-2) * n_o * n_q * est
+            got = _rabitq_dist(q32, code, d, orc.L2, 32)
+            assert got == float(expect), (forced, got, float(expect))
+    # zero raw norms
+    for metric in (orc.IP, orc.COSINE):
+        for qbits in (4, 32):
+            codes = orc.rabitq_encode(x, rot, cen, metric, qbits=qbits)
+            qc = orc.rabitq_process_query(q, rot, cen, metric, qbits)[0]
+            normal = _rabitq_dist(qc, codes[0], d, metric, qbits)
+            assert normal != 1.0
+            code = codes[0].copy()
+            code[-4:].view(np.float32)[0] = 5e-6  # the base's raw norm is the last field
+            assert _rabitq_dist(qc, code, d, metric, qbits) == 1.0
+            qz = qc.copy()
+            qz[-4:].view(np.float32)[0] = 0.0  # and so is the query's
+            assert _rabitq_dist(qz, codes[0], d, metric, qbits) == 1.0
+            zero_q = orc.rabitq_process_query(np.zeros((1, d), np.float32), rot, cen, metric, qbits)[0]
+            assert _rabitq_dist(zero_q, codes[0], d, metric, qbits) == 1.0
+
+
+@pytest.mark.parametrize("d", [6, 15, 128, 200, 768])
+def test_rabitq_4bit_estimate_equals_the_fp32_form_on_the_dequantised_query(d):
+    """The 4-bit branch (rabitq_quantizer.cpp:924-939, equation 19-20 of the paper) is algebra on
+    <bits, lb + delta c> : feeding the dequantised query lb + delta c_d through the fp32 branch (RaBitQFloatBinaryIP,
+    pinned against the reference's own compiled kernel) must give the same distance up to fp32 rounding.  A dropped
+    or mis-signed term of the four (2 delta ip, 2 lb sum_b, delta sum_q, lb d) is off by far more."""
+    rng, x, rot, cen = _rabitq_case(80 + d, d, 40, orc.IP, unit=True)
+    q = rng.standard_normal((6, d)).astype(np.float32)
+    q /= np.linalg.norm(q, axis=1, keepdims=True)
+    nb = (d + 7) // 8
+    nb4 = (nb + 3) // 4 * 4
+    for metric in (orc.L2, orc.IP, orc.COSINE):
+        codes4 = orc.rabitq_encode(x, rot, cen, metric, qbits=4)
+        codes32 = orc.rabitq_encode(x, rot, cen, metric, qbits=32)
+        # the two base layouts hold the same bits, norm, error and raw norm
+        assert np.array_equal(codes4[:, :nb4 + 8], codes32[:, :nb4 + 8])
+        q4 = orc.rabitq_process_query(q, rot, cen, metric, 4)
+        q32 = orc.rabitq_process_query(q, rot, cen, metric, 32)
+        qs32 = q32.shape[1]
+        pb = (d + 511) // 512 * 512 // 8
+        for i in range(q.shape[0]):
+            planes = q4[i, :4 * pb].reshape(4, pb)
+            c = np.zeros(d, np.int64)
+            for b in range(4):
+                c += np.unpackbits(planes[b], bitorder="little")[:d].astype(np.int64) << b
+            tail = q4[i, 4 * pb:].view(np.float32)  # lb, delta, sum, norm, (raw norm)
+            lb, delta, qsum = tail[0], tail[1], tail[2]
+            assert qsum == np.float32(c.sum())
+            deq = np.zeros(qs32, np.uint8)
+            deq[:4 * d] = (np.float32(lb) + np.float32(delta) * c.astype(np.float32)).astype(np.float32).view(np.uint8)
+            deq[4 * d:] = q32[i, 4 * d:]  # same norm and raw norm fields
+            assert np.array_equal(tail[3:].view(np.uint8), q32[i, 4 * d:])
+            for j in range(x.shape[0]):
+                a = _rabitq_dist(q4[i], codes4[j], d, metric, 4)
+                b = _rabitq_dist(deq, codes32[j], d, metric, 32)
+                assert abs(a - b) <= 2e-5 * (1.0 + abs(b)), (metric, i, j, a, b)
+
+
 def test_kmeans_assign_is_the_exact_argmin():
     rng = np.random.default_rng(7)
     x = rng.standard_normal((800, 24)).astype(np.float32)

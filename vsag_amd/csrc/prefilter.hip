@@ -320,10 +320,13 @@ code_term_kernel(const uint4* tiles, uint32_t G, const float* scale, uint64_t fi
         }
         term[slot] = static_cast<float>(s);
     }
+    // A code with a NaN or infinite norm (fp32 stores hold whatever the caller gave) must not decide the maximum: it
+    // would hide the largest finite norm, which the thresholds of all the other codes are built on.  Such a code's own
+    // distances are NaN or infinite and order behind every finite one.
     float m = static_cast<float>(sqrt(s)) * (1.0F + 2.0e-7F);
+    m = m < __builtin_inff() ? m : 0.0F;
     for (int off = 32; off > 0; off >>= 1) {
-        float o = __shfl_xor(m, off);
-        m = o > m ? o : m;
+        m = fmaxf(m, __shfl_xor(m, off));
     }
     if ((threadIdx.x & 63) == 0 && m > 0.0F) {
         atomicMax(ymax_bits, __float_as_uint(m));

@@ -53,6 +53,9 @@ prepare_float_queries(const float* q, uint64_t nq, uint32_t dim, int kind, int m
         }
         s = block_sum(s, red);
         inv_norm = sqrtf(s);
+        if (inv_norm == 0.0F) {
+            inv_norm = 1.0F;  // DivScalarImpl (src/simd/kernels/scalar_op.h:40-42): a zero norm divides by 1
+        }
     }
     float bias = 0;
     for (uint32_t d = threadIdx.x; d < qstride; d += blockDim.x) {

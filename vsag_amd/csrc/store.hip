@@ -54,6 +54,9 @@ retile_kernel(RetileArgs a) {
             s = fmaf(x[d], x[d], s);
         }
         float norm = sqrtf(s);
+        if (norm == 0.0F) {
+            norm = 1.0F;  // DivScalarImpl (src/simd/kernels/scalar_op.h:40-42): a zero norm divides by 1
+        }
         for (uint32_t e = 0; e < 4; ++e) {
             uint32_t d = 4 * j + e;
             if (d < a.dim) {
