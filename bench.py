@@ -27,6 +27,8 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 HBM_PEAK_GBS = 8000.0
 MFMA_F32_PEAK_TFLOPS = 157.3
 MFMA_I8_PEAK_TOPS = 5000.0  # dense int8, published
+# HBM/fabric bytes of the last-level launch of prefilter_i8_kernel<l2> on configs[1] (profiles/prefilter_i8_sq8_c2.md)
+PROFILE_TRAFFIC_I8_C2 = 2422324.4 * 2.00 * 1024 + 68345.8 * 1024
 
 
 def mt(seed):
@@ -163,6 +165,10 @@ class Env:
     def base_line(self, metric, unit, value, sec_per_step, dtype, workload, extra, roofline, cpu):
         cfg = {"workload": workload, "device": self.dev_name, "compute_units": self.cus}
         cfg.update(extra)
+        if roofline is not None and "traffic_source" not in roofline:
+            roofline["traffic_source"] = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, from the committed "
+                                          "summary under profiles/; not measured in this run"
+                                          if roofline.get("traffic") is not None else None)
         return {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": self.args.steps,
                 "warmup": self.args.warmup, "ms_per_step": 1e3 * sec_per_step, "higher_is_better": True,
                 "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic", "config": cfg,
@@ -220,6 +226,37 @@ def run_c2(env):
                   "hbm_frac": bpp / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS}
         ws.free()
 
+    # The same search through the index API with host buffers on both sides, as a user of the reference calls it
+    # (tools/eval/case/search_eval_case.cpp:233-277): Factory::CreateIndex("brute_force") -> Build -> KnnSearch.
+    # A step uploads the queries, runs the scan above, downloads ids and distances and maps inner ids to labels.
+    api = None
+    if not args.no_api:
+        from vsag_amd import pyvsag
+        params = json.dumps({"dtype": "float32", "metric_type": "l2", "dim": d,
+                             "index_param": {"base_quantization_type": "sq8"}})
+        index = pyvsag.Index("brute_force", params)
+        labels = np.arange(n, dtype=np.int64) + 1000000007
+        t0 = time.perf_counter()
+        index.build(x, labels, n, d)
+        api_build = time.perf_counter() - t0
+        for _ in range(max(1, args.warmup)):
+            aids, adist = index.knn_search_batch(q, k, "{}")
+        capi.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            aids, adist = index.knn_search_batch(q, k, "{}")
+        api_sec = (time.perf_counter() - t0) / args.steps
+        t0 = time.perf_counter()
+        for i in range(200):
+            index.knn_search(q[i % nq], k, "{}")
+        api_one = (time.perf_counter() - t0) / 200
+        api = {"qps": nq / api_sec, "ms_per_step": 1e3 * api_sec, "build_seconds": api_build,
+               "one_query_per_call_us": 1e6 * api_one,
+               "same_ids_as_resident_path": float(np.mean(aids - 1000000007 == results["l2"]["ids"])),
+               "what": "vsag::Factory::CreateIndex(brute_force, sq8) -> Build(%d x %d host floats) -> KnnSearch(%d host "
+                       "queries, k=%d) -> host ids / distances, PCIe copies and label mapping included" % (n, d, nq, k)}
+        index.close()
+
     recall = {}
     if not args.no_recall:
         nrec = min(nq, 500)
@@ -267,39 +304,41 @@ def run_c2(env):
              "ip_kernel_ms": ri["kernel_ms"],
              "ip_algorithmic_gbs": ri["passes"] * ri["bytes_per_pass"] / (ri["kernel_ms"] * 1e-3) / 1e9,
              "query_tile": r["tile"], "passes_per_step": r["passes"], "bytes_per_pass": r["bytes_per_pass"],
-             "single_query_l2": single, "build_seconds": t_build, "datagen_seconds": t_gen}
-    # HBM/fabric bytes of one launch of this exact configuration, from rocprofv3 --pmc FETCH_SIZE (x 2.00, the
-    # factor that makes kernels of known size read their size) + WRITE_SIZE (x 1.00): profiles/flat_scan_sq8_c2.md.
-    traffic = None
-    # the same two counters for the last-level launch of the int8 kernel: profiles/prefilter_i8_sq8_c2.md
-    traffic_i8 = 2422324.4 * 2.00 * 1024 + 68345.8 * 1024
+             "single_query_l2": single, "index_api_l2": api, "build_seconds": t_build, "datagen_seconds": t_gen}
+    # HBM/fabric bytes of one launch of this exact configuration come from rocprofv3 --pmc runs of this command
+    # (FETCH_SIZE x 2.00, the factor that makes kernels of known size read their size, + WRITE_SIZE x 1.00); they are
+    # constants of the committed profile, not measurements of this run, and are labelled so.
+    traffic, traffic_source = None, None
     if (n, d, nq, k, r["tile"]) == (1000000, 128, 10000, 10, 4):
-        traffic = 115043826 * 2.00 * 1024 + 28593 * 1024
+        traffic, traffic_source = 115043826 * 2.00 * 1024 + 28593 * 1024, "profiles/flat_scan_sq8_c2.md"
+    elif (n, d, nq, k, r["tile"]) == (1000000, 128, 10000, 10, 256):
+        traffic, traffic_source = PROFILE_TRAFFIC_I8_C2, "profiles/prefilter_i8_sq8_c2.md"
+    if traffic_source is not None:
+        traffic_source += " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command; not measured in this run)"
     roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+            "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": traffic_source,
             "kernel": "flat_scan_kernel<sq8, l2, T=%d>" % r["tile"], "kernel_ms": r["kernel_ms"],
             "algorithmic_bytes_per_launch": algo_bytes}
-    if r["tile"] == 256:
-        # The batch went through the int8 matrix cores (256 queries per workgroup): the timed kernel multiplies
-        # every code of the last level (bytes_per_pass / d of them) with two int8 planes of every query.
+    if r["tile"] >= 64:
+        # The batch went through a matrix-core pre-selection (query tile 256: int8, 128: fp32): the timed kernel meets
+        # every code of the last level (bytes_per_pass / padded code bytes of them) with every query.  Algorithmic work
+        # of the launch = 2 d operations per (query, code) pair; the int8 kernel executes twice that (two int8 planes
+        # per query), reported beside it.  The same launch by the memory figure: passes x code bytes.
+        i8 = r["tile"] == 256
         codes = r["bytes_per_pass"] / float(-(-d // 16) * 16)
-        ops = 2.0 * 2.0 * codes * (-(-d // 32) * 32) * nq
-        tops = ops / (r["kernel_ms"] * 1e-3) / 1e12
-        roof = {"bound": "mfma", "achieved": tops, "peak": MFMA_I8_PEAK_TOPS, "unit": "TOP/s",
-                "frac": tops / MFMA_I8_PEAK_TOPS, "traffic": traffic_i8 if (n, d, nq, k) == (1000000, 128, 10000, 10)
-                else None, "kernel": "prefilter_i8_kernel<l2> (int8 MFMA, last level)", "kernel_ms": r["kernel_ms"],
-                "ops_per_launch": ops, "codes_per_launch": codes,
-                "algorithmic_bytes_per_launch": algo_bytes, "algorithmic_gbs": achieved}
-    elif r["tile"] >= 64:
-        # The batch went through the fp32 matrix-core contraction (query tile 128): the timed kernel multiplies
-        # every code of the last level with every query, 2 d flops per pair.
-        codes = r["bytes_per_pass"] / float(-(-d // 16) * 16)
-        flops = 2.0 * codes * d * nq
-        tf = flops / (r["kernel_ms"] * 1e-3) / 1e12
-        roof = {"bound": "mfma", "achieved": tf, "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": tf / MFMA_F32_PEAK_TFLOPS, "traffic": None, "kernel": "prefilter_kernel<sq8> (fp32 MFMA)",
-                "kernel_ms": r["kernel_ms"], "flops_per_launch": flops,
-                "algorithmic_bytes_per_launch": algo_bytes, "algorithmic_gbs": achieved}
+        ops = 2.0 * codes * d * nq
+        rate = ops / (r["kernel_ms"] * 1e-3) / 1e12
+        peak = MFMA_I8_PEAK_TOPS if i8 else MFMA_F32_PEAK_TFLOPS
+        roof = {"bound": "mfma", "achieved": rate, "peak": peak, "unit": "TOP/s" if i8 else "TFLOP/s",
+                "frac": rate / peak, "traffic": traffic, "traffic_source": traffic_source,
+                "kernel": "prefilter_i8_kernel<l2> (int8 MFMA, last level)" if i8 else "prefilter_kernel<sq8> (fp32 MFMA)",
+                "kernel_ms": r["kernel_ms"], "ops_per_launch": ops, "codes_per_launch": codes,
+                "mfma_frac": rate / peak,
+                "executed_ops_per_launch": (2.0 if i8 else 1.0) * 2.0 * codes * (-(-d // 32) * 32) * nq,
+                "executed_frac": (2.0 if i8 else 1.0) * 2.0 * codes * (-(-d // 32) * 32) * nq /
+                                 (r["kernel_ms"] * 1e-3) / 1e12 / peak,
+                "algorithmic_bytes_per_launch": algo_bytes, "algorithmic_gbs": achieved,
+                "hbm_frac_algorithmic": achieved / HBM_PEAK_GBS}
     return env.base_line("QPS @ recall@10 (1M x 128 SQ8 scan)", "queries/s", r["qps"], r["sec"],
                          "u8 codes; i8 x i8 -> i32 pre-selection, f32 results" if r["tile"] == 256 else
                          "u8 codes, f32 accumulate",
@@ -384,7 +423,7 @@ def run_c3(env):
         capi.check(lib.vsag_amd_kmeans_assign(x_dev.ptr, n, d, cent.ptr, k, labels.ptr, None, loss.ptr, ws.ptr, wsb,
                                               None))
     sec, kms = env.timed(step, args.steps, args.warmup)
-    ws.free()
+    ws_a, wsb_a = ws, wsb
     # the full Lloyd run: 10 iterations from the same initial centroids
     cent2 = env.upload(init)
     wsb = lib.vsag_amd_kmeans_run_workspace_bytes(n, d, k)
@@ -395,23 +434,40 @@ def run_c3(env):
                                        None))
     t_run = time.perf_counter() - t0
     cpu = None
+    inertia = None
     if not args.no_cpu:
         import oracle as orc
         xs = sample_rows[0]
         threads = min(os.cpu_count() or 1, 16)
+        orc.set_threads(threads)
         orc.kmeans_assign(xs[:256], init)
         t0 = time.perf_counter()
         ol, _, oloss = orc.kmeans_assign(xs, init)
         t_cpu = time.perf_counter() - t0
-        gl = labels  # noqa: F841
         step()
         capi.synchronize()
         glabels = labels.to_numpy(np.int32, (n,))[:xs.shape[0]]
         cpu = {"value": xs.shape[0] / t_cpu, "unit": "rows/s", "cores": threads, "kind": "port",
                "sample": "first %d of the %d rows against all %d centroids, CPU restatement of "
-                         "find_nearest_one_with_blas (scalar dot instead of OpenBLAS SGEMM), OpenMP over rows" %
-                         (xs.shape[0], n, k),
+                         "find_nearest_one_with_blas (fp32 dot products in element order, eight centroids per vector, "
+                         "instead of OpenBLAS SGEMM), OpenMP over rows" % (xs.shape[0], n, k),
                "label_agreement_with_gpu": float((ol == glabels).mean())}
+        # Final inertia against the CPU: the centroids after the ten iterations, assigned once more by both sides on
+        # the sample rows (inertia = mean over rows of the squared distance to the nearest centroid).
+        mind = env.buf(n * 4)
+        capi.check(lib.vsag_amd_kmeans_assign(x_dev.ptr, n, d, cent2.ptr, k, labels.ptr, mind.ptr, loss.ptr, ws_a.ptr,
+                                              wsb_a, None))
+        capi.synchronize()
+        final_cent = cent2.to_numpy(np.float32, (k, d))
+        fl, _, floss = orc.kmeans_assign(xs, final_cent)
+        gmin = mind.to_numpy(np.float32, (n,))[:xs.shape[0]].astype(np.float64)
+        gfl = labels.to_numpy(np.int32, (n,))[:xs.shape[0]]
+        g_inertia = float(np.mean(gmin + (xs.astype(np.float64) ** 2).sum(1)))
+        inertia = {"gpu_on_sample": g_inertia, "cpu_on_sample": float(floss),
+                   "relative_difference": abs(g_inertia - floss) / abs(floss),
+                   "label_agreement": float((fl == gfl).mean()), "sample_rows": int(xs.shape[0]),
+                   "gpu_all_rows_after_assignment": float(loss.to_numpy(np.float64, (1,))[0])}
+        mind.free()
     flops = 2.0 * n * k * d
     tf = flops / (kms * 1e-3) / 1e12
     roof = {"bound": "mfma", "achieved": tf, "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -425,7 +481,7 @@ def run_c3(env):
     return env.base_line("k-means assign rows/s", "rows/s", n / sec, sec, "f32",
                          "configs[2]: k-means assignment, N=%d, d=%d, k=%d (one step = one assignment pass)" % (n, d, k),
                          {"lloyd_iterations": iters, "lloyd_seconds": t_run, "final_loss": final.value,
-                          "datagen_seconds": t_gen}, roof, cpu)
+                          "final_inertia_vs_cpu": inertia, "datagen_seconds": t_gen}, roof, cpu)
 
 
 # ------------------------------------------------------------------------------------------- C4
@@ -736,6 +792,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-recall", action="store_true", help="skip the recall check")
     ap.add_argument("--no-single", action="store_true", help="skip the one-query-per-call measurement")
+    ap.add_argument("--no-api", action="store_true", help="skip the index-API leg (host buffers on both sides)")
+    ap.add_argument("--no-kmeans", action="store_true", help="default line only: skip the k-means block (configs[2])")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the search core is single-GPU by design (sharding it means splitting "
@@ -745,6 +803,17 @@ def main():
     env = Env(args)
     env.capi.check(env.lib.vsag_amd_set_scan_contraction(args.contraction))
     line = {"c1": run_c1, "c2": run_c2, "c3": run_c3, "c4": run_c4, "c5": run_c5}[args.config](env)
+    if args.config == "c2" and not args.no_kmeans and not (args.n or args.dim or args.nq):
+        # The metric's second figure, "k-means assign rows/s": configs[2] in the same line.
+        env.capi.check(env.lib.vsag_amd_set_scan_tuning(0, 0))
+        km = run_c3(env)
+        line["kmeans"] = {"metric": km["metric"], "value": km["value"], "unit": km["unit"],
+                          "ms_per_step": km["ms_per_step"], "dtype": km["dtype"], "workload": km["config"]["workload"],
+                          "lloyd_iterations": km["config"]["lloyd_iterations"],
+                          "lloyd_seconds": km["config"]["lloyd_seconds"], "final_loss": km["config"]["final_loss"],
+                          "final_inertia_vs_cpu": km["config"]["final_inertia_vs_cpu"],
+                          "datagen_seconds": km["config"]["datagen_seconds"],
+                          "roofline": km["roofline"], "cpu_baseline": km["cpu_baseline"]}
     print(json.dumps(line))
 
 

@@ -558,6 +558,14 @@ store_dist(const Store& s, const RabitqLayout* rl, const uint8_t* q, const uint8
 
 // ================================================================= exported C entry points
 
+// Threads of the OpenMP loops below (0 = leave as is); the loops that take a `threads` argument set it themselves.
+ORC_API void
+orc_set_threads(int threads) {
+    if (threads > 0) {
+        omp_set_num_threads(threads);
+    }
+}
+
 ORC_API float
 orc_fp32_l2sqr(const float* q, const float* x, uint64_t dim) {
     return fp32_l2sqr(q, x, dim);
@@ -983,25 +991,68 @@ orc_kmeans_assign(const float* x, uint64_t n, uint64_t dim, const float* cent, u
     for (uint64_t j = 0; j < k; ++j) {
         y_sqr[j] = fp32_ip(cent + j * dim, cent + j * dim, dim);
     }
+    // Eight centroids side by side (ct[block][d][lane]) so that the compiler can run eight of the dot products
+    // in one vector; every dot product is still the element-order fp32 sum of fp32_ip (multiply, then add).
+    const uint64_t kb = (k + 7) / 8;
+    std::vector<float> ct(kb * dim * 8, 0.0F);
+    for (uint64_t j = 0; j < k; ++j) {
+        for (uint64_t d = 0; d < dim; ++d) {
+            ct[(j / 8) * dim * 8 + d * 8 + (j % 8)] = cent[j * dim + d];
+        }
+    }
     double error = 0.0;
+    // Rows go four at a time through a block of centroids (the block stays in cache, four independent sums hide the
+    // latency of the adds); the per-row results do not depend on the grouping.
+    constexpr int R = 4;
+    const int64_t ngroups = static_cast<int64_t>((n + R - 1) / R);
 #pragma omp parallel
     {
-        std::vector<float> dist(k);
+        std::vector<float> dist(static_cast<size_t>(R) * kb * 8);
         double local = 0.0;
 #pragma omp for schedule(static)
-        for (int64_t i = 0; i < static_cast<int64_t>(n); ++i) {
-            const float* xi = x + i * dim;
-            for (uint64_t j = 0; j < k; ++j) {
-                dist[j] = -2.0F * fp32_ip(cent + j * dim, xi, dim);
-                dist[j] = 1.0F * y_sqr[j] + dist[j];
+        for (int64_t g = 0; g < ngroups; ++g) {
+            const uint64_t i0 = static_cast<uint64_t>(g) * R;
+            const int rows = static_cast<int>(std::min<uint64_t>(R, n - i0));
+            const float* xr[R];
+            for (int r = 0; r < R; ++r) {
+                xr[r] = x + (i0 + (r < rows ? r : 0)) * dim;
             }
-            auto* me = std::min_element(dist.data(), dist.data() + k);
-            float x_sqr = fp32_ip(xi, xi, dim);
-            labels[i] = static_cast<int32_t>(me - dist.data());
-            if (min_dist != nullptr) {
-                min_dist[i] = *me;
+            for (uint64_t b = 0; b < kb; ++b) {
+                const float* cb = ct.data() + b * dim * 8;
+                float acc[R][8];
+                for (int r = 0; r < R; ++r) {
+                    for (int l = 0; l < 8; ++l) {
+                        acc[r][l] = 0.0F;
+                    }
+                }
+                for (uint64_t d = 0; d < dim; ++d) {
+                    for (int r = 0; r < R; ++r) {
+                        const float xv = xr[r][d];
+                        for (int l = 0; l < 8; ++l) {
+                            acc[r][l] = cb[d * 8 + l] * xv + acc[r][l];
+                        }
+                    }
+                }
+                for (int r = 0; r < R; ++r) {
+                    for (int l = 0; l < 8; ++l) {
+                        dist[(r * kb + b) * 8 + l] = -2.0F * acc[r][l];
+                    }
+                }
             }
-            local += static_cast<double>(*me + x_sqr);
+            for (int r = 0; r < rows; ++r) {
+                float* dr = dist.data() + static_cast<size_t>(r) * kb * 8;
+                for (uint64_t j = 0; j < k; ++j) {
+                    dr[j] = 1.0F * y_sqr[j] + dr[j];
+                }
+                auto* me = std::min_element(dr, dr + k);
+                const float* xi = xr[r];
+                float x_sqr = fp32_ip(xi, xi, dim);
+                labels[i0 + r] = static_cast<int32_t>(me - dr);
+                if (min_dist != nullptr) {
+                    min_dist[i0 + r] = *me;
+                }
+                local += static_cast<double>(*me + x_sqr);
+            }
         }
 #pragma omp critical
         error += local;

@@ -54,6 +54,11 @@ def u64(v):
     return C.c_uint64(int(v))
 
 
+def set_threads(threads):
+    """OpenMP threads of the checker's parallel loops from now on."""
+    lib().orc_set_threads(int(threads))
+
+
 def sq_train(x, bits, metric=L2, mode=3, trunc_rate=0.05, max_sample=0):
     x = f32(x)
     n, d = x.shape

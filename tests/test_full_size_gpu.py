@@ -162,9 +162,40 @@ def test_kmeans_assign_1m_x_960(lib):
         b.free()
 
 
+def test_kmeans_lloyd_10_iterations_on_a_64k_slice(lib):
+    """configs[2], the first 65 536 rows: ten Lloyd iterations from the seeded random-sample initialisation against
+    the checker's KMeansCluster::Run restatement (same initial centroids, same re-seeding of empty clusters)."""
+    n, d, k, iters = 65536, 960, 4096, 10
+    means = mt(315).standard_normal((k, d), dtype=np.float32)
+    x = np.empty((n, d), np.float32)
+    for s, blk in mixture_chunks(47, n, d, means, 0.2, step=1 << 15):
+        x[s:s + blk.shape[0]] = blk
+    cent0 = x[np.sort(mt(7).choice(n, k, replace=False))].copy()
+    xb, cb = dev(x), dev(cent0)
+    labels = capi.DeviceBuffer(n * 4)
+    loss = C.c_double()
+    wsb = lib.vsag_amd_kmeans_run_workspace_bytes(n, d, k)
+    ws = capi.DeviceBuffer(wsb)
+    capi.check(lib.vsag_amd_kmeans_run(xb.ptr, n, d, cb.ptr, k, iters, 7, labels.ptr, C.byref(loss), ws.ptr, wsb, None))
+    gl = labels.to_numpy(np.int32, (n,))
+    gc = cb.to_numpy(np.float32, (k, d))
+    rc, rl, rloss = orc.kmeans_run(x, cent0, iters, 7)
+    assert np.mean(gl == rl) >= 0.999, float(np.mean(gl == rl))
+    assert abs(loss.value - rloss) <= 1e-4 * abs(rloss), (loss.value, rloss)
+    # centroids of clusters whose members agree are the same means (fp32 sums in a different order)
+    same = np.array([np.array_equal(np.nonzero(gl == j)[0], np.nonzero(rl == j)[0]) for j in range(0, k, 16)])
+    assert same.mean() > 0.99
+    np.testing.assert_allclose(gc[::16][same], rc[::16][same], rtol=1e-4, atol=1e-4)
+    # the inertia went down from that of the initial centroids (estimated on the first 2048 rows)
+    _, _, loss0 = orc.kmeans_assign(x[:2048], cent0)
+    assert loss.value < loss0
+    for b in (xb, cb, labels, ws):
+        b.free()
+
+
 def test_ivf_sq4_uniform_10m(lib):
     """configs[3]: 10 000 000 x 128 rows, 4096 lists of SQ4-uniform codes, 64 probes, rerank of 100."""
-    n, d, nq, k, nlist, nprobe, kcand = 10000000, 128, 256, 10, 4096, 64, 100
+    n, d, nq, k, nlist, nprobe, kcand = 10000000, 128, 1024, 10, 4096, 64, 100
     means = mt(315).random((10000, d), dtype=np.float32)
     x_dev = capi.DeviceBuffer(n * d * 4)
     pick = np.sort(mt(7).choice(n, nlist, replace=False))
@@ -224,6 +255,19 @@ def test_ivf_sq4_uniform_10m(lib):
 
     cand, cand_d = lists.ivf_scan(q, b, kcand)
     check_result_shape(cand, cand_d, n)
+    # a batch of this size sends the probe columns behind the first through the int8 matrix cores (ivf_i8_kernel);
+    # the streaming kernel alone must return the same bits
+    info = capi.C.c_int()
+    lib.vsag_amd_last_scan_info(capi.C.byref(info), None, None)
+    assert info.value == 256, "the int8 pass over the posting lists did not run"
+    capi.check(lib.vsag_amd_set_scan_contraction(-1))
+    try:
+        si, sd = lists.ivf_scan(q, b, kcand)
+        lib.vsag_amd_last_scan_info(capi.C.byref(info), None, None)
+        assert info.value <= 8
+    finally:
+        capi.check(lib.vsag_amd_set_scan_contraction(0))
+    assert np.array_equal(si, cand) and np.array_equal(sd.view(np.uint32), cand_d.view(np.uint32))
     # the checker on the same codes, lists and probes: integer distances, so bit-equal; ids up to equal distances
     offsets, order = orc.ivf_build_lists(hlabels, nlist)
     posting = hcodes[order]
@@ -232,7 +276,7 @@ def test_ivf_sq4_uniform_10m(lib):
     assert np.array_equal(od.view(np.uint32), cand_d[:64].view(np.uint32))
     assert_topk_close(cand[:64], cand_d[:64], oi, od, rtol=0, atol=0, tie_rtol=0, label="ivf sq4u 10M")
     # the batch split does not matter: the same queries alone and in groups of 7
-    for s, e in ((0, 1), (5, 6), (10, 17), (100, 107)):
+    for s, e in ((0, 1), (5, 6), (10, 17), (100, 107), (1000, 1024)):
         ci, cd = lists.ivf_scan(q[s:e], b[s:e], kcand)
         assert np.array_equal(ci, cand[s:e]) and np.array_equal(cd.view(np.uint32), cand_d[s:e].view(np.uint32)), (s, e)
 
@@ -244,7 +288,7 @@ def test_ivf_sq4_uniform_10m(lib):
     ri, rd = out_i.to_numpy(np.uint32, (nq, k)), out_d.to_numpy(np.float32, (nq, k))
     check_result_shape(ri, rd, n)
     row = np.empty(d, np.float32)
-    for i in range(0, nq, 8):
+    for i in range(0, nq, 32):
         dd = np.empty(kcand)
         for j, c in enumerate(cand[i]):
             capi.check(lib.vsag_amd_memcpy_d2h(row.ctypes.data, x_dev.ptr + int(c) * d * 4, d * 4, None))
@@ -260,7 +304,7 @@ def test_ivf_sq4_uniform_10m(lib):
 
 def test_rabitq_scan_5m_x_768(lib):
     """configs[4]: 5 000 000 x 768 unit rows, 1-bit codes, 4-bit queries, inner product, 200 candidates."""
-    n, d, nq, kcand = 5000000, 768, 64, 200
+    n, d, nq, kcand = 5000000, 768, 512, 200
     rng = mt(47)
     x_dev = capi.DeviceBuffer(n * d * 4)
     head = None
@@ -294,11 +338,24 @@ def test_rabitq_scan_5m_x_768(lib):
     codes.free()
     ids, dists = store.flat_scan(q, kcand)
     check_result_shape(ids, dists, n)
+    # 512 queries take the matrix-core route (prefilter_rb_kernel: code bits x 4-bit queries on the int8 matrix cores,
+    # exact rescoring); the checker and the streaming kernel alone must agree with it
+    info = capi.C.c_int()
+    lib.vsag_amd_last_scan_info(capi.C.byref(info), None, None)
+    assert info.value == 128, "the matrix-core pre-selection did not run"
     qcodes = orc.rabitq_process_query(q[:16], rot, hcen, orc.IP, 4)
     oi, od = orc.flat_scan_topk(orc.RABITQ, orc.IP, d, hcodes, qcodes, kcand, qbits=4)
     assert_topk_close(ids[:16], dists[:16], oi, od, label="rabitq 5M")
-    ti, td = scan_with_tile(lib, store, q, kcand, 1)
-    assert np.array_equal(ti, ids) and np.array_equal(td.view(np.uint32), dists.view(np.uint32))
+    capi.check(lib.vsag_amd_set_scan_contraction(-1))
+    try:
+        si, sd = store.flat_scan(q[:128], kcand)
+        lib.vsag_amd_last_scan_info(capi.C.byref(info), None, None)
+        assert info.value <= 8
+        ti, td = scan_with_tile(lib, store, q[:32], kcand, 1)
+    finally:
+        capi.check(lib.vsag_amd_set_scan_contraction(0))
+    assert np.array_equal(si, ids[:128]) and np.array_equal(sd.view(np.uint32), dists[:128].view(np.uint32))
+    assert np.array_equal(ti, ids[:32]) and np.array_equal(td.view(np.uint32), dists[:32].view(np.uint32))
     for b in (rot_dev, cen):
         b.free()
     store.destroy()
