@@ -194,6 +194,20 @@ VSAG_AMD_API int vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* store, const
                                uint32_t k, const vsag_amd_search_options_t* options, uint32_t* ids_dev,
                                float* dists_dev, void* workspace_dev, size_t workspace_bytes, void* stream);
 
+/* vsag_amd_flat_scan_topk_ex without a workspace argument and without any allocation: the scan's intermediate
+ * buffers live in a scratch array inside the library's device image (vsag_amd_flat_scan_noalloc_max_bytes() bytes,
+ * 32 MiB, held on every GPU the library runs on until the process ends).  No counterpart in the reference; it is for
+ * callers that cannot call hipMalloc -- code under HIP graph capture, tight serving loops, harnesses that forbid
+ * allocation.  Same results as vsag_amd_flat_scan_topk_ex (options may be NULL).  A scan whose
+ * vsag_amd_flat_scan_workspace_bytes() exceeds the array is rejected with VSAG_AMD_INVALID_ARGUMENT (10^6 sq8 codes
+ * and k = 10: about a thousand queries per call fit).  All calls on one GPU share the array: calls that overlap on
+ * one GPU race, whatever their streams.  Calls no hipMalloc / hipFree and creates no events (the measurement hook is
+ * off for the call). */
+VSAG_AMD_API size_t vsag_amd_flat_scan_noalloc_max_bytes(void);
+VSAG_AMD_API int vsag_amd_flat_scan_topk_noalloc(const vsag_amd_store_t* store, const float* queries_dev, uint64_t nq,
+                                    uint32_t k, const vsag_amd_search_options_t* options, uint32_t* ids_dev,
+                                    float* dists_dev, void* stream);
+
 /* Large batches on flat fp32 / sq8 / sq8_uniform / sq4_uniform (the uniform kinds: at most 128 dimensions) / rabitq stores are served by a matrix-core contraction that pre-selects
  * candidates, which are then recomputed and selected exactly as the streaming scan does (same results, bit for bit).
  * rabitq stores with 4-bit queries and at most 1024 dimensions (L2, inner product) expand code bits and query nibbles to

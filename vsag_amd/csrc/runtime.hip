@@ -18,6 +18,8 @@ static int g_cu_count = 0;
 static char g_name[256] = {0};
 static uint64_t g_hbm = 0;
 
+int static_scratch_setup(int device);  // scan.hip: address of the library's own scratch array on `device`
+
 __global__ void
 probe_kernel(int* out) {
     *out = 950;
@@ -52,6 +54,7 @@ init_device(int device) {
         return fail(VSAG_AMD_INTERNAL_ERROR, "gfx950 code object did not load or run: %s",
                     hipGetErrorString(launch != hipSuccess ? launch : copy));
     }
+    VA_TRY(static_scratch_setup(device));
     g_cu_count = prop.multiProcessorCount;
     g_hbm = prop.totalGlobalMem;
     snprintf(g_name, sizeof(g_name), "%s (%s)", prop.name, prop.gcnArchName);
@@ -87,10 +90,19 @@ struct KernelTimer {
     bool recorded = false;
 };
 static thread_local KernelTimer tl_timer;
+static thread_local bool tl_timing_off = false;
+
+// Calls that must not create anything (events included) switch the measurement hook off for their duration.
+bool
+timing_suppress(bool off) {
+    const bool was = tl_timing_off;
+    tl_timing_off = off;
+    return was;
+}
 
 void
 timing_begin(hipStream_t st) {
-    if (g_timing.load() == 0) {
+    if (g_timing.load() == 0 || tl_timing_off) {
         return;
     }
     if (tl_timer.start == nullptr) {
@@ -103,7 +115,7 @@ timing_begin(hipStream_t st) {
 
 void
 timing_end(hipStream_t st) {
-    if (g_timing.load() == 0 || !tl_timer.recorded) {
+    if (g_timing.load() == 0 || tl_timing_off || !tl_timer.recorded) {
         return;
     }
     tl_timer.recorded = hipEventRecord(tl_timer.stop, st) == hipSuccess;

@@ -13,6 +13,8 @@
 // survivors that the bound still admits; a merge kernel picks the k best per query.  All waves of a query
 // share a handful of addresses (its bound, its seed row), and atomics on one address serialise in L2, so
 // every atomicMin is preceded by a plain load and issued only when it would lower the value.
+#include <mutex>
+
 #include "distance.h"
 #include "store.h"
 #include "topk.h"
@@ -998,6 +1000,10 @@ vsag_amd_flat_scan_topk(const vsag_amd_store_t* s, const float* queries_dev, uin
 
 namespace {
 
+int flat_scan_call(const vsag_amd_store_t* s, const float* queries_dev, uint64_t nq, uint32_t k,
+                   const vsag_amd_search_options_t* options, uint32_t* ids_dev, float* dists_dev, void* workspace_dev,
+                   size_t workspace_bytes, void* stream);
+
 // One streaming launch over tiles [tile0, tile_end), writing partial lists slot0, slot0 + 1, ...
 int
 run_streaming(const vsag_amd_store* s, const ScanPlan& p, const ScanArgs& a, const ScanBuffers& b, uint64_t nq,
@@ -1029,6 +1035,16 @@ vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, 
                            const vsag_amd_search_options_t* options, uint32_t* ids_dev, float* dists_dev,
                            void* workspace_dev, size_t workspace_bytes, void* stream) {
     VA_TRY(ensure_init());
+    return flat_scan_call(s, queries_dev, nq, k, options, ids_dev, dists_dev, workspace_dev, workspace_bytes, stream);
+}
+
+namespace {
+
+// The whole flat scan of one call on `stream`, with every intermediate buffer carved out of the given workspace.
+int
+flat_scan_call(const vsag_amd_store_t* s, const float* queries_dev, uint64_t nq, uint32_t k,
+               const vsag_amd_search_options_t* options, uint32_t* ids_dev, float* dists_dev, void* workspace_dev,
+               size_t workspace_bytes, void* stream) {
     VA_TRY(check_scan_call(s, nq, k));
     VA_CHECK_ARG(s->nlist == 0, "flat scan on a posting-list store");
     VA_CHECK_ARG(queries_dev && ids_dev && dists_dev, "null query / output pointer");
@@ -1095,6 +1111,74 @@ vsag_amd_flat_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, 
     const uint64_t timed_tiles = contraction ? s->ntiles - cp.level_begin[cp.levels - 1] : s->ntiles;
     tl_last_bytes = timed_tiles * s->G * kWave * kGranule;
     return 0;
+}
+
+}  // namespace
+
+// ---- the flat scan for callers that cannot allocate ------------------------------------------------------------
+// The intermediate buffers of a scan (query tables, bounds, seed rows, counted partial lists, candidate lists)
+// normally sit in a workspace the caller allocates.  Code under HIP graph capture, tight serving loops and
+// harnesses that forbid hipMalloc cannot do that: for them the library keeps one scratch array of fixed size in
+// its own device image.  Every GPU the library runs on holds its own copy at its own address until the process
+// ends; the address is looked up once per device with that device current.  All calls on one GPU share the array
+// and it keeps the last call's contents: every buffer carved from it is (re)initialised by the call that uses
+// it, and two calls that overlap on one GPU race.
+constexpr size_t kStaticScratchBytes = 32ull << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxScratchDevices = 64;
+static void* g_scratch_ptr[kMaxScratchDevices] = {};
+static std::mutex g_scratch_mutex;
+
+namespace vsag_amd {
+// Looks up the device address of `scratch` on `device`, which must be the current device.
+int
+static_scratch_setup(int device) {
+    VA_CHECK_ARG(device >= 0 && device < kMaxScratchDevices, "device %d out of range [0, %d)", device, kMaxScratchDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[device] != nullptr) {
+        return 0;
+    }
+    void* ptr = nullptr;
+    VA_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (ptr == nullptr) {
+        return fail(VSAG_AMD_INTERNAL_ERROR, "the library's scratch array has no address on device %d", device);
+    }
+    g_scratch_ptr[device] = ptr;
+    return 0;
+}
+bool timing_suppress(bool off);
+}  // namespace vsag_amd
+
+extern "C" size_t
+vsag_amd_flat_scan_noalloc_max_bytes(void) {
+    return kStaticScratchBytes;
+}
+
+extern "C" int
+vsag_amd_flat_scan_topk_noalloc(const vsag_amd_store_t* s, const float* queries_dev, uint64_t nq, uint32_t k,
+                                const vsag_amd_search_options_t* options, uint32_t* ids_dev, float* dists_dev,
+                                void* stream) {
+    VA_TRY(ensure_init());
+    VA_TRY(check_scan_call(s, nq, k));
+    int device = 0;
+    VA_HIP(hipGetDevice(&device));
+    VA_CHECK_ARG(device >= 0 && device < kMaxScratchDevices, "device %d out of range [0, %d)", device, kMaxScratchDevices);
+    if (g_scratch_ptr[device] == nullptr) {
+        // A device the library was not initialised on: first call there.
+        VA_TRY(static_scratch_setup(device));
+    }
+    const size_t need = vsag_amd_flat_scan_workspace_bytes(s, nq, k);
+    VA_CHECK_ARG(need != 0 && need <= kStaticScratchBytes,
+                 "this scan needs %zu bytes of scratch memory, the library's own array holds %zu: send fewer queries "
+                 "per call or use vsag_amd_flat_scan_topk_ex with a workspace",
+                 need, kStaticScratchBytes);
+    // The measurement hook creates events on first use: not in this call.
+    const bool was = timing_suppress(true);
+    const int rc = flat_scan_call(s, queries_dev, nq, k, options, ids_dev, dists_dev, g_scratch_ptr[device],
+                                  kStaticScratchBytes, stream);
+    timing_suppress(was);
+    return rc;
 }
 
 namespace vsag_amd {
