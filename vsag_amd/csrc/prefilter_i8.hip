@@ -48,8 +48,9 @@ struct QuantizeArgs {
     const uint32_t* ymax_bits;  // largest |y| of the store (l2: scaled codes, ip: raw codes)
     uint64_t nq, nq_pad;
     uint8_t* q8;     // nq_pad x 256 bytes
-    float* u;        // l2: -2 s2
-    uint32_t* tau;   // l2: float bits of the threshold on |y|^2 + u T; ip: smallest T that passes (int32)
+    float* amax;     // l2: per query max |b| (rounded up; 0 for queries that take no part), written by query_amax_kernel
+    float* ginv;     // l2: per group of kI8Group queries, 1 / (2 s2) of the scale the group shares (0: no scale)
+    uint32_t* tau;   // smallest T that passes (int32); l2: T is the matrix product minus the code's integer term
 };
 
 __device__ inline double
@@ -69,12 +70,67 @@ wave_max_f64(double v) {
     return v;
 }
 
+// The l2 test compares the matrix product with a per-code integer (|y|^2 / 2 s2, see prefilter_i8_kernel), so the
+// kI8Group queries that meet a code in one workgroup must share the scale s2: it is taken from the largest |b| of the
+// group.  A query much smaller than its group's largest loses resolution (more candidates, never a wrong result).
+// One wave per query: amax[q] = max_d |b_d|, rounded up to a float; 0 for padding rows and rows with NaN / infinite
+// entries (they pass everything anyway and must not blow up the scale of their group).
+__global__ void __launch_bounds__(64)
+query_amax_kernel(QuantizeArgs p) {
+    const uint64_t q = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    double m = 0.0;
+    if (q < p.nq) {
+        const float* row = p.qtab + q * p.qstride;
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const uint32_t d = lane + 64 * r;
+            if (d < p.kdim) {
+                const double a = static_cast<double>(row[d]);
+                const double b = fabs(p.scale != nullptr ? a * static_cast<double>(p.scale[d]) : a);
+                m = b > m || !(b < 1.0e300) ? b : m;
+            }
+        }
+    }
+    // NaN wins the reduction so that a bad row is seen as such.
+    for (int off = 32; off > 0; off >>= 1) {
+        const double o = __shfl_xor(m, off);
+        m = o > m || !(o < 1.0e300) ? o : m;
+    }
+    if (lane == 0) {
+        float f = 0.0F;
+        if (m < 1.0e30) {
+            f = static_cast<float>(m);
+            f = static_cast<double>(f) < m ? __uint_as_float(__float_as_uint(f) + 1U) : f;  // m > 0 here: next float up
+        }
+        p.amax[q] = f;
+    }
+}
+
 // One wave per query; lane l owns dimensions l and l + 64.
 __global__ void __launch_bounds__(64)
 quantize_queries_i8_kernel(QuantizeArgs p) {
     const uint64_t q = blockIdx.x;
     const uint32_t lane = threadIdx.x;
     uint8_t* out = p.q8 + q * kI8QueryBytes;
+    // l2: the scale of the whole group.
+    double gmax = 0.0;
+    if (p.is_l2) {
+        const uint64_t g0 = q / kI8Group * kI8Group;
+        float m = 0.0F;
+#pragma unroll
+        for (int r = 0; r < static_cast<int>(kI8Group / kWave); ++r) {
+            m = fmaxf(m, p.amax[g0 + lane + kWave * r]);
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            m = fmaxf(m, __shfl_xor(m, off));
+        }
+        gmax = static_cast<double>(m);
+        if (q == g0 && lane == 0) {
+            // 1 / (2 s2) as the kernel multiplies the code terms with it.
+            p.ginv[q / kI8Group] = gmax > 0.0 ? static_cast<float>(127.0 * 256.0 / (2.0 * gmax)) : 0.0F;
+        }
+    }
     if (q >= p.nq) {
         // Padding rows: zero operands and a threshold nothing meets.
         out[lane] = 0;
@@ -82,8 +138,7 @@ quantize_queries_i8_kernel(QuantizeArgs p) {
         out[128 + lane] = 0;
         out[192 + lane] = 0;
         if (lane == 0) {
-            p.u[q] = 0.0F;
-            p.tau[q] = p.is_l2 ? __float_as_uint(-__builtin_inff()) : 0x7FFFFFFFU;
+            p.tau[q] = 0x7FFFFFFFU;
         }
         return;
     }
@@ -96,7 +151,11 @@ quantize_queries_i8_kernel(QuantizeArgs p) {
         // The product of two floats is exact in double.
         b[r] = p.scale != nullptr && d < p.kdim ? a[r] * static_cast<double>(p.scale[d]) : a[r];
     }
-    const double amax = wave_max_f64(fmax(fabs(b[0]), fabs(b[1])));
+    const double own_max = wave_max_f64(fmax(fabs(b[0]), fabs(b[1])));
+    // A row with NaN / infinite entries is not part of its group's maximum; it keeps zero operands and passes
+    // everything (below).
+    const bool bad_row = !(own_max < 1.0e30);
+    const double amax = p.is_l2 ? (bad_row ? 0.0 : gmax) : own_max;
     const double s1 = amax / 127.0;
     const double s2 = s1 / 256.0;
     double e_pos = 0.0, e_neg = 0.0, w = 0.0;
@@ -124,12 +183,10 @@ quantize_queries_i8_kernel(QuantizeArgs p) {
         return;
     }
     const uint32_t bbits = p.bound[q];
-    const float u = static_cast<float>(-2.0 * s2);
-    p.u[q] = u;
-    if (bbits == 0xFFFFFFFFU || !(b1 < 1.0e300) || !(a2 < 1.0e300)) {
-        // No bound yet, or a query with NaN / infinite entries: everything is a candidate (and the query will
-        // overflow into the streaming kernel).
-        p.tau[q] = p.is_l2 ? __float_as_uint(3.0e38F) : 0x80000000U;
+    if (bbits == 0xFFFFFFFFU || !(b1 < 1.0e300) || !(a2 < 1.0e300) || bad_row || (p.is_l2 && !(s2 > 0.0))) {
+        // No bound yet, a query with NaN / infinite entries, or (l2) a group of all-zero queries, whose test would
+        // have no scale: everything is a candidate (and the query will overflow into the streaming kernel).
+        p.tau[q] = 0x80000000U;
         return;
     }
     constexpr double kU = 5.9604644775390625e-8;  // 2^-24, the unit roundoff of fp32
@@ -144,13 +201,18 @@ quantize_queries_i8_kernel(QuantizeArgs p) {
         const double e_stream = 4.0 * kU * sqrt(s_abs) * ymax + 2.0 * (p.kdim + 4) * kU * s_abs;
         // |y|^2 per code is accumulated in double and rounded once.
         const double e_term = 2.0 * kU * ymax * ymax;
-        // dist = a2 + |y|^2 - 2 s2 (T + 128 w) - 2 <e, c>, T the integer the matrix cores deliver.
+        // dist = a2 + |y|^2 - 2 s2 (M + 128 w) - 2 <e, c>, M the integer the matrix cores deliver: the pair can matter
+        // when |y|^2 - 2 s2 M <= t_real, i.e. M >= |y|^2 / (2 s2) - t_real / (2 s2).
         const double t_real = bd - a2 + 256.0 * s2 * w + 2.0 * q_err + e_stream + e_term;
-        // The test itself runs in fp32: fl(T) u + |y|^2 in one fma against the rounded threshold.
-        const double reach = 2.0 * (255.0 + 129.0) * b1;  // bounds |2 s2 T|
-        const double slack = 4.0 * kU * (reach + ymax * ymax + fabs(t_real));
-        const double t = t_real + slack;
-        p.tau[q] = __float_as_uint(t < 3.0e38 ? static_cast<float>(t) : 3.0e38F);
+        // The kernel subtracts I = rn(fl(|y|^2 inv)) from M, inv = fl(1 / (2 s2)) (ginv above): I differs from the real
+        // |y|^2 / (2 s2) by at most a half plus two fp32 roundings of a value of at most ymax^2 / (2 s2); the kernel
+        // clamps I from above only, which admits more.  So M - I >= floor(-t_real / (2 s2) - that - 1) keeps every
+        // pair the real test keeps.
+        const double x_max = ymax * ymax / (2.0 * s2);
+        const double x = floor(-t_real / (2.0 * s2) - 0.5 - 4.0 * kU * x_max - 1.0);
+        const int32_t ti = x >= 2147483647.0 ? 0x7FFFFFFF : (x <= -2147483648.0 ? static_cast<int32_t>(0x80000000U)
+                                                                                 : static_cast<int32_t>(x));
+        p.tau[q] = static_cast<uint32_t>(ti);
     } else {
         // dist = 1 - (fl(sum c a) + qmeta): the fp32 sum is off by at most n u sum |c a|, the two closing
         // operations by u of their results; twice that is allowed for.
@@ -283,8 +345,9 @@ struct PrefilterI8Args {
     uint64_t n;
     const uint4* q8;      // [query][plane][granule]
     uint64_t nq;
-    const float* term;    // per slot |y|^2 (l2)
-    const float* u;       // per query (l2)
+    const float* term;    // per slot: |y|^2 (sq8 l2) or the uniform kinds' term
+    const float* u;       // per query (fma test)
+    const float* ginv;    // per group of kI8Group queries: 1 / (2 s2) (integer test with a code term)
     const uint32_t* tau;  // per query
     // Candidates go to private lists: list (group, lane / 32) of a query belongs to one lane of one wave for the
     // whole kernel, so appending needs no atomic and nobody waits for one.
@@ -296,35 +359,31 @@ struct PrefilterI8Args {
 
 constexpr int kI8StageTiles = 2;  // storage tiles per LDS stage (one barrier per stage)
 
+// How a (query, code) pair is judged from M = 256 H + L, the two matrix products:
+//   kI8TestFma      fl(fl(M) u_q + term_o) <= tau_q in fp32 (the uniform kinds: term_o and u_q from their formulas);
+//   kI8TestInt      M >= tau_q (sq8 inner product: the per-code part of the distance is in M already);
+//   kI8TestIntTerm  M - I_o >= tau_q (sq8 l2) with I_o = rn(term_o / 2 s2) the code's |y|^2 in units of the product.
+//                   -I_o is what the accumulator of L starts from, so the matrix pipe does the subtraction and the
+//                   test costs what the plain integer test costs.
+constexpr int kI8TestFma = 0;
+constexpr int kI8TestInt = 1;
+constexpr int kI8TestIntTerm = 2;
+
 struct I8Stage {
     uint4 codes[kI8StageTiles][8 * kWave];  // granule-major, as in the store; bytes are c - 128
-    float term[kI8StageTiles][kWave];
+    float term[kI8StageTiles][kWave];       // kI8TestIntTerm: the bits of the int32 -I_o
 };
 
-// The sixteen verdicts of one 32 x 32 block for this lane's query; returns the lanes with any verdict set.
-template <int METRIC>
-__device__ inline uint64_t
-i8_verdicts(const intx16& hi, const intx16& lo, const float (&tm)[16], float uq, uint32_t tau, bool (&pass)[16]) {
-    uint64_t any = 0;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-        const int32_t tt = (hi[e] << 8) + lo[e];
-        if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
-            pass[e] = fmaf(static_cast<float>(tt), uq, tm[e]) <= __uint_as_float(tau);
-        } else {
-            pass[e] = tt >= static_cast<int32_t>(tau);
-        }
-        any |= __ballot(pass[e]);
-    }
-    return any;
-}
+// Largest code term in units of the product; beyond it the term is clamped (which only admits more).
+constexpr float kI8TermClamp = 1073741824.0F;  // 2^30
 
 // NIBBLE: the codes hold two 4-bit values per byte (sq4_uniform, at most four granules per code): a granule is staged
 // as two, its low nibbles and its high nibbles, as they are (0..15 needs no shift to fit a signed byte).
-template <int METRIC, bool NIBBLE = false>
+template <int TEST, bool NIBBLE = false>
 __global__ void __launch_bounds__(256, 2)
 prefilter_i8_kernel(PrefilterI8Args p) {
     __shared__ I8Stage stage[2];
+    constexpr bool kTerm = TEST != kI8TestInt;  // a per-code term takes part in the test
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
     const uint32_t wave = tid >> 6;
@@ -354,10 +413,11 @@ prefilter_i8_kernel(PrefilterI8Args p) {
             ql[j][s] = intx4{static_cast<int>(lv.x), static_cast<int>(lv.y), static_cast<int>(lv.z),
                              static_cast<int>(lv.w)};
         }
-        uq[j] = p.u[q];
+        uq[j] = TEST == kI8TestFma ? p.u[q] : 0.0F;
         tau[j] = p.tau[q];
         my_list[j] = p.cand + ((q < p.nq ? q : 0) * 2 * p.groups + 2 * blockIdx.x + half) * p.sub_cap;
     }
+    const float ginv = TEST == kI8TestIntTerm ? p.ginv[blockIdx.y] : 0.0F;
 
     // Staging: wave w copies granules w and w + 4 of each tile of the stage, a lane per code.
     uint4 regs[kI8StageTiles][2];
@@ -377,7 +437,7 @@ prefilter_i8_kernel(PrefilterI8Args p) {
                     regs[tt][r] = p.tiles[(tile * p.G + j) * kWave + lane];
                 }
             }
-            if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+            if constexpr (kTerm) {
                 my_term[tt] = 0.0F;
                 if (wave == 0) {
                     const uint64_t slot = tile * kWave + lane;
@@ -403,17 +463,25 @@ prefilter_i8_kernel(PrefilterI8Args p) {
                         make_uint4(v.x ^ 0x80808080U, v.y ^ 0x80808080U, v.z ^ 0x80808080U, v.w ^ 0x80808080U);
                 }
             }
-            if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+            if constexpr (kTerm) {
                 if (wave == 0) {
-                    st.term[tt][lane] = my_term[tt];
+                    if constexpr (TEST == kI8TestIntTerm) {
+                        // -I_o, I_o = rn(term / 2 s2) clamped from above (a slot without a code: the clamp itself,
+                        // such a slot is never appended).  A term of NaN compares false and converts to 0.
+                        const float x = my_term[tt] * ginv;
+                        const int32_t io = x >= kI8TermClamp ? static_cast<int32_t>(kI8TermClamp) : __float2int_rn(x);
+                        st.term[tt][lane] = __int_as_float(-io);
+                    } else {
+                        st.term[tt][lane] = my_term[tt];
+                    }
                 }
             }
         }
     };
 
     // A stage is a run of 32 x 32 blocks: block b = (tile b / 4 of the stage, codes 32 ((b / 2) % 2) ..., queries
-    // 32 (b % 2) ...).  The matrix instructions of block b + 1 are issued among the verdicts of block b, so that
-    // the matrix pipe and the vector ALU of the wave run side by side.
+    // 32 (b % 2) ...).  The matrix instructions of block b + 1 are issued among the verdict instructions of block b,
+    // so that the matrix pipe and the vector ALU of the wave run side by side.
     constexpr int kBlocks = 4 * kI8StageTiles;
     // The grid never has more columns than there are stages, so the first stage exists.  Fetching it without a
     // condition also lets every load issued so far (the query operands) complete here, once, instead of being
@@ -433,7 +501,7 @@ prefilter_i8_kernel(PrefilterI8Args p) {
             const uint64_t slot0 = (p.tile_begin + sg * kI8StageTiles) * kWave;
             intx16 hi[2], lo[2];  // two sets: one being filled, one being judged
             // Row r of the stage = codes 32 (r % 2) ... of its tile r / 2; blocks 2 r and 2 r + 1 are its two query
-            // halves.  Code operands and |y|^2 terms of a row are read from LDS one block before their first use
+            // halves.  Code operands and terms of a row are read from LDS one block before their first use
             // (two register sets each), so that no matrix instruction and no verdict waits for LDS.
             intx4 av[2][4];
             float tm[2][16];
@@ -445,7 +513,7 @@ prefilter_i8_kernel(PrefilterI8Args p) {
                     av[r & 1][s] = intx4{static_cast<int>(c.x), static_cast<int>(c.y), static_cast<int>(c.z),
                                          static_cast<int>(c.w)};
                 }
-                if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                if constexpr (kTerm) {
                     // Element e of a lane is code 32 i + 8 (e / 4) + 4 (lane / 32) + e % 4 of the tile.
 #pragma unroll
                     for (int g = 0; g < 4; ++g) {
@@ -462,7 +530,8 @@ prefilter_i8_kernel(PrefilterI8Args p) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     h[e] = 0;
-                    l[e] = 0;
+                    // The low product starts from minus the code's integer term: M - I_o comes out of the matrix pipe.
+                    l[e] = TEST == kI8TestIntTerm ? __float_as_int(tm[r & 1][e]) : 0;
                 }
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
@@ -470,12 +539,17 @@ prefilter_i8_kernel(PrefilterI8Args p) {
                     l = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[r & 1][s], ql[j][s], l, 0, 0, 0);
                 }
             };
+            // The quantity of element e that is compared with the query's threshold.
+            auto judged_int = [&](int b, int e) { return (hi[b & 1][e] << 8) + lo[b & 1][e]; };
+            auto judged_fma = [&](int b, int e) {
+                return fmaf(static_cast<float>(judged_int(b, e)), uq[b & 1], tm[(b >> 1) & 1][e]);
+            };
             read_row(0);
             multiply(0, hi[0], lo[0]);
 #pragma unroll
             for (int b = 0; b < kBlocks; ++b) {
                 const int r = b >> 1, j = b & 1;
-                constexpr int kDsReads = METRIC == VSAG_AMD_METRIC_L2 ? 8 : 4;
+                constexpr int kDsReads = kTerm ? 8 : 4;
                 const bool reads = j == 0 && b + 2 < kBlocks;
                 if (reads) {
                     read_row(r + 1);
@@ -483,10 +557,26 @@ prefilter_i8_kernel(PrefilterI8Args p) {
                 if (b + 1 < kBlocks) {
                     multiply(b + 1, hi[(b + 1) & 1], lo[(b + 1) & 1]);
                 }
-                // Nearly nothing passes: the sixteen verdicts stay in scalar registers, and only when one of them
-                // has a bit set does the wave turn them into a bit mask per lane.
-                bool pass[16];
-                const uint64_t any = i8_verdicts<METRIC>(hi[b & 1], lo[b & 1], tm[r & 1], uq[j], tau[j], pass);
+                // Nearly nothing passes.  The sixteen elements of a lane are reduced to their best one with
+                // three-operand max / min instructions (three vector instructions per two elements, none of them
+                // writing a scalar register), and one compare decides whether the block needs a second look.
+                bool hit;
+                if constexpr (TEST == kI8TestFma) {
+                    float best = __builtin_inff();
+#pragma unroll
+                    for (int e = 0; e < 16; e += 2) {
+                        best = fminf(fminf(best, judged_fma(b, e)), judged_fma(b, e + 1));
+                    }
+                    hit = best <= __uint_as_float(tau[j]);
+                } else {
+                    int32_t best = static_cast<int32_t>(0x80000000U);
+#pragma unroll
+                    for (int e = 0; e < 16; e += 2) {
+                        best = max(max(best, judged_int(b, e)), judged_int(b, e + 1));
+                    }
+                    hit = best >= static_cast<int32_t>(tau[j]);
+                }
+                const uint64_t any = __ballot(hit);
                 if (b + 1 < kBlocks) {
                     // The LDS reads first; then one matrix instruction (32 cycles of the pipe) at a time, each
                     // followed by its share of the verdict instructions.
@@ -496,24 +586,29 @@ prefilter_i8_kernel(PrefilterI8Args p) {
 #pragma unroll
                     for (int m = 0; m < 8; ++m) {
                         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x002, METRIC == VSAG_AMD_METRIC_L2 ? 8 : 4, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, TEST == kI8TestFma ? 7 : 3, 0);
                     }
                 }
                 if (any != 0) {
-                    uint32_t bits = 0;
+                    // Some lane has an element that passes: judge the elements one by one (the accumulators of this
+                    // block are not touched before the next block has been judged) and let the lanes under each
+                    // element's mask append.
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
-                        bits |= pass[e] ? 1U << e : 0U;
-                    }
-                    while (bits != 0) {
-                        const uint32_t e = static_cast<uint32_t>(__builtin_ctz(bits));
-                        bits &= bits - 1;
-                        const uint64_t slot = slot0 + 32 * r + 8 * (e >> 2) + 4 * half + (e & 3);
-                        if (slot < p.n) {
-                            if (ncand[j] < p.sub_cap) {
-                                my_list[j][ncand[j]] = static_cast<uint32_t>(slot);
+                        bool pass;
+                        if constexpr (TEST == kI8TestFma) {
+                            pass = judged_fma(b, e) <= __uint_as_float(tau[j]);
+                        } else {
+                            pass = judged_int(b, e) >= static_cast<int32_t>(tau[j]);
+                        }
+                        if (__ballot(pass) != 0) {
+                            const uint64_t slot = slot0 + 32 * r + 8 * (e >> 2) + 4 * half + (e & 3);
+                            if (pass && slot < p.n) {
+                                if (ncand[j] < p.sub_cap) {
+                                    my_list[j][ncand[j]] = static_cast<uint32_t>(slot);
+                                }
+                                ++ncand[j];
                             }
-                            ++ncand[j];
                         }
                     }
                 }
@@ -551,6 +646,13 @@ prefilter_i8_query_bytes(uint64_t nq) {
     return static_cast<size_t>(div_up(nq, static_cast<uint64_t>(kI8Group)) * kI8Group) * kI8QueryBytes;
 }
 
+// Floats of per-query and per-group scalars the quantizing kernels keep for nq queries.
+size_t
+prefilter_i8_scalar_floats(uint64_t nq) {
+    const uint64_t groups = div_up(nq, static_cast<uint64_t>(kI8Group));
+    return static_cast<size_t>(groups * kI8Group + groups);
+}
+
 // Candidate lists per query (two per workgroup column) for nq queries over `span` tiles.
 uint32_t
 prefilter_i8_sub_lists(uint64_t nq, uint64_t span) {
@@ -570,9 +672,10 @@ launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride
                     uint32_t sub_cap, hipStream_t st) {
     const bool nibbles = s->kind == VSAG_AMD_KIND_SQ4_UNIFORM;
     const bool uniform = s->kind == VSAG_AMD_KIND_SQ8_UNIFORM || nibbles;
-    // The uniform kinds use the l2 form of the test (fma of the integer and a per-code term) for every metric.
-    const bool l2 = s->metric == VSAG_AMD_METRIC_L2 || uniform;
+    const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
     const uint64_t nq_pad = div_up(nq, static_cast<uint64_t>(kI8Group)) * kI8Group;
+    // `u` holds a float per padded query and one per group of kI8Group queries behind them (prefilter_i8_scalar_floats).
+    float* ginv = u + nq_pad;
     if (uniform) {
         UniformQuantizeArgs z{};
         z.qtab = reinterpret_cast<const uint32_t*>(qtab);
@@ -580,7 +683,7 @@ launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride
         z.kdim = s->dpad;
         z.qmeta = qmeta;
         z.qmeta_stride = qmeta_stride;
-        z.is_l2 = s->metric == VSAG_AMD_METRIC_L2 ? 1 : 0;
+        z.is_l2 = l2 ? 1 : 0;
         z.nibbles = nibbles ? 1 : 0;
         z.lb = s->ulb;
         z.rate = s->scalar_rate;
@@ -592,23 +695,26 @@ launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride
         z.u = u;
         z.tau = tau;
         hipLaunchKernelGGL(quantize_uniform_i8_kernel, dim3(static_cast<uint32_t>(nq_pad)), dim3(kWave), 0, st, z);
-    }
-    QuantizeArgs z{};
-    z.qtab = qtab;
-    z.qstride = qstride;
-    z.kdim = s->dpad;
-    z.scale = l2 ? s->scale_dev : nullptr;
-    z.qmeta = l2 ? nullptr : qmeta;
-    z.qmeta_stride = qmeta_stride;
-    z.is_l2 = l2 ? 1 : 0;
-    z.bound = bound;
-    z.ymax_bits = s->pf_ymax;
-    z.nq = nq;
-    z.nq_pad = nq_pad;
-    z.q8 = q8;
-    z.u = u;
-    z.tau = tau;
-    if (!uniform) {
+    } else {
+        QuantizeArgs z{};
+        z.qtab = qtab;
+        z.qstride = qstride;
+        z.kdim = s->dpad;
+        z.scale = l2 ? s->scale_dev : nullptr;
+        z.qmeta = l2 ? nullptr : qmeta;
+        z.qmeta_stride = qmeta_stride;
+        z.is_l2 = l2 ? 1 : 0;
+        z.bound = bound;
+        z.ymax_bits = s->pf_ymax;
+        z.nq = nq;
+        z.nq_pad = nq_pad;
+        z.q8 = q8;
+        z.amax = u;
+        z.ginv = ginv;
+        z.tau = tau;
+        if (l2) {
+            hipLaunchKernelGGL(query_amax_kernel, dim3(static_cast<uint32_t>(nq_pad)), dim3(kWave), 0, st, z);
+        }
         hipLaunchKernelGGL(quantize_queries_i8_kernel, dim3(static_cast<uint32_t>(nq_pad)), dim3(kWave), 0, st, z);
     }
     VA_HIP(hipGetLastError());
@@ -623,6 +729,7 @@ launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride
     p.nq = nq;
     p.term = s->pf_term;
     p.u = u;
+    p.ginv = ginv;
     p.tau = tau;
     p.cand = cand;
     p.cand_cnt = cand_cnt;
@@ -632,11 +739,13 @@ launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride
     dim3 grid(p.groups, static_cast<uint32_t>(nq_pad / kI8Group));
     timing_begin(st);
     if (nibbles) {
-        hipLaunchKernelGGL((prefilter_i8_kernel<VSAG_AMD_METRIC_L2, true>), grid, dim3(256), 0, st, p);
+        hipLaunchKernelGGL((prefilter_i8_kernel<kI8TestFma, true>), grid, dim3(256), 0, st, p);
+    } else if (uniform) {
+        hipLaunchKernelGGL(prefilter_i8_kernel<kI8TestFma>, grid, dim3(256), 0, st, p);
     } else if (l2) {
-        hipLaunchKernelGGL(prefilter_i8_kernel<VSAG_AMD_METRIC_L2>, grid, dim3(256), 0, st, p);
+        hipLaunchKernelGGL(prefilter_i8_kernel<kI8TestIntTerm>, grid, dim3(256), 0, st, p);
     } else {
-        hipLaunchKernelGGL(prefilter_i8_kernel<VSAG_AMD_METRIC_IP>, grid, dim3(256), 0, st, p);
+        hipLaunchKernelGGL(prefilter_i8_kernel<kI8TestInt>, grid, dim3(256), 0, st, p);
     }
     timing_end(st);
     VA_HIP(hipGetLastError());

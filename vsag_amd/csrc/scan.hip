@@ -743,6 +743,7 @@ int launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, ui
                      uint32_t* gate, uint8_t* q8, float* q8_u, uint32_t sub_lists, uint32_t sub_cap, hipStream_t st);
 bool prefilter_i8_supports(const vsag_amd_store* s);
 size_t prefilter_i8_query_bytes(uint64_t nq);
+size_t prefilter_i8_scalar_floats(uint64_t nq);
 uint32_t prefilter_i8_sub_lists(uint64_t nq, uint64_t span);
 bool prefilter_rb_supports(const vsag_amd_store* s);
 size_t prefilter_rb_scratch_bytes(const vsag_amd_store* s, uint64_t nq);
@@ -876,7 +877,7 @@ carve_scan(Carver& c, const CallPlan& cp, uint64_t nq, uint32_t k, ScanBuffers* 
     b->partial = c.take<uint64_t>(nq * cp.nslots * k);
     const uint64_t nq_pad8 = prefilter_i8_query_bytes(nq) / 256;  // whole workgroups of the int8 prefilter
     b->tau = c.take<float>(cp.contraction ? nq_pad8 : 0);
-    b->q8_u = c.take<float>(cp.int8 ? nq_pad8 : 0);
+    b->q8_u = c.take<float>(cp.int8 ? prefilter_i8_scalar_floats(nq) : 0);
     b->q8 = c.take<uint8_t>(cp.int8 ? prefilter_i8_query_bytes(nq) : (cp.rb ? cp.rb_scratch : 0));
     if (!cp.int8 && !cp.rb) {
         b->q8 = nullptr;
