@@ -354,7 +354,8 @@ struct PrefilterI8Args {
     uint32_t* cand;       // [query][2 groups][sub_cap]
     uint32_t* cand_cnt;   // [query][2 groups]; a count above sub_cap means the list overflowed
     uint32_t sub_cap;
-    uint32_t groups;      // grid x; stage g of the span (kI8StageTiles tiles) is walked by group g % groups
+    uint32_t groups;      // stage g of the span (kI8StageTiles tiles) is walked by group g % groups
+    uint32_t qgroups;     // groups of kI8Group queries; the grid is groups x qgroups workgroups in one dimension
 };
 
 constexpr int kI8StageTiles = 2;  // storage tiles per LDS stage (one barrier per stage)
@@ -389,7 +390,19 @@ prefilter_i8_kernel(PrefilterI8Args p) {
     const uint32_t wave = tid >> 6;
     const uint32_t half = lane >> 5;
     const uint32_t l32 = lane & 31;
-    const uint64_t q_base = (static_cast<uint64_t>(blockIdx.y) * 4 + wave) * kWave;
+    // Workgroups are handed to the eight XCDs (each with its own L2) in turn.  All query groups that walk the same
+    // stages are made neighbours on one XCD, so that a tile is fetched into that L2 once and found there by the
+    // others: the fabric carries the codes once instead of once per query group.
+    uint32_t gx, gy;
+    if ((p.groups & 7U) == 0) {
+        const uint32_t xcd = blockIdx.x & 7U, local = blockIdx.x >> 3;
+        gy = local % p.qgroups;
+        gx = (local / p.qgroups) * 8 + xcd;
+    } else {
+        gx = blockIdx.x % p.groups;
+        gy = blockIdx.x / p.groups;
+    }
+    const uint64_t q_base = (static_cast<uint64_t>(gy) * 4 + wave) * kWave;
     const bool active = q_base < p.nq;  // the query table is padded to whole workgroups
     const uint64_t span = p.tile_end - p.tile_begin;
     const uint64_t nstages = (span + kI8StageTiles - 1) / kI8StageTiles;
@@ -415,9 +428,9 @@ prefilter_i8_kernel(PrefilterI8Args p) {
         }
         uq[j] = TEST == kI8TestFma ? p.u[q] : 0.0F;
         tau[j] = p.tau[q];
-        my_list[j] = p.cand + ((q < p.nq ? q : 0) * 2 * p.groups + 2 * blockIdx.x + half) * p.sub_cap;
+        my_list[j] = p.cand + ((q < p.nq ? q : 0) * 2 * p.groups + 2 * gx + half) * p.sub_cap;
     }
-    const float ginv = TEST == kI8TestIntTerm ? p.ginv[blockIdx.y] : 0.0F;
+    const float ginv = TEST == kI8TestIntTerm ? p.ginv[gy] : 0.0F;
 
     // Staging: wave w copies granules w and w + 4 of each tile of the stage, a lane per code.
     uint4 regs[kI8StageTiles][2];
@@ -486,7 +499,7 @@ prefilter_i8_kernel(PrefilterI8Args p) {
     // The grid never has more columns than there are stages, so the first stage exists.  Fetching it without a
     // condition also lets every load issued so far (the query operands) complete here, once, instead of being
     // waited for inside the loop, where that wait would hold up the prefetch of the next stage.
-    uint64_t sg = blockIdx.x;
+    uint64_t sg = gx;
     fetch(sg);
     park(stage[0]);
     __syncthreads();
@@ -558,23 +571,26 @@ prefilter_i8_kernel(PrefilterI8Args p) {
                     multiply(b + 1, hi[(b + 1) & 1], lo[(b + 1) & 1]);
                 }
                 // Nearly nothing passes.  The sixteen elements of a lane are reduced to their best one with
-                // three-operand max / min instructions (three vector instructions per two elements, none of them
-                // writing a scalar register), and one compare decides whether the block needs a second look.
+                // three-operand max / min instructions (none of them writing a scalar register) -- four at a time, so
+                // that a block with a hit finds it group by group -- and one compare decides whether the block needs a
+                // second look.
                 bool hit;
+                float gbest_f[4];
+                int32_t gbest_i[4];
                 if constexpr (TEST == kI8TestFma) {
-                    float best = __builtin_inff();
 #pragma unroll
-                    for (int e = 0; e < 16; e += 2) {
-                        best = fminf(fminf(best, judged_fma(b, e)), judged_fma(b, e + 1));
+                    for (int g = 0; g < 4; ++g) {
+                        gbest_f[g] = fminf(fminf(fminf(judged_fma(b, 4 * g), judged_fma(b, 4 * g + 1)), judged_fma(b, 4 * g + 2)),
+                                           judged_fma(b, 4 * g + 3));
                     }
-                    hit = best <= __uint_as_float(tau[j]);
+                    hit = fminf(fminf(fminf(gbest_f[0], gbest_f[1]), gbest_f[2]), gbest_f[3]) <= __uint_as_float(tau[j]);
                 } else {
-                    int32_t best = static_cast<int32_t>(0x80000000U);
 #pragma unroll
-                    for (int e = 0; e < 16; e += 2) {
-                        best = max(max(best, judged_int(b, e)), judged_int(b, e + 1));
+                    for (int g = 0; g < 4; ++g) {
+                        gbest_i[g] = max(max(max(judged_int(b, 4 * g), judged_int(b, 4 * g + 1)), judged_int(b, 4 * g + 2)),
+                                         judged_int(b, 4 * g + 3));
                     }
-                    hit = best >= static_cast<int32_t>(tau[j]);
+                    hit = max(max(max(gbest_i[0], gbest_i[1]), gbest_i[2]), gbest_i[3]) >= static_cast<int32_t>(tau[j]);
                 }
                 const uint64_t any = __ballot(hit);
                 if (b + 1 < kBlocks) {
@@ -586,28 +602,40 @@ prefilter_i8_kernel(PrefilterI8Args p) {
 #pragma unroll
                     for (int m = 0; m < 8; ++m) {
                         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x002, TEST == kI8TestFma ? 7 : 3, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, TEST == kI8TestFma ? 8 : 4, 0);
                     }
                 }
                 if (any != 0) {
-                    // Some lane has an element that passes: judge the elements one by one (the accumulators of this
-                    // block are not touched before the next block has been judged) and let the lanes under each
-                    // element's mask append.
+                    // Some lane has an element that passes: find the groups of four with a hit, judge their elements
+                    // one by one (the accumulators of this block are not touched before the next block has been
+                    // judged) and let the lanes under each element's mask append.
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) {
-                        bool pass;
+                    for (int g = 0; g < 4; ++g) {
+                        bool ghit;
                         if constexpr (TEST == kI8TestFma) {
-                            pass = judged_fma(b, e) <= __uint_as_float(tau[j]);
+                            ghit = gbest_f[g] <= __uint_as_float(tau[j]);
                         } else {
-                            pass = judged_int(b, e) >= static_cast<int32_t>(tau[j]);
+                            ghit = gbest_i[g] >= static_cast<int32_t>(tau[j]);
                         }
-                        if (__ballot(pass) != 0) {
-                            const uint64_t slot = slot0 + 32 * r + 8 * (e >> 2) + 4 * half + (e & 3);
-                            if (pass && slot < p.n) {
-                                if (ncand[j] < p.sub_cap) {
-                                    my_list[j][ncand[j]] = static_cast<uint32_t>(slot);
+                        if (__ballot(ghit) == 0) {
+                            continue;
+                        }
+#pragma unroll
+                        for (int e = 4 * g; e < 4 * g + 4; ++e) {
+                            bool pass;
+                            if constexpr (TEST == kI8TestFma) {
+                                pass = judged_fma(b, e) <= __uint_as_float(tau[j]);
+                            } else {
+                                pass = judged_int(b, e) >= static_cast<int32_t>(tau[j]);
+                            }
+                            if (__ballot(pass) != 0) {
+                                const uint64_t slot = slot0 + 32 * r + 8 * (e >> 2) + 4 * half + (e & 3);
+                                if (pass && slot < p.n) {
+                                    if (ncand[j] < p.sub_cap) {
+                                        my_list[j][ncand[j]] = static_cast<uint32_t>(slot);
+                                    }
+                                    ++ncand[j];
                                 }
-                                ++ncand[j];
                             }
                         }
                     }
@@ -625,7 +653,7 @@ prefilter_i8_kernel(PrefilterI8Args p) {
         for (int j = 0; j < 2; ++j) {
             const uint64_t q = q_base + 32 * j + l32;
             if (q < p.nq) {
-                p.cand_cnt[q * 2 * p.groups + 2 * blockIdx.x + half] = ncand[j];
+                p.cand_cnt[q * 2 * p.groups + 2 * gx + half] = ncand[j];
             }
         }
     }
@@ -657,9 +685,27 @@ prefilter_i8_scalar_floats(uint64_t nq) {
 uint32_t
 prefilter_i8_sub_lists(uint64_t nq, uint64_t span) {
     const uint64_t qgroups = div_up(nq, static_cast<uint64_t>(kI8Group));
-    // Two workgroups fit a compute unit; just under four full rounds of them (never a nearly empty last round).
-    uint64_t groups = static_cast<uint64_t>(device_cu_count()) * 8 / qgroups;
-    groups = std::max<uint64_t>(1, std::min<uint64_t>(groups, div_up(span, static_cast<uint64_t>(kI8StageTiles))));
+    // Two workgroups fit a compute unit.  The workgroups of a launch take about equally long, so they run in rounds of
+    // 2 x compute units: the number of columns is the multiple of eight (whole turns of the XCDs, see the kernel's
+    // workgroup mapping) between six and twelve rounds that leaves the last round fullest (few rounds: the slowest
+    // workgroup of the last one is a larger share of the launch; many: every workgroup loads its queries anew).
+    constexpr uint64_t rounds_lo = 6, rounds_hi = 12;
+    const uint64_t per_round = static_cast<uint64_t>(device_cu_count()) * 2;
+    const uint64_t stages = div_up(span, static_cast<uint64_t>(kI8StageTiles));
+    uint64_t groups = std::max<uint64_t>(1, std::min<uint64_t>(per_round * rounds_lo / qgroups, stages));
+    if (groups >= 8) {
+        uint64_t best = groups / 8 * 8;
+        double best_fill = 0.0;
+        for (uint64_t g = best; g <= stages && g * qgroups <= per_round * rounds_hi; g += 8) {
+            const uint64_t rem = g * qgroups % per_round;
+            const double fill = rem == 0 ? 1.0 : static_cast<double>(rem) / static_cast<double>(per_round);
+            if (fill > best_fill + 1e-9) {
+                best_fill = fill;
+                best = g;
+            }
+        }
+        groups = best;
+    }
     return static_cast<uint32_t>(2 * groups);
 }
 
@@ -736,7 +782,8 @@ launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride
     p.sub_cap = sub_cap;
     p.groups = sub_lists / 2;
     VA_CHECK_ARG(sub_lists == prefilter_i8_sub_lists(nq, tile_end - tile_begin), "candidate lists do not match the grid");
-    dim3 grid(p.groups, static_cast<uint32_t>(nq_pad / kI8Group));
+    p.qgroups = static_cast<uint32_t>(nq_pad / kI8Group);
+    dim3 grid(p.groups * p.qgroups);
     timing_begin(st);
     if (nibbles) {
         hipLaunchKernelGGL((prefilter_i8_kernel<kI8TestFma, true>), grid, dim3(256), 0, st, p);
