@@ -163,8 +163,38 @@ VSAG_AMD_API int vsag_amd_store_append(vsag_amd_store_t* store, const uint8_t* c
  * previous content. */
 VSAG_AMD_API int vsag_amd_store_set_lists(vsag_amd_store_t* store, const uint8_t* codes_dev, const int32_t* labels_dev,
                              uint64_t n, uint32_t nlist, void* stream);
+/* IVF::Add on a filled index (ivf.cpp:590-724, BucketDataCell::InsertVector, bucket_datacell.h:670-709): n more codes
+ * (reference byte layout; source row r gets inner id size + r) go behind the codes their lists already hold, in input
+ * order.  Lists have some room behind their last tile; when one outgrows it, all lists move once to a layout with a
+ * quarter more room.  residual_bias_dev: per source row, for stores with residual centroids and the l2 metric
+ * (vsag_amd_residual_bias), else NULL.  Blocking. */
+VSAG_AMD_API int vsag_amd_store_append_lists(vsag_amd_store_t* store, const uint8_t* codes_dev, const int32_t* labels_dev,
+                                const float* residual_bias_dev, uint64_t n, void* stream);
+
+/* use_residual of BucketDataCell (bucket_datacell.h:527-572,594-639): the lists hold codes of x - c, c the centroid of
+ * the list (x normalised first for cosine), and a scan puts every distance right with the slot's bias and <q, c>.
+ * vsag_amd_store_set_residual copies the nlist x dim centroids into an empty store (before vsag_amd_store_set_lists with
+ * n = 0 and vsag_amd_store_append_lists); vsag_amd_residual_rows writes x_i - c[labels_i]; vsag_amd_residual_bias
+ * decodes the codes (DecodeOneImpl of fp32 / sq8 / sq4 / sq8_uniform / sq4_uniform) into decoded_dev (n x dim floats of
+ * scratch) and writes -2 <c, decoded> - <c, c> per row (encode_vector, bucket_datacell.h:626-636; l2 only). */
+VSAG_AMD_API int vsag_amd_store_set_residual(vsag_amd_store_t* store, const float* centroids_dev, uint32_t nlist, void* stream);
+VSAG_AMD_API int vsag_amd_residual_rows(const float* x_dev, uint64_t n, uint32_t dim, int metric, const int32_t* labels_dev,
+                           const float* centroids_dev, float* out_dev, void* stream);
+VSAG_AMD_API int vsag_amd_residual_bias(const vsag_amd_store_t* store, const uint8_t* codes_dev, uint64_t n,
+                           const int32_t* labels_dev, const float* centroids_dev, float* bias_dev, float* decoded_dev,
+                           void* stream);
+
 /* Sizes of the posting lists (nlist values) copied to host memory. */
 VSAG_AMD_API int vsag_amd_store_list_sizes(const vsag_amd_store_t* store, uint32_t* sizes, uint32_t nlist);
+
+/* FlattenDataCell::Query / BucketDataCell::QueryOneById (flatten_datacell.h:334-440, bucket_datacell.h:353-383; what
+ * Index::CalDistanceById and a reorder over quantised codes call): distance of query i to each of its own `count`
+ * codes named by inner id (ids_dev: nq x count; VSAG_AMD_INVALID_ID or an id the store does not hold gives -1).
+ * Same arithmetic as the scans.  nq <= 65535. */
+VSAG_AMD_API size_t vsag_amd_store_distances_workspace_bytes(const vsag_amd_store_t* store, uint64_t nq);
+VSAG_AMD_API int vsag_amd_store_distances(const vsag_amd_store_t* store, const float* queries_dev, uint64_t nq,
+                             const uint32_t* ids_dev, uint32_t count, float* dists_dev, void* workspace_dev,
+                             size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------ flat scan + top-k -------- */
 

@@ -1295,6 +1295,101 @@ orc_ivf_scan(int kind, int metric, uint64_t dim, const uint8_t* codes, uint64_t 
     }
 }
 
+// ---- use_residual of BucketDataCell ------------------------------------------------------------------------
+// Train / encode_vector (bucket_datacell.h:594-625): the quantizer sees x - c of the row's bucket, x normalised first
+// for cosine.
+ORC_API void
+orc_residual_rows(const float* x, uint64_t n, uint64_t dim, int metric, const int32_t* labels, const float* cent,
+                  float* out) {
+    std::vector<float> tmp(dim);
+    for (uint64_t i = 0; i < n; ++i) {
+        const float* cur = x + i * dim;
+        if (metric == kCosine) {
+            normalize(cur, tmp.data(), dim);
+            cur = tmp.data();
+        }
+        const float* c = cent + static_cast<uint64_t>(labels[i]) * dim;
+        for (uint64_t d = 0; d < dim; ++d) {
+            out[i * dim + d] = cur[d] - c[d];
+        }
+    }
+}
+
+// DecodeOneImpl of the uniform quantizers (sq4_uniform_quantizer.cpp:160-170, sq8_uniform_quantizer.cpp:140-145):
+// double arithmetic, rounded to float on the store.
+ORC_API void
+orc_squ_decode(const uint8_t* codes, uint64_t n, uint64_t dim, int bits, int metric, float lb, float diff, float* data) {
+    UniformLayout l = uniform_layout(dim, bits, metric);
+    for (uint64_t i = 0; i < n; ++i) {
+        const uint8_t* c = codes + i * l.code_size;
+        for (uint64_t d = 0; d < dim; ++d) {
+            if (bits == 4) {
+                int v = (d & 1) != 0 ? (c[d >> 1] & 0xf0) >> 4 : (c[d >> 1] & 0x0f);
+                data[i * dim + d] = v / 15.0 * diff + lb;
+            } else {
+                data[i * dim + d] = c[d] / 255.0 * diff + lb;
+            }
+        }
+    }
+}
+
+// encode_vector, l2 (bucket_datacell.h:626-636): -2 <c, decoded> - <c, c>.
+ORC_API void
+orc_residual_bias(const float* decoded, uint64_t n, uint64_t dim, const int32_t* labels, const float* cent, float* bias) {
+    for (uint64_t i = 0; i < n; ++i) {
+        const float* c = cent + static_cast<uint64_t>(labels[i]) * dim;
+        bias[i] = -2 * fp32_ip(c, decoded + i * dim, dim) - fp32_ip(c, c, dim);
+    }
+}
+
+// IVF::search<KNN> over residual lists: ScanBucketById (bucket_datacell.h:527-572) takes the list's residual bias
+// (l2) and <q, c> (twice for l2) off every distance; the computer's query is the raw query, normalised for cosine
+// (FactoryComputer, :574-592).  `queries` holds the processed queries as in orc_ivf_scan, `raw_queries` the float
+// rows the <q, c> terms are formed from, `bias` one value per posting position (null: zeros).
+ORC_API void
+orc_ivf_scan_residual(int kind, int metric, uint64_t dim, const uint8_t* codes, uint64_t code_size, const float* lb,
+                      const float* diff, int query_bits, const uint64_t* offsets, const uint32_t* order,
+                      const uint8_t* queries, uint64_t nq, uint64_t query_stride, const float* raw_queries,
+                      const float* cent, const float* bias, const int32_t* buckets, uint64_t nprobe, uint64_t kcand,
+                      uint32_t* out_ids, float* out_dists) {
+    Store s{kind, metric, dim, code_size, codes, lb, diff, query_bits};
+    RabitqLayout rl = rabitq_layout(dim, metric, query_bits ? query_bits : 4);
+#pragma omp parallel for schedule(dynamic)
+    for (int64_t qi = 0; qi < static_cast<int64_t>(nq); ++qi) {
+        StrictMaxHeap h(kcand);
+        const uint8_t* q = queries + qi * query_stride;
+        std::vector<float> rq(dim);
+        if (metric == kCosine) {
+            normalize(raw_queries + qi * dim, rq.data(), dim);
+        } else {
+            std::memcpy(rq.data(), raw_queries + qi * dim, dim * sizeof(float));
+        }
+        for (uint64_t p = 0; p < nprobe; ++p) {
+            int32_t b = buckets[qi * nprobe + p];
+            if (b < 0) {
+                continue;
+            }
+            float ip_distance = fp32_ip(rq.data(), cent + static_cast<uint64_t>(b) * dim, dim);
+            if (metric == kL2) {
+                ip_distance *= 2;
+            }
+            for (uint64_t pos = offsets[b]; pos < offsets[b + 1]; ++pos) {
+                float d = store_dist(s, &rl, q, codes + pos * code_size);
+                if (metric == kL2 && bias != nullptr) {
+                    d = d - bias[pos];
+                }
+                d -= ip_distance;
+                h.push(d, order[pos]);
+            }
+        }
+        uint64_t cnt = h.drain(out_ids + qi * kcand, out_dists + qi * kcand);
+        for (uint64_t j = cnt; j < kcand; ++j) {
+            out_ids[qi * kcand + j] = 0xFFFFFFFFU;
+            out_dists[qi * kcand + j] = std::numeric_limits<float>::infinity();
+        }
+    }
+}
+
 // FlattenReorder::Reorder (impl/reorder/flatten_reorder.cpp:52-114): exact fp32 distance of every
 // candidate (in candidate order) into a strict-`<` heap of size k, packed ascending.
 ORC_API void

@@ -248,6 +248,51 @@ def ivf_scan(kind, metric, d, codes_posting, offsets, order, queries, buckets, k
     return ids, dists
 
 
+def residual_rows(x, labels, cent, metric=L2):
+    x = f32(x)
+    n, d = x.shape
+    out = np.empty((n, d), np.float32)
+    lib().orc_residual_rows(_p(x), u64(n), u64(d), metric, _p(np.ascontiguousarray(labels, np.int32)), _p(f32(cent)),
+                            _p(out))
+    return out
+
+
+def squ_decode(codes, d, bits, lb, diff, metric=L2):
+    codes = np.ascontiguousarray(codes)
+    n = codes.shape[0]
+    out = np.empty((n, d), np.float32)
+    lib().orc_squ_decode(_p(codes), u64(n), u64(d), bits, metric, C.c_float(lb), C.c_float(diff), _p(out))
+    return out
+
+
+def residual_bias(decoded, labels, cent):
+    decoded = f32(decoded)
+    n, d = decoded.shape
+    out = np.empty(n, np.float32)
+    lib().orc_residual_bias(_p(decoded), u64(n), u64(d), _p(np.ascontiguousarray(labels, np.int32)), _p(f32(cent)), _p(out))
+    return out
+
+
+def ivf_scan_residual(kind, metric, d, codes_posting, offsets, order, queries, raw_queries, cent, bias_posting, buckets,
+                      kcand, lb=None, diff=None, qbits=4):
+    codes = np.ascontiguousarray(codes_posting)
+    queries = np.ascontiguousarray(queries)
+    buckets = np.ascontiguousarray(buckets, np.int32)
+    cs = codes.shape[1] * codes.itemsize
+    nq, nprobe = buckets.shape
+    qstride = queries.shape[1] * queries.itemsize
+    ids = np.empty((nq, kcand), np.uint32)
+    dists = np.empty((nq, kcand), np.float32)
+    lbp = _p(f32(np.atleast_1d(lb))) if lb is not None else None
+    dfp = _p(f32(np.atleast_1d(diff))) if diff is not None else None
+    bp = _p(f32(bias_posting)) if bias_posting is not None else None
+    lib().orc_ivf_scan_residual(kind, metric, u64(d), _p(codes), u64(cs), lbp, dfp, qbits,
+                                _p(np.ascontiguousarray(offsets, np.uint64)), _p(np.ascontiguousarray(order, np.uint32)),
+                                _p(queries), u64(nq), u64(qstride), _p(f32(raw_queries)), _p(f32(cent)), bp, _p(buckets),
+                                u64(nprobe), u64(kcand), _p(ids), _p(dists))
+    return ids, dists
+
+
 def rerank_fp32(raw, queries, cand, k, metric=L2):
     raw = f32(raw)
     queries = f32(queries)

@@ -110,3 +110,171 @@ def test_rerank_matches_oracle(lib, metric):
     ri, rd = orc.rerank_fp32(x, q, cand, k, metric)
     assert_topk_close(gi, gd, ri, rd, atol=2e-6, label="rerank")
     assert np.all(gi[0, 5:] == 0xFFFFFFFF)
+
+
+def _append_lists(lib, store, codes, labels, bias=None):
+    cbuf, lbuf = dev(np.ascontiguousarray(codes)), dev(np.ascontiguousarray(labels, np.int32))
+    bbuf = dev(np.ascontiguousarray(bias, np.float32)) if bias is not None else None
+    capi.check(lib.load_library().vsag_amd_store_append_lists(store.handle, cbuf.ptr, lbuf.ptr,
+                                                             bbuf.ptr if bbuf is not None else None, codes.shape[0], None))
+    for b in (cbuf, lbuf, bbuf):
+        if b is not None:
+            b.free()
+
+
+@pytest.mark.parametrize("kind", ["sq8", "sq4u", "fp32"])
+def test_lists_appended_in_pieces_equal_one_fill(lib, kind):
+    """IVF::Add on a filled index (ivf.cpp:590-724): codes appended to their lists piece by piece -- the first pieces fit
+    the room of the first fill's last tiles, later ones make every list move -- give the lists one fill of everything
+    gives: same sizes, and the same scan results bit for bit (in-list order = insertion order either way)."""
+    rng = np.random.default_rng(77)
+    n, d, nlist, nq, nprobe, kcand = 9000, 64, 37, 25, 9, 50
+    x, q, cent, labels = _ivf_case(rng, n, d, nlist, nq)
+    labels[labels == 5] = 6  # an empty list
+    if kind == "sq8":
+        lb, diff = orc.sq_train(x, 8)
+        codes = orc.sq_encode(x, 8, lb, diff)
+        make = lambda: Store(capi.KIND_SQ8, orc.L2, d, lb=lb, diff=diff)
+    elif kind == "sq4u":
+        l, dd = orc.sq_train_uniform(x, 4, orc.L2, mode=3)
+        codes = orc.squ_encode(x, 4, l, dd, orc.L2)
+        make = lambda: Store(capi.KIND_SQ4_UNIFORM, orc.L2, d, bounds=[l, dd])
+    else:
+        codes = x.view(np.uint8).reshape(n, 4 * d)
+        make = lambda: Store(capi.KIND_FP32, orc.L2, d)
+    whole = make()
+    whole.set_lists(codes, labels, nlist)
+    grown = make()
+    cuts = [0, 3000, 3001, 3010, 3500, 6000, 9000]
+    grown.set_lists(codes[:cuts[1]], labels[:cuts[1]], nlist)
+    for s, e in zip(cuts[1:-1], cuts[2:]):
+        _append_lists(lib, grown, codes[s:e], labels[s:e])
+    assert grown.size() == n
+    L = lib.load_library()
+    sa, sb = np.zeros(nlist, np.uint32), np.zeros(nlist, np.uint32)
+    capi.check(L.vsag_amd_store_list_sizes(whole.handle, sa.ctypes.data, nlist))
+    capi.check(L.vsag_amd_store_list_sizes(grown.handle, sb.ctypes.data, nlist))
+    assert np.array_equal(sa, sb) and sa[5] == 0
+    routed, _ = orc.ivf_route(cent, q, nprobe)
+    i1, d1 = whole.ivf_scan(q, routed, kcand)
+    i2, d2 = grown.ivf_scan(q, routed, kcand)
+    assert np.array_equal(i1, i2) and np.array_equal(d1.view(np.uint32), d2.view(np.uint32))
+    # a store that starts empty and is only ever appended to
+    empty = make()
+    empty.set_lists(codes[:0], labels[:0], nlist)
+    assert empty.ivf_scan(q, routed, kcand)[0].max() == 0xFFFFFFFF
+    _append_lists(lib, empty, codes[:4000], labels[:4000])
+    _append_lists(lib, empty, codes[4000:], labels[4000:])
+    i3, d3 = empty.ivf_scan(q, routed, kcand)
+    assert np.array_equal(i1, i3) and np.array_equal(d1.view(np.uint32), d3.view(np.uint32))
+    for st in (whole, grown, empty):
+        st.destroy()
+
+
+def _store_distances(lib, store, q, ids):
+    L = lib.load_library()
+    nq, count = ids.shape
+    qb, ib = dev(np.ascontiguousarray(q, np.float32)), dev(np.ascontiguousarray(ids, np.uint32))
+    out = capi.DeviceBuffer(nq * count * 4)
+    wsb = L.vsag_amd_store_distances_workspace_bytes(store.handle, nq)
+    ws = capi.DeviceBuffer(wsb)
+    capi.check(L.vsag_amd_store_distances(store.handle, qb.ptr, nq, ib.ptr, count, out.ptr, ws.ptr, wsb, None))
+    res = out.to_numpy(np.float32, (nq, count))
+    for b in (qb, ib, out, ws):
+        b.free()
+    return res
+
+
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP])
+def test_distances_by_inner_id(lib, metric):
+    """CalDistanceById's core: the distance of a query to codes named by inner id equals the scan's distance to the
+    same code, on a flat store and on posting lists; unknown ids give -1."""
+    rng = np.random.default_rng(31)
+    n, d, nlist, nq, count = 5000, 96, 23, 6, 150
+    x, q, cent, labels = _ivf_case(rng, n, d, nlist, nq)
+    lb, diff = orc.sq_train(x, 8, metric)
+    codes = orc.sq_encode(x, 8, lb, diff, metric)
+    ids = rng.integers(0, n, (nq, count)).astype(np.uint32)
+    ids[1, 3] = 0xFFFFFFFF
+    ids[2, 7] = n + 5
+    expect = orc.flat_dists(orc.SQ8, metric, d, codes, q, lb=lb, diff=diff)
+    want = np.take_along_axis(expect, np.minimum(ids, n - 1).astype(np.int64), 1)
+    want[1, 3] = want[2, 7] = -1.0
+    flat = Store(capi.KIND_SQ8, metric, d, lb=lb, diff=diff)
+    flat.append(codes)
+    lists = Store(capi.KIND_SQ8, metric, d, lb=lb, diff=diff)
+    lists.set_lists(codes[:3000], labels[:3000], nlist)
+    _append_lists(lib, lists, codes[3000:], labels[3000:])
+    for st in (flat, lists):
+        got = _store_distances(lib, st, q, ids)
+        np.testing.assert_allclose(got, want, rtol=1e-4, atol=2e-6)
+        st.destroy()
+
+
+@pytest.mark.parametrize("metric,mname", [(orc.L2, "l2"), (orc.IP, "ip"), (orc.COSINE, "cosine")])
+@pytest.mark.parametrize("kind", ["fp32", "sq8", "sq4u"])
+def test_residual_lists_match_oracle(lib, kind, metric, mname):
+    """use_residual (bucket_datacell.h:527-572,594-639): codes of x - c scanned with the list's bias and <q, c> taken
+    off, against the checker's restatement; with fp32 codes that is the plain distance to x again."""
+    if kind == "fp32" and metric == orc.COSINE:
+        pytest.skip("the fp32 quantizer normalises what it stores under cosine: residuals lose their length")
+    L = lib.load_library()
+    rng = np.random.default_rng(41 + metric)
+    n, d, nlist, nq, nprobe, kcand = 6000, 48, 29, 19, 7, 40
+    x, q, cent, labels = _ivf_case(rng, n, d, nlist, nq)
+    x = (x - 0.3).astype(np.float32)
+    q = (q - 0.3).astype(np.float32)
+    res = orc.residual_rows(x, labels, cent, metric)
+    xb, lb_dev, cb = dev(x), dev(labels.astype(np.int32)), dev(cent)
+    rb = capi.DeviceBuffer(n * d * 4)
+    capi.check(L.vsag_amd_residual_rows(xb.ptr, n, d, metric, lb_dev.ptr, cb.ptr, rb.ptr, None))
+    assert np.array_equal(rb.to_numpy(np.float32, (n, d)).view(np.uint32), res.view(np.uint32))
+    qproc = q if metric != orc.COSINE else (q / np.linalg.norm(q, axis=1, keepdims=True)).astype(np.float32)
+    lb = diff = None
+    if kind == "fp32":
+        codes = res.view(np.uint8).reshape(n, 4 * d)
+        dec = res
+        st = Store(capi.KIND_FP32, metric, d)
+        okind = orc.FP32
+    elif kind == "sq8":
+        lb, diff = orc.sq_train(res, 8, metric)
+        codes = orc.sq_encode(res, 8, lb, diff, metric)
+        dec = orc.sq_decode(codes, d, 8, lb, diff)
+        st = Store(capi.KIND_SQ8, metric, d, lb=lb, diff=diff)
+        okind = orc.SQ8
+    else:
+        l, dd = orc.sq_train_uniform(res, 4, metric, mode=3)
+        codes = orc.squ_encode(res, 4, l, dd, metric)
+        dec = orc.squ_decode(codes, d, 4, l, dd, metric)
+        lb, diff = l, dd
+        st = Store(capi.KIND_SQ4_UNIFORM, metric, d, bounds=[l, dd])
+        okind = orc.SQ4U
+        qproc = orc.squ_encode(q, 4, l, dd, metric)
+    bias = orc.residual_bias(dec, labels, cent) if metric == orc.L2 else None
+    capi.check(L.vsag_amd_store_set_residual(st.handle, cb.ptr, nlist, None))
+    st.set_lists(codes[:0], labels[:0], nlist)
+    if metric == orc.L2:
+        cdev, bdev, scratch = dev(codes), capi.DeviceBuffer(n * 4), capi.DeviceBuffer(n * d * 4)
+        capi.check(L.vsag_amd_residual_bias(st.handle, cdev.ptr, n, lb_dev.ptr, cb.ptr, bdev.ptr, scratch.ptr, None))
+        gbias = bdev.to_numpy(np.float32, (n,))
+        np.testing.assert_allclose(gbias, bias, rtol=1e-5, atol=1e-5)
+        for b in (cdev, bdev, scratch):
+            b.free()
+    _append_lists(lib, st, codes[:2500], labels[:2500], None if bias is None else bias[:2500])
+    _append_lists(lib, st, codes[2500:], labels[2500:], None if bias is None else bias[2500:])
+    offsets, order = orc.ivf_build_lists(labels, nlist)
+    routed, _ = orc.ivf_route(cent, q, nprobe)
+    ids, ds = st.ivf_scan(q, routed, kcand)
+    rids, rds = orc.ivf_scan_residual(okind, metric, d, codes[order], offsets, order, qproc, q, cent,
+                                      None if bias is None else bias[order], routed, kcand, lb=lb, diff=diff)
+    assert_topk_close(ids, ds, rids, rds, rtol=2e-4, atol=2e-5, tie_rtol=2e-4, label="residual %s %s" % (kind, mname))
+    if kind == "fp32":
+        # closed form: the residual scan of fp32 codes is the plain distance to the original vectors
+        plain = Store(capi.KIND_FP32, metric, d)
+        plain.set_lists(x.view(np.uint8).reshape(n, 4 * d), labels, nlist)
+        pi, pd = plain.ivf_scan(q, routed, kcand)
+        assert_topk_close(ids, ds, pi, pd, rtol=2e-4, atol=5e-5, tie_rtol=5e-4, label="residual fp32 closed form")
+        plain.destroy()
+    for b in (xb, lb_dev, cb, rb):
+        b.free()
+    st.destroy()

@@ -545,3 +545,45 @@ def test_ivf_probing_every_list_equals_the_flat_scan():
     assert np.array_equal(b, np.argsort(dc, 1, kind="stable")[:, :4].astype(np.int32))
     rids, rds = orc.rerank_fp32(x, q, ids, 5)
     assert np.array_equal(rds, fds[:, :5])
+
+
+def test_residual_scan_closed_forms():
+    """use_residual: with fp32 codes of x - c the corrected distance is the plain distance to x (l2: |q - x|^2, ip:
+    1 - <q, x>); with sq8 codes it is the distance to c + decoded.  A dropped bias, a missing factor 2 or a wrong sign
+    of <q, c> is off by the size of |c|^2."""
+    rng = np.random.default_rng(12)
+    n, d, nlist, nq, k = 900, 24, 7, 5, 30
+    x = (rng.random((n, d), dtype=np.float32) - 0.2).astype(np.float32)
+    q = (rng.random((nq, d), dtype=np.float32) - 0.2).astype(np.float32)
+    cent = x[:nlist].copy() + 0.5
+    labels, _, _ = orc.kmeans_assign(x, cent)
+    offsets, order = orc.ivf_build_lists(labels, nlist)
+    buckets = np.tile(np.arange(nlist, dtype=np.int32), (nq, 1))
+    for metric in (orc.L2, orc.IP):
+        res = orc.residual_rows(x, labels, cent, metric)
+        assert np.array_equal(res, x - cent[labels])
+        bias = orc.residual_bias(res, labels, cent) if metric == orc.L2 else None
+        ids, ds = orc.ivf_scan_residual(orc.FP32, metric, d, res.view(np.uint8).reshape(n, 4 * d)[order], offsets, order, q,
+                                        q, cent, None if bias is None else bias[order], buckets, k)
+        x64, q64 = x.astype(np.float64), q.astype(np.float64)
+        full = ((q64[:, None, :] - x64[None]) ** 2).sum(2) if metric == orc.L2 else 1.0 - q64 @ x64.T
+        want = np.sort(full, axis=1)[:, :k]
+        assert np.allclose(ds, want, rtol=1e-4, atol=2e-5)
+        # sq8 codes of the residual: distance to c + decoded
+        lb, diff = orc.sq_train(res, 8, metric)
+        codes = orc.sq_encode(res, 8, lb, diff, metric)
+        dec = orc.sq_decode(codes, d, 8, lb, diff)
+        bias = orc.residual_bias(dec, labels, cent) if metric == orc.L2 else None
+        ids, ds = orc.ivf_scan_residual(orc.SQ8, metric, d, codes[order], offsets, order, q, q, cent,
+                                        None if bias is None else bias[order], buckets, k, lb=lb, diff=diff)
+        y64 = (dec + cent[labels]).astype(np.float64)
+        full = ((q64[:, None, :] - y64[None]) ** 2).sum(2) if metric == orc.L2 else 1.0 - q64 @ y64.T
+        assert np.allclose(ds, np.sort(full, axis=1)[:, :k], rtol=1e-4, atol=5e-5)
+    # cosine normalises the row before the centroid comes off; uniform decode is lb + code / levels * diff
+    res = orc.residual_rows(x, labels, cent, orc.COSINE)
+    xn = x / np.linalg.norm(x, axis=1, keepdims=True)
+    assert np.allclose(res, xn - cent[labels], atol=1e-6)
+    l, dd = orc.sq_train_uniform(res, 4, orc.L2, mode=3)
+    c4 = orc.squ_encode(res, 4, l, dd, orc.L2)
+    raw = np.stack([(c4[:, i // 2] >> (4 * (i % 2))) & 15 for i in range(d)], 1)
+    assert np.allclose(orc.squ_decode(c4, d, 4, l, dd, orc.L2), l + raw / 15.0 * dd, atol=1e-6)

@@ -69,7 +69,13 @@ PROTOTYPES = {
     "vsag_amd_store_size": (_u64, [_vp]),
     "vsag_amd_store_append": (C.c_int, [_vp, _vp, _u64, _vp]),
     "vsag_amd_store_set_lists": (C.c_int, [_vp, _vp, _vp, _u64, _u32, _vp]),
+    "vsag_amd_store_append_lists": (C.c_int, [_vp, _vp, _vp, _vp, _u64, _vp]),
+    "vsag_amd_store_set_residual": (C.c_int, [_vp, _vp, _u32, _vp]),
+    "vsag_amd_residual_rows": (C.c_int, [_vp, _u64, _u32, _i32, _vp, _vp, _vp, _vp]),
+    "vsag_amd_residual_bias": (C.c_int, [_vp, _vp, _u64, _vp, _vp, _vp, _vp, _vp]),
     "vsag_amd_store_list_sizes": (C.c_int, [_vp, _vp, _u32]),
+    "vsag_amd_store_distances_workspace_bytes": (_sz, [_vp, _u64]),
+    "vsag_amd_store_distances": (C.c_int, [_vp, _vp, _u64, _vp, _u32, _vp, _vp, _sz, _vp]),
     "vsag_amd_flat_scan_workspace_bytes": (_sz, [_vp, _u64, _u32]),
     "vsag_amd_flat_scan_topk": (C.c_int, [_vp, _vp, _u64, _u32, _vp, _vp, _vp, _sz, _vp]),
     "vsag_amd_flat_scan_topk_ex": (C.c_int, [_vp, _vp, _u64, _u32, _vp, _vp, _vp, _vp, _sz, _vp]),

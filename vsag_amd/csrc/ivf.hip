@@ -48,6 +48,8 @@ int prepare_queries(const vsag_amd_store* s, const float* queries, uint64_t nq, 
 ScanArgs make_scan_args(const vsag_amd_store* s, const QueryLayout& ql, const uint32_t* qtab, const float* qmeta);
 void timing_begin(hipStream_t st);
 void timing_end(hipStream_t st);
+int launch_residual_terms(const vsag_amd_store* s, const float* queries, uint64_t nq, const int32_t* buckets, uint32_t nprobe,
+                          float* terms, hipStream_t st);
 int launch_merge_partials(const uint64_t* partial, const uint32_t* partial_cnt, const uint32_t* bound, uint32_t nslots,
                           uint32_t stride, uint32_t k, uint32_t S, uint64_t nq, uint32_t* ids, float* dists,
                           hipStream_t st);
@@ -149,7 +151,7 @@ offsets_kernel(const uint32_t* counts, const uint32_t* list_tile, uint32_t nlist
     uint32_t sp = 0, si = 0;
     for (uint32_t i = begin; i < end; ++i) {
         sp += counts[i];
-        si += list_items(counts[i], T, list_tile[i + 1] - list_tile[i], tiles_per_item, chunks_max);
+        si += list_items(counts[i], T, list_tile[2 * i + 1] - list_tile[2 * i], tiles_per_item, chunks_max);
     }
     uint32_t rp = sp, ri = si, all_pairs, all_items;
     block_exclusive_scan2(rp, ri, wave_sums, all_pairs, all_items);
@@ -161,7 +163,7 @@ offsets_kernel(const uint32_t* counts, const uint32_t* list_tile, uint32_t nlist
         pair_off[i] = rp;
         item_off[i] = ri;
         rp += counts[i];
-        ri += list_items(counts[i], T, list_tile[i + 1] - list_tile[i], tiles_per_item, chunks_max);
+        ri += list_items(counts[i], T, list_tile[2 * i + 1] - list_tile[2 * i], tiles_per_item, chunks_max);
     }
 }
 
@@ -210,7 +212,7 @@ regroup_small_kernel(const int32_t* buckets, uint64_t nq, uint32_t nprobe, const
     uint32_t sp = 0, si = 0;
     for (uint32_t i = begin; i < end; ++i) {
         sp += counts[i];
-        si += list_items(counts[i], T, list_tile[i + 1] - list_tile[i], tiles_per_item, chunks_max);
+        si += list_items(counts[i], T, list_tile[2 * i + 1] - list_tile[2 * i], tiles_per_item, chunks_max);
     }
     uint32_t rp = sp, ri = si, all_pairs, all_items;
     block_exclusive_scan2(rp, ri, wave_sums, all_pairs, all_items);
@@ -222,7 +224,7 @@ regroup_small_kernel(const int32_t* buckets, uint64_t nq, uint32_t nprobe, const
         pair_off[i] = rp;
         item_off[i] = ri;
         rp += counts[i];
-        ri += list_items(counts[i], T, list_tile[i + 1] - list_tile[i], tiles_per_item, chunks_max);
+        ri += list_items(counts[i], T, list_tile[2 * i + 1] - list_tile[2 * i], tiles_per_item, chunks_max);
     }
     __syncthreads();
     for (uint64_t i = threadIdx.x; i < npairs; i += blockDim.x) {
@@ -236,7 +238,7 @@ regroup_small_kernel(const int32_t* buckets, uint64_t nq, uint32_t nprobe, const
 
 struct IvfArgs {
     const uint32_t* ids;         // inner id per tile slot
-    const uint32_t* list_tile;   // nlist+1
+    const uint32_t* list_tile;   // 2 nlist: first tile and end of the used tiles of every list
     const uint32_t* pair_off;    // nlist+1
     const uint32_t* item_off;    // nlist+1
     const uint32_t* sorted_pair; // pair index (q * nprobe + p) grouped by list
@@ -260,6 +262,10 @@ struct IvfArgs {
     const uint32_t* direct_count;
     uint32_t direct_cap;
     const int32_t* buckets;      // direct mode: list of a pair
+    // Residual lists (bucket_datacell.h:553-566): the codes hold x - c of their list's centroid c, and a distance is
+    // put right by taking off the slot's bias (l2: -2 <c, decoded> - |c|^2) and the pair's term (<q, c>, twice for l2).
+    const float* res_bias;       // per slot, or null
+    const float* res_term;       // per pair (q * nprobe + p), or null: no residual
 };
 
 constexpr uint32_t kIvfSeedTiles = 4;
@@ -282,8 +288,8 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
         }
         pairs_src = as_const(v.direct);
         const int32_t bk = v.buckets[pairs_src[vi]];  // a real list: pairs without one are never queued
-        list_begin = as_const(v.list_tile)[bk];
-        list_end = as_const(v.list_tile)[bk + 1];
+        list_begin = as_const(v.list_tile)[2 * bk];
+        list_end = as_const(v.list_tile)[2 * bk + 1];
         local = item % v.chunks_max;
         pfirst = vi;
         plast = vi + 1;
@@ -311,8 +317,8 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
                 hi = mid;
             }
         }
-        list_begin = as_const(v.list_tile)[lo];
-        list_end = as_const(v.list_tile)[lo + 1];
+        list_begin = as_const(v.list_tile)[2 * lo];
+        list_end = as_const(v.list_tile)[2 * lo + 1];
         local = item - ioff[lo];
         pfirst = as_const(v.pair_off)[lo];
         plast = as_const(v.pair_off)[lo + 1];
@@ -369,6 +375,11 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
     wave_lds_fence();
 
     const QueryRows<T> qrows = query_rows<T>(a, qidx);
+    float rterm[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+        rterm[t] = v.res_term != nullptr && pair[t] != 0xFFFFFFFFU ? v.res_term[pair[t]] : 0.0F;
+    }
     constexpr int GROUP = GroupOf<T>::value;
     TileStream<GROUP> cur{a.tiles, lane, tbeg, tend, 1, 0, a.G};
     TileStream<GROUP> nxt = cur;
@@ -393,6 +404,13 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
         float d[T];
         finish_distances<KIND, METRIC, T>(a, qidx, slot, acc, d);
         acc_reset(acc);
+        if (v.res_term != nullptr) {
+            const float bias = v.res_bias != nullptr ? v.res_bias[slot] : 0.0F;
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                d[t] = (d[t] - bias) - rterm[t];
+            }
+        }
         const uint32_t id = v.ids[slot];
         const bool valid = id != VSAG_AMD_INVALID_ID && !denied(v.deny, id);
 #pragma unroll
@@ -684,6 +702,7 @@ struct IvfBuffers {
     uint32_t* gate;       // mfma: nq + 2 (flags, raised gates, their pairs)
     int32_t* tq;          // mfma: nq + 1
     uint32_t* gpairs;     // mfma: pairs of gated queries, kGatedPairsCap
+    float* res_term;      // residual lists: per pair
 };
 
 // Pairs of gated queries the direct fallback launch takes; more go through the per-list grouping.
@@ -735,6 +754,7 @@ plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, 
     // Large batches on sq4_uniform / L2 lists: the streaming kernel scans the nearest list of every query, the int8
     // matrix cores the other columns, into two private lists per (query, list) pair.
     p->mfma = !p->chunked && nprobe > 1 && scan_contraction_mode() >= 0 && ivf_i8_supports(s) &&
+              s->residual_centroids_dev == nullptr &&
               npairs * ivf_i8_lists_per_pair() * kcand * 8 <= (8ull << 30);
     if (p->mfma) {
         p->chunks_max = ivf_i8_lists_per_pair();
@@ -758,6 +778,7 @@ carve_ivf(Carver& c, const vsag_amd_store* s, const ScanPlanIvf& p, uint64_t nq,
     b->gate = c.take<uint32_t>(p.mfma ? nq + 2 : 0);
     b->gpairs = c.take<uint32_t>(p.mfma ? kGatedPairsCap : 0);
     b->tq = c.take<int32_t>(p.mfma ? nq + 1 : 0);
+    b->res_term = c.take<float>(s->residual_centroids_dev != nullptr ? p.npairs : 0);
     return c.used;
 }
 
@@ -865,6 +886,11 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
     v.seed = p.seeded ? b.seed : nullptr;
     v.partial = b.partial;
     v.partial_cnt = b.partial_cnt;
+    if (s->residual_centroids_dev != nullptr) {
+        VA_TRY(launch_residual_terms(s, queries_dev, nq, buckets_dev, nprobe, b.res_term, st));
+        v.res_term = b.res_term;
+        v.res_bias = s->residual_bias_dev;
+    }
 
     uint32_t waves = 4;
     while (waves > 1 && static_cast<size_t>(waves) * p.T * p.S * 8 > 65536) {

@@ -103,7 +103,7 @@ struct IvfI8Args {
     uint32_t G;                  // granules per code (<= 4)
     const uint32_t* meta;        // per slot: No as float bits
     const uint32_t* ids;         // inner id per tile slot
-    const uint32_t* list_tile;   // nlist + 1
+    const uint32_t* list_tile;   // 2 nlist: first tile and end of the used tiles of every list
     const uint32_t* pair_off;    // nlist + 1
     const uint32_t* item_off;    // nlist + 1: workgroups per list (256 pairs each), prefix sums
     const uint32_t* sorted_pair; // pair index (q * nprobe + p) grouped by list
@@ -153,7 +153,7 @@ ivf_i8_kernel(IvfI8Args p) {
     }
     const uint32_t b = lo_b;
     // Items of a list: (block of 256 pairs) x (tile chunk), chunk fastest.
-    const uint32_t list_begin = as_const(p.list_tile)[b], list_end = as_const(p.list_tile)[b + 1];
+    const uint32_t list_begin = as_const(p.list_tile)[2 * b], list_end = as_const(p.list_tile)[2 * b + 1];
     const uint32_t chunks = ivf_i8_list_chunks(list_end - list_begin);
     const uint32_t per = chunks != 0 ? (list_end - list_begin + chunks - 1) / chunks : 0;
     const uint32_t chunk = chunks != 0 ? (item - ioff[b]) % chunks : 0;

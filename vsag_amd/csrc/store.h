@@ -43,13 +43,21 @@ struct vsag_amd_store {
     uint64_t ntiles = 0;
     uint64_t n = 0;
 
-    // posting lists (nlist == 0: flat store)
+    // posting lists (nlist == 0: flat store).  Every list owns a run of tiles with some room behind the tiles it
+    // uses, so that codes can be appended in place; a list that outgrows its room moves all lists once.
     uint32_t nlist = 0;
     uint32_t* ids_dev = nullptr;         // inner id per tile slot, VSAG_AMD_INVALID_ID in padding
-    uint32_t* list_tile_dev = nullptr;   // nlist+1 tile offsets
-    std::vector<uint32_t> list_sizes;    // host copy
-    std::vector<uint32_t> list_tile;     // host copy, nlist+1
-    uint32_t max_list_tiles = 0;         // tiles of the longest list
+    uint32_t* list_tile_dev = nullptr;   // 2 * nlist: first tile of list l at [2 l], end of its used tiles at [2 l + 1]
+    std::vector<uint32_t> list_sizes;    // codes per list
+    std::vector<uint32_t> list_begin;    // first tile per list
+    std::vector<uint32_t> list_room;     // tiles of room per list
+    uint32_t max_list_tiles = 0;         // used tiles of the longest list
+    uint32_t* slot_of_id_dev = nullptr;  // tile slot of every inner id (the reference's location_map_, ivf.h:300-306)
+    uint64_t slot_of_id_cap = 0;
+    // use_residual (bucket_datacell.h:527-572,612-639): per slot -2 <c, decoded> - |c|^2 of its list's centroid c
+    // (l2 only, else null) and the centroids the codes are residuals of.
+    float* residual_bias_dev = nullptr;
+    float* residual_centroids_dev = nullptr;  // nlist x dim, null: no residual
 
     // flat fp32 / sq8 stores: per slot |y|^2 and the largest |y| (float bits) of the code as the batched
     // contraction sees it, kept up to date by append

@@ -31,6 +31,10 @@ struct RetileArgs {
     const uint32_t* src_index;    // list form: sorted position -> source row (may be null)
     const uint32_t* dst_slot;     // list form: sorted position -> tile slot (may be null)
     uint32_t* ids;                // list form: inner id per slot
+    uint32_t id_base;             // list form: inner id of source row 0
+    uint32_t* slot_of_id;         // list form: slot per inner id
+    const float* bias_src;        // list form: per source row residual bias (may be null)
+    float* bias_dst;              // list form: per slot
     int normalize;                // fp32 + cosine: store x / ||x||
     uint32_t dim;
 };
@@ -93,7 +97,12 @@ retile_kernel(RetileArgs a) {
             a.meta[m * a.meta_stride + slot] = word;
         }
         if (a.ids != nullptr) {
-            a.ids[slot] = static_cast<uint32_t>(row);
+            const uint32_t id = a.id_base + static_cast<uint32_t>(row);
+            a.ids[slot] = id;
+            a.slot_of_id[id] = static_cast<uint32_t>(slot);
+            if (a.bias_dst != nullptr) {
+                a.bias_dst[slot] = a.bias_src != nullptr ? a.bias_src[row] : 0.0F;
+            }
         }
     }
 }
@@ -138,15 +147,73 @@ iota_kernel(uint32_t* p, uint64_t n) {
     }
 }
 
-// sorted position p (codes ordered by label, stable) -> tile slot inside its list.
+// sorted position p (the new codes ordered by label, stable) -> tile slot: slot_base[l] + p, slot_base[l] = first free
+// slot of list l minus the position of the list's first new code (modulo 2^32).
 __global__ void
-list_slot_kernel(const int32_t* sorted_labels, uint64_t n, const uint32_t* list_start /* prefix of sizes */,
-                 const uint32_t* list_tile, uint32_t* dst_slot) {
+list_slot_kernel(const int32_t* sorted_labels, uint64_t n, const uint32_t* slot_base, uint32_t* dst_slot) {
     uint64_t p = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (p < n) {
-        uint32_t l = static_cast<uint32_t>(sorted_labels[p]);
-        uint32_t rank = static_cast<uint32_t>(p) - list_start[l];
-        dst_slot[p] = list_tile[l] * kWave + rank;
+        dst_slot[p] = slot_base[static_cast<uint32_t>(sorted_labels[p])] + static_cast<uint32_t>(p);
+    }
+}
+
+// Moves the used tiles of every list to the list's new place (one workgroup per old tile).
+struct RelocateArgs {
+    const uint4* old_tiles;
+    uint4* new_tiles;
+    uint32_t G;
+    const uint32_t* old_lt;     // 2 * nlist (first tile, end of used tiles)
+    const uint32_t* new_begin;  // nlist
+    uint32_t nlist;
+    const uint32_t* old_meta;
+    uint32_t* new_meta;
+    uint32_t nmeta;
+    uint64_t old_stride, new_stride;
+    const uint32_t* old_ids;
+    uint32_t* new_ids;
+    uint32_t* slot_of_id;
+    const float* old_bias;  // may be null
+    float* new_bias;
+};
+
+__global__ void __launch_bounds__(256)
+relocate_tiles_kernel(RelocateArgs a) {
+    __shared__ uint32_t target;
+    const uint32_t t = blockIdx.x;
+    if (threadIdx.x == 0) {
+        // the last list whose first tile is at or before t (first tiles ascend)
+        uint32_t lo = 0, hi = a.nlist;
+        while (hi - lo > 1) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (a.old_lt[2 * mid] <= t) {
+                lo = mid;
+            } else {
+                hi = mid;
+            }
+        }
+        target = t >= a.old_lt[2 * lo] && t < a.old_lt[2 * lo + 1] ? a.new_begin[lo] + (t - a.old_lt[2 * lo]) : 0xFFFFFFFFU;
+    }
+    __syncthreads();
+    const uint32_t nt = target;
+    if (nt == 0xFFFFFFFFU) {
+        return;  // room behind a list, not in use
+    }
+    for (uint32_t i = threadIdx.x; i < a.G * kWave; i += blockDim.x) {
+        a.new_tiles[static_cast<uint64_t>(nt) * a.G * kWave + i] = a.old_tiles[static_cast<uint64_t>(t) * a.G * kWave + i];
+    }
+    if (threadIdx.x < kWave) {
+        const uint64_t os = static_cast<uint64_t>(t) * kWave + threadIdx.x, ns = static_cast<uint64_t>(nt) * kWave + threadIdx.x;
+        for (uint32_t m = 0; m < a.nmeta; ++m) {
+            a.new_meta[m * a.new_stride + ns] = a.old_meta[m * a.old_stride + os];
+        }
+        const uint32_t id = a.old_ids[os];
+        a.new_ids[ns] = id;
+        if (id != VSAG_AMD_INVALID_ID) {
+            a.slot_of_id[id] = static_cast<uint32_t>(ns);
+        }
+        if (a.new_bias != nullptr) {
+            a.new_bias[ns] = a.old_bias != nullptr ? a.old_bias[os] : 0.0F;
+        }
     }
 }
 
@@ -429,7 +496,7 @@ vsag_amd_store_destroy(vsag_amd_store_t* s) {
     }
     void* ptrs[] = {s->scale_dev, s->lb_dev,  s->diff_dev, s->bounds_dev,    s->rotation_dev, s->centroid_dev,
                     s->tiles,     s->meta,    s->ids_dev,  s->list_tile_dev, s->pf_term,      s->pf_ymax,
-                    s->rows};
+                    s->rows,      s->slot_of_id_dev, s->residual_bias_dev, s->residual_centroids_dev};
     for (void* p : ptrs) {
         if (p != nullptr) {
             (void)hipFree(p);
@@ -473,6 +540,233 @@ vsag_amd_store_append(vsag_amd_store_t* s, const uint8_t* codes_dev, uint64_t n,
     return 0;
 }
 
+namespace {
+
+// Frees the posting lists of a store (not its quantizer state).
+int
+drop_lists(vsag_amd_store* s) {
+    for (void* p : {static_cast<void*>(s->tiles), static_cast<void*>(s->meta), static_cast<void*>(s->ids_dev),
+                    static_cast<void*>(s->list_tile_dev), static_cast<void*>(s->slot_of_id_dev),
+                    static_cast<void*>(s->residual_bias_dev)}) {
+        if (p != nullptr) {
+            VA_HIP(hipFree(p));
+        }
+    }
+    s->tiles = nullptr;
+    s->meta = nullptr;
+    s->ids_dev = nullptr;
+    s->list_tile_dev = nullptr;
+    s->slot_of_id_dev = nullptr;
+    s->residual_bias_dev = nullptr;
+    s->slot_of_id_cap = 0;
+    s->cap_tiles = 0;
+    s->ntiles = 0;
+    s->n = 0;
+    s->max_list_tiles = 0;
+    s->list_sizes.clear();
+    s->list_begin.clear();
+    s->list_room.clear();
+    return 0;
+}
+
+// Device buffers of one call that are freed whatever way the call ends.
+struct Temporaries {
+    std::vector<void*> ptrs;
+    ~Temporaries() {
+        for (void* p : ptrs) {
+            if (p != nullptr) {
+                (void)hipFree(p);
+            }
+        }
+    }
+    template <typename T>
+    hipError_t
+    alloc(T** out, size_t bytes) {
+        void* p = nullptr;
+        hipError_t e = hipMalloc(&p, bytes ? bytes : 4);
+        if (e == hipSuccess) {
+            ptrs.push_back(p);
+        }
+        *out = static_cast<T*>(p);
+        return e;
+    }
+};
+
+// Appends n codes (reference byte layout, source row r gets inner id s->n + r) to the lists named by labels_dev, in
+// input order inside every list.  bias_dev: per source row residual bias, or null.
+int
+append_to_lists(vsag_amd_store* s, const uint8_t* codes_dev, const int32_t* labels_dev, const float* bias_dev, uint64_t n,
+                hipStream_t st) {
+    const uint32_t nlist = s->nlist;
+    if (n == 0) {
+        return 0;
+    }
+    Temporaries tmp;
+    // 1. how many new codes per list
+    uint32_t* counts = nullptr;
+    VA_HIP(tmp.alloc(&counts, (nlist + 1) * sizeof(uint32_t)));
+    VA_HIP(hipMemsetAsync(counts, 0, (nlist + 1) * sizeof(uint32_t), st));
+    hipLaunchKernelGGL(histogram_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, labels_dev, n,
+                       nlist, counts, counts + nlist);
+    std::vector<uint32_t> added(nlist + 1);
+    VA_HIP(hipMemcpyAsync(added.data(), counts, (nlist + 1) * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+    VA_HIP(hipStreamSynchronize(st));
+    VA_CHECK_ARG(added[nlist] == 0, "%u labels are outside [0, %u)", added[nlist], nlist);
+
+    // 2. room: a list that outgrows its tiles moves every list to a new layout, with a quarter more room than it
+    // needs now (the first fill takes exactly what it needs).
+    const bool first_fill = s->n == 0;
+    bool move = s->tiles == nullptr;
+    std::vector<uint32_t> need(nlist), room(nlist);
+    for (uint32_t l = 0; l < nlist; ++l) {
+        need[l] = static_cast<uint32_t>(div_up(static_cast<uint64_t>(s->list_sizes[l]) + added[l], kWave));
+        move = move || need[l] > s->list_room[l];
+    }
+    if (move) {
+        uint64_t total = 0;
+        std::vector<uint32_t> begin(nlist);
+        for (uint32_t l = 0; l < nlist; ++l) {
+            room[l] = need[l] > s->list_room[l] && !first_fill ? need[l] + need[l] / 4 + 1 : std::max(need[l], s->list_room[l]);
+            begin[l] = static_cast<uint32_t>(total);
+            total += room[l];
+        }
+        VA_CHECK_ARG(total * kWave < 0xFFFFFFFFull, "the posting lists would span 2^32 slots or more");
+        const uint64_t cap = total > 0 ? total : 1;
+        // Everything new is built beside the old; the store changes hands only when all of it exists.
+        uint4* tiles = nullptr;
+        uint32_t *meta = nullptr, *ids = nullptr, *lt = nullptr, *new_begin = nullptr;
+        float* bias = nullptr;
+        Temporaries fresh;
+        VA_HIP(fresh.alloc(&tiles, cap * s->G * kWave * sizeof(uint4) + kTileSlackBytes));
+        VA_HIP(hipMemsetAsync(tiles, 0, cap * s->G * kWave * sizeof(uint4), st));
+        if (s->nmeta > 0) {
+            VA_HIP(fresh.alloc(&meta, cap * kWave * s->nmeta * sizeof(uint32_t)));
+            VA_HIP(hipMemsetAsync(meta, 0, cap * kWave * s->nmeta * sizeof(uint32_t), st));
+        }
+        VA_HIP(fresh.alloc(&ids, cap * kWave * sizeof(uint32_t)));
+        hipLaunchKernelGGL(fill_u32_kernel, dim3(static_cast<uint32_t>(div_up(cap * kWave, 256))), dim3(256), 0, st, ids,
+                           VSAG_AMD_INVALID_ID, cap * kWave);
+        if (s->residual_centroids_dev != nullptr && s->metric == VSAG_AMD_METRIC_L2) {
+            VA_HIP(fresh.alloc(&bias, cap * kWave * sizeof(float)));
+            VA_HIP(hipMemsetAsync(bias, 0, cap * kWave * sizeof(float), st));
+        }
+        VA_HIP(fresh.alloc(&lt, 2 * static_cast<size_t>(nlist) * sizeof(uint32_t)));
+        if (s->n > 0) {
+            VA_HIP(tmp.alloc(&new_begin, nlist * sizeof(uint32_t)));
+            VA_HIP(hipMemcpyAsync(new_begin, begin.data(), nlist * sizeof(uint32_t), hipMemcpyHostToDevice, st));
+            RelocateArgs r{};
+            r.old_tiles = s->tiles;
+            r.new_tiles = tiles;
+            r.G = s->G;
+            r.old_lt = s->list_tile_dev;
+            r.new_begin = new_begin;
+            r.nlist = nlist;
+            r.old_meta = s->meta;
+            r.new_meta = meta;
+            r.nmeta = s->nmeta;
+            r.old_stride = s->cap_tiles * kWave;
+            r.new_stride = cap * kWave;
+            r.old_ids = s->ids_dev;
+            r.new_ids = ids;
+            r.slot_of_id = s->slot_of_id_dev;
+            r.old_bias = s->residual_bias_dev;
+            r.new_bias = bias;
+            hipLaunchKernelGGL(relocate_tiles_kernel, dim3(static_cast<uint32_t>(s->cap_tiles)), dim3(256), 0, st, r);
+            VA_HIP(hipGetLastError());
+            VA_HIP(hipStreamSynchronize(st));
+        }
+        for (void* p : {static_cast<void*>(s->tiles), static_cast<void*>(s->meta), static_cast<void*>(s->ids_dev),
+                        static_cast<void*>(s->list_tile_dev), static_cast<void*>(s->residual_bias_dev)}) {
+            if (p != nullptr) {
+                (void)hipFree(p);
+            }
+        }
+        fresh.ptrs.clear();  // the store owns them now
+        s->tiles = tiles;
+        s->meta = meta;
+        s->ids_dev = ids;
+        s->list_tile_dev = lt;
+        s->residual_bias_dev = bias;
+        s->cap_tiles = cap;
+        s->list_begin = begin;
+        s->list_room = room;
+    }
+    // 3. inner id -> slot map with room for the new ids
+    if (s->n + n > s->slot_of_id_cap) {
+        uint64_t cap = std::max<uint64_t>(s->n + n, s->slot_of_id_cap + s->slot_of_id_cap / 2);
+        uint32_t* map = nullptr;
+        VA_HIP(hipMalloc(&map, cap * sizeof(uint32_t)));
+        if (s->n > 0) {
+            VA_HIP(hipMemcpyAsync(map, s->slot_of_id_dev, s->n * sizeof(uint32_t), hipMemcpyDeviceToDevice, st));
+            VA_HIP(hipStreamSynchronize(st));
+        }
+        if (s->slot_of_id_dev != nullptr) {
+            (void)hipFree(s->slot_of_id_dev);
+        }
+        s->slot_of_id_dev = map;
+        s->slot_of_id_cap = cap;
+    }
+
+    // 4. the new codes in list order (stable: the order the reference gets by appending vectors to their bucket one
+    // after another, ivf.cpp:661-675 without a thread pool), each to the first free slots of its list
+    std::vector<uint32_t> slot_base(nlist), lt_host(2 * static_cast<size_t>(nlist));
+    uint32_t first_new = 0;
+    for (uint32_t l = 0; l < nlist; ++l) {
+        slot_base[l] = s->list_begin[l] * kWave + s->list_sizes[l] - first_new;  // modulo 2^32
+        first_new += added[l];
+    }
+    int32_t* keys_out = nullptr;
+    uint32_t *vals_in = nullptr, *vals_out = nullptr, *base_dev = nullptr, *dst_slot = nullptr;
+    void* sort_tmp = nullptr;
+    size_t sort_bytes = 0;
+    VA_HIP(tmp.alloc(&keys_out, n * 4));
+    VA_HIP(tmp.alloc(&vals_in, n * 4));
+    VA_HIP(tmp.alloc(&vals_out, n * 4));
+    VA_HIP(tmp.alloc(&dst_slot, n * 4));
+    VA_HIP(tmp.alloc(&base_dev, nlist * 4));
+    VA_HIP(hipMemcpyAsync(base_dev, slot_base.data(), nlist * 4, hipMemcpyHostToDevice, st));
+    hipLaunchKernelGGL(iota_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, vals_in, n);
+    int end_bit = 1;
+    while ((1u << end_bit) < nlist) {
+        ++end_bit;
+    }
+    VA_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, sort_bytes, labels_dev, keys_out, vals_in, vals_out,
+                                              static_cast<int>(n), 0, end_bit, st));
+    VA_HIP(tmp.alloc(&sort_tmp, sort_bytes));
+    VA_HIP(hipcub::DeviceRadixSort::SortPairs(sort_tmp, sort_bytes, labels_dev, keys_out, vals_in, vals_out,
+                                              static_cast<int>(n), 0, end_bit, st));
+    hipLaunchKernelGGL(list_slot_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, keys_out, n,
+                       base_dev, dst_slot);
+    RetileArgs a = retile_args(s, codes_dev, n);
+    a.src_index = vals_out;
+    a.dst_slot = dst_slot;
+    a.ids = s->ids_dev;
+    a.id_base = static_cast<uint32_t>(s->n);
+    a.slot_of_id = s->slot_of_id_dev;
+    a.bias_src = bias_dev;
+    a.bias_dst = s->residual_bias_dev;
+    hipLaunchKernelGGL(retile_kernel, dim3(static_cast<uint32_t>(div_up(n * s->G, 256))), dim3(256), 0, st, a);
+    VA_HIP(hipGetLastError());
+
+    // 5. the lists' new extents
+    uint64_t used = 0;
+    s->max_list_tiles = 0;
+    for (uint32_t l = 0; l < nlist; ++l) {
+        s->list_sizes[l] += added[l];
+        lt_host[2 * l] = s->list_begin[l];
+        lt_host[2 * l + 1] = s->list_begin[l] + need[l];
+        used += need[l];
+        s->max_list_tiles = std::max(s->max_list_tiles, need[l]);
+    }
+    VA_HIP(hipMemcpyAsync(s->list_tile_dev, lt_host.data(), lt_host.size() * sizeof(uint32_t), hipMemcpyHostToDevice, st));
+    VA_HIP(hipStreamSynchronize(st));
+    s->ntiles = used;
+    s->n += n;
+    return 0;
+}
+
+}  // namespace
+
 extern "C" int
 vsag_amd_store_set_lists(vsag_amd_store_t* s, const uint8_t* codes_dev, const int32_t* labels_dev, uint64_t n,
                          uint32_t nlist, void* stream) {
@@ -482,105 +776,60 @@ vsag_amd_store_set_lists(vsag_amd_store_t* s, const uint8_t* codes_dev, const in
     VA_CHECK_ARG(n < 0xFFFFFFFFull, "a store holds fewer than 2^32 - 1 codes");
     VA_CHECK_ARG(n == 0 || (codes_dev && labels_dev), "null codes / labels");
     hipStream_t st = static_cast<hipStream_t>(stream);
-
-    // 1. list sizes
-    uint32_t* counts = nullptr;
-    VA_HIP(hipMalloc(&counts, (nlist + 1) * sizeof(uint32_t)));
-    VA_HIP(hipMemsetAsync(counts, 0, (nlist + 1) * sizeof(uint32_t), st));
-    if (n > 0) {
-        hipLaunchKernelGGL(histogram_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, labels_dev,
-                           n, nlist, counts, counts + nlist);
-    }
-    std::vector<uint32_t> sizes(nlist + 1);
-    VA_HIP(hipMemcpyAsync(sizes.data(), counts, (nlist + 1) * sizeof(uint32_t), hipMemcpyDeviceToHost, st));
     VA_HIP(hipStreamSynchronize(st));
-    VA_HIP(hipFree(counts));
-    VA_CHECK_ARG(sizes[nlist] == 0, "%u labels are outside [0, %u)", sizes[nlist], nlist);
-
-    // 2. tile offsets (each list padded to whole tiles) and code offsets
-    std::vector<uint32_t> list_tile(nlist + 1, 0), list_start(nlist + 1, 0);
-    for (uint32_t l = 0; l < nlist; ++l) {
-        list_tile[l + 1] = list_tile[l] + static_cast<uint32_t>(div_up(sizes[l], kWave));
-        list_start[l + 1] = list_start[l] + sizes[l];
-    }
-    uint64_t ntiles = list_tile[nlist];
-
-    // 3. fresh storage
-    for (void* p : {static_cast<void*>(s->tiles), static_cast<void*>(s->meta), static_cast<void*>(s->ids_dev),
-                    static_cast<void*>(s->list_tile_dev)}) {
-        if (p != nullptr) {
-            VA_HIP(hipFree(p));
-        }
-    }
-    s->tiles = nullptr;
-    s->meta = nullptr;
-    s->ids_dev = nullptr;
-    s->list_tile_dev = nullptr;
-    s->cap_tiles = 0;
-    s->ntiles = 0;
-    s->n = 0;
-    uint64_t cap = ntiles > 0 ? ntiles : 1;
-    VA_HIP(hipMalloc(&s->tiles, cap * s->G * kWave * sizeof(uint4) + kTileSlackBytes));
-    VA_HIP(hipMemsetAsync(s->tiles, 0, cap * s->G * kWave * sizeof(uint4), st));
-    if (s->nmeta > 0) {
-        VA_HIP(hipMalloc(&s->meta, cap * kWave * s->nmeta * sizeof(uint32_t)));
-        VA_HIP(hipMemsetAsync(s->meta, 0, cap * kWave * s->nmeta * sizeof(uint32_t), st));
-    }
-    VA_HIP(hipMalloc(&s->ids_dev, cap * kWave * sizeof(uint32_t)));
-    hipLaunchKernelGGL(fill_u32_kernel, dim3(static_cast<uint32_t>(div_up(cap * kWave, 256))), dim3(256), 0, st,
-                       s->ids_dev, VSAG_AMD_INVALID_ID, cap * kWave);
-    VA_HIP(hipMalloc(&s->list_tile_dev, (nlist + 1) * sizeof(uint32_t)));
-    VA_HIP(hipMemcpyAsync(s->list_tile_dev, list_tile.data(), (nlist + 1) * sizeof(uint32_t), hipMemcpyHostToDevice,
-                          st));
-    s->cap_tiles = cap;
-    s->ntiles = ntiles;
+    VA_TRY(drop_lists(s));
     s->nlist = nlist;
-    s->list_sizes.assign(sizes.begin(), sizes.begin() + nlist);
-    s->list_tile = list_tile;
-    s->max_list_tiles = 0;
-    for (uint32_t b = 0; b < nlist; ++b) {
-        s->max_list_tiles = std::max(s->max_list_tiles, list_tile[b + 1] - list_tile[b]);
-    }
-
-    if (n > 0) {
-        // 4. stable sort of inner ids by label: the order the reference gets by appending vectors to their
-        // bucket one after another (ivf.cpp:661-675 without a thread pool).
-        int32_t* keys_out = nullptr;
-        uint32_t *vals_in = nullptr, *vals_out = nullptr, *start_dev = nullptr, *dst_slot = nullptr;
-        void* tmp = nullptr;
-        size_t tmp_bytes = 0;
-        VA_HIP(hipMalloc(&keys_out, n * 4));
-        VA_HIP(hipMalloc(&vals_in, n * 4));
-        VA_HIP(hipMalloc(&vals_out, n * 4));
-        VA_HIP(hipMalloc(&dst_slot, n * 4));
-        VA_HIP(hipMalloc(&start_dev, (nlist + 1) * 4));
-        VA_HIP(hipMemcpyAsync(start_dev, list_start.data(), (nlist + 1) * 4, hipMemcpyHostToDevice, st));
-        hipLaunchKernelGGL(iota_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, vals_in, n);
-        int end_bit = 1;
-        while ((1u << end_bit) < nlist) {
-            ++end_bit;
+    s->list_sizes.assign(nlist, 0);
+    s->list_begin.assign(nlist, 0);
+    s->list_room.assign(nlist, 0);
+    if (n == 0) {
+        // Empty lists still need their offset table: every list begins and ends at tile 0.
+        VA_HIP(hipMalloc(&s->list_tile_dev, 2 * static_cast<size_t>(nlist) * sizeof(uint32_t)));
+        VA_HIP(hipMemsetAsync(s->list_tile_dev, 0, 2 * static_cast<size_t>(nlist) * sizeof(uint32_t), st));
+        VA_HIP(hipMalloc(&s->tiles, kTileSlackBytes + kWave * s->G * sizeof(uint4)));
+        VA_HIP(hipMalloc(&s->ids_dev, kWave * sizeof(uint32_t)));
+        hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(256), 0, st, s->ids_dev, VSAG_AMD_INVALID_ID,
+                           static_cast<uint64_t>(kWave));
+        if (s->nmeta > 0) {
+            VA_HIP(hipMalloc(&s->meta, kWave * s->nmeta * sizeof(uint32_t)));
         }
-        VA_HIP(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, labels_dev, keys_out, vals_in, vals_out,
-                                                  static_cast<int>(n), 0, end_bit, st));
-        VA_HIP(hipMalloc(&tmp, tmp_bytes));
-        VA_HIP(hipcub::DeviceRadixSort::SortPairs(tmp, tmp_bytes, labels_dev, keys_out, vals_in, vals_out,
-                                                  static_cast<int>(n), 0, end_bit, st));
-        hipLaunchKernelGGL(list_slot_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, keys_out, n,
-                           start_dev, s->list_tile_dev, dst_slot);
-        RetileArgs a = retile_args(s, codes_dev, n);
-        a.src_index = vals_out;
-        a.dst_slot = dst_slot;
-        a.ids = s->ids_dev;
-        hipLaunchKernelGGL(retile_kernel, dim3(static_cast<uint32_t>(div_up(n * s->G, 256))), dim3(256), 0, st, a);
-        VA_HIP(hipGetLastError());
+        s->cap_tiles = 1;
         VA_HIP(hipStreamSynchronize(st));
-        for (void* p : {static_cast<void*>(keys_out), static_cast<void*>(vals_in), static_cast<void*>(vals_out),
-                        static_cast<void*>(dst_slot), static_cast<void*>(start_dev), tmp}) {
-            VA_HIP(hipFree(p));
-        }
+        return 0;
     }
-    s->n = n;
+    return append_to_lists(s, codes_dev, labels_dev, nullptr, n, st);
+}
+
+extern "C" int
+vsag_amd_store_set_residual(vsag_amd_store_t* s, const float* centroids_dev, uint32_t nlist, void* stream) {
+    VA_TRY(ensure_init());
+    VA_CHECK_ARG(s != nullptr && centroids_dev != nullptr, "null store / centroids");
+    VA_CHECK_ARG(s->n == 0, "the residual centroids are set before the first code is stored");
+    VA_CHECK_ARG(s->kind != VSAG_AMD_KIND_RABITQ, "residual codes of a rabitq store are not supported");
+    VA_CHECK_ARG(nlist >= 1 && (s->nlist == 0 || s->nlist == nlist), "nlist does not match the store's lists");
+    if (s->residual_centroids_dev != nullptr) {
+        VA_HIP(hipFree(s->residual_centroids_dev));
+        s->residual_centroids_dev = nullptr;
+    }
+    const size_t bytes = static_cast<size_t>(nlist) * s->dim * sizeof(float);
+    VA_HIP(hipMalloc(&s->residual_centroids_dev, bytes));
+    VA_HIP(hipMemcpyAsync(s->residual_centroids_dev, centroids_dev, bytes, hipMemcpyDeviceToDevice,
+                          static_cast<hipStream_t>(stream)));
+    VA_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
     return 0;
+}
+
+extern "C" int
+vsag_amd_store_append_lists(vsag_amd_store_t* s, const uint8_t* codes_dev, const int32_t* labels_dev,
+                            const float* residual_bias_dev, uint64_t n, void* stream) {
+    VA_TRY(ensure_init());
+    VA_CHECK_ARG(s != nullptr, "store is null");
+    VA_CHECK_ARG(s->nlist > 0, "append_lists on a store without posting lists: call vsag_amd_store_set_lists first");
+    VA_CHECK_ARG(s->n + n < 0xFFFFFFFFull, "a store holds fewer than 2^32 - 1 codes");
+    VA_CHECK_ARG(n == 0 || (codes_dev && labels_dev), "null codes / labels");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    VA_HIP(hipStreamSynchronize(st));
+    return append_to_lists(s, codes_dev, labels_dev, residual_bias_dev, n, st);
 }
 
 extern "C" int
