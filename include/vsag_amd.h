@@ -73,6 +73,9 @@ VSAG_AMD_API int vsag_amd_memcpy_d2h(void* dst, const void* src_dev, size_t byte
 VSAG_AMD_API int vsag_amd_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
 VSAG_AMD_API int vsag_amd_memset(void* dst_dev, int value, size_t bytes, void* stream);
 VSAG_AMD_API int vsag_amd_stream_synchronize(void* stream);
+/* A stream of default priority that does not synchronise with the null stream: one per concurrent search. */
+VSAG_AMD_API int vsag_amd_stream_create(void** stream);
+VSAG_AMD_API int vsag_amd_stream_destroy(void* stream);
 
 /* ------------------------------------------------------------------ quantizer training ------- */
 
@@ -314,12 +317,24 @@ VSAG_AMD_API int vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* lists, const 
                               const vsag_amd_search_options_t* options, uint32_t* ids_dev, float* dists_dev,
                               void* workspace_dev, size_t workspace_bytes, void* stream);
 
+/* Number of codes in the lists a batch probes, summed over all (query, probe) pairs: the approximate-phase
+ * distance_evaluations of SearchStatistics (src/query_context.h:215-246).  total_dev: 8 bytes of device memory. */
+VSAG_AMD_API int vsag_amd_ivf_probed_codes(const vsag_amd_store_t* lists, const int32_t* buckets_dev, uint64_t nq,
+                              uint32_t nprobe, uint64_t* total_dev, void* stream);
+
 /* FlattenReorder::Reorder (impl/reorder/flatten_reorder.cpp:52-114): exact fp32 distances of the
  * candidates (nq x kcand inner ids into raw_dev, n x dim fp32 row-major; VSAG_AMD_INVALID_ID skipped),
  * best k kept, ascending. */
 VSAG_AMD_API int vsag_amd_rerank_fp32(const float* raw_dev, uint64_t n, uint32_t dim, int metric,
                          const float* queries_dev, uint64_t nq, const uint32_t* cand_ids_dev,
                          uint32_t kcand, uint32_t k, uint32_t* ids_dev, float* dists_dev, void* stream);
+
+/* FlattenDataCell::Query over fp32 codes (flatten_datacell.h:334-440; IVF::CalDistanceById with precise distances,
+ * ivf.cpp:2462-2465): the exact distance of every (query, inner id) pair in the order given, nq x count, with the
+ * arithmetic of vsag_amd_rerank_fp32; -1 where the id is VSAG_AMD_INVALID_ID or beyond the rows. */
+VSAG_AMD_API int vsag_amd_rows_distances_fp32(const float* raw_dev, uint64_t n, uint32_t dim, int metric,
+                                 const float* queries_dev, uint64_t nq, const uint32_t* ids_dev, uint32_t count,
+                                 float* dists_dev, void* stream);
 
 #ifdef __cplusplus
 }

@@ -54,6 +54,8 @@ PROTOTYPES = {
     "vsag_amd_memcpy_d2d": (C.c_int, [_vp, _vp, _sz, _vp]),
     "vsag_amd_memset": (C.c_int, [_vp, C.c_int, _sz, _vp]),
     "vsag_amd_stream_synchronize": (C.c_int, [_vp]),
+    "vsag_amd_stream_create": (C.c_int, [C.POINTER(_vp)]),
+    "vsag_amd_stream_destroy": (C.c_int, [_vp]),
     "vsag_amd_sq_train_workspace_bytes": (_sz, [_u64, _u32, _u64]),
     "vsag_amd_sq_train": (C.c_int, [_vp, _u64, _u32, _i32, _i32, _i32, _f32, _u64, _vp, _vp, _vp, _sz, _vp]),
     "vsag_amd_sq_train_uniform": (C.c_int, [_vp, _u64, _u32, _i32, _i32, _i32, _f32, _u64, _vp, _vp, _sz, _vp]),
@@ -98,7 +100,9 @@ PROTOTYPES = {
     "vsag_amd_ivf_scan_workspace_bytes": (_sz, [_vp, _u64, _u32, _u32]),
     "vsag_amd_ivf_scan_topk": (C.c_int, [_vp, _vp, _u64, _vp, _u32, _u32, _vp, _vp, _vp, _sz, _vp]),
     "vsag_amd_ivf_scan_topk_ex": (C.c_int, [_vp, _vp, _u64, _vp, _u32, _u32, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "vsag_amd_ivf_probed_codes": (C.c_int, [_vp, _vp, _u64, _u32, _vp, _vp]),
     "vsag_amd_rerank_fp32": (C.c_int, [_vp, _u64, _u32, _i32, _vp, _u64, _vp, _u32, _u32, _vp, _vp, _vp]),
+    "vsag_amd_rows_distances_fp32": (C.c_int, [_vp, _u64, _u32, _i32, _vp, _u64, _vp, _u32, _vp, _vp]),
 }
 
 _lib = None

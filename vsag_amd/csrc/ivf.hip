@@ -614,6 +614,86 @@ rerank_kernel(const float* raw, uint64_t n, uint32_t dim, int metric, const floa
     }
 }
 
+// Exact fp32 distance of every (query, inner id) pair, in the order given: what the rerank computes for a candidate,
+// without the selection.  Sixteen lanes share a pair; ids beyond the rows (or VSAG_AMD_INVALID_ID) give -1.
+__global__ void __launch_bounds__(kRerankThreads)
+rows_distances_kernel(const float* raw, uint64_t n, uint32_t dim, int metric, const float* queries, const uint32_t* ids,
+                      uint32_t count, float* dists) {
+    const uint32_t tid = threadIdx.x;
+    const uint32_t sub = tid >> 4, l = tid & 15;
+    const uint64_t q = blockIdx.y;
+    const float* qv = queries + q * dim;
+    float inv_norm = 1.0F;
+    if (metric == VSAG_AMD_METRIC_COSINE) {
+        float s = 0.0F;
+        for (uint32_t d = l; d < dim; d += 16) {
+            s = fmaf(qv[d], qv[d], s);
+        }
+        for (int off = 8; off > 0; off >>= 1) {
+            s += __shfl_xor(s, off);
+        }
+        inv_norm = s > 0.0F ? 1.0F / sqrtf(s) : 1.0F;
+    }
+    const uint32_t j = blockIdx.x * (kRerankThreads / 16) + sub;
+    const uint32_t id = j < count ? ids[q * count + j] : VSAG_AMD_INVALID_ID;
+    const bool live = id != VSAG_AMD_INVALID_ID && id < n;
+    const float* x = raw + static_cast<uint64_t>(live ? id : 0) * dim;
+    float s = 0.0F, xx = 0.0F;
+    if (live) {
+        if ((dim & 3) == 0) {
+            for (uint32_t d = l * 4; d < dim; d += 64) {
+                const float4 xv = *reinterpret_cast<const float4*>(x + d);
+                const float4 qq = *reinterpret_cast<const float4*>(qv + d);
+                if (metric == VSAG_AMD_METRIC_L2) {
+                    const float t0 = qq.x - xv.x, t1 = qq.y - xv.y, t2 = qq.z - xv.z, t3 = qq.w - xv.w;
+                    s = fmaf(t0, t0, s);
+                    s = fmaf(t1, t1, s);
+                    s = fmaf(t2, t2, s);
+                    s = fmaf(t3, t3, s);
+                } else {
+                    s = fmaf(qq.x, xv.x, s);
+                    s = fmaf(qq.y, xv.y, s);
+                    s = fmaf(qq.z, xv.z, s);
+                    s = fmaf(qq.w, xv.w, s);
+                    xx = fmaf(xv.x, xv.x, xx);
+                    xx = fmaf(xv.y, xv.y, xx);
+                    xx = fmaf(xv.z, xv.z, xx);
+                    xx = fmaf(xv.w, xv.w, xx);
+                }
+            }
+        } else {
+            for (uint32_t d = l; d < dim; d += 16) {
+                const float xv = x[d];
+                if (metric == VSAG_AMD_METRIC_L2) {
+                    const float t = qv[d] - xv;
+                    s = fmaf(t, t, s);
+                } else {
+                    s = fmaf(qv[d], xv, s);
+                    xx = fmaf(xv, xv, xx);
+                }
+            }
+        }
+    }
+    for (int off = 8; off > 0; off >>= 1) {
+        s += __shfl_xor(s, off);
+        xx += __shfl_xor(xx, off);
+    }
+    if (j < count && l == 0) {
+        float dist = -1.0F;
+        if (live) {
+            if (metric == VSAG_AMD_METRIC_L2) {
+                dist = s;
+            } else if (metric == VSAG_AMD_METRIC_IP) {
+                dist = 1.0F - s;
+            } else {
+                const float xn = xx > 0.0F ? 1.0F / sqrtf(xx) : 1.0F;
+                dist = 1.0F - s * inv_norm * xn;
+            }
+        }
+        dists[q * count + j] = dist;
+    }
+}
+
 template <int KIND, int METRIC, int T>
 static void
 launch_ivf_c(dim3 grid, dim3 block, size_t lds, hipStream_t st, const ScanArgs& a, const IvfArgs& v) {
@@ -972,6 +1052,44 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
                                  p.S, nq, ids_dev, dists_dev, st);
 }
 
+namespace vsag_amd {
+// Codes in the lists the queries probe, summed over all (query, probe) pairs.
+__global__ void __launch_bounds__(256)
+probed_codes_kernel(const int32_t* buckets, uint64_t npairs, uint32_t nlist, const uint32_t* list_sizes,
+                    unsigned long long* total) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    unsigned long long mine = 0;
+    if (i < npairs) {
+        const int32_t b = buckets[i];
+        if (b >= 0 && static_cast<uint32_t>(b) < nlist) {
+            mine = list_sizes[b];
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        mine += __shfl_xor(mine, off);
+    }
+    if ((threadIdx.x & 63) == 0 && mine != 0) {
+        atomicAdd(total, mine);
+    }
+}
+}  // namespace vsag_amd
+
+extern "C" int
+vsag_amd_ivf_probed_codes(const vsag_amd_store_t* s, const int32_t* buckets_dev, uint64_t nq, uint32_t nprobe,
+                          uint64_t* total_dev, void* stream) {
+    VA_TRY(ensure_init());
+    VA_CHECK_ARG(s != nullptr && s->nlist > 0, "not a posting-list store");
+    VA_CHECK_ARG(buckets_dev && total_dev, "null pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(fill_jobs_kernel, dim3(1), dim3(256), 0, st,
+                       FillJob{{reinterpret_cast<uint32_t*>(total_dev), nullptr, nullptr, nullptr, nullptr}, {0, 0, 0, 0, 0},
+                               {2, 0, 0, 0, 0}});
+    hipLaunchKernelGGL(probed_codes_kernel, dim3(blocks_for(nq * nprobe)), dim3(256), 0, st, buckets_dev, nq * nprobe,
+                       s->nlist, s->list_sizes_dev, reinterpret_cast<unsigned long long*>(total_dev));
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
 extern "C" int
 vsag_amd_rerank_fp32(const float* raw_dev, uint64_t n, uint32_t dim, int metric, const float* queries_dev, uint64_t nq,
                      const uint32_t* cand_ids_dev, uint32_t kcand, uint32_t k, uint32_t* ids_dev, float* dists_dev,
@@ -989,6 +1107,21 @@ vsag_amd_rerank_fp32(const float* raw_dev, uint64_t n, uint32_t dim, int metric,
     hipLaunchKernelGGL(rerank_kernel, dim3(static_cast<uint32_t>(nq)), dim3(kRerankThreads), S * 8,
                        static_cast<hipStream_t>(stream), raw_dev, n, dim, metric, queries_dev, cand_ids_dev, kcand, k,
                        S, ids_dev, dists_dev);
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
+extern "C" int
+vsag_amd_rows_distances_fp32(const float* raw_dev, uint64_t n, uint32_t dim, int metric, const float* queries_dev,
+                             uint64_t nq, const uint32_t* ids_dev, uint32_t count, float* dists_dev, void* stream) {
+    VA_TRY(ensure_init());
+    VA_CHECK_ARG(raw_dev && queries_dev && ids_dev && dists_dev, "null pointer");
+    VA_CHECK_ARG(metric >= VSAG_AMD_METRIC_L2 && metric <= VSAG_AMD_METRIC_COSINE, "unknown metric %d", metric);
+    VA_CHECK_ARG(nq >= 1 && nq <= 65535, "nq must be in [1, 65535]");
+    VA_CHECK_ARG(count >= 1, "count must be positive");
+    hipLaunchKernelGGL(rows_distances_kernel, dim3(static_cast<uint32_t>(div_up(count, kRerankThreads / 16)), static_cast<uint32_t>(nq)),
+                       dim3(kRerankThreads), 0, static_cast<hipStream_t>(stream), raw_dev, n, dim, metric, queries_dev,
+                       ids_dev, count, dists_dev);
     VA_HIP(hipGetLastError());
     return 0;
 }

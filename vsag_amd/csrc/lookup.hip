@@ -35,6 +35,38 @@ fill_dists_kernel(float* p, uint64_t n, float v) {
     }
 }
 
+// <q, c> and <q, q> summed by one lane in the order a wave sums them in residual_terms_kernel (lane l takes the
+// dimensions l, l + 64, ...; the lanes are then added pairwise at distances 32, 16, ... 1), so that a distance looked
+// up by id is bit for bit the distance a scan of the list reports.
+__device__ inline void
+dot_in_wave_order(const float* qv, const float* c, uint32_t dim, float* ip_out, float* qq_out) {
+    float ip_stack[7], qq_stack[7];
+    int sp = 0;
+#pragma unroll
+    for (uint32_t j = 0; j < kWave; ++j) {
+        // the lane whose partial sum is the j-th leaf of the addition tree: j with its six bits reversed
+        const uint32_t leaf = ((j & 1) << 5) | ((j & 2) << 3) | ((j & 4) << 1) | ((j & 8) >> 1) | ((j & 16) >> 3) |
+                              ((j & 32) >> 5);
+        float ip = 0.0F, qq = 0.0F;
+        for (uint32_t d = leaf; d < dim; d += kWave) {
+            ip = fmaf(qv[d], c[d], ip);
+            qq = fmaf(qv[d], qv[d], qq);
+        }
+        uint32_t m = j;
+        while (m & 1) {
+            --sp;
+            ip = ip_stack[sp] + ip;
+            qq = qq_stack[sp] + qq;
+            m >>= 1;
+        }
+        ip_stack[sp] = ip;
+        qq_stack[sp] = qq;
+        ++sp;
+    }
+    *ip_out = ip_stack[0];
+    *qq_out = qq_stack[0];
+}
+
 // One wave per (query, 64 ids): every lane gathers the granules of its own code.
 template <int KIND, int METRIC>
 __global__ void __launch_bounds__(64)
@@ -72,18 +104,11 @@ store_distances_kernel(ScanArgs a, LookupArgs p) {
         }
         const float* c = p.centroids + static_cast<uint64_t>(lo) * a.dim;
         const float* qv = p.queries + static_cast<uint64_t>(q) * a.dim;
-        float norm = 1.0F;
+        float ip, qq;
+        dot_in_wave_order(qv, c, a.dim, &ip, &qq);
         if (p.metric == VSAG_AMD_METRIC_COSINE) {
-            float s = 0.0F;
-            for (uint32_t k = 0; k < a.dim; ++k) {
-                s = fmaf(qv[k], qv[k], s);
-            }
-            norm = sqrtf(s);
-            norm = norm == 0.0F ? 1.0F : norm;
-        }
-        float ip = 0.0F;
-        for (uint32_t k = 0; k < a.dim; ++k) {
-            ip = fmaf(qv[k] / norm, c[k], ip);
+            const float norm = sqrtf(qq);
+            ip = ip / (norm == 0.0F ? 1.0F : norm);
         }
         if (p.metric == VSAG_AMD_METRIC_L2) {
             out = (out - (p.bias != nullptr ? p.bias[slot] : 0.0F)) - 2.0F * ip;

@@ -230,6 +230,25 @@ vsag_amd_memset(void* dst_dev, int value, size_t bytes, void* stream) {
 }
 
 extern "C" int
+vsag_amd_stream_create(void** stream) {
+    VA_TRY(ensure_init());
+    VA_CHECK_ARG(stream != nullptr, "stream is null");
+    hipStream_t st = nullptr;
+    // Default priority; independent of the null stream, so that searches on different streams overlap.
+    VA_HIP(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+    *stream = st;
+    return 0;
+}
+
+extern "C" int
+vsag_amd_stream_destroy(void* stream) {
+    if (stream != nullptr) {
+        VA_HIP(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+    }
+    return 0;
+}
+
+extern "C" int
 vsag_amd_stream_synchronize(void* stream) {
     VA_TRY(ensure_init());
     VA_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));

@@ -49,6 +49,7 @@ struct vsag_amd_store {
     uint32_t* ids_dev = nullptr;         // inner id per tile slot, VSAG_AMD_INVALID_ID in padding
     uint32_t* list_tile_dev = nullptr;   // 2 * nlist: first tile of list l at [2 l], end of its used tiles at [2 l + 1]
     std::vector<uint32_t> list_sizes;    // codes per list
+    uint32_t* list_sizes_dev = nullptr;  // the same on the device
     std::vector<uint32_t> list_begin;    // first tile per list
     std::vector<uint32_t> list_room;     // tiles of room per list
     uint32_t max_list_tiles = 0;         // used tiles of the longest list

@@ -496,7 +496,8 @@ vsag_amd_store_destroy(vsag_amd_store_t* s) {
     }
     void* ptrs[] = {s->scale_dev, s->lb_dev,  s->diff_dev, s->bounds_dev,    s->rotation_dev, s->centroid_dev,
                     s->tiles,     s->meta,    s->ids_dev,  s->list_tile_dev, s->pf_term,      s->pf_ymax,
-                    s->rows,      s->slot_of_id_dev, s->residual_bias_dev, s->residual_centroids_dev};
+                    s->rows,      s->slot_of_id_dev, s->residual_bias_dev, s->residual_centroids_dev,
+                    s->list_sizes_dev};
     for (void* p : ptrs) {
         if (p != nullptr) {
             (void)hipFree(p);
@@ -547,11 +548,12 @@ int
 drop_lists(vsag_amd_store* s) {
     for (void* p : {static_cast<void*>(s->tiles), static_cast<void*>(s->meta), static_cast<void*>(s->ids_dev),
                     static_cast<void*>(s->list_tile_dev), static_cast<void*>(s->slot_of_id_dev),
-                    static_cast<void*>(s->residual_bias_dev)}) {
+                    static_cast<void*>(s->residual_bias_dev), static_cast<void*>(s->list_sizes_dev)}) {
         if (p != nullptr) {
             VA_HIP(hipFree(p));
         }
     }
+    s->list_sizes_dev = nullptr;
     s->tiles = nullptr;
     s->meta = nullptr;
     s->ids_dev = nullptr;
@@ -759,6 +761,7 @@ append_to_lists(vsag_amd_store* s, const uint8_t* codes_dev, const int32_t* labe
         s->max_list_tiles = std::max(s->max_list_tiles, need[l]);
     }
     VA_HIP(hipMemcpyAsync(s->list_tile_dev, lt_host.data(), lt_host.size() * sizeof(uint32_t), hipMemcpyHostToDevice, st));
+    VA_HIP(hipMemcpyAsync(s->list_sizes_dev, s->list_sizes.data(), nlist * sizeof(uint32_t), hipMemcpyHostToDevice, st));
     VA_HIP(hipStreamSynchronize(st));
     s->ntiles = used;
     s->n += n;
@@ -782,6 +785,8 @@ vsag_amd_store_set_lists(vsag_amd_store_t* s, const uint8_t* codes_dev, const in
     s->list_sizes.assign(nlist, 0);
     s->list_begin.assign(nlist, 0);
     s->list_room.assign(nlist, 0);
+    VA_HIP(hipMalloc(&s->list_sizes_dev, nlist * sizeof(uint32_t)));
+    VA_HIP(hipMemsetAsync(s->list_sizes_dev, 0, nlist * sizeof(uint32_t), st));
     if (n == 0) {
         // Empty lists still need their offset table: every list begins and ends at tile 0.
         VA_HIP(hipMalloc(&s->list_tile_dev, 2 * static_cast<size_t>(nlist) * sizeof(uint32_t)));

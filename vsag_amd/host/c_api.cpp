@@ -7,6 +7,9 @@
 #include <cstring>
 #include <limits>
 #include <memory>
+#include <mutex>
+#include <unordered_map>
+#include <unordered_set>
 
 #include "vsag_host.h"
 
@@ -36,6 +39,11 @@ success() {
     static const Error_t ok = make_error(VSAG_SUCCESS, "success");
     return ok;
 }
+
+// src/vsag_c_api.cpp:70-140: statistics are kept per SearchResult_t that asked for them.
+std::mutex statistics_mutex;
+std::unordered_set<const SearchResult_t*> statistics_requests;
+std::unordered_map<const SearchResult_t*, std::unique_ptr<std::string>> statistics_results;
 
 thread_local Error_t tl_factory_error = make_error(VSAG_SUCCESS, "success");
 thread_local int64_t tl_failed_ids = 0;
@@ -142,6 +150,12 @@ search_one(vsag_index_t index, const float* query, uint64_t dim, bool range, flo
         search_result->dists[i] = result.value()->GetDistances()[i];
     }
     search_result->count = to_write;
+    {
+        std::lock_guard<std::mutex> lock(statistics_mutex);
+        if (statistics_requests.erase(search_result) != 0) {
+            statistics_results[search_result] = std::make_unique<std::string>(result.value()->GetStatistics());
+        }
+    }
     return success();
 }
 
@@ -211,4 +225,118 @@ vsag_index_get_num_elements(vsag_index_t index) {
 extern "C" int64_t
 vsag_last_failed_id_count(void) {
     return tl_failed_ids;
+}
+
+extern "C" Error_t
+vsag_index_search_buckets(vsag_index_t index, const float* queries, uint64_t nq, uint64_t dim, int64_t k,
+                          const char* parameters, const int64_t* bucket_ids, const uint64_t* bucket_offsets, int64_t* ids,
+                          float* dists, int64_t* result_dim) {
+    auto* vi = static_cast<VsagIndex*>(index);
+    if (vi == nullptr) {
+        return make_error(VSAG_UNKNOWN_ERROR, "index is NULL");
+    }
+    if (ids == nullptr || dists == nullptr) {
+        return make_error(VSAG_INVALID_ARGUMENT, "result arrays are NULL");
+    }
+    vsag::SearchRequest request;
+    request.query_ = vsag::Dataset::Make();
+    request.query_->Owner(false)
+        ->Dim(static_cast<int64_t>(dim))
+        ->NumElements(static_cast<int64_t>(nq))
+        ->Float32Vectors(queries);
+    request.topk_ = k;
+    request.params_str_ = parameters ? parameters : "";
+    if (bucket_offsets != nullptr && bucket_ids != nullptr) {
+        request.bucket_ids_.resize(nq);
+        for (uint64_t i = 0; i < nq; ++i) {
+            request.bucket_ids_[i].assign(bucket_ids + bucket_offsets[i], bucket_ids + bucket_offsets[i + 1]);
+        }
+    }
+    auto result = vi->index_->SearchWithRequest(request);
+    if (!result.has_value()) {
+        return make_error(result.error());
+    }
+    const auto& r = result.value();
+    const int64_t rows = r->GetNumElements(), cols = r->GetDim();
+    for (uint64_t i = 0; i < nq; ++i) {
+        for (int64_t j = 0; j < k; ++j) {
+            bool have = static_cast<int64_t>(i) < rows && j < cols;
+            ids[i * k + j] = have ? r->GetIds()[i * cols + j] : -1;
+            dists[i * k + j] = have ? r->GetDistances()[i * cols + j] : std::numeric_limits<float>::infinity();
+        }
+    }
+    if (result_dim != nullptr) {
+        *result_dim = cols;
+    }
+    return success();
+}
+
+extern "C" Error_t
+vsag_index_train(vsag_index_t index, const float* data, const int64_t* ids, uint64_t dim, uint64_t count) {
+    auto* vi = static_cast<VsagIndex*>(index);
+    if (vi == nullptr) {
+        return make_error(VSAG_UNKNOWN_ERROR, "index is NULL");
+    }
+    auto result = vi->index_->Train(base_dataset(data, ids, dim, count));
+    return result.has_value() ? success() : make_error(result.error());
+}
+
+extern "C" Error_t
+vsag_index_calculate_distance_by_ids(vsag_index_t index, const float* query, uint64_t dim, const int64_t* ids,
+                                     uint64_t count, float* dists) {
+    return vsag_index_calculate_distances(index, query, 1, dim, ids, count, true, -1, nullptr, dists);
+}
+
+extern "C" Error_t
+vsag_index_calculate_distances(vsag_index_t index, const float* queries, uint64_t nq, uint64_t dim, const int64_t* ids,
+                               uint64_t count, bool precise, int64_t topk, int64_t* out_ids, float* out_dists) {
+    auto* vi = static_cast<VsagIndex*>(index);
+    if (vi == nullptr) {
+        return make_error(VSAG_UNKNOWN_ERROR, "index is NULL");
+    }
+    if (out_dists == nullptr && count > 0) {
+        return make_error(VSAG_INVALID_ARGUMENT, "output array is NULL");
+    }
+    auto q = vsag::Dataset::Make();
+    q->Owner(false)->Dim(static_cast<int64_t>(dim))->NumElements(static_cast<int64_t>(nq))->Float32Vectors(queries);
+    auto result = vi->index_->CalDistanceById(q, ids, static_cast<int64_t>(count), precise, topk);
+    if (!result.has_value()) {
+        return make_error(result.error());
+    }
+    const auto& r = result.value();
+    const int64_t total = r->GetNumElements() * r->GetDim();
+    if (total > 0) {
+        std::memcpy(out_dists, r->GetDistances(), static_cast<size_t>(total) * sizeof(float));
+        if (out_ids != nullptr && r->GetIds() != nullptr) {
+            std::memcpy(out_ids, r->GetIds(), static_cast<size_t>(total) * sizeof(int64_t));
+        }
+    }
+    return success();
+}
+
+extern "C" Error_t
+vsag_search_result_enable_statistics(SearchResult_t* search_result) {
+    if (search_result == nullptr) {
+        return make_error(VSAG_UNKNOWN_ERROR, "search result is NULL");
+    }
+    std::lock_guard<std::mutex> lock(statistics_mutex);
+    if (statistics_requests.count(search_result) != 0 || statistics_results.count(search_result) != 0) {
+        return make_error(VSAG_UNKNOWN_ERROR, "search result statistics are already enabled");
+    }
+    statistics_requests.insert(search_result);
+    return success();
+}
+
+extern "C" const char*
+vsag_search_result_get_statistics(const SearchResult_t* search_result) {
+    std::lock_guard<std::mutex> lock(statistics_mutex);
+    auto it = statistics_results.find(search_result);
+    return it == statistics_results.end() ? nullptr : it->second->c_str();
+}
+
+extern "C" void
+vsag_search_result_destroy_statistics(SearchResult_t* search_result) {
+    std::lock_guard<std::mutex> lock(statistics_mutex);
+    statistics_requests.erase(search_result);
+    statistics_results.erase(search_result);
 }

@@ -9,10 +9,13 @@
 #include <cstring>
 #include <functional>
 #include <limits>
+#include <map>
 #include <mutex>
+#include <shared_mutex>
 #include <random>
 #include <set>
 #include <stdexcept>
+#include <unordered_map>
 #include <unordered_set>
 
 #include "../../include/vsag_amd.h"
@@ -74,6 +77,23 @@ safe_call(F&& f) {
     }
 }
 
+template <typename F>
+Expected<void>
+safe_run(F&& f) {
+    try {
+        f();
+        return Expected<void>();
+    } catch (const VsagException& e) {
+        return Expected<void>(Error(e.type, e.message));
+    } catch (const std::bad_alloc&) {
+        return Expected<void>(Error(ErrorType::NO_ENOUGH_MEMORY, "not enough memory"));
+    } catch (const std::invalid_argument& e) {
+        return Expected<void>(Error(ErrorType::INVALID_ARGUMENT, e.what()));
+    } catch (const std::exception& e) {
+        return Expected<void>(Error(ErrorType::UNKNOWN_ERROR, e.what()));
+    }
+}
+
 struct DevBuf {
     void* p = nullptr;
     size_t bytes = 0;
@@ -126,6 +146,80 @@ struct DevBuf {
     as() const {
         return static_cast<T*>(p);
     }
+};
+
+// What one search in flight owns on the device: a stream of its own and its buffers.  Searches are const and may run
+// concurrently on one index (SUPPORT_SEARCH_CONCURRENT, bruteforce.cpp:1112-1116, ivf.cpp:498; tools/eval drives one
+// query per call from an OpenMP loop, tools/eval/case/search_eval_case.cpp:233-248): each takes a context from the
+// index's pool and gives it back, so the buffers are reused without being shared.
+struct SearchContext {
+    void* stream = nullptr;
+    DevBuf queries, buckets, bucket_d, cand_ids, cand_d, out_ids, out_d, workspace, deny, scalar;
+    SearchContext() {
+        dev(vsag_amd_stream_create(&stream));
+    }
+    SearchContext(const SearchContext&) = delete;
+    SearchContext&
+    operator=(const SearchContext&) = delete;
+    ~SearchContext() {
+        if (stream != nullptr) {
+            vsag_amd_stream_destroy(stream);
+        }
+    }
+    void
+    upload(DevBuf& buf, const void* src, size_t n) {
+        buf.reserve(std::max<size_t>(n, 4));
+        dev(vsag_amd_memcpy_h2d(buf.p, src, n, stream));
+    }
+    void
+    download(void* dst, const void* src_dev, size_t n) {
+        dev(vsag_amd_memcpy_d2h(dst, src_dev, n, stream));
+    }
+};
+
+class ContextPool {
+public:
+    class Lease {
+    public:
+        Lease(ContextPool* pool, std::unique_ptr<SearchContext> ctx) : pool_(pool), ctx_(std::move(ctx)) {
+        }
+        Lease(Lease&&) = default;
+        ~Lease() {
+            if (ctx_ != nullptr) {
+                std::lock_guard<std::mutex> lock(pool_->mutex_);
+                pool_->free_.push_back(std::move(ctx_));
+            }
+        }
+        SearchContext*
+        operator->() {
+            return ctx_.get();
+        }
+        SearchContext&
+        operator*() {
+            return *ctx_;
+        }
+
+    private:
+        ContextPool* pool_;
+        std::unique_ptr<SearchContext> ctx_;
+    };
+
+    Lease
+    acquire() {
+        {
+            std::lock_guard<std::mutex> lock(mutex_);
+            if (!free_.empty()) {
+                auto ctx = std::move(free_.back());
+                free_.pop_back();
+                return Lease(this, std::move(ctx));
+            }
+        }
+        return Lease(this, std::make_unique<SearchContext>());
+    }
+
+private:
+    std::mutex mutex_;
+    std::vector<std::unique_ptr<SearchContext>> free_;
 };
 
 struct CommonParam {
@@ -392,14 +486,18 @@ pack_results(const std::vector<uint32_t>& ids, const std::vector<float>& dists, 
     return result;
 }
 
-// Ids of `base` that are already present (or repeated inside `base`): they are reported back and skipped,
-// as BruteForce::Add / IVF::Add do through the label table.
+using LabelMap = std::unordered_map<int64_t, uint32_t>;  // label -> inner id (LabelTable)
+
+// Rows of `base` whose ids are new; the ids already present (or repeated inside `base`) are reported back and
+// skipped, as BruteForce::Add / IVF::Add do through the label table.  Nothing is recorded yet: the caller adds the
+// new labels to the table once the device holds the vectors, so that a failed insert leaves the index as it was.
 std::vector<int64_t>
-split_new_rows(const DatasetPtr& base, std::unordered_set<int64_t>& known, std::vector<int64_t>& rows) {
+split_new_rows(const DatasetPtr& base, const LabelMap& known, std::vector<int64_t>& rows) {
     std::vector<int64_t> failed;
+    std::unordered_set<int64_t> batch;
     const int64_t* ids = base->GetIds();
     for (int64_t i = 0; i < base->GetNumElements(); ++i) {
-        if (known.insert(ids[i]).second) {
+        if (known.count(ids[i]) == 0 && batch.insert(ids[i]).second) {
             rows.push_back(i);
         } else {
             failed.push_back(ids[i]);
@@ -408,19 +506,22 @@ split_new_rows(const DatasetPtr& base, std::unordered_set<int64_t>& known, std::
     return failed;
 }
 
-// Uploads the selected rows (all rows when nothing was skipped) as one n x dim device matrix.
+// Uploads the selected rows (all rows when nothing was skipped) as one n x dim device matrix, every row `repeat`
+// times in a row.
 void
-upload_rows(const DatasetPtr& base, const std::vector<int64_t>& rows, uint32_t dim, DevBuf& out) {
+upload_rows(const DatasetPtr& base, const std::vector<int64_t>& rows, uint32_t dim, DevBuf& out, uint32_t repeat = 1) {
     const float* src = base->GetFloat32Vectors();
     size_t row_bytes = static_cast<size_t>(dim) * 4;
-    out.reserve(std::max<size_t>(rows.size() * row_bytes, 4));
-    if (static_cast<int64_t>(rows.size()) == base->GetNumElements()) {
+    out.reserve(std::max<size_t>(rows.size() * row_bytes * repeat, 4));
+    if (repeat == 1 && static_cast<int64_t>(rows.size()) == base->GetNumElements()) {
         dev(vsag_amd_memcpy_h2d(out.p, src, rows.size() * row_bytes, nullptr));
         return;
     }
-    std::vector<float> staged(rows.size() * dim);
+    std::vector<float> staged(rows.size() * dim * repeat);
     for (size_t i = 0; i < rows.size(); ++i) {
-        std::memcpy(staged.data() + i * dim, src + rows[i] * dim, row_bytes);
+        for (uint32_t r = 0; r < repeat; ++r) {
+            std::memcpy(staged.data() + (i * repeat + r) * dim, src + rows[i] * dim, row_bytes);
+        }
     }
     dev(vsag_amd_memcpy_h2d(out.p, staged.data(), staged.size() * 4, nullptr));
 }
@@ -434,50 +535,57 @@ reject_unknown_keys(const Json& index_param, const std::set<std::string>& known)
     }
 }
 
-// What a search asks for beyond (query, k): a pre-filter on labels and / or a radius.
+// What a search asks for beyond (query, k): a pre-filter on labels, a radius, the buckets to scan.
 struct SearchSpec {
     bool range = false;
     float radius = 0.0F;
     int64_t limited_size = -1;
     std::function<bool(int64_t)> valid;  // empty = every label is kept
+    const std::vector<std::vector<int64_t>>* bucket_ids = nullptr;
 };
 
-// Deny mask over inner ids for the device scans (bit set = filtered out), kept on the host as well so that
-// a range search can add the ids it has already returned.
+// Deny mask over the ids the device scans see (inner ids; posting ids = inner id * per_id + j for an ivf index with
+// buckets_per_data = per_id), bit set = filtered out; kept on the host as well so that a range search can add the ids
+// it has already returned.
 struct DenyMask {
     std::vector<uint32_t> words;
-    DevBuf dev_words;
     bool active = false;
+    uint32_t per_id = 1;
 
     void
-    init(const std::vector<int64_t>& labels, const std::function<bool(int64_t)>& valid, bool force) {
+    init(SearchContext& ctx, const std::vector<int64_t>& labels, const std::function<bool(int64_t)>& valid, bool force,
+         uint32_t postings_per_id) {
         active = static_cast<bool>(valid) || force;
+        per_id = postings_per_id;
         if (!active) {
             return;
         }
-        words.assign((labels.size() + 31) / 32, 0U);
+        const size_t bits = labels.size() * per_id;
+        words.assign((bits + 31) / 32, 0U);
         if (valid) {
             for (size_t i = 0; i < labels.size(); ++i) {
                 if (!valid(labels[i])) {
-                    words[i >> 5] |= 1U << (i & 31);
+                    deny(static_cast<uint32_t>(i));
                 }
             }
         }
-        upload();
+        upload(ctx);
     }
     void
-    deny(uint32_t id) {
-        words[id >> 5] |= 1U << (id & 31);
+    deny(uint32_t inner_id) {
+        for (uint32_t j = 0; j < per_id; ++j) {
+            const uint64_t bit = static_cast<uint64_t>(inner_id) * per_id + j;
+            words[bit >> 5] |= 1U << (bit & 31);
+        }
     }
     void
-    upload() {
-        dev_words.reserve(std::max<size_t>(words.size() * 4, 4));
-        dev(vsag_amd_memcpy_h2d(dev_words.p, words.data(), words.size() * 4, nullptr));
+    upload(SearchContext& ctx) {
+        ctx.upload(ctx.deny, words.data(), words.size() * 4);
     }
     vsag_amd_search_options_t
-    options(const SearchSpec& spec, float radius_slack) const {
+    options(const SearchContext& ctx, const SearchSpec& spec, float radius_slack) const {
         vsag_amd_search_options_t o{};
-        o.deny_bits_dev = active ? dev_words.as<uint32_t>() : nullptr;
+        o.deny_bits_dev = active ? ctx.deny.as<uint32_t>() : nullptr;
         o.use_radius = spec.range ? 1 : 0;
         o.radius = spec.radius + radius_slack;
         return o;
@@ -485,6 +593,47 @@ struct DenyMask {
 };
 
 constexpr int64_t kMaxDeviceK = 1024;  // largest k of one device scan
+
+const char*
+kind_name(int kind) {
+    static const char* names[] = {"fp32", "sq8", "sq4", "sq4_uniform", "sq8_uniform", "rabitq"};
+    return kind >= 0 && kind <= VSAG_AMD_KIND_RABITQ ? names[kind] : "unknown";
+}
+
+// SearchStatistics::ToJson (src/query_context.h:215-246): distance evaluations of one call by phase and backend.  The
+// device scans do not count comparisons one by one; the figures are what the call's plan evaluates: every centroid per
+// query (routing), every code of the scanned lists or of the store (approximate), every candidate handed to the
+// rerank (at most; a list shorter than the candidate count hands over less).
+struct SearchStats {
+    uint64_t routing = 0, approximate = 0, rerank = 0;
+    int base_kind = VSAG_AMD_KIND_FP32, precise_kind = VSAG_AMD_KIND_FP32;
+
+    std::string
+    dump() const {
+        std::map<std::string, uint64_t> backend;
+        backend["fp32"] += routing;
+        backend[kind_name(base_kind)] += approximate;
+        backend[kind_name(precise_kind)] += rerank;
+        const uint64_t total = routing + approximate + rerank;
+        std::string s = "{\"is_timeout\":false,\"dist_cmp\":" + std::to_string(std::min<uint64_t>(total, 0xFFFFFFFFULL)) +
+                        ",\"hops\":0,\"io_cnt\":0,\"io_time_ms\":0,\"reorder_distance_count\":" +
+                        std::to_string(std::min<uint64_t>(rerank, 0xFFFFFFFFULL)) +
+                        ",\"distance_evaluations\":" + std::to_string(total) +
+                        ",\"distance_evaluations_by_phase\":{\"routing\":" + std::to_string(routing) +
+                        ",\"approximate\":" + std::to_string(approximate) + ",\"rerank\":" + std::to_string(rerank) +
+                        "},\"distance_evaluations_by_backend\":{";
+        bool first = true;
+        for (const auto& b : backend) {
+            if (b.second == 0) {
+                continue;
+            }
+            s += std::string(first ? "" : ",") + "\"" + b.first + "\":" + std::to_string(b.second);
+            first = false;
+        }
+        s += "},\"complete\":true}";
+        return s;
+    }
+};
 
 // One ascending row of (distance, inner id) as a single-query result dataset.
 DatasetPtr
@@ -497,6 +646,55 @@ pack_row(const std::vector<std::pair<float, uint32_t>>& row, const std::vector<i
         ids[i] = row[i].second;
     }
     return pack_results(ids, dists, 1, static_cast<int64_t>(ids.size()), labels, stats);
+}
+
+// ApplyTopkWithValidity (src/algorithm/inner_index_interface.cpp:611-669): the distances of CalDistanceById as they
+// are (topk == -1) or the topk smallest per row with their labels; unknown labels (distance -1) come last, NaN
+// distances before them.  inner[i] == VSAG_AMD_INVALID_ID marks an unknown label.
+DatasetPtr
+pack_distances(const std::vector<float>& dists, const std::vector<uint32_t>& inner, const int64_t* ids, int64_t rows,
+               int64_t count, int64_t topk) {
+    auto result = Dataset::Make();
+    const int64_t out_count = topk == -1 ? count : std::min(topk, count);
+    result->NumElements(rows)->Dim(out_count)->Owner(true);
+    if (count == 0) {
+        return result;
+    }
+    auto* out_d = new float[rows * out_count];
+    result->Distances(out_d);
+    if (topk == -1) {
+        std::copy(dists.begin(), dists.begin() + rows * count, out_d);
+        return result;
+    }
+    auto* out_ids = new int64_t[rows * out_count];
+    result->Ids(out_ids);
+    std::vector<int64_t> order(count);
+    for (int64_t r = 0; r < rows; ++r) {
+        const float* d = dists.data() + r * count;
+        const uint32_t* in = inner.data() + r * count;
+        for (int64_t i = 0; i < count; ++i) {
+            order[i] = i;
+        }
+        std::partial_sort(order.begin(), order.begin() + out_count, order.end(), [&](int64_t a, int64_t b) {
+            const bool va = in[a] != VSAG_AMD_INVALID_ID, vb = in[b] != VSAG_AMD_INVALID_ID;
+            if (va != vb) {
+                return va;
+            }
+            const bool na = std::isnan(d[a]), nb = std::isnan(d[b]);
+            if (na != nb) {
+                return !na;
+            }
+            if (na) {
+                return a < b;
+            }
+            return d[a] < d[b];
+        });
+        for (int64_t i = 0; i < out_count; ++i) {
+            out_d[r * out_count + i] = d[order[i]];
+            out_ids[r * out_count + i] = ids[r * count + order[i]];
+        }
+    }
+    return result;
 }
 
 // The search overloads of the public interface, reduced to one virtual search().
@@ -541,9 +739,70 @@ public:
         return run(query, 1, parameters, with_filter(range_spec(radius, limited_size), filter));
     }
 
+    // BruteForce::SearchWithRequest / IVF::SearchWithRequest (bruteforce.cpp:481-597, ivf.cpp:2052-2354): mode, k or
+    // radius, parameters, the bitset and the filter object (both, when both are enabled), injected buckets.
+    Expected<DatasetPtr>
+    SearchWithRequest(const SearchRequest& request) const override {
+        SearchSpec spec = request.mode_ == SearchMode::RANGE_SEARCH ? range_spec(request.radius_, request.limited_size_)
+                                                                   : SearchSpec{};
+        const BitsetPtr bits = request.enable_bitset_filter_ ? request.bitset_filter_ : nullptr;
+        const FilterPtr filter = request.enable_filter_ ? request.filter_ : nullptr;
+        if (bits != nullptr || filter != nullptr) {
+            spec.valid = [bits, filter](int64_t label) {
+                return (bits == nullptr || !bits->Test(label & 0xFFFFFFFFLL)) &&
+                       (filter == nullptr || filter->CheckValid(label));
+            };
+        }
+        if (!request.bucket_ids_.empty()) {
+            spec.bucket_ids = &request.bucket_ids_;
+        }
+        return run(request.query_, spec.range ? 1 : request.topk_, request.params_str_, spec);
+    }
+
+    Expected<DatasetPtr>
+    CalDistanceById(const float* query, const int64_t* ids, int64_t count, bool calculate_precise_distance,
+                    int64_t topk) const override {
+        return safe_call<DatasetPtr>([&]() {
+            CHECK_ARGUMENT(count >= 0, "CalDistanceById count must be non-negative");
+            CHECK_ARGUMENT(topk == -1 || topk > 0, "CalDistanceById topk must be -1 or positive");
+            if (count > 0) {
+                CHECK_ARGUMENT(query != nullptr, "CalDistanceById query must not be null");
+                CHECK_ARGUMENT(ids != nullptr, "CalDistanceById ids must not be null");
+            }
+            return distances_by_id(query, 1, ids, count, calculate_precise_distance, topk);
+        });
+    }
+    Expected<DatasetPtr>
+    CalDistanceById(const DatasetPtr& query, const int64_t* ids, int64_t count, bool calculate_precise_distance,
+                    int64_t topk) const override {
+        return safe_call<DatasetPtr>([&]() {
+            CHECK_ARGUMENT(query != nullptr, "CalDistanceById query must not be null");
+            CHECK_ARGUMENT(count >= 0, "CalDistanceById count must be non-negative");
+            CHECK_ARGUMENT(topk == -1 || topk > 0, "CalDistanceById topk must be -1 or positive");
+            CHECK_ARGUMENT(query->GetNumElements() > 0, "CalDistanceById query count must be positive");
+            if (count > 0) {
+                CHECK_ARGUMENT(ids != nullptr, "CalDistanceById ids must not be null");
+                CHECK_ARGUMENT(query->GetFloat32Vectors() != nullptr, "query.float_vector is nullptr");
+                CHECK_ARGUMENT(query->GetDim() == static_cast<int64_t>(dimension()), "query.dim must be equal to index.dim");
+            }
+            return distances_by_id(query->GetFloat32Vectors(), query->GetNumElements(), ids, count,
+                                   calculate_precise_distance, topk);
+        });
+    }
+
 protected:
     virtual DatasetPtr
     search(const DatasetPtr& query, int64_t k, const std::string& parameters, const SearchSpec& spec) const = 0;
+    // rows x count distances (row r: query r against ids[r * count ...]), packed by pack_distances.
+    virtual DatasetPtr
+    distances_by_id(const float* queries, int64_t rows, const int64_t* ids, int64_t count, bool precise,
+                    int64_t topk) const = 0;
+    virtual uint32_t
+    dimension() const = 0;
+
+    // Searches share the lock; Build / Add / Train hold it alone (bruteforce.cpp:373,1386).
+    mutable std::shared_mutex mutex_;
+    mutable ContextPool pool_;
 
 private:
     Expected<DatasetPtr>
@@ -590,7 +849,78 @@ private:
     }
 };
 
-// ------------------------------------------------------------------------------------------- brute_force
+// Labels of a CalDistanceById call as inner ids (VSAG_AMD_INVALID_ID where the label is unknown).
+std::vector<uint32_t>
+inner_ids_of(const LabelMap& known, const int64_t* ids, int64_t total) {
+    std::vector<uint32_t> inner(static_cast<size_t>(total));
+    for (int64_t i = 0; i < total; ++i) {
+        auto it = known.find(ids[i]);
+        inner[i] = it == known.end() ? VSAG_AMD_INVALID_ID : it->second;
+    }
+    return inner;
+}
+
+// Distances of `rows` queries to `count` codes each, named by inner id, from a store (chunks of queries the device
+// entry point takes at a time).
+void
+store_distances(SearchContext& ctx, const vsag_amd_store_t* store, const float* queries, int64_t rows, uint32_t dim,
+                const std::vector<uint32_t>& inner, int64_t count, uint32_t scale, std::vector<float>& out) {
+    out.assign(static_cast<size_t>(rows * count), -1.0F);
+    if (count == 0) {
+        return;
+    }
+    std::vector<uint32_t> scaled;
+    const std::vector<uint32_t>* src = &inner;
+    if (scale != 1) {
+        scaled = inner;
+        for (auto& v : scaled) {
+            v = v == VSAG_AMD_INVALID_ID ? v : v * scale;
+        }
+        src = &scaled;
+    }
+    const int64_t chunk = 32768;
+    for (int64_t r0 = 0; r0 < rows; r0 += chunk) {
+        const int64_t nr = std::min(chunk, rows - r0);
+        ctx.upload(ctx.queries, queries + r0 * dim, static_cast<size_t>(nr) * dim * 4);
+        ctx.upload(ctx.cand_ids, src->data() + r0 * count, static_cast<size_t>(nr * count) * 4);
+        ctx.out_d.reserve(static_cast<size_t>(nr * count) * 4);
+        const size_t wsb = vsag_amd_store_distances_workspace_bytes(store, nr);
+        ctx.workspace.reserve(wsb);
+        dev(vsag_amd_store_distances(store, ctx.queries.as<float>(), nr, ctx.cand_ids.as<uint32_t>(),
+                                     static_cast<uint32_t>(count), ctx.out_d.as<float>(), ctx.workspace.p, wsb, ctx.stream));
+        ctx.download(out.data() + r0 * count, ctx.out_d.p, static_cast<size_t>(nr * count) * 4);
+    }
+}
+
+DatasetPtr
+empty_result(const std::string& stats = std::string()) {
+    auto empty = Dataset::Make();
+    empty->NumElements(1)->Dim(0);
+    if (!stats.empty()) {
+        empty->Statistics(stats);
+    }
+    return empty;
+}
+
+void
+read_rabitq_params(const Json& index_param, Quantizer& q) {
+    if (index_param.Contains("rabitq_bits_per_dim_query")) {
+        q.rabitq_query_bits = static_cast<int>(index_param["rabitq_bits_per_dim_query"].GetInt());
+    }
+    if (q.kind == VSAG_AMD_KIND_RABITQ) {
+        CHECK_ARGUMENT(q.rabitq_query_bits == 4 || q.rabitq_query_bits == 32,
+                       "rabitq_bits_per_dim_query must be 4 or 32");
+        if (index_param.Contains("rabitq_bits_per_dim_base")) {
+            CHECK_ARGUMENT(index_param["rabitq_bits_per_dim_base"].GetInt() == 1,
+                           "the GPU path supports rabitq_bits_per_dim_base = 1 only");
+        }
+        if (index_param.Contains("rabitq_use_fht")) {
+            CHECK_ARGUMENT(!index_param["rabitq_use_fht"].GetBool(), "rabitq_use_fht is not supported");
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------- brute force
 class BruteForce : public GpuIndex {
 public:
     BruteForce(const CommonParam& common, const Json& index_param) {
@@ -605,26 +935,32 @@ public:
         if (index_param.Contains("base_quantization_type")) {
             q_.kind = kind_from_name(index_param["base_quantization_type"].GetString());
         }
-        if (index_param.Contains("rabitq_bits_per_dim_query")) {
-            q_.rabitq_query_bits = static_cast<int>(index_param["rabitq_bits_per_dim_query"].GetInt());
-        }
-        if (q_.kind == VSAG_AMD_KIND_RABITQ) {
-            CHECK_ARGUMENT(q_.rabitq_query_bits == 4 || q_.rabitq_query_bits == 32,
-                           "rabitq_bits_per_dim_query must be 4 or 32");
-            if (index_param.Contains("rabitq_bits_per_dim_base")) {
-                CHECK_ARGUMENT(index_param["rabitq_bits_per_dim_base"].GetInt() == 1,
-                               "the GPU path supports rabitq_bits_per_dim_base = 1 only");
+        read_rabitq_params(index_param, q_);
+    }
+
+    // BruteForce::Train (bruteforce.cpp:123-126): the quantizer of the codes is trained on the data.
+    Expected<void>
+    Train(const DatasetPtr& data) override {
+        return safe_run([&]() {
+            std::unique_lock<std::shared_mutex> lock(mutex_);
+            check_base(data, q_.dim);
+            if (q_.trained || data->GetNumElements() == 0) {
+                return;
             }
-            if (index_param.Contains("rabitq_use_fht")) {
-                CHECK_ARGUMENT(!index_param["rabitq_use_fht"].GetBool(), "rabitq_use_fht is not supported");
+            std::vector<int64_t> rows(static_cast<size_t>(data->GetNumElements()));
+            for (size_t i = 0; i < rows.size(); ++i) {
+                rows[i] = static_cast<int64_t>(i);
             }
-        }
+            DevBuf x;
+            upload_rows(data, rows, q_.dim, x);
+            q_.train(x.as<float>(), rows.size());
+        });
     }
 
     Expected<std::vector<int64_t>>
     Build(const DatasetPtr& base) override {
         return safe_call<std::vector<int64_t>>([&]() {
-            std::lock_guard<std::mutex> lock(mutex_);
+            std::unique_lock<std::shared_mutex> lock(mutex_);
             if (!labels_.empty()) {
                 throw VsagException(ErrorType::BUILD_TWICE, "failed to build index: index is not empty");
             }
@@ -635,12 +971,23 @@ public:
     Expected<std::vector<int64_t>>
     Add(const DatasetPtr& base) override {
         return safe_call<std::vector<int64_t>>([&]() {
-            std::lock_guard<std::mutex> lock(mutex_);
+            std::unique_lock<std::shared_mutex> lock(mutex_);
             return add_locked(base);
         });
     }
 
+    int64_t
+    GetNumElements() const override {
+        std::shared_lock<std::shared_mutex> lock(mutex_);
+        return static_cast<int64_t>(labels_.size());
+    }
+
 protected:
+    uint32_t
+    dimension() const override {
+        return q_.dim;
+    }
+
     DatasetPtr
     search(const DatasetPtr& query, int64_t k, const std::string& parameters, const SearchSpec& spec) const override {
         check_query(query, k, q_.dim);
@@ -648,12 +995,11 @@ protected:
             Json p = Json::Parse(parameters);  // {"parallelism": p}, optionally under "brute_force"
             CHECK_ARGUMENT(p.IsObject(), "search parameters must be a JSON object");
         }
-        std::lock_guard<std::mutex> lock(mutex_);
+        CHECK_ARGUMENT(spec.bucket_ids == nullptr, "bucket_ids_ is supported by the ivf index only");
+        std::shared_lock<std::shared_mutex> lock(mutex_);
         const int64_t nq = query->GetNumElements();
         if (labels_.empty()) {
-            auto empty = Dataset::Make();
-            empty->NumElements(1)->Dim(0);
-            return empty;
+            return empty_result();
         }
         // One device scan returns at most 1024 results per query.  A range search, and a KnnSearch with a larger
         // k, run scan after scan for one query: what a scan returned is denied to the next one, so the rows come
@@ -661,20 +1007,22 @@ protected:
         const bool looped = spec.range || k > kMaxDeviceK;
         CHECK_ARGUMENT(!looped || nq == 1, spec.range ? "range search takes one query"
                                                       : "k above 1024 is supported for one query per call");
-        queries_.reserve(static_cast<size_t>(nq) * q_.dim * 4);
-        dev(vsag_amd_memcpy_h2d(queries_.p, query->GetFloat32Vectors(), static_cast<size_t>(nq) * q_.dim * 4, nullptr));
+        auto ctx = pool_.acquire();
+        ctx->upload(ctx->queries, query->GetFloat32Vectors(), static_cast<size_t>(nq) * q_.dim * 4);
         DenyMask mask;
-        mask.init(labels_, spec.valid, looped);
-        const vsag_amd_search_options_t opt = mask.options(spec, 0.0F);
-        // distance_evaluations as the reference counts them: every stored vector once per query
-        const std::string stats = "{\"dist_cmp\":" + std::to_string(labels_.size() * static_cast<size_t>(nq)) + "}";
+        mask.init(*ctx, labels_, spec.valid, looped, 1);
+        const vsag_amd_search_options_t opt = mask.options(*ctx, spec, 0.0F);
+        // every stored vector once per query and scan
+        SearchStats stats;
+        stats.base_kind = q_.kind;
         const auto n = static_cast<int64_t>(labels_.size());
         if (!looped) {
             const auto kk = static_cast<uint32_t>(k);
             std::vector<uint32_t> ids;
             std::vector<float> dists;
-            scan(nq, kk, opt, ids, dists);
-            return pack_results(ids, dists, nq, k, labels_, stats);
+            scan(*ctx, nq, kk, opt, ids, dists);
+            stats.approximate = static_cast<uint64_t>(n) * static_cast<uint64_t>(nq);
+            return pack_results(ids, dists, nq, k, labels_, stats.dump());
         }
         std::vector<std::pair<float, uint32_t>> row;
         int64_t remaining = spec.range ? (spec.limited_size > 0 ? spec.limited_size : n) : k;
@@ -682,7 +1030,8 @@ protected:
             const auto kk = static_cast<uint32_t>(std::min<int64_t>({remaining, kMaxDeviceK, n}));
             std::vector<uint32_t> ids;
             std::vector<float> dists;
-            scan(1, kk, opt, ids, dists);
+            scan(*ctx, 1, kk, opt, ids, dists);
+            stats.approximate += static_cast<uint64_t>(n);
             uint32_t got = 0;
             while (got < kk && ids[got] != VSAG_AMD_INVALID_ID) {
                 row.emplace_back(dists[got], ids[got]);
@@ -693,38 +1042,44 @@ protected:
             if (got < kk) {
                 break;
             }
-            mask.upload();
+            mask.upload(*ctx);
         }
         if (row.empty()) {
-            auto empty = Dataset::Make();
-            empty->NumElements(1)->Dim(0)->Statistics(stats);
-            return empty;
+            return empty_result(stats.dump());
         }
-        return pack_row(row, labels_, stats);
+        return pack_row(row, labels_, stats.dump());
     }
 
-public:
-    int64_t
-    GetNumElements() const override {
-        std::lock_guard<std::mutex> lock(mutex_);
-        return static_cast<int64_t>(labels_.size());
+    // BruteForce::CalDistanceById through InnerIndexInterface (inner_index_interface.cpp:448-609): the distance the
+    // stored code gives, whatever calculate_precise_distance says (the index keeps one set of codes).
+    DatasetPtr
+    distances_by_id(const float* queries, int64_t rows, const int64_t* ids, int64_t count, bool /*precise*/,
+                    int64_t topk) const override {
+        std::shared_lock<std::shared_mutex> lock(mutex_);
+        const std::vector<uint32_t> inner = inner_ids_of(known_, ids, rows * count);
+        std::vector<float> dists(static_cast<size_t>(rows * count), -1.0F);
+        if (count > 0 && store_.s != nullptr) {
+            auto ctx = pool_.acquire();
+            store_distances(*ctx, store_.s, queries, rows, q_.dim, inner, count, 1, dists);
+        }
+        return pack_distances(dists, inner, ids, rows, count, topk);
     }
 
 private:
     // One device scan of the uploaded queries; results copied to the host.
     void
-    scan(int64_t nq, uint32_t kk, const vsag_amd_search_options_t& opt, std::vector<uint32_t>& ids,
+    scan(SearchContext& ctx, int64_t nq, uint32_t kk, const vsag_amd_search_options_t& opt, std::vector<uint32_t>& ids,
          std::vector<float>& dists) const {
-        out_ids_.reserve(static_cast<size_t>(nq) * kk * 4);
-        out_d_.reserve(static_cast<size_t>(nq) * kk * 4);
+        ctx.out_ids.reserve(static_cast<size_t>(nq) * kk * 4);
+        ctx.out_d.reserve(static_cast<size_t>(nq) * kk * 4);
         size_t wsb = vsag_amd_flat_scan_workspace_bytes(store_.s, nq, kk);
-        workspace_.reserve(wsb);
-        dev(vsag_amd_flat_scan_topk_ex(store_.s, queries_.as<float>(), nq, kk, &opt, out_ids_.as<uint32_t>(),
-                                       out_d_.as<float>(), workspace_.p, wsb, nullptr));
+        ctx.workspace.reserve(wsb);
+        dev(vsag_amd_flat_scan_topk_ex(store_.s, ctx.queries.as<float>(), nq, kk, &opt, ctx.out_ids.as<uint32_t>(),
+                                       ctx.out_d.as<float>(), ctx.workspace.p, wsb, ctx.stream));
         ids.resize(static_cast<size_t>(nq) * kk);
         dists.resize(ids.size());
-        dev(vsag_amd_memcpy_d2h(ids.data(), out_ids_.p, ids.size() * 4, nullptr));
-        dev(vsag_amd_memcpy_d2h(dists.data(), out_d_.p, dists.size() * 4, nullptr));
+        ctx.download(ids.data(), ctx.out_ids.p, ids.size() * 4);
+        ctx.download(dists.data(), ctx.out_d.p, dists.size() * 4);
     }
 
     std::vector<int64_t>
@@ -735,6 +1090,7 @@ private:
         if (rows.empty()) {
             return failed;
         }
+        CHECK_ARGUMENT(labels_.size() + rows.size() < VSAG_AMD_INVALID_ID, "the index holds at most 2^32 - 2 vectors");
         DevBuf x;
         upload_rows(base, rows, q_.dim, x);
         q_.train(x.as<float>(), rows.size());
@@ -748,10 +1104,11 @@ private:
             codes.reserve(rows.size() * q_.code_size());
             q_.encode(x.as<float>(), rows.size(), codes.as<uint8_t>());
             dev(vsag_amd_store_append(store_.s, codes.as<uint8_t>(), rows.size(), nullptr));
-            dev(vsag_amd_stream_synchronize(nullptr));
         }
         dev(vsag_amd_stream_synchronize(nullptr));
+        // the labels are recorded once the device holds the vectors: a failed insert leaves the index as it was
         for (int64_t r : rows) {
+            known_.emplace(base->GetIds()[r], static_cast<uint32_t>(labels_.size()));
             labels_.push_back(base->GetIds()[r]);
         }
         return failed;
@@ -760,9 +1117,7 @@ private:
     Quantizer q_;
     StoreHandle store_;
     std::vector<int64_t> labels_;  // inner id -> label (LabelTable)
-    std::unordered_set<int64_t> known_;
-    mutable std::mutex mutex_;
-    mutable DevBuf queries_, out_ids_, out_d_, workspace_;
+    LabelMap known_;
 };
 
 // ------------------------------------------------------------------------------------------- ivf
@@ -780,16 +1135,12 @@ public:
         reject_unknown_keys(index_param, known);
         q_.metric = common.metric;
         q_.dim = common.dim;
+        pq_.metric = common.metric;
+        pq_.dim = common.dim;
         if (index_param.Contains("base_quantization_type")) {
             q_.kind = kind_from_name(index_param["base_quantization_type"].GetString());
         }
-        if (index_param.Contains("rabitq_bits_per_dim_query")) {
-            q_.rabitq_query_bits = static_cast<int>(index_param["rabitq_bits_per_dim_query"].GetInt());
-        }
-        if (q_.kind == VSAG_AMD_KIND_RABITQ) {
-            CHECK_ARGUMENT(q_.rabitq_query_bits == 4 || q_.rabitq_query_bits == 32,
-                           "rabitq_bits_per_dim_query must be 4 or 32");
-        }
+        read_rabitq_params(index_param, q_);
         if (index_param.Contains("buckets_count")) {
             int64_t b = index_param["buckets_count"].GetInt();
             CHECK_ARGUMENT(b >= 1 && b <= (1 << 24), "buckets_count must be in [1, 2^24], got " + std::to_string(b));
@@ -799,8 +1150,15 @@ public:
             use_reorder_ = index_param["use_reorder"].GetBool();
         }
         if (index_param.Contains("precise_quantization_type")) {
-            CHECK_ARGUMENT(index_param["precise_quantization_type"].GetString() == "fp32",
-                           "the GPU path reranks with precise_quantization_type = fp32 only");
+            pq_.kind = kind_from_name(index_param["precise_quantization_type"].GetString());
+            CHECK_ARGUMENT(pq_.kind != VSAG_AMD_KIND_RABITQ, "precise_quantization_type must not be rabitq");
+        }
+        if (index_param.Contains("precise_codes_layout")) {
+            // "bucket" keeps the precise codes list by list instead of in one array (ivf.cpp:441-455); the distances are
+            // the same, and here both are one array addressed by inner id.
+            const std::string layout = index_param["precise_codes_layout"].GetString();
+            CHECK_ARGUMENT(layout == "flat" || layout == "bucket", "precise_codes_layout must be flat or bucket");
+            CHECK_ARGUMENT(layout == "flat" || use_reorder_, "precise_codes_layout=bucket requires use_reorder=true");
         }
         if (index_param.Contains("ivf_train_type")) {
             const std::string t = index_param["ivf_train_type"].GetString();
@@ -808,15 +1166,28 @@ public:
             train_random_ = t == "random";
         }
         if (index_param.Contains("buckets_per_data")) {
-            CHECK_ARGUMENT(index_param["buckets_per_data"].GetInt() == 1,
-                           "the GPU path supports buckets_per_data = 1 only");
+            // ivf_parameter.cpp:36-46
+            const int64_t b = index_param["buckets_per_data"].GetInt();
+            CHECK_ARGUMENT(b >= 1 && b <= static_cast<int64_t>(nlist_),
+                           "buckets_per_data must be in [1, buckets_count], got " + std::to_string(b));
+            CHECK_ARGUMENT(b <= 64, "the GPU path supports buckets_per_data up to 64");
+            bpd_ = static_cast<uint32_t>(b);
         }
         if (index_param.Contains("use_residual")) {
-            CHECK_ARGUMENT(!index_param["use_residual"].GetBool(), "the GPU path does not support use_residual");
+            use_residual_ = index_param["use_residual"].GetBool();
+        }
+        if (use_residual_) {
+            CHECK_ARGUMENT(q_.kind != VSAG_AMD_KIND_RABITQ, "the GPU path does not support use_residual with rabitq");
+            CHECK_ARGUMENT(!(q_.kind == VSAG_AMD_KIND_FP32 && q_.metric == VSAG_AMD_METRIC_COSINE),
+                           "the GPU path does not support use_residual with fp32 codes under cosine");
         }
         if (index_param.Contains("partition_strategy_type")) {
             CHECK_ARGUMENT(index_param["partition_strategy_type"].GetString() == "ivf",
                            "the GPU path supports the nearest-centroid partition strategy only");
+        }
+        if (index_param.Contains("graph_build_threshold")) {
+            CHECK_ARGUMENT(index_param["graph_build_threshold"].GetInt() <= 0,
+                           "the GPU path scans lists flat: graph_build_threshold must be 0");
         }
         // ivf_parameter.cpp:88-98: default max(65536, 64 * buckets_count), at least 512.
         train_sample_count_ = std::max<int64_t>(65536, 64LL * nlist_);
@@ -826,26 +1197,55 @@ public:
         }
     }
 
+    // IVF::Train (ivf.cpp:564-588).
+    Expected<void>
+    Train(const DatasetPtr& data) override {
+        return safe_run([&]() {
+            std::unique_lock<std::shared_mutex> lock(mutex_);
+            check_base(data, q_.dim);
+            if (trained_) {
+                return;
+            }
+            std::vector<int64_t> rows(static_cast<size_t>(data->GetNumElements()));
+            for (size_t i = 0; i < rows.size(); ++i) {
+                rows[i] = static_cast<int64_t>(i);
+            }
+            train_locked(data, rows, nullptr);
+        });
+    }
+
+    // IVF::Build = Train + Add (ivf.cpp:547-562).
     Expected<std::vector<int64_t>>
     Build(const DatasetPtr& base) override {
         return safe_call<std::vector<int64_t>>([&]() {
-            std::lock_guard<std::mutex> lock(mutex_);
+            std::unique_lock<std::shared_mutex> lock(mutex_);
             if (!labels_.empty()) {
                 throw VsagException(ErrorType::BUILD_TWICE, "failed to build index: index is not empty");
             }
-            return add_locked(base);
+            return add_locked(base, true);
         });
     }
 
     Expected<std::vector<int64_t>>
     Add(const DatasetPtr& base) override {
         return safe_call<std::vector<int64_t>>([&]() {
-            std::lock_guard<std::mutex> lock(mutex_);
-            return add_locked(base);
+            std::unique_lock<std::shared_mutex> lock(mutex_);
+            return add_locked(base, false);
         });
     }
 
+    int64_t
+    GetNumElements() const override {
+        std::shared_lock<std::shared_mutex> lock(mutex_);
+        return static_cast<int64_t>(labels_.size());
+    }
+
 protected:
+    uint32_t
+    dimension() const override {
+        return q_.dim;
+    }
+
     DatasetPtr
     search(const DatasetPtr& query, int64_t k, const std::string& parameters, const SearchSpec& spec) const override {
         check_query(query, k, q_.dim);
@@ -865,17 +1265,35 @@ protected:
         if (ivf.Contains("enable_reorder")) {
             enable_reorder = ivf["enable_reorder"].GetBool();
         }
-        bool disable_scan = ivf.Contains("disable_bucket_scan") && ivf["disable_bucket_scan"].GetBool();
-
-        std::lock_guard<std::mutex> lock(mutex_);
+        const bool disable_scan = ivf.Contains("disable_bucket_scan") && ivf["disable_bucket_scan"].GetBool();
         const int64_t nq = query->GetNumElements();
+        if (spec.bucket_ids != nullptr) {
+            // IVF::SearchWithRequest (ivf.cpp:2076-2110)
+            CHECK_ARGUMENT(static_cast<int64_t>(spec.bucket_ids->size()) == nq,
+                           "bucket_ids_ size must match the number of query vectors; got " +
+                               std::to_string(spec.bucket_ids->size()) + " bucket lists for " + std::to_string(nq) +
+                               " queries");
+            CHECK_ARGUMENT(!disable_scan, "bucket_ids_ is incompatible with disable_bucket_scan mode");
+            for (size_t qi = 0; qi < spec.bucket_ids->size(); ++qi) {
+                const auto& ids = (*spec.bucket_ids)[qi];
+                CHECK_ARGUMENT(!ids.empty(), "bucket_ids_[" + std::to_string(qi) +
+                                                 "] must not be empty; use empty outer vector for default routing");
+                std::set<int64_t> seen;
+                for (int64_t id : ids) {
+                    CHECK_ARGUMENT(id >= 0 && id < static_cast<int64_t>(nlist_),
+                                   "bucket_id " + std::to_string(id) + " out of range [0, " + std::to_string(nlist_) + ")");
+                    CHECK_ARGUMENT(seen.insert(id).second, "duplicate bucket_id " + std::to_string(id));
+                }
+            }
+        }
+
+        std::shared_lock<std::shared_mutex> lock(mutex_);
+        check_usable();
         if (labels_.empty()) {
-            auto empty = Dataset::Make();
-            empty->NumElements(1)->Dim(0);
-            return empty;
+            return empty_result();
         }
         const auto n = static_cast<int64_t>(labels_.size());
-        const auto nprobe = static_cast<uint32_t>(std::min<int64_t>(scan, nlist_));  // ivf.cpp:1573-1574
+        uint32_t nprobe = static_cast<uint32_t>(std::min<int64_t>(scan, nlist_));  // ivf.cpp:1573-1574
         const bool reorder = use_reorder_ && enable_reorder;
         if (reorder) {
             CHECK_ARGUMENT(factor > 0.0F, "factor must be positive when use_reorder is true");
@@ -885,46 +1303,93 @@ protected:
             kcand = std::max<int64_t>(static_cast<int64_t>(factor * static_cast<float>(k)), 1);  // ivf.cpp:2316
         }
         // One device scan returns at most 1024 candidates per query; more (and every range search) run scan
-        // after scan for one query, each denied what the earlier ones returned.
-        const bool looped = spec.range || kcand > kMaxDeviceK;
-        CHECK_ARGUMENT(!looped || nq == 1, spec.range ? "range search takes one query"
-                                                      : "factor * k above 1024 is supported for one query per call");
+        // after scan for one query, each denied what the earlier ones returned.  With buckets_per_data = b a vector
+        // has b postings, so a scan asks for b times the candidates (ivf.cpp:1722-1730).
+        const bool looped = spec.range || kcand * bpd_ > kMaxDeviceK;
+        CHECK_ARGUMENT(!looped || nq == 1,
+                       spec.range ? "range search takes one query"
+                                  : "factor * k * buckets_per_data above 1024 is supported for one query per call");
 
-        queries_.reserve(static_cast<size_t>(nq) * q_.dim * 4);
-        dev(vsag_amd_memcpy_h2d(queries_.p, query->GetFloat32Vectors(), static_cast<size_t>(nq) * q_.dim * 4, nullptr));
-        // 1. route (exact nearest centroids)
-        buckets_.reserve(static_cast<size_t>(nq) * nprobe * 4);
-        bucket_d_.reserve(static_cast<size_t>(nq) * nprobe * 4);
-        size_t wsb = vsag_amd_ivf_route_workspace_bytes(centroid_store_.s, nq, nprobe);
-        workspace_.reserve(wsb);
-        dev(vsag_amd_ivf_route(centroid_store_.s, queries_.as<float>(), nq, nprobe, buckets_.as<int32_t>(),
-                               bucket_d_.as<float>(), workspace_.p, wsb, nullptr));
+        auto lease = pool_.acquire();
+        SearchContext& ctx = *lease;
+        ctx.upload(ctx.queries, query->GetFloat32Vectors(), static_cast<size_t>(nq) * q_.dim * 4);
+        SearchStats stats;
+        stats.base_kind = q_.kind;
+        stats.precise_kind = pq_.kind;
+        if (spec.bucket_ids != nullptr) {
+            // the caller names the lists (ivf.cpp:1702-1706); shorter rows are padded with "no list"
+            size_t widest = 0;
+            for (const auto& ids : *spec.bucket_ids) {
+                widest = std::max(widest, ids.size());
+            }
+            nprobe = static_cast<uint32_t>(widest);
+            std::vector<int32_t> padded(static_cast<size_t>(nq) * nprobe, -1);
+            for (int64_t qi = 0; qi < nq; ++qi) {
+                const auto& ids = (*spec.bucket_ids)[qi];
+                for (size_t j = 0; j < ids.size(); ++j) {
+                    padded[qi * nprobe + j] = static_cast<int32_t>(ids[j]);
+                }
+            }
+            ctx.upload(ctx.buckets, padded.data(), padded.size() * 4);
+        } else {
+            // 1. route (exact nearest centroids)
+            ctx.buckets.reserve(static_cast<size_t>(nq) * nprobe * 4);
+            ctx.bucket_d.reserve(static_cast<size_t>(nq) * nprobe * 4);
+            const size_t wsb = vsag_amd_ivf_route_workspace_bytes(centroid_store_.s, nq, nprobe);
+            ctx.workspace.reserve(wsb);
+            dev(vsag_amd_ivf_route(centroid_store_.s, ctx.queries.as<float>(), nq, nprobe, ctx.buckets.as<int32_t>(),
+                                   ctx.bucket_d.as<float>(), ctx.workspace.p, wsb, ctx.stream));
+            stats.routing = static_cast<uint64_t>(nq) * nlist_;
+        }
         if (disable_scan && !spec.range) {
             // routing only: bucket ids + centroid distances (ivf.cpp:1589-1660)
             std::vector<uint32_t> ids(static_cast<size_t>(nq) * nprobe);
             std::vector<float> dists(ids.size());
-            dev(vsag_amd_memcpy_d2h(ids.data(), buckets_.p, ids.size() * 4, nullptr));
-            dev(vsag_amd_memcpy_d2h(dists.data(), bucket_d_.p, dists.size() * 4, nullptr));
+            ctx.download(ids.data(), ctx.buckets.p, ids.size() * 4);
+            ctx.download(dists.data(), ctx.bucket_d.p, dists.size() * 4);
             std::vector<int64_t> identity(nlist_);
             for (uint32_t i = 0; i < nlist_; ++i) {
                 identity[i] = i;
             }
-            return pack_results(ids, dists, nq, nprobe, identity, "{}");
+            return pack_results(ids, dists, nq, nprobe, identity, stats.dump());
         }
+        const uint64_t probed = probed_codes(ctx, nq, nprobe);
         DenyMask mask;
-        mask.init(labels_, spec.valid, looped);
+        mask.init(ctx, labels_, spec.valid, looped, bpd_);
         // FlatBucketSearcher compares against radius + THRESHOLD_ERROR (flat_bucket_searcher.cpp:121,
         // impl/searcher/basic_searcher.h:39).
-        const vsag_amd_search_options_t opt = mask.options(spec, 2e-6F);
+        const vsag_amd_search_options_t opt = mask.options(ctx, spec, 2e-6F);
 
         if (!looped) {
             // 2. scan the probed lists; 3. exact rerank, best min(k, candidates) kept (flatten_reorder.cpp:77)
+            const auto kc = static_cast<uint32_t>(kcand * bpd_);
             const int64_t kout = reorder ? std::min<int64_t>(k, kcand) : kcand;
+            scan_lists(ctx, nq, nprobe, kc, opt);
+            stats.approximate = probed;
             std::vector<uint32_t> ids;
             std::vector<float> dists;
-            scan_lists(nq, nprobe, static_cast<uint32_t>(kcand), opt, reorder ? static_cast<uint32_t>(kout) : 0U, ids,
-                       dists);
-            return pack_results(ids, dists, nq, kout, labels_, "{}");
+            if (bpd_ == 1 && reorder && pq_.kind == VSAG_AMD_KIND_FP32) {
+                // the whole batch stays on the device
+                ctx.out_ids.reserve(static_cast<size_t>(nq) * kout * 4);
+                ctx.out_d.reserve(static_cast<size_t>(nq) * kout * 4);
+                dev(vsag_amd_rerank_fp32(raw_.as<float>(), labels_.size(), q_.dim, q_.metric, ctx.queries.as<float>(), nq,
+                                         ctx.cand_ids.as<uint32_t>(), kc, static_cast<uint32_t>(kout),
+                                         ctx.out_ids.as<uint32_t>(), ctx.out_d.as<float>(), ctx.stream));
+                fetch(ctx, ctx.out_ids, ctx.out_d, static_cast<size_t>(nq) * kout, ids, dists);
+                stats.rerank = static_cast<uint64_t>(nq) * kc;  // at most: lists may hold fewer candidates
+                return pack_results(ids, dists, nq, kout, labels_, stats.dump());
+            }
+            fetch(ctx, ctx.cand_ids, ctx.cand_d, static_cast<size_t>(nq) * kc, ids, dists);
+            if (bpd_ > 1) {
+                merge_postings(ids, dists, nq, kc, static_cast<uint32_t>(kcand));
+            }
+            if (reorder) {
+                std::vector<uint32_t> best;
+                std::vector<float> best_d;
+                stats.rerank = rerank(ctx, nq, ids, static_cast<uint32_t>(kcand), static_cast<uint32_t>(kout), best, best_d);
+                return pack_results(best, best_d, nq, kout, labels_, stats.dump());
+            }
+            return pack_results(ids, dists, nq, kout, labels_, stats.dump());
         }
         // Range (ivf.cpp:2282-2307): candidates within the radius by the list codes, at most factor *
         // limited_size of them when a rerank follows; the rerank keeps the nearest limited_size (all of them
@@ -939,81 +1404,229 @@ protected:
             }
         }
         std::vector<std::pair<float, uint32_t>> row;
+        std::unordered_set<uint32_t> seen;
         int64_t remaining = want;
         while (remaining > 0) {
-            const auto kc = static_cast<uint32_t>(std::min<int64_t>({remaining, kMaxDeviceK, n}));
+            const auto kc = static_cast<uint32_t>(
+                std::min<int64_t>({remaining * bpd_, kMaxDeviceK, n * static_cast<int64_t>(bpd_)}));
+            scan_lists(ctx, 1, nprobe, kc, opt);
+            stats.approximate += probed;
             std::vector<uint32_t> ids;
             std::vector<float> dists;
-            scan_lists(1, nprobe, kc, opt, reorder ? kc : 0U, ids, dists);
+            fetch(ctx, ctx.cand_ids, ctx.cand_d, kc, ids, dists);
             uint32_t got = 0;
             while (got < kc && ids[got] != VSAG_AMD_INVALID_ID) {
-                row.emplace_back(dists[got], ids[got]);
-                mask.deny(ids[got]);
+                // ascending: the first posting of a vector carries its smallest distance (ivf.cpp:1799-1812)
+                const uint32_t origin = ids[got] / bpd_;
+                if (remaining > 0 && seen.insert(origin).second) {
+                    row.emplace_back(dists[got], origin);
+                    mask.deny(origin);
+                    --remaining;
+                }
                 ++got;
             }
-            remaining -= got;
             if (got < kc) {
                 break;
             }
-            mask.upload();
+            mask.upload(ctx);
         }
-        if (reorder) {
-            // batches were reranked one by one: order the whole row by exact distance
-            std::sort(row.begin(), row.end());
-            if (static_cast<int64_t>(row.size()) > keep) {
-                row.resize(static_cast<size_t>(keep));
+        if (reorder && !row.empty()) {
+            // exact distances of everything gathered, a device call per 1024 candidates
+            std::vector<std::pair<float, uint32_t>> exact;
+            for (size_t i0 = 0; i0 < row.size(); i0 += kMaxDeviceK) {
+                const auto m = static_cast<uint32_t>(std::min<size_t>(kMaxDeviceK, row.size() - i0));
+                std::vector<uint32_t> cand(m);
+                for (uint32_t i = 0; i < m; ++i) {
+                    cand[i] = row[i0 + i].second;
+                }
+                std::vector<uint32_t> best;
+                std::vector<float> best_d;
+                stats.rerank += rerank(ctx, 1, cand, m, m, best, best_d);
+                for (uint32_t i = 0; i < m && best[i] != VSAG_AMD_INVALID_ID; ++i) {
+                    exact.emplace_back(best_d[i], best[i]);
+                }
             }
+            std::sort(exact.begin(), exact.end());
+            if (static_cast<int64_t>(exact.size()) > keep) {
+                exact.resize(static_cast<size_t>(keep));
+            }
+            row.swap(exact);
         }
         if (row.empty()) {
-            auto empty = Dataset::Make();
-            empty->NumElements(1)->Dim(0)->Statistics("{}");
-            return empty;
+            return empty_result(stats.dump());
         }
-        return pack_row(row, labels_, "{}");
+        return pack_row(row, labels_, stats.dump());
     }
 
-public:
-    int64_t
-    GetNumElements() const override {
-        std::lock_guard<std::mutex> lock(mutex_);
-        return static_cast<int64_t>(labels_.size());
+    // IVF::CalDistanceById (ivf.cpp:2429-2508): the precise codes when the index reorders and the caller asks for
+    // precise distances, else the codes of the lists (the first posting of the vector, ivf.cpp:670-675).
+    DatasetPtr
+    distances_by_id(const float* queries, int64_t rows, const int64_t* ids, int64_t count, bool precise,
+                    int64_t topk) const override {
+        std::shared_lock<std::shared_mutex> lock(mutex_);
+        check_usable();
+        const std::vector<uint32_t> inner = inner_ids_of(known_, ids, rows * count);
+        std::vector<float> dists(static_cast<size_t>(rows * count), -1.0F);
+        if (count > 0 && !labels_.empty()) {
+            auto lease = pool_.acquire();
+            SearchContext& ctx = *lease;
+            if (use_reorder_ && precise && pq_.kind == VSAG_AMD_KIND_FP32) {
+                const int64_t chunk = 32768;
+                for (int64_t r0 = 0; r0 < rows; r0 += chunk) {
+                    const int64_t nr = std::min(chunk, rows - r0);
+                    ctx.upload(ctx.queries, queries + r0 * q_.dim, static_cast<size_t>(nr) * q_.dim * 4);
+                    ctx.upload(ctx.cand_ids, inner.data() + r0 * count, static_cast<size_t>(nr * count) * 4);
+                    ctx.out_d.reserve(static_cast<size_t>(nr * count) * 4);
+                    dev(vsag_amd_rows_distances_fp32(raw_.as<float>(), labels_.size(), q_.dim, q_.metric,
+                                                     ctx.queries.as<float>(), nr, ctx.cand_ids.as<uint32_t>(),
+                                                     static_cast<uint32_t>(count), ctx.out_d.as<float>(), ctx.stream));
+                    ctx.download(dists.data() + r0 * count, ctx.out_d.p, static_cast<size_t>(nr * count) * 4);
+                }
+            } else if (use_reorder_ && precise) {
+                store_distances(ctx, precise_.s, queries, rows, q_.dim, inner, count, 1, dists);
+            } else {
+                store_distances(ctx, lists_.s, queries, rows, q_.dim, inner, count, bpd_, dists);
+            }
+        }
+        return pack_distances(dists, inner, ids, rows, count, topk);
     }
 
 private:
-    // Scan of the routed lists for the uploaded queries, then (rerank_k > 0) the exact fp32 rerank that keeps
-    // rerank_k; results copied to the host, kcand or rerank_k per query.
     void
-    scan_lists(int64_t nq, uint32_t nprobe, uint32_t kcand, const vsag_amd_search_options_t& opt, uint32_t rerank_k,
-               std::vector<uint32_t>& ids, std::vector<float>& dists) const {
-        cand_ids_.reserve(static_cast<size_t>(nq) * kcand * 4);
-        cand_d_.reserve(static_cast<size_t>(nq) * kcand * 4);
-        size_t wsb = vsag_amd_ivf_scan_workspace_bytes(lists_.s, nq, nprobe, kcand);
-        workspace_.reserve(wsb);
-        dev(vsag_amd_ivf_scan_topk_ex(lists_.s, queries_.as<float>(), nq, buckets_.as<int32_t>(), nprobe, kcand, &opt,
-                                      cand_ids_.as<uint32_t>(), cand_d_.as<float>(), workspace_.p, wsb, nullptr));
-        const DevBuf* final_ids = &cand_ids_;
-        const DevBuf* final_d = &cand_d_;
-        uint32_t kout = kcand;
-        if (rerank_k > 0) {
-            kout = rerank_k;
-            out_ids_.reserve(static_cast<size_t>(nq) * kout * 4);
-            out_d_.reserve(static_cast<size_t>(nq) * kout * 4);
-            dev(vsag_amd_rerank_fp32(raw_.as<float>(), labels_.size(), q_.dim, q_.metric, queries_.as<float>(), nq,
-                                     cand_ids_.as<uint32_t>(), kcand, kout, out_ids_.as<uint32_t>(), out_d_.as<float>(),
-                                     nullptr));
-            final_ids = &out_ids_;
-            final_d = &out_d_;
+    check_usable() const {
+        if (broken_) {
+            throw VsagException(ErrorType::INTERNAL_ERROR, "an insert failed part-way on the device: the index is unusable");
         }
-        ids.resize(static_cast<size_t>(nq) * kout);
-        dists.resize(ids.size());
-        dev(vsag_amd_memcpy_d2h(ids.data(), final_ids->p, ids.size() * 4, nullptr));
-        dev(vsag_amd_memcpy_d2h(dists.data(), final_d->p, dists.size() * 4, nullptr));
     }
 
-    // IVF::Train (ivf.cpp:564-588): sample, k-means (25 iterations, hard-coded in
-    // ivf_nearest_partition.cpp:65-70), quantizer training on the same sample.
+    static void
+    fetch(SearchContext& ctx, const DevBuf& ids_dev, const DevBuf& d_dev, size_t count, std::vector<uint32_t>& ids,
+          std::vector<float>& dists) {
+        ids.resize(count);
+        dists.resize(count);
+        ctx.download(ids.data(), ids_dev.p, count * 4);
+        ctx.download(dists.data(), d_dev.p, count * 4);
+    }
+
+    // Codes in the lists of ctx.buckets, over all (query, list) pairs.
+    uint64_t
+    probed_codes(SearchContext& ctx, int64_t nq, uint32_t nprobe) const {
+        ctx.scalar.reserve(8);
+        dev(vsag_amd_ivf_probed_codes(lists_.s, ctx.buckets.as<int32_t>(), nq, nprobe, ctx.scalar.as<uint64_t>(),
+                                      ctx.stream));
+        uint64_t total = 0;
+        ctx.download(&total, ctx.scalar.p, 8);
+        return total;
+    }
+
+    // Scan of the lists in ctx.buckets for the uploaded queries: kc (distance, posting id) per query, ascending, in
+    // ctx.cand_ids / ctx.cand_d.
     void
-    train(const DatasetPtr& base, const std::vector<int64_t>& rows, const DevBuf& x_all) {
+    scan_lists(SearchContext& ctx, int64_t nq, uint32_t nprobe, uint32_t kc, const vsag_amd_search_options_t& opt) const {
+        ctx.cand_ids.reserve(static_cast<size_t>(nq) * kc * 4);
+        ctx.cand_d.reserve(static_cast<size_t>(nq) * kc * 4);
+        const size_t wsb = vsag_amd_ivf_scan_workspace_bytes(lists_.s, nq, nprobe, kc);
+        ctx.workspace.reserve(wsb);
+        dev(vsag_amd_ivf_scan_topk_ex(lists_.s, ctx.queries.as<float>(), nq, ctx.buckets.as<int32_t>(), nprobe, kc, &opt,
+                                      ctx.cand_ids.as<uint32_t>(), ctx.cand_d.as<float>(), ctx.workspace.p, wsb,
+                                      ctx.stream));
+    }
+
+    // Posting ids to vectors (ivf.cpp:1799-1826): per query the smallest distance of every vector, ascending, the best
+    // `keep` kept.  The rows shrink from kc to keep entries.
+    void
+    merge_postings(std::vector<uint32_t>& ids, std::vector<float>& dists, int64_t nq, uint32_t kc, uint32_t keep) const {
+        std::vector<uint32_t> out_ids(static_cast<size_t>(nq) * keep, VSAG_AMD_INVALID_ID);
+        std::vector<float> out_d(out_ids.size(), std::numeric_limits<float>::infinity());
+        std::unordered_set<uint32_t> seen;
+        for (int64_t q = 0; q < nq; ++q) {
+            seen.clear();
+            uint32_t w = 0;
+            for (uint32_t i = 0; i < kc && w < keep; ++i) {
+                const uint32_t id = ids[q * kc + i];
+                if (id == VSAG_AMD_INVALID_ID) {
+                    break;
+                }
+                if (seen.insert(id / bpd_).second) {
+                    out_ids[q * keep + w] = id / bpd_;
+                    out_d[q * keep + w] = dists[q * kc + i];
+                    ++w;
+                }
+            }
+        }
+        ids.swap(out_ids);
+        dists.swap(out_d);
+    }
+
+    // FlattenReorder::Reorder (impl/reorder/flatten_reorder.cpp:52-114): distances of the candidates (nq x kcand inner
+    // ids, VSAG_AMD_INVALID_ID = none) by the precise codes, the best `keep` per query, ascending.  Returns the number
+    // of distances evaluated.
+    uint64_t
+    rerank(SearchContext& ctx, int64_t nq, const std::vector<uint32_t>& cand, uint32_t kcand, uint32_t keep,
+           std::vector<uint32_t>& ids, std::vector<float>& dists) const {
+        uint64_t evaluated = 0;
+        for (uint32_t id : cand) {
+            evaluated += id != VSAG_AMD_INVALID_ID ? 1 : 0;
+        }
+        ctx.upload(ctx.cand_ids, cand.data(), cand.size() * 4);
+        if (pq_.kind == VSAG_AMD_KIND_FP32) {
+            ctx.out_ids.reserve(static_cast<size_t>(nq) * keep * 4);
+            ctx.out_d.reserve(static_cast<size_t>(nq) * keep * 4);
+            dev(vsag_amd_rerank_fp32(raw_.as<float>(), labels_.size(), q_.dim, q_.metric, ctx.queries.as<float>(), nq,
+                                     ctx.cand_ids.as<uint32_t>(), kcand, keep, ctx.out_ids.as<uint32_t>(),
+                                     ctx.out_d.as<float>(), ctx.stream));
+            fetch(ctx, ctx.out_ids, ctx.out_d, static_cast<size_t>(nq) * keep, ids, dists);
+            return evaluated;
+        }
+        ctx.out_d.reserve(static_cast<size_t>(nq) * kcand * 4);
+        const size_t wsb = vsag_amd_store_distances_workspace_bytes(precise_.s, nq);
+        ctx.workspace.reserve(wsb);
+        dev(vsag_amd_store_distances(precise_.s, ctx.queries.as<float>(), nq, ctx.cand_ids.as<uint32_t>(), kcand,
+                                     ctx.out_d.as<float>(), ctx.workspace.p, wsb, ctx.stream));
+        std::vector<float> exact(static_cast<size_t>(nq) * kcand);
+        ctx.download(exact.data(), ctx.out_d.p, exact.size() * 4);
+        ids.assign(static_cast<size_t>(nq) * keep, VSAG_AMD_INVALID_ID);
+        dists.assign(ids.size(), std::numeric_limits<float>::infinity());
+        std::vector<std::pair<float, uint32_t>> row;
+        for (int64_t q = 0; q < nq; ++q) {
+            row.clear();
+            for (uint32_t i = 0; i < kcand; ++i) {
+                if (cand[q * kcand + i] != VSAG_AMD_INVALID_ID) {
+                    row.emplace_back(exact[q * kcand + i], cand[q * kcand + i]);
+                }
+            }
+            std::sort(row.begin(), row.end());
+            for (uint32_t i = 0; i < keep && i < row.size(); ++i) {
+                dists[q * keep + i] = row[i].first;
+                ids[q * keep + i] = row[i].second;
+            }
+        }
+        return evaluated;
+    }
+
+    // The nearest `per_row` centroids of n rows under the index metric (IVFNearestPartition::ClassifyDatas,
+    // ivf_nearest_partition.cpp:88-147, exact instead of through the router graph): n x per_row list numbers.
+    void
+    classify(const float* x_dev, uint64_t n, uint32_t per_row, DevBuf& buckets) const {
+        buckets.reserve(std::max<size_t>(n * per_row * 4, 4));
+        DevBuf d, ws;
+        const uint64_t chunk = 65536;
+        d.reserve(std::min(n, chunk) * per_row * 4);
+        for (uint64_t r0 = 0; r0 < n; r0 += chunk) {
+            const uint64_t nr = std::min(chunk, n - r0);
+            const size_t wsb = vsag_amd_ivf_route_workspace_bytes(centroid_store_.s, nr, per_row);
+            ws.reserve(wsb);
+            dev(vsag_amd_ivf_route(centroid_store_.s, x_dev + r0 * q_.dim, nr, per_row,
+                                   buckets.as<int32_t>() + r0 * per_row, d.as<float>(), ws.p, wsb, nullptr));
+        }
+        dev(vsag_amd_stream_synchronize(nullptr));
+    }
+
+    // IVF::Train (ivf.cpp:564-588): sample, k-means (25 iterations, hard-coded in ivf_nearest_partition.cpp:65-70),
+    // quantizer training on the same sample (on its residuals with use_residual, bucket_datacell.h:594-619); the
+    // precise quantizer is trained on all of the data.  x_all_dev: the rows on the device when the caller has them.
+    void
+    train_locked(const DatasetPtr& base, const std::vector<int64_t>& rows, const float* x_all_dev) {
         const uint64_t n = rows.size();
         uint64_t sample_n = std::min<uint64_t>(n, static_cast<uint64_t>(train_sample_count_));
         if (n < nlist_) {
@@ -1040,35 +1653,88 @@ private:
         dev(vsag_amd_memcpy_h2d(sample_dev.p, sample.data(), sample.size() * 4, nullptr));
         // Initial centroids: the first nlist rows of the shuffled sample (random-sample initialisation;
         // the reference defaults to k-means++ drawn from std::random_device).
-        centroids_.reserve(static_cast<size_t>(nlist_) * q_.dim * 4);
-        dev(vsag_amd_memcpy_d2d(centroids_.p, sample_dev.p, static_cast<size_t>(nlist_) * q_.dim * 4, nullptr));
+        DevBuf centroids;
+        centroids.reserve(static_cast<size_t>(nlist_) * q_.dim * 4);
+        dev(vsag_amd_memcpy_d2d(centroids.p, sample_dev.p, static_cast<size_t>(nlist_) * q_.dim * 4, nullptr));
         if (!train_random_) {
             DevBuf labels, ws;
             labels.reserve(sample_n * 4);
             size_t wsb = vsag_amd_kmeans_run_workspace_bytes(sample_n, q_.dim, nlist_);
             ws.reserve(wsb);
             double loss = 0;
-            dev(vsag_amd_kmeans_run(sample_dev.as<float>(), sample_n, q_.dim, centroids_.as<float>(), nlist_, 25, 47,
+            dev(vsag_amd_kmeans_run(sample_dev.as<float>(), sample_n, q_.dim, centroids.as<float>(), nlist_, 25, 47,
                                     labels.as<int32_t>(), &loss, ws.p, wsb, nullptr));
         }
-        // Router: an fp32 store of the centroids under the index metric (cosine normalises them,
-        // ivf_nearest_partition.cpp:81-85).
+        if (q_.metric == VSAG_AMD_METRIC_COSINE) {
+            // the router keeps unit centroids (ivf_nearest_partition.cpp:81-85), and so do the residuals
+            std::vector<float> c(static_cast<size_t>(nlist_) * q_.dim);
+            dev(vsag_amd_memcpy_d2h(c.data(), centroids.p, c.size() * 4, nullptr));
+            for (uint32_t l = 0; l < nlist_; ++l) {
+                float* row = c.data() + static_cast<size_t>(l) * q_.dim;
+                float s = 0.0F;
+                for (uint32_t d = 0; d < q_.dim; ++d) {
+                    s += row[d] * row[d];
+                }
+                const float norm = std::sqrt(s);
+                for (uint32_t d = 0; d < q_.dim && norm > 0.0F; ++d) {
+                    row[d] /= norm;
+                }
+            }
+            dev(vsag_amd_memcpy_h2d(centroids.p, c.data(), c.size() * 4, nullptr));
+        }
+        // Router: an fp32 store of the centroids under the index metric.
         Quantizer cq;
         cq.kind = VSAG_AMD_KIND_FP32;
         cq.metric = q_.metric;
         cq.dim = q_.dim;
-        centroid_store_.s = cq.make_store();
-        dev(vsag_amd_store_append(centroid_store_.s, centroids_.as<uint8_t>(), nlist_, nullptr));
-        q_.train(sample_dev.as<float>(), sample_n);
-        lists_.s = q_.make_store();
+        StoreHandle router;
+        router.s = cq.make_store();
+        dev(vsag_amd_store_append(router.s, centroids.as<uint8_t>(), nlist_, nullptr));
         dev(vsag_amd_stream_synchronize(nullptr));
-        (void)x_all;
+        std::swap(centroid_store_.s, router.s);
+        centroids_.release();
+        std::swap(centroids_.p, centroids.p);
+        std::swap(centroids_.bytes, centroids.bytes);
+        if (use_residual_) {
+            DevBuf nearest, residuals;
+            classify(sample_dev.as<float>(), sample_n, 1, nearest);
+            residuals.reserve(sample.size() * 4);
+            dev(vsag_amd_residual_rows(sample_dev.as<float>(), sample_n, q_.dim, q_.metric, nearest.as<int32_t>(),
+                                       centroids_.as<float>(), residuals.as<float>(), nullptr));
+            q_.train(residuals.as<float>(), sample_n);
+        } else {
+            q_.train(sample_dev.as<float>(), sample_n);
+        }
+        StoreHandle lists;
+        lists.s = q_.make_store();
+        if (use_residual_) {
+            dev(vsag_amd_store_set_residual(lists.s, centroids_.as<float>(), nlist_, nullptr));
+        }
+        dev(vsag_amd_store_set_lists(lists.s, nullptr, nullptr, 0, nlist_, nullptr));
+        if (use_reorder_ && pq_.kind != VSAG_AMD_KIND_FP32) {
+            DevBuf x;
+            if (x_all_dev == nullptr) {
+                upload_rows(base, rows, q_.dim, x);
+                x_all_dev = x.as<float>();
+            }
+            pq_.train(x_all_dev, n);
+            StoreHandle precise;
+            precise.s = pq_.make_store();
+            std::swap(precise_.s, precise.s);
+        }
+        dev(vsag_amd_stream_synchronize(nullptr));
+        std::swap(lists_.s, lists.s);
         trained_ = true;
     }
 
+    // IVF::Add (ivf.cpp:590-724).
     std::vector<int64_t>
-    add_locked(const DatasetPtr& base) {
+    add_locked(const DatasetPtr& base, bool train_first) {
+        check_usable();
         check_base(base, q_.dim);
+        if (!train_first && !trained_) {
+            throw VsagException(ErrorType::INTERNAL_ERROR, "ivf index add without train error");
+        }
         std::vector<int64_t> rows;
         std::vector<int64_t> failed = split_new_rows(base, known_, rows);
         if (rows.empty()) {
@@ -1076,64 +1742,86 @@ private:
         }
         const uint64_t n_new = rows.size();
         const uint64_t n_old = labels_.size();
+        CHECK_ARGUMENT((n_old + n_new) * bpd_ < VSAG_AMD_INVALID_ID, "the lists hold at most 2^32 - 2 postings");
         DevBuf x;
         upload_rows(base, rows, q_.dim, x);
         if (!trained_) {
-            try {
-                train(base, rows, x);
-            } catch (...) {
-                for (int64_t r : rows) {
-                    known_.erase(base->GetIds()[r]);
-                }
-                throw;
-            }
+            train_locked(base, rows, x.as<float>());
         }
-        // IVFPartitionStrategy::ClassifyDatas with exact nearest centroids: k-means assignment always
-        // measures plain L2 on the raw vectors (ivf_nearest_partition.cpp:63-70).
-        bucket_labels_.grow((n_old + n_new) * 4, n_old * 4);
-        {
-            DevBuf ws;
-            size_t wsb = vsag_amd_kmeans_assign_workspace_bytes(n_new, q_.dim, nlist_);
-            ws.reserve(wsb);
-            dev(vsag_amd_kmeans_assign(x.as<float>(), n_new, q_.dim, centroids_.as<float>(), nlist_,
-                                       bucket_labels_.as<int32_t>() + n_old, nullptr, nullptr, ws.p, wsb, nullptr));
+        // the lists of every row, nearest first; posting (i, j) is row i in list buckets[i * bpd + j]
+        DevBuf buckets;
+        classify(x.as<float>(), n_new, bpd_, buckets);
+        const uint64_t postings = n_new * bpd_;
+        DevBuf expanded;
+        const float* xe = x.as<float>();
+        if (bpd_ > 1) {
+            upload_rows(base, rows, q_.dim, expanded, bpd_);
+            xe = expanded.as<float>();
+        }
+        DevBuf residuals, codes, bias;
+        if (use_residual_) {
+            residuals.reserve(postings * q_.dim * 4);
+            dev(vsag_amd_residual_rows(xe, postings, q_.dim, q_.metric, buckets.as<int32_t>(), centroids_.as<float>(),
+                                       residuals.as<float>(), nullptr));
+            xe = residuals.as<float>();
+        }
+        const uint8_t* code_src = reinterpret_cast<const uint8_t*>(xe);
+        if (q_.kind != VSAG_AMD_KIND_FP32) {
+            codes.reserve(postings * q_.code_size());
+            q_.encode(xe, postings, codes.as<uint8_t>());
+            code_src = codes.as<uint8_t>();
+        }
+        const float* bias_src = nullptr;
+        if (use_residual_ && q_.metric == VSAG_AMD_METRIC_L2) {
+            DevBuf decoded;
+            bias.reserve(postings * 4);
+            decoded.reserve(postings * q_.dim * 4);
+            dev(vsag_amd_residual_bias(lists_.s, code_src, postings, buckets.as<int32_t>(), centroids_.as<float>(),
+                                       bias.as<float>(), decoded.as<float>(), nullptr));
             dev(vsag_amd_stream_synchronize(nullptr));
+            bias_src = bias.as<float>();
         }
-        // Codes of every vector in inner-id order; the posting lists are rebuilt from them.
-        const uint64_t cs = q_.code_size();
-        codes_.grow((n_old + n_new) * cs, n_old * cs);
-        if (q_.kind == VSAG_AMD_KIND_FP32) {
-            dev(vsag_amd_memcpy_d2d(codes_.as<uint8_t>() + n_old * cs, x.p, n_new * cs, nullptr));
-        } else {
-            q_.encode(x.as<float>(), n_new, codes_.as<uint8_t>() + n_old * cs);
+        // From here on two structures change; a failure between them leaves them out of step.
+        try {
+            if (use_reorder_ && pq_.kind == VSAG_AMD_KIND_FP32) {
+                const size_t row_bytes = static_cast<size_t>(q_.dim) * 4;
+                raw_.grow((n_old + n_new) * row_bytes, n_old * row_bytes);
+                dev(vsag_amd_memcpy_d2d(raw_.as<uint8_t>() + n_old * row_bytes, x.p, n_new * row_bytes, nullptr));
+            } else if (use_reorder_) {
+                DevBuf pcodes;
+                pcodes.reserve(n_new * pq_.code_size());
+                pq_.encode(x.as<float>(), n_new, pcodes.as<uint8_t>());
+                dev(vsag_amd_store_append(precise_.s, pcodes.as<uint8_t>(), n_new, nullptr));
+                dev(vsag_amd_stream_synchronize(nullptr));
+            }
+            dev(vsag_amd_store_append_lists(lists_.s, code_src, buckets.as<int32_t>(), bias_src, postings, nullptr));
+            dev(vsag_amd_stream_synchronize(nullptr));
+        } catch (...) {
+            broken_ = n_old > 0 || vsag_amd_store_size(lists_.s) != 0;
+            throw;
         }
-        dev(vsag_amd_store_set_lists(lists_.s, codes_.as<uint8_t>(), bucket_labels_.as<int32_t>(), n_old + n_new,
-                                     nlist_, nullptr));
-        if (use_reorder_) {
-            const size_t row_bytes = static_cast<size_t>(q_.dim) * 4;
-            raw_.grow((n_old + n_new) * row_bytes, n_old * row_bytes);
-            dev(vsag_amd_memcpy_d2d(raw_.as<uint8_t>() + n_old * row_bytes, x.p, n_new * row_bytes, nullptr));
-        }
-        dev(vsag_amd_stream_synchronize(nullptr));
         for (int64_t r : rows) {
+            known_.emplace(base->GetIds()[r], static_cast<uint32_t>(labels_.size()));
             labels_.push_back(base->GetIds()[r]);
         }
         return failed;
     }
 
     CommonParam common_;
-    Quantizer q_;
+    Quantizer q_;   // codes of the lists
+    Quantizer pq_;  // precise codes of the rerank (fp32: the raw rows)
     uint32_t nlist_ = 10;
+    uint32_t bpd_ = 1;  // buckets_per_data
     bool use_reorder_ = false;
+    bool use_residual_ = false;
     bool train_random_ = false;
     int64_t train_sample_count_ = 65536;
     bool trained_ = false;
-    StoreHandle centroid_store_, lists_;
-    DevBuf centroids_, codes_, bucket_labels_, raw_;
+    bool broken_ = false;
+    StoreHandle centroid_store_, lists_, precise_;
+    DevBuf centroids_, raw_;
     std::vector<int64_t> labels_;
-    std::unordered_set<int64_t> known_;
-    mutable std::mutex mutex_;
-    mutable DevBuf queries_, buckets_, bucket_d_, cand_ids_, cand_d_, out_ids_, out_d_, workspace_;
+    LabelMap known_;
 };
 
 }  // namespace

@@ -85,6 +85,31 @@ private:
     Error error_;
 };
 
+// The reference's tl::expected<void, Error> of Train and the like.
+template <>
+class Expected<void> {
+public:
+    Expected() : has_(true), error_(ErrorType::UNKNOWN_ERROR, "") {
+    }
+    Expected(Error error) : has_(false), error_(std::move(error)) {
+    }
+    bool
+    has_value() const {
+        return has_;
+    }
+    explicit operator bool() const {
+        return has_;
+    }
+    const Error&
+    error() const {
+        return error_;
+    }
+
+private:
+    bool has_;
+    Error error_;
+};
+
 class Dataset;
 using DatasetPtr = std::shared_ptr<Dataset>;
 
@@ -224,9 +249,51 @@ public:
 };
 using FilterPtr = std::shared_ptr<Filter>;
 
+// include/vsag/search_request.h:34-230, the fields the brute_force and ivf indexes read.
+enum class SearchMode {
+    KNN_SEARCH = 1,
+    RANGE_SEARCH = 2,
+};
+
+class SearchRequest {
+public:
+    DatasetPtr query_{nullptr};
+    SearchMode mode_{SearchMode::KNN_SEARCH};
+    int64_t topk_{10};
+    float radius_{0.5F};
+    int64_t limited_size_{-1};
+    std::string params_str_{};
+    bool enable_filter_{false};
+    FilterPtr filter_{nullptr};
+    bool enable_bitset_filter_{false};
+    BitsetPtr bitset_filter_{nullptr};
+    // ivf: the buckets every query scans, in scan order, instead of the routed ones (one list per query; empty =
+    // default routing).  The hook by which a caller injects its own routing (ivf.cpp:2075-2112).
+    std::vector<std::vector<int64_t>> bucket_ids_{};
+};
+
 class VSAG_HOST_EXPORT Index {
 public:
     virtual ~Index() = default;
+
+    // Trains the quantizers (and, for ivf, the partition) without inserting anything (include/vsag/index.h:150).
+    virtual Expected<void>
+    Train(const DatasetPtr& data) = 0;
+
+    // include/vsag/index.h:333: the search described by `request` (filters are ANDed).
+    virtual Expected<DatasetPtr>
+    SearchWithRequest(const SearchRequest& request) const = 0;
+
+    // include/vsag/index.h:575-633: distances between the query and the vectors with the given labels; -1 for a label
+    // the index does not hold.  topk == -1: Dim = count, distances in the order of `ids`, no ids; topk > 0: the
+    // min(topk, count) smallest, ascending, with their labels, unknown labels last.  calculate_precise_distance uses
+    // the reorder vectors of an ivf index built with use_reorder, else the base codes.
+    virtual Expected<DatasetPtr>
+    CalDistanceById(const float* query, const int64_t* ids, int64_t count, bool calculate_precise_distance = true,
+                    int64_t topk = -1) const = 0;
+    virtual Expected<DatasetPtr>
+    CalDistanceById(const DatasetPtr& query, const int64_t* ids, int64_t count, bool calculate_precise_distance = true,
+                    int64_t topk = -1) const = 0;
 
     // Train + Add.  Returns the ids that could not be inserted (duplicates of ids already present).
     virtual Expected<std::vector<int64_t>>

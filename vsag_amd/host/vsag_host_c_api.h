@@ -1,7 +1,8 @@
 /* C view of the host layer, shaped like the reference's include/vsag/vsag_c_api.h:20-160 (same error
  * codes, Error_t by value, caller-owned result arrays), so that a program written against the reference's
- * C API drives the GPU-backed index classes unchanged.  vsag_index_knn_search_batch is the only addition:
- * the reference's C entry point takes one query per call. */
+ * C API drives the GPU-backed index classes unchanged.  Additions, marked below: vsag_index_knn_search_batch and
+ * vsag_index_search_buckets (the reference's C entry points take one query per call and cannot name buckets), and
+ * vsag_index_calculate_distances (rows of queries, precise / top-k selection of Index::CalDistanceById). */
 #ifndef VSAG_HOST_C_API_H
 #define VSAG_HOST_C_API_H
 
@@ -68,6 +69,31 @@ VSAG_HOST_API Error_t vsag_index_range_search_with_filter(vsag_index_t index, co
 VSAG_HOST_API Error_t vsag_index_knn_search_batch(vsag_index_t index, const float* queries, uint64_t nq, uint64_t dim,
                                                   int64_t k, const char* parameters, int64_t* ids, float* dists,
                                                   int64_t* result_dim);
+/* Addition: Index::SearchWithRequest with bucket_ids_ (include/vsag/search_request.h): query i scans the lists
+ * bucket_ids[bucket_offsets[i] .. bucket_offsets[i + 1]) instead of the routed ones; bucket_offsets has nq + 1 entries
+ * (NULL: default routing).  Output as vsag_index_knn_search_batch. */
+VSAG_HOST_API Error_t vsag_index_search_buckets(vsag_index_t index, const float* queries, uint64_t nq, uint64_t dim,
+                                                int64_t k, const char* parameters, const int64_t* bucket_ids,
+                                                const uint64_t* bucket_offsets, int64_t* ids, float* dists,
+                                                int64_t* result_dim);
+/* include/vsag/vsag_c_api.h:128-133: trains the index (centroids, quantizers); no data is added. */
+VSAG_HOST_API Error_t vsag_index_train(vsag_index_t index, const float* data, const int64_t* ids, uint64_t dim,
+                                       uint64_t count);
+/* include/vsag/vsag_c_api.h:250-255: distances between the query and the vectors with the given labels, in the order
+ * of `ids`; -1 for a label the index does not hold. */
+VSAG_HOST_API Error_t vsag_index_calculate_distance_by_ids(vsag_index_t index, const float* query, uint64_t dim,
+                                                           const int64_t* ids, uint64_t count, float* dists);
+/* Addition: Index::CalDistanceById in full (include/vsag/index.h:575-633): nq queries, row i against
+ * ids[i * count ...]; topk == -1 writes nq x count distances in the order of ids (out_ids may be NULL), topk > 0 the
+ * min(topk, count) smallest per row with their labels. */
+VSAG_HOST_API Error_t vsag_index_calculate_distances(vsag_index_t index, const float* queries, uint64_t nq, uint64_t dim,
+                                                     const int64_t* ids, uint64_t count, bool precise, int64_t topk,
+                                                     int64_t* out_ids, float* out_dists);
+/* include/vsag/vsag_c_api.h:50-65: statistics of the next search that writes search_result (a JSON string with
+ * dist_cmp, distance_evaluations_by_phase, ...; NULL when none were recorded). */
+VSAG_HOST_API Error_t vsag_search_result_enable_statistics(SearchResult_t* search_result);
+VSAG_HOST_API const char* vsag_search_result_get_statistics(const SearchResult_t* search_result);
+VSAG_HOST_API void vsag_search_result_destroy_statistics(SearchResult_t* search_result);
 VSAG_HOST_API int64_t vsag_index_get_num_elements(vsag_index_t index);
 /* Number of ids the last build / add on this thread could not insert (duplicates). */
 VSAG_HOST_API int64_t vsag_last_failed_id_count(void);
