@@ -472,11 +472,11 @@ def run_c3(env):
     tf = flops / (kms * 1e-3) / 1e12
     roof = {"bound": "mfma", "achieved": tf, "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": tf / MFMA_F32_PEAK_TFLOPS,
-            # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of one launch: profiles/kmeans_assign_c3.md.  Far above
-            # the 3.9 GB of inputs: every row tile re-reads the centroids from beyond the L2 (they come from the
-            # last-level cache, the kernel stays bound by the matrix cores).
-            "traffic": 65124676.8 * 2.00 * 1024 + 125000.0 * 1024 if (n, d, k) == (1000000, 960, 4096) else None,
-            "kernel": "kmeans_assign_kernel", "kernel_ms": kms,
+            # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of one launch: profiles/kmeans_assign_c3.md.  Above the
+            # 3.9 GB of inputs: an XCD's L2 holds the k-slices of one macro tile (1024 rows x 2048 centroids) at a time.
+            "traffic": 11786276.4 * 2.00 * 1024 + 2125360.1 * 1024 if (n, d, k) == (1000000, 960, 4096) else None,
+            "kernel": "kmeans_assign_tile_kernel<4>" if d % 4 == 0 and k > 384 else
+                      "kmeans_assign_tile_kernel<2>" if d % 4 == 0 else "kmeans_assign_kernel", "kernel_ms": kms,
             "flops_per_launch": flops}
     return env.base_line("k-means assign rows/s", "rows/s", n / sec, sec, "f32",
                          "configs[2]: k-means assignment, N=%d, d=%d, k=%d (one step = one assignment pass)" % (n, d, k),

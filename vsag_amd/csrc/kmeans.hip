@@ -14,6 +14,7 @@
 // quarter-to-eighth of the centroids and keeps them in its own L2, while the X tile is what streams.
 #include <hipcub/hipcub.hpp>
 
+#include <mutex>
 #include <random>
 #include <vector>
 
@@ -198,6 +199,264 @@ kmeans_assign_kernel(const float* __restrict__ X, uint64_t n, const float* __res
         unsigned long long other = __shfl_xor(my_best[j], 32);
         unsigned long long key = other < my_best[j] ? other : my_best[j];
         uint64_t row = row0 + wn * 64 + j * 32 + l32;
+        if (half == 0 && row < n && key != ~0ull) {
+            atomicMin(&best[row], key);
+        }
+    }
+}
+
+// v or zeros, component by component (a conditional on the whole float4 would go through memory).
+__device__ inline float4
+keep_if(bool in, float4 v) {
+    v.x = in ? v.x : 0.0F;
+    v.y = in ? v.y : 0.0F;
+    v.z = in ? v.z : 0.0F;
+    v.w = in ? v.w : 0.0F;
+    return v;
+}
+
+// The same contraction for dim % 4 == 0 (every row is a whole number of float4), one (row tile, centroid tile) per
+// workgroup of eight waves: 256 data rows x (64 MI) centroids, MI = 2 or 4.  What bounds this kernel next to the matrix
+// pipe is the stream of operand tiles from L2 into the CUs, so the tile is as large as LDS and registers allow: one
+// workgroup per CU, 16 MI accumulator registers per 32 data rows.
+//
+// Stages of 16 k travel through a ring of three LDS slots.  In iteration s a wave stores the rows it loaded for
+// stage s + 2 (the loads went out an iteration ago), sends the loads for stage s + 3, and contracts stage s; the
+// operands of the first MFMAs of stage s + 1 are read from LDS while the last ones of stage s run, so the matrix pipe
+// never waits for LDS across the one barrier per stage.  Slot (s + 2) % 3 last held stage s - 1, which every wave
+// finished before the barrier that ended iteration s - 1.
+//
+// LDS layout per slot and operand: four planes of float4, plane g = 2c + h holds for every row the float4 of
+// k = 8c + 4h .. 8c + 4h + 3 of the stage.  The contraction runs over all k, so the k a lane feeds to an MFMA step may
+// be any bijection as long as both operands use the same one: lane (row, h) takes k = 8c + 4h + e in step 4c + e,
+// which makes a global float4 one ds_write_b128 and a lane's operands for four steps one ds_read_b128.  Row r of
+// plane g sits in slot r ^ (10 (g & 1) + 4 (g >> 1)): the float4 written by 8 (16) neighbouring lanes, 2 (4) rows of
+// all planes, fall into different 16-byte columns of a 128 (256) byte bank period, and a read of 32 consecutive rows
+// stays a permutation of 32 consecutive slots.
+//
+// Grid: one dimension.  Workgroups are dealt round-robin to the eight XCDs, so id % 8 is the XCD; the ids of one XCD
+// walk macro tiles of (32 / mc) row tiles x mc centroid tiles, the 32 workgroups that run at the same time on that
+// XCD and advance through k together: a k-slice of a row tile or centroid tile is fetched into the XCD's L2 once and
+// hit by the other workgroups of its macro row / column.
+struct TilePlan {
+    uint32_t rtiles, ctiles;
+    uint32_t mc_log2;  // macro tile: (32 >> mc_log2) row tiles x (1 << mc_log2) centroid tiles
+    uint32_t mcols;    // macro tiles per macro row
+    uint32_t macros;
+};
+
+constexpr int kTileRows = 256;  // data rows per workgroup tile
+constexpr int kTileThreads = 512;
+constexpr int kStageK = 16;     // contraction depth per stage
+constexpr int kRing = 3;
+
+constexpr size_t
+tile_lds_bytes(int mi) {
+    return kRing * static_cast<size_t>(4 * (64 * mi + kTileRows)) * sizeof(float4);
+}
+
+template <int MI>
+__global__ void __launch_bounds__(kTileThreads, 1)
+kmeans_assign_tile_kernel(const float* __restrict__ X, uint64_t n, const float* __restrict__ C, uint32_t k, uint32_t dim,
+                          const float* __restrict__ ynorm, unsigned long long* __restrict__ best, TilePlan plan) {
+    constexpr uint32_t TM = 64 * MI;                   // centroids per tile
+    constexpr uint32_t kSlot = 4 * (TM + kTileRows);   // float4 per ring slot: A planes, then B planes
+    constexpr int RA = MI / 2;                         // float4 of A a thread loads per stage
+    extern __shared__ float4 lds[];
+
+    const uint32_t xcd = blockIdx.x & 7;
+    const uint32_t local = blockIdx.x >> 3;
+    const uint32_t macro = (local >> 5) * 8 + xcd;
+    if (macro >= plan.macros) {
+        return;
+    }
+    const uint32_t within = local & 31;
+    const uint32_t rt = (macro / plan.mcols) * (32U >> plan.mc_log2) + (within >> plan.mc_log2);
+    const uint32_t ct = ((macro % plan.mcols) << plan.mc_log2) + (within & ((1U << plan.mc_log2) - 1));
+    if (rt >= plan.rtiles || ct >= plan.ctiles) {
+        return;
+    }
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    const uint32_t wave = tid >> 6;
+    const uint32_t wm = wave & 1;   // which half of the tile's centroids
+    const uint32_t wn = wave >> 1;  // which 64 data rows of the tile
+    const uint32_t half = lane >> 5;
+    const uint32_t l32 = lane & 31;
+    const uint64_t row0 = static_cast<uint64_t>(rt) * kTileRows;
+    const uint64_t c0 = static_cast<uint64_t>(ct) * TM;
+    const uint32_t stages = (dim + kStageK - 1) / kStageK;
+
+    // Loader: thread (r, g) of 128 x 4 moves float4 g of rows r, r + 128 of both operands (A: one row when the tile
+    // has 128 centroids).  Rows past the end repeat the last one: their results are dropped at the end.
+    const uint32_t lr = tid >> 2, lg = tid & 3;
+    const float* pa[RA];
+    const float* pb[2];
+#pragma unroll
+    for (int r = 0; r < RA; ++r) {
+        const uint64_t ca = c0 + lr + 128 * r;
+        pa[r] = C + (ca < k ? ca : k - 1) * dim;
+    }
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+        const uint64_t xb = row0 + lr + 128 * r;
+        pb[r] = X + (xb < n ? xb : n - 1) * dim;
+    }
+    const uint32_t wslot = lr ^ (10 * (lg & 1) + 4 * (lg >> 1));  // + 128 r
+    const uint32_t wa = lg * TM + wslot;
+    const uint32_t wb = 4 * TM + lg * kTileRows + wslot;
+    // Reader: lane (l32, half) takes plane 2c + half, rows wm * 32 MI + 32 i + l32 of A and wn * 64 + 32 j + l32 of B.
+    uint32_t ra_off[2], rb_off[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+        const uint32_t sw = 10 * half + 4 * c;
+        ra_off[c] = (2 * c + half) * TM + wm * 32 * MI + (l32 ^ sw);
+        rb_off[c] = 4 * TM + (2 * c + half) * kTileRows + wn * 64 + (l32 ^ sw);
+    }
+
+    floatx16 acc[MI][2];
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                acc[i][j][e] = 0.0F;
+            }
+        }
+    }
+    float4 ga[RA], gb[2];
+    // Loads of stage t; past the last stage they repeat it and what they bring is never read.
+    auto load_column = [&](uint32_t t) {
+        const uint32_t k0 = (t < stages ? t : stages - 1) * kStageK + 4 * lg;
+        return k0 < dim ? k0 : 0;
+    };
+    auto issue_loads = [&](uint32_t t) {
+        const uint32_t col = load_column(t);
+#pragma unroll
+        for (int r = 0; r < RA; ++r) {
+            ga[r] = *reinterpret_cast<const float4*>(pa[r] + col);
+        }
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            gb[r] = *reinterpret_cast<const float4*>(pb[r] + col);
+        }
+    };
+    auto store_stage = [&](uint32_t t, float4* slot) {
+        const bool in = t * kStageK + 4 * lg < dim;
+#pragma unroll
+        for (int r = 0; r < RA; ++r) {
+            slot[wa + 128 * r] = keep_if(in, ga[r]);
+        }
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            slot[wb + 128 * r] = keep_if(in, gb[r]);
+        }
+    };
+    float4 fa[2][MI], fb[2][2];
+    // Operand m of 6 (MI = 4) or 4 (MI = 2) of chunk c of a slot into buffer u.
+    auto read_operand = [&](const float4* slot, int c, int u, int m) {
+        if (m < MI) {
+            fa[u][m] = slot[ra_off[c] + 32 * m];
+        } else {
+            fb[u][m - MI] = slot[rb_off[c] + 32 * (m - MI)];
+        }
+    };
+    // The 2 MI MFMAs of step e of the chunk in buffer u; side(m) runs behind the m-th of them, so that the loads,
+    // stores and LDS reads of the pipeline are issued while the matrix pipe works on an MFMA of this wave.
+    auto mfma_step = [&](int u, int e, auto side) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+            const float av = e == 0 ? fa[u][i].x : e == 1 ? fa[u][i].y : e == 2 ? fa[u][i].z : fa[u][i].w;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const float bv = e == 0 ? fb[u][j].x : e == 1 ? fb[u][j].y : e == 2 ? fb[u][j].z : fb[u][j].w;
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[i][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                side(2 * i + j);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+    auto nothing = [](int) {};
+    float4* s0 = lds;              // slot of the stage being contracted
+    float4* s1 = lds + kSlot;      // of the next one
+    float4* s2 = lds + 2 * kSlot;  // of the one after
+    issue_loads(0);
+    store_stage(0, s0);
+    issue_loads(1);
+    store_stage(1, s1);
+    issue_loads(2);
+    __syncthreads();
+#pragma unroll
+    for (int m = 0; m < MI + 2; ++m) {
+        read_operand(s0, 0, 0, m);
+    }
+    for (uint32_t st = 0; st < stages; ++st) {
+        const bool in = (st + 2) * kStageK + 4 * lg < dim;
+        const uint32_t col = load_column(st + 3);
+        // chunk 0; the operands of chunk 1 are read behind its first MFMAs
+        mfma_step(0, 0, [&](int m) {
+            if (m < MI + 2) {
+                read_operand(s0, 1, 1, m);
+            }
+        });
+        mfma_step(0, 1, nothing);
+        mfma_step(0, 2, nothing);
+        mfma_step(0, 3, nothing);
+        // chunk 1; behind it the first operands of stage st + 1 (stored an iteration ago, behind the last barrier),
+        // then the rows loaded for stage st + 2 go to LDS and the loads of stage st + 3 go out
+        mfma_step(1, 0, [&](int m) {
+            if (m < MI + 2) {
+                read_operand(s1, 0, 0, m);
+            }
+        });
+        mfma_step(1, 1, [&](int m) {
+            if (m < RA) {
+                s2[wa + 128 * m] = keep_if(in, ga[m]);
+            } else if (m < RA + 2) {
+                s2[wb + 128 * (m - RA)] = keep_if(in, gb[m - RA]);
+            }
+        });
+        mfma_step(1, 2, [&](int m) {
+            if (m < RA) {
+                ga[m] = *reinterpret_cast<const float4*>(pa[m] + col);
+            } else if (m < RA + 2) {
+                gb[m - RA] = *reinterpret_cast<const float4*>(pb[m - RA] + col);
+            }
+        });
+        mfma_step(1, 3, nothing);
+        __syncthreads();
+        float4* t = s0;
+        s0 = s1;
+        s1 = s2;
+        s2 = t;
+    }
+    // Fused argmin: acc[i][j][e] = <c_m, x_n> with m = c0 + wm*32*MI + i*32 + 8*(e/4) + 4*half + e%4 and
+    // n = row0 + wn*64 + j*32 + l32.  m grows with (i, e), so a strict `<` keeps the first minimum.
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        float bd = __builtin_inff();
+        uint32_t bi = 0xFFFFFFFFU;
+#pragma unroll
+        for (int i = 0; i < MI; ++i) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const uint32_t ml = wm * 32 * MI + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+                const bool ok = c0 + ml < k;
+                const float dist = (ok ? ynorm[c0 + ml] : 0.0F) + (-2.0F * acc[i][j][e]);
+                if (ok && dist < bd) {
+                    bd = dist;
+                    bi = static_cast<uint32_t>(c0) + ml;
+                }
+            }
+        }
+        // the two halves of the wave hold different centroids of the same data row
+        unsigned long long key = bi != 0xFFFFFFFFU ? make_key(bd, bi) : ~0ull;
+        const unsigned long long other = __shfl_xor(key, 32);
+        key = other < key ? other : key;
+        const uint64_t row = row0 + wn * 64 + j * 32 + l32;
         if (half == 0 && row < n && key != ~0ull) {
             atomicMin(&best[row], key);
         }
@@ -412,15 +671,54 @@ assign_launch(const float* x, uint64_t n, uint32_t dim, const float* cent, uint3
     hipLaunchKernelGGL(fill_u64_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, b.best, ~0ull,
                        n);
     uint32_t ctiles = (k + BM - 1) / BM;
-    uint32_t groups = ctiles < 8 ? ctiles : 8;
-    // grid.y is limited to 65535 row tiles: larger inputs go slab by slab.
-    const uint64_t slab_rows = 65535ull * BN;
     timing_begin(st);
-    for (uint64_t r0 = 0; r0 < n; r0 += slab_rows) {
-        uint64_t rows = n - r0 < slab_rows ? n - r0 : slab_rows;
-        dim3 grid(groups, static_cast<uint32_t>(div_up(rows, BN)));
-        hipLaunchKernelGGL(kmeans_assign_kernel, grid, dim3(256), 0, st, x + r0 * dim, rows, cent, k, dim, b.ynorm,
-                           b.best + r0, groups);
+    if ((dim & 3) == 0) {
+        // 256 centroids per tile when there are enough of them to fill it, else 128
+        const int mi = k > 384 ? 4 : 2;
+        const uint32_t tile_m = 64 * mi;
+        static std::once_flag lds_once;
+        static hipError_t lds_rc = hipSuccess;
+        std::call_once(lds_once, []() {
+            lds_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kmeans_assign_tile_kernel<2>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(tile_lds_bytes(2)));
+            if (lds_rc == hipSuccess) {
+                lds_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kmeans_assign_tile_kernel<4>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             static_cast<int>(tile_lds_bytes(4)));
+            }
+        });
+        VA_HIP(lds_rc);
+        // rows go slab by slab so that the tile count stays far inside the grid limit
+        const uint64_t slab_rows = (1ull << 20) * kTileRows;
+        for (uint64_t r0 = 0; r0 < n; r0 += slab_rows) {
+            const uint64_t rows = n - r0 < slab_rows ? n - r0 : slab_rows;
+            TilePlan plan;
+            plan.rtiles = static_cast<uint32_t>(div_up(rows, kTileRows));
+            plan.ctiles = (k + tile_m - 1) / tile_m;
+            plan.mc_log2 = plan.ctiles >= 8 ? 3 : plan.ctiles >= 4 ? 2 : plan.ctiles >= 2 ? 1 : 0;
+            plan.mcols = (plan.ctiles + (1U << plan.mc_log2) - 1) >> plan.mc_log2;
+            const uint32_t mrows = (plan.rtiles + (32U >> plan.mc_log2) - 1) / (32U >> plan.mc_log2);
+            plan.macros = mrows * plan.mcols;
+            const uint32_t per_xcd = (plan.macros + 7) / 8;
+            const dim3 grid(per_xcd * 32 * 8);
+            if (mi == 4) {
+                hipLaunchKernelGGL(kmeans_assign_tile_kernel<4>, grid, dim3(kTileThreads), tile_lds_bytes(4), st,
+                                   x + r0 * dim, rows, cent, k, dim, b.ynorm, b.best + r0, plan);
+            } else {
+                hipLaunchKernelGGL(kmeans_assign_tile_kernel<2>, grid, dim3(kTileThreads), tile_lds_bytes(2), st,
+                                   x + r0 * dim, rows, cent, k, dim, b.ynorm, b.best + r0, plan);
+            }
+        }
+    } else {
+        uint32_t groups = ctiles < 8 ? ctiles : 8;
+        // grid.y is limited to 65535 row tiles: larger inputs go slab by slab.
+        const uint64_t slab_rows = 65535ull * BN;
+        for (uint64_t r0 = 0; r0 < n; r0 += slab_rows) {
+            uint64_t rows = n - r0 < slab_rows ? n - r0 : slab_rows;
+            dim3 grid(groups, static_cast<uint32_t>(div_up(rows, BN)));
+            hipLaunchKernelGGL(kmeans_assign_kernel, grid, dim3(256), 0, st, x + r0 * dim, rows, cent, k, dim, b.ynorm,
+                               b.best + r0, groups);
+        }
     }
     timing_end(st);
     hipLaunchKernelGGL(kmeans_finalize_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, b.best,
