@@ -194,6 +194,11 @@ ivf_i8_kernel(IvfI8Args p) {
                                          static_cast<int>(x1.z)}
                                  : intx4{static_cast<int>(x0.y), static_cast<int>(x0.w), static_cast<int>(x1.y),
                                          static_cast<int>(x1.w)};
+            if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                // Twice the query (0..30 still fits a signed byte): with the accumulator started from -No the matrix
+                // pipe delivers 2 <q, o> - No, the quantity the test compares.
+                qv[j][s] = qv[j][s] << 1;
+            }
         }
         tq[j] = p.tq[qidx[j]];
         my_list[j] = (static_cast<uint64_t>(live ? pair[j] : 0) * kIvfI8Chunks + chunk) * 2 + half;
@@ -273,7 +278,7 @@ ivf_i8_kernel(IvfI8Args p) {
                 const int r = blk >> 1, j = blk & 1;
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    c[e] = 0;
+                    c[e] = METRIC == VSAG_AMD_METRIC_L2 ? tm[r & 1][e] : 0;
                 }
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
@@ -292,57 +297,77 @@ ivf_i8_kernel(IvfI8Args p) {
                 if (blk + 1 < kBlocks) {
                     multiply(blk + 1, acc[(blk + 1) & 1]);
                 }
-                // The sixteen verdicts stay in scalar registers; only a block with a hit builds a mask per lane.
-                bool pass[16];
-                uint64_t any = 0;
+                // What passes is recorded as (slot, accumulator) and turned into (distance, id) by
+                // ivf_i8_finish_kernel: nothing here waits for a load from global memory.
+                auto record = [&](int e) {
+                    const uint64_t slot = slot0 + 32 * r + 8 * (e >> 2) + 4 * half + (e & 3);
+                    if (ncand[j] < p.k) {
+                        p.partial[my_list[j] * p.k + ncand[j]] =
+                            (slot << 32) | static_cast<uint32_t>(acc[blk & 1][e]);
+                    }
+                    ++ncand[j];
+                };
+                if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                    // Nearly nothing passes.  The sixteen elements of a lane are reduced to their best one with
+                    // three-operand max instructions, four at a time, so that a block with a hit finds it group by
+                    // group, and one compare decides whether the block needs a second look.
+                    int32_t gbest[4];
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
-                        pass[e] = (acc[blk & 1][e] << 1) + tm[r & 1][e] >= tq[j];
-                    } else {
-                        pass[e] = static_cast<float>(acc[blk & 1][e]) >=
-                                  __int_as_float(tm[r & 1][e]) + __int_as_float(tq[j]);
+                    for (int g = 0; g < 4; ++g) {
+                        gbest[g] = max(max(max(acc[blk & 1][4 * g], acc[blk & 1][4 * g + 1]), acc[blk & 1][4 * g + 2]),
+                                       acc[blk & 1][4 * g + 3]);
                     }
-                    any |= __ballot(pass[e]);
-                }
-                if (blk + 1 < kBlocks) {
-                    if (reads) {
-                        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-                    }
+                    const bool hit = max(max(max(gbest[0], gbest[1]), gbest[2]), gbest[3]) >= tq[j];
+                    const uint64_t any = __ballot(hit);
+                    if (blk + 1 < kBlocks) {
+                        if (reads) {
+                            __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+                        }
 #pragma unroll
-                    for (int m = 0; m < 4; ++m) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x002, METRIC == VSAG_AMD_METRIC_L2 ? 8 : 12, 0);
+                        for (int m = 0; m < 4; ++m) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                        }
                     }
-                }
-                if (any != 0) {
-                    uint32_t bits = 0;
+                    if (any != 0) {
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            if (__ballot(gbest[g] >= tq[j]) == 0) {
+                                continue;
+                            }
+#pragma unroll
+                            for (int e = 4 * g; e < 4 * g + 4; ++e) {
+                                const bool pass = acc[blk & 1][e] >= tq[j] && pair[j] != 0xFFFFFFFFU;
+                                if (__ballot(pass) != 0 && pass) {
+                                    record(e);
+                                }
+                            }
+                        }
+                    }
+                } else {
+                    // The sixteen verdicts stay in scalar registers; only a block with a hit builds a mask per lane.
+                    bool pass[16];
+                    uint64_t any = 0;
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
-                        bits |= pass[e] ? 1U << e : 0U;
+                        pass[e] = static_cast<float>(acc[blk & 1][e]) >= __int_as_float(tm[r & 1][e]) + __int_as_float(tq[j]);
+                        any |= __ballot(pass[e]);
                     }
-                    while (bits != 0) {
-                        const uint32_t e = static_cast<uint32_t>(__builtin_ctz(bits));
-                        bits &= bits - 1;
-                        const uint64_t slot = slot0 + 32 * r + 8 * (e >> 2) + 4 * half + (e & 3);
-                        const uint32_t id = p.ids[slot];
-                        if (id != VSAG_AMD_INVALID_ID && pair[j] != 0xFFFFFFFFU) {
-                            // The streaming kernel's own three operations on the same integers.
-                            const float result = static_cast<float>(acc[blk & 1][e]);
-                            const float qm = p.qmeta[static_cast<uint64_t>(qidx[j]) * p.qmeta_stride];
-                            const float m0 = __uint_as_float(p.meta[slot]);
-                            float dist;
-                            if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
-                                dist = (qm + m0 - 2 * result) * p.rate;
-                            } else {
-                                const float rr = p.lb * (qm + m0) + p.rate * result + p.lb2;
-                                dist = 1 - rr;
-                            }
-                            if (float_to_ordered(dist) <= as_const(p.bound)[qidx[j]]) {
-                                if (ncand[j] < p.k) {
-                                    p.partial[my_list[j] * p.k + ncand[j]] = make_key(dist, id);
-                                }
-                                ++ncand[j];
+                    if (blk + 1 < kBlocks) {
+                        if (reads) {
+                            __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+                        }
+#pragma unroll
+                        for (int m = 0; m < 4; ++m) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x002, 12, 0);
+                        }
+                    }
+                    if (any != 0) {
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) {
+                            if (pass[e] && pair[j] != 0xFFFFFFFFU) {
+                                record(e);
                             }
                         }
                     }
@@ -368,6 +393,68 @@ ivf_i8_kernel(IvfI8Args p) {
             }
         }
     }
+}
+
+// One thread per private list: its (slot, accumulator) records become (distance, id) keys through the streaming
+// kernel's own three operations on the same integers; records of empty slots and of distances beyond the query's
+// bound (the integer test is a level wider than the bound) are dropped and the list is closed up.
+struct IvfI8FinishArgs {
+    uint64_t* partial;
+    uint32_t* partial_cnt;
+    uint64_t lists;  // pairs x lists per pair
+    uint32_t k, nprobe, p0, per_pair;  // probe columns p0 .. nprobe - 1 hold records, the ones before them keys
+    const uint32_t* ids;
+    const uint32_t* meta;
+    const float* qmeta;
+    uint32_t qmeta_stride;
+    const uint32_t* bound;
+    float lb, rate, lb2;
+};
+
+template <int METRIC>
+__global__ void __launch_bounds__(256)
+ivf_i8_finish_kernel(IvfI8FinishArgs p) {
+    const uint64_t list = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (list >= p.lists) {
+        return;
+    }
+    const uint64_t pair = list / p.per_pair;
+    if (pair % p.nprobe < p.p0) {
+        return;
+    }
+    const uint32_t count = p.partial_cnt[list];
+    if (count == 0) {
+        return;
+    }
+    const uint64_t q = pair / p.nprobe;
+    const float qm = p.qmeta[q * p.qmeta_stride];
+    const uint32_t bound = p.bound[q];
+    uint64_t* keys = p.partial + list * p.k;
+    uint32_t kept = 0;
+    for (uint32_t i = 0; i < count; ++i) {
+        const uint64_t rec = keys[i];
+        const uint64_t slot = rec >> 32;
+        const int32_t acc = static_cast<int32_t>(static_cast<uint32_t>(rec));
+        const uint32_t id = p.ids[slot];
+        if (id == VSAG_AMD_INVALID_ID) {
+            continue;
+        }
+        const float m0 = __uint_as_float(p.meta[slot]);
+        float dist;
+        if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+            // acc = 2 <q, o> - No with No = m0, an integer
+            const float result = static_cast<float>((acc + static_cast<int32_t>(m0)) >> 1);
+            dist = (qm + m0 - 2 * result) * p.rate;
+        } else {
+            const float result = static_cast<float>(acc);
+            const float rr = p.lb * (qm + m0) + p.rate * result + p.lb2;
+            dist = 1 - rr;
+        }
+        if (float_to_ordered(dist) <= bound) {
+            keys[kept++] = make_key(dist, id);
+        }
+    }
+    p.partial_cnt[list] = kept;
 }
 
 // Gated queries: the streaming kernel rescans their lists, so what the matrix-core pass left must not count.  Their
@@ -456,6 +543,29 @@ launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     VA_HIP(hipGetLastError());
     hipLaunchKernelGGL(ivf_i8_clear_gated_kernel, dim3(static_cast<uint32_t>(div_up(pairs, 256))), dim3(256), 0, st, gate,
                        nq, nprobe, p0, partial_cnt, buckets, gpairs, gpairs_cap);
+    VA_HIP(hipGetLastError());
+    IvfI8FinishArgs f{};
+    f.partial = partial;
+    f.partial_cnt = partial_cnt;
+    f.per_pair = ivf_i8_lists_per_pair();
+    f.lists = nq * nprobe * f.per_pair;
+    f.k = kcand;
+    f.nprobe = nprobe;
+    f.p0 = p0;
+    f.ids = s->ids_dev;
+    f.meta = a.meta;
+    f.qmeta = a.qmeta;
+    f.qmeta_stride = a.qmeta_stride;
+    f.bound = bound;
+    f.lb = a.f0;
+    f.rate = a.f1;
+    f.lb2 = a.f2;
+    const dim3 fgrid(static_cast<uint32_t>(div_up(f.lists, 256)));
+    if (l2) {
+        hipLaunchKernelGGL(ivf_i8_finish_kernel<VSAG_AMD_METRIC_L2>, fgrid, dim3(256), 0, st, f);
+    } else {
+        hipLaunchKernelGGL(ivf_i8_finish_kernel<VSAG_AMD_METRIC_IP>, fgrid, dim3(256), 0, st, f);
+    }
     VA_HIP(hipGetLastError());
     return 0;
 }
