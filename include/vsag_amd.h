@@ -187,6 +187,21 @@ VSAG_AMD_API int vsag_amd_residual_bias(const vsag_amd_store_t* store, const uin
                            const int32_t* labels_dev, const float* centroids_dev, float* bias_dev, float* decoded_dev,
                            void* stream);
 
+/* The payload of FlattenDataCell::Serialize (flatten_datacell.h:481-486, io/common/basic_io.h:196-207): codes
+ * [first, first + n) of a flat store back in the reference byte layout (n x code_size bytes).  The store keeps the
+ * u64 sums of squares of the uniform kinds as floats; the exported code carries them recomputed from its bytes. */
+VSAG_AMD_API int vsag_amd_store_export_codes(const vsag_amd_store_t* store, uint64_t first, uint64_t n, uint8_t* codes_dev,
+                                void* stream);
+/* The payload of BucketDataCell::Serialize (bucket_datacell.h:892-904): every list's codes, list by list in list
+ * order (vsag_amd_store_list_sizes gives the cuts), with their inner ids and, for residual stores with the l2 metric,
+ * their bias (bias_dev may be NULL).  Blocking. */
+VSAG_AMD_API int vsag_amd_store_export_lists(const vsag_amd_store_t* store, uint8_t* codes_dev, uint32_t* ids_dev,
+                                float* bias_dev, void* stream);
+
+/* Deserialize (flatten_datacell.h:488-497): while on, appended codes are taken as they were exported -- an fp32 store
+ * under cosine does not normalise rows that are unit vectors already. */
+VSAG_AMD_API int vsag_amd_store_expect_stored_codes(vsag_amd_store_t* store, int on);
+
 /* Sizes of the posting lists (nlist values) copied to host memory. */
 VSAG_AMD_API int vsag_amd_store_list_sizes(const vsag_amd_store_t* store, uint32_t* sizes, uint32_t nlist);
 

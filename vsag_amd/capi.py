@@ -102,6 +102,9 @@ PROTOTYPES = {
     "vsag_amd_ivf_scan_topk_ex": (C.c_int, [_vp, _vp, _u64, _vp, _u32, _u32, _vp, _vp, _vp, _vp, _sz, _vp]),
     "vsag_amd_ivf_probed_codes": (C.c_int, [_vp, _vp, _u64, _u32, _vp, _vp]),
     "vsag_amd_rerank_fp32": (C.c_int, [_vp, _u64, _u32, _i32, _vp, _u64, _vp, _u32, _u32, _vp, _vp, _vp]),
+    "vsag_amd_store_expect_stored_codes": (C.c_int, [_vp, C.c_int]),
+    "vsag_amd_store_export_codes": (C.c_int, [_vp, _u64, _u64, _vp, _vp]),
+    "vsag_amd_store_export_lists": (C.c_int, [_vp, _vp, _vp, _vp, _vp]),
     "vsag_amd_rows_distances_fp32": (C.c_int, [_vp, _u64, _u32, _i32, _vp, _u64, _vp, _u32, _vp, _vp]),
 }
 

@@ -26,6 +26,7 @@ struct vsag_amd_store {
     uint32_t nmeta = 0;          // 4-byte metadata words per code
     uint32_t meta_offset[4] = {0, 0, 0, 0};  // byte offsets of those words in the reference code
     uint32_t meta_is_u64 = 0;    // bit m set: word m is a u64 in the reference code, kept as float
+    bool stored_codes = false;   // appended codes come out of a serialized index: fp32 + cosine rows are unit already
 
     // quantizer state
     float* scale_dev = nullptr;  // sq8/sq4: diff[d]/levels, zero beyond dim

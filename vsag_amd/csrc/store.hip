@@ -313,7 +313,7 @@ retile_args(const vsag_amd_store* s, const uint8_t* codes, uint64_t n) {
     a.tiles = s->tiles;
     a.meta = s->meta;
     a.meta_stride = s->cap_tiles * kWave;
-    a.normalize = (s->kind == VSAG_AMD_KIND_FP32 && s->metric == VSAG_AMD_METRIC_COSINE) ? 1 : 0;
+    a.normalize = (s->kind == VSAG_AMD_KIND_FP32 && s->metric == VSAG_AMD_METRIC_COSINE && !s->stored_codes) ? 1 : 0;
     a.dim = s->dim;
     return a;
 }
@@ -842,5 +842,12 @@ vsag_amd_store_list_sizes(const vsag_amd_store_t* s, uint32_t* sizes, uint32_t n
     VA_CHECK_ARG(s != nullptr && sizes != nullptr, "null store / output");
     VA_CHECK_ARG(s->nlist == nlist, "store has %u lists, asked for %u", s->nlist, nlist);
     memcpy(sizes, s->list_sizes.data(), nlist * sizeof(uint32_t));
+    return 0;
+}
+
+extern "C" int
+vsag_amd_store_expect_stored_codes(vsag_amd_store_t* s, int on) {
+    VA_CHECK_ARG(s != nullptr, "store is null");
+    s->stored_codes = on != 0;
     return 0;
 }

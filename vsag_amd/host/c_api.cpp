@@ -5,6 +5,7 @@
 #include <functional>
 #include <cstdio>
 #include <cstring>
+#include <fstream>
 #include <limits>
 #include <memory>
 #include <mutex>
@@ -339,4 +340,33 @@ vsag_search_result_destroy_statistics(SearchResult_t* search_result) {
     std::lock_guard<std::mutex> lock(statistics_mutex);
     statistics_requests.erase(search_result);
     statistics_results.erase(search_result);
+}
+
+extern "C" Error_t
+vsag_serialize_file(vsag_index_t index, const char* file_path) {
+    auto* vi = static_cast<VsagIndex*>(index);
+    if (vi == nullptr || file_path == nullptr) {
+        return make_error(VSAG_UNKNOWN_ERROR, "index or file path is NULL");
+    }
+    std::ofstream file(file_path, std::ios::binary | std::ios::trunc);
+    if (!file.is_open()) {
+        return make_error(VSAG_INTERNAL_ERROR, std::string("failed to open file for writing: ") + file_path);
+    }
+    auto result = vi->index_->Serialize(file);
+    file.close();
+    return result.has_value() ? success() : make_error(result.error());
+}
+
+extern "C" Error_t
+vsag_deserialize_file(vsag_index_t index, const char* file_path) {
+    auto* vi = static_cast<VsagIndex*>(index);
+    if (vi == nullptr || file_path == nullptr) {
+        return make_error(VSAG_UNKNOWN_ERROR, "index or file path is NULL");
+    }
+    std::ifstream file(file_path, std::ios::binary);
+    if (!file.is_open()) {
+        return make_error(VSAG_MISSING_FILE, std::string("failed to open file for reading: ") + file_path);
+    }
+    auto result = vi->index_->Deserialize(file);
+    return result.has_value() ? success() : make_error(result.error());
 }

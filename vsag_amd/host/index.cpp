@@ -8,9 +8,11 @@
 #include <cmath>
 #include <cstring>
 #include <functional>
+#include <istream>
 #include <limits>
 #include <map>
 #include <mutex>
+#include <ostream>
 #include <shared_mutex>
 #include <random>
 #include <set>
@@ -101,6 +103,10 @@ struct DevBuf {
     DevBuf(const DevBuf&) = delete;
     DevBuf&
     operator=(const DevBuf&) = delete;
+    DevBuf(DevBuf&& other) noexcept : p(other.p), bytes(other.bytes) {
+        other.p = nullptr;
+        other.bytes = 0;
+    }
     ~DevBuf() {
         release();
     }
@@ -221,6 +227,189 @@ private:
     std::mutex mutex_;
     std::vector<std::unique_ptr<SearchContext>> free_;
 };
+
+// ------------------------------------------------------------------------------------------- serialized form
+// StreamWriter / StreamReader of the reference (src/storage/stream_writer.h:28-60, stream_reader.h): objects as their
+// bytes, vectors and strings behind a u64 count.
+class Writer {
+public:
+    explicit Writer(std::ostream& os) : os_(os) {
+    }
+    void
+    write(const void* p, size_t n) {
+        os_.write(static_cast<const char*>(p), static_cast<std::streamsize>(n));
+        if (!os_) {
+            throw VsagException(ErrorType::INTERNAL_ERROR, "writing the serialized index failed");
+        }
+        cursor_ += n;
+    }
+    template <typename T>
+    void
+    obj(const T& v) {
+        write(&v, sizeof(T));
+    }
+    template <typename T>
+    void
+    vec(const std::vector<T>& v) {
+        const uint64_t n = v.size();
+        obj(n);
+        if (n > 0) {
+            write(v.data(), n * sizeof(T));
+        }
+    }
+    void
+    str(const std::string& v) {
+        const uint64_t n = v.size();
+        obj(n);
+        write(v.data(), n);
+    }
+    uint64_t
+    cursor() const {
+        return cursor_;
+    }
+
+private:
+    std::ostream& os_;
+    uint64_t cursor_ = 0;
+};
+
+class Reader {
+public:
+    explicit Reader(std::istream& is) : is_(is) {
+        base_ = is_.tellg();
+        is_.seekg(0, std::ios::end);
+        const std::streampos end = is_.tellg();
+        if (base_ < 0 || end < base_) {
+            throw VsagException(ErrorType::READ_ERROR, "the stream of a serialized index must be seekable");
+        }
+        length_ = static_cast<uint64_t>(end - base_);
+        is_.seekg(base_);
+    }
+    void
+    read(void* p, uint64_t n) {
+        if (n > length_ - cursor_) {
+            throw VsagException(ErrorType::INVALID_BINARY, "the serialized index ends early");
+        }
+        is_.read(static_cast<char*>(p), static_cast<std::streamsize>(n));
+        if (static_cast<uint64_t>(is_.gcount()) != n) {
+            throw VsagException(ErrorType::READ_ERROR, "reading the serialized index failed");
+        }
+        cursor_ += n;
+    }
+    template <typename T>
+    void
+    obj(T& v) {
+        read(&v, sizeof(T));
+    }
+    template <typename T>
+    T
+    get() {
+        T v;
+        obj(v);
+        return v;
+    }
+    template <typename T>
+    void
+    vec(std::vector<T>& v) {
+        const uint64_t n = get<uint64_t>();
+        if (n > (length_ - cursor_) / sizeof(T)) {
+            throw VsagException(ErrorType::INVALID_BINARY, "a vector of the serialized index is longer than the stream");
+        }
+        v.resize(n);
+        if (n > 0) {
+            read(v.data(), n * sizeof(T));
+        }
+    }
+    uint64_t
+    cursor() const {
+        return cursor_;
+    }
+    uint64_t
+    length() const {
+        return length_;
+    }
+    void
+    seek(uint64_t pos) {
+        if (pos > length_) {
+            throw VsagException(ErrorType::INVALID_BINARY, "the serialized index ends early");
+        }
+        is_.clear();
+        is_.seekg(base_ + static_cast<std::streamoff>(pos));
+        cursor_ = pos;
+    }
+    void
+    skip(uint64_t n) {
+        if (n > length_ - cursor_) {
+            throw VsagException(ErrorType::INVALID_BINARY, "the serialized index ends early");
+        }
+        seek(cursor_ + n);
+    }
+
+private:
+    std::istream& is_;
+    std::streampos base_;
+    uint64_t length_ = 0;
+    uint64_t cursor_ = 0;
+};
+
+// Footer (src/storage/serialization.cpp:122-222, serialization.h:193-205):
+// [magic "vsag0000"][u64 metadata length][metadata JSON][u32 CRC-32 of the JSON][u64 footer length][cigam "0000gasv"].
+uint32_t
+footer_checksum(const std::string& bytes) {
+    uint32_t crc = 0xFFFFFFFFU;
+    for (const char byte : bytes) {
+        crc ^= static_cast<uint32_t>(static_cast<int32_t>(byte));  // `crc ^= byte` on a char: sign-extended
+        for (int j = 0; j < 8; ++j) {
+            crc = (crc >> 1) ^ ((crc & 1U) != 0 ? 0xEDB88320U : 0U);
+        }
+    }
+    return crc ^ 0xFFFFFFFFU;
+}
+
+void
+write_footer(Writer& w, const std::string& metadata) {
+    w.write("vsag0000", 8);
+    w.str(metadata);
+    w.obj(footer_checksum(metadata));
+    const uint64_t length = 8 + 8 + metadata.size() + 4 + 8 + 8;
+    w.obj(length);
+    w.write("0000gasv", 8);
+}
+
+// The metadata JSON of the footer at the end of the stream and the footer's length; false when there is none.
+bool
+read_footer(Reader& r, std::string* metadata, uint64_t* footer_length) {
+    constexpr uint64_t kTrailer = 16, kMin = 36;
+    if (r.length() < kMin) {
+        return false;
+    }
+    const uint64_t back = r.cursor();
+    char trailer[kTrailer];
+    r.seek(r.length() - kTrailer);
+    r.read(trailer, kTrailer);
+    uint64_t length = 0;
+    std::memcpy(&length, trailer, 8);
+    bool ok = std::memcmp(trailer + 8, "0000gasv", 8) == 0 && length >= kMin && length <= r.length();
+    if (ok) {
+        std::vector<char> body(length);
+        r.seek(r.length() - length);
+        r.read(body.data(), length);
+        uint64_t mlen = 0;
+        std::memcpy(&mlen, body.data() + 8, 8);
+        ok = std::memcmp(body.data(), "vsag0000", 8) == 0 && mlen == length - kMin;
+        if (ok) {
+            metadata->assign(body.data() + 16, mlen);
+            uint32_t crc = 0;
+            std::memcpy(&crc, body.data() + 16 + mlen, 4);
+            ok = crc == footer_checksum(*metadata);
+            *footer_length = length;
+        }
+    }
+    r.seek(back);
+    return ok;
+}
+
+constexpr uint64_t kIoChunkBytes = 64ull << 20;  // codes cross the host 64 MiB at a time
 
 struct CommonParam {
     int metric = VSAG_AMD_METRIC_L2;
@@ -387,6 +576,142 @@ struct Quantizer {
                                            rabitq_query_bits, codes, nullptr));
                 break;
         }
+    }
+
+    // The same parameters, untrained; and taking over what another one was loaded with.
+    Quantizer
+    blank() const {
+        Quantizer q;
+        q.kind = kind;
+        q.metric = metric;
+        q.dim = dim;
+        q.rabitq_query_bits = rabitq_query_bits;
+        return q;
+    }
+    void
+    take(Quantizer& other) {
+        trained = other.trained;
+        for (auto pair : {std::make_pair(&lb, &other.lb), std::make_pair(&diff, &other.diff),
+                          std::make_pair(&bounds, &other.bounds), std::make_pair(&rotation, &other.rotation),
+                          std::make_pair(&centroid, &other.centroid)}) {
+            std::swap(pair.first->p, pair.second->p);
+            std::swap(pair.first->bytes, pair.second->bytes);
+        }
+    }
+
+    // Quantizer::Serialize (src/quantization/quantizer.h:161-168) and the SerializeImpl of each kind
+    // (scalar_quantizer.cpp:199-204, sq8_uniform_quantizer.cpp:273-281, sq4_uniform_quantizer.cpp:225-234,
+    // rabitq_quantizer.cpp:2245-2252 with random_orthogonal_transformer.cpp:193-196; fp32 writes nothing).
+    void
+    save(Writer& w) const {
+        w.obj(static_cast<uint64_t>(dim));
+        w.obj(static_cast<int32_t>(metric));  // MetricType: l2 0, ip 1, cosine 2, as here
+        w.obj(code_size());
+        w.obj(static_cast<uint8_t>(trained ? 1 : 0));
+        auto floats = [&](const DevBuf& buf, size_t n) {
+            std::vector<float> v(n, 0.0F);
+            if (trained && buf.p != nullptr) {
+                dev(vsag_amd_memcpy_d2h(v.data(), buf.p, n * 4, nullptr));
+            }
+            return v;
+        };
+        auto up = [](uint64_t v, uint64_t a) { return (v + a - 1) / a * a; };
+        switch (kind) {
+            case VSAG_AMD_KIND_FP32:
+                break;
+            case VSAG_AMD_KIND_SQ8:
+            case VSAG_AMD_KIND_SQ4:
+                w.vec(floats(diff, dim));
+                w.vec(floats(lb, dim));
+                break;
+            case VSAG_AMD_KIND_SQ8_UNIFORM: {
+                const std::vector<float> b = floats(bounds, 2);  // lower bound, diff
+                const bool norm = metric == VSAG_AMD_METRIC_L2;
+                const uint64_t behind = up(dim, norm ? 8 : 4);
+                w.obj(b[1]);
+                w.obj(b[0]);
+                w.obj(static_cast<uint64_t>(0));               // offset_code_
+                w.obj(static_cast<uint64_t>(norm ? behind : 0));  // offset_norm_
+                w.obj(static_cast<uint64_t>(norm ? 0 : behind));  // offset_sum_
+                break;
+            }
+            case VSAG_AMD_KIND_SQ4_UNIFORM: {
+                const std::vector<float> b = floats(bounds, 2);
+                const bool norm = metric != VSAG_AMD_METRIC_IP, sum = metric != VSAG_AMD_METRIC_L2;
+                const uint64_t align = norm ? 8 : 4;
+                uint64_t cur = up((static_cast<uint64_t>(dim) + 1) / 2, align);
+                uint64_t off_norm = 0, off_sum = 0, off_codes_sum = 0;
+                if (norm) {
+                    off_norm = cur;
+                    cur += up(8, align);
+                }
+                if (sum) {
+                    off_sum = cur;
+                    cur += up(4, align);
+                    off_codes_sum = cur;
+                }
+                w.obj(b[1]);
+                w.obj(b[0]);
+                w.obj(static_cast<uint64_t>(0));
+                w.obj(off_norm);
+                w.obj(off_sum);
+                w.obj(off_codes_sum);
+                break;
+            }
+            case VSAG_AMD_KIND_RABITQ:
+                w.vec(floats(centroid, dim));
+                w.vec(floats(rotation, static_cast<size_t>(dim) * dim));
+                break;
+        }
+    }
+
+    void
+    load(Reader& r) {
+        const auto fdim = r.get<uint64_t>();
+        const auto fmetric = r.get<int32_t>();
+        const auto fsize = r.get<uint64_t>();
+        const auto ftrained = r.get<uint8_t>();
+        if (fdim != dim || fmetric != metric || fsize != code_size()) {
+            throw VsagException(ErrorType::INVALID_ARGUMENT,
+                                "the serialized quantizer (dim " + std::to_string(fdim) + ", metric " +
+                                    std::to_string(fmetric) + ", code size " + std::to_string(fsize) +
+                                    ") does not match the index (dim " + std::to_string(dim) + ", metric " +
+                                    std::to_string(metric) + ", code size " + std::to_string(code_size()) + ")");
+        }
+        auto upload = [&](DevBuf& buf, const std::vector<float>& v, size_t want) {
+            if (v.size() != want) {
+                throw VsagException(ErrorType::INVALID_BINARY, "a table of the serialized quantizer has the wrong length");
+            }
+            buf.reserve(std::max<size_t>(want * 4, 4));
+            dev(vsag_amd_memcpy_h2d(buf.p, v.data(), want * 4, nullptr));
+        };
+        std::vector<float> a, b;
+        switch (kind) {
+            case VSAG_AMD_KIND_FP32:
+                break;
+            case VSAG_AMD_KIND_SQ8:
+            case VSAG_AMD_KIND_SQ4:
+                r.vec(a);
+                r.vec(b);
+                upload(diff, a, dim);
+                upload(lb, b, dim);
+                break;
+            case VSAG_AMD_KIND_SQ8_UNIFORM:
+            case VSAG_AMD_KIND_SQ4_UNIFORM: {
+                const auto fdiff = r.get<float>();
+                const auto flb = r.get<float>();
+                r.skip(kind == VSAG_AMD_KIND_SQ4_UNIFORM ? 32 : 24);  // the offsets of the code's fields
+                upload(bounds, {flb, fdiff}, 2);
+                break;
+            }
+            case VSAG_AMD_KIND_RABITQ:
+                r.vec(a);
+                r.vec(b);
+                upload(centroid, a, dim);
+                upload(rotation, b, static_cast<size_t>(dim) * dim);
+                break;
+        }
+        trained = ftrained != 0;
     }
 
     vsag_amd_store_t*
@@ -790,7 +1115,30 @@ public:
         });
     }
 
+    // Index::Serialize(std::ostream&) / Deserialize(std::istream&) (include/vsag/index.h:903-940); the stream of a
+    // Deserialize must be seekable (the footer is at its end), the index empty.
+    Expected<void>
+    Serialize(std::ostream& out) const override {
+        return safe_run([&]() {
+            std::shared_lock<std::shared_mutex> lock(mutex_);
+            Writer w(out);
+            save(w);
+        });
+    }
+    Expected<void>
+    Deserialize(std::istream& in) override {
+        return safe_run([&]() {
+            std::unique_lock<std::shared_mutex> lock(mutex_);
+            Reader r(in);
+            load(r);
+        });
+    }
+
 protected:
+    virtual void
+    save(Writer& w) const = 0;
+    virtual void
+    load(Reader& r) = 0;
     virtual DatasetPtr
     search(const DatasetPtr& query, int64_t k, const std::string& parameters, const SearchSpec& spec) const = 0;
     // rows x count distances (row r: query r against ids[r * count ...]), packed by pack_distances.
@@ -889,6 +1237,88 @@ store_distances(SearchContext& ctx, const vsag_amd_store_t* store, const float* 
         dev(vsag_amd_store_distances(store, ctx.queries.as<float>(), nr, ctx.cand_ids.as<uint32_t>(),
                                      static_cast<uint32_t>(count), ctx.out_d.as<float>(), ctx.workspace.p, wsb, ctx.stream));
         ctx.download(out.data() + r0 * count, ctx.out_d.p, static_cast<size_t>(nr * count) * 4);
+    }
+}
+
+// FlattenDataCell::Serialize (src/datacell/flatten_datacell.h:481-497): [u32 total count][u32 capacity][u32 code size]
+// [u64 bytes][codes by inner id][quantizer].  `rows`: the codes are fp32 rows kept outside a store.
+void
+write_flat_cell(Writer& w, const vsag_amd_store_t* store, const DevBuf* rows, const Quantizer& q, uint64_t total) {
+    const uint64_t cs = q.code_size();
+    w.obj(static_cast<uint32_t>(total));
+    w.obj(static_cast<uint32_t>(std::max<uint64_t>(total, 800)));  // max_capacity_: never below its initial value
+    w.obj(static_cast<uint32_t>(cs));
+    w.obj(total * cs);
+    const uint64_t step = std::max<uint64_t>(1, kIoChunkBytes / cs);
+    std::vector<uint8_t> host(static_cast<size_t>(std::min(step, std::max<uint64_t>(total, 1)) * cs));
+    DevBuf staged;
+    for (uint64_t first = 0; first < total; first += step) {
+        const uint64_t n = std::min(step, total - first);
+        if (rows != nullptr) {
+            dev(vsag_amd_memcpy_d2h(host.data(), rows->as<uint8_t>() + first * cs, n * cs, nullptr));
+        } else {
+            staged.reserve(n * cs);
+            dev(vsag_amd_store_export_codes(store, first, n, staged.as<uint8_t>(), nullptr));
+            dev(vsag_amd_memcpy_d2h(host.data(), staged.p, n * cs, nullptr));
+        }
+        w.write(host.data(), n * cs);
+    }
+    q.save(w);
+}
+
+// The cell back: the quantizer lies behind the codes, and the store is made from it, so the codes are read second.
+// Returns the number of codes.
+uint64_t
+read_flat_cell(Reader& r, Quantizer& q, StoreHandle* store, DevBuf* rows) {
+    const auto total = r.get<uint32_t>();
+    (void)r.get<uint32_t>();
+    const auto cs = r.get<uint32_t>();
+    const auto bytes = r.get<uint64_t>();
+    if (cs != q.code_size() || bytes < static_cast<uint64_t>(total) * cs) {
+        throw VsagException(ErrorType::INVALID_ARGUMENT,
+                            "the serialized codes (code size " + std::to_string(cs) + ", " + std::to_string(bytes) +
+                                " bytes for " + std::to_string(total) + " codes) do not match the index (code size " +
+                                std::to_string(q.code_size()) + ")");
+    }
+    const uint64_t codes_at = r.cursor();
+    r.skip(bytes);
+    q.load(r);
+    const uint64_t behind = r.cursor();
+    r.seek(codes_at);
+    if (store != nullptr) {
+        store->s = q.make_store();
+        dev(vsag_amd_store_expect_stored_codes(store->s, 1));
+    } else {
+        rows->reserve(std::max<uint64_t>(static_cast<uint64_t>(total) * cs, 4));
+    }
+    const uint64_t step = std::max<uint64_t>(1, kIoChunkBytes / cs);
+    std::vector<uint8_t> host(static_cast<size_t>(std::min<uint64_t>(step, std::max<uint32_t>(total, 1)) * cs));
+    DevBuf staged;
+    for (uint64_t first = 0; first < total; first += step) {
+        const uint64_t n = std::min<uint64_t>(step, total - first);
+        r.read(host.data(), n * cs);
+        if (store != nullptr) {
+            staged.reserve(n * cs);
+            dev(vsag_amd_memcpy_h2d(staged.p, host.data(), n * cs, nullptr));
+            dev(vsag_amd_store_append(store->s, staged.as<uint8_t>(), n, nullptr));
+            dev(vsag_amd_stream_synchronize(nullptr));
+        } else {
+            dev(vsag_amd_memcpy_h2d(rows->as<uint8_t>() + first * cs, host.data(), n * cs, nullptr));
+        }
+    }
+    if (store != nullptr) {
+        dev(vsag_amd_store_expect_stored_codes(store->s, 0));
+    }
+    r.seek(behind);
+    return total;
+}
+
+void
+rebuild_label_map(const std::vector<int64_t>& labels, LabelMap& known) {
+    known.clear();
+    known.reserve(labels.size());
+    for (size_t i = 0; i < labels.size(); ++i) {
+        known.emplace(labels[i], static_cast<uint32_t>(i));
     }
 }
 
@@ -1063,6 +1493,65 @@ protected:
             store_distances(*ctx, store_.s, queries, rows, q_.dim, inner, count, 1, dists);
         }
         return pack_distances(dists, inner, ids, rows, count, topk);
+    }
+
+    // BruteForce::Serialize (bruteforce.cpp:684-705): the codes' cell, the label table, the footer with basic_info.
+    // index_param is left out of basic_info (a reader checks it only when it is there, bruteforce.cpp:1020-1037).
+    void
+    save(Writer& w) const override {
+        const uint64_t total = labels_.size();
+        write_flat_cell(w, store_.s, nullptr, q_, total);
+        w.vec(labels_);
+        write_footer(w, "{\"_update_time\":\"1970-01-01 00:00:00\",\"basic_info\":{\"dim\":" + std::to_string(q_.dim) +
+                            ",\"extra_info_size\":0,\"has_extra_info\":false,\"is_multi_vector\":false,\"total_count\":" +
+                            std::to_string(total) + "}}");
+    }
+
+    // BruteForce::Deserialize (bruteforce.cpp:1001-1075), both the footer form and the older one that starts with
+    // dim and count.
+    void
+    load(Reader& r) override {
+        if (!labels_.empty()) {
+            throw VsagException(ErrorType::INDEX_NOT_EMPTY, "failed to deserialize: index is not empty");
+        }
+        std::string metadata;
+        uint64_t footer_bytes = 0;
+        int64_t file_dim = q_.dim;
+        uint64_t file_total = 0;
+        const bool footer = read_footer(r, &metadata, &footer_bytes);
+        if (footer) {
+            const Json m = Json::Parse(metadata);
+            if (m.Contains("_empty") && m["_empty"].GetBool()) {
+                throw VsagException(ErrorType::INDEX_EMPTY, "index is empty");
+            }
+            CHECK_ARGUMENT(m.Contains("basic_info"), "the footer of the serialized index has no basic_info");
+            const Json& info = m["basic_info"];
+            file_dim = info["dim"].GetInt();
+            file_total = static_cast<uint64_t>(info["total_count"].GetInt());
+            if (info.Contains("extra_info_size")) {
+                CHECK_ARGUMENT(info["extra_info_size"].GetInt() == 0, "BruteForce index extra_info_size not match");
+            }
+        } else {
+            file_dim = r.get<int64_t>();
+            file_total = r.get<uint64_t>();
+        }
+        CHECK_ARGUMENT(file_dim == static_cast<int64_t>(q_.dim), "the serialized index has dim " + std::to_string(file_dim) +
+                                                                    ", this one " + std::to_string(q_.dim));
+        Quantizer q = q_.blank();
+        StoreHandle store;
+        const uint64_t total = read_flat_cell(r, q, &store, nullptr);
+        std::vector<int64_t> labels;
+        r.vec(labels);
+        if (total != file_total || labels.size() < total) {
+            throw VsagException(ErrorType::INVALID_BINARY, "the serialized index holds " + std::to_string(total) +
+                                                               " codes, " + std::to_string(labels.size()) +
+                                                               " labels and a count of " + std::to_string(file_total));
+        }
+        labels.resize(total);
+        q_.take(q);
+        std::swap(store_.s, store.s);
+        labels_.swap(labels);
+        rebuild_label_map(labels_, known_);
     }
 
 private:
@@ -1489,6 +1978,344 @@ protected:
             }
         }
         return pack_distances(dists, inner, ids, rows, count, topk);
+    }
+
+    // IVF::Serialize (ivf.cpp:990-1057): the cells "bucket", "partition_strategy", "label_table" and "reorder_codes",
+    // their offsets and sizes in the footer next to basic_info.  The bucket cell is BucketDataCell::Serialize
+    // (bucket_datacell.h:892-904).  The partition cell starts like IVFPartitionStrategy::Serialize
+    // (ivf_partition_strategy.h:76-80); behind that the reference writes the image of its router graph, this index
+    // (which routes exactly) a tag and the centroids -- load() reads both, the reference reads only its own.
+    static constexpr uint64_t kCentroidTag = 0x52444D4147415356ULL;  // "VSAGAMDR"
+
+    void
+    save(Writer& w) const override {
+        check_usable();
+        std::string offsets = "{", sizes = "{";
+        auto cell = [&](const char* name, uint64_t begin) {
+            offsets += std::string(offsets.size() > 1 ? "," : "") + "\"" + name + "\":" + std::to_string(begin);
+            sizes += std::string(sizes.size() > 1 ? "," : "") + "\"" + name + "\":" + std::to_string(w.cursor() - begin);
+        };
+        const uint64_t postings = labels_.size() * bpd_;
+        const uint64_t cs = q_.code_size();
+        // bucket
+        uint64_t begin = w.cursor();
+        w.obj(static_cast<int32_t>(nlist_));
+        w.obj(static_cast<uint32_t>(cs));
+        q_.save(w);
+        std::vector<uint32_t> list_sizes(nlist_, 0);
+        std::vector<uint8_t> codes;
+        std::vector<uint32_t> ids;
+        std::vector<float> bias;
+        const bool with_bias = use_residual_ && q_.metric == VSAG_AMD_METRIC_L2;
+        if (postings > 0) {
+            dev(vsag_amd_store_list_sizes(lists_.s, list_sizes.data(), nlist_));
+            DevBuf dcodes, dids, dbias;
+            dcodes.reserve(postings * cs);
+            dids.reserve(postings * 4);
+            if (with_bias) {
+                dbias.reserve(postings * 4);
+            }
+            dev(vsag_amd_store_export_lists(lists_.s, dcodes.as<uint8_t>(), dids.as<uint32_t>(),
+                                            with_bias ? dbias.as<float>() : nullptr, nullptr));
+            codes.resize(postings * cs);
+            ids.resize(postings);
+            dev(vsag_amd_memcpy_d2h(codes.data(), dcodes.p, codes.size(), nullptr));
+            dev(vsag_amd_memcpy_d2h(ids.data(), dids.p, ids.size() * 4, nullptr));
+            if (with_bias) {
+                bias.resize(postings);
+                dev(vsag_amd_memcpy_d2h(bias.data(), dbias.p, bias.size() * 4, nullptr));
+            }
+        }
+        uint64_t at = 0;
+        for (uint32_t l = 0; l < nlist_; ++l) {
+            const uint64_t n = list_sizes[l];
+            w.obj(n * cs);
+            w.write(codes.data() + at * cs, n * cs);
+            w.obj(n);
+            w.write(ids.data() + at, n * 4);
+            if (use_residual_) {
+                const uint64_t nb = with_bias ? n : 0;
+                w.obj(nb);
+                if (nb > 0) {
+                    w.write(bias.data() + at, nb * 4);
+                }
+            }
+            at += n;
+        }
+        w.vec(list_sizes);
+        cell("bucket", begin);
+        // partition_strategy
+        begin = w.cursor();
+        w.obj(static_cast<uint8_t>(trained_ ? 1 : 0));
+        w.obj(static_cast<int32_t>(nlist_));
+        w.obj(static_cast<int64_t>(q_.dim));
+        w.obj(kCentroidTag);
+        std::vector<float> centroids(trained_ ? static_cast<size_t>(nlist_) * q_.dim : 0);
+        if (!centroids.empty()) {
+            dev(vsag_amd_memcpy_d2h(centroids.data(), centroids_.p, centroids.size() * 4, nullptr));
+        }
+        w.vec(centroids);
+        cell("partition_strategy", begin);
+        // label_table
+        begin = w.cursor();
+        w.vec(labels_);
+        cell("label_table", begin);
+        if (use_reorder_) {
+            begin = w.cursor();
+            if (pq_.kind == VSAG_AMD_KIND_FP32) {
+                Quantizer fp = pq_.blank();
+                fp.trained = trained_;
+                write_flat_cell(w, nullptr, &raw_, fp, labels_.size());
+            } else {
+                write_flat_cell(w, precise_.s, nullptr, pq_, labels_.size());
+            }
+            cell("reorder_codes", begin);
+        }
+        write_footer(w, "{\"_update_time\":\"1970-01-01 00:00:00\",\"basic_info\":{\"data_type\":0,\"dim\":" +
+                            std::to_string(q_.dim) + ",\"extra_info_size\":0,\"is_trained\":" +
+                            (trained_ ? "true" : "false") + ",\"metric\":" + std::to_string(q_.metric) +
+                            ",\"total_elements\":" + std::to_string(labels_.size()) + ",\"use_reorder\":" +
+                            (use_reorder_ ? "true" : "false") + "},\"datacell_offsets\":" + offsets +
+                            "},\"datacell_sizes\":" + sizes + "}}");
+    }
+
+    // IVF::Deserialize (ivf.cpp:1429-1530), footer form.
+    void
+    load(Reader& r) override {
+        if (!labels_.empty() || trained_) {
+            throw VsagException(ErrorType::INDEX_NOT_EMPTY, "failed to deserialize: index is not empty");
+        }
+        std::string metadata;
+        uint64_t footer_bytes = 0;
+        if (!read_footer(r, &metadata, &footer_bytes)) {
+            throw VsagException(ErrorType::INVALID_BINARY, "the serialized ivf index has no footer");
+        }
+        const Json m = Json::Parse(metadata);
+        if (m.Contains("_empty") && m["_empty"].GetBool()) {
+            return;
+        }
+        CHECK_ARGUMENT(m.Contains("basic_info") && m.Contains("datacell_offsets") && m.Contains("datacell_sizes"),
+                       "the footer of the serialized index lacks basic_info or the cells' offsets and sizes");
+        const Json& info = m["basic_info"];
+        const Json& offsets = m["datacell_offsets"];
+        const auto total = static_cast<uint64_t>(info["total_elements"].GetInt());
+        CHECK_ARGUMENT(info["dim"].GetInt() == static_cast<int64_t>(q_.dim), "the serialized index has another dim");
+        CHECK_ARGUMENT(!info.Contains("metric") || info["metric"].GetInt() == q_.metric,
+                       "the serialized index has another metric");
+        CHECK_ARGUMENT(info["use_reorder"].GetBool() == use_reorder_,
+                       "the serialized index and this one differ in use_reorder");
+        CHECK_ARGUMENT(total * bpd_ < VSAG_AMD_INVALID_ID, "the serialized index holds too many postings");
+        for (const char* name : {"bucket", "partition_strategy", "label_table"}) {
+            CHECK_ARGUMENT(offsets.Contains(name), std::string("the serialized index has no cell ") + name);
+        }
+        const bool file_trained = info["is_trained"].GetBool();
+
+        // partition_strategy first: the lists of a residual index need its centroids
+        r.seek(static_cast<uint64_t>(offsets["partition_strategy"].GetInt()));
+        (void)r.get<uint8_t>();
+        const auto file_lists = r.get<int32_t>();
+        const auto file_dim = r.get<int64_t>();
+        CHECK_ARGUMENT(file_lists == static_cast<int32_t>(nlist_) && file_dim == static_cast<int64_t>(q_.dim),
+                       "the serialized partition has " + std::to_string(file_lists) + " buckets of dim " +
+                           std::to_string(file_dim) + ", this index " + std::to_string(nlist_) + " of dim " +
+                           std::to_string(q_.dim));
+        std::vector<float> centroids;
+        if (r.get<uint64_t>() == kCentroidTag) {
+            r.vec(centroids);
+        } else {
+            r.seek(r.cursor() - 8);
+            read_router_image(r, centroids);
+        }
+        CHECK_ARGUMENT(!file_trained || centroids.size() == static_cast<size_t>(nlist_) * q_.dim,
+                       "the serialized partition does not hold one centroid per bucket");
+        DevBuf centroids_dev;
+        StoreHandle router;
+        if (file_trained) {
+            centroids_dev.reserve(centroids.size() * 4);
+            dev(vsag_amd_memcpy_h2d(centroids_dev.p, centroids.data(), centroids.size() * 4, nullptr));
+            Quantizer cq;
+            cq.kind = VSAG_AMD_KIND_FP32;
+            cq.metric = q_.metric;
+            cq.dim = q_.dim;
+            router.s = cq.make_store();
+            dev(vsag_amd_store_expect_stored_codes(router.s, 1));  // cosine: unit vectors already
+            dev(vsag_amd_store_append(router.s, centroids_dev.as<uint8_t>(), nlist_, nullptr));
+            dev(vsag_amd_store_expect_stored_codes(router.s, 0));
+        }
+
+        // bucket
+        r.seek(static_cast<uint64_t>(offsets["bucket"].GetInt()));
+        const auto buckets = r.get<int32_t>();
+        const auto cs = r.get<uint32_t>();
+        CHECK_ARGUMENT(buckets == static_cast<int32_t>(nlist_) && cs == q_.code_size(),
+                       "the serialized lists (" + std::to_string(buckets) + " of code size " + std::to_string(cs) +
+                           ") do not match the index (" + std::to_string(nlist_) + " of code size " +
+                           std::to_string(q_.code_size()) + ")");
+        Quantizer q = q_.blank();
+        q.load(r);
+        // the sizes lie behind the lists: a first walk finds them, the second one reads the lists
+        const uint64_t lists_at = r.cursor();
+        for (uint32_t l = 0; l < nlist_; ++l) {
+            r.skip(r.get<uint64_t>());
+            r.skip(r.get<uint64_t>() * 4);
+            if (use_residual_) {
+                r.skip(r.get<uint64_t>() * 4);
+            }
+        }
+        std::vector<uint32_t> list_sizes;
+        r.vec(list_sizes);
+        CHECK_ARGUMENT(list_sizes.size() == nlist_, "serialized bucket size vector does not match bucket count");
+        uint64_t postings = 0;
+        for (uint32_t n : list_sizes) {
+            postings += n;
+        }
+        if (postings != total * bpd_) {
+            throw VsagException(ErrorType::INVALID_BINARY, "the lists hold " + std::to_string(postings) + " codes for " +
+                                                               std::to_string(total) + " vectors with buckets_per_data " +
+                                                               std::to_string(bpd_));
+        }
+        const bool with_bias = use_residual_ && q_.metric == VSAG_AMD_METRIC_L2;
+        std::vector<uint8_t> codes(postings * cs);
+        std::vector<int32_t> bucket_of(postings, -1);
+        std::vector<float> bias(with_bias ? postings : 0, 0.0F);
+        std::vector<uint8_t> list_codes;
+        std::vector<uint32_t> list_ids;
+        std::vector<float> list_bias;
+        r.seek(lists_at);
+        for (uint32_t l = 0; l < nlist_; ++l) {
+            const uint64_t n = list_sizes[l];
+            const auto bytes = r.get<uint64_t>();
+            if (bytes < n * cs) {
+                throw VsagException(ErrorType::INVALID_BINARY, "a serialized list is shorter than its size");
+            }
+            list_codes.resize(n * cs);
+            r.read(list_codes.data(), n * cs);
+            r.skip(bytes - n * cs);
+            r.vec(list_ids);
+            if (list_ids.size() < n) {
+                throw VsagException(ErrorType::INVALID_BINARY,
+                                    "serialized bucket " + std::to_string(l) + " inner id count is smaller than bucket size");
+            }
+            if (use_residual_) {
+                r.vec(list_bias);
+                if (with_bias && list_bias.size() < n) {
+                    throw VsagException(ErrorType::INVALID_BINARY, "a serialized list lacks residual bias values");
+                }
+            }
+            for (uint64_t i = 0; i < n; ++i) {
+                const uint32_t id = list_ids[i];
+                if (id >= postings || bucket_of[id] != -1) {
+                    throw VsagException(ErrorType::INVALID_BINARY, "the serialized lists name inner id " +
+                                                                       std::to_string(id) + " twice or out of range");
+                }
+                bucket_of[id] = static_cast<int32_t>(l);
+                std::memcpy(codes.data() + static_cast<uint64_t>(id) * cs, list_codes.data() + i * cs, cs);
+                if (with_bias) {
+                    bias[id] = list_bias[i];
+                }
+            }
+        }
+        StoreHandle lists;
+        if (file_trained) {
+            lists.s = q.make_store();
+            dev(vsag_amd_store_expect_stored_codes(lists.s, 1));
+            if (use_residual_) {
+                dev(vsag_amd_store_set_residual(lists.s, centroids_dev.as<float>(), nlist_, nullptr));
+            }
+            dev(vsag_amd_store_set_lists(lists.s, nullptr, nullptr, 0, nlist_, nullptr));
+            const uint64_t step = std::max<uint64_t>(1, kIoChunkBytes / cs);
+            DevBuf dcodes, dlabels, dbias;
+            for (uint64_t first = 0; first < postings; first += step) {
+                const uint64_t n = std::min(step, postings - first);
+                dcodes.reserve(n * cs);
+                dlabels.reserve(n * 4);
+                dev(vsag_amd_memcpy_h2d(dcodes.p, codes.data() + first * cs, n * cs, nullptr));
+                dev(vsag_amd_memcpy_h2d(dlabels.p, bucket_of.data() + first, n * 4, nullptr));
+                if (with_bias) {
+                    dbias.reserve(n * 4);
+                    dev(vsag_amd_memcpy_h2d(dbias.p, bias.data() + first, n * 4, nullptr));
+                }
+                dev(vsag_amd_store_append_lists(lists.s, dcodes.as<uint8_t>(), dlabels.as<int32_t>(),
+                                                with_bias ? dbias.as<float>() : nullptr, n, nullptr));
+            }
+            dev(vsag_amd_store_expect_stored_codes(lists.s, 0));
+        }
+
+        // label_table
+        r.seek(static_cast<uint64_t>(offsets["label_table"].GetInt()));
+        std::vector<int64_t> labels;
+        r.vec(labels);
+        if (labels.size() < total) {
+            throw VsagException(ErrorType::INVALID_BINARY, "the serialized label table is shorter than the index");
+        }
+        labels.resize(total);
+
+        // reorder_codes
+        Quantizer pq = pq_.blank();
+        StoreHandle precise;
+        DevBuf raw;
+        if (use_reorder_) {
+            CHECK_ARGUMENT(offsets.Contains("reorder_codes"),
+                           "the serialized index keeps its precise codes list by list (precise_codes_layout = bucket), "
+                           "which is not read here");
+            r.seek(static_cast<uint64_t>(offsets["reorder_codes"].GetInt()));
+            const uint64_t n = pq_.kind == VSAG_AMD_KIND_FP32 ? read_flat_cell(r, pq, nullptr, &raw)
+                                                              : read_flat_cell(r, pq, &precise, nullptr);
+            if (n != total) {
+                throw VsagException(ErrorType::INVALID_BINARY, "the serialized precise codes do not cover the index");
+            }
+        }
+        dev(vsag_amd_stream_synchronize(nullptr));
+
+        q_.take(q);
+        pq_.take(pq);
+        std::swap(lists_.s, lists.s);
+        std::swap(centroid_store_.s, router.s);
+        std::swap(precise_.s, precise.s);
+        std::swap(centroids_.p, centroids_dev.p);
+        std::swap(centroids_.bytes, centroids_dev.bytes);
+        std::swap(raw_.p, raw.p);
+        std::swap(raw_.bytes, raw.bytes);
+        labels_.swap(labels);
+        rebuild_label_map(labels_, known_);
+        trained_ = file_trained;
+    }
+
+    // The router of the reference is an hgraph over the centroids (ivf_nearest_partition.cpp:150-153); of its image
+    // (hgraph_serialize.cpp:286-311,397-401) the label table and the flat cell of fp32 codes that follows it are read:
+    // centroid b is the code whose label is b.
+    void
+    read_router_image(Reader& r, std::vector<float>& centroids) const {
+        std::vector<int64_t> labels;
+        r.vec(labels);
+        r.skip(r.get<uint64_t>() * 12);  // the label -> inner id pairs
+        if (r.length() - r.cursor() >= 8) {
+            if (r.get<uint64_t>() == 0x534F555243454944ULL) {  // a table of source ids
+                const auto count = r.get<uint64_t>();
+                for (uint64_t i = 0; i < count; ++i) {
+                    r.skip(r.get<uint64_t>());
+                }
+            } else {
+                r.seek(r.cursor() - 8);
+            }
+        }
+        const auto total = r.get<uint32_t>();
+        (void)r.get<uint32_t>();
+        const auto cs = r.get<uint32_t>();
+        const auto bytes = r.get<uint64_t>();
+        if (cs != 4 * q_.dim || total != labels.size() || total != nlist_ || bytes < static_cast<uint64_t>(total) * cs) {
+            throw VsagException(ErrorType::INVALID_BINARY, "the router image does not hold one fp32 centroid per bucket");
+        }
+        std::vector<float> rows(static_cast<size_t>(total) * q_.dim);
+        r.read(rows.data(), rows.size() * 4);
+        centroids.assign(rows.size(), 0.0F);
+        for (uint32_t i = 0; i < total; ++i) {
+            if (labels[i] < 0 || labels[i] >= static_cast<int64_t>(nlist_)) {
+                throw VsagException(ErrorType::INVALID_BINARY, "the router image names a bucket that does not exist");
+            }
+            std::memcpy(centroids.data() + static_cast<size_t>(labels[i]) * q_.dim, rows.data() + static_cast<size_t>(i) * q_.dim,
+                        static_cast<size_t>(q_.dim) * 4);
+        }
     }
 
 private:

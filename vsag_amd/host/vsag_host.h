@@ -11,6 +11,7 @@
 
 #include <cstdint>
 #include <functional>
+#include <iosfwd>
 #include <memory>
 #include <string>
 #include <utility>
@@ -294,6 +295,14 @@ public:
     virtual Expected<DatasetPtr>
     CalDistanceById(const DatasetPtr& query, const int64_t* ids, int64_t count, bool calculate_precise_distance = true,
                     int64_t topk = -1) const = 0;
+
+    // include/vsag/index.h:903-940: the index as one stream (cells of codes, quantizer state and labels in the layout
+    // of the reference, a footer with basic_info at the end) and back; Deserialize wants an empty index and a seekable
+    // stream.
+    virtual Expected<void>
+    Serialize(std::ostream& out) const = 0;
+    virtual Expected<void>
+    Deserialize(std::istream& in) = 0;
 
     // Train + Add.  Returns the ids that could not be inserted (duplicates of ids already present).
     virtual Expected<std::vector<int64_t>>

@@ -94,6 +94,10 @@ VSAG_HOST_API Error_t vsag_index_calculate_distances(vsag_index_t index, const f
 VSAG_HOST_API Error_t vsag_search_result_enable_statistics(SearchResult_t* search_result);
 VSAG_HOST_API const char* vsag_search_result_get_statistics(const SearchResult_t* search_result);
 VSAG_HOST_API void vsag_search_result_destroy_statistics(SearchResult_t* search_result);
+/* include/vsag/vsag_c_api.h:327-330: the index to a file (Index::Serialize(std::ostream&)) and back into an empty
+ * index made with the same parameters. */
+VSAG_HOST_API Error_t vsag_serialize_file(vsag_index_t index, const char* file_path);
+VSAG_HOST_API Error_t vsag_deserialize_file(vsag_index_t index, const char* file_path);
 VSAG_HOST_API int64_t vsag_index_get_num_elements(vsag_index_t index);
 /* Number of ids the last build / add on this thread could not insert (duplicates). */
 VSAG_HOST_API int64_t vsag_last_failed_id_count(void);

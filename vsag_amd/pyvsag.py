@@ -1,7 +1,8 @@
 """Python view of the GPU-backed index classes with the call shapes of the reference's pyvsag.Index
 (python_bindings/index_binding.cpp:641-716): Index(name, parameters), build(vectors, ids, num_elements, dim),
 add(...), knn_search(vector, k, parameters) -> (ids, dists), range_search(point, threshold, parameters),
-get_num_elements(), train(...), cal_distance_by_id(query, ids, ...).  Additions: knn_search_batch (many queries per
+get_num_elements(), train(...), cal_distance_by_id(query, ids, ...), serialize(path) / deserialize(path) (the file forms of
+the binding's save / load).  Additions: knn_search_batch (many queries per
 call, optionally with the buckets every query scans), the `filter` / `limit` keywords (the C API's *_with_filter entry
 points: filter(label) == True filters the vector out) and `statistics=True` (the search's statistics JSON as a third
 result).  Everything goes through libvsag_amd_host.so's C API; errors raise
@@ -16,7 +17,8 @@ HOST_LIB_PATH = os.path.join(_HERE, "lib", "libvsag_amd_host.so")
 
 ERROR_NAMES = {0: "SUCCESS", -1: "UNKNOWN_ERROR", -2: "INTERNAL_ERROR", -3: "INVALID_ARGUMENT", -4: "WRONG_STATUS",
                -5: "BUILD_TWICE", -6: "INDEX_NOT_EMPTY", -7: "UNSUPPORTED_INDEX", -8: "UNSUPPORTED_INDEX_OPERATION",
-               -9: "DIMENSION_NOT_EQUAL", -10: "INDEX_EMPTY", -11: "NO_ENOUGH_MEMORY"}
+               -9: "DIMENSION_NOT_EQUAL", -10: "INDEX_EMPTY", -11: "NO_ENOUGH_MEMORY", -12: "READ_ERROR",
+               -13: "MISSING_FILE", -14: "INVALID_BINARY"}
 
 
 class ErrorT(C.Structure):
@@ -88,6 +90,10 @@ def _load():
         lib.vsag_search_result_get_statistics.argtypes = [C.POINTER(SearchResult)]
         lib.vsag_search_result_destroy_statistics.restype = None
         lib.vsag_search_result_destroy_statistics.argtypes = [C.POINTER(SearchResult)]
+        for name in ("vsag_serialize_file", "vsag_deserialize_file"):
+            fn = getattr(lib, name)
+            fn.restype = ErrorT
+            fn.argtypes = [C.c_void_p, C.c_char_p]
         lib.vsag_index_get_num_elements.restype = C.c_int64
         lib.vsag_index_get_num_elements.argtypes = [C.c_void_p]
         lib.vsag_last_failed_id_count.restype = C.c_int64
@@ -209,6 +215,14 @@ class Index:
                                                  flat.ctypes.data, offsets.ctypes.data,
                                                  ids.ctypes.data, dists.ctypes.data, C.byref(rdim)))
         return ids, dists
+
+    def serialize(self, path):
+        """The index as one file in the reference's stream layout (cells of codes, quantizer state, labels, footer)."""
+        _check(_load().vsag_serialize_file(self._h, str(path).encode()))
+
+    def deserialize(self, path):
+        """Loads a file written by serialize() (or by the reference) into this empty index."""
+        _check(_load().vsag_deserialize_file(self._h, str(path).encode()))
 
     def get_num_elements(self):
         return int(_load().vsag_index_get_num_elements(self._h))
