@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F32_PEAK_TFLOPS = 157.3
 MFMA_I8_PEAK_TOPS = 5000.0  # dense int8, published
 # HBM/fabric bytes of the last-level launch of prefilter_i8_kernel<l2> on configs[1] (profiles/prefilter_i8_sq8_c2.md)
-PROFILE_TRAFFIC_I8_C2 = 2422324.4 * 2.00 * 1024 + 68345.8 * 1024
+PROFILE_TRAFFIC_I8_C2 = 235670.3 * 2.00 * 1024 + 60099.9 * 1024
 
 
 def mt(seed):
