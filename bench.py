@@ -489,6 +489,10 @@ def run_c4(env):
     args, capi, lib = env.args, env.capi, env.lib
     n, d, nq, k = args.n or 10000000, args.dim or 128, args.nq or 10000, args.k
     nlist, nprobe, kcand = args.nlist or 4096, 64, 100
+    # --list-codes sq8_uniform: the same search over sq8_uniform lists (a byte per dimension)
+    bits = 8 if args.list_codes == "sq8_uniform" else 4
+    kind = capi.KIND_SQ8_UNIFORM if bits == 8 else capi.KIND_SQ4_UNIFORM
+    kind_name = "sq8_uniform" if bits == 8 else "sq4_uniform"
     means = mt(315).random((10000, d), dtype=np.float32)
     x_dev = env.buf(n * d * 4)
     pick = np.sort(mt(7).choice(n, nlist, replace=False))
@@ -515,13 +519,13 @@ def run_c4(env):
     bounds = env.buf(8)
     wsb = lib.vsag_amd_sq_train_workspace_bytes(ns, d, 0)
     ws = env.buf(wsb)
-    capi.check(lib.vsag_amd_sq_train_uniform(x_dev.ptr, ns, d, 4, capi.METRIC_L2, capi.SQ_TRAIN_TRUNC_BOUND, 0.05, 0,
+    capi.check(lib.vsag_amd_sq_train_uniform(x_dev.ptr, ns, d, bits, capi.METRIC_L2, capi.SQ_TRAIN_TRUNC_BOUND, 0.05, 0,
                                              bounds.ptr, ws.ptr, wsb, None))
     ws.free()
-    cs = int(lib.vsag_amd_code_size(capi.KIND_SQ4_UNIFORM, capi.METRIC_L2, d, 0))
+    cs = int(lib.vsag_amd_code_size(kind, capi.METRIC_L2, d, 0))
     codes = env.buf(n * cs)
-    capi.check(lib.vsag_amd_squ_encode(x_dev.ptr, n, d, 4, capi.METRIC_L2, bounds.ptr, codes.ptr, None))
-    lists = env.make_store(capi.KIND_SQ4_UNIFORM, capi.METRIC_L2, d, bounds=bounds)
+    capi.check(lib.vsag_amd_squ_encode(x_dev.ptr, n, d, bits, capi.METRIC_L2, bounds.ptr, codes.ptr, None))
+    lists = env.make_store(kind, capi.METRIC_L2, d, bounds=bounds)
     capi.check(lib.vsag_amd_store_set_lists(lists, codes.ptr, labels.ptr, n, nlist, None))
     cstore = env.make_store(capi.KIND_FP32, capi.METRIC_L2, d)
     capi.check(lib.vsag_amd_store_append(cstore, cent.ptr, nlist, None))
@@ -593,11 +597,12 @@ def run_c4(env):
         hb = bounds.to_numpy(np.float32, (2,))
         offsets, order = orc.ivf_build_lists(hlabels, nlist)
         posting = hcodes[order]
-        qcodes = orc.squ_encode(q[:sample], 4, hb[0], hb[1], orc.L2)
-        orc.ivf_scan(orc.SQ4U, orc.L2, d, posting, offsets, order, qcodes[:threads], b[:threads], kcand,
+        okind = orc.SQ8U if bits == 8 else orc.SQ4U
+        qcodes = orc.squ_encode(q[:sample], bits, hb[0], hb[1], orc.L2)
+        orc.ivf_scan(okind, orc.L2, d, posting, offsets, order, qcodes[:threads], b[:threads], kcand,
                      lb=hb[0], diff=hb[1], threads=threads)
         t0 = time.perf_counter()
-        cids, cds = orc.ivf_scan(orc.SQ4U, orc.L2, d, posting, offsets, order, qcodes, b[:sample], kcand,
+        cids, cds = orc.ivf_scan(okind, orc.L2, d, posting, offsets, order, qcodes, b[:sample], kcand,
                                  lb=hb[0], diff=hb[1], threads=threads)
         t_cpu = time.perf_counter() - t0
         gcand = cand.to_numpy(np.uint32, (nq, kcand))[:sample]
@@ -612,8 +617,8 @@ def run_c4(env):
             rids[i] = cids[i][np.lexsort((cids[i], dd))[:k]]
         cpu = {"value": sample / t_cpu, "unit": "queries/s", "cores": threads, "kind": "port",
                "sample": "%d of the %d queries, CPU restatement of IVF::search (scan of the same %d probed lists per "
-                         "query with the strict-< heap) on the same SQ4-uniform codes, OpenMP over queries; rerank in "
-                         "fp64 on the host" % (sample, nq, nprobe),
+                         "query with the strict-< heap) on the same %s codes, OpenMP over queries; rerank in "
+                         "fp64 on the host" % (sample, nq, nprobe, kind_name),
                "candidate_distances_bit_equal": bool(np.array_equal(cds.view(np.uint32), gcd.view(np.uint32))),
                "candidate_overlap_with_gpu": float(np.mean([len(set(a) & set(bb)) / float(kcand)
                                                             for a, bb in zip(cids, gcand)])),
@@ -629,10 +634,10 @@ def run_c4(env):
     # configuration, profiles/ivf_scan_sq4u_c4.md.  Work items that share a list are co-scheduled and read it
     # through L2 once per <= 4 queries, so the fraction against HBM exceeds 1: this kernel is bound by VALU issue.
     traffic = None
-    if (n, d, nq, k, nlist) == (10000000, 128, 10000, 10, 4096) and tile.value != 256:
+    if (n, d, nq, k, nlist, bits) == (10000000, 128, 10000, 10, 4096, 4) and tile.value != 256:
         traffic = (482513.06 + 1698762.06) * 2.00 * 1024 + (9817.03 + 19915.53) * 1024
     roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-            "traffic": traffic, "kernel": "ivf_scan_kernel<sq4_uniform, l2> (2 launches per step)", "kernel_ms": kms,
+            "traffic": traffic, "kernel": "ivf_scan_kernel<%s, l2> (2 launches per step)" % kind_name, "kernel_ms": kms,
             "algorithmic_bytes_per_launch": algo,
             "distance_evaluations_per_second": float(scanned) / (kms * 1e-3)}
     if tile.value == 256:
@@ -645,13 +650,14 @@ def run_c4(env):
                 "frac": tops / MFMA_I8_PEAK_TOPS,
                 # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this launch: profiles/ivf_i8_sq4u_c4.md
                 "traffic": 490258.9 * 2.00 * 1024 + 73488.6 * 1024
-                if (n, d, nq, k, nlist) == (10000000, 128, 10000, 10, 4096) else None,
-                "kernel": "ivf_i8_kernel (int8 MFMA, probe columns 1..%d)" % (nprobe - 1), "kernel_ms": kms,
+                if (n, d, nq, k, nlist, bits) == (10000000, 128, 10000, 10, 4096, 4) else None,
+                "kernel": "ivf_i8_kernel<%s> (int8 MFMA, probe columns 1..%d)" % (kind_name, nprobe - 1), "kernel_ms": kms,
                 "ops_per_launch": ops, "distance_evaluations_per_launch": float(rest),
                 "distance_evaluations_per_second": float(rest) / (kms * 1e-3)}
-    return env.base_line("QPS @ recall@10 (IVF SQ4-uniform, 10M x 128)", "queries/s", nq / sec, sec,
-                         "u4 codes, i32 dot", "configs[3]: IVF search, N=%d, d=%d, nlist=%d, nprobe=%d, rerank %d, "
-                         "%d queries, k=%d" % (n, d, nlist, nprobe, kcand, nq, k),
+    return env.base_line("QPS @ recall@10 (IVF %s, 10M x 128)" % ("SQ4-uniform" if bits == 4 else "SQ8-uniform"),
+                         "queries/s", nq / sec, sec, "u%d codes, i32 dot" % bits,
+                         "configs[3]%s: IVF search, N=%d, d=%d, nlist=%d, nprobe=%d, rerank %d, %d queries, k=%d"
+                         % ("" if bits == 4 else " with sq8_uniform lists", n, d, nlist, nprobe, kcand, nq, k),
                          {"recall_at_10": rec, "build_seconds": t_build, "scanned_codes_per_query": float(scanned) / nq,
                           "bytes_per_scanned_code": cs + 4, "single_query": single}, roof, cpu)
 
@@ -789,6 +795,8 @@ def main():
     ap.add_argument("--chunks", type=int, default=0, help="base chunk override (0 = library default)")
     ap.add_argument("--contraction", type=int, default=0, choices=[-1, 0, 1],
                     help="matrix-core path of the flat scans: -1 never, 0 library default, 1 whenever supported")
+    ap.add_argument("--list-codes", default="sq4_uniform", choices=["sq4_uniform", "sq8_uniform"],
+                    help="c4 only: the quantizer of the posting lists (configs[3] names sq4_uniform)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-recall", action="store_true", help="skip the recall check")
     ap.add_argument("--no-single", action="store_true", help="skip the one-query-per-call measurement")

@@ -56,6 +56,17 @@ class Store:
         cbuf.free()
         lbuf.free()
 
+    def append_lists(self, codes, labels, bias=None):
+        codes = np.ascontiguousarray(codes)
+        cbuf, lbuf = dev(codes), dev(np.ascontiguousarray(labels, np.int32))
+        bbuf = dev(np.ascontiguousarray(bias, np.float32)) if bias is not None else None
+        capi.check(self.lib.vsag_amd_store_append_lists(self.handle, cbuf.ptr, lbuf.ptr,
+                                                        bbuf.ptr if bbuf is not None else None, codes.shape[0], None))
+        capi.synchronize()
+        for b in (cbuf, lbuf, bbuf):
+            if b is not None:
+                b.free()
+
     def size(self):
         return int(self.lib.vsag_amd_store_size(self.handle))
 

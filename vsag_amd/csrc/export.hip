@@ -51,6 +51,9 @@ untile_kernel(UntileArgs a) {
         dst[off] = 0;
     }
     for (uint32_t m = 0; m < a.nmeta; ++m) {
+        if (a.meta_offset[m] == kMetaPayloadSum) {
+            continue;  // no field of the code
+        }
         uint8_t* p = dst + a.meta_offset[m];
         if ((a.meta_is_u64 >> m) & 1U) {
             // The store keeps this integer as a float; the code holds it exactly: the sum of the squared code values

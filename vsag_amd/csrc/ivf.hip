@@ -780,7 +780,7 @@ struct IvfBuffers {
     uint32_t* partial_cnt;
     uint64_t* partial;
     uint32_t* gate;       // mfma: nq + 2 (flags, raised gates, their pairs)
-    int32_t* tq;          // mfma: nq + 1
+    int32_t* tq;          // mfma: 2 (nq + 1)
     uint32_t* gpairs;     // mfma: pairs of gated queries, kGatedPairsCap
     float* res_term;      // residual lists: per pair
 };
@@ -831,7 +831,7 @@ plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, 
         p->chunks_max = static_cast<uint32_t>(cap);
     }
     p->seeded = p->chunked && kcand <= 256;
-    // Large batches on sq4_uniform / L2 lists: the streaming kernel scans the nearest list of every query, the int8
+    // Large batches on sq4_uniform (and sq8_uniform / l2) lists: the streaming kernel scans the nearest list of every query, the int8
     // matrix cores the other columns, into two private lists per (query, list) pair.
     p->mfma = !p->chunked && nprobe > 1 && scan_contraction_mode() >= 0 && ivf_i8_supports(s) &&
               s->residual_centroids_dev == nullptr &&
@@ -857,7 +857,7 @@ carve_ivf(Carver& c, const vsag_amd_store* s, const ScanPlanIvf& p, uint64_t nq,
     b->partial = c.take<uint64_t>(p.npairs * p.chunks_max * kcand);
     b->gate = c.take<uint32_t>(p.mfma ? nq + 2 : 0);
     b->gpairs = c.take<uint32_t>(p.mfma ? kGatedPairsCap : 0);
-    b->tq = c.take<int32_t>(p.mfma ? nq + 1 : 0);
+    b->tq = c.take<int32_t>(p.mfma ? 2 * (nq + 1) : 0);  // thresholds, then (sq8_uniform) the sums of the query values
     b->res_term = c.take<float>(s->residual_centroids_dev != nullptr ? p.npairs : 0);
     return c.used;
 }

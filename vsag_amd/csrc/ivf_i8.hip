@@ -1,4 +1,5 @@
-// Posting lists of sq4_uniform codes (at most 128 dimensions) against large query batches, on the int8 matrix cores.
+// Posting lists of sq4_uniform codes (and, l2 only, sq8_uniform codes; at most 128 dimensions) against large query
+// batches, on the int8 matrix cores.
 //
 // The streaming IVF kernel (ivf.hip) is bound by vector-ALU issue: every (query, code) pair costs sixteen dot4
 // instructions.  The distance of this quantizer is a function of integers only,
@@ -14,6 +15,16 @@
 // charged against A_q, and what passes is re-checked with the streaming kernel's own operations.
 // The kernel serves the probe columns behind the first one: the nearest list of every query has been
 // scanned by the streaming kernel, which leaves the bound.
+//
+// sq8_uniform, l2 (sq8_uniform_quantizer.cpp:204-250): the same distance formula with byte values 0..255 on both
+// sides; every integer in it stays below 2^24 up to 128 dimensions, so the test is an integer test again.  The
+// matrix cores take signed bytes: code and query are both centred, o' = o - 128, q' = q - 128 (q' = 0 beyond the
+// dimension), and with X = <q', o'> over the real dimensions
+//      <q, o> = X + 128 sum_q + 128 sum_o - 128^2 dim.
+// sum_o is kept per slot next to No (store.h, kMetaPayloadSum), sum_q is formed once per query.  The accumulator
+// starts from C_o = ceil((256 sum_o - No) / 2), so the pipe delivers X + C_o, and 2 <q, o> - No >= Tq becomes
+// X + C_o >= floor((Tq - 256 sum_q + 2 128^2 dim) / 2) -- a test that keeps every pair of the real one and at most
+// the pairs one unit beyond it, which ivf_i8_finish_kernel drops when it forms the distance.
 //
 // Work split: the (query, list) pairs are grouped by list as for the streaming kernel; a workgroup is a chunk of a
 // list's tiles and up to 256 of its pairs, four waves of 64.  It walks the chunk two tiles per LDS stage; staging
@@ -98,10 +109,42 @@ ivf_i8_threshold_kernel(const uint32_t* bound, const float* qmeta, uint32_t qmet
     tq[q] = static_cast<int32_t>(v);
 }
 
+// sq8_uniform: sum_q per query from its byte row, and the threshold of the centred product (see the header) in place
+// of Tq.  One thread per query; tq[nq] (the dummy row) and the two sentinels stay as they are.
+__global__ void __launch_bounds__(256)
+ivf_i8_centre_threshold_kernel(const uint32_t* qtab, uint32_t qstride, uint32_t dim, uint64_t nq, int32_t* tq,
+                               int32_t* qsum) {
+    const uint64_t q = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (q > nq) {
+        return;
+    }
+    uint32_t sum = 0;
+    if (q < nq) {
+        const uint32_t* row = qtab + q * qstride;
+        for (uint32_t w = 0; 4 * w < dim; ++w) {
+            uint32_t v = row[w];
+            if (4 * w + 4 > dim) {
+                v &= 0xFFFFFFFFU >> (8 * (4 * w + 4 - dim));
+            }
+            sum = __builtin_amdgcn_udot4(v, 0x01010101U, sum, false);
+        }
+    }
+    qsum[q] = static_cast<int32_t>(sum);
+    const int32_t t = tq[q];
+    if (t == 0x7FFFFFFF || t == static_cast<int32_t>(0x80000000U)) {
+        return;
+    }
+    int64_t v = (static_cast<int64_t>(t) - 256LL * sum + 32768LL * dim) >> 1;  // floor
+    v = v > 0x7FFFFFFELL ? 0x7FFFFFFELL : (v < -0x7FFFFFFFLL ? -0x7FFFFFFFLL : v);
+    tq[q] = static_cast<int32_t>(v);
+}
+
 struct IvfI8Args {
     const uint4* tiles;
-    uint32_t G;                  // granules per code (<= 4)
+    uint32_t G;                  // granules per code (sq4_uniform <= 4, sq8_uniform <= 8)
+    uint32_t dim;
     const uint32_t* meta;        // per slot: No as float bits
+    const uint32_t* meta_sum;    // sq8_uniform: per slot, the sum of the code values
     const uint32_t* ids;         // inner id per tile slot
     const uint32_t* list_tile;   // 2 nlist: first tile and end of the used tiles of every list
     const uint32_t* pair_off;    // nlist + 1
@@ -123,13 +166,22 @@ struct IvfI8Args {
 };
 
 struct IvfI8Stage {
-    uint4 codes[kIvfI8StageTiles][8 * kWave];  // [2 granule + nibble half][code]: one nibble per byte
-    int32_t term[kIvfI8StageTiles][kWave];     // -No per code
+    // sq4_uniform: [2 granule + nibble half][code], one nibble per byte; sq8_uniform: [granule][code], bytes - 128
+    uint4 codes[kIvfI8StageTiles][8 * kWave];
+    int32_t term[kIvfI8StageTiles][kWave];     // what the accumulator of a code starts from (-No; sq8_uniform: C_o)
 };
 
-template <int METRIC>
+// ceil((256 sum_o - No) / 2); 256 sum_o >= No because every value is at most 255.
+__device__ inline int32_t
+ivf_i8_centre_term(uint32_t sum_o, float no) {
+    return (static_cast<int32_t>(256U * sum_o) - static_cast<int32_t>(no) + 1) >> 1;
+}
+
+template <int KIND, int METRIC>
 __global__ void __launch_bounds__(256, 2)
 ivf_i8_kernel(IvfI8Args p) {
+    constexpr bool kBytes = KIND == VSAG_AMD_KIND_SQ8_UNIFORM;  // a byte per dimension (l2 only)
+    static_assert(!kBytes || METRIC == VSAG_AMD_METRIC_L2, "sq8_uniform lists take this route under l2 only");
     __shared__ IvfI8Stage stage[2];
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
@@ -185,6 +237,22 @@ ivf_i8_kernel(IvfI8Args p) {
         const uint4* rowp = reinterpret_cast<const uint4*>(p.qtab + static_cast<uint64_t>(qidx[j]) * p.qstride);
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
+            if constexpr (kBytes) {
+                // Step s, this half: dimensions 32 s + 16 half ... + 15, centred; zero beyond the dimension (and for
+                // the dummy row, whose threshold nothing meets anyway).
+                const uint32_t d0 = 32 * s + 16 * half;
+                uint4 x = make_uint4(0, 0, 0, 0);
+                if (2 * s + half < p.G) {
+                    x = rowp[2 * s + half];
+                }
+                auto centre = [&](uint32_t w, uint32_t d) {
+                    const uint32_t c = w ^ 0x80808080U;
+                    return d + 4 <= p.dim ? c : (d >= p.dim ? 0U : c & (0xFFFFFFFFU >> (8 * (d + 4 - p.dim))));
+                };
+                qv[j][s] = intx4{static_cast<int>(centre(x.x, d0)), static_cast<int>(centre(x.y, d0 + 4)),
+                                 static_cast<int>(centre(x.z, d0 + 8)), static_cast<int>(centre(x.w, d0 + 12))};
+                continue;
+            }
             uint4 x0 = make_uint4(0, 0, 0, 0), x1 = make_uint4(0, 0, 0, 0);
             if (static_cast<uint32_t>(s) < p.G) {
                 x0 = rowp[2 * s];
@@ -206,23 +274,33 @@ ivf_i8_kernel(IvfI8Args p) {
 
     // Staging: wave w copies granule w of both tiles of the stage, a lane per code; the nibbles are split on the
     // way into LDS.  Wave t also brings the -No terms of tile t.
-    uint4 regs[kIvfI8StageTiles];
+    // (sq8_uniform: wave w copies granules w and w + 4, centring the bytes.)
+    uint4 regs[kIvfI8StageTiles][kBytes ? 2 : 1];
     int32_t my_term = 0;
     auto fetch = [&](uint32_t sg) {
 #pragma unroll
         for (int tt = 0; tt < kIvfI8StageTiles; ++tt) {
             const uint32_t tile = tile_begin + sg * kIvfI8StageTiles + tt;
-            regs[tt] = make_uint4(0, 0, 0, 0);
-            if (tile < tile_end && wave < p.G) {
-                regs[tt] = p.tiles[(static_cast<uint64_t>(tile) * p.G + wave) * kWave + lane];
+#pragma unroll
+            for (int r = 0; r < (kBytes ? 2 : 1); ++r) {
+                const uint32_t g = wave + 4 * r;
+                const uint32_t none = kBytes ? 0x80808080U : 0U;
+                regs[tt][r] = make_uint4(none, none, none, none);
+                if (tile < tile_end && g < p.G) {
+                    regs[tt][r] = p.tiles[(static_cast<uint64_t>(tile) * p.G + g) * kWave + lane];
+                }
             }
             if (wave == static_cast<uint32_t>(tt)) {
                 // l2: -No; inner product: the bits of g * sum_o, g = -lb / rate.  Padding tiles never pass.
                 my_term = METRIC == VSAG_AMD_METRIC_L2 ? static_cast<int32_t>(0xC0000000U) : 0x7F800000;
                 if (tile < tile_end) {
                     const float m0 = __uint_as_float(p.meta[static_cast<uint64_t>(tile) * kWave + lane]);
-                    my_term = METRIC == VSAG_AMD_METRIC_L2 ? -static_cast<int32_t>(m0)
-                                                           : __float_as_int(m0 * (-p.lb / p.rate));
+                    if constexpr (kBytes) {
+                        my_term = ivf_i8_centre_term(p.meta_sum[static_cast<uint64_t>(tile) * kWave + lane], m0);
+                    } else {
+                        my_term = METRIC == VSAG_AMD_METRIC_L2 ? -static_cast<int32_t>(m0)
+                                                               : __float_as_int(m0 * (-p.lb / p.rate));
+                    }
                 }
             }
         }
@@ -230,11 +308,21 @@ ivf_i8_kernel(IvfI8Args p) {
     auto park = [&](IvfI8Stage& st) {
 #pragma unroll
         for (int tt = 0; tt < kIvfI8StageTiles; ++tt) {
-            const uint4 v = regs[tt];
-            st.codes[tt][(2 * wave) * kWave + lane] =
-                make_uint4(v.x & 0x0F0F0F0FU, v.y & 0x0F0F0F0FU, v.z & 0x0F0F0F0FU, v.w & 0x0F0F0F0FU);
-            st.codes[tt][(2 * wave + 1) * kWave + lane] = make_uint4((v.x >> 4) & 0x0F0F0F0FU, (v.y >> 4) & 0x0F0F0F0FU,
-                                                                       (v.z >> 4) & 0x0F0F0F0FU, (v.w >> 4) & 0x0F0F0F0FU);
+            if constexpr (kBytes) {
+#pragma unroll
+                for (int r = 0; r < 2; ++r) {
+                    const uint4 v = regs[tt][r];
+                    st.codes[tt][(wave + 4 * r) * kWave + lane] =
+                        make_uint4(v.x ^ 0x80808080U, v.y ^ 0x80808080U, v.z ^ 0x80808080U, v.w ^ 0x80808080U);
+                }
+            } else {
+                const uint4 v = regs[tt][0];
+                st.codes[tt][(2 * wave) * kWave + lane] =
+                    make_uint4(v.x & 0x0F0F0F0FU, v.y & 0x0F0F0F0FU, v.z & 0x0F0F0F0FU, v.w & 0x0F0F0F0FU);
+                st.codes[tt][(2 * wave + 1) * kWave + lane] =
+                    make_uint4((v.x >> 4) & 0x0F0F0F0FU, (v.y >> 4) & 0x0F0F0F0FU, (v.z >> 4) & 0x0F0F0F0FU,
+                               (v.w >> 4) & 0x0F0F0F0FU);
+            }
             if (wave == static_cast<uint32_t>(tt)) {
                 st.term[tt][lane] = my_term;
             }
@@ -405,13 +493,16 @@ struct IvfI8FinishArgs {
     uint32_t k, nprobe, p0, per_pair;  // probe columns p0 .. nprobe - 1 hold records, the ones before them keys
     const uint32_t* ids;
     const uint32_t* meta;
+    const uint32_t* meta_sum;  // sq8_uniform: sum of the code values per slot
+    const int32_t* qsum;       // sq8_uniform: sum of the query's values
+    uint32_t dim;
     const float* qmeta;
     uint32_t qmeta_stride;
     const uint32_t* bound;
     float lb, rate, lb2;
 };
 
-template <int METRIC>
+template <int KIND, int METRIC>
 __global__ void __launch_bounds__(256)
 ivf_i8_finish_kernel(IvfI8FinishArgs p) {
     const uint64_t list = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
@@ -441,7 +532,14 @@ ivf_i8_finish_kernel(IvfI8FinishArgs p) {
         }
         const float m0 = __uint_as_float(p.meta[slot]);
         float dist;
-        if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+        if constexpr (KIND == VSAG_AMD_KIND_SQ8_UNIFORM) {
+            // acc = X + C_o, <q, o> = X + 128 sum_q + 128 sum_o - 128^2 dim (see the header)
+            const uint32_t so = p.meta_sum[slot];
+            const int32_t ip = acc - ivf_i8_centre_term(so, m0) + 128 * p.qsum[q] + static_cast<int32_t>(128U * so) -
+                               static_cast<int32_t>(16384U * p.dim);
+            const float result = static_cast<float>(ip);
+            dist = (qm + m0 - 2 * result) * p.rate;
+        } else if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
             // acc = 2 <q, o> - No with No = m0, an integer
             const float result = static_cast<float>((acc + static_cast<int32_t>(m0)) >> 1);
             dist = (qm + m0 - 2 * result) * p.rate;
@@ -490,24 +588,36 @@ ivf_i8_lists_per_pair() {
 
 bool
 ivf_i8_supports(const vsag_amd_store* s) {
+    if (s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
+        return s->metric == VSAG_AMD_METRIC_L2 && s->G <= 8 && s->dim <= 128 && s->nmeta == 2 && s->nlist > 0 &&
+               s->scalar_rate > 0.0F;
+    }
     return s->kind == VSAG_AMD_KIND_SQ4_UNIFORM && s->G <= 4 && s->nlist > 0 && s->scalar_rate > 0.0F;
 }
 
 // The pairs of probe columns [p0, nprobe) are grouped by list (pair_off, sorted_pair) and item_off counts
 // workgroups per list (blocks of 256 pairs x tile chunks: offsets_kernel with T = 256, kIvfI8ChunkTiles,
-// kIvfI8Chunks); `bound` holds what the first columns left.  tq: nq + 1 words; gate: nq + 2 words, zeroed.
+// kIvfI8Chunks); `bound` holds what the first columns left.  tq: 2 (nq + 1) words; gate: nq + 2 words, zeroed.
 int
 launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
               const uint32_t* pair_off, const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound,
               int32_t* tq, uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, const int32_t* buckets,
               uint32_t* gpairs, uint32_t gpairs_cap, hipStream_t st) {
     const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
+    const bool bytes = s->kind == VSAG_AMD_KIND_SQ8_UNIFORM;
+    int32_t* qsum = tq + nq + 1;
     hipLaunchKernelGGL(ivf_i8_threshold_kernel, dim3(static_cast<uint32_t>(div_up(nq + 1, 256))), dim3(256), 0, st, bound,
                        a.qmeta, a.qmeta_stride, l2 ? 1 : 0, a.f0, a.f1, a.f2, s->dpad, nq, tq);
+    if (bytes) {
+        hipLaunchKernelGGL(ivf_i8_centre_threshold_kernel, dim3(static_cast<uint32_t>(div_up(nq + 1, 256))), dim3(256), 0,
+                           st, a.qtab, a.qstride, s->dim, nq, tq, qsum);
+    }
     IvfI8Args p{};
     p.tiles = s->tiles;
     p.G = s->G;
+    p.dim = s->dim;
     p.meta = a.meta;
+    p.meta_sum = bytes ? a.meta + a.meta_stride : nullptr;
     p.ids = s->ids_dev;
     p.list_tile = s->list_tile_dev;
     p.pair_off = pair_off;
@@ -533,11 +643,14 @@ launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     const uint64_t pairs = nq * (nprobe - p0);
     const uint64_t max_items =
         (div_up(pairs, static_cast<uint64_t>(kIvfI8Pairs)) + std::min<uint64_t>(s->nlist, pairs)) * kIvfI8Chunks;
+    const dim3 grid(static_cast<uint32_t>(max_items));
     timing_begin(st);
-    if (l2) {
-        hipLaunchKernelGGL(ivf_i8_kernel<VSAG_AMD_METRIC_L2>, dim3(static_cast<uint32_t>(max_items)), dim3(256), 0, st, p);
+    if (bytes) {
+        hipLaunchKernelGGL((ivf_i8_kernel<VSAG_AMD_KIND_SQ8_UNIFORM, VSAG_AMD_METRIC_L2>), grid, dim3(256), 0, st, p);
+    } else if (l2) {
+        hipLaunchKernelGGL((ivf_i8_kernel<VSAG_AMD_KIND_SQ4_UNIFORM, VSAG_AMD_METRIC_L2>), grid, dim3(256), 0, st, p);
     } else {
-        hipLaunchKernelGGL(ivf_i8_kernel<VSAG_AMD_METRIC_IP>, dim3(static_cast<uint32_t>(max_items)), dim3(256), 0, st, p);
+        hipLaunchKernelGGL((ivf_i8_kernel<VSAG_AMD_KIND_SQ4_UNIFORM, VSAG_AMD_METRIC_IP>), grid, dim3(256), 0, st, p);
     }
     timing_end(st);
     VA_HIP(hipGetLastError());
@@ -554,6 +667,9 @@ launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     f.p0 = p0;
     f.ids = s->ids_dev;
     f.meta = a.meta;
+    f.meta_sum = p.meta_sum;
+    f.qsum = qsum;
+    f.dim = s->dim;
     f.qmeta = a.qmeta;
     f.qmeta_stride = a.qmeta_stride;
     f.bound = bound;
@@ -561,10 +677,12 @@ launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     f.rate = a.f1;
     f.lb2 = a.f2;
     const dim3 fgrid(static_cast<uint32_t>(div_up(f.lists, 256)));
-    if (l2) {
-        hipLaunchKernelGGL(ivf_i8_finish_kernel<VSAG_AMD_METRIC_L2>, fgrid, dim3(256), 0, st, f);
+    if (bytes) {
+        hipLaunchKernelGGL((ivf_i8_finish_kernel<VSAG_AMD_KIND_SQ8_UNIFORM, VSAG_AMD_METRIC_L2>), fgrid, dim3(256), 0, st, f);
+    } else if (l2) {
+        hipLaunchKernelGGL((ivf_i8_finish_kernel<VSAG_AMD_KIND_SQ4_UNIFORM, VSAG_AMD_METRIC_L2>), fgrid, dim3(256), 0, st, f);
     } else {
-        hipLaunchKernelGGL(ivf_i8_finish_kernel<VSAG_AMD_METRIC_IP>, fgrid, dim3(256), 0, st, f);
+        hipLaunchKernelGGL((ivf_i8_finish_kernel<VSAG_AMD_KIND_SQ4_UNIFORM, VSAG_AMD_METRIC_IP>), fgrid, dim3(256), 0, st, f);
     }
     VA_HIP(hipGetLastError());
     return 0;

@@ -13,6 +13,11 @@
 
 #include "common.h"
 
+// A metadata word that is no field of the reference code but the sum of its payload bytes, formed when the code is
+// re-tiled (sq8_uniform, l2: the int8 matrix cores take code and query centred by 128, and putting the product right
+// needs the plain sum of the code values next to the sum of their squares the code carries).
+constexpr uint32_t kMetaPayloadSum = 0xFFFFFFFFU;
+
 struct vsag_amd_store {
     int kind = 0;
     int metric = 0;
@@ -25,6 +30,7 @@ struct vsag_amd_store {
     uint32_t dpad = 0;           // dims covered by G granules (per-dim tables are this long)
     uint32_t nmeta = 0;          // 4-byte metadata words per code
     uint32_t meta_offset[4] = {0, 0, 0, 0};  // byte offsets of those words in the reference code
+                                             // (kMetaPayloadSum: no field of the code, see below)
     uint32_t meta_is_u64 = 0;    // bit m set: word m is a u64 in the reference code, kept as float
     bool stored_codes = false;   // appended codes come out of a serialized index: fp32 + cosine rows are unit already
 

@@ -80,6 +80,14 @@ retile_kernel(RetileArgs a) {
     a.tiles[(tile * a.G + j) * kWave + lane] = make_uint4(w[0], w[1], w[2], w[3]);
     if (j == 0) {
         for (uint32_t m = 0; m < a.nmeta; ++m) {
+            if (a.meta_offset[m] == kMetaPayloadSum) {
+                uint32_t sum = 0;
+                for (uint32_t b = 0; b < a.payload_bytes; ++b) {
+                    sum += src[b];
+                }
+                a.meta[m * a.meta_stride + slot] = sum;
+                continue;
+            }
             const uint8_t* p = src + a.meta_offset[m];
             uint32_t word;
             if ((a.meta_is_u64 >> m) & 1) {
@@ -415,6 +423,10 @@ vsag_amd_store_create(const vsag_amd_store_params_t* p, vsag_amd_store_t** out) 
             s->nmeta = 1;
             s->meta_offset[0] = static_cast<uint32_t>(up(p->dim, align));
             s->meta_is_u64 = p->metric == VSAG_AMD_METRIC_L2 ? 1 : 0;
+            if (p->metric == VSAG_AMD_METRIC_L2) {
+                s->nmeta = 2;
+                s->meta_offset[1] = kMetaPayloadSum;
+            }
             break;
         }
         case VSAG_AMD_KIND_RABITQ: {
