@@ -272,6 +272,13 @@ VSAG_AMD_API int vsag_amd_set_scan_contraction(int mode);
 /* Tuning knobs of the scan (query tile T in {1,2,4,8}, 0 = automatic; number of base chunks, 0 =
  * automatic).  Process-wide; meant for benchmarks. */
 VSAG_AMD_API int vsag_amd_set_scan_tuning(int query_tile, int base_chunks);
+
+/* The same two settings for one store; they go before the process-wide ones, so that callers with different needs can
+ * share a process (and searches on other stores are not disturbed by a change).  mode -2 / query_tile -1 /
+ * base_chunks -1 = follow the process-wide setting (the default).  Set them while no search runs on the store.  No
+ * counterpart in the reference. */
+VSAG_AMD_API int vsag_amd_store_set_scan_contraction(vsag_amd_store_t* store, int mode);
+VSAG_AMD_API int vsag_amd_store_set_scan_tuning(vsag_amd_store_t* store, int query_tile, int base_chunks);
 /* What the last flat scan on this thread used: query tile (128 / 256: the batch went through the fp32 / int8
  * matrix cores), passes over the code array, bytes of codes one pass reads.  After a posting-list scan: query tile
  * only (256: the columns behind the first went through the int8 matrix cores). */

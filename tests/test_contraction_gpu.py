@@ -227,3 +227,47 @@ def test_sq4_uniform_contraction_equals_streaming(lib, modes, metric, n, d, nq, 
     assert tile == 256, "the int8 route did not run"
     assert same(plain, fast)
     st.destroy()
+
+
+def test_settings_of_one_store_leave_the_others_alone(lib):
+    """vsag_amd_store_set_scan_contraction / _set_scan_tuning: a store's own settings go before the process-wide ones
+    and do not touch searches on another store."""
+    L = capi.load_library()
+    n, d, nq, k = 70000, 64, 600, 10
+    rng = np.random.default_rng(21)
+    x, means = gaussian_mixture(rng, n, d, 30, 0.05)
+    q, _ = gaussian_mixture(rng, nq, d, 30, 0.05, means=means)
+    lb, diff = orc.sq_train(x, 8, orc.L2)
+    codes = orc.sq_encode(x, 8, lb, diff, orc.L2)
+    a = Store(capi.KIND_SQ8, orc.L2, d, lb=lb, diff=diff)
+    b = Store(capi.KIND_SQ8, orc.L2, d, lb=lb, diff=diff)
+    a.append(codes)
+    b.append(codes)
+    tile = capi.C.c_int()
+
+    def last_tile():
+        L.vsag_amd_last_scan_info(capi.C.byref(tile), None, None)
+        return tile.value
+    capi.check(L.vsag_amd_store_set_scan_contraction(a.handle, -1))
+    ws_a, ws_b = (int(L.vsag_amd_flat_scan_workspace_bytes(s.handle, nq, k)) for s in (a, b))
+    assert ws_a < ws_b, "the streaming scan needs no candidate buffers"
+    ra = a.flat_scan(q, k)
+    assert last_tile() == 4, "store a was told to stream"
+    rb = b.flat_scan(q, k)
+    assert last_tile() == 256, "store b follows the process-wide default"
+    assert same(ra, rb)
+    capi.check(L.vsag_amd_store_set_scan_tuning(a.handle, 2, -1))
+    ra2 = a.flat_scan(q, k)
+    assert last_tile() == 2
+    assert same(ra, ra2)
+    b.flat_scan(q[:8], k)
+    assert last_tile() == 4, "store b keeps the default tile"
+    # back to the process-wide settings; a bad mode is refused
+    capi.check(L.vsag_amd_store_set_scan_contraction(a.handle, -2))
+    capi.check(L.vsag_amd_store_set_scan_tuning(a.handle, -1, -1))
+    a.flat_scan(q, k)
+    assert last_tile() == 256
+    assert L.vsag_amd_store_set_scan_contraction(a.handle, 3) == capi.INVALID_ARGUMENT
+    assert L.vsag_amd_store_set_scan_tuning(a.handle, 3, 0) == capi.INVALID_ARGUMENT
+    a.destroy()
+    b.destroy()

@@ -85,6 +85,8 @@ PROTOTYPES = {
     "vsag_amd_flat_scan_topk_noalloc": (C.c_int, [_vp, _vp, _u64, _u32, _vp, _vp, _vp, _vp]),
     "vsag_amd_set_scan_tuning": (C.c_int, [_i32, _i32]),
     "vsag_amd_set_scan_contraction": (C.c_int, [_i32]),
+    "vsag_amd_store_set_scan_contraction": (C.c_int, [_vp, _i32]),
+    "vsag_amd_store_set_scan_tuning": (C.c_int, [_vp, _i32, _i32]),
     "vsag_amd_last_scan_info": (C.c_int, [C.POINTER(C.c_int), C.POINTER(_u64), C.POINTER(_u64)]),
     "vsag_amd_set_kernel_timing": (C.c_int, [_i32]),
     "vsag_amd_last_kernel_ms": (C.c_int, [C.POINTER(_f32)]),

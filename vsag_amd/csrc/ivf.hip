@@ -35,7 +35,7 @@ struct ScanPlanIvf {
 };
 
 uint64_t rabitq_query_code_size(uint32_t dim, int metric, int query_bits);
-int scan_contraction_mode();
+int scan_contraction_mode(const vsag_amd_store* s);
 void note_last_scan(int query_tile, uint64_t passes, uint64_t bytes_per_pass);
 bool ivf_i8_supports(const vsag_amd_store* s);
 uint32_t ivf_i8_lists_per_pair();
@@ -833,7 +833,7 @@ plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, 
     p->seeded = p->chunked && kcand <= 256;
     // Large batches on sq4_uniform (and sq8_uniform / l2) lists: the streaming kernel scans the nearest list of every query, the int8
     // matrix cores the other columns, into two private lists per (query, list) pair.
-    p->mfma = !p->chunked && nprobe > 1 && scan_contraction_mode() >= 0 && ivf_i8_supports(s) &&
+    p->mfma = !p->chunked && nprobe > 1 && scan_contraction_mode(s) >= 0 && ivf_i8_supports(s) &&
               s->residual_centroids_dev == nullptr &&
               npairs * ivf_i8_lists_per_pair() * kcand * 8 <= (8ull << 30);
     if (p->mfma) {

@@ -610,6 +610,9 @@ launch_merge_partials(const uint64_t* partial, const uint32_t* partial_cnt, cons
 
 static int g_tile_override = 0;
 static int g_chunk_override = 0;
+// A store's own setting (vsag_amd_store_set_scan_tuning) goes before the process-wide one.
+static int tile_override(const vsag_amd_store* s) { return s->tile_override >= 0 ? s->tile_override : g_tile_override; }
+static int chunk_override(const vsag_amd_store* s) { return s->chunk_override >= 0 ? s->chunk_override : g_chunk_override; }
 static thread_local int tl_last_tile = 0;
 static thread_local uint64_t tl_last_passes = 0;
 static thread_local uint64_t tl_last_bytes = 0;
@@ -646,8 +649,8 @@ struct ScanPlan {
 static void
 make_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, uint64_t ntiles, ScanPlan* p) {
     p->S = selector_slots(k);
-    int T = g_tile_override > 0 ? g_tile_override : default_query_tile(s);
-    if (g_tile_override <= 0 && s->kind == VSAG_AMD_KIND_FP32 && ntiles >= 1024) {
+    int T = tile_override(s) > 0 ? tile_override(s) : default_query_tile(s);
+    if (tile_override(s) <= 0 && s->kind == VSAG_AMD_KIND_FP32 && ntiles >= 1024) {
         // 512 bytes per code and pass: on a long scan the passes are what costs (100k x 128: a quarter faster than 4);
         // short scans (centroid routing, the exact prefix of a pre-selected batch) live on their selectors instead.
         T = 8;
@@ -669,8 +672,8 @@ make_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, uint64_t ntiles, Sca
     p->groups = div_up(nq, static_cast<uint64_t>(T));
     p->nq_pad = p->groups * T;
     uint64_t chunks;
-    if (g_chunk_override > 0) {
-        chunks = g_chunk_override;
+    if (chunk_override(s) > 0) {
+        chunks = chunk_override(s);
     } else {
         // Workgroups in the grid: about 64 per query group, but at least two per compute unit (few queries:
         // every wave still has a long run of tiles behind its cold start) and at most eight rounds of
@@ -735,6 +738,8 @@ struct CallPlan {
 
 // -1 never, 0 when it pays, 1 whenever the store supports it, 2 like 1 but on the fp32 matrix cores only
 static int g_prefilter_mode = 0;
+// A store's own setting (vsag_amd_store_set_scan_contraction) goes before the process-wide one.
+static int prefilter_mode(const vsag_amd_store* s) { return s->contraction_mode >= -1 ? s->contraction_mode : g_prefilter_mode; }
 
 bool prefilter_supports(const vsag_amd_store* s);
 int launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t k, uint32_t S, uint64_t tile_begin,
@@ -755,10 +760,10 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
     c->nslots = static_cast<uint32_t>(c->all.chunks * c->all.waves);
     c->any_seeded = c->all.seeded;
     c->contraction = false;
-    if (g_prefilter_mode < 0 || !prefilter_supports(s)) {
+    if (prefilter_mode(s) < 0 || !prefilter_supports(s)) {
         return;
     }
-    const bool forced = g_prefilter_mode > 0;
+    const bool forced = prefilter_mode(s) > 0;
     const bool rb = prefilter_rb_supports(s);
     if (!forced && (nq < 512 || k > (rb ? 256U : 128U) || s->ntiles < 1024)) {
         return;
@@ -814,7 +819,7 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
     }
     c->contraction = true;
     // Mode 2 asks for the fp32 matrix cores, which the uniform kinds have no route for.
-    c->int8 = prefilter_i8_supports(s) && (g_prefilter_mode != 2 || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM ||
+    c->int8 = prefilter_i8_supports(s) && (prefilter_mode(s) != 2 || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM ||
                                            s->kind == VSAG_AMD_KIND_SQ4_UNIFORM);
     c->rb = rb;
     c->rb_scratch = rb ? prefilter_rb_scratch_bytes(s, nq) : 0;
@@ -1190,8 +1195,8 @@ vsag_amd_flat_scan_topk_noalloc(const vsag_amd_store_t* s, const float* queries_
 
 namespace vsag_amd {
 int
-scan_contraction_mode() {
-    return g_prefilter_mode;
+scan_contraction_mode(const vsag_amd_store* s) {
+    return prefilter_mode(s);
 }
 
 // What vsag_amd_last_scan_info reports, for the posting-list scan.
@@ -1208,6 +1213,26 @@ vsag_amd_set_scan_contraction(int mode) {
     VA_CHECK_ARG(mode >= -1 && mode <= 2,
                  "mode must be -1 (never), 0 (when it pays), 1 (whenever supported) or 2 (1 on the fp32 matrix cores)");
     g_prefilter_mode = mode;
+    return 0;
+}
+
+extern "C" int
+vsag_amd_store_set_scan_contraction(vsag_amd_store_t* s, int mode) {
+    VA_CHECK_ARG(s != nullptr, "store is null");
+    VA_CHECK_ARG(mode >= -2 && mode <= 2, "mode must be -2 (follow the process-wide setting), -1, 0, 1 or 2");
+    s->contraction_mode = mode;
+    return 0;
+}
+
+extern "C" int
+vsag_amd_store_set_scan_tuning(vsag_amd_store_t* s, int query_tile, int base_chunks) {
+    VA_CHECK_ARG(s != nullptr, "store is null");
+    VA_CHECK_ARG(query_tile == -1 || query_tile == 0 || query_tile == 1 || query_tile == 2 || query_tile == 4 ||
+                     query_tile == 8,
+                 "query_tile must be -1 (follow the process-wide setting), 0, 1, 2, 4 or 8");
+    VA_CHECK_ARG(base_chunks >= -1 && base_chunks <= 65535, "base_chunks must be in [-1, 65535]");
+    s->tile_override = query_tile;
+    s->chunk_override = base_chunks;
     return 0;
 }
 

@@ -28,6 +28,12 @@ struct vsag_amd_store {
     uint32_t payload_bytes = 0;  // leading bytes consumed by the distance loop
     uint32_t G = 0;              // 16-byte granules per code
     uint32_t dpad = 0;           // dims covered by G granules (per-dim tables are this long)
+    // Scan settings of this store; the values below follow the process-wide ones (vsag_amd_set_scan_contraction /
+    // vsag_amd_set_scan_tuning).
+    int contraction_mode = -2;
+    int tile_override = -1;
+    int chunk_override = -1;
+
     uint32_t nmeta = 0;          // 4-byte metadata words per code
     uint32_t meta_offset[4] = {0, 0, 0, 0};  // byte offsets of those words in the reference code
                                              // (kMetaPayloadSum: no field of the code, see below)
