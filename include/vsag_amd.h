@@ -313,6 +313,17 @@ VSAG_AMD_API int vsag_amd_kmeans_run(const float* x_dev, uint64_t n, uint32_t di
                         int iters, uint64_t seed, int32_t* labels_dev, double* loss,
                         void* workspace_dev, size_t workspace_bytes, void* stream);
 
+/* KMeansCluster::select_initial_centroids_kmeans_plus_plus (kmeans_cluster.cpp:383-435), the reference's default
+ * initialisation, with its random draws as inputs (the reference takes them from an mt19937 seeded by
+ * std::random_device): `first` = the row that becomes centroid 0; draws (HOST array, k - 1 doubles in [0, 1)): centroid
+ * j is the first row at which the running sum of the rows' smallest squared distances to the centroids so far reaches
+ * draws[j - 1] * their total (any row, floor(draw * n), when the total is 0).  picks_dev (k words, may be NULL) receives
+ * the chosen rows. */
+VSAG_AMD_API size_t vsag_amd_kmeans_init_plus_plus_workspace_bytes(uint64_t n);
+VSAG_AMD_API int vsag_amd_kmeans_init_plus_plus(const float* x_dev, uint64_t n, uint32_t dim, uint32_t k, uint64_t first,
+                                   const double* draws, float* centroids_dev, uint64_t* picks_dev,
+                                   void* workspace_dev, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------ IVF ---------------------- */
 
 /* Routing (IVFNearestPartition::ClassifyDatasForSearch, ivf_nearest_partition.cpp:99-147, done exactly

@@ -18,7 +18,9 @@
 //                                          composition (nprobe=nlist), rabitq_dist (a stored vector as
 //                                          32-bit query: estimate exactly 0 / 1 - |x|^2; the +-1 clamp of
 //                                          a tiny error field; zero raw norms -> 1; the 4-bit branch
-//                                          against the fp32 branch on the dequantised query)
+//                                          against the fp32 branch on the dequantised query),
+//                                          kmeans_init_pp (numpy restatement with cumsum / searchsorted in
+//                                          float64; k = n picks every row once; coincident rows)
 //   parity unpinned ...................... nothing; what the formulas leave open is the order of fp32
 //                                          operations inside rabitq_dist and the k-means loss (no
 //                                          executable reference class), which the 1e-4 relative
@@ -1099,6 +1101,46 @@ orc_kmeans_update(const float* x, const int32_t* labels, uint64_t n, uint64_t di
                 cent[j * dim + d] = sums[j * dim + d] * inv;
             }
         }
+    }
+}
+
+// KMeansCluster::select_initial_centroids_kmeans_plus_plus (kmeans_cluster.cpp:383-435) with the random draws as
+// inputs: `first` is what first_dis(gen) returned, draws[c - 1] in [0, 1) stands for the c-th prob_dis(gen) /
+// total_weight (uniform_real_distribution<double>(0, w)(gen) = w * generate_canonical) or, when the total weight is 0,
+// for dis(gen) / count.
+ORC_API void
+orc_kmeans_init_pp(const float* x, uint64_t n, uint64_t dim, uint64_t k, uint64_t first, const double* draws, float* cent,
+                   uint64_t* picks) {
+    std::memcpy(cent, x + first * dim, dim * sizeof(float));
+    picks[0] = first;
+    std::vector<float> min_distances(n, std::numeric_limits<float>::max());
+    for (uint64_t c = 1; c < k; ++c) {
+        const float* centroid = cent + (c - 1) * dim;
+        for (uint64_t i = 0; i < n; ++i) {
+            float dist = fp32_l2sqr(x + i * dim, centroid, dim);
+            min_distances[i] = std::min(min_distances[i], dist);
+        }
+        double total_weight = 0.0;
+        for (uint64_t i = 0; i < n; ++i) {
+            total_weight += min_distances[i];
+        }
+        uint64_t selected = n - 1;
+        if (total_weight <= 0.0) {
+            double f = draws[c - 1] * static_cast<double>(n);
+            selected = f >= static_cast<double>(n - 1) ? n - 1 : static_cast<uint64_t>(f);
+        } else {
+            double threshold = draws[c - 1] * total_weight;
+            double cumulative = 0.0;
+            for (uint64_t i = 0; i < n; ++i) {
+                cumulative += min_distances[i];
+                if (cumulative >= threshold) {
+                    selected = i;
+                    break;
+                }
+            }
+        }
+        picks[c] = selected;
+        std::memcpy(cent + c * dim, x + selected * dim, dim * sizeof(float));
     }
 }
 

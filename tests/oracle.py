@@ -199,6 +199,18 @@ def kmeans_update(x, labels, cent):
     return cent, counts
 
 
+def kmeans_init_pp(x, k, first, draws):
+    """k-means++ seeding with the random draws given: (centroids, picked rows)."""
+    x = f32(x)
+    n, d = x.shape
+    draws = np.ascontiguousarray(draws, np.float64)
+    assert draws.shape[0] >= k - 1
+    cent = np.empty((k, d), np.float32)
+    picks = np.empty(k, np.uint64)
+    lib().orc_kmeans_init_pp(_p(x), u64(n), u64(d), u64(k), u64(first), _p(draws), _p(cent), _p(picks))
+    return cent, picks
+
+
 def kmeans_run(x, cent0, iters, seed):
     x = f32(x)
     cent = f32(cent0).copy()

@@ -111,3 +111,46 @@ def test_kmeans_argument_errors(lib):
     assert rc == capi.INVALID_ARGUMENT and b"k cannot be larger than count" in L.vsag_amd_last_error()
     rc = L.vsag_amd_kmeans_assign(x.ptr, 4, 4, x.ptr, 0, x.ptr, None, None, None, 0, None)
     assert rc == capi.INVALID_ARGUMENT and b"k must be positive" in L.vsag_amd_last_error()
+
+
+def gpu_init_pp(x, k, first, draws):
+    L = capi.load_library()
+    n, d = x.shape
+    xb = dev(x)
+    cent, picks = capi.DeviceBuffer(k * d * 4), capi.DeviceBuffer(k * 8)
+    wsb = L.vsag_amd_kmeans_init_plus_plus_workspace_bytes(n)
+    ws = capi.DeviceBuffer(wsb)
+    draws = np.ascontiguousarray(draws, np.float64)
+    capi.check(L.vsag_amd_kmeans_init_plus_plus(xb.ptr, n, d, k, first, draws.ctypes.data, cent.ptr, picks.ptr, ws.ptr,
+                                                wsb, None))
+    capi.synchronize()
+    out = cent.to_numpy(np.float32, (k, d)), picks.to_numpy(np.uint64, (k,))
+    for b in (xb, cent, picks, ws):
+        b.free()
+    return out
+
+
+@pytest.mark.parametrize("n,d,k", [(5000, 128, 64), (777, 7, 100), (20000, 65, 33), (64, 960, 64), (130, 16, 130)])
+def test_plus_plus_seeding_matches_oracle(lib, n, d, k):
+    """k-means++ seeding (kmeans_cluster.cpp:383-435) with the same draws as the checker: the same rows, except where a
+    threshold falls within the rounding of the (differently associated) double sums of a boundary."""
+    rng = np.random.default_rng(n + d + k)
+    x, _ = gaussian_mixture(rng, n, d, max(2, k // 4), 0.2, uniform_means=False)
+    draws = rng.random(k - 1)
+    first = int(rng.integers(n))
+    cent, picks = gpu_init_pp(x, k, first, draws)
+    rcent, rpicks = orc.kmeans_init_pp(x, k, first, draws)
+    assert np.array_equal(picks, rpicks), np.nonzero(picks != rpicks)[0][:5]
+    assert np.array_equal(cent, rcent)
+    assert len(set(picks.tolist())) == k
+
+
+def test_plus_plus_seeding_on_coincident_rows(lib):
+    rng = np.random.default_rng(4)
+    y = np.repeat(rng.standard_normal((3, 20)).astype(np.float32), 50, axis=0)
+    draws = np.array([0.5, 0.99, 0.0, 0.5, 0.999])
+    cent, picks = gpu_init_pp(y, 6, 0, draws)
+    _, rpicks = orc.kmeans_init_pp(y, 6, 0, draws)
+    assert np.array_equal(picks, rpicks) and list(picks[3:]) == [0, 75, 149]
+    L = capi.load_library()
+    assert L.vsag_amd_kmeans_init_plus_plus(1, 10, 4, 3, 10, draws.ctypes.data, 1, None, None, 0, None) == capi.INVALID_ARGUMENT

@@ -506,6 +506,36 @@ def test_kmeans_assign_is_the_exact_argmin():
             assert np.array_equal(newc[j], cent[j])
 
 
+def test_kmeans_plus_plus_seeding_follows_the_squared_distance_law():
+    """select_initial_centroids_kmeans_plus_plus (kmeans_cluster.cpp:383-435) with the draws given, against an
+    independent restatement: smallest squared distances in float64 from the definition, cumulative sums and the first
+    index that reaches the threshold by searchsorted.  Draws that land within rounding of a boundary are left out."""
+    rng = np.random.default_rng(12)
+    n, d, k = 500, 9, 40
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    draws = rng.random(k - 1)
+    cent, picks = orc.kmeans_init_pp(x, k, 17, draws)
+    assert picks[0] == 17 and np.array_equal(cent, x[picks.astype(np.int64)])
+    x64 = x.astype(np.float64)
+    chosen = [17]
+    for c in range(1, k):
+        d2 = ((x64[:, None, :] - x64[chosen][None]) ** 2).sum(2).min(1)
+        cum = np.cumsum(d2)
+        thr = draws[c - 1] * cum[-1]
+        i = int(np.searchsorted(cum, thr, side="left"))
+        near = np.abs(cum[max(i - 1, 0):i + 1] - thr).min() < 1e-5 * cum[-1]  # fp32 distances vs float64 ones
+        assert near or picks[c] == i, (c, picks[c], i)
+        chosen.append(int(picks[c]))
+    assert len(set(chosen)) == k, "a chosen row has distance 0 and cannot be drawn again"
+    # k = n: every row is picked exactly once, whatever the draws
+    _, all_picks = orc.kmeans_init_pp(x[:60], 60, 3, rng.random(59))
+    assert sorted(all_picks.tolist()) == list(range(60))
+    # coincident rows: once every distinct point is a centroid the total weight is 0 and the draw picks any row
+    y = np.repeat(rng.standard_normal((3, d)).astype(np.float32), 5, axis=0)
+    _, p = orc.kmeans_init_pp(y, 6, 0, np.array([0.5, 0.99, 0.0, 0.5, 0.999]))
+    assert len({int(v) // 5 for v in p[:3]}) == 3 and list(p[3:]) == [0, 7, 14]
+
+
 def test_heaps_equal_sorting():
     rng = np.random.default_rng(8)
     n, d, k = 700, 10, 13

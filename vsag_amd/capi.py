@@ -94,6 +94,8 @@ PROTOTYPES = {
     "vsag_amd_kmeans_assign": (C.c_int, [_vp, _u64, _u32, _vp, _u32, _vp, _vp, _vp, _vp, _sz, _vp]),
     "vsag_amd_kmeans_update_workspace_bytes": (_sz, [_u64, _u32, _u32]),
     "vsag_amd_kmeans_update": (C.c_int, [_vp, _vp, _u64, _u32, _u32, _vp, _vp, _vp, _sz, _vp]),
+    "vsag_amd_kmeans_init_plus_plus_workspace_bytes": (_sz, [_u64]),
+    "vsag_amd_kmeans_init_plus_plus": (C.c_int, [_vp, _u64, _u32, _u32, _u64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "vsag_amd_kmeans_run_workspace_bytes": (_sz, [_u64, _u32, _u32]),
     "vsag_amd_kmeans_run": (C.c_int, [_vp, _u64, _u32, _vp, _u32, _i32, _u64, _vp, C.POINTER(C.c_double), _vp, _sz,
                                       _vp]),

@@ -796,9 +796,233 @@ check_kmeans(const void* x, uint64_t n, uint32_t dim, const void* cent, uint32_t
     return 0;
 }
 
+// ---- k-means++ seeding (KMeansCluster::select_initial_centroids_kmeans_plus_plus, kmeans_cluster.cpp:383-435) -------
+// One step = two launches: the distance of every row to the centroid chosen last lowers the row's smallest distance
+// so far, and a row is drawn with a probability proportional to that distance -- the first row at which the running
+// sum of the distances (a double, in row order) reaches the step's threshold draw * total.  The reference sums
+// sequentially; here a block of 64 rows is summed in row order, blocks in chunks in block order, chunks in chunk
+// order, chunks in runs: the same sums apart from the association of the double additions.
+constexpr uint32_t kPpRows = 64;      // rows per workgroup of the distance launch (one wave, a lane per row)
+constexpr uint32_t kPpChunks = 1024;  // threads of the picking workgroup: each sums a run of block sums
+
+__global__ void __launch_bounds__(64)
+kpp_distance_kernel(const float* x, uint64_t n, uint32_t dim, const float* centroid, float* min_dist, double* block_sum,
+                    int first_step) {
+    __shared__ float rows[kPpRows][kPpRows + 1];
+    __shared__ float cent[kPpRows];
+    __shared__ float md[kPpRows];
+    const uint32_t lane = threadIdx.x;
+    const uint64_t row0 = static_cast<uint64_t>(blockIdx.x) * kPpRows;
+    // FP32ComputeL2Sqr in element order (simd/generic.cpp): result += (a - b) * (a - b), one row per lane.
+    float result = 0.0F;
+    for (uint32_t c0 = 0; c0 < dim; c0 += kPpRows) {
+        const uint32_t d = c0 + lane;
+        cent[lane] = d < dim ? centroid[d] : 0.0F;
+        // All 64 loads of the chunk are issued before the first is used (no branch around a load: addresses are
+        // clamped, what lies beyond the data is never used).
+        const uint32_t dc = d < dim ? d : dim - 1;
+        float v[kPpRows];
+#pragma unroll
+        for (uint32_t r = 0; r < kPpRows; ++r) {
+            const uint64_t row = row0 + r < n ? row0 + r : n - 1;
+            v[r] = x[row * dim + dc];
+        }
+#pragma unroll
+        for (uint32_t r = 0; r < kPpRows; ++r) {
+            rows[r][lane] = v[r];
+        }
+        __syncthreads();
+        const uint32_t width = dim - c0 < kPpRows ? dim - c0 : kPpRows;
+        for (uint32_t j = 0; j < width; ++j) {
+            const float diff = rows[lane][j] - cent[j];
+            result += diff * diff;
+        }
+        __syncthreads();
+    }
+    const uint64_t row = row0 + lane;
+    float m = 0.0F;
+    if (row < n) {
+        const float old = first_step ? 3.402823466e38F : min_dist[row];
+        m = result < old ? result : old;  // std::min(min_distances[i], dist)
+        min_dist[row] = m;
+    }
+    md[lane] = m;
+    __syncthreads();
+    if (lane == 0) {
+        double sum = 0.0;
+        for (uint32_t r = 0; r < kPpRows; ++r) {
+            sum += static_cast<double>(md[r]);
+        }
+        block_sum[blockIdx.x] = sum;
+    }
+}
+
+// One workgroup.  The walk along the running sum goes down four levels -- 32 runs of 32 chunks, the chunks of a run,
+// the block sums of a chunk, the 64 rows of a block -- and one thread does each walk over values the others have
+// brought into LDS, so that no step of a walk waits for global memory.
+__global__ void __launch_bounds__(kPpChunks)
+kpp_pick_kernel(const float* x, uint64_t n, uint32_t dim, const float* min_dist, const double* block_sum,
+                uint64_t nblocks, double draw, float* centroid_out, uint64_t* pick_out) {
+    constexpr uint32_t kRuns = 32, kPerRun = kPpChunks / kRuns;
+    __shared__ double chunk_sum[kPpChunks];
+    __shared__ double run_sum[kRuns];
+    __shared__ double staged[kPpChunks];
+    __shared__ double cumulative_s, threshold_s;
+    __shared__ uint64_t at_s;  // the chunk, then the block, then the row the walk has reached
+    __shared__ int done_s;
+    const uint32_t t = threadIdx.x;
+    const uint64_t per = (nblocks + kPpChunks - 1) / kPpChunks;
+    const uint64_t b0 = t * per, b1 = b0 + per < nblocks ? b0 + per : nblocks;
+    double mine = 0.0;
+    for (uint64_t b = b0; b < b1; ++b) {
+        mine += block_sum[b];
+    }
+    chunk_sum[t] = mine;
+    __syncthreads();
+    if (t < kRuns) {
+        double r = 0.0;
+        for (uint32_t c = 0; c < kPerRun; ++c) {
+            r += chunk_sum[t * kPerRun + c];
+        }
+        run_sum[t] = r;
+    }
+    __syncthreads();
+    if (t == 0) {
+        double total = 0.0;
+        for (uint32_t r = 0; r < kRuns; ++r) {
+            total += run_sum[r];
+        }
+        done_s = 0;
+        if (!(total > 0.0)) {
+            // Every row coincides with a centroid: any row (uniform_int_distribution in the reference).
+            const double f = draw * static_cast<double>(n);
+            at_s = f >= static_cast<double>(n - 1) ? n - 1 : static_cast<uint64_t>(f);
+            done_s = 1;
+        } else {
+            const double threshold = draw * total;
+            double cumulative = 0.0;
+            uint32_t r = 0;
+            while (r + 1 < kRuns && !(cumulative + run_sum[r] >= threshold)) {
+                cumulative += run_sum[r];
+                ++r;
+            }
+            uint32_t c = r * kPerRun;
+            while (c + 1 < (r + 1) * kPerRun && !(cumulative + chunk_sum[c] >= threshold)) {
+                cumulative += chunk_sum[c];
+                ++c;
+            }
+            cumulative_s = cumulative;
+            threshold_s = threshold;
+            at_s = c;
+        }
+    }
+    __syncthreads();
+    if (done_s == 0) {
+        // The block sums of the chunk, kPpChunks at a time.
+        const uint64_t first = at_s * per;
+        const uint64_t last = first + per < nblocks ? first + per : nblocks;  // may be <= first: a chunk without blocks
+        __syncthreads();
+        if (t == 0) {
+            at_s = last > first ? last - 1 : (nblocks - 1);
+        }
+        for (uint64_t base = first; base < last; base += kPpChunks) {
+            if (base + t < last) {
+                staged[t] = block_sum[base + t];
+            }
+            __syncthreads();
+            if (t == 0 && done_s == 0) {
+                const uint64_t m = last - base < kPpChunks ? last - base : kPpChunks;
+                double cumulative = cumulative_s;
+                for (uint64_t i = 0; i < m; ++i) {
+                    if (base + i + 1 == last || cumulative + staged[i] >= threshold_s) {
+                        at_s = base + i;
+                        done_s = 2;
+                        break;
+                    }
+                    cumulative += staged[i];
+                }
+                cumulative_s = cumulative;
+            }
+            __syncthreads();
+            if (done_s != 0) {
+                break;
+            }
+        }
+        __syncthreads();
+        const uint64_t blk = at_s;
+        const uint64_t r0 = blk * kPpRows, r1 = r0 + kPpRows < n ? r0 + kPpRows : n;
+        if (t < kPpRows) {
+            staged[t] = r0 + t < r1 ? static_cast<double>(min_dist[r0 + t]) : 0.0;
+        }
+        __syncthreads();
+        if (t == 0) {
+            uint64_t idx = r1 - 1;
+            double cumulative = cumulative_s;
+            for (uint64_t r = r0; r < r1; ++r) {
+                cumulative += staged[r - r0];
+                if (cumulative >= threshold_s) {
+                    idx = r;
+                    break;
+                }
+            }
+            at_s = idx;
+        }
+        __syncthreads();
+    }
+    const uint64_t idx = at_s;
+    if (t == 0 && pick_out != nullptr) {
+        *pick_out = idx;
+    }
+    for (uint32_t d = t; d < dim; d += kPpChunks) {
+        centroid_out[d] = x[idx * dim + d];
+    }
+}
+
 }  // namespace vsag_amd
 
 using namespace vsag_amd;
+
+extern "C" size_t
+vsag_amd_kmeans_init_plus_plus_workspace_bytes(uint64_t n) {
+    Carver c(nullptr, 0);
+    c.take<float>(n);
+    c.take<double>(div_up(n, static_cast<uint64_t>(kPpRows)));
+    return c.used + 256;
+}
+
+extern "C" int
+vsag_amd_kmeans_init_plus_plus(const float* x_dev, uint64_t n, uint32_t dim, uint32_t k, uint64_t first,
+                               const double* draws, float* centroids_dev, uint64_t* picks_dev, void* workspace_dev,
+                               size_t workspace_bytes, void* stream) {
+    VA_TRY(ensure_init());
+    VA_TRY(check_kmeans(x_dev, n, dim, centroids_dev, k));
+    VA_CHECK_ARG(k <= n, "k cannot be larger than count");
+    VA_CHECK_ARG(first < n, "the first centroid must be a row of the data");
+    VA_CHECK_ARG(k == 1 || draws != nullptr, "draws is null");
+    for (uint32_t c = 1; c < k; ++c) {
+        VA_CHECK_ARG(draws[c - 1] >= 0.0 && draws[c - 1] < 1.0, "draws must lie in [0, 1)");
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    Carver c(workspace_dev, workspace_bytes);
+    float* min_dist = c.take<float>(n);
+    const uint64_t nblocks = div_up(n, static_cast<uint64_t>(kPpRows));
+    double* block_sum = c.take<double>(nblocks);
+    VA_CHECK_ARG(c.ok(), "workspace too small: need %zu bytes, got %zu", c.used, workspace_bytes);
+    VA_HIP(hipMemcpyAsync(centroids_dev, x_dev + first * dim, dim * sizeof(float), hipMemcpyDeviceToDevice, st));
+    if (picks_dev != nullptr) {
+        VA_HIP(hipMemcpyAsync(picks_dev, &first, sizeof(uint64_t), hipMemcpyHostToDevice, st));
+        VA_HIP(hipStreamSynchronize(st));  // `first` lives on this frame
+    }
+    for (uint32_t j = 1; j < k; ++j) {
+        hipLaunchKernelGGL(kpp_distance_kernel, dim3(static_cast<uint32_t>(nblocks)), dim3(kPpRows), 0, st, x_dev, n, dim,
+                           centroids_dev + static_cast<uint64_t>(j - 1) * dim, min_dist, block_sum, j == 1 ? 1 : 0);
+        hipLaunchKernelGGL(kpp_pick_kernel, dim3(1), dim3(kPpChunks), 0, st, x_dev, n, dim, min_dist, block_sum, nblocks,
+                           draws[j - 1], centroids_dev + static_cast<uint64_t>(j) * dim,
+                           picks_dev != nullptr ? picks_dev + j : nullptr);
+    }
+    VA_HIP(hipGetLastError());
+    return 0;
+}
 
 extern "C" size_t
 vsag_amd_kmeans_assign_workspace_bytes(uint64_t n, uint32_t dim, uint32_t k) {

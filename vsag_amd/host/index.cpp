@@ -2478,12 +2478,29 @@ private:
         DevBuf sample_dev;
         sample_dev.reserve(sample.size() * 4);
         dev(vsag_amd_memcpy_h2d(sample_dev.p, sample.data(), sample.size() * 4, nullptr));
-        // Initial centroids: the first nlist rows of the shuffled sample (random-sample initialisation;
-        // the reference defaults to k-means++ drawn from std::random_device).
+        // "random": the centroids are nlist rows of the shuffled sample.  "kmeans": k-means++ seeding, the default
+        // of KMeansCluster::Run (kmeans_cluster.cpp:78-82, 383-435), with draws from the seeded generator where the
+        // reference seeds an mt19937 from std::random_device; then the Lloyd iterations.
         DevBuf centroids;
         centroids.reserve(static_cast<size_t>(nlist_) * q_.dim * 4);
         dev(vsag_amd_memcpy_d2d(centroids.p, sample_dev.p, static_cast<size_t>(nlist_) * q_.dim * 4, nullptr));
         if (!train_random_) {
+            {
+                std::uniform_int_distribution<uint64_t> first_dis(0, sample_n - 1);
+                const uint64_t first = first_dis(gen);
+                std::uniform_real_distribution<double> unit(0.0, 1.0);
+                std::vector<double> draws(nlist_ > 1 ? nlist_ - 1 : 0);
+                for (double& d : draws) {
+                    d = unit(gen);
+                    d = d < 1.0 ? d : 0.0;
+                }
+                DevBuf ws;
+                size_t wsb = vsag_amd_kmeans_init_plus_plus_workspace_bytes(sample_n);
+                ws.reserve(wsb);
+                dev(vsag_amd_kmeans_init_plus_plus(sample_dev.as<float>(), sample_n, q_.dim, nlist_, first, draws.data(),
+                                                   centroids.as<float>(), nullptr, ws.p, wsb, nullptr));
+                dev(vsag_amd_stream_synchronize(nullptr));
+            }
             DevBuf labels, ws;
             labels.reserve(sample_n * 4);
             size_t wsb = vsag_amd_kmeans_run_workspace_bytes(sample_n, q_.dim, nlist_);
