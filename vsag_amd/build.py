@@ -72,9 +72,25 @@ def build_host(verbose=True):
     return lib
 
 
+def build_host_example(verbose=True):
+    """tests/cpp/host_api.cpp: a C++ program against vsag_host.h, run by the tests (it must be built before them)."""
+    src = os.path.join(ROOT, "..", "tests", "cpp", "host_api.cpp")
+    if not os.path.exists(src):
+        return None
+    exe = os.path.join(LIB, "host_api_test")
+    out = _run(["g++", "-O2", "-std=c++17", "-Wall", "-I" + HOST, "-o", exe, src, "-L" + LIB, "-lvsag_amd_host",
+                "-lvsag_amd", "-Wl,-rpath,$ORIGIN", "-lpthread"])
+    if verbose:
+        if out:
+            print(out)
+        print("built", exe)
+    return exe
+
+
 def build_all(verbose=True):
     build_kernels(verbose)
     build_host(verbose)
+    build_host_example(verbose)
 
 
 if __name__ == "__main__":

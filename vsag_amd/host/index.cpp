@@ -1023,8 +1023,39 @@ pack_distances(const std::vector<float>& dists, const std::vector<uint32_t>& inn
 }
 
 // The search overloads of the public interface, reduced to one virtual search().
+// The arrays of a result moved into the caller's allocator (an index created with one hands out only such results).
+DatasetPtr
+rehome(const DatasetPtr& result, Allocator* allocator) {
+    if (allocator == nullptr || result == nullptr) {
+        return result;
+    }
+    const int64_t cells = result->GetNumElements() * result->GetDim();
+    auto moved = Dataset::Make();
+    moved->NumElements(result->GetNumElements())->Dim(result->GetDim())->Statistics(result->GetStatistics());
+    moved->Owner(true, allocator);
+    auto copy = [&](const auto* src) -> decltype(src) {
+        using T = std::remove_const_t<std::remove_pointer_t<decltype(src)>>;
+        if (src == nullptr) {
+            return nullptr;
+        }
+        auto* dst = static_cast<T*>(allocator->Allocate(sizeof(T) * static_cast<uint64_t>(std::max<int64_t>(cells, 1))));
+        if (dst == nullptr) {
+            throw VsagException(ErrorType::NO_ENOUGH_MEMORY, "the allocator returned no memory for a search result");
+        }
+        std::copy(src, src + cells, dst);
+        return dst;
+    };
+    moved->Ids(copy(result->GetIds()));
+    moved->Distances(copy(result->GetDistances()));
+    return moved;
+}
+
 class GpuIndex : public Index {
 public:
+    void
+    set_allocator(Allocator* allocator) {
+        allocator_ = allocator;
+    }
     Expected<DatasetPtr>
     KnnSearch(const DatasetPtr& query, int64_t k, const std::string& parameters) const override {
         return run(query, k, parameters, SearchSpec{});
@@ -1094,7 +1125,7 @@ public:
                 CHECK_ARGUMENT(query != nullptr, "CalDistanceById query must not be null");
                 CHECK_ARGUMENT(ids != nullptr, "CalDistanceById ids must not be null");
             }
-            return distances_by_id(query, 1, ids, count, calculate_precise_distance, topk);
+            return rehome(distances_by_id(query, 1, ids, count, calculate_precise_distance, topk), allocator_);
         });
     }
     Expected<DatasetPtr>
@@ -1110,8 +1141,9 @@ public:
                 CHECK_ARGUMENT(query->GetFloat32Vectors() != nullptr, "query.float_vector is nullptr");
                 CHECK_ARGUMENT(query->GetDim() == static_cast<int64_t>(dimension()), "query.dim must be equal to index.dim");
             }
-            return distances_by_id(query->GetFloat32Vectors(), query->GetNumElements(), ids, count,
-                                   calculate_precise_distance, topk);
+            return rehome(distances_by_id(query->GetFloat32Vectors(), query->GetNumElements(), ids, count,
+                                          calculate_precise_distance, topk),
+                          allocator_);
         });
     }
 
@@ -1151,6 +1183,7 @@ protected:
     // Searches share the lock; Build / Add / Train hold it alone (bruteforce.cpp:373,1386).
     mutable std::shared_mutex mutex_;
     mutable ContextPool pool_;
+    Allocator* allocator_ = nullptr;
 
 private:
     Expected<DatasetPtr>
@@ -1163,7 +1196,7 @@ private:
                                "radius(" + std::to_string(spec.radius) + ") must be greater equal than 0");
                 CHECK_ARGUMENT(spec.limited_size != 0, "limited_size(0) must not be equal to 0");
             }
-            return search(query, k, parameters, spec);
+            return rehome(search(query, k, parameters, spec), allocator_);
         });
     }
     static SearchSpec
@@ -2671,7 +2704,7 @@ private:
 }  // namespace
 
 Expected<std::shared_ptr<Index>>
-Factory::CreateIndex(const std::string& name, const std::string& parameters) {
+Factory::CreateIndex(const std::string& name, const std::string& parameters, Allocator* allocator) {
     return safe_call<std::shared_ptr<Index>>([&]() -> std::shared_ptr<Index> {
         Json params = Json::Parse(parameters);
         CommonParam common = parse_common(params);
@@ -2683,13 +2716,14 @@ Factory::CreateIndex(const std::string& name, const std::string& parameters) {
         }
         // The constructors only validate parameters; the device is touched afterwards, so that parameter
         // errors are reported the same way with or without a GPU.
-        std::shared_ptr<Index> index;
+        std::shared_ptr<GpuIndex> index;
         if (name == "brute_force") {
             index = std::make_shared<BruteForce>(common, index_param);
         } else if (name == "ivf") {
             index = std::make_shared<IVF>(common, index_param);
         }
         if (index != nullptr) {
+            index->set_allocator(allocator);
             static std::once_flag once;
             static int init_rc = 0;
             static std::string init_message;

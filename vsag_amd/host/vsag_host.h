@@ -111,11 +111,28 @@ private:
     Error error_;
 };
 
+// include/vsag/allocator.h:34-96: the caller's memory management.  An index created with an allocator takes the arrays
+// of its results (ids, distances) from it; the dataset that owns them gives them back to it.  Device memory is not the
+// allocator's business.
+class Allocator {
+public:
+    virtual ~Allocator() = default;
+    virtual std::string
+    Name() = 0;
+    virtual void*
+    Allocate(uint64_t size) = 0;
+    virtual void
+    Deallocate(void* p) = 0;
+    virtual void*
+    Reallocate(void* p, uint64_t size) = 0;
+};
+
 class Dataset;
 using DatasetPtr = std::shared_ptr<Dataset>;
 
-// Column container with the reference's builder style.  An owning dataset frees ids / distances / vectors
-// with delete[] when it dies (results of a search are owning).
+// Column container with the reference's builder style.  An owning dataset frees ids / distances / vectors when it
+// dies (results of a search are owning): through its allocator when it was given one (Owner(true, allocator),
+// include/vsag/dataset.h:140-147), else with delete[].
 class VSAG_HOST_EXPORT Dataset : public std::enable_shared_from_this<Dataset> {
 public:
     static DatasetPtr
@@ -123,15 +140,20 @@ public:
         return DatasetPtr(new Dataset());
     }
     ~Dataset() {
-        if (owner_) {
+        if (owner_ && allocator_ != nullptr) {
+            allocator_->Deallocate(const_cast<int64_t*>(ids_));
+            allocator_->Deallocate(const_cast<float*>(distances_));
+            allocator_->Deallocate(const_cast<float*>(vectors_));
+        } else if (owner_) {
             delete[] ids_;
             delete[] distances_;
             delete[] vectors_;
         }
     }
     DatasetPtr
-    Owner(bool is_owner) {
+    Owner(bool is_owner, Allocator* allocator = nullptr) {
         owner_ = is_owner;
+        allocator_ = allocator;
         return shared_from_this();
     }
     DatasetPtr
@@ -192,6 +214,7 @@ public:
 private:
     Dataset() = default;
     bool owner_ = true;
+    Allocator* allocator_ = nullptr;
     int64_t num_elements_ = 0;
     int64_t dim_ = 0;
     const int64_t* ids_ = nullptr;
@@ -351,8 +374,10 @@ public:
     // name: "brute_force" or "ivf".  parameters: {"dtype":"float32","metric_type":"l2"|"ip"|"cosine","dim":N,
     // "index_param":{...}} with the reference's keys (src/constants.cpp:195-216,255-265); unknown index_param
     // keys are INVALID_ARGUMENT "invalid config param: <key>" (src/utils/util_functions.cpp:45-66).
+    // allocator (include/vsag/factory.h:47-50): where the index takes the host arrays of its results from; nullptr =
+    // new[] / delete[].  It must outlive the index and every result the index returned.
     static Expected<std::shared_ptr<Index>>
-    CreateIndex(const std::string& name, const std::string& parameters);
+    CreateIndex(const std::string& name, const std::string& parameters, Allocator* allocator = nullptr);
 };
 
 }  // namespace vsag
