@@ -659,7 +659,11 @@ def run_c4(env):
                          "configs[3]%s: IVF search, N=%d, d=%d, nlist=%d, nprobe=%d, rerank %d, %d queries, k=%d"
                          % ("" if bits == 4 else " with sq8_uniform lists", n, d, nlist, nprobe, kcand, nq, k),
                          {"recall_at_10": rec, "build_seconds": t_build, "scanned_codes_per_query": float(scanned) / nq,
-                          "bytes_per_scanned_code": cs + 4, "single_query": single}, roof, cpu)
+                          "bytes_per_scanned_code": cs + 4, "single_query": single,
+                          "list_sizes": {"mean": float(sizes.mean()), "max": int(sizes.max()), "min": int(sizes.min()),
+                                         "p99": float(np.percentile(sizes, 99))},
+                          "queries_per_first_list": {"max": int(np.bincount(b[:, 0].clip(0), minlength=nlist).max()),
+                                                     "mean": float(nq) / nlist}}, roof, cpu)
 
 
 # ------------------------------------------------------------------------------------------- C5

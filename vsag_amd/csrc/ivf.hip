@@ -89,6 +89,75 @@ count_pairs_kernel(const int32_t* buckets, uint64_t nq, uint32_t nprobe, uint32_
     }
 }
 
+// The same grouping for many pairs without an atomic per pair in global memory (hundreds of thousands of them on a
+// few thousand counters take 0.1 ms per launch): a counting sort in three launches.  kRegroupGroups workgroups each
+// take a run of the pairs; regroup_hist_kernel counts a run's pairs per list in LDS, regroup_prefix_kernel turns
+// the counts of a list into the offsets of the runs inside the list (and their sum into counts[]), and
+// regroup_scatter_kernel hands out the places of a run with a cursor per list in LDS.
+constexpr uint32_t kRegroupGroups = 128;
+constexpr uint32_t kRegroupLists = 8192;  // lists a workgroup's LDS holds a counter for
+
+__global__ void __launch_bounds__(1024)
+regroup_hist_kernel(const int32_t* buckets, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t p1, uint32_t nlist,
+                    uint32_t* hist) {
+    __shared__ uint32_t h[kRegroupLists];
+    for (uint32_t b = threadIdx.x; b < nlist; b += blockDim.x) {
+        h[b] = 0;
+    }
+    __syncthreads();
+    const uint32_t w = p1 - p0;
+    const uint64_t total = nq * w, per = (total + gridDim.x - 1) / gridDim.x;
+    const uint64_t begin = blockIdx.x * per, end = begin + per < total ? begin + per : total;
+    for (uint64_t i = begin + threadIdx.x; i < end; i += blockDim.x) {
+        const uint64_t q = i / w;
+        const int32_t b = buckets[q * nprobe + p0 + static_cast<uint32_t>(i - q * w)];
+        if (b >= 0 && static_cast<uint32_t>(b) < nlist) {
+            atomicAdd(&h[b], 1U);
+        }
+    }
+    __syncthreads();
+    for (uint32_t b = threadIdx.x; b < nlist; b += blockDim.x) {
+        hist[static_cast<uint64_t>(blockIdx.x) * nlist + b] = h[b];
+    }
+}
+
+__global__ void __launch_bounds__(256)
+regroup_prefix_kernel(uint32_t* hist, uint32_t groups, uint32_t nlist, uint32_t* counts) {
+    const uint32_t b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nlist) {
+        return;
+    }
+    uint32_t running = 0;
+    for (uint32_t g = 0; g < groups; ++g) {
+        const uint32_t c = hist[static_cast<uint64_t>(g) * nlist + b];
+        hist[static_cast<uint64_t>(g) * nlist + b] = running;
+        running += c;
+    }
+    counts[b] = running;
+}
+
+__global__ void __launch_bounds__(1024)
+regroup_scatter_kernel(const int32_t* buckets, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t p1, uint32_t nlist,
+                       const uint32_t* pair_off, const uint32_t* hist, uint32_t* sorted_pair) {
+    __shared__ uint32_t cursor[kRegroupLists];
+    for (uint32_t b = threadIdx.x; b < nlist; b += blockDim.x) {
+        cursor[b] = 0;
+    }
+    __syncthreads();
+    const uint32_t w = p1 - p0;
+    const uint64_t total = nq * w, per = (total + gridDim.x - 1) / gridDim.x;
+    const uint64_t begin = blockIdx.x * per, end = begin + per < total ? begin + per : total;
+    for (uint64_t i = begin + threadIdx.x; i < end; i += blockDim.x) {
+        const uint64_t q = i / w;
+        const uint32_t p = p0 + static_cast<uint32_t>(i - q * w);
+        const int32_t b = buckets[q * nprobe + p];
+        if (b >= 0 && static_cast<uint32_t>(b) < nlist) {
+            const uint32_t pos = pair_off[b] + hist[static_cast<uint64_t>(blockIdx.x) * nlist + b] + atomicAdd(&cursor[b], 1U);
+            sorted_pair[pos] = static_cast<uint32_t>(q * nprobe + p);
+        }
+    }
+}
+
 // Chunks a list of `tiles` tiles is cut into: about tiles_per_item tiles each, at most chunks_max chunks
 // (longer lists get longer chunks); 0xFFFFFFFF = never cut.
 __device__ inline uint32_t
@@ -775,6 +844,7 @@ struct IvfBuffers {
     uint32_t* pair_off;   // nlist + 1
     uint32_t* item_off;   // nlist + 1
     uint32_t* sorted_pair;
+    uint32_t* hist;       // counting sort of many pairs: kRegroupGroups x nlist
     uint32_t* bound;
     uint32_t* seed;
     uint32_t* partial_cnt;
@@ -841,6 +911,13 @@ plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, 
     }
 }
 
+// Whether the pairs of a call are grouped by the counting sort (regroup_hist_kernel ...) rather than with an atomic
+// per pair.
+static bool
+regroup_by_sort(const vsag_amd_store* s, uint64_t npairs) {
+    return npairs >= 65536 && s->nlist <= kRegroupLists;
+}
+
 static size_t
 carve_ivf(Carver& c, const vsag_amd_store* s, const ScanPlanIvf& p, uint64_t nq, uint32_t kcand, IvfBuffers* b) {
     b->qtab = c.take<uint32_t>((nq + 1) * p.ql.qstride);
@@ -851,6 +928,7 @@ carve_ivf(Carver& c, const vsag_amd_store* s, const ScanPlanIvf& p, uint64_t nq,
     b->pair_off = c.take<uint32_t>(s->nlist + 1);
     b->item_off = c.take<uint32_t>(s->nlist + 1);
     b->sorted_pair = c.take<uint32_t>(p.npairs);
+    b->hist = c.take<uint32_t>(regroup_by_sort(s, p.npairs) ? static_cast<size_t>(kRegroupGroups) * s->nlist : 0);
     b->bound = c.take<uint32_t>(nq);
     b->seed = c.take<uint32_t>(p.seeded ? nq * kcand : 0);
     b->partial_cnt = c.take<uint32_t>(p.npairs * p.chunks_max);
@@ -982,6 +1060,27 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
     uint32_t cols[3] = {0, p.chunked ? nprobe : 1, nprobe};
     // A pre-filter or a radius goes the streaming way (the matrix-core pass knows neither).
     const bool mfma = p.mfma && (options == nullptr || (options->deny_bits_dev == nullptr && options->use_radius == 0));
+    // The pairs of columns [c0, c1) grouped by list (pair_off, sorted_pair) and the work items of every list (item_off).
+    auto regroup = [&](uint32_t c0, uint32_t c1, uint64_t pairs, uint32_t per_item, uint32_t tiles_per_item,
+                       uint32_t chunks_max) {
+        if (b.hist != nullptr && pairs >= 65536) {
+            hipLaunchKernelGGL(regroup_hist_kernel, dim3(kRegroupGroups), dim3(1024), 0, st, buckets_dev, nq, nprobe, c0,
+                               c1, s->nlist, b.hist);
+            hipLaunchKernelGGL(regroup_prefix_kernel, dim3(static_cast<uint32_t>(div_up(s->nlist, 256))), dim3(256), 0, st,
+                               b.hist, kRegroupGroups, s->nlist, b.counts);
+            hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, st, b.counts, s->list_tile_dev, s->nlist, per_item,
+                               tiles_per_item, chunks_max, b.pair_off, b.item_off);
+            hipLaunchKernelGGL(regroup_scatter_kernel, dim3(kRegroupGroups), dim3(1024), 0, st, buckets_dev, nq, nprobe,
+                               c0, c1, s->nlist, b.pair_off, b.hist, b.sorted_pair);
+            return;
+        }
+        hipLaunchKernelGGL(count_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq, nprobe, c0, c1,
+                           s->nlist, b.counts);
+        hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, st, b.counts, s->list_tile_dev, s->nlist, per_item,
+                           tiles_per_item, chunks_max, b.pair_off, b.item_off);
+        hipLaunchKernelGGL(scatter_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq, nprobe, c0,
+                           c1, s->nlist, b.pair_off, b.cursor, b.sorted_pair);
+    };
     timing_begin(st);
     for (int pass = 0; pass < 2; ++pass) {
         uint32_t p0 = cols[pass], p1 = cols[pass + 1];
@@ -996,12 +1095,8 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
         if (pass == 1 && mfma) {
             // Pairs grouped by list once; workgroups of 256 pairs for the matrix cores, then -- for the queries whose
             // lists overflowed -- the streaming kernel's items over the same grouping.
-            hipLaunchKernelGGL(count_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq, nprobe,
-                               p0, p1, s->nlist, b.counts);
-            hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, st, b.counts, s->list_tile_dev, s->nlist, 256U,
-                               32U, 4U, b.pair_off, b.item_off);  // ivf_i8.hip: kIvfI8ChunkTiles, kIvfI8Chunks
-            hipLaunchKernelGGL(scatter_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq,
-                               nprobe, p0, p1, s->nlist, b.pair_off, b.cursor, b.sorted_pair);
+            // ivf_i8.hip: items of 256 pairs, kIvfI8ChunkTiles, kIvfI8Chunks
+            regroup(p0, p1, pairs, 256U, 32U, 4U);
             VA_TRY(launch_ivf_i8(s, a, nq, nprobe, p0, kcand, b.pair_off, b.item_off, b.sorted_pair, b.bound, b.tq,
                                  b.partial, b.partial_cnt, b.gate, buckets_dev, b.gpairs, kGatedPairsCap, st));
             // Few gated pairs (the usual case): one wave per pair and chunk of its list.
@@ -1027,22 +1122,28 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
             VA_TRY(launch_ivf(s, p.T, grid, dim3(waves * kWave), lds, st, a, v));
             continue;
         }
+        // The nearest-list pass ahead of the matrix cores: a list several times the average length (k-means leaves
+        // such lists) would keep one wave busy long after the others are done, so lists are cut into chunks of about
+        // the average list's length; a pair's chunks use the private lists the matrix-core pass has per pair anyway.
+        IvfArgs first = v;
+        const bool cut_first = mfma && pass == 0;
+        if (cut_first) {
+            const uint32_t avg_tiles = std::max<uint32_t>(1, static_cast<uint32_t>(s->ntiles / s->nlist));
+            first.tiles_per_item = std::max<uint32_t>(std::max<uint32_t>(16, avg_tiles + avg_tiles / 4),
+                                                      static_cast<uint32_t>(div_up(s->max_list_tiles, p.chunks_max)));
+        }
         if (p.chunked) {
             hipLaunchKernelGGL(regroup_small_kernel, dim3(1), dim3(1024), 0, st, buckets_dev, nq, nprobe,
                                s->list_tile_dev, s->nlist, static_cast<uint32_t>(p.T), p.tiles_per_item, p.chunks_max,
                                b.counts, b.cursor, b.pair_off, b.item_off, b.sorted_pair);
         } else {
-            hipLaunchKernelGGL(count_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq, nprobe,
-                               p0, p1, s->nlist, b.counts);
-            hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, st, b.counts, s->list_tile_dev, s->nlist,
-                               static_cast<uint32_t>(p.T), p.tiles_per_item, p.chunks_max, b.pair_off, b.item_off);
-            hipLaunchKernelGGL(scatter_pairs_kernel, dim3(blocks_for(pairs)), dim3(256), 0, st, buckets_dev, nq,
-                               nprobe, p0, p1, s->nlist, b.pair_off, b.cursor, b.sorted_pair);
+            regroup(p0, p1, pairs, static_cast<uint32_t>(p.T), first.tiles_per_item, p.chunks_max);
         }
         // At most one partly filled query group per probed list, each cut into at most chunks_max items.
-        uint64_t max_items = (div_up(pairs, p.T) + std::min<uint64_t>(s->nlist, pairs)) * (p.chunked ? p.chunks_max : 1);
+        uint64_t max_items =
+            (div_up(pairs, p.T) + std::min<uint64_t>(s->nlist, pairs)) * (p.chunked || cut_first ? p.chunks_max : 1);
         dim3 grid(static_cast<uint32_t>(div_up(max_items, waves)));
-        VA_TRY(launch_ivf(s, p.T, grid, dim3(waves * kWave), lds, st, a, v));
+        VA_TRY(launch_ivf(s, p.T, grid, dim3(waves * kWave), lds, st, a, first));
     }
     if (!mfma) {
         timing_end(st);  // the matrix-core pass is timed on its own (ivf_i8.hip)
