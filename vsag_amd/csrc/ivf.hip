@@ -411,6 +411,7 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
     const uint32_t pend = plast;
 
     const uint32_t S = v.S, k = v.k;
+    const uint32_t spend = selector_base(S, k);  // where a selector's pending keys start
     uint64_t* sel = lds + static_cast<size_t>(wave) * T * S;
     uint32_t qidx[T], pair[T];
     uint64_t tau[T];
@@ -512,7 +513,7 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
             }
             uint64_t* keys = sel + t * S;
             uint32_t np = __popcll(mask);
-            if (k + cnt[t] + np > S) {
+            if (spend + cnt[t] + np > S) {
                 uint64_t th = selector_flush(keys, S, k, cnt[t], lane);
                 cnt[t] = 0;
                 cold[t] = 0;
@@ -524,7 +525,7 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
                 }
             }
             if (pass) {
-                keys[k + cnt[t] + mask_rank(mask)] = key;
+                keys[spend + cnt[t] + mask_rank(mask)] = key;
             }
             cnt[t] += np;
         }
@@ -553,7 +554,7 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
         uint64_t* keys = sel + t * S;
         wave_lds_fence();
         uint32_t bs = __builtin_amdgcn_readfirstlane(__atomic_load_n(&v.bound[qidx[t]], __ATOMIC_RELAXED));
-        uint32_t total = k + cnt[t];
+        uint32_t total = spend + cnt[t];
         uint32_t admitted = selector_count_admitted(keys, total, bs, lane);
         if (admitted > k) {
             uint64_t th = selector_flush(keys, S, k, cnt[t], lane);

@@ -422,6 +422,7 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
         return;
     }
     const uint32_t S = r.S, k = r.k;
+    const uint32_t pend = selector_base(S, k);  // where the selector's pending keys start
     selector_init(keys, S, lane);
     uint32_t cnt = 0;
     uint32_t bs = __builtin_amdgcn_readfirstlane(__atomic_load_n(&r.bound[q], __ATOMIC_RELAXED));
@@ -462,7 +463,7 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
             uint64_t mask = __ballot(pass);
             if (mask != 0) {
                 uint32_t np = __popcll(mask);
-                if (k + cnt + np > S) {
+                if (pend + cnt + np > S) {
                     uint64_t th = selector_flush(keys, S, k, cnt, lane);
                     cnt = 0;
                     uint32_t b = lower_shared(&r.bound[q], static_cast<uint32_t>(th >> 32), lane);
@@ -470,7 +471,7 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
                     tau = th < shared_tau ? th : shared_tau;
                 }
                 if (pass) {
-                    keys[k + cnt + mask_rank(mask)] = key;
+                    keys[pend + cnt + mask_rank(mask)] = key;
                 }
                 cnt += np;
             }
@@ -542,7 +543,7 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
     }
     wave_lds_fence();
     bs = __builtin_amdgcn_readfirstlane(__atomic_load_n(&r.bound[q], __ATOMIC_RELAXED));
-    uint32_t kept = k + cnt;
+    uint32_t kept = pend + cnt;
     uint32_t admitted = selector_count_admitted(keys, kept, bs, lane);
     if (admitted > k) {
         uint64_t th = selector_flush(keys, S, k, cnt, lane);

@@ -152,6 +152,7 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
     Acc<KIND, T> acc;
     acc_reset(acc);
 
+    const uint32_t pend = selector_base(S, k);  // where a selector's pending keys start
     // Sorts selector t and folds its k-th key and the shared bound into thr[t].
     auto flush = [&](int t) {
         uint64_t* keys = sel + t * S;
@@ -212,11 +213,11 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
             uint64_t mask = __ballot(pass);
             if (mask != 0) {
                 uint32_t np = __popcll(mask);
-                if (k + cnt[t] + np > S) {
+                if (pend + cnt[t] + np > S) {
                     flush(t);
                 }
                 if (pass) {
-                    sel[t * S + k + cnt[t] + mask_rank(mask)] = (static_cast<uint64_t>(od) << 32) | static_cast<uint32_t>(id);
+                    sel[t * S + pend + cnt[t] + mask_rank(mask)] = (static_cast<uint64_t>(od) << 32) | static_cast<uint32_t>(id);
                 }
                 cnt[t] += np;
             }
@@ -248,7 +249,7 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
         uint64_t* keys = sel + t * S;
         wave_lds_fence();
         uint32_t bs = __builtin_amdgcn_readfirstlane(__atomic_load_n(&f.bound[qidx[t]], __ATOMIC_RELAXED));
-        uint32_t total = k + cnt[t];
+        uint32_t total = pend + cnt[t];
         uint32_t admitted = selector_count_admitted(keys, total, bs, lane);
         if (admitted > k) {
             uint64_t th = selector_flush(keys, S, k, cnt[t], lane);

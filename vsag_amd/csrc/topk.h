@@ -1,10 +1,12 @@
 // Wave-level streaming top-k selector kept in LDS.
 //
 // One wavefront owns one selector per query it serves.  A selector is an array of S 64-bit keys
-// (S a power of two, S >= k + 96): slots [0,k) hold the best keys found so far, slots [k,k+cnt) hold
-// pending candidates that passed the current threshold.  When an append would overflow the pending
-// region, the wave first sorts the whole array (bitonic, in LDS) which leaves the k best in front and
-// yields the new threshold keys[k-1].  No workgroup barrier is involved: only the owning
+// (S a power of two, S >= k + 96): slots [0,k) hold the best keys found so far, slots [base, base+cnt), base =
+// selector_base(S, k), hold pending candidates that passed the current threshold.  When an append would overflow
+// the pending region, the wave flushes: the k best of everything end up in front, in ascending order, and
+// keys[k-1] is the new threshold.  With k <= S / 2 (and S >= 256) the pending region is the upper half and a flush
+// sorts only that half (downwards) and merges it into the sorted front -- half the compare-exchange steps of sorting
+// the whole array, which is what the other selectors do.  No workgroup barrier is involved: only the owning
 // wave touches a selector, and LDS operations of one wave complete in program order.
 //
 // This replaces the reference's per-query bounded max-heap (src/impl/heap/standard_heap.cpp:24-53,
@@ -52,6 +54,12 @@ selector_slots(uint32_t k) {
     return s;
 }
 
+// First slot of the pending region.
+__host__ __device__ inline uint32_t
+selector_base(uint32_t S, uint32_t k) {
+    return S >= 256 && 2 * k <= S ? S / 2 : k;
+}
+
 __device__ inline void
 selector_init(uint64_t* keys, uint32_t S, uint32_t lane) {
     for (uint32_t i = lane; i < S; i += kWave) {
@@ -80,29 +88,62 @@ wave_bitonic_sort(uint64_t* keys, uint32_t S, uint32_t lane) {
     }
 }
 
-// Sorts, keeps the k best in front, returns the new threshold key (wave-uniform).
+// One compare-exchange step of a bitonic network over keys[0, n): pairs `stride` apart, ascending where
+// (pos & size) == 0 (size = 0: everywhere), descending elsewhere; `flip` turns the directions round.
+__device__ inline void
+wave_bitonic_step(uint64_t* keys, uint32_t n, uint32_t size, uint32_t stride, bool flip, uint32_t lane) {
+    for (uint32_t i = lane; i < (n >> 1); i += kWave) {
+        uint32_t pos = 2 * i - (i & (stride - 1));
+        uint64_t a = keys[pos];
+        uint64_t b = keys[pos + stride];
+        bool up = ((pos & size) == 0) != flip;
+        if ((a > b) == up) {
+            keys[pos] = b;
+            keys[pos + stride] = a;
+        }
+    }
+    wave_lds_fence();
+}
+
+// Keeps the k best in front, in ascending order, and returns the new threshold key (wave-uniform).  keys[0, k) are in
+// ascending order on entry (they are after selector_init and after every flush), cnt keys are pending.
 __device__ inline uint64_t
 selector_flush(uint64_t* keys, uint32_t S, uint32_t k, uint32_t cnt, uint32_t lane) {
-    for (uint32_t i = k + cnt + lane; i < S; i += kWave) {
+    const uint32_t base = selector_base(S, k);
+    for (uint32_t i = base + cnt + lane; i < S; i += kWave) {
         keys[i] = kInfKey;
     }
     wave_lds_fence();
-    wave_bitonic_sort(keys, S, lane);
-    return wave_uniform_u64(keys[k - 1]);
-}
-
-// Appends the keys of the lanes with `pass` set behind the pending region; returns the new count.
-// The caller guarantees k + cnt + 64 <= S.
-__device__ inline uint32_t
-selector_append(uint64_t* keys, uint32_t k, uint32_t cnt, bool pass, uint64_t key) {
-    uint64_t mask = __ballot(pass);
-    if (mask != 0) {
-        if (pass) {
-            keys[k + cnt + mask_rank(mask)] = key;
-        }
-        cnt += __popcll(mask);
+    if (base == k) {
+        wave_bitonic_sort(keys, S, lane);
+        return wave_uniform_u64(keys[k - 1]);
     }
-    return cnt;
+    // The front half is ascending (k keys, then kInfKey).  The pending half sorted downwards behind it makes the
+    // whole array bitonic; one step across the halves leaves the smaller half in front, itself bitonic, and a
+    // merge puts it in order.
+    uint64_t* pending = keys + base;
+    for (uint32_t size = 2; size <= base; size <<= 1) {
+        for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+            wave_bitonic_step(pending, base, size == base ? 0 : size, stride, true, lane);
+        }
+    }
+    for (uint32_t i = lane; i < base; i += kWave) {
+        uint64_t a = keys[i];
+        uint64_t b = keys[i + base];
+        if (b < a) {
+            keys[i] = b;
+        }
+    }
+    wave_lds_fence();
+    for (uint32_t stride = base >> 1; stride > 0; stride >>= 1) {
+        wave_bitonic_step(keys, base, 0, stride, false, lane);
+    }
+    // Only the k best stay.
+    for (uint32_t i = k + lane; i < base; i += kWave) {
+        keys[i] = kInfKey;
+    }
+    wave_lds_fence();
+    return wave_uniform_u64(keys[k - 1]);
 }
 
 // How many of keys[0,total) are real and have an ordered distance of at most `bound` (wave-uniform).
