@@ -128,10 +128,20 @@ regroup_prefix_kernel(uint32_t* hist, uint32_t groups, uint32_t nlist, uint32_t*
         return;
     }
     uint32_t running = 0;
-    for (uint32_t g = 0; g < groups; ++g) {
-        const uint32_t c = hist[static_cast<uint64_t>(g) * nlist + b];
-        hist[static_cast<uint64_t>(g) * nlist + b] = running;
-        running += c;
+    // Sixteen loads in flight at a time (the stores into the same array would otherwise keep them apart).
+    for (uint32_t g0 = 0; g0 < groups; g0 += 16) {
+        uint32_t c[16];
+#pragma unroll
+        for (uint32_t u = 0; u < 16; ++u) {
+            c[u] = g0 + u < groups ? hist[static_cast<uint64_t>(g0 + u) * nlist + b] : 0U;
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 16; ++u) {
+            if (g0 + u < groups) {
+                hist[static_cast<uint64_t>(g0 + u) * nlist + b] = running;
+                running += c[u];
+            }
+        }
     }
     counts[b] = running;
 }

@@ -407,6 +407,9 @@ merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, cons
     __shared__ uint32_t npool;
     __shared__ uint32_t nout;
     __shared__ SelectScratch scratch;
+    constexpr uint32_t kLongLists = 128;
+    __shared__ uint32_t nlong;
+    __shared__ uint32_t long_slot[kLongLists];
     uint64_t* pool = lds + S;
     const uint64_t q = blockIdx.x;
     const uint32_t* cnts = partial_cnt + q * stride;  // the first nslots of the query's `stride` lists
@@ -421,6 +424,7 @@ merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, cons
         if (threadIdx.x == 0) {
             npool = 0;
             nout = 0;
+            nlong = 0;
         }
         __syncthreads();
         if (nslots * 4 <= blockDim.x) {
@@ -449,9 +453,24 @@ merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, cons
                 }
             }
         } else {
-            // A thread per list: most lists are empty or nearly so once the bound is known.
+            // A thread per list: most lists are empty or nearly so once the bound is known.  The few long ones (the
+            // lists of a query's nearest bucket hold up to k keys each) are noted and read a wave per list afterwards:
+            // one thread walking such a list would outlast the whole workgroup.
+            auto pool_key = [&](uint64_t key) {
+                uint32_t pos = atomicAdd(&npool, 1U);
+                if (pos < pool_keys) {
+                    pool[pos] = key;
+                }
+            };
             for (uint32_t slot = threadIdx.x; slot < nslots; slot += blockDim.x) {
                 const uint32_t c = cnts[slot];
+                if (c > 4) {
+                    const uint32_t at = atomicAdd(&nlong, 1U);
+                    if (at < kLongLists) {
+                        long_slot[at] = slot;
+                        continue;
+                    }
+                }
                 const uint64_t* list = src + static_cast<uint64_t>(slot) * k;
                 // Four loads in flight at a time: the pool's atomics would otherwise serialise them.
                 for (uint32_t i = 0; i < c; i += 4) {
@@ -463,11 +482,34 @@ merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, cons
 #pragma unroll
                     for (uint32_t j = 0; j < 4; ++j) {
                         if (i + j < c && key[j] <= admit) {
-                            uint32_t pos = atomicAdd(&npool, 1U);
-                            if (pos < pool_keys) {
-                                pool[pos] = key[j];
-                            }
+                            pool_key(key[j]);
                         }
+                    }
+                }
+            }
+            __syncthreads();
+            const uint32_t lane = threadIdx.x & (kWave - 1);
+            const uint32_t nl = nlong < kLongLists ? nlong : kLongLists;
+            for (uint32_t w = threadIdx.x / kWave; w < nl; w += blockDim.x / kWave) {
+                const uint32_t slot = long_slot[w];
+                const uint32_t c = cnts[slot];
+                const uint64_t* list = src + static_cast<uint64_t>(slot) * k;
+                for (uint32_t i0 = 0; i0 < c; i0 += kWave) {
+                    const uint32_t i = i0 + lane;
+                    const uint64_t key = i < c ? list[i] : kInfKey;
+                    const bool keep = i < c && key <= admit;
+                    const uint64_t votes = __ballot(keep);
+                    if (votes == 0) {
+                        continue;
+                    }
+                    uint32_t base = 0;
+                    if (lane == 0) {
+                        base = atomicAdd(&npool, static_cast<uint32_t>(__popcll(votes)));
+                    }
+                    base = __shfl(base, 0);
+                    const uint32_t pos = base + static_cast<uint32_t>(__popcll(votes & ((1ULL << lane) - 1)));
+                    if (keep && pos < pool_keys) {
+                        pool[pos] = key;
                     }
                 }
             }
