@@ -709,6 +709,13 @@ make_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, uint64_t ntiles, Sca
     while (waves > 1 && static_cast<size_t>(waves) * T * p->S * 8 > lds_budget) {
         waves >>= 1;
     }
+    // A short scan under many queries (centroid routing, the exact prefix of a pre-selected batch): every wave of a
+    // workgroup keeps selectors of its own for the same queries, so with a few tiles per wave the selecting outweighs
+    // the scanning.  Fewer waves then, as long as the grid still holds two waves per SIMD of the machine.
+    const uint64_t groups_all = div_up(nq, static_cast<uint64_t>(T));
+    while (waves > 1 && ntiles / waves < 32 && groups_all * (waves / 2) >= static_cast<uint64_t>(device_cu_count()) * 8) {
+        waves >>= 1;
+    }
     p->T = T;
     p->waves = waves;
     p->lds_bytes = static_cast<size_t>(waves) * T * p->S * 8;
