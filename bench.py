@@ -649,7 +649,7 @@ def run_c4(env):
         roof = {"bound": "mfma", "achieved": tops, "peak": MFMA_I8_PEAK_TOPS, "unit": "TOP/s",
                 "frac": tops / MFMA_I8_PEAK_TOPS,
                 # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this launch: profiles/ivf_i8_sq4u_c4.md
-                "traffic": 490258.9 * 2.00 * 1024 + 73488.6 * 1024
+                "traffic": 491061.0 * 2.00 * 1024 + 73550.7 * 1024
                 if (n, d, nq, k, nlist, bits) == (10000000, 128, 10000, 10, 4096, 4) else None,
                 "kernel": "ivf_i8_kernel<%s> (int8 MFMA, probe columns 1..%d)" % (kind_name, nprobe - 1), "kernel_ms": kms,
                 "ops_per_launch": ops, "distance_evaluations_per_launch": float(rest),
