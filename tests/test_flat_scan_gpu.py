@@ -108,6 +108,44 @@ def test_append_in_pieces_equals_one_append(lib):
     b.destroy()
 
 
+@pytest.mark.parametrize("kind,d", [("sq8", 128), ("sq8", 16), ("fp32", 128), ("sq4u", 128), ("fp32", 4)])
+@pytest.mark.parametrize("n", [1024, 2048, 16384])
+def test_store_filled_to_the_last_tile_of_its_buffer(lib, kind, d, n):
+    """A store grows by doubling from 16 tiles, so these sizes fill the tile buffer to its last byte.  The scan fetches
+    tile rows in groups with fixed offsets and no branch around a load, which reads past the last tile by design: the
+    buffer ends with slack for that, and nothing read there may reach a result.  One query per call (eight rows per
+    group) and a small batch."""
+    rng = np.random.default_rng(n + d)
+    x, means = gaussian_mixture(rng, n, d, 10, 0.05)
+    q, _ = gaussian_mixture(rng, 9, d, 10, 0.05, means=means)
+    if kind == "sq8":
+        lb, diff = orc.sq_train(x, 8)
+        codes = orc.sq_encode(x, 8, lb, diff)
+        st = Store(lib.KIND_SQ8, orc.L2, d, lb=lb, diff=diff)
+        ref = lambda qq, k: orc.flat_scan_topk(orc.SQ8, orc.L2, d, codes, qq, k, lb=lb, diff=diff)
+    elif kind == "sq4u":
+        lb, diff = orc.sq_train_uniform(x, 4, orc.L2, mode=3)
+        codes = orc.squ_encode(x, 4, lb, diff, orc.L2)
+        st = Store(lib.KIND_SQ4_UNIFORM, orc.L2, d, bounds=[lb, diff])
+        ref = lambda qq, k: orc.flat_scan_topk(orc.SQ4U, orc.L2, d, codes, orc.squ_encode(qq, 4, lb, diff, orc.L2), k,
+                                               lb=lb, diff=diff)
+    else:
+        codes = x.view(np.uint8).reshape(n, 4 * d)
+        st = Store(lib.KIND_FP32, orc.L2, d)
+        ref = lambda qq, k: orc.flat_scan_topk(orc.FP32, orc.L2, d, codes, qq, k)
+    # in pieces, so that the buffer has grown (and been copied) several times on the way
+    st.append(codes[:1000])
+    st.append(codes[1000:n - 1])
+    st.append(codes[n - 1:])
+    assert st.size() == n
+    for qq in (q[:1], q):
+        ids, ds = st.flat_scan(qq, 10)
+        rids, rds = ref(qq, 10)
+        assert_topk_close(ids, ds, rids, rds, atol=2e-6, label="%s filled to capacity" % kind)
+        assert ids.max() < n
+    st.destroy()
+
+
 def test_empty_store_and_bad_arguments(lib):
     st = Store(lib.KIND_FP32, orc.L2, 8)
     ids, ds = st.flat_scan(np.zeros((2, 8), np.float32), 3)
