@@ -76,6 +76,53 @@ def test_ivf_scan_matches_oracle(lib, kind, okind, bits, n, d, nlist, nq, nprobe
     st.destroy()
 
 
+@pytest.mark.parametrize("kind", ["sq8", "sq4u"])
+def test_many_pairs_are_grouped_by_the_counting_sort(lib, kind):
+    """From 65 536 (query, list) pairs of a pass on, the pairs are grouped by list with a counting sort in LDS instead of
+    an atomic per pair; what a query finds does not depend on where its pairs land inside a list's group.  Streaming
+    kernels only (sq8 lists; sq4_uniform with the matrix cores switched off), a ragged bucket table, one list much
+    longer than the others."""
+    rng = np.random.default_rng(5)
+    n, d, nlist, nq, nprobe, kcand = 30000, 32, 48, 10000, 9, 10
+    x, q, cent, labels = _ivf_case(rng, n, d, nlist, nq)
+    labels = labels.copy()
+    labels[rng.random(n) < 0.3] = 7  # a long list
+    offsets, order = orc.ivf_build_lists(labels, nlist)
+    routed, _ = orc.ivf_route(cent, q, nprobe)
+    buckets = routed.copy()
+    buckets[::5, 6:] = -1
+    buckets[3, :] = -1
+    if kind == "sq4u":
+        l, dd = orc.sq_train_uniform(x, 4, orc.L2, mode=3)
+        codes = orc.squ_encode(x, 4, l, dd, orc.L2)
+        qproc = orc.squ_encode(q, 4, l, dd, orc.L2)
+        lb, diff, okind = l, dd, orc.SQ4U
+        st = Store(capi.KIND_SQ4_UNIFORM, orc.L2, d, bounds=[l, dd])
+    else:
+        lb, diff = orc.sq_train(x, 8)
+        codes = orc.sq_encode(x, 8, lb, diff)
+        qproc, okind = q, orc.SQ8
+        st = Store(capi.KIND_SQ8, orc.L2, d, lb=lb, diff=diff)
+    st.set_lists(codes, labels, nlist)
+    L = lib.load_library()
+    capi.check(L.vsag_amd_store_set_scan_contraction(st.handle, -1))
+    ids, ds = st.ivf_scan(q, buckets, kcand)
+    rids, rds = orc.ivf_scan(okind, orc.L2, d, codes[order], offsets, order, qproc, buckets, kcand, lb=lb, diff=diff)
+    if kind == "sq4u":
+        assert np.array_equal(ds.view(np.uint32), rds.view(np.uint32))
+        # and the matrix-core pass over the same grouping
+        capi.check(L.vsag_amd_store_set_scan_contraction(st.handle, -2))
+        fids, fds = st.ivf_scan(q, buckets, kcand)
+        tile = capi.C.c_int()
+        L.vsag_amd_last_scan_info(capi.C.byref(tile), None, None)
+        assert tile.value == 256
+        assert np.array_equal(fids, ids) and np.array_equal(fds.view(np.uint32), ds.view(np.uint32))
+    else:
+        assert_topk_close(ids, ds, rids, rds, atol=2e-6, label="ivf sq8, many pairs")
+    assert np.all(ids[3] == 0xFFFFFFFF)
+    st.destroy()
+
+
 def test_probe_all_lists_equals_flat_scan(lib):
     rng = np.random.default_rng(9)
     n, d, nlist, nq = 5000, 48, 32, 12
