@@ -25,6 +25,7 @@
 #include "vsag_host.h"
 
 namespace vsag {
+inline namespace amd_gpu {
 namespace {
 
 using vsag_host::Json;
@@ -2742,4 +2743,5 @@ Factory::CreateIndex(const std::string& name, const std::string& parameters, All
     });
 }
 
+}  // namespace amd_gpu
 }  // namespace vsag

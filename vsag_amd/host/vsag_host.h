@@ -17,7 +17,11 @@
 #include <utility>
 #include <vector>
 
+// The classes live in an inline namespace: source code says vsag::Index as with the reference, while the symbols
+// (vsag::amd_gpu::Index ...) differ from the reference's, so that a program may link this library beside the real
+// libvsag (one translation unit includes one of the two headers).
 namespace vsag {
+inline namespace amd_gpu {
 
 #define VSAG_HOST_EXPORT __attribute__((visibility("default")))
 
@@ -380,4 +384,5 @@ public:
     CreateIndex(const std::string& name, const std::string& parameters, Allocator* allocator = nullptr);
 };
 
+}  // namespace amd_gpu
 }  // namespace vsag
