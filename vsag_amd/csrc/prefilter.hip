@@ -624,7 +624,8 @@ launch_rescore_m(int metric, dim3 grid, size_t lds, hipStream_t st, const ScanAr
 int launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride, const float* qmeta,
                         uint32_t qmeta_stride, uint64_t nq, uint64_t tile_begin, uint64_t tile_end,
                         const uint32_t* bound, uint8_t* q8, float* u, uint32_t* tau, uint32_t* cand, uint32_t* cand_cnt,
-                        uint32_t sub_lists, uint32_t sub_cap, hipStream_t st);
+                        uint32_t sub_lists, uint32_t sub_cap, bool first_level, const float* merged_dists, uint32_t k,
+                        uint32_t* bound_rw, hipStream_t st);
 
 // Step 3 of the header comment: exact distances of the collected candidates.
 static int
@@ -674,7 +675,8 @@ int
 launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t k, uint32_t S, uint64_t tile_begin,
                  uint64_t tile_end, uint32_t* bound, float* tau, uint32_t* cand, uint32_t* cand_cnt, uint32_t cap,
                  uint64_t* partial, uint32_t* partial_cnt, uint32_t nslots, uint32_t first_slot, uint32_t out_slot,
-                 uint32_t* gate, uint8_t* q8, float* q8_u, uint32_t sub_lists, uint32_t sub_cap, hipStream_t st) {
+                 uint32_t* gate, uint8_t* q8, float* q8_u, uint32_t sub_lists, uint32_t sub_cap,
+                 const float* merged_dists, hipStream_t st) {
     const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
     const bool sq8 = s->kind == VSAG_AMD_KIND_SQ8;
     if (s->kind == VSAG_AMD_KIND_RABITQ) {
@@ -687,7 +689,7 @@ launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32
         // At most 128 dimensions of sq8: the int8 matrix cores pre-select (prefilter_i8.hip).
         VA_TRY(launch_prefilter_i8(s, reinterpret_cast<const float*>(a.qtab), a.qstride, a.qmeta, a.qmeta_stride, nq,
                                    tile_begin, tile_end, bound, q8, q8_u, reinterpret_cast<uint32_t*>(tau), cand,
-                                   cand_cnt, sub_lists, sub_cap, st));
+                                   cand_cnt, sub_lists, sub_cap, out_slot == first_slot, merged_dists, k, bound, st));
         return launch_rescore(s, a, nq, k, S, bound, cand, cand_cnt, 0, sub_lists, sub_cap, partial, partial_cnt, nslots,
                               first_slot, out_slot, gate, st);
     }

@@ -51,7 +51,63 @@ struct QuantizeArgs {
     float* amax;     // l2: per query max |b| (rounded up; 0 for queries that take no part), written by query_amax_kernel
     float* ginv;     // l2: per group of kI8Group queries, 1 / (2 s2) of the scale the group shares (0: no scale)
     uint32_t* tau;   // smallest T that passes (int32); l2: T is the matrix product minus the code's integer term
+    // Per query, what the threshold needs besides the bound (kI8Scalars doubles: q_err, w, a2, b1, s2, usable): kept
+    // so that a later level of the same call only redoes the threshold (retau_queries_i8_kernel).
+    double* scal;
 };
+
+constexpr uint32_t kI8Scalars = 6;
+
+// The threshold of one query against its current bound from the scalars of its quantization: see
+// quantize_queries_i8_kernel for what they are.
+__device__ inline uint32_t
+query_tau_i8(const QuantizeArgs& p, uint64_t q, double q_err, double w, double a2, double b1, double s2, bool usable) {
+    const uint32_t bbits = p.bound[q];
+    if (bbits == 0xFFFFFFFFU || !usable) {
+        // No bound yet, a query with NaN / infinite entries, or (l2) a group of all-zero queries, whose test would
+        // have no scale: everything is a candidate (and the query will overflow into the streaming kernel).
+        return 0x80000000U;
+    }
+    constexpr double kU = 5.9604644775390625e-8;  // 2^-24, the unit roundoff of fp32
+    const double bd = static_cast<double>(ordered_to_float(bbits));
+    const double ymax = static_cast<double>(__uint_as_float(*p.ymax_bits)) * (1.0 + 1.0e-6);
+    if (p.is_l2) {
+        // The streaming kernel sums fl(fl(c s) - a)^2 in fp32: off from the real sum S by at most
+        // 2u sum |y - a| |y| + (n + 2) u S <= 2u sqrt(S) |y| + (n + 2) u S to first order; twice that is allowed for.
+        const double s_abs = fabs(bd);
+        const double e_stream = 4.0 * kU * sqrt(s_abs) * ymax + 2.0 * (p.kdim + 4) * kU * s_abs;
+        // |y|^2 per code is accumulated in double and rounded once.
+        const double e_term = 2.0 * kU * ymax * ymax;
+        // dist = a2 + |y|^2 - 2 s2 (M + 128 w) - 2 <e, c>, M the integer the matrix cores deliver: the pair can matter
+        // when |y|^2 - 2 s2 M <= t_real, i.e. M >= |y|^2 / (2 s2) - t_real / (2 s2).
+        const double t_real = bd - a2 + 256.0 * s2 * w + 2.0 * q_err + e_stream + e_term;
+        // The kernel subtracts I = rn(fl(|y|^2 inv)) from M, inv = fl(1 / (2 s2)) (ginv): I differs from the real
+        // |y|^2 / (2 s2) by at most a half plus two fp32 roundings of a value of at most ymax^2 / (2 s2); the kernel
+        // clamps I from above only, which admits more.  So M - I >= floor(-t_real / (2 s2) - that - 1) keeps every
+        // pair the real test keeps.
+        const double x_max = ymax * ymax / (2.0 * s2);
+        const double x = floor(-t_real / (2.0 * s2) - 0.5 - 4.0 * kU * x_max - 1.0);
+        const int32_t ti = x >= 2147483647.0 ? 0x7FFFFFFF : (x <= -2147483648.0 ? static_cast<int32_t>(0x80000000U)
+                                                                                 : static_cast<int32_t>(x));
+        return static_cast<uint32_t>(ti);
+    }
+    // dist = 1 - (fl(sum c a) + qmeta): the fp32 sum is off by at most n u sum |c a|, the two closing
+    // operations by u of their results; twice that is allowed for.
+    const double qm = p.qmeta != nullptr ? static_cast<double>(p.qmeta[q * p.qmeta_stride]) : 0.0;
+    const double m = fmin(255.0 * b1, sqrt(a2) * ymax * (1.0 + 1.0e-6));
+    const double e_stream = 2.0 * (p.kdim + 2) * kU * m + 4.0 * kU * (m + fabs(qm) + 1.0 + fabs(bd));
+    // 1 - qm - s2 (T + 128 w) - <e, c> <= bd   <=>   T >= -(bd - 1 + qm + errors) / s2 - 128 w.
+    const double rhs = bd - 1.0 + qm + q_err + e_stream;
+    int32_t ti;
+    if (s2 > 0.0) {
+        const double x = floor(-rhs / s2 - 128.0 * w) - 2.0;
+        ti = x >= 2147483647.0 ? 0x7FFFFFFF : (x <= -2147483648.0 ? static_cast<int32_t>(0x80000000U)
+                                                                  : static_cast<int32_t>(x));
+    } else {
+        ti = rhs >= 0.0 ? static_cast<int32_t>(0x80000000U) : 0x7FFFFFFF;
+    }
+    return static_cast<uint32_t>(ti);
+}
 
 __device__ inline double
 wave_sum_f64(double v) {
@@ -182,55 +238,40 @@ quantize_queries_i8_kernel(QuantizeArgs p) {
     if (lane != 0) {
         return;
     }
-    const uint32_t bbits = p.bound[q];
-    if (bbits == 0xFFFFFFFFU || !(b1 < 1.0e300) || !(a2 < 1.0e300) || bad_row || (p.is_l2 && !(s2 > 0.0))) {
-        // No bound yet, a query with NaN / infinite entries, or (l2) a group of all-zero queries, whose test would
-        // have no scale: everything is a candidate (and the query will overflow into the streaming kernel).
-        p.tau[q] = 0x80000000U;
-        return;
-    }
-    constexpr double kU = 5.9604644775390625e-8;  // 2^-24, the unit roundoff of fp32
-    const double bd = static_cast<double>(ordered_to_float(bbits));
-    const double ymax = static_cast<double>(__uint_as_float(*p.ymax_bits)) * (1.0 + 1.0e-6);
     // |<e, c>| for any code, plus the rounding of the double arithmetic above.
     const double q_err = 255.0 * fmax(e_pos, e_neg) + 1.0e-12 * 255.0 * b1;
-    if (p.is_l2) {
-        // The streaming kernel sums fl(fl(c s) - a)^2 in fp32: off from the real sum S by at most
-        // 2u sum |y - a| |y| + (n + 2) u S <= 2u sqrt(S) |y| + (n + 2) u S to first order; twice that is allowed for.
-        const double s_abs = fabs(bd);
-        const double e_stream = 4.0 * kU * sqrt(s_abs) * ymax + 2.0 * (p.kdim + 4) * kU * s_abs;
-        // |y|^2 per code is accumulated in double and rounded once.
-        const double e_term = 2.0 * kU * ymax * ymax;
-        // dist = a2 + |y|^2 - 2 s2 (M + 128 w) - 2 <e, c>, M the integer the matrix cores deliver: the pair can matter
-        // when |y|^2 - 2 s2 M <= t_real, i.e. M >= |y|^2 / (2 s2) - t_real / (2 s2).
-        const double t_real = bd - a2 + 256.0 * s2 * w + 2.0 * q_err + e_stream + e_term;
-        // The kernel subtracts I = rn(fl(|y|^2 inv)) from M, inv = fl(1 / (2 s2)) (ginv above): I differs from the real
-        // |y|^2 / (2 s2) by at most a half plus two fp32 roundings of a value of at most ymax^2 / (2 s2); the kernel
-        // clamps I from above only, which admits more.  So M - I >= floor(-t_real / (2 s2) - that - 1) keeps every
-        // pair the real test keeps.
-        const double x_max = ymax * ymax / (2.0 * s2);
-        const double x = floor(-t_real / (2.0 * s2) - 0.5 - 4.0 * kU * x_max - 1.0);
-        const int32_t ti = x >= 2147483647.0 ? 0x7FFFFFFF : (x <= -2147483648.0 ? static_cast<int32_t>(0x80000000U)
-                                                                                 : static_cast<int32_t>(x));
-        p.tau[q] = static_cast<uint32_t>(ti);
-    } else {
-        // dist = 1 - (fl(sum c a) + qmeta): the fp32 sum is off by at most n u sum |c a|, the two closing
-        // operations by u of their results; twice that is allowed for.
-        const double qm = p.qmeta != nullptr ? static_cast<double>(p.qmeta[q * p.qmeta_stride]) : 0.0;
-        const double m = fmin(255.0 * b1, sqrt(a2) * ymax * (1.0 + 1.0e-6));
-        const double e_stream = 2.0 * (p.kdim + 2) * kU * m + 4.0 * kU * (m + fabs(qm) + 1.0 + fabs(bd));
-        // 1 - qm - s2 (T + 128 w) - <e, c> <= bd   <=>   T >= -(bd - 1 + qm + errors) / s2 - 128 w.
-        const double rhs = bd - 1.0 + qm + q_err + e_stream;
-        int32_t ti;
-        if (s2 > 0.0) {
-            const double x = floor(-rhs / s2 - 128.0 * w) - 2.0;
-            ti = x >= 2147483647.0 ? 0x7FFFFFFF : (x <= -2147483648.0 ? static_cast<int32_t>(0x80000000U)
-                                                                      : static_cast<int32_t>(x));
-        } else {
-            ti = rhs >= 0.0 ? static_cast<int32_t>(0x80000000U) : 0x7FFFFFFF;
-        }
-        p.tau[q] = static_cast<uint32_t>(ti);
+    const bool usable = (b1 < 1.0e300) && (a2 < 1.0e300) && !bad_row && !(p.is_l2 && !(s2 > 0.0));
+    if (p.scal != nullptr) {
+        double* keep = p.scal + q * kI8Scalars;
+        keep[0] = q_err;
+        keep[1] = w;
+        keep[2] = a2;
+        keep[3] = b1;
+        keep[4] = s2;
+        keep[5] = usable ? 1.0 : 0.0;
     }
+    p.tau[q] = query_tau_i8(p, q, q_err, w, a2, b1, s2, usable);
+}
+
+// A later level of the same call: the planes stand, only the bound has moved.  One thread per query; merged_dists
+// (may be null) holds the k best distances of everything before this level, whose k-th lowers the bound first.
+__global__ void __launch_bounds__(256)
+retau_queries_i8_kernel(QuantizeArgs p, const float* merged_dists, uint32_t k, uint32_t* bound) {
+    const uint64_t q = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (q >= p.nq) {
+        return;
+    }
+    if (merged_dists != nullptr) {
+        const float kth = merged_dists[q * k + k - 1];
+        if (kth < __builtin_inff()) {
+            const uint32_t o = float_to_ordered(kth);
+            if (o < bound[q]) {
+                bound[q] = o;
+            }
+        }
+    }
+    const double* keep = p.scal + q * kI8Scalars;
+    p.tau[q] = query_tau_i8(p, q, keep[0], keep[1], keep[2], keep[3], keep[4], keep[5] != 0.0);
 }
 
 // sq8_uniform (and, with 4-bit values, sq4_uniform) stores: the query is a row of bytes itself (its uniform code, 0..255), so the product with the code is
@@ -254,7 +295,51 @@ struct UniformQuantizeArgs {
     uint8_t* q8;
     float* u;
     uint32_t* tau;
+    double* scal;  // per query kI8Scalars doubles, the first holds the sum of the query's values (see QuantizeArgs)
 };
+
+// The threshold of one query of a uniform kind against its current bound; sum = the sum of the query's values.
+__device__ inline uint32_t
+uniform_tau_i8(const UniformQuantizeArgs& p, uint64_t q, double sum) {
+    const uint32_t bbits = p.bound[q];
+    const double rate = static_cast<double>(p.rate);
+    if (bbits == 0xFFFFFFFFU) {
+        return __float_as_uint(3.0e38F);  // no bound yet: everything is a candidate
+    }
+    constexpr double kU = 5.9604644775390625e-8;  // 2^-24
+    const double bd = static_cast<double>(ordered_to_float(bbits));
+    const double qm = static_cast<double>(p.qmeta[q * p.qmeta_stride]);
+    const double cmax = p.nibbles ? 15.0 : 255.0;      // largest code value
+    const double shift = p.nibbles ? 0.0 : 128.0;      // the codes are staged as c - shift
+    const double ip_max = cmax * sum;                  // <code, query> of any code
+    const double t_max = 128.0 * 256.0 * p.kdim;       // |T| of any code
+    const double m_max = p.is_l2 ? cmax * cmax * p.kdim : cmax * p.kdim;  // norm_o, sum_o of any code
+    double t;
+    if (p.is_l2) {
+        // Streaming: fl(fl(fl(qm + m) - 2 R) rate), R the integer as a float (exact below 2^24).  The two sums round
+        // by at most u of their magnitude each, the product by u of itself.
+        if (!(rate > 0.0)) {
+            return __float_as_uint(3.0e38F);
+        }
+        const double reach = fabs(qm) + m_max + 2.0 * ip_max;
+        const double x_max = bd / rate * (1.0 + 4.0 * kU) + 4.0 * kU * reach;  // what qm + m - 2 ip may reach
+        // qm + m - 2 (T + shift sum) <= x_max   <=>   m - 2 T <= x_max - qm + 2 shift sum
+        t = x_max - qm + 2.0 * shift * sum;
+        // The test itself: fl(m - 2 T) in one fma against the rounded threshold.
+        t += 4.0 * kU * (m_max + 2.0 * t_max + fabs(t));
+    } else {
+        // Streaming: r = fl(fl(fl(lb fl(qm + m)) + fl(rate R)) + lb2), distance fl(1 - r).
+        const double lb = fabs(static_cast<double>(p.lb)), lb2 = fabs(static_cast<double>(p.lb2));
+        const double reach = lb * (fabs(qm) + m_max) + rate * ip_max + lb2 + 1.0 + fabs(bd);
+        const double e_stream = 8.0 * kU * reach;
+        // 1 - lb (qm + m) - rate (T + shift sum) - lb2 <= bd + e
+        //     <=>   -rate T - lb m <= bd + e - 1 + lb qm + shift rate sum + lb2
+        t = bd + e_stream - 1.0 + static_cast<double>(p.lb) * qm + shift * rate * sum + static_cast<double>(p.lb2);
+        // term_o = fl(-lb m) and the fma of the test.
+        t += 4.0 * kU * (2.0 * lb * m_max + rate * t_max + fabs(t));
+    }
+    return __float_as_uint(t < 3.0e38 ? (t > -3.0e38 ? static_cast<float>(t) : -3.0e38F) : 3.0e38F);
+}
 
 // One wave per query; lane l owns dimensions l and l + 64.
 __global__ void __launch_bounds__(64)
@@ -295,47 +380,30 @@ quantize_uniform_i8_kernel(UniformQuantizeArgs p) {
     if (lane != 0) {
         return;
     }
-    const uint32_t bbits = p.bound[q];
-    const double rate = static_cast<double>(p.rate);
     p.u[q] = p.is_l2 ? -2.0F : -p.rate;
-    if (bbits == 0xFFFFFFFFU) {
-        p.tau[q] = __float_as_uint(3.0e38F);  // no bound yet: everything is a candidate
+    if (p.scal != nullptr) {
+        p.scal[q * kI8Scalars] = sum;
+    }
+    p.tau[q] = uniform_tau_i8(p, q, sum);
+}
+
+// A later level of the same call (see retau_queries_i8_kernel).
+__global__ void __launch_bounds__(256)
+retau_uniform_i8_kernel(UniformQuantizeArgs p, const float* merged_dists, uint32_t k, uint32_t* bound) {
+    const uint64_t q = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (q >= p.nq) {
         return;
     }
-    constexpr double kU = 5.9604644775390625e-8;  // 2^-24
-    const double bd = static_cast<double>(ordered_to_float(bbits));
-    const double qm = static_cast<double>(p.qmeta[q * p.qmeta_stride]);
-    const double cmax = p.nibbles ? 15.0 : 255.0;      // largest code value
-    const double shift = p.nibbles ? 0.0 : 128.0;      // the codes are staged as c - shift
-    const double ip_max = cmax * sum;                  // <code, query> of any code
-    const double t_max = 128.0 * 256.0 * p.kdim;       // |T| of any code
-    const double m_max = p.is_l2 ? cmax * cmax * p.kdim : cmax * p.kdim;  // norm_o, sum_o of any code
-    double t;
-    if (p.is_l2) {
-        // Streaming: fl(fl(fl(qm + m) - 2 R) rate), R the integer as a float (exact below 2^24).  The two sums round
-        // by at most u of their magnitude each, the product by u of itself.
-        if (!(rate > 0.0)) {
-            p.tau[q] = __float_as_uint(3.0e38F);
-            return;
+    if (merged_dists != nullptr) {
+        const float kth = merged_dists[q * k + k - 1];
+        if (kth < __builtin_inff()) {
+            const uint32_t o = float_to_ordered(kth);
+            if (o < bound[q]) {
+                bound[q] = o;
+            }
         }
-        const double reach = fabs(qm) + m_max + 2.0 * ip_max;
-        const double x_max = bd / rate * (1.0 + 4.0 * kU) + 4.0 * kU * reach;  // what qm + m - 2 ip may reach
-        // qm + m - 2 (T + shift sum) <= x_max   <=>   m - 2 T <= x_max - qm + 2 shift sum
-        t = x_max - qm + 2.0 * shift * sum;
-        // The test itself: fl(m - 2 T) in one fma against the rounded threshold.
-        t += 4.0 * kU * (m_max + 2.0 * t_max + fabs(t));
-    } else {
-        // Streaming: r = fl(fl(fl(lb fl(qm + m)) + fl(rate R)) + lb2), distance fl(1 - r).
-        const double lb = fabs(static_cast<double>(p.lb)), lb2 = fabs(static_cast<double>(p.lb2));
-        const double reach = lb * (fabs(qm) + m_max) + rate * ip_max + lb2 + 1.0 + fabs(bd);
-        const double e_stream = 8.0 * kU * reach;
-        // 1 - lb (qm + m) - rate (T + shift sum) - lb2 <= bd + e
-        //     <=>   -rate T - lb m <= bd + e - 1 + lb qm + shift rate sum + lb2
-        t = bd + e_stream - 1.0 + static_cast<double>(p.lb) * qm + shift * rate * sum + static_cast<double>(p.lb2);
-        // term_o = fl(-lb m) and the fma of the test.
-        t += 4.0 * kU * (2.0 * lb * m_max + rate * t_max + fabs(t));
     }
-    p.tau[q] = __float_as_uint(t < 3.0e38 ? (t > -3.0e38 ? static_cast<float>(t) : -3.0e38F) : 3.0e38F);
+    p.tau[q] = uniform_tau_i8(p, q, p.scal[q * kI8Scalars]);
 }
 
 struct PrefilterI8Args {
@@ -678,7 +746,9 @@ prefilter_i8_query_bytes(uint64_t nq) {
 size_t
 prefilter_i8_scalar_floats(uint64_t nq) {
     const uint64_t groups = div_up(nq, static_cast<uint64_t>(kI8Group));
-    return static_cast<size_t>(groups * kI8Group + groups);
+    // a float per padded query, one per group, then (8-byte aligned) kI8Scalars doubles per padded query
+    const uint64_t head = (groups * kI8Group + groups + 1) / 2 * 2;
+    return static_cast<size_t>(head + 2 * kI8Scalars * groups * kI8Group);
 }
 
 // Candidate lists per query (two per workgroup column) for nq queries over `span` tiles.
@@ -710,18 +780,24 @@ prefilter_i8_sub_lists(uint64_t nq, uint64_t span) {
 }
 
 // Quantizes the queries against their current bounds and collects the candidates of tiles [tile_begin, tile_end)
-// into sub_lists lists of sub_cap slots per query (sub_lists as prefilter_i8_sub_lists gives it).
+// into sub_lists lists of sub_cap slots per query (sub_lists as prefilter_i8_sub_lists gives it).  first_level: the
+// first level of a call quantizes; the later ones keep the planes and only redo the thresholds, after lowering the
+// bounds to the k-th of merged_dists (k per query; null: the bounds are up to date).
 int
 launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride, const float* qmeta,
                     uint32_t qmeta_stride, uint64_t nq, uint64_t tile_begin, uint64_t tile_end, const uint32_t* bound,
                     uint8_t* q8, float* u, uint32_t* tau, uint32_t* cand, uint32_t* cand_cnt, uint32_t sub_lists,
-                    uint32_t sub_cap, hipStream_t st) {
+                    uint32_t sub_cap, bool first_level, const float* merged_dists, uint32_t k, uint32_t* bound_rw,
+                    hipStream_t st) {
     const bool nibbles = s->kind == VSAG_AMD_KIND_SQ4_UNIFORM;
     const bool uniform = s->kind == VSAG_AMD_KIND_SQ8_UNIFORM || nibbles;
     const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
     const uint64_t nq_pad = div_up(nq, static_cast<uint64_t>(kI8Group)) * kI8Group;
     // `u` holds a float per padded query and one per group of kI8Group queries behind them (prefilter_i8_scalar_floats).
     float* ginv = u + nq_pad;
+    const uint64_t head = (nq_pad + nq_pad / kI8Group + 1) / 2 * 2;
+    double* scal = reinterpret_cast<double*>(u + head);
+    const dim3 per_query(static_cast<uint32_t>(div_up(nq, 256)));
     if (uniform) {
         UniformQuantizeArgs z{};
         z.qtab = reinterpret_cast<const uint32_t*>(qtab);
@@ -740,7 +816,12 @@ launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride
         z.q8 = q8;
         z.u = u;
         z.tau = tau;
-        hipLaunchKernelGGL(quantize_uniform_i8_kernel, dim3(static_cast<uint32_t>(nq_pad)), dim3(kWave), 0, st, z);
+        z.scal = scal;
+        if (first_level) {
+            hipLaunchKernelGGL(quantize_uniform_i8_kernel, dim3(static_cast<uint32_t>(nq_pad)), dim3(kWave), 0, st, z);
+        } else {
+            hipLaunchKernelGGL(retau_uniform_i8_kernel, per_query, dim3(256), 0, st, z, merged_dists, k, bound_rw);
+        }
     } else {
         QuantizeArgs z{};
         z.qtab = qtab;
@@ -758,10 +839,15 @@ launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride
         z.amax = u;
         z.ginv = ginv;
         z.tau = tau;
-        if (l2) {
-            hipLaunchKernelGGL(query_amax_kernel, dim3(static_cast<uint32_t>(nq_pad)), dim3(kWave), 0, st, z);
+        z.scal = scal;
+        if (first_level) {
+            if (l2) {
+                hipLaunchKernelGGL(query_amax_kernel, dim3(static_cast<uint32_t>(nq_pad)), dim3(kWave), 0, st, z);
+            }
+            hipLaunchKernelGGL(quantize_queries_i8_kernel, dim3(static_cast<uint32_t>(nq_pad)), dim3(kWave), 0, st, z);
+        } else {
+            hipLaunchKernelGGL(retau_queries_i8_kernel, per_query, dim3(256), 0, st, z, merged_dists, k, bound_rw);
         }
-        hipLaunchKernelGGL(quantize_queries_i8_kernel, dim3(static_cast<uint32_t>(nq_pad)), dim3(kWave), 0, st, z);
     }
     VA_HIP(hipGetLastError());
 

@@ -795,7 +795,8 @@ bool prefilter_supports(const vsag_amd_store* s);
 int launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t k, uint32_t S, uint64_t tile_begin,
                      uint64_t tile_end, uint32_t* bound, float* tau, uint32_t* cand, uint32_t* cand_cnt, uint32_t cap,
                      uint64_t* partial, uint32_t* partial_cnt, uint32_t nslots, uint32_t first_slot, uint32_t out_slot,
-                     uint32_t* gate, uint8_t* q8, float* q8_u, uint32_t sub_lists, uint32_t sub_cap, hipStream_t st);
+                     uint32_t* gate, uint8_t* q8, float* q8_u, uint32_t sub_lists, uint32_t sub_cap,
+                     const float* merged_dists, hipStream_t st);
 bool prefilter_i8_supports(const vsag_amd_store* s);
 size_t prefilter_i8_query_bytes(uint64_t nq);
 size_t prefilter_i8_scalar_floats(uint64_t nq);
@@ -1153,15 +1154,21 @@ flat_scan_call(const vsag_amd_store_t* s, const float* queries_dev, uint64_t nq,
             // filter it with.
             VA_TRY(launch_merge_partials(b.partial, b.partial_cnt, b.bound, slots_prefix + l, nslots, k, p.S, nq, ids_dev,
                                          dists_dev, st));
-            hipLaunchKernelGGL(tighten_bound_kernel, dim3(static_cast<uint32_t>(div_up(nq, 256))), dim3(256), 0, st,
-                               dists_dev, k, nq, b.bound);
+            // (The int8 route lowers the bounds itself from its second level on, in the launch that renews its
+            // thresholds.)
+            const bool folded = cp.int8 && !cp.rb && l > 0;
+            if (!folded) {
+                hipLaunchKernelGGL(tighten_bound_kernel, dim3(static_cast<uint32_t>(div_up(nq, 256))), dim3(256), 0, st,
+                                   dists_dev, k, nq, b.bound);
+            }
             if (!cp.int8 && !cp.rb) {
                 hipLaunchKernelGGL(fill_words2_kernel, dim3(static_cast<uint32_t>(div_up(nq, 256))), dim3(256), 0, st,
                                    b.cand_cnt, nq, static_cast<uint32_t*>(nullptr), 0);
             }
             VA_TRY(launch_prefilter(s, a, nq, k, p.S, cp.level_begin[l], cp.level_begin[l + 1], b.bound, b.tau, b.cand,
                                     b.cand_cnt, cp.cap, b.partial, b.partial_cnt, nslots, slots_prefix, slots_prefix + l,
-                                    b.gate, b.q8, b.q8_u, cp.sub_lists[l], cp.sub_cap[l], st));
+                                    b.gate, b.q8, b.q8_u, cp.sub_lists[l], cp.sub_cap[l], folded ? dists_dev : nullptr,
+                                    st));
         }
         VA_TRY(run_streaming(s, cp.rest, a, b, nq, k, nullptr, cp.prefix_tiles, s->ntiles, slots_prefix + levels, nslots,
                              b.gate, st));
