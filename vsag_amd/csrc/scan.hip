@@ -168,8 +168,24 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
         thr[t] = tl < tb ? tl : tb;
     };
 
+    // What a cold wave reads of its queries' seed rows (largest entry over this lane's share): fetched when a tile
+    // begins, looked at when its distances are done, so that the read waits under the tile's arithmetic.
+    uint32_t seed_seen[T];
     auto consume = [&](const uint4(&regs)[GROUP]) {
         const uint32_t first = cur.first();
+        if (SEED && cur.j0 == 0) {
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                seed_seen[t] = 0;
+                if (cold[t] != 0) {
+                    const uint32_t* row = f.seed + static_cast<uint64_t>(qidx[t]) * k;
+                    for (uint32_t i = lane; i < k; i += kWave) {
+                        const uint32_t v = __atomic_load_n(&row[i], __ATOMIC_RELAXED);
+                        seed_seen[t] = v > seed_seen[t] ? v : seed_seen[t];
+                    }
+                }
+            }
+        }
 #pragma unroll
         for (int u = 0; u < GROUP; ++u) {
             const uint32_t g = first + u;
@@ -193,20 +209,17 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
             if (SEED && cold[t] != 0) {
                 uint32_t* row = f.seed + static_cast<uint64_t>(qidx[t]) * k;
                 if (cold[t] == kSeedTiles) {
+                    // This wave's entry (its own first look at the row came before it, the next one will see it).
                     uint32_t m = wave_min_u32(valid ? od : 0xFFFFFFFFU);
                     lower_shared(&row[seed_slot], m, lane);
                 }
                 --cold[t];
-                uint32_t mx = 0;
-                for (uint32_t i = lane; i < k; i += kWave) {
-                    uint32_t v = __atomic_load_n(&row[i], __ATOMIC_RELAXED);
-                    mx = v > mx ? v : mx;
-                }
-                mx = wave_max_u32(mx);
+                const uint32_t mx = wave_max_u32(seed_seen[t]);
                 if (mx != 0xFFFFFFFFU) {
+                    // Every slot filled: k different codes reach mx.
                     cold[t] = 0;
-                    mx = lower_shared(&f.bound[qidx[t]], mx, lane);
-                    thr[t] = mx + 1 < thr[t] ? mx + 1 : thr[t];
+                    const uint32_t b = lower_shared(&f.bound[qidx[t]], mx, lane);
+                    thr[t] = b + 1 < thr[t] ? b + 1 : thr[t];
                 }
             }
             bool pass = valid && od < thr[t];
