@@ -32,6 +32,7 @@ struct ScanPlanIvf {
     bool chunked;             // one launch over all probe columns, seeded cold start
     bool seeded;
     bool mfma;                // probe columns behind the first go through the int8 matrix cores (ivf_i8.hip)
+    bool planes;              // ... with sq8 codes: two int8 planes per query, records rescored (prefilter_i8.hip)
 };
 
 uint64_t rabitq_query_code_size(uint32_t dim, int metric, int query_bits);
@@ -39,6 +40,20 @@ int scan_contraction_mode(const vsag_amd_store* s);
 void note_last_scan(int query_tile, uint64_t passes, uint64_t bytes_per_pass);
 bool ivf_i8_supports(const vsag_amd_store* s);
 uint32_t ivf_i8_lists_per_pair();
+// sq8 lists: the two-plane test of prefilter_i8.hip over the same work split, records rescored by prefilter.hip.
+bool ivf_sq8_i8_supports(const vsag_amd_store* s);
+size_t ivf_sq8_i8_query_bytes(uint64_t nq);
+size_t ivf_sq8_i8_scalar_floats(uint64_t nq);
+size_t ivf_sq8_i8_tau_words(uint64_t nq);
+uint32_t ivf_rescore_capacity();
+int launch_ivf_sq8_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride, const float* qmeta, uint32_t qmeta_stride,
+                      uint64_t nq, uint32_t nprobe, uint32_t p0, const uint32_t* pair_off, const uint32_t* item_off,
+                      const uint32_t* sorted_pair, const uint32_t* bound, uint32_t kcand, uint8_t* q8, float* u, uint32_t* tau,
+                      uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st);
+int launch_ivf_clear_gated(uint32_t* gate, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t* partial_cnt,
+                           const int32_t* buckets, uint32_t* gpairs, uint32_t gpairs_cap, hipStream_t st);
+int launch_ivf_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
+                       uint32_t per_pair, uint64_t* partial, uint32_t* partial_cnt, const uint32_t* bound, hipStream_t st);
 int launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
                   const uint32_t* pair_off, const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound,
                   int32_t* tq, uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, const int32_t* buckets,
@@ -863,6 +878,9 @@ struct IvfBuffers {
     uint32_t* gate;       // mfma: nq + 2 (flags, raised gates, their pairs)
     int32_t* tq;          // mfma: 2 (nq + 1)
     uint32_t* gpairs;     // mfma: pairs of gated queries, kGatedPairsCap
+    uint8_t* q8;          // sq8 lists on the matrix cores: the planes of the queries, their scalars and thresholds
+    float* q8_u;
+    uint32_t* q8_tau;
     float* res_term;      // residual lists: per pair
 };
 
@@ -917,6 +935,10 @@ plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, 
     p->mfma = !p->chunked && nprobe > 1 && scan_contraction_mode(s) >= 0 && ivf_i8_supports(s) &&
               s->residual_centroids_dev == nullptr &&
               npairs * ivf_i8_lists_per_pair() * kcand * 8 <= (8ull << 30);
+    // sq8 lists of at most 128 dimensions: the same split with the two-plane test and an exact rescoring.
+    p->planes = !p->mfma && !p->chunked && nprobe > 1 && scan_contraction_mode(s) >= 0 && ivf_sq8_i8_supports(s) &&
+                kcand <= ivf_rescore_capacity() && npairs * ivf_i8_lists_per_pair() * kcand * 8 <= (8ull << 30);
+    p->mfma = p->mfma || p->planes;
     if (p->mfma) {
         p->chunks_max = ivf_i8_lists_per_pair();
     }
@@ -947,6 +969,9 @@ carve_ivf(Carver& c, const vsag_amd_store* s, const ScanPlanIvf& p, uint64_t nq,
     b->gate = c.take<uint32_t>(p.mfma ? nq + 2 : 0);
     b->gpairs = c.take<uint32_t>(p.mfma ? kGatedPairsCap : 0);
     b->tq = c.take<int32_t>(p.mfma ? 2 * (nq + 1) : 0);  // thresholds, then (sq8_uniform) the sums of the query values
+    b->q8 = c.take<uint8_t>(p.planes ? ivf_sq8_i8_query_bytes(nq) : 0);
+    b->q8_u = c.take<float>(p.planes ? ivf_sq8_i8_scalar_floats(nq) : 0);
+    b->q8_tau = c.take<uint32_t>(p.planes ? ivf_sq8_i8_tau_words(nq) : 0);
     b->res_term = c.take<float>(s->residual_centroids_dev != nullptr ? p.npairs : 0);
     return c.used;
 }
@@ -1108,8 +1133,17 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
             // lists overflowed -- the streaming kernel's items over the same grouping.
             // ivf_i8.hip: items of 256 pairs, kIvfI8ChunkTiles, kIvfI8Chunks
             regroup(p0, p1, pairs, 256U, 32U, 4U);
-            VA_TRY(launch_ivf_i8(s, a, nq, nprobe, p0, kcand, b.pair_off, b.item_off, b.sorted_pair, b.bound, b.tq,
-                                 b.partial, b.partial_cnt, b.gate, buckets_dev, b.gpairs, kGatedPairsCap, st));
+            if (p.planes) {
+                VA_TRY(launch_ivf_sq8_i8(s, reinterpret_cast<const float*>(a.qtab), a.qstride, a.qmeta, a.qmeta_stride, nq,
+                                         nprobe, p0, b.pair_off, b.item_off, b.sorted_pair, b.bound, kcand, b.q8, b.q8_u,
+                                         b.q8_tau, b.partial, b.partial_cnt, b.gate, st));
+                VA_TRY(launch_ivf_clear_gated(b.gate, nq, nprobe, p0, b.partial_cnt, buckets_dev, b.gpairs,
+                                              kGatedPairsCap, st));
+                VA_TRY(launch_ivf_rescore(s, a, nq, nprobe, p0, kcand, p.chunks_max, b.partial, b.partial_cnt, b.bound, st));
+            } else {
+                VA_TRY(launch_ivf_i8(s, a, nq, nprobe, p0, kcand, b.pair_off, b.item_off, b.sorted_pair, b.bound, b.tq,
+                                     b.partial, b.partial_cnt, b.gate, buckets_dev, b.gpairs, kGatedPairsCap, st));
+            }
             // Few gated pairs (the usual case): one wave per pair and chunk of its list.
             IvfArgs d = v;
             d.direct = b.gpairs;

@@ -595,6 +595,18 @@ ivf_i8_supports(const vsag_amd_store* s) {
     return s->kind == VSAG_AMD_KIND_SQ4_UNIFORM && s->G <= 4 && s->nlist > 0 && s->scalar_rate > 0.0F;
 }
 
+// After a matrix-core pass over probe columns [p0, nprobe): the private lists of the queries whose gate it raised are
+// emptied and their pairs queued (see ivf_i8_clear_gated_kernel).
+int
+launch_ivf_clear_gated(uint32_t* gate, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t* partial_cnt,
+                       const int32_t* buckets, uint32_t* gpairs, uint32_t gpairs_cap, hipStream_t st) {
+    const uint64_t pairs = nq * (nprobe - p0);
+    hipLaunchKernelGGL(ivf_i8_clear_gated_kernel, dim3(static_cast<uint32_t>(div_up(pairs, 256))), dim3(256), 0, st, gate,
+                       nq, nprobe, p0, partial_cnt, buckets, gpairs, gpairs_cap);
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
 // The pairs of probe columns [p0, nprobe) are grouped by list (pair_off, sorted_pair) and item_off counts
 // workgroups per list (blocks of 256 pairs x tile chunks: offsets_kernel with T = 256, kIvfI8ChunkTiles,
 // kIvfI8Chunks); `bound` holds what the first columns left.  tq: 2 (nq + 1) words; gate: nq + 2 words, zeroed.
@@ -654,9 +666,7 @@ launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     }
     timing_end(st);
     VA_HIP(hipGetLastError());
-    hipLaunchKernelGGL(ivf_i8_clear_gated_kernel, dim3(static_cast<uint32_t>(div_up(pairs, 256))), dim3(256), 0, st, gate,
-                       nq, nprobe, p0, partial_cnt, buckets, gpairs, gpairs_cap);
-    VA_HIP(hipGetLastError());
+    VA_TRY(launch_ivf_clear_gated(gate, nq, nprobe, p0, partial_cnt, buckets, gpairs, gpairs_cap, st));
     IvfI8FinishArgs f{};
     f.partial = partial;
     f.partial_cnt = partial_cnt;

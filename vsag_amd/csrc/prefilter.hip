@@ -559,6 +559,150 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
     }
 }
 
+// Posting lists: the matrix-core pass over sq8 lists (prefilter_i8.hip, ivf_sq8_i8_kernel) leaves, per (query, list)
+// pair, per_pair private lists of tile slots in the partial lists of an ivf scan.  One wave per query turns the
+// records of probe columns [p0, nprobe) into (distance, id) keys by the streaming kernel's arithmetic, in place: the
+// records of 64 lists (or, when those hold many, of as many lists as always fit) are gathered in LDS, a lane computes
+// a record's key, and the lane that owns a list writes the keys that count back to its front.  Records of empty slots
+// and of distances beyond the query's bound are dropped.
+struct IvfRescoreArgs {
+    uint64_t* partial;
+    uint32_t* partial_cnt;
+    uint32_t k;  // capacity of a private list, at most kIvfRescoreGather
+    uint32_t nprobe, p0, per_pair;
+    const uint32_t* ids;
+    const uint32_t* bound;
+};
+
+constexpr uint32_t kIvfRescoreGather = 1024;
+
+template <int KIND, int METRIC>
+__global__ void __launch_bounds__(64)
+ivf_rescore_kernel(ScanArgs a, IvfRescoreArgs r) {
+    __shared__ uint32_t where[kIvfRescoreGather];
+    __shared__ uint64_t fkey[kIvfRescoreGather];
+    const uint32_t lane = threadIdx.x;
+    const uint32_t q = blockIdx.x;
+    const uint32_t lists = (r.nprobe - r.p0) * r.per_pair;
+    const uint64_t base = (static_cast<uint64_t>(q) * r.nprobe + r.p0) * r.per_pair;
+    uint64_t* mine = r.partial + base * r.k;
+    uint32_t* counts = r.partial_cnt + base;
+    const uint32_t bound = as_const(r.bound)[q];
+    const uint32_t qidx[1] = {q};
+    const QueryRows<1> qrows = query_rows<1>(a, qidx);
+    uint32_t piece = kIvfRescoreGather / r.k;
+    piece = piece > kWave ? kWave : piece;
+    constexpr uint64_t kDropped = ~0ULL;
+    auto round = [&](uint32_t g, uint32_t c) {
+        // c = records of this lane's list g that take part (0: none).
+        uint32_t incl = c;
+        for (int off = 1; off < 64; off <<= 1) {
+            const uint32_t o = __shfl_up(incl, off);
+            incl += lane >= static_cast<uint32_t>(off) ? o : 0U;
+        }
+        const uint32_t sum = __shfl(incl, 63);
+        if (sum == 0) {
+            return;
+        }
+        const uint32_t at = incl - c;
+        for (uint32_t i = 0; i < c; ++i) {
+            where[at + i] = g * r.k + i;
+        }
+        wave_lds_fence();
+        for (uint32_t e0 = 0; e0 < sum; e0 += kWave) {
+            const bool have = e0 + lane < sum;
+            const uint32_t slot = have ? static_cast<uint32_t>(mine[where[e0 + lane]]) : 0U;
+            const uint64_t tile = slot >> 6;
+            const uint32_t ln = slot & 63;
+            Acc<KIND, 1> acc;
+            acc_reset(acc);
+            constexpr uint32_t kAhead = KIND == VSAG_AMD_KIND_SQ8 && METRIC == VSAG_AMD_METRIC_L2 ? 2 : 4;
+            for (uint32_t j0 = 0; j0 < a.G; j0 += kAhead) {
+                uint4 c4[kAhead];
+#pragma unroll
+                for (uint32_t u = 0; u < kAhead; ++u) {
+                    const uint32_t j = j0 + u < a.G ? j0 + u : a.G - 1;
+                    c4[u] = a.tiles[(tile * a.G + j) * kWave + ln];
+                }
+#pragma unroll
+                for (uint32_t u = 0; u < kAhead; ++u) {
+                    if (j0 + u < a.G) {
+                        accumulate_granule<KIND, METRIC, 1>(a, qrows, j0 + u, c4[u], acc);
+                    }
+                }
+            }
+            float d[1];
+            finish_distances<KIND, METRIC, 1>(a, qidx, slot, acc, d);
+            if (have) {
+                const uint32_t id = as_const(r.ids)[slot];
+                fkey[e0 + lane] =
+                    id != VSAG_AMD_INVALID_ID && float_to_ordered(d[0]) <= bound ? make_key(d[0], id) : kDropped;
+            }
+        }
+        wave_lds_fence();
+        if (c != 0) {
+            uint32_t kept = 0;
+            for (uint32_t i = 0; i < c; ++i) {
+                const uint64_t key = fkey[at + i];
+                if (key != kDropped) {
+                    mine[static_cast<uint64_t>(g) * r.k + kept++] = key;
+                }
+            }
+            counts[g] = kept;
+        }
+        wave_lds_fence();  // the next round writes the same LDS
+    };
+    for (uint32_t g0 = 0; g0 < lists; g0 += kWave) {
+        const uint32_t g = g0 + lane;
+        const uint32_t c = g < lists ? as_const(counts)[g] : 0U;
+        uint32_t total = c;
+        for (int off = 32; off > 0; off >>= 1) {
+            total += __shfl_xor(total, off);
+        }
+        if (total == 0) {
+            continue;
+        }
+        if (total <= kIvfRescoreGather) {
+            round(g, c);
+        } else {
+            for (uint32_t b0 = 0; b0 < kWave; b0 += piece) {
+                round(g, lane >= b0 && lane < b0 + piece ? c : 0U);
+            }
+        }
+    }
+}
+
+uint32_t
+ivf_rescore_capacity() {
+    return kIvfRescoreGather;
+}
+
+int
+launch_ivf_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
+                   uint32_t per_pair, uint64_t* partial, uint32_t* partial_cnt, const uint32_t* bound, hipStream_t st) {
+    if (s->kind != VSAG_AMD_KIND_SQ8 || kcand > kIvfRescoreGather || s->ids_dev == nullptr) {
+        return fail(VSAG_AMD_INVALID_ARGUMENT, "rescoring of list records: sq8 lists with kcand <= %u only",
+                    kIvfRescoreGather);
+    }
+    IvfRescoreArgs r{};
+    r.partial = partial;
+    r.partial_cnt = partial_cnt;
+    r.k = kcand;
+    r.nprobe = nprobe;
+    r.p0 = p0;
+    r.per_pair = per_pair;
+    r.ids = s->ids_dev;
+    r.bound = bound;
+    const dim3 grid(static_cast<uint32_t>(nq));
+    if (s->metric == VSAG_AMD_METRIC_L2) {
+        hipLaunchKernelGGL((ivf_rescore_kernel<VSAG_AMD_KIND_SQ8, VSAG_AMD_METRIC_L2>), grid, dim3(kWave), 0, st, a, r);
+    } else {
+        hipLaunchKernelGGL((ivf_rescore_kernel<VSAG_AMD_KIND_SQ8, VSAG_AMD_METRIC_IP>), grid, dim3(kWave), 0, st, a, r);
+    }
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
 // ------------------------------------------------------------------ host side
 bool prefilter_rb_supports(const vsag_amd_store* s);
 int launch_prefilter_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint64_t tile_begin, uint64_t tile_end,

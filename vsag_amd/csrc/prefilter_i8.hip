@@ -21,6 +21,7 @@
 // for the whole kernel and meets every 64-code storage tile the workgroup walks, which is staged in LDS in the
 // tile's own granule-major order -- that order is the operand order of the matrix instruction (lane % 32 = code,
 // lane / 32 = which 16 of the 32 dimensions of a step), so staging is a plain copy.
+#include "distance.h"
 #include "store.h"
 #include "topk.h"
 
@@ -734,6 +735,387 @@ prefilter_i8_supports(const vsag_amd_store* s) {
     }
     return (s->kind == VSAG_AMD_KIND_SQ8 || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) && s->nlist == 0 && s->pf_term != nullptr &&
            s->dpad <= kI8Dims && s->G <= 8;
+}
+
+size_t prefilter_i8_query_bytes(uint64_t nq);
+size_t prefilter_i8_scalar_floats(uint64_t nq);
+
+// ---- sq8 posting lists against large batches --------------------------------------------------------------------
+// The same two-plane test over the (query, list) pairs of an ivf search that the streaming kernel has already given a
+// bound (the probe columns behind the nearest list, see ivf_i8.hip for the work split this kernel shares: a
+// workgroup = a chunk of a list's tiles x up to 256 of the pairs that probe the list, four waves of 64 pairs).  The
+// queries of a workgroup are whatever queries probe the list, so they cannot share a scale by groups of neighbours:
+// the whole batch shares one (spread_amax_kernel), and 1 / (2 s2) is one number.  What passes is recorded as a tile
+// slot in the private list of (pair, chunk, lane / 32) -- the lists the streaming kernel's partial results use -- and
+// turned into a (distance, id) key by ivf_rescore_kernel (prefilter.hip).
+constexpr uint32_t kIvfSq8Pairs = 256;
+constexpr uint32_t kIvfSq8ChunkTiles = 32;  // as ivf_i8.hip: kIvfI8ChunkTiles, kIvfI8Chunks
+constexpr uint32_t kIvfSq8Chunks = 4;
+
+// amax[q] = the largest amax of the batch, for every row (one workgroup).
+__global__ void __launch_bounds__(1024)
+spread_amax_kernel(float* amax, uint64_t n) {
+    __shared__ float part[16];
+    float m = 0.0F;
+    for (uint64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        m = fmaxf(m, amax[i]);
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        m = fmaxf(m, __shfl_xor(m, off));
+    }
+    if ((threadIdx.x & 63) == 0) {
+        part[threadIdx.x >> 6] = m;
+    }
+    __syncthreads();
+    m = 0.0F;
+    for (uint32_t w = 0; w < blockDim.x / kWave; ++w) {
+        m = fmaxf(m, part[w]);
+    }
+    for (uint64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        amax[i] = m;
+    }
+}
+
+struct IvfSq8Args {
+    const uint4* tiles;
+    uint32_t G;
+    const float* term;           // per slot |y|^2 (l2)
+    const uint32_t* list_tile;   // 2 nlist: first tile and end of the used tiles of every list
+    const uint32_t* pair_off;    // nlist + 1
+    const uint32_t* item_off;    // nlist + 1: workgroups per list, prefix sums
+    const uint32_t* sorted_pair; // pair index (q * nprobe + p) grouped by list
+    uint32_t nlist, nprobe;
+    uint32_t dummy_query;        // a padding row of the query table: zero operands, a threshold nothing meets
+    const uint4* q8;             // [query][plane][granule]
+    const uint32_t* tau;         // per query
+    const float* ginv;           // 1 / (2 s2) of the batch (l2)
+    uint32_t k;                  // capacity of a private list
+    uint64_t* partial;           // [pair][chunk][lane / 32][k]: tile slots
+    uint32_t* partial_cnt;       // [pair][chunk][lane / 32]
+    uint32_t* gate;              // per query: raised when one of its lists overflowed; gate[dummy_query] counts them
+};
+
+template <int TEST>
+__global__ void __launch_bounds__(256, 2)
+ivf_sq8_i8_kernel(IvfSq8Args p) {
+    __shared__ I8Stage stage[2];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    const uint32_t wave = tid >> 6;
+    const uint32_t half = lane >> 5;
+    const uint32_t l32 = lane & 31;
+    const uint32_t item = blockIdx.x;
+    cu32_p ioff = as_const(p.item_off);
+    if (item >= ioff[p.nlist]) {
+        return;  // the whole workgroup
+    }
+    uint32_t lo_b = 0, hi_b = p.nlist;
+    while (hi_b - lo_b > 1) {
+        const uint32_t mid = (lo_b + hi_b) >> 1;
+        if (ioff[mid] <= item) {
+            lo_b = mid;
+        } else {
+            hi_b = mid;
+        }
+    }
+    const uint32_t b = lo_b;
+    const uint32_t list_begin = as_const(p.list_tile)[2 * b], list_end = as_const(p.list_tile)[2 * b + 1];
+    uint32_t chunks = (list_end - list_begin + kIvfSq8ChunkTiles - 1) / kIvfSq8ChunkTiles;
+    chunks = chunks < kIvfSq8Chunks ? chunks : kIvfSq8Chunks;
+    const uint32_t per = chunks != 0 ? (list_end - list_begin + chunks - 1) / chunks : 0;
+    const uint32_t chunk = chunks != 0 ? (item - ioff[b]) % chunks : 0;
+    const uint32_t group = chunks != 0 ? (item - ioff[b]) / chunks : 0;
+    uint32_t tile_begin = list_begin + chunk * per;
+    tile_begin = tile_begin < list_end ? tile_begin : list_end;
+    const uint32_t tile_end = tile_begin + per < list_end ? tile_begin + per : list_end;
+    const uint32_t pbeg = as_const(p.pair_off)[b] + group * kIvfSq8Pairs + wave * kWave;
+    const uint32_t pend = as_const(p.pair_off)[b + 1];
+    const bool active = pbeg < pend;
+    const uint32_t nstages = (tile_end - tile_begin + kI8StageTiles - 1) / kI8StageTiles;
+    if (nstages == 0) {
+        return;
+    }
+    constexpr bool kTerm = TEST == kI8TestIntTerm;
+
+    intx4 qh[2][4], ql[2][4];
+    uint32_t tau[2], qidx[2];
+    uint32_t ncand[2] = {0, 0};
+    uint64_t my_list[2];
+    bool live[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint32_t idx = pbeg + 32 * j + l32;
+        live[j] = idx < pend;
+        const uint32_t pair = live[j] ? as_const(p.sorted_pair)[idx] : 0U;
+        qidx[j] = live[j] ? pair / p.nprobe : p.dummy_query;
+        const uint4* rowp = p.q8 + static_cast<uint64_t>(qidx[j]) * (kI8QueryBytes / 16);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const uint4 hv = rowp[2 * s + half];
+            const uint4 lv = rowp[8 + 2 * s + half];
+            qh[j][s] = intx4{static_cast<int>(hv.x), static_cast<int>(hv.y), static_cast<int>(hv.z),
+                             static_cast<int>(hv.w)};
+            ql[j][s] = intx4{static_cast<int>(lv.x), static_cast<int>(lv.y), static_cast<int>(lv.z),
+                             static_cast<int>(lv.w)};
+        }
+        tau[j] = live[j] ? p.tau[qidx[j]] : 0x7FFFFFFFU;
+        my_list[j] = (static_cast<uint64_t>(pair) * kIvfSq8Chunks + chunk) * 2 + half;
+    }
+    const float ginv = kTerm ? p.ginv[0] : 0.0F;
+
+    uint4 regs[kI8StageTiles][2];
+    float my_term[kI8StageTiles];
+    auto fetch = [&](uint32_t sg) {
+#pragma unroll
+        for (int tt = 0; tt < kI8StageTiles; ++tt) {
+            const uint32_t tile = tile_begin + sg * kI8StageTiles + tt;
+            const bool real = tile < tile_end;
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const uint32_t j = wave + 4 * r;
+                regs[tt][r] = make_uint4(0x80808080U, 0x80808080U, 0x80808080U, 0x80808080U);
+                if (real && j < p.G) {
+                    regs[tt][r] = p.tiles[(static_cast<uint64_t>(tile) * p.G + j) * kWave + lane];
+                }
+            }
+            if constexpr (kTerm) {
+                my_term[tt] = 0.0F;
+                if (wave == 0) {
+                    // Slots without a code hold zero codes: their term is that of the zero vector, and the rescoring
+                    // leaves them out by their id.
+                    my_term[tt] = real ? p.term[static_cast<uint64_t>(tile) * kWave + lane] : __builtin_inff();
+                }
+            }
+        }
+    };
+    auto park = [&](I8Stage& st) {
+#pragma unroll
+        for (int tt = 0; tt < kI8StageTiles; ++tt) {
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const uint4 v = regs[tt][r];
+                st.codes[tt][(wave + 4 * r) * kWave + lane] =
+                    make_uint4(v.x ^ 0x80808080U, v.y ^ 0x80808080U, v.z ^ 0x80808080U, v.w ^ 0x80808080U);
+            }
+            if constexpr (kTerm) {
+                if (wave == 0) {
+                    const float x = my_term[tt] * ginv;
+                    const int32_t io = x >= kI8TermClamp ? static_cast<int32_t>(kI8TermClamp) : __float2int_rn(x);
+                    st.term[tt][lane] = __int_as_float(-io);
+                }
+            }
+        }
+    };
+
+    constexpr int kBlocks = 4 * kI8StageTiles;
+    fetch(0);
+    park(stage[0]);
+    __syncthreads();
+    uint32_t cur = 0;
+    for (uint32_t sg = 0; sg < nstages; ++sg) {
+        if (sg + 1 < nstages) {
+            fetch(sg + 1);
+        }
+        if (active) {
+            const I8Stage& st = stage[cur];
+            const uint64_t slot0 = (static_cast<uint64_t>(tile_begin) + sg * kI8StageTiles) * kWave;
+            intx16 hi[2], lo[2];
+            intx4 av[2][4];
+            float tm[2][16];
+            auto read_row = [&](int r) {
+                const int tt = r >> 1, i = r & 1;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const uint4 c = st.codes[tt][(2 * s + half) * kWave + 32 * i + l32];
+                    av[r & 1][s] = intx4{static_cast<int>(c.x), static_cast<int>(c.y), static_cast<int>(c.z),
+                                         static_cast<int>(c.w)};
+                }
+                if constexpr (kTerm) {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const float4 v = *reinterpret_cast<const float4*>(&st.term[tt][32 * i + 8 * g + 4 * half]);
+                        tm[r & 1][4 * g] = v.x;
+                        tm[r & 1][4 * g + 1] = v.y;
+                        tm[r & 1][4 * g + 2] = v.z;
+                        tm[r & 1][4 * g + 3] = v.w;
+                    }
+                }
+            };
+            auto multiply = [&](int blk, intx16& h, intx16& l) {
+                const int r = blk >> 1, j = blk & 1;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    h[e] = 0;
+                    l[e] = kTerm ? __float_as_int(tm[r & 1][e]) : 0;
+                }
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    h = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[r & 1][s], qh[j][s], h, 0, 0, 0);
+                    l = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[r & 1][s], ql[j][s], l, 0, 0, 0);
+                }
+            };
+            auto judged = [&](int blk, int e) { return (hi[blk & 1][e] << 8) + lo[blk & 1][e]; };
+            read_row(0);
+            multiply(0, hi[0], lo[0]);
+#pragma unroll
+            for (int blk = 0; blk < kBlocks; ++blk) {
+                const int r = blk >> 1, j = blk & 1;
+                const bool reads = j == 0 && blk + 2 < kBlocks;
+                if (reads) {
+                    read_row(r + 1);
+                }
+                if (blk + 1 < kBlocks) {
+                    multiply(blk + 1, hi[(blk + 1) & 1], lo[(blk + 1) & 1]);
+                }
+                int32_t gbest[4];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    gbest[g] = max(max(max(judged(blk, 4 * g), judged(blk, 4 * g + 1)), judged(blk, 4 * g + 2)),
+                                   judged(blk, 4 * g + 3));
+                }
+                const bool hit = max(max(max(gbest[0], gbest[1]), gbest[2]), gbest[3]) >= static_cast<int32_t>(tau[j]);
+                const uint64_t any = __ballot(hit);
+                if (blk + 1 < kBlocks) {
+                    if (reads) {
+                        __builtin_amdgcn_sched_group_barrier(0x100, kTerm ? 8 : 4, 0);
+                    }
+#pragma unroll
+                    for (int m = 0; m < 8; ++m) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+                    }
+                }
+                if (any != 0) {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        if (__ballot(gbest[g] >= static_cast<int32_t>(tau[j])) == 0) {
+                            continue;
+                        }
+#pragma unroll
+                        for (int e = 4 * g; e < 4 * g + 4; ++e) {
+                            const bool pass = judged(blk, e) >= static_cast<int32_t>(tau[j]) && live[j];
+                            if (__ballot(pass) != 0 && pass) {
+                                const uint64_t slot = slot0 + 32 * r + 8 * (e >> 2) + 4 * half + (e & 3);
+                                if (ncand[j] < p.k) {
+                                    p.partial[my_list[j] * p.k + ncand[j]] = slot;
+                                }
+                                ++ncand[j];
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        if (sg + 1 < nstages) {
+            park(stage[cur ^ 1]);
+        }
+        __syncthreads();
+        cur ^= 1;
+    }
+    if (active) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            if (live[j]) {
+                p.partial_cnt[my_list[j]] = ncand[j] < p.k ? ncand[j] : p.k;
+                if (ncand[j] > p.k) {
+                    if (atomicExch(&p.gate[qidx[j]], 1U) == 0U) {
+                        atomicAdd(&p.gate[p.dummy_query], 1U);
+                    }
+                }
+            }
+        }
+    }
+}
+
+bool
+ivf_sq8_i8_supports(const vsag_amd_store* s) {
+    return s->kind == VSAG_AMD_KIND_SQ8 && s->nlist > 0 && s->G <= 8 && s->dpad <= kI8Dims && s->pf_term != nullptr &&
+           s->pf_ymax != nullptr && s->residual_centroids_dev == nullptr;
+}
+
+// Bytes of the query planes, floats of the scalars and words of the thresholds for nq queries and one padding row.
+size_t
+ivf_sq8_i8_query_bytes(uint64_t nq) {
+    return prefilter_i8_query_bytes(nq + 1);
+}
+
+size_t
+ivf_sq8_i8_scalar_floats(uint64_t nq) {
+    return prefilter_i8_scalar_floats(nq + 1);
+}
+
+size_t
+ivf_sq8_i8_tau_words(uint64_t nq) {
+    return static_cast<size_t>(div_up(nq + 1, static_cast<uint64_t>(kI8Group)) * kI8Group);
+}
+
+// Quantizes the queries against their bounds (one scale for the batch) and collects, for the pairs of probe columns
+// [p0, nprobe) grouped by list (pair_off, sorted_pair; item_off as for ivf_i8.hip), the tile slots whose distance may
+// still matter: private list (pair * 8 + chunk * 2 + lane / 32) of kcand records in `partial`, counts in partial_cnt
+// (zero before).  gate: nq + 2 words as in ivf_i8.hip.
+int
+launch_ivf_sq8_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride, const float* qmeta, uint32_t qmeta_stride,
+                  uint64_t nq, uint32_t nprobe, uint32_t p0, const uint32_t* pair_off, const uint32_t* item_off,
+                  const uint32_t* sorted_pair, const uint32_t* bound, uint32_t kcand, uint8_t* q8, float* u, uint32_t* tau,
+                  uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st) {
+    const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
+    const uint64_t nq_pad = ivf_sq8_i8_tau_words(nq);
+    float* ginv = u + nq_pad;
+    const uint64_t head = (nq_pad + nq_pad / kI8Group + 1) / 2 * 2;
+    QuantizeArgs z{};
+    z.qtab = qtab;
+    z.qstride = qstride;
+    z.kdim = s->dpad;
+    z.scale = l2 ? s->scale_dev : nullptr;
+    z.qmeta = l2 ? nullptr : qmeta;
+    z.qmeta_stride = qmeta_stride;
+    z.is_l2 = l2 ? 1 : 0;
+    z.bound = bound;
+    z.ymax_bits = s->pf_ymax;
+    z.nq = nq;
+    z.nq_pad = nq_pad;
+    z.q8 = q8;
+    z.amax = u;
+    z.ginv = ginv;
+    z.tau = tau;
+    z.scal = reinterpret_cast<double*>(u + head);
+    if (l2) {
+        hipLaunchKernelGGL(query_amax_kernel, dim3(static_cast<uint32_t>(nq_pad)), dim3(kWave), 0, st, z);
+        hipLaunchKernelGGL(spread_amax_kernel, dim3(1), dim3(1024), 0, st, u, nq_pad);
+    }
+    hipLaunchKernelGGL(quantize_queries_i8_kernel, dim3(static_cast<uint32_t>(nq_pad)), dim3(kWave), 0, st, z);
+    VA_HIP(hipGetLastError());
+    IvfSq8Args p{};
+    p.tiles = s->tiles;
+    p.G = s->G;
+    p.term = s->pf_term;
+    p.list_tile = s->list_tile_dev;
+    p.pair_off = pair_off;
+    p.item_off = item_off;
+    p.sorted_pair = sorted_pair;
+    p.nlist = s->nlist;
+    p.nprobe = nprobe;
+    p.dummy_query = static_cast<uint32_t>(nq);
+    p.q8 = reinterpret_cast<const uint4*>(q8);
+    p.tau = tau;
+    p.ginv = ginv;
+    p.k = kcand;
+    p.partial = partial;
+    p.partial_cnt = partial_cnt;
+    p.gate = gate;
+    const uint64_t pairs = nq * (nprobe - p0);
+    const uint64_t max_items =
+        (div_up(pairs, static_cast<uint64_t>(kIvfSq8Pairs)) + std::min<uint64_t>(s->nlist, pairs)) * kIvfSq8Chunks;
+    const dim3 grid(static_cast<uint32_t>(max_items));
+    timing_begin(st);
+    if (l2) {
+        hipLaunchKernelGGL(ivf_sq8_i8_kernel<kI8TestIntTerm>, grid, dim3(256), 0, st, p);
+    } else {
+        hipLaunchKernelGGL(ivf_sq8_i8_kernel<kI8TestInt>, grid, dim3(256), 0, st, p);
+    }
+    timing_end(st);
+    VA_HIP(hipGetLastError());
+    return 0;
 }
 
 // Bytes of the quantized query table for nq queries.

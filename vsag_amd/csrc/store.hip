@@ -565,6 +565,11 @@ drop_lists(vsag_amd_store* s) {
             VA_HIP(hipFree(p));
         }
     }
+    if (s->pf_term_slots != 0 && s->pf_term != nullptr) {
+        VA_HIP(hipFree(s->pf_term));
+        s->pf_term = nullptr;
+    }
+    s->pf_term_slots = 0;
     s->list_sizes_dev = nullptr;
     s->tiles = nullptr;
     s->meta = nullptr;
@@ -777,6 +782,22 @@ append_to_lists(vsag_amd_store* s, const uint8_t* codes_dev, const int32_t* labe
     VA_HIP(hipStreamSynchronize(st));
     s->ntiles = used;
     s->n += n;
+    // The per-slot terms of the int8 pass over sq8 lists (ivf_i8.hip): recomputed over the whole buffer, which costs a
+    // pass over the codes (0.4 ms for ten million of them) against the classification and encoding an append has
+    // behind it already.
+    if (s->kind == VSAG_AMD_KIND_SQ8 && s->pf_ymax != nullptr && s->dpad <= 128 && s->residual_centroids_dev == nullptr) {
+        const uint64_t slots = s->cap_tiles * kWave;
+        if (s->pf_term == nullptr || s->pf_term_slots < slots) {
+            if (s->pf_term != nullptr) {
+                VA_HIP(hipFree(s->pf_term));
+                s->pf_term = nullptr;
+            }
+            VA_HIP(hipMalloc(&s->pf_term, slots * sizeof(float)));
+            s->pf_term_slots = slots;
+        }
+        VA_TRY(launch_code_terms(s, 0, slots, st));
+        VA_HIP(hipStreamSynchronize(st));
+    }
     return 0;
 }
 
