@@ -489,10 +489,12 @@ def run_c4(env):
     args, capi, lib = env.args, env.capi, env.lib
     n, d, nq, k = args.n or 10000000, args.dim or 128, args.nq or 10000, args.k
     nlist, nprobe, kcand = args.nlist or 4096, 64, 100
-    # --list-codes sq8_uniform: the same search over sq8_uniform lists (a byte per dimension)
-    bits = 8 if args.list_codes == "sq8_uniform" else 4
-    kind = capi.KIND_SQ8_UNIFORM if bits == 8 else capi.KIND_SQ4_UNIFORM
-    kind_name = "sq8_uniform" if bits == 8 else "sq4_uniform"
+    # --list-codes sq8_uniform / sq8: the same search over lists of a byte per dimension (one range for all
+    # dimensions / a range per dimension)
+    bits = 4 if args.list_codes == "sq4_uniform" else 8
+    per_dim = args.list_codes == "sq8"
+    kind = capi.KIND_SQ8 if per_dim else capi.KIND_SQ8_UNIFORM if bits == 8 else capi.KIND_SQ4_UNIFORM
+    kind_name = args.list_codes
     means = mt(315).random((10000, d), dtype=np.float32)
     x_dev = env.buf(n * d * 4)
     pick = np.sort(mt(7).choice(n, nlist, replace=False))
@@ -517,15 +519,22 @@ def run_c4(env):
     capi.check(lib.vsag_amd_kmeans_assign(x_dev.ptr, n, d, cent.ptr, nlist, labels.ptr, None, None, ws.ptr, wsb, None))
     ws.free()
     bounds = env.buf(8)
+    lb_dev, diff_dev = env.buf(d * 4), env.buf(d * 4)
     wsb = lib.vsag_amd_sq_train_workspace_bytes(ns, d, 0)
     ws = env.buf(wsb)
-    capi.check(lib.vsag_amd_sq_train_uniform(x_dev.ptr, ns, d, bits, capi.METRIC_L2, capi.SQ_TRAIN_TRUNC_BOUND, 0.05, 0,
-                                             bounds.ptr, ws.ptr, wsb, None))
-    ws.free()
     cs = int(lib.vsag_amd_code_size(kind, capi.METRIC_L2, d, 0))
     codes = env.buf(n * cs)
-    capi.check(lib.vsag_amd_squ_encode(x_dev.ptr, n, d, bits, capi.METRIC_L2, bounds.ptr, codes.ptr, None))
-    lists = env.make_store(kind, capi.METRIC_L2, d, bounds=bounds)
+    if per_dim:
+        capi.check(lib.vsag_amd_sq_train(x_dev.ptr, ns, d, 8, capi.METRIC_L2, capi.SQ_TRAIN_TRUNC_BOUND, 0.05, 0,
+                                         lb_dev.ptr, diff_dev.ptr, ws.ptr, wsb, None))
+        capi.check(lib.vsag_amd_sq_encode(x_dev.ptr, n, d, 8, capi.METRIC_L2, lb_dev.ptr, diff_dev.ptr, codes.ptr, None))
+        lists = env.make_store(kind, capi.METRIC_L2, d, lb=lb_dev, diff=diff_dev)
+    else:
+        capi.check(lib.vsag_amd_sq_train_uniform(x_dev.ptr, ns, d, bits, capi.METRIC_L2, capi.SQ_TRAIN_TRUNC_BOUND, 0.05,
+                                                 0, bounds.ptr, ws.ptr, wsb, None))
+        capi.check(lib.vsag_amd_squ_encode(x_dev.ptr, n, d, bits, capi.METRIC_L2, bounds.ptr, codes.ptr, None))
+        lists = env.make_store(kind, capi.METRIC_L2, d, bounds=bounds)
+    ws.free()
     capi.check(lib.vsag_amd_store_set_lists(lists, codes.ptr, labels.ptr, n, nlist, None))
     cstore = env.make_store(capi.KIND_FP32, capi.METRIC_L2, d)
     capi.check(lib.vsag_amd_store_append(cstore, cent.ptr, nlist, None))
@@ -594,11 +603,15 @@ def run_c4(env):
         sample = min(nq, 16 * threads)
         hcodes = codes.to_numpy(np.uint8, (n, cs))
         hlabels = labels.to_numpy(np.int32, (n,))
-        hb = bounds.to_numpy(np.float32, (2,))
         offsets, order = orc.ivf_build_lists(hlabels, nlist)
         posting = hcodes[order]
-        okind = orc.SQ8U if bits == 8 else orc.SQ4U
-        qcodes = orc.squ_encode(q[:sample], bits, hb[0], hb[1], orc.L2)
+        if per_dim:
+            hb = (lb_dev.to_numpy(np.float32, (d,)), diff_dev.to_numpy(np.float32, (d,)))
+            okind, qcodes = orc.SQ8, q[:sample]
+        else:
+            hb = bounds.to_numpy(np.float32, (2,))
+            okind = orc.SQ8U if bits == 8 else orc.SQ4U
+            qcodes = orc.squ_encode(q[:sample], bits, hb[0], hb[1], orc.L2)
         orc.ivf_scan(okind, orc.L2, d, posting, offsets, order, qcodes[:threads], b[:threads], kcand,
                      lb=hb[0], diff=hb[1], threads=threads)
         t0 = time.perf_counter()
@@ -620,6 +633,7 @@ def run_c4(env):
                          "query with the strict-< heap) on the same %s codes, OpenMP over queries; rerank in "
                          "fp64 on the host" % (sample, nq, nprobe, kind_name),
                "candidate_distances_bit_equal": bool(np.array_equal(cds.view(np.uint32), gcd.view(np.uint32))),
+               "candidate_distances_max_abs_difference": float(np.abs(cds.astype(np.float64) - gcd).max()),
                "candidate_overlap_with_gpu": float(np.mean([len(set(a) & set(bb)) / float(kcand)
                                                             for a, bb in zip(cids, gcand)])),
                "topk_overlap_with_gpu": float(np.mean([len(set(a) & set(bb)) / float(k)
@@ -651,13 +665,15 @@ def run_c4(env):
                 # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this launch: profiles/ivf_i8_sq4u_c4.md
                 "traffic": 491061.0 * 2.00 * 1024 + 73550.7 * 1024
                 if (n, d, nq, k, nlist, bits) == (10000000, 128, 10000, 10, 4096, 4) else None,
-                "kernel": "ivf_i8_kernel<%s> (int8 MFMA, probe columns 1..%d)" % (kind_name, nprobe - 1), "kernel_ms": kms,
+                "kernel": "%s<%s> (int8 MFMA, probe columns 1..%d)" % ("ivf_sq8_i8_kernel" if per_dim else "ivf_i8_kernel",
+                                                                        kind_name, nprobe - 1), "kernel_ms": kms,
                 "ops_per_launch": ops, "distance_evaluations_per_launch": float(rest),
                 "distance_evaluations_per_second": float(rest) / (kms * 1e-3)}
-    return env.base_line("QPS @ recall@10 (IVF %s, 10M x 128)" % ("SQ4-uniform" if bits == 4 else "SQ8-uniform"),
-                         "queries/s", nq / sec, sec, "u%d codes, i32 dot" % bits,
+    return env.base_line("QPS @ recall@10 (IVF %s, 10M x 128)" % {"sq4_uniform": "SQ4-uniform", "sq8_uniform": "SQ8-uniform",
+                                                                  "sq8": "SQ8"}[kind_name],
+                         "queries/s", nq / sec, sec, "u8 codes x f32 scale, f32 (pre-selection: i8 x i8, i32 sums)" if per_dim else "u%d codes, i32 dot" % bits,
                          "configs[3]%s: IVF search, N=%d, d=%d, nlist=%d, nprobe=%d, rerank %d, %d queries, k=%d"
-                         % ("" if bits == 4 else " with sq8_uniform lists", n, d, nlist, nprobe, kcand, nq, k),
+                         % ("" if bits == 4 else " with %s lists" % kind_name, n, d, nlist, nprobe, kcand, nq, k),
                          {"recall_at_10": rec, "build_seconds": t_build, "scanned_codes_per_query": float(scanned) / nq,
                           "bytes_per_scanned_code": cs + 4, "single_query": single,
                           "list_sizes": {"mean": float(sizes.mean()), "max": int(sizes.max()), "min": int(sizes.min()),
@@ -799,7 +815,7 @@ def main():
     ap.add_argument("--chunks", type=int, default=0, help="base chunk override (0 = library default)")
     ap.add_argument("--contraction", type=int, default=0, choices=[-1, 0, 1],
                     help="matrix-core path of the flat scans: -1 never, 0 library default, 1 whenever supported")
-    ap.add_argument("--list-codes", default="sq4_uniform", choices=["sq4_uniform", "sq8_uniform"],
+    ap.add_argument("--list-codes", default="sq4_uniform", choices=["sq4_uniform", "sq8_uniform", "sq8"],
                     help="c4 only: the quantizer of the posting lists (configs[3] names sq4_uniform)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-recall", action="store_true", help="skip the recall check")
