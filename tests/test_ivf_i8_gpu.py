@@ -1,4 +1,4 @@
-"""Large batches on sq4_uniform (and, l2, sq8_uniform) posting lists: the probe columns behind the first go through the
+"""Large batches on sq4_uniform and sq8_uniform posting lists: the probe columns behind the first go through the
 int8 matrix cores.  The integer test selects exactly what the streaming kernel would admit and the distances are formed by the
 same operations, so ids and distance bits must equal the streaming scan's (and the checker's distances)."""
 import numpy as np
@@ -84,20 +84,24 @@ def test_missing_buckets_and_ragged_lists(lib):
     st.destroy()
 
 
+@pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("metric", [orc.IP, orc.COSINE])
-@pytest.mark.parametrize("n,d,nlist,nq,nprobe,kcand", [(60000, 128, 64, 2100, 16, 100), (30000, 100, 37, 4500, 8, 10)])
-def test_inner_product_and_cosine_columns_equal_streaming(lib, metric, n, d, nlist, nq, nprobe, kcand):
+@pytest.mark.parametrize("n,d,nlist,nq,nprobe,kcand", [(60000, 128, 64, 2100, 16, 100), (30000, 100, 37, 4500, 8, 10),
+                                                       (20000, 7, 16, 9000, 4, 5)])
+def test_inner_product_and_cosine_columns_equal_streaming(lib, bits, metric, n, d, nlist, nq, nprobe, kcand):
     """No integer form for these metrics: a float threshold with every rounding charged against it, then the
-    streaming kernel's own operations on what passes."""
-    x, q, cent, labels, codes, (l, dd), st = _case(n + d + metric, n, d, nlist, nq, metric=metric)
+    streaming kernel's own operations on what passes.  Byte codes (sq8_uniform): the same test on the product of the
+    centred operands."""
+    x, q, cent, labels, codes, (l, dd), st = _case(n + d + metric, n, d, nlist, nq, metric=metric, bits=bits)
     buckets, _ = orc.ivf_route(cent, q, nprobe)
     buckets = buckets.copy()
     buckets[70:73, 0] = -1
     plain, fast = _both(lib, st, q, buckets, kcand)
     assert _same(plain, fast)
     offsets, order = orc.ivf_build_lists(labels, nlist)
-    qproc = orc.squ_encode(q[:64], 4, l, dd, metric)
-    _, rds = orc.ivf_scan(orc.SQ4U, metric, d, codes[order], offsets, order, qproc, buckets[:64], kcand, lb=l, diff=dd)
+    qproc = orc.squ_encode(q[:64], bits, l, dd, metric)
+    _, rds = orc.ivf_scan(orc.SQ4U if bits == 4 else orc.SQ8U, metric, d, codes[order], offsets, order, qproc, buckets[:64],
+                          kcand, lb=l, diff=dd)
     assert np.array_equal(fast[1][:64].view(np.uint32), rds.view(np.uint32))
     st.destroy()
 

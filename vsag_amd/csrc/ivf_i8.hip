@@ -24,7 +24,10 @@
 // sum_o is kept per slot next to No (store.h, kMetaPayloadSum), sum_q is formed once per query.  The accumulator
 // starts from C_o = ceil((256 sum_o - No) / 2), so the pipe delivers X + C_o, and 2 <q, o> - No >= Tq becomes
 // X + C_o >= floor((Tq - 256 sum_q + 2 128^2 dim) / 2) -- a test that keeps every pair of the real one and at most
-// the pairs one unit beyond it, which ivf_i8_finish_kernel drops when it forms the distance.
+// the pairs one unit beyond it, which ivf_i8_finish_kernel drops when it forms the distance.  Inner product and
+// cosine: the float test of the 4-bit codes on the centred product, float(X) >= A'_q + g' sum_o with
+// A'_q = A_q - 128 sum_q + 128^2 dim and the per-code term g m_o - 128 sum_o (m_o the code's stored scalar, the sum of
+// the vector's values; sum_o the sum of its code values as under l2).
 //
 // Work split: the (query, list) pairs are grouped by list as for the streaming kernel; a workgroup is a chunk of a
 // list's tiles and up to 256 of its pairs, four waves of 64.  It walks the chunk two tiles per LDS stage; staging
@@ -59,7 +62,8 @@ ivf_i8_list_chunks(uint32_t tiles) {
 // Per query: Tq = Nq - tmax(bound) (see the header), widened by one level; the slow path re-checks exactly.
 __global__ void __launch_bounds__(256)
 ivf_i8_threshold_kernel(const uint32_t* bound, const float* qmeta, uint32_t qmeta_stride, int is_l2, float lb, float rate,
-                        float lb2, uint32_t dpad, uint64_t nq, int32_t* tq) {
+                        float lb2, uint32_t dpad, uint32_t centred_dim, const uint32_t* qtab, uint32_t qstride, uint64_t nq,
+                        int32_t* tq) {
     const uint64_t q = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (q > nq) {
         return;
@@ -82,12 +86,29 @@ ivf_i8_threshold_kernel(const uint32_t* bound, const float* qmeta, uint32_t qmet
         // out <= bd implies rate ip >= 1 - bd - lb2 - lb qm - lb m0 - eps.
         constexpr double kU = 5.9604644775390625e-8;
         const double qm = static_cast<double>(qmeta[q * qmeta_stride]);
-        const double m0_max = 15.0 * dpad, ip_max = 225.0 * dpad;
+        // centred_dim != 0: byte codes (values up to 255), the product centred by 128 on both sides.
+        const double vmax = centred_dim != 0 ? 255.0 : 15.0;
+        const double m0_max = vmax * dpad, ip_max = vmax * vmax * dpad;
         const double mag = fabs(static_cast<double>(lb)) * (fabs(qm) + m0_max) + static_cast<double>(rate) * ip_max +
                            fabs(static_cast<double>(lb2)) + 1.0 + fabs(static_cast<double>(bd));
         double aq = (1.0 - bd - lb2 - static_cast<double>(lb) * qm - 16.0 * kU * mag) / static_cast<double>(rate);
-        // the test adds fl(g m0) to A_q in fp32
-        aq -= 8.0 * kU * (fabs(aq) + fabs(static_cast<double>(lb) / rate) * m0_max + ip_max);
+        double slope = fabs(static_cast<double>(lb) / rate);
+        if (centred_dim != 0) {
+            // <q, o> = X + 128 sum_q + 128 sum_o - 128^2 dim: the test is on X.
+            uint32_t sum = 0;
+            const uint32_t* row = qtab + q * qstride;
+            for (uint32_t w = 0; 4 * w < centred_dim; ++w) {
+                uint32_t v = row[w];
+                if (4 * w + 4 > centred_dim) {
+                    v &= 0xFFFFFFFFU >> (8 * (4 * w + 4 - centred_dim));
+                }
+                sum = __builtin_amdgcn_udot4(v, 0x01010101U, sum, false);
+            }
+            aq += -128.0 * sum + 16384.0 * centred_dim;
+            slope += 128.0;
+        }
+        // the test adds fl(g m0) to A_q in fp32 (g itself rounded, for byte codes twice)
+        aq -= 8.0 * kU * (fabs(aq) + slope * m0_max + ip_max);
         float f = static_cast<float>(aq);
         if (static_cast<double>(f) > aq) {
             f = nextafterf(f, -__builtin_inff());
@@ -112,7 +133,7 @@ ivf_i8_threshold_kernel(const uint32_t* bound, const float* qmeta, uint32_t qmet
 // sq8_uniform: sum_q per query from its byte row, and the threshold of the centred product (see the header) in place
 // of Tq.  One thread per query; tq[nq] (the dummy row) and the two sentinels stay as they are.
 __global__ void __launch_bounds__(256)
-ivf_i8_centre_threshold_kernel(const uint32_t* qtab, uint32_t qstride, uint32_t dim, uint64_t nq, int32_t* tq,
+ivf_i8_centre_threshold_kernel(const uint32_t* qtab, uint32_t qstride, uint32_t dim, uint64_t nq, int is_l2, int32_t* tq,
                                int32_t* qsum) {
     const uint64_t q = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (q > nq) {
@@ -130,6 +151,9 @@ ivf_i8_centre_threshold_kernel(const uint32_t* qtab, uint32_t qstride, uint32_t 
         }
     }
     qsum[q] = static_cast<int32_t>(sum);
+    if (!is_l2) {
+        return;  // the float threshold is centred where it is formed
+    }
     const int32_t t = tq[q];
     if (t == 0x7FFFFFFF || t == static_cast<int32_t>(0x80000000U)) {
         return;
@@ -180,8 +204,7 @@ ivf_i8_centre_term(uint32_t sum_o, float no) {
 template <int KIND, int METRIC>
 __global__ void __launch_bounds__(256, 2)
 ivf_i8_kernel(IvfI8Args p) {
-    constexpr bool kBytes = KIND == VSAG_AMD_KIND_SQ8_UNIFORM;  // a byte per dimension (l2 only)
-    static_assert(!kBytes || METRIC == VSAG_AMD_METRIC_L2, "sq8_uniform lists take this route under l2 only");
+    constexpr bool kBytes = KIND == VSAG_AMD_KIND_SQ8_UNIFORM;  // a byte per dimension
     __shared__ IvfI8Stage stage[2];
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
@@ -295,8 +318,11 @@ ivf_i8_kernel(IvfI8Args p) {
                 my_term = METRIC == VSAG_AMD_METRIC_L2 ? static_cast<int32_t>(0xC0000000U) : 0x7F800000;
                 if (tile < tile_end) {
                     const float m0 = __uint_as_float(p.meta[static_cast<uint64_t>(tile) * kWave + lane]);
-                    if constexpr (kBytes) {
+                    if constexpr (kBytes && METRIC == VSAG_AMD_METRIC_L2) {
                         my_term = ivf_i8_centre_term(p.meta_sum[static_cast<uint64_t>(tile) * kWave + lane], m0);
+                    } else if constexpr (kBytes) {
+                        const uint32_t so = p.meta_sum[static_cast<uint64_t>(tile) * kWave + lane];
+                        my_term = __float_as_int(m0 * (-p.lb / p.rate) - 128.0F * static_cast<float>(so));
                     } else {
                         my_term = METRIC == VSAG_AMD_METRIC_L2 ? -static_cast<int32_t>(m0)
                                                                : __float_as_int(m0 * (-p.lb / p.rate));
@@ -532,7 +558,14 @@ ivf_i8_finish_kernel(IvfI8FinishArgs p) {
         }
         const float m0 = __uint_as_float(p.meta[slot]);
         float dist;
-        if constexpr (KIND == VSAG_AMD_KIND_SQ8_UNIFORM) {
+        if constexpr (KIND == VSAG_AMD_KIND_SQ8_UNIFORM && METRIC != VSAG_AMD_METRIC_L2) {
+            // acc = X, <q, o> = X + 128 sum_q + 128 sum_o - 128^2 dim
+            const int32_t ip = acc + 128 * p.qsum[q] + static_cast<int32_t>(128U * p.meta_sum[slot]) -
+                               static_cast<int32_t>(16384U * p.dim);
+            const float result = static_cast<float>(ip);
+            const float rr = p.lb * (qm + m0) + p.rate * result + p.lb2;
+            dist = 1 - rr;
+        } else if constexpr (KIND == VSAG_AMD_KIND_SQ8_UNIFORM) {
             // acc = X + C_o, <q, o> = X + 128 sum_q + 128 sum_o - 128^2 dim (see the header)
             const uint32_t so = p.meta_sum[slot];
             const int32_t ip = acc - ivf_i8_centre_term(so, m0) + 128 * p.qsum[q] + static_cast<int32_t>(128U * so) -
@@ -589,8 +622,7 @@ ivf_i8_lists_per_pair() {
 bool
 ivf_i8_supports(const vsag_amd_store* s) {
     if (s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
-        return s->metric == VSAG_AMD_METRIC_L2 && s->G <= 8 && s->dim <= 128 && s->nmeta == 2 && s->nlist > 0 &&
-               s->scalar_rate > 0.0F;
+        return s->G <= 8 && s->dim <= 128 && s->nmeta == 2 && s->nlist > 0 && s->scalar_rate > 0.0F;
     }
     return s->kind == VSAG_AMD_KIND_SQ4_UNIFORM && s->G <= 4 && s->nlist > 0 && s->scalar_rate > 0.0F;
 }
@@ -619,10 +651,11 @@ launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     const bool bytes = s->kind == VSAG_AMD_KIND_SQ8_UNIFORM;
     int32_t* qsum = tq + nq + 1;
     hipLaunchKernelGGL(ivf_i8_threshold_kernel, dim3(static_cast<uint32_t>(div_up(nq + 1, 256))), dim3(256), 0, st, bound,
-                       a.qmeta, a.qmeta_stride, l2 ? 1 : 0, a.f0, a.f1, a.f2, s->dpad, nq, tq);
+                       a.qmeta, a.qmeta_stride, l2 ? 1 : 0, a.f0, a.f1, a.f2, s->dpad, bytes ? s->dim : 0U, a.qtab, a.qstride, nq,
+                       tq);
     if (bytes) {
         hipLaunchKernelGGL(ivf_i8_centre_threshold_kernel, dim3(static_cast<uint32_t>(div_up(nq + 1, 256))), dim3(256), 0,
-                           st, a.qtab, a.qstride, s->dim, nq, tq, qsum);
+                           st, a.qtab, a.qstride, s->dim, nq, l2 ? 1 : 0, tq, qsum);
     }
     IvfI8Args p{};
     p.tiles = s->tiles;
@@ -657,8 +690,10 @@ launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
         (div_up(pairs, static_cast<uint64_t>(kIvfI8Pairs)) + std::min<uint64_t>(s->nlist, pairs)) * kIvfI8Chunks;
     const dim3 grid(static_cast<uint32_t>(max_items));
     timing_begin(st);
-    if (bytes) {
+    if (bytes && l2) {
         hipLaunchKernelGGL((ivf_i8_kernel<VSAG_AMD_KIND_SQ8_UNIFORM, VSAG_AMD_METRIC_L2>), grid, dim3(256), 0, st, p);
+    } else if (bytes) {
+        hipLaunchKernelGGL((ivf_i8_kernel<VSAG_AMD_KIND_SQ8_UNIFORM, VSAG_AMD_METRIC_IP>), grid, dim3(256), 0, st, p);
     } else if (l2) {
         hipLaunchKernelGGL((ivf_i8_kernel<VSAG_AMD_KIND_SQ4_UNIFORM, VSAG_AMD_METRIC_L2>), grid, dim3(256), 0, st, p);
     } else {
@@ -687,8 +722,10 @@ launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     f.rate = a.f1;
     f.lb2 = a.f2;
     const dim3 fgrid(static_cast<uint32_t>(div_up(f.lists, 256)));
-    if (bytes) {
+    if (bytes && l2) {
         hipLaunchKernelGGL((ivf_i8_finish_kernel<VSAG_AMD_KIND_SQ8_UNIFORM, VSAG_AMD_METRIC_L2>), fgrid, dim3(256), 0, st, f);
+    } else if (bytes) {
+        hipLaunchKernelGGL((ivf_i8_finish_kernel<VSAG_AMD_KIND_SQ8_UNIFORM, VSAG_AMD_METRIC_IP>), fgrid, dim3(256), 0, st, f);
     } else if (l2) {
         hipLaunchKernelGGL((ivf_i8_finish_kernel<VSAG_AMD_KIND_SQ4_UNIFORM, VSAG_AMD_METRIC_L2>), fgrid, dim3(256), 0, st, f);
     } else {

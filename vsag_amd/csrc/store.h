@@ -14,8 +14,8 @@
 #include "common.h"
 
 // A metadata word that is no field of the reference code but the sum of its payload bytes, formed when the code is
-// re-tiled (sq8_uniform, l2: the int8 matrix cores take code and query centred by 128, and putting the product right
-// needs the plain sum of the code values next to the sum of their squares the code carries).
+// re-tiled (sq8_uniform: the int8 matrix cores take code and query centred by 128, and putting the product right
+// needs the plain sum of the code values next to the scalar the code carries).
 constexpr uint32_t kMetaPayloadSum = 0xFFFFFFFFU;
 
 struct vsag_amd_store {

@@ -423,10 +423,8 @@ vsag_amd_store_create(const vsag_amd_store_params_t* p, vsag_amd_store_t** out) 
             s->nmeta = 1;
             s->meta_offset[0] = static_cast<uint32_t>(up(p->dim, align));
             s->meta_is_u64 = p->metric == VSAG_AMD_METRIC_L2 ? 1 : 0;
-            if (p->metric == VSAG_AMD_METRIC_L2) {
-                s->nmeta = 2;
-                s->meta_offset[1] = kMetaPayloadSum;
-            }
+            s->nmeta = 2;
+            s->meta_offset[1] = kMetaPayloadSum;
             break;
         }
         case VSAG_AMD_KIND_RABITQ: {
