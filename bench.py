@@ -493,7 +493,9 @@ def run_c4(env):
     # dimensions / a range per dimension)
     bits = 4 if args.list_codes == "sq4_uniform" else 8
     per_dim = args.list_codes == "sq8"
-    kind = capi.KIND_SQ8 if per_dim else capi.KIND_SQ8_UNIFORM if bits == 8 else capi.KIND_SQ4_UNIFORM
+    one_bit = args.list_codes == "rabitq"  # 1-bit codes, 4-bit queries, a seeded random rotation
+    kind = (capi.KIND_RABITQ if one_bit else capi.KIND_SQ8 if per_dim else capi.KIND_SQ8_UNIFORM if bits == 8
+            else capi.KIND_SQ4_UNIFORM)
     kind_name = args.list_codes
     means = mt(315).random((10000, d), dtype=np.float32)
     x_dev = env.buf(n * d * 4)
@@ -522,9 +524,18 @@ def run_c4(env):
     lb_dev, diff_dev = env.buf(d * 4), env.buf(d * 4)
     wsb = lib.vsag_amd_sq_train_workspace_bytes(ns, d, 0)
     ws = env.buf(wsb)
-    cs = int(lib.vsag_amd_code_size(kind, capi.METRIC_L2, d, 0))
+    cs = int(lib.vsag_amd_code_size(kind, capi.METRIC_L2, d, 4 if one_bit else 0))
     codes = env.buf(n * cs)
-    if per_dim:
+    rot = None
+    if one_bit:
+        g = mt(316).standard_normal((d, d))
+        rot, r = np.linalg.qr(g)
+        rot = (rot * np.sign(np.diag(r))).astype(np.float32)
+        rot_dev, cen_dev = env.upload(rot), env.buf(d * 4)
+        capi.check(lib.vsag_amd_rabitq_train(x_dev.ptr, ns, d, rot_dev.ptr, cen_dev.ptr, None))
+        capi.check(lib.vsag_amd_rabitq_encode(x_dev.ptr, n, d, rot_dev.ptr, cen_dev.ptr, capi.METRIC_L2, 4, codes.ptr, None))
+        lists = env.make_store(kind, capi.METRIC_L2, d, rot=rot_dev, cen=cen_dev, qbits=4)
+    elif per_dim:
         capi.check(lib.vsag_amd_sq_train(x_dev.ptr, ns, d, 8, capi.METRIC_L2, capi.SQ_TRAIN_TRUNC_BOUND, 0.05, 0,
                                          lb_dev.ptr, diff_dev.ptr, ws.ptr, wsb, None))
         capi.check(lib.vsag_amd_sq_encode(x_dev.ptr, n, d, 8, capi.METRIC_L2, lb_dev.ptr, diff_dev.ptr, codes.ptr, None))
@@ -605,7 +616,11 @@ def run_c4(env):
         hlabels = labels.to_numpy(np.int32, (n,))
         offsets, order = orc.ivf_build_lists(hlabels, nlist)
         posting = hcodes[order]
-        if per_dim:
+        if one_bit:
+            hb = (None, None)
+            okind = orc.RABITQ
+            qcodes = orc.rabitq_process_query(q[:sample], rot, cen_dev.to_numpy(np.float32, (d,)), orc.L2)
+        elif per_dim:
             hb = (lb_dev.to_numpy(np.float32, (d,)), diff_dev.to_numpy(np.float32, (d,)))
             okind, qcodes = orc.SQ8, q[:sample]
         else:
@@ -665,13 +680,15 @@ def run_c4(env):
                 # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this launch: profiles/ivf_i8_sq4u_c4.md
                 "traffic": 491061.0 * 2.00 * 1024 + 73550.7 * 1024
                 if (n, d, nq, k, nlist, bits) == (10000000, 128, 10000, 10, 4096, 4) else None,
-                "kernel": "%s<%s> (int8 MFMA, probe columns 1..%d)" % ("ivf_sq8_i8_kernel" if per_dim else "ivf_i8_kernel",
+                "kernel": "%s<%s> (int8 MFMA, probe columns 1..%d)" % ("prefilter_rb_kernel<lists>" if one_bit else
+                                                                        "ivf_sq8_i8_kernel" if per_dim else "ivf_i8_kernel",
                                                                         kind_name, nprobe - 1), "kernel_ms": kms,
                 "ops_per_launch": ops, "distance_evaluations_per_launch": float(rest),
                 "distance_evaluations_per_second": float(rest) / (kms * 1e-3)}
     return env.base_line("QPS @ recall@10 (IVF %s, 10M x 128)" % {"sq4_uniform": "SQ4-uniform", "sq8_uniform": "SQ8-uniform",
-                                                                  "sq8": "SQ8"}[kind_name],
-                         "queries/s", nq / sec, sec, "u8 codes x f32 scale, f32 (pre-selection: i8 x i8, i32 sums)" if per_dim else "u%d codes, i32 dot" % bits,
+                                                                  "sq8": "SQ8", "rabitq": "RaBitQ"}[kind_name],
+                         "queries/s", nq / sec, sec, "1-bit codes x u4 queries, i32 popcount sums, f32 estimator" if one_bit else
+                         "u8 codes x f32 scale, f32 (pre-selection: i8 x i8, i32 sums)" if per_dim else "u%d codes, i32 dot" % bits,
                          "configs[3]%s: IVF search, N=%d, d=%d, nlist=%d, nprobe=%d, rerank %d, %d queries, k=%d"
                          % ("" if bits == 4 else " with %s lists" % kind_name, n, d, nlist, nprobe, kcand, nq, k),
                          {"recall_at_10": rec, "build_seconds": t_build, "scanned_codes_per_query": float(scanned) / nq,
@@ -815,7 +832,7 @@ def main():
     ap.add_argument("--chunks", type=int, default=0, help="base chunk override (0 = library default)")
     ap.add_argument("--contraction", type=int, default=0, choices=[-1, 0, 1],
                     help="matrix-core path of the flat scans: -1 never, 0 library default, 1 whenever supported")
-    ap.add_argument("--list-codes", default="sq4_uniform", choices=["sq4_uniform", "sq8_uniform", "sq8"],
+    ap.add_argument("--list-codes", default="sq4_uniform", choices=["sq4_uniform", "sq8_uniform", "sq8", "rabitq"],
                     help="c4 only: the quantizer of the posting lists (configs[3] names sq4_uniform)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-recall", action="store_true", help="skip the recall check")

@@ -325,3 +325,27 @@ def test_residual_lists_match_oracle(lib, kind, metric, mname):
     for b in (xb, lb_dev, cb, rb):
         b.free()
     st.destroy()
+
+
+@pytest.mark.parametrize("nq,kcand", [(40, 32), (40, 33), (6000, 32), (6000, 7)])
+def test_a_list_probed_twice_brings_every_key_twice(lib, nq, kcand):
+    """Injected buckets may name a list twice; then every (distance, id) key exists twice, also the k-th one, and the
+    closing merge must keep the right number of copies of it: positions 2i and 2i + 1 of a result are equal."""
+    rng = np.random.default_rng(kcand)
+    n, d, nlist = 20000, 32, 16
+    x, q, cent, labels = _ivf_case(rng, n, d, nlist, nq)
+    lb, diff = orc.sq_train(x, 8)
+    codes = orc.sq_encode(x, 8, lb, diff)
+    st = Store(capi.KIND_SQ8, orc.L2, d, lb=lb, diff=diff)
+    st.set_lists(codes, labels, nlist)
+    routed, _ = orc.ivf_route(cent, q, 2)
+    buckets = np.ascontiguousarray(routed[:, [0, 1, 0, 1]])
+    ids, ds = st.ivf_scan(q, buckets, kcand)
+    once, od = st.ivf_scan(q, np.ascontiguousarray(routed), kcand)
+    half = kcand // 2
+    assert np.array_equal(ids[:, 0:2 * half:2], ids[:, 1:2 * half:2])
+    assert np.array_equal(ids[:, 0:2 * half:2], once[:, :half])
+    assert np.array_equal(ds[:, 0:2 * half:2].view(np.uint32), od[:, :half].view(np.uint32))
+    if kcand % 2:
+        assert np.array_equal(ids[:, -1], once[:, half])
+    st.destroy()

@@ -33,6 +33,7 @@ struct ScanPlanIvf {
     bool seeded;
     bool mfma;                // probe columns behind the first go through the int8 matrix cores (ivf_i8.hip)
     bool planes;              // ... with sq8 codes: two int8 planes per query, records rescored (prefilter_i8.hip)
+    bool bits1;               // ... with rabitq codes: expanded bits, records rescored (prefilter_rb.hip)
 };
 
 uint64_t rabitq_query_code_size(uint32_t dim, int metric, int query_bits);
@@ -50,6 +51,14 @@ int launch_ivf_sq8_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstri
                       uint64_t nq, uint32_t nprobe, uint32_t p0, const uint32_t* pair_off, const uint32_t* item_off,
                       const uint32_t* sorted_pair, const uint32_t* bound, uint32_t kcand, uint8_t* q8, float* u, uint32_t* tau,
                       uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st);
+// rabitq lists (1-bit codes, 4-bit queries): the expanded-bits contraction of prefilter_rb.hip over 128 pairs per item.
+bool ivf_rb_supports(const vsag_amd_store* s);
+uint32_t ivf_rb_pairs_per_item();
+uint32_t ivf_rb_chunk_tiles();
+size_t ivf_rb_scratch_bytes(const vsag_amd_store* s, uint64_t nq);
+int launch_ivf_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, const uint32_t* pair_off,
+                  const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound, uint32_t kcand, uint8_t* scratch,
+                  uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st);
 int launch_ivf_clear_gated(uint32_t* gate, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t* partial_cnt,
                            const int32_t* buckets, uint32_t* gpairs, uint32_t gpairs_cap, hipStream_t st);
 int launch_ivf_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
@@ -879,13 +888,14 @@ struct IvfBuffers {
     int32_t* tq;          // mfma: 2 (nq + 1)
     uint32_t* gpairs;     // mfma: pairs of gated queries, kGatedPairsCap
     uint8_t* q8;          // sq8 lists on the matrix cores: the planes of the queries, their scalars and thresholds
+                          // (rabitq lists: the queries as bytes and their four factors)
     float* q8_u;
     uint32_t* q8_tau;
     float* res_term;      // residual lists: per pair
 };
 
 // Pairs of gated queries the direct fallback launch takes; more go through the per-list grouping.
-constexpr uint32_t kGatedPairsCap = 4096;
+constexpr uint32_t kGatedPairsCap = 32768;
 
 static void
 plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, ScanPlanIvf* p) {
@@ -938,7 +948,9 @@ plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, 
     // sq8 lists of at most 128 dimensions: the same split with the two-plane test and an exact rescoring.
     p->planes = !p->mfma && !p->chunked && nprobe > 1 && scan_contraction_mode(s) >= 0 && ivf_sq8_i8_supports(s) &&
                 kcand <= ivf_rescore_capacity() && npairs * ivf_i8_lists_per_pair() * kcand * 8 <= (8ull << 30);
-    p->mfma = p->mfma || p->planes;
+    p->bits1 = !p->mfma && !p->planes && !p->chunked && nprobe > 1 && scan_contraction_mode(s) >= 0 && ivf_rb_supports(s) &&
+               kcand <= ivf_rescore_capacity() && npairs * ivf_i8_lists_per_pair() * kcand * 8 <= (8ull << 30);
+    p->mfma = p->mfma || p->planes || p->bits1;
     if (p->mfma) {
         p->chunks_max = ivf_i8_lists_per_pair();
     }
@@ -969,7 +981,7 @@ carve_ivf(Carver& c, const vsag_amd_store* s, const ScanPlanIvf& p, uint64_t nq,
     b->gate = c.take<uint32_t>(p.mfma ? nq + 2 : 0);
     b->gpairs = c.take<uint32_t>(p.mfma ? kGatedPairsCap : 0);
     b->tq = c.take<int32_t>(p.mfma ? 2 * (nq + 1) : 0);  // thresholds, then (sq8_uniform) the sums of the query values
-    b->q8 = c.take<uint8_t>(p.planes ? ivf_sq8_i8_query_bytes(nq) : 0);
+    b->q8 = c.take<uint8_t>(p.planes ? ivf_sq8_i8_query_bytes(nq) : p.bits1 ? ivf_rb_scratch_bytes(s, nq) : 0);
     b->q8_u = c.take<float>(p.planes ? ivf_sq8_i8_scalar_floats(nq) : 0);
     b->q8_tau = c.take<uint32_t>(p.planes ? ivf_sq8_i8_tau_words(nq) : 0);
     b->res_term = c.take<float>(s->residual_centroids_dev != nullptr ? p.npairs : 0);
@@ -1132,8 +1144,14 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
             // Pairs grouped by list once; workgroups of 256 pairs for the matrix cores, then -- for the queries whose
             // lists overflowed -- the streaming kernel's items over the same grouping.
             // ivf_i8.hip: items of 256 pairs, kIvfI8ChunkTiles, kIvfI8Chunks
-            regroup(p0, p1, pairs, 256U, 32U, 4U);
-            if (p.planes) {
+            regroup(p0, p1, pairs, p.bits1 ? ivf_rb_pairs_per_item() : 256U, p.bits1 ? ivf_rb_chunk_tiles() : 32U, 4U);
+            if (p.bits1) {
+                VA_TRY(launch_ivf_rb(s, a, nq, nprobe, p0, b.pair_off, b.item_off, b.sorted_pair, b.bound, kcand, b.q8,
+                                     b.partial, b.partial_cnt, b.gate, st));
+                VA_TRY(launch_ivf_clear_gated(b.gate, nq, nprobe, p0, b.partial_cnt, buckets_dev, b.gpairs,
+                                              kGatedPairsCap, st));
+                VA_TRY(launch_ivf_rescore(s, a, nq, nprobe, p0, kcand, p.chunks_max, b.partial, b.partial_cnt, b.bound, st));
+            } else if (p.planes) {
                 VA_TRY(launch_ivf_sq8_i8(s, reinterpret_cast<const float*>(a.qtab), a.qstride, a.qmeta, a.qmeta_stride, nq,
                                          nprobe, p0, b.pair_off, b.item_off, b.sorted_pair, b.bound, kcand, b.q8, b.q8_u,
                                          b.q8_tau, b.partial, b.partial_cnt, b.gate, st));

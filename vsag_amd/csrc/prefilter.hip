@@ -680,8 +680,9 @@ ivf_rescore_capacity() {
 int
 launch_ivf_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
                    uint32_t per_pair, uint64_t* partial, uint32_t* partial_cnt, const uint32_t* bound, hipStream_t st) {
-    if (s->kind != VSAG_AMD_KIND_SQ8 || kcand > kIvfRescoreGather || s->ids_dev == nullptr) {
-        return fail(VSAG_AMD_INVALID_ARGUMENT, "rescoring of list records: sq8 lists with kcand <= %u only",
+    if ((s->kind != VSAG_AMD_KIND_SQ8 && s->kind != VSAG_AMD_KIND_RABITQ) || kcand > kIvfRescoreGather ||
+        s->ids_dev == nullptr) {
+        return fail(VSAG_AMD_INVALID_ARGUMENT, "rescoring of list records: sq8 or rabitq lists with kcand <= %u only",
                     kIvfRescoreGather);
     }
     IvfRescoreArgs r{};
@@ -694,7 +695,13 @@ launch_ivf_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint
     r.ids = s->ids_dev;
     r.bound = bound;
     const dim3 grid(static_cast<uint32_t>(nq));
-    if (s->metric == VSAG_AMD_METRIC_L2) {
+    if (s->kind == VSAG_AMD_KIND_RABITQ) {
+        if (s->metric == VSAG_AMD_METRIC_L2) {
+            hipLaunchKernelGGL((ivf_rescore_kernel<VSAG_AMD_KIND_RABITQ, VSAG_AMD_METRIC_L2>), grid, dim3(kWave), 0, st, a, r);
+        } else {
+            hipLaunchKernelGGL((ivf_rescore_kernel<VSAG_AMD_KIND_RABITQ, VSAG_AMD_METRIC_IP>), grid, dim3(kWave), 0, st, a, r);
+        }
+    } else if (s->metric == VSAG_AMD_METRIC_L2) {
         hipLaunchKernelGGL((ivf_rescore_kernel<VSAG_AMD_KIND_SQ8, VSAG_AMD_METRIC_L2>), grid, dim3(kWave), 0, st, a, r);
     } else {
         hipLaunchKernelGGL((ivf_rescore_kernel<VSAG_AMD_KIND_SQ8, VSAG_AMD_METRIC_IP>), grid, dim3(kWave), 0, st, a, r);

@@ -39,6 +39,10 @@ constexpr uint32_t kRbQueries = 128;  // queries per workgroup
 constexpr uint32_t kRbMaxG = 8;       // granules per code (1024 dimensions): the query group has to fit the LDS
 constexpr uint32_t kRbWaves = 8;      // waves per workgroup, two per SIMD: one multiplies while the other decides
 constexpr uint32_t kRbThreads = kRbWaves * kWave;
+// Largest per-code factors the fp32 threshold takes (A_c, |B_c|; codes beyond them are candidates of every query): the
+// per-query slack below is sized for them.  B_c grows with the square of the data's scale (norm x error factor / 2).
+constexpr float kRbMaxA = 64.0F;
+constexpr float kRbMaxB = 4096.0F;
 
 // 4-bit queries as bytes: row q holds, per code dword w, the 32 values of dimensions 32 w ... (dpad bytes per row).
 __global__ void __launch_bounds__(256)
@@ -78,8 +82,8 @@ rabitq_query_bytes_kernel(const uint32_t* qtab, uint32_t qstride, uint32_t ndw, 
 
 // Per query: u1..u4 of the header (u[j * nq_pad + q]).  -inf in u4: everything passes; +inf: nothing does.
 __global__ void __launch_bounds__(256)
-rabitq_tau_kernel(const float* qmeta, uint32_t qmeta_stride, const uint32_t* bound, int is_l2, uint64_t nq, uint64_t nq_pad,
-                  float* u) {
+rabitq_tau_kernel(const float* qmeta, uint32_t qmeta_stride, const uint32_t* bound, int is_l2, uint32_t dpad, uint64_t nq,
+                  uint64_t nq_pad, float* u) {
     const uint64_t q = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (q >= nq_pad) {
         return;
@@ -116,7 +120,11 @@ rabitq_tau_kernel(const float* qmeta, uint32_t qmeta_stride, const uint32_t* bou
                     u1 = static_cast<float>(v1 * lower);
                     u2 = static_cast<float>(inv * lower);
                     u3 = static_cast<float>(v3 * lower);
-                    u4 = static_cast<float>(v4 * lower);
+                    // The threshold is a chain of three fp32 fma over terms that may cancel: it is off by at most
+                    // 3 x 2^-24 of the sum of their magnitudes, whatever it comes to itself.  2^-20 of the largest
+                    // magnitudes any code can bring (A_c <= kRbMaxA, |B_c| <= kRbMaxB, set bits <= dpad) is taken off.
+                    const double reach = kRbMaxA * fabs(v1) + kRbMaxB * inv + dpad * fabs(v3) + fabs(v4);
+                    u4 = static_cast<float>(v4 * lower - 9.5367431640625e-7 * reach);
                 }
             }
         }
@@ -141,7 +149,27 @@ struct PrefilterRbArgs {
     uint32_t* cand_cnt;    // [query][sub_lists]
     uint32_t sub_cap;
     uint32_t groups;       // grid x; the grid has groups * kRbWaves waves per query group
+    // Posting lists (LISTS): a workgroup is a chunk of a list's tiles x up to 128 of the (query, list) pairs that probe
+    // the list -- the work split of ivf_i8.hip with 128 pairs per item -- and its queries are gathered by pair.
+    const uint32_t* ids;          // inner id per tile slot (slots without a code hold VSAG_AMD_INVALID_ID)
+    const uint32_t* list_tile;    // 2 nlist: first tile and end of the used tiles of every list
+    const uint32_t* pair_off;     // nlist + 1
+    const uint32_t* item_off;     // nlist + 1: workgroups per list, prefix sums
+    const uint32_t* sorted_pair;  // pair index (q * nprobe + p) grouped by list
+    uint32_t nlist, nprobe;
+    uint32_t dummy_query;         // a padding row of the query tables: zero operands, a threshold nothing meets
+    uint32_t k;                   // capacity of a private list
+    uint64_t* partial;            // [pair][8][k]: tile slots; the waves of a pair's items share its eight lists
+    uint32_t* partial_cnt;        // [pair][8]: appended so far, also beyond k
+    uint32_t* gate;               // per query: raised when one of its lists overflowed; gate[dummy_query] counts them
 };
+
+// Lists are cut into chunks of about kIvfRbChunkTiles tiles, at most kIvfRbChunks per list (the private lists of a pair
+// are laid out for four chunks, as in ivf_i8.hip).  Long chunks: a workgroup fills a compute unit alone (the registers
+// of its eight waves), so what it does before its first tile -- finding its list, gathering its queries -- is not
+// hidden behind another workgroup and has to be spread over many tiles.
+constexpr uint32_t kIvfRbChunkTiles = 128;
+constexpr uint32_t kIvfRbChunks = 4;
 
 __device__ inline int
 rb_spread(uint32_t nibble) {
@@ -149,24 +177,85 @@ rb_spread(uint32_t nibble) {
     return static_cast<int>((nibble * 0x00204081U) & 0x01010101U);
 }
 
-template <int METRIC>
+template <int METRIC, bool LISTS = false>
 __global__ void __launch_bounds__(kRbThreads, 2)
 prefilter_rb_kernel(PrefilterRbArgs p) {
     extern __shared__ uint4 rb_lds[];
+    __shared__ uint32_t pair_q[LISTS ? kRbQueries : 1];     // LISTS: the query of each of the item's pairs
+    __shared__ uint32_t pair_list[LISTS ? kRbQueries : 1];  // and the first of its private lists in this chunk
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
     const uint32_t wave = tid >> 6;
     const uint32_t half = lane >> 5;
     const uint32_t l32 = lane & 31;
     const uint32_t nchunks = 8 * p.G;  // 16-byte chunks per query row: chunk 2 s + h of step s = code dword s
-    const uint64_t q0 = static_cast<uint64_t>(blockIdx.y) * kRbQueries;
+    uint64_t q0 = static_cast<uint64_t>(blockIdx.y) * kRbQueries;
     uint4* qs = rb_lds;                                                           // [chunk][128 queries]
     float* cc = reinterpret_cast<float*>(rb_lds + nchunks * kRbQueries) + wave * 3 * kWave;  // [3][64] per wave
+    uint64_t tile_first = p.tile_begin, span = p.tile_end - p.tile_begin;
+    uint64_t t_first = static_cast<uint64_t>(blockIdx.x) * kRbWaves + wave, t_step = static_cast<uint64_t>(p.groups) * kRbWaves;
+
+    if constexpr (LISTS) {
+        const uint32_t item = blockIdx.x;
+        cu32_p ioff = as_const(p.item_off);
+        if (item >= ioff[p.nlist]) {
+            return;  // the whole workgroup
+        }
+        // Which list: last b with item_off[b] <= item; its items are (block of 128 pairs) x (tile chunk), chunk fastest.
+        uint32_t lo_b = 0, hi_b = p.nlist;
+        while (hi_b - lo_b > 1) {
+            const uint32_t mid = (lo_b + hi_b) >> 1;
+            if (ioff[mid] <= item) {
+                lo_b = mid;
+            } else {
+                hi_b = mid;
+            }
+        }
+        const uint32_t b = lo_b;
+        const uint32_t list_begin = as_const(p.list_tile)[2 * b], list_end = as_const(p.list_tile)[2 * b + 1];
+        uint32_t chunks = (list_end - list_begin + kIvfRbChunkTiles - 1) / kIvfRbChunkTiles;
+        chunks = chunks < kIvfRbChunks ? chunks : kIvfRbChunks;
+        if (chunks == 0) {
+            return;
+        }
+        const uint32_t per = (list_end - list_begin + chunks - 1) / chunks;
+        const uint32_t chunk = (item - ioff[b]) % chunks;
+        const uint32_t group = (item - ioff[b]) / chunks;
+        uint32_t tile_begin = list_begin + chunk * per;
+        tile_begin = tile_begin < list_end ? tile_begin : list_end;
+        const uint32_t tile_end = tile_begin + per < list_end ? tile_begin + per : list_end;
+        if (tile_end == tile_begin) {
+            return;  // an empty chunk: its lists keep their zero counts
+        }
+        const uint32_t pbeg = as_const(p.pair_off)[b] + group * kRbQueries;
+        const uint32_t pend = as_const(p.pair_off)[b + 1];
+        if (tid < kRbQueries) {
+            const uint32_t idx = pbeg + tid;
+            const bool live = idx < pend;
+            const uint32_t pair = live ? as_const(p.sorted_pair)[idx] : 0U;
+            pair_q[tid] = live ? pair / p.nprobe : p.dummy_query;
+            pair_list[tid] = live ? pair * kIvfRbChunks * 2 : 0xFFFFFFFFU;
+        }
+        __syncthreads();
+        q0 = 0;
+        tile_first = tile_begin;
+        span = tile_end - tile_begin;
+        t_first = wave;
+        t_step = kRbWaves;
+    }
+    // The row of the query tables behind local query ql of the workgroup.
+    auto query_row = [&](uint32_t ql) -> uint64_t {
+        if constexpr (LISTS) {
+            return pair_q[ql];
+        } else {
+            return q0 + ql;
+        }
+    };
 
     // The query group, once: chunk c of query q to qs[c][q].
     for (uint32_t i = tid; i < nchunks * kRbQueries; i += blockDim.x) {
         const uint32_t ql = i / nchunks, c = i % nchunks;
-        qs[c * kRbQueries + ql] = p.qbytes[(q0 + ql) * nchunks + c];
+        qs[c * kRbQueries + ql] = p.qbytes[query_row(ql) * nchunks + c];
     }
     float u1[4], u2[4], u3[4], u4[4];
     uint32_t ncand[4] = {0, 0, 0, 0};
@@ -174,18 +263,31 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
     const uint32_t my_sub = (blockIdx.x * kRbWaves + wave) * 2 + half;
 #pragma unroll
     for (int qb = 0; qb < 4; ++qb) {
-        const uint64_t q = q0 + 32 * qb + l32;
+        const uint64_t q = query_row(32 * qb + l32);
         u1[qb] = p.u[q];
         u2[qb] = p.u[p.nq_pad + q];
         u3[qb] = p.u[2 * p.nq_pad + q];
         u4[qb] = p.u[3 * p.nq_pad + q];
     }
     __syncthreads();
+    // LISTS: a pair has eight private lists (two per chunk in ivf_i8.hip's layout); here a hit goes to the one of
+    // (wave % 4, lane / 32), so that the waves of an item -- and of the other chunks of a long list, which use the same
+    // eight -- spread what passes over all of them: the estimator is noisy, and a pair may bring hundreds.
+    auto append_shared = [&](uint32_t ql, uint64_t slot) {
+        const uint32_t first = pair_list[ql];
+        if (first != 0xFFFFFFFFU) {
+            const uint64_t list = static_cast<uint64_t>(first) + 2 * (wave & 3U) + half;
+            const uint32_t pos = atomicAdd(&p.partial_cnt[list], 1U);
+            if (pos < p.k) {
+                p.partial[list * p.k + pos] = slot;
+            } else if (atomicExch(&p.gate[pair_q[ql]], 1U) == 0U) {
+                atomicAdd(&p.gate[p.dummy_query], 1U);
+            }
+        }
+    };
 
-    const uint64_t span = p.tile_end - p.tile_begin;
-    for (uint64_t t = static_cast<uint64_t>(blockIdx.x) * kRbWaves + wave; t < span;
-         t += static_cast<uint64_t>(p.groups) * kRbWaves) {
-        const uint64_t tile = p.tile_begin + t;
+    for (uint64_t t = t_first; t < span; t += t_step) {
+        const uint64_t tile = tile_first + t;
         // The bits of this lane's two codes (rows l32 and 32 + l32 of the tile), a granule at a time and one ahead.
         const uint4* code_rows = p.tiles + tile * p.G * kWave + l32;
         uint4 bits[2], ahead[2];
@@ -207,15 +309,20 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
         }
         float a_c = odd ? 0.0F : berr / (2.0F * bn);
         float b_c = odd ? 0.0F : (bn * bn - braw * braw) * a_c;
-        odd = odd || !(a_c <= 64.0F) || !(fabsf(b_c) <= 64.0F) || !(fabsf(bsum) <= 65536.0F);
+        odd = odd || !(a_c <= kRbMaxA) || !(fabsf(b_c) <= kRbMaxB) || !(fabsf(bsum) <= static_cast<float>(128 * p.G));
         a_c = odd ? 0.0F : a_c;
         b_c = odd ? 0.0F : b_c;
-        const bool special = odd && my_slot < p.n;
+        bool holds_code = my_slot < p.n;
+        if constexpr (LISTS) {
+            holds_code = as_const(p.ids)[my_slot] != VSAG_AMD_INVALID_ID;
+        }
+        const bool special = odd && holds_code;
         wave_lds_fence();  // the previous tile's verdicts have read these
         cc[lane] = a_c;
         cc[kWave + lane] = b_c;
         cc[2 * kWave + lane] = odd ? 0.0F : bsum;
         const uint64_t special_mask = __ballot(special);
+        const uint64_t code_mask = __ballot(holds_code);
         wave_lds_fence();
 
         intx16 acc[4][2];
@@ -291,17 +398,21 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
                             hits |= pass[j] ? 1U << j : 0U;
                         }
                         const uint64_t q = q0 + 32 * qb + l32;
-                        uint32_t* list = p.cand + ((q < p.nq ? q : 0) * sub_lists + my_sub) * p.sub_cap;
+                        uint32_t* list = LISTS ? nullptr : p.cand + ((q < p.nq ? q : 0) * sub_lists + my_sub) * p.sub_cap;
                         while (hits != 0) {
                             const uint32_t j = static_cast<uint32_t>(__builtin_ctz(hits));
                             hits &= hits - 1;
                             const uint32_t code = row + j;
                             const uint64_t slot = tile * kWave + code;
-                            if (slot < p.n && ((special_mask >> code) & 1ULL) == 0) {
-                                if (ncand[qb] < p.sub_cap) {
-                                    list[ncand[qb]] = static_cast<uint32_t>(slot);
+                            if (((code_mask >> code) & 1ULL) != 0 && ((special_mask >> code) & 1ULL) == 0) {
+                                if constexpr (LISTS) {
+                                    append_shared(32 * qb + l32, slot);
+                                } else {
+                                    if (ncand[qb] < p.sub_cap) {
+                                        list[ncand[qb]] = static_cast<uint32_t>(slot);
+                                    }
+                                    ++ncand[qb];
                                 }
-                                ++ncand[qb];
                             }
                         }
                     }
@@ -316,6 +427,10 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
                 rest &= rest - 1;
 #pragma unroll
                 for (int qb = 0; qb < 4; ++qb) {
+                    if constexpr (LISTS) {
+                        append_shared(32 * qb + l32, tile * kWave + code);
+                        continue;
+                    }
                     const uint64_t q = q0 + 32 * qb + l32;
                     if (q < p.nq) {
                         if (ncand[qb] < p.sub_cap) {
@@ -327,11 +442,13 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
             }
         }
     }
+    if constexpr (!LISTS) {
 #pragma unroll
-    for (int qb = 0; qb < 4; ++qb) {
-        const uint64_t q = q0 + 32 * qb + l32;
-        if (q < p.nq) {
-            p.cand_cnt[q * sub_lists + my_sub] = ncand[qb];
+        for (int qb = 0; qb < 4; ++qb) {
+            const uint64_t q = q0 + 32 * qb + l32;
+            if (q < p.nq) {
+                p.cand_cnt[q * sub_lists + my_sub] = ncand[qb];
+            }
         }
     }
 }
@@ -387,7 +504,7 @@ launch_prefilter_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uin
     hipLaunchKernelGGL(rabitq_query_bytes_kernel, dim3(static_cast<uint32_t>(div_up(nq_pad * ndw, 256))), dim3(256), 0, st,
                        a.qtab, a.qstride, ndw, nq, nq_pad, qbytes);
     hipLaunchKernelGGL(rabitq_tau_kernel, dim3(static_cast<uint32_t>(div_up(nq_pad, 256))), dim3(256), 0, st, a.qmeta,
-                       a.qmeta_stride, bound, l2 ? 1 : 0, nq, nq_pad, u);
+                       a.qmeta_stride, bound, l2 ? 1 : 0, s->G * 128, nq, nq_pad, u);
     VA_HIP(hipGetLastError());
     PrefilterRbArgs p{};
     p.tiles = s->tiles;
@@ -417,6 +534,92 @@ launch_prefilter_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uin
         VA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(prefilter_rb_kernel<VSAG_AMD_METRIC_IP>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
         hipLaunchKernelGGL(prefilter_rb_kernel<VSAG_AMD_METRIC_IP>, grid, dim3(kRbThreads), lds, st, p);
+    }
+    timing_end(st);
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
+// ---- posting lists ------------------------------------------------------------------------------------------------
+bool
+ivf_rb_supports(const vsag_amd_store* s) {
+    return s->kind == VSAG_AMD_KIND_RABITQ && s->query_bits == 4 && s->nlist > 0 && s->G <= kRbMaxG &&
+           s->residual_centroids_dev == nullptr &&
+           (s->metric == VSAG_AMD_METRIC_L2 || s->metric == VSAG_AMD_METRIC_IP);
+}
+
+// Pairs per work item of the list kernel (offsets_kernel's T) and the tiles of a chunk.
+uint32_t
+ivf_rb_pairs_per_item() {
+    return kRbQueries;
+}
+
+uint32_t
+ivf_rb_chunk_tiles() {
+    return kIvfRbChunkTiles;
+}
+
+// Bytes of scratch for nq queries and one padding row.
+size_t
+ivf_rb_scratch_bytes(const vsag_amd_store* s, uint64_t nq) {
+    return prefilter_rb_scratch_bytes(s, nq + 1);
+}
+
+// The pairs of probe columns [p0, nprobe) grouped by list (pair_off, sorted_pair; item_off: offsets_kernel with
+// T = 128, ivf_rb_chunk_tiles(), four chunks at most) against the bounds the nearest lists left: what may still matter is
+// recorded as a tile slot in one of the pair's eight private lists of kcand records in `partial`, counted in
+// partial_cnt (zero before; a count above kcand raised the query's gate).  gate: nq + 2 words as in ivf_i8.hip.
+int
+launch_ivf_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, const uint32_t* pair_off,
+              const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound, uint32_t kcand, uint8_t* scratch,
+              uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st) {
+    const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
+    const uint64_t nq_pad = prefilter_rb_padded_queries(nq + 1);
+    const uint32_t ndw = s->G * 4;
+    uint8_t* qbytes = scratch;
+    float* u = reinterpret_cast<float*>(scratch + round_up(static_cast<size_t>(nq_pad) * ndw * 32, 256));
+    hipLaunchKernelGGL(rabitq_query_bytes_kernel, dim3(static_cast<uint32_t>(div_up(nq_pad * ndw, 256))), dim3(256), 0, st,
+                       a.qtab, a.qstride, ndw, nq, nq_pad, qbytes);
+    hipLaunchKernelGGL(rabitq_tau_kernel, dim3(static_cast<uint32_t>(div_up(nq_pad, 256))), dim3(256), 0, st, a.qmeta,
+                       a.qmeta_stride, bound, l2 ? 1 : 0, s->G * 128, nq, nq_pad, u);
+    VA_HIP(hipGetLastError());
+    PrefilterRbArgs p{};
+    p.tiles = s->tiles;
+    p.G = s->G;
+    p.n = s->n;
+    p.meta = a.meta;
+    p.meta_stride = a.meta_stride;
+    p.qbytes = reinterpret_cast<const uint4*>(qbytes);
+    p.u = u;
+    p.nq = nq;
+    p.nq_pad = nq_pad;
+    p.groups = 1;
+    p.ids = s->ids_dev;
+    p.list_tile = s->list_tile_dev;
+    p.pair_off = pair_off;
+    p.item_off = item_off;
+    p.sorted_pair = sorted_pair;
+    p.nlist = s->nlist;
+    p.nprobe = nprobe;
+    p.dummy_query = static_cast<uint32_t>(nq);
+    p.k = kcand;
+    p.partial = partial;
+    p.partial_cnt = partial_cnt;
+    p.gate = gate;
+    const size_t lds = static_cast<size_t>(8 * s->G) * kRbQueries * 16 + kRbWaves * 3 * kWave * sizeof(float);
+    const uint64_t pairs = nq * (nprobe - p0);
+    const uint64_t max_items =
+        (div_up(pairs, static_cast<uint64_t>(kRbQueries)) + std::min<uint64_t>(s->nlist, pairs)) * kIvfRbChunks;
+    const dim3 grid(static_cast<uint32_t>(max_items));
+    timing_begin(st);
+    if (l2) {
+        VA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(prefilter_rb_kernel<VSAG_AMD_METRIC_L2, true>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        hipLaunchKernelGGL((prefilter_rb_kernel<VSAG_AMD_METRIC_L2, true>), grid, dim3(kRbThreads), lds, st, p);
+    } else {
+        VA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(prefilter_rb_kernel<VSAG_AMD_METRIC_IP, true>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        hipLaunchKernelGGL((prefilter_rb_kernel<VSAG_AMD_METRIC_IP, true>), grid, dim3(kRbThreads), lds, st, p);
     }
     timing_end(st);
     VA_HIP(hipGetLastError());

@@ -543,12 +543,27 @@ merge_partials_kernel(const uint64_t* partial, const uint32_t* partial_cnt, cons
         }
         const uint64_t kth = block_kth_smallest(pool, n, k, scratch);
         if (total <= pool_keys) {
-            // The k smallest (all of them when fewer than k) go to the front of the output area.
+            // The k smallest (all of them when fewer than k) go to the front of the output area: what lies below the
+            // k-th first, then as many copies of the k-th key as still fit (a list probed twice by one query brings
+            // every key twice).
             for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
                 uint64_t key = pool[i];
-                if (key <= kth) {
+                if (key < kth) {
                     lds[atomicAdd(&nout, 1U)] = key;
                 }
+            }
+            __syncthreads();
+            for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) {
+                if (pool[i] == kth) {
+                    const uint32_t pos = atomicAdd(&nout, 1U);
+                    if (pos < sort_room) {
+                        lds[pos] = kth;
+                    }
+                }
+            }
+            __syncthreads();
+            if (threadIdx.x == 0 && nout > sort_room) {
+                nout = sort_room;
             }
             break;
         }
