@@ -326,18 +326,20 @@ def test_k_above_one_device_scan(lib, name, params, search):
     idx.close()
 
 
+@pytest.mark.parametrize("quant,metric", [("sq4_uniform", "l2"), ("sq8_uniform", "ip"), ("sq8", "l2"), ("sq8", "cosine"),
+                                          ("rabitq", "l2")])
 @pytest.mark.parametrize("reorder", [True, False])
-def test_ivf_large_batch_equals_one_by_one(lib, reorder):
-    """A batch large enough for the matrix-core pass over sq4_uniform posting lists returns what single queries
-    (chunked streaming scan) return."""
+def test_ivf_large_batch_equals_one_by_one(lib, reorder, quant, metric):
+    """A batch large enough for the matrix-core pass over the posting lists (sq4_uniform, sq8_uniform, sq8, rabitq)
+    returns what single queries (chunked streaming scan) return."""
     n, d, nq, k = 60000, 64, 2200, 10
     x = vectors(n, d, normalize=False)
     q = vectors(nq, d, seed=165, normalize=False)
     labels = np.arange(n, dtype=np.int64) * 2 + 1
-    params = dict(buckets_count=64, base_quantization_type="sq4_uniform", train_sample_count=20000)
+    params = dict(buckets_count=64, base_quantization_type=quant, train_sample_count=20000)
     if reorder:
         params.update(use_reorder=True, precise_quantization_type="fp32")
-    idx = make("ivf", d, "l2", **params)
+    idx = make("ivf", d, metric, **params)
     assert idx.build(x, labels, n, d) == 0
     search = json.dumps({"ivf": {"scan_buckets_count": 16, "factor": 4.0}})
     ids, dists = idx.knn_search_batch(q, k, search)
