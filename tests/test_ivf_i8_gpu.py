@@ -63,7 +63,9 @@ def test_matrix_core_columns_equal_streaming(lib, n, d, nlist, nq, nprobe, kcand
 def test_overflowing_lists_fall_back_to_streaming(lib):
     """Queries routed to a far list first: the bound the first column leaves is so loose that the other lists hold
     hundreds of better codes, more than a private list takes; those queries go back to the streaming kernel."""
-    n, d, nlist, nq, nprobe, kcand = 40000, 64, 8, 9000, 4, 10
+    # 12 000 queries x 3 columns: more gated pairs than the direct fallback launch takes (32 768), so the streaming
+    # kernel serves them over the per-list grouping
+    n, d, nlist, nq, nprobe, kcand = 40000, 64, 8, 12000, 4, 10
     x, q, cent, labels, codes, (l, dd), st = _case(11, n, d, nlist, nq, components=8, sigma=0.02)
     routed, _ = orc.ivf_route(cent, q, nlist)
     buckets = np.ascontiguousarray(routed[:, [nlist - 1, 0, 1, 2]])  # farthest list first, then the nearest three
