@@ -253,9 +253,31 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
     };
 
     // The query group, once: chunk c of query q to qs[c][q].
-    for (uint32_t i = tid; i < nchunks * kRbQueries; i += blockDim.x) {
-        const uint32_t ql = i / nchunks, c = i % nchunks;
-        qs[c * kRbQueries + ql] = p.qbytes[query_row(ql) * nchunks + c];
+    if constexpr (LISTS) {
+        // A list item lives for a few tiles per wave only: the rows are fetched four loads at a time, so that the
+        // gather takes a few memory round trips instead of one per 16 bytes.
+        const uint32_t total = nchunks * kRbQueries;
+        for (uint32_t i0 = tid; i0 < total; i0 += 4 * blockDim.x) {
+            uint4 v[4];
+#pragma unroll
+            for (uint32_t r = 0; r < 4; ++r) {
+                const uint32_t i = i0 + r * blockDim.x;
+                const uint32_t ic = i < total ? i : total - 1;
+                v[r] = p.qbytes[query_row(ic / nchunks) * nchunks + ic % nchunks];
+            }
+#pragma unroll
+            for (uint32_t r = 0; r < 4; ++r) {
+                const uint32_t i = i0 + r * blockDim.x;
+                if (i < total) {
+                    qs[(i % nchunks) * kRbQueries + i / nchunks] = v[r];
+                }
+            }
+        }
+    } else {
+        for (uint32_t i = tid; i < nchunks * kRbQueries; i += blockDim.x) {
+            const uint32_t ql = i / nchunks, c = i % nchunks;
+            qs[c * kRbQueries + ql] = p.qbytes[query_row(ql) * nchunks + c];
+        }
     }
     float u1[4], u2[4], u3[4], u4[4];
     uint32_t ncand[4] = {0, 0, 0, 0};
@@ -325,6 +347,7 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
         const uint64_t code_mask = __ballot(holds_code);
         wave_lds_fence();
 
+        uint32_t tile_hits[4] = {0, 0, 0, 0};
         intx16 acc[4][2];
 #pragma unroll
         for (int qb = 0; qb < 4; ++qb) {
@@ -397,6 +420,12 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
                         for (int j = 0; j < 4; ++j) {
                             hits |= pass[j] ? 1U << j : 0U;
                         }
+                        if constexpr (LISTS) {
+                            // Bit 16 i + 4 gq + j of the tile's verdicts for this lane's pair of block qb; appended
+                            // after the tile, one atomic per pair instead of one per hit.
+                            tile_hits[qb] |= hits << (16 * i + 4 * gq);
+                            continue;
+                        }
                         const uint64_t q = q0 + 32 * qb + l32;
                         uint32_t* list = LISTS ? nullptr : p.cand + ((q < p.nq ? q : 0) * sub_lists + my_sub) * p.sub_cap;
                         while (hits != 0) {
@@ -415,6 +444,47 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
                                 }
                             }
                         }
+                    }
+                }
+            }
+        }
+        if constexpr (LISTS) {
+            // Room for all hits of a pair in one go: the four counts are asked for before the first answer is needed.
+            uint32_t count[4], base[4];
+            uint64_t list[4];
+#pragma unroll
+            for (int qb = 0; qb < 4; ++qb) {
+                uint32_t mask = tile_hits[qb];
+                // bit 16 i + 4 gq + j is code 32 i + 8 gq + 4 half + j
+                uint32_t keep = 0;
+                for (uint32_t m = mask; m != 0; m &= m - 1) {
+                    const uint32_t bit = static_cast<uint32_t>(__builtin_ctz(m));
+                    const uint32_t code = 32 * (bit >> 4) + 8 * ((bit >> 2) & 3U) + 4 * half + (bit & 3U);
+                    if (((code_mask >> code) & 1ULL) != 0 && ((special_mask >> code) & 1ULL) == 0) {
+                        keep |= 1U << bit;
+                    }
+                }
+                const uint32_t first = pair_list[32 * qb + l32];
+                keep = first != 0xFFFFFFFFU ? keep : 0U;
+                tile_hits[qb] = keep;
+                count[qb] = static_cast<uint32_t>(__builtin_popcount(keep));
+                list[qb] = static_cast<uint64_t>(first) + 2 * (wave & 3U) + half;
+                base[qb] = count[qb] != 0 ? atomicAdd(&p.partial_cnt[list[qb]], count[qb]) : 0U;
+            }
+#pragma unroll
+            for (int qb = 0; qb < 4; ++qb) {
+                uint32_t pos = base[qb];
+                for (uint32_t m = tile_hits[qb]; m != 0; m &= m - 1) {
+                    const uint32_t bit = static_cast<uint32_t>(__builtin_ctz(m));
+                    const uint32_t code = 32 * (bit >> 4) + 8 * ((bit >> 2) & 3U) + 4 * half + (bit & 3U);
+                    if (pos < p.k) {
+                        p.partial[list[qb] * p.k + pos] = tile * kWave + code;
+                    }
+                    ++pos;
+                }
+                if (count[qb] != 0 && pos > p.k) {
+                    if (atomicExch(&p.gate[pair_q[32 * qb + l32]], 1U) == 0U) {
+                        atomicAdd(&p.gate[p.dummy_query], 1U);
                     }
                 }
             }
