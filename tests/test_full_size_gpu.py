@@ -302,6 +302,97 @@ def test_ivf_sq4_uniform_10m(lib):
     cstore.destroy()
 
 
+def test_ivf_sq8_and_rabitq_lists_10m(lib):
+    """configs[3]'s rows, lists and probes with sq8 and with RaBitQ codes in the lists: the probe columns behind the
+    first go through the int8 matrix cores (two planes per query / expanded code bits), and what they return must be
+    the streaming kernel's result bit for bit, the checker's on a sample, and independent of the batch split."""
+    n, d, nq, nlist, nprobe, kcand = 10000000, 128, 1024, 4096, 64, 100
+    means = mt(315).random((10000, d), dtype=np.float32)
+    x_dev = capi.DeviceBuffer(n * d * 4)
+    pick = np.sort(mt(7).choice(n, nlist, replace=False))
+    init = np.empty((nlist, d), np.float32)
+    for s, blk in mixture_chunks(47, n, d, means, 0.05):
+        capi.check(lib.vsag_amd_memcpy_h2d(x_dev.ptr + s * d * 4, blk.ctypes.data, blk.nbytes, None))
+        lo, hi = np.searchsorted(pick, [s, s + blk.shape[0]])
+        init[lo:hi] = blk[pick[lo:hi] - s]
+    q, _ = mixture(315, 165, nq, d, 10000, 0.05, means=means)
+    ns = 64 * nlist
+    cent = dev(init)
+    slabels = capi.DeviceBuffer(ns * 4)
+    wsb = lib.vsag_amd_kmeans_run_workspace_bytes(ns, d, nlist)
+    ws = capi.DeviceBuffer(wsb)
+    capi.check(lib.vsag_amd_kmeans_run(x_dev.ptr, ns, d, cent.ptr, nlist, 10, 7, slabels.ptr, None, ws.ptr, wsb, None))
+    ws.free()
+    labels = capi.DeviceBuffer(n * 4)
+    wsb = lib.vsag_amd_kmeans_assign_workspace_bytes(n, d, nlist)
+    ws = capi.DeviceBuffer(wsb)
+    capi.check(lib.vsag_amd_kmeans_assign(x_dev.ptr, n, d, cent.ptr, nlist, labels.ptr, None, None, ws.ptr, wsb, None))
+    ws.free()
+    hlabels = labels.to_numpy(np.int32, (n,))
+    hcent = cent.to_numpy(np.float32, (nlist, d))
+    offsets, order = orc.ivf_build_lists(hlabels, nlist)
+    b, _ = orc.ivf_route(hcent, q, nprobe)
+    info = capi.C.c_int()
+
+    def both(lists):
+        fast = lists.ivf_scan(q, b, kcand)
+        lib.vsag_amd_last_scan_info(capi.C.byref(info), None, None)
+        assert info.value == 256, "the int8 pass over the posting lists did not run"
+        check_result_shape(fast[0], fast[1], n)
+        capi.check(lib.vsag_amd_store_set_scan_contraction(lists.handle, -1))
+        plain = lists.ivf_scan(q, b, kcand)
+        capi.check(lib.vsag_amd_store_set_scan_contraction(lists.handle, -2))
+        assert np.array_equal(plain[0], fast[0]) and np.array_equal(plain[1].view(np.uint32), fast[1].view(np.uint32))
+        for s, e in ((0, 1), (10, 17), (1000, 1024)):
+            ci, cd = lists.ivf_scan(q[s:e], b[s:e], kcand)
+            assert np.array_equal(ci, fast[0][s:e]) and np.array_equal(cd.view(np.uint32), fast[1][s:e].view(np.uint32))
+        return fast
+
+    # sq8: a range per dimension
+    lb_dev, diff_dev = capi.DeviceBuffer(d * 4), capi.DeviceBuffer(d * 4)
+    wsb = lib.vsag_amd_sq_train_workspace_bytes(ns, d, 0)
+    ws = capi.DeviceBuffer(wsb)
+    capi.check(lib.vsag_amd_sq_train(x_dev.ptr, ns, d, 8, capi.METRIC_L2, capi.SQ_TRAIN_TRUNC_BOUND, 0.05, 0, lb_dev.ptr,
+                                     diff_dev.ptr, ws.ptr, wsb, None))
+    ws.free()
+    codes = capi.DeviceBuffer(n * d)
+    capi.check(lib.vsag_amd_sq_encode(x_dev.ptr, n, d, 8, capi.METRIC_L2, lb_dev.ptr, diff_dev.ptr, codes.ptr, None))
+    hlb, hdiff = lb_dev.to_numpy(np.float32, (d,)), diff_dev.to_numpy(np.float32, (d,))
+    hcodes = codes.to_numpy(np.uint8, (n, d))
+    lists = Store(capi.KIND_SQ8, capi.METRIC_L2, d, lb=hlb, diff=hdiff)
+    capi.check(lib.vsag_amd_store_set_lists(lists.handle, codes.ptr, labels.ptr, n, nlist, None))
+    capi.synchronize()
+    codes.free()
+    fast = both(lists)
+    oi, od = orc.ivf_scan(orc.SQ8, orc.L2, d, hcodes[order], offsets, order, q[:32], b[:32], kcand, lb=hlb, diff=hdiff)
+    assert_topk_close(fast[0][:32], fast[1][:32], oi, od, atol=4e-6, label="ivf sq8 10M")
+    lists.destroy()
+    del hcodes
+
+    # RaBitQ: 1-bit codes, 4-bit queries, a seeded rotation
+    g = mt(316).standard_normal((d, d))
+    rot, r = np.linalg.qr(g)
+    rot = (rot * np.sign(np.diag(r))).astype(np.float32)
+    rot_dev, cen = dev(rot), capi.DeviceBuffer(d * 4)
+    capi.check(lib.vsag_amd_rabitq_train(x_dev.ptr, ns, d, rot_dev.ptr, cen.ptr, None))
+    cs = int(lib.vsag_amd_code_size(capi.KIND_RABITQ, capi.METRIC_L2, d, 4))
+    codes = capi.DeviceBuffer(n * cs)
+    capi.check(lib.vsag_amd_rabitq_encode(x_dev.ptr, n, d, rot_dev.ptr, cen.ptr, capi.METRIC_L2, 4, codes.ptr, None))
+    hcen = cen.to_numpy(np.float32, (d,))
+    hcodes = codes.to_numpy(np.uint8, (n, cs))
+    lists = Store(capi.KIND_RABITQ, capi.METRIC_L2, d, rot=rot, centroid=hcen, qbits=4)
+    capi.check(lib.vsag_amd_store_set_lists(lists.handle, codes.ptr, labels.ptr, n, nlist, None))
+    capi.synchronize()
+    codes.free()
+    fast = both(lists)
+    qcodes = orc.rabitq_process_query(q[:32], rot, hcen, orc.L2)
+    oi, od = orc.ivf_scan(orc.RABITQ, orc.L2, d, hcodes[order], offsets, order, qcodes, b[:32], kcand)
+    assert np.array_equal(od.view(np.uint32), fast[1][:32].view(np.uint32))
+    lists.destroy()
+    for x in (x_dev, cent, slabels, labels, lb_dev, diff_dev, rot_dev, cen):
+        x.free()
+
+
 def test_rabitq_scan_5m_x_768(lib):
     """configs[4]: 5 000 000 x 768 unit rows, 1-bit codes, 4-bit queries, inner product, 200 candidates."""
     n, d, nq, kcand = 5000000, 768, 512, 200
