@@ -85,6 +85,40 @@ def test_sq8_int8_planes_hold_for_awkward_queries(lib, modes, metric, d):
 
 
 @pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
+@pytest.mark.parametrize("n,d,nq,k", [(40000, 128, 300, 10), (20001, 100, 129, 100), (9000, 31, 640, 7),
+                                      (30000, 16, 320, 10)])
+def test_sq4_contraction_equals_streaming(lib, modes, metric, n, d, nq, k):
+    """sq4 (a range per dimension, two 4-bit values per byte): the two int8 planes of a query against the nibbles as
+    they are; awkward queries among the ordinary ones."""
+    rng = np.random.default_rng(n + d + k + metric)
+    x, means = gaussian_mixture(rng, n, d, 30, 0.05)
+    q, _ = gaussian_mixture(rng, nq, d, 30, 0.05, means=means)
+    if metric != orc.COSINE:
+        q[0] = 0.0
+        q[1] = 1e-20
+    q[2] *= 1e6
+    q[3] *= 1e-6
+    q[5:40] = x[5:40]
+    q[60:80] += 100.0
+    lb, diff = orc.sq_train(x, 4, metric)
+    codes = orc.sq_encode(x, 4, lb, diff, metric)
+    st = Store(capi.KIND_SQ4, metric, d, lb=lb, diff=diff)
+    st.append(codes[:n // 3])
+    st.append(codes[n // 3:])  # the per-code terms follow appends
+    plain, fast, tile = modes(st, q, k)
+    assert tile == 256, "the contraction path did not run"
+    assert same(plain, fast)
+    # asking for the fp32 matrix cores finds no route for this kind and the int8 one serves
+    plain, fast, tile = modes(st, q, k, 2)
+    assert tile == 256 and same(plain, fast)
+    om, oq = (orc.IP, (q[100:116] / np.linalg.norm(q[100:116], axis=1, keepdims=True)).astype(np.float32)) \
+        if metric == orc.COSINE else (metric, q[100:116])
+    ri, rd = orc.flat_scan_topk(orc.SQ4, om, d, codes, oq, k, lb=lb, diff=diff)
+    assert_topk_close(fast[0][100:116], fast[1][100:116], ri, rd, atol=4e-6, label="sq4 contraction")
+    st.destroy()
+
+
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
 @pytest.mark.parametrize("n,d,nq,k", [(30000, 128, 200, 10), (7000, 65, 77, 32)])
 def test_fp32_contraction_equals_streaming(lib, modes, metric, n, d, nq, k):
     rng = np.random.default_rng(n + d + k + metric)

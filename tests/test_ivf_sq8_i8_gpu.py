@@ -1,6 +1,6 @@
-"""Large batches on sq8 posting lists of at most 128 dimensions: the probe columns behind the first are pre-selected on
-the int8 matrix cores (two int8 planes per query, one scale for the batch) and what passes is rescored with the
-streaming kernel's arithmetic, so ids and distance bits must equal the streaming scan's."""
+"""Large batches on sq8 (and sq4) posting lists of at most 128 dimensions: the probe columns behind the first are
+pre-selected on the int8 matrix cores (two int8 planes per query, one scale for the batch) and what passes is rescored
+with the streaming kernel's arithmetic, so ids and distance bits must equal the streaming scan's."""
 import numpy as np
 import pytest
 
@@ -11,15 +11,15 @@ from vsag_amd import capi
 pytestmark = pytest.mark.gpu
 
 
-def _case(seed, n, d, nlist, nq, components=40, sigma=0.05, metric=orc.L2):
+def _case(seed, n, d, nlist, nq, components=40, sigma=0.05, metric=orc.L2, bits=8):
     rng = np.random.default_rng(seed)
     x, means = gaussian_mixture(rng, n, d, components, sigma)
     q, _ = gaussian_mixture(rng, nq, d, components, sigma, means=means)
     cent = x[rng.choice(n, nlist, replace=False)].copy()
     labels, _, _ = orc.kmeans_assign(x, cent)
-    lb, diff = orc.sq_train(x, 8, metric)
-    codes = orc.sq_encode(x, 8, lb, diff, metric)
-    st = Store(capi.KIND_SQ8, metric, d, lb=lb, diff=diff)
+    lb, diff = orc.sq_train(x, bits, metric)
+    codes = orc.sq_encode(x, bits, lb, diff, metric)
+    st = Store(capi.KIND_SQ8 if bits == 8 else capi.KIND_SQ4, metric, d, lb=lb, diff=diff)
     st.set_lists(codes, labels, nlist)
     return x, q, cent, labels, codes, (lb, diff), st
 
@@ -40,11 +40,12 @@ def _same(a, b):
     return np.array_equal(a[0], b[0]) and np.array_equal(a[1].view(np.uint32), b[1].view(np.uint32))
 
 
+@pytest.mark.parametrize("bits", [8, 4])
 @pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
 @pytest.mark.parametrize("n,d,nlist,nq,nprobe,kcand", [(60000, 128, 64, 2100, 16, 100), (30000, 100, 37, 4500, 8, 10),
                                                        (20000, 33, 16, 9000, 4, 32), (20000, 7, 16, 9000, 4, 5)])
-def test_matrix_core_columns_equal_streaming(lib, metric, n, d, nlist, nq, nprobe, kcand):
-    x, q, cent, labels, codes, (lb, diff), st = _case(n + d + metric, n, d, nlist, nq, metric=metric)
+def test_matrix_core_columns_equal_streaming(lib, bits, metric, n, d, nlist, nq, nprobe, kcand):
+    x, q, cent, labels, codes, (lb, diff), st = _case(n + d + metric, n, d, nlist, nq, metric=metric, bits=bits)
     buckets, _ = orc.ivf_route(cent, q, nprobe)
     buckets = buckets.copy()
     buckets[70:73, 0] = -1      # three queries without a first list: no bound, served by the direct fallback launch
@@ -56,7 +57,8 @@ def test_matrix_core_columns_equal_streaming(lib, metric, n, d, nlist, nq, nprob
     qs, om = q[:64], metric
     if metric == orc.COSINE:  # inner product of the unit query with the codes of the unit rows
         qs, om = (qs / np.linalg.norm(qs, axis=1, keepdims=True)).astype(np.float32), orc.IP
-    rids, rds = orc.ivf_scan(orc.SQ8, om, d, codes[order], offsets, order, qs, buckets[:64], kcand, lb=lb, diff=diff)
+    rids, rds = orc.ivf_scan(orc.SQ8 if bits == 8 else orc.SQ4, om, d, codes[order], offsets, order, qs, buckets[:64], kcand,
+                             lb=lb, diff=diff)
     assert_topk_close(fast[0][:64], fast[1][:64], rids, rds, atol=4e-6, label="ivf sq8 on the matrix cores")
     st.destroy()
 
@@ -103,7 +105,8 @@ def test_queries_of_very_different_sizes_share_one_scale(lib):
     st.destroy()
 
 
-def test_lists_that_grew_by_appending(lib):
+@pytest.mark.parametrize("bits", [8, 4])
+def test_lists_that_grew_by_appending(lib, bits):
     """The per-slot terms are renewed when codes are appended (lists move, room behind each list holds no code)."""
     n, d, nlist, nq, nprobe, kcand = 40000, 96, 24, 6000, 6, 20
     rng = np.random.default_rng(2)
@@ -111,14 +114,15 @@ def test_lists_that_grew_by_appending(lib):
     q, _ = gaussian_mixture(rng, nq, d, 30, 0.05, means=means)
     cent = x[rng.choice(n, nlist, replace=False)].copy()
     labels, _, _ = orc.kmeans_assign(x, cent)
-    lb, diff = orc.sq_train(x, 8)
-    codes = orc.sq_encode(x, 8, lb, diff)
-    st = Store(capi.KIND_SQ8, orc.L2, d, lb=lb, diff=diff)
+    kind = capi.KIND_SQ8 if bits == 8 else capi.KIND_SQ4
+    lb, diff = orc.sq_train(x, bits)
+    codes = orc.sq_encode(x, bits, lb, diff)
+    st = Store(kind, orc.L2, d, lb=lb, diff=diff)
     half = n // 2
     st.set_lists(codes[:half], labels[:half], nlist)
     st.append_lists(codes[half:half + 7000], labels[half:half + 7000])
     st.append_lists(codes[half + 7000:], labels[half + 7000:])
-    whole = Store(capi.KIND_SQ8, orc.L2, d, lb=lb, diff=diff)
+    whole = Store(kind, orc.L2, d, lb=lb, diff=diff)
     whole.set_lists(codes, labels, nlist)
     buckets, _ = orc.ivf_route(cent, q, nprobe)
     plain, fast = _both(lib, st, q, buckets, kcand)

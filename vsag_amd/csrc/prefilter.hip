@@ -310,6 +310,16 @@ code_term_kernel(const uint4* tiles, uint32_t G, const float* scale, uint64_t fi
                     }
                     s = fma(y, y, s);
                 }
+            } else if constexpr (KIND == VSAG_AMD_KIND_SQ4) {
+                // byte b of the granule: dimension 32 j + 2 b in its low nibble, 32 j + 2 b + 1 in its high one
+#pragma unroll
+                for (int e = 0; e < 32; ++e) {
+                    double y = static_cast<double>((w[e >> 3] >> (8 * ((e >> 1) & 3) + 4 * (e & 1))) & 0xfU);
+                    if (scale != nullptr) {
+                        y *= static_cast<double>(scale[32 * j + e]);
+                    }
+                    s = fma(y, y, s);
+                }
             } else {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -440,8 +450,10 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
             acc_reset(acc);
             const uint4* row = r.rows != nullptr ? r.rows + static_cast<uint64_t>(slot) * a.G : nullptr;
             // A few granules are fetched before the first is used: a candidate's loads wait for memory together.
-            // (sq8 l2 holds scale and query of every dimension in flight in scalar registers: two granules' worth.)
-            constexpr uint32_t kAhead = KIND == VSAG_AMD_KIND_SQ8 && METRIC == VSAG_AMD_METRIC_L2 ? 2 : 4;
+            // (sq8 l2 holds scale and query of every dimension in flight in scalar registers: two granules' worth; an sq4
+            // granule is 32 dimensions.)
+            constexpr uint32_t kAhead = KIND == VSAG_AMD_KIND_SQ4 ? (METRIC == VSAG_AMD_METRIC_L2 ? 1 : 2)
+                                       : (KIND == VSAG_AMD_KIND_SQ8 && METRIC == VSAG_AMD_METRIC_L2 ? 2 : 4);
             for (uint32_t j0 = 0; j0 < a.G; j0 += kAhead) {
                 uint4 c[kAhead];
 #pragma unroll
@@ -616,7 +628,8 @@ ivf_rescore_kernel(ScanArgs a, IvfRescoreArgs r) {
             const uint32_t ln = slot & 63;
             Acc<KIND, 1> acc;
             acc_reset(acc);
-            constexpr uint32_t kAhead = KIND == VSAG_AMD_KIND_SQ8 && METRIC == VSAG_AMD_METRIC_L2 ? 2 : 4;
+            constexpr uint32_t kAhead = KIND == VSAG_AMD_KIND_SQ4 ? (METRIC == VSAG_AMD_METRIC_L2 ? 1 : 2)
+                                       : (KIND == VSAG_AMD_KIND_SQ8 && METRIC == VSAG_AMD_METRIC_L2 ? 2 : 4);
             for (uint32_t j0 = 0; j0 < a.G; j0 += kAhead) {
                 uint4 c4[kAhead];
 #pragma unroll
@@ -680,9 +693,9 @@ ivf_rescore_capacity() {
 int
 launch_ivf_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
                    uint32_t per_pair, uint64_t* partial, uint32_t* partial_cnt, const uint32_t* bound, hipStream_t st) {
-    if ((s->kind != VSAG_AMD_KIND_SQ8 && s->kind != VSAG_AMD_KIND_RABITQ) || kcand > kIvfRescoreGather ||
-        s->ids_dev == nullptr) {
-        return fail(VSAG_AMD_INVALID_ARGUMENT, "rescoring of list records: sq8 or rabitq lists with kcand <= %u only",
+    if ((s->kind != VSAG_AMD_KIND_SQ8 && s->kind != VSAG_AMD_KIND_SQ4 && s->kind != VSAG_AMD_KIND_RABITQ) ||
+        kcand > kIvfRescoreGather || s->ids_dev == nullptr) {
+        return fail(VSAG_AMD_INVALID_ARGUMENT, "rescoring of list records: sq8, sq4 or rabitq lists with kcand <= %u only",
                     kIvfRescoreGather);
     }
     IvfRescoreArgs r{};
@@ -700,6 +713,12 @@ launch_ivf_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint
             hipLaunchKernelGGL((ivf_rescore_kernel<VSAG_AMD_KIND_RABITQ, VSAG_AMD_METRIC_L2>), grid, dim3(kWave), 0, st, a, r);
         } else {
             hipLaunchKernelGGL((ivf_rescore_kernel<VSAG_AMD_KIND_RABITQ, VSAG_AMD_METRIC_IP>), grid, dim3(kWave), 0, st, a, r);
+        }
+    } else if (s->kind == VSAG_AMD_KIND_SQ4) {
+        if (s->metric == VSAG_AMD_METRIC_L2) {
+            hipLaunchKernelGGL((ivf_rescore_kernel<VSAG_AMD_KIND_SQ4, VSAG_AMD_METRIC_L2>), grid, dim3(kWave), 0, st, a, r);
+        } else {
+            hipLaunchKernelGGL((ivf_rescore_kernel<VSAG_AMD_KIND_SQ4, VSAG_AMD_METRIC_IP>), grid, dim3(kWave), 0, st, a, r);
         }
     } else if (s->metric == VSAG_AMD_METRIC_L2) {
         hipLaunchKernelGGL((ivf_rescore_kernel<VSAG_AMD_KIND_SQ8, VSAG_AMD_METRIC_L2>), grid, dim3(kWave), 0, st, a, r);
@@ -723,7 +742,7 @@ prefilter_supports(const vsag_amd_store* s) {
     if (prefilter_rb_supports(s)) {
         return true;
     }
-    if (s->kind == VSAG_AMD_KIND_SQ8_UNIFORM || s->kind == VSAG_AMD_KIND_SQ4_UNIFORM) {
+    if (s->kind == VSAG_AMD_KIND_SQ8_UNIFORM || s->kind == VSAG_AMD_KIND_SQ4_UNIFORM || s->kind == VSAG_AMD_KIND_SQ4) {
         return prefilter_i8_supports(s);  // the int8 matrix cores or nothing
     }
     return s->nlist == 0 && (s->kind == VSAG_AMD_KIND_FP32 || s->kind == VSAG_AMD_KIND_SQ8) && s->pf_term != nullptr;
@@ -753,6 +772,10 @@ launch_code_terms(vsag_amd_store* s, uint64_t first, uint64_t count, hipStream_t
     } else if (s->kind == VSAG_AMD_KIND_SQ8) {
         const float* scale = s->metric == VSAG_AMD_METRIC_L2 ? s->scale_dev : nullptr;
         hipLaunchKernelGGL(code_term_kernel<VSAG_AMD_KIND_SQ8>, grid, dim3(256), 0, st, s->tiles, s->G, scale, first,
+                           count, s->pf_term, s->pf_ymax);
+    } else if (s->kind == VSAG_AMD_KIND_SQ4) {
+        const float* scale = s->metric == VSAG_AMD_METRIC_L2 ? s->scale_dev : nullptr;
+        hipLaunchKernelGGL(code_term_kernel<VSAG_AMD_KIND_SQ4>, grid, dim3(256), 0, st, s->tiles, s->G, scale, first,
                            count, s->pf_term, s->pf_ymax);
     } else {
         hipLaunchKernelGGL(code_term_kernel<VSAG_AMD_KIND_FP32>, grid, dim3(256), 0, st, s->tiles, s->G,
@@ -806,6 +829,8 @@ launch_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t
     const size_t lds = S * 8 + (sub_lists != 0 ? r.gather * 4 : 0);
     if (s->kind == VSAG_AMD_KIND_SQ8) {
         launch_rescore_m<VSAG_AMD_KIND_SQ8>(s->metric, rgrid, lds, st, a, r);
+    } else if (s->kind == VSAG_AMD_KIND_SQ4) {
+        launch_rescore_m<VSAG_AMD_KIND_SQ4>(s->metric, rgrid, lds, st, a, r);
     } else if (s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
         launch_rescore_m<VSAG_AMD_KIND_SQ8_UNIFORM>(s->metric, rgrid, lds, st, a, r);
     } else if (s->kind == VSAG_AMD_KIND_SQ4_UNIFORM) {

@@ -1,5 +1,5 @@
-// Pre-selection for large query batches on a flat sq8 (or sq8_uniform, see UniformQuantizeArgs) store of at most 128
-// dimensions, on the int8 matrix cores.
+// Pre-selection for large query batches on a flat sq8 (or sq8_uniform, see UniformQuantizeArgs; or sq4, see
+// QuantizeArgs::nibbles) store of at most 128 dimensions, on the int8 matrix cores.
 //
 // The streaming distance of an sq8 code is a function of <b, c>: c the code bytes (0..255), b the query folded
 // with the per-dimension scale (l2: b_d = (q_d - lb_d) scale_d, ip: b_d = q_d scale_d).  Each query row b is split
@@ -45,6 +45,11 @@ struct QuantizeArgs {
     const float* qmeta;   // ip: sum q_d lb_d per query
     uint32_t qmeta_stride;
     int is_l2;
+    // sq4: the codes hold two 4-bit values per byte (byte b of a 32-dimension granule: dimension 2 b low, 2 b + 1
+    // high).  They are staged as they are (0..15 needs no shift to fit a signed byte), a granule as its low and its high
+    // nibbles, so operand position 16 g + p (staged granule g, byte p) is dimension 32 (g / 2) + 2 p + g % 2, and
+    // the terms that make up for the shift by 128 of byte codes fall away.
+    int nibbles;
     const uint32_t* bound;      // per query, ordered-float bits; 0xFFFFFFFF = none yet
     const uint32_t* ymax_bits;  // largest |y| of the store (l2: scaled codes, ip: raw codes)
     uint64_t nq, nq_pad;
@@ -72,6 +77,8 @@ query_tau_i8(const QuantizeArgs& p, uint64_t q, double q_err, double w, double a
     constexpr double kU = 5.9604644775390625e-8;  // 2^-24, the unit roundoff of fp32
     const double bd = static_cast<double>(ordered_to_float(bbits));
     const double ymax = static_cast<double>(__uint_as_float(*p.ymax_bits)) * (1.0 + 1.0e-6);
+    const double shift = p.nibbles ? 0.0 : 128.0;  // the codes are staged as c - shift
+    const double cmax = p.nibbles ? 15.0 : 255.0;  // largest code value
     if (p.is_l2) {
         // The streaming kernel sums fl(fl(c s) - a)^2 in fp32: off from the real sum S by at most
         // 2u sum |y - a| |y| + (n + 2) u S <= 2u sqrt(S) |y| + (n + 2) u S to first order; twice that is allowed for.
@@ -79,9 +86,9 @@ query_tau_i8(const QuantizeArgs& p, uint64_t q, double q_err, double w, double a
         const double e_stream = 4.0 * kU * sqrt(s_abs) * ymax + 2.0 * (p.kdim + 4) * kU * s_abs;
         // |y|^2 per code is accumulated in double and rounded once.
         const double e_term = 2.0 * kU * ymax * ymax;
-        // dist = a2 + |y|^2 - 2 s2 (M + 128 w) - 2 <e, c>, M the integer the matrix cores deliver: the pair can matter
+        // dist = a2 + |y|^2 - 2 s2 (M + shift w) - 2 <e, c>, M the integer the matrix cores deliver: the pair can matter
         // when |y|^2 - 2 s2 M <= t_real, i.e. M >= |y|^2 / (2 s2) - t_real / (2 s2).
-        const double t_real = bd - a2 + 256.0 * s2 * w + 2.0 * q_err + e_stream + e_term;
+        const double t_real = bd - a2 + 2.0 * shift * s2 * w + 2.0 * q_err + e_stream + e_term;
         // The kernel subtracts I = rn(fl(|y|^2 inv)) from M, inv = fl(1 / (2 s2)) (ginv): I differs from the real
         // |y|^2 / (2 s2) by at most a half plus two fp32 roundings of a value of at most ymax^2 / (2 s2); the kernel
         // clamps I from above only, which admits more.  So M - I >= floor(-t_real / (2 s2) - that - 1) keeps every
@@ -95,13 +102,13 @@ query_tau_i8(const QuantizeArgs& p, uint64_t q, double q_err, double w, double a
     // dist = 1 - (fl(sum c a) + qmeta): the fp32 sum is off by at most n u sum |c a|, the two closing
     // operations by u of their results; twice that is allowed for.
     const double qm = p.qmeta != nullptr ? static_cast<double>(p.qmeta[q * p.qmeta_stride]) : 0.0;
-    const double m = fmin(255.0 * b1, sqrt(a2) * ymax * (1.0 + 1.0e-6));
+    const double m = fmin(cmax * b1, sqrt(a2) * ymax * (1.0 + 1.0e-6));
     const double e_stream = 2.0 * (p.kdim + 2) * kU * m + 4.0 * kU * (m + fabs(qm) + 1.0 + fabs(bd));
-    // 1 - qm - s2 (T + 128 w) - <e, c> <= bd   <=>   T >= -(bd - 1 + qm + errors) / s2 - 128 w.
+    // 1 - qm - s2 (T + shift w) - <e, c> <= bd   <=>   T >= -(bd - 1 + qm + errors) / s2 - shift w.
     const double rhs = bd - 1.0 + qm + q_err + e_stream;
     int32_t ti;
     if (s2 > 0.0) {
-        const double x = floor(-rhs / s2 - 128.0 * w) - 2.0;
+        const double x = floor(-rhs / s2 - shift * w) - 2.0;
         ti = x >= 2147483647.0 ? 0x7FFFFFFF : (x <= -2147483648.0 ? static_cast<int32_t>(0x80000000U)
                                                                   : static_cast<int32_t>(x));
     } else {
@@ -228,8 +235,10 @@ quantize_queries_i8_kernel(QuantizeArgs p) {
         e_pos += e > 0.0 ? e : 0.0;
         e_neg += e < 0.0 ? -e : 0.0;
         w += whole;
-        out[lane + 64 * r] = static_cast<uint8_t>(static_cast<int8_t>(h));
-        out[128 + lane + 64 * r] = static_cast<uint8_t>(static_cast<int8_t>(l));
+        const uint32_t d = lane + 64 * r;
+        const uint32_t at = p.nibbles ? 16 * (2 * (d >> 5) + (d & 1U)) + ((d & 31U) >> 1) : d;
+        out[at] = static_cast<uint8_t>(static_cast<int8_t>(h));
+        out[128 + at] = static_cast<uint8_t>(static_cast<int8_t>(l));
     }
     e_pos = wave_sum_f64(e_pos);
     e_neg = wave_sum_f64(e_neg);
@@ -240,7 +249,8 @@ quantize_queries_i8_kernel(QuantizeArgs p) {
         return;
     }
     // |<e, c>| for any code, plus the rounding of the double arithmetic above.
-    const double q_err = 255.0 * fmax(e_pos, e_neg) + 1.0e-12 * 255.0 * b1;
+    const double cmax = p.nibbles ? 15.0 : 255.0;
+    const double q_err = cmax * fmax(e_pos, e_neg) + 1.0e-12 * cmax * b1;
     const bool usable = (b1 < 1.0e300) && (a2 < 1.0e300) && !bad_row && !(p.is_l2 && !(s2 > 0.0));
     if (p.scal != nullptr) {
         double* keep = p.scal + q * kI8Scalars;
@@ -730,7 +740,7 @@ prefilter_i8_kernel(PrefilterI8Args p) {
 
 bool
 prefilter_i8_supports(const vsag_amd_store* s) {
-    if (s->kind == VSAG_AMD_KIND_SQ4_UNIFORM) {
+    if (s->kind == VSAG_AMD_KIND_SQ4_UNIFORM || s->kind == VSAG_AMD_KIND_SQ4) {
         return s->nlist == 0 && s->pf_term != nullptr && s->dpad <= kI8Dims && s->G <= 4;
     }
     return (s->kind == VSAG_AMD_KIND_SQ8 || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) && s->nlist == 0 && s->pf_term != nullptr &&
@@ -740,7 +750,7 @@ prefilter_i8_supports(const vsag_amd_store* s) {
 size_t prefilter_i8_query_bytes(uint64_t nq);
 size_t prefilter_i8_scalar_floats(uint64_t nq);
 
-// ---- sq8 posting lists against large batches --------------------------------------------------------------------
+// ---- sq8 (and, NIBBLE, sq4) posting lists against large batches --------------------------------------------------------------------
 // The same two-plane test over the (query, list) pairs of an ivf search that the streaming kernel has already given a
 // bound (the probe columns behind the nearest list, see ivf_i8.hip for the work split this kernel shares: a
 // workgroup = a chunk of a list's tiles x up to 256 of the pairs that probe the list, four waves of 64 pairs).  The
@@ -795,7 +805,7 @@ struct IvfSq8Args {
     uint32_t* gate;              // per query: raised when one of its lists overflowed; gate[dummy_query] counts them
 };
 
-template <int TEST>
+template <int TEST, bool NIBBLE = false>
 __global__ void __launch_bounds__(256, 2)
 ivf_sq8_i8_kernel(IvfSq8Args p) {
     __shared__ I8Stage stage[2];
@@ -871,9 +881,10 @@ ivf_sq8_i8_kernel(IvfSq8Args p) {
             const uint32_t tile = tile_begin + sg * kI8StageTiles + tt;
             const bool real = tile < tile_end;
 #pragma unroll
-            for (int r = 0; r < 2; ++r) {
+            for (int r = 0; r < (NIBBLE ? 1 : 2); ++r) {
                 const uint32_t j = wave + 4 * r;
-                regs[tt][r] = make_uint4(0x80808080U, 0x80808080U, 0x80808080U, 0x80808080U);
+                const uint32_t none = NIBBLE ? 0U : 0x80808080U;
+                regs[tt][r] = make_uint4(none, none, none, none);
                 if (real && j < p.G) {
                     regs[tt][r] = p.tiles[(static_cast<uint64_t>(tile) * p.G + j) * kWave + lane];
                 }
@@ -891,11 +902,20 @@ ivf_sq8_i8_kernel(IvfSq8Args p) {
     auto park = [&](I8Stage& st) {
 #pragma unroll
         for (int tt = 0; tt < kI8StageTiles; ++tt) {
+            if constexpr (NIBBLE) {
+                // sq4: a granule is staged as two, its low and its high nibbles, as they are
+                const uint4 v = regs[tt][0];
+                const uint32_t m = 0x0F0F0F0FU;
+                st.codes[tt][(2 * wave) * kWave + lane] = make_uint4(v.x & m, v.y & m, v.z & m, v.w & m);
+                st.codes[tt][(2 * wave + 1) * kWave + lane] =
+                    make_uint4((v.x >> 4) & m, (v.y >> 4) & m, (v.z >> 4) & m, (v.w >> 4) & m);
+            } else {
 #pragma unroll
-            for (int r = 0; r < 2; ++r) {
-                const uint4 v = regs[tt][r];
-                st.codes[tt][(wave + 4 * r) * kWave + lane] =
-                    make_uint4(v.x ^ 0x80808080U, v.y ^ 0x80808080U, v.z ^ 0x80808080U, v.w ^ 0x80808080U);
+                for (int r = 0; r < 2; ++r) {
+                    const uint4 v = regs[tt][r];
+                    st.codes[tt][(wave + 4 * r) * kWave + lane] =
+                        make_uint4(v.x ^ 0x80808080U, v.y ^ 0x80808080U, v.z ^ 0x80808080U, v.w ^ 0x80808080U);
+                }
             }
             if constexpr (kTerm) {
                 if (wave == 0) {
@@ -1029,8 +1049,9 @@ ivf_sq8_i8_kernel(IvfSq8Args p) {
 
 bool
 ivf_sq8_i8_supports(const vsag_amd_store* s) {
-    return s->kind == VSAG_AMD_KIND_SQ8 && s->nlist > 0 && s->G <= 8 && s->dpad <= kI8Dims && s->pf_term != nullptr &&
-           s->pf_ymax != nullptr && s->residual_centroids_dev == nullptr;
+    const bool kind_ok = (s->kind == VSAG_AMD_KIND_SQ8 && s->G <= 8) || (s->kind == VSAG_AMD_KIND_SQ4 && s->G <= 4);
+    return kind_ok && s->nlist > 0 && s->dpad <= kI8Dims && s->pf_term != nullptr && s->pf_ymax != nullptr &&
+           s->residual_centroids_dev == nullptr;
 }
 
 // Bytes of the query planes, floats of the scalars and words of the thresholds for nq queries and one padding row.
@@ -1070,6 +1091,7 @@ launch_ivf_sq8_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride, 
     z.qmeta = l2 ? nullptr : qmeta;
     z.qmeta_stride = qmeta_stride;
     z.is_l2 = l2 ? 1 : 0;
+    z.nibbles = s->kind == VSAG_AMD_KIND_SQ4 ? 1 : 0;
     z.bound = bound;
     z.ymax_bits = s->pf_ymax;
     z.nq = nq;
@@ -1108,7 +1130,13 @@ launch_ivf_sq8_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride, 
         (div_up(pairs, static_cast<uint64_t>(kIvfSq8Pairs)) + std::min<uint64_t>(s->nlist, pairs)) * kIvfSq8Chunks;
     const dim3 grid(static_cast<uint32_t>(max_items));
     timing_begin(st);
-    if (l2) {
+    if (z.nibbles) {
+        if (l2) {
+            hipLaunchKernelGGL((ivf_sq8_i8_kernel<kI8TestIntTerm, true>), grid, dim3(256), 0, st, p);
+        } else {
+            hipLaunchKernelGGL((ivf_sq8_i8_kernel<kI8TestInt, true>), grid, dim3(256), 0, st, p);
+        }
+    } else if (l2) {
         hipLaunchKernelGGL(ivf_sq8_i8_kernel<kI8TestIntTerm>, grid, dim3(256), 0, st, p);
     } else {
         hipLaunchKernelGGL(ivf_sq8_i8_kernel<kI8TestInt>, grid, dim3(256), 0, st, p);
@@ -1171,8 +1199,8 @@ launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride
                     uint8_t* q8, float* u, uint32_t* tau, uint32_t* cand, uint32_t* cand_cnt, uint32_t sub_lists,
                     uint32_t sub_cap, bool first_level, const float* merged_dists, uint32_t k, uint32_t* bound_rw,
                     hipStream_t st) {
-    const bool nibbles = s->kind == VSAG_AMD_KIND_SQ4_UNIFORM;
-    const bool uniform = s->kind == VSAG_AMD_KIND_SQ8_UNIFORM || nibbles;
+    const bool nibbles = s->kind == VSAG_AMD_KIND_SQ4_UNIFORM || s->kind == VSAG_AMD_KIND_SQ4;
+    const bool uniform = s->kind == VSAG_AMD_KIND_SQ8_UNIFORM || s->kind == VSAG_AMD_KIND_SQ4_UNIFORM;
     const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
     const uint64_t nq_pad = div_up(nq, static_cast<uint64_t>(kI8Group)) * kI8Group;
     // `u` holds a float per padded query and one per group of kI8Group queries behind them (prefilter_i8_scalar_floats).
@@ -1213,6 +1241,7 @@ launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride
         z.qmeta = l2 ? nullptr : qmeta;
         z.qmeta_stride = qmeta_stride;
         z.is_l2 = l2 ? 1 : 0;
+        z.nibbles = nibbles ? 1 : 0;
         z.bound = bound;
         z.ymax_bits = s->pf_ymax;
         z.nq = nq;
@@ -1253,8 +1282,12 @@ launch_prefilter_i8(const vsag_amd_store* s, const float* qtab, uint32_t qstride
     p.qgroups = static_cast<uint32_t>(nq_pad / kI8Group);
     dim3 grid(p.groups * p.qgroups);
     timing_begin(st);
-    if (nibbles) {
+    if (nibbles && uniform) {
         hipLaunchKernelGGL((prefilter_i8_kernel<kI8TestFma, true>), grid, dim3(256), 0, st, p);
+    } else if (nibbles && l2) {
+        hipLaunchKernelGGL((prefilter_i8_kernel<kI8TestIntTerm, true>), grid, dim3(256), 0, st, p);
+    } else if (nibbles) {
+        hipLaunchKernelGGL((prefilter_i8_kernel<kI8TestInt, true>), grid, dim3(256), 0, st, p);
     } else if (uniform) {
         hipLaunchKernelGGL(prefilter_i8_kernel<kI8TestFma>, grid, dim3(256), 0, st, p);
     } else if (l2) {

@@ -899,7 +899,7 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
     c->contraction = true;
     // Mode 2 asks for the fp32 matrix cores, which the uniform kinds have no route for.
     c->int8 = prefilter_i8_supports(s) && (prefilter_mode(s) != 2 || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM ||
-                                           s->kind == VSAG_AMD_KIND_SQ4_UNIFORM);
+                                           s->kind == VSAG_AMD_KIND_SQ4_UNIFORM || s->kind == VSAG_AMD_KIND_SQ4);
     c->rb = rb;
     c->rb_scratch = rb ? prefilter_rb_scratch_bytes(s, nq) : 0;
     c->prefix_tiles = prefix;

@@ -80,7 +80,7 @@ struct vsag_amd_store {
     uint4* rows = nullptr;
     float* pf_term = nullptr;
     uint32_t* pf_ymax = nullptr;
-    // sq8 posting lists of at most 128 dimensions keep the same per-slot term (over all cap_tiles * 64 slots, renewed
+    // sq8 / sq4 posting lists of at most 128 dimensions keep the same per-slot term (over all cap_tiles * 64 slots, renewed
     // when codes are added) for the int8 pass over lists; pf_term_slots = the slots pf_term has room for there.
     uint64_t pf_term_slots = 0;
 };

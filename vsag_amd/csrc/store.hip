@@ -489,7 +489,8 @@ vsag_amd_store_create(const vsag_amd_store_params_t* p, vsag_amd_store_t** out) 
     }
     // Stores the matrix cores can pre-select on keep a per-code term (and the largest norm, where a threshold needs it).
     if (p->kind == VSAG_AMD_KIND_FP32 || p->kind == VSAG_AMD_KIND_SQ8 ||
-        ((p->kind == VSAG_AMD_KIND_SQ8_UNIFORM || p->kind == VSAG_AMD_KIND_SQ4_UNIFORM) && s->dpad <= 128)) {
+        ((p->kind == VSAG_AMD_KIND_SQ8_UNIFORM || p->kind == VSAG_AMD_KIND_SQ4_UNIFORM || p->kind == VSAG_AMD_KIND_SQ4) &&
+         s->dpad <= 128)) {
         if (hipMalloc(&s->pf_ymax, 4) != hipSuccess || hipMemset(s->pf_ymax, 0, 4) != hipSuccess) {
             return fail_free(fail(VSAG_AMD_NO_ENOUGH_MEMORY, "hipMalloc of the norm scalar failed"));
         }
@@ -783,7 +784,8 @@ append_to_lists(vsag_amd_store* s, const uint8_t* codes_dev, const int32_t* labe
     // The per-slot terms of the int8 pass over sq8 lists (ivf_i8.hip): recomputed over the whole buffer, which costs a
     // pass over the codes (0.4 ms for ten million of them) against the classification and encoding an append has
     // behind it already.
-    if (s->kind == VSAG_AMD_KIND_SQ8 && s->pf_ymax != nullptr && s->dpad <= 128 && s->residual_centroids_dev == nullptr) {
+    if ((s->kind == VSAG_AMD_KIND_SQ8 || s->kind == VSAG_AMD_KIND_SQ4) && s->pf_ymax != nullptr && s->dpad <= 128 &&
+        s->residual_centroids_dev == nullptr) {
         const uint64_t slots = s->cap_tiles * kWave;
         if (s->pf_term == nullptr || s->pf_term_slots < slots) {
             if (s->pf_term != nullptr) {
