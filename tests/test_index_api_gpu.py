@@ -327,10 +327,10 @@ def test_k_above_one_device_scan(lib, name, params, search):
 
 
 @pytest.mark.parametrize("quant,metric", [("sq4_uniform", "l2"), ("sq8_uniform", "ip"), ("sq8", "l2"), ("sq8", "cosine"),
-                                          ("rabitq", "l2")])
+                                          ("sq4", "l2"), ("rabitq", "l2")])
 @pytest.mark.parametrize("reorder", [True, False])
 def test_ivf_large_batch_equals_one_by_one(lib, reorder, quant, metric):
-    """A batch large enough for the matrix-core pass over the posting lists (sq4_uniform, sq8_uniform, sq8, rabitq)
+    """A batch large enough for the matrix-core pass over the posting lists (sq4_uniform, sq8_uniform, sq8, sq4, rabitq)
     returns what single queries (chunked streaming scan) return."""
     n, d, nq, k = 60000, 64, 2200, 10
     x = vectors(n, d, normalize=False)
@@ -368,7 +368,7 @@ def test_rabitq_large_batch_equals_one_by_one(lib):
     idx.close()
 
 
-@pytest.mark.parametrize("quant", ["fp32", "sq8", "sq8_uniform", "sq4_uniform"])
+@pytest.mark.parametrize("quant", ["fp32", "sq8", "sq4", "sq8_uniform", "sq4_uniform"])
 def test_large_batch_equals_one_by_one(lib, quant):
     """A batch large enough for the matrix-core path of the flat scan returns what single queries return."""
     n, d, nq, k = 70000, 32, 600, 10
