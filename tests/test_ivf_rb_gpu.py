@@ -102,3 +102,34 @@ def test_vectors_equal_to_the_centroid(lib):
     plain, fast = _both(lib, st, q, buckets, kcand)
     assert _same(plain, fast)
     st.destroy()
+
+
+def test_one_long_list_among_short_and_empty_ones(lib):
+    """A list long enough for several chunks of the matrix-core pass (128 tiles each), lists of a single code and lists
+    without any."""
+    n, d, nlist, nq, nprobe, kcand = 40000, 64, 40, 6000, 6, 20
+    rng = np.random.default_rng(12)
+    x, means = gaussian_mixture(rng, n, d, 30, 0.3)
+    q, _ = gaussian_mixture(rng, nq, d, 30, 0.3, means=means)
+    cent = x[rng.choice(n, nlist, replace=False)].copy()
+    labels, _, _ = orc.kmeans_assign(x, cent)
+    labels = labels.copy()
+    labels[rng.random(n) < 0.45] = 7          # about 18 000 codes: three chunks
+    labels[labels == 3] = 7                   # list 3 is empty
+    labels[labels == 4] = 7
+    labels[11] = 4                            # list 4 holds one code
+    g = rng.standard_normal((d, d))
+    rot, r = np.linalg.qr(g)
+    rot = (rot * np.sign(np.diag(r))).astype(np.float32)
+    cen = orc.rabitq_train(x, rot)
+    codes = orc.rabitq_encode(x, rot, cen, orc.L2)
+    st = Store(capi.KIND_RABITQ, orc.L2, d, rot=rot, centroid=cen)
+    st.set_lists(codes, labels, nlist)
+    buckets, _ = orc.ivf_route(cent, q, nprobe)
+    buckets = buckets.copy()
+    buckets[::2, 1] = 7
+    buckets[1::2, 2] = 3
+    buckets[::5, 3] = 4
+    plain, fast = _both(lib, st, q, buckets, kcand)
+    assert _same(plain, fast)
+    st.destroy()

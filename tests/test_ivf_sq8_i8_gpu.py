@@ -131,3 +131,31 @@ def test_lists_that_grew_by_appending(lib, bits):
     assert np.array_equal(ref[1].view(np.uint32), fast[1].view(np.uint32))
     st.destroy()
     whole.destroy()
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_one_long_list_among_short_and_empty_ones(lib, bits):
+    """A list long enough for all four chunks of the matrix-core pass, lists of a single code and lists without any."""
+    n, d, nlist, nq, nprobe, kcand = 40000, 64, 40, 6000, 6, 20
+    rng = np.random.default_rng(12)
+    x, means = gaussian_mixture(rng, n, d, 30, 0.05)
+    q, _ = gaussian_mixture(rng, nq, d, 30, 0.05, means=means)
+    cent = x[rng.choice(n, nlist, replace=False)].copy()
+    labels, _, _ = orc.kmeans_assign(x, cent)
+    labels = labels.copy()
+    labels[rng.random(n) < 0.45] = 7          # about 18 000 codes: four chunks of 70 tiles
+    labels[labels == 3] = 7                   # list 3 is empty
+    labels[labels == 4] = 7
+    labels[11] = 4                            # list 4 holds one code
+    lb, diff = orc.sq_train(x, bits)
+    codes = orc.sq_encode(x, bits, lb, diff)
+    st = Store(capi.KIND_SQ8 if bits == 8 else capi.KIND_SQ4, orc.L2, d, lb=lb, diff=diff)
+    st.set_lists(codes, labels, nlist)
+    buckets, _ = orc.ivf_route(cent, q, nprobe)
+    buckets = buckets.copy()
+    buckets[::2, 1] = 7
+    buckets[1::2, 2] = 3
+    buckets[::5, 3] = 4
+    plain, fast = _both(lib, st, q, buckets, kcand)
+    assert _same(plain, fast)
+    st.destroy()
