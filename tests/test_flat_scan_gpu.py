@@ -198,3 +198,61 @@ def test_cosine_with_zero_rows_and_a_zero_query(lib, kind, contraction):
     if kind == "fp32":
         assert np.all(ds[2] == 1.0), "a zero query is at distance 1 from everything"
     st.destroy()
+
+
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
+@pytest.mark.parametrize("n,d,nq,k", [(4096, 128, 1500, 64), (5000, 100, 1030, 10), (8192, 32, 2000, 1), (1024, 16, 1100, 256),
+                                      (3000, 30, 1024, 100), (2047, 7, 1300, 5)])
+def test_many_queries_against_a_small_fp32_store(lib, metric, n, d, nq, k):
+    """A few thousand fp32 codes against a thousand queries and more (the routing of an ivf search): the fp32 matrix
+    cores fill a table of approximate distances, every query takes the codes within reach of its k-th table value and
+    scores them with the streaming arithmetic.  Ids and distance bits equal the streaming scan's."""
+    rng = np.random.default_rng(n + d + k)
+    x, means = gaussian_mixture(rng, n, d, 20, 0.1)
+    q, _ = gaussian_mixture(rng, nq, d, 20, 0.1, means=means)
+    q[3] *= 1e4
+    q[4] *= 1e-4
+    q[5] = x[17]
+    if metric != orc.COSINE:
+        q[6] = 0.0
+    st = Store(lib.KIND_FP32, metric, d)
+    st.append(x.view(np.uint8).reshape(n, 4 * d))
+    L = lib.load_library()
+    lib.check(L.vsag_amd_set_scan_contraction(-1))
+    try:
+        plain = st.flat_scan(q, k)
+    finally:
+        lib.check(L.vsag_amd_set_scan_contraction(0))
+    fast = st.flat_scan(q, k)
+    tile = lib.C.c_int()
+    L.vsag_amd_last_scan_info(lib.C.byref(tile), None, None)
+    assert tile.value == 64, "the table route did not run"
+    assert np.array_equal(plain[0], fast[0]) and np.array_equal(plain[1].view(np.uint32), fast[1].view(np.uint32))
+    st.destroy()
+
+
+def test_small_fp32_store_with_thousands_of_equal_rows(lib):
+    """More codes at the k-th distance than a query's candidate pool takes (and a query with a NaN): those queries are
+    redone by a full scan of their own."""
+    n, d, nq, k = 8192, 32, 1200, 40
+    rng = np.random.default_rng(9)
+    x = (rng.random((n, d), dtype=np.float32) * 10 + 20).astype(np.float32)
+    x[5::4] = x[5]  # 2047 copies of one row: the same distance, ids apart
+    q = (x[5] + rng.random((nq, d), dtype=np.float32) * 0.1).astype(np.float32)
+    q[100:] = (rng.random((nq - 100, d), dtype=np.float32) * 10 + 20).astype(np.float32)
+    q[7, 3] = np.nan
+    st = Store(lib.KIND_FP32, orc.L2, d)
+    st.append(x.view(np.uint8).reshape(n, 4 * d))
+    L = lib.load_library()
+    lib.check(L.vsag_amd_set_scan_contraction(-1))
+    try:
+        plain = st.flat_scan(q, k)
+    finally:
+        lib.check(L.vsag_amd_set_scan_contraction(0))
+    fast = st.flat_scan(q, k)
+    ok = np.ones(nq, bool)
+    ok[7] = False
+    assert np.array_equal(plain[0][ok], fast[0][ok])
+    assert np.array_equal(plain[1][ok].view(np.uint32), fast[1][ok].view(np.uint32))
+    assert np.all(fast[0][:100][ok[:100]] % 4 == 1)
+    st.destroy()

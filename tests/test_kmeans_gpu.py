@@ -38,7 +38,8 @@ def check_assignment(x, cent, labels, mind, rel=1e-5):
     return int(wrong.sum())
 
 
-@pytest.mark.parametrize("n,d,k", [(3000, 128, 100), (1000, 960, 257), (129, 7, 3), (5000, 33, 1000), (64, 16, 64)])
+@pytest.mark.parametrize("n,d,k", [(3000, 128, 100), (1000, 960, 257), (129, 7, 3), (5000, 33, 1000), (64, 16, 64),
+                                   (3000, 100, 100), (2000, 104, 500), (1500, 12, 40)])
 def test_assign_matches_bruteforce_and_oracle(lib, n, d, k):
     rng = np.random.default_rng(n + d + k)
     x, _ = gaussian_mixture(rng, n, d, max(2, k // 4), 0.2, uniform_means=False)

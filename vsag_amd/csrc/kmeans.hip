@@ -242,6 +242,8 @@ struct TilePlan {
     uint32_t rtiles, ctiles;
     uint32_t mc_log2;  // macro tile: (32 >> mc_log2) row tiles x (1 << mc_log2) centroid tiles
     uint32_t mcols;    // macro tiles per macro row
+    uint64_t ld;       // STORE: floats per row of the output
+    float alpha;       // STORE: factor of the product
     uint32_t macros;
 };
 
@@ -255,7 +257,10 @@ tile_lds_bytes(int mi) {
     return kRing * static_cast<size_t>(4 * (64 * mi + kTileRows)) * sizeof(float4);
 }
 
-template <int MI>
+// STORE: instead of the argmin, every product goes out as out[m * plan.ld + n] = (ynorm ? ynorm[n] : 0) + plan.alpha *
+// <c_m, x_n> (m a row of C, n a row of X; `best` is that float matrix, ynorm is indexed by rows of X): the table of
+// approximate distances a routing call selects from (scan.hip, route_select_kernel).
+template <int MI, bool STORE = false>
 __global__ void __launch_bounds__(kTileThreads, 1)
 kmeans_assign_tile_kernel(const float* __restrict__ X, uint64_t n, const float* __restrict__ C, uint32_t k, uint32_t dim,
                           const float* __restrict__ ynorm, unsigned long long* __restrict__ best, TilePlan plan) {
@@ -432,6 +437,25 @@ kmeans_assign_tile_kernel(const float* __restrict__ X, uint64_t n, const float* 
         s0 = s1;
         s1 = s2;
         s2 = t;
+    }
+    if constexpr (STORE) {
+        float* out = reinterpret_cast<float*>(best);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint64_t row = row0 + wn * 64 + j * 32 + l32;
+            const float base = row < n && ynorm != nullptr ? ynorm[row] : 0.0F;
+#pragma unroll
+            for (int i = 0; i < MI; ++i) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const uint32_t ml = wm * 32 * MI + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+                    if (row < n && c0 + ml < k) {
+                        out[(c0 + ml) * plan.ld + row] = base + plan.alpha * acc[i][j][e];
+                    }
+                }
+            }
+        }
+        return;
     }
     // Fused argmin: acc[i][j][e] = <c_m, x_n> with m = c0 + wm*32*MI + i*32 + 8*(e/4) + 4*half + e%4 and
     // n = row0 + wn*64 + j*32 + l32.  m grows with (i, e), so a strict `<` keeps the first minimum.
@@ -641,6 +665,72 @@ centroid_mean_kernel(const float* x, uint32_t dim, const uint32_t* sorted_rows, 
 void timing_begin(hipStream_t st);
 void timing_end(hipStream_t st);
 
+// out[m * ld + n] = (base ? base[n] : 0) + alpha <c_m, x_n> for the rows x_n of x (nx x dim) and c_m of c (nc x dim), on
+// the fp32 matrix cores; dim a multiple of 4, rows 16-byte aligned.
+int
+launch_row_products(const float* x, uint64_t nx, const float* c, uint32_t nc, uint32_t dim, const float* base, float alpha,
+                    float* out, uint64_t ld, hipStream_t st) {
+    if ((dim & 3) != 0 || nx == 0 || nc == 0 || nx > (1ull << 20) * kTileRows) {
+        return fail(VSAG_AMD_INVALID_ARGUMENT, "row products: the dimension must be a multiple of 4");
+    }
+    static std::once_flag lds_once;
+    static hipError_t lds_rc = hipSuccess;
+    std::call_once(lds_once, []() {
+        lds_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kmeans_assign_tile_kernel<4, true>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(tile_lds_bytes(4)));
+    });
+    VA_HIP(lds_rc);
+    TilePlan plan;
+    plan.rtiles = static_cast<uint32_t>(div_up(nx, kTileRows));
+    plan.ctiles = (nc + 255) / 256;
+    plan.mc_log2 = plan.ctiles >= 8 ? 3 : plan.ctiles >= 4 ? 2 : plan.ctiles >= 2 ? 1 : 0;
+    plan.mcols = (plan.ctiles + (1U << plan.mc_log2) - 1) >> plan.mc_log2;
+    const uint32_t mrows = (plan.rtiles + (32U >> plan.mc_log2) - 1) / (32U >> plan.mc_log2);
+    plan.macros = mrows * plan.mcols;
+    plan.ld = ld;
+    plan.alpha = alpha;
+    const uint32_t per_xcd = (plan.macros + 7) / 8;
+    const dim3 grid(per_xcd * 32 * 8);
+    hipLaunchKernelGGL((kmeans_assign_tile_kernel<4, true>), grid, dim3(kTileThreads), tile_lds_bytes(4), st, x, nx, c, nc,
+                       dim, base, reinterpret_cast<unsigned long long*>(out), plan);
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
+// The largest finite value of out[0, n) as float bits (norms: not negative, so the bits order like the values); one
+// workgroup.
+__global__ void __launch_bounds__(1024)
+max_norm_kernel(const float* out, uint64_t n, uint32_t* max_bits) {
+    __shared__ float part[16];
+    float m = 0.0F;
+    for (uint64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        const float v = out[i];
+        m = v < __builtin_inff() ? fmaxf(m, v) : m;
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        m = fmaxf(m, __shfl_xor(m, off));
+    }
+    if ((threadIdx.x & 63) == 0) {
+        part[threadIdx.x >> 6] = m;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (uint32_t w = 1; w < blockDim.x / 64; ++w) {
+            m = fmaxf(m, part[w]);
+        }
+        *max_bits = __float_as_uint(m);
+    }
+}
+
+// ||row||^2 of nx rows and the largest of them (as float bits).
+int
+launch_row_sqnorms(const float* x, uint64_t nx, uint32_t dim, float* out, uint32_t* max_bits, hipStream_t st) {
+    hipLaunchKernelGGL(row_sqnorm_kernel, dim3(static_cast<uint32_t>(div_up(nx, 4))), dim3(256), 0, st, x, nx, dim, out);
+    hipLaunchKernelGGL(max_norm_kernel, dim3(1), dim3(1024), 0, st, out, nx, max_bits);
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
 struct AssignBuffers {
     float* ynorm;
     float* xnorm;
@@ -699,6 +789,8 @@ assign_launch(const float* x, uint64_t n, uint32_t dim, const float* cent, uint3
             plan.mcols = (plan.ctiles + (1U << plan.mc_log2) - 1) >> plan.mc_log2;
             const uint32_t mrows = (plan.rtiles + (32U >> plan.mc_log2) - 1) / (32U >> plan.mc_log2);
             plan.macros = mrows * plan.mcols;
+            plan.ld = 0;
+            plan.alpha = 0.0F;
             const uint32_t per_xcd = (plan.macros + 7) / 8;
             const dim3 grid(per_xcd * 32 * 8);
             if (mi == 4) {

@@ -812,6 +812,10 @@ struct CallPlan {
     size_t rb_scratch = 0;     // rb: bytes of the expanded queries and per-query factors
     uint32_t nslots = 0;       // partial lists per query
     bool any_seeded = false;
+    // Many queries against a small fp32 store (the routing of an ivf search): a table of approximate distances from the
+    // fp32 matrix cores, then per query the exact distances of the few codes that can be among the k best.
+    bool table = false;
+    uint64_t table_ld = 0;     // floats per row of the table
 };
 
 // -1 never, 0 when it pays, 1 whenever the store supports it, 2 like 1 but on the fp32 matrix cores only
@@ -833,12 +837,26 @@ bool prefilter_rb_supports(const vsag_amd_store* s);
 size_t prefilter_rb_scratch_bytes(const vsag_amd_store* s, uint64_t nq);
 uint32_t prefilter_rb_sub_lists(uint64_t nq, uint64_t span);
 
+// Whether a call goes through the table of approximate distances (see CallPlan::table).
+constexpr uint64_t kTableMinCodes = 1024, kTableMaxCodes = 8192;
+constexpr uint32_t kTableMaxK = 256;
+static bool
+small_store_table(const vsag_amd_store* s, uint64_t nq, uint32_t k) {
+    return s->kind == VSAG_AMD_KIND_FP32 && s->nlist == 0 && prefilter_mode(s) == 0 && nq >= 1024 && k <= kTableMaxK &&
+           s->n >= kTableMinCodes && s->ntiles * kWave <= kTableMaxCodes && nq * (s->ntiles * kWave) * 4 <= (2ull << 30);
+}
+
 static void
 make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
     make_plan(s, nq, k, s->ntiles, &c->all);
     c->nslots = static_cast<uint32_t>(c->all.chunks * c->all.waves);
     c->any_seeded = c->all.seeded;
     c->contraction = false;
+    c->table = small_store_table(s, nq, k);
+    c->table_ld = c->table ? round_up(s->ntiles * kWave, 64) : 0;
+    if (c->table) {
+        return;
+    }
     if (prefilter_mode(s) < 0 || !prefilter_supports(s)) {
         return;
     }
@@ -950,6 +968,10 @@ struct ScanBuffers {
     uint32_t* cand;
     uint8_t* q8;   // int8 planes of the queries, null on the fp32 matrix cores
     float* q8_u;
+    // table route only
+    float* table;       // nq x table_ld approximate distances
+    float* table_rows;  // the codes a row per code
+    float* table_norms; // their squared norms, then (one word) the largest as float bits
 };
 
 static size_t
@@ -975,6 +997,9 @@ carve_scan(Carver& c, const CallPlan& cp, uint64_t nq, uint32_t k, ScanBuffers* 
     b->cand_cnt = c.take<uint32_t>(cp.contraction ? nq * std::max<uint32_t>(1, cp.max_lists) : 0);
     b->gate = c.take<uint32_t>(cp.contraction ? nq : 0);
     b->cand = c.take<uint32_t>(cp.contraction ? nq * cp.cap : 0);
+    b->table = c.take<float>(cp.table ? nq * cp.table_ld : 0);
+    b->table_rows = c.take<float>(cp.table ? cp.table_ld * p.ql.qstride : 0);
+    b->table_norms = c.take<float>(cp.table ? cp.table_ld + 64 : 0);
     return c.used;
 }
 
@@ -1054,6 +1079,276 @@ launch_flat(const vsag_amd_store* s, const ScanPlan& p, const ScanArgs& a, const
     }
     VA_HIP(hipGetLastError());
     return 0;
+}
+
+// ---- many queries against a small fp32 store: selection from a table of approximate distances ------------------
+// (the routing of an ivf search over its centroids: 10 000 queries x 4096 centroids x 128 dimensions).  The streaming
+// distance sum (q_d - c_d)^2 is a subtraction and an fma per dimension; on the vector ALU that alone is 0.27 ms here.
+// The fp32 matrix cores deliver |c|^2 - 2 <q, c> (inner product: -<q, c>) for every pair in a third of that
+// (kmeans.hip, launch_row_products), but rounded differently.  So the table only selects: with a_k the k-th smallest
+// table value of a query and eps a bound on |table - streaming distance| (up to the query's own constant), every code
+// among the k best by streaming distance has a table value of at most a_k + 2 eps; those few codes -- k and a
+// handful -- get their streaming distance, and the k best of them are the result, bit for bit what the streaming
+// scan returns.
+int launch_row_products(const float* x, uint64_t nx, const float* c, uint32_t nc, uint32_t dim, const float* base, float alpha,
+                        float* out, uint64_t ld, hipStream_t st);
+int launch_row_sqnorms(const float* x, uint64_t nx, uint32_t dim, float* out, uint32_t* max_bits, hipStream_t st);
+
+constexpr uint32_t kTablePool = 512;  // candidates a query may have before it is redone by a full scan
+
+// rows[slot][4 j ...] = granule j of the code in `slot`: rows of `row_granules` granules like the rows of the query
+// table (zero behind the code's own G granules, zero rows behind the last code).
+__global__ void __launch_bounds__(256)
+table_rows_kernel(const uint4* tiles, uint32_t G, uint32_t row_granules, uint64_t n, uint64_t slots, float* rows,
+                  uint32_t* max_bits) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i == 0) {
+        *max_bits = 0;
+    }
+    if (i >= slots * row_granules) {
+        return;
+    }
+    const uint64_t slot = i / row_granules;
+    const uint32_t j = static_cast<uint32_t>(i % row_granules);
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (slot < n && j < G) {
+        v = tiles[((slot / kWave) * G + j) * kWave + slot % kWave];
+    }
+    reinterpret_cast<uint4*>(rows)[slot * row_granules + j] = v;
+}
+
+// The exact scan of one query (row qi of the query table) by one wave: all keys at or below `limit`, the k best written
+// out.  The pool takes kTablePool keys; when more lie at or below the limit, the k-th of what was pooled (an upper bound
+// of the k-th of all that lies below at least kTablePool - k pooled keys) is the limit of another pass.
+template <int METRIC>
+__device__ inline void
+table_redo(const ScanArgs& a, uint64_t n, uint64_t ntiles, uint32_t k, uint32_t qi, uint32_t* ids, float* dists,
+           uint64_t limit, uint64_t* pool, uint32_t lane) {
+    const uint32_t qidx[1] = {qi};
+    const QueryRows<1> qrows = query_rows<1>(a, qidx);
+    for (;;) {
+        uint32_t count = 0;
+        for (uint64_t tile = 0; tile < ntiles; ++tile) {
+            Acc<VSAG_AMD_KIND_FP32, 1> acc;
+            acc_reset(acc);
+            for (uint32_t j = 0; j < a.G; ++j) {
+                accumulate_granule<VSAG_AMD_KIND_FP32, METRIC, 1>(a, qrows, j, a.tiles[(tile * a.G + j) * kWave + lane], acc);
+            }
+            const uint64_t slot = tile * kWave + lane;
+            float d[1];
+            finish_distances<VSAG_AMD_KIND_FP32, METRIC, 1>(a, qidx, slot, acc, d);
+            const uint64_t key = make_key(d[0], static_cast<uint32_t>(slot));
+            const bool pass = slot < n && key <= limit;
+            const uint64_t mask = __ballot(pass);
+            const uint32_t at = count + mask_rank(mask);
+            if (pass && at < kTablePool) {
+                pool[at] = key;
+            }
+            count += static_cast<uint32_t>(__popcll(mask));
+        }
+        const uint32_t kept = count < kTablePool ? count : kTablePool;
+        for (uint32_t i = kept + lane; i < kTablePool; i += kWave) {
+            pool[i] = kInfKey;
+        }
+        wave_lds_fence();
+        wave_bitonic_sort(pool, kTablePool, lane);
+        if (count <= kTablePool) {
+            break;
+        }
+        limit = wave_uniform_u64(pool[k - 1]);
+        wave_lds_fence();
+    }
+    for (uint32_t i = lane; i < k; i += kWave) {
+        const uint64_t key = pool[i];
+        ids[i] = key == kInfKey ? VSAG_AMD_INVALID_ID : static_cast<uint32_t>(key);
+        dists[i] = key == kInfKey ? __builtin_inff() : ordered_to_float(static_cast<uint32_t>(key >> 32));
+    }
+}
+
+struct TableSelectArgs {
+    const float* table;  // nq x ld
+    uint64_t ld;
+    uint64_t nq, n, ntiles;
+    uint32_t k, dim;
+    const uint32_t* max_norm_bits;  // the largest |c|^2
+    uint32_t* ids;
+    float* dists;
+};
+
+// One wave per query; NV table values per lane (NV * 64 >= the codes of the store).
+template <int METRIC, int NV>
+__global__ void __launch_bounds__(64)
+table_select_kernel(ScanArgs a, TableSelectArgs p) {
+    __shared__ uint64_t pool[kTablePool];
+    __shared__ uint32_t hist[256];
+    __shared__ uint32_t cand[kTablePool];
+    const uint32_t lane = threadIdx.x;
+    const uint64_t q = blockIdx.x;
+    const float* row = p.table + q * p.ld;
+    float val[NV];
+    bool odd = false;  // a value that is no number: the table cannot order this query
+    float vmin = __builtin_inff(), vmax = -__builtin_inff();
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint64_t c = static_cast<uint64_t>(i) * kWave + lane;
+        val[i] = c < p.n ? row[c] : __builtin_inff();
+        odd = odd || val[i] != val[i];
+        if (c < p.n) {
+            vmin = fminf(vmin, val[i]);
+            vmax = fmaxf(vmax, val[i]);
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        vmin = fminf(vmin, __shfl_xor(vmin, off));
+        vmax = fmaxf(vmax, __shfl_xor(vmax, off));
+    }
+    // |table - streaming| <= eps: both sums run over dim terms in fp32, whatever their order.
+    const uint32_t* qrow = a.qtab + q * a.qstride;
+    float qn2 = 0.0F;
+    for (uint32_t d = lane; d < a.qstride; d += kWave) {
+        const float x = __uint_as_float(qrow[d]);
+        qn2 = fmaf(x, x, qn2);
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        qn2 += __shfl_xor(qn2, off);
+    }
+    const float cn2 = __uint_as_float(*p.max_norm_bits);
+    const float u = 5.9604644775390625e-8F;
+    float eps;
+    if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+        const float reach = sqrtf(qn2) + sqrtf(cn2);
+        eps = 2.0F * static_cast<float>(p.dim + 8) * u * reach * reach * 1.001F;
+    } else {
+        eps = 2.0F * static_cast<float>(p.dim + 8) * u * (sqrtf(qn2) * sqrtf(cn2) + 1.0F) * 1.001F;
+    }
+    odd = odd || !(eps < 1.0e30F) || !(vmax < 1.0e30F) || !(vmin > -1.0e30F);
+    const uint32_t qi[1] = {static_cast<uint32_t>(q)};
+    if (__ballot(odd) != 0 || p.k > p.n) {
+        table_redo<METRIC>(a, p.n, p.ntiles, p.k, qi[0], p.ids + q * p.k, p.dists + q * p.k, kInfKey, pool, lane);
+        return;
+    }
+    // Any value with at least k table values at or below it serves as a_k (a larger one only admits more): 256 bins
+    // between the smallest and the largest value, the first bin at which the running count reaches k, and two bins more
+    // for the rounding of the binning itself.
+    const float width = (vmax - vmin) * (1.0F / 256.0F);
+    const float inv_width = width > 0.0F ? 1.0F / width : 0.0F;
+    for (uint32_t b = lane; b < 256; b += kWave) {
+        hist[b] = 0;
+    }
+    wave_lds_fence();
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t c = static_cast<uint32_t>(i) * kWave + lane;
+        if (c < p.n) {
+            const float f = (val[i] - vmin) * inv_width;
+            atomicAdd(&hist[f < 255.0F ? static_cast<uint32_t>(f) : 255U], 1U);
+        }
+    }
+    wave_lds_fence();
+    uint32_t bin;
+    {
+        const uint32_t h0 = hist[4 * lane], h1 = hist[4 * lane + 1], h2 = hist[4 * lane + 2], h3 = hist[4 * lane + 3];
+        uint32_t incl = h0 + h1 + h2 + h3;
+        const uint32_t mine = incl;
+        for (int off = 1; off < 64; off <<= 1) {
+            const uint32_t o = __shfl_up(incl, off);
+            incl += lane >= static_cast<uint32_t>(off) ? o : 0U;
+        }
+        const uint64_t reached = __ballot(incl >= p.k);
+        const uint32_t owner = static_cast<uint32_t>(__builtin_ctzll(reached));  // k <= n: some lane reaches it
+        uint32_t before = __shfl(incl - mine, static_cast<int>(owner));
+        const uint32_t o0 = __shfl(h0, static_cast<int>(owner)), o1 = __shfl(h1, static_cast<int>(owner)),
+                       o2 = __shfl(h2, static_cast<int>(owner));
+        bin = 4 * owner;
+        if (before + o0 < p.k) {
+            before += o0;
+            ++bin;
+            if (before + o1 < p.k) {
+                before += o1;
+                ++bin;
+                if (before + o2 < p.k) {
+                    ++bin;
+                }
+            }
+        }
+    }
+    const float kth = vmin + static_cast<float>(bin + 3) * width;  // the upper edge of bin + 2
+    // rounded up: what is added here only admits more
+    const float thr = (kth + 2.0F * eps) + fabsf(kth + 2.0F * eps) * 4.0F * u;
+    uint32_t count = 0;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t c = static_cast<uint32_t>(i) * kWave + lane;
+        const bool pass = c < p.n && val[i] <= thr;
+        const uint64_t mask = __ballot(pass);
+        const uint32_t at = count + mask_rank(mask);
+        if (pass && at < kTablePool) {
+            cand[at] = c;
+        }
+        count += static_cast<uint32_t>(__popcll(mask));
+    }
+    wave_lds_fence();
+    if (count > kTablePool) {
+        // many codes at nearly the same distance: the full scan sorts it out
+        table_redo<METRIC>(a, p.n, p.ntiles, p.k, qi[0], p.ids + q * p.k, p.dists + q * p.k, kInfKey, pool, lane);
+        return;
+    }
+    const QueryRows<1> qrows = query_rows<1>(a, qi);
+    uint32_t sorted = kWave;  // the power of two from the candidates on
+    while (sorted < count) {
+        sorted <<= 1;
+    }
+    for (uint32_t base = 0; base < sorted; base += kWave) {
+        if (base >= count) {
+            pool[base + lane] = kInfKey;
+            continue;
+        }
+        const bool have = base + lane < count;
+        const uint32_t slot = have ? cand[base + lane] : 0U;
+        const uint64_t tile = slot >> 6;
+        const uint32_t ln = slot & 63;
+        Acc<VSAG_AMD_KIND_FP32, 1> acc;
+        acc_reset(acc);
+        constexpr uint32_t kAhead = 8;
+        for (uint32_t j0 = 0; j0 < a.G; j0 += kAhead) {
+            uint4 c4[kAhead];
+#pragma unroll
+            for (uint32_t v = 0; v < kAhead; ++v) {
+                const uint32_t j = j0 + v < a.G ? j0 + v : a.G - 1;
+                c4[v] = a.tiles[(tile * a.G + j) * kWave + ln];
+            }
+#pragma unroll
+            for (uint32_t v = 0; v < kAhead; ++v) {
+                if (j0 + v < a.G) {
+                    accumulate_granule<VSAG_AMD_KIND_FP32, METRIC, 1>(a, qrows, j0 + v, c4[v], acc);
+                }
+            }
+        }
+        float d[1];
+        finish_distances<VSAG_AMD_KIND_FP32, METRIC, 1>(a, qi, slot, acc, d);
+        pool[base + lane] = have ? make_key(d[0], slot) : kInfKey;
+    }
+    wave_lds_fence();
+    wave_bitonic_sort(pool, sorted, lane);
+    for (uint32_t i = lane; i < p.k; i += kWave) {
+        const uint64_t key64 = i < sorted ? pool[i] : kInfKey;
+        p.ids[q * p.k + i] = key64 == kInfKey ? VSAG_AMD_INVALID_ID : static_cast<uint32_t>(key64);
+        p.dists[q * p.k + i] = key64 == kInfKey ? __builtin_inff() : ordered_to_float(static_cast<uint32_t>(key64 >> 32));
+    }
+}
+
+template <int METRIC>
+static void
+launch_table_select(uint64_t codes, dim3 grid, hipStream_t st, const ScanArgs& a, const TableSelectArgs& p) {
+    if (codes <= 1024) {
+        hipLaunchKernelGGL((table_select_kernel<METRIC, 16>), grid, dim3(kWave), 0, st, a, p);
+    } else if (codes <= 2048) {
+        hipLaunchKernelGGL((table_select_kernel<METRIC, 32>), grid, dim3(kWave), 0, st, a, p);
+    } else if (codes <= 4096) {
+        hipLaunchKernelGGL((table_select_kernel<METRIC, 64>), grid, dim3(kWave), 0, st, a, p);
+    } else {
+        hipLaunchKernelGGL((table_select_kernel<METRIC, 128>), grid, dim3(kWave), 0, st, a, p);
+    }
 }
 
 static int
@@ -1152,6 +1447,31 @@ flat_scan_call(const vsag_amd_store_t* s, const float* queries_dev, uint64_t nq,
     const ScanPlan& p = cp.all;
 
     VA_TRY(prepare_queries(s, queries_dev, nq, p.nq_pad, p.ql, b.qtab, b.qmeta, b.qcodes, st));
+    if (cp.table && plain) {
+        const ScanArgs ta = make_scan_args(s, p.ql, b.qtab, b.qmeta);
+        const uint64_t slots = cp.table_ld;
+        const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
+        uint32_t* max_bits = reinterpret_cast<uint32_t*>(b.table_norms + slots);
+        const uint32_t row_words = p.ql.qstride;  // a multiple of 16: the rows of the query table, zero behind the dimension
+        hipLaunchKernelGGL(table_rows_kernel, dim3(static_cast<uint32_t>(div_up(slots * (row_words / 4), 256))), dim3(256),
+                           0, st, s->tiles, s->G, row_words / 4, s->n, slots, b.table_rows, max_bits);
+        VA_TRY(launch_row_sqnorms(b.table_rows, slots, row_words, b.table_norms, max_bits, st));
+        timing_begin(st);
+        VA_TRY(launch_row_products(b.table_rows, slots, reinterpret_cast<const float*>(b.qtab), static_cast<uint32_t>(nq),
+                                   row_words, l2 ? b.table_norms : nullptr, l2 ? -2.0F : -1.0F, b.table, cp.table_ld, st));
+        TableSelectArgs tp{b.table, cp.table_ld, nq, s->n, s->ntiles, k, row_words, max_bits, ids_dev, dists_dev};
+        const dim3 grid(static_cast<uint32_t>(nq));
+        if (l2) {
+            launch_table_select<VSAG_AMD_METRIC_L2>(slots, grid, st, ta, tp);
+        } else {
+            launch_table_select<VSAG_AMD_METRIC_IP>(slots, grid, st, ta, tp);
+        }
+        timing_end(st);
+        VA_HIP(hipGetLastError());
+        tl_last_tile = 64;
+        tl_last_passes = nq;
+        return 0;
+    }
     const uint64_t nseed = b.seed != nullptr ? nq * k : 0;
     hipLaunchKernelGGL(reset_queries_kernel, dim3(static_cast<uint32_t>(div_up(nq > nseed ? nq : nseed, 256))), dim3(256),
                        0, st, b.bound, initial_bound(options), nq, b.seed, nseed);
