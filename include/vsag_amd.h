@@ -328,7 +328,9 @@ VSAG_AMD_API int vsag_amd_kmeans_init_plus_plus(const float* x_dev, uint64_t n, 
 
 /* Routing (IVFNearestPartition::ClassifyDatasForSearch, ivf_nearest_partition.cpp:99-147, done exactly
  * instead of through the reference's HGraph): the nprobe nearest centroids of every query, ascending.
- * centroids are an fp32 store created with vsag_amd_store_create + append. */
+ * centroids are an fp32 store created with vsag_amd_store_create + append.  From 1024 queries on, 1024 to 8192
+ * centroids are ranked through a table of approximate distances (nq x centroids x 4 bytes of the workspace) and the
+ * ones that can be among the nprobe nearest are scored exactly: the same buckets and distances as for fewer queries. */
 VSAG_AMD_API size_t vsag_amd_ivf_route_workspace_bytes(const vsag_amd_store_t* centroids, uint64_t nq, uint32_t nprobe);
 VSAG_AMD_API int vsag_amd_ivf_route(const vsag_amd_store_t* centroids, const float* queries_dev, uint64_t nq,
                        uint32_t nprobe, int32_t* buckets_dev, float* dists_dev, void* workspace_dev,
