@@ -1173,6 +1173,8 @@ struct TableSelectArgs {
     const uint32_t* max_norm_bits;  // the largest |c|^2
     uint32_t* ids;
     float* dists;
+    const uint4* rows;      // the codes a row per code, row_granules granules each: a candidate's granules lie together
+    uint32_t row_granules;  // there (eight cache lines for 128 dimensions against 32 in the tiles)
 };
 
 // One wave per query; NV table values per lane (NV * 64 >= the codes of the store).
@@ -1305,8 +1307,7 @@ table_select_kernel(ScanArgs a, TableSelectArgs p) {
         }
         const bool have = base + lane < count;
         const uint32_t slot = have ? cand[base + lane] : 0U;
-        const uint64_t tile = slot >> 6;
-        const uint32_t ln = slot & 63;
+        const uint4* code = p.rows + static_cast<uint64_t>(slot) * p.row_granules;
         Acc<VSAG_AMD_KIND_FP32, 1> acc;
         acc_reset(acc);
         constexpr uint32_t kAhead = 8;
@@ -1315,7 +1316,7 @@ table_select_kernel(ScanArgs a, TableSelectArgs p) {
 #pragma unroll
             for (uint32_t v = 0; v < kAhead; ++v) {
                 const uint32_t j = j0 + v < a.G ? j0 + v : a.G - 1;
-                c4[v] = a.tiles[(tile * a.G + j) * kWave + ln];
+                c4[v] = code[j];
             }
 #pragma unroll
             for (uint32_t v = 0; v < kAhead; ++v) {
@@ -1459,7 +1460,8 @@ flat_scan_call(const vsag_amd_store_t* s, const float* queries_dev, uint64_t nq,
         timing_begin(st);
         VA_TRY(launch_row_products(b.table_rows, slots, reinterpret_cast<const float*>(b.qtab), static_cast<uint32_t>(nq),
                                    row_words, l2 ? b.table_norms : nullptr, l2 ? -2.0F : -1.0F, b.table, cp.table_ld, st));
-        TableSelectArgs tp{b.table, cp.table_ld, nq, s->n, s->ntiles, k, row_words, max_bits, ids_dev, dists_dev};
+        TableSelectArgs tp{b.table, cp.table_ld, nq, s->n, s->ntiles, k, row_words, max_bits, ids_dev, dists_dev,
+                           reinterpret_cast<const uint4*>(b.table_rows), row_words / 4};
         const dim3 grid(static_cast<uint32_t>(nq));
         if (l2) {
             launch_table_select<VSAG_AMD_METRIC_L2>(slots, grid, st, ta, tp);
