@@ -726,6 +726,12 @@ make_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, uint64_t ntiles, Sca
         // short scans (centroid routing, the exact prefix of a pre-selected batch) live on their selectors instead.
         T = 8;
     }
+    if (tile_override(s) <= 0 && T > 2 && ntiles <= 32 && nq >= 2048) {
+        // A few tiles under thousands of queries (the exact prefix of a pre-selected batch): the scan lives on its
+        // selectors, and two queries per wave mean twice the waves to overlap each other's flushes (1M x 128 sq8 codes,
+        // 10 000 queries: the prefix launch 188 -> 157 us).
+        T = 2;
+    }
     while (T > 1 && static_cast<uint64_t>(T) > nq) {
         T >>= 1;
     }
