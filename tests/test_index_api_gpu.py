@@ -385,3 +385,25 @@ def test_large_batch_equals_one_by_one(lib, quant):
         gt, _ = ground_truth(x, q[:50], k, "l2")
         assert recall(ids[:50], gt, labels) >= 0.999
     idx.close()
+
+
+def test_ivf_with_a_thousand_buckets_routes_large_batches_through_the_table(lib):
+    """1024 buckets: Add classifies 65 536 rows a call and a search batch of 1100 queries routes through the table of
+    approximate centroid distances; both must give what single queries give (exact routing either way)."""
+    n, d, nq, k = 70000, 32, 1100, 10
+    x = vectors(n, d, normalize=False)
+    q = vectors(nq, d, seed=165, normalize=False)
+    labels = np.arange(n, dtype=np.int64) * 3 + 7
+    idx = make("ivf", d, "l2", buckets_count=1024, base_quantization_type="sq8", train_sample_count=30000)
+    assert idx.build(x, labels, n, d) == 0
+    search = json.dumps({"ivf": {"scan_buckets_count": 32}})
+    ids, dists = idx.knn_search_batch(q, k, search)
+    for i in range(0, nq, 53):
+        si, sd = idx.knn_search(q[i], k, search)
+        assert np.array_equal(si, ids[i]) and np.array_equal(sd.view(np.uint32), dists[i].view(np.uint32)), i
+    # every bucket probed: the exact sq8 neighbours, whichever way the rows were classified
+    every = json.dumps({"ivf": {"scan_buckets_count": 1024}})
+    ai, _ = idx.knn_search_batch(q[:1024], k, every)
+    gt, _ = ground_truth(x, q[:100], k, "l2")
+    assert recall(ai[:100], gt, labels) >= 0.9
+    idx.close()
