@@ -1173,6 +1173,13 @@ prefilter_i8_sub_lists(uint64_t nq, uint64_t span) {
     const uint64_t per_round = static_cast<uint64_t>(device_cu_count()) * 2;
     const uint64_t stages = div_up(span, static_cast<uint64_t>(kI8StageTiles));
     uint64_t groups = std::max<uint64_t>(1, std::min<uint64_t>(per_round * rounds_lo / qgroups, stages));
+    // A workgroup loads the planes of its 256 queries (64 KB) before its first stage, and every column is two more
+    // private lists per query whose counts the rescoring reads: on a short level a workgroup walks at least sixteen
+    // stages, as long as two rounds of workgroups remain (1M codes, 10 000 queries: 2.89 -> 2.84 ms per call).
+    const uint64_t by_length = std::max<uint64_t>(1, stages / 16);
+    if (groups > by_length) {
+        groups = std::max(by_length, std::min(groups, div_up(per_round * 2, qgroups)));
+    }
     if (groups >= 8) {
         uint64_t best = groups / 8 * 8;
         double best_fill = 0.0;
