@@ -6,10 +6,12 @@ one step = one pass of the hot path (query preparation + scan with fused top-k +
 query batch, inputs resident in HBM.  Prints ONE JSON line with the metric, the roofline of the dominant
 kernel (HIP events recorded by the library around that kernel on its own stream) and the CPU baseline
 (the reference's own SIMD kernel compiled from its sources when oracle/_ref is present, else the CPU
-restatement), timed on this host's cores on a bounded sample of the same workload.
+restatement), timed on this host's cores on a bounded sample of the same workload.  The same line carries
+one block per other configuration -- "kmeans" (configs[2]), "c1" (configs[0]), "c4" (configs[3]), "c5"
+(configs[4]) -- each with its own value, recall, roofline and CPU baseline (--only leaves them out).
 
-Other configs (--config c1 | c3 | c4 | c5) print one line each in the same shape for the fp32 brute-force
-scan, k-means assignment, the IVF SQ4-uniform search and the RaBitQ scan + rerank.
+--config c1 | c3 | c4 | c5 print one line each in the same shape for the fp32 brute-force scan, k-means
+assignment, the IVF SQ4-uniform search and the RaBitQ scan + rerank alone.
 """
 import argparse
 import ctypes as C
@@ -85,6 +87,46 @@ def exact_topk_host(x, q, k, metric):
     return out
 
 
+def blas_name():
+    try:
+        cfg = np.show_config(mode="dicts")
+        b = cfg["Build Dependencies"]["blas"]
+        return "%s %s" % (b.get("name", "blas"), b.get("version", ""))
+    except Exception:  # noqa: BLE001 - older numpy: no dict form
+        return "numpy's BLAS"
+
+
+def cpu_assign_sgemm(x, cent, threads):
+    """KMeansCluster::find_nearest_one_with_blas (impl/cluster/kmeans_cluster.cpp:193-305) with the BLAS numpy links:
+    per chunk of 65 536 rows distances = -2 C X^T by SGEMM, then per row (blocks of 1024 rows on the thread pool)
+    += |c|^2, first minimum, error += double(float(min + |x|^2)).  Returns (labels, error / n)."""
+    from concurrent.futures import ThreadPoolExecutor
+    n, k = x.shape[0], cent.shape[0]
+    y_sqr = np.einsum("ij,ij->i", cent, cent).astype(np.float32)
+    labels = np.empty(n, np.int32)
+    ct = np.ascontiguousarray(cent.T)
+    err = 0.0
+
+    def block(args):
+        dist, xb, lo, hi = args
+        blk = dist[lo:hi]
+        blk += y_sqr[None, :]
+        idx = blk.argmin(1)
+        labels_chunk[lo:hi] = idx
+        x_sqr = np.einsum("ij,ij->i", xb[lo:hi], xb[lo:hi]).astype(np.float32)
+        return float((blk[np.arange(hi - lo), idx] + x_sqr).astype(np.float64).sum())
+
+    with ThreadPoolExecutor(max_workers=threads) as pool:
+        for s in range(0, n, 65536):
+            xb = x[s:s + 65536]
+            dist = np.matmul(xb, ct)
+            dist *= np.float32(-2.0)
+            labels_chunk = labels[s:s + 65536]
+            m = xb.shape[0]
+            err += sum(pool.map(block, [(dist, xb, lo, min(lo + 1024, m)) for lo in range(0, m, 1024)]))
+    return labels, err / float(n)
+
+
 def device_rows(env, x_dev, rows, d):
     """Rows of a device-resident n x d fp32 matrix, copied one by one (a few thousand at most)."""
     rows = np.asarray(rows, np.int64)
@@ -109,6 +151,7 @@ class Env:
         capi.init(0)
         self.dev_name, self.cus, self.hbm = capi.device_info()
         self.args = args
+        self.stores = []
         capi.check(self.lib.vsag_amd_set_kernel_timing(1))
 
     def buf(self, nbytes):
@@ -133,7 +176,17 @@ class Env:
             p.rotation_dev, p.centroid_dev = rot.ptr, cen.ptr
         h = C.c_void_p()
         self.capi.check(self.lib.vsag_amd_store_create(C.byref(p), C.byref(h)))
+        self.stores.append(h)
         return h
+
+    def release(self):
+        """Destroys the stores of the configuration that just ran (its buffers go with their Python objects)."""
+        import gc
+        self.capi.synchronize()
+        for h in self.stores:
+            self.lib.vsag_amd_store_destroy(h)
+        self.stores = []
+        gc.collect()
 
     def timed(self, step, steps, warmup):
         for _ in range(warmup):
@@ -411,8 +464,8 @@ def run_c3(env):
         capi.check(lib.vsag_amd_memcpy_h2d(x_dev.ptr + s * d * 4, blk.ctypes.data, blk.nbytes, None))
         lo, hi = np.searchsorted(pick, [s, s + blk.shape[0]])
         init[lo:hi] = blk[pick[lo:hi] - s]
-        if s < (1 << 15):
-            sample_rows.append(blk[:8192].copy())
+        if s < (1 << 16):
+            sample_rows.append(blk.copy())  # the first 65 536 rows stay on the host for the CPU legs
     t_gen = time.time() - t0
     cent = env.upload(init)
     labels, loss = env.buf(n * 4), env.buf(8)
@@ -437,37 +490,61 @@ def run_c3(env):
     inertia = None
     if not args.no_cpu:
         import oracle as orc
-        xs = sample_rows[0]
         threads = min(os.cpu_count() or 1, 16)
         orc.set_threads(threads)
-        orc.kmeans_assign(xs[:256], init)
+        # (1) Assignment as the reference does it (find_nearest_one_with_blas): SGEMM per 65 536-row chunk through the
+        # OpenBLAS that numpy links, + |c|^2, first minimum, loss in double.  Timed on the first rows of the workload.
+        xs = np.concatenate(sample_rows)
+        cpu_assign_sgemm(xs[:4096], init, threads)  # BLAS thread pool and page warm-up
         t0 = time.perf_counter()
-        ol, _, oloss = orc.kmeans_assign(xs, init)
+        ol, oloss = cpu_assign_sgemm(xs, init, threads)
         t_cpu = time.perf_counter() - t0
         step()
         capi.synchronize()
         glabels = labels.to_numpy(np.int32, (n,))[:xs.shape[0]]
+        sl, _, _ = orc.kmeans_assign(xs[:1024], init)  # the scalar restatement on a few rows, for the record
         cpu = {"value": xs.shape[0] / t_cpu, "unit": "rows/s", "cores": threads, "kind": "port",
-               "sample": "first %d of the %d rows against all %d centroids, CPU restatement of "
-                         "find_nearest_one_with_blas (fp32 dot products in element order, eight centroids per vector, "
-                         "instead of OpenBLAS SGEMM), OpenMP over rows" % (xs.shape[0], n, k),
-               "label_agreement_with_gpu": float((ol == glabels).mean())}
-        # Final inertia against the CPU: the centroids after the ten iterations, assigned once more by both sides on
-        # the sample rows (inertia = mean over rows of the squared distance to the nearest centroid).
-        mind = env.buf(n * 4)
-        capi.check(lib.vsag_amd_kmeans_assign(x_dev.ptr, n, d, cent2.ptr, k, labels.ptr, mind.ptr, loss.ptr, ws_a.ptr,
-                                              wsb_a, None))
-        capi.synchronize()
-        final_cent = cent2.to_numpy(np.float32, (k, d))
-        fl, _, floss = orc.kmeans_assign(xs, final_cent)
-        gmin = mind.to_numpy(np.float32, (n,))[:xs.shape[0]].astype(np.float64)
-        gfl = labels.to_numpy(np.int32, (n,))[:xs.shape[0]]
-        g_inertia = float(np.mean(gmin + (xs.astype(np.float64) ** 2).sum(1)))
-        inertia = {"gpu_on_sample": g_inertia, "cpu_on_sample": float(floss),
-                   "relative_difference": abs(g_inertia - floss) / abs(floss),
-                   "label_agreement": float((fl == gfl).mean()), "sample_rows": int(xs.shape[0]),
-                   "gpu_all_rows_after_assignment": float(loss.to_numpy(np.float64, (1,))[0])}
-        mind.free()
+               "blas": blas_name(),
+               "sample": "first %d of the %d rows against all %d centroids; find_nearest_one_with_blas restated with "
+                         "its own steps: chunks of 65 536 rows, -2 C X^T by SGEMM (%s through numpy, %d threads), + |c|^2, "
+                         "std::min_element per row in blocks of 1024 rows on %d threads, loss in double" %
+                         (xs.shape[0], n, k, blas_name(), threads, threads),
+               "label_agreement_with_gpu": float((ol == glabels).mean()),
+               "label_agreement_sgemm_vs_scalar_restatement": float((ol[:1024] == sl).mean())}
+        # (2) Final inertia against the CPU: ten Lloyd iterations by both sides on one slice of the workload (its
+        # first 65 536 rows), from the same initial centroids (a seeded sample of the slice) and with the same
+        # re-seeding of empty clusters; the CPU side assigns through SGEMM as above.
+        ns = min(n, xs.shape[0], 65536)
+        xsl = np.ascontiguousarray(xs[:ns])
+        init_s = xsl[np.sort(mt(7).choice(ns, k, replace=False))].copy()
+        xs_dev, cs_dev = env.upload(xsl), env.upload(init_s)
+        ls_dev = env.buf(ns * 4)
+        wsb_s = lib.vsag_amd_kmeans_run_workspace_bytes(ns, d, k)
+        ws_s = env.buf(wsb_s)
+        g_loss = C.c_double()
+        capi.check(lib.vsag_amd_kmeans_run(xs_dev.ptr, ns, d, cs_dev.ptr, k, iters, 7, ls_dev.ptr, C.byref(g_loss),
+                                           ws_s.ptr, wsb_s, None))
+        g_lab = ls_dev.to_numpy(np.int32, (ns,))
+        g_cent = cs_dev.to_numpy(np.float32, (k, d))
+        t0 = time.perf_counter()
+        c_cent, c_lab, c_loss = orc.kmeans_run_with(xsl, init_s, iters, 7,
+                                                    lambda cc: cpu_assign_sgemm(xsl, np.array(cc), threads))
+        t_lloyd_cpu = time.perf_counter() - t0
+        # inertia of the final centroids (after the tenth update), by one more SGEMM assignment of the slice
+        _, g_final = cpu_assign_sgemm(xsl, g_cent, threads)
+        _, c_final = cpu_assign_sgemm(xsl, c_cent, threads)
+        inertia = {"slice_rows": int(ns), "iterations": iters,
+                   "gpu_loss_of_last_assignment": g_loss.value, "cpu_loss_of_last_assignment": float(c_loss),
+                   "relative_difference": abs(g_loss.value - c_loss) / abs(c_loss),
+                   "gpu_inertia_of_final_centroids": float(g_final), "cpu_inertia_of_final_centroids": float(c_final),
+                   "relative_difference_final": abs(g_final - c_final) / abs(c_final),
+                   "label_agreement_after_10_iterations": float((g_lab == c_lab).mean()),
+                   "cpu_lloyd_seconds": t_lloyd_cpu,
+                   "gpu_all_rows_loss_after_10_iterations": final.value,
+                   "what": "KMeansCluster::Run restated (SGEMM assignment, mean update, empty clusters re-seeded from "
+                           "mt19937(7)) on the CPU against vsag_amd_kmeans_run on the same %d x %d slice" % (ns, d)}
+        for b in (xs_dev, cs_dev, ls_dev, ws_s):
+            b.free()
     flops = 2.0 * n * k * d
     tf = flops / (kms * 1e-3) / 1e12
     roof = {"bound": "mfma", "achieved": tf, "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -604,7 +681,6 @@ def run_c4(env):
         gt_ids = gi.to_numpy(np.uint32, (nrec, k))
         rec = recall_at_k(ids[:nrec], gt_ids)
         w2.free()
-        lib.vsag_amd_store_destroy(flat)
     cpu = None
     if not args.no_cpu:
         # CPU restatement of IVF::search + reorder on a sample of the same queries, routing injected (the GPU's
@@ -751,7 +827,6 @@ def run_c5(env):
         gt_ids = gi.to_numpy(np.uint32, (nrec, k))
         rec = recall_at_k(ids[:nrec], gt_ids)
         w2.free()
-        lib.vsag_amd_store_destroy(flat)
     cpu = None
     if not args.no_cpu:
         # CPU restatement of the RaBitQ scan (ProcessQueryImpl + ComputeQueryBaseImpl + heap) on a sample of the same
@@ -839,6 +914,8 @@ def main():
     ap.add_argument("--no-single", action="store_true", help="skip the one-query-per-call measurement")
     ap.add_argument("--no-api", action="store_true", help="skip the index-API leg (host buffers on both sides)")
     ap.add_argument("--no-kmeans", action="store_true", help="default line only: skip the k-means block (configs[2])")
+    ap.add_argument("--only", action="store_true", help="--config c2 alone, without the blocks of the other configurations")
+    ap.add_argument("--skip", default="", help="default line only: blocks to leave out, e.g. c4,c5")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the search core is single-GPU by design (sharding it means splitting "
@@ -847,18 +924,33 @@ def main():
         sys.exit(2)
     env = Env(args)
     env.capi.check(env.lib.vsag_amd_set_scan_contraction(args.contraction))
-    line = {"c1": run_c1, "c2": run_c2, "c3": run_c3, "c4": run_c4, "c5": run_c5}[args.config](env)
-    if args.config == "c2" and not args.no_kmeans and not (args.n or args.dim or args.nq):
-        # The metric's second figure, "k-means assign rows/s": configs[2] in the same line.
-        env.capi.check(env.lib.vsag_amd_set_scan_tuning(0, 0))
-        km = run_c3(env)
-        line["kmeans"] = {"metric": km["metric"], "value": km["value"], "unit": km["unit"],
-                          "ms_per_step": km["ms_per_step"], "dtype": km["dtype"], "workload": km["config"]["workload"],
-                          "lloyd_iterations": km["config"]["lloyd_iterations"],
-                          "lloyd_seconds": km["config"]["lloyd_seconds"], "final_loss": km["config"]["final_loss"],
-                          "final_inertia_vs_cpu": km["config"]["final_inertia_vs_cpu"],
-                          "datagen_seconds": km["config"]["datagen_seconds"],
-                          "roofline": km["roofline"], "cpu_baseline": km["cpu_baseline"]}
+    runs = {"c1": run_c1, "c2": run_c2, "c3": run_c3, "c4": run_c4, "c5": run_c5}
+    line = runs[args.config](env)
+    env.release()
+    if args.config == "c2" and not args.only and not (args.n or args.dim or args.nq):
+        # The default line carries all five configurations: configs[1] is the line itself (the headline metric), the
+        # others are blocks of the same shape -- "kmeans" (configs[2], the metric's second figure), "c1" (configs[0]),
+        # "c4" (configs[3]) and "c5" (configs[4]) -- each timed with the same --steps / --warmup, with its own roofline
+        # and its own CPU baseline on a bounded sample.
+        def block(cfg):
+            env.capi.check(env.lib.vsag_amd_set_scan_tuning(0, 0))
+            t0 = time.perf_counter()
+            full = runs[cfg](env)
+            env.release()
+            c = full["config"]
+            out = {"metric": full["metric"], "value": full["value"], "unit": full["unit"],
+                   "ms_per_step": full["ms_per_step"], "steps": full["steps"], "warmup": full["warmup"],
+                   "dtype": full["dtype"], "workload": c["workload"]}
+            out.update({k: v for k, v in c.items() if k not in ("workload", "device", "compute_units")})
+            out["roofline"] = full["roofline"]
+            out["cpu_baseline"] = full["cpu_baseline"]
+            out["block_wall_seconds"] = time.perf_counter() - t0
+            return out
+        if not args.no_kmeans:
+            line["kmeans"] = block("c3")
+        for cfg in ("c1", "c4", "c5"):
+            if cfg not in args.skip:
+                line[cfg] = block(cfg)
     print(json.dumps(line))
 
 

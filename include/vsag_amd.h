@@ -68,6 +68,11 @@ VSAG_AMD_API int vsag_amd_device_info(char* name, size_t name_bytes, int* comput
  * touch host memory return after the copy has finished; d2d and memset are asynchronous. */
 VSAG_AMD_API int vsag_amd_malloc(void** ptr_dev, size_t bytes);
 VSAG_AMD_API int vsag_amd_free(void* ptr_dev);
+/* Free and total device memory (hipMemGetInfo) and the high-water mark of the stream-ordered allocator's default
+ * pool since it was last reset (reset_high != 0 resets it after reading): what a caller needs to check that a
+ * call allocated nothing.  Any pointer may be NULL. */
+VSAG_AMD_API int vsag_amd_memory_info(uint64_t* free_bytes, uint64_t* total_bytes, uint64_t* async_pool_high_bytes,
+                                      int reset_high);
 VSAG_AMD_API int vsag_amd_memcpy_h2d(void* dst_dev, const void* src, size_t bytes, void* stream);
 VSAG_AMD_API int vsag_amd_memcpy_d2h(void* dst, const void* src_dev, size_t bytes, void* stream);
 VSAG_AMD_API int vsag_amd_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);

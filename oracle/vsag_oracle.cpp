@@ -1146,15 +1146,19 @@ orc_kmeans_init_pp(const float* x, uint64_t n, uint64_t dim, uint64_t k, uint64_
 
 // Lloyd driver (kmeans_cluster.cpp:46-190) with the initial centroids given and empty clusters
 // re-seeded from mt19937(seed) + uniform_int_distribution<uint64_t>(0, n-1), drawn in cluster order.
-// Returns the loss of the last assignment (err / n).
+// Returns the loss of the last assignment (err / n).  `assign` replaces the assignment step when given
+// (a caller with a BLAS runs find_nearest_one_with_blas as the reference does, through SGEMM): it fills
+// labels for the centroids it is handed and returns err / n.
+typedef double (*orc_assign_fn)(const float* cent, int32_t* labels, void* user);
+
 ORC_API double
-orc_kmeans_run(const float* x, uint64_t n, uint64_t dim, float* cent /* in: init, out: final */, uint64_t k, int iters,
-               uint64_t seed, int32_t* labels) {
+orc_kmeans_run_with(const float* x, uint64_t n, uint64_t dim, float* cent /* in: init, out: final */, uint64_t k,
+                    int iters, uint64_t seed, int32_t* labels, orc_assign_fn assign, void* user) {
     std::mt19937 gen(static_cast<uint32_t>(seed));
     std::vector<int32_t> counts(k);
     double err = 0;
     for (int it = 0; it < iters; ++it) {
-        err = orc_kmeans_assign(x, n, dim, cent, k, labels, nullptr);
+        err = assign != nullptr ? assign(cent, labels, user) : orc_kmeans_assign(x, n, dim, cent, k, labels, nullptr);
         orc_kmeans_update(x, labels, n, dim, k, cent, counts.data());
         std::uniform_int_distribution<uint64_t> dis(0, n - 1);
         for (uint64_t j = 0; j < k; ++j) {
@@ -1165,6 +1169,12 @@ orc_kmeans_run(const float* x, uint64_t n, uint64_t dim, float* cent /* in: init
         }
     }
     return err;
+}
+
+ORC_API double
+orc_kmeans_run(const float* x, uint64_t n, uint64_t dim, float* cent, uint64_t k, int iters, uint64_t seed,
+               int32_t* labels) {
+    return orc_kmeans_run_with(x, n, dim, cent, k, iters, seed, labels, nullptr, nullptr);
 }
 
 // ---- flat scan with bounded heap (BruteForce::SearchWithRequest hot loop) ----------------------

@@ -32,6 +32,7 @@ def lib():
         _lib = C.CDLL(LIB)
         _lib.orc_kmeans_assign.restype = C.c_double
         _lib.orc_kmeans_run.restype = C.c_double
+        _lib.orc_kmeans_run_with.restype = C.c_double
         for name in ("orc_fp32_l2sqr", "orc_fp32_ip", "orc_sq8_ip", "orc_sq8_l2sqr", "orc_sq4_ip", "orc_sq4_l2sqr",
                      "orc_squ_dist", "orc_rabitq_dist", "orc_normalize", "orc_normalize_with_centroid",
                      "orc_rabitq_float_binary_ip"):
@@ -218,6 +219,26 @@ def kmeans_run(x, cent0, iters, seed):
     k = cent.shape[0]
     labels = np.empty(n, np.int32)
     loss = lib().orc_kmeans_run(_p(x), u64(n), u64(d), _p(cent), u64(k), iters, u64(seed), _p(labels))
+    return cent, labels, loss
+
+
+def kmeans_run_with(x, cent0, iters, seed, assign):
+    """kmeans_run with the assignment step done by `assign(cent[k, d]) -> (labels[n], err / n)` (the update and the
+    re-seeding of empty clusters stay the checker's)."""
+    x = f32(x)
+    cent = f32(cent0).copy()
+    n, d = x.shape
+    k = cent.shape[0]
+    labels = np.empty(n, np.int32)
+
+    @C.CFUNCTYPE(C.c_double, C.POINTER(C.c_float), C.POINTER(C.c_int32), C.c_void_p)
+    def step(cent_p, labels_p, _user):
+        c = np.ctypeslib.as_array(cent_p, shape=(k, d))
+        out, err = assign(c)
+        np.ctypeslib.as_array(labels_p, shape=(n,))[:] = out
+        return float(err)
+
+    loss = lib().orc_kmeans_run_with(_p(x), u64(n), u64(d), _p(cent), u64(k), iters, u64(seed), _p(labels), step, None)
     return cent, labels, loss
 
 

@@ -53,6 +53,7 @@ PROTOTYPES = {
     "vsag_amd_memcpy_d2h": (C.c_int, [_vp, _vp, _sz, _vp]),
     "vsag_amd_memcpy_d2d": (C.c_int, [_vp, _vp, _sz, _vp]),
     "vsag_amd_memset": (C.c_int, [_vp, C.c_int, _sz, _vp]),
+    "vsag_amd_memory_info": (C.c_int, [_vp, _vp, _vp, C.c_int]),
     "vsag_amd_stream_synchronize": (C.c_int, [_vp]),
     "vsag_amd_stream_create": (C.c_int, [C.POINTER(_vp)]),
     "vsag_amd_stream_destroy": (C.c_int, [_vp]),

@@ -80,6 +80,9 @@ div_up(uint64_t v, uint64_t a) {
     return (v + a - 1) / a;
 }
 
+// The RaBitQ rotation y = R x is done for this many rows at a time, so that its temporary stays bounded.
+constexpr uint64_t kRotateSlabRows = 1ull << 18;
+
 // Carves 256-byte aligned pieces out of a caller-supplied workspace.
 struct Carver {
     uint8_t* base;

@@ -915,12 +915,7 @@ plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, 
     }
     p->T = t;
     p->ql = query_layout(s);
-    p->qcode_bytes = 0;
-    if (s->kind == VSAG_AMD_KIND_SQ4_UNIFORM || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
-        p->qcode_bytes = nq * s->code_size;
-    } else if (s->kind == VSAG_AMD_KIND_RABITQ) {
-        p->qcode_bytes = nq * rabitq_query_code_size(s->dim, s->metric, s->query_bits);
-    }
+    p->qcode_bytes = query_staging_bytes(s, nq);
     p->npairs = npairs;
     // Enough (list, query group) items to fill the machine: every item walks its whole list, the nearest list
     // of every query goes first.  Otherwise lists are cut into chunks of at least four tiles for about 4096 items in all (a probed

@@ -142,12 +142,7 @@ struct LookupBuffers {
 static size_t
 carve_lookup(Carver& c, const vsag_amd_store* s, uint64_t nq, LookupBuffers* b) {
     const QueryLayout ql = query_layout(s);
-    size_t qcode_bytes = 0;
-    if (s->kind == VSAG_AMD_KIND_SQ4_UNIFORM || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
-        qcode_bytes = nq * s->code_size;
-    } else if (s->kind == VSAG_AMD_KIND_RABITQ) {
-        qcode_bytes = nq * rabitq_query_code_size(s->dim, s->metric, s->query_bits);
-    }
+    size_t qcode_bytes = query_staging_bytes(s, nq);
     b->qtab = c.take<uint32_t>(nq * ql.qstride);
     b->qmeta = c.take<float>(nq * ql.qmeta);
     b->qcodes = c.take<uint8_t>(qcode_bytes);

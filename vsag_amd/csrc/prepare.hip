@@ -196,9 +196,41 @@ prepare_rabitq_queries(const uint8_t* qcodes, uint64_t nq, uint32_t qcode_size, 
 
 uint64_t rabitq_query_code_size(uint32_t dim, int metric, int query_bits);
 int squ_encode_launch(const float* x, uint64_t n, uint32_t dim, int bits, int metric, const float* bounds,
-                      uint8_t* codes, hipStream_t st);
+                      uint8_t* codes, hipStream_t st, float* norm_scratch);
 int rabitq_process_query_launch(const float* q, uint64_t nq, uint32_t dim, const float* rot, const float* centroid,
-                                int metric, int query_bits, uint8_t* qcodes, hipStream_t st);
+                                int metric, int query_bits, uint8_t* qcodes, hipStream_t st, float* scratch);
+
+// Bytes of the encoded queries of a call (uniform kinds, rabitq; zero for the kinds that keep fp32 queries).
+static size_t
+query_code_bytes(const vsag_amd_store* s, uint64_t nq) {
+    if (s->kind == VSAG_AMD_KIND_SQ4_UNIFORM || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
+        return nq * s->code_size;
+    }
+    if (s->kind == VSAG_AMD_KIND_RABITQ) {
+        return nq * rabitq_query_code_size(s->dim, s->metric, s->query_bits);
+    }
+    return 0;
+}
+
+// What the query encoders need besides their output: the rotated queries of one slab (rabitq), a norm per
+// query (uniform kinds under cosine).
+static size_t
+query_scratch_bytes(const vsag_amd_store* s, uint64_t nq) {
+    if (s->kind == VSAG_AMD_KIND_RABITQ) {
+        return static_cast<size_t>(nq < kRotateSlabRows ? nq : kRotateSlabRows) * s->dim * 4;
+    }
+    if ((s->kind == VSAG_AMD_KIND_SQ4_UNIFORM || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) &&
+        s->metric == VSAG_AMD_METRIC_COSINE) {
+        return nq * 4;
+    }
+    return 0;
+}
+
+size_t
+query_staging_bytes(const vsag_amd_store* s, uint64_t nq) {
+    size_t scratch = query_scratch_bytes(s, nq);
+    return scratch == 0 ? query_code_bytes(s, nq) : round_up(query_code_bytes(s, nq), 256) + scratch;
+}
 
 QueryLayout
 query_layout(const vsag_amd_store* s) {
@@ -282,11 +314,15 @@ prepare_rabitq_f32_queries(const uint8_t* qcodes, uint64_t nq, uint32_t qcode_si
     }
 }
 
-// Runs ProcessQueryImpl of the store's quantizer for nq raw queries and fills the scan tables.
+// Runs ProcessQueryImpl of the store's quantizer for nq raw queries and fills the scan tables.  `qcodes` is
+// query_staging_bytes(s, nq) of device memory (the encoded queries, then the encoders' scratch): nothing is
+// allocated here.
 int
 prepare_queries(const vsag_amd_store* s, const float* queries, uint64_t nq, uint64_t nq_pad, const QueryLayout& ql,
                 uint32_t* qtab, float* qmeta, uint8_t* qcodes, hipStream_t st) {
     dim3 grid(static_cast<uint32_t>(nq_pad));
+    float* scratch = query_scratch_bytes(s, nq) == 0 ? nullptr :
+                     reinterpret_cast<float*>(qcodes + round_up(query_code_bytes(s, nq), 256));
     switch (s->kind) {
         case VSAG_AMD_KIND_FP32:
         case VSAG_AMD_KIND_SQ8:
@@ -297,7 +333,7 @@ prepare_queries(const vsag_amd_store* s, const float* queries, uint64_t nq, uint
         case VSAG_AMD_KIND_SQ4_UNIFORM:
         case VSAG_AMD_KIND_SQ8_UNIFORM: {
             int bits = s->kind == VSAG_AMD_KIND_SQ4_UNIFORM ? 4 : 8;
-            VA_TRY(squ_encode_launch(queries, nq, s->dim, bits, s->metric, s->bounds_dev, qcodes, st));
+            VA_TRY(squ_encode_launch(queries, nq, s->dim, bits, s->metric, s->bounds_dev, qcodes, st, scratch));
             hipLaunchKernelGGL(prepare_uniform_queries, grid, dim3(256), 0, st, qcodes, nq, s->code_size,
                                s->payload_bytes, bits, s->meta_offset[0], static_cast<int>(s->meta_is_u64 & 1),
                                s->G * 4, qtab, ql.qstride, qmeta, ql.qmeta);
@@ -306,7 +342,7 @@ prepare_queries(const vsag_amd_store* s, const float* queries, uint64_t nq, uint
         case VSAG_AMD_KIND_RABITQ: {
             VA_CHECK_ARG(s->query_bits == 4 || s->query_bits == 32, "rabitq scan supports 4-bit and fp32 queries");
             VA_TRY(rabitq_process_query_launch(queries, nq, s->dim, s->rotation_dev, s->centroid_dev, s->metric,
-                                               s->query_bits, qcodes, st));
+                                               s->query_bits, qcodes, st, scratch));
             if (s->query_bits == 32) {
                 hipLaunchKernelGGL(prepare_rabitq_f32_queries, grid, dim3(256), 0, st, qcodes, nq,
                                    static_cast<uint32_t>(rabitq_query_code_size(s->dim, s->metric, 32)), s->dim,

@@ -570,7 +570,7 @@ rabitq_finish_query_wave_kernel(const float* raw, const float* rotated, uint64_t
 
 int
 squ_encode_launch(const float* x, uint64_t n, uint32_t dim, int bits, int metric, const float* bounds, uint8_t* codes,
-                  hipStream_t st) {
+                  hipStream_t st, float* norm_scratch) {
     if (n == 0) {
         return 0;
     }
@@ -583,29 +583,37 @@ squ_encode_launch(const float* x, uint64_t n, uint32_t dim, int bits, int metric
     uint32_t off_norm = off;
     uint32_t off_sum = off + (norm ? 8 : 0);
     uint32_t off_codes_sum = off_sum + align;
+    // Cosine needs a float per row; a caller that must not allocate brings them (norm_scratch, n floats).
     float* norms = nullptr;
     if (metric == VSAG_AMD_METRIC_COSINE) {
-        VA_HIP(hipMallocAsync(reinterpret_cast<void**>(&norms), n * 4, st));
+        norms = norm_scratch;
+        if (norms == nullptr) {
+            VA_HIP(hipMallocAsync(reinterpret_cast<void**>(&norms), n * 4, st));
+        }
         hipLaunchKernelGGL(row_norm_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, x, n, dim,
                            norms);
     }
     hipLaunchKernelGGL(squ_encode_kernel, dim3(static_cast<uint32_t>(div_up(n, 4))), dim3(256), 0, st, x, n, dim, bits,
                        metric, bounds, norms, code_size, payload, off_norm, off_sum, off_codes_sum, codes);
     VA_HIP(hipGetLastError());
-    if (norms != nullptr) {
+    if (norms != nullptr && norms != norm_scratch) {
         VA_HIP(hipFreeAsync(norms, st));
     }
     return 0;
 }
 
-// Rotates rows in slabs so that the temporary stays bounded, then runs `finish` on each slab.
+// Rotates rows in slabs so that the temporary stays bounded, then runs `finish` on each slab.  The temporary
+// (min(n, kRotateSlabRows) x dim floats) is `scratch` when the caller brings one, else allocated on the stream.
 template <typename Finish>
 static int
-rabitq_rotate_slabs(const float* x, uint64_t n, uint32_t dim, const float* rot, hipStream_t st, Finish finish) {
-    const uint64_t slab = 1ull << 18;
+rabitq_rotate_slabs(const float* x, uint64_t n, uint32_t dim, const float* rot, hipStream_t st, float* scratch,
+                    Finish finish) {
+    const uint64_t slab = kRotateSlabRows;
     uint64_t rows = n < slab ? n : slab;
-    float* tmp = nullptr;
-    VA_HIP(hipMallocAsync(reinterpret_cast<void**>(&tmp), rows * dim * 4, st));
+    float* tmp = scratch;
+    if (tmp == nullptr) {
+        VA_HIP(hipMallocAsync(reinterpret_cast<void**>(&tmp), rows * dim * 4, st));
+    }
     int rc = 0;
     for (uint64_t s = 0; s < n && rc == 0; s += slab) {
         uint64_t m = n - s < slab ? n - s : slab;
@@ -614,21 +622,23 @@ rabitq_rotate_slabs(const float* x, uint64_t n, uint32_t dim, const float* rot, 
             rc = finish(s, m, tmp);
         }
     }
-    hipError_t e = hipFreeAsync(tmp, st);
-    if (rc == 0 && e != hipSuccess) {
-        return fail(VSAG_AMD_INTERNAL_ERROR, "hipFreeAsync failed: %s", hipGetErrorString(e));
+    if (tmp != scratch) {
+        hipError_t e = hipFreeAsync(tmp, st);
+        if (rc == 0 && e != hipSuccess) {
+            return fail(VSAG_AMD_INTERNAL_ERROR, "hipFreeAsync failed: %s", hipGetErrorString(e));
+        }
     }
     return rc;
 }
 
 int
 rabitq_process_query_launch(const float* q, uint64_t nq, uint32_t dim, const float* rot, const float* centroid,
-                            int metric, int query_bits, uint8_t* qcodes, hipStream_t st) {
+                            int metric, int query_bits, uint8_t* qcodes, hipStream_t st, float* scratch) {
     if (nq == 0) {
         return 0;
     }
     uint64_t qsize = rabitq_query_code_size(dim, metric, query_bits);
-    return rabitq_rotate_slabs(q, nq, dim, rot, st, [&](uint64_t s, uint64_t m, const float* rotated) {
+    return rabitq_rotate_slabs(q, nq, dim, rot, st, scratch, [&](uint64_t s, uint64_t m, const float* rotated) {
         const size_t lds = static_cast<size_t>(dim) * 4 * (rabitq_layout(dim, metric, query_bits).has_raw_norm ? 2 : 1);
         if (lds <= 48 * 1024) {
             hipLaunchKernelGGL(rabitq_finish_query_wave_kernel, dim3(static_cast<uint32_t>(m)), dim3(64), lds, st,
@@ -878,7 +888,8 @@ vsag_amd_squ_encode(const float* x_dev, uint64_t n, uint32_t dim, int bits, int 
     VA_CHECK_ARG(bits == 4 || bits == 8, "bits must be 4 or 8, got %d", bits);
     VA_CHECK_ARG(dim >= 1 && dim <= 65536, "dim must be in [1, 65536], got %u", dim);
     VA_CHECK_ARG(n == 0 || (x_dev && bounds_dev && codes_dev), "null pointer");
-    return squ_encode_launch(x_dev, n, dim, bits, metric, bounds_dev, codes_dev, static_cast<hipStream_t>(stream));
+    return squ_encode_launch(x_dev, n, dim, bits, metric, bounds_dev, codes_dev, static_cast<hipStream_t>(stream),
+                             nullptr);
 }
 
 extern "C" int
@@ -909,7 +920,7 @@ vsag_amd_rabitq_encode(const float* x_dev, uint64_t n, uint32_t dim, const float
     VA_CHECK_ARG(x_dev && rotation_dev && centroid_dev && codes_dev, "null pointer");
     hipStream_t st = static_cast<hipStream_t>(stream);
     uint64_t csize = rabitq_code_size(dim, metric, query_bits);
-    return rabitq_rotate_slabs(x_dev, n, dim, rotation_dev, st, [&](uint64_t s, uint64_t m, const float* rotated) {
+    return rabitq_rotate_slabs(x_dev, n, dim, rotation_dev, st, nullptr, [&](uint64_t s, uint64_t m, const float* rotated) {
         hipLaunchKernelGGL(rabitq_finish_encode_kernel, dim3(static_cast<uint32_t>(div_up(m, 64))), dim3(64), 0, st,
                            x_dev + s * dim, rotated, m, dim, centroid_dev, metric, query_bits, codes_dev + s * csize);
         VA_HIP(hipGetLastError());
@@ -931,5 +942,5 @@ vsag_amd_rabitq_process_query(const float* q_dev, uint64_t nq, uint32_t dim, con
     VA_CHECK_ARG(dim >= 1 && dim <= 65536, "dim must be in [1, 65536], got %u", dim);
     VA_CHECK_ARG(nq == 0 || (q_dev && rotation_dev && centroid_dev && qcodes_dev), "null pointer");
     return rabitq_process_query_launch(q_dev, nq, dim, rotation_dev, centroid_dev, metric, query_bits, qcodes_dev,
-                                       static_cast<hipStream_t>(stream));
+                                       static_cast<hipStream_t>(stream), nullptr);
 }

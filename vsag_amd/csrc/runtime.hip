@@ -188,6 +188,33 @@ vsag_amd_free(void* ptr_dev) {
 }
 
 extern "C" int
+vsag_amd_memory_info(uint64_t* free_bytes, uint64_t* total_bytes, uint64_t* async_pool_high_bytes, int reset_high) {
+    VA_TRY(ensure_init());
+    size_t f = 0, t = 0;
+    VA_HIP(hipMemGetInfo(&f, &t));
+    if (free_bytes != nullptr) {
+        *free_bytes = f;
+    }
+    if (total_bytes != nullptr) {
+        *total_bytes = t;
+    }
+    int device = 0;
+    VA_HIP(hipGetDevice(&device));
+    hipMemPool_t pool = nullptr;
+    VA_HIP(hipDeviceGetDefaultMemPool(&pool, device));
+    if (async_pool_high_bytes != nullptr) {
+        uint64_t high = 0;
+        VA_HIP(hipMemPoolGetAttribute(pool, hipMemPoolAttrUsedMemHigh, &high));
+        *async_pool_high_bytes = high;
+    }
+    if (reset_high) {
+        uint64_t zero = 0;
+        VA_HIP(hipMemPoolSetAttribute(pool, hipMemPoolAttrUsedMemHigh, &zero));
+    }
+    return 0;
+}
+
+extern "C" int
 vsag_amd_memcpy_h2d(void* dst_dev, const void* src, size_t bytes, void* stream) {
     VA_TRY(ensure_init());
     if (bytes == 0) {

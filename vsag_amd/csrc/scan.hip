@@ -13,6 +13,7 @@
 // survivors that the bound still admits; a merge kernel picks the k best per query.  All waves of a query
 // share a handful of addresses (its bound, its seed row), and atomics on one address serialise in L2, so
 // every atomicMin is preceded by a plain load and issued only when it would lower the value.
+#include <atomic>
 #include <mutex>
 
 #include "distance.h"
@@ -788,12 +789,7 @@ make_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, uint64_t ntiles, Sca
     // Seeding pays when a query's waves all start cold together, i.e. when the whole grid is resident at once.
     p->seeded = p->chunks * waves >= 2ull * k && k <= 256 && p->groups * p->chunks * waves <= 8192;
     p->ql = query_layout(s);
-    p->qcode_bytes = 0;
-    if (s->kind == VSAG_AMD_KIND_SQ4_UNIFORM || s->kind == VSAG_AMD_KIND_SQ8_UNIFORM) {
-        p->qcode_bytes = nq * s->code_size;
-    } else if (s->kind == VSAG_AMD_KIND_RABITQ) {
-        p->qcode_bytes = nq * rabitq_query_code_size(s->dim, s->metric, s->query_bits);
-    }
+    p->qcode_bytes = query_staging_bytes(s, nq);
 }
 
 // A call is served either by one streaming launch over all tiles, or -- large batches on fp32 / sq8 stores
@@ -1552,7 +1548,7 @@ constexpr size_t kStaticScratchBytes = 32ull << 20;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 constexpr int kMaxScratchDevices = 64;
-static void* g_scratch_ptr[kMaxScratchDevices] = {};
+static std::atomic<void*> g_scratch_ptr[kMaxScratchDevices] = {};
 static std::mutex g_scratch_mutex;
 
 namespace vsag_amd {
@@ -1561,7 +1557,7 @@ int
 static_scratch_setup(int device) {
     VA_CHECK_ARG(device >= 0 && device < kMaxScratchDevices, "device %d out of range [0, %d)", device, kMaxScratchDevices);
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    if (g_scratch_ptr[device] != nullptr) {
+    if (g_scratch_ptr[device].load(std::memory_order_acquire) != nullptr) {
         return 0;
     }
     void* ptr = nullptr;
@@ -1569,7 +1565,7 @@ static_scratch_setup(int device) {
     if (ptr == nullptr) {
         return fail(VSAG_AMD_INTERNAL_ERROR, "the library's scratch array has no address on device %d", device);
     }
-    g_scratch_ptr[device] = ptr;
+    g_scratch_ptr[device].store(ptr, std::memory_order_release);
     return 0;
 }
 bool timing_suppress(bool off);
@@ -1589,10 +1585,11 @@ vsag_amd_flat_scan_topk_noalloc(const vsag_amd_store_t* s, const float* queries_
     int device = 0;
     VA_HIP(hipGetDevice(&device));
     VA_CHECK_ARG(device >= 0 && device < kMaxScratchDevices, "device %d out of range [0, %d)", device, kMaxScratchDevices);
-    if (g_scratch_ptr[device] == nullptr) {
+    if (g_scratch_ptr[device].load(std::memory_order_acquire) == nullptr) {
         // A device the library was not initialised on: first call there.
         VA_TRY(static_scratch_setup(device));
     }
+    void* const scratch_dev = g_scratch_ptr[device].load(std::memory_order_acquire);
     const size_t need = vsag_amd_flat_scan_workspace_bytes(s, nq, k);
     VA_CHECK_ARG(need != 0 && need <= kStaticScratchBytes,
                  "this scan needs %zu bytes of scratch memory, the library's own array holds %zu: send fewer queries "
@@ -1600,7 +1597,7 @@ vsag_amd_flat_scan_topk_noalloc(const vsag_amd_store_t* s, const float* queries_
                  need, kStaticScratchBytes);
     // The measurement hook creates events on first use: not in this call.
     const bool was = timing_suppress(true);
-    const int rc = flat_scan_call(s, queries_dev, nq, k, options, ids_dev, dists_dev, g_scratch_ptr[device],
+    const int rc = flat_scan_call(s, queries_dev, nq, k, options, ids_dev, dists_dev, scratch_dev,
                                   kStaticScratchBytes, stream);
     timing_suppress(was);
     return rc;

@@ -94,6 +94,9 @@ struct QueryLayout {
 };
 
 QueryLayout query_layout(const vsag_amd_store* s);
+// Device bytes prepare_queries needs behind its `qcodes` pointer for nq queries: the encoded queries of the kinds
+// that encode them, then whatever their encoders use as scratch.
+size_t query_staging_bytes(const vsag_amd_store* s, uint64_t nq);
 int launch_code_terms(vsag_amd_store* s, uint64_t first, uint64_t count, hipStream_t st);
 
 }  // namespace vsag_amd
