@@ -326,7 +326,7 @@ def run_c2(env):
         threads = min(os.cpu_count() or 1, 16)
         isa = orc.ref_best_isa()
         fn = orc.ref_sq8_fn(orc.L2, isa)
-        sample = min(nq, 8 * threads)
+        sample = min(nq, 64 * threads)
 
         def run_cpu(qs, th):
             if fn is not None:
@@ -420,14 +420,22 @@ def run_c1(env):
     if not args.no_cpu:
         import oracle as orc
         threads = min(os.cpu_count() or 1, 16)
-        sample = min(nq, 16 * threads)
+        sample = nq
         codes = x.view(np.uint8).reshape(n, 4 * d)
+        ref = orc.use_reference_kernels(orc.ref_best_isa())
         orc.flat_scan_topk(orc.FP32, orc.L2, d, codes, q[:threads], k, threads=threads)
         t0 = time.perf_counter()
-        orc.flat_scan_topk(orc.FP32, orc.L2, d, codes, q[:sample], k, threads=threads)
-        cpu = {"value": sample / (time.perf_counter() - t0), "unit": "queries/s", "cores": threads, "kind": "port",
-               "sample": "%d of the %d queries over all %d vectors, CPU restatement of generic::FP32ComputeL2Sqr + "
-                         "BruteForce loop, OpenMP over queries" % (sample, nq, n)}
+        cids, _ = orc.flat_scan_topk(orc.FP32, orc.L2, d, codes, q[:sample], k, threads=threads)
+        t_cpu = time.perf_counter() - t0
+        orc.use_reference_kernels(None)
+        cpu = {"value": sample / t_cpu, "unit": "queries/s", "cores": threads,
+               "kind": "reference" if ref else "port",
+               "sample": "%d of the %d queries over all %d vectors, one query per call, OpenMP dynamic over queries; "
+                         "distance = %s, loop and heap = restated BruteForce::SearchWithRequest" %
+                         (sample, nq, n, (ref["FP32ComputeL2Sqr"] + " compiled from the reference sources") if ref
+                          else "CPU restatement of generic::FP32ComputeL2Sqr"),
+               "topk_overlap_with_gpu": float(np.mean([len(set(a) & set(b)) / float(k)
+                                                       for a, b in zip(cids, ids[:sample])]))}
     algo = passes * bpp
     achieved = algo / (kms * 1e-3) / 1e9
     roof = {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
@@ -464,8 +472,8 @@ def run_c3(env):
         capi.check(lib.vsag_amd_memcpy_h2d(x_dev.ptr + s * d * 4, blk.ctypes.data, blk.nbytes, None))
         lo, hi = np.searchsorted(pick, [s, s + blk.shape[0]])
         init[lo:hi] = blk[pick[lo:hi] - s]
-        if s < (1 << 16):
-            sample_rows.append(blk.copy())  # the first 65 536 rows stay on the host for the CPU legs
+        if s < (1 << 18):
+            sample_rows.append(blk.copy())  # the first 262 144 rows stay on the host for the CPU legs
     t_gen = time.time() - t0
     cent = env.upload(init)
     labels, loss = env.buf(n * 4), env.buf(8)
@@ -687,7 +695,7 @@ def run_c4(env):
         # exact routing), same codes and lists: candidates, reranked ids and recall must agree.
         import oracle as orc
         threads = min(os.cpu_count() or 1, 16)
-        sample = min(nq, 16 * threads)
+        sample = min(nq, 64 * threads)
         hcodes = codes.to_numpy(np.uint8, (n, cs))
         hlabels = labels.to_numpy(np.int32, (n,))
         offsets, order = orc.ivf_build_lists(hlabels, nlist)
@@ -703,12 +711,17 @@ def run_c4(env):
             hb = bounds.to_numpy(np.float32, (2,))
             okind = orc.SQ8U if bits == 8 else orc.SQ4U
             qcodes = orc.squ_encode(q[:sample], bits, hb[0], hb[1], orc.L2)
+        ref = orc.use_reference_kernels(orc.ref_best_isa())
+        ref_name = {orc.SQ4U: "SQ4UniformComputeCodesIP", orc.SQ8U: "SQ8UniformComputeCodesIP",
+                    orc.RABITQ: "RaBitQSQ4UBinaryIP"}.get(okind)
+        ref = ref if ref and ref_name in ref else None
         orc.ivf_scan(okind, orc.L2, d, posting, offsets, order, qcodes[:threads], b[:threads], kcand,
                      lb=hb[0], diff=hb[1], threads=threads)
         t0 = time.perf_counter()
         cids, cds = orc.ivf_scan(okind, orc.L2, d, posting, offsets, order, qcodes, b[:sample], kcand,
                                  lb=hb[0], diff=hb[1], threads=threads)
         t_cpu = time.perf_counter() - t0
+        orc.use_reference_kernels(None)
         gcand = cand.to_numpy(np.uint32, (nq, kcand))[:sample]
         gcd = cand_d.to_numpy(np.float32, (nq, kcand))[:sample]
         uniq = np.unique(cids[cids != 0xFFFFFFFF])
@@ -719,10 +732,12 @@ def run_c4(env):
             rows = raw[[pos[int(v)] for v in cids[i]]]
             dd = ((rows.astype(np.float64) - q[i].astype(np.float64)) ** 2).sum(1)
             rids[i] = cids[i][np.lexsort((cids[i], dd))[:k]]
-        cpu = {"value": sample / t_cpu, "unit": "queries/s", "cores": threads, "kind": "port",
-               "sample": "%d of the %d queries, CPU restatement of IVF::search (scan of the same %d probed lists per "
-                         "query with the strict-< heap) on the same %s codes, OpenMP over queries; rerank in "
-                         "fp64 on the host" % (sample, nq, nprobe, kind_name),
+        cpu = {"value": sample / t_cpu, "unit": "queries/s", "cores": threads, "kind": "reference" if ref else "port",
+               "sample": "%d of the %d queries, one query per call, OpenMP dynamic over queries; restated IVF::search "
+                         "(scan of the same %d probed lists per query with the strict-< heap) on the same %s codes, lists "
+                         "and routing; distance kernel = %s; rerank in fp64 on the host (not timed)" %
+                         (sample, nq, nprobe, kind_name, (ref[ref_name] + " compiled from the reference sources") if ref
+                          else "CPU restatement"),
                "candidate_distances_bit_equal": bool(np.array_equal(cds.view(np.uint32), gcd.view(np.uint32))),
                "candidate_distances_max_abs_difference": float(np.abs(cds.astype(np.float64) - gcd).max()),
                "candidate_overlap_with_gpu": float(np.mean([len(set(a) & set(bb)) / float(kcand)
@@ -833,13 +848,16 @@ def run_c5(env):
         # queries against the same codes, then fp64 rerank of its 200 candidates.
         import oracle as orc
         threads = min(os.cpu_count() or 1, 16)
-        sample = min(nq, 2 * threads)
+        sample = min(nq, 8 * threads)
         hcodes = codes.to_numpy(np.uint8, (n, cs))
         hcen = cen.to_numpy(np.float32, (d,))
         qcodes = orc.rabitq_process_query(q[:sample], rot, hcen, orc.IP, 4)
+        ref = orc.use_reference_kernels(orc.ref_best_isa())
+        ref = ref if ref and "RaBitQSQ4UBinaryIP" in ref else None
         t0 = time.perf_counter()
         cids, cds = orc.flat_scan_topk(orc.RABITQ, orc.IP, d, hcodes, qcodes, kcand, qbits=4, threads=threads)
         t_cpu = time.perf_counter() - t0
+        orc.use_reference_kernels(None)
         gcand = cand.to_numpy(np.uint32, (nq, kcand))[:sample]
         uniq = np.unique(cids)
         raw = device_rows(env, x_dev, uniq, d)
@@ -849,10 +867,12 @@ def run_c5(env):
             rows = raw[[pos[int(v)] for v in cids[i]]]
             dd = 1.0 - rows.astype(np.float64) @ q[i].astype(np.float64)
             rids[i] = cids[i][np.lexsort((cids[i], dd))[:k]]
-        cpu = {"value": sample / t_cpu, "unit": "queries/s", "cores": threads, "kind": "port",
-               "sample": "%d of the %d queries over all %d codes, CPU restatement of RaBitQuantizer::ProcessQueryImpl + "
-                         "ComputeQueryBaseImpl + BruteForce heap, OpenMP over queries; rerank in fp64 on the host" %
-                         (sample, nq, n),
+        cpu = {"value": sample / t_cpu, "unit": "queries/s", "cores": threads, "kind": "reference" if ref else "port",
+               "sample": "%d of the %d queries over all %d codes, one query per call, OpenMP dynamic over queries; restated "
+                         "RaBitQuantizer::ComputeQueryBaseImpl + BruteForce heap, popcount kernel = %s; rerank in fp64 on "
+                         "the host (not timed)" %
+                         (sample, nq, n, (ref["RaBitQSQ4UBinaryIP"] + " compiled from the reference sources") if ref
+                          else "CPU restatement"),
                "candidate_overlap_with_gpu": float(np.mean([len(set(a) & set(bb)) / float(kcand)
                                                             for a, bb in zip(cids, gcand)])),
                "topk_overlap_with_gpu": float(np.mean([len(set(a) & set(bb)) / float(k)

@@ -363,6 +363,19 @@ recover_sq4u(uint32_t ip, float base_sum, float query_sum, float lb, float delta
     return p1 + p2 - p3 - p4;
 }
 
+// ---------------------------------------------------------------- the reference's compiled kernels (timing only)
+// When oracle/_ref is built, a benchmark's CPU leg can put the reference's own SIMD kernels (vsag::<isa>::*) under
+// the loops restated below, through orc_set_reference_kernels.  All null by default: parity checks always run the
+// scalar restatements above.
+struct RefKernels {
+    float (*fp32_l2)(const float*, const float*, uint64_t) = nullptr;
+    float (*fp32_ip)(const float*, const float*, uint64_t) = nullptr;
+    float (*sq4u_ip)(const uint8_t*, const uint8_t*, uint64_t) = nullptr;
+    float (*sq8u_ip)(const uint8_t*, const uint8_t*, uint64_t) = nullptr;
+    uint32_t (*rabitq_sq4u_ip)(const uint8_t*, const uint8_t*, uint64_t) = nullptr;
+};
+RefKernels g_ref;
+
 // ---------------------------------------------------------------- bounded heaps
 using Rec = std::pair<float, uint32_t>;
 struct CmpMax {
@@ -471,7 +484,12 @@ uniform_dist(const Store& s, const uint8_t* qcode, const uint8_t* code) {
     float diff = *s.diff;
     float lb = *s.lb;
     float scalar_rate = static_cast<float>((diff / static_cast<double>(levels)) * (diff / static_cast<double>(levels)));
-    float result = static_cast<float>(bits == 4 ? sq4u_codes_ip(qcode, code, s.dim) : sq8u_codes_ip(qcode, code, s.dim));
+    float result;
+    if (bits == 4) {
+        result = g_ref.sq4u_ip ? g_ref.sq4u_ip(qcode, code, s.dim) : static_cast<float>(sq4u_codes_ip(qcode, code, s.dim));
+    } else {
+        result = g_ref.sq8u_ip ? g_ref.sq8u_ip(qcode, code, s.dim) : static_cast<float>(sq8u_codes_ip(qcode, code, s.dim));
+    }
     if (s.metric == kL2) {
         uint64_t n1, n2;
         std::memcpy(&n1, qcode + l.offset_norm, 8);
@@ -492,7 +510,8 @@ rabitq_dist(const RabitqLayout& l, int metric, int query_bits, const uint8_t* qc
     if (query_bits == 4) {
         std::vector<uint8_t> tmp(l.aligned_dim / 8, 0);
         std::memcpy(tmp.data(), code, l.offset_norm);
-        uint32_t ip = rabitq_sq4u_binary_ip(qcode, tmp.data(), l.aligned_dim);
+        uint32_t ip = g_ref.rabitq_sq4u_ip ? g_ref.rabitq_sq4u_ip(qcode, tmp.data(), l.aligned_dim)
+                                           : rabitq_sq4u_binary_ip(qcode, tmp.data(), l.aligned_dim);
         float base_sum = rd_f32(code + l.offset_sum);
         float query_sum = rd_f32(qcode + l.q_offset_sum);
         float lb = rd_f32(qcode + l.q_offset_lb);
@@ -539,7 +558,10 @@ store_dist(const Store& s, const RabitqLayout* rl, const uint8_t* q, const uint8
     switch (s.kind) {
         case kFP32: {
             const float* x = reinterpret_cast<const float*>(code);
-            return s.metric == kL2 ? fp32_l2sqr(qf, x, s.dim) : 1 - fp32_ip(qf, x, s.dim);
+            if (s.metric == kL2) {
+                return g_ref.fp32_l2 ? g_ref.fp32_l2(qf, x, s.dim) : fp32_l2sqr(qf, x, s.dim);
+            }
+            return 1 - (g_ref.fp32_ip ? g_ref.fp32_ip(qf, x, s.dim) : fp32_ip(qf, x, s.dim));
         }
         case kSQ8:
             return s.metric == kL2 ? sq8_l2sqr(qf, code, s.lb, s.diff, s.dim)
@@ -559,6 +581,18 @@ store_dist(const Store& s, const RabitqLayout* rl, const uint8_t* q, const uint8
 }  // namespace
 
 // ================================================================= exported C entry points
+
+// Puts compiled kernels of the reference (addresses of vsag::<isa>::FP32ComputeL2Sqr, FP32ComputeIP,
+// SQ4UniformComputeCodesIP, SQ8UniformComputeCodesIP, RaBitQSQ4UBinaryIP; null = keep the restatement) under the
+// scan loops of this file.  For timing the CPU baseline only; call with all nulls to go back.
+ORC_API void
+orc_set_reference_kernels(void* fp32_l2, void* fp32_ip, void* sq4u_ip, void* sq8u_ip, void* rabitq_sq4u_ip) {
+    g_ref.fp32_l2 = reinterpret_cast<decltype(g_ref.fp32_l2)>(fp32_l2);
+    g_ref.fp32_ip = reinterpret_cast<decltype(g_ref.fp32_ip)>(fp32_ip);
+    g_ref.sq4u_ip = reinterpret_cast<decltype(g_ref.sq4u_ip)>(sq4u_ip);
+    g_ref.sq8u_ip = reinterpret_cast<decltype(g_ref.sq8u_ip)>(sq8u_ip);
+    g_ref.rabitq_sq4u_ip = reinterpret_cast<decltype(g_ref.rabitq_sq4u_ip)>(rabitq_sq4u_ip);
+}
 
 // Threads of the OpenMP loops below (0 = leave as is); the loops that take a `threads` argument set it themselves.
 ORC_API void
@@ -1475,6 +1509,10 @@ orc_cpu_has_avx512() {
            __builtin_cpu_supports("avx512dq") && __builtin_cpu_supports("avx512vl") &&
            __builtin_cpu_supports("avx512cd") && __builtin_cpu_supports("avx512ifma") &&
            __builtin_cpu_supports("avx512vbmi");
+}
+ORC_API int
+orc_cpu_has_avx512vpopcntdq() {
+    return __builtin_cpu_supports("avx512vpopcntdq");
 }
 ORC_API int
 orc_cpu_has_avx2() {

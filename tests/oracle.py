@@ -392,6 +392,36 @@ def ref_sq8_fn(metric, isa):
     return C.cast(getattr(dll, sym), C.c_void_p)
 
 
+def use_reference_kernels(isa):
+    """Puts the reference's compiled kernels of tier `isa` (oracle/_ref) under the checker's scan loops, for timing
+    a CPU baseline; None restores the scalar restatements.  Returns the names that were found, or None when
+    oracle/_ref is not built."""
+    if isa is None or not os.path.exists(REF_SIMD):
+        lib().orc_set_reference_kernels(None, None, None, None, None)
+        return None
+    dll = C.CDLL(REF_SIMD)
+    found = {}
+
+    def sym(name, args, tiers):
+        for t in tiers:
+            s = "_ZN4vsag%d%s%d%sE%s" % (len(t), t, len(name), name, args)
+            try:
+                found[name] = "vsag::%s::%s" % (t, name)
+                return C.cast(getattr(dll, s), C.c_void_p)
+            except AttributeError:
+                found.pop(name, None)
+        return None
+
+    tiers = {"avx512": ["avx512", "avx2", "avx", "sse", "generic"], "avx2": ["avx2", "avx", "sse", "generic"],
+             "generic": ["generic"]}[isa]
+    pop = (["avx512vpopcntdq"] if isa == "avx512" and lib().orc_cpu_has_avx512vpopcntdq() else []) + tiers
+    lib().orc_set_reference_kernels(sym("FP32ComputeL2Sqr", "PKfS2_m", tiers), sym("FP32ComputeIP", "PKfS2_m", tiers),
+                                    sym("SQ4UniformComputeCodesIP", "PKhS2_m", tiers),
+                                    sym("SQ8UniformComputeCodesIP", "PKhS2_m", tiers),
+                                    sym("RaBitQSQ4UBinaryIP", "PKhS2_m", pop))
+    return found
+
+
 def flat_scan_topk_fn(fn, metric, d, codes, queries, k, lb, diff, threads=0):
     codes = np.ascontiguousarray(codes)
     queries = f32(queries)

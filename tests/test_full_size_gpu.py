@@ -34,10 +34,26 @@ def check_result_shape(ids, dists, n):
 
 
 def scan_with_tile(lib, store, queries, k, tile):
-    capi.check(lib.vsag_amd_set_scan_tuning(tile, 0))
-    out = store.flat_scan(queries, k)
-    capi.check(lib.vsag_amd_set_scan_tuning(0, 0))
-    return out
+    """A flat scan with the store's own query-tile setting (process-wide settings stay untouched)."""
+    capi.check(lib.vsag_amd_store_set_scan_tuning(store.handle, tile, -1))
+    try:
+        return store.flat_scan(queries, k)
+    finally:
+        capi.check(lib.vsag_amd_store_set_scan_tuning(store.handle, -1, -1))
+
+
+def streaming_only(lib, store):
+    """Context manager: the store's scans stay on the streaming kernels (its own setting, not the process-wide one)."""
+    import contextlib
+
+    @contextlib.contextmanager
+    def cm():
+        capi.check(lib.vsag_amd_store_set_scan_contraction(store.handle, -1))
+        try:
+            yield
+        finally:
+            capi.check(lib.vsag_amd_store_set_scan_contraction(store.handle, -2))
+    return cm()
 
 
 def test_fp32_bruteforce_100k(lib):
@@ -65,8 +81,9 @@ def test_fp32_bruteforce_100k(lib):
 
 @pytest.mark.parametrize("metric,ometric", [(capi.METRIC_L2, orc.L2), (capi.METRIC_IP, orc.IP)])
 def test_sq8_scan_1m(lib, metric, ometric):
-    """configs[1]: 1 000 000 x 128 mixture rows as SQ8 codes; trained and encoded on the device."""
-    n, d, nq, k = 1000000, 128, 512, 10
+    """configs[1] at the benchmark's own batch: 1 000 000 x 128 mixture rows as SQ8 codes (trained and encoded on the
+    device), all 10 000 queries in one call."""
+    n, d, nq, k = 1000000, 128, 10000, 10
     x, means = mixture(315, 47, n, d, 1000, 0.05)
     q, _ = mixture(315, 165, nq, d, 1000, 0.05, means=means)
     x_dev = dev(x)
@@ -93,16 +110,19 @@ def test_sq8_scan_1m(lib, metric, ometric):
     check_result_shape(ids, dists, n)
     oi, od = orc.flat_scan_topk(orc.SQ8, ometric, d, codes, q[:32], k, lb=lb, diff=diff)
     assert_topk_close(ids[:32], dists[:32], oi, od, label="sq8 1M")
-    # 512 queries go through the int8 matrix-core pre-selection; the streaming kernel alone must return the same bits
+    # the batch goes through the int8 matrix-core pre-selection (40 query groups, the XCD-grouped grid of the
+    # benchmark); the streaming kernel alone must return the same bits for every one of the 10 000 queries
     info = capi.C.c_int()
     lib.vsag_amd_last_scan_info(capi.C.byref(info), None, None)
     assert info.value == 256, "the int8 pre-selection did not run"
-    capi.check(lib.vsag_amd_set_scan_contraction(-1))
-    try:
+    with streaming_only(lib, store):
         si, sd = store.flat_scan(q, k)
-    finally:
-        capi.check(lib.vsag_amd_set_scan_contraction(0))
+        lib.vsag_amd_last_scan_info(capi.C.byref(info), None, None)
+        assert info.value <= 8
     assert np.array_equal(si, ids) and np.array_equal(sd.view(np.uint32), dists.view(np.uint32))
+    # a smaller batch takes another grid (2 query groups): same bits again
+    pi, pd = store.flat_scan(q[:512], k)
+    assert np.array_equal(pi, ids[:512]) and np.array_equal(pd.view(np.uint32), dists[:512].view(np.uint32))
     # the same answer whatever the query tile, and one query per call (a different grid and cold start)
     for tile in (1, 2):
         ti, td = scan_with_tile(lib, store, q[:256], k, tile)
@@ -194,8 +214,9 @@ def test_kmeans_lloyd_10_iterations_on_a_64k_slice(lib):
 
 
 def test_ivf_sq4_uniform_10m(lib):
-    """configs[3]: 10 000 000 x 128 rows, 4096 lists of SQ4-uniform codes, 64 probes, rerank of 100."""
-    n, d, nq, k, nlist, nprobe, kcand = 10000000, 128, 1024, 10, 4096, 64, 100
+    """configs[3] at the benchmark's own batch: 10 000 000 x 128 rows, 4096 lists of SQ4-uniform codes, 64 probes,
+    rerank of 100, all 10 000 queries in one call (640 000 (query, list) pairs)."""
+    n, d, nq, k, nlist, nprobe, kcand = 10000000, 128, 10000, 10, 4096, 64, 100
     means = mt(315).random((10000, d), dtype=np.float32)
     x_dev = capi.DeviceBuffer(n * d * 4)
     pick = np.sort(mt(7).choice(n, nlist, replace=False))
@@ -260,13 +281,10 @@ def test_ivf_sq4_uniform_10m(lib):
     info = capi.C.c_int()
     lib.vsag_amd_last_scan_info(capi.C.byref(info), None, None)
     assert info.value == 256, "the int8 pass over the posting lists did not run"
-    capi.check(lib.vsag_amd_set_scan_contraction(-1))
-    try:
+    with streaming_only(lib, lists):
         si, sd = lists.ivf_scan(q, b, kcand)
         lib.vsag_amd_last_scan_info(capi.C.byref(info), None, None)
         assert info.value <= 8
-    finally:
-        capi.check(lib.vsag_amd_set_scan_contraction(0))
     assert np.array_equal(si, cand) and np.array_equal(sd.view(np.uint32), cand_d.view(np.uint32))
     # the checker on the same codes, lists and probes: integer distances, so bit-equal; ids up to equal distances
     offsets, order = orc.ivf_build_lists(hlabels, nlist)
@@ -276,7 +294,7 @@ def test_ivf_sq4_uniform_10m(lib):
     assert np.array_equal(od.view(np.uint32), cand_d[:64].view(np.uint32))
     assert_topk_close(cand[:64], cand_d[:64], oi, od, rtol=0, atol=0, tie_rtol=0, label="ivf sq4u 10M")
     # the batch split does not matter: the same queries alone and in groups of 7
-    for s, e in ((0, 1), (5, 6), (10, 17), (100, 107), (1000, 1024)):
+    for s, e in ((0, 1), (5, 6), (10, 17), (100, 107), (1000, 2024), (9990, 10000)):
         ci, cd = lists.ivf_scan(q[s:e], b[s:e], kcand)
         assert np.array_equal(ci, cand[s:e]) and np.array_equal(cd.view(np.uint32), cand_d[s:e].view(np.uint32)), (s, e)
 
@@ -288,7 +306,7 @@ def test_ivf_sq4_uniform_10m(lib):
     ri, rd = out_i.to_numpy(np.uint32, (nq, k)), out_d.to_numpy(np.float32, (nq, k))
     check_result_shape(ri, rd, n)
     row = np.empty(d, np.float32)
-    for i in range(0, nq, 32):
+    for i in range(0, nq, 250):
         dd = np.empty(kcand)
         for j, c in enumerate(cand[i]):
             capi.check(lib.vsag_amd_memcpy_d2h(row.ctypes.data, x_dev.ptr + int(c) * d * 4, d * 4, None))
@@ -306,7 +324,7 @@ def test_ivf_sq8_and_rabitq_lists_10m(lib):
     """configs[3]'s rows, lists and probes with sq8 and with RaBitQ codes in the lists: the probe columns behind the
     first go through the int8 matrix cores (two planes per query / expanded code bits), and what they return must be
     the streaming kernel's result bit for bit, the checker's on a sample, and independent of the batch split."""
-    n, d, nq, nlist, nprobe, kcand = 10000000, 128, 1024, 4096, 64, 100
+    n, d, nq, nlist, nprobe, kcand = 10000000, 128, 10000, 4096, 64, 100
     means = mt(315).random((10000, d), dtype=np.float32)
     x_dev = capi.DeviceBuffer(n * d * 4)
     pick = np.sort(mt(7).choice(n, nlist, replace=False))
@@ -343,7 +361,7 @@ def test_ivf_sq8_and_rabitq_lists_10m(lib):
         plain = lists.ivf_scan(q, b, kcand)
         capi.check(lib.vsag_amd_store_set_scan_contraction(lists.handle, -2))
         assert np.array_equal(plain[0], fast[0]) and np.array_equal(plain[1].view(np.uint32), fast[1].view(np.uint32))
-        for s, e in ((0, 1), (10, 17), (1000, 1024)):
+        for s, e in ((0, 1), (10, 17), (1000, 2024), (9990, 10000)):
             ci, cd = lists.ivf_scan(q[s:e], b[s:e], kcand)
             assert np.array_equal(ci, fast[0][s:e]) and np.array_equal(cd.view(np.uint32), fast[1][s:e].view(np.uint32))
         return fast
@@ -394,8 +412,9 @@ def test_ivf_sq8_and_rabitq_lists_10m(lib):
 
 
 def test_rabitq_scan_5m_x_768(lib):
-    """configs[4]: 5 000 000 x 768 unit rows, 1-bit codes, 4-bit queries, inner product, 200 candidates."""
-    n, d, nq, kcand = 5000000, 768, 512, 200
+    """configs[4] at the benchmark's own batch: 5 000 000 x 768 unit rows, 1-bit codes, 4-bit queries, inner product,
+    200 candidates, all 10 000 queries in one call."""
+    n, d, nq, kcand = 5000000, 768, 10000, 200
     rng = mt(47)
     x_dev = capi.DeviceBuffer(n * d * 4)
     head = None
@@ -429,24 +448,27 @@ def test_rabitq_scan_5m_x_768(lib):
     codes.free()
     ids, dists = store.flat_scan(q, kcand)
     check_result_shape(ids, dists, n)
-    # 512 queries take the matrix-core route (prefilter_rb_kernel: code bits x 4-bit queries on the int8 matrix cores,
-    # exact rescoring); the checker and the streaming kernel alone must agree with it
+    # the batch takes the matrix-core route (prefilter_rb_kernel: code bits x 4-bit queries on the int8 matrix cores,
+    # exact rescoring); the checker on a sample and the streaming kernel alone on 1000 queries spread over the batch
+    # must agree with it, and so must a smaller batch (another grid)
     info = capi.C.c_int()
     lib.vsag_amd_last_scan_info(capi.C.byref(info), None, None)
     assert info.value == 128, "the matrix-core pre-selection did not run"
     qcodes = orc.rabitq_process_query(q[:16], rot, hcen, orc.IP, 4)
     oi, od = orc.flat_scan_topk(orc.RABITQ, orc.IP, d, hcodes, qcodes, kcand, qbits=4)
     assert_topk_close(ids[:16], dists[:16], oi, od, label="rabitq 5M")
-    capi.check(lib.vsag_amd_set_scan_contraction(-1))
-    try:
-        si, sd = store.flat_scan(q[:128], kcand)
+    sel = np.arange(0, nq, 10)
+    with streaming_only(lib, store):
+        si, sd = store.flat_scan(q[sel], kcand)
         lib.vsag_amd_last_scan_info(capi.C.byref(info), None, None)
         assert info.value <= 8
         ti, td = scan_with_tile(lib, store, q[:32], kcand, 1)
-    finally:
-        capi.check(lib.vsag_amd_set_scan_contraction(0))
-    assert np.array_equal(si, ids[:128]) and np.array_equal(sd.view(np.uint32), dists[:128].view(np.uint32))
+    assert np.array_equal(si, ids[sel]) and np.array_equal(sd.view(np.uint32), dists[sel].view(np.uint32))
     assert np.array_equal(ti, ids[:32]) and np.array_equal(td.view(np.uint32), dists[:32].view(np.uint32))
+    pi, pd = store.flat_scan(q[:512], kcand)
+    lib.vsag_amd_last_scan_info(capi.C.byref(info), None, None)
+    assert info.value == 128
+    assert np.array_equal(pi, ids[:512]) and np.array_equal(pd.view(np.uint32), dists[:512].view(np.uint32))
     for b in (rot_dev, cen):
         b.free()
     store.destroy()
