@@ -47,6 +47,7 @@ extern "C" {
 #define VSAG_AMD_KIND_SQ4_UNIFORM 3
 #define VSAG_AMD_KIND_SQ8_UNIFORM 4
 #define VSAG_AMD_KIND_RABITQ 5
+#define VSAG_AMD_KIND_PQFS 6
 
 /* SQTrainMode of src/quantization/scalar_quantization/scalar_quantization_trainer.h:24-28. */
 #define VSAG_AMD_SQ_TRAIN_CLASSIC 1
@@ -105,7 +106,8 @@ VSAG_AMD_API int vsag_amd_sq_train_uniform(const float* x_dev, uint64_t n, uint3
 
 /* Bytes per code in the reference's layout (Quantizer::GetCodeSize): fp32 4*dim; sq8 dim; sq4
  * ceil(dim/2) (scalar_quantizer.cpp:28-36); uniform kinds sq4_uniform_quantizer.cpp:33-72 and
- * sq8_uniform_quantizer.cpp:30-62; rabitq 1-bit base rabitq_quantizer.cpp:102-133. */
+ * sq8_uniform_quantizer.cpp:30-62; rabitq 1-bit base rabitq_quantizer.cpp:102-133.  (pqfs: ceil(pq_dim / 2),
+ * pq_fastscan_quantizer.cpp:38 -- it depends on pq_dim, not on dim: call it with dim = pq_dim.) */
 VSAG_AMD_API uint64_t vsag_amd_code_size(int kind, int metric, uint32_t dim, int rabitq_query_bits);
 
 /* ScalarQuantizer::EncodeBatch (scalar_quantizer.cpp:85-112): fp32 rows -> sq8 / sq4 codes in the
@@ -137,6 +139,30 @@ VSAG_AMD_API int vsag_amd_rabitq_process_query(const float* q_dev, uint64_t nq, 
                                   const float* rotation_dev, const float* centroid_dev, int metric,
                                   int query_bits, uint8_t* qcodes_dev, void* stream);
 
+/* PQFastScanQuantizer (src/quantization/product_quantization/pq_fastscan_quantizer.cpp): pq_dim subspaces of
+ * dim / pq_dim dimensions, 16 centroids each; codebooks_dev is pq_dim x 16 x (dim / pq_dim) floats.
+ * vsag_amd_pq_train = TrainImpl (:62-94): 16 centroids per subspace from the first min(n, 65536) rows by k-means++ and
+ * 25 Lloyd iterations (the reference's draws come from std::random_device; here subspace i draws from
+ * mt19937(seed + i)); blocking.  vsag_amd_pq_encode = EncodeBatchImpl (:97-138): n x ceil(pq_dim / 2) code bytes,
+ * subspace i in byte i / 2, low nibble for even i (norm_scratch_dev: n floats under cosine, else NULL).
+ * vsag_amd_pq_decode = DecodeBatchImpl (:140-156).  vsag_amd_pqfs_process_query = ProcessQueryImpl (:299-361):
+ * nq x (pq_dim * 16 + 8) bytes, the byte table of a query, then diff and lower bound as floats.
+ * vsag_amd_pqfs_package / _unpack = Package32 / Unpack32 (:241-297) over ceil(n / 32) blocks of 32 codes, the order in
+ * which BucketDataCell keeps and serializes pqfs codes (bucket_datacell.h:943-992). */
+VSAG_AMD_API size_t vsag_amd_pq_train_workspace_bytes(uint64_t n, uint32_t dim, uint32_t pq_dim);
+VSAG_AMD_API int vsag_amd_pq_train(const float* x_dev, uint64_t n, uint32_t dim, uint32_t pq_dim, int metric, uint64_t seed,
+                      float* codebooks_dev, void* workspace_dev, size_t workspace_bytes, void* stream);
+VSAG_AMD_API int vsag_amd_pq_encode(const float* x_dev, uint64_t n, uint32_t dim, uint32_t pq_dim, const float* codebooks_dev,
+                       int metric, uint8_t* codes_dev, float* norm_scratch_dev, void* stream);
+VSAG_AMD_API int vsag_amd_pq_decode(const uint8_t* codes_dev, uint64_t n, uint32_t dim, uint32_t pq_dim,
+                       const float* codebooks_dev, float* out_dev, void* stream);
+VSAG_AMD_API int vsag_amd_pqfs_process_query(const float* q_dev, uint64_t nq, uint32_t dim, uint32_t pq_dim,
+                                const float* codebooks_dev, int metric, uint8_t* qcodes_dev, void* stream);
+VSAG_AMD_API int vsag_amd_pqfs_package(const uint8_t* codes_dev, uint64_t n, uint32_t pq_dim, uint8_t* packaged_dev,
+                          void* stream);
+VSAG_AMD_API int vsag_amd_pqfs_unpack(const uint8_t* packaged_dev, uint64_t n, uint32_t pq_dim, uint8_t* codes_dev,
+                         void* stream);
+
 /* ------------------------------------------------------------------ code stores -------------- */
 
 /* A store is the device-resident replacement of one FlattenDataCell / BucketDataCell
@@ -154,6 +180,8 @@ typedef struct vsag_amd_store_params {
     const float* rotation_dev;    /* rabitq: dim x dim row-major.  otherwise NULL. */
     const float* centroid_dev;    /* rabitq: dim floats (already rotated). */
     int rabitq_query_bits;        /* rabitq: 4 or 32 (only 4 is scanned on the device). */
+    uint32_t pq_dim;              /* pqfs: number of subspaces (divides dim, at most 1024). */
+    const float* codebooks_dev;   /* pqfs: pq_dim x 16 x (dim / pq_dim) floats. */
 } vsag_amd_store_params_t;
 
 VSAG_AMD_API int vsag_amd_store_create(const vsag_amd_store_params_t* params, vsag_amd_store_t** store);

@@ -363,6 +363,155 @@ recover_sq4u(uint32_t ip, float base_sum, float query_sum, float lb, float delta
     return p1 + p2 - p3 - p4;
 }
 
+// ---------------------------------------------------------------- product quantization, fast-scan form (pqfs)
+// pq_fastscan_quantizer.cpp: pq_dim subspaces of dim / pq_dim dimensions, 16 centroids each
+// (codebooks[subspace][centroid][subspace_dim], :117-122 of the header); a code is one 4-bit centroid index per
+// subspace, subspace i in byte i / 2, low nibble for even i (:97-127).
+constexpr uint64_t kPqCentroids = 16;
+
+inline uint8_t
+pq_nibble(const uint8_t* code, uint64_t i) {
+    return (i & 1) ? static_cast<uint8_t>(code[i >> 1] >> 4) : static_cast<uint8_t>(code[i >> 1] & 0x0F);
+}
+
+// EncodeOneImpl (pq_fastscan_quantizer.cpp:97-127): per subspace the first centroid of smallest FP32ComputeL2Sqr
+// (strict <, starting from FLT_MAX); cosine normalises the row first.
+inline void
+pq_encode_one(const float* x, uint64_t dim, uint64_t pq_dim, const float* codebooks, int metric, uint8_t* code) {
+    const uint64_t sd = dim / pq_dim;
+    std::vector<float> tmp;
+    const float* cur = x;
+    if (metric == kCosine) {
+        tmp.resize(dim);
+        normalize(x, tmp.data(), dim);
+        cur = tmp.data();
+    }
+    std::memset(code, 0, (pq_dim + 1) / 2);
+    for (uint64_t i = 0; i < pq_dim; ++i) {
+        float nearest = std::numeric_limits<float>::max();
+        uint8_t id = 0;
+        const float* base = codebooks + i * sd * kPqCentroids;
+        for (uint64_t j = 0; j < kPqCentroids; ++j) {
+            float dist = fp32_l2sqr(cur + i * sd, base + j * sd, sd);
+            if (dist < nearest) {
+                nearest = dist;
+                id = static_cast<uint8_t>(j);
+            }
+        }
+        code[i / 2] |= (i & 1) ? static_cast<uint8_t>(id << 4) : id;
+    }
+}
+
+// ProcessQueryImpl (pq_fastscan_quantizer.cpp:299-361): the float table lut[i][j] = FP32ComputeL2Sqr(sub-query i,
+// centroid j) (l2) or their inner product (ip, cosine: the reference takes it from cblas_sgemv, whose order of
+// summation is the library's; here in element order), quantised to bytes between its own smallest and largest
+// entry (ScalarQuantizationTrainer::TrainUniform, CLASSIC: scalar_quantization_trainer.cpp:47-61,72-86):
+// byte = uint8((v - lower) / diff * 255).  Output: pq_dim * 16 bytes, then diff and lower as floats.
+inline void
+pqfs_process_query(const float* q, uint64_t dim, uint64_t pq_dim, const float* codebooks, int metric, uint8_t* out) {
+    const uint64_t sd = dim / pq_dim;
+    std::vector<float> tmp;
+    const float* cur = q;
+    if (metric == kCosine) {
+        tmp.resize(dim);
+        normalize(q, tmp.data(), dim);
+        cur = tmp.data();
+    }
+    std::vector<float> lut(pq_dim * kPqCentroids);
+    for (uint64_t i = 0; i < pq_dim; ++i) {
+        for (uint64_t j = 0; j < kPqCentroids; ++j) {
+            const float* c = codebooks + (i * kPqCentroids + j) * sd;
+            lut[i * kPqCentroids + j] = metric == kL2 ? fp32_l2sqr(cur + i * sd, c, sd) : fp32_ip(c, cur + i * sd, sd);
+        }
+    }
+    float upper = std::numeric_limits<float>::lowest();
+    float lower = std::numeric_limits<float>::max();
+    for (float v : lut) {
+        upper = std::max(upper, v);
+        lower = std::min(lower, v);
+    }
+    const float diff = upper - lower;
+    for (uint64_t j = 0; j < pq_dim * kPqCentroids; ++j) {
+        // a float converted to uint8_t as the reference's assignment does; 0 / 0 (every entry equal) gives 0 here
+        const float v = (lut[j] - lower) / diff * 255;
+        out[j] = v == v ? static_cast<uint8_t>(static_cast<int32_t>(v)) : 0;
+    }
+    wr_f32(out + pq_dim * kPqCentroids, diff);
+    wr_f32(out + pq_dim * kPqCentroids + 4, lower);
+}
+
+// The 32 codes of a block in the fast-scan order (pq_fastscan_quantizer.h:115-118, .cpp:241-266): subspace i takes 16
+// bytes; byte j / 2 holds the code of vector MAPPER[j] in its low (even j) or high (odd j) nibble.
+constexpr int32_t kPqMapper[32] = {0, 16, 8, 24, 1, 17, 9, 25, 2, 18, 10, 26, 3, 19, 11, 27,
+                                   4, 20, 12, 28, 5, 21, 13, 29, 6, 22, 14, 30, 7, 23, 15, 31};
+
+inline void
+pqfs_package32(const uint8_t* codes, uint64_t pq_dim, int64_t valid, uint8_t* packaged) {
+    const uint64_t cs = (pq_dim + 1) / 2;
+    if (valid < 0) {
+        valid = 32;
+    }
+    std::memset(packaged, 0, cs * 32);
+    for (uint64_t i = 0; i < pq_dim; ++i) {
+        for (int j = 0; j < 32; ++j) {
+            const int v = kPqMapper[j];
+            uint8_t code = v >= valid ? 0 : pq_nibble(codes + v * cs, i);
+            packaged[i * 16 + j / 2] |= (j & 1) ? static_cast<uint8_t>(code << 4) : code;
+        }
+    }
+}
+
+inline void
+pqfs_unpack32(const uint8_t* packaged, uint64_t pq_dim, uint8_t* codes) {
+    const uint64_t cs = (pq_dim + 1) / 2;
+    for (uint64_t i = 0; i < pq_dim; ++i) {
+        for (int j = 0; j < 32; ++j) {
+            const uint8_t byte = packaged[i * 16 + j / 2];
+            const uint8_t code = (j & 1) ? static_cast<uint8_t>(byte >> 4) : static_cast<uint8_t>(byte & 0x0F);
+            uint8_t* dst = codes + kPqMapper[j] * cs + i / 2;
+            *dst = (i & 1) ? static_cast<uint8_t>((*dst & 0x0F) | (code << 4)) : static_cast<uint8_t>((*dst & 0xF0) | code);
+        }
+    }
+}
+
+// generic::PQFastScanLookUp32 (src/simd/generic.cpp:902-921): adds to result[32] the table bytes of the 32 packaged
+// codes, subspace by subspace.
+inline void
+pqfs_lookup32(const uint8_t* lut, const uint8_t* packaged, uint64_t pq_dim, int32_t* result) {
+    for (uint64_t i = 0; i < pq_dim; ++i) {
+        const uint8_t* dict = lut + 16 * i;
+        const uint8_t* code = packaged + 16 * i;
+        for (uint64_t j = 0; j < 16; ++j) {
+            if (j % 2 == 0) {
+                result[j / 2] += dict[code[j] & 0x0F];
+                result[16 + j / 2] += dict[code[j] >> 4];
+            } else {
+                result[8 + j / 2] += dict[code[j] & 0x0F];
+                result[24 + j / 2] += dict[code[j] >> 4];
+            }
+        }
+    }
+}
+
+// ScanBatchDistImpl's map (pq_fastscan_quantizer.cpp:166-199): int32 sum -> float(sum) / 255 * diff + lower, and
+// 1 - that for ip / cosine.
+inline float
+pqfs_map(int32_t sum, float diff, float lower, int metric) {
+    float v = static_cast<float>(sum) / 255.0F * diff + lower;
+    return metric == kL2 ? v : 1.0F - v;
+}
+
+// One processed query against one code in the plain (not packaged) layout: the sum PQFastScanLookUp32 forms for
+// that vector, mapped as above.
+inline float
+pqfs_dist(const uint8_t* q, const uint8_t* code, uint64_t pq_dim, int metric) {
+    int32_t sum = 0;
+    for (uint64_t i = 0; i < pq_dim; ++i) {
+        sum += q[16 * i + pq_nibble(code, i)];
+    }
+    return pqfs_map(sum, rd_f32(q + pq_dim * kPqCentroids), rd_f32(q + pq_dim * kPqCentroids + 4), metric);
+}
+
 // ---------------------------------------------------------------- the reference's compiled kernels (timing only)
 // When oracle/_ref is built, a benchmark's CPU leg can put the reference's own SIMD kernels (vsag::<isa>::*) under
 // the loops restated below, through orc_set_reference_kernels.  All null by default: parity checks always run the
@@ -462,7 +611,7 @@ struct StrictMaxHeap {
 
 // One (query, code) distance of the chosen store kind, as the quantizers' ComputeDistImpl return it:
 // L2 -> squared L2, IP/cosine -> 1 - ip (fp32_quantizer.cpp:164-188, scalar_quantizer.cpp:180-196).
-enum Kind { kFP32 = 0, kSQ8 = 1, kSQ4 = 2, kSQ4U = 3, kSQ8U = 4, kRaBitQ = 5 };
+enum Kind { kFP32 = 0, kSQ8 = 1, kSQ4 = 2, kSQ4U = 3, kSQ8U = 4, kRaBitQ = 5, kPQFS = 6 };
 
 struct Store {
     int kind;
@@ -574,6 +723,8 @@ store_dist(const Store& s, const RabitqLayout* rl, const uint8_t* q, const uint8
             return uniform_dist(s, q, code);
         case kRaBitQ:
             return rabitq_dist(*rl, s.metric, s.query_bits, q, code);
+        case kPQFS:
+            return pqfs_dist(q, code, s.dim, s.metric);  // s.dim: the number of subspaces
     }
     return 0;
 }
@@ -1209,6 +1360,106 @@ ORC_API double
 orc_kmeans_run(const float* x, uint64_t n, uint64_t dim, float* cent, uint64_t k, int iters, uint64_t seed,
                int32_t* labels) {
     return orc_kmeans_run_with(x, n, dim, cent, k, iters, seed, labels, nullptr, nullptr);
+}
+
+// ---- pqfs ------------------------------------------------------------------------------------
+ORC_API void
+orc_pq_encode(const float* x, uint64_t n, uint64_t dim, uint64_t pq_dim, const float* codebooks, int metric,
+              uint8_t* codes) {
+    const uint64_t cs = (pq_dim + 1) / 2;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < static_cast<int64_t>(n); ++i) {
+        pq_encode_one(x + i * dim, dim, pq_dim, codebooks, metric, codes + i * cs);
+    }
+}
+
+// DecodeOneImpl (pq_fastscan_quantizer.cpp:140-156): the centroids the code names, subspace by subspace.
+ORC_API void
+orc_pq_decode(const uint8_t* codes, uint64_t n, uint64_t dim, uint64_t pq_dim, const float* codebooks, float* out) {
+    const uint64_t cs = (pq_dim + 1) / 2, sd = dim / pq_dim;
+    for (uint64_t r = 0; r < n; ++r) {
+        for (uint64_t i = 0; i < pq_dim; ++i) {
+            const float* c = codebooks + (i * kPqCentroids + pq_nibble(codes + r * cs, i)) * sd;
+            std::memcpy(out + r * dim + i * sd, c, sd * sizeof(float));
+        }
+    }
+}
+
+ORC_API void
+orc_pqfs_process_query(const float* q, uint64_t nq, uint64_t dim, uint64_t pq_dim, const float* codebooks, int metric,
+                       uint8_t* out /* nq x (pq_dim * 16 + 8) */) {
+    for (uint64_t i = 0; i < nq; ++i) {
+        pqfs_process_query(q + i * dim, dim, pq_dim, codebooks, metric, out + i * (pq_dim * kPqCentroids + 8));
+    }
+}
+
+ORC_API void
+orc_pqfs_package32(const uint8_t* codes, uint64_t pq_dim, int64_t valid, uint8_t* packaged) {
+    pqfs_package32(codes, pq_dim, valid, packaged);
+}
+
+ORC_API void
+orc_pqfs_unpack32(const uint8_t* packaged, uint64_t pq_dim, uint8_t* codes) {
+    pqfs_unpack32(packaged, pq_dim, codes);
+}
+
+ORC_API void
+orc_pqfs_lookup32(const uint8_t* lut, const uint8_t* packaged, uint64_t pq_dim, int32_t* result) {
+    pqfs_lookup32(lut, packaged, pq_dim, result);
+}
+
+// ScanBatchDistImpl (pq_fastscan_quantizer.cpp:166-199) over `count` codes packaged in blocks of 32 (the last
+// block padded): dists[count].
+ORC_API void
+orc_pqfs_scan_batch(const uint8_t* q, const uint8_t* packaged, uint64_t count, uint64_t pq_dim, int metric,
+                    float* dists) {
+    const uint64_t cs = (pq_dim + 1) / 2;
+    const float diff = rd_f32(q + pq_dim * kPqCentroids), lower = rd_f32(q + pq_dim * kPqCentroids + 4);
+    for (uint64_t b = 0; b * 32 < count; ++b) {
+        int32_t tmp[32] = {0};
+        pqfs_lookup32(q, packaged + b * 32 * cs, pq_dim, tmp);
+        for (uint64_t j = 0; j < 32 && b * 32 + j < count; ++j) {
+            dists[b * 32 + j] = pqfs_map(tmp[j], diff, lower, metric);
+        }
+    }
+}
+
+// PQFastScanQuantizer::TrainImpl (pq_fastscan_quantizer.cpp:62-94): the first min(n, 65536) rows (normalised for
+// cosine), sliced per subspace, 16 centroids by KMeansCluster::Run (k-means++ seeding, 25 Lloyd iterations).  The
+// reference draws from std::random_device; here subspace i seeds mt19937(seed + i): `first` and the k-means++ draws
+// come from it in that order, and the Lloyd run re-seeds empty clusters from mt19937(seed + i) as orc_kmeans_run does.
+ORC_API void
+orc_pq_train(const float* x, uint64_t n, uint64_t dim, uint64_t pq_dim, int metric, uint64_t seed, float* codebooks) {
+    const uint64_t count = std::min<uint64_t>(n, 65536), sd = dim / pq_dim;
+    std::vector<float> norm;
+    const float* data = x;
+    if (metric == kCosine) {
+        norm.resize(count * dim);
+        for (uint64_t i = 0; i < count; ++i) {
+            normalize(x + i * dim, norm.data() + i * dim, dim);
+        }
+        data = norm.data();
+    }
+    std::vector<float> slice(count * sd);
+    std::vector<int32_t> labels(count);
+    for (uint64_t i = 0; i < pq_dim; ++i) {
+        for (uint64_t j = 0; j < count; ++j) {
+            std::memcpy(slice.data() + j * sd, data + j * dim + i * sd, sd * sizeof(float));
+        }
+        std::mt19937 gen(static_cast<uint32_t>(seed + i));
+        std::uniform_int_distribution<uint64_t> first_dis(0, count - 1);
+        const uint64_t first = first_dis(gen);
+        std::uniform_real_distribution<double> unit(0.0, 1.0);
+        std::vector<double> draws(kPqCentroids - 1);
+        for (double& d : draws) {
+            d = unit(gen);
+            d = d < 1.0 ? d : 0.0;
+        }
+        float* cb = codebooks + i * kPqCentroids * sd;
+        std::vector<uint64_t> picks(kPqCentroids);
+        orc_kmeans_init_pp(slice.data(), count, sd, kPqCentroids, first, draws.data(), cb, picks.data());
+        orc_kmeans_run(slice.data(), count, sd, cb, kPqCentroids, 25, seed + i, labels.data());
+    }
 }
 
 // ---- flat scan with bounded heap (BruteForce::SearchWithRequest hot loop) ----------------------

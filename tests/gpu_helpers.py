@@ -13,9 +13,10 @@ def dev(arr):
 class Store:
     """A vsag_amd store handle plus the device buffers that must outlive it."""
 
-    def __init__(self, kind, metric, dim, lb=None, diff=None, bounds=None, rot=None, centroid=None, qbits=4):
+    def __init__(self, kind, metric, dim, lb=None, diff=None, bounds=None, rot=None, centroid=None, qbits=4,
+                 pq_dim=0, codebooks=None):
         self.lib = capi.load_library()
-        self.kind, self.metric, self.dim, self.qbits = kind, metric, dim, qbits
+        self.kind, self.metric, self.dim, self.qbits, self.pq_dim = kind, metric, dim, qbits, pq_dim
         self._keep = []
         p = capi.StoreParams()
         p.kind, p.metric, p.dim, p.rabitq_query_bits = kind, metric, dim, qbits
@@ -31,12 +32,17 @@ class Store:
             a, b = dev(np.asarray(rot, np.float32)), dev(np.asarray(centroid, np.float32))
             self._keep += [a, b]
             p.rotation_dev, p.centroid_dev = a.ptr, b.ptr
+        elif kind == capi.KIND_PQFS:
+            a = dev(np.asarray(codebooks, np.float32))
+            self._keep.append(a)
+            p.pq_dim, p.codebooks_dev = pq_dim, a.ptr
         h = C.c_void_p()
         capi.check(self.lib.vsag_amd_store_create(C.byref(p), C.byref(h)))
         self.handle = h
 
     def code_size(self):
-        return int(self.lib.vsag_amd_code_size(self.kind, self.metric, self.dim, self.qbits))
+        dim = self.pq_dim if self.kind == capi.KIND_PQFS else self.dim  # a pqfs code depends on pq_dim alone
+        return int(self.lib.vsag_amd_code_size(self.kind, self.metric, dim, self.qbits))
 
     def append(self, codes):
         codes = np.ascontiguousarray(codes)

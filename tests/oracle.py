@@ -12,7 +12,7 @@ LIB = os.path.join(ORACLE_DIR, "liboracle.so")
 REF_SIMD = os.path.join(ORACLE_DIR, "_ref", "libvsag_simd.so")
 
 L2, IP, COSINE = 0, 1, 2
-FP32, SQ8, SQ4, SQ4U, SQ8U, RABITQ = range(6)
+FP32, SQ8, SQ4, SQ4U, SQ8U, RABITQ, PQFS = range(7)
 KIND_BITS = {SQ8: 8, SQ4: 4, SQ4U: 4, SQ8U: 8}
 
 _f32p = C.POINTER(C.c_float)
@@ -144,6 +144,80 @@ def rabitq_process_query(q, rot, centroid, metric, qbits=4):
         lib().orc_rabitq_process_query(_p(q[i]), u64(d), _p(rot), _p(centroid), metric, qbits,
                                        C.c_void_p(out.ctypes.data + i * qs))
     return out
+
+
+# ---- pqfs (for the scans below a PQFS store's `d` is its number of subspaces, pq_dim) ----
+def pq_train(x, pq_dim, metric=L2, seed=11):
+    x = f32(x)
+    n, d = x.shape
+    cb = np.empty((pq_dim, 16, d // pq_dim), np.float32)
+    lib().orc_pq_train(_p(x), u64(n), u64(d), u64(pq_dim), metric, u64(seed), _p(cb))
+    return cb
+
+
+def pq_encode(x, pq_dim, codebooks, metric=L2):
+    x = f32(x)
+    n, d = x.shape
+    codes = np.zeros((n, (pq_dim + 1) // 2), np.uint8)
+    lib().orc_pq_encode(_p(x), u64(n), u64(d), u64(pq_dim), _p(f32(codebooks)), metric, _p(codes))
+    return codes
+
+
+def pq_decode(codes, d, pq_dim, codebooks):
+    codes = np.ascontiguousarray(codes)
+    out = np.empty((codes.shape[0], d), np.float32)
+    lib().orc_pq_decode(_p(codes), u64(codes.shape[0]), u64(d), u64(pq_dim), _p(f32(codebooks)), _p(out))
+    return out
+
+
+def pqfs_process_query(q, pq_dim, codebooks, metric=L2):
+    """nq x (pq_dim * 16 + 8) bytes: the byte table, then diff and lower as floats."""
+    q = f32(np.atleast_2d(q))
+    nq, d = q.shape
+    out = np.zeros((nq, pq_dim * 16 + 8), np.uint8)
+    lib().orc_pqfs_process_query(_p(q), u64(nq), u64(d), u64(pq_dim), _p(f32(codebooks)), metric, _p(out))
+    return out
+
+
+def pqfs_package32(codes, pq_dim, valid=-1):
+    codes = np.ascontiguousarray(codes)
+    cs = (pq_dim + 1) // 2
+    assert codes.shape == (32, cs)
+    out = np.zeros(32 * cs, np.uint8)
+    lib().orc_pqfs_package32(_p(codes), u64(pq_dim), C.c_int64(valid), _p(out))
+    return out
+
+
+def pqfs_unpack32(packaged, pq_dim):
+    packaged = np.ascontiguousarray(packaged)
+    cs = (pq_dim + 1) // 2
+    out = np.zeros((32, cs), np.uint8)
+    lib().orc_pqfs_unpack32(_p(packaged), u64(pq_dim), _p(out))
+    return out
+
+
+def pqfs_lookup32(lut, packaged, pq_dim):
+    out = np.zeros(32, np.int32)
+    lib().orc_pqfs_lookup32(_p(np.ascontiguousarray(lut)), _p(np.ascontiguousarray(packaged)), u64(pq_dim), _p(out))
+    return out
+
+
+def pqfs_scan_batch(qcode, packaged, count, pq_dim, metric):
+    out = np.empty(count, np.float32)
+    lib().orc_pqfs_scan_batch(_p(np.ascontiguousarray(qcode)), _p(np.ascontiguousarray(packaged)), u64(count),
+                              u64(pq_dim), metric, _p(out))
+    return out
+
+
+def ref_pqfs_lookup32(isa):
+    """vsag::<isa>::PQFastScanLookUp32 of oracle/_ref as a ctypes function, or None."""
+    if not os.path.exists(REF_SIMD):
+        return None
+    name = "PQFastScanLookUp32"
+    try:
+        return getattr(C.CDLL(REF_SIMD), "_ZN4vsag%d%s%d%sEPKhS2_mPi" % (len(isa), isa, len(name), name))
+    except AttributeError:
+        return None
 
 
 def flat_scan_topk(kind, metric, d, codes, queries, k, lb=None, diff=None, qbits=4, strict=False, threads=0):

@@ -617,3 +617,133 @@ def test_residual_scan_closed_forms():
     c4 = orc.squ_encode(res, 4, l, dd, orc.L2)
     raw = np.stack([(c4[:, i // 2] >> (4 * (i % 2))) & 15 for i in range(d)], 1)
     assert np.allclose(orc.squ_decode(c4, d, 4, l, dd, orc.L2), l + raw / 15.0 * dd, atol=1e-6)
+
+
+# ------------------------------------------------------------------ pqfs (PQ fast scan)
+def _pqfs_lookup_cases():
+    """The reference's own shapes (src/simd/pqfs_simd_test.cpp: pq_dim 8, 16, 31, 256), seeded."""
+    rng = np.random.default_rng(903)
+    for pq_dim in (8, 16, 31, 256):
+        lut = rng.integers(0, 256, pq_dim * 16).astype(np.uint8)
+        packaged = rng.integers(0, 256, pq_dim * 16).astype(np.uint8)
+        yield pq_dim, lut, packaged
+
+
+def test_pqfs_lookup32_matches_compiled_reference_and_golden_vectors():
+    gold = json.load(open(os.path.join(GOLDEN, "pqfs_lookup32.json")))
+    for (pq_dim, lut, packaged), want in zip(_pqfs_lookup_cases(), gold["values"]):
+        got = orc.pqfs_lookup32(lut, packaged, pq_dim)
+        assert got.tolist() == want, pq_dim
+        # the function accumulates into its output (the caller zeroes it between blocks)
+        L = orc.lib()
+        twice = got.copy()
+        L.orc_pqfs_lookup32(_p(lut), _p(packaged), C.c_uint64(pq_dim), _p(twice))
+        assert np.array_equal(twice, 2 * got)
+    tiers = ["generic", "sse", "avx"] + (["avx2"] if orc.lib().orc_cpu_has_avx2() else []) + \
+            (["avx512"] if orc.lib().orc_cpu_has_avx512() else [])
+    ran = 0
+    for isa in tiers:
+        fn = orc.ref_pqfs_lookup32(isa)
+        if fn is None:
+            continue
+        ran += 1
+        for pq_dim, lut, packaged in _pqfs_lookup_cases():
+            out = np.zeros(32, np.int32)
+            fn(_p(lut), _p(packaged), C.c_uint64(pq_dim), _p(out))
+            assert np.array_equal(out, orc.pqfs_lookup32(lut, packaged, pq_dim)), (isa, pq_dim)
+    if orc.ref() is not None:
+        assert ran >= 3
+
+
+@pytest.mark.parametrize("pq_dim", [1, 7, 64, 128])
+def test_pqfs_package32_round_trip_and_order(pq_dim):
+    """Package32 / Unpack32 (pq_fastscan_quantizer.cpp:241-297; the reference's own round-trip test) and what the
+    order means: entry v of PQFastScanLookUp32's result on a packaged block is the table sum of vector v."""
+    rng = np.random.default_rng(pq_dim)
+    cs = (pq_dim + 1) // 2
+    codes = rng.integers(0, 256, (32, cs)).astype(np.uint8)
+    if pq_dim % 2:
+        codes[:, -1] &= 0x0F
+    packaged = orc.pqfs_package32(codes, pq_dim)
+    assert np.array_equal(orc.pqfs_unpack32(packaged, pq_dim), codes)
+    lut = rng.integers(0, 256, pq_dim * 16).astype(np.uint8)
+    sums = orc.pqfs_lookup32(lut, packaged, pq_dim)
+    for v in range(32):
+        nib = [int(codes[v, i // 2] >> 4) if i % 2 else int(codes[v, i // 2] & 15) for i in range(pq_dim)]
+        assert sums[v] == sum(int(lut[16 * i + n]) for i, n in enumerate(nib)), v
+    # a partly filled block: the vectors beyond valid_size read as code 0 in every subspace
+    part = orc.pqfs_package32(codes, pq_dim, valid=5)
+    back = orc.pqfs_unpack32(part, pq_dim)
+    assert np.array_equal(back[:5], codes[:5]) and not back[5:].any()
+
+
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
+def test_pqfs_encode_table_and_distance_closed_forms(metric):
+    rng = np.random.default_rng(31 + metric)
+    n, d, pq_dim = 200, 24, 6
+    sd = d // pq_dim
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    cb = rng.standard_normal((pq_dim, 16, sd)).astype(np.float32)
+    xn = x / np.linalg.norm(x, axis=1, keepdims=True) if metric == orc.COSINE else x
+    codes = orc.pq_encode(x, pq_dim, cb, metric)
+    # the nearest centroid per subspace, in float64, ties aside
+    sub = xn.reshape(n, pq_dim, 1, sd).astype(np.float64)
+    dist = ((sub - cb[None].astype(np.float64)) ** 2).sum(-1)  # n x pq_dim x 16
+    nib = np.stack([(codes[:, i // 2] >> 4) if i % 2 else (codes[:, i // 2] & 15) for i in range(pq_dim)], 1)
+    best = dist.min(-1)
+    got = np.take_along_axis(dist, nib[..., None].astype(np.int64), -1)[..., 0]
+    assert np.all(got <= best * (1 + 1e-5) + 1e-6)
+    # decode returns the named centroids; encoding them again names them again
+    dec = orc.pq_decode(codes, d, pq_dim, cb)
+    assert np.array_equal(dec.reshape(n, pq_dim, sd), cb[np.arange(pq_dim)[None], nib])
+    if metric != orc.COSINE:
+        assert np.array_equal(orc.pq_encode(dec, pq_dim, cb, metric), codes)
+    # the query table: bytes = trunc((value - lower) / diff * 255) between the smallest and largest entry
+    q = rng.standard_normal((3, d)).astype(np.float32)
+    qn = q / np.linalg.norm(q, axis=1, keepdims=True) if metric == orc.COSINE else q
+    qc = orc.pqfs_process_query(q, pq_dim, cb, metric)
+    for r in range(3):
+        qs = qn[r].reshape(pq_dim, 1, sd).astype(np.float64)
+        c64 = cb.astype(np.float64)
+        table = ((qs - c64) ** 2).sum(-1) if metric == orc.L2 else (qs * c64).sum(-1)  # pq_dim x 16
+        diff, lower = qc[r, pq_dim * 16:].view(np.float32)
+        assert abs(lower - table.min()) <= 1e-5 * max(1.0, abs(table.min()))
+        assert abs(diff - (table.max() - table.min())) <= 1e-5 * (table.max() - table.min())
+        want = (table - table.min()) / (table.max() - table.min()) * 255.0
+        lut8 = qc[r, :pq_dim * 16].reshape(pq_dim, 16).astype(np.float64)
+        assert np.all(np.abs(lut8 - np.floor(want)) <= 1.0 + 1e-9) and np.mean(lut8 == np.floor(want)) > 0.98
+        assert lut8.min() == 0 and lut8.max() == 255
+        # distance of a code = float(sum of its table bytes) / 255 * diff + lower (1 - that for ip / cosine),
+        # and the block scan over packaged codes returns the same floats
+        sums = lut8[np.arange(pq_dim)[None], nib].sum(1)
+        d_flat = orc.flat_dists(orc.PQFS, metric, pq_dim, codes, qc[r:r + 1])[0]
+        v = (sums.astype(np.float32) / np.float32(255.0)) * np.float32(diff) + np.float32(lower)
+        v = v if metric == orc.L2 else np.float32(1.0) - v
+        assert np.array_equal(d_flat.view(np.uint32), v.astype(np.float32).view(np.uint32))
+        pad = np.zeros((224, codes.shape[1]), np.uint8)
+        pad[:n] = codes
+        packaged = np.concatenate([orc.pqfs_package32(pad[b:b + 32], pq_dim, valid=min(32, n - b)) for b in range(0, 224, 32)])
+        d_scan = orc.pqfs_scan_batch(qc[r], packaged, n, pq_dim, metric)
+        assert np.array_equal(d_scan.view(np.uint32), d_flat.view(np.uint32))
+
+
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
+def test_pqfs_distances_meet_the_reference_tests_bound(metric):
+    """pq_fastscan_quantizer_test.cpp "PQFSQuantizer Compute": with one subspace per dimension, trained codebooks and
+    unit vectors, every distance is within 0.08 of the true one (dim 128, 300 vectors, 100 queries)."""
+    rng = np.random.default_rng(128 + metric)
+    n, nq, d = 300, 100, 128
+    x = rng.random((n, d), dtype=np.float32)
+    q = rng.random((nq, d), dtype=np.float32)
+    if metric != orc.COSINE:  # the reference's fixture normalises the vectors for l2 / ip and lets cosine do it
+        x /= np.linalg.norm(x, axis=1, keepdims=True)
+        q /= np.linalg.norm(q, axis=1, keepdims=True)
+    cb = orc.pq_train(x, d, metric)
+    codes = orc.pq_encode(x, d, cb, metric)
+    got = orc.flat_dists(orc.PQFS, metric, d, codes, orc.pqfs_process_query(q, d, cb, metric))
+    x64, q64 = x.astype(np.float64), q.astype(np.float64)
+    if metric == orc.COSINE:
+        x64 /= np.linalg.norm(x64, axis=1, keepdims=True)
+        q64 /= np.linalg.norm(q64, axis=1, keepdims=True)
+    true = ((q64[:, None] - x64[None]) ** 2).sum(-1) if metric == orc.L2 else 1.0 - q64 @ x64.T
+    assert np.abs(got - true).max() <= 0.08, float(np.abs(got - true).max())

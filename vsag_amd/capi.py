@@ -15,13 +15,13 @@ LIB_PATH = os.path.join(_HERE, "lib", "libvsag_amd.so")
 SUCCESS = 0
 INVALID_ARGUMENT = -3
 METRIC_L2, METRIC_IP, METRIC_COSINE = 0, 1, 2
-KIND_FP32, KIND_SQ8, KIND_SQ4, KIND_SQ4_UNIFORM, KIND_SQ8_UNIFORM, KIND_RABITQ = range(6)
+KIND_FP32, KIND_SQ8, KIND_SQ4, KIND_SQ4_UNIFORM, KIND_SQ8_UNIFORM, KIND_RABITQ, KIND_PQFS = range(7)
 SQ_TRAIN_CLASSIC, SQ_TRAIN_TRUNC_BOUND = 1, 3
 INVALID_ID = 0xFFFFFFFF
 
 METRICS = {"l2": METRIC_L2, "ip": METRIC_IP, "cosine": METRIC_COSINE}
 KINDS = {"fp32": KIND_FP32, "sq8": KIND_SQ8, "sq4": KIND_SQ4, "sq4_uniform": KIND_SQ4_UNIFORM,
-         "sq8_uniform": KIND_SQ8_UNIFORM, "rabitq": KIND_RABITQ}
+         "sq8_uniform": KIND_SQ8_UNIFORM, "rabitq": KIND_RABITQ, "pqfs": KIND_PQFS}
 
 
 class VsagAmdError(RuntimeError):
@@ -33,7 +33,8 @@ class VsagAmdError(RuntimeError):
 class StoreParams(C.Structure):
     _fields_ = [("kind", C.c_int), ("metric", C.c_int), ("dim", C.c_uint32),
                 ("lower_bound_dev", C.c_void_p), ("diff_dev", C.c_void_p), ("rotation_dev", C.c_void_p),
-                ("centroid_dev", C.c_void_p), ("rabitq_query_bits", C.c_int)]
+                ("centroid_dev", C.c_void_p), ("rabitq_query_bits", C.c_int), ("pq_dim", C.c_uint32),
+                ("codebooks_dev", C.c_void_p)]
 
 
 class SearchOptions(C.Structure):
@@ -67,6 +68,13 @@ PROTOTYPES = {
     "vsag_amd_rabitq_encode": (C.c_int, [_vp, _u64, _u32, _vp, _vp, _i32, _i32, _vp, _vp]),
     "vsag_amd_rabitq_query_code_size": (_u64, [_u32, _i32, _i32]),
     "vsag_amd_rabitq_process_query": (C.c_int, [_vp, _u64, _u32, _vp, _vp, _i32, _i32, _vp, _vp]),
+    "vsag_amd_pq_train_workspace_bytes": (_sz, [_u64, _u32, _u32]),
+    "vsag_amd_pq_train": (C.c_int, [_vp, _u64, _u32, _u32, _i32, _u64, _vp, _vp, _sz, _vp]),
+    "vsag_amd_pq_encode": (C.c_int, [_vp, _u64, _u32, _u32, _vp, _i32, _vp, _vp, _vp]),
+    "vsag_amd_pq_decode": (C.c_int, [_vp, _u64, _u32, _u32, _vp, _vp, _vp]),
+    "vsag_amd_pqfs_process_query": (C.c_int, [_vp, _u64, _u32, _u32, _vp, _i32, _vp, _vp]),
+    "vsag_amd_pqfs_package": (C.c_int, [_vp, _u64, _u32, _vp, _vp]),
+    "vsag_amd_pqfs_unpack": (C.c_int, [_vp, _u64, _u32, _vp, _vp]),
     "vsag_amd_store_create": (C.c_int, [C.POINTER(StoreParams), C.POINTER(_vp)]),
     "vsag_amd_store_destroy": (C.c_int, [_vp]),
     "vsag_amd_store_size": (_u64, [_vp]),

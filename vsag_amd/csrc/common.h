@@ -16,7 +16,9 @@ constexpr int kWave = 64;          // gfx950 wavefront width; one code tile hold
 constexpr int kGranule = 16;       // bytes per lane per tile row (one dwordx4)
 // Scan-kernel variant of VSAG_AMD_KIND_RABITQ for stores whose queries stay fp32 (rabitq_bits_per_dim_query = 32);
 // only the kernel templates and their dispatch know it.
-constexpr int kKindRabitqF32 = VSAG_AMD_KIND_RABITQ + 1;
+constexpr int kKindRabitqF32 = 100;  // a tag of the kernels only, beyond the public kinds
+// pqfs: the float table of a query (16 entries per subspace) must fit 64 KB of LDS while it is quantised
+constexpr uint32_t kMaxPqDim = 1024;
 constexpr int kMaxGroup = 8;       // most granule rows the scans fetch together
 // Readable bytes past the last tile of every tile buffer: the last group of a tile is fetched whole.
 constexpr size_t kTileSlackBytes = static_cast<size_t>(kMaxGroup - 1) * kWave * kGranule;

@@ -12,6 +12,7 @@
 //   SQ4U   src/simd/generic.cpp:406-422 + sq4_uniform_quantizer.cpp:166-201
 //   SQ8U   src/simd/generic.cpp:424-431 + sq8_uniform_quantizer.cpp:141-170
 //   RaBitQ src/simd/generic.cpp:832-872 + rabitq_quantizer.cpp:915-939,1775-1860
+//   PQFS   src/simd/generic.cpp:902-921 (PQFastScanLookUp32) + pq_fastscan_quantizer.cpp:166-199
 #pragma once
 
 #include "common.h"
@@ -187,6 +188,23 @@ accumulate_granule(const ScanArgs& a, const QueryRows<T>& q, uint32_t j, uint4 c
                 }
             }
         }
+    } else if constexpr (KIND == VSAG_AMD_KIND_PQFS) {
+        // qtab row: 16 table bytes per subspace.  A granule holds the centroid indices of 32 subspaces (byte b:
+        // subspace 2 b in the low nibble, 2 b + 1 in the high one); every lane looks its own entries up, so these
+        // are vector loads of one byte (all lanes inside the 16 bytes of one subspace: one memory line).
+        typedef const uint8_t __attribute__((address_space(4))) * cu8_p;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t nib = (w[m] >> (4 * e)) & 15U;
+                const uint32_t at = (32 * j + 8 * m + e) * 16 + nib;
+#pragma unroll
+                for (int t = 0; t < T; ++t) {
+                    acc.lo[t] += reinterpret_cast<cu8_p>(q.row[t])[at];
+                }
+            }
+        }
     } else if constexpr (KIND == VSAG_AMD_KIND_RABITQ) {
         // qtab row: per code dword the four query bit planes.
 #pragma unroll
@@ -237,6 +255,14 @@ finish_distances(const ScanArgs& a, const uint32_t (&qidx)[T], uint64_t slot, co
                 float r = a.f0 * (qm + m0) + a.f1 * result + a.f2;
                 out[t] = 1 - r;
             }
+        }
+    } else if constexpr (KIND == VSAG_AMD_KIND_PQFS) {
+        // qmeta: {diff, lower} of the query's byte table; float(sum) / 255 * diff + lower, 1 - that for ip / cosine.
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const float* qm = a.qmeta + static_cast<size_t>(qidx[t]) * a.qmeta_stride;
+            const float v = static_cast<float>(static_cast<int32_t>(acc.lo[t])) / 255.0F * qm[0] + qm[1];
+            out[t] = METRIC == VSAG_AMD_METRIC_L2 ? v : 1.0F - v;
         }
     } else if constexpr (KIND == VSAG_AMD_KIND_RABITQ || KIND == kKindRabitqF32) {
         // qmeta, 4-bit queries: {2 delta/sqrt(d), 2 lb/sqrt(d), delta sum_q/sqrt(d), lb d/sqrt(d), ||Rq - c||, ||q||};

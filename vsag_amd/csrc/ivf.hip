@@ -856,6 +856,9 @@ launch_ivf(const vsag_amd_store* s, int T, dim3 grid, dim3 block, size_t lds, hi
         case VSAG_AMD_KIND_SQ8_UNIFORM:
             launch_ivf_m<VSAG_AMD_KIND_SQ8_UNIFORM>(s->metric, T, grid, block, lds, st, a, v);
             break;
+        case VSAG_AMD_KIND_PQFS:
+            launch_ivf_m<VSAG_AMD_KIND_PQFS>(s->metric, T, grid, block, lds, st, a, v);
+            break;
         case VSAG_AMD_KIND_RABITQ:
             if (s->query_bits == 32) {
                 launch_ivf_m<kKindRabitqF32>(s->metric, T, grid, block, lds, st, a, v);

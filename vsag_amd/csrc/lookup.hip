@@ -342,6 +342,9 @@ vsag_amd_store_distances(const vsag_amd_store_t* s, const float* queries_dev, ui
         case VSAG_AMD_KIND_SQ8_UNIFORM:
             launch_lookup_m<VSAG_AMD_KIND_SQ8_UNIFORM>(s->metric, grid, st, a, p);
             break;
+        case VSAG_AMD_KIND_PQFS:
+            launch_lookup_m<VSAG_AMD_KIND_PQFS>(s->metric, grid, st, a, p);
+            break;
         case VSAG_AMD_KIND_RABITQ:
             if (s->query_bits == 32) {
                 launch_lookup_m<kKindRabitqF32>(s->metric, grid, st, a, p);
@@ -381,8 +384,12 @@ vsag_amd_residual_bias(const vsag_amd_store_t* s, const uint8_t* codes_dev, uint
     VA_CHECK_ARG(s && codes_dev && labels_dev && centroids_dev && bias_dev && decoded_dev, "null pointer");
     VA_CHECK_ARG(s->kind != VSAG_AMD_KIND_RABITQ, "residual codes of a rabitq store are not supported");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(decode_kernel, dim3(static_cast<uint32_t>(div_up(n * s->dim, 256))), dim3(256), 0, st, s->kind,
-                       codes_dev, n, s->dim, s->code_size, s->lb_dev, s->diff_dev, s->ulb, s->udiff, decoded_dev);
+    if (s->kind == VSAG_AMD_KIND_PQFS) {
+        VA_TRY(vsag_amd_pq_decode(codes_dev, n, s->dim, s->pq_dim, s->codebooks_dev, decoded_dev, stream));
+    } else {
+        hipLaunchKernelGGL(decode_kernel, dim3(static_cast<uint32_t>(div_up(n * s->dim, 256))), dim3(256), 0, st, s->kind,
+                           codes_dev, n, s->dim, s->code_size, s->lb_dev, s->diff_dev, s->ulb, s->udiff, decoded_dev);
+    }
     hipLaunchKernelGGL(residual_bias_kernel, dim3(static_cast<uint32_t>(div_up(n, 256))), dim3(256), 0, st, decoded_dev, n,
                        s->dim, labels_dev, centroids_dev, bias_dev);
     VA_HIP(hipGetLastError());

@@ -232,11 +232,18 @@ query_staging_bytes(const vsag_amd_store* s, uint64_t nq) {
     return scratch == 0 ? query_code_bytes(s, nq) : round_up(query_code_bytes(s, nq), 256) + scratch;
 }
 
+int pqfs_prepare_launch(const vsag_amd_store* s, const float* queries, uint64_t nq, uint64_t nq_pad, uint32_t* qtab,
+                        uint32_t qstride, float* qmeta, uint32_t qmeta_stride, hipStream_t st);
+
 QueryLayout
 query_layout(const vsag_amd_store* s) {
     QueryLayout l{};
     uint32_t ndw = s->G * 4;
     switch (s->kind) {
+        case VSAG_AMD_KIND_PQFS:
+            l.qstride = s->G * 128;  // 16 table bytes for each of the 32 subspaces of a granule
+            l.qmeta = 2;
+            break;
         case VSAG_AMD_KIND_FP32:
             l.qstride = s->dpad;
             l.qmeta = 1;
@@ -356,6 +363,9 @@ prepare_queries(const vsag_amd_store* s, const float* queries, uint64_t nq, uint
                                ql.qstride, qmeta, ql.qmeta);
             break;
         }
+        case VSAG_AMD_KIND_PQFS:
+            VA_TRY(pqfs_prepare_launch(s, queries, nq, nq_pad, qtab, ql.qstride, qmeta, ql.qmeta, st));
+            break;
         default:
             return fail(VSAG_AMD_INVALID_ARGUMENT, "unknown store kind %d", s->kind);
     }

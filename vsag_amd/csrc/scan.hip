@@ -1069,6 +1069,9 @@ launch_flat(const vsag_amd_store* s, const ScanPlan& p, const ScanArgs& a, const
         case VSAG_AMD_KIND_SQ8_UNIFORM:
             launch_flat_m<VSAG_AMD_KIND_SQ8_UNIFORM>(s->metric, p.T, grid, block, lds, st, a, f);
             break;
+        case VSAG_AMD_KIND_PQFS:
+            launch_flat_m<VSAG_AMD_KIND_PQFS>(s->metric, p.T, grid, block, lds, st, a, f);
+            break;
         case VSAG_AMD_KIND_RABITQ:
             if (s->query_bits == 32) {
                 launch_flat_m<kKindRabitqF32>(s->metric, p.T, grid, block, lds, st, a, f);

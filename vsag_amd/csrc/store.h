@@ -48,6 +48,8 @@ struct vsag_amd_store {
     float* bounds_dev = nullptr;                // uniform kinds: {lb, diff}
     float* rotation_dev = nullptr;              // rabitq
     float* centroid_dev = nullptr;              // rabitq
+    uint32_t pq_dim = 0;                        // pqfs: subspaces
+    float* codebooks_dev = nullptr;             // pqfs: pq_dim x 16 x (dim / pq_dim)
 
     // codes
     uint4* tiles = nullptr;

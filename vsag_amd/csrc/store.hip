@@ -362,6 +362,8 @@ vsag_amd_code_size(int kind, int metric, uint32_t dim, int rabitq_query_bits) {
         }
         case VSAG_AMD_KIND_RABITQ:
             return rabitq_code_size(dim, metric, rabitq_query_bits ? rabitq_query_bits : 4);
+        case VSAG_AMD_KIND_PQFS:
+            return (static_cast<uint64_t>(dim) + 1) / 2;  // dim = the number of subspaces here
         default:
             return 0;
     }
@@ -372,7 +374,13 @@ vsag_amd_store_create(const vsag_amd_store_params_t* p, vsag_amd_store_t** out) 
     VA_TRY(ensure_init());
     VA_CHECK_ARG(p != nullptr && out != nullptr, "null params / output");
     *out = nullptr;
-    VA_CHECK_ARG(p->kind >= VSAG_AMD_KIND_FP32 && p->kind <= VSAG_AMD_KIND_RABITQ, "unknown store kind %d", p->kind);
+    VA_CHECK_ARG(p->kind >= VSAG_AMD_KIND_FP32 && p->kind <= VSAG_AMD_KIND_PQFS, "unknown store kind %d", p->kind);
+    if (p->kind == VSAG_AMD_KIND_PQFS) {
+        VA_CHECK_ARG(p->pq_dim >= 1 && p->dim % p->pq_dim == 0, "pq_dim(%u) does not divide evenly into dim(%u)", p->pq_dim,
+                     p->dim);
+        VA_CHECK_ARG(p->pq_dim <= kMaxPqDim, "pq_dim must be at most %u, got %u", kMaxPqDim, p->pq_dim);
+        VA_CHECK_ARG(p->codebooks_dev != nullptr, "pqfs store needs codebooks_dev");
+    }
     VA_CHECK_ARG(p->metric >= VSAG_AMD_METRIC_L2 && p->metric <= VSAG_AMD_METRIC_COSINE, "unknown metric %d",
                  p->metric);
     VA_CHECK_ARG(p->dim >= 1 && p->dim <= 65536, "dim must be in [1, 65536], got %u", p->dim);
@@ -384,7 +392,9 @@ vsag_amd_store_create(const vsag_amd_store_params_t* p, vsag_amd_store_t** out) 
     s->metric = p->metric;
     s->dim = p->dim;
     s->query_bits = p->rabitq_query_bits ? p->rabitq_query_bits : 4;
-    s->code_size = static_cast<uint32_t>(vsag_amd_code_size(p->kind, p->metric, p->dim, s->query_bits));
+    s->pq_dim = p->kind == VSAG_AMD_KIND_PQFS ? p->pq_dim : 0;
+    s->code_size = static_cast<uint32_t>(
+        vsag_amd_code_size(p->kind, p->metric, p->kind == VSAG_AMD_KIND_PQFS ? p->pq_dim : p->dim, s->query_bits));
     uint32_t dims_per_granule = 16;
     auto up = [](uint64_t v, uint64_t a) { return (v + a - 1) / a * a; };
     int rc = 0;
@@ -439,6 +449,11 @@ vsag_amd_store_create(const vsag_amd_store_params_t* p, vsag_amd_store_t** out) 
             s->meta_offset[3] = p->metric != VSAG_AMD_METRIC_L2 ? s->code_size - 4 : off + 4;
             break;
         }
+        case VSAG_AMD_KIND_PQFS:
+            // a granule holds the 4-bit centroid indices of 32 subspaces (dpad counts subspaces for this kind)
+            s->payload_bytes = s->code_size;
+            dims_per_granule = 32;
+            break;
     }
     s->G = static_cast<uint32_t>((s->payload_bytes + kGranule - 1) / kGranule);
     s->dpad = s->G * dims_per_granule;
@@ -486,6 +501,12 @@ vsag_amd_store_create(const vsag_amd_store_params_t* p, vsag_amd_store_t** out) 
             hipMemcpy(s->centroid_dev, p->centroid_dev, p->dim * 4, hipMemcpyDeviceToDevice) != hipSuccess) {
             return fail_free(fail(VSAG_AMD_NO_ENOUGH_MEMORY, "copying the rabitq rotation failed"));
         }
+    } else if (p->kind == VSAG_AMD_KIND_PQFS) {
+        const size_t cb = static_cast<size_t>(p->dim) * 16 * 4;
+        if (hipMalloc(&s->codebooks_dev, cb) != hipSuccess ||
+            hipMemcpy(s->codebooks_dev, p->codebooks_dev, cb, hipMemcpyDeviceToDevice) != hipSuccess) {
+            return fail_free(fail(VSAG_AMD_NO_ENOUGH_MEMORY, "copying the pq codebooks failed"));
+        }
     }
     // Stores the matrix cores can pre-select on keep a per-code term (and the largest norm, where a threshold needs it).
     if (p->kind == VSAG_AMD_KIND_FP32 || p->kind == VSAG_AMD_KIND_SQ8 ||
@@ -508,7 +529,7 @@ vsag_amd_store_destroy(vsag_amd_store_t* s) {
     void* ptrs[] = {s->scale_dev, s->lb_dev,  s->diff_dev, s->bounds_dev,    s->rotation_dev, s->centroid_dev,
                     s->tiles,     s->meta,    s->ids_dev,  s->list_tile_dev, s->pf_term,      s->pf_ymax,
                     s->rows,      s->slot_of_id_dev, s->residual_bias_dev, s->residual_centroids_dev,
-                    s->list_sizes_dev};
+                    s->list_sizes_dev, s->codebooks_dev};
     for (void* p : ptrs) {
         if (p != nullptr) {
             (void)hipFree(p);
