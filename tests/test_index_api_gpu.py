@@ -407,3 +407,52 @@ def test_ivf_with_a_thousand_buckets_routes_large_batches_through_the_table(lib)
     gt, _ = ground_truth(x, q[:100], k, "l2")
     assert recall(ai[:100], gt, labels) >= 0.9
     idx.close()
+
+
+@pytest.mark.parametrize("metric", ["l2", "ip", "cosine"])
+@pytest.mark.parametrize("residual", [False, True])
+def test_ivf_pqfs_recall_floor_and_conventions(lib, metric, residual):
+    """base_quantization_type "pqfs" with fp32 reorder: the reference's floor for "pqfs,fp32" is 0.82, with a subspace
+    per dimension (tests/test_ivf.cpp:94-102,166-172,1292-1300), with and without use_residual."""
+    n, d, nq, k = 2400, 64, 100, 10
+    x = vectors(n, d)
+    q = vectors(nq, d, seed=165)
+    labels = np.arange(n, dtype=np.int64) + 1000
+    idx = make("ivf", d, metric, buckets_count=50, base_quantization_type="pqfs", base_pq_dim=d, use_reorder=True,
+               precise_quantization_type="fp32", train_sample_count=2400, use_residual=residual)
+    assert idx.build(x, labels, n, d) == 0
+    gt, _ = ground_truth(x, q, k, metric)
+    search = json.dumps({"ivf": {"scan_buckets_count": 30, "factor": 4.0}})
+    ids, dists = idx.knn_search_batch(q, k, search)
+    r = recall(ids, gt, labels)
+    assert r >= 0.82 * RECALL_THRESHOLD, r
+    assert np.all(np.diff(dists, axis=1) >= 0)
+    for i in range(8):  # batch == serial, bit for bit
+        sid, sd = idx.knn_search(q[i], k, search)
+        assert np.array_equal(sid, ids[i]) and np.array_equal(sd, dists[i])
+    idx.close()
+
+
+def test_pqfs_parameters_and_brute_force(lib):
+    d = 48
+    # pq_fastscan_quantizer.cpp:31-36: pq_dim must divide the dimension; the default pq_dim is 1
+    with pytest.raises(pyvsag.VsagError) as e:
+        make("ivf", d, "l2", buckets_count=8, base_quantization_type="pqfs", base_pq_dim=7)
+    assert "does not divide evenly" in str(e.value)
+    with pytest.raises(pyvsag.VsagError):
+        make("ivf", d, "l2", buckets_count=8, base_quantization_type="sq8", use_reorder=True,
+             precise_quantization_type="pqfs")
+    # a flat store of pqfs codes scans like any other kind: against the checker on the same codebooks it would be
+    # bit-exact (tests/test_pqfs_gpu.py); here the approximation itself, with a subspace per dimension
+    n, nq, k = 3000, 40, 10
+    x = vectors(n, d)
+    q = vectors(nq, d, seed=165)
+    labels = np.arange(n, dtype=np.int64)
+    idx = make("brute_force", d, "l2", base_quantization_type="pqfs", base_pq_dim=d)
+    assert idx.build(x, labels, n, d) == 0
+    ids, dists = idx.knn_search_batch(q, k, "{}")
+    gt, gt_d = ground_truth(x, q, k, "l2")
+    assert recall(ids, gt, labels) >= 0.5
+    true = ((q[:, None].astype(np.float64) - x[ids].astype(np.float64)) ** 2).sum(-1)
+    assert np.abs(dists - true).max() <= 0.08  # the bound of the reference's own quantizer test
+    idx.close()

@@ -158,6 +158,9 @@ IVF_CASES = [
     ({"base_quantization_type": "sq8", "use_residual": True}, "l2", None),
     ({"base_quantization_type": "fp32", "buckets_per_data": 2}, "cosine", None),
     ({"base_quantization_type": "rabitq", "use_reorder": True, "precise_quantization_type": "fp32"}, "l2", 10.0),
+    ({"base_quantization_type": "pqfs", "base_pq_dim": 16, "use_reorder": True, "precise_quantization_type": "fp32"},
+     "l2", 5.0),
+    ({"base_quantization_type": "pqfs", "base_pq_dim": 32, "use_residual": True}, "cosine", None),
 ]
 
 
@@ -342,3 +345,39 @@ def test_deserialize_errors(lib, tmp_path):
     fresh.deserialize(tmp_path / "empty.index")
     assert fresh.get_num_elements() == 0
     a.close()
+
+
+def test_ivf_pqfs_bucket_cell_holds_packaged_blocks(lib, tmp_path):
+    """A pqfs bucket is serialized as BucketDataCell keeps it (package_fastscan, bucket_datacell.h:943-966): whole
+    blocks of 32 codes in the fast-scan order of PQFastScanQuantizer::Package32; the quantizer writes pq_dim, the
+    subspace dimension and the codebooks (pq_fastscan_quantizer.cpp:201-207)."""
+    n, d, nlist, pq_dim = 1500, 24, 6, 12
+    x = vectors(n, d, normalize=False)
+    labels = np.arange(n, dtype=np.int64)
+    idx = make("ivf", d, "l2", buckets_count=nlist, train_sample_count=1500, base_quantization_type="pqfs",
+               base_pq_dim=pq_dim)
+    idx.build(x, labels, n, d)
+    path = tmp_path / "ivf.index"
+    idx.serialize(path)
+    data = path.read_bytes()
+    meta, _ = footer_of(data)
+    cs = pq_dim // 2
+    c = Cursor(data, meta["datacell_offsets"]["bucket"])
+    assert c.take("iI") == (nlist, cs)
+    assert c.take("QiQB") == (d, 0, cs, 1)
+    assert c.take("qq") == (pq_dim, d // pq_dim)
+    cb = c.vector(np.float32).reshape(pq_dim, 16, d // pq_dim)
+    seen = []
+    for _ in range(nlist):
+        size = c.take("Q")
+        packaged = c.array(np.uint8, size)
+        ids = c.vector(np.uint32)
+        assert size == (ids.size + 31) // 32 * 32 * cs
+        want = orc.pq_encode(x[ids], pq_dim, cb, orc.L2)
+        for b in range(0, ids.size, 32):
+            blk = np.zeros((32, cs), np.uint8)
+            blk[:min(32, ids.size - b)] = want[b:b + 32]
+            assert np.array_equal(packaged[b * cs:(b + 32) * cs], orc.pqfs_package32(blk, pq_dim, valid=min(32, ids.size - b)))
+        seen.append(ids)
+    assert np.array_equal(np.sort(np.concatenate(seen)), np.arange(n, dtype=np.uint32))
+    idx.close()

@@ -449,7 +449,7 @@ kind_from_name(const std::string& name) {
     static const std::pair<const char*, int> kinds[] = {
         {"fp32", VSAG_AMD_KIND_FP32}, {"sq8", VSAG_AMD_KIND_SQ8}, {"sq4", VSAG_AMD_KIND_SQ4},
         {"sq4_uniform", VSAG_AMD_KIND_SQ4_UNIFORM}, {"sq8_uniform", VSAG_AMD_KIND_SQ8_UNIFORM},
-        {"rabitq", VSAG_AMD_KIND_RABITQ}};
+        {"rabitq", VSAG_AMD_KIND_RABITQ}, {"pqfs", VSAG_AMD_KIND_PQFS}};
     for (const auto& k : kinds) {
         if (name == k.first) {
             return k.second;
@@ -464,12 +464,13 @@ struct Quantizer {
     int metric = VSAG_AMD_METRIC_L2;
     uint32_t dim = 0;
     int rabitq_query_bits = 32;
+    uint32_t pq_dim = 1;  // pqfs: subspaces (PQFastScanQuantizerParameter::pq_dim_, default 1)
     bool trained = false;
-    DevBuf lb, diff, bounds, rotation, centroid;
+    DevBuf lb, diff, bounds, rotation, centroid, codebooks;
 
     uint64_t
     code_size() const {
-        return vsag_amd_code_size(kind, metric, dim, rabitq_query_bits);
+        return vsag_amd_code_size(kind, metric, kind == VSAG_AMD_KIND_PQFS ? pq_dim : dim, rabitq_query_bits);
     }
 
     // Random orthogonal matrix: Gram-Schmidt on a Gaussian matrix (the reference takes the Q of a LAPACK QR,
@@ -551,6 +552,15 @@ struct Quantizer {
                 dev(vsag_amd_rabitq_train(x_dev, n, dim, rotation.as<float>(), centroid.as<float>(), nullptr));
                 break;
             }
+            case VSAG_AMD_KIND_PQFS: {
+                // PQFastScanQuantizer::TrainImpl (pq_fastscan_quantizer.cpp:62-94); the seed is fixed so that a build
+                // is reproducible (the reference draws from std::random_device)
+                codebooks.reserve(static_cast<size_t>(dim) * 16 * 4);
+                size_t wsb = vsag_amd_pq_train_workspace_bytes(n, dim, pq_dim);
+                ws.reserve(wsb);
+                dev(vsag_amd_pq_train(x_dev, n, dim, pq_dim, metric, 20240301U, codebooks.as<float>(), ws.p, wsb, nullptr));
+                break;
+            }
         }
         dev(vsag_amd_stream_synchronize(nullptr));
         trained = true;
@@ -576,6 +586,16 @@ struct Quantizer {
                 dev(vsag_amd_rabitq_encode(x_dev, n, dim, rotation.as<float>(), centroid.as<float>(), metric,
                                            rabitq_query_bits, codes, nullptr));
                 break;
+            case VSAG_AMD_KIND_PQFS: {
+                DevBuf norms;
+                if (metric == VSAG_AMD_METRIC_COSINE) {
+                    norms.reserve(n * 4);
+                }
+                dev(vsag_amd_pq_encode(x_dev, n, dim, pq_dim, codebooks.as<float>(), metric, codes, norms.as<float>(),
+                                       nullptr));
+                dev(vsag_amd_stream_synchronize(nullptr));  // the scratch goes with this scope
+                break;
+            }
         }
     }
 
@@ -587,6 +607,7 @@ struct Quantizer {
         q.metric = metric;
         q.dim = dim;
         q.rabitq_query_bits = rabitq_query_bits;
+        q.pq_dim = pq_dim;
         return q;
     }
     void
@@ -594,7 +615,7 @@ struct Quantizer {
         trained = other.trained;
         for (auto pair : {std::make_pair(&lb, &other.lb), std::make_pair(&diff, &other.diff),
                           std::make_pair(&bounds, &other.bounds), std::make_pair(&rotation, &other.rotation),
-                          std::make_pair(&centroid, &other.centroid)}) {
+                          std::make_pair(&centroid, &other.centroid), std::make_pair(&codebooks, &other.codebooks)}) {
             std::swap(pair.first->p, pair.second->p);
             std::swap(pair.first->bytes, pair.second->bytes);
         }
@@ -663,6 +684,12 @@ struct Quantizer {
                 w.vec(floats(centroid, dim));
                 w.vec(floats(rotation, static_cast<size_t>(dim) * dim));
                 break;
+            case VSAG_AMD_KIND_PQFS:
+                // PQFastScanQuantizer::SerializeImpl (pq_fastscan_quantizer.cpp:201-207)
+                w.obj(static_cast<int64_t>(pq_dim));
+                w.obj(static_cast<int64_t>(dim / pq_dim));
+                w.vec(floats(codebooks, static_cast<size_t>(dim) * 16));
+                break;
         }
     }
 
@@ -711,6 +738,18 @@ struct Quantizer {
                 upload(centroid, a, dim);
                 upload(rotation, b, static_cast<size_t>(dim) * dim);
                 break;
+            case VSAG_AMD_KIND_PQFS: {
+                const auto fpq = r.get<int64_t>();
+                const auto fsd = r.get<int64_t>();
+                if (fpq != static_cast<int64_t>(pq_dim) || fsd != static_cast<int64_t>(dim / pq_dim)) {
+                    throw VsagException(ErrorType::INVALID_ARGUMENT,
+                                        "the serialized pqfs quantizer has pq_dim " + std::to_string(fpq) +
+                                            ", the index " + std::to_string(pq_dim));
+                }
+                r.vec(a);
+                upload(codebooks, a, static_cast<size_t>(dim) * 16);
+                break;
+            }
         }
         trained = ftrained != 0;
     }
@@ -730,6 +769,9 @@ struct Quantizer {
         } else if (kind == VSAG_AMD_KIND_RABITQ) {
             p.rotation_dev = rotation.as<float>();
             p.centroid_dev = centroid.as<float>();
+        } else if (kind == VSAG_AMD_KIND_PQFS) {
+            p.pq_dim = pq_dim;
+            p.codebooks_dev = codebooks.as<float>();
         }
         vsag_amd_store_t* s = nullptr;
         dev(vsag_amd_store_create(&p, &s));
@@ -1274,6 +1316,51 @@ store_distances(SearchContext& ctx, const vsag_amd_store_t* store, const float* 
     }
 }
 
+// A posting list of pqfs codes as BucketDataCell keeps and serializes it (package_fastscan, bucket_datacell.h:943-966;
+// PQFastScanQuantizer::Package32, pq_fastscan_quantizer.cpp:241-266): blocks of 32 codes, subspace i of a block in 16
+// bytes, byte j / 2 holding the code of vector MAPPER[j] of the block in its low (even j) or high nibble; the last
+// block is padded with zeros.  n plain codes of cs bytes -> ceil(n / 32) * 32 * cs bytes, and back.
+constexpr int kPqMapper[32] = {0, 16, 8, 24, 1, 17, 9, 25, 2, 18, 10, 26, 3, 19, 11, 27,
+                               4, 20, 12, 28, 5, 21, 13, 29, 6, 22, 14, 30, 7, 23, 15, 31};
+
+void
+pqfs_package_list(const uint8_t* codes, uint64_t n, uint32_t pq_dim, std::vector<uint8_t>& out) {
+    const uint64_t cs = (pq_dim + 1) / 2, blocks = (n + 31) / 32;
+    out.assign(blocks * 32 * cs, 0);
+    for (uint64_t b = 0; b < blocks; ++b) {
+        uint8_t* dst = out.data() + b * 32 * cs;
+        for (uint32_t i = 0; i < pq_dim; ++i) {
+            for (int j = 0; j < 32; ++j) {
+                const uint64_t v = b * 32 + static_cast<uint64_t>(kPqMapper[j]);
+                if (v >= n) {
+                    continue;
+                }
+                const uint8_t nib = (codes[v * cs + i / 2] >> (4 * (i & 1))) & 15;
+                dst[i * 16 + j / 2] |= static_cast<uint8_t>(nib << (4 * (j & 1)));
+            }
+        }
+    }
+}
+
+void
+pqfs_unpack_list(const uint8_t* packaged, uint64_t n, uint32_t pq_dim, uint8_t* codes) {
+    const uint64_t cs = (pq_dim + 1) / 2;
+    std::memset(codes, 0, n * cs);
+    for (uint64_t b = 0; b * 32 < n; ++b) {
+        const uint8_t* src = packaged + b * 32 * cs;
+        for (uint32_t i = 0; i < pq_dim; ++i) {
+            for (int j = 0; j < 32; ++j) {
+                const uint64_t v = b * 32 + static_cast<uint64_t>(kPqMapper[j]);
+                if (v >= n) {
+                    continue;
+                }
+                const uint8_t nib = (src[i * 16 + j / 2] >> (4 * (j & 1))) & 15;
+                codes[v * cs + i / 2] |= static_cast<uint8_t>(nib << (4 * (i & 1)));
+            }
+        }
+    }
+}
+
 // FlattenDataCell::Serialize (src/datacell/flatten_datacell.h:481-497): [u32 total count][u32 capacity][u32 code size]
 // [u64 bytes][codes by inner id][quantizer].  `rows`: the codes are fp32 rows kept outside a store.
 void
@@ -1384,6 +1471,24 @@ read_rabitq_params(const Json& index_param, Quantizer& q) {
     }
 }
 
+// base_pq_dim (constants.cpp:197,211 -> PRODUCT_QUANTIZATION_DIM_KEY): the number of subspaces of a pqfs quantizer;
+// the constructor of PQFastScanQuantizer rejects one that does not divide the dimension
+// (pq_fastscan_quantizer.cpp:31-36).
+void
+read_pq_params(const Json& index_param, Quantizer& q) {
+    if (q.kind != VSAG_AMD_KIND_PQFS) {
+        return;
+    }
+    int64_t pq_dim = 1;
+    if (index_param.Contains("base_pq_dim")) {
+        pq_dim = index_param["base_pq_dim"].GetInt();
+    }
+    CHECK_ARGUMENT(pq_dim >= 1 && static_cast<int64_t>(q.dim) % pq_dim == 0,
+                   "pq_dim(" + std::to_string(pq_dim) + ") does not divide evenly into dim(" + std::to_string(q.dim) + ")");
+    CHECK_ARGUMENT(pq_dim <= 1024, "the GPU path supports base_pq_dim up to 1024, got " + std::to_string(pq_dim));
+    q.pq_dim = static_cast<uint32_t>(pq_dim);
+}
+
 // ------------------------------------------------------------------------------------------- brute force
 class BruteForce : public GpuIndex {
 public:
@@ -1400,6 +1505,7 @@ public:
             q_.kind = kind_from_name(index_param["base_quantization_type"].GetString());
         }
         read_rabitq_params(index_param, q_);
+        read_pq_params(index_param, q_);
     }
 
     // BruteForce::Train (bruteforce.cpp:123-126): the quantizer of the codes is trained on the data.
@@ -1664,6 +1770,7 @@ public:
             q_.kind = kind_from_name(index_param["base_quantization_type"].GetString());
         }
         read_rabitq_params(index_param, q_);
+        read_pq_params(index_param, q_);
         if (index_param.Contains("buckets_count")) {
             int64_t b = index_param["buckets_count"].GetInt();
             CHECK_ARGUMENT(b >= 1 && b <= (1 << 24), "buckets_count must be in [1, 2^24], got " + std::to_string(b));
@@ -1675,6 +1782,9 @@ public:
         if (index_param.Contains("precise_quantization_type")) {
             pq_.kind = kind_from_name(index_param["precise_quantization_type"].GetString());
             CHECK_ARGUMENT(pq_.kind != VSAG_AMD_KIND_RABITQ, "precise_quantization_type must not be rabitq");
+            // the reference's reorder asks a pqfs cell for single distances, which it refuses
+            // (pq_fastscan_quantizer.cpp:158-164)
+            CHECK_ARGUMENT(pq_.kind != VSAG_AMD_KIND_PQFS, "precise_quantization_type must not be pqfs");
         }
         if (index_param.Contains("precise_codes_layout")) {
             // "bucket" keeps the precise codes list by list instead of in one array (ivf.cpp:441-455); the distances are
@@ -2061,10 +2171,17 @@ protected:
             }
         }
         uint64_t at = 0;
+        std::vector<uint8_t> packaged;
         for (uint32_t l = 0; l < nlist_; ++l) {
             const uint64_t n = list_sizes[l];
-            w.obj(n * cs);
-            w.write(codes.data() + at * cs, n * cs);
+            if (q_.kind == VSAG_AMD_KIND_PQFS) {
+                pqfs_package_list(codes.data() + at * cs, n, q_.pq_dim, packaged);
+                w.obj(static_cast<uint64_t>(packaged.size()));
+                w.write(packaged.data(), packaged.size());
+            } else {
+                w.obj(n * cs);
+                w.write(codes.data() + at * cs, n * cs);
+            }
             w.obj(n);
             w.write(ids.data() + at, n * 4);
             if (use_residual_) {
@@ -2223,8 +2340,20 @@ protected:
                 throw VsagException(ErrorType::INVALID_BINARY, "a serialized list is shorter than its size");
             }
             list_codes.resize(n * cs);
-            r.read(list_codes.data(), n * cs);
-            r.skip(bytes - n * cs);
+            if (q_.kind == VSAG_AMD_KIND_PQFS) {
+                // whole blocks of 32 codes in the fast-scan order
+                const uint64_t padded = (n + 31) / 32 * 32 * cs;
+                if (bytes < padded) {
+                    throw VsagException(ErrorType::INVALID_BINARY, "a serialized pqfs list is not made of whole blocks");
+                }
+                std::vector<uint8_t> packaged(padded);
+                r.read(packaged.data(), padded);
+                r.skip(bytes - padded);
+                pqfs_unpack_list(packaged.data(), n, q_.pq_dim, list_codes.data());
+            } else {
+                r.read(list_codes.data(), n * cs);
+                r.skip(bytes - n * cs);
+            }
             r.vec(list_ids);
             if (list_ids.size() < n) {
                 throw VsagException(ErrorType::INVALID_BINARY,
