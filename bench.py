@@ -165,9 +165,12 @@ class Env:
         self.capi.check(self.lib.vsag_amd_last_kernel_ms(C.byref(ms)))
         return ms.value
 
-    def make_store(self, kind, metric, dim, lb=None, diff=None, bounds=None, rot=None, cen=None, qbits=4):
+    def make_store(self, kind, metric, dim, lb=None, diff=None, bounds=None, rot=None, cen=None, qbits=4, pq_dim=0,
+                   codebooks=None):
         p = self.capi.StoreParams()
         p.kind, p.metric, p.dim, p.rabitq_query_bits = kind, metric, dim, qbits
+        if codebooks is not None:
+            p.pq_dim, p.codebooks_dev = pq_dim, codebooks.ptr
         if lb is not None:
             p.lower_bound_dev, p.diff_dev = lb.ptr, diff.ptr
         if bounds is not None:
@@ -579,8 +582,10 @@ def run_c4(env):
     bits = 4 if args.list_codes == "sq4_uniform" else 8
     per_dim = args.list_codes == "sq8"
     one_bit = args.list_codes == "rabitq"  # 1-bit codes, 4-bit queries, a seeded random rotation
-    kind = (capi.KIND_RABITQ if one_bit else capi.KIND_SQ8 if per_dim else capi.KIND_SQ8_UNIFORM if bits == 8
-            else capi.KIND_SQ4_UNIFORM)
+    pqfs = args.list_codes == "pqfs"       # 4-bit product quantization, --pq-dim subspaces (default: one per dimension)
+    pq_dim = (args.pq_dim or d) if pqfs else 0
+    kind = (capi.KIND_PQFS if pqfs else capi.KIND_RABITQ if one_bit else capi.KIND_SQ8 if per_dim
+            else capi.KIND_SQ8_UNIFORM if bits == 8 else capi.KIND_SQ4_UNIFORM)
     kind_name = args.list_codes
     means = mt(315).random((10000, d), dtype=np.float32)
     x_dev = env.buf(n * d * 4)
@@ -609,10 +614,18 @@ def run_c4(env):
     lb_dev, diff_dev = env.buf(d * 4), env.buf(d * 4)
     wsb = lib.vsag_amd_sq_train_workspace_bytes(ns, d, 0)
     ws = env.buf(wsb)
-    cs = int(lib.vsag_amd_code_size(kind, capi.METRIC_L2, d, 4 if one_bit else 0))
+    cs = int(lib.vsag_amd_code_size(kind, capi.METRIC_L2, pq_dim if pqfs else d, 4 if one_bit else 0))
     codes = env.buf(n * cs)
     rot = None
-    if one_bit:
+    if pqfs:
+        cb_dev = env.buf(d * 16 * 4)
+        wsp = lib.vsag_amd_pq_train_workspace_bytes(ns, d, pq_dim)
+        wp = env.buf(wsp)
+        capi.check(lib.vsag_amd_pq_train(x_dev.ptr, ns, d, pq_dim, capi.METRIC_L2, 11, cb_dev.ptr, wp.ptr, wsp, None))
+        wp.free()
+        capi.check(lib.vsag_amd_pq_encode(x_dev.ptr, n, d, pq_dim, cb_dev.ptr, capi.METRIC_L2, codes.ptr, None, None))
+        lists = env.make_store(kind, capi.METRIC_L2, d, pq_dim=pq_dim, codebooks=cb_dev)
+    elif one_bit:
         g = mt(316).standard_normal((d, d))
         rot, r = np.linalg.qr(g)
         rot = (rot * np.sign(np.diag(r))).astype(np.float32)
@@ -700,7 +713,12 @@ def run_c4(env):
         hlabels = labels.to_numpy(np.int32, (n,))
         offsets, order = orc.ivf_build_lists(hlabels, nlist)
         posting = hcodes[order]
-        if one_bit:
+        od = d
+        if pqfs:
+            hb = (None, None)
+            okind, od = orc.PQFS, pq_dim
+            qcodes = orc.pqfs_process_query(q[:sample], pq_dim, cb_dev.to_numpy(np.float32, (pq_dim, 16, d // pq_dim)), orc.L2)
+        elif one_bit:
             hb = (None, None)
             okind = orc.RABITQ
             qcodes = orc.rabitq_process_query(q[:sample], rot, cen_dev.to_numpy(np.float32, (d,)), orc.L2)
@@ -715,10 +733,10 @@ def run_c4(env):
         ref_name = {orc.SQ4U: "SQ4UniformComputeCodesIP", orc.SQ8U: "SQ8UniformComputeCodesIP",
                     orc.RABITQ: "RaBitQSQ4UBinaryIP"}.get(okind)
         ref = ref if ref and ref_name in ref else None
-        orc.ivf_scan(okind, orc.L2, d, posting, offsets, order, qcodes[:threads], b[:threads], kcand,
+        orc.ivf_scan(okind, orc.L2, od, posting, offsets, order, qcodes[:threads], b[:threads], kcand,
                      lb=hb[0], diff=hb[1], threads=threads)
         t0 = time.perf_counter()
-        cids, cds = orc.ivf_scan(okind, orc.L2, d, posting, offsets, order, qcodes, b[:sample], kcand,
+        cids, cds = orc.ivf_scan(okind, orc.L2, od, posting, offsets, order, qcodes, b[:sample], kcand,
                                  lb=hb[0], diff=hb[1], threads=threads)
         t_cpu = time.perf_counter() - t0
         orc.use_reference_kernels(None)
@@ -777,8 +795,9 @@ def run_c4(env):
                 "ops_per_launch": ops, "distance_evaluations_per_launch": float(rest),
                 "distance_evaluations_per_second": float(rest) / (kms * 1e-3)}
     return env.base_line("QPS @ recall@10 (IVF %s, 10M x 128)" % {"sq4_uniform": "SQ4-uniform", "sq8_uniform": "SQ8-uniform",
-                                                                  "sq8": "SQ8", "rabitq": "RaBitQ"}[kind_name],
-                         "queries/s", nq / sec, sec, "1-bit codes x u4 queries, i32 popcount sums, f32 estimator" if one_bit else
+                                                                  "sq8": "SQ8", "rabitq": "RaBitQ", "pqfs": "PQFS"}[kind_name],
+                         "queries/s", nq / sec, sec, "4-bit pq codes, u8 table sums in i32" if pqfs else
+                         "1-bit codes x u4 queries, i32 popcount sums, f32 estimator" if one_bit else
                          "u8 codes x f32 scale, f32 (pre-selection: i8 x i8, i32 sums)" if per_dim else "u%d codes, i32 dot" % bits,
                          "configs[3]%s: IVF search, N=%d, d=%d, nlist=%d, nprobe=%d, rerank %d, %d queries, k=%d"
                          % ("" if bits == 4 else " with %s lists" % kind_name, n, d, nlist, nprobe, kcand, nq, k),
@@ -927,8 +946,9 @@ def main():
     ap.add_argument("--chunks", type=int, default=0, help="base chunk override (0 = library default)")
     ap.add_argument("--contraction", type=int, default=0, choices=[-1, 0, 1],
                     help="matrix-core path of the flat scans: -1 never, 0 library default, 1 whenever supported")
-    ap.add_argument("--list-codes", default="sq4_uniform", choices=["sq4_uniform", "sq8_uniform", "sq8", "rabitq"],
+    ap.add_argument("--list-codes", default="sq4_uniform", choices=["sq4_uniform", "sq8_uniform", "sq8", "rabitq", "pqfs"],
                     help="c4 only: the quantizer of the posting lists (configs[3] names sq4_uniform)")
+    ap.add_argument("--pq-dim", type=int, default=0, help="c4 with --list-codes pqfs: subspaces (default: the dimension)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-recall", action="store_true", help="skip the recall check")
     ap.add_argument("--no-single", action="store_true", help="skip the one-query-per-call measurement")

@@ -160,3 +160,52 @@ def test_pqfs_posting_lists_and_lookup(lib, metric, mname):
     for b in (qb, ib, out, ws):
         b.free()
     st.destroy()
+
+
+@pytest.mark.parametrize("metric,mname", METRICS)
+@pytest.mark.parametrize("d,pq_dim", [(128, 128), (64, 32), (62, 31), (96, 8)])
+def test_pqfs_lists_on_the_matrix_cores_equal_the_streaming_scan(lib, metric, mname, d, pq_dim):
+    """A large batch sends the probe columns behind the first through the int8 matrix cores (one-hot centroid indices
+    against the byte tables, ivf_pq.hip): ids and distance bits must be the streaming kernel's, and the checker's on
+    a sample.  Lists shorter than the candidate count (queries without a bound overflow into the streaming fallback),
+    missing buckets and a list probed twice are part of the batch."""
+    L = lib.load_library()
+    rng = np.random.default_rng(d + pq_dim + metric)
+    n, nlist, nprobe, nq, kcand = 150000, 256, 12, 3000, 40
+    x, means = gaussian_mixture(rng, n, d, 200, 0.08)
+    q, _ = gaussian_mixture(rng, nq, d, 200, 0.08, means=means)
+    cb = orc.pq_train(x[:4000], pq_dim, metric)
+    codes = orc.pq_encode(x, pq_dim, cb, metric)
+    labels = rng.integers(0, nlist, n).astype(np.int32)
+    labels[labels < 3] = 3 + rng.integers(0, nlist - 3, int((labels < 3).sum()))  # lists 0..2: nearly empty
+    labels[:20] = 0
+    labels[20:25] = 1
+    buckets = np.stack([rng.permutation(nlist)[:nprobe] for _ in range(nq)]).astype(np.int32)
+    buckets[:200, 0] = rng.integers(0, 3, 200)   # a first list that leaves no bound
+    buckets[200:300, 5] = -1                     # missing buckets
+    buckets[300:320, 7] = buckets[300:320, 3]    # a list probed twice
+    st = Store(capi.KIND_PQFS, metric, d, pq_dim=pq_dim, codebooks=cb)
+    st.set_lists(codes, labels, nlist)
+    fast = st.ivf_scan(q, buckets, kcand)
+    info = C.c_int()
+    L.vsag_amd_last_scan_info(C.byref(info), None, None)
+    assert info.value == 256, "the matrix-core pass over the posting lists did not run"
+    capi.check(L.vsag_amd_store_set_scan_contraction(st.handle, -1))
+    plain = st.ivf_scan(q, buckets, kcand)
+    L.vsag_amd_last_scan_info(C.byref(info), None, None)
+    assert info.value <= 8
+    capi.check(L.vsag_amd_store_set_scan_contraction(st.handle, -2))
+    assert np.array_equal(fast[0], plain[0]) and np.array_equal(fast[1].view(np.uint32), plain[1].view(np.uint32))
+    offsets, order = orc.ivf_build_lists(labels, nlist)
+    sel = np.r_[0:40, 200:240, 300:320, 2900:2940]
+    # the checker keeps what it meets first among equal distances and scans a list probed twice twice
+    sel = sel[~np.isin(sel, np.arange(300, 320))]
+    qc = orc.pqfs_process_query(q[sel], pq_dim, cb, metric)
+    rids, rds = orc.ivf_scan(orc.PQFS, metric, pq_dim, codes[order], offsets, order, qc, buckets[sel], kcand)
+    assert np.array_equal(fast[1][sel].view(np.uint32), rds.view(np.uint32))
+    assert_topk_close(fast[0][sel], fast[1][sel], rids, rds, rtol=0, atol=0, tie_rtol=0, label="pqfs mfma " + mname)
+    # the batch split does not matter
+    for s, e in ((0, 1), (250, 257), (1000, 2024)):
+        ci, cd = st.ivf_scan(q[s:e], buckets[s:e], kcand)
+        assert np.array_equal(ci, fast[0][s:e]) and np.array_equal(cd.view(np.uint32), fast[1][s:e].view(np.uint32)), (s, e)
+    st.destroy()
