@@ -782,14 +782,16 @@ def run_c4(env):
         # The probe columns behind the first went through the int8 matrix cores; the timed kernel is that pass alone:
         # every code of those lists against every query probing them, 2 x 128 integer operations per pair.
         rest = sizes[b[:, 1:].clip(0)].astype(np.int64).sum() - (b[:, 1:] < 0).sum() * int(sizes[0])
-        ops = 2.0 * (-(-d // 32) * 32) * float(rest)
+        # (pqfs: a pair is a contraction of the one-hot centroid indices with the byte table, 16 products per subspace)
+        ops = 2.0 * (16 * (-(-pq_dim // 32) * 32) if pqfs else -(-d // 32) * 32) * float(rest)
         tops = ops / (kms * 1e-3) / 1e12
         roof = {"bound": "mfma", "achieved": tops, "peak": MFMA_I8_PEAK_TOPS, "unit": "TOP/s",
                 "frac": tops / MFMA_I8_PEAK_TOPS,
                 # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this launch: profiles/ivf_i8_sq4u_c4.md
                 "traffic": 491061.0 * 2.00 * 1024 + 73550.7 * 1024
                 if (n, d, nq, k, nlist, bits) == (10000000, 128, 10000, 10, 4096, 4) else None,
-                "kernel": "%s<%s> (int8 MFMA, probe columns 1..%d)" % ("prefilter_rb_kernel<lists>" if one_bit else
+                "kernel": "%s<%s> (int8 MFMA, probe columns 1..%d)" % ("ivf_pq_kernel" if pqfs else
+                                                                        "prefilter_rb_kernel<lists>" if one_bit else
                                                                         "ivf_sq8_i8_kernel" if per_dim else "ivf_i8_kernel",
                                                                         kind_name, nprobe - 1), "kernel_ms": kms,
                 "ops_per_launch": ops, "distance_evaluations_per_launch": float(rest),

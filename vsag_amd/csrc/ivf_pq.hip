@@ -16,7 +16,7 @@
 // Work split (the grouping of ivf_i8.hip): a workgroup is a chunk of a list's tiles and up to 64 of the (query, list)
 // pairs that probe the list.  The tables of its 64 queries stay in LDS for the whole kernel (16 bytes per subspace and
 // query, 128 KB for 128 subspaces), laid out [subspace][query] so that the 32 lanes of an operand read 512 contiguous
-// bytes.  Each of the four waves walks its own tiles: it keeps a tile's code bytes in registers as they lie in the
+// bytes.  Each of the eight waves walks its own tiles: it keeps a tile's code bytes in registers as they lie in the
 // store (a lane per code), swaps the halves it needs with the lane 32 apart, builds the one-hot operands with a shift
 // and four selects per subspace, and meets all 64 queries (four accumulators of 32 x 32).  Candidates of a pair go to
 // one list per chunk through a counter in LDS; a list that overflows raises the query's gate and the streaming kernel
@@ -37,6 +37,7 @@ typedef int intx4 __attribute__((ext_vector_type(4)));
 typedef int intx16 __attribute__((ext_vector_type(16)));
 
 constexpr uint32_t kIvfPqPairs = 64;       // pairs per workgroup
+constexpr uint32_t kIvfPqWaves = 8;        // two per SIMD: one waits for its table rows while the other multiplies
 constexpr uint32_t kIvfPqMaxSubspaces = 128;
 constexpr uint32_t kIvfPqChunkTiles = 32;  // as ivf_i8.hip: kIvfI8ChunkTiles, kIvfI8Chunks
 constexpr uint32_t kIvfPqChunks = 4;
@@ -115,7 +116,7 @@ pq_one_hot(uint32_t nib) {
 }
 
 template <int METRIC>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(kIvfPqWaves * kWave)
 ivf_pq_kernel(IvfPqArgs p) {
     extern __shared__ uint4 lut[];  // [subspace][kIvfPqPairs]
     __shared__ uint32_t cnt[kIvfPqPairs];
@@ -157,7 +158,9 @@ ivf_pq_kernel(IvfPqArgs p) {
     }
     const uint32_t pbeg = as_const(p.pair_off)[b] + group * kIvfPqPairs;
     const uint32_t pend = as_const(p.pair_off)[b + 1];
-    const uint32_t nsteps = (p.pq_dim + 1) / 2;  // matrix steps: two subspaces each
+    // Matrix steps, two subspaces each: whole granules (a granule's 16 bytes are 16 steps), so that the loop over a
+    // granule has no branch in it; the tables are zero behind the last subspace and so are the codes' indices.
+    const uint32_t nsteps = 16 * p.G;
 
     // The tables of the workgroup's queries into LDS, staged signed; zero behind the last subspace.
     {
@@ -172,7 +175,7 @@ ivf_pq_kernel(IvfPqArgs p) {
         }
         const uint4* row = reinterpret_cast<const uint4*>(p.qtab + static_cast<uint64_t>(q) * p.qstride);
         const uint32_t flip = METRIC == VSAG_AMD_METRIC_L2 ? 0x7F7F7F7FU : 0x80808080U;
-        for (uint32_t sub = tid / kIvfPqPairs; sub < 2 * nsteps; sub += 256 / kIvfPqPairs) {
+        for (uint32_t sub = tid / kIvfPqPairs; sub < 2 * nsteps; sub += kIvfPqWaves * kWave / kIvfPqPairs) {
             uint4 v = make_uint4(0, 0, 0, 0);
             if (sub < p.pq_dim) {
                 v = row[sub];
@@ -191,7 +194,7 @@ ivf_pq_kernel(IvfPqArgs p) {
         tq[j] = p.tq[pair[j] != 0xFFFFFFFFU ? pair[j] / p.nprobe : p.dummy_query];
     }
 
-    // A wave's tiles: tile_begin + wave, + 4, ...; the code bytes of the next tile are fetched while this one is met.
+    // A wave's tiles: tile_begin + wave, + 8, ...; the code bytes of the next tile are fetched while this one is met.
     uint4 cw[4], nw[4];
     auto fetch = [&](uint32_t tile, uint4(&regs)[4]) {
 #pragma unroll
@@ -203,8 +206,8 @@ ivf_pq_kernel(IvfPqArgs p) {
         }
     };
     fetch(tile_begin + wave, cw);
-    for (uint32_t tile = tile_begin + wave; tile < tile_end; tile += 4) {
-        fetch(tile + 4, nw);
+    for (uint32_t tile = tile_begin + wave; tile < tile_end; tile += kIvfPqWaves) {
+        fetch(tile + kIvfPqWaves, nw);
         intx16 acc[2][2];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -218,15 +221,12 @@ ivf_pq_kernel(IvfPqArgs p) {
         }
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            if (16U * g >= nsteps) {
+            if (static_cast<uint32_t>(g) >= p.G) {
                 break;
             }
             const uint32_t w4[4] = {cw[g].x, cw[g].y, cw[g].z, cw[g].w};
 #pragma unroll
             for (int m = 0; m < 4; ++m) {
-                if (16U * g + 4U * m >= nsteps) {
-                    break;
-                }
                 // Byte s of a code holds subspaces 2 s (low nibble) and 2 s + 1 (high nibble).  In a matrix step the
                 // lanes below 32 supply subspace 2 s of codes lane and lane + 32, the lanes from 32 on subspace
                 // 2 s + 1 of codes lane - 32 and lane: each takes what it lacks from the lane 32 apart.
@@ -237,9 +237,6 @@ ivf_pq_kernel(IvfPqArgs p) {
 #pragma unroll
                 for (int bb = 0; bb < 4; ++bb) {
                     const uint32_t s = 16U * g + 4U * m + bb;
-                    if (s >= nsteps) {
-                        break;
-                    }
                     const intx4 a0 = pq_one_hot((n0 >> (8 * bb)) & 15U);
                     const intx4 a1 = pq_one_hot((n1 >> (8 * bb)) & 15U);
                     const uint4 t0 = lut[(2 * s + half) * kIvfPqPairs + l32];
@@ -396,8 +393,7 @@ launch_ivf_pq(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     p.partial = partial;
     p.partial_cnt = partial_cnt;
     p.gate = gate;
-    const uint32_t nsteps = (s->pq_dim + 1) / 2;
-    const size_t lds = static_cast<size_t>(2 * nsteps) * kIvfPqPairs * sizeof(uint4);
+    const size_t lds = static_cast<size_t>(32) * s->G * kIvfPqPairs * sizeof(uint4);
     static bool attr_set = false;
     if (!attr_set) {
         const int bytes = static_cast<int>(kIvfPqMaxSubspaces * kIvfPqPairs * sizeof(uint4));
@@ -414,9 +410,9 @@ launch_ivf_pq(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     const dim3 grid(static_cast<uint32_t>(max_items));
     timing_begin(st);
     if (l2) {
-        hipLaunchKernelGGL(ivf_pq_kernel<VSAG_AMD_METRIC_L2>, grid, dim3(256), lds, st, p);
+        hipLaunchKernelGGL(ivf_pq_kernel<VSAG_AMD_METRIC_L2>, grid, dim3(kIvfPqWaves * kWave), lds, st, p);
     } else {
-        hipLaunchKernelGGL(ivf_pq_kernel<VSAG_AMD_METRIC_IP>, grid, dim3(256), lds, st, p);
+        hipLaunchKernelGGL(ivf_pq_kernel<VSAG_AMD_METRIC_IP>, grid, dim3(kIvfPqWaves * kWave), lds, st, p);
     }
     timing_end(st);
     VA_HIP(hipGetLastError());

@@ -856,9 +856,83 @@ carve_update(Carver& c, uint64_t n, uint32_t k, UpdateBuffers* b) {
     return c.used;
 }
 
+// Few, short centroids (the 16 centroids of a product-quantizer subspace): sorting the rows by label and giving a
+// workgroup to each centroid leaves the machine idle.  Instead a workgroup sums a block of 1024 rows per (centroid,
+// dimension) in row order, and a second launch adds the block sums in block order -- the order of the reference's own
+// update, which sums per task of 1024 rows and merges the tasks (kmeans_cluster.cpp:108-154).
+constexpr uint32_t kSmallUpdateRows = 1024;
+
+__global__ void __launch_bounds__(256)
+small_update_partial_kernel(const float* x, const int32_t* labels, uint64_t n, uint32_t dim, uint32_t k, float* psum,
+                            uint32_t* pcount) {
+    __shared__ int32_t lab[kSmallUpdateRows];
+    const uint64_t row0 = static_cast<uint64_t>(blockIdx.x) * kSmallUpdateRows;
+    const uint32_t rows = static_cast<uint32_t>(n - row0 < kSmallUpdateRows ? n - row0 : kSmallUpdateRows);
+    for (uint32_t r = threadIdx.x; r < rows; r += blockDim.x) {
+        lab[r] = labels[row0 + r];
+    }
+    __syncthreads();
+    const uint32_t entries = k * dim;
+    for (uint32_t e = threadIdx.x; e < entries; e += blockDim.x) {
+        const int32_t c = static_cast<int32_t>(e / dim);
+        const uint32_t d = e % dim;
+        const float* col = x + row0 * dim + d;
+        float s = 0.0F;
+        uint32_t cnt = 0;
+        for (uint32_t r = 0; r < rows; ++r) {
+            if (lab[r] == c) {
+                s += col[static_cast<uint64_t>(r) * dim];
+                ++cnt;
+            }
+        }
+        psum[static_cast<uint64_t>(blockIdx.x) * entries + e] = s;
+        if (d == 0) {
+            pcount[static_cast<uint64_t>(blockIdx.x) * k + c] = cnt;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256)
+small_update_final_kernel(const float* psum, const uint32_t* pcount, uint32_t blocks, uint32_t dim, uint32_t k,
+                          float* centroids, int32_t* counts_out) {
+    const uint32_t e = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t entries = k * dim;
+    if (e >= entries) {
+        return;
+    }
+    const uint32_t c = e / dim;
+    float s = 0.0F;
+    uint32_t cnt = 0;
+    for (uint32_t b = 0; b < blocks; ++b) {
+        const uint32_t bc = pcount[static_cast<uint64_t>(b) * k + c];
+        if (bc != 0) {
+            s += psum[static_cast<uint64_t>(b) * entries + e];
+            cnt += bc;
+        }
+    }
+    if (e % dim == 0) {
+        counts_out[c] = static_cast<int32_t>(cnt);
+    }
+    if (cnt != 0) {
+        centroids[e] = s * (1.0F / static_cast<float>(cnt));  // empty clusters keep their centroid
+    }
+}
+
 static int
 update_launch(const float* x, const int32_t* labels, uint64_t n, uint32_t dim, uint32_t k, float* cent,
               int32_t* counts_dev, const UpdateBuffers& b, hipStream_t st) {
+    const uint64_t small_blocks = div_up(n, static_cast<uint64_t>(kSmallUpdateRows));
+    if (k <= 64 && static_cast<uint64_t>(k) * dim <= 512 && small_blocks * k * dim <= n && small_blocks * k <= n) {
+        // the block sums and counts live where the sort of the general path keeps its row lists
+        float* psum = reinterpret_cast<float*>(b.rows_in);
+        uint32_t* pcount = b.rows_out;
+        hipLaunchKernelGGL(small_update_partial_kernel, dim3(static_cast<uint32_t>(small_blocks)), dim3(256), 0, st, x,
+                           labels, n, dim, k, psum, pcount);
+        hipLaunchKernelGGL(small_update_final_kernel, dim3((k * dim + 255) / 256), dim3(256), 0, st, psum, pcount,
+                           static_cast<uint32_t>(small_blocks), dim, k, cent, counts_dev);
+        VA_HIP(hipGetLastError());
+        return 0;
+    }
     uint32_t blocks = static_cast<uint32_t>(div_up(n, 256));
     hipLaunchKernelGGL(fill_u64_kernel, dim3((k / 2 + 1 + 255) / 256), dim3(256), 0, st,
                        reinterpret_cast<unsigned long long*>(b.counts), 0ull, static_cast<uint64_t>(k / 2 + 1));
