@@ -302,12 +302,18 @@ def run_c2(env):
         for _ in range(args.steps):
             aids, adist = index.knn_search_batch(q, k, "{}")
         api_sec = (time.perf_counter() - t0) / args.steps
-        t0 = time.perf_counter()
-        for i in range(200):
-            index.knn_search(q[i % nq], k, "{}")
-        api_one = (time.perf_counter() - t0) / 200
+        # one query per call, the reference evaluator's protocol (tools/eval/case/search_eval_case.cpp:233-277): from
+        # one caller thread, then from as many as the CPU baseline uses, all on the one index
+        index.eval_knn_search(q[:64], k, "{}", 1)
+        e_ids, _, e_sec = index.eval_knn_search(q[:2000], k, "{}", 1)
+        api_one = e_sec / 2000
+        threads = min(os.cpu_count() or 1, 16)
+        index.eval_knn_search(q[:256], k, "{}", threads)
+        c_ids, _, c_sec = index.eval_knn_search(q, k, "{}", threads)
         api = {"qps": nq / api_sec, "ms_per_step": 1e3 * api_sec, "build_seconds": api_build,
                "one_query_per_call_us": 1e6 * api_one,
+               "concurrent_one_query_qps": nq / c_sec, "concurrent_threads": threads,
+               "concurrent_same_ids_as_batch": float(np.mean(c_ids == aids)),
                "same_ids_as_resident_path": float(np.mean(aids - 1000000007 == results["l2"]["ids"])),
                "what": "vsag::Factory::CreateIndex(brute_force, sq8) -> Build(%d x %d host floats) -> KnnSearch(%d host "
                        "queries, k=%d) -> host ids / distances, PCIe copies and label mapping included" % (n, d, nq, k)}

@@ -77,6 +77,13 @@ VSAG_AMD_API int vsag_amd_memory_info(uint64_t* free_bytes, uint64_t* total_byte
 VSAG_AMD_API int vsag_amd_memcpy_h2d(void* dst_dev, const void* src, size_t bytes, void* stream);
 VSAG_AMD_API int vsag_amd_memcpy_d2h(void* dst, const void* src_dev, size_t bytes, void* stream);
 VSAG_AMD_API int vsag_amd_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
+/* Pinned host memory (hipHostMalloc) and the two host copies without their wait: a search that stages its queries
+ * and results through pinned buffers needs one vsag_amd_stream_synchronize, at its end.  With pageable host memory
+ * the copies are still correct, but may block. */
+VSAG_AMD_API int vsag_amd_host_malloc(void** ptr, size_t bytes);
+VSAG_AMD_API int vsag_amd_host_free(void* ptr);
+VSAG_AMD_API int vsag_amd_memcpy_h2d_async(void* dst_dev, const void* src, size_t bytes, void* stream);
+VSAG_AMD_API int vsag_amd_memcpy_d2h_async(void* dst, const void* src_dev, size_t bytes, void* stream);
 VSAG_AMD_API int vsag_amd_memset(void* dst_dev, int value, size_t bytes, void* stream);
 VSAG_AMD_API int vsag_amd_stream_synchronize(void* stream);
 /* A stream of default priority that does not synchronise with the null stream: one per concurrent search. */

@@ -394,4 +394,14 @@ def test_concurrent_searches_equal_serial(lib, name, params, search):
         th.join(timeout=100)
     assert not any(th.is_alive() for th in pool)
     assert not errors, errors[:5]
+    # The evaluator's loop natively (tools/eval/case/search_eval_case.cpp:233-277): sixteen caller threads, one query per
+    # call; calls that meet are served as one device batch and must still return the single-query results, also with
+    # another k and other parameters in between, and short rows (k above what a probe can return) as short rows.
+    for t in (1, threads):
+        ids, dists, seconds = idx.eval_knn_search(q, k, search, t)
+        assert np.array_equal(ids, want_ids) and np.array_equal(dists, want_d) and seconds > 0
+    ids3, dists3, _ = idx.eval_knn_search(q[:64], 3, search, threads)
+    assert np.array_equal(ids3, want_ids[:64, :3]) and np.array_equal(dists3, want_d[:64, :3])
+    one_i, one_d = idx.knn_search(q[5], k, search, statistics=False)
+    assert np.array_equal(one_i, want_ids[5]) and np.array_equal(one_d, want_d[5])
     idx.close()

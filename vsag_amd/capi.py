@@ -53,6 +53,10 @@ PROTOTYPES = {
     "vsag_amd_memcpy_h2d": (C.c_int, [_vp, _vp, _sz, _vp]),
     "vsag_amd_memcpy_d2h": (C.c_int, [_vp, _vp, _sz, _vp]),
     "vsag_amd_memcpy_d2d": (C.c_int, [_vp, _vp, _sz, _vp]),
+    "vsag_amd_host_malloc": (C.c_int, [C.POINTER(_vp), _sz]),
+    "vsag_amd_host_free": (C.c_int, [_vp]),
+    "vsag_amd_memcpy_h2d_async": (C.c_int, [_vp, _vp, _sz, _vp]),
+    "vsag_amd_memcpy_d2h_async": (C.c_int, [_vp, _vp, _sz, _vp]),
     "vsag_amd_memset": (C.c_int, [_vp, C.c_int, _sz, _vp]),
     "vsag_amd_memory_info": (C.c_int, [_vp, _vp, _vp, C.c_int]),
     "vsag_amd_stream_synchronize": (C.c_int, [_vp]),

@@ -236,6 +236,49 @@ vsag_amd_memcpy_d2h(void* dst, const void* src_dev, size_t bytes, void* stream) 
     return 0;
 }
 
+// Pinned host memory (allocated, never registered) and copies that do not wait: what a serving loop stages its
+// queries and results through, with one vsag_amd_stream_synchronize per search.
+extern "C" int
+vsag_amd_host_malloc(void** ptr, size_t bytes) {
+    VA_TRY(ensure_init());
+    VA_CHECK_ARG(ptr != nullptr, "ptr is null");
+    *ptr = nullptr;
+    if (bytes == 0) {
+        return 0;
+    }
+    VA_HIP(hipHostMalloc(ptr, bytes, hipHostMallocDefault));
+    return 0;
+}
+
+extern "C" int
+vsag_amd_host_free(void* ptr) {
+    if (ptr == nullptr) {
+        return 0;
+    }
+    VA_HIP(hipHostFree(ptr));
+    return 0;
+}
+
+extern "C" int
+vsag_amd_memcpy_h2d_async(void* dst_dev, const void* src, size_t bytes, void* stream) {
+    VA_TRY(ensure_init());
+    if (bytes == 0) {
+        return 0;
+    }
+    VA_HIP(hipMemcpyAsync(dst_dev, src, bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)));
+    return 0;
+}
+
+extern "C" int
+vsag_amd_memcpy_d2h_async(void* dst, const void* src_dev, size_t bytes, void* stream) {
+    VA_TRY(ensure_init());
+    if (bytes == 0) {
+        return 0;
+    }
+    VA_HIP(hipMemcpyAsync(dst, src_dev, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
+    return 0;
+}
+
 extern "C" int
 vsag_amd_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream) {
     VA_TRY(ensure_init());

@@ -2,6 +2,10 @@
 #include "vsag_host_c_api.h"
 
 #include <algorithm>
+#include <atomic>
+#include <chrono>
+#include <thread>
+#include <vector>
 #include <functional>
 #include <cstdio>
 #include <cstring>
@@ -215,6 +219,62 @@ vsag_index_knn_search_batch(vsag_index_t index, const float* queries, uint64_t n
         *result_dim = cols;
     }
     return success();
+}
+
+extern "C" Error_t
+vsag_index_eval_knn_search(vsag_index_t index, const float* queries, uint64_t nq, uint64_t dim, int64_t k,
+                           const char* parameters, int threads, int64_t* ids, float* dists, double* seconds) {
+    auto* vi = static_cast<VsagIndex*>(index);
+    if (vi == nullptr) {
+        return make_error(VSAG_UNKNOWN_ERROR, "index is NULL");
+    }
+    if (ids == nullptr || dists == nullptr || queries == nullptr || k <= 0 || threads <= 0) {
+        return make_error(VSAG_INVALID_ARGUMENT, "null array, k or thread count not positive");
+    }
+    const std::string params = parameters ? parameters : "";
+    std::atomic<uint64_t> next{0};
+    std::mutex error_mutex;
+    bool failed = false;
+    vsag::Error first_error(vsag::ErrorType::UNKNOWN_ERROR, "");
+    auto worker = [&]() {
+        for (;;) {
+            const uint64_t i = next.fetch_add(1);
+            if (i >= nq) {
+                return;
+            }
+            auto q = vsag::Dataset::Make();
+            q->Owner(false)->Dim(static_cast<int64_t>(dim))->NumElements(1)->Float32Vectors(queries + i * dim);
+            auto result = vi->index_->KnnSearch(q, k, params);
+            if (!result.has_value()) {
+                std::lock_guard<std::mutex> lock(error_mutex);
+                if (!failed) {
+                    failed = true;
+                    first_error = result.error();
+                }
+                return;
+            }
+            const auto& r = result.value();
+            const int64_t cols = r->GetDim();
+            for (int64_t j = 0; j < k; ++j) {
+                const bool have = r->GetNumElements() > 0 && j < cols;
+                ids[i * k + j] = have ? r->GetIds()[j] : -1;
+                dists[i * k + j] = have ? r->GetDistances()[j] : std::numeric_limits<float>::infinity();
+            }
+        }
+    };
+    const auto t0 = std::chrono::steady_clock::now();
+    std::vector<std::thread> pool;
+    for (int t = 1; t < threads; ++t) {
+        pool.emplace_back(worker);
+    }
+    worker();
+    for (auto& th : pool) {
+        th.join();
+    }
+    if (seconds != nullptr) {
+        *seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    }
+    return failed ? make_error(first_error) : success();
 }
 
 extern "C" int64_t

@@ -6,6 +6,7 @@
 // code and every centroid is computed by libvsag_amd.so.  There is no host arithmetic to fall back to.
 #include <algorithm>
 #include <cmath>
+#include <condition_variable>
 #include <cstring>
 #include <functional>
 #include <istream>
@@ -159,6 +160,11 @@ struct DevBuf {
 // concurrently on one index (SUPPORT_SEARCH_CONCURRENT, bruteforce.cpp:1112-1116, ivf.cpp:498; tools/eval drives one
 // query per call from an OpenMP loop, tools/eval/case/search_eval_case.cpp:233-248): each takes a context from the
 // index's pool and gives it back, so the buffers are reused without being shared.
+//
+// Host data crosses through a pinned staging area of the context: an upload copies into it and queues the transfer
+// without waiting, a download queues the transfer into it and hands the bytes over at finish(), which is the one
+// point where a search waits for the device.  (A copy from or to pageable memory waits on its own, and the caller's
+// arrays cannot be pinned after the fact.)  Transfers too large for the area go the plain, waiting way.
 struct SearchContext {
     void* stream = nullptr;
     DevBuf queries, buckets, bucket_d, cand_ids, cand_d, out_ids, out_d, workspace, deny, scalar;
@@ -170,18 +176,83 @@ struct SearchContext {
     operator=(const SearchContext&) = delete;
     ~SearchContext() {
         if (stream != nullptr) {
+            vsag_amd_stream_synchronize(stream);
             vsag_amd_stream_destroy(stream);
         }
+        vsag_amd_host_free(stage_);
     }
     void
     upload(DevBuf& buf, const void* src, size_t n) {
         buf.reserve(std::max<size_t>(n, 4));
-        dev(vsag_amd_memcpy_h2d(buf.p, src, n, stream));
+        void* s = staged(n);
+        if (s == nullptr) {
+            dev(vsag_amd_memcpy_h2d(buf.p, src, n, stream));
+            return;
+        }
+        std::memcpy(s, src, n);
+        dev(vsag_amd_memcpy_h2d_async(buf.p, s, n, stream));
+    }
+    // The bytes are in `dst` after the next finish().
+    void
+    download_later(void* dst, const void* src_dev, size_t n) {
+        void* s = staged(n);
+        if (s == nullptr) {
+            dev(vsag_amd_memcpy_d2h(dst, src_dev, n, stream));
+            return;
+        }
+        dev(vsag_amd_memcpy_d2h_async(s, src_dev, n, stream));
+        pending_.push_back({dst, s, n});
     }
     void
     download(void* dst, const void* src_dev, size_t n) {
-        dev(vsag_amd_memcpy_d2h(dst, src_dev, n, stream));
+        download_later(dst, src_dev, n);
+        finish();
     }
+    // Waits for everything queued on the stream and hands over the downloads.
+    void
+    finish() {
+        dev(vsag_amd_stream_synchronize(stream));
+        for (const Pending& p : pending_) {
+            std::memcpy(p.dst, p.staged, p.bytes);
+        }
+        pending_.clear();
+        stage_used_ = 0;
+    }
+
+private:
+    struct Pending {
+        void* dst;
+        const void* staged;
+        size_t bytes;
+    };
+    static constexpr size_t kStageLimit = 8u << 20;  // larger transfers are not staged
+    // Room for n bytes in the pinned area (null: too large).  A full area is emptied by finish() first.
+    void*
+    staged(size_t n) {
+        const size_t need = (n + 63) / 64 * 64;
+        if (need > kStageLimit) {
+            return nullptr;
+        }
+        if (stage_used_ + need > stage_cap_) {
+            finish();
+            if (need > stage_cap_) {
+                vsag_amd_host_free(stage_);
+                stage_ = nullptr;
+                stage_cap_ = 0;
+                const size_t cap = std::max<size_t>(need, 1u << 16);
+                void* p = nullptr;
+                dev(vsag_amd_host_malloc(&p, cap));
+                stage_ = static_cast<uint8_t*>(p);
+                stage_cap_ = cap;
+            }
+        }
+        void* s = stage_ + stage_used_;
+        stage_used_ += need;
+        return s;
+    }
+    uint8_t* stage_ = nullptr;
+    size_t stage_cap_ = 0, stage_used_ = 0;
+    std::vector<Pending> pending_;
 };
 
 class ContextPool {
@@ -1239,9 +1310,158 @@ private:
                                "radius(" + std::to_string(spec.radius) + ") must be greater equal than 0");
                 CHECK_ARGUMENT(spec.limited_size != 0, "limited_size(0) must not be equal to 0");
             }
+            if (combinable(query, k, spec)) {
+                return rehome(search_combined(query, k, parameters), allocator_);
+            }
             return rehome(search(query, k, parameters, spec), allocator_);
         });
     }
+
+    // ---- single queries of concurrent callers, combined ---------------------------------------------------------
+    // The reference's evaluator and its users call KnnSearch with one query from many threads
+    // (tools/eval/case/search_eval_case.cpp:233-248).  A device scan of one query leaves most of the machine idle and
+    // a scan of sixteen costs little more, so plain single-query calls that meet here are served together: a caller
+    // that finds no search under way becomes the leader, takes every queued call with its own k and parameters,
+    // runs them as one batch (whose rows equal the single-query results bit for bit) and hands the rows out; calls
+    // that arrive meanwhile queue up for the next leader.  Up to kCombineLeaders batches are under way at a time (each
+    // on a stream of its own), so the device works on one while the host prepares and unpacks others.  A lone caller
+    // pays two uncontended lock operations.
+    // The statistics of a combined call are the batch's, divided evenly among its queries.
+    struct PendingCall {
+        const float* query;
+        int64_t k;
+        const std::string* parameters;
+        DatasetPtr result;
+        std::exception_ptr error;
+        bool taken = false;  // in some leader's batch
+        bool done = false;
+    };
+    mutable std::mutex combine_mutex_;
+    mutable std::condition_variable combine_cv_;
+    mutable std::vector<PendingCall*> combine_queue_;
+    mutable int combine_leaders_ = 0;
+    static constexpr int kCombineLeaders = 3;
+    static constexpr size_t kCombineMax = 64;
+
+    bool
+    combinable(const DatasetPtr& query, int64_t k, const SearchSpec& spec) const {
+        return !spec.range && !spec.valid && spec.bucket_ids == nullptr && query != nullptr &&
+               query->GetNumElements() == 1 && query->GetFloat32Vectors() != nullptr &&
+               query->GetDim() == static_cast<int64_t>(dimension()) && k >= 1 && k <= kMaxDeviceK;
+    }
+
+    // Every integer of a statistics string divided by `parts` (they are all counts of one batch).
+    static std::string
+    divide_counts(const std::string& stats, uint64_t parts) {
+        std::string out;
+        bool quoted = false;
+        for (size_t i = 0; i < stats.size();) {
+            const char c = stats[i];
+            if (c == '"') {
+                quoted = !quoted;
+            }
+            if (!quoted && c >= '0' && c <= '9') {
+                uint64_t v = 0;
+                while (i < stats.size() && stats[i] >= '0' && stats[i] <= '9') {
+                    v = v * 10 + static_cast<uint64_t>(stats[i] - '0');
+                    ++i;
+                }
+                out += std::to_string(v / parts);
+                continue;
+            }
+            out += c;
+            ++i;
+        }
+        return out;
+    }
+
+    DatasetPtr
+    search_combined(const DatasetPtr& query, int64_t k, const std::string& parameters) const {
+        PendingCall mine{query->GetFloat32Vectors(), k, &parameters, nullptr, nullptr, false, false};
+        std::vector<PendingCall*> batch;
+        {
+            std::unique_lock<std::mutex> lock(combine_mutex_);
+            combine_queue_.push_back(&mine);
+            combine_cv_.wait(lock,
+                             [&]() { return mine.done || (!mine.taken && combine_leaders_ < kCombineLeaders); });
+            if (mine.done) {
+                if (mine.error) {
+                    std::rethrow_exception(mine.error);
+                }
+                return mine.result;
+            }
+            ++combine_leaders_;
+            // this call and every queued one with the same k and parameters
+            std::vector<PendingCall*> rest;
+            batch.push_back(&mine);
+            mine.taken = true;
+            for (PendingCall* c : combine_queue_) {
+                if (c == &mine) {
+                    continue;
+                }
+                if (batch.size() < kCombineMax && c->k == k && *c->parameters == parameters) {
+                    c->taken = true;
+                    batch.push_back(c);
+                } else {
+                    rest.push_back(c);
+                }
+            }
+            combine_queue_.swap(rest);
+        }
+        auto release = [&]() {
+            std::lock_guard<std::mutex> lock(combine_mutex_);
+            for (PendingCall* c : batch) {
+                c->done = true;
+            }
+            --combine_leaders_;
+            combine_cv_.notify_all();
+        };
+        try {
+            if (batch.size() == 1) {
+                mine.result = search(query, k, parameters, SearchSpec{});
+            } else {
+                const uint32_t dim = dimension();
+                std::vector<float> rows(batch.size() * dim);
+                for (size_t i = 0; i < batch.size(); ++i) {
+                    std::memcpy(rows.data() + i * dim, batch[i]->query, static_cast<size_t>(dim) * 4);
+                }
+                auto all = Dataset::Make();
+                all->Owner(false)->Dim(dim)->NumElements(static_cast<int64_t>(batch.size()))->Float32Vectors(rows.data());
+                const DatasetPtr found = search(all, k, parameters, SearchSpec{});
+                const std::string stats = divide_counts(found->GetStatistics(), batch.size());
+                const int64_t cols = found->GetDim();
+                const bool none = found->GetNumElements() < static_cast<int64_t>(batch.size());  // an empty index
+                for (size_t i = 0; i < batch.size(); ++i) {
+                    int64_t count = 0;
+                    if (!none) {
+                        const int64_t* ids = found->GetIds() + static_cast<int64_t>(i) * cols;
+                        const float* ds = found->GetDistances() + static_cast<int64_t>(i) * cols;
+                        while (count < cols && !(ids[count] == -1 && std::isinf(ds[count]))) {
+                            ++count;
+                        }
+                        auto* out_ids = new int64_t[std::max<int64_t>(count, 1)];
+                        auto* out_d = new float[std::max<int64_t>(count, 1)];
+                        std::copy(ids, ids + count, out_ids);
+                        std::copy(ds, ds + count, out_d);
+                        auto one = Dataset::Make();
+                        one->NumElements(1)->Dim(count)->Ids(out_ids)->Distances(out_d)->Owner(true)->Statistics(stats);
+                        batch[i]->result = one;
+                    } else {
+                        batch[i]->result = found;
+                    }
+                }
+            }
+        } catch (...) {
+            for (PendingCall* c : batch) {
+                c->error = std::current_exception();
+            }
+            release();
+            throw;
+        }
+        release();
+        return mine.result;
+    }
+
     static SearchSpec
     range_spec(float radius, int64_t limited_size) {
         SearchSpec s;
@@ -1707,7 +1927,7 @@ private:
                                        ctx.out_d.as<float>(), ctx.workspace.p, wsb, ctx.stream));
         ids.resize(static_cast<size_t>(nq) * kk);
         dists.resize(ids.size());
-        ctx.download(ids.data(), ctx.out_ids.p, ids.size() * 4);
+        ctx.download_later(ids.data(), ctx.out_ids.p, ids.size() * 4);
         ctx.download(dists.data(), ctx.out_d.p, dists.size() * 4);
     }
 
@@ -1978,7 +2198,7 @@ protected:
             // routing only: bucket ids + centroid distances (ivf.cpp:1589-1660)
             std::vector<uint32_t> ids(static_cast<size_t>(nq) * nprobe);
             std::vector<float> dists(ids.size());
-            ctx.download(ids.data(), ctx.buckets.p, ids.size() * 4);
+            ctx.download_later(ids.data(), ctx.buckets.p, ids.size() * 4);
             ctx.download(dists.data(), ctx.bucket_d.p, dists.size() * 4);
             std::vector<int64_t> identity(nlist_);
             for (uint32_t i = 0; i < nlist_; ++i) {
@@ -2494,7 +2714,7 @@ private:
           std::vector<float>& dists) {
         ids.resize(count);
         dists.resize(count);
-        ctx.download(ids.data(), ids_dev.p, count * 4);
+        ctx.download_later(ids.data(), ids_dev.p, count * 4);
         ctx.download(dists.data(), d_dev.p, count * 4);
     }
 

@@ -98,6 +98,12 @@ VSAG_HOST_API void vsag_search_result_destroy_statistics(SearchResult_t* search_
  * index made with the same parameters. */
 VSAG_HOST_API Error_t vsag_serialize_file(vsag_index_t index, const char* file_path);
 VSAG_HOST_API Error_t vsag_deserialize_file(vsag_index_t index, const char* file_path);
+/* Addition: the search loop of the reference's evaluator (tools/eval/case/search_eval_case.cpp:233-277): one query
+ * per KnnSearch call, the queries handed out dynamically to `threads` caller threads that share the index; ids and
+ * distances as vsag_index_knn_search_batch writes them, the wall-clock seconds of the loop in *seconds. */
+VSAG_HOST_API Error_t vsag_index_eval_knn_search(vsag_index_t index, const float* queries, uint64_t nq, uint64_t dim,
+                                                 int64_t k, const char* parameters, int threads, int64_t* ids,
+                                                 float* dists, double* seconds);
 VSAG_HOST_API int64_t vsag_index_get_num_elements(vsag_index_t index);
 /* Number of ids the last build / add on this thread could not insert (duplicates). */
 VSAG_HOST_API int64_t vsag_last_failed_id_count(void);

@@ -75,6 +75,9 @@ def _load():
         lib.vsag_index_knn_search_batch.restype = ErrorT
         lib.vsag_index_knn_search_batch.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint64, C.c_int64,
                                                     C.c_char_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_int64)]
+        lib.vsag_index_eval_knn_search.restype = ErrorT
+        lib.vsag_index_eval_knn_search.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint64, C.c_int64, C.c_char_p,
+                                                   C.c_int, C.c_void_p, C.c_void_p, C.POINTER(C.c_double)]
         lib.vsag_index_search_buckets.restype = ErrorT
         lib.vsag_index_search_buckets.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint64, C.c_int64, C.c_char_p,
                                                   C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_int64)]
@@ -215,6 +218,18 @@ class Index:
                                                  flat.ctypes.data, offsets.ctypes.data,
                                                  ids.ctypes.data, dists.ctypes.data, C.byref(rdim)))
         return ids, dists
+
+    def eval_knn_search(self, vectors, k, parameters, threads):
+        """The reference evaluator's loop (tools/eval/case/search_eval_case.cpp:233-277): one query per KnnSearch call
+        from `threads` caller threads on this index.  Returns (ids, distances, wall seconds of the loop)."""
+        q = np.ascontiguousarray(vectors, np.float32)
+        nq, dim = q.shape
+        ids = np.empty((nq, k), np.int64)
+        dists = np.empty((nq, k), np.float32)
+        seconds = C.c_double()
+        _check(_load().vsag_index_eval_knn_search(self._h, q.ctypes.data, nq, dim, k, parameters.encode(), int(threads),
+                                                  ids.ctypes.data, dists.ctypes.data, C.byref(seconds)))
+        return ids, dists, seconds.value
 
     def serialize(self, path):
         """The index as one file in the reference's stream layout (cells of codes, quantizer state, labels, footer)."""
