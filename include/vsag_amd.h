@@ -113,8 +113,13 @@ VSAG_AMD_API int vsag_amd_sq_train_uniform(const float* x_dev, uint64_t n, uint3
 
 /* Bytes per code in the reference's layout (Quantizer::GetCodeSize): fp32 4*dim; sq8 dim; sq4
  * ceil(dim/2) (scalar_quantizer.cpp:28-36); uniform kinds sq4_uniform_quantizer.cpp:33-72 and
- * sq8_uniform_quantizer.cpp:30-62; rabitq 1-bit base rabitq_quantizer.cpp:102-133.  (pqfs: ceil(pq_dim / 2),
- * pq_fastscan_quantizer.cpp:38 -- it depends on pq_dim, not on dim: call it with dim = pq_dim.) */
+ * sq8_uniform_quantizer.cpp:30-62; rabitq rabitq_quantizer.cpp:102-133.  (pqfs: ceil(pq_dim / 2),
+ * pq_fastscan_quantizer.cpp:38 -- it depends on pq_dim, not on dim: call it with dim = pq_dim.)
+ *
+ * Every `query_bits` / `rabitq_query_bits` argument of this header is a bits word: rabitq_bits_per_dim_query (4 or 32)
+ * plus 256 * rabitq_bits_per_dim_base for multi-bit base codes (2..8 bits, fp32 queries only; 0 in the second byte
+ * means 1 bit). */
+#define VSAG_AMD_RABITQ_BITS(query_bits, base_bits) ((query_bits) | ((base_bits) > 1 ? (base_bits) << 8 : 0))
 VSAG_AMD_API uint64_t vsag_amd_code_size(int kind, int metric, uint32_t dim, int rabitq_query_bits);
 
 /* ScalarQuantizer::EncodeBatch (scalar_quantizer.cpp:85-112): fp32 rows -> sq8 / sq4 codes in the
@@ -139,8 +144,16 @@ VSAG_AMD_API int vsag_amd_rabitq_train(const float* x_dev, uint64_t n, uint32_t 
 VSAG_AMD_API int vsag_amd_rabitq_encode(const float* x_dev, uint64_t n, uint32_t dim, const float* rotation_dev,
                            const float* centroid_dev, int metric, int query_bits, uint8_t* codes_dev,
                            void* stream);
+/* RaBitQuantizer::EncodeOneInternal, multi-bit base (rabitq_quantizer.cpp:774-809; bits_word =
+ * VSAG_AMD_RABITQ_BITS(32, 2..8)): n x code_size codes [bit planes, plane b = bit b of every dimension (PackIntoPlanes,
+ * :431-453) | norm of the centred code | norm | error | raw norm (ip, cosine)].  fast_encode chooses FastEncodeRaBitQ
+ * (:609-704, the reference's default, fast_encode_rounds 1..32) over EncodeExtendRaBitQ (:455-607). */
+VSAG_AMD_API int vsag_amd_rabitq_encode_multibit(const float* x_dev, uint64_t n, uint32_t dim, const float* rotation_dev,
+                                    const float* centroid_dev, int metric, int bits_word, int fast_encode,
+                                    uint32_t fast_encode_rounds, uint8_t* codes_dev, void* stream);
 /* RaBitQuantizer::ProcessQueryImpl (rabitq_quantizer.cpp:2130-2217): nq x query_code_size processed
- * queries (4-bit: four bit planes of aligned_dim/8 bytes, lb, delta, code sum, norm, raw norm). */
+ * queries (4-bit: four bit planes of aligned_dim/8 bytes, lb, delta, code sum, norm, raw norm; fp32: the values, their
+ * sum where the base code is multi-bit, norm, raw norm). */
 VSAG_AMD_API uint64_t vsag_amd_rabitq_query_code_size(uint32_t dim, int metric, int query_bits);
 VSAG_AMD_API int vsag_amd_rabitq_process_query(const float* q_dev, uint64_t nq, uint32_t dim,
                                   const float* rotation_dev, const float* centroid_dev, int metric,
@@ -186,7 +199,7 @@ typedef struct vsag_amd_store_params {
     const float* diff_dev;        /* sq8/sq4: dim floats.  otherwise NULL. */
     const float* rotation_dev;    /* rabitq: dim x dim row-major.  otherwise NULL. */
     const float* centroid_dev;    /* rabitq: dim floats (already rotated). */
-    int rabitq_query_bits;        /* rabitq: 4 or 32 (only 4 is scanned on the device). */
+    int rabitq_query_bits;        /* rabitq: the bits word, VSAG_AMD_RABITQ_BITS(4 | 32, base bits); 0 = 4-bit queries. */
     uint32_t pq_dim;              /* pqfs: number of subspaces (divides dim, at most 1024). */
     const float* codebooks_dev;   /* pqfs: pq_dim x 16 x (dim / pq_dim) floats. */
 } vsag_amd_store_params_t;

@@ -230,10 +230,14 @@ uniform_layout(uint64_t dim, int bits, int metric) {
     return l;
 }
 
-// ---------------------------------------------------------------- RaBitQ (1-bit base)
-// rabitq_quantizer.cpp:102-176: field offsets of the base code and of the processed query.
+// ---------------------------------------------------------------- RaBitQ
+// rabitq_quantizer.cpp:102-176: field offsets of the base code and of the processed query ("standard" version: no
+// PCA, no MRQ term, no split storage).  Every function below that takes `query_bits` reads the bits per dimension
+// of the base code from its second byte: query_bits = 4 or 32, plus 256 * base_bits (0 stands for 1 bit).
 struct RabitqLayout {
     uint64_t dim;
+    int base_bits;
+    uint64_t offset_norm_code;  // base_bits != 1 only
     uint64_t offset_norm, offset_error, offset_sum, offset_raw_norm, code_size;
     bool has_sum, has_raw_norm;
     uint64_t aligned_dim, plane_bytes;
@@ -244,8 +248,14 @@ inline RabitqLayout
 rabitq_layout(uint64_t dim, int metric, int query_bits) {
     RabitqLayout l{};
     l.dim = dim;
+    l.base_bits = (query_bits >> 8) == 0 ? 1 : (query_bits >> 8);
+    query_bits &= 255;
     const uint64_t a = 4;
-    uint64_t cs = align_up((dim + 7) / 8, a);
+    uint64_t cs = align_up((dim + 7) / 8 * l.base_bits, a);
+    if (l.base_bits != 1) {
+        l.offset_norm_code = cs;
+        cs += 4;
+    }
     l.offset_norm = cs;
     cs += 4;
     l.offset_error = cs;
@@ -274,6 +284,10 @@ rabitq_layout(uint64_t dim, int metric, int query_bits) {
         qs += 4;
     } else {
         qs = align_up(4 * dim, a);
+        if (l.base_bits != 1) {
+            l.q_offset_sum = qs;
+            qs += 4;
+        }
     }
     l.q_offset_norm = qs;
     qs += 4;
@@ -323,6 +337,261 @@ rabitq_sq4u_binary_ip(const uint8_t* planes, const uint8_t* bits, uint64_t dim) 
         r += cnt << b;
     }
     return r;
+}
+
+// src/simd/generic.cpp:799-811
+inline float
+rabitq_float_sq_ip(const float* v, const uint8_t* codes, uint64_t dim) {
+    float r = 0.0F;
+    for (uint64_t d = 0; d < dim; ++d) {
+        r += static_cast<float>(codes[d]) * v[d];
+    }
+    return r;
+}
+
+// src/simd/generic.cpp:743-771 as RaBitQFloatSQIPByPlanes calls it without split storage (rabitq_quantizer.cpp:354-374):
+// plane b of ceil(dim / 8) bytes holds bit b of every dimension's code (PackIntoPlanes, :431-453); the top plane is
+// the "one bit" code, the planes below it the supplement.
+inline float
+rabitq_float_planes_ip(const float* v, const uint8_t* planes, uint64_t dim, int base_bits) {
+    if (dim == 0) {
+        return 0.0F;
+    }
+    const uint64_t plane_bytes = (dim + 7) / 8;
+    const uint32_t supplement_bits = static_cast<uint32_t>(base_bits - 1);
+    const uint8_t* one_bit = planes + supplement_bits * plane_bytes;
+    float r = 0.0F;
+    for (uint64_t d = 0; d < dim; ++d) {
+        const uint64_t byte = d >> 3;
+        const uint8_t mask = static_cast<uint8_t>(1U << (d & 7));
+        uint32_t code = (one_bit[byte] & mask) != 0 ? 1U << supplement_bits : 0U;
+        for (uint32_t bit = 0; bit < supplement_bits; ++bit) {
+            if ((planes[bit * plane_bytes + byte] & mask) != 0) {
+                code += 1U << bit;
+            }
+        }
+        r += v[d] * static_cast<float>(code);
+    }
+    return r;
+}
+
+// rabitq_quantizer.cpp:256-267
+inline float
+ip_obar_q(float ip_yu_q, float q_prime_sum, float y_norm, int bits) {
+    const float c = 0.5F * static_cast<float>((1U << bits) - 1U);
+    if (y_norm <= 0.0F) {
+        return 0.0F;
+    }
+    float ret = ip_yu_q - c * q_prime_sum;
+    ret /= y_norm;
+    return ret;
+}
+
+// RaBitQuantizer::FastEncodeRaBitQ (rabitq_quantizer.cpp:609-704): a floor grid over [-max|o|, max|o|], then rounds of
+// one-level moves per coordinate that raise <o, y>^2 / |y|^2 (y = code - centre), all sums in double.
+inline void
+rabitq_fast_encode(const float* o, uint64_t dim, int bits, uint64_t rounds, uint8_t* code, float* y_norm) {
+    constexpr double adjustment_epsilon = 1e-8;
+    const uint32_t code_max = (1U << bits) - 1U;
+    const double center = 0.5 * static_cast<double>(code_max);
+    double max_abs = 0.0;
+    for (uint64_t d = 0; d < dim; ++d) {
+        max_abs = std::max(max_abs, std::fabs(static_cast<double>(o[d])));
+    }
+    if (max_abs <= 0.0) {
+        for (uint64_t d = 0; d < dim; ++d) {
+            code[d] = static_cast<uint8_t>(code_max / 2U);
+        }
+        *y_norm = 1.0F;
+        return;
+    }
+    const double delta = 2.0 * max_abs / static_cast<double>(code_max + 1U);
+    const double inv_delta = 1.0 / delta;
+    double ip = 0.0, norm_sqr = 0.0;
+    for (uint64_t d = 0; d < dim; ++d) {
+        const double scaled = (static_cast<double>(o[d]) + max_abs) * inv_delta;
+        int64_t q = static_cast<int64_t>(std::floor(scaled));
+        q = std::min<int64_t>(std::max<int64_t>(q, 0), code_max);
+        code[d] = static_cast<uint8_t>(q);
+        const double centered = static_cast<double>(q) - center;
+        ip += static_cast<double>(o[d]) * centered;
+        norm_sqr += centered * centered;
+    }
+    auto score = [](double inner, double squared) { return squared > 0.0 ? inner * inner / squared : 0.0; };
+    for (uint64_t round = 0; round < rounds; ++round) {
+        bool adjusted = false;
+        for (uint64_t d = 0; d < dim; ++d) {
+            const int32_t cur = code[d];
+            const double cur_value = static_cast<double>(cur) - center;
+            int32_t best_code = cur;
+            double best_ip = ip, best_norm = norm_sqr, best_score = score(ip, norm_sqr);
+            for (int32_t dir = -1; dir <= 1; dir += 2) {
+                const int32_t cand = cur + dir;
+                if (cand < 0 || cand > static_cast<int32_t>(code_max)) {
+                    continue;
+                }
+                const double cand_ip = ip + static_cast<double>(dir) * static_cast<double>(o[d]);
+                if (cand_ip < 0.0) {
+                    continue;
+                }
+                const double cand_norm = norm_sqr + 2.0 * cur_value * static_cast<double>(dir) + 1.0;
+                const double cand_score = score(cand_ip, cand_norm);
+                const double tolerance = adjustment_epsilon * std::max(1.0, std::fabs(best_score));
+                if (cand_score > best_score + tolerance) {
+                    best_code = cand;
+                    best_ip = cand_ip;
+                    best_norm = cand_norm;
+                    best_score = cand_score;
+                }
+            }
+            if (best_code != cur) {
+                code[d] = static_cast<uint8_t>(best_code);
+                ip = best_ip;
+                norm_sqr = best_norm;
+                adjusted = true;
+            }
+        }
+        if (!adjusted) {
+            break;
+        }
+    }
+    norm_sqr = 0.0;
+    for (uint64_t d = 0; d < dim; ++d) {
+        const double centered = static_cast<double>(code[d]) - center;
+        norm_sqr += centered * centered;
+    }
+    *y_norm = static_cast<float>(std::sqrt(norm_sqr));
+    if (!std::isfinite(*y_norm) || *y_norm <= 0.0F) {
+        *y_norm = 1.0F;
+    }
+}
+
+// RaBitQuantizer::EncodeExtendRaBitQ (rabitq_quantizer.cpp:455-607): walks the scale t upwards, one grid step of one
+// coordinate per event (events ordered by (t, coordinate)), keeps the t with the largest <y2, o> / |y2|, then rounds
+// 2 t o to the grid of the parity of 2^bits - 1.
+inline void
+rabitq_extend_encode(const float* o, uint64_t dim, int bits, uint8_t* code, float* y_norm) {
+    constexpr double eps = 1e-12;
+    const int y2_max = static_cast<int>((1U << bits) - 1U);
+    const double c = 0.5 * static_cast<double>(y2_max);
+    const int step = 2;
+    auto clamp_int = [](int x, int lo, int hi) { return x < lo ? lo : (x > hi ? hi : x); };
+    auto round_clamp_parity = [&](double val) {
+        const int lo = -y2_max, hi = +y2_max;
+        const long long r = std::llround(val);
+        const int ri = clamp_int(static_cast<int>(r), lo, hi);
+        if ((ri & 1) == (y2_max & 1)) {
+            return ri;
+        }
+        const int s = (val >= 0.0) ? +1 : -1;
+        int cand = ri + s;
+        if (cand < lo || cand > hi) {
+            cand = ri - s;
+        }
+        return clamp_int(cand, lo, hi);
+    };
+    double max_o = 0.0;
+    for (uint64_t i = 0; i < dim; ++i) {
+        max_o = std::max(max_o, std::fabs(static_cast<double>(o[i])));
+    }
+    if (max_o <= 0.0) {
+        for (uint64_t i = 0; i < dim; ++i) {
+            code[i] = static_cast<uint8_t>(y2_max / 2);
+        }
+        *y_norm = 1.0F;
+        return;
+    }
+    std::vector<int> y2_cur(dim, 0);
+    const double t_end = (static_cast<double>(y2_max) + 2.0) / (2.0 * max_o);
+    double ip_y2_o = 0.0, norm_y2 = 0.0;
+    typedef std::pair<double, size_t> Event;
+    std::priority_queue<Event, std::vector<Event>, std::greater<Event>> pq;
+    auto next_t = [&](size_t i) {
+        const double oi = static_cast<double>(o[i]);
+        if (std::fabs(oi) < 1e-3) {
+            return std::numeric_limits<double>::infinity();
+        }
+        const int sign = (oi > 0.0) ? +1 : -1;
+        const int y2_next = y2_cur[i] + sign * step;
+        if (y2_next < -y2_max || y2_next > +y2_max) {
+            return std::numeric_limits<double>::infinity();
+        }
+        double t = static_cast<double>(y2_cur[i] + sign) / (2.0 * oi);
+        if (t < 0.0) {
+            t = 0.0;
+        }
+        return t;
+    };
+    for (size_t i = 0; i < dim; ++i) {
+        if (static_cast<double>(o[i]) == 0.0) {
+            continue;
+        }
+        const double t0 = next_t(i);
+        if (std::isfinite(t0) && t0 <= t_end) {
+            pq.emplace(t0, i);
+        }
+    }
+    double best_ip = eps, best_t = 0.0;
+    while (!pq.empty()) {
+        const double cur_t = pq.top().first;
+        const size_t k = pq.top().second;
+        pq.pop();
+        if (cur_t >= t_end) {
+            break;
+        }
+        const int sign = (o[k] > 0.0) ? +1 : -1;
+        const int y2_old = y2_cur[k];
+        const int y2_new = y2_old + sign * step;
+        if (y2_new < -y2_max || y2_new > +y2_max) {
+            continue;
+        }
+        y2_cur[k] = y2_new;
+        ip_y2_o += (static_cast<double>(y2_new) - static_cast<double>(y2_old)) * o[k];
+        norm_y2 += static_cast<double>(y2_new) * static_cast<double>(y2_new) -
+                   static_cast<double>(y2_old) * static_cast<double>(y2_old);
+        const double cur_ip = (norm_y2 > 0.0) ? (ip_y2_o / std::sqrt(norm_y2)) : 0.0;
+        if (cur_ip > best_ip) {
+            best_ip = cur_ip;
+            best_t = cur_t;
+        }
+        double t_next = next_t(k);
+        if (t_next <= cur_t) {
+            t_next = std::nextafter(cur_t, std::numeric_limits<double>::infinity());
+        }
+        if (std::isfinite(t_next) && t_next < t_end) {
+            pq.emplace(t_next, k);
+        }
+    }
+    for (size_t i = 0; i < dim; ++i) {
+        const double val = 2.0 * best_t * static_cast<double>(o[i]);
+        const int y2 = round_clamp_parity(val + ((val >= 0) ? eps : -eps));
+        int u = (y2 + y2_max) / 2;
+        u = clamp_int(u, 0, y2_max);
+        code[i] = static_cast<uint8_t>(u);
+    }
+    double sum_y2 = 0.0;
+    for (size_t i = 0; i < dim; ++i) {
+        const double y = static_cast<double>(code[i]) - c;
+        sum_y2 += y * y;
+    }
+    *y_norm = static_cast<float>(std::sqrt(sum_y2));
+    if (!std::isfinite(*y_norm) || *y_norm <= 0.0F) {
+        *y_norm = 1.0F;
+    }
+}
+
+// RaBitQuantizer::PackIntoPlanes (rabitq_quantizer.cpp:431-453), planes in logical order (no split storage).
+inline void
+rabitq_pack_planes(const uint8_t* scalar, uint64_t dim, int bits, uint8_t* planes) {
+    const uint64_t plane_bytes = (dim + 7) / 8;
+    std::memset(planes, 0, plane_bytes * bits);
+    for (uint64_t i = 0; i < dim; ++i) {
+        for (int b = 0; b < bits; ++b) {
+            if ((scalar[i] >> b) & 1U) {
+                planes[b * plane_bytes + (i >> 3)] |= static_cast<uint8_t>(1U << (i & 7));
+            }
+        }
+    }
 }
 
 inline float
@@ -651,12 +920,17 @@ uniform_dist(const Store& s, const uint8_t* qcode, const uint8_t* code) {
     return 1 - result;
 }
 
-// rabitq_quantizer.cpp:1775-1860, 1-bit base and 4-bit or 32-bit query.
+// rabitq_quantizer.cpp:1775-1860: 1-bit base with a 4-bit or 32-bit query, multi-bit base with a 32-bit query.
 inline float
 rabitq_dist(const RabitqLayout& l, int metric, int query_bits, const uint8_t* qcode, const uint8_t* code) {
     float inv_sqrt_d = 1.0F / std::sqrt(static_cast<float>(l.dim));
     float ip_bq;
-    if (query_bits == 4) {
+    query_bits &= 255;
+    if (l.base_bits != 1) {
+        const float query_raw_sum = rd_f32(qcode + l.q_offset_sum);
+        const float ip_yu_q = rabitq_float_planes_ip(reinterpret_cast<const float*>(qcode), code, l.dim, l.base_bits);
+        ip_bq = ip_obar_q(ip_yu_q, query_raw_sum, rd_f32(code + l.offset_norm_code), l.base_bits);
+    } else if (query_bits == 4) {
         std::vector<uint8_t> tmp(l.aligned_dim / 8, 0);
         std::memcpy(tmp.data(), code, l.offset_norm);
         uint32_t ip = g_ref.rabitq_sq4u_ip ? g_ref.rabitq_sq4u_ip(qcode, tmp.data(), l.aligned_dim)
@@ -1087,6 +1361,75 @@ orc_rabitq_encode(const float* data, uint64_t n, uint64_t dim, const float* rot,
     }
 }
 
+// RaBitQuantizer::EncodeOneInternal, multi-bit branch (rabitq_quantizer.cpp:774-809): the scalar code of the rotated,
+// centred, normalised row by FastEncodeRaBitQ or EncodeExtendRaBitQ, packed into bit planes; norm_code = |code - centre|,
+// error = ip_obar_q(<o, code>, sum o, norm_code).  query_bits carries the base bits in its second byte.
+ORC_API void
+orc_rabitq_encode_multibit(const float* data, uint64_t n, uint64_t dim, const float* rot, const float* centroid,
+                           int metric, int query_bits, int fast, uint64_t rounds, uint8_t* codes) {
+    RabitqLayout l = rabitq_layout(dim, metric, query_bits);
+#pragma omp parallel
+    {
+        std::vector<float> t(dim), nd(dim);
+        std::vector<uint8_t> scalar(dim);
+#pragma omp for schedule(static)
+        for (int64_t i = 0; i < static_cast<int64_t>(n); ++i) {
+            const float* x = data + i * dim;
+            uint8_t* c = codes + i * l.code_size;
+            std::memset(c, 0, l.code_size);
+            float raw_norm = 0;
+            if (l.has_raw_norm) {
+                for (uint64_t d = 0; d < dim; ++d) {
+                    raw_norm += x[d] * x[d];
+                }
+            }
+            raw_norm = std::sqrt(raw_norm);
+            rotate(rot, x, t.data(), dim);
+            float norm = normalize_with_centroid(t.data(), centroid, nd.data(), dim);
+            float norm_code = 0;
+            if (fast) {
+                rabitq_fast_encode(nd.data(), dim, l.base_bits, rounds, scalar.data(), &norm_code);
+            } else {
+                rabitq_extend_encode(nd.data(), dim, l.base_bits, scalar.data(), &norm_code);
+            }
+            float query_sum = 0.0F;
+            for (uint64_t d = 0; d < dim; ++d) {
+                query_sum += nd[d];
+            }
+            rabitq_pack_planes(scalar.data(), dim, l.base_bits, c);
+            wr_f32(c + l.offset_norm_code, norm_code);
+            const float scalar_ip = rabitq_float_sq_ip(nd.data(), scalar.data(), dim);
+            const float error = ip_obar_q(scalar_ip, query_sum, norm_code, l.base_bits);
+            wr_f32(c + l.offset_norm, norm);
+            wr_f32(c + l.offset_error, error);
+            if (l.has_raw_norm) {
+                wr_f32(c + l.offset_raw_norm, raw_norm);
+            }
+        }
+    }
+}
+
+ORC_API void
+orc_rabitq_fast_encode(const float* o, uint64_t dim, int bits, uint64_t rounds, uint8_t* code, float* y_norm) {
+    rabitq_fast_encode(o, dim, bits, rounds, code, y_norm);
+}
+ORC_API void
+orc_rabitq_extend_encode(const float* o, uint64_t dim, int bits, uint8_t* code, float* y_norm) {
+    rabitq_extend_encode(o, dim, bits, code, y_norm);
+}
+ORC_API void
+orc_rabitq_pack_planes(const uint8_t* scalar, uint64_t dim, int bits, uint8_t* planes) {
+    rabitq_pack_planes(scalar, dim, bits, planes);
+}
+ORC_API float
+orc_rabitq_float_planes_ip(const float* v, const uint8_t* planes, uint64_t dim, int bits) {
+    return rabitq_float_planes_ip(v, planes, dim, bits);
+}
+ORC_API float
+orc_rabitq_float_sq_ip(const float* v, const uint8_t* codes, uint64_t dim) {
+    return rabitq_float_sq_ip(v, codes, dim);
+}
+
 // RaBitQuantizer::EncodeSQ + ReOrderSQ (rabitq_quantizer.cpp:2049-2088): per-query min/max, round to
 // nearest of 15 levels, then bit b of every dim goes to plane b (planes aligned_dim/8 bytes apart).
 ORC_API void
@@ -1144,7 +1487,7 @@ orc_rabitq_process_query(const float* query, uint64_t dim, const float* rot, con
     raw = std::sqrt(raw);
     rotate(rot, query, t.data(), dim);
     float qnorm = normalize_with_centroid(t.data(), centroid, nd.data(), dim);
-    if (query_bits == 4) {
+    if ((query_bits & 255) == 4) {
         std::vector<uint8_t> quant(dim, 0);
         float ub, lb, delta, qsum;
         orc_rabitq_encode_sq(nd.data(), dim, quant.data(), &ub, &lb, &delta, &qsum);
@@ -1154,6 +1497,13 @@ orc_rabitq_process_query(const float* query, uint64_t dim, const float* rot, con
         wr_f32(qcode + l.q_offset_sum, qsum);
     } else {
         std::memcpy(qcode, nd.data(), dim * sizeof(float));
+    }
+    if (l.base_bits != 1) {
+        float query_raw_sum = 0;
+        for (uint64_t d = 0; d < dim; ++d) {
+            query_raw_sum += nd[d];
+        }
+        wr_f32(qcode + l.q_offset_sum, query_raw_sum);
     }
     wr_f32(qcode + l.q_offset_norm, qnorm);
     if (l.has_raw_norm) {

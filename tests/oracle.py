@@ -35,7 +35,7 @@ def lib():
         _lib.orc_kmeans_run_with.restype = C.c_double
         for name in ("orc_fp32_l2sqr", "orc_fp32_ip", "orc_sq8_ip", "orc_sq8_l2sqr", "orc_sq4_ip", "orc_sq4_l2sqr",
                      "orc_squ_dist", "orc_rabitq_dist", "orc_normalize", "orc_normalize_with_centroid",
-                     "orc_rabitq_float_binary_ip"):
+                     "orc_rabitq_float_binary_ip", "orc_rabitq_float_planes_ip", "orc_rabitq_float_sq_ip"):
             getattr(_lib, name).restype = C.c_float
         for name in ("orc_squ_code_size", "orc_rabitq_code_size", "orc_rabitq_query_code_size"):
             getattr(_lib, name).restype = C.c_uint64
@@ -131,6 +131,58 @@ def rabitq_encode(x, rot, centroid, metric, qbits=4):
     codes = np.zeros((n, rabitq_code_size(d, metric, qbits)), np.uint8)
     lib().orc_rabitq_encode(_p(x), u64(n), u64(d), _p(f32(rot)), _p(f32(centroid)), metric, qbits, _p(codes))
     return codes
+
+
+def rabitq_bits(qbits, base_bits=1):
+    """The `qbits` argument of every rabitq function here: query bits (4 | 32) plus 256 * base bits for multi-bit base
+    codes (rabitq_bits_per_dim_base 2..8, fp32 queries only)."""
+    return qbits if base_bits == 1 else (qbits | (base_bits << 8))
+
+
+def rabitq_encode_multibit(x, rot, centroid, metric, base_bits, fast=True, rounds=6):
+    """RaBitQuantizer::EncodeOneInternal with rabitq_bits_per_dim_base = base_bits (2..8) and fp32 queries."""
+    x = f32(x)
+    n, d = x.shape
+    qbits = rabitq_bits(32, base_bits)
+    codes = np.zeros((n, rabitq_code_size(d, metric, qbits)), np.uint8)
+    lib().orc_rabitq_encode_multibit(_p(x), u64(n), u64(d), _p(f32(rot)), _p(f32(centroid)), metric, qbits,
+                                     1 if fast else 0, u64(rounds), _p(codes))
+    return codes
+
+
+def rabitq_fast_encode(o, bits, rounds=6):
+    o = f32(o)
+    code = np.zeros(o.shape[0], np.uint8)
+    norm = C.c_float()
+    lib().orc_rabitq_fast_encode(_p(o), u64(o.shape[0]), bits, u64(rounds), _p(code), C.byref(norm))
+    return code, norm.value
+
+
+def rabitq_extend_encode(o, bits):
+    o = f32(o)
+    code = np.zeros(o.shape[0], np.uint8)
+    norm = C.c_float()
+    lib().orc_rabitq_extend_encode(_p(o), u64(o.shape[0]), bits, _p(code), C.byref(norm))
+    return code, norm.value
+
+
+def rabitq_pack_planes(scalar, bits):
+    scalar = np.ascontiguousarray(scalar, np.uint8)
+    d = scalar.shape[0]
+    planes = np.zeros((d + 7) // 8 * bits, np.uint8)
+    lib().orc_rabitq_pack_planes(_p(scalar), u64(d), bits, _p(planes))
+    return planes
+
+
+def rabitq_float_planes_ip(v, planes, bits):
+    v = f32(v)
+    return float(lib().orc_rabitq_float_planes_ip(_p(v), _p(np.ascontiguousarray(planes, np.uint8)), u64(v.shape[0]),
+                                                  bits))
+
+
+def rabitq_float_sq_ip(v, codes):
+    v = f32(v)
+    return float(lib().orc_rabitq_float_sq_ip(_p(v), _p(np.ascontiguousarray(codes, np.uint8)), u64(v.shape[0])))
 
 
 def rabitq_process_query(q, rot, centroid, metric, qbits=4):
@@ -426,6 +478,8 @@ _REF_SYMBOLS = {
     "SQ8UniformComputeCodesIP": "_ZN4vsag7generic24SQ8UniformComputeCodesIPEPKhS2_m",
     "RaBitQSQ4UBinaryIP": "_ZN4vsag7generic18RaBitQSQ4UBinaryIPEPKhS2_m",
     "RaBitQFloatBinaryIP": "_ZN4vsag7generic19RaBitQFloatBinaryIPEPKfPKhmf",
+    "RaBitQFloatSQIP": "_ZN4vsag7generic15RaBitQFloatSQIPEPKfPKhm",
+    "RaBitQFloatSplitCodeIP": "_ZN4vsag7generic22RaBitQFloatSplitCodeIPEPKfPKhS4_mj",
     "NormalizeWithCentroid": "_ZN4vsag7generic21NormalizeWithCentroidEPKfS2_Pfm",
     "Normalize": "_ZN4vsag7generic9NormalizeEPKfPfm",
 }

@@ -209,6 +209,75 @@ def test_ivf_rabitq_with_reorder(lib, query_bits):
     idx.close()
 
 
+@pytest.mark.parametrize("metric", ["l2", "ip", "cosine"])
+@pytest.mark.parametrize("bits,fast,floor", [(2, True, 0.55), (4, True, 0.85), (8, True, 0.97), (4, False, 0.85)])
+def test_ivf_rabitq_multibit_base_codes(lib, tmp_path, metric, bits, fast, floor):
+    """rabitq_bits_per_dim_base 2..8 (rabitq_quantizer.cpp:774-809,1799-1808) WITHOUT reorder: the recall of the code
+    itself rises with the bits, and 8 bits all but equal the exact search.  Single queries, batches and a reloaded
+    index agree."""
+    n, d, nq, k = 3000, 64, 40, 10
+    x = vectors(n, d)
+    q = vectors(nq, d, seed=165)
+    labels = np.arange(n, dtype=np.int64) + 7
+    idx = make("ivf", d, metric, buckets_count=10, base_quantization_type="rabitq", rabitq_bits_per_dim_base=bits,
+               fast_encode_rabitq=fast, train_sample_count=3000)
+    idx.build(x, labels, n, d)
+    gt, _ = ground_truth(x, q, k, metric)
+    search = json.dumps({"ivf": {"scan_buckets_count": 10}})
+    ids, dists = idx.knn_search_batch(q, k, search)
+    r = recall(ids, gt, labels)
+    assert r >= floor, r
+    one_bit = make("ivf", d, metric, buckets_count=10, base_quantization_type="rabitq", train_sample_count=3000)
+    one_bit.build(x, labels, n, d)
+    ids1, _ = one_bit.knn_search_batch(q, k, search)
+    assert r > recall(ids1, gt, labels)
+    one_bit.close()
+    for i in range(5):
+        sid, sd = idx.knn_search(q[i], k, search)
+        assert np.array_equal(sid, ids[i]) and np.allclose(sd, dists[i], rtol=1e-5, atol=1e-6)
+    path = tmp_path / "multibit.index"
+    idx.serialize(path)
+    again = make("ivf", d, metric, buckets_count=10, base_quantization_type="rabitq", rabitq_bits_per_dim_base=bits,
+                 fast_encode_rabitq=fast, train_sample_count=3000)
+    again.deserialize(path)
+    ids2, dists2 = again.knn_search_batch(q, k, search)
+    assert np.array_equal(ids2, ids) and np.array_equal(dists2, dists)
+    again.close()
+    idx.close()
+
+
+def test_rabitq_multibit_parameters(lib):
+    """RaBitQuantizerParameter::FromJson (rabitq_quantizer_parameter.cpp:30-112) and the constructor
+    (rabitq_quantizer.cpp:67-100): the reference's ranges and messages."""
+    d = 32
+    for extra, text in (({"rabitq_bits_per_dim_base": 0}, "rabitq_bits_per_dim_base in [1, 8], but got 0"),
+                        ({"rabitq_bits_per_dim_base": 9}, "rabitq_bits_per_dim_base in [1, 8], but got 9"),
+                        ({"rabitq_bits_per_dim_base": 4, "rabitq_bits_per_dim_query": 4},
+                         "not support num_bits_per_dim_query_ == 4 with num_bits_per_dim_base_ != 1"),
+                        ({"rabitq_bits_per_dim_base": 4, "fast_encode_rabitq_rounds": 0},
+                         "fast_encode_rabitq_rounds must be in [1, 32], but got 0"),
+                        ({"rabitq_bits_per_dim_base": 4, "fast_encode_rabitq_rounds": 33},
+                         "fast_encode_rabitq_rounds must be in [1, 32], but got 33"),
+                        ({"rabitq_version": "v9"}, "unsupported rabitq_version: v9"),
+                        ({"rabitq_version": "split"}, "split"),
+                        ({"rabitq_error_rate": -1.0}, "rabitq_error_rate must be finite and positive")):
+        with pytest.raises(pyvsag.VsagError) as e:
+            make("ivf", d, "l2", buckets_count=4, base_quantization_type="rabitq", **extra)
+        assert e.value.code == -3 and text in e.value.message, (extra, e.value.message)
+    # brute force takes the same codes
+    n, nq, k = 1500, 20, 10
+    x = vectors(n, d)
+    q = vectors(nq, d, seed=3)
+    labels = np.arange(n, dtype=np.int64)
+    idx = make("brute_force", d, "l2", base_quantization_type="rabitq", rabitq_bits_per_dim_base=8,
+               fast_encode_rabitq_rounds=3)
+    idx.build(x, labels, n, d)
+    gt, _ = ground_truth(x, q, k, "l2")
+    ids, _ = idx.knn_search_batch(q, k, "{}")
+    assert recall(ids, gt, labels) >= 0.97
+    idx.close()
+
+
 # ------------------------------------------------------------------------------------------------------------------
 # Pre-filters and range search, after TestIndex::TestFilterSearch / TestRangeSearch
 # (tests/test_index/test_index_search.cpp:100-160,263-350): filter(label) == True filters the vector out; the range

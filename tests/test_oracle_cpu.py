@@ -222,6 +222,33 @@ def test_rabitq_bit_kernels_match_reference():
         assert abs(n1 - n2) <= 2e-6 * n2 and np.allclose(o1, o2, rtol=2e-6, atol=1e-7)
 
 
+def test_rabitq_multibit_kernels_match_reference():
+    """The bit-plane inner product against the reference's compiled RaBitQFloatSplitCodeIP (generic.cpp:743-771, as
+    RaBitQFloatSQIPByPlanes calls it: top plane = one-bit code, lower planes = supplement) and RaBitQFloatSQIP
+    (:799-811) on the unpacked codes: the two agree by construction in the reference, and so must the restatements."""
+    ref = orc.ref()
+    if ref is None:
+        pytest.skip("oracle/_ref is not built (reference sources not mounted)")
+    rng = np.random.default_rng(744)
+    for d in DIMS:
+        nb = (d + 7) // 8
+        v = rng.standard_normal(d).astype(np.float32)
+        for bits in (2, 3, 4, 5, 8):
+            scalar = rng.integers(0, 1 << bits, d).astype(np.uint8)
+            planes = orc.rabitq_pack_planes(scalar, bits)
+            # plane b holds bit b of every dimension
+            for b in range(bits):
+                want = np.packbits((scalar >> b) & 1, bitorder="little")
+                assert np.array_equal(planes[b * nb:(b + 1) * nb], want)
+            mine = orc.rabitq_float_planes_ip(v, planes, bits)
+            one_bit = np.ascontiguousarray(planes[(bits - 1) * nb:])
+            theirs = ref["RaBitQFloatSplitCodeIP"](_p(v), _p(one_bit), _p(planes), C.c_uint64(d), C.c_uint32(bits - 1))
+            assert mine == theirs
+            sq_mine = orc.rabitq_float_sq_ip(v, scalar)
+            sq_theirs = ref["RaBitQFloatSQIP"](_p(v), _p(scalar), C.c_uint64(d))
+            assert sq_mine == sq_theirs == mine
+
+
 # ------------------------------------------------------------------ closed forms and brute force
 def test_popcount_identity_of_the_binary_ip():
     # sum_b 2^b popcount(plane_b & bits) == sum over set bits of the 4-bit code
@@ -747,3 +774,152 @@ def test_pqfs_distances_meet_the_reference_tests_bound(metric):
         q64 /= np.linalg.norm(q64, axis=1, keepdims=True)
     true = ((q64[:, None] - x64[None]) ** 2).sum(-1) if metric == orc.L2 else 1.0 - q64 @ x64.T
     assert np.abs(got - true).max() <= 0.08, float(np.abs(got - true).max())
+
+
+# ------------------------------------------------------------------ multi-bit RaBitQ (rabitq_bits_per_dim_base 2..8)
+def _alignment(o, code, bits):
+    y = code.astype(np.float64) - 0.5 * ((1 << bits) - 1)
+    ip = float(o.astype(np.float64) @ y)
+    return ip * ip / float(y @ y)
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_rabitq_fast_encode_known_input_of_the_reference_test(bits):
+    """rabitq_quantizer_test.cpp:107-183: on sin(0.37 d) + 0.2 cos(0.11 d), one round is at least as aligned as the
+    floor grid it starts from, six rounds at least as one, codes stay in range, and the norm is |code - centre|."""
+    dgrid = np.arange(64, dtype=np.float32)
+    data = (np.sin(dgrid * np.float32(0.37)) + np.float32(0.2) * np.cos(dgrid * np.float32(0.11))).astype(np.float32)
+    code_max = (1 << bits) - 1
+    max_abs = float(np.abs(data.astype(np.float64)).max())
+    delta = 2.0 * max_abs / (code_max + 1)
+    lvq = np.clip(np.floor((data.astype(np.float64) + max_abs) / delta), 0, code_max).astype(np.uint8)
+    one, _ = orc.rabitq_fast_encode(data, bits, rounds=1)
+    six, norm = orc.rabitq_fast_encode(data, bits, rounds=6)
+    assert _alignment(data, one, bits) + 1e-7 >= _alignment(data, lvq, bits)
+    assert _alignment(data, six, bits) + 1e-7 >= _alignment(data, one, bits)
+    assert six.max() <= code_max and norm > 0
+    y = six.astype(np.float64) - 0.5 * code_max
+    assert abs(norm - np.sqrt(float(y @ y))) <= 1e-5
+    # a fixed point: after convergence no single one-level move raises the alignment by more than the tolerance
+    conv, _ = orc.rabitq_fast_encode(data, bits, rounds=32)
+    base = _alignment(data, conv, bits)
+    for dd in range(64):
+        for step in (-1, 1):
+            c = int(conv[dd]) + step
+            if 0 <= c <= code_max:
+                moved = conv.copy()
+                moved[dd] = c
+                y = moved.astype(np.float64) - 0.5 * code_max
+                if float(data.astype(np.float64) @ y) >= 0:
+                    assert _alignment(data, moved, bits) <= base + 1e-8 * max(1.0, base) + 1e-12
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+def test_rabitq_encoders_against_the_exhaustive_optimum(bits):
+    """rabitq_quantizer_test.cpp:185-226 for the fast encoder (never above the best of all 2^(3 bits) codes).  The
+    extended encoder (rabitq_quantizer.cpp:455-607) walks the scale on the even grid 0, +-2, ... but rounds to the odd
+    one, so it is near the optimum, not at it: within 3 % at 4 bits; at 2 bits the walk is traced by hand below."""
+    import itertools
+    levels = 1 << bits
+    rng = np.random.default_rng(bits)
+    cases = [np.array([0.73, -0.41, 0.19], np.float32)] + [rng.standard_normal(3).astype(np.float32) for _ in range(20)]
+    for data in cases:
+        data = (data / np.linalg.norm(data)).astype(np.float32)
+        best = 0.0
+        for cand in itertools.product(range(levels), repeat=3):
+            y = np.array(cand, np.float64) - 0.5 * (levels - 1)
+            ip = float(data.astype(np.float64) @ y)
+            if ip > 0:
+                best = max(best, ip * ip / float(y @ y))
+        fast, _ = orc.rabitq_fast_encode(data, bits)
+        assert _alignment(data, fast, bits) <= best + 1e-10
+        ext, norm = orc.rabitq_extend_encode(data, bits)
+        y = ext.astype(np.float64) - 0.5 * (levels - 1)
+        assert float(data.astype(np.float64) @ y) > 0
+        if bits == 4 and np.abs(data).min() > 0.05:
+            assert _alignment(data, ext, bits) >= best * 0.97, (data, ext, best)
+        assert abs(norm - np.sqrt(float(y @ y))) <= 1e-5
+    # By hand from the source, 2 bits (y2_max = 3, one event per coordinate at t = 1 / (2 |o|)): events in order
+    # coordinate 1 (t 0.662: <y2, o> / |y2| = 0.755), coordinate 2 (t 0.838: 0.955, the best), coordinate 0 (t 1.83:
+    # 0.938).  At t = 0.838: 2 t o = (0.458, -1.266, -1.000 - eps) -> odd grid (1, -1, -1) -> codes (2, 1, 1), norm
+    # sqrt(0.75).
+    ext, norm = orc.rabitq_extend_encode(np.array([0.2729807, -0.75481445, -0.5964367], np.float32), 2)
+    assert ext.tolist() == [2, 1, 1] and abs(norm - np.sqrt(0.75)) < 1e-6
+    # 3 bits (y2_max = 7, steps to +-2, +-4, +-6 at t = (1, 3, 5) / (2 |o|)) on (0.6, -0.8): events t = 0.625 (c1),
+    # 0.833 (c0), 1.875 (c1), 2.5 (c0), 3.125 (c1), 4.167 (c0) with y2 = (0,-2), (2,-2), (2,-4), (4,-4), (4,-6), (6,-6)
+    # and <y2, o> / |y2| = 0.8, 0.98995, 0.98387, 0.98995, 0.99846 (the best), 0.98995.  At t = 3.125:
+    # 2 t o = (3.75, -5) -> round to (4, -5), 4 is even -> 5 -> odd grid (5, -5) -> codes ((5 + 7) / 2, (-5 + 7) / 2).
+    ext, norm = orc.rabitq_extend_encode(np.array([0.6, -0.8], np.float32), 3)
+    assert ext.tolist() == [6, 1] and abs(norm - np.sqrt(2.5 ** 2 * 2)) < 1e-6
+
+
+def test_rabitq_multibit_zero_vector():
+    """rabitq_quantizer_test.cpp:227-238: a zero vector encodes to code_max / 2 everywhere with norm 1."""
+    for enc in (lambda o: orc.rabitq_fast_encode(o, 8), lambda o: orc.rabitq_extend_encode(o, 8)):
+        code, norm = enc(np.zeros(16, np.float32))
+        assert norm == 1.0 and np.all(code == 127)
+
+
+@pytest.mark.parametrize("fast", [True, False])
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_rabitq_multibit_self_distance_and_accuracy(bits, fast):
+    """rabitq_quantizer_test.cpp:75-105: a query equal to a stored vector is at distance |d| <= 1e-3 (the error field
+    is the same <o, code> the scan computes, so ip_est = 1); and more bits estimate better than fewer."""
+    d, n = 32, 200
+    rng, x, rot, cen = _rabitq_case(900 + bits, d, n, orc.L2, unit=False)
+    qb = orc.rabitq_bits(32, bits)
+    for metric in (orc.L2, orc.IP, orc.COSINE):
+        codes = orc.rabitq_encode_multibit(x, rot, cen, metric, bits, fast=fast)
+        assert codes.shape[1] == orc.rabitq_code_size(d, metric, qb)
+        qcodes = orc.rabitq_process_query(x, rot, cen, metric, qb)
+        for i in range(n):
+            got = _rabitq_dist(qcodes[i], codes[i], d, metric, qb)
+            if metric == orc.L2:
+                assert abs(got) <= 1e-3
+            elif metric == orc.COSINE:
+                assert abs(got) <= 1e-5
+            else:
+                assert abs(got - (1.0 - float((x[i].astype(np.float64) ** 2).sum()))) <= 1e-3 * d
+    # layout: planes, norm_code, norm, error (rabitq_quantizer.cpp:102-133)
+    codes = orc.rabitq_encode_multibit(x, rot, cen, orc.L2, bits, fast=fast)
+    nb = (d + 7) // 8 * bits
+    f = codes[:, nb:].copy().view(np.float32)
+    assert codes.shape[1] == nb + 12
+    assert np.all(f[:, 0] > 0) and np.all(f[:, 1] > 0) and np.all((f[:, 2] > 0.5) & (f[:, 2] <= 1.0 + 1e-6))
+    # error = cos(o, y): closer to 1 with more bits
+    assert f[:, 2].mean() > {2: 0.85, 4: 0.98, 8: 0.9995}[bits]
+    q = rng.standard_normal((30, d)).astype(np.float32)
+    true = ((q[:, None, :].astype(np.float64) - x[None].astype(np.float64)) ** 2).sum(-1)
+    est = orc.flat_dists(orc.RABITQ, orc.L2, d, codes, orc.rabitq_process_query(q, rot, cen, orc.L2, qb), qbits=qb)
+    one = orc.flat_dists(orc.RABITQ, orc.L2, d, orc.rabitq_encode(x, rot, cen, orc.L2, 32),
+                         orc.rabitq_process_query(q, rot, cen, orc.L2, 32), qbits=32)
+    err, err1 = np.abs(est - true).mean(), np.abs(one - true).mean()
+    assert err < err1 * {2: 0.8, 4: 0.3, 8: 0.05}[bits], (err, err1)
+
+
+def test_rabitq_multibit_estimator_closed_form():
+    """ip_obar_q (rabitq_quantizer.cpp:256-267) and the branch at :1799-1808 by hand on a 3-dimensional code: the
+    estimate is (<q, u> - c sum q) / |u - c| / error inside l2_ube.  A dropped centre term, the wrong plane weight or
+    a missing division each change the number."""
+    d, bits = 3, 3
+    rot = np.eye(d, dtype=np.float32)
+    cen = np.zeros(d, np.float32)
+    x = np.array([[3.0, -1.0, 0.5]], np.float32)
+    q = np.array([[1.0, 2.0, -0.5]], np.float32)
+    qb = orc.rabitq_bits(32, bits)
+    code = orc.rabitq_encode_multibit(x, rot, cen, orc.L2, bits, fast=True)[0]
+    qcode = orc.rabitq_process_query(q, rot, cen, orc.L2, qb)[0]
+    planes = code[:3]
+    u = np.array([sum(((int(planes[b]) >> dd) & 1) << b for b in range(bits)) for dd in range(d)], np.float64)
+    c = 0.5 * 7
+    norm_code, norm, error = code[4:16].view(np.float32)
+    o = x[0].astype(np.float64) / np.linalg.norm(x[0])
+    assert abs(norm - np.linalg.norm(x[0])) < 1e-6 and abs(norm_code - np.linalg.norm(u - c)) < 1e-6
+    assert abs(error - float(o @ (u - c)) / np.linalg.norm(u - c)) < 1e-6
+    qn = q[0].astype(np.float64) / np.linalg.norm(q[0])
+    qf = qcode.view(np.float32)
+    assert np.allclose(qf[:3], qn, atol=1e-6) and abs(qf[3] - qn.sum()) < 1e-6 and abs(qf[4] - np.linalg.norm(q[0])) < 1e-6
+    ip_est = (float(qn @ u) - c * qn.sum()) / np.linalg.norm(u - c) / float(error)
+    want = norm ** 2 + np.linalg.norm(q[0]) ** 2 - 2 * norm * np.linalg.norm(q[0]) * ip_est
+    got = _rabitq_dist(qcode, code, d, orc.L2, qb)
+    assert abs(got - want) < 1e-5

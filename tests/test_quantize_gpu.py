@@ -186,3 +186,91 @@ def test_rabitq_flat_scan_fp32_queries(lib, metric, mname, n, d, nq, k):
     # the sum over set bits is taken in another order than the checker's running sum
     assert_topk_close(ids, ds, rids, rds, rtol=1e-4, atol=2e-5, tie_rtol=2e-4, label="rabitq fp32 query " + mname)
     st.destroy()
+
+
+# ------------------------------------------------------------------ multi-bit RaBitQ base codes
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
+@pytest.mark.parametrize("fast", [True, False])
+@pytest.mark.parametrize("bits,n,d", [(2, 700, 128), (4, 500, 128), (8, 300, 128), (3, 200, 15), (4, 150, 200),
+                                      (5, 120, 768), (8, 130, 64)])
+def test_rabitq_multibit_encode_and_query(lib, metric, fast, bits, n, d):
+    """rabitq_bits_per_dim_base 2..8 (rabitq_quantizer.cpp:774-809): FastEncodeRaBitQ / EncodeExtendRaBitQ, bit planes,
+    norm of the code, norm, error -- byte for byte the checker's codes; the processed query carries its sum."""
+    rng = np.random.default_rng(bits * 1000 + d + int(fast))
+    L = lib.load_library()
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    x[3] = 0.0  # a zero row: the centred vector still is not zero, a plain case
+    q = rng.standard_normal((7, d)).astype(np.float32)
+    rot = _rotation(rng, d)
+    cen = orc.rabitq_train(x, rot)
+    word = orc.rabitq_bits(32, bits)
+    ref = orc.rabitq_encode_multibit(x, rot, cen, metric, bits, fast=fast, rounds=6)
+    cs = ref.shape[1]
+    assert cs == L.vsag_amd_code_size(capi.KIND_RABITQ, metric, d, word)
+    xb, rb, cb = dev(x), dev(rot), dev(cen)
+    out = capi.DeviceBuffer(n * cs)
+    capi.check(L.vsag_amd_rabitq_encode_multibit(xb.ptr, n, d, rb.ptr, cb.ptr, metric, word, 1 if fast else 0, 6,
+                                                 out.ptr, None))
+    codes = out.to_numpy(np.uint8, (n, cs))
+    bad = np.flatnonzero((codes != ref).any(axis=1))
+    assert bad.size == 0, (bad[:5], codes[bad[0]], ref[bad[0]])
+
+    qref = orc.rabitq_process_query(q, rot, cen, metric, word)
+    qs = qref.shape[1]
+    assert qs == L.vsag_amd_rabitq_query_code_size(d, metric, word)
+    qb = dev(q)
+    qout = capi.DeviceBuffer(q.shape[0] * qs)
+    capi.check(L.vsag_amd_rabitq_process_query(qb.ptr, q.shape[0], d, rb.ptr, cb.ptr, metric, word, qout.ptr, None))
+    assert np.array_equal(qout.to_numpy(np.uint8, (q.shape[0], qs)), qref)
+
+
+def test_rabitq_multibit_rounds_and_arguments(lib):
+    lib = lib.load_library()
+    rng = np.random.default_rng(77)
+    n, d, bits = 300, 96, 4
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    rot = _rotation(rng, d)
+    cen = orc.rabitq_train(x, rot)
+    word = orc.rabitq_bits(32, bits)
+    xb, rb, cb = dev(x), dev(rot), dev(cen)
+    cs = orc.rabitq_code_size(d, orc.L2, word)
+    out = capi.DeviceBuffer(n * cs)
+    for rounds in (1, 2, 32):
+        capi.check(lib.vsag_amd_rabitq_encode_multibit(xb.ptr, n, d, rb.ptr, cb.ptr, orc.L2, word, 1, rounds, out.ptr, None))
+        assert np.array_equal(out.to_numpy(np.uint8, (n, cs)),
+                              orc.rabitq_encode_multibit(x, rot, cen, orc.L2, bits, fast=True, rounds=rounds))
+    for bad_word, fast, rounds in ((orc.rabitq_bits(4, 4), 1, 6), (32 | (9 << 8), 1, 6), (32 | (1 << 8), 1, 6),
+                                   (word, 1, 0), (word, 1, 33)):
+        assert lib.vsag_amd_rabitq_encode_multibit(xb.ptr, n, d, rb.ptr, cb.ptr, orc.L2, bad_word, fast, rounds, out.ptr,
+                                                   None) == capi.INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("metric,mname", [(orc.L2, "l2"), (orc.IP, "ip"), (orc.COSINE, "cosine")])
+@pytest.mark.parametrize("bits,n,d,nq,k", [(2, 6000, 128, 11, 10), (4, 3000, 128, 70, 10), (8, 2000, 128, 5, 100),
+                                           (4, 900, 768, 5, 50), (3, 300, 15, 3, 7), (5, 1500, 200, 1, 10),
+                                           (8, 500, 960, 9, 20)])
+def test_rabitq_multibit_flat_scan(lib, metric, mname, bits, n, d, nq, k):
+    """Multi-bit codes against fp32 queries (rabitq_quantizer.cpp:1799-1808 over RaBitQFloatSplitCodeIP,
+    generic.cpp:743-771).  Floating point: the device adds the query values plane by plane, the checker dimension by
+    dimension, so distances agree to 1e-4 relative (2e-5 absolute) and ids up to ties of that width."""
+    from gpu_helpers import Store, assert_topk_close
+    lib = lib.load_library()
+    rng = np.random.default_rng(n + d + bits)
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    q = rng.standard_normal((nq, d)).astype(np.float32)
+    rot = _rotation(rng, d)
+    cen = orc.rabitq_train(x, rot)
+    word = orc.rabitq_bits(32, bits)
+    codes = orc.rabitq_encode_multibit(x, rot, cen, metric, bits)
+    qcodes = orc.rabitq_process_query(q, rot, cen, metric, word)
+    st = Store(capi.KIND_RABITQ, metric, d, rot=rot, centroid=cen, qbits=word)
+    assert st.code_size() == codes.shape[1]
+    st.append(codes)
+    # the codes come back out of the tiles as they went in
+    back = capi.DeviceBuffer(codes.size)
+    capi.check(lib.vsag_amd_store_export_codes(st.handle, 0, n, back.ptr, None))
+    assert np.array_equal(back.to_numpy(np.uint8, codes.shape), codes)
+    ids, ds = st.flat_scan(q, k)
+    rids, rds = orc.flat_scan_topk(orc.RABITQ, metric, d, codes, qcodes, k, qbits=word)
+    assert_topk_close(ids, ds, rids, rds, rtol=1e-4, atol=2e-5, tie_rtol=2e-4, label="rabitq %d-bit %s" % (bits, mname))
+    st.destroy()

@@ -42,6 +42,8 @@ struct ScanArgs {
     uint32_t qmeta_stride;
     uint32_t G;
     uint32_t dim;
+    // multi-bit rabitq: granule j belongs to bit plane j / plane_granules ((j * plane_recip) >> 16 for the j in range)
+    uint32_t planes, plane_granules, plane_recip;
     float f0, f1, f2;       // uniform kinds: lb, scalar_rate, lb*lb
 };
 
@@ -51,8 +53,9 @@ struct ScanArgs {
 // Running sums of T queries against the code owned by this lane.
 template <int KIND, int T>
 struct Acc {
-    float f[T];         // fp32 / sq8 / sq4
-    uint32_t lo[T];     // uniform kinds (and plane 0 of rabitq)
+    float f[T];         // fp32 / sq8 / sq4; rabitq with fp32 queries: the sum under the bits of the current plane
+    uint32_t lo[T];     // uniform kinds (and plane 0 of rabitq); multi-bit rabitq: the weighted sum of finished planes
+                        // (float bits)
     uint32_t hi[T];     // sq4_uniform high nibbles (x16); rabitq plane 1
     uint32_t p2[T];     // rabitq plane 2
     uint32_t p3[T];     // rabitq plane 3
@@ -176,7 +179,14 @@ accumulate_granule(const ScanArgs& a, const QueryRows<T>& q, uint32_t j, uint4 c
     } else if constexpr (KIND == kKindRabitqF32) {
         // qtab row: the rotated, centred, normalised query as fp32; a granule holds the bits of 128 dimensions.
         // Sum of the query values under set bits: a sign-extended one-bit extract is an all-ones / all-zeros
-        // mask for the value.
+        // mask for the value.  Multi-bit codes (RaBitQFloatSplitCodeIP, generic.cpp:743-771: sum q[d] code[d]) are bit
+        // planes of ceil(dim / 128) granules each, plane b first to last bit 0 to the top one: the sum under a plane
+        // enters the total with weight 2^b when the plane ends.
+        uint32_t plane = 0, jj = j;
+        if (a.planes > 1) {
+            plane = (j * a.plane_recip) >> 16;
+            jj = j - plane * a.plane_granules;
+        }
 #pragma unroll
         for (int m = 0; m < 4; ++m) {
 #pragma unroll
@@ -184,8 +194,16 @@ accumulate_granule(const ScanArgs& a, const QueryRows<T>& q, uint32_t j, uint4 c
                 uint32_t mask = static_cast<uint32_t>(__builtin_amdgcn_sbfe(static_cast<int32_t>(w[m]), e, 1));
 #pragma unroll
                 for (int t = 0; t < T; ++t) {
-                    acc.f[t] += __uint_as_float(mask & q.row[t][128 * j + 32 * m + e]);
+                    acc.f[t] += __uint_as_float(mask & q.row[t][128 * jj + 32 * m + e]);
                 }
+            }
+        }
+        if (a.planes > 1 && jj + 1 == a.plane_granules) {
+            const float weight = static_cast<float>(1U << plane);
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                acc.lo[t] = __float_as_uint(fmaf(weight, acc.f[t], __uint_as_float(acc.lo[t])));
+                acc.f[t] = 0.0F;
             }
         }
     } else if constexpr (KIND == VSAG_AMD_KIND_PQFS) {
@@ -284,6 +302,11 @@ finish_distances(const ScanArgs& a, const uint32_t (&qidx)[T], uint64_t slot, co
                 float p1 = qm[0] * static_cast<float>(ip);
                 float p2 = qm[1] * base_sum;
                 ip_bq = p1 + p2 - qm[2] - qm[3];
+            } else if (a.planes > 1) {
+                // ip_obar_q (rabitq_quantizer.cpp:256-267) of the plane-weighted sum; qm[1] = sum of the query values
+                const float norm_code = __uint_as_float(a.meta[2 * a.meta_stride + slot]);
+                const float c = 0.5F * static_cast<float>((1U << a.planes) - 1U);
+                ip_bq = norm_code <= 0.0F ? 0.0F : (__uint_as_float(acc.lo[t]) - c * qm[1]) / norm_code;
             } else {
                 ip_bq = qm[0] * acc.f[t] - qm[2];
             }

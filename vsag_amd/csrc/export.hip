@@ -15,6 +15,7 @@ struct UntileArgs {
     uint32_t meta_offset[4];
     uint32_t meta_is_u64;
     uint32_t code_size, payload_bytes;
+    uint32_t plane_bytes, plane_granules;  // the payload as zero-padded planes (see vsag_amd_store)
     int nibbles;               // the u64 word is the sum of squared 4-bit values (sq4_uniform), else of squared bytes
     uint64_t n;
     uint64_t first_slot;       // slot of output row i: first_slot + i ...
@@ -37,10 +38,11 @@ untile_kernel(UntileArgs a) {
     uint8_t* dst = a.out + i * a.code_size;
     const uint4 v = a.tiles[(tile * a.G + j) * kWave + lane];
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    const uint32_t plane = j / a.plane_granules;
     for (uint32_t b = 0; b < 16; ++b) {
-        const uint32_t off = 16 * j + b;
-        if (off < a.payload_bytes) {
-            dst[off] = static_cast<uint8_t>(w[b >> 2] >> (8 * (b & 3)));
+        const uint32_t off = 16 * (j - plane * a.plane_granules) + b;
+        if (off < a.plane_bytes) {
+            dst[plane * a.plane_bytes + off] = static_cast<uint8_t>(w[b >> 2] >> (8 * (b & 3)));
         }
     }
     if (j != 0) {
@@ -124,6 +126,8 @@ untile_args(const vsag_amd_store* s, uint64_t n, uint8_t* out) {
     a.meta_is_u64 = s->meta_is_u64;
     a.code_size = s->code_size;
     a.payload_bytes = s->payload_bytes;
+    a.plane_bytes = s->plane_bytes;
+    a.plane_granules = s->plane_granules;
     a.nibbles = s->kind == VSAG_AMD_KIND_SQ4_UNIFORM ? 1 : 0;
     a.n = n;
     a.out = out;

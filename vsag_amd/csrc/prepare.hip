@@ -207,7 +207,7 @@ query_code_bytes(const vsag_amd_store* s, uint64_t nq) {
         return nq * s->code_size;
     }
     if (s->kind == VSAG_AMD_KIND_RABITQ) {
-        return nq * rabitq_query_code_size(s->dim, s->metric, s->query_bits);
+        return nq * rabitq_query_code_size(s->dim, s->metric, rabitq_bits_word(s));
     }
     return 0;
 }
@@ -275,7 +275,7 @@ query_layout(const vsag_amd_store* s) {
 // rabitq_quantizer.cpp:2049-2088) -> table row padded with zeros + the factors of the estimator.
 __global__ void __launch_bounds__(256)
 prepare_rabitq_f32_queries(const uint8_t* qcodes, uint64_t nq, uint32_t qcode_size, uint32_t dim, int has_raw_norm,
-                           uint32_t* qtab, uint32_t qstride, float* qmeta, uint32_t qmeta_stride) {
+                           int has_sum, uint32_t* qtab, uint32_t qstride, float* qmeta, uint32_t qmeta_stride) {
     __shared__ float partial[256];
     uint64_t row = blockIdx.x;
     uint32_t* out = qtab + row * qstride;
@@ -309,11 +309,12 @@ prepare_rabitq_f32_queries(const uint8_t* qcodes, uint64_t nq, uint32_t qcode_si
         for (uint32_t i = 0; i < blockDim.x; ++i) {
             total += partial[i];
         }
-        uint32_t tail = (4 * dim + 3) / 4 * 4;
+        // behind the values: (their running sum, multi-bit base codes only,) the norm, (the raw norm)
+        uint32_t tail = (4 * dim + 3) / 4 * 4 + (has_sum ? 4 : 0);
         float inv_sqrt_d = 1.0F / sqrtf(static_cast<float>(dim));
         float* m = qmeta + row * qmeta_stride;
         m[0] = 2.0F * inv_sqrt_d;
-        m[1] = 0.0F;
+        m[1] = has_sum ? __uint_as_float(rd(4 * dim)) : 0.0F;
         m[2] = inv_sqrt_d * total;
         m[3] = 0.0F;
         m[4] = __uint_as_float(rd(tail));
@@ -349,11 +350,12 @@ prepare_queries(const vsag_amd_store* s, const float* queries, uint64_t nq, uint
         case VSAG_AMD_KIND_RABITQ: {
             VA_CHECK_ARG(s->query_bits == 4 || s->query_bits == 32, "rabitq scan supports 4-bit and fp32 queries");
             VA_TRY(rabitq_process_query_launch(queries, nq, s->dim, s->rotation_dev, s->centroid_dev, s->metric,
-                                               s->query_bits, qcodes, st, scratch));
+                                               rabitq_bits_word(s), qcodes, st, scratch));
             if (s->query_bits == 32) {
                 hipLaunchKernelGGL(prepare_rabitq_f32_queries, grid, dim3(256), 0, st, qcodes, nq,
-                                   static_cast<uint32_t>(rabitq_query_code_size(s->dim, s->metric, 32)), s->dim,
-                                   s->metric != VSAG_AMD_METRIC_L2 ? 1 : 0, qtab, ql.qstride, qmeta, ql.qmeta);
+                                   static_cast<uint32_t>(rabitq_query_code_size(s->dim, s->metric, rabitq_bits_word(s))),
+                                   s->dim, s->metric != VSAG_AMD_METRIC_L2 ? 1 : 0, s->base_bits != 1 ? 1 : 0, qtab,
+                                   ql.qstride, qmeta, ql.qmeta);
                 break;
             }
             uint32_t aligned_dim = (s->dim + 511) / 512 * 512;
@@ -386,6 +388,9 @@ make_scan_args(const vsag_amd_store* s, const QueryLayout& ql, const uint32_t* q
     a.qmeta_stride = ql.qmeta;
     a.G = s->G;
     a.dim = s->dim;
+    a.planes = s->planes;
+    a.plane_granules = s->plane_granules;
+    a.plane_recip = (65536U + s->plane_granules - 1) / s->plane_granules;
     a.f0 = s->ulb;
     a.f1 = s->scalar_rate;
     a.f2 = s->ulb * s->ulb;

@@ -210,19 +210,27 @@ gemm_nt_seq(const float* A, const float* B, float* C, uint64_t M, uint32_t N, ui
 // ------------------------------------------------------------------ RaBitQ
 struct RabitqLayout {
     uint32_t dim, code_bytes;
+    uint32_t base_bits, offset_norm_code;  // bits per dimension of the base code; |code - centre| where base_bits != 1
     uint32_t offset_norm, offset_error, offset_sum, offset_raw_norm, code_size;
     int has_sum, has_raw_norm;
     uint32_t aligned_dim, plane_bytes;
     uint32_t q_offset_lb, q_offset_delta, q_offset_sum, q_offset_norm, q_offset_raw_norm, query_code_size;
 };
 
-// rabitq_quantizer.cpp:102-176 (1-bit base, standard version, no PCA / MRQ / split storage).
+// rabitq_quantizer.cpp:102-176 (standard version, no PCA / MRQ / split storage).  `query_bits` is the bits word of the
+// C interface: 4 or 32 for the query, plus 256 * base bits for multi-bit base codes (VSAG_AMD_RABITQ_BITS).
 __host__ __device__ inline RabitqLayout
 rabitq_layout(uint32_t dim, int metric, int query_bits) {
     RabitqLayout l{};
     l.dim = dim;
-    l.code_bytes = (dim + 7) / 8;
+    l.base_bits = (query_bits >> 8) == 0 ? 1U : static_cast<uint32_t>(query_bits >> 8);
+    query_bits &= 255;
+    l.code_bytes = (dim + 7) / 8 * l.base_bits;
     uint32_t cs = (l.code_bytes + 3) / 4 * 4;
+    if (l.base_bits != 1) {
+        l.offset_norm_code = cs;
+        cs += 4;
+    }
     l.offset_norm = cs;
     cs += 4;
     l.offset_error = cs;
@@ -251,6 +259,10 @@ rabitq_layout(uint32_t dim, int metric, int query_bits) {
         qs += 4;
     } else {
         qs = 4 * dim;
+        if (l.base_bits != 1) {
+            l.q_offset_sum = qs;
+            qs += 4;
+        }
     }
     l.q_offset_norm = qs;
     qs += 4;
@@ -397,6 +409,339 @@ rabitq_finish_encode_kernel(const float* raw, const float* rotated, uint64_t n, 
     }
 }
 
+// ---- multi-bit base codes (rabitq_bits_per_dim_base 2..8) ----
+// Norm of (rotated row - centroid) as NormalizeWithCentroid takes it (kernels/normalize.h:35-83).
+__device__ inline float
+rabitq_row_norm(const float* y, const float* centroid, uint32_t dim) {
+    float norm_sq = 0.0F;
+    for (uint32_t d = 0; d < dim; ++d) {
+        float t = y[d] - centroid[d];
+        norm_sq = t * t + norm_sq;
+    }
+    return norm_sq < 1e-5F ? 1.0F : sqrtf(norm_sq);
+}
+
+// RaBitQuantizer::FastEncodeRaBitQ (rabitq_quantizer.cpp:609-704): a floor grid over [-max|o|, max|o|], then `rounds`
+// sweeps of one-level moves per coordinate that raise <o, y>^2 / |y|^2 (y = code - centre).  The sweep is sequential
+// per row (every move changes the sums the next coordinate is judged by), so one thread owns a row; all sums are
+// doubles in the reference's order.  scalar: n x dim code values; norm_code: n floats.
+__global__ void __launch_bounds__(64)
+rabitq_fast_encode_kernel(const float* rotated, uint64_t n, uint32_t dim, const float* centroid, uint32_t bits,
+                          uint32_t rounds, uint8_t* scalar, float* norm_code) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) {
+        return;
+    }
+    const float* y = rotated + i * dim;
+    uint8_t* code = scalar + i * dim;
+    const float norm = rabitq_row_norm(y, centroid, dim);
+    const uint32_t code_max = (1U << bits) - 1U;
+    const double center = 0.5 * static_cast<double>(code_max);
+    double max_abs = 0.0;
+    for (uint32_t d = 0; d < dim; ++d) {
+        const float o = (y[d] - centroid[d]) / norm;
+        max_abs = fmax(max_abs, fabs(static_cast<double>(o)));
+    }
+    if (max_abs <= 0.0) {
+        for (uint32_t d = 0; d < dim; ++d) {
+            code[d] = static_cast<uint8_t>(code_max / 2U);
+        }
+        norm_code[i] = 1.0F;
+        return;
+    }
+    const double delta = 2.0 * max_abs / static_cast<double>(code_max + 1U);
+    const double inv_delta = 1.0 / delta;
+    double ip = 0.0, norm_sqr = 0.0;
+    for (uint32_t d = 0; d < dim; ++d) {
+        const float o = (y[d] - centroid[d]) / norm;
+        const double scaled = (static_cast<double>(o) + max_abs) * inv_delta;
+        long long q = static_cast<long long>(floor(scaled));
+        q = q < 0 ? 0 : (q > static_cast<long long>(code_max) ? static_cast<long long>(code_max) : q);
+        code[d] = static_cast<uint8_t>(q);
+        const double centered = static_cast<double>(q) - center;
+        ip += static_cast<double>(o) * centered;
+        norm_sqr += centered * centered;
+    }
+    for (uint32_t round = 0; round < rounds; ++round) {
+        bool adjusted = false;
+        for (uint32_t d = 0; d < dim; ++d) {
+            const double o = static_cast<double>((y[d] - centroid[d]) / norm);
+            const int cur = code[d];
+            const double cur_value = static_cast<double>(cur) - center;
+            int best_code = cur;
+            double best_ip = ip, best_norm = norm_sqr;
+            double best_score = norm_sqr > 0.0 ? ip * ip / norm_sqr : 0.0;
+#pragma unroll
+            for (int dir = -1; dir <= 1; dir += 2) {
+                const int cand = cur + dir;
+                if (cand < 0 || cand > static_cast<int>(code_max)) {
+                    continue;
+                }
+                const double cand_ip = ip + static_cast<double>(dir) * o;
+                if (cand_ip < 0.0) {
+                    continue;
+                }
+                const double cand_norm = norm_sqr + 2.0 * cur_value * static_cast<double>(dir) + 1.0;
+                const double cand_score = cand_norm > 0.0 ? cand_ip * cand_ip / cand_norm : 0.0;
+                const double tolerance = 1e-8 * fmax(1.0, fabs(best_score));
+                if (cand_score > best_score + tolerance) {
+                    best_code = cand;
+                    best_ip = cand_ip;
+                    best_norm = cand_norm;
+                    best_score = cand_score;
+                }
+            }
+            if (best_code != cur) {
+                code[d] = static_cast<uint8_t>(best_code);
+                ip = best_ip;
+                norm_sqr = best_norm;
+                adjusted = true;
+            }
+        }
+        if (!adjusted) {
+            break;
+        }
+    }
+    norm_sqr = 0.0;
+    for (uint32_t d = 0; d < dim; ++d) {
+        const double centered = static_cast<double>(code[d]) - center;
+        norm_sqr += centered * centered;
+    }
+    float yn = static_cast<float>(sqrt(norm_sqr));
+    if (!isfinite(yn) || yn <= 0.0F) {
+        yn = 1.0F;
+    }
+    norm_code[i] = yn;
+}
+
+// RaBitQuantizer::EncodeExtendRaBitQ (rabitq_quantizer.cpp:455-607): the scale t walks upwards, one grid step of one
+// coordinate per event, events in (t, coordinate) order -- the reference's priority queue always holds at most one
+// pending event per coordinate, so "pop" is the minimum over the coordinates' next event times.  One wave per row:
+// the lanes share that minimum search, every lane repeats the running sums (doubles, the reference's order).
+// LDS per row: dim doubles (next event), dim ints (grid position), dim floats (o).
+__global__ void __launch_bounds__(64)
+rabitq_extend_encode_kernel(const float* rotated, uint64_t n, uint32_t dim, const float* centroid, uint32_t bits,
+                            uint8_t* scalar, float* norm_code) {
+    extern __shared__ double ee_lds[];
+    double* next_t = ee_lds;
+    int* y2_cur = reinterpret_cast<int*>(next_t + dim);
+    float* o = reinterpret_cast<float*>(y2_cur + dim);
+    const uint64_t i = blockIdx.x;
+    const uint32_t lane = threadIdx.x;
+    const float* y = rotated + i * dim;
+    uint8_t* code = scalar + i * dim;
+    float norm = 0.0F;
+    if (lane == 0) {
+        norm = rabitq_row_norm(y, centroid, dim);
+    }
+    norm = __shfl(norm, 0);
+    const int y2_max = static_cast<int>((1U << bits) - 1U);
+    const double c = 0.5 * static_cast<double>(y2_max);
+    const double inf = __builtin_huge_val();
+    double max_o = 0.0;
+    for (uint32_t d = lane; d < dim; d += kWave) {
+        const float v = (y[d] - centroid[d]) / norm;
+        o[d] = v;
+        max_o = fmax(max_o, fabs(static_cast<double>(v)));
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        max_o = fmax(max_o, __shfl_xor(max_o, off));
+    }
+    if (max_o <= 0.0) {
+        for (uint32_t d = lane; d < dim; d += kWave) {
+            code[d] = static_cast<uint8_t>(y2_max / 2);
+        }
+        if (lane == 0) {
+            norm_code[i] = 1.0F;
+        }
+        return;
+    }
+    const double t_end = (static_cast<double>(y2_max) + 2.0) / (2.0 * max_o);
+    // Next event time of a coordinate at grid position `pos` (compute_next_t_for_dim, :513-531).
+    auto next_event = [&](double oi, int pos) {
+        if (fabs(oi) < 1e-3) {
+            return inf;
+        }
+        const int sign = (oi > 0.0) ? +1 : -1;
+        const int y2_next = pos + sign * 2;
+        if (y2_next < -y2_max || y2_next > +y2_max) {
+            return inf;
+        }
+        double t = static_cast<double>(pos + sign) / (2.0 * oi);
+        if (t < 0.0) {
+            t = 0.0;
+        }
+        return t;
+    };
+    for (uint32_t d = lane; d < dim; d += kWave) {
+        const double oi = static_cast<double>(o[d]);
+        double t0 = inf;
+        if (oi != 0.0) {
+            t0 = next_event(oi, 0);
+            if (!(t0 <= t_end)) {
+                t0 = inf;
+            }
+        }
+        next_t[d] = t0;
+        y2_cur[d] = 0;
+    }
+    wave_lds_fence();
+    double ip_y2_o = 0.0, norm_y2 = 0.0;
+    double best_ip = 1e-12, best_t = 0.0;
+    // Every pass retires one event; a coordinate has at most 2^(bits - 1) of them, so the walk ends.
+    const uint64_t max_events = static_cast<uint64_t>(dim) << bits;
+    for (uint64_t ev = 0; ev < max_events; ++ev) {
+        double bt = inf;
+        uint32_t bi = 0xFFFFFFFFU;
+        for (uint32_t d = lane; d < dim; d += kWave) {
+            const double t = next_t[d];
+            if (t < bt) {
+                bt = t;
+                bi = d;
+            }
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            const double ot = __shfl_xor(bt, off);
+            const uint32_t oi = __shfl_xor(bi, off);
+            if (ot < bt || (ot == bt && oi < bi)) {
+                bt = ot;
+                bi = oi;
+            }
+        }
+        if (bi == 0xFFFFFFFFU || !(bt < t_end)) {
+            break;
+        }
+        const double cur_t = bt;
+        const uint32_t k = bi;
+        const double ok = static_cast<double>(o[k]);
+        const int sign = (o[k] > 0.0F) ? +1 : -1;
+        const int y2_old = y2_cur[k];
+        const int y2_new = y2_old + sign * 2;
+        wave_lds_fence();
+        if (y2_new < -y2_max || y2_new > +y2_max) {
+            if (lane == 0) {
+                next_t[k] = inf;
+            }
+            wave_lds_fence();
+            continue;
+        }
+        ip_y2_o += (static_cast<double>(y2_new) - static_cast<double>(y2_old)) * ok;
+        norm_y2 += static_cast<double>(y2_new) * static_cast<double>(y2_new) -
+                   static_cast<double>(y2_old) * static_cast<double>(y2_old);
+        const double cur_ip = (norm_y2 > 0.0) ? (ip_y2_o / sqrt(norm_y2)) : 0.0;
+        if (cur_ip > best_ip) {
+            best_ip = cur_ip;
+            best_t = cur_t;
+        }
+        double t_next = next_event(ok, y2_new);
+        if (t_next <= cur_t) {
+            t_next = __longlong_as_double(__double_as_longlong(cur_t) + 1);  // nextafter(cur_t, +inf), cur_t >= 0
+        }
+        if (lane == 0) {
+            y2_cur[k] = y2_new;
+            next_t[k] = (t_next < t_end) ? t_next : inf;  // a finite time below the end, else no further event
+        }
+        wave_lds_fence();
+    }
+    double sum_y2 = 0.0;  // a sum of k + 0.25 terms: exact in any order
+    for (uint32_t d = lane; d < dim; d += kWave) {
+        const double val = 2.0 * best_t * static_cast<double>(o[d]);
+        const double shifted = val + ((val >= 0) ? 1e-12 : -1e-12);
+        long long r = llround(shifted);
+        int ri = r < -y2_max ? -y2_max : (r > y2_max ? y2_max : static_cast<int>(r));
+        if ((ri & 1) != (y2_max & 1)) {
+            const int step = (shifted >= 0.0) ? +1 : -1;
+            int cand = ri + step;
+            if (cand < -y2_max || cand > y2_max) {
+                cand = ri - step;
+            }
+            ri = cand < -y2_max ? -y2_max : (cand > y2_max ? y2_max : cand);
+        }
+        int u = (ri + y2_max) / 2;
+        u = u < 0 ? 0 : (u > y2_max ? y2_max : u);
+        code[d] = static_cast<uint8_t>(u);
+        const double yy = static_cast<double>(u) - c;
+        sum_y2 += yy * yy;
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        sum_y2 += __shfl_xor(sum_y2, off);
+    }
+    if (lane == 0) {
+        float yn = static_cast<float>(sqrt(sum_y2));
+        if (!isfinite(yn) || yn <= 0.0F) {
+            yn = 1.0F;
+        }
+        norm_code[i] = yn;
+    }
+}
+
+// Rest of the multi-bit branch of RaBitQuantizer::EncodeOneInternal (rabitq_quantizer.cpp:789-809, 852-855): bit planes
+// (PackIntoPlanes, :431-453: plane b holds bit b of every dimension), |code - centre|, the norms, and error =
+// ip_obar_q(<o, code>, sum o, |code - centre|) with both sums as running floats in element order.  One thread per row.
+__global__ void __launch_bounds__(64)
+rabitq_multibit_finish_kernel(const float* raw, const float* rotated, uint64_t n, uint32_t dim, const float* centroid,
+                              int metric, int bits_word, const uint8_t* scalar, const float* norm_code,
+                              uint8_t* codes) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) {
+        return;
+    }
+    const RabitqLayout l = rabitq_layout(dim, metric, bits_word);
+    const float* y = rotated + i * dim;
+    const uint8_t* sc = scalar + i * dim;
+    uint8_t* c = codes + i * l.code_size;
+    float raw_norm = 0.0F;
+    if (l.has_raw_norm) {
+        const float* x = raw + i * dim;
+        for (uint32_t d = 0; d < dim; ++d) {
+            raw_norm += x[d] * x[d];
+        }
+    }
+    raw_norm = sqrtf(raw_norm);
+    const float norm = rabitq_row_norm(y, centroid, dim);
+    const uint32_t plane_bytes = (dim + 7) / 8;
+    float query_sum = 0.0F, scalar_ip = 0.0F;
+    for (uint32_t b = 0; b < plane_bytes; ++b) {
+        uint32_t plane[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (uint32_t e = 0; e < 8; ++e) {
+            const uint32_t d = b * 8 + e;
+            if (d >= dim) {
+                break;
+            }
+            const float nd = (y[d] - centroid[d]) / norm;
+            const uint32_t v = sc[d];
+            query_sum += nd;
+            scalar_ip += static_cast<float>(v) * nd;
+#pragma unroll
+            for (uint32_t p = 0; p < 8; ++p) {
+                plane[p] |= ((v >> p) & 1U) << e;
+            }
+        }
+#pragma unroll
+        for (uint32_t p = 0; p < 8; ++p) {
+            if (p < l.base_bits) {
+                c[p * plane_bytes + b] = static_cast<uint8_t>(plane[p]);
+            }
+        }
+    }
+    for (uint32_t b = l.code_bytes; b < l.offset_norm_code; ++b) {
+        c[b] = 0;
+    }
+    const float yn = norm_code[i];
+    // ip_obar_q (rabitq_quantizer.cpp:256-267)
+    float error = 0.0F;
+    if (yn > 0.0F) {
+        error = scalar_ip - 0.5F * static_cast<float>((1U << l.base_bits) - 1U) * query_sum;
+        error /= yn;
+    }
+    store_f32(c + l.offset_norm_code, yn);
+    store_f32(c + l.offset_norm, norm);
+    store_f32(c + l.offset_error, error);
+    if (l.has_raw_norm) {
+        store_f32(c + l.offset_raw_norm, raw_norm);
+    }
+}
+
 // Second half of RaBitQuantizer::ProcessQueryImpl (rabitq_quantizer.cpp:2130-2217) with EncodeSQ and
 // ReOrderSQ (:2049-2088) for queries already rotated.  One thread per query.
 __global__ void __launch_bounds__(64)
@@ -423,7 +768,14 @@ rabitq_finish_query_kernel(const float* raw, const float* rotated, uint64_t nq, 
         norm_sq = t * t + norm_sq;
     }
     float norm = norm_sq < 1e-5F ? 1.0F : sqrtf(norm_sq);
-    if (query_bits == 4) {
+    if (l.base_bits != 1) {
+        float sum = 0.0F;
+        for (uint32_t d = 0; d < dim; ++d) {
+            sum += (y[d] - centroid[d]) / norm;
+        }
+        store_f32(qc + l.q_offset_sum, sum);
+    }
+    if ((query_bits & 255) == 4) {
         float lb = FLT_MAX, ub = -FLT_MAX;
         for (uint32_t d = 0; d < dim; ++d) {
             float v = (y[d] - centroid[d]) / norm;
@@ -505,7 +857,14 @@ rabitq_finish_query_wave_kernel(const float* raw, const float* rotated, uint64_t
     raw_norm = sqrtf(__shfl(raw_norm, 0));
     norm_sq = __shfl(norm_sq, 0);
     const float norm = norm_sq < 1e-5F ? 1.0F : sqrtf(norm_sq);
-    if (query_bits == 4) {
+    if (l.base_bits != 1 && lane == 0) {
+        float sum = 0.0F;  // in element order, like the reference (rabitq_quantizer.cpp:2199-2205)
+        for (uint32_t d = 0; d < dim; ++d) {
+            sum += t[d] / norm;
+        }
+        store_f32(qc + l.q_offset_sum, sum);
+    }
+    if ((query_bits & 255) == 4) {
         float lb = FLT_MAX, ub = -FLT_MAX;
         for (uint32_t d = lane; d < dim; d += kWave) {
             const float v = t[d] / norm;
@@ -928,6 +1287,55 @@ vsag_amd_rabitq_encode(const float* x_dev, uint64_t n, uint32_t dim, const float
     });
 }
 
+extern "C" int
+vsag_amd_rabitq_encode_multibit(const float* x_dev, uint64_t n, uint32_t dim, const float* rotation_dev,
+                                const float* centroid_dev, int metric, int bits_word, int fast_encode,
+                                uint32_t fast_encode_rounds, uint8_t* codes_dev, void* stream) {
+    VA_TRY(ensure_init());
+    const int base_bits = bits_word >> 8;
+    VA_CHECK_ARG((bits_word & 255) == 32, "multi-bit base codes need fp32 queries (query bits 32), got %d", bits_word & 255);
+    VA_CHECK_ARG(base_bits >= 2 && base_bits <= 8, "base bits must be in [2, 8], got %d", base_bits);
+    VA_CHECK_ARG(dim >= 1 && dim <= 65536, "dim must be in [1, 65536], got %u", dim);
+    VA_CHECK_ARG(!fast_encode || (fast_encode_rounds >= 1 && fast_encode_rounds <= 32),
+                 "fast_encode_rabitq_rounds must be in [1, 32], but got %u", fast_encode_rounds);
+    VA_CHECK_ARG(fast_encode || dim <= 3072, "the exhaustive encoder supports at most 3072 dimensions, got %u", dim);
+    if (n == 0) {
+        return 0;
+    }
+    VA_CHECK_ARG(x_dev && rotation_dev && centroid_dev && codes_dev, "null pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint64_t csize = rabitq_code_size(dim, metric, bits_word);
+    const uint64_t rows = n < kRotateSlabRows ? n : kRotateSlabRows;
+    uint8_t* scalar = nullptr;
+    float* norm_code = nullptr;
+    VA_HIP(hipMallocAsync(reinterpret_cast<void**>(&scalar), rows * dim, st));
+    hipError_t e = hipMallocAsync(reinterpret_cast<void**>(&norm_code), rows * 4, st);
+    if (e != hipSuccess) {
+        (void)hipFreeAsync(scalar, st);
+        return fail(VSAG_AMD_NO_ENOUGH_MEMORY, "hipMallocAsync failed: %s", hipGetErrorString(e));
+    }
+    int rc = rabitq_rotate_slabs(x_dev, n, dim, rotation_dev, st, nullptr, [&](uint64_t s, uint64_t m, const float* rotated) {
+        if (fast_encode) {
+            hipLaunchKernelGGL(rabitq_fast_encode_kernel, dim3(static_cast<uint32_t>(div_up(m, 64))), dim3(64), 0, st,
+                               rotated, m, dim, centroid_dev, static_cast<uint32_t>(base_bits), fast_encode_rounds, scalar,
+                               norm_code);
+        } else {
+            const size_t lds = static_cast<size_t>(dim) * 16;
+            hipLaunchKernelGGL(rabitq_extend_encode_kernel, dim3(static_cast<uint32_t>(m)), dim3(64), lds, st, rotated, m,
+                               dim, centroid_dev, static_cast<uint32_t>(base_bits), scalar, norm_code);
+        }
+        VA_HIP(hipGetLastError());
+        hipLaunchKernelGGL(rabitq_multibit_finish_kernel, dim3(static_cast<uint32_t>(div_up(m, 64))), dim3(64), 0, st,
+                           x_dev + s * dim, rotated, m, dim, centroid_dev, metric, bits_word, scalar, norm_code,
+                           codes_dev + s * csize);
+        VA_HIP(hipGetLastError());
+        return 0;
+    });
+    (void)hipFreeAsync(scalar, st);
+    (void)hipFreeAsync(norm_code, st);
+    return rc;
+}
+
 extern "C" uint64_t
 vsag_amd_rabitq_query_code_size(uint32_t dim, int metric, int query_bits) {
     return rabitq_query_code_size(dim, metric, query_bits);
@@ -938,7 +1346,10 @@ vsag_amd_rabitq_process_query(const float* q_dev, uint64_t nq, uint32_t dim, con
                               const float* centroid_dev, int metric, int query_bits, uint8_t* qcodes_dev,
                               void* stream) {
     VA_TRY(ensure_init());
-    VA_CHECK_ARG(query_bits == 4 || query_bits == 32, "query_bits must be 4 or 32, got %d", query_bits);
+    VA_CHECK_ARG((query_bits & 255) == 4 || (query_bits & 255) == 32, "query_bits must be 4 or 32, got %d",
+                 query_bits & 255);
+    VA_CHECK_ARG((query_bits >> 8) == 0 || ((query_bits & 255) == 32 && (query_bits >> 8) <= 8),
+                 "multi-bit base codes (%d bits) need fp32 queries and at most 8 bits", query_bits >> 8);
     VA_CHECK_ARG(dim >= 1 && dim <= 65536, "dim must be in [1, 65536], got %u", dim);
     VA_CHECK_ARG(nq == 0 || (q_dev && rotation_dev && centroid_dev && qcodes_dev), "null pointer");
     return rabitq_process_query_launch(q_dev, nq, dim, rotation_dev, centroid_dev, metric, query_bits, qcodes_dev,

@@ -22,11 +22,17 @@ struct vsag_amd_store {
     int kind = 0;
     int metric = 0;
     uint32_t dim = 0;
-    int query_bits = 4;
+    int query_bits = 4;          // rabitq: 4 or 32
+    uint32_t base_bits = 1;      // rabitq: bits per dimension of the base code (more than 1: fp32 queries only)
 
     uint32_t code_size = 0;      // bytes per code in the reference layout
     uint32_t payload_bytes = 0;  // leading bytes consumed by the distance loop
     uint32_t G = 0;              // 16-byte granules per code
+    // The payload as planes: `planes` runs of plane_bytes source bytes, each padded to plane_granules granules in the
+    // tiles (multi-bit rabitq: one run per bit plane; every other kind: one run, the whole payload).
+    uint32_t planes = 1;
+    uint32_t plane_bytes = 0;
+    uint32_t plane_granules = 0;
     uint32_t dpad = 0;           // dims covered by G granules (per-dim tables are this long)
     // Scan settings of this store; the values below follow the process-wide ones (vsag_amd_set_scan_contraction /
     // vsag_amd_set_scan_tuning).
@@ -99,6 +105,11 @@ QueryLayout query_layout(const vsag_amd_store* s);
 // Device bytes prepare_queries needs behind its `qcodes` pointer for nq queries: the encoded queries of the kinds
 // that encode them, then whatever their encoders use as scratch.
 size_t query_staging_bytes(const vsag_amd_store* s, uint64_t nq);
+// The bits word of the rabitq entry points for a store: query bits plus 256 * base bits for multi-bit base codes.
+inline int
+rabitq_bits_word(const vsag_amd_store* s) {
+    return s->query_bits | (s->base_bits > 1 ? static_cast<int>(s->base_bits) << 8 : 0);
+}
 int launch_code_terms(vsag_amd_store* s, uint64_t first, uint64_t count, hipStream_t st);
 
 }  // namespace vsag_amd

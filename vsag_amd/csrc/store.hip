@@ -20,6 +20,8 @@ struct RetileArgs {
     uint64_t n;
     uint32_t code_size;
     uint32_t payload_bytes;
+    uint32_t plane_bytes;     // source bytes of one plane of the payload ...
+    uint32_t plane_granules;  // ... which fill this many granules (zero padded)
     uint32_t G;
     uint32_t nmeta;
     uint32_t meta_offset[4];
@@ -68,10 +70,12 @@ retile_kernel(RetileArgs a) {
             }
         }
     } else {
+        const uint32_t plane = j / a.plane_granules;
+        const uint8_t* run = src + plane * a.plane_bytes;
         for (uint32_t b = 0; b < 16; ++b) {
-            uint32_t off = 16 * j + b;
-            if (off < a.payload_bytes) {
-                w[b >> 2] |= static_cast<uint32_t>(src[off]) << (8 * (b & 3));
+            uint32_t off = 16 * (j - plane * a.plane_granules) + b;
+            if (off < a.plane_bytes) {
+                w[b >> 2] |= static_cast<uint32_t>(run[off]) << (8 * (b & 3));
             }
         }
     }
@@ -312,6 +316,8 @@ retile_args(const vsag_amd_store* s, const uint8_t* codes, uint64_t n) {
     a.n = n;
     a.code_size = s->code_size;
     a.payload_bytes = s->payload_bytes;
+    a.plane_bytes = s->plane_bytes;
+    a.plane_granules = s->plane_granules;
     a.G = s->G;
     a.nmeta = s->nmeta;
     for (int m = 0; m < 4; ++m) {
@@ -361,7 +367,7 @@ vsag_amd_code_size(int kind, int metric, uint32_t dim, int rabitq_query_bits) {
             return up(dim, align) + (norm ? 8 : 4);
         }
         case VSAG_AMD_KIND_RABITQ:
-            return rabitq_code_size(dim, metric, rabitq_query_bits ? rabitq_query_bits : 4);
+            return rabitq_code_size(dim, metric, (rabitq_query_bits & 255) ? rabitq_query_bits : (rabitq_query_bits | 4));
         case VSAG_AMD_KIND_PQFS:
             return (static_cast<uint64_t>(dim) + 1) / 2;  // dim = the number of subspaces here
         default:
@@ -391,10 +397,17 @@ vsag_amd_store_create(const vsag_amd_store_params_t* p, vsag_amd_store_t** out) 
     s->kind = p->kind;
     s->metric = p->metric;
     s->dim = p->dim;
-    s->query_bits = p->rabitq_query_bits ? p->rabitq_query_bits : 4;
+    s->query_bits = (p->rabitq_query_bits & 255) ? (p->rabitq_query_bits & 255) : 4;
+    s->base_bits = (p->rabitq_query_bits >> 8) ? static_cast<uint32_t>(p->rabitq_query_bits >> 8) : 1U;
+    if (p->kind == VSAG_AMD_KIND_RABITQ && s->base_bits != 1 && (s->query_bits != 32 || s->base_bits > 8)) {
+        delete s;
+        return fail(VSAG_AMD_INVALID_ARGUMENT, "multi-bit rabitq base codes take 2 to 8 bits and fp32 queries (got %u bits, "
+                    "%d-bit queries)", s->base_bits, s->query_bits);
+    }
     s->pq_dim = p->kind == VSAG_AMD_KIND_PQFS ? p->pq_dim : 0;
     s->code_size = static_cast<uint32_t>(
-        vsag_amd_code_size(p->kind, p->metric, p->kind == VSAG_AMD_KIND_PQFS ? p->pq_dim : p->dim, s->query_bits));
+        vsag_amd_code_size(p->kind, p->metric, p->kind == VSAG_AMD_KIND_PQFS ? p->pq_dim : p->dim,
+                           p->kind == VSAG_AMD_KIND_RABITQ ? rabitq_bits_word(s) : s->query_bits));
     uint32_t dims_per_granule = 16;
     auto up = [](uint64_t v, uint64_t a) { return (v + a - 1) / a * a; };
     int rc = 0;
@@ -438,14 +451,23 @@ vsag_amd_store_create(const vsag_amd_store_params_t* p, vsag_amd_store_t** out) 
             break;
         }
         case VSAG_AMD_KIND_RABITQ: {
-            s->payload_bytes = (p->dim + 7) / 8;
+            s->planes = s->base_bits;
+            s->plane_bytes = (p->dim + 7) / 8;
+            s->payload_bytes = s->plane_bytes * s->planes;
             dims_per_granule = 128;
             uint32_t off = static_cast<uint32_t>(up(s->payload_bytes, 4));
-            // norm, error, sum, raw norm (rabitq_quantizer.cpp:102-133); sum exists for query_bits != 32.
+            // (norm of the code,) norm, error, sum, raw norm (rabitq_quantizer.cpp:102-133); the code's norm exists for
+            // multi-bit codes, the sum for query_bits != 32.  Word 2 holds whichever of those two the store has.
             s->nmeta = 4;
+            if (s->base_bits != 1) {
+                s->meta_offset[2] = off;
+                off += 4;
+            }
             s->meta_offset[0] = off;
             s->meta_offset[1] = off + 4;
-            s->meta_offset[2] = s->query_bits != 32 ? off + 8 : off + 4;
+            if (s->base_bits == 1) {
+                s->meta_offset[2] = s->query_bits != 32 ? off + 8 : off + 4;
+            }
             s->meta_offset[3] = p->metric != VSAG_AMD_METRIC_L2 ? s->code_size - 4 : off + 4;
             break;
         }
@@ -455,8 +477,12 @@ vsag_amd_store_create(const vsag_amd_store_params_t* p, vsag_amd_store_t** out) 
             dims_per_granule = 32;
             break;
     }
-    s->G = static_cast<uint32_t>((s->payload_bytes + kGranule - 1) / kGranule);
-    s->dpad = s->G * dims_per_granule;
+    if (s->plane_bytes == 0) {
+        s->plane_bytes = s->payload_bytes;
+    }
+    s->plane_granules = static_cast<uint32_t>((s->plane_bytes + kGranule - 1) / kGranule);
+    s->G = s->plane_granules * s->planes;
+    s->dpad = s->plane_granules * dims_per_granule;
 
     auto fail_free = [&](int code) {
         vsag_amd_store_destroy(s);

@@ -535,13 +535,22 @@ struct Quantizer {
     int metric = VSAG_AMD_METRIC_L2;
     uint32_t dim = 0;
     int rabitq_query_bits = 32;
+    // RaBitQuantizerParameter (rabitq_quantizer_parameter.h:57-64): bits per dimension of the base code and the encoder
+    // of multi-bit codes (FastEncodeRaBitQ with this many rounds, else EncodeExtendRaBitQ).
+    int rabitq_base_bits = 1;
+    bool rabitq_fast_encode = true;
+    uint32_t rabitq_fast_rounds = 6;
     uint32_t pq_dim = 1;  // pqfs: subspaces (PQFastScanQuantizerParameter::pq_dim_, default 1)
     bool trained = false;
     DevBuf lb, diff, bounds, rotation, centroid, codebooks;
 
+    int
+    rabitq_bits() const {
+        return VSAG_AMD_RABITQ_BITS(rabitq_query_bits, rabitq_base_bits);
+    }
     uint64_t
     code_size() const {
-        return vsag_amd_code_size(kind, metric, kind == VSAG_AMD_KIND_PQFS ? pq_dim : dim, rabitq_query_bits);
+        return vsag_amd_code_size(kind, metric, kind == VSAG_AMD_KIND_PQFS ? pq_dim : dim, rabitq_bits());
     }
 
     // Random orthogonal matrix: Gram-Schmidt on a Gaussian matrix (the reference takes the Q of a LAPACK QR,
@@ -654,6 +663,12 @@ struct Quantizer {
                                         bounds.as<float>(), codes, nullptr));
                 break;
             case VSAG_AMD_KIND_RABITQ:
+                if (rabitq_base_bits != 1) {
+                    dev(vsag_amd_rabitq_encode_multibit(x_dev, n, dim, rotation.as<float>(), centroid.as<float>(), metric,
+                                                        rabitq_bits(), rabitq_fast_encode ? 1 : 0, rabitq_fast_rounds,
+                                                        codes, nullptr));
+                    break;
+                }
                 dev(vsag_amd_rabitq_encode(x_dev, n, dim, rotation.as<float>(), centroid.as<float>(), metric,
                                            rabitq_query_bits, codes, nullptr));
                 break;
@@ -678,6 +693,9 @@ struct Quantizer {
         q.metric = metric;
         q.dim = dim;
         q.rabitq_query_bits = rabitq_query_bits;
+        q.rabitq_base_bits = rabitq_base_bits;
+        q.rabitq_fast_encode = rabitq_fast_encode;
+        q.rabitq_fast_rounds = rabitq_fast_rounds;
         q.pq_dim = pq_dim;
         return q;
     }
@@ -831,7 +849,7 @@ struct Quantizer {
         p.kind = kind;
         p.metric = metric;
         p.dim = dim;
-        p.rabitq_query_bits = rabitq_query_bits;
+        p.rabitq_query_bits = rabitq_bits();
         if (kind == VSAG_AMD_KIND_SQ8 || kind == VSAG_AMD_KIND_SQ4) {
             p.lower_bound_dev = lb.as<float>();
             p.diff_dev = diff.as<float>();
@@ -1679,11 +1697,41 @@ read_rabitq_params(const Json& index_param, Quantizer& q) {
         q.rabitq_query_bits = static_cast<int>(index_param["rabitq_bits_per_dim_query"].GetInt());
     }
     if (q.kind == VSAG_AMD_KIND_RABITQ) {
+        // RaBitQuantizerParameter::FromJson (rabitq_quantizer_parameter.cpp:30-112) and the constructor's checks
+        // (rabitq_quantizer.cpp:67-100).
         CHECK_ARGUMENT(q.rabitq_query_bits == 4 || q.rabitq_query_bits == 32,
-                       "rabitq_bits_per_dim_query must be 4 or 32");
+                       "currently, only support rabitq_bits_per_dim_query = 4 or 32, but got " +
+                           std::to_string(q.rabitq_query_bits));
         if (index_param.Contains("rabitq_bits_per_dim_base")) {
-            CHECK_ARGUMENT(index_param["rabitq_bits_per_dim_base"].GetInt() == 1,
-                           "the GPU path supports rabitq_bits_per_dim_base = 1 only");
+            const int64_t bits = index_param["rabitq_bits_per_dim_base"].GetInt();
+            CHECK_ARGUMENT(bits >= 1 && bits <= 8,
+                           "currently, only support rabitq_bits_per_dim_base in [1, 8], but got " + std::to_string(bits));
+            q.rabitq_base_bits = static_cast<int>(bits);
+        }
+        if (index_param.Contains("rabitq_version")) {
+            const std::string version = index_param["rabitq_version"].GetString();
+            CHECK_ARGUMENT(version == "standard" || version == "split" || version == "split_1bit_7bit",
+                           "unsupported rabitq_version: " + version + ". Supported values are standard, split");
+            // The split layout belongs to the flatten cell of the graph indexes (datacell/rabitq_split_datacell.h).
+            CHECK_ARGUMENT(version == "standard", "rabitq_version=split is not supported on the GPU path");
+        }
+        CHECK_ARGUMENT(q.rabitq_query_bits != 4 || q.rabitq_base_bits == 1,
+                       "not support num_bits_per_dim_query_ == 4 with num_bits_per_dim_base_ != 1");
+        if (index_param.Contains("rabitq_error_rate")) {
+            const double rate = index_param["rabitq_error_rate"].GetFloat();
+            CHECK_ARGUMENT(std::isfinite(rate) && rate > 0.0,
+                           "rabitq_error_rate must be finite and positive, got " + std::to_string(rate));
+        }
+        if (index_param.Contains("fast_encode_rabitq")) {
+            q.rabitq_fast_encode = index_param["fast_encode_rabitq"].GetBool();
+        }
+        if (index_param.Contains("fast_encode_rabitq_rounds")) {
+            CHECK_ARGUMENT(index_param["fast_encode_rabitq_rounds"].IsNumberInteger(),
+                           "fast_encode_rabitq_rounds must be an integer");
+            const int64_t rounds = index_param["fast_encode_rabitq_rounds"].GetInt();
+            CHECK_ARGUMENT(rounds >= 1 && rounds <= 32,
+                           "fast_encode_rabitq_rounds must be in [1, 32], but got " + std::to_string(rounds));
+            q.rabitq_fast_rounds = static_cast<uint32_t>(rounds);
         }
         if (index_param.Contains("rabitq_use_fht")) {
             CHECK_ARGUMENT(!index_param["rabitq_use_fht"].GetBool(), "rabitq_use_fht is not supported");
@@ -1716,7 +1764,8 @@ public:
         static const std::set<std::string> known = {
             "base_quantization_type", "base_io_type", "base_pq_dim", "base_file_path", "precise_quantization_type",
             "precise_io_type", "precise_file_path", "thread_count", "use_residual", "use_reorder",
-            "use_attribute_filter", "rabitq_bits_per_dim_query", "rabitq_bits_per_dim_base", "rabitq_use_fht"};
+            "use_attribute_filter", "rabitq_bits_per_dim_query", "rabitq_bits_per_dim_base", "rabitq_use_fht",
+            "rabitq_version", "rabitq_error_rate", "fast_encode_rabitq", "fast_encode_rabitq_rounds"};
         reject_unknown_keys(index_param, known);
         q_.metric = common.metric;
         q_.dim = common.dim;

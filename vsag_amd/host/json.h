@@ -67,6 +67,10 @@ public:
         }
         return static_cast<int64_t>(number);
     }
+    bool
+    IsNumberInteger() const {
+        return type == Type::Number && number == static_cast<double>(static_cast<int64_t>(number));
+    }
     double
     GetFloat() const {
         if (type != Type::Number) {
