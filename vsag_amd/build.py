@@ -22,7 +22,7 @@ HIP_FLAGS = [
     "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
 ]
 KERNEL_SOURCES = ["runtime.hip", "store.hip", "quantize.hip", "prepare.hip", "scan.hip", "prefilter.hip", "prefilter_i8.hip", "prefilter_rb.hip", "ivf.hip", "ivf_i8.hip", "ivf_pq.hip",
-                  "kmeans.hip", "lookup.hip", "export.hip", "pq.hip"]
+                  "kmeans.hip", "lookup.hip", "export.hip", "scan_one.hip", "pq.hip"]
 
 
 def _run(cmd):

@@ -90,7 +90,7 @@ query_rows(const ScanArgs& a, const uint32_t (&qidx)[T]) {
 
 // One granule (16 bytes of this lane's code, granule index j) against the T queries.
 template <int KIND, int METRIC, int T>
-__device__ inline void
+__device__ __forceinline__ void
 accumulate_granule(const ScanArgs& a, const QueryRows<T>& q, uint32_t j, uint4 c, Acc<KIND, T>& acc) {
     const uint32_t w[4] = {c.x, c.y, c.z, c.w};
     if constexpr (KIND == VSAG_AMD_KIND_FP32) {
@@ -241,7 +241,7 @@ accumulate_granule(const ScanArgs& a, const QueryRows<T>& q, uint32_t j, uint4 c
 
 // Distances of the finished code (tile slot `slot`) to the T queries.
 template <int KIND, int METRIC, int T>
-__device__ inline void
+__device__ __forceinline__ void
 finish_distances(const ScanArgs& a, const uint32_t (&qidx)[T], uint64_t slot, const Acc<KIND, T>& acc,
                  float (&out)[T]) {
     if constexpr (KIND == VSAG_AMD_KIND_FP32) {

@@ -501,7 +501,7 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
     Acc<KIND, T> acc;
     acc_reset(acc);
 
-    auto consume = [&](const uint4(&regs)[GROUP]) {
+    auto consume = [&](const uint4(&regs)[GROUP]) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < GROUP; ++u) {
             if (cur.j0 + u < a.G) {

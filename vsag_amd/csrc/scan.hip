@@ -155,7 +155,7 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
 
     const uint32_t pend = selector_base(S, k);  // where a selector's pending keys start
     // Sorts selector t and folds its k-th key and the shared bound into thr[t].
-    auto flush = [&](int t) {
+    auto flush = [&](int t) __attribute__((always_inline)) {
         uint64_t* keys = sel + t * S;
         uint64_t th = selector_flush(keys, S, k, cnt[t], lane);
         cnt[t] = 0;
@@ -172,7 +172,7 @@ flat_scan_kernel(ScanArgs a, FlatArgs f) {
     // What a cold wave reads of its queries' seed rows (largest entry over this lane's share): fetched when a tile
     // begins, looked at when its distances are done, so that the read waits under the tile's arithmetic.
     uint32_t seed_seen[T];
-    auto consume = [&](const uint4(&regs)[GROUP]) {
+    auto consume = [&](const uint4(&regs)[GROUP]) __attribute__((always_inline)) {
         const uint32_t first = cur.first();
         if (SEED && cur.j0 == 0) {
 #pragma unroll
@@ -818,6 +818,11 @@ struct CallPlan {
     // fp32 matrix cores, then per query the exact distances of the few codes that can be among the k best.
     bool table = false;
     uint64_t table_ld = 0;     // floats per row of the table
+    // One query against a large store (scan_one.hip): a pass that writes every distance and a minimum per run of
+    // tiles, then a one-workgroup selection.
+    bool one = false;
+    uint32_t one_runs = 0;
+    uint64_t one_tiles = 0;
 };
 
 // -1 never, 0 when it pays, 1 whenever the store supports it, 2 like 1 but on the fp32 matrix cores only
@@ -825,6 +830,10 @@ static int g_prefilter_mode = 0;
 // A store's own setting (vsag_amd_store_set_scan_contraction) goes before the process-wide one.
 static int prefilter_mode(const vsag_amd_store* s) { return s->contraction_mode >= -1 ? s->contraction_mode : g_prefilter_mode; }
 
+bool one_query_supports(const vsag_amd_store* s, uint64_t nq, uint32_t k);
+uint32_t one_query_run_tiles(const vsag_amd_store* s);
+int launch_one_query(const vsag_amd_store* s, const ScanArgs& a, uint32_t k, const vsag_amd_search_options_t* options,
+                     uint32_t* dist, uint64_t* mins, uint32_t* ids_dev, float* dists_dev, hipStream_t st);
 bool prefilter_supports(const vsag_amd_store* s);
 int launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t k, uint32_t S, uint64_t tile_begin,
                      uint64_t tile_end, uint32_t* bound, float* tau, uint32_t* cand, uint32_t* cand_cnt, uint32_t cap,
@@ -859,6 +868,10 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
     if (c->table) {
         return;
     }
+    // (an explicit query tile asks for the streaming kernel)
+    c->one = tile_override(s) <= 0 && one_query_supports(s, nq, k);
+    c->one_runs = c->one ? static_cast<uint32_t>(div_up(s->ntiles, static_cast<uint64_t>(one_query_run_tiles(s)))) : 0;
+    c->one_tiles = c->one ? s->ntiles : 0;
     if (prefilter_mode(s) < 0 || !prefilter_supports(s)) {
         return;
     }
@@ -974,6 +987,9 @@ struct ScanBuffers {
     float* table;       // nq x table_ld approximate distances
     float* table_rows;  // the codes a row per code
     float* table_norms; // their squared norms, then (one word) the largest as float bits
+    // one-query route only
+    uint32_t* one_dist;  // an ordered distance per tile slot
+    uint64_t* one_mins;  // the smallest key per run of tiles
 };
 
 static size_t
@@ -1002,6 +1018,8 @@ carve_scan(Carver& c, const CallPlan& cp, uint64_t nq, uint32_t k, ScanBuffers* 
     b->table = c.take<float>(cp.table ? nq * cp.table_ld : 0);
     b->table_rows = c.take<float>(cp.table ? cp.table_ld * p.ql.qstride : 0);
     b->table_norms = c.take<float>(cp.table ? cp.table_ld + 64 : 0);
+    b->one_mins = c.take<uint64_t>(cp.one ? cp.one_runs : 0);
+    b->one_dist = c.take<uint32_t>(cp.one ? cp.one_tiles * kWave : 0);
     return c.used;
 }
 
@@ -1446,6 +1464,13 @@ flat_scan_call(const vsag_amd_store_t* s, const float* queries_dev, uint64_t nq,
     Carver c(workspace_dev, workspace_bytes);
     ScanBuffers b;
     carve_scan(c, cp, nq, k, &b);
+    if (!c.ok() && cp.one) {
+        // A workspace sized without the one-query route's distance array (the fixed scratch of the entry point that
+        // allocates nothing): the query streams like a batch.
+        cp.one = false;
+        c = Carver(workspace_dev, workspace_bytes);
+        carve_scan(c, cp, nq, k, &b);
+    }
     VA_CHECK_ARG(c.ok(), "workspace too small: need %zu bytes, got %zu", c.used, workspace_bytes);
     // A pre-filter or a radius goes the streaming way (the prefilter knows neither).
     const bool plain = options == nullptr || (options->deny_bits_dev == nullptr && options->use_radius == 0);
@@ -1477,6 +1502,14 @@ flat_scan_call(const vsag_amd_store_t* s, const float* queries_dev, uint64_t nq,
         VA_HIP(hipGetLastError());
         tl_last_tile = 64;
         tl_last_passes = nq;
+        return 0;
+    }
+    if (cp.one && s->ntiles == cp.one_tiles) {
+        const ScanArgs oa = make_scan_args(s, p.ql, b.qtab, b.qmeta);
+        VA_TRY(launch_one_query(s, oa, k, options, b.one_dist, b.one_mins, ids_dev, dists_dev, st));
+        tl_last_tile = 1;
+        tl_last_passes = 1;
+        tl_last_bytes = s->ntiles * s->G * kWave * kGranule;
         return 0;
     }
     const uint64_t nseed = b.seed != nullptr ? nq * k : 0;
