@@ -589,8 +589,9 @@ def run_c4(env):
     per_dim = args.list_codes == "sq8"
     one_bit = args.list_codes == "rabitq"  # 1-bit codes, 4-bit queries, a seeded random rotation
     pqfs = args.list_codes == "pqfs"       # 4-bit product quantization, --pq-dim subspaces (default: one per dimension)
+    raw32 = args.list_codes == "fp32"      # the reference's default ivf codec: the vectors themselves
     pq_dim = (args.pq_dim or d) if pqfs else 0
-    kind = (capi.KIND_PQFS if pqfs else capi.KIND_RABITQ if one_bit else capi.KIND_SQ8 if per_dim
+    kind = (capi.KIND_FP32 if raw32 else capi.KIND_PQFS if pqfs else capi.KIND_RABITQ if one_bit else capi.KIND_SQ8 if per_dim
             else capi.KIND_SQ8_UNIFORM if bits == 8 else capi.KIND_SQ4_UNIFORM)
     kind_name = args.list_codes
     means = mt(315).random((10000, d), dtype=np.float32)
@@ -621,9 +622,11 @@ def run_c4(env):
     wsb = lib.vsag_amd_sq_train_workspace_bytes(ns, d, 0)
     ws = env.buf(wsb)
     cs = int(lib.vsag_amd_code_size(kind, capi.METRIC_L2, pq_dim if pqfs else d, 4 if one_bit else 0))
-    codes = env.buf(n * cs)
+    codes = x_dev if raw32 else env.buf(n * cs)
     rot = None
-    if pqfs:
+    if raw32:
+        lists = env.make_store(kind, capi.METRIC_L2, d)
+    elif pqfs:
         cb_dev = env.buf(d * 16 * 4)
         wsp = lib.vsag_amd_pq_train_workspace_bytes(ns, d, pq_dim)
         wp = env.buf(wsp)
@@ -720,7 +723,10 @@ def run_c4(env):
         offsets, order = orc.ivf_build_lists(hlabels, nlist)
         posting = hcodes[order]
         od = d
-        if pqfs:
+        if raw32:
+            hb = (None, None)
+            okind, qcodes = orc.FP32, q[:sample]
+        elif pqfs:
             hb = (None, None)
             okind, od = orc.PQFS, pq_dim
             qcodes = orc.pqfs_process_query(q[:sample], pq_dim, cb_dev.to_numpy(np.float32, (pq_dim, 16, d // pq_dim)), orc.L2)
@@ -737,7 +743,7 @@ def run_c4(env):
             qcodes = orc.squ_encode(q[:sample], bits, hb[0], hb[1], orc.L2)
         ref = orc.use_reference_kernels(orc.ref_best_isa())
         ref_name = {orc.SQ4U: "SQ4UniformComputeCodesIP", orc.SQ8U: "SQ8UniformComputeCodesIP",
-                    orc.RABITQ: "RaBitQSQ4UBinaryIP"}.get(okind)
+                    orc.RABITQ: "RaBitQSQ4UBinaryIP", orc.FP32: "FP32ComputeL2Sqr"}.get(okind)
         ref = ref if ref and ref_name in ref else None
         orc.ivf_scan(okind, orc.L2, od, posting, offsets, order, qcodes[:threads], b[:threads], kcand,
                      lb=hb[0], diff=hb[1], threads=threads)
@@ -770,7 +776,8 @@ def run_c4(env):
                                                        for a, bb in zip(rids, ids[:sample])])),
                "recall_at_10": None if gt_ids is None else recall_at_k(rids, gt_ids[:sample]),
                "gpu_recall_at_10_same_queries": None if gt_ids is None else recall_at_k(ids[:sample], gt_ids[:sample])}
-    codes.free()
+    if not raw32:
+        codes.free()
     achieved = algo / (kms * 1e-3) / 1e9
     # One step launches the scan kernel twice (nearest list of every query first, then the other lists); kernel_ms,
     # the algorithmic bytes (76 B per (query, scanned code), the reference's per-query list reads) and the traffic
@@ -791,20 +798,23 @@ def run_c4(env):
         # (pqfs: a pair is a contraction of the one-hot centroid indices with the byte table, 16 products per subspace)
         ops = 2.0 * (16 * (-(-pq_dim // 32) * 32) if pqfs else -(-d // 32) * 32) * float(rest)
         tops = ops / (kms * 1e-3) / 1e12
-        roof = {"bound": "mfma", "achieved": tops, "peak": MFMA_I8_PEAK_TOPS, "unit": "TOP/s",
-                "frac": tops / MFMA_I8_PEAK_TOPS,
+        peak = MFMA_F32_PEAK_TFLOPS if raw32 or (per_dim and d > 128) else MFMA_I8_PEAK_TOPS
+        roof = {"bound": "mfma", "achieved": tops, "peak": peak, "unit": "TFLOP/s" if peak == MFMA_F32_PEAK_TFLOPS else "TOP/s",
+                "frac": tops / peak,
                 # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this launch: profiles/ivf_i8_sq4u_c4.md
                 "traffic": 491061.0 * 2.00 * 1024 + 73550.7 * 1024
                 if (n, d, nq, k, nlist, bits) == (10000000, 128, 10000, 10, 4096, 4) else None,
-                "kernel": "%s<%s> (int8 MFMA, probe columns 1..%d)" % ("ivf_pq_kernel" if pqfs else
+                "kernel": "%s<%s> (%s MFMA, probe columns 1..%d)" % ("ivf_f32_kernel" if peak == MFMA_F32_PEAK_TFLOPS else
+                                                                        "ivf_pq_kernel" if pqfs else
                                                                         "prefilter_rb_kernel<lists>" if one_bit else
                                                                         "ivf_sq8_i8_kernel" if per_dim else "ivf_i8_kernel",
-                                                                        kind_name, nprobe - 1), "kernel_ms": kms,
+                                                                        kind_name, "fp32" if peak == MFMA_F32_PEAK_TFLOPS else "int8",
+                                                                        nprobe - 1), "kernel_ms": kms,
                 "ops_per_launch": ops, "distance_evaluations_per_launch": float(rest),
                 "distance_evaluations_per_second": float(rest) / (kms * 1e-3)}
     return env.base_line("QPS @ recall@10 (IVF %s, 10M x 128)" % {"sq4_uniform": "SQ4-uniform", "sq8_uniform": "SQ8-uniform",
-                                                                  "sq8": "SQ8", "rabitq": "RaBitQ", "pqfs": "PQFS"}[kind_name],
-                         "queries/s", nq / sec, sec, "4-bit pq codes, u8 table sums in i32" if pqfs else
+                                                                  "sq8": "SQ8", "rabitq": "RaBitQ", "pqfs": "PQFS", "fp32": "FP32"}[kind_name],
+                         "queries/s", nq / sec, sec, "f32" if raw32 else "4-bit pq codes, u8 table sums in i32" if pqfs else
                          "1-bit codes x u4 queries, i32 popcount sums, f32 estimator" if one_bit else
                          "u8 codes x f32 scale, f32 (pre-selection: i8 x i8, i32 sums)" if per_dim else "u%d codes, i32 dot" % bits,
                          "configs[3]%s: IVF search, N=%d, d=%d, nlist=%d, nprobe=%d, rerank %d, %d queries, k=%d"
@@ -954,7 +964,7 @@ def main():
     ap.add_argument("--chunks", type=int, default=0, help="base chunk override (0 = library default)")
     ap.add_argument("--contraction", type=int, default=0, choices=[-1, 0, 1],
                     help="matrix-core path of the flat scans: -1 never, 0 library default, 1 whenever supported")
-    ap.add_argument("--list-codes", default="sq4_uniform", choices=["sq4_uniform", "sq8_uniform", "sq8", "rabitq", "pqfs"],
+    ap.add_argument("--list-codes", default="sq4_uniform", choices=["sq4_uniform", "sq8_uniform", "sq8", "rabitq", "pqfs", "fp32"],
                     help="c4 only: the quantizer of the posting lists (configs[3] names sq4_uniform)")
     ap.add_argument("--pq-dim", type=int, default=0, help="c4 with --list-codes pqfs: subspaces (default: the dimension)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")

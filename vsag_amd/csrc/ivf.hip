@@ -35,6 +35,8 @@ struct ScanPlanIvf {
     bool planes;              // ... with sq8 codes: two int8 planes per query, records rescored (prefilter_i8.hip)
     bool bits1;               // ... with rabitq codes: expanded bits, records rescored (prefilter_rb.hip)
     bool pq;                  // ... with pqfs codes: one-hot centroid indices against the byte tables (ivf_pq.hip)
+    bool f32;                 // ... with fp32 codes (sq8 beyond 128 dimensions): the fp32 matrix cores, records rescored
+                              // (prefilter.hip)
 };
 
 uint64_t rabitq_query_code_size(uint32_t dim, int metric, int query_bits);
@@ -68,6 +70,11 @@ int launch_ivf_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint3
                   uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st);
 int launch_ivf_clear_gated(uint32_t* gate, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t* partial_cnt,
                            const int32_t* buckets, uint32_t* gpairs, uint32_t gpairs_cap, hipStream_t st);
+bool ivf_f32_supports(const vsag_amd_store* s);
+uint32_t ivf_f32_pairs_per_item();
+int launch_ivf_f32(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, const uint32_t* pair_off,
+                   const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound, uint32_t kcand, float* tau,
+                   uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st);
 int launch_ivf_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
                        uint32_t per_pair, uint64_t* partial, uint32_t* partial_cnt, const uint32_t* bound, hipStream_t st);
 int launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
@@ -958,7 +965,11 @@ plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, 
     p->pq = !p->mfma && !p->planes && !p->bits1 && !p->chunked && nprobe > 1 && scan_contraction_mode(s) >= 0 &&
             ivf_pq_supports(s) && s->residual_centroids_dev == nullptr &&
             npairs * ivf_i8_lists_per_pair() * kcand * 8 <= (8ull << 30);
-    p->mfma = p->mfma || p->planes || p->bits1 || p->pq;
+    // fp32 lists, sq8 lists of more than 128 dimensions: the fp32 matrix cores pre-select, the same exact rescoring.
+    p->f32 = !p->mfma && !p->planes && !p->bits1 && !p->pq && !p->chunked && nprobe > 1 && scan_contraction_mode(s) >= 0 &&
+             ivf_f32_supports(s) && kcand <= ivf_rescore_capacity() &&
+             npairs * ivf_i8_lists_per_pair() * kcand * 8 <= (8ull << 30);
+    p->mfma = p->mfma || p->planes || p->bits1 || p->pq || p->f32;
     if (p->mfma) {
         p->chunks_max = ivf_i8_lists_per_pair();
     }
@@ -1152,9 +1163,16 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
             // Pairs grouped by list once; workgroups of 256 pairs for the matrix cores, then -- for the queries whose
             // lists overflowed -- the streaming kernel's items over the same grouping.
             // ivf_i8.hip: items of 256 pairs, kIvfI8ChunkTiles, kIvfI8Chunks
-            regroup(p0, p1, pairs, p.bits1 ? ivf_rb_pairs_per_item() : p.pq ? ivf_pq_pairs_per_item() : 256U,
+            regroup(p0, p1, pairs,
+                    p.bits1 ? ivf_rb_pairs_per_item() : p.pq ? ivf_pq_pairs_per_item() : p.f32 ? ivf_f32_pairs_per_item() : 256U,
                     p.bits1 ? ivf_rb_chunk_tiles() : 32U, 4U);
-            if (p.pq) {
+            if (p.f32) {
+                VA_TRY(launch_ivf_f32(s, a, nq, nprobe, p0, b.pair_off, b.item_off, b.sorted_pair, b.bound, kcand,
+                                      reinterpret_cast<float*>(b.tq), b.partial, b.partial_cnt, b.gate, st));
+                VA_TRY(launch_ivf_clear_gated(b.gate, nq, nprobe, p0, b.partial_cnt, buckets_dev, b.gpairs,
+                                              kGatedPairsCap, st));
+                VA_TRY(launch_ivf_rescore(s, a, nq, nprobe, p0, kcand, p.chunks_max, b.partial, b.partial_cnt, b.bound, st));
+            } else if (p.pq) {
                 VA_TRY(launch_ivf_pq(s, a, nq, nprobe, p0, kcand, b.pair_off, b.item_off, b.sorted_pair, b.bound, b.tq,
                                      b.partial, b.partial_cnt, b.gate, buckets_dev, b.gpairs, kGatedPairsCap, st));
             } else if (p.bits1) {

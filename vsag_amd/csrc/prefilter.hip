@@ -693,10 +693,11 @@ ivf_rescore_capacity() {
 int
 launch_ivf_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
                    uint32_t per_pair, uint64_t* partial, uint32_t* partial_cnt, const uint32_t* bound, hipStream_t st) {
-    if ((s->kind != VSAG_AMD_KIND_SQ8 && s->kind != VSAG_AMD_KIND_SQ4 && s->kind != VSAG_AMD_KIND_RABITQ) ||
+    if ((s->kind != VSAG_AMD_KIND_SQ8 && s->kind != VSAG_AMD_KIND_SQ4 && s->kind != VSAG_AMD_KIND_RABITQ &&
+         s->kind != VSAG_AMD_KIND_FP32) ||
         kcand > kIvfRescoreGather || s->ids_dev == nullptr) {
-        return fail(VSAG_AMD_INVALID_ARGUMENT, "rescoring of list records: sq8, sq4 or rabitq lists with kcand <= %u only",
-                    kIvfRescoreGather);
+        return fail(VSAG_AMD_INVALID_ARGUMENT,
+                    "rescoring of list records: fp32, sq8, sq4 or rabitq lists with kcand <= %u only", kIvfRescoreGather);
     }
     IvfRescoreArgs r{};
     r.partial = partial;
@@ -708,7 +709,14 @@ launch_ivf_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint
     r.ids = s->ids_dev;
     r.bound = bound;
     const dim3 grid(static_cast<uint32_t>(nq));
-    if (s->kind == VSAG_AMD_KIND_RABITQ) {
+    if (s->kind == VSAG_AMD_KIND_FP32) {
+        // (cosine stores hold normalised vectors and scan as inner product)
+        if (s->metric == VSAG_AMD_METRIC_L2) {
+            hipLaunchKernelGGL((ivf_rescore_kernel<VSAG_AMD_KIND_FP32, VSAG_AMD_METRIC_L2>), grid, dim3(kWave), 0, st, a, r);
+        } else {
+            hipLaunchKernelGGL((ivf_rescore_kernel<VSAG_AMD_KIND_FP32, VSAG_AMD_METRIC_IP>), grid, dim3(kWave), 0, st, a, r);
+        }
+    } else if (s->kind == VSAG_AMD_KIND_RABITQ) {
         if (s->metric == VSAG_AMD_METRIC_L2) {
             hipLaunchKernelGGL((ivf_rescore_kernel<VSAG_AMD_KIND_RABITQ, VSAG_AMD_METRIC_L2>), grid, dim3(kWave), 0, st, a, r);
         } else {
@@ -725,6 +733,342 @@ launch_ivf_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint
     } else {
         hipLaunchKernelGGL((ivf_rescore_kernel<VSAG_AMD_KIND_SQ8, VSAG_AMD_METRIC_IP>), grid, dim3(kWave), 0, st, a, r);
     }
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
+// ---- fp32 (and sq8 of any dimension) posting lists against large batches ------------------------------------------
+// The contraction of prefilter_kernel over the (query, list) pairs of an ivf search that the streaming kernel has already
+// given a bound (the probe columns behind the nearest list; ivf_i8.hip describes the work split this kernel shares: the
+// pairs are grouped by list, a work item = a chunk of a list's tiles x up to 128 of the pairs that probe the list).
+// The B operand rows of an item are whatever queries probe the list, fetched through the pair table.  What passes is
+// recorded as a tile slot in the private list (pair, chunk, which 64 codes of the 128-code tile) -- the lists the
+// streaming kernel's partial results use -- and turned into a (distance, id) key by ivf_rescore_kernel.
+constexpr uint32_t kIvfF32Pairs = PN;
+constexpr uint32_t kIvfF32ChunkTiles = 32;  // as ivf_i8.hip: kIvfI8ChunkTiles, kIvfI8Chunks
+constexpr uint32_t kIvfF32Chunks = 4;
+
+struct IvfF32Args {
+    const uint4* tiles;
+    uint32_t G;
+    const float* scale;             // sq8, l2: y_d = c_d * scale_d; null: y_d = c_d
+    const float* qtab;
+    uint32_t qstride;
+    uint32_t kdim;
+    const float* term;              // per slot |y|^2
+    float term_factor, dot_factor;  // as PrefilterArgs
+    const float* tau;               // per query
+    const uint32_t* list_tile;      // per list: first tile, end tile
+    const uint32_t* pair_off;       // pairs of list b: sorted_pair[pair_off[b] .. pair_off[b + 1])
+    const uint32_t* item_off;       // items of list b: item_off[b] .. item_off[b + 1]
+    const uint32_t* sorted_pair;    // query * nprobe + column
+    uint32_t nlist, nprobe;
+    uint64_t nq;
+    uint32_t k;                     // records per private list
+    uint64_t* partial;
+    uint32_t* partial_cnt;          // zero before the launch; may end above k (overflow: the query is gated)
+    uint32_t* gate;                 // nq + 2 words as in ivf_i8.hip
+};
+
+template <int KIND>
+__global__ void __launch_bounds__(256, 3)
+ivf_f32_kernel(IvfF32Args p) {
+    __shared__ PfStage stage[1];
+    __shared__ float code_term[PM];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    const uint32_t wave = tid >> 6;
+    const uint32_t wm = wave & 1;
+    const uint32_t wn = wave >> 1;
+    const uint32_t half = lane >> 5;
+    const uint32_t l32 = lane & 31;
+    const uint32_t item = blockIdx.x;
+    const cu32_p ioff = as_const(p.item_off);
+    if (item >= ioff[p.nlist]) {
+        return;  // the whole workgroup
+    }
+    uint32_t lo_b = 0, hi_b = p.nlist;
+    while (hi_b - lo_b > 1) {
+        const uint32_t mid = (lo_b + hi_b) >> 1;
+        if (ioff[mid] <= item) {
+            lo_b = mid;
+        } else {
+            hi_b = mid;
+        }
+    }
+    const uint32_t b = lo_b;
+    const uint32_t list_begin = as_const(p.list_tile)[2 * b], list_end = as_const(p.list_tile)[2 * b + 1];
+    uint32_t chunks = (list_end - list_begin + kIvfF32ChunkTiles - 1) / kIvfF32ChunkTiles;
+    chunks = chunks < kIvfF32Chunks ? chunks : kIvfF32Chunks;
+    if (chunks == 0) {
+        return;
+    }
+    const uint32_t per = (list_end - list_begin + chunks - 1) / chunks;
+    const uint32_t chunk = (item - ioff[b]) % chunks;
+    const uint32_t group = (item - ioff[b]) / chunks;
+    uint32_t tile_begin = list_begin + chunk * per;
+    tile_begin = tile_begin < list_end ? tile_begin : list_end;
+    const uint32_t tile_end = tile_begin + per < list_end ? tile_begin + per : list_end;
+    const uint32_t pbeg = as_const(p.pair_off)[b] + group * kIvfF32Pairs;
+    const uint32_t pend = as_const(p.pair_off)[b + 1];
+    const uint32_t mtiles = (tile_end - tile_begin + 1) / 2;
+    if (mtiles == 0 || pbeg >= pend) {
+        return;
+    }
+    const uint32_t ktiles = (p.kdim + PK - 1) / PK;
+
+    // Query loader roles as in prefilter_kernel; the rows are the queries of this item's pairs.
+    uint32_t qc[2];
+    uint64_t qsrc[2];
+    uint32_t qrow[2];
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+        const uint32_t idx = tid + 256 * r;
+        qrow[r] = idx >> 2;
+        qc[r] = idx & 3;
+        const uint32_t at = pbeg + qrow[r];
+        qsrc[r] = at < pend ? as_const(p.sorted_pair)[at] / p.nprobe : p.nq;  // p.nq: no such row, zeros
+    }
+    float tau_n[2];
+    uint32_t pair_n[2], query_n[2];
+    bool live[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint32_t at = pbeg + wn * 64 + j * 32 + l32;
+        live[j] = at < pend;
+        pair_n[j] = live[j] ? as_const(p.sorted_pair)[at] : 0U;
+        query_n[j] = pair_n[j] / p.nprobe;
+        tau_n[j] = live[j] ? p.tau[query_n[j]] : -__builtin_inff();
+    }
+
+    const uint32_t crow = tid & 127;
+    const uint32_t cpart = tid >> 7;
+    auto code_granule = [&](uint32_t mt, uint32_t j) {
+        const uint32_t tile = tile_begin + 2 * mt + (crow >> 6);
+        if (tile < tile_end && j < p.G) {
+            return p.tiles[(static_cast<uint64_t>(tile) * p.G + j) * kWave + (crow & 63)];
+        }
+        return make_uint4(0, 0, 0, 0);
+    };
+    constexpr int kCodeRegs = KIND == VSAG_AMD_KIND_SQ8 ? 1 : 4;
+    auto fetch_codes = [&](uint32_t mt, uint32_t kt, uint4 (&regs)[kCodeRegs]) {
+        if constexpr (KIND == VSAG_AMD_KIND_SQ8) {
+            regs[0] = code_granule(mt, 2 * kt + cpart);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                regs[2 * r] = code_granule(mt, 8 * kt + 2 * (cpart + 2 * r));
+                regs[2 * r + 1] = code_granule(mt, 8 * kt + 2 * (cpart + 2 * r) + 1);
+            }
+        }
+    };
+    auto as_floats = [](uint4 v) {
+        return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w));
+    };
+    auto park_codes = [&](float4* plane, uint32_t kt, const uint4 (&regs)[kCodeRegs]) {
+        if constexpr (KIND == VSAG_AMD_KIND_SQ8) {
+            const uint32_t w[4] = {regs[0].x, regs[0].y, regs[0].z, regs[0].w};
+            const uint32_t d0 = PK * kt + 16 * cpart;
+            float4 v[4];
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                v[m] = make_float4(static_cast<float>(w[m] & 0xffU), static_cast<float>((w[m] >> 8) & 0xffU),
+                                   static_cast<float>((w[m] >> 16) & 0xffU), static_cast<float>(w[m] >> 24));
+                if (p.scale != nullptr && d0 + 16 <= p.kdim) {
+                    float4 sc = *reinterpret_cast<const float4*>(p.scale + d0 + 4 * m);
+                    v[m].x *= sc.x;
+                    v[m].y *= sc.y;
+                    v[m].z *= sc.z;
+                    v[m].w *= sc.w;
+                }
+            }
+            pf_stage_store8(plane, crow, 2 * cpart, v[0], v[1]);
+            pf_stage_store8(plane, crow, 2 * cpart + 1, v[2], v[3]);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                pf_stage_store8(plane, crow, cpart + 2 * r, as_floats(regs[2 * r]), as_floats(regs[2 * r + 1]));
+            }
+        }
+    };
+    uint4 rc[kCodeRegs];
+    float4 rq[4];
+    auto fetch_queries = [&](uint32_t kt) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            rq[2 * r] = pf_query_chunk(p.qtab, qsrc[r], p.nq, PK * kt + 8 * qc[r], p.qstride);
+            rq[2 * r + 1] = pf_query_chunk(p.qtab, qsrc[r], p.nq, PK * kt + 8 * qc[r] + 4, p.qstride);
+        }
+    };
+    auto park_queries = [&](float4* plane) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            pf_stage_store8(plane, qrow[r], qc[r], rq[2 * r], rq[2 * r + 1]);
+        }
+    };
+    fetch_codes(0, 0, rc);
+    fetch_queries(0);
+    for (uint32_t mt = 0; mt < mtiles; ++mt) {
+        floatx16 acc[2][2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    acc[i][j][e] = 0.0F;
+                }
+            }
+        }
+        const uint64_t slot0 = (static_cast<uint64_t>(tile_begin) + 2 * mt) * kWave;
+        park_codes(stage[0].a, 0, rc);
+        park_queries(stage[0].b);
+        float my_term = 0.0F;
+        if (tid < PM) {
+            const bool real = tile_begin + 2 * mt + (tid >> 6) < tile_end;
+            my_term = real ? p.term_factor * p.term[slot0 + tid] : __builtin_inff();
+        }
+        __syncthreads();
+        for (uint32_t kt = 0; kt < ktiles; ++kt) {
+            if (kt + 1 < ktiles) {
+                fetch_codes(mt, kt + 1, rc);
+                fetch_queries(kt + 1);
+            } else if (mt + 1 < mtiles) {
+                fetch_codes(mt + 1, 0, rc);
+                fetch_queries(0);
+            }
+            const float4* pa = stage[0].a + half * 4 * kPfPlane + wm * 64 + l32;
+            const float4* pb = stage[0].b + half * 4 * kPfPlane + wn * 64 + l32;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                float4 a0 = pa[c * kPfPlane];
+                float4 a1 = pa[c * kPfPlane + 32];
+                float4 b0 = pb[c * kPfPlane];
+                float4 b1 = pb[c * kPfPlane + 32];
+                const float av0[4] = {a0.x, a0.y, a0.z, a0.w};
+                const float av1[4] = {a1.x, a1.y, a1.z, a1.w};
+                const float bv0[4] = {b0.x, b0.y, b0.z, b0.w};
+                const float bv1[4] = {b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[e], bv0[e], acc[0][0], 0, 0, 0);
+                    acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av0[e], bv1[e], acc[0][1], 0, 0, 0);
+                    acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[e], bv0[e], acc[1][0], 0, 0, 0);
+                    acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(av1[e], bv1[e], acc[1][1], 0, 0, 0);
+                }
+            }
+            if (kt + 1 == ktiles && tid < PM) {
+                code_term[tid] = my_term;
+            }
+            __syncthreads();
+            if (kt + 1 < ktiles) {
+                park_codes(stage[0].a, kt + 1, rc);
+                park_queries(stage[0].b);
+                __syncthreads();
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            uint32_t hits = 0;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const uint32_t ml = wm * 64 + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+                    const float v = code_term[ml] + p.dot_factor * acc[i][j][e];
+                    hits |= (v <= tau_n[j] ? 1U : 0U) << (16 * i + e);
+                }
+            }
+            if (hits != 0 && live[j]) {
+                const uint64_t list = (static_cast<uint64_t>(pair_n[j]) * kIvfF32Chunks + chunk) * 2 + wm;
+                while (hits != 0) {
+                    const uint32_t bit = static_cast<uint32_t>(__builtin_ctz(hits));
+                    hits &= hits - 1;
+                    const uint32_t i = bit >> 4, e = bit & 15;
+                    const uint32_t ml = wm * 64 + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+                    const uint32_t pos = atomicAdd(&p.partial_cnt[list], 1U);
+                    if (pos < p.k) {
+                        p.partial[list * p.k + pos] = slot0 + ml;
+                    } else if (pos == p.k) {
+                        if (atomicExch(&p.gate[query_n[j]], 1U) == 0U) {
+                            atomicAdd(&p.gate[p.nq], 1U);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// counts[i] = min(counts[i], k): the lists of ivf_f32_kernel are counted with atomics that run past the capacity.
+__global__ void
+clamp_counts_kernel(uint32_t* counts, uint64_t n, uint32_t k) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n && counts[i] > k) {
+        counts[i] = k;
+    }
+}
+
+bool
+ivf_f32_supports(const vsag_amd_store* s) {
+    return (s->kind == VSAG_AMD_KIND_FP32 || s->kind == VSAG_AMD_KIND_SQ8) && s->nlist > 0 && s->pf_term != nullptr &&
+           s->pf_ymax != nullptr && s->residual_centroids_dev == nullptr && s->ids_dev != nullptr;
+}
+
+uint32_t
+ivf_f32_pairs_per_item() {
+    return kIvfF32Pairs;
+}
+
+// Thresholds from the bounds (tau: nq floats), then the candidates of probe columns [p0, nprobe) grouped by list
+// (pair_off, sorted_pair; item_off counted with ivf_f32_pairs_per_item() pairs per item) into the private lists
+// (pair * 8 + chunk * 2 + half tile) of kcand records in `partial`; partial_cnt zero before.  gate: nq + 2 words.
+int
+launch_ivf_f32(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, const uint32_t* pair_off,
+               const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound, uint32_t kcand, float* tau,
+               uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st) {
+    const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
+    const bool sq8 = s->kind == VSAG_AMD_KIND_SQ8;
+    hipLaunchKernelGGL(prefilter_tau_kernel, dim3(static_cast<uint32_t>(nq)), dim3(kWave), 0, st,
+                       reinterpret_cast<const float*>(a.qtab), a.qstride, s->dpad, sq8 && !l2 ? a.qmeta : nullptr,
+                       a.qmeta_stride, l2 ? 1 : 0, bound, s->pf_ymax, nq, tau);
+    IvfF32Args p{};
+    p.tiles = s->tiles;
+    p.G = s->G;
+    p.scale = sq8 && l2 ? s->scale_dev : nullptr;
+    p.qtab = reinterpret_cast<const float*>(a.qtab);
+    p.qstride = a.qstride;
+    p.kdim = s->dpad;
+    p.term = s->pf_term;
+    p.term_factor = l2 ? 1.0F : 0.0F;
+    p.dot_factor = l2 ? -2.0F : -1.0F;
+    p.tau = tau;
+    p.list_tile = s->list_tile_dev;
+    p.pair_off = pair_off;
+    p.item_off = item_off;
+    p.sorted_pair = sorted_pair;
+    p.nlist = s->nlist;
+    p.nprobe = nprobe;
+    p.nq = nq;
+    p.k = kcand;
+    p.partial = partial;
+    p.partial_cnt = partial_cnt;
+    p.gate = gate;
+    const uint64_t pairs = nq * (nprobe - p0);
+    const uint64_t max_items =
+        (div_up(pairs, static_cast<uint64_t>(kIvfF32Pairs)) + std::min<uint64_t>(s->nlist, pairs)) * kIvfF32Chunks;
+    const dim3 grid(static_cast<uint32_t>(max_items));
+    timing_begin(st);
+    if (sq8) {
+        hipLaunchKernelGGL(ivf_f32_kernel<VSAG_AMD_KIND_SQ8>, grid, dim3(256), 0, st, p);
+    } else {
+        hipLaunchKernelGGL(ivf_f32_kernel<VSAG_AMD_KIND_FP32>, grid, dim3(256), 0, st, p);
+    }
+    timing_end(st);
+    VA_HIP(hipGetLastError());
+    const uint64_t lists = nq * nprobe * 2 * kIvfF32Chunks;
+    hipLaunchKernelGGL(clamp_counts_kernel, dim3(static_cast<uint32_t>(div_up(lists, 256))), dim3(256), 0, st, partial_cnt,
+                       lists, kcand);
     VA_HIP(hipGetLastError());
     return 0;
 }

@@ -828,11 +828,12 @@ append_to_lists(vsag_amd_store* s, const uint8_t* codes_dev, const int32_t* labe
     VA_HIP(hipStreamSynchronize(st));
     s->ntiles = used;
     s->n += n;
-    // The per-slot terms of the int8 pass over sq8 lists (ivf_i8.hip): recomputed over the whole buffer, which costs a
-    // pass over the codes (0.4 ms for ten million of them) against the classification and encoding an append has
-    // behind it already.
-    if ((s->kind == VSAG_AMD_KIND_SQ8 || s->kind == VSAG_AMD_KIND_SQ4) && s->pf_ymax != nullptr && s->dpad <= 128 &&
-        s->residual_centroids_dev == nullptr) {
+    // The per-slot terms of the matrix-core passes over sq8 / sq4 lists (prefilter_i8.hip) and over fp32 and longer sq8
+    // lists (prefilter.hip): recomputed over the whole buffer, which costs a pass over the codes (0.4 ms for ten million
+    // sq8 codes) against the classification and encoding an append has behind it already.
+    const bool list_terms = s->kind == VSAG_AMD_KIND_FP32 || s->kind == VSAG_AMD_KIND_SQ8 ||
+                            (s->kind == VSAG_AMD_KIND_SQ4 && s->dpad <= 128);
+    if (list_terms && s->pf_ymax != nullptr && s->residual_centroids_dev == nullptr) {
         const uint64_t slots = s->cap_tiles * kWave;
         if (s->pf_term == nullptr || s->pf_term_slots < slots) {
             if (s->pf_term != nullptr) {
