@@ -9,6 +9,8 @@ import json
 import struct
 import zlib
 
+import os
+
 import numpy as np
 import pytest
 
@@ -106,8 +108,9 @@ def test_brute_force_sq8_layout_field_by_field(lib, tmp_path):
     idx.serialize(path)
     data = path.read_bytes()
     meta, foot = footer_of(data)
-    assert meta["basic_info"] == {"dim": d, "extra_info_size": 0, "has_extra_info": False, "is_multi_vector": False,
-                                  "total_count": n}
+    info = dict(meta["basic_info"])
+    assert json.loads(info.pop("index_param"))["base_codes"]["quantization_params"] == {"type": "sq8"}
+    assert info == {"dim": d, "extra_info_size": 0, "has_extra_info": False, "is_multi_vector": False, "total_count": n}
     c = Cursor(data)
     total, cap, code_size = c.take("III")  # FlattenInterface::Serialize
     assert (total, code_size) == (n, d) and cap >= n
@@ -344,6 +347,10 @@ def test_deserialize_errors(lib, tmp_path):
     fresh = make("brute_force", d, "l2")
     fresh.deserialize(tmp_path / "empty.index")
     assert fresh.get_num_elements() == 0
+    # a device that takes no bytes: the write (at the latest the closing flush) fails, and the call says so
+    if os.path.exists("/dev/full"):
+        with pytest.raises(pyvsag.VsagError):
+            a.serialize("/dev/full")
     a.close()
 
 
@@ -381,3 +388,114 @@ def test_ivf_pqfs_bucket_cell_holds_packaged_blocks(lib, tmp_path):
         seen.append(ids)
     assert np.array_equal(np.sort(np.concatenate(seen)), np.arange(n, dtype=np.uint32))
     idx.close()
+
+
+def _reparam(data, edit):
+    """The same stream with its index_param edited (edit(dict) -> dict or None to drop it) and the footer rewritten."""
+    meta, start = footer_of(data)
+    info = meta["basic_info"]
+    param = edit(json.loads(info["index_param"]))
+    if param is None:
+        del info["index_param"]
+    else:
+        info["index_param"] = json.dumps(param, separators=(",", ":"))
+    return with_footer(data[:start], meta)
+
+
+def test_index_param_in_the_footer_and_its_compatibility_check(lib, tmp_path):
+    """basic_info carries index_param, the creating parameters in the reference's internal form (ivf.cpp:1045,
+    bruteforce.cpp:703); a reader refuses a file whose parameters its own are not compatible with
+    (ivf.cpp:1201-1208 with IVFParameter::CheckCompatibility, ivf_parameter.cpp:133-148; bruteforce.cpp:887-891) and
+    reads a file without the field (older writers)."""
+    n, d = 1500, 32
+    x = vectors(n, d)
+    labels = np.arange(n, dtype=np.int64)
+    params = dict(buckets_count=10, base_quantization_type="sq8", use_reorder=True, precise_quantization_type="fp32",
+                  train_sample_count=1500)
+    a = make("ivf", d, "l2", **params)
+    a.build(x, labels, n, d)
+    path = tmp_path / "ivf.index"
+    a.serialize(path)
+    data = path.read_bytes()
+    meta, _ = footer_of(data)
+    p = json.loads(meta["basic_info"]["index_param"])
+    assert p["type"] == "ivf" and p["use_reorder"] is True and p["reorder_source"] == "precise"
+    assert p["buckets_params"] == {"buckets_count": 10, "io_params": {"type": "memory_io"},
+                                   "quantization_params": {"type": "sq8"}, "use_residual": False}
+    assert p["precise_codes"]["quantization_params"] == {"type": "fp32"} and p["precise_codes"]["codes_type"] == "flatten"
+    assert p["partition_strategy"]["partition_strategy_type"] == "ivf" and p["partition_strategy"]["ivf_train_type"] == "kmeans"
+    assert p["precise_codes_layout"] == "flat" and p["buckets_per_data"] == 1 and p["graph_build_threshold"] == 0
+    q = vectors(10, d, seed=3)
+    search = json.dumps({"ivf": {"scan_buckets_count": 10, "factor": 2.0}})
+
+    def load(blob, **override):
+        f = tmp_path / "edited.index"
+        f.write_bytes(blob)
+        b = make("ivf", d, "l2", **{**params, **override})
+        try:
+            b.deserialize(f)
+            return b
+        except pyvsag.VsagError:
+            b.close()
+            raise
+
+    # unchanged, and without the field: read
+    for blob in (data, _reparam(data, lambda p: None)):
+        b = load(blob)
+        assert same_results(a, b, q, 5, search)
+        b.close()
+    # every field the reference compares, one at a time
+    def edited(path_keys, value):
+        def edit(p):
+            node = p
+            for key in path_keys[:-1]:
+                node = node[key]
+            node[path_keys[-1]] = value
+            return p
+        return _reparam(data, edit)
+    for keys, value in ((("buckets_params", "quantization_params", "type"), "sq4"), (("buckets_params", "buckets_count"), 11),
+                        (("buckets_params", "use_residual"), True), (("precise_codes", "quantization_params", "type"), "sq8"),
+                        (("use_reorder",), False), (("reorder_source",), "base"), (("use_attribute_filter",), True),
+                        (("label_remap_type",), "robin"), (("precise_codes_layout",), "bucket"), (("buckets_per_data",), 2),
+                        (("graph_build_threshold",), 100), (("partition_strategy", "partition_strategy_type"), "gno_imi"),
+                        (("partition_strategy", "route_max_degree"), 32)):
+        with pytest.raises(pyvsag.VsagError) as e:
+            load(edited(keys, value))
+        assert e.value.code == -3 and "IVF index parameter not match, current: " in e.value.message, (keys, e.value.message)
+    # fields it does not compare do not matter
+    for keys, value in ((("train_sample_count",), 99999), (("build_thread_count",), 8),
+                        (("partition_strategy", "ivf_train_type"), "random")):
+        load(edited(keys, value)).close()
+    a.close()
+
+    # quantizer fields: rabitq bits, pq_dim
+    r = make("ivf", d, "l2", buckets_count=4, base_quantization_type="rabitq", rabitq_bits_per_dim_base=4, train_sample_count=1500)
+    r.build(x, labels, n, d)
+    r.serialize(tmp_path / "rabitq.index")
+    rp = json.loads(footer_of((tmp_path / "rabitq.index").read_bytes())[0]["basic_info"]["index_param"])
+    assert rp["buckets_params"]["quantization_params"]["rabitq_bits_per_dim_base"] == 4
+    assert rp["buckets_params"]["quantization_params"]["rabitq_bits_per_dim_query"] == 32
+    with pytest.raises(pyvsag.VsagError) as e:
+        make("ivf", d, "l2", buckets_count=4, base_quantization_type="rabitq", rabitq_bits_per_dim_base=2,
+             train_sample_count=1500).deserialize(tmp_path / "rabitq.index")
+    assert e.value.code == -3 and "parameter not match" in e.value.message
+    r.close()
+
+    # brute force
+    bf = make("brute_force", d, "l2", base_quantization_type="sq8")
+    bf.build(x, labels, n, d)
+    bf.serialize(tmp_path / "bf.index")
+    bdata = (tmp_path / "bf.index").read_bytes()
+    bp = json.loads(footer_of(bdata)[0]["basic_info"]["index_param"])
+    assert bp["type"] == "brute_force" and bp["base_codes"]["quantization_params"] == {"type": "sq8"}
+    (tmp_path / "bf_sq4.index").write_bytes(_reparam(bdata, lambda p: {**p, "base_codes": {**p["base_codes"],
+                                                                                             "quantization_params": {"type": "sq4"}}}))
+    with pytest.raises(pyvsag.VsagError) as e:
+        make("brute_force", d, "l2", base_quantization_type="sq8").deserialize(tmp_path / "bf_sq4.index")
+    assert e.value.code == -3 and "BruteForce index parameter not match" in e.value.message
+    (tmp_path / "bf_plain.index").write_bytes(_reparam(bdata, lambda p: None))
+    c = make("brute_force", d, "l2", base_quantization_type="sq8")
+    c.deserialize(tmp_path / "bf_plain.index")
+    assert c.get_num_elements() == n
+    c.close()
+    bf.close()

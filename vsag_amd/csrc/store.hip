@@ -740,6 +740,15 @@ append_to_lists(vsag_amd_store* s, const uint8_t* codes_dev, const int32_t* labe
             VA_HIP(hipGetLastError());
             VA_HIP(hipStreamSynchronize(st));
         }
+        // The tile extents of the codes the lists hold now, at their new places: whatever fails from here on (the id map,
+        // the temporaries and the sort below) leaves a store that a scan can still walk.
+        std::vector<uint32_t> lt_now(2 * static_cast<size_t>(nlist));
+        for (uint32_t l = 0; l < nlist; ++l) {
+            lt_now[2 * l] = begin[l];
+            lt_now[2 * l + 1] = begin[l] + static_cast<uint32_t>(div_up(static_cast<uint64_t>(s->list_sizes[l]), kWave));
+        }
+        VA_HIP(hipMemcpyAsync(lt, lt_now.data(), lt_now.size() * sizeof(uint32_t), hipMemcpyHostToDevice, st));
+        VA_HIP(hipStreamSynchronize(st));
         for (void* p : {static_cast<void*>(s->tiles), static_cast<void*>(s->meta), static_cast<void*>(s->ids_dev),
                         static_cast<void*>(s->list_tile_dev), static_cast<void*>(s->residual_bias_dev)}) {
             if (p != nullptr) {

@@ -414,7 +414,14 @@ vsag_serialize_file(vsag_index_t index, const char* file_path) {
     }
     auto result = vi->index_->Serialize(file);
     file.close();
-    return result.has_value() ? success() : make_error(result.error());
+    if (!result.has_value()) {
+        return make_error(result.error());
+    }
+    if (file.fail()) {
+        // a write or the closing flush did not reach the file (a full disk): the file is truncated
+        return make_error(VSAG_INTERNAL_ERROR, std::string("failed to write file: ") + file_path);
+    }
+    return success();
 }
 
 extern "C" Error_t

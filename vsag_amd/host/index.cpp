@@ -1053,8 +1053,117 @@ constexpr int64_t kMaxDeviceK = 1024;  // largest k of one device scan
 
 const char*
 kind_name(int kind) {
-    static const char* names[] = {"fp32", "sq8", "sq4", "sq4_uniform", "sq8_uniform", "rabitq"};
-    return kind >= 0 && kind <= VSAG_AMD_KIND_RABITQ ? names[kind] : "unknown";
+    static const char* names[] = {"fp32", "sq8", "sq4", "sq4_uniform", "sq8_uniform", "rabitq", "pqfs"};
+    return kind >= 0 && kind <= VSAG_AMD_KIND_PQFS ? names[kind] : "unknown";
+}
+
+// ---- index_param of the footer's basic_info ----
+// The creating parameters in the reference's internal form, as Parameter::ToString() dumps them (ivf.cpp:1045,
+// bruteforce.cpp:703): a reader rebuilds the parameter object from the string and refuses a file whose parameters its
+// own index is not compatible with (ivf.cpp:1201-1208, bruteforce.cpp:887-891).  Written here: the fields those
+// CheckCompatibility functions compare, under the reference's keys (inner_string_params.h).
+
+// QuantizerParameter::ToJson of each kind (fp32_quantizer_parameter.cpp:33-37, scalar_quantizer_parameter.h:54-58,
+// sq4_uniform_quantizer_parameter.cpp:47-52, sq8_uniform_quantizer_parameter.cpp:30-34,
+// rabitq_quantizer_parameter.cpp:116-129, pq_fastscan_quantizer_parameter.cpp:36-41).
+std::string
+quantization_params_json(const Quantizer& q) {
+    std::string s = std::string("{\"type\":\"") + kind_name(q.kind) + "\"";
+    if (q.kind == VSAG_AMD_KIND_SQ4_UNIFORM) {
+        s += ",\"sq4_uniform_trunc_rate\":0.05";
+    } else if (q.kind == VSAG_AMD_KIND_PQFS) {
+        s += ",\"pq_dim\":" + std::to_string(q.pq_dim);
+    } else if (q.kind == VSAG_AMD_KIND_RABITQ) {
+        s += ",\"pca_dim\":0,\"rabitq_version\":\"standard\",\"rabitq_bits_per_dim_query\":" +
+             std::to_string(q.rabitq_query_bits) + ",\"rabitq_bits_per_dim_base\":" + std::to_string(q.rabitq_base_bits) +
+             ",\"rabitq_bits_per_dim_filter\":1,\"rabitq_error_rate\":1.9,\"use_fht\":false,\"fast_encode_rabitq\":" +
+             (q.rabitq_fast_encode ? "true" : "false") +
+             ",\"fast_encode_rabitq_rounds\":" + std::to_string(q.rabitq_fast_rounds);
+    }
+    return s + "}";
+}
+
+// FlattenDataCellParameter::ToJson (flatten_datacell_parameter.cpp:87-97).
+std::string
+flatten_params_json(const Quantizer& q) {
+    return "{\"codes_type\":\"flatten\",\"io_params\":{\"type\":\"block_memory_io\"},\"quantization_params\":" +
+           quantization_params_json(q) + "}";
+}
+
+// A JSON text as the value of a JSON string.
+std::string
+json_quoted(const std::string& text) {
+    std::string s = "\"";
+    for (char c : text) {
+        if (c == '"' || c == '\\') {
+            s += '\\';
+        }
+        s += c;
+    }
+    return s + "\"";
+}
+
+// The CheckCompatibility of the quantizer parameters: the same type, and the fields each kind compares
+// (sq4_uniform_quantizer_parameter.cpp:54-58, rabitq_quantizer_parameter.cpp:131-141,
+// pq_fastscan_quantizer_parameter.cpp:43-48).  Fields a file does not carry are not compared.
+bool
+quantization_params_compatible(const Json& file, const Quantizer& q) {
+    if (!file.IsObject() || !file.Contains("type") || file["type"].GetString() != kind_name(q.kind)) {
+        return false;
+    }
+    auto same_int = [&](const char* key, int64_t mine) { return !file.Contains(key) || file[key].GetInt() == mine; };
+    if (q.kind == VSAG_AMD_KIND_SQ4_UNIFORM && file.Contains("sq4_uniform_trunc_rate") &&
+        std::fabs(file["sq4_uniform_trunc_rate"].GetFloat() - 0.05) > 1e-6) {
+        return false;
+    }
+    if (q.kind == VSAG_AMD_KIND_PQFS && !same_int("pq_dim", q.pq_dim)) {
+        return false;
+    }
+    if (q.kind == VSAG_AMD_KIND_RABITQ) {
+        if (!same_int("rabitq_bits_per_dim_query", q.rabitq_query_bits) ||
+            !same_int("rabitq_bits_per_dim_base", q.rabitq_base_bits) || !same_int("rabitq_bits_per_dim_filter", 1)) {
+            return false;
+        }
+        if (file.Contains("pca_dim") && file["pca_dim"].GetInt() != 0 && file["pca_dim"].GetInt() != q.dim) {
+            return false;
+        }
+        if (file.Contains("rabitq_version") && file["rabitq_version"].GetString() != "standard") {
+            return false;
+        }
+        if (file.Contains("use_fht") && file["use_fht"].GetBool()) {
+            return false;
+        }
+    }
+    return true;
+}
+
+// InnerIndexParameter::CheckCompatibility (inner_index_parameter.cpp:275-286) for an index without attribute filters
+// whose reorder source is its precise codes.
+bool
+inner_params_compatible(const Json& file, bool use_reorder, const Quantizer& precise) {
+    if (file.Contains("use_reorder") && file["use_reorder"].GetBool() != use_reorder) {
+        return false;
+    }
+    if (file.Contains("reorder_source") && file["reorder_source"].GetString() != "precise") {
+        return false;
+    }
+    if (use_reorder && file.Contains("precise_codes")) {
+        const Json& pc = file["precise_codes"];
+        if (pc.Contains("codes_type") && pc["codes_type"].GetString() != "flatten" &&
+            pc["codes_type"].GetString() != "flatten_codes") {
+            return false;
+        }
+        if (pc.Contains("quantization_params") && !quantization_params_compatible(pc["quantization_params"], precise)) {
+            return false;
+        }
+    }
+    if (file.Contains("use_attribute_filter") && file["use_attribute_filter"].GetBool()) {
+        return false;
+    }
+    if (file.Contains("label_remap_type") && file["label_remap_type"].GetString() != "pg") {
+        return false;
+    }
+    return true;
 }
 
 // SearchStatistics::ToJson (src/query_context.h:215-246): distance evaluations of one call by phase and backend.  The
@@ -1904,15 +2013,25 @@ protected:
         return pack_distances(dists, inner, ids, rows, count, topk);
     }
 
+    // BruteForceParameter::ToJson over InnerIndexParameter::ToJson (bruteforce_parameter.cpp:57-63,
+    // inner_index_parameter.cpp:249-274).
+    std::string
+    index_param_json() const {
+        return "{\"base_codes\":" + flatten_params_json(q_) +
+               ",\"build_thread_count\":1,\"label_remap_type\":\"pg\",\"reorder_source\":\"precise\","
+               "\"resize_increase_count_bit\":10,\"store_raw_vector\":false,\"train_sample_count\":65536,"
+               "\"type\":\"brute_force\",\"use_attribute_filter\":false,\"use_reorder\":false}";
+    }
+
     // BruteForce::Serialize (bruteforce.cpp:684-705): the codes' cell, the label table, the footer with basic_info.
-    // index_param is left out of basic_info (a reader checks it only when it is there, bruteforce.cpp:1020-1037).
     void
     save(Writer& w) const override {
         const uint64_t total = labels_.size();
         write_flat_cell(w, store_.s, nullptr, q_, total);
         w.vec(labels_);
         write_footer(w, "{\"_update_time\":\"1970-01-01 00:00:00\",\"basic_info\":{\"dim\":" + std::to_string(q_.dim) +
-                            ",\"extra_info_size\":0,\"has_extra_info\":false,\"is_multi_vector\":false,\"total_count\":" +
+                            ",\"extra_info_size\":0,\"has_extra_info\":false,\"index_param\":" +
+                            json_quoted(index_param_json()) + ",\"is_multi_vector\":false,\"total_count\":" +
                             std::to_string(total) + "}}");
     }
 
@@ -1939,6 +2058,19 @@ protected:
             file_total = static_cast<uint64_t>(info["total_count"].GetInt());
             if (info.Contains("extra_info_size")) {
                 CHECK_ARGUMENT(info["extra_info_size"].GetInt() == 0, "BruteForce index extra_info_size not match");
+            }
+            if (info.Contains("index_param")) {
+                // bruteforce.cpp:887-898 with BruteForceParameter::CheckCompatibility (bruteforce_parameter.cpp:65-73)
+                const std::string text = info["index_param"].GetString();
+                const Json file = Json::Parse(text);
+                bool ok = inner_params_compatible(file, false, q_);
+                if (ok && file.Contains("base_codes")) {
+                    const Json& bc = file["base_codes"];
+                    ok = (!bc.Contains("codes_type") || bc["codes_type"].GetString() == "flatten") &&
+                         (!bc.Contains("quantization_params") ||
+                          quantization_params_compatible(bc["quantization_params"], q_));
+                }
+                CHECK_ARGUMENT(ok, "BruteForce index parameter not match, current: " + index_param_json() + ", new: " + text);
             }
         } else {
             file_dim = r.get<int64_t>();
@@ -2492,11 +2624,72 @@ protected:
             cell("reorder_codes", begin);
         }
         write_footer(w, "{\"_update_time\":\"1970-01-01 00:00:00\",\"basic_info\":{\"data_type\":0,\"dim\":" +
-                            std::to_string(q_.dim) + ",\"extra_info_size\":0,\"is_trained\":" +
+                            std::to_string(q_.dim) + ",\"extra_info_size\":0,\"index_param\":" +
+                            json_quoted(index_param_json()) + ",\"is_trained\":" +
                             (trained_ ? "true" : "false") + ",\"metric\":" + std::to_string(q_.metric) +
                             ",\"total_elements\":" + std::to_string(labels_.size()) + ",\"use_reorder\":" +
                             (use_reorder_ ? "true" : "false") + "},\"datacell_offsets\":" + offsets +
                             "},\"datacell_sizes\":" + sizes + "}}");
+    }
+
+    // IVFParameter::ToJson over InnerIndexParameter::ToJson (ivf_parameter.cpp:121-132, inner_index_parameter.cpp:249-274)
+    // with BucketDataCellParameter::ToJson (bucket_datacell_parameter.cpp:48-55) and
+    // IVFPartitionStrategyParameters::ToJson (ivf_partition_strategy_parameter.cpp:69-88).
+    std::string
+    index_param_json() const {
+        std::string s = "{\"build_thread_count\":1,\"buckets_params\":{\"buckets_count\":" + std::to_string(nlist_) +
+                        ",\"io_params\":{\"type\":\"memory_io\"},\"quantization_params\":" + quantization_params_json(q_) +
+                        ",\"use_residual\":" + (use_residual_ ? "true" : "false") + "},\"buckets_per_data\":" +
+                        std::to_string(bpd_) + ",\"graph_build_threshold\":0,\"label_remap_type\":\"pg\","
+                        "\"partition_strategy\":{\"ivf_train_type\":\"" + (train_random_ ? "random" : "kmeans") +
+                        "\",\"partition_strategy_type\":\"ivf\",\"route_ef_construction\":300,\"route_max_degree\":64}";
+        if (use_reorder_) {
+            s += ",\"precise_codes\":" + flatten_params_json(pq_);
+        }
+        s += ",\"precise_codes_layout\":\"flat\",\"reorder_source\":\"precise\",\"store_raw_vector\":false,"
+             "\"train_sample_count\":" + std::to_string(train_sample_count_) +
+             ",\"type\":\"ivf\",\"use_attribute_filter\":false,\"use_reorder\":" + (use_reorder_ ? "true" : "false") + "}";
+        return s;
+    }
+
+    // IVFParameter::CheckCompatibility (ivf_parameter.cpp:133-148) against the parameters a file carries.
+    bool
+    index_param_compatible(const Json& file) const {
+        if (!inner_params_compatible(file, use_reorder_, pq_)) {
+            return false;
+        }
+        if (file.Contains("precise_codes_layout") && file["precise_codes_layout"].GetString() != "flat") {
+            return false;
+        }
+        if (file.Contains("buckets_per_data") && file["buckets_per_data"].GetInt() != static_cast<int64_t>(bpd_)) {
+            return false;
+        }
+        if (file.Contains("graph_build_threshold") && file["graph_build_threshold"].GetInt() != 0) {
+            return false;
+        }
+        if (file.Contains("buckets_params")) {
+            const Json& bp = file["buckets_params"];
+            if (bp.Contains("quantization_params") && !quantization_params_compatible(bp["quantization_params"], q_)) {
+                return false;
+            }
+            if (bp.Contains("buckets_count") && bp["buckets_count"].GetInt() != static_cast<int64_t>(nlist_)) {
+                return false;
+            }
+            if (bp.Contains("use_residual") && bp["use_residual"].GetBool() != use_residual_) {
+                return false;
+            }
+        }
+        if (file.Contains("partition_strategy")) {
+            const Json& ps = file["partition_strategy"];
+            if (ps.Contains("partition_strategy_type") && ps["partition_strategy_type"].GetString() != "ivf") {
+                return false;
+            }
+            if ((ps.Contains("route_max_degree") && ps["route_max_degree"].GetInt() != 64) ||
+                (ps.Contains("route_ef_construction") && ps["route_ef_construction"].GetInt() != 300)) {
+                return false;
+            }
+        }
+        return true;
     }
 
     // IVF::Deserialize (ivf.cpp:1429-1530), footer form.
@@ -2524,6 +2717,11 @@ protected:
                        "the serialized index has another metric");
         CHECK_ARGUMENT(info["use_reorder"].GetBool() == use_reorder_,
                        "the serialized index and this one differ in use_reorder");
+        if (info.Contains("index_param")) {  // ivf.cpp:1201-1208
+            const std::string text = info["index_param"].GetString();
+            CHECK_ARGUMENT(index_param_compatible(Json::Parse(text)),
+                           "IVF index parameter not match, current: " + index_param_json() + ", new: " + text);
+        }
         CHECK_ARGUMENT(total * bpd_ < VSAG_AMD_INVALID_ID, "the serialized index holds too many postings");
         for (const char* name : {"bucket", "partition_strategy", "label_table"}) {
             CHECK_ARGUMENT(offsets.Contains(name), std::string("the serialized index has no cell ") + name);
@@ -2867,15 +3065,19 @@ private:
     // ivf_nearest_partition.cpp:88-147, exact instead of through the router graph): n x per_row list numbers.
     void
     classify(const float* x_dev, uint64_t n, uint32_t per_row, DevBuf& buckets) const {
+        classify_with(centroid_store_.s, x_dev, n, per_row, buckets);
+    }
+    void
+    classify_with(const vsag_amd_store_t* router, const float* x_dev, uint64_t n, uint32_t per_row, DevBuf& buckets) const {
         buckets.reserve(std::max<size_t>(n * per_row * 4, 4));
         DevBuf d, ws;
         const uint64_t chunk = 65536;
         d.reserve(std::min(n, chunk) * per_row * 4);
         for (uint64_t r0 = 0; r0 < n; r0 += chunk) {
             const uint64_t nr = std::min(chunk, n - r0);
-            const size_t wsb = vsag_amd_ivf_route_workspace_bytes(centroid_store_.s, nr, per_row);
+            const size_t wsb = vsag_amd_ivf_route_workspace_bytes(router, nr, per_row);
             ws.reserve(wsb);
-            dev(vsag_amd_ivf_route(centroid_store_.s, x_dev + r0 * q_.dim, nr, per_row,
+            dev(vsag_amd_ivf_route(router, x_dev + r0 * q_.dim, nr, per_row,
                                    buckets.as<int32_t>() + r0 * per_row, d.as<float>(), ws.p, wsb, nullptr));
         }
         dev(vsag_amd_stream_synchronize(nullptr));
@@ -2967,38 +3169,46 @@ private:
         router.s = cq.make_store();
         dev(vsag_amd_store_append(router.s, centroids.as<uint8_t>(), nlist_, nullptr));
         dev(vsag_amd_stream_synchronize(nullptr));
-        std::swap(centroid_store_.s, router.s);
-        centroids_.release();
-        std::swap(centroids_.p, centroids.p);
-        std::swap(centroids_.bytes, centroids.bytes);
+        // Router, quantizers, lists and precise store are built beside what the index holds and change hands together
+        // at the end: a step that throws leaves the index as it was.
+        Quantizer q = q_.blank();
         if (use_residual_) {
             DevBuf nearest, residuals;
-            classify(sample_dev.as<float>(), sample_n, 1, nearest);
+            classify_with(router.s, sample_dev.as<float>(), sample_n, 1, nearest);
             residuals.reserve(sample.size() * 4);
             dev(vsag_amd_residual_rows(sample_dev.as<float>(), sample_n, q_.dim, q_.metric, nearest.as<int32_t>(),
-                                       centroids_.as<float>(), residuals.as<float>(), nullptr));
-            q_.train(residuals.as<float>(), sample_n);
+                                       centroids.as<float>(), residuals.as<float>(), nullptr));
+            q.train(residuals.as<float>(), sample_n);
         } else {
-            q_.train(sample_dev.as<float>(), sample_n);
+            q.train(sample_dev.as<float>(), sample_n);
         }
         StoreHandle lists;
-        lists.s = q_.make_store();
+        lists.s = q.make_store();
         if (use_residual_) {
-            dev(vsag_amd_store_set_residual(lists.s, centroids_.as<float>(), nlist_, nullptr));
+            dev(vsag_amd_store_set_residual(lists.s, centroids.as<float>(), nlist_, nullptr));
         }
         dev(vsag_amd_store_set_lists(lists.s, nullptr, nullptr, 0, nlist_, nullptr));
-        if (use_reorder_ && pq_.kind != VSAG_AMD_KIND_FP32) {
+        Quantizer pq = pq_.blank();
+        StoreHandle precise;
+        const bool precise_codes = use_reorder_ && pq_.kind != VSAG_AMD_KIND_FP32;
+        if (precise_codes) {
             DevBuf x;
             if (x_all_dev == nullptr) {
                 upload_rows(base, rows, q_.dim, x);
                 x_all_dev = x.as<float>();
             }
-            pq_.train(x_all_dev, n);
-            StoreHandle precise;
-            precise.s = pq_.make_store();
-            std::swap(precise_.s, precise.s);
+            pq.train(x_all_dev, n);
+            precise.s = pq.make_store();
         }
         dev(vsag_amd_stream_synchronize(nullptr));
+        q_.take(q);
+        if (precise_codes) {
+            pq_.take(pq);
+            std::swap(precise_.s, precise.s);
+        }
+        std::swap(centroid_store_.s, router.s);
+        std::swap(centroids_.p, centroids.p);
+        std::swap(centroids_.bytes, centroids.bytes);
         std::swap(lists_.s, lists.s);
         trained_ = true;
     }
