@@ -371,7 +371,8 @@ def test_range_search(lib, name, params, search):
              "precise_quantization_type": "fp32"}, json.dumps({"ivf": {"scan_buckets_count": 16, "factor": 1.5}})),
 ])
 def test_k_above_one_device_scan(lib, name, params, search):
-    """k larger than the 1024 results of one device scan: one query per call, several scans."""
+    """k larger than the 1024 results of one device scan: several scans per query, for one query per call and for a
+    batch (whose rows are the single-query results)."""
     n, d, k = 6000, 16, 2500
     x = vectors(n, d)
     q = vectors(3, d, seed=165)
@@ -379,6 +380,8 @@ def test_k_above_one_device_scan(lib, name, params, search):
     idx = make(name, d, "l2", **params)
     assert idx.build(x, labels, n, d) == 0
     gt, gt_d = ground_truth(x, q, k, "l2")
+    bids, bdists = idx.knn_search_batch(q, k, search)
+    assert bids.shape == (3, k)
     for i in range(3):
         ids, dists = idx.knn_search(q[i], k, search)
         assert ids.size == k and np.unique(ids).size == k
@@ -389,9 +392,14 @@ def test_k_above_one_device_scan(lib, name, params, search):
             np.testing.assert_allclose(dists, gt_d[i], rtol=1e-4, atol=1e-6)
         else:
             assert hit >= 0.9
-    with pytest.raises(pyvsag.VsagError) as e:
-        idx.knn_search_batch(q, k, search)
-    assert e.value.code == -3
+        assert np.array_equal(bids[i], ids) and np.array_equal(bdists[i], dists)
+    # more than the index holds: the rows end with -1 / inf
+    few = make(name, d, "l2", **params)
+    few.build(x[:1500], labels[:1500], 1500, d)
+    fids, fd = few.knn_search_batch(q, 2000, search)
+    assert fids.shape == (3, 2000) and np.all(fids[:, 1500:] == -1) and np.all(np.isinf(fd[:, 1500:]))
+    assert all(np.unique(fids[i, :1500]).size == 1500 for i in range(3)) or params["base_quantization_type"] != "fp32"
+    few.close()
     idx.close()
 
 
@@ -499,6 +507,34 @@ def test_ivf_pqfs_recall_floor_and_conventions(lib, metric, residual):
     for i in range(8):  # batch == serial, bit for bit
         sid, sd = idx.knn_search(q[i], k, search)
         assert np.array_equal(sid, ids[i]) and np.array_equal(sd, dists[i])
+    idx.close()
+
+
+def test_ivf_fp32_cosine_with_residual(lib, tmp_path):
+    """use_residual with fp32 codes under cosine: FP32Quantizer::EncodeOneImpl (fp32_quantizer.cpp:58-72) normalises
+    the residual it is handed, so the lists estimate the angle from the direction of x - c alone; with the fp32
+    reorder behind it the search still finds the neighbours, and a reloaded index answers alike."""
+    n, d, nq, k = 3000, 32, 50, 10
+    x = vectors(n, d)
+    q = vectors(nq, d, seed=165)
+    labels = np.arange(n, dtype=np.int64)
+    params = dict(buckets_count=20, base_quantization_type="fp32", use_residual=True, use_reorder=True,
+                  precise_quantization_type="fp32", train_sample_count=3000)
+    idx = make("ivf", d, "cosine", **params)
+    assert idx.build(x, labels, n, d) == 0
+    gt, _ = ground_truth(x, q, k, "cosine")
+    search = json.dumps({"ivf": {"scan_buckets_count": 20, "factor": 10.0}})
+    ids, dists = idx.knn_search_batch(q, k, search)
+    assert recall(ids, gt, labels) >= 0.9
+    assert np.all(np.diff(dists, axis=1) >= 0)
+    sid, sd = idx.knn_search(q[0], k, search)
+    assert np.array_equal(sid, ids[0]) and np.allclose(sd, dists[0], rtol=1e-5, atol=1e-6)
+    idx.serialize(tmp_path / "res.index")
+    again = make("ivf", d, "cosine", **params)
+    again.deserialize(tmp_path / "res.index")
+    ids2, dists2 = again.knn_search_batch(q, k, search)
+    assert np.array_equal(ids2, ids) and np.array_equal(dists2, dists)
+    again.close()
     idx.close()
 
 

@@ -262,9 +262,9 @@ def test_distances_by_inner_id(lib, metric):
 @pytest.mark.parametrize("kind", ["fp32", "sq8", "sq4u"])
 def test_residual_lists_match_oracle(lib, kind, metric, mname):
     """use_residual (bucket_datacell.h:527-572,594-639): codes of x - c scanned with the list's bias and <q, c> taken
-    off, against the checker's restatement; with fp32 codes that is the plain distance to x again."""
-    if kind == "fp32" and metric == orc.COSINE:
-        pytest.skip("the fp32 quantizer normalises what it stores under cosine: residuals lose their length")
+    off, against the checker's restatement; with fp32 codes that is the plain distance to x again -- except under
+    cosine, where FP32Quantizer::EncodeOneImpl (fp32_quantizer.cpp:58-72) normalises what it is given, the residual
+    too: the stored code is the unit residual and the figure is 1 - <q, r / |r|> - <q, c>, as in the reference."""
     L = lib.load_library()
     rng = np.random.default_rng(41 + metric)
     n, d, nlist, nq, nprobe, kcand = 6000, 48, 29, 19, 7, 40
@@ -278,11 +278,15 @@ def test_residual_lists_match_oracle(lib, kind, metric, mname):
     assert np.array_equal(rb.to_numpy(np.float32, (n, d)).view(np.uint32), res.view(np.uint32))
     qproc = q if metric != orc.COSINE else (q / np.linalg.norm(q, axis=1, keepdims=True)).astype(np.float32)
     lb = diff = None
+    ocodes = None
     if kind == "fp32":
         codes = res.view(np.uint8).reshape(n, 4 * d)
         dec = res
         st = Store(capi.KIND_FP32, metric, d)
         okind = orc.FP32
+        if metric == orc.COSINE:
+            unit = (res / np.linalg.norm(res.astype(np.float64), axis=1, keepdims=True)).astype(np.float32)
+            ocodes = unit.view(np.uint8).reshape(n, 4 * d)
     elif kind == "sq8":
         lb, diff = orc.sq_train(res, 8, metric)
         codes = orc.sq_encode(res, 8, lb, diff, metric)
@@ -312,10 +316,10 @@ def test_residual_lists_match_oracle(lib, kind, metric, mname):
     offsets, order = orc.ivf_build_lists(labels, nlist)
     routed, _ = orc.ivf_route(cent, q, nprobe)
     ids, ds = st.ivf_scan(q, routed, kcand)
-    rids, rds = orc.ivf_scan_residual(okind, metric, d, codes[order], offsets, order, qproc, q, cent,
+    rids, rds = orc.ivf_scan_residual(okind, metric, d, (codes if ocodes is None else ocodes)[order], offsets, order, qproc, q, cent,
                                       None if bias is None else bias[order], routed, kcand, lb=lb, diff=diff)
     assert_topk_close(ids, ds, rids, rds, rtol=2e-4, atol=2e-5, tie_rtol=2e-4, label="residual %s %s" % (kind, mname))
-    if kind == "fp32":
+    if kind == "fp32" and metric != orc.COSINE:
         # closed form: the residual scan of fp32 codes is the plain distance to the original vectors
         plain = Store(capi.KIND_FP32, metric, d)
         plain.set_lists(x.view(np.uint8).reshape(n, 4 * d), labels, nlist)

@@ -1502,6 +1502,44 @@ private:
         return out;
     }
 
+protected:
+    // A batch whose k (or candidate count) is beyond one device scan: the queries one at a time, each through the
+    // scan-after-scan loop a single query takes, assembled into the batch form (k columns, -1 / inf behind a row's end).
+    DatasetPtr
+    search_rows_one_by_one(const DatasetPtr& query, int64_t k, const std::string& parameters, const SearchSpec& spec) const {
+        const int64_t nq = query->GetNumElements();
+        const int64_t dim = query->GetDim();
+        const size_t cells = static_cast<size_t>(nq) * static_cast<size_t>(k);
+        std::unique_ptr<int64_t[]> ids(new int64_t[cells]);
+        std::unique_ptr<float[]> dists(new float[cells]);
+        std::fill(ids.get(), ids.get() + cells, static_cast<int64_t>(-1));
+        std::fill(dists.get(), dists.get() + cells, std::numeric_limits<float>::infinity());
+        std::string stats;
+        for (int64_t i = 0; i < nq; ++i) {
+            auto one = Dataset::Make();
+            one->Owner(false)->Dim(dim)->NumElements(1)->Float32Vectors(query->GetFloat32Vectors() + i * dim);
+            SearchSpec own = spec;
+            std::vector<std::vector<int64_t>> own_buckets(1);
+            if (spec.bucket_ids != nullptr && static_cast<size_t>(i) < spec.bucket_ids->size()) {
+                own_buckets[0] = (*spec.bucket_ids)[static_cast<size_t>(i)];
+                own.bucket_ids = &own_buckets;
+            }
+            const DatasetPtr found = search(one, k, parameters, own);
+            const int64_t count = std::min<int64_t>(found->GetDim(), k);
+            if (found->GetNumElements() == 1 && count > 0) {
+                std::copy(found->GetIds(), found->GetIds() + count, ids.get() + i * k);
+                std::copy(found->GetDistances(), found->GetDistances() + count, dists.get() + i * k);
+            }
+            if (i == 0) {
+                stats = found->GetStatistics();
+            }
+        }
+        auto result = Dataset::Make();
+        result->NumElements(nq)->Dim(k)->Ids(ids.release())->Distances(dists.release())->Owner(true)->Statistics(stats);
+        return result;
+    }
+
+private:
     DatasetPtr
     search_combined(const DatasetPtr& query, int64_t k, const std::string& parameters) const {
         PendingCall mine{query->GetFloat32Vectors(), k, &parameters, nullptr, nullptr, false, false};
@@ -1953,8 +1991,11 @@ protected:
         // k, run scan after scan for one query: what a scan returned is denied to the next one, so the rows come
         // out in ascending order.
         const bool looped = spec.range || k > kMaxDeviceK;
-        CHECK_ARGUMENT(!looped || nq == 1, spec.range ? "range search takes one query"
-                                                      : "k above 1024 is supported for one query per call");
+        CHECK_ARGUMENT(!spec.range || nq == 1, "range search takes one query");
+        if (looped && nq > 1) {
+            lock.unlock();
+            return search_rows_one_by_one(query, k, parameters, spec);
+        }
         auto ctx = pool_.acquire();
         ctx->upload(ctx->queries, query->GetFloat32Vectors(), static_cast<size_t>(nq) * q_.dim * 4);
         DenyMask mask;
@@ -2212,8 +2253,6 @@ public:
         }
         if (use_residual_) {
             CHECK_ARGUMENT(q_.kind != VSAG_AMD_KIND_RABITQ, "the GPU path does not support use_residual with rabitq");
-            CHECK_ARGUMENT(!(q_.kind == VSAG_AMD_KIND_FP32 && q_.metric == VSAG_AMD_METRIC_COSINE),
-                           "the GPU path does not support use_residual with fp32 codes under cosine");
         }
         if (index_param.Contains("partition_strategy_type")) {
             CHECK_ARGUMENT(index_param["partition_strategy_type"].GetString() == "ivf",
@@ -2340,9 +2379,11 @@ protected:
         // after scan for one query, each denied what the earlier ones returned.  With buckets_per_data = b a vector
         // has b postings, so a scan asks for b times the candidates (ivf.cpp:1722-1730).
         const bool looped = spec.range || kcand * bpd_ > kMaxDeviceK;
-        CHECK_ARGUMENT(!looped || nq == 1,
-                       spec.range ? "range search takes one query"
-                                  : "factor * k * buckets_per_data above 1024 is supported for one query per call");
+        CHECK_ARGUMENT(!spec.range || nq == 1, "range search takes one query");
+        if (looped && nq > 1) {
+            lock.unlock();
+            return search_rows_one_by_one(query, k, parameters, spec);
+        }
 
         auto lease = pool_.acquire();
         SearchContext& ctx = *lease;
