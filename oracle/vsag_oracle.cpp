@@ -21,6 +21,18 @@
 //                                          against the fp32 branch on the dequantised query),
 //                                          kmeans_init_pp (numpy restatement with cumsum / searchsorted in
 //                                          float64; k = n picks every row once; coincident rows)
+//   pqfs ................................. pqfs_lookup32 against the reference's compiled PQFastScanLookUp32 and
+//                                          committed vectors; Package32 / Unpack32 by round trip and the mapper
+//                                          order; encode, query table and distance by brute-force argmin and the
+//                                          closed form (table entry = the exact subspace distance within one
+//                                          quantisation step); the reference test's own error bound
+//   multi-bit rabitq ..................... the float x plane / float x code inner products against the reference's
+//                                          compiled RaBitQFloatSplitCodeIP / RaBitQFloatSQIP; the fast encoder on
+//                                          the known input of the reference's test; both encoders against the
+//                                          exhaustive optimum on tiny inputs (the extended one against hand-traced
+//                                          answers of the reference's walk, which is not optimal); zero vectors;
+//                                          the estimator's closed form (ip_obar_q) and a stored vector's self
+//                                          distance
 //   parity unpinned ...................... nothing; what the formulas leave open is the order of fp32
 //                                          operations inside rabitq_dist and the k-means loss (no
 //                                          executable reference class), which the 1e-4 relative
