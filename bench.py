@@ -29,6 +29,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 HBM_PEAK_GBS = 8000.0
 MFMA_F32_PEAK_TFLOPS = 157.3
 MFMA_I8_PEAK_TOPS = 5000.0  # dense int8, published
+MFMA_F6F4_PEAK_TFLOPS = 10100.0  # dense fp6 / fp4, published
 # HBM/fabric bytes of the last-level launch of prefilter_i8_kernel<l2> on configs[1] (profiles/prefilter_i8_sq8_c2.md)
 PROFILE_TRAFFIC_I8_C2 = 235670.3 * 2.00 * 1024 + 60099.9 * 1024
 
@@ -798,8 +799,9 @@ def run_c4(env):
         # (pqfs: a pair is a contraction of the one-hot centroid indices with the byte table, 16 products per subspace)
         ops = 2.0 * (16 * (-(-pq_dim // 32) * 32) if pqfs else -(-d // 32) * 32) * float(rest)
         tops = ops / (kms * 1e-3) / 1e12
-        peak = MFMA_F32_PEAK_TFLOPS if raw32 or (per_dim and d > 128) else MFMA_I8_PEAK_TOPS
-        roof = {"bound": "mfma", "achieved": tops, "peak": peak, "unit": "TFLOP/s" if peak == MFMA_F32_PEAK_TFLOPS else "TOP/s",
+        peak = (MFMA_F32_PEAK_TFLOPS if raw32 or (per_dim and d > 128) else
+                MFMA_F6F4_PEAK_TFLOPS if one_bit else MFMA_I8_PEAK_TOPS)
+        roof = {"bound": "mfma", "achieved": tops, "peak": peak, "unit": "TOP/s" if peak == MFMA_I8_PEAK_TOPS else "TFLOP/s",
                 "frac": tops / peak,
                 # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this launch: profiles/ivf_i8_sq4u_c4.md
                 "traffic": 491061.0 * 2.00 * 1024 + 73550.7 * 1024
@@ -808,7 +810,8 @@ def run_c4(env):
                                                                         "ivf_pq_kernel" if pqfs else
                                                                         "prefilter_rb_kernel<lists>" if one_bit else
                                                                         "ivf_sq8_i8_kernel" if per_dim else "ivf_i8_kernel",
-                                                                        kind_name, "fp32" if peak == MFMA_F32_PEAK_TFLOPS else "int8",
+                                                                        kind_name, "fp32" if peak == MFMA_F32_PEAK_TFLOPS else
+                                                                        "fp4 x fp6" if one_bit else "int8",
                                                                         nprobe - 1), "kernel_ms": kms,
                 "ops_per_launch": ops, "distance_evaluations_per_launch": float(rest),
                 "distance_evaluations_per_second": float(rest) / (kms * 1e-3)}
@@ -928,19 +931,18 @@ def run_c5(env):
             "algorithmic_bytes_per_launch": algo}
     dtype = "1-bit codes x 4-bit queries, u32 popcount"
     if tile >= 64:
-        # The batch was pre-selected on the int8 matrix cores (1-bit codes and 4-bit queries expanded to bytes) and
-        # the survivors rescored with the popcount arithmetic.  The timed kernel is the last level: bpp bytes of
-        # d / 8-byte codes against every query.
+        # The batch was pre-selected on the matrix cores (1-bit codes as fp4, 4-bit queries as fp6, exact sums in
+        # fp32) and the survivors rescored with the popcount arithmetic.  The timed kernel is the last level: bpp
+        # bytes of d / 8-byte codes against every query.
         lcodes = bpp / (d / 8.0)
         ops = 2.0 * lcodes * d * nq
         tops = ops / (kms * 1e-3) / 1e12
-        roof = {"bound": "mfma", "achieved": tops, "peak": MFMA_I8_PEAK_TOPS, "unit": "TOP/s",
-                # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this launch: profiles/prefilter_rb_rabitq_c5.md
-                "frac": tops / MFMA_I8_PEAK_TOPS,
-                "traffic": 1056537.4 * 2.00 * 1024 + 213139.2 * 1024 if (n, d, nq, k) == (5000000, 768, 10000, 10) else None,
-                "kernel": "prefilter_rb_kernel<ip> (int8 MFMA, last level)", "kernel_ms": kms, "ops_per_launch": ops,
+        roof = {"bound": "mfma", "achieved": tops, "peak": MFMA_F6F4_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": tops / MFMA_F6F4_PEAK_TFLOPS,
+                "traffic": None,
+                "kernel": "prefilter_rb_kernel<ip> (fp4 x fp6 MFMA, last level)", "kernel_ms": kms, "ops_per_launch": ops,
                 "codes_per_launch": lcodes}
-        dtype = "1-bit codes x 4-bit queries: int8 MFMA pre-selection, u32 popcount rescoring"
+        dtype = "1-bit codes x 4-bit queries: fp4 x fp6 MFMA pre-selection (exact fp32 sums), u32 popcount rescoring"
     return env.base_line("QPS @ recall@10 (RaBitQ 1-bit scan + rerank 200, 5M x 768)", "queries/s", nq / sec, sec,
                          dtype,
                          "configs[4]: RaBitQ full scan + fp32 rerank of %d, N=%d, d=%d, %d queries, k=%d, IP" %

@@ -216,6 +216,47 @@ def test_rabitq_contraction_equals_streaming(lib, modes, metric, n, d, nq, k, ce
     st.destroy()
 
 
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP])
+def test_rabitq_store_of_many_appends_and_codes_outside_the_pass(lib, modes, metric):
+    """The store keeps its code bits and per-code constants once more for the matrix cores, renewed by every append
+    (also of the tile an earlier append left part full).  Codes the pre-selection's derivation does not cover -- a zero
+    norm, a non-positive error factor, a sum field that is not the number of set bits -- must still come out as the
+    streaming scan has them."""
+    n, d, nq, k = 21000, 200, 200, 30
+    rng = np.random.default_rng(77 + metric)
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    x /= np.linalg.norm(x, axis=1, keepdims=True)
+    g = rng.standard_normal((d, d))
+    rot, r = np.linalg.qr(g)
+    rot = (rot * np.sign(np.diag(r))).astype(np.float32)
+    cen = orc.rabitq_train(x, rot)
+    x[5] = cen @ rot                    # the centroid itself (rotated back): a zero norm after centring
+    codes = orc.rabitq_encode(x, rot, cen, metric)
+    tail = codes[:, -(12 if metric == orc.L2 else 16):].view(np.float32)  # norm, error factor, sum[, raw norm]
+    tail[70, 1] = -0.5                  # a negative error factor
+    tail[131, 2] += 3.0                 # a sum field that is not the set bits
+    tail[4000, 0] = 0.0                 # a zero norm
+    tail[20999, 2] = 0.0
+    st = Store(capi.KIND_RABITQ, metric, d, rot=rot, centroid=cen)
+    at = 0
+    for step in (1, 63, 64, 65, 1000, 37, 12000, 3, n):   # ragged: tiles left part full and filled later
+        end = min(n, at + step)
+        if end > at:
+            st.append(codes[at:end])
+        at = end
+    assert at == n
+    q = rng.standard_normal((nq, d)).astype(np.float32)
+    q /= np.linalg.norm(q, axis=1, keepdims=True)
+    plain, fast, tile = modes(st, q, k)
+    assert tile == 128, "the contraction path did not run"
+    assert same(plain, fast)
+    whole = Store(capi.KIND_RABITQ, metric, d, rot=rot, centroid=cen)
+    whole.append(codes)
+    assert same(plain, whole.flat_scan(q, k))
+    whole.destroy()
+    st.destroy()
+
+
 @pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
 @pytest.mark.parametrize("n,d,nq,k", [(40000, 128, 300, 10), (20001, 100, 129, 100), (5000, 33, 1000, 7),
                                       (70000, 64, 600, 1)])

@@ -1,9 +1,13 @@
 // Pre-selection for large query batches on a flat RaBitQ store (1-bit codes, 4-bit queries, L2 or inner product),
-// on the int8 matrix cores.
+// on the matrix cores.
 //
 // The streaming kernel forms <code bits, 4-bit query> with sixteen and/popcount pairs per code dword and query; that
-// is what bounds it.  The same integer is a contraction of 0/1 bytes with 0..15 bytes, exact on
-// v_mfma_i32_32x32x32_i8.  The estimator that turns it into a distance (distance.h, finish_distances) is, for a given
+// is what bounds it.  The same integer is a contraction of 0/1 values with the values 0..15.  The matrix cores take
+// 4-bit and 6-bit floats at twice the rate of bytes (v_mfma_scale_f32_32x32x64_f8f6f4): a code bit is the fp4 value 1.0
+// or 0, and a query value v goes in as the fp6 (e2m3) value v - 7.5, one of +-0.5 .. +-7.5, all of which that format
+// holds exactly; the fp32 sums of at most 1024 such products are exact, and the contraction comes out as
+// ip - 7.5 x (set bits of the code), which moves the third factor below by 7.5.  The estimator that turns ip into a
+// distance (distance.h, finish_distances) is, for a given
 // query and code, an affine function of that integer with a slope of known sign, so "distance <= bound" is
 // "ip >= thr(query, code)" with
 //
@@ -17,10 +21,11 @@
 // Codes the derivation does not cover (zero norm, non-positive error factor, zero raw norm) are candidates of every
 // query.
 //
-// Work split: the 4-bit queries of a group of 128 are expanded to bytes once and stay in LDS (96 KB for 768
-// dimensions) in the operand order of the instruction; a wave owns storage tiles (64 codes; their bits come a granule
-// at a time, one granule ahead, and are expanded to 0/1 bytes with three vector instructions per nibble) and meets all
-// 128 queries of the group: 8 accumulators, 8 matrix instructions per expanded step.  A workgroup is eight waves,
+// Work split: the 4-bit queries of a group of 128 are turned into fp6 once and stay in LDS (72 KB for 768
+// dimensions) in the operand order of the instruction; a wave owns storage tiles (64 codes; their bits come from the
+// store's copy in operand order, 128 dimensions at a time and one load ahead, and become fp4 with seven vector
+// instructions per 32 dimensions) and meets all
+// 128 queries of the group: 8 accumulators, 8 matrix instructions per step of 64 dimensions.  A workgroup is eight waves,
 // two per SIMD, so that one wave's verdicts run under the other's matrix instructions; no barrier inside the loop.
 // What passes goes into the private list of (query, wave of the grid, lane / 32).
 #include "distance.h"
@@ -35,52 +40,56 @@ void timing_end(hipStream_t st);
 typedef int intx4 __attribute__((ext_vector_type(4)));
 typedef int intx16 __attribute__((ext_vector_type(16)));
 
-constexpr uint32_t kRbQueries = 128;  // queries per workgroup
-constexpr uint32_t kRbMaxG = 8;       // granules per code (1024 dimensions): the query group has to fit the LDS
+typedef int intx8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr uint32_t kRbQueries = 128;  // queries per workgroup; kRbMaxG granules per code: the query group has to fit the LDS
 constexpr uint32_t kRbWaves = 8;      // waves per workgroup, two per SIMD: one multiplies while the other decides
 constexpr uint32_t kRbThreads = kRbWaves * kWave;
-// Largest per-code factors the fp32 threshold takes (A_c, |B_c|; codes beyond them are candidates of every query): the
-// per-query slack below is sized for them.  B_c grows with the square of the data's scale (norm x error factor / 2).
-constexpr float kRbMaxA = 64.0F;
-constexpr float kRbMaxB = 4096.0F;
+constexpr uint32_t kRbWaveFloats = 3 * kWave + 4 * 8;  // LDS floats of a wave's per-code constants
 
-// 4-bit queries as bytes: row q holds, per code dword w, the 32 values of dimensions 32 w ... (dpad bytes per row).
+// The fp6 (e2m3) pattern of v - 7.5 for a 4-bit query value v: sign | exponent (2) | mantissa (3).
+__device__ inline uint32_t
+rb_fp6(uint32_t v) {
+    // magnitudes 0.5, 1.5, ... 7.5 by index: 0.5 = 0.100 x 2^0 (subnormal), 1.5 = 1.100 x 2^0, 2.5 = 1.010 x 2^1,
+    // 3.5 = 1.110 x 2^1, 4.5 = 1.001 x 2^2, 5.5 = 1.011 x 2^2, 6.5 = 1.101 x 2^2, 7.5 = 1.111 x 2^2
+    const uint32_t idx = v >= 8 ? v - 8 : 7 - v;
+    const uint64_t table = 4ULL | (12ULL << 8) | (18ULL << 16) | (22ULL << 24) | (25ULL << 32) | (27ULL << 40) |
+                           (29ULL << 48) | (31ULL << 56);
+    return static_cast<uint32_t>((table >> (8 * idx)) & 63ULL) | (v >= 8 ? 0U : 32U);
+}
+
+// 4-bit queries as fp6: per query row and code dword w, the 32 values of dimensions 32 w ... as 24 bytes, value t in
+// bits 6 t .. 6 t + 5; the first 16 bytes go to qa[q ndw + w], the last 8 to qb[q ndw + w].  Padding rows are zero
+// (the fp6 value 0).
 __global__ void __launch_bounds__(256)
-rabitq_query_bytes_kernel(const uint32_t* qtab, uint32_t qstride, uint32_t ndw, uint64_t nq, uint64_t nq_pad,
-                          uint8_t* qbytes) {
+rabitq_query_f6_kernel(const uint32_t* qtab, uint32_t qstride, uint32_t ndw, uint64_t nq, uint64_t nq_pad, uint4* qa,
+                       uint2* qb) {
     const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= nq_pad * ndw) {
         return;
     }
     const uint64_t q = i / ndw;
     const uint32_t w = static_cast<uint32_t>(i % ndw);
-    uint32_t planes[4] = {0, 0, 0, 0};
+    uint32_t out[6] = {0, 0, 0, 0, 0, 0};
     if (q < nq) {
         const uint4 v = *reinterpret_cast<const uint4*>(qtab + q * qstride + 4 * w);
-        planes[0] = v.x;
-        planes[1] = v.y;
-        planes[2] = v.z;
-        planes[3] = v.w;
-    }
-    uint32_t out[8];
 #pragma unroll
-    for (int b = 0; b < 8; ++b) {
-        uint32_t word = 0;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const uint32_t t = 4 * b + k;
-            const uint32_t val = ((planes[0] >> t) & 1U) | (((planes[1] >> t) & 1U) << 1) | (((planes[2] >> t) & 1U) << 2) |
-                                 (((planes[3] >> t) & 1U) << 3);
-            word |= val << (8 * k);
+        for (uint32_t t = 0; t < 32; ++t) {
+            const uint32_t val = ((v.x >> t) & 1U) | (((v.y >> t) & 1U) << 1) | (((v.z >> t) & 1U) << 2) |
+                                 (((v.w >> t) & 1U) << 3);
+            const uint64_t code = static_cast<uint64_t>(rb_fp6(val)) << ((6 * t) % 32);
+            out[(6 * t) / 32] |= static_cast<uint32_t>(code);
+            if ((6 * t) % 32 > 26) {
+                out[(6 * t) / 32 + 1] |= static_cast<uint32_t>(code >> 32);
+            }
         }
-        out[b] = word;
     }
-    uint4* dst = reinterpret_cast<uint4*>(qbytes + (q * ndw + w) * 32);
-    dst[0] = make_uint4(out[0], out[1], out[2], out[3]);
-    dst[1] = make_uint4(out[4], out[5], out[6], out[7]);
+    qa[i] = make_uint4(out[0], out[1], out[2], out[3]);
+    qb[i] = make_uint2(out[4], out[5]);
 }
 
-// Per query: u1..u4 of the header (u[j * nq_pad + q]).  -inf in u4: everything passes; +inf: nothing does.
+// Per query: u1..u4 of the header and u5 (u[j * nq_pad + q]).  -inf in u4: everything passes; +inf: nothing does.
 __global__ void __launch_bounds__(256)
 rabitq_tau_kernel(const float* qmeta, uint32_t qmeta_stride, const uint32_t* bound, int is_l2, uint32_t dpad, uint64_t nq,
                   uint64_t nq_pad, float* u) {
@@ -88,7 +97,7 @@ rabitq_tau_kernel(const float* qmeta, uint32_t qmeta_stride, const uint32_t* bou
     if (q >= nq_pad) {
         return;
     }
-    float u1 = 0.0F, u2 = 0.0F, u3 = 0.0F, u4 = __builtin_inff();
+    float u1 = 0.0F, u2 = 0.0F, u3 = 0.0F, u4 = __builtin_inff(), u5 = 0.0F;
     if (q < nq) {
         const float* qm = qmeta + q * qmeta_stride;
         const uint32_t b = bound[q];
@@ -119,7 +128,14 @@ rabitq_tau_kernel(const float* qmeta, uint32_t qmeta_stride, const uint32_t* bou
                     const double lower = 1.0 - 1.0e-4;
                     u1 = static_cast<float>(v1 * lower);
                     u2 = static_cast<float>(inv * lower);
-                    u3 = static_cast<float>(v3 * lower);
+                    // Less 7.5: the contraction of the matrix cores is ip - 7.5 x set bits.  The factor of the set bits is
+                    // split: its nearest multiple of 1/4 (u5) is taken off in the accumulators, where set bits x u5 and
+                    // every sum on top of it are exact, and only the rest (u3, at most 1/8) stays in the threshold --
+                    // with it the thresholds of a group of codes differ by little, which the group test lives on.
+                    const double x3 = v3 * lower - 7.5;
+                    const double coarse = rint(x3 * 4.0) * 0.25;
+                    u5 = static_cast<float>(coarse);
+                    u3 = static_cast<float>(x3 - coarse);
                     // The threshold is a chain of three fp32 fma over terms that may cancel: it is off by at most
                     // 3 x 2^-24 of the sum of their magnitudes, whatever it comes to itself.  2^-20 of the largest
                     // magnitudes any code can bring (A_c <= kRbMaxA, |B_c| <= kRbMaxB, set bits <= dpad) is taken off.
@@ -133,16 +149,17 @@ rabitq_tau_kernel(const float* qmeta, uint32_t qmeta_stride, const uint32_t* bou
     u[nq_pad + q] = u2;
     u[2 * nq_pad + q] = u3;
     u[3 * nq_pad + q] = u4;
+    u[4 * nq_pad + q] = u5;
 }
 
 struct PrefilterRbArgs {
-    const uint4* tiles;
+    const uint4* f4tiles;    // the code bits in operand order (store.h)
+    const float4* f4const;   // per slot: A_c, B_c, S_c of the header and the flags
+    const float* f4group;    // per tile: 32 floats, the extremes of the constants over each group of sixteen codes
     uint32_t G;
     uint64_t tile_begin, tile_end;
-    uint64_t n;
-    const uint32_t* meta;  // norm, error factor, set bits, raw norm: meta_stride words apart
-    uint64_t meta_stride;
-    const uint4* qbytes;   // [query][2 G * 4 chunks of 16 bytes]
+    const uint4* qa;       // fp6 queries: [query][4 G code dwords] first 16 bytes of the 24 of a dword's 32 values
+    const uint2* qb;       // and the last 8
     const float* u;        // [4][nq_pad]
     uint64_t nq, nq_pad;
     uint32_t* cand;        // [query][sub_lists][sub_cap]
@@ -151,7 +168,6 @@ struct PrefilterRbArgs {
     uint32_t groups;       // grid x; the grid has groups * kRbWaves waves per query group
     // Posting lists (LISTS): a workgroup is a chunk of a list's tiles x up to 128 of the (query, list) pairs that probe
     // the list -- the work split of ivf_i8.hip with 128 pairs per item -- and its queries are gathered by pair.
-    const uint32_t* ids;          // inner id per tile slot (slots without a code hold VSAG_AMD_INVALID_ID)
     const uint32_t* list_tile;    // 2 nlist: first tile and end of the used tiles of every list
     const uint32_t* pair_off;     // nlist + 1
     const uint32_t* item_off;     // nlist + 1: workgroups per list, prefix sums
@@ -171,10 +187,13 @@ struct PrefilterRbArgs {
 constexpr uint32_t kIvfRbChunkTiles = 128;
 constexpr uint32_t kIvfRbChunks = 4;
 
-__device__ inline int
-rb_spread(uint32_t nibble) {
-    // bit j of the nibble into byte j
-    return static_cast<int>((nibble * 0x00204081U) & 0x01010101U);
+// The fp4 operand of 32 code bits in the store's operand order: register v = elements 8 v .. 8 v + 7, 1.0 = 0b0010.
+__device__ inline intx8
+rb_fp4(uint32_t w) {
+    const uint32_t m = 0x22222222U;
+    intx4 v = intx4{static_cast<int>((w << 1) & m), static_cast<int>(w & m), static_cast<int>((w >> 1) & m),
+                    static_cast<int>((w >> 2) & m)};
+    return __builtin_shufflevector(v, v, 0, 1, 2, 3, -1, -1, -1, -1);
 }
 
 template <int METRIC, bool LISTS = false>
@@ -188,10 +207,12 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
     const uint32_t wave = tid >> 6;
     const uint32_t half = lane >> 5;
     const uint32_t l32 = lane & 31;
-    const uint32_t nchunks = 8 * p.G;  // 16-byte chunks per query row: chunk 2 s + h of step s = code dword s
+    const uint32_t ndw = 4 * p.G;  // code dwords: dword 2 s + h is what half h of the wave brings to step s
     uint64_t q0 = static_cast<uint64_t>(blockIdx.y) * kRbQueries;
-    uint4* qs = rb_lds;                                                           // [chunk][128 queries]
-    float* cc = reinterpret_cast<float*>(rb_lds + nchunks * kRbQueries) + wave * 3 * kWave;  // [3][64] per wave
+    uint4* qs = rb_lds;                                                  // [dword][128 queries]: 16 of its 24 bytes
+    uint2* qt = reinterpret_cast<uint2*>(rb_lds + ndw * kRbQueries);     // [dword][128 queries]: the other 8
+    float* cc = reinterpret_cast<float*>(qt + ndw * kRbQueries) + wave * kRbWaveFloats;  // [3][64] per wave
+    float* cg = cc + 3 * kWave;  // then [4 groups of 16 codes][8]: the extremes of the three constants
     uint64_t tile_first = p.tile_begin, span = p.tile_end - p.tile_begin;
     uint64_t t_first = static_cast<uint64_t>(blockIdx.x) * kRbWaves + wave, t_step = static_cast<uint64_t>(p.groups) * kRbWaves;
 
@@ -256,31 +277,42 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
     if constexpr (LISTS) {
         // A list item lives for a few tiles per wave only: the rows are fetched four loads at a time, so that the
         // gather takes a few memory round trips instead of one per 16 bytes.
-        const uint32_t total = nchunks * kRbQueries;
+        const uint32_t total = ndw * kRbQueries;
         for (uint32_t i0 = tid; i0 < total; i0 += 4 * blockDim.x) {
             uint4 v[4];
+            uint2 t[4];
 #pragma unroll
             for (uint32_t r = 0; r < 4; ++r) {
                 const uint32_t i = i0 + r * blockDim.x;
                 const uint32_t ic = i < total ? i : total - 1;
-                v[r] = p.qbytes[query_row(ic / nchunks) * nchunks + ic % nchunks];
+                const uint64_t at = query_row(ic / ndw) * ndw + ic % ndw;
+                v[r] = p.qa[at];
+                t[r] = p.qb[at];
             }
 #pragma unroll
             for (uint32_t r = 0; r < 4; ++r) {
                 const uint32_t i = i0 + r * blockDim.x;
                 if (i < total) {
-                    qs[(i % nchunks) * kRbQueries + i / nchunks] = v[r];
+                    qs[(i % ndw) * kRbQueries + i / ndw] = v[r];
+                    qt[(i % ndw) * kRbQueries + i / ndw] = t[r];
                 }
             }
         }
     } else {
-        for (uint32_t i = tid; i < nchunks * kRbQueries; i += blockDim.x) {
-            const uint32_t ql = i / nchunks, c = i % nchunks;
-            qs[c * kRbQueries + ql] = p.qbytes[query_row(ql) * nchunks + c];
+        for (uint32_t i = tid; i < ndw * kRbQueries; i += blockDim.x) {
+            const uint32_t ql = i / ndw, c = i % ndw;
+            const uint64_t at = query_row(ql) * ndw + c;
+            qs[c * kRbQueries + ql] = p.qa[at];
+            qt[c * kRbQueries + ql] = p.qb[at];
         }
     }
-    float u1[4], u2[4], u3[4], u4[4];
-    uint32_t ncand[4] = {0, 0, 0, 0};
+    float u1[4], u2[4], u3[4], u4[4], u5n[4];
+    // Candidates so far of this lane's four queries (flat stores): in LDS, the registers go to the accumulators.
+    uint32_t* ncand = reinterpret_cast<uint32_t*>(cc - wave * kRbWaveFloats + kRbWaves * kRbWaveFloats) + tid;
+#pragma unroll
+    for (int qb = 0; qb < 4; ++qb) {
+        ncand[qb * kRbThreads] = 0;
+    }
     const uint32_t sub_lists = p.groups * 2 * kRbWaves;
     const uint32_t my_sub = (blockIdx.x * kRbWaves + wave) * 2 + half;
 #pragma unroll
@@ -290,6 +322,7 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
         u2[qb] = p.u[p.nq_pad + q];
         u3[qb] = p.u[2 * p.nq_pad + q];
         u4[qb] = p.u[3 * p.nq_pad + q];
+        u5n[qb] = -p.u[4 * p.nq_pad + q];
     }
     __syncthreads();
     // LISTS: a pair has eight private lists (two per chunk in ivf_i8.hip's layout); here a hit goes to the one of
@@ -308,110 +341,136 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
         }
     };
 
+    // A tile's constants and the first of its bits are asked for one tile ahead: with two waves on a SIMD nothing else
+    // would hide their way from memory.
+    float4 next_const = make_float4(0.0F, 0.0F, 0.0F, 0.0F);
+    float next_group = 0.0F;
+    uint4 bits = make_uint4(0U, 0U, 0U, 0U);
+    if (t_first < span) {
+        const uint64_t tile = tile_first + t_first;
+        next_const = p.f4const[tile * kWave + lane];
+        next_group = p.f4group[tile * 32 + l32];
+        bits = p.f4tiles[tile * p.G * kWave + lane];
+    }
     for (uint64_t t = t_first; t < span; t += t_step) {
         const uint64_t tile = tile_first + t;
-        // The bits of this lane's two codes (rows l32 and 32 + l32 of the tile), a granule at a time and one ahead.
-        const uint4* code_rows = p.tiles + tile * p.G * kWave + l32;
-        uint4 bits[2], ahead[2];
-        bits[0] = code_rows[0];
-        bits[1] = code_rows[32];
-        // Per-code constants, a lane per code.
-        const uint64_t my_slot = tile * kWave + lane;
-        const float bn = __uint_as_float(p.meta[my_slot]);
-        float berr = __uint_as_float(p.meta[p.meta_stride + my_slot]);
-        const float bsum = __uint_as_float(p.meta[2 * p.meta_stride + my_slot]);
-        const float braw = METRIC == VSAG_AMD_METRIC_L2 ? 0.0F : __uint_as_float(p.meta[3 * p.meta_stride + my_slot]);
-        if (fabsf(berr) < 1e-5F) {
-            berr = berr >= 0 ? 1.0F : -1.0F;
-        }
-        // Outside the derivation, or with factors so large that the fp32 threshold would lose its margin.
-        bool odd = !(bn > 0.0F) || !(berr > 0.0F) || !(bn < 1.0e18F) || !(berr < 1.0e18F);
-        if (METRIC != VSAG_AMD_METRIC_L2) {
-            odd = odd || !(fabsf(braw) >= 1e-5F) || !(fabsf(braw) < 1.0e18F);
-        }
-        float a_c = odd ? 0.0F : berr / (2.0F * bn);
-        float b_c = odd ? 0.0F : (bn * bn - braw * braw) * a_c;
-        odd = odd || !(a_c <= kRbMaxA) || !(fabsf(b_c) <= kRbMaxB) || !(fabsf(bsum) <= static_cast<float>(128 * p.G));
-        a_c = odd ? 0.0F : a_c;
-        b_c = odd ? 0.0F : b_c;
-        bool holds_code = my_slot < p.n;
-        if constexpr (LISTS) {
-            holds_code = as_const(p.ids)[my_slot] != VSAG_AMD_INVALID_ID;
-        }
-        const bool special = odd && holds_code;
+        // The bits of this lane's two codes (rows l32 and 32 + l32 of the tile) that its half of the wave brings to
+        // the two steps of a granule, one load ahead.
+        const uint4* code_rows = p.f4tiles + tile * p.G * kWave + lane;
+        uint4 ahead = bits;
+        // Per-code constants, a lane per code; the extremes of each group of sixteen, a lane of either half per value.
+        const float4 mine = next_const;
+        const float group_value = next_group;
+        const uint64_t tile_after = t + t_step < span ? tile + t_step : tile;
+        next_const = p.f4const[tile_after * kWave + lane];
+        next_group = p.f4group[tile_after * 32 + l32];
+        const uint4* rows_after = p.f4tiles + tile_after * p.G * kWave + lane;
+        const uint32_t flags = __float_as_uint(mine.w);
         wave_lds_fence();  // the previous tile's verdicts have read these
-        cc[lane] = a_c;
-        cc[kWave + lane] = b_c;
-        cc[2 * kWave + lane] = odd ? 0.0F : bsum;
-        const uint64_t special_mask = __ballot(special);
-        const uint64_t code_mask = __ballot(holds_code);
+        cc[lane] = mine.x;
+        cc[kWave + lane] = mine.y;
+        cc[2 * kWave + lane] = mine.z;
+        if (half == 0) {
+            cg[l32] = group_value;
+        }
+        const uint64_t special_mask = __ballot((flags & 2U) != 0);
+        const uint64_t code_mask = __ballot((flags & 1U) != 0);
         wave_lds_fence();
 
         uint32_t tile_hits[4] = {0, 0, 0, 0};
-        intx16 acc[4][2];
+        // The accumulators start at -(set bits) x u5: exact, as everything added to it (multiples of 1/4 below 2^17).
+        floatx16 acc[4][2];
 #pragma unroll
-        for (int qb = 0; qb < 4; ++qb) {
+        for (int i = 0; i < 2; ++i) {
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
+            for (int gq = 0; gq < 4; ++gq) {
+                const float4 vs = *reinterpret_cast<const float4*>(&cc[2 * kWave + 32 * i + 8 * gq + 4 * half]);
+                const float cs[4] = {vs.x, vs.y, vs.z, vs.w};
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    acc[qb][i][e] = 0;
+                for (int qb = 0; qb < 4; ++qb) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        acc[qb][i][4 * gq + j] = cs[j] * u5n[qb];
+                    }
                 }
             }
         }
 #pragma unroll
         for (uint32_t g = 0; g < kRbMaxG; ++g) {
             if (g < p.G) {
-                if (g + 1 < p.G) {
-                    ahead[0] = code_rows[(g + 1) * kWave];
-                    ahead[1] = code_rows[(g + 1) * kWave + 32];
-                }
+                // the next granule, or the first of the next tile
+                ahead = *(g + 1 < p.G ? code_rows + (g + 1) * kWave : rows_after);
 #pragma unroll
-                for (int m = 0; m < 4; ++m) {
-                    const uint32_t s = 4 * g + m;
-                    intx4 av[2];
-#pragma unroll
-                    for (int i = 0; i < 2; ++i) {
-                        const uint32_t dw = m == 0 ? bits[i].x : (m == 1 ? bits[i].y : (m == 2 ? bits[i].z : bits[i].w));
-                        const uint32_t hb = dw >> (16 * half);
-                        av[i] = intx4{rb_spread(hb & 15U), rb_spread((hb >> 4) & 15U), rb_spread((hb >> 8) & 15U),
-                                      rb_spread((hb >> 12) & 15U)};
-                    }
+                for (int m = 0; m < 2; ++m) {
+                    const uint32_t dw = 4 * g + 2 * m + half;
+                    const intx8 a0 = rb_fp4(m == 0 ? bits.x : bits.y);
+                    const intx8 a1 = rb_fp4(m == 0 ? bits.z : bits.w);
 #pragma unroll
                     for (int qb = 0; qb < 4; ++qb) {
-                        const uint4 b = qs[(2 * s + half) * kRbQueries + 32 * qb + l32];
-                        const intx4 bv = intx4{static_cast<int>(b.x), static_cast<int>(b.y), static_cast<int>(b.z),
+                        const uint4 b = qs[dw * kRbQueries + 32 * qb + l32];
+                        const uint2 t = qt[dw * kRbQueries + 32 * qb + l32];
+                        // six of the eight operand registers hold fp6 values; the other two stay undefined
+                        const intx4 b4 = intx4{static_cast<int>(b.x), static_cast<int>(b.y), static_cast<int>(b.z),
                                                static_cast<int>(b.w)};
-                        acc[qb][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[0], bv, acc[qb][0], 0, 0, 0);
-                        acc[qb][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[1], bv, acc[qb][1], 0, 0, 0);
+                        const intx4 t4 = intx4{static_cast<int>(t.x), static_cast<int>(t.y), 0, 0};
+                        const intx8 bv = __builtin_shufflevector(b4, t4, 0, 1, 2, 3, 4, 5, -1, -1);
+                        // A: fp4 (4), B: fp6 e2m3 (2); both scales 2^0 (the e8m0 pattern 127)
+                        acc[qb][0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a0, bv, acc[qb][0], 4, 2, 0, 0x7F7F7F7F,
+                                                                                      0, 0x7F7F7F7F);
+                        acc[qb][1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a1, bv, acc[qb][1], 4, 2, 0, 0x7F7F7F7F,
+                                                                                      0, 0x7F7F7F7F);
                     }
                 }
-                bits[0] = ahead[0];
-                bits[1] = ahead[1];
+                bits = ahead;
             }
         }
 
         // Element e of a lane is code 32 i + 8 (e / 4) + 4 (lane / 32) + e % 4 of the tile against query l32 of block qb.
         // Four elements (one float4 of each per-code constant) at a time keeps the registers of two waves per SIMD.
+        // First the sixteen of a lane at once: their largest sum against the smallest threshold any of them can have
+        // (the fp32 chain of five and the rounded centres are off by less than 10 x 2^-24 of the magnitudes, inside the
+        // 2^-20 taken off u4; u2 is never negative).  Only where a lane of the wave gets past that are the sixteen
+        // looked at one by one.
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
+            const float4 ge = *reinterpret_cast<const float4*>(&cg[(2 * i + half) * 8]);
+            const float ge_half_s = cg[(2 * i + half) * 8 + 4];
 #pragma unroll
-            for (int gq = 0; gq < 4; ++gq) {
-                const uint32_t row = 32 * i + 8 * gq + 4 * half;
-                const float4 va = *reinterpret_cast<const float4*>(&cc[row]);
-                const float4 vb = *reinterpret_cast<const float4*>(&cc[kWave + row]);
-                const float4 vs = *reinterpret_cast<const float4*>(&cc[2 * kWave + row]);
-                const float ca[4] = {va.x, va.y, va.z, va.w};
-                const float cb[4] = {vb.x, vb.y, vb.z, vb.w};
-                const float cs[4] = {vs.x, vs.y, vs.z, vs.w};
+            for (int qb = 0; qb < 4; ++qb) {
+                const float least = fmaf(ge.x, u1[qb], fmaf(-ge.y, fabsf(u1[qb]), fmaf(ge.z, u2[qb], fmaf(ge.w, u3[qb],
+                                    fmaf(-ge_half_s, fabsf(u3[qb]), u4[qb])))));
+                const floatx16& r = acc[qb][i];
+                float top = fmaxf(fmaxf(r[0], r[1]), r[2]);
+                top = fmaxf(fmaxf(top, r[3]), r[4]);
+                top = fmaxf(fmaxf(top, r[5]), r[6]);
+                top = fmaxf(fmaxf(top, r[7]), r[8]);
+                top = fmaxf(fmaxf(top, r[9]), r[10]);
+                top = fmaxf(fmaxf(top, r[11]), r[12]);
+                top = fmaxf(fmaxf(top, r[13]), r[14]);
+                top = fmaxf(top, r[15]);
+                if (__ballot(top >= least) == 0) {
+                    continue;
+                }
 #pragma unroll
-                for (int qb = 0; qb < 4; ++qb) {
+                for (int gq = 0; gq < 4; ++gq) {
+                    // the same test on the four of a quarter before their own thresholds are formed
+                    const float top4 = fmaxf(fmaxf(fmaxf(r[4 * gq], r[4 * gq + 1]), r[4 * gq + 2]), r[4 * gq + 3]);
+                    if (__ballot(top4 >= least) == 0) {
+                        continue;
+                    }
+                    const uint32_t row = 32 * i + 8 * gq + 4 * half;
+                    const float4 va = *reinterpret_cast<const float4*>(&cc[row]);
+                    const float4 vb = *reinterpret_cast<const float4*>(&cc[kWave + row]);
+                    const float4 vs = *reinterpret_cast<const float4*>(&cc[2 * kWave + row]);
+                    const float ca[4] = {va.x, va.y, va.z, va.w};
+                    const float cb[4] = {vb.x, vb.y, vb.z, vb.w};
+                    const float cs[4] = {vs.x, vs.y, vs.z, vs.w};
                     bool pass[4];
                     uint64_t any = 0;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
                         const float thr = fmaf(cs[j], u3[qb], fmaf(cb[j], u2[qb], fmaf(ca[j], u1[qb], u4[qb])));
-                        pass[j] = static_cast<float>(acc[qb][i][4 * gq + j]) >= thr;
+                        pass[j] = acc[qb][i][4 * gq + j] >= thr;
                         any |= __ballot(pass[j]);
                     }
                     if (any != 0) {
@@ -437,10 +496,11 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
                                 if constexpr (LISTS) {
                                     append_shared(32 * qb + l32, slot);
                                 } else {
-                                    if (ncand[qb] < p.sub_cap) {
-                                        list[ncand[qb]] = static_cast<uint32_t>(slot);
+                                    const uint32_t have = ncand[qb * kRbThreads];
+                                    if (have < p.sub_cap) {
+                                        list[have] = static_cast<uint32_t>(slot);
                                     }
-                                    ++ncand[qb];
+                                    ncand[qb * kRbThreads] = have + 1;
                                 }
                             }
                         }
@@ -503,10 +563,11 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
                     }
                     const uint64_t q = q0 + 32 * qb + l32;
                     if (q < p.nq) {
-                        if (ncand[qb] < p.sub_cap) {
-                            p.cand[(q * sub_lists + my_sub) * p.sub_cap + ncand[qb]] = static_cast<uint32_t>(tile * kWave + code);
+                        const uint32_t have = ncand[qb * kRbThreads];
+                        if (have < p.sub_cap) {
+                            p.cand[(q * sub_lists + my_sub) * p.sub_cap + have] = static_cast<uint32_t>(tile * kWave + code);
                         }
-                        ++ncand[qb];
+                        ncand[qb * kRbThreads] = have + 1;
                     }
                 }
             }
@@ -517,7 +578,7 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
         for (int qb = 0; qb < 4; ++qb) {
             const uint64_t q = q0 + 32 * qb + l32;
             if (q < p.nq) {
-                p.cand_cnt[q * sub_lists + my_sub] = ncand[qb];
+                p.cand_cnt[q * sub_lists + my_sub] = ncand[qb * kRbThreads];
             }
         }
     }
@@ -525,7 +586,7 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
 
 bool
 prefilter_rb_supports(const vsag_amd_store* s) {
-    return s->kind == VSAG_AMD_KIND_RABITQ && s->query_bits == 4 && s->nlist == 0 && s->G <= kRbMaxG &&
+    return s->kind == VSAG_AMD_KIND_RABITQ && s->query_bits == 4 && s->nlist == 0 && s->G <= kRbMaxG && s->f4tiles != nullptr &&
            (s->metric == VSAG_AMD_METRIC_L2 || s->metric == VSAG_AMD_METRIC_IP);
 }
 
@@ -538,7 +599,7 @@ prefilter_rb_padded_queries(uint64_t nq) {
 size_t
 prefilter_rb_scratch_bytes(const vsag_amd_store* s, uint64_t nq) {
     const uint64_t nq_pad = prefilter_rb_padded_queries(nq);
-    return static_cast<size_t>(nq_pad) * s->G * 128 + static_cast<size_t>(nq_pad) * 16 + 512;
+    return static_cast<size_t>(nq_pad) * s->G * 128 + static_cast<size_t>(nq_pad) * 20 + 512;
 }
 
 // Private candidate lists per query for nq queries over `span` tiles.
@@ -569,22 +630,23 @@ launch_prefilter_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uin
     const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
     const uint64_t nq_pad = prefilter_rb_padded_queries(nq);
     const uint32_t ndw = s->G * 4;
-    uint8_t* qbytes = scratch;
+    uint4* qa = reinterpret_cast<uint4*>(scratch);
+    uint2* qb = reinterpret_cast<uint2*>(scratch + static_cast<size_t>(nq_pad) * ndw * 16);
     float* u = reinterpret_cast<float*>(scratch + round_up(static_cast<size_t>(nq_pad) * ndw * 32, 256));
-    hipLaunchKernelGGL(rabitq_query_bytes_kernel, dim3(static_cast<uint32_t>(div_up(nq_pad * ndw, 256))), dim3(256), 0, st,
-                       a.qtab, a.qstride, ndw, nq, nq_pad, qbytes);
+    hipLaunchKernelGGL(rabitq_query_f6_kernel, dim3(static_cast<uint32_t>(div_up(nq_pad * ndw, 256))), dim3(256), 0, st,
+                       a.qtab, a.qstride, ndw, nq, nq_pad, qa, qb);
     hipLaunchKernelGGL(rabitq_tau_kernel, dim3(static_cast<uint32_t>(div_up(nq_pad, 256))), dim3(256), 0, st, a.qmeta,
                        a.qmeta_stride, bound, l2 ? 1 : 0, s->G * 128, nq, nq_pad, u);
     VA_HIP(hipGetLastError());
     PrefilterRbArgs p{};
-    p.tiles = s->tiles;
+    p.f4tiles = s->f4tiles;
+    p.f4const = s->f4const;
+    p.f4group = reinterpret_cast<const float*>(s->f4group);
     p.G = s->G;
     p.tile_begin = tile_begin;
     p.tile_end = tile_end;
-    p.n = s->n;
-    p.meta = a.meta;
-    p.meta_stride = a.meta_stride;
-    p.qbytes = reinterpret_cast<const uint4*>(qbytes);
+    p.qa = qa;
+    p.qb = qb;
     p.u = u;
     p.nq = nq;
     p.nq_pad = nq_pad;
@@ -593,7 +655,8 @@ launch_prefilter_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uin
     p.sub_cap = sub_cap;
     p.groups = sub_lists / (2 * kRbWaves);
     VA_CHECK_ARG(sub_lists == prefilter_rb_sub_lists(nq, tile_end - tile_begin), "candidate lists do not match the grid");
-    const size_t lds = static_cast<size_t>(8 * s->G) * kRbQueries * 16 + kRbWaves * 3 * kWave * sizeof(float);
+    const size_t lds = static_cast<size_t>(4 * s->G) * kRbQueries * 24 + kRbWaves * kRbWaveFloats * sizeof(float) +
+                       4 * kRbThreads * sizeof(uint32_t);
     dim3 grid(p.groups, static_cast<uint32_t>(nq_pad / kRbQueries));
     timing_begin(st);
     if (l2) {
@@ -613,7 +676,7 @@ launch_prefilter_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uin
 // ---- posting lists ------------------------------------------------------------------------------------------------
 bool
 ivf_rb_supports(const vsag_amd_store* s) {
-    return s->kind == VSAG_AMD_KIND_RABITQ && s->query_bits == 4 && s->nlist > 0 && s->G <= kRbMaxG &&
+    return s->kind == VSAG_AMD_KIND_RABITQ && s->query_bits == 4 && s->nlist > 0 && s->G <= kRbMaxG && s->f4tiles != nullptr &&
            s->residual_centroids_dev == nullptr &&
            (s->metric == VSAG_AMD_METRIC_L2 || s->metric == VSAG_AMD_METRIC_IP);
 }
@@ -646,25 +709,25 @@ launch_ivf_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
     const uint64_t nq_pad = prefilter_rb_padded_queries(nq + 1);
     const uint32_t ndw = s->G * 4;
-    uint8_t* qbytes = scratch;
+    uint4* qa = reinterpret_cast<uint4*>(scratch);
+    uint2* qb = reinterpret_cast<uint2*>(scratch + static_cast<size_t>(nq_pad) * ndw * 16);
     float* u = reinterpret_cast<float*>(scratch + round_up(static_cast<size_t>(nq_pad) * ndw * 32, 256));
-    hipLaunchKernelGGL(rabitq_query_bytes_kernel, dim3(static_cast<uint32_t>(div_up(nq_pad * ndw, 256))), dim3(256), 0, st,
-                       a.qtab, a.qstride, ndw, nq, nq_pad, qbytes);
+    hipLaunchKernelGGL(rabitq_query_f6_kernel, dim3(static_cast<uint32_t>(div_up(nq_pad * ndw, 256))), dim3(256), 0, st,
+                       a.qtab, a.qstride, ndw, nq, nq_pad, qa, qb);
     hipLaunchKernelGGL(rabitq_tau_kernel, dim3(static_cast<uint32_t>(div_up(nq_pad, 256))), dim3(256), 0, st, a.qmeta,
                        a.qmeta_stride, bound, l2 ? 1 : 0, s->G * 128, nq, nq_pad, u);
     VA_HIP(hipGetLastError());
     PrefilterRbArgs p{};
-    p.tiles = s->tiles;
+    p.f4tiles = s->f4tiles;
+    p.f4const = s->f4const;
+    p.f4group = reinterpret_cast<const float*>(s->f4group);
     p.G = s->G;
-    p.n = s->n;
-    p.meta = a.meta;
-    p.meta_stride = a.meta_stride;
-    p.qbytes = reinterpret_cast<const uint4*>(qbytes);
+    p.qa = qa;
+    p.qb = qb;
     p.u = u;
     p.nq = nq;
     p.nq_pad = nq_pad;
     p.groups = 1;
-    p.ids = s->ids_dev;
     p.list_tile = s->list_tile_dev;
     p.pair_off = pair_off;
     p.item_off = item_off;
@@ -676,7 +739,8 @@ launch_ivf_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     p.partial = partial;
     p.partial_cnt = partial_cnt;
     p.gate = gate;
-    const size_t lds = static_cast<size_t>(8 * s->G) * kRbQueries * 16 + kRbWaves * 3 * kWave * sizeof(float);
+    const size_t lds = static_cast<size_t>(4 * s->G) * kRbQueries * 24 + kRbWaves * kRbWaveFloats * sizeof(float) +
+                       4 * kRbThreads * sizeof(uint32_t);
     const uint64_t pairs = nq * (nprobe - p0);
     const uint64_t max_items =
         (div_up(pairs, static_cast<uint64_t>(kRbQueries)) + std::min<uint64_t>(s->nlist, pairs)) * kIvfRbChunks;

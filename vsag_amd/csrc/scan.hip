@@ -897,7 +897,7 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
     // unless r is small.
     uint64_t r = std::min<uint64_t>(16, std::max<uint64_t>(2, cap / (8ull * k)));
     if (rb) {
-        r = std::min<uint64_t>(r, std::max<uint64_t>(4, 800 / k));
+        r = std::min<uint64_t>(r, std::max<uint64_t>(3, 600 / k));
     }
     // The int8 matrix cores pass a tile forty times faster than the streaming kernel: there a short exact prefix and
     // one more level beat a long prefix.

@@ -88,6 +88,20 @@ struct vsag_amd_store {
     uint4* rows = nullptr;
     float* pf_term = nullptr;
     uint32_t* pf_ymax = nullptr;
+    // 1-bit rabitq stores with 4-bit queries (l2 / ip, at most kRbMaxG granules, no residual), flat or lists: the code
+    // bits once more as the fp4 operand of the matrix cores wants them (prefilter_rb.hip).  f4tiles[(tile G + g) 64 +
+    // lane], lane = 32 h + r: dwords 4 g + h and 4 g + 2 + h of code r of the tile (x, y) and of code 32 + r (z, w),
+    // each with bit 8 v + j of the code's dword moved to bit 4 j + v, so that ((w >> v) << 1) & 0x22222222 is register
+    // v of the operand (elements 8 v .. 8 v + 7 as fp4 1.0 or 0).  f4const: per slot the three constants the pass
+    // takes from a code's factors and two flags as the bits of w (1: the slot holds a code, 2: the code stands outside
+    // the pass and is a candidate of every query).  f4group: per tile and group of sixteen codes (those whose verdicts
+    // share a lane: 32 i + 8 gq + 4 h + j of group 2 i + h) the centre and half width of the first constant, the least
+    // second, the centre and half width of the third, in two float4.  Flat stores keep all of it up to date in append;
+    // posting lists renew it over all cap_tiles when codes are added (f4_slots = their room).
+    uint4* f4tiles = nullptr;
+    float4* f4const = nullptr;
+    float4* f4group = nullptr;
+    uint64_t f4_slots = 0;
     // sq8 / sq4 posting lists of at most 128 dimensions keep the same per-slot term (over all cap_tiles * 64 slots, renewed
     // when codes are added) for the int8 pass over lists; pf_term_slots = the slots pf_term has room for there.
     uint64_t pf_term_slots = 0;
@@ -96,6 +110,13 @@ struct vsag_amd_store {
 namespace vsag_amd {
 
 // Query-side table geometry of one store kind (what the prepare kernel writes per query).
+constexpr uint32_t kRbMaxG = 8;  // granules per code (1024 dimensions) of the rabitq matrix-core pass
+// Largest per-code factors the fp32 threshold of that pass takes (A_c, |B_c| of prefilter_rb.hip; codes beyond them stand
+// outside the pass, as candidates of every query): the per-query slack there is sized for them.  The second grows with
+// the square of the data's scale (norm x error factor / 2).
+constexpr float kRbMaxA = 64.0F;
+constexpr float kRbMaxB = 4096.0F;
+
 struct QueryLayout {
     uint32_t qstride;  // 4-byte words per query in the main table
     uint32_t qmeta;    // floats per query in the scalar table

@@ -249,6 +249,128 @@ rows_from_tiles_kernel(const uint4* tiles, uint32_t G, uint64_t first_slot, uint
     rows[slot * G + j] = tiles[((slot / kWave) * G + j) * kWave + slot % kWave];
 }
 
+// Stores whose code bits are kept as fp4 operands as well (prefilter_rb.hip).
+static bool
+keeps_f4(const vsag_amd_store* s) {
+    return s->kind == VSAG_AMD_KIND_RABITQ && s->query_bits == 4 && s->base_bits == 1 && s->G <= kRbMaxG &&
+           (s->metric == VSAG_AMD_METRIC_L2 || s->metric == VSAG_AMD_METRIC_IP);
+}
+
+__device__ inline uint32_t
+f4_order(uint32_t w) {
+    // bit 8 v + j -> bit 4 j + v
+    uint32_t out = 0;
+#pragma unroll
+    for (uint32_t v = 0; v < 4; ++v) {
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {
+            out |= ((w >> (8 * v + j)) & 1U) << (4 * j + v);
+        }
+    }
+    return out;
+}
+
+// f4tiles of tiles [first_tile, first_tile + ntiles) from the tiles; a thread per (tile, granule, lane).
+__global__ void __launch_bounds__(256)
+f4_from_tiles_kernel(const uint4* tiles, uint32_t G, uint64_t first_tile, uint64_t ntiles, uint4* f4tiles) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= ntiles * G * kWave) {
+        return;
+    }
+    const uint64_t at = first_tile * G * kWave + i;  // (tile G + g) 64 + lane
+    const uint32_t lane = static_cast<uint32_t>(at % kWave);
+    const uint64_t granule = at - lane;
+    const uint32_t h = lane >> 5, r = lane & 31;
+    const uint4 lo = tiles[granule + r], hi = tiles[granule + 32 + r];
+    uint4 out;
+    out.x = f4_order(h == 0 ? lo.x : lo.y);
+    out.y = f4_order(h == 0 ? lo.z : lo.w);
+    out.z = f4_order(h == 0 ? hi.x : hi.y);
+    out.w = f4_order(h == 0 ? hi.z : hi.w);
+    f4tiles[at] = out;
+}
+
+// f4const of slots [first_slot, first_slot + count).  With err the error factor, norm and raw the norms of a code and
+// S its sum field: A = err / (2 norm), B = (norm^2 [- raw^2]) A, S.  Codes the derivation of the pass does not cover
+// (zero norm, non-positive error factor, zero raw norm, factors so large that the fp32 threshold would lose its margin,
+// a sum field that is not the number of set bits -- the matrix cores count the bits themselves) stand outside.
+__global__ void __launch_bounds__(256)
+f4_const_kernel(const uint4* tiles, uint32_t G, const uint32_t* meta, uint64_t meta_stride, int is_l2, const uint32_t* ids,
+                uint64_t n, uint64_t first_slot, uint64_t count, float4* f4const) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= count) {
+        return;
+    }
+    const uint64_t slot = first_slot + i;
+    const uint4* code = tiles + (slot / kWave) * G * kWave + slot % kWave;
+    uint32_t bits = 0;
+    for (uint32_t g = 0; g < G; ++g) {
+        const uint4 v = code[static_cast<uint64_t>(g) * kWave];
+        bits += __popc(v.x) + __popc(v.y) + __popc(v.z) + __popc(v.w);
+    }
+    const float bn = __uint_as_float(meta[slot]);
+    float berr = __uint_as_float(meta[meta_stride + slot]);
+    const float bsum = __uint_as_float(meta[2 * meta_stride + slot]);
+    const float braw = is_l2 ? 0.0F : __uint_as_float(meta[3 * meta_stride + slot]);
+    if (fabsf(berr) < 1e-5F) {
+        berr = berr >= 0 ? 1.0F : -1.0F;  // as the estimator does (distance.h, finish_distances)
+    }
+    bool odd = !(bn > 0.0F) || !(berr > 0.0F) || !(bn < 1.0e18F) || !(berr < 1.0e18F);
+    if (!is_l2) {
+        odd = odd || !(fabsf(braw) >= 1e-5F) || !(fabsf(braw) < 1.0e18F);
+    }
+    float a_c = odd ? 0.0F : berr / (2.0F * bn);
+    float b_c = odd ? 0.0F : (bn * bn - braw * braw) * a_c;
+    odd = odd || !(a_c <= kRbMaxA) || !(fabsf(b_c) <= kRbMaxB) || !(bsum == static_cast<float>(bits));
+    const bool holds = ids != nullptr ? ids[slot] != VSAG_AMD_INVALID_ID : slot < n;
+    const uint32_t flags = (holds ? 1U : 0U) | (odd && holds ? 2U : 0U);
+    f4const[slot] = make_float4(odd ? 0.0F : a_c, odd ? 0.0F : b_c, odd ? 0.0F : bsum, __uint_as_float(flags));
+}
+
+// f4group of tiles [first_tile, first_tile + ntiles); a thread per (tile, group).  Slots without a verdict (no code, or
+// a code outside the pass) stay out; a group of nothing else gets a threshold nothing reaches (1e30 stays finite
+// through the chain of multiply-adds it goes into).
+__global__ void __launch_bounds__(256)
+f4_group_kernel(const float4* f4const, uint64_t first_tile, uint64_t ntiles, float4* f4group) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= ntiles * 4) {
+        return;
+    }
+    const uint64_t tile = first_tile + i / 4;
+    const uint32_t group = static_cast<uint32_t>(i % 4), gi = group >> 1, gh = group & 1U;
+    float lo_a = 1e30F, hi_a = -1e30F, lo_b = 1e30F, lo_s = 1e30F, hi_s = -1e30F;
+    for (uint32_t c = 0; c < 16; ++c) {
+        const float4 v = f4const[tile * kWave + 32 * gi + 8 * (c >> 2) + 4 * gh + (c & 3U)];
+        if (__float_as_uint(v.w) == 1U) {
+            lo_a = fminf(lo_a, v.x);
+            hi_a = fmaxf(hi_a, v.x);
+            lo_b = fminf(lo_b, v.y);
+            lo_s = fminf(lo_s, v.z);
+            hi_s = fmaxf(hi_s, v.z);
+        }
+    }
+    // factor x constant is least at factor x centre - |factor| x half width
+    f4group[(tile * 4 + group) * 2] = make_float4(0.5F * (lo_a + hi_a), 0.5F * (hi_a - lo_a), lo_b, 0.5F * (lo_s + hi_s));
+    f4group[(tile * 4 + group) * 2 + 1] = make_float4(0.5F * (hi_s - lo_s), 0.0F, 0.0F, 0.0F);
+}
+
+// Renews f4tiles / f4const / f4group over tiles [first_tile, first_tile + ntiles) of a store of n codes.
+static int
+launch_f4(const vsag_amd_store* s, uint64_t n, uint64_t first_tile, uint64_t ntiles, hipStream_t st) {
+    if (s->f4tiles == nullptr || ntiles == 0) {
+        return 0;
+    }
+    hipLaunchKernelGGL(f4_from_tiles_kernel, dim3(static_cast<uint32_t>(div_up(ntiles * s->G * kWave, 256))), dim3(256), 0,
+                       st, s->tiles, s->G, first_tile, ntiles, s->f4tiles);
+    hipLaunchKernelGGL(f4_const_kernel, dim3(static_cast<uint32_t>(div_up(ntiles * kWave, 256))), dim3(256), 0, st, s->tiles,
+                       s->G, s->meta, s->cap_tiles * kWave, s->metric == VSAG_AMD_METRIC_L2 ? 1 : 0,
+                       s->nlist > 0 ? s->ids_dev : nullptr, n, first_tile * kWave, ntiles * kWave, s->f4const);
+    hipLaunchKernelGGL(f4_group_kernel, dim3(static_cast<uint32_t>(div_up(ntiles * 4, 256))), dim3(256), 0, st, s->f4const,
+                       first_tile, ntiles, s->f4group);
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
 static int
 grow(vsag_amd_store* s, uint64_t need_tiles, hipStream_t st) {
     if (need_tiles <= s->cap_tiles) {
@@ -288,7 +410,29 @@ grow(vsag_amd_store* s, uint64_t need_tiles, hipStream_t st) {
             VA_HIP(hipMemcpyAsync(rows, s->rows, s->ntiles * kWave * s->G * sizeof(uint4), hipMemcpyDeviceToDevice, st));
         }
     }
+    uint4* f4tiles = nullptr;
+    float4* f4const = nullptr;
+    float4* f4group = nullptr;
+    if (keeps_f4(s)) {
+        VA_HIP(hipMalloc(&f4tiles, cap * kWave * s->G * sizeof(uint4)));
+        VA_HIP(hipMalloc(&f4const, cap * kWave * sizeof(float4)));
+        VA_HIP(hipMalloc(&f4group, cap * 8 * sizeof(float4)));
+        if (s->ntiles > 0) {
+            VA_HIP(hipMemcpyAsync(f4tiles, s->f4tiles, s->ntiles * kWave * s->G * sizeof(uint4), hipMemcpyDeviceToDevice, st));
+            VA_HIP(hipMemcpyAsync(f4const, s->f4const, s->ntiles * kWave * sizeof(float4), hipMemcpyDeviceToDevice, st));
+            VA_HIP(hipMemcpyAsync(f4group, s->f4group, s->ntiles * 8 * sizeof(float4), hipMemcpyDeviceToDevice, st));
+        }
+    }
     VA_HIP(hipStreamSynchronize(st));
+    for (void* p : {static_cast<void*>(s->f4tiles), static_cast<void*>(s->f4const), static_cast<void*>(s->f4group)}) {
+        if (p != nullptr) {
+            VA_HIP(hipFree(p));
+        }
+    }
+    s->f4tiles = f4tiles;
+    s->f4const = f4const;
+    s->f4group = f4group;
+    s->f4_slots = f4tiles != nullptr ? cap * kWave : 0;
     if (s->tiles) {
         VA_HIP(hipFree(s->tiles));
     }
@@ -555,7 +699,7 @@ vsag_amd_store_destroy(vsag_amd_store_t* s) {
     void* ptrs[] = {s->scale_dev, s->lb_dev,  s->diff_dev, s->bounds_dev,    s->rotation_dev, s->centroid_dev,
                     s->tiles,     s->meta,    s->ids_dev,  s->list_tile_dev, s->pf_term,      s->pf_ymax,
                     s->rows,      s->slot_of_id_dev, s->residual_bias_dev, s->residual_centroids_dev,
-                    s->list_sizes_dev, s->codebooks_dev};
+                    s->list_sizes_dev, s->codebooks_dev, s->f4tiles, s->f4const, s->f4group};
     for (void* p : ptrs) {
         if (p != nullptr) {
             (void)hipFree(p);
@@ -594,6 +738,7 @@ vsag_amd_store_append(vsag_amd_store_t* s, const uint8_t* codes_dev, uint64_t n,
         VA_HIP(hipGetLastError());
     }
     VA_TRY(launch_code_terms(s, s->n, n, st));
+    VA_TRY(launch_f4(s, s->n + n, s->n / kWave, need - s->n / kWave, st));
     s->n += n;
     s->ntiles = need;
     return 0;
@@ -616,6 +761,15 @@ drop_lists(vsag_amd_store* s) {
         s->pf_term = nullptr;
     }
     s->pf_term_slots = 0;
+    for (void* p : {static_cast<void*>(s->f4tiles), static_cast<void*>(s->f4const), static_cast<void*>(s->f4group)}) {
+        if (p != nullptr) {
+            VA_HIP(hipFree(p));
+        }
+    }
+    s->f4tiles = nullptr;
+    s->f4const = nullptr;
+    s->f4group = nullptr;
+    s->f4_slots = 0;
     s->list_sizes_dev = nullptr;
     s->tiles = nullptr;
     s->meta = nullptr;
@@ -853,6 +1007,27 @@ append_to_lists(vsag_amd_store* s, const uint8_t* codes_dev, const int32_t* labe
             s->pf_term_slots = slots;
         }
         VA_TRY(launch_code_terms(s, 0, slots, st));
+        VA_HIP(hipStreamSynchronize(st));
+    }
+    // The fp4 copy of 1-bit rabitq lists, renewed the same way.
+    if (keeps_f4(s) && s->residual_centroids_dev == nullptr) {
+        const uint64_t slots = s->cap_tiles * kWave;
+        if (s->f4tiles == nullptr || s->f4_slots < slots) {
+            for (void* p : {static_cast<void*>(s->f4tiles), static_cast<void*>(s->f4const), static_cast<void*>(s->f4group)}) {
+                if (p != nullptr) {
+                    VA_HIP(hipFree(p));
+                }
+            }
+            s->f4tiles = nullptr;
+            s->f4const = nullptr;
+            s->f4group = nullptr;
+            s->f4_slots = 0;
+            VA_HIP(hipMalloc(&s->f4tiles, slots * s->G * sizeof(uint4)));
+            VA_HIP(hipMalloc(&s->f4const, slots * sizeof(float4)));
+            VA_HIP(hipMalloc(&s->f4group, s->cap_tiles * 8 * sizeof(float4)));
+            s->f4_slots = slots;
+        }
+        VA_TRY(launch_f4(s, s->n, 0, s->cap_tiles, st));
         VA_HIP(hipStreamSynchronize(st));
     }
     return 0;
