@@ -196,7 +196,16 @@ rb_fp4(uint32_t w) {
     return __builtin_shufflevector(v, v, 0, 1, 2, 3, -1, -1, -1, -1);
 }
 
-template <int METRIC, bool LISTS = false>
+// Granules of code bits a wave keeps on their way from memory: a granule feeds sixteen matrix instructions, about a
+// quarter of the time its load takes, and two waves on a SIMD do not hide the rest.  The depth divides the granules of a
+// code, so that granule j of every tile sits in register set j % depth.
+__host__ __device__ constexpr uint32_t
+rb_ring(uint32_t granules) {
+    return granules > 1 && granules % 2 == 0 ? 2 : 1;
+}
+
+// KG: the granules of a code (the store's G), a parameter so that the registers of the ring are fixed.
+template <bool LISTS, uint32_t KG>
 __global__ void __launch_bounds__(kRbThreads, 2)
 prefilter_rb_kernel(PrefilterRbArgs p) {
     extern __shared__ uint4 rb_lds[];
@@ -207,7 +216,9 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
     const uint32_t wave = tid >> 6;
     const uint32_t half = lane >> 5;
     const uint32_t l32 = lane & 31;
-    const uint32_t ndw = 4 * p.G;  // code dwords: dword 2 s + h is what half h of the wave brings to step s
+    constexpr uint32_t kRing = rb_ring(KG);
+    constexpr uint32_t kUnroll = KG <= 6 ? KG : kRing;  // seven and eight granules, all unrolled, run out of registers
+    const uint32_t ndw = 4 * KG;  // code dwords: dword 2 s + h is what half h of the wave brings to step s
     uint64_t q0 = static_cast<uint64_t>(blockIdx.y) * kRbQueries;
     uint4* qs = rb_lds;                                                  // [dword][128 queries]: 16 of its 24 bytes
     uint2* qt = reinterpret_cast<uint2*>(rb_lds + ndw * kRbQueries);     // [dword][128 queries]: the other 8
@@ -306,9 +317,10 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
             qt[c * kRbQueries + ql] = p.qb[at];
         }
     }
-    float u1[4], u2[4], u3[4], u4[4], u5n[4];
     // Candidates so far of this lane's four queries (flat stores): in LDS, the registers go to the accumulators.
     uint32_t* ncand = reinterpret_cast<uint32_t*>(cc - wave * kRbWaveFloats + kRbWaves * kRbWaveFloats) + tid;
+    // So do the five factors of each of those queries: uq[(5 qb + j) kRbThreads] is u(j + 1), u5 negated.
+    float* uq = reinterpret_cast<float*>(ncand + 4 * kRbThreads);
 #pragma unroll
     for (int qb = 0; qb < 4; ++qb) {
         ncand[qb * kRbThreads] = 0;
@@ -318,11 +330,11 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
 #pragma unroll
     for (int qb = 0; qb < 4; ++qb) {
         const uint64_t q = query_row(32 * qb + l32);
-        u1[qb] = p.u[q];
-        u2[qb] = p.u[p.nq_pad + q];
-        u3[qb] = p.u[2 * p.nq_pad + q];
-        u4[qb] = p.u[3 * p.nq_pad + q];
-        u5n[qb] = -p.u[4 * p.nq_pad + q];
+        uq[(5 * qb + 0) * kRbThreads] = p.u[q];
+        uq[(5 * qb + 1) * kRbThreads] = p.u[p.nq_pad + q];
+        uq[(5 * qb + 2) * kRbThreads] = p.u[2 * p.nq_pad + q];
+        uq[(5 * qb + 3) * kRbThreads] = p.u[3 * p.nq_pad + q];
+        uq[(5 * qb + 4) * kRbThreads] = -p.u[4 * p.nq_pad + q];
     }
     __syncthreads();
     // LISTS: a pair has eight private lists (two per chunk in ivf_i8.hip's layout); here a hit goes to the one of
@@ -341,30 +353,44 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
         }
     };
 
-    // A tile's constants and the first of its bits are asked for one tile ahead: with two waves on a SIMD nothing else
-    // would hide their way from memory.
+    // A tile's constants are asked for one tile ahead, its bits kRing granules ahead (across the end of a tile): with
+    // two waves on a SIMD nothing else would hide their way from memory.
     float4 next_const = make_float4(0.0F, 0.0F, 0.0F, 0.0F);
     float next_group = 0.0F;
-    uint4 bits = make_uint4(0U, 0U, 0U, 0U);
+    uint4 ring[kRing];
+#pragma unroll
+    for (uint32_t j = 0; j < kRing; ++j) {
+        ring[j] = make_uint4(0U, 0U, 0U, 0U);
+    }
     if (t_first < span) {
         const uint64_t tile = tile_first + t_first;
         next_const = p.f4const[tile * kWave + lane];
         next_group = p.f4group[tile * 32 + l32];
-        bits = p.f4tiles[tile * p.G * kWave + lane];
+#pragma unroll
+        for (uint32_t j = 0; j < kRing; ++j) {
+            ring[j] = p.f4tiles[(tile * KG + j) * kWave + lane];
+        }
+    }
+    // The query operands of the first two pairs of matrix instructions of a tile.
+    uint4 qb_a[2];
+    uint2 qb_t[2];
+#pragma unroll
+    for (uint32_t j = 0; j < 2; ++j) {
+        qb_a[j] = qs[half * kRbQueries + 32 * j + l32];
+        qb_t[j] = qt[half * kRbQueries + 32 * j + l32];
     }
     for (uint64_t t = t_first; t < span; t += t_step) {
         const uint64_t tile = tile_first + t;
         // The bits of this lane's two codes (rows l32 and 32 + l32 of the tile) that its half of the wave brings to
-        // the two steps of a granule, one load ahead.
-        const uint4* code_rows = p.f4tiles + tile * p.G * kWave + lane;
-        uint4 ahead = bits;
+        // the two steps of a granule.
+        const uint4* code_rows = p.f4tiles + tile * KG * kWave + lane;
         // Per-code constants, a lane per code; the extremes of each group of sixteen, a lane of either half per value.
         const float4 mine = next_const;
         const float group_value = next_group;
         const uint64_t tile_after = t + t_step < span ? tile + t_step : tile;
         next_const = p.f4const[tile_after * kWave + lane];
         next_group = p.f4group[tile_after * 32 + l32];
-        const uint4* rows_after = p.f4tiles + tile_after * p.G * kWave + lane;
+        const uint4* rows_after = p.f4tiles + tile_after * KG * kWave + lane;
         const uint32_t flags = __float_as_uint(mine.w);
         wave_lds_fence();  // the previous tile's verdicts have read these
         cc[lane] = mine.x;
@@ -380,35 +406,42 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
         uint32_t tile_hits[4] = {0, 0, 0, 0};
         // The accumulators start at -(set bits) x u5: exact, as everything added to it (multiples of 1/4 below 2^17).
         floatx16 acc[4][2];
+        {
+            const float u5n[4] = {uq[4 * kRbThreads], uq[9 * kRbThreads], uq[14 * kRbThreads], uq[19 * kRbThreads]};
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+            for (int i = 0; i < 2; ++i) {
 #pragma unroll
-            for (int gq = 0; gq < 4; ++gq) {
-                const float4 vs = *reinterpret_cast<const float4*>(&cc[2 * kWave + 32 * i + 8 * gq + 4 * half]);
-                const float cs[4] = {vs.x, vs.y, vs.z, vs.w};
+                for (int gq = 0; gq < 4; ++gq) {
+                    const float4 vs = *reinterpret_cast<const float4*>(&cc[2 * kWave + 32 * i + 8 * gq + 4 * half]);
+                    const float cs[4] = {vs.x, vs.y, vs.z, vs.w};
 #pragma unroll
-                for (int qb = 0; qb < 4; ++qb) {
+                    for (int qb = 0; qb < 4; ++qb) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        acc[qb][i][4 * gq + j] = cs[j] * u5n[qb];
+                        for (int j = 0; j < 4; ++j) {
+                            acc[qb][i][4 * gq + j] = cs[j] * u5n[qb];
+                        }
                     }
                 }
             }
         }
-#pragma unroll
-        for (uint32_t g = 0; g < kRbMaxG; ++g) {
+#pragma unroll kUnroll
+        for (uint32_t g = 0; g < KG; ++g) {
+            // p.G is KG: asked at run time, the question keeps every granule a block of its own.  In one block the
+            // compiler gathers the matrix instructions by accumulator, which takes every query operand of the tile into
+            // registers at once.
             if (g < p.G) {
-                // the next granule, or the first of the next tile
-                ahead = *(g + 1 < p.G ? code_rows + (g + 1) * kWave : rows_after);
+                const uint4 bits = ring[g % kRing];
 #pragma unroll
                 for (int m = 0; m < 2; ++m) {
-                    const uint32_t dw = 4 * g + 2 * m + half;
                     const intx8 a0 = rb_fp4(m == 0 ? bits.x : bits.y);
                     const intx8 a1 = rb_fp4(m == 0 ? bits.z : bits.w);
 #pragma unroll
                     for (int qb = 0; qb < 4; ++qb) {
-                        const uint4 b = qs[dw * kRbQueries + 32 * qb + l32];
-                        const uint2 t = qt[dw * kRbQueries + 32 * qb + l32];
+                        // The query operand was asked for two pairs of matrix instructions ago; its registers go to the
+                        // pair after the next (of the next step, granule or -- the queries being the same -- tile).
+                        const uint32_t pair = 4 * m + qb;
+                        const uint4 b = qb_a[pair % 2];
+                        const uint2 t = qb_t[pair % 2];
                         // six of the eight operand registers hold fp6 values; the other two stay undefined
                         const intx4 b4 = intx4{static_cast<int>(b.x), static_cast<int>(b.y), static_cast<int>(b.z),
                                                static_cast<int>(b.w)};
@@ -419,9 +452,15 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
                                                                                       0, 0x7F7F7F7F);
                         acc[qb][1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a1, bv, acc[qb][1], 4, 2, 0, 0x7F7F7F7F,
                                                                                       0, 0x7F7F7F7F);
+                        const uint32_t pair_then = pair + 2;
+                        const uint32_t g_then = pair_then < 8 ? g : (g + 1 < KG ? g + 1 : 0);
+                        const uint32_t dw_then = 4 * g_then + 2 * ((pair_then % 8) / 4) + half;
+                        qb_a[pair % 2] = qs[dw_then * kRbQueries + 32 * (pair_then % 4) + l32];
+                        qb_t[pair % 2] = qt[dw_then * kRbQueries + 32 * (pair_then % 4) + l32];
                     }
                 }
-                bits = ahead;
+                // its register set goes to the granule kRing further on, of this tile or the next
+                ring[g % kRing] = g + kRing < KG ? code_rows[(g + kRing) * kWave] : rows_after[(g + kRing - KG) * kWave];
             }
         }
 
@@ -437,8 +476,10 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
             const float ge_half_s = cg[(2 * i + half) * 8 + 4];
 #pragma unroll
             for (int qb = 0; qb < 4; ++qb) {
-                const float least = fmaf(ge.x, u1[qb], fmaf(-ge.y, fabsf(u1[qb]), fmaf(ge.z, u2[qb], fmaf(ge.w, u3[qb],
-                                    fmaf(-ge_half_s, fabsf(u3[qb]), u4[qb])))));
+                const float u1 = uq[(5 * qb) * kRbThreads], u2 = uq[(5 * qb + 1) * kRbThreads];
+                const float u3 = uq[(5 * qb + 2) * kRbThreads], u4 = uq[(5 * qb + 3) * kRbThreads];
+                const float least = fmaf(ge.x, u1, fmaf(-ge.y, fabsf(u1), fmaf(ge.z, u2, fmaf(ge.w, u3,
+                                    fmaf(-ge_half_s, fabsf(u3), u4)))));
                 const floatx16& r = acc[qb][i];
                 float top = fmaxf(fmaxf(r[0], r[1]), r[2]);
                 top = fmaxf(fmaxf(top, r[3]), r[4]);
@@ -469,7 +510,7 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
                     uint64_t any = 0;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const float thr = fmaf(cs[j], u3[qb], fmaf(cb[j], u2[qb], fmaf(ca[j], u1[qb], u4[qb])));
+                        const float thr = fmaf(cs[j], u3, fmaf(cb[j], u2, fmaf(ca[j], u1, u4)));
                         pass[j] = acc[qb][i][4 * gq + j] >= thr;
                         any |= __ballot(pass[j]);
                     }
@@ -584,6 +625,33 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
     }
 }
 
+template <bool LISTS, uint32_t KG>
+static int
+launch_rb_kernel_g(dim3 grid, size_t lds, hipStream_t st, const PrefilterRbArgs& p) {
+    VA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(prefilter_rb_kernel<LISTS, KG>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+    hipLaunchKernelGGL((prefilter_rb_kernel<LISTS, KG>), grid, dim3(kRbThreads), lds, st, p);
+    return 0;
+}
+
+template <bool LISTS>
+static int
+launch_rb_kernel(uint32_t granules, dim3 grid, size_t lds, hipStream_t st, const PrefilterRbArgs& p) {
+    switch (granules) {
+        case 1: return launch_rb_kernel_g<LISTS, 1>(grid, lds, st, p);
+        case 2: return launch_rb_kernel_g<LISTS, 2>(grid, lds, st, p);
+        case 3: return launch_rb_kernel_g<LISTS, 3>(grid, lds, st, p);
+        case 4: return launch_rb_kernel_g<LISTS, 4>(grid, lds, st, p);
+        case 5: return launch_rb_kernel_g<LISTS, 5>(grid, lds, st, p);
+        case 6: return launch_rb_kernel_g<LISTS, 6>(grid, lds, st, p);
+        case 7: return launch_rb_kernel_g<LISTS, 7>(grid, lds, st, p);
+        case 8: return launch_rb_kernel_g<LISTS, 8>(grid, lds, st, p);
+        default: break;
+    }
+    return fail(VSAG_AMD_INVALID_ARGUMENT, "the rabitq matrix-core pass takes codes of at most %u granules, got %u", kRbMaxG,
+                granules);
+}
+
 bool
 prefilter_rb_supports(const vsag_amd_store* s) {
     return s->kind == VSAG_AMD_KIND_RABITQ && s->query_bits == 4 && s->nlist == 0 && s->G <= kRbMaxG && s->f4tiles != nullptr &&
@@ -656,18 +724,10 @@ launch_prefilter_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uin
     p.groups = sub_lists / (2 * kRbWaves);
     VA_CHECK_ARG(sub_lists == prefilter_rb_sub_lists(nq, tile_end - tile_begin), "candidate lists do not match the grid");
     const size_t lds = static_cast<size_t>(4 * s->G) * kRbQueries * 24 + kRbWaves * kRbWaveFloats * sizeof(float) +
-                       4 * kRbThreads * sizeof(uint32_t);
+                       (4 + 20) * kRbThreads * sizeof(uint32_t);
     dim3 grid(p.groups, static_cast<uint32_t>(nq_pad / kRbQueries));
     timing_begin(st);
-    if (l2) {
-        VA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(prefilter_rb_kernel<VSAG_AMD_METRIC_L2>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        hipLaunchKernelGGL(prefilter_rb_kernel<VSAG_AMD_METRIC_L2>, grid, dim3(kRbThreads), lds, st, p);
-    } else {
-        VA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(prefilter_rb_kernel<VSAG_AMD_METRIC_IP>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        hipLaunchKernelGGL(prefilter_rb_kernel<VSAG_AMD_METRIC_IP>, grid, dim3(kRbThreads), lds, st, p);
-    }
+    VA_TRY(launch_rb_kernel<false>(s->G, grid, lds, st, p));
     timing_end(st);
     VA_HIP(hipGetLastError());
     return 0;
@@ -740,21 +800,13 @@ launch_ivf_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     p.partial_cnt = partial_cnt;
     p.gate = gate;
     const size_t lds = static_cast<size_t>(4 * s->G) * kRbQueries * 24 + kRbWaves * kRbWaveFloats * sizeof(float) +
-                       4 * kRbThreads * sizeof(uint32_t);
+                       (4 + 20) * kRbThreads * sizeof(uint32_t);
     const uint64_t pairs = nq * (nprobe - p0);
     const uint64_t max_items =
         (div_up(pairs, static_cast<uint64_t>(kRbQueries)) + std::min<uint64_t>(s->nlist, pairs)) * kIvfRbChunks;
     const dim3 grid(static_cast<uint32_t>(max_items));
     timing_begin(st);
-    if (l2) {
-        VA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(prefilter_rb_kernel<VSAG_AMD_METRIC_L2, true>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        hipLaunchKernelGGL((prefilter_rb_kernel<VSAG_AMD_METRIC_L2, true>), grid, dim3(kRbThreads), lds, st, p);
-    } else {
-        VA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(prefilter_rb_kernel<VSAG_AMD_METRIC_IP, true>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        hipLaunchKernelGGL((prefilter_rb_kernel<VSAG_AMD_METRIC_IP, true>), grid, dim3(kRbThreads), lds, st, p);
-    }
+    VA_TRY(launch_rb_kernel<true>(s->G, grid, lds, st, p));
     timing_end(st);
     VA_HIP(hipGetLastError());
     return 0;
