@@ -440,7 +440,7 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
     uint64_t tau = (static_cast<uint64_t>(bs) << 32) | 0xFFFFFFFFULL;
     const uint32_t qidx[1] = {q};
     const QueryRows<1> qrows = query_rows<1>(a, qidx);
-    auto rescore = [&](const uint32_t* mine, uint32_t total) {
+    auto rescore = [&](const uint32_t* mine, uint32_t total) __attribute__((always_inline)) {
         for (uint32_t base = 0; base < total; base += kWave) {
             const bool have = base + lane < total;
             const uint32_t slot = have ? mine[base + lane] : 0U;
@@ -535,12 +535,15 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
             }
             fill += sum;
         };
-        for (uint32_t g0 = 0; g0 < r.sub_lists; g0 += kWave) {
-            const uint32_t g = g0 + lane;
-            const uint32_t c = g < r.sub_lists ? as_const(counts)[g] : 0U;
+        // The counts of four rounds are asked for together: a query with thousands of (mostly empty) private lists
+        // would otherwise wait for memory once per 64 of them.
+        auto round = [&](uint32_t g, uint32_t c) {
             uint32_t total = c;
             for (int off = 32; off > 0; off >>= 1) {
                 total += __shfl_xor(total, off);
+            }
+            if (total == 0) {
+                return;
             }
             if (total <= r.gather) {
                 gather(g, c);
@@ -548,6 +551,18 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
                 for (uint32_t b0 = 0; b0 < kWave; b0 += piece) {
                     gather(g, lane >= b0 && lane < b0 + piece ? c : 0U);
                 }
+            }
+        };
+        for (uint32_t g4 = 0; g4 < r.sub_lists; g4 += 4 * kWave) {
+            const uint32_t ga = g4 + lane, gb = ga + kWave, gc = gb + kWave, gd = gc + kWave;
+            const uint32_t ca = ga < r.sub_lists ? as_const(counts)[ga] : 0U;
+            const uint32_t cb = gb < r.sub_lists ? as_const(counts)[gb] : 0U;
+            const uint32_t cc = gc < r.sub_lists ? as_const(counts)[gc] : 0U;
+            const uint32_t cd = gd < r.sub_lists ? as_const(counts)[gd] : 0U;
+            // (one call in a loop that stays a loop: four calls would make the rounds a function with a stack frame)
+#pragma nounroll
+            for (uint32_t u = 0; u < 4; ++u) {
+                round(ga + u * kWave, u == 0 ? ca : (u == 1 ? cb : (u == 2 ? cc : cd)));
             }
         }
         wave_lds_fence();

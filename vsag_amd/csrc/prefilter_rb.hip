@@ -4,9 +4,11 @@
 // The streaming kernel forms <code bits, 4-bit query> with sixteen and/popcount pairs per code dword and query; that
 // is what bounds it.  The same integer is a contraction of 0/1 values with the values 0..15.  The matrix cores take
 // 4-bit and 6-bit floats at twice the rate of bytes (v_mfma_scale_f32_32x32x64_f8f6f4): a code bit is the fp4 value 1.0
-// or 0, and a query value v goes in as the fp6 (e2m3) value v - 7.5, one of +-0.5 .. +-7.5, all of which that format
-// holds exactly; the fp32 sums of at most 1024 such products are exact, and the contraction comes out as
-// ip - 7.5 x (set bits of the code), which moves the third factor below by 7.5.  The estimator that turns ip into a
+// or 0, and a query value v goes in as the fp6 (e2m3) value (v - m) / 2 with an integer m of the query's own, one of
+// 0, +-0.5 .. +-7.5, all of which that format holds exactly; the fp32 sums of at most 1024 such products are exact, and
+// the contraction comes out as (ip - m x (set bits of the code)) / 2, which moves the third factor below by m and halves
+// all four.  m is the integer nearest to -u3: what is left of the third factor is at most a half, so the thresholds of
+// neighbouring codes differ by little -- the group test below lives on that.  The estimator that turns ip into a
 // distance (distance.h, finish_distances) is, for a given
 // query and code, an affine function of that integer with a slope of known sign, so "distance <= bound" is
 // "ip >= thr(query, code)" with
@@ -48,23 +50,21 @@ constexpr uint32_t kRbWaves = 8;      // waves per workgroup, two per SIMD: one 
 constexpr uint32_t kRbThreads = kRbWaves * kWave;
 constexpr uint32_t kRbWaveFloats = 3 * kWave + 4 * 8;  // LDS floats of a wave's per-code constants
 
-// The fp6 (e2m3) pattern of v - 7.5 for a 4-bit query value v: sign | exponent (2) | mantissa (3).
+// The fp6 (e2m3) pattern (sign | exponent (2) | mantissa (3)) of k / 2 for an integer k in [-15, 15].
 __device__ inline uint32_t
-rb_fp6(uint32_t v) {
-    // magnitudes 0.5, 1.5, ... 7.5 by index: 0.5 = 0.100 x 2^0 (subnormal), 1.5 = 1.100 x 2^0, 2.5 = 1.010 x 2^1,
-    // 3.5 = 1.110 x 2^1, 4.5 = 1.001 x 2^2, 5.5 = 1.011 x 2^2, 6.5 = 1.101 x 2^2, 7.5 = 1.111 x 2^2
-    const uint32_t idx = v >= 8 ? v - 8 : 7 - v;
-    const uint64_t table = 4ULL | (12ULL << 8) | (18ULL << 16) | (22ULL << 24) | (25ULL << 32) | (27ULL << 40) |
-                           (29ULL << 48) | (31ULL << 56);
-    return static_cast<uint32_t>((table >> (8 * idx)) & 63ULL) | (v >= 8 ? 0U : 32U);
+rb_fp6_half(int k) {
+    // 0, 0.5 (subnormal 0.100), 1, 1.5 | 2, 2.5, 3, 3.5 (steps of 1/4 from 010.000) | 4 .. 7.5 (steps of 1/2 from 011.000)
+    const uint32_t a = static_cast<uint32_t>(k < 0 ? -k : k);
+    const uint32_t mag = a < 4 ? 4 * a : (a < 8 ? 16 + 2 * (a - 4) : 24 + (a - 8));
+    return mag | (k < 0 ? 32U : 0U);
 }
 
-// 4-bit queries as fp6: per query row and code dword w, the 32 values of dimensions 32 w ... as 24 bytes, value t in
-// bits 6 t .. 6 t + 5; the first 16 bytes go to qa[q ndw + w], the last 8 to qb[q ndw + w].  Padding rows are zero
-// (the fp6 value 0).
+// 4-bit queries as fp6: per query row and code dword w, the 32 values of dimensions 32 w ... less the query's offset
+// (offset[q], an integer in [0, 15], rabitq_tau_kernel's u5) and halved, as 24 bytes, value t in bits 6 t .. 6 t + 5;
+// the first 16 bytes go to qa[q ndw + w], the last 8 to qb[q ndw + w].  Padding rows are zero (the fp6 value 0).
 __global__ void __launch_bounds__(256)
-rabitq_query_f6_kernel(const uint32_t* qtab, uint32_t qstride, uint32_t ndw, uint64_t nq, uint64_t nq_pad, uint4* qa,
-                       uint2* qb) {
+rabitq_query_f6_kernel(const uint32_t* qtab, uint32_t qstride, uint32_t ndw, uint64_t nq, uint64_t nq_pad,
+                       const float* offset, uint4* qa, uint2* qb) {
     const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= nq_pad * ndw) {
         return;
@@ -74,11 +74,12 @@ rabitq_query_f6_kernel(const uint32_t* qtab, uint32_t qstride, uint32_t ndw, uin
     uint32_t out[6] = {0, 0, 0, 0, 0, 0};
     if (q < nq) {
         const uint4 v = *reinterpret_cast<const uint4*>(qtab + q * qstride + 4 * w);
+        const int m = static_cast<int>(offset[q]);
 #pragma unroll
         for (uint32_t t = 0; t < 32; ++t) {
             const uint32_t val = ((v.x >> t) & 1U) | (((v.y >> t) & 1U) << 1) | (((v.z >> t) & 1U) << 2) |
                                  (((v.w >> t) & 1U) << 3);
-            const uint64_t code = static_cast<uint64_t>(rb_fp6(val)) << ((6 * t) % 32);
+            const uint64_t code = static_cast<uint64_t>(rb_fp6_half(static_cast<int>(val) - m)) << ((6 * t) % 32);
             out[(6 * t) / 32] |= static_cast<uint32_t>(code);
             if ((6 * t) % 32 > 26) {
                 out[(6 * t) / 32 + 1] |= static_cast<uint32_t>(code >> 32);
@@ -89,7 +90,8 @@ rabitq_query_f6_kernel(const uint32_t* qtab, uint32_t qstride, uint32_t ndw, uin
     qb[i] = make_uint2(out[4], out[5]);
 }
 
-// Per query: u1..u4 of the header and u5 (u[j * nq_pad + q]).  -inf in u4: everything passes; +inf: nothing does.
+// Per query: u1..u4 of the header, halved, and the offset m as u5 (u[j * nq_pad + q]).  -inf in u4: everything passes;
+// +inf: nothing does.
 __global__ void __launch_bounds__(256)
 rabitq_tau_kernel(const float* qmeta, uint32_t qmeta_stride, const uint32_t* bound, int is_l2, uint32_t dpad, uint64_t nq,
                   uint64_t nq_pad, float* u) {
@@ -125,22 +127,19 @@ rabitq_tau_kernel(const float* qmeta, uint32_t qmeta_stride, const uint32_t* bou
                 if (fabs(v1) <= 1.0e4 && inv <= 1.0e4 && fabs(v3) <= 64.0 && fabs(v4) <= 1.0e5) {
                     // The relative margin rides on the factors: a positive threshold comes out 1e-4 lower, a
                     // negative one is passed by every (non-negative) product anyway.
+                    // Everything is halved with the contraction (exactly: a power of two).
                     const double lower = 1.0 - 1.0e-4;
-                    u1 = static_cast<float>(v1 * lower);
-                    u2 = static_cast<float>(inv * lower);
-                    // Less 7.5: the contraction of the matrix cores is ip - 7.5 x set bits.  The factor of the set bits is
-                    // split: its nearest multiple of 1/4 (u5) is taken off in the accumulators, where set bits x u5 and
-                    // every sum on top of it are exact, and only the rest (u3, at most 1/8) stays in the threshold --
-                    // with it the thresholds of a group of codes differ by little, which the group test lives on.
-                    const double x3 = v3 * lower - 7.5;
-                    const double coarse = rint(x3 * 4.0) * 0.25;
-                    u5 = static_cast<float>(coarse);
-                    u3 = static_cast<float>(x3 - coarse);
+                    u1 = static_cast<float>(0.5 * v1 * lower);
+                    u2 = static_cast<float>(0.5 * inv * lower);
+                    // Less the query's offset m: the contraction of the matrix cores is (ip - m x set bits) / 2.
+                    const double m = fmin(15.0, fmax(0.0, rint(v3 * lower)));
+                    u5 = static_cast<float>(m);
+                    u3 = static_cast<float>(0.5 * (v3 * lower - m));
                     // The threshold is a chain of three fp32 fma over terms that may cancel: it is off by at most
                     // 3 x 2^-24 of the sum of their magnitudes, whatever it comes to itself.  2^-20 of the largest
                     // magnitudes any code can bring (A_c <= kRbMaxA, |B_c| <= kRbMaxB, set bits <= dpad) is taken off.
                     const double reach = kRbMaxA * fabs(v1) + kRbMaxB * inv + dpad * fabs(v3) + fabs(v4);
-                    u4 = static_cast<float>(v4 * lower - 9.5367431640625e-7 * reach);
+                    u4 = static_cast<float>(0.5 * (v4 * lower - 9.5367431640625e-7 * reach));
                 }
             }
         }
@@ -319,22 +318,27 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
     }
     // Candidates so far of this lane's four queries (flat stores): in LDS, the registers go to the accumulators.
     uint32_t* ncand = reinterpret_cast<uint32_t*>(cc - wave * kRbWaveFloats + kRbWaves * kRbWaveFloats) + tid;
-    // So do the five factors of each of those queries: uq[(5 qb + j) kRbThreads] is u(j + 1), u5 negated.
+    // So do the four factors of each of those queries: uq[(4 qb + j) kRbThreads] is u(j + 1).
     float* uq = reinterpret_cast<float*>(ncand + 4 * kRbThreads);
 #pragma unroll
     for (int qb = 0; qb < 4; ++qb) {
         ncand[qb * kRbThreads] = 0;
     }
-    const uint32_t sub_lists = p.groups * 2 * kRbWaves;
-    const uint32_t my_sub = (blockIdx.x * kRbWaves + wave) * 2 + half;
+    // Which private list of query q is this lane's (flat stores).  Formed where it is needed -- rarely: the empty
+    // statement keeps the compiler from forming it once, ahead of the loop, and holding it in registers the matrix
+    // instructions want.
+    auto list_of = [&](uint64_t q) -> uint64_t {
+        uint32_t groups = p.groups;
+        asm volatile("" : "+s"(groups));
+        return q * (groups * 2 * kRbWaves) + (blockIdx.x * kRbWaves + wave) * 2 + half;
+    };
 #pragma unroll
     for (int qb = 0; qb < 4; ++qb) {
         const uint64_t q = query_row(32 * qb + l32);
-        uq[(5 * qb + 0) * kRbThreads] = p.u[q];
-        uq[(5 * qb + 1) * kRbThreads] = p.u[p.nq_pad + q];
-        uq[(5 * qb + 2) * kRbThreads] = p.u[2 * p.nq_pad + q];
-        uq[(5 * qb + 3) * kRbThreads] = p.u[3 * p.nq_pad + q];
-        uq[(5 * qb + 4) * kRbThreads] = -p.u[4 * p.nq_pad + q];
+        uq[(4 * qb + 0) * kRbThreads] = p.u[q];
+        uq[(4 * qb + 1) * kRbThreads] = p.u[p.nq_pad + q];
+        uq[(4 * qb + 2) * kRbThreads] = p.u[2 * p.nq_pad + q];
+        uq[(4 * qb + 3) * kRbThreads] = p.u[3 * p.nq_pad + q];
     }
     __syncthreads();
     // LISTS: a pair has eight private lists (two per chunk in ivf_i8.hip's layout); here a hit goes to the one of
@@ -404,25 +408,12 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
         wave_lds_fence();
 
         uint32_t tile_hits[4] = {0, 0, 0, 0};
-        // The accumulators start at -(set bits) x u5: exact, as everything added to it (multiples of 1/4 below 2^17).
+        // The first matrix instruction of an accumulator starts from zero.
         floatx16 acc[4][2];
-        {
-            const float u5n[4] = {uq[4 * kRbThreads], uq[9 * kRbThreads], uq[14 * kRbThreads], uq[19 * kRbThreads]};
+        floatx16 zero;
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-#pragma unroll
-                for (int gq = 0; gq < 4; ++gq) {
-                    const float4 vs = *reinterpret_cast<const float4*>(&cc[2 * kWave + 32 * i + 8 * gq + 4 * half]);
-                    const float cs[4] = {vs.x, vs.y, vs.z, vs.w};
-#pragma unroll
-                    for (int qb = 0; qb < 4; ++qb) {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            acc[qb][i][4 * gq + j] = cs[j] * u5n[qb];
-                        }
-                    }
-                }
-            }
+        for (int e = 0; e < 16; ++e) {
+            zero[e] = 0.0F;
         }
 #pragma unroll kUnroll
         for (uint32_t g = 0; g < KG; ++g) {
@@ -448,10 +439,11 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
                         const intx4 t4 = intx4{static_cast<int>(t.x), static_cast<int>(t.y), 0, 0};
                         const intx8 bv = __builtin_shufflevector(b4, t4, 0, 1, 2, 3, 4, 5, -1, -1);
                         // A: fp4 (4), B: fp6 e2m3 (2); both scales 2^0 (the e8m0 pattern 127)
-                        acc[qb][0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a0, bv, acc[qb][0], 4, 2, 0, 0x7F7F7F7F,
-                                                                                      0, 0x7F7F7F7F);
-                        acc[qb][1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a1, bv, acc[qb][1], 4, 2, 0, 0x7F7F7F7F,
-                                                                                      0, 0x7F7F7F7F);
+                        const bool first = g == 0 && m == 0;
+                        acc[qb][0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a0, bv, first ? zero : acc[qb][0], 4, 2,
+                                                                                      0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+                        acc[qb][1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a1, bv, first ? zero : acc[qb][1], 4, 2,
+                                                                                      0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
                         const uint32_t pair_then = pair + 2;
                         const uint32_t g_then = pair_then < 8 ? g : (g + 1 < KG ? g + 1 : 0);
                         const uint32_t dw_then = 4 * g_then + 2 * ((pair_then % 8) / 4) + half;
@@ -476,8 +468,8 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
             const float ge_half_s = cg[(2 * i + half) * 8 + 4];
 #pragma unroll
             for (int qb = 0; qb < 4; ++qb) {
-                const float u1 = uq[(5 * qb) * kRbThreads], u2 = uq[(5 * qb + 1) * kRbThreads];
-                const float u3 = uq[(5 * qb + 2) * kRbThreads], u4 = uq[(5 * qb + 3) * kRbThreads];
+                const float u1 = uq[(4 * qb) * kRbThreads], u2 = uq[(4 * qb + 1) * kRbThreads];
+                const float u3 = uq[(4 * qb + 2) * kRbThreads], u4 = uq[(4 * qb + 3) * kRbThreads];
                 const float least = fmaf(ge.x, u1, fmaf(-ge.y, fabsf(u1), fmaf(ge.z, u2, fmaf(ge.w, u3,
                                     fmaf(-ge_half_s, fabsf(u3), u4)))));
                 const floatx16& r = acc[qb][i];
@@ -527,7 +519,7 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
                             continue;
                         }
                         const uint64_t q = q0 + 32 * qb + l32;
-                        uint32_t* list = LISTS ? nullptr : p.cand + ((q < p.nq ? q : 0) * sub_lists + my_sub) * p.sub_cap;
+                        uint32_t* list = LISTS ? nullptr : p.cand + list_of(q < p.nq ? q : 0) * p.sub_cap;
                         while (hits != 0) {
                             const uint32_t j = static_cast<uint32_t>(__builtin_ctz(hits));
                             hits &= hits - 1;
@@ -606,7 +598,7 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
                     if (q < p.nq) {
                         const uint32_t have = ncand[qb * kRbThreads];
                         if (have < p.sub_cap) {
-                            p.cand[(q * sub_lists + my_sub) * p.sub_cap + have] = static_cast<uint32_t>(tile * kWave + code);
+                            p.cand[list_of(q) * p.sub_cap + have] = static_cast<uint32_t>(tile * kWave + code);
                         }
                         ncand[qb * kRbThreads] = have + 1;
                     }
@@ -619,7 +611,7 @@ prefilter_rb_kernel(PrefilterRbArgs p) {
         for (int qb = 0; qb < 4; ++qb) {
             const uint64_t q = q0 + 32 * qb + l32;
             if (q < p.nq) {
-                p.cand_cnt[q * sub_lists + my_sub] = ncand[qb * kRbThreads];
+                p.cand_cnt[list_of(q)] = ncand[qb * kRbThreads];
             }
         }
     }
@@ -701,10 +693,10 @@ launch_prefilter_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uin
     uint4* qa = reinterpret_cast<uint4*>(scratch);
     uint2* qb = reinterpret_cast<uint2*>(scratch + static_cast<size_t>(nq_pad) * ndw * 16);
     float* u = reinterpret_cast<float*>(scratch + round_up(static_cast<size_t>(nq_pad) * ndw * 32, 256));
-    hipLaunchKernelGGL(rabitq_query_f6_kernel, dim3(static_cast<uint32_t>(div_up(nq_pad * ndw, 256))), dim3(256), 0, st,
-                       a.qtab, a.qstride, ndw, nq, nq_pad, qa, qb);
     hipLaunchKernelGGL(rabitq_tau_kernel, dim3(static_cast<uint32_t>(div_up(nq_pad, 256))), dim3(256), 0, st, a.qmeta,
                        a.qmeta_stride, bound, l2 ? 1 : 0, s->G * 128, nq, nq_pad, u);
+    hipLaunchKernelGGL(rabitq_query_f6_kernel, dim3(static_cast<uint32_t>(div_up(nq_pad * ndw, 256))), dim3(256), 0, st,
+                       a.qtab, a.qstride, ndw, nq, nq_pad, u + 4 * nq_pad, qa, qb);
     VA_HIP(hipGetLastError());
     PrefilterRbArgs p{};
     p.f4tiles = s->f4tiles;
@@ -724,7 +716,7 @@ launch_prefilter_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uin
     p.groups = sub_lists / (2 * kRbWaves);
     VA_CHECK_ARG(sub_lists == prefilter_rb_sub_lists(nq, tile_end - tile_begin), "candidate lists do not match the grid");
     const size_t lds = static_cast<size_t>(4 * s->G) * kRbQueries * 24 + kRbWaves * kRbWaveFloats * sizeof(float) +
-                       (4 + 20) * kRbThreads * sizeof(uint32_t);
+                       (4 + 16) * kRbThreads * sizeof(uint32_t);
     dim3 grid(p.groups, static_cast<uint32_t>(nq_pad / kRbQueries));
     timing_begin(st);
     VA_TRY(launch_rb_kernel<false>(s->G, grid, lds, st, p));
@@ -772,10 +764,10 @@ launch_ivf_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     uint4* qa = reinterpret_cast<uint4*>(scratch);
     uint2* qb = reinterpret_cast<uint2*>(scratch + static_cast<size_t>(nq_pad) * ndw * 16);
     float* u = reinterpret_cast<float*>(scratch + round_up(static_cast<size_t>(nq_pad) * ndw * 32, 256));
-    hipLaunchKernelGGL(rabitq_query_f6_kernel, dim3(static_cast<uint32_t>(div_up(nq_pad * ndw, 256))), dim3(256), 0, st,
-                       a.qtab, a.qstride, ndw, nq, nq_pad, qa, qb);
     hipLaunchKernelGGL(rabitq_tau_kernel, dim3(static_cast<uint32_t>(div_up(nq_pad, 256))), dim3(256), 0, st, a.qmeta,
                        a.qmeta_stride, bound, l2 ? 1 : 0, s->G * 128, nq, nq_pad, u);
+    hipLaunchKernelGGL(rabitq_query_f6_kernel, dim3(static_cast<uint32_t>(div_up(nq_pad * ndw, 256))), dim3(256), 0, st,
+                       a.qtab, a.qstride, ndw, nq, nq_pad, u + 4 * nq_pad, qa, qb);
     VA_HIP(hipGetLastError());
     PrefilterRbArgs p{};
     p.f4tiles = s->f4tiles;
@@ -800,7 +792,7 @@ launch_ivf_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     p.partial_cnt = partial_cnt;
     p.gate = gate;
     const size_t lds = static_cast<size_t>(4 * s->G) * kRbQueries * 24 + kRbWaves * kRbWaveFloats * sizeof(float) +
-                       (4 + 20) * kRbThreads * sizeof(uint32_t);
+                       (4 + 16) * kRbThreads * sizeof(uint32_t);
     const uint64_t pairs = nq * (nprobe - p0);
     const uint64_t max_items =
         (div_up(pairs, static_cast<uint64_t>(kRbQueries)) + std::min<uint64_t>(s->nlist, pairs)) * kIvfRbChunks;
