@@ -395,6 +395,7 @@ struct RescoreArgs {
     // (a count above sub_cap = that list overflowed); they are gathered into `gather` words of LDS.
     uint32_t sub_lists, sub_cap, gather;
     const uint4* rows;  // the codes a row per code (store.h), or null: read the tiles
+    uint32_t row_granules;  // granules of a row: G, or G + 1 with the code's metadata words behind the code
 };
 
 // Words of LDS for gathered candidates: small, so that many of these one-wave workgroups share a compute unit (the
@@ -448,7 +449,7 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
             const uint32_t ln = slot & 63;
             Acc<KIND, 1> acc;
             acc_reset(acc);
-            const uint4* row = r.rows != nullptr ? r.rows + static_cast<uint64_t>(slot) * a.G : nullptr;
+            const uint4* row = r.rows != nullptr ? r.rows + static_cast<uint64_t>(slot) * r.row_granules : nullptr;
             // A few granules are fetched before the first is used: a candidate's loads wait for memory together.
             // (sq8 l2 holds scale and query of every dimension in flight in scalar registers: two granules' worth; an sq4
             // granule is 32 dimensions.)
@@ -469,7 +470,16 @@ rescore_kernel(ScanArgs a, RescoreArgs r) {
                 }
             }
             float d[1];
-            finish_distances<KIND, METRIC, 1>(a, qidx, slot, acc, d);
+            if (r.row_granules > a.G) {
+                // The metadata words of the code sit behind it in the row: the same words in the same arithmetic, but one
+                // run of memory per candidate instead of a line per word.
+                ScanArgs b = a;
+                b.meta = reinterpret_cast<const uint32_t*>(row + a.G);
+                b.meta_stride = 1;
+                finish_distances<KIND, METRIC, 1>(b, qidx, 0, acc, d);
+            } else {
+                finish_distances<KIND, METRIC, 1>(a, qidx, slot, acc, d);
+            }
             const uint64_t key = make_key(d[0], slot);
             bool pass = have && slot < r.n && key <= tau;
             uint64_t mask = __ballot(pass);
@@ -1184,6 +1194,7 @@ launch_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t
     r.sub_cap = sub_cap;
     r.gather = std::max(kRescoreGather, sub_cap);
     r.rows = s->rows;
+    r.row_granules = s->row_granules;
     dim3 rgrid(static_cast<uint32_t>(nq));
     const size_t lds = S * 8 + (sub_lists != 0 ? r.gather * 4 : 0);
     if (s->kind == VSAG_AMD_KIND_SQ8) {

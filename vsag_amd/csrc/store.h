@@ -85,7 +85,10 @@ struct vsag_amd_store {
     // contraction sees it, kept up to date by append
     // Flat stores the matrix cores pre-select on: the codes once more, a row per code (G granules in a run), for the
     // rescoring of scattered candidates -- one or two memory lines per candidate instead of one per granule.
+    // With metadata words (nmeta > 0) a row is one granule longer: the code's words, so that a candidate is one run of
+    // memory (row_granules = G or G + 1).
     uint4* rows = nullptr;
+    uint32_t row_granules = 0;
     float* pf_term = nullptr;
     uint32_t* pf_ymax = nullptr;
     // 1-bit rabitq stores with 4-bit queries (l2 / ip, at most kRbMaxG granules, no residual), flat or lists: the code

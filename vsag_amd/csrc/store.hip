@@ -237,16 +237,26 @@ keeps_rows(const vsag_amd_store* s) {
            (s->kind == VSAG_AMD_KIND_RABITQ && s->query_bits == 4);
 }
 
-// rows[slot][j] = granule j of the code in `slot`, from the tiles.
+// rows[slot][j] = granule j of the code in `slot`, from the tiles; with row_granules = G + 1 the last granule of a row
+// holds the code's metadata words (zero beyond nmeta).
 __global__ void __launch_bounds__(256)
-rows_from_tiles_kernel(const uint4* tiles, uint32_t G, uint64_t first_slot, uint64_t count, uint4* rows) {
+rows_from_tiles_kernel(const uint4* tiles, uint32_t G, uint32_t row_granules, const uint32_t* meta, uint64_t meta_stride,
+                       uint32_t nmeta, uint64_t first_slot, uint64_t count, uint4* rows) {
     const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (i >= count * G) {
+    if (i >= count * row_granules) {
         return;
     }
-    const uint64_t slot = first_slot + i / G;
-    const uint32_t j = static_cast<uint32_t>(i % G);
-    rows[slot * G + j] = tiles[((slot / kWave) * G + j) * kWave + slot % kWave];
+    const uint64_t slot = first_slot + i / row_granules;
+    const uint32_t j = static_cast<uint32_t>(i % row_granules);
+    if (j < G) {
+        rows[slot * row_granules + j] = tiles[((slot / kWave) * G + j) * kWave + slot % kWave];
+    } else {
+        uint32_t w[4] = {0, 0, 0, 0};
+        for (uint32_t m = 0; m < nmeta && m < 4; ++m) {
+            w[m] = meta[m * meta_stride + slot];
+        }
+        rows[slot * row_granules + j] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
 }
 
 // Stores whose code bits are kept as fp4 operands as well (prefilter_rb.hip).
@@ -405,9 +415,11 @@ grow(vsag_amd_store* s, uint64_t need_tiles, hipStream_t st) {
     }
     uint4* rows = nullptr;
     if (keeps_rows(s)) {
-        VA_HIP(hipMalloc(&rows, cap * kWave * s->G * sizeof(uint4)));
+        s->row_granules = s->G + (s->nmeta > 0 ? 1 : 0);
+        VA_HIP(hipMalloc(&rows, cap * kWave * s->row_granules * sizeof(uint4)));
         if (s->ntiles > 0) {
-            VA_HIP(hipMemcpyAsync(rows, s->rows, s->ntiles * kWave * s->G * sizeof(uint4), hipMemcpyDeviceToDevice, st));
+            VA_HIP(hipMemcpyAsync(rows, s->rows, s->ntiles * kWave * s->row_granules * sizeof(uint4),
+                                  hipMemcpyDeviceToDevice, st));
         }
     }
     uint4* f4tiles = nullptr;
@@ -733,8 +745,8 @@ vsag_amd_store_append(vsag_amd_store_t* s, const uint8_t* codes_dev, uint64_t n,
     hipLaunchKernelGGL(retile_kernel, dim3(static_cast<uint32_t>(div_up(threads, 256))), dim3(256), 0, st, a);
     VA_HIP(hipGetLastError());
     if (s->rows != nullptr) {
-        hipLaunchKernelGGL(rows_from_tiles_kernel, dim3(static_cast<uint32_t>(div_up(threads, 256))), dim3(256), 0, st,
-                           s->tiles, s->G, s->n, n, s->rows);
+        hipLaunchKernelGGL(rows_from_tiles_kernel, dim3(static_cast<uint32_t>(div_up(n * s->row_granules, 256))), dim3(256),
+                           0, st, s->tiles, s->G, s->row_granules, s->meta, s->cap_tiles * kWave, s->nmeta, s->n, n, s->rows);
         VA_HIP(hipGetLastError());
     }
     VA_TRY(launch_code_terms(s, s->n, n, st));
