@@ -939,7 +939,8 @@ def run_c5(env):
         tops = ops / (kms * 1e-3) / 1e12
         roof = {"bound": "mfma", "achieved": tops, "peak": MFMA_F6F4_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": tops / MFMA_F6F4_PEAK_TFLOPS,
-                "traffic": None,
+                # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this launch: profiles/prefilter_rb_rabitq_c5.md
+                "traffic": 951461.0 * 2.00 * 1024 + 218608.0 * 1024 if (n, d, nq, k) == (5000000, 768, 10000, 10) else None,
                 "kernel": "prefilter_rb_kernel<ip> (fp4 x fp6 MFMA, last level)", "kernel_ms": kms, "ops_per_launch": ops,
                 "codes_per_launch": lcodes}
         dtype = "1-bit codes x 4-bit queries: fp4 x fp6 MFMA pre-selection (exact fp32 sums), u32 popcount rescoring"
