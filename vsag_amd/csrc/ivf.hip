@@ -69,7 +69,7 @@ int launch_ivf_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint3
                   const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound, uint32_t kcand, uint8_t* scratch,
                   uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st);
 int launch_ivf_clear_gated(uint32_t* gate, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t* partial_cnt,
-                           const int32_t* buckets, uint32_t* gpairs, uint32_t gpairs_cap, hipStream_t st);
+                           const int32_t* buckets, uint32_t* gpairs, uint32_t gpairs_cap, uint32_t k, hipStream_t st);
 bool ivf_f32_supports(const vsag_amd_store* s);
 uint32_t ivf_f32_pairs_per_item();
 int launch_ivf_f32(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, const uint32_t* pair_off,
@@ -901,7 +901,7 @@ struct IvfBuffers {
     uint32_t* seed;
     uint32_t* partial_cnt;
     uint64_t* partial;
-    uint32_t* gate;       // mfma: nq + 2 (flags, raised gates, their pairs)
+    uint32_t* gate;       // mfma: nq + 3 (flags, raised gates, the pairs to scan again, the pairs queued)
     int32_t* tq;          // mfma: 2 (nq + 1)
     uint32_t* gpairs;     // mfma: pairs of gated queries, kGatedPairsCap
     uint8_t* q8;          // sq8 lists on the matrix cores: the planes of the queries, their scalars and thresholds
@@ -997,7 +997,7 @@ carve_ivf(Carver& c, const vsag_amd_store* s, const ScanPlanIvf& p, uint64_t nq,
     b->seed = c.take<uint32_t>(p.seeded ? nq * kcand : 0);
     b->partial_cnt = c.take<uint32_t>(p.npairs * p.chunks_max);
     b->partial = c.take<uint64_t>(p.npairs * p.chunks_max * kcand);
-    b->gate = c.take<uint32_t>(p.mfma ? nq + 2 : 0);
+    b->gate = c.take<uint32_t>(p.mfma ? nq + 3 : 0);
     b->gpairs = c.take<uint32_t>(p.mfma ? kGatedPairsCap : 0);
     b->tq = c.take<int32_t>(p.mfma ? 2 * (nq + 1) : 0);  // thresholds, then (sq8_uniform) the sums of the query values
     b->q8 = c.take<uint8_t>(p.planes ? ivf_sq8_i8_query_bytes(nq) : p.bits1 ? ivf_rb_scratch_bytes(s, nq) : 0);
@@ -1157,7 +1157,7 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
         uint64_t pairs = nq * (p1 - p0);
         if (pass == 1) {
             fill(FillJob{{b.counts, b.cursor, mfma ? b.gate : nullptr, nullptr, nullptr}, {0U, 0U, 0U, 0U, 0U},
-                         {nlists1, nlists1, mfma ? nq + 2 : 0, 0, 0}});
+                         {nlists1, nlists1, mfma ? nq + 3 : 0, 0, 0}});
         }
         if (pass == 1 && mfma) {
             // Pairs grouped by list once; workgroups of 256 pairs for the matrix cores, then -- for the queries whose
@@ -1170,7 +1170,7 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
                 VA_TRY(launch_ivf_f32(s, a, nq, nprobe, p0, b.pair_off, b.item_off, b.sorted_pair, b.bound, kcand,
                                       reinterpret_cast<float*>(b.tq), b.partial, b.partial_cnt, b.gate, st));
                 VA_TRY(launch_ivf_clear_gated(b.gate, nq, nprobe, p0, b.partial_cnt, buckets_dev, b.gpairs,
-                                              kGatedPairsCap, st));
+                                              kGatedPairsCap, kcand, st));
                 VA_TRY(launch_ivf_rescore(s, a, nq, nprobe, p0, kcand, p.chunks_max, b.partial, b.partial_cnt, b.bound, st));
             } else if (p.pq) {
                 VA_TRY(launch_ivf_pq(s, a, nq, nprobe, p0, kcand, b.pair_off, b.item_off, b.sorted_pair, b.bound, b.tq,
@@ -1179,14 +1179,14 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
                 VA_TRY(launch_ivf_rb(s, a, nq, nprobe, p0, b.pair_off, b.item_off, b.sorted_pair, b.bound, kcand, b.q8,
                                      b.partial, b.partial_cnt, b.gate, st));
                 VA_TRY(launch_ivf_clear_gated(b.gate, nq, nprobe, p0, b.partial_cnt, buckets_dev, b.gpairs,
-                                              kGatedPairsCap, st));
+                                              kGatedPairsCap, kcand, st));
                 VA_TRY(launch_ivf_rescore(s, a, nq, nprobe, p0, kcand, p.chunks_max, b.partial, b.partial_cnt, b.bound, st));
             } else if (p.planes) {
                 VA_TRY(launch_ivf_sq8_i8(s, reinterpret_cast<const float*>(a.qtab), a.qstride, a.qmeta, a.qmeta_stride, nq,
                                          nprobe, p0, b.pair_off, b.item_off, b.sorted_pair, b.bound, kcand, b.q8, b.q8_u,
                                          b.q8_tau, b.partial, b.partial_cnt, b.gate, st));
                 VA_TRY(launch_ivf_clear_gated(b.gate, nq, nprobe, p0, b.partial_cnt, buckets_dev, b.gpairs,
-                                              kGatedPairsCap, st));
+                                              kGatedPairsCap, kcand, st));
                 VA_TRY(launch_ivf_rescore(s, a, nq, nprobe, p0, kcand, p.chunks_max, b.partial, b.partial_cnt, b.bound, st));
             } else {
                 VA_TRY(launch_ivf_i8(s, a, nq, nprobe, p0, kcand, b.pair_off, b.item_off, b.sorted_pair, b.bound, b.tq,

@@ -498,7 +498,8 @@ ivf_i8_kernel(IvfI8Args p) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             if (pair[j] != 0xFFFFFFFFU) {
-                p.partial_cnt[my_list[j]] = ncand[j] < p.k ? ncand[j] : p.k;
+                // k + 1 for a list that overflowed: that is how the pair is told from the query's other pairs afterwards
+                p.partial_cnt[my_list[j]] = ncand[j] <= p.k ? ncand[j] : p.k + 1;
                 if (ncand[j] > p.k) {
                     if (atomicExch(&p.gate[qidx[j]], 1U) == 0U) {
                         atomicAdd(&p.gate[p.dummy_query], 1U);
@@ -588,11 +589,25 @@ ivf_i8_finish_kernel(IvfI8FinishArgs p) {
     p.partial_cnt[list] = kept;
 }
 
-// Gated queries: the streaming kernel rescans their lists, so what the matrix-core pass left must not count.  Their
-// pairs with a list are queued for that rescan (gate[nq + 1] counts them, also beyond the queue's capacity).
+// Gated queries: one of their private lists overflowed, so the streaming kernel scans lists again for them.  Which:
+// the pairs (query, list) whose own private lists overflowed -- the other lists of the query are whole and stay -- as
+// long as the direct launch has room for all such pairs (gpairs_cap); beyond that every pair of a gated query, through
+// the streaming kernel's own grouping, and then nothing the matrix-core pass left for the query may count.  Two
+// launches, a thread per pair: the first counts the overflowed pairs (gate[nq + 1]), the second empties the private lists
+// of the pairs to scan again and queues them (gate[nq + 2] counts the queue; in the second case gate[nq + 1] is left
+// above the capacity, which is what the streaming launches look at).
+__device__ inline bool
+ivf_pair_overflowed(const uint32_t* partial_cnt, uint64_t pair, uint32_t k) {
+    bool over = false;
+    for (uint32_t l = 0; l < 2 * kIvfI8Chunks; ++l) {
+        over = over || partial_cnt[2 * kIvfI8Chunks * pair + l] > k;
+    }
+    return over;
+}
+
 __global__ void __launch_bounds__(256)
-ivf_i8_clear_gated_kernel(uint32_t* gate, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t* partial_cnt,
-                          const int32_t* buckets, uint32_t* gpairs, uint32_t gpairs_cap) {
+ivf_i8_count_gated_kernel(uint32_t* gate, uint64_t nq, uint32_t nprobe, uint32_t p0, const uint32_t* partial_cnt,
+                          const int32_t* buckets, uint32_t k) {
     const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     const uint64_t per = nprobe - p0;
     if (i >= nq * per || gate[nq] == 0) {
@@ -601,14 +616,32 @@ ivf_i8_clear_gated_kernel(uint32_t* gate, uint64_t nq, uint32_t nprobe, uint32_t
     const uint64_t q = i / per;
     if (gate[q] != 0) {
         const uint64_t pair = q * nprobe + p0 + i % per;
+        if (buckets[pair] >= 0 && ivf_pair_overflowed(partial_cnt, pair, k)) {
+            atomicAdd(&gate[nq + 1], 1U);
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256)
+ivf_i8_clear_gated_kernel(uint32_t* gate, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t* partial_cnt,
+                          const int32_t* buckets, uint32_t* gpairs, uint32_t gpairs_cap, uint32_t k) {
+    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const uint64_t per = nprobe - p0;
+    if (i >= nq * per || gate[nq] == 0) {
+        return;
+    }
+    const uint64_t q = i / per;
+    if (gate[q] != 0) {
+        const uint64_t pair = q * nprobe + p0 + i % per;
+        const bool by_pair = gate[nq + 1] <= gpairs_cap;  // fixed by the first launch
+        if (by_pair && !ivf_pair_overflowed(partial_cnt, pair, k)) {
+            return;
+        }
         for (uint32_t l = 0; l < 2 * kIvfI8Chunks; ++l) {
             partial_cnt[2 * kIvfI8Chunks * pair + l] = 0;
         }
-        if (buckets[pair] >= 0) {
-            const uint32_t pos = atomicAdd(&gate[nq + 1], 1U);
-            if (pos < gpairs_cap) {
-                gpairs[pos] = static_cast<uint32_t>(pair);
-            }
+        if (by_pair && buckets[pair] >= 0) {
+            gpairs[atomicAdd(&gate[nq + 2], 1U)] = static_cast<uint32_t>(pair);
         }
     }
 }
@@ -631,10 +664,12 @@ ivf_i8_supports(const vsag_amd_store* s) {
 // emptied and their pairs queued (see ivf_i8_clear_gated_kernel).
 int
 launch_ivf_clear_gated(uint32_t* gate, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t* partial_cnt,
-                       const int32_t* buckets, uint32_t* gpairs, uint32_t gpairs_cap, hipStream_t st) {
+                       const int32_t* buckets, uint32_t* gpairs, uint32_t gpairs_cap, uint32_t k, hipStream_t st) {
     const uint64_t pairs = nq * (nprobe - p0);
+    hipLaunchKernelGGL(ivf_i8_count_gated_kernel, dim3(static_cast<uint32_t>(div_up(pairs, 256))), dim3(256), 0, st, gate,
+                       nq, nprobe, p0, partial_cnt, buckets, k);
     hipLaunchKernelGGL(ivf_i8_clear_gated_kernel, dim3(static_cast<uint32_t>(div_up(pairs, 256))), dim3(256), 0, st, gate,
-                       nq, nprobe, p0, partial_cnt, buckets, gpairs, gpairs_cap);
+                       nq, nprobe, p0, partial_cnt, buckets, gpairs, gpairs_cap, k);
     VA_HIP(hipGetLastError());
     return 0;
 }
@@ -701,7 +736,7 @@ launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     }
     timing_end(st);
     VA_HIP(hipGetLastError());
-    VA_TRY(launch_ivf_clear_gated(gate, nq, nprobe, p0, partial_cnt, buckets, gpairs, gpairs_cap, st));
+    VA_TRY(launch_ivf_clear_gated(gate, nq, nprobe, p0, partial_cnt, buckets, gpairs, gpairs_cap, kcand, st));
     IvfI8FinishArgs f{};
     f.partial = partial;
     f.partial_cnt = partial_cnt;

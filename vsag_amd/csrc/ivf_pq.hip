@@ -30,7 +30,7 @@ namespace vsag_amd {
 void timing_begin(hipStream_t st);
 void timing_end(hipStream_t st);
 int launch_ivf_clear_gated(uint32_t* gate, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t* partial_cnt,
-                           const int32_t* buckets, uint32_t* gpairs, uint32_t gpairs_cap, hipStream_t st);
+                           const int32_t* buckets, uint32_t* gpairs, uint32_t gpairs_cap, uint32_t k, hipStream_t st);
 uint32_t ivf_i8_lists_per_pair();
 
 typedef int intx4 __attribute__((ext_vector_type(4)));
@@ -289,7 +289,8 @@ ivf_pq_kernel(IvfPqArgs p) {
         const uint32_t pr = spair[tid];
         if (pr != 0xFFFFFFFFU) {
             const uint32_t n = cnt[tid];
-            p.partial_cnt[static_cast<uint64_t>(pr) * p.lists_per_pair + chunk] = n < p.k ? n : p.k;
+            // k + 1 for a list that overflowed: that is how the pair is told from the query's other pairs afterwards
+            p.partial_cnt[static_cast<uint64_t>(pr) * p.lists_per_pair + chunk] = n <= p.k ? n : p.k + 1;
             if (n > p.k) {
                 const uint32_t q = pr / p.nprobe;
                 if (atomicExch(&p.gate[q], 1U) == 0U) {
@@ -416,7 +417,7 @@ launch_ivf_pq(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t 
     }
     timing_end(st);
     VA_HIP(hipGetLastError());
-    VA_TRY(launch_ivf_clear_gated(gate, nq, nprobe, p0, partial_cnt, buckets, gpairs, gpairs_cap, st));
+    VA_TRY(launch_ivf_clear_gated(gate, nq, nprobe, p0, partial_cnt, buckets, gpairs, gpairs_cap, kcand, st));
     IvfPqFinishArgs f{};
     f.partial = partial;
     f.partial_cnt = partial_cnt;

@@ -1025,15 +1025,6 @@ ivf_f32_kernel(IvfF32Args p) {
     }
 }
 
-// counts[i] = min(counts[i], k): the lists of ivf_f32_kernel are counted with atomics that run past the capacity.
-__global__ void
-clamp_counts_kernel(uint32_t* counts, uint64_t n, uint32_t k) {
-    const uint64_t i = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (i < n && counts[i] > k) {
-        counts[i] = k;
-    }
-}
-
 bool
 ivf_f32_supports(const vsag_amd_store* s) {
     return (s->kind == VSAG_AMD_KIND_FP32 || s->kind == VSAG_AMD_KIND_SQ8) && s->nlist > 0 && s->pf_term != nullptr &&
@@ -1091,10 +1082,8 @@ launch_ivf_f32(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t
     }
     timing_end(st);
     VA_HIP(hipGetLastError());
-    const uint64_t lists = nq * nprobe * 2 * kIvfF32Chunks;
-    hipLaunchKernelGGL(clamp_counts_kernel, dim3(static_cast<uint32_t>(div_up(lists, 256))), dim3(256), 0, st, partial_cnt,
-                       lists, kcand);
-    VA_HIP(hipGetLastError());
+    // (Counts run past the capacity where a list overflowed; those lists are emptied with their pair's, or their
+    // query's, before anything reads them: launch_ivf_clear_gated.)
     return 0;
 }
 

@@ -1016,6 +1016,12 @@ ivf_sq8_i8_kernel(IvfSq8Args p) {
                             const bool pass = judged(blk, e) >= static_cast<int32_t>(tau[j]) && live[j];
                             if (__ballot(pass) != 0 && pass) {
                                 const uint64_t slot = slot0 + 32 * r + 8 * (e >> 2) + 4 * half + (e & 3);
+                                // The second tile of the last stage may lie behind the chunk: its staged codes and term
+                                // fail every threshold but that of a query without a bound, which everything passes --
+                                // and behind the chunk lies the next chunk, or the next list.
+                                if (slot >= static_cast<uint64_t>(tile_end) * kWave) {
+                                    continue;
+                                }
                                 if (ncand[j] < p.k) {
                                     p.partial[my_list[j] * p.k + ncand[j]] = slot;
                                 }
@@ -1036,7 +1042,8 @@ ivf_sq8_i8_kernel(IvfSq8Args p) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             if (live[j]) {
-                p.partial_cnt[my_list[j]] = ncand[j] < p.k ? ncand[j] : p.k;
+                // k + 1 for a list that overflowed: that is how the pair is told from the query's other pairs afterwards
+                p.partial_cnt[my_list[j]] = ncand[j] <= p.k ? ncand[j] : p.k + 1;
                 if (ncand[j] > p.k) {
                     if (atomicExch(&p.gate[qidx[j]], 1U) == 0U) {
                         atomicAdd(&p.gate[p.dummy_query], 1U);
