@@ -815,8 +815,10 @@ def run_c4(env):
                                                                         nprobe - 1), "kernel_ms": kms,
                 "ops_per_launch": ops, "distance_evaluations_per_launch": float(rest),
                 "distance_evaluations_per_second": float(rest) / (kms * 1e-3)}
-    return env.base_line("QPS @ recall@10 (IVF %s, 10M x 128)" % {"sq4_uniform": "SQ4-uniform", "sq8_uniform": "SQ8-uniform",
-                                                                  "sq8": "SQ8", "rabitq": "RaBitQ", "pqfs": "PQFS", "fp32": "FP32"}[kind_name],
+    return env.base_line("QPS @ recall@10 (IVF %s, %s x %d)" % ({"sq4_uniform": "SQ4-uniform", "sq8_uniform": "SQ8-uniform",
+                                                                "sq8": "SQ8", "rabitq": "RaBitQ", "pqfs": "PQFS",
+                                                                "fp32": "FP32"}[kind_name],
+                                                               "%dM" % (n // 1000000) if n % 1000000 == 0 else str(n), d),
                          "queries/s", nq / sec, sec, "f32" if raw32 else "4-bit pq codes, u8 table sums in i32" if pqfs else
                          "1-bit codes x u4 queries, i32 popcount sums, f32 estimator" if one_bit else
                          "u8 codes x f32 scale, f32 (pre-selection: i8 x i8, i32 sums)" if per_dim else "u%d codes, i32 dot" % bits,

@@ -389,12 +389,10 @@ constexpr uint32_t kIvfSeedTiles = 4;
 
 // CHUNKED: work items are chunks of lists and start cold together (few queries); otherwise whole lists.
 template <int KIND, int METRIC, int T, bool CHUNKED>
-__global__ void __launch_bounds__(256)
-ivf_scan_kernel(ScanArgs a, IvfArgs v) {
-    extern __shared__ uint64_t lds[];
+__device__ __forceinline__ void
+ivf_scan_item(const ScanArgs& a, const IvfArgs& v, uint64_t* lds, uint32_t item) {
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t item = blockIdx.x * (blockDim.x >> 6) + wave;
     uint32_t list_begin, list_end, local, pfirst, plast;
     cu32_p pairs_src = as_const(v.sorted_pair);
     if (v.direct != nullptr) {
@@ -626,6 +624,29 @@ ivf_scan_kernel(ScanArgs a, IvfArgs v) {
         if (admitted != 0) {
             selector_copy_admitted(keys, total, bs, v.partial + list * k, lane);
         }
+    }
+}
+
+// A wave is a work item.  The direct launch (v.direct) serves a queue whose length only the device knows: a grid sized
+// for its capacity would be tens of thousands of workgroups that find nothing to do, so there the waves of a smaller
+// grid take the items in turn.
+template <int KIND, int METRIC, int T, bool CHUNKED>
+__global__ void __launch_bounds__(256)
+ivf_scan_kernel(ScanArgs a, IvfArgs v) {
+    extern __shared__ uint64_t lds[];
+    const uint32_t waves = blockDim.x >> 6;
+    uint32_t item = blockIdx.x * waves + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (v.direct == nullptr) {
+        ivf_scan_item<KIND, METRIC, T, CHUNKED>(a, v, lds, item);
+        return;
+    }
+    const uint32_t count = as_const(v.direct_count)[0];
+    const uint32_t stride = gridDim.x * waves;
+    const uint32_t limit = count <= v.direct_cap ? count * v.chunks_max : 0;
+    for (; item < limit; item += stride) {
+        ivf_scan_item<KIND, METRIC, T, CHUNKED>(a, v, lds, item);
+        // the selectors of the item in LDS have been read before the next item resets them
+        wave_lds_fence();
     }
 }
 
@@ -1203,7 +1224,9 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
             while (dwaves > 1 && static_cast<size_t>(dwaves) * p.S * 8 > 65536) {
                 dwaves >>= 1;
             }
-            dim3 dgrid(static_cast<uint32_t>(div_up(static_cast<uint64_t>(kGatedPairsCap) * d.chunks_max, dwaves)));
+            // (the waves of this grid take the queued items in turn: see ivf_scan_kernel)
+            dim3 dgrid(static_cast<uint32_t>(std::min<uint64_t>(div_up(static_cast<uint64_t>(kGatedPairsCap) * d.chunks_max, dwaves),
+                                                                8ull * static_cast<uint64_t>(device_cu_count()))));
             VA_TRY(launch_ivf(s, 1, dgrid, dim3(dwaves * kWave), static_cast<size_t>(dwaves) * p.S * 8, st, a, d));
             // Many: the streaming kernel's items over the same grouping (stands back otherwise).
             hipLaunchKernelGGL(offsets_kernel, dim3(1), dim3(1024), 0, st, b.counts, s->list_tile_dev, s->nlist,

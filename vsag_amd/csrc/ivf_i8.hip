@@ -548,42 +548,59 @@ ivf_i8_finish_kernel(IvfI8FinishArgs p) {
     const float qm = p.qmeta[q * p.qmeta_stride];
     const uint32_t bound = p.bound[q];
     uint64_t* keys = p.partial + list * p.k;
+    // Four records at a time: their loads (record, then id and scalars of its slot) are in flight together, which is
+    // what a full list -- a query with a loose bound -- waits for.  Kept keys go to the front of the list, never past
+    // the records already read.
     uint32_t kept = 0;
-    for (uint32_t i = 0; i < count; ++i) {
-        const uint64_t rec = keys[i];
-        const uint64_t slot = rec >> 32;
-        const int32_t acc = static_cast<int32_t>(static_cast<uint32_t>(rec));
-        const uint32_t id = p.ids[slot];
-        if (id == VSAG_AMD_INVALID_ID) {
-            continue;
+    for (uint32_t i0 = 0; i0 < count; i0 += 4) {
+        uint64_t recs[4];
+        uint32_t idv[4];
+        float m0v[4];
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            recs[u] = keys[i0 + u < count ? i0 + u : count - 1];
         }
-        const float m0 = __uint_as_float(p.meta[slot]);
-        float dist;
-        if constexpr (KIND == VSAG_AMD_KIND_SQ8_UNIFORM && METRIC != VSAG_AMD_METRIC_L2) {
-            // acc = X, <q, o> = X + 128 sum_q + 128 sum_o - 128^2 dim
-            const int32_t ip = acc + 128 * p.qsum[q] + static_cast<int32_t>(128U * p.meta_sum[slot]) -
-                               static_cast<int32_t>(16384U * p.dim);
-            const float result = static_cast<float>(ip);
-            const float rr = p.lb * (qm + m0) + p.rate * result + p.lb2;
-            dist = 1 - rr;
-        } else if constexpr (KIND == VSAG_AMD_KIND_SQ8_UNIFORM) {
-            // acc = X + C_o, <q, o> = X + 128 sum_q + 128 sum_o - 128^2 dim (see the header)
-            const uint32_t so = p.meta_sum[slot];
-            const int32_t ip = acc - ivf_i8_centre_term(so, m0) + 128 * p.qsum[q] + static_cast<int32_t>(128U * so) -
-                               static_cast<int32_t>(16384U * p.dim);
-            const float result = static_cast<float>(ip);
-            dist = (qm + m0 - 2 * result) * p.rate;
-        } else if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
-            // acc = 2 <q, o> - No with No = m0, an integer
-            const float result = static_cast<float>((acc + static_cast<int32_t>(m0)) >> 1);
-            dist = (qm + m0 - 2 * result) * p.rate;
-        } else {
-            const float result = static_cast<float>(acc);
-            const float rr = p.lb * (qm + m0) + p.rate * result + p.lb2;
-            dist = 1 - rr;
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            idv[u] = p.ids[recs[u] >> 32];
+            m0v[u] = __uint_as_float(p.meta[recs[u] >> 32]);
         }
-        if (float_to_ordered(dist) <= bound) {
-            keys[kept++] = make_key(dist, id);
+#pragma unroll
+        for (uint32_t u = 0; u < 4; ++u) {
+            const uint64_t slot = recs[u] >> 32;
+            const int32_t acc = static_cast<int32_t>(static_cast<uint32_t>(recs[u]));
+            const uint32_t id = idv[u];
+            if (i0 + u >= count || id == VSAG_AMD_INVALID_ID) {
+                continue;
+            }
+            const float m0 = m0v[u];
+            float dist;
+            if constexpr (KIND == VSAG_AMD_KIND_SQ8_UNIFORM && METRIC != VSAG_AMD_METRIC_L2) {
+                // acc = X, <q, o> = X + 128 sum_q + 128 sum_o - 128^2 dim
+                const int32_t ip = acc + 128 * p.qsum[q] + static_cast<int32_t>(128U * p.meta_sum[slot]) -
+                                   static_cast<int32_t>(16384U * p.dim);
+                const float result = static_cast<float>(ip);
+                const float rr = p.lb * (qm + m0) + p.rate * result + p.lb2;
+                dist = 1 - rr;
+            } else if constexpr (KIND == VSAG_AMD_KIND_SQ8_UNIFORM) {
+                // acc = X + C_o, <q, o> = X + 128 sum_q + 128 sum_o - 128^2 dim (see the header)
+                const uint32_t so = p.meta_sum[slot];
+                const int32_t ip = acc - ivf_i8_centre_term(so, m0) + 128 * p.qsum[q] + static_cast<int32_t>(128U * so) -
+                                   static_cast<int32_t>(16384U * p.dim);
+                const float result = static_cast<float>(ip);
+                dist = (qm + m0 - 2 * result) * p.rate;
+            } else if constexpr (METRIC == VSAG_AMD_METRIC_L2) {
+                // acc = 2 <q, o> - No with No = m0, an integer
+                const float result = static_cast<float>((acc + static_cast<int32_t>(m0)) >> 1);
+                dist = (qm + m0 - 2 * result) * p.rate;
+            } else {
+                const float result = static_cast<float>(acc);
+                const float rr = p.lb * (qm + m0) + p.rate * result + p.lb2;
+                dist = 1 - rr;
+            }
+            if (float_to_ordered(dist) <= bound) {
+                keys[kept++] = make_key(dist, id);
+            }
         }
     }
     p.partial_cnt[list] = kept;
