@@ -66,13 +66,14 @@ def test_random_configuration(lib, seed):
     st.destroy()
 
 
-@pytest.mark.parametrize("seed", range(8))
+@pytest.mark.parametrize("seed", range(14))
 def test_random_rabitq_configuration(lib, seed):
-    """1-bit RaBitQ codes against 4-bit queries: the int8 pre-selection against the streaming popcount kernel on seeded
-    random sizes, dimensions (padded and unpadded), k, metrics, centred and far-off data, duplicated queries."""
+    """1-bit RaBitQ codes against 4-bit queries: the matrix-core pre-selection against the streaming popcount kernel on
+    seeded random sizes, dimensions (padded and unpadded; one to eight granules per code, each of which has a kernel of its
+    own), k, metrics, centred and far-off data, duplicated queries."""
     L = lib.load_library()
     rng = np.random.default_rng(2000 + seed)
-    d = int(rng.choice([32, 64, 100, 128, 200, 256, 384, 512, 960]))
+    d = [32, 100, 128, 200, 384, 512, 600, 640, 768, 800, 896, 960, 64, 256][seed % 14]
     n = int(rng.integers(8000, 60000))
     nq = int(rng.integers(130, 900))
     k = int(rng.choice([1, 10, 50, 100, 200, 256]))
