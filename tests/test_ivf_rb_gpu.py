@@ -50,7 +50,14 @@ def _same(a, b):
 @pytest.mark.parametrize("n,d,nlist,nq,nprobe,kcand,unit", [(60000, 128, 64, 2100, 16, 100, False),
                                                             (30000, 100, 37, 4500, 8, 10, True),
                                                             (20000, 768, 16, 5000, 4, 32, True),
-                                                            (20000, 33, 16, 9000, 4, 5, False)])
+                                                            (20000, 33, 16, 9000, 4, 5, False),
+                                                            # the other granule counts (a kernel each): 2, 3, 4, 5, 7, 8
+                                                            (12000, 256, 16, 5000, 4, 20, True),
+                                                            (12000, 384, 16, 5000, 4, 20, False),
+                                                            (12000, 500, 16, 5000, 4, 20, True),
+                                                            (12000, 640, 16, 5000, 4, 20, True),
+                                                            (12000, 800, 16, 5000, 4, 20, False),
+                                                            (12000, 1024, 16, 5000, 4, 20, True)])
 def test_matrix_core_columns_equal_streaming(lib, metric, n, d, nlist, nq, nprobe, kcand, unit):
     x, q, cent, labels, codes, (rot, cen), st = _case(n + d + metric, n, d, nlist, nq, metric, unit=unit)
     buckets, _ = orc.ivf_route(cent, q, nprobe)
