@@ -140,3 +140,32 @@ def test_one_long_list_among_short_and_empty_ones(lib):
     plain, fast = _both(lib, st, q, buckets, kcand)
     assert _same(plain, fast)
     st.destroy()
+
+
+def test_lists_grown_by_appends_keep_their_matrix_core_copies(lib):
+    """The store keeps the code bits and per-code constants of rabitq lists once more for the matrix cores and renews
+    them whenever codes are added (lists outgrow their room and move): a store grown in ragged pieces, one of them into
+    empty lists, must answer like one built at once, on both paths."""
+    from gpu_helpers import dev
+    n, d, nlist, nq, nprobe, kcand, metric = 30000, 200, 24, 4000, 6, 40, orc.L2
+    x, q, cent, labels, codes, (rot, cen), whole = _case(91, n, d, nlist, nq, metric)
+    grown = Store(capi.KIND_RABITQ, metric, d, rot=rot, centroid=cen)
+    grown.set_lists(codes[:1], labels[:1], nlist)
+    L = lib.load_library()
+    at = 1
+    for step in (63, 1, 500, 7000, 64, 9000, n):
+        end = min(n, at + step)
+        if end > at:
+            cbuf, lbuf = dev(np.ascontiguousarray(codes[at:end])), dev(np.ascontiguousarray(labels[at:end], np.int32))
+            capi.check(L.vsag_amd_store_append_lists(grown.handle, cbuf.ptr, lbuf.ptr, None, end - at, None))
+            cbuf.free()
+            lbuf.free()
+        at = end
+    buckets, _ = orc.ivf_route(cent, q, nprobe)
+    plain_w, fast_w = _both(lib, whole, q, buckets, kcand)
+    plain_g, fast_g = _both(lib, grown, q, buckets, kcand)
+    assert _same(plain_w, fast_w) and _same(plain_g, fast_g)
+    # the two stores hold the same codes under the same ids (lists in another order of arrival: ties aside, the same answers)
+    assert np.array_equal(fast_w[1].view(np.uint32), fast_g[1].view(np.uint32))
+    whole.destroy()
+    grown.destroy()
