@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import oracle as orc
-from gpu_helpers import Store, assert_topk_close, gaussian_mixture
+from gpu_helpers import Store, assert_topk_close, dev, gaussian_mixture
 from vsag_amd import capi
 
 pytestmark = pytest.mark.gpu
@@ -96,4 +96,52 @@ def test_fp32_duplicates_and_ragged_lists(lib):
     buckets, _ = orc.ivf_route(cent, q, nprobe)
     plain, fast = _both(lib, st, q, buckets, kcand)
     assert _same(plain, fast)
+    st.destroy()
+
+
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP])
+@pytest.mark.parametrize("kind,n,d,nlist,nq,nprobe,kcand", [
+    ("fp32", 30000, 96, 40, 4500, 8, 10), ("fp32", 20000, 33, 16, 9000, 4, 32), ("fp32", 12000, 960, 16, 9000, 4, 10),
+    ("sq8", 20000, 64, 20, 7000, 6, 10), ("sq8", 20000, 200, 20, 7000, 6, 100)])
+def test_residual_lists_on_the_matrix_cores_equal_streaming(lib, metric, kind, n, d, nlist, nq, nprobe, kcand):
+    """use_residual (bucket_datacell.h:527-572,594-639): codes of x - c.  The slot's bias joins the code's term and the
+    pair's <q, c> the threshold of the fp32 matrix-core test, and the rescoring takes both off in the streaming kernel's
+    order, so ids and distance bits equal the streaming scan's; with fp32 codes the result is the plain scan of x again."""
+    L = lib.load_library()
+    rng = np.random.default_rng(n + d + metric)
+    x, means = gaussian_mixture(rng, n, d, 40, 0.05)
+    q, _ = gaussian_mixture(rng, nq, d, 40, 0.05, means=means)
+    x, q = (x - 0.3).astype(np.float32), (q - 0.3).astype(np.float32)
+    cent = x[rng.choice(n, nlist, replace=False)].copy()
+    labels, _, _ = orc.kmeans_assign(x, cent)
+    res = orc.residual_rows(x, labels, cent, metric)
+    if kind == "fp32":
+        codes, dec = res.view(np.uint8).reshape(n, 4 * d), res
+        st = Store(capi.KIND_FP32, metric, d)
+    else:
+        lb, diff = orc.sq_train(res, 8, metric)
+        codes = orc.sq_encode(res, 8, lb, diff, metric)
+        dec = orc.sq_decode(codes, d, 8, lb, diff)
+        st = Store(capi.KIND_SQ8, metric, d, lb=lb, diff=diff)
+    bias = orc.residual_bias(dec, labels, cent) if metric == orc.L2 else None
+    cb = dev(cent)
+    capi.check(L.vsag_amd_store_set_residual(st.handle, cb.ptr, nlist, None))
+    st.set_lists(codes[:0], labels[:0], nlist)
+    half = n // 3
+    st.append_lists(codes[:half], labels[:half], None if bias is None else bias[:half])
+    st.append_lists(codes[half:], labels[half:], None if bias is None else bias[half:])
+    buckets, _ = orc.ivf_route(cent, q, nprobe)
+    buckets = buckets.copy()
+    buckets[70:73, 0] = -1
+    buckets[80, 0] = buckets[80, nprobe - 1]
+    plain, fast = _both(lib, st, q, buckets, kcand)
+    assert _same(plain, fast)
+    if kind == "fp32":
+        direct = Store(capi.KIND_FP32, metric, d)
+        direct.set_lists(x.view(np.uint8).reshape(n, 4 * d), labels, nlist)
+        pi, pd = direct.ivf_scan(q[:256], buckets[:256], kcand)
+        assert_topk_close(fast[0][:256], fast[1][:256], pi, pd, rtol=2e-4, atol=5e-4 if d > 500 else 5e-5, tie_rtol=5e-4,
+                          label="residual fp32 lists against the plain scan")
+        direct.destroy()
+    cb.free()
     st.destroy()

@@ -74,9 +74,10 @@ bool ivf_f32_supports(const vsag_amd_store* s);
 uint32_t ivf_f32_pairs_per_item();
 int launch_ivf_f32(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, const uint32_t* pair_off,
                    const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound, uint32_t kcand, float* tau,
-                   uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st);
+                   uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, const float* res_term, hipStream_t st);
 int launch_ivf_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
-                       uint32_t per_pair, uint64_t* partial, uint32_t* partial_cnt, const uint32_t* bound, hipStream_t st);
+                       uint32_t per_pair, uint64_t* partial, uint32_t* partial_cnt, const uint32_t* bound,
+                       const float* res_term, hipStream_t st);
 int launch_ivf_i8(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
                   const uint32_t* pair_off, const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound,
                   int32_t* tq, uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, const int32_t* buckets,
@@ -1189,10 +1190,11 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
                     p.bits1 ? ivf_rb_chunk_tiles() : 32U, 4U);
             if (p.f32) {
                 VA_TRY(launch_ivf_f32(s, a, nq, nprobe, p0, b.pair_off, b.item_off, b.sorted_pair, b.bound, kcand,
-                                      reinterpret_cast<float*>(b.tq), b.partial, b.partial_cnt, b.gate, st));
+                                      reinterpret_cast<float*>(b.tq), b.partial, b.partial_cnt, b.gate, v.res_term, st));
                 VA_TRY(launch_ivf_clear_gated(b.gate, nq, nprobe, p0, b.partial_cnt, buckets_dev, b.gpairs,
                                               kGatedPairsCap, kcand, st));
-                VA_TRY(launch_ivf_rescore(s, a, nq, nprobe, p0, kcand, p.chunks_max, b.partial, b.partial_cnt, b.bound, st));
+                VA_TRY(launch_ivf_rescore(s, a, nq, nprobe, p0, kcand, p.chunks_max, b.partial, b.partial_cnt, b.bound,
+                                          v.res_term, st));
             } else if (p.pq) {
                 VA_TRY(launch_ivf_pq(s, a, nq, nprobe, p0, kcand, b.pair_off, b.item_off, b.sorted_pair, b.bound, b.tq,
                                      b.partial, b.partial_cnt, b.gate, buckets_dev, b.gpairs, kGatedPairsCap, st));
@@ -1201,14 +1203,16 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
                                      b.partial, b.partial_cnt, b.gate, st));
                 VA_TRY(launch_ivf_clear_gated(b.gate, nq, nprobe, p0, b.partial_cnt, buckets_dev, b.gpairs,
                                               kGatedPairsCap, kcand, st));
-                VA_TRY(launch_ivf_rescore(s, a, nq, nprobe, p0, kcand, p.chunks_max, b.partial, b.partial_cnt, b.bound, st));
+                VA_TRY(launch_ivf_rescore(s, a, nq, nprobe, p0, kcand, p.chunks_max, b.partial, b.partial_cnt, b.bound,
+                                          nullptr, st));
             } else if (p.planes) {
                 VA_TRY(launch_ivf_sq8_i8(s, reinterpret_cast<const float*>(a.qtab), a.qstride, a.qmeta, a.qmeta_stride, nq,
                                          nprobe, p0, b.pair_off, b.item_off, b.sorted_pair, b.bound, kcand, b.q8, b.q8_u,
                                          b.q8_tau, b.partial, b.partial_cnt, b.gate, st));
                 VA_TRY(launch_ivf_clear_gated(b.gate, nq, nprobe, p0, b.partial_cnt, buckets_dev, b.gpairs,
                                               kGatedPairsCap, kcand, st));
-                VA_TRY(launch_ivf_rescore(s, a, nq, nprobe, p0, kcand, p.chunks_max, b.partial, b.partial_cnt, b.bound, st));
+                VA_TRY(launch_ivf_rescore(s, a, nq, nprobe, p0, kcand, p.chunks_max, b.partial, b.partial_cnt, b.bound,
+                                          nullptr, st));
             } else {
                 VA_TRY(launch_ivf_i8(s, a, nq, nprobe, p0, kcand, b.pair_off, b.item_off, b.sorted_pair, b.bound, b.tq,
                                      b.partial, b.partial_cnt, b.gate, buckets_dev, b.gpairs, kGatedPairsCap, st));

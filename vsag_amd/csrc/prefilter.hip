@@ -349,7 +349,8 @@ code_term_kernel(const uint4* tiles, uint32_t G, const float* scale, uint64_t fi
 // result when B <a, y> + F |y|^2 <= bound - C + |B| * err, plus the rounding of these few terms themselves.
 __global__ void __launch_bounds__(64)
 prefilter_tau_kernel(const float* qtab, uint32_t qstride, uint32_t kdim, const float* qmeta, uint32_t qmeta_stride,
-                     int is_l2, const uint32_t* bound, const uint32_t* ymax_bits, uint64_t nq, float* tau) {
+                     int is_l2, const uint32_t* bound, const uint32_t* ymax_bits, uint64_t nq, float* tau,
+                     float* magnitude_out = nullptr) {
     uint64_t q = blockIdx.x;
     uint32_t lane = threadIdx.x;
     const float* row = qtab + q * qstride;
@@ -366,6 +367,9 @@ prefilter_tau_kernel(const float* qtab, uint32_t qstride, uint32_t kdim, const f
     uint32_t b = bound[q];
     if (b == 0xFFFFFFFFU) {
         tau[q] = 3.0e38F;  // no bound yet: everything is a candidate (and the query will overflow)
+        if (magnitude_out != nullptr) {
+            magnitude_out[q] = 0.0F;
+        }
         return;
     }
     float bd = ordered_to_float(b);
@@ -376,6 +380,9 @@ prefilter_tau_kernel(const float* qtab, uint32_t qstride, uint32_t kdim, const f
     float magnitude = fabsf(bd) + fabsf(cq) + (is_l2 ? ymax * ymax : 0.0F) + factor * sqrtf(a2) * ymax;
     float t = bd - cq + err + 1.0e-6F * magnitude;
     tau[q] = t < 3.0e38F ? t : 3.0e38F;
+    if (magnitude_out != nullptr) {
+        magnitude_out[q] = magnitude;  // residual lists add their own terms' share to the margin (ivf_f32_kernel)
+    }
 }
 
 struct RescoreArgs {
@@ -609,6 +616,10 @@ struct IvfRescoreArgs {
     uint32_t nprobe, p0, per_pair;
     const uint32_t* ids;
     const uint32_t* bound;
+    // Residual lists (ivf.hip, IvfArgs): the slot's bias and the pair's term come off the distance, in the streaming
+    // kernel's order.  res_term null: no residual.
+    const float* res_bias;
+    const float* res_term;
 };
 
 constexpr uint32_t kIvfRescoreGather = 1024;
@@ -671,6 +682,12 @@ ivf_rescore_kernel(ScanArgs a, IvfRescoreArgs r) {
             }
             float d[1];
             finish_distances<KIND, METRIC, 1>(a, qidx, slot, acc, d);
+            if (r.res_term != nullptr && have) {
+                // list g of the query belongs to its pair p0 + g / per_pair
+                const uint32_t gl = where[e0 + lane] / r.k;
+                const float bias = r.res_bias != nullptr ? r.res_bias[slot] : 0.0F;
+                d[0] = (d[0] - bias) - r.res_term[static_cast<uint64_t>(q) * r.nprobe + r.p0 + gl / r.per_pair];
+            }
             if (have) {
                 const uint32_t id = as_const(r.ids)[slot];
                 fkey[e0 + lane] =
@@ -717,7 +734,8 @@ ivf_rescore_capacity() {
 
 int
 launch_ivf_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t kcand,
-                   uint32_t per_pair, uint64_t* partial, uint32_t* partial_cnt, const uint32_t* bound, hipStream_t st) {
+                   uint32_t per_pair, uint64_t* partial, uint32_t* partial_cnt, const uint32_t* bound, const float* res_term,
+                   hipStream_t st) {
     if ((s->kind != VSAG_AMD_KIND_SQ8 && s->kind != VSAG_AMD_KIND_SQ4 && s->kind != VSAG_AMD_KIND_RABITQ &&
          s->kind != VSAG_AMD_KIND_FP32) ||
         kcand > kIvfRescoreGather || s->ids_dev == nullptr) {
@@ -733,6 +751,8 @@ launch_ivf_rescore(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint
     r.per_pair = per_pair;
     r.ids = s->ids_dev;
     r.bound = bound;
+    r.res_term = res_term;
+    r.res_bias = res_term != nullptr ? s->residual_bias_dev : nullptr;
     const dim3 grid(static_cast<uint32_t>(nq));
     if (s->kind == VSAG_AMD_KIND_FP32) {
         // (cosine stores hold normalised vectors and scan as inner product)
@@ -783,6 +803,15 @@ struct IvfF32Args {
     const float* term;              // per slot |y|^2
     float term_factor, dot_factor;  // as PrefilterArgs
     const float* tau;               // per query
+    // Residual lists: distance = (base - bias of the slot) - term of the pair, so the bias joins the code's term, the
+    // pair's term the threshold, and the margin grows by their rounding: res_margin x (the query's magnitudes +
+    // |term| + res_bias_max).  res_term null: no residual.
+    const float* res_bias;          // per slot, or null (inner product)
+    const float* res_term;          // per pair (query * nprobe + column)
+    const float* magnitude;         // per query, from prefilter_tau_kernel
+    const uint32_t* ymax_bits;      // the largest norm among the stored vectors
+    float res_cmax;                 // the largest norm among the lists' centroids
+    const uint32_t* ids;            // per slot; the padding behind a list's last code holds no id and never passes
     const uint32_t* list_tile;      // per list: first tile, end tile
     const uint32_t* pair_off;       // pairs of list b: sorted_pair[pair_off[b] .. pair_off[b + 1])
     const uint32_t* item_off;       // items of list b: item_off[b] .. item_off[b + 1]
@@ -864,6 +893,16 @@ ivf_f32_kernel(IvfF32Args p) {
         pair_n[j] = live[j] ? as_const(p.sorted_pair)[at] : 0U;
         query_n[j] = pair_n[j] / p.nprobe;
         tau_n[j] = live[j] ? p.tau[query_n[j]] : -__builtin_inff();
+        if (p.res_term != nullptr && live[j]) {
+            const float rt = p.res_term[pair_n[j]];
+            // |bias| = |2 <c, y> + |c|^2| (l2; inner product has none)
+            const float res_bias_max =
+                p.res_bias != nullptr ? (2.0F * __uint_as_float(*p.ymax_bits) + p.res_cmax) * p.res_cmax : 0.0F;
+            // five more roundings between this test and the streaming result (the slot's term less its bias, the
+            // threshold plus the pair's term, and the two subtractions of the streaming kernel): 2e-6 of the magnitudes
+            // is several times their sum
+            tau_n[j] = tau_n[j] + rt + 2.0e-6F * (p.magnitude[query_n[j]] + fabsf(rt) + res_bias_max);
+        }
     }
 
     const uint32_t crow = tid & 127;
@@ -950,8 +989,12 @@ ivf_f32_kernel(IvfF32Args p) {
         park_queries(stage[0].b);
         float my_term = 0.0F;
         if (tid < PM) {
-            const bool real = tile_begin + 2 * mt + (tid >> 6) < tile_end;
+            // (a padding slot is all zeros: under inner product, and with a residual bias, that is a good distance)
+            const bool real = tile_begin + 2 * mt + (tid >> 6) < tile_end && p.ids[slot0 + tid] != VSAG_AMD_INVALID_ID;
             my_term = real ? p.term_factor * p.term[slot0 + tid] : __builtin_inff();
+            if (real && p.res_bias != nullptr) {
+                my_term -= p.res_bias[slot0 + tid];
+            }
         }
         __syncthreads();
         for (uint32_t kt = 0; kt < ktiles; ++kt) {
@@ -1028,7 +1071,8 @@ ivf_f32_kernel(IvfF32Args p) {
 bool
 ivf_f32_supports(const vsag_amd_store* s) {
     return (s->kind == VSAG_AMD_KIND_FP32 || s->kind == VSAG_AMD_KIND_SQ8) && s->nlist > 0 && s->pf_term != nullptr &&
-           s->pf_ymax != nullptr && s->residual_centroids_dev == nullptr && s->ids_dev != nullptr;
+           s->pf_ymax != nullptr && s->ids_dev != nullptr &&
+           (s->residual_centroids_dev == nullptr || s->metric != VSAG_AMD_METRIC_COSINE);
 }
 
 uint32_t
@@ -1042,12 +1086,13 @@ ivf_f32_pairs_per_item() {
 int
 launch_ivf_f32(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, const uint32_t* pair_off,
                const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound, uint32_t kcand, float* tau,
-               uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st) {
+               uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, const float* res_term, hipStream_t st) {
     const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
     const bool sq8 = s->kind == VSAG_AMD_KIND_SQ8;
+    // tau: nq thresholds, then (residual lists) nq magnitudes behind a spare word
     hipLaunchKernelGGL(prefilter_tau_kernel, dim3(static_cast<uint32_t>(nq)), dim3(kWave), 0, st,
                        reinterpret_cast<const float*>(a.qtab), a.qstride, s->dpad, sq8 && !l2 ? a.qmeta : nullptr,
-                       a.qmeta_stride, l2 ? 1 : 0, bound, s->pf_ymax, nq, tau);
+                       a.qmeta_stride, l2 ? 1 : 0, bound, s->pf_ymax, nq, tau, res_term != nullptr ? tau + nq + 1 : nullptr);
     IvfF32Args p{};
     p.tiles = s->tiles;
     p.G = s->G;
@@ -1059,6 +1104,14 @@ launch_ivf_f32(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t
     p.term_factor = l2 ? 1.0F : 0.0F;
     p.dot_factor = l2 ? -2.0F : -1.0F;
     p.tau = tau;
+    if (res_term != nullptr) {
+        p.res_term = res_term;
+        p.res_bias = s->residual_bias_dev;
+        p.magnitude = tau + nq + 1;
+        p.ymax_bits = s->pf_ymax;
+        p.res_cmax = s->residual_cmax;
+    }
+    p.ids = s->ids_dev;
     p.list_tile = s->list_tile_dev;
     p.pair_off = pair_off;
     p.item_off = item_off;

@@ -80,6 +80,7 @@ struct vsag_amd_store {
     // (l2 only, else null) and the centroids the codes are residuals of.
     float* residual_bias_dev = nullptr;
     float* residual_centroids_dev = nullptr;  // nlist x dim, null: no residual
+    float residual_cmax = 0.0F;               // the largest norm among those centroids (rounded up)
 
     // flat fp32 / sq8 stores: per slot |y|^2 and the largest |y| (float bits) of the code as the batched
     // contraction sees it, kept up to date by append

@@ -1008,7 +1008,12 @@ append_to_lists(vsag_amd_store* s, const uint8_t* codes_dev, const int32_t* labe
     // sq8 codes) against the classification and encoding an append has behind it already.
     const bool list_terms = s->kind == VSAG_AMD_KIND_FP32 || s->kind == VSAG_AMD_KIND_SQ8 ||
                             (s->kind == VSAG_AMD_KIND_SQ4 && s->dpad <= 128);
-    if (list_terms && s->pf_ymax != nullptr && s->residual_centroids_dev == nullptr) {
+    // (Residual lists: fp32 and sq8 under l2 / inner product go through the fp32 matrix cores, the int8 passes do not take
+    // them.)
+    const bool residual_ok = s->residual_centroids_dev == nullptr ||
+                             ((s->kind == VSAG_AMD_KIND_FP32 || s->kind == VSAG_AMD_KIND_SQ8) &&
+                              s->metric != VSAG_AMD_METRIC_COSINE);
+    if (list_terms && s->pf_ymax != nullptr && residual_ok) {
         const uint64_t slots = s->cap_tiles * kWave;
         if (s->pf_term == nullptr || s->pf_term_slots < slots) {
             if (s->pf_term != nullptr) {
@@ -1097,7 +1102,21 @@ vsag_amd_store_set_residual(vsag_amd_store_t* s, const float* centroids_dev, uin
     VA_HIP(hipMalloc(&s->residual_centroids_dev, bytes));
     VA_HIP(hipMemcpyAsync(s->residual_centroids_dev, centroids_dev, bytes, hipMemcpyDeviceToDevice,
                           static_cast<hipStream_t>(stream)));
+    // The largest centroid norm bounds the per-slot bias of the residual arithmetic (2 |c| |y| + |c|^2), which the
+    // matrix-core pass over residual lists needs for its error margin.
+    std::vector<float> host(static_cast<size_t>(nlist) * s->dim);
+    VA_HIP(hipMemcpyAsync(host.data(), centroids_dev, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
     VA_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    double cmax = 0.0;
+    for (uint32_t l = 0; l < nlist; ++l) {
+        double sq = 0.0;
+        for (uint32_t d = 0; d < s->dim; ++d) {
+            const double v = host[static_cast<size_t>(l) * s->dim + d];
+            sq += v * v;
+        }
+        cmax = std::max(cmax, std::sqrt(sq));
+    }
+    s->residual_cmax = std::isfinite(cmax) ? static_cast<float>(cmax * (1.0 + 1.0e-6)) : std::numeric_limits<float>::infinity();
     return 0;
 }
 
