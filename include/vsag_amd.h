@@ -144,6 +144,10 @@ VSAG_AMD_API int vsag_amd_rabitq_train(const float* x_dev, uint64_t n, uint32_t 
 VSAG_AMD_API int vsag_amd_rabitq_encode(const float* x_dev, uint64_t n, uint32_t dim, const float* rotation_dev,
                            const float* centroid_dev, int metric, int query_bits, uint8_t* codes_dev,
                            void* stream);
+/* RaBitQuantizer::DecodeOneImpl (rabitq_quantizer.cpp:871-899): n x dim floats, x = R^T ((+-1 / sqrt(dim)) norm + centroid).
+ * 1-bit codes only (the reference returns false for the others: INVALID_ARGUMENT here).  bits_word as for the encoders. */
+VSAG_AMD_API int vsag_amd_rabitq_decode(const uint8_t* codes_dev, uint64_t n, uint32_t dim, const float* rotation_dev,
+                           const float* centroid_dev, int metric, int bits_word, float* out_dev, void* stream);
 /* RaBitQuantizer::EncodeOneInternal, multi-bit base (rabitq_quantizer.cpp:774-809; bits_word =
  * VSAG_AMD_RABITQ_BITS(32, 2..8)): n x code_size codes [bit planes, plane b = bit b of every dimension (PackIntoPlanes,
  * :431-453) | norm of the centred code | norm | error | raw norm (ip, cosine)].  fast_encode chooses FastEncodeRaBitQ

@@ -33,6 +33,10 @@
 //                                          answers of the reference's walk, which is not optimal); zero vectors;
 //                                          the estimator's closed form (ip_obar_q) and a stored vector's self
 //                                          distance
+//   rabitq decode (residual lists) ....... the scale step against the reference's compiled
+//                                          InverseNormalizeWithCentroid; the whole against what the definition
+//                                          fixes: R x - centroid has the code's signs and one magnitude, norm / sqrt(d),
+//                                          and a row built to sit exactly on such a point decodes to itself
 //   parity unpinned ...................... nothing; what the formulas leave open is the order of fp32
 //                                          operations inside rabitq_dist and the k-means loss (no
 //                                          executable reference class), which the 1e-4 relative
@@ -1371,6 +1375,45 @@ orc_rabitq_encode(const float* data, uint64_t n, uint64_t dim, const float* rot,
             }
         }
     }
+}
+
+// RaBitQuantizer::DecodeOneImpl (rabitq_quantizer.cpp:871-899), which use_residual needs for the l2 bias of a code
+// (bucket_datacell.h:645-650): 1-bit codes only (other widths return false and write nothing: 0 here, rows left as
+// they are).  The sign vector over sqrt(d), InverseNormalizeWithCentroid (simd/kernels/normalize.h:88-119:
+// from * norm + centroid per element), then x = R^T y (RandomOrthogonalMatrix::InverseTransform,
+// random_orthogonal_transformer.cpp:80-94: a row-major sgemv with Trans; summed over the rows in order here, BLAS
+// leaves the order open).
+ORC_API int
+orc_rabitq_decode(const uint8_t* codes, uint64_t n, uint64_t dim, const float* rot, const float* centroid, int metric,
+                  int query_bits, float* out) {
+    RabitqLayout l = rabitq_layout(dim, metric, query_bits);
+    if (l.base_bits != 1) {
+        return 0;
+    }
+    const float inv_sqrt_d = 1.0F / std::sqrt(static_cast<float>(dim));
+#pragma omp parallel
+    {
+        std::vector<float> y(dim);
+#pragma omp for schedule(static)
+        for (int64_t i = 0; i < static_cast<int64_t>(n); ++i) {
+            const uint8_t* c = codes + i * l.code_size;
+            const float norm = rd_f32(c + l.offset_norm);
+            for (uint64_t d = 0; d < dim; ++d) {
+                const bool bit = ((c[d / 8] >> (d % 8)) & 1) != 0;
+                const float from = bit ? inv_sqrt_d : -inv_sqrt_d;
+                y[d] = from * norm + centroid[d];
+            }
+            float* x = out + i * dim;
+            for (uint64_t j = 0; j < dim; ++j) {
+                float acc = 0.0F;
+                for (uint64_t r = 0; r < dim; ++r) {
+                    acc += rot[r * dim + j] * y[r];
+                }
+                x[j] = acc;
+            }
+        }
+    }
+    return 1;
 }
 
 // RaBitQuantizer::EncodeOneInternal, multi-bit branch (rabitq_quantizer.cpp:774-809): the scalar code of the rotated,

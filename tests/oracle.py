@@ -133,6 +133,15 @@ def rabitq_encode(x, rot, centroid, metric, qbits=4):
     return codes
 
 
+def rabitq_decode(codes, d, rot, centroid, metric, qbits=4):
+    """RaBitQuantizer::DecodeOneImpl; None where the reference returns false (multi-bit codes)."""
+    codes = np.ascontiguousarray(codes, np.uint8)
+    out = np.zeros((codes.shape[0], d), np.float32)
+    ok = lib().orc_rabitq_decode(_p(codes), u64(codes.shape[0]), u64(d), _p(f32(rot)), _p(f32(centroid)), metric, qbits,
+                                 _p(out))
+    return out if ok else None
+
+
 def rabitq_bits(qbits, base_bits=1):
     """The `qbits` argument of every rabitq function here: query bits (4 | 32) plus 256 * base bits for multi-bit base
     codes (rabitq_bits_per_dim_base 2..8, fp32 queries only)."""
@@ -481,6 +490,7 @@ _REF_SYMBOLS = {
     "RaBitQFloatSQIP": "_ZN4vsag7generic15RaBitQFloatSQIPEPKfPKhm",
     "RaBitQFloatSplitCodeIP": "_ZN4vsag7generic22RaBitQFloatSplitCodeIPEPKfPKhS4_mj",
     "NormalizeWithCentroid": "_ZN4vsag7generic21NormalizeWithCentroidEPKfS2_Pfm",
+    "InverseNormalizeWithCentroid": "_ZN4vsag7generic28InverseNormalizeWithCentroidEPKfS2_Pfmf",
     "Normalize": "_ZN4vsag7generic9NormalizeEPKfPfm",
 }
 

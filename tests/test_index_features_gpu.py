@@ -109,7 +109,8 @@ def test_ivf_buckets_per_data(lib):
 # quantizer trained on the residuals, which clips it (bucket_datacell.h:575-591 hands the raw query to SetQuery).
 @pytest.mark.parametrize("metric,quant,improves", [("l2", "fp32", False), ("ip", "fp32", False), ("l2", "sq8", True),
                                                    ("ip", "sq8", True), ("l2", "sq4", True), ("cosine", "sq8", False),
-                                                   ("l2", "sq8_uniform", False)])
+                                                   ("l2", "sq8_uniform", False), ("l2", "rabitq", False),
+                                                   ("ip", "rabitq", False)])
 def test_ivf_use_residual(lib, metric, quant, improves):
     n, d, nq, k, nlist = 4000, 32, 50, 10, 32
     # fewer clusters than lists, so that k-means splits clusters rather than merging them

@@ -353,3 +353,50 @@ def test_a_list_probed_twice_brings_every_key_twice(lib, nq, kcand):
     if kcand % 2:
         assert np.array_equal(ids[:, -1], once[:, half])
     st.destroy()
+
+
+@pytest.mark.parametrize("metric,mname", [(orc.L2, "l2"), (orc.IP, "ip")])
+@pytest.mark.parametrize("qbits", [4, 32])
+def test_residual_rabitq_lists_match_oracle(lib, metric, mname, qbits):
+    """use_residual with rabitq lists (bucket_datacell.h:594-650): the quantizer is trained on and encodes x - c; under
+    l2 the bias of a code comes from RaBitQuantizer::DecodeOneImpl (rabitq_quantizer.cpp:871-899), the sign point
+    rotated back.  The decoder and the bias against the checker's, then the scan against its restatement."""
+    L = lib.load_library()
+    rng = np.random.default_rng(97 + metric + qbits)
+    n, d, nlist, nq, nprobe, kcand = 5000, 72, 23, 17, 6, 30
+    x, q, cent, labels = _ivf_case(rng, n, d, nlist, nq)
+    x = (x - 0.3).astype(np.float32)
+    q = (q - 0.3).astype(np.float32)
+    res = orc.residual_rows(x, labels, cent, metric)
+    g = rng.standard_normal((d, d))
+    rot, r = np.linalg.qr(g)
+    rot = (rot * np.sign(np.diag(r))).astype(np.float32)
+    cen = orc.rabitq_train(res, rot)
+    codes = orc.rabitq_encode(res, rot, cen, metric, qbits)
+    dec = orc.rabitq_decode(codes, d, rot, cen, metric, qbits)
+    st = Store(capi.KIND_RABITQ, metric, d, rot=rot, centroid=cen, qbits=qbits)
+    cdev, rdev, cendev, out = dev(codes), dev(rot), dev(cen), capi.DeviceBuffer(n * d * 4)
+    capi.check(L.vsag_amd_rabitq_decode(cdev.ptr, n, d, rdev.ptr, cendev.ptr, metric, qbits, out.ptr, None))
+    np.testing.assert_allclose(out.to_numpy(np.float32, (n, d)), dec, rtol=0, atol=2e-6 * (1 + np.abs(dec).max()))
+    cb, lb_dev = dev(cent), dev(labels.astype(np.int32))
+    capi.check(L.vsag_amd_store_set_residual(st.handle, cb.ptr, nlist, None))
+    st.set_lists(codes[:0], labels[:0], nlist)
+    bias = None
+    if metric == orc.L2:
+        bias = orc.residual_bias(dec, labels, cent)
+        bdev = capi.DeviceBuffer(n * 4)
+        capi.check(L.vsag_amd_residual_bias(st.handle, cdev.ptr, n, lb_dev.ptr, cb.ptr, bdev.ptr, out.ptr, None))
+        np.testing.assert_allclose(bdev.to_numpy(np.float32, (n,)), bias, rtol=1e-5, atol=1e-5)
+        bdev.free()
+    _append_lists(lib, st, codes[:2000], labels[:2000], None if bias is None else bias[:2000])
+    _append_lists(lib, st, codes[2000:], labels[2000:], None if bias is None else bias[2000:])
+    offsets, order = orc.ivf_build_lists(labels, nlist)
+    routed, _ = orc.ivf_route(cent, q, nprobe)
+    ids, ds = st.ivf_scan(q, routed, kcand)
+    qproc = orc.rabitq_process_query(q, rot, cen, metric, qbits)
+    rids, rds = orc.ivf_scan_residual(orc.RABITQ, metric, d, codes[order], offsets, order, qproc, q, cent,
+                                      None if bias is None else bias[order], routed, kcand, qbits=qbits)
+    assert_topk_close(ids, ds, rids, rds, rtol=2e-4, atol=5e-5, tie_rtol=2e-4, label="residual rabitq %s" % mname)
+    for b in (cdev, rdev, cendev, out, cb, lb_dev):
+        b.free()
+    st.destroy()

@@ -390,6 +390,55 @@ def test_rabitq_encode_invariants_and_estimator():
     assert np.corrcoef(d4.ravel(), true.ravel())[0, 1] > 0.7
 
 
+@pytest.mark.parametrize("d", [8, 33, 128, 200])
+def test_rabitq_decode_is_the_sign_point_rotated_back(d):
+    """RaBitQuantizer::DecodeOneImpl (rabitq_quantizer.cpp:871-899), which the l2 bias of residual lists is computed
+    from.  (1) The scale step equals the reference's compiled InverseNormalizeWithCentroid on the identity rotation.
+    (2) What the definition fixes for any rotation: R x' - centroid has the code's signs and the single magnitude
+    norm / sqrt(d).  (3) A row built to sit exactly on such a point encodes to those signs and decodes to itself.
+    (4) Multi-bit codes: the reference returns false."""
+    rng = np.random.default_rng(90 + d)
+    rot = _rotation(rng, d)
+    n = 40
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    cen = orc.rabitq_train(x, rot)
+    for metric in (orc.L2, orc.IP):
+        codes = orc.rabitq_encode(x, rot, cen, metric)
+        dec = orc.rabitq_decode(codes, d, rot, cen, metric)
+        nb = (d + 7) // 8
+        bits = np.unpackbits(codes[:, :nb], axis=1, bitorder="little")[:, :d].astype(np.float64)
+        norms = np.ascontiguousarray(codes[:, -(16 if metric == orc.IP else 12):][:, :4]).view(np.float32)[:, 0].astype(np.float64)
+        back = dec.astype(np.float64) @ rot.astype(np.float64).T - cen.astype(np.float64)
+        want = (2.0 * bits - 1.0) * norms[:, None] / np.sqrt(d)
+        np.testing.assert_allclose(back, want, rtol=0, atol=2e-5 * (1.0 + np.abs(want).max() + np.abs(cen).max()))
+        # the stored norm is |R x - centroid|: the decoded point lies at that distance from the centroid as well
+        np.testing.assert_allclose(np.linalg.norm(back, axis=1), norms, rtol=1e-5)
+    ref = orc.ref()
+    if ref is not None:
+        eye = np.eye(d, dtype=np.float32)
+        codes = orc.rabitq_encode(x, eye, cen, orc.L2)
+        dec = orc.rabitq_decode(codes, d, eye, cen, orc.L2)
+        inv = np.float32(1.0) / np.sqrt(np.float32(d))
+        for i in range(n):
+            signs = np.where(np.unpackbits(codes[i, :(d + 7) // 8], bitorder="little")[:d] != 0, inv, -inv).astype(np.float32)
+            norm = np.ascontiguousarray(codes[i, -12:-8]).view(np.float32)[0]
+            out = np.empty(d, np.float32)
+            ref["InverseNormalizeWithCentroid"].restype = None
+            ref["InverseNormalizeWithCentroid"](_p(signs), _p(cen), _p(out), C.c_uint64(d), C.c_float(norm))
+            # (a fused and an unfused multiply-add differ by an ulp of the result)
+            np.testing.assert_allclose(dec[i], out, rtol=3e-7, atol=1e-7)
+    # (3) a fixed point: x = R^T (centroid + r s / sqrt(d)) for a sign vector s
+    s = np.where(rng.random((n, d)) < 0.5, -1.0, 1.0)
+    r = rng.uniform(0.5, 2.0, n)
+    pts = ((cen.astype(np.float64) + s * r[:, None] / np.sqrt(d)) @ rot.astype(np.float64)).astype(np.float32)
+    codes = orc.rabitq_encode(pts, rot, cen, orc.L2)
+    got_bits = np.unpackbits(codes[:, :(d + 7) // 8], axis=1, bitorder="little")[:, :d]
+    assert np.array_equal(got_bits, (s > 0).astype(np.uint8))
+    np.testing.assert_allclose(orc.rabitq_decode(codes, d, rot, cen, orc.L2), pts, rtol=0, atol=1e-5 * (1 + np.abs(pts).max()))
+    x4 = orc.rabitq_encode_multibit(x, rot, cen, orc.L2, 4)
+    assert orc.rabitq_decode(x4, d, rot, cen, orc.L2, qbits=orc.rabitq_bits(32, 4)) is None
+
+
 def _rabitq_dist(qcode, code, d, metric, qbits):
     L = orc.lib()
     return float(L.orc_rabitq_dist(_p(np.ascontiguousarray(qcode)), _p(np.ascontiguousarray(code)), C.c_uint64(d), metric,

@@ -164,6 +164,7 @@ IVF_CASES = [
     ({"base_quantization_type": "pqfs", "base_pq_dim": 16, "use_reorder": True, "precise_quantization_type": "fp32"},
      "l2", 5.0),
     ({"base_quantization_type": "pqfs", "base_pq_dim": 32, "use_residual": True}, "cosine", None),
+    ({"base_quantization_type": "rabitq", "use_residual": True}, "l2", None),
 ]
 
 

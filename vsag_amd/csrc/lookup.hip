@@ -382,9 +382,17 @@ vsag_amd_residual_bias(const vsag_amd_store_t* s, const uint8_t* codes_dev, uint
         return 0;
     }
     VA_CHECK_ARG(s && codes_dev && labels_dev && centroids_dev && bias_dev && decoded_dev, "null pointer");
-    VA_CHECK_ARG(s->kind != VSAG_AMD_KIND_RABITQ, "residual codes of a rabitq store are not supported");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (s->kind == VSAG_AMD_KIND_PQFS) {
+    if (s->kind == VSAG_AMD_KIND_RABITQ) {
+        if (s->base_bits == 1) {
+            VA_TRY(vsag_amd_rabitq_decode(codes_dev, n, s->dim, s->rotation_dev, s->centroid_dev, s->metric,
+                                          rabitq_bits_word(s), decoded_dev, stream));
+        } else {
+            // RaBitQuantizer::DecodeOneImpl returns false for multi-bit codes and writes nothing: encode_vector
+            // (bucket_datacell.h:645-650) then takes the products with its zero-initialised buffer.
+            VA_HIP(hipMemsetAsync(decoded_dev, 0, n * s->dim * sizeof(float), st));
+        }
+    } else if (s->kind == VSAG_AMD_KIND_PQFS) {
         VA_TRY(vsag_amd_pq_decode(codes_dev, n, s->dim, s->pq_dim, s->codebooks_dev, decoded_dev, stream));
     } else {
         hipLaunchKernelGGL(decode_kernel, dim3(static_cast<uint32_t>(div_up(n * s->dim, 256))), dim3(256), 0, st, s->kind,

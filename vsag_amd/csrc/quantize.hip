@@ -283,6 +283,15 @@ rabitq_query_code_size(uint32_t dim, int metric, int query_bits) {
     return rabitq_layout(dim, metric, query_bits).query_code_size;
 }
 
+__device__ inline float
+load_f32(const uint8_t* p) {
+    uint32_t u = 0;
+    for (int b = 0; b < 4; ++b) {
+        u |= static_cast<uint32_t>(p[b]) << (8 * b);
+    }
+    return __uint_as_float(u);
+}
+
 __device__ inline void
 store_f32(uint8_t* p, float v) {
     uint32_t u = __float_as_uint(v);
@@ -1285,6 +1294,47 @@ vsag_amd_rabitq_encode(const float* x_dev, uint64_t n, uint32_t dim, const float
         VA_HIP(hipGetLastError());
         return 0;
     });
+}
+
+// RaBitQuantizer::DecodeOneImpl (rabitq_quantizer.cpp:871-899), 1-bit codes: y = (+-1 / sqrt(d)) * norm + centroid
+// per dimension (InverseNormalizeWithCentroid, simd/kernels/normalize.h:88-119), x = R^T y.  A workgroup per code, a
+// thread per output dimension, the rows of R summed in order.
+__global__ void __launch_bounds__(256)
+rabitq_decode_kernel(const uint8_t* codes, uint32_t dim, const float* rot, const float* centroid, uint32_t code_size,
+                     uint32_t offset_norm, float* out) {
+    const uint64_t i = blockIdx.x;
+    const uint8_t* c = codes + i * code_size;
+    const float norm = load_f32(c + offset_norm);
+    const float inv_sqrt_d = 1.0F / sqrtf(static_cast<float>(dim));
+    for (uint32_t j = threadIdx.x; j < dim; j += blockDim.x) {
+        float acc = 0.0F;
+        for (uint32_t r = 0; r < dim; ++r) {
+            const bool bit = ((c[r >> 3] >> (r & 7)) & 1) != 0;
+            const float y = (bit ? inv_sqrt_d : -inv_sqrt_d) * norm + centroid[r];
+            acc += rot[static_cast<uint64_t>(r) * dim + j] * y;
+        }
+        out[i * dim + j] = acc;
+    }
+}
+
+extern "C" int
+vsag_amd_rabitq_decode(const uint8_t* codes_dev, uint64_t n, uint32_t dim, const float* rotation_dev,
+                       const float* centroid_dev, int metric, int bits_word, float* out_dev, void* stream) {
+    VA_TRY(ensure_init());
+    const int query_bits = bits_word & 255;
+    VA_CHECK_ARG(query_bits == 4 || query_bits == 32, "query_bits must be 4 or 32, got %d", query_bits);
+    VA_CHECK_ARG((bits_word >> 8) <= 1, "only 1-bit codes decode (RaBitQuantizer::DecodeOneImpl returns false for the others)");
+    VA_CHECK_ARG(dim >= 1 && dim <= 65536, "dim must be in [1, 65536], got %u", dim);
+    if (n == 0) {
+        return 0;
+    }
+    VA_CHECK_ARG(codes_dev && rotation_dev && centroid_dev && out_dev, "null pointer");
+    VA_CHECK_ARG(n < (1ull << 31), "n must be below 2^31");
+    const RabitqLayout l = rabitq_layout(dim, metric, query_bits);
+    hipLaunchKernelGGL(rabitq_decode_kernel, dim3(static_cast<uint32_t>(n)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       codes_dev, dim, rotation_dev, centroid_dev, l.code_size, l.offset_norm, out_dev);
+    VA_HIP(hipGetLastError());
+    return 0;
 }
 
 extern "C" int

@@ -1092,7 +1092,6 @@ vsag_amd_store_set_residual(vsag_amd_store_t* s, const float* centroids_dev, uin
     VA_TRY(ensure_init());
     VA_CHECK_ARG(s != nullptr && centroids_dev != nullptr, "null store / centroids");
     VA_CHECK_ARG(s->n == 0, "the residual centroids are set before the first code is stored");
-    VA_CHECK_ARG(s->kind != VSAG_AMD_KIND_RABITQ, "residual codes of a rabitq store are not supported");
     VA_CHECK_ARG(nlist >= 1 && (s->nlist == 0 || s->nlist == nlist), "nlist does not match the store's lists");
     if (s->residual_centroids_dev != nullptr) {
         VA_HIP(hipFree(s->residual_centroids_dev));

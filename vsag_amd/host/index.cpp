@@ -2251,9 +2251,6 @@ public:
         if (index_param.Contains("use_residual")) {
             use_residual_ = index_param["use_residual"].GetBool();
         }
-        if (use_residual_) {
-            CHECK_ARGUMENT(q_.kind != VSAG_AMD_KIND_RABITQ, "the GPU path does not support use_residual with rabitq");
-        }
         if (index_param.Contains("partition_strategy_type")) {
             CHECK_ARGUMENT(index_param["partition_strategy_type"].GetString() == "ivf",
                            "the GPU path supports the nearest-centroid partition strategy only");
