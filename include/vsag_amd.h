@@ -144,6 +144,10 @@ VSAG_AMD_API int vsag_amd_rabitq_train(const float* x_dev, uint64_t n, uint32_t 
 VSAG_AMD_API int vsag_amd_rabitq_encode(const float* x_dev, uint64_t n, uint32_t dim, const float* rotation_dev,
                            const float* centroid_dev, int metric, int query_bits, uint8_t* codes_dev,
                            void* stream);
+/* FhtKacRotator::Transform (src/impl/transform/fht_kac_rotate_transformer.cpp:64-96; `rabitq_use_fht`) as the dense
+ * row-major rotation the rabitq entry points take: y = R x.  flip_host: 4 x ceil(dim / 8) bytes of sign bits (what
+ * FhtKacRotator::Serialize writes); rotation_host: dim x dim floats.  Host memory on both sides, no device work. */
+VSAG_AMD_API int vsag_amd_fht_kac_matrix(const uint8_t* flip_host, uint32_t dim, float* rotation_host);
 /* RaBitQuantizer::DecodeOneImpl (rabitq_quantizer.cpp:871-899): n x dim floats, x = R^T ((+-1 / sqrt(dim)) norm + centroid).
  * 1-bit codes only (the reference returns false for the others: INVALID_ARGUMENT here).  bits_word as for the encoders. */
 VSAG_AMD_API int vsag_amd_rabitq_decode(const uint8_t* codes_dev, uint64_t n, uint32_t dim, const float* rotation_dev,

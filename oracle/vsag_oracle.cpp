@@ -37,6 +37,10 @@
 //                                          InverseNormalizeWithCentroid; the whole against what the definition
 //                                          fixes: R x - centroid has the code's signs and one magnitude, norm / sqrt(d),
 //                                          and a row built to sit exactly on such a point decodes to itself
+//   FhtKacRotator (rabitq_use_fht) ....... the four primitives against the reference's compiled FlipSign, VecRescale,
+//                                          FHTRotate and KacsWalk; the transform by the reference test's own
+//                                          properties (lengths kept, the inverse returns the input within 1e-4) and
+//                                          the closed form without flips on a power of two ((H / sqrt(d))^4 = I)
 //   parity unpinned ...................... nothing; what the formulas leave open is the order of fp32
 //                                          operations inside rabitq_dist and the k-means loss (no
 //                                          executable reference class), which the 1e-4 relative
@@ -1374,6 +1378,114 @@ orc_rabitq_encode(const float* data, uint64_t n, uint64_t dim, const float* rot,
                 wr_f32(c + l.offset_raw_norm, raw_norm);
             }
         }
+    }
+}
+
+// ---- FhtKacRotator (rabitq_use_fht) -----------------------------------------------------------------------
+// The primitives of simd/generic.cpp:953-985 (FlipSign, VecRescale, FHTRotate over RotateOp of
+// simd/kernels/butterfly.h:36-55, KacsWalk of butterfly.h:61-94).
+static void
+fht_flip_sign(const uint8_t* flip, float* data, uint64_t dim) {
+    for (uint64_t i = 0; i < dim; ++i) {
+        if ((flip[i / 8] & (1 << (i % 8))) != 0) {
+            data[i] = -data[i];
+        }
+    }
+}
+static void
+fht_rescale(float* data, uint64_t dim, float val) {
+    for (uint64_t i = 0; i < dim; ++i) {
+        data[i] *= val;
+    }
+}
+static void
+fht_rotate(float* data, uint64_t n) {
+    for (uint64_t step = 1; step < n; step *= 2) {
+        for (uint64_t i = 0; i < n; i += step * 2) {
+            for (uint64_t j = 0; j < step; ++j) {
+                const float g1 = data[i + j], g2 = data[i + j + step];
+                data[i + j] = g1 + g2;
+                data[i + j + step] = g1 - g2;
+            }
+        }
+    }
+}
+static void
+fht_kacs_walk(float* data, uint64_t len) {
+    const uint64_t base = len % 2, offset = base + len / 2;
+    for (uint64_t i = 0; i < len / 2; ++i) {
+        const float x = data[i], y = data[i + offset];
+        data[i] = x + y;
+        data[i + offset] = x - y;
+    }
+    if (base != 0) {
+        data[len / 2] *= std::sqrt(2.0F);
+    }
+}
+ORC_API void
+orc_fht_primitive(int which, const uint8_t* flip, float* data, uint64_t dim, float val) {
+    switch (which) {
+        case 0: fht_flip_sign(flip, data, dim); break;
+        case 1: fht_rescale(data, dim, val); break;
+        case 2: fht_rotate(data, dim); break;
+        default: fht_kacs_walk(data, dim); break;
+    }
+}
+
+// FhtKacRotator::Transform / InverseTransform (impl/transform/fht_kac_rotate_transformer.cpp:64-120): four rounds
+// (ROUND, fht_kac_rotate_transformer.h:53) of sign flips (flip: 4 x ceil(dim / 8) bytes), a Hadamard transform of the
+// leading power-of-two block and a rescale; other dimensions alternate the leading and the trailing block with a
+// Kac walk in between and close with a factor 1/4.
+ORC_API void
+orc_fht_kac_transform(const uint8_t* flip, uint64_t dim, int inverse, const float* in, float* out) {
+    const uint64_t flip_offset = (dim + 7) / 8;
+    uint64_t trunc = 1;
+    while (trunc * 2 <= dim) {
+        trunc *= 2;
+    }
+    const float fac = 1.0F / std::sqrt(static_cast<float>(trunc));
+    std::memcpy(out, in, dim * sizeof(float));
+    const uint64_t start = dim - trunc;
+    if (!inverse) {
+        if (trunc == dim) {
+            for (int t = 0; t < 4; ++t) {
+                fht_flip_sign(flip + t * flip_offset, out, dim);
+                fht_rotate(out, trunc);
+                fht_rescale(out, trunc, fac);
+            }
+            return;
+        }
+        for (int t = 0; t < 4; t += 2) {
+            fht_flip_sign(flip + t * flip_offset, out, dim);
+            fht_rotate(out, trunc);
+            fht_rescale(out, trunc, fac);
+            fht_kacs_walk(out, dim);
+            fht_flip_sign(flip + (t + 1) * flip_offset, out, dim);
+            fht_rotate(out + start, trunc);
+            fht_rescale(out + start, trunc, fac);
+            fht_kacs_walk(out, dim);
+        }
+        fht_rescale(out, dim, 0.25F);
+        return;
+    }
+    if (trunc == dim) {
+        for (int t = 3; t >= 0; --t) {
+            fht_rotate(out, trunc);
+            fht_rescale(out, trunc, fac);
+            fht_flip_sign(flip + t * flip_offset, out, dim);
+        }
+        return;
+    }
+    fht_rescale(out, dim, 0.25F);
+    for (int t = 3; t > 0; t -= 2) {
+        fht_kacs_walk(out, dim);
+        fht_rotate(out + start, trunc);
+        fht_rescale(out + start, trunc, fac);
+        fht_flip_sign(flip + t * flip_offset, out, dim);
+        fht_kacs_walk(out, dim);
+        fht_rotate(out, trunc);
+        fht_rescale(out, trunc, fac);
+        fht_flip_sign(flip + (t - 1) * flip_offset, out, dim);
     }
 }
 

@@ -142,6 +142,24 @@ def rabitq_decode(codes, d, rot, centroid, metric, qbits=4):
     return out if ok else None
 
 
+def fht_primitive(which, data, flip=None, val=0.0):
+    """0 FlipSign, 1 VecRescale, 2 FHTRotate, 3 KacsWalk of the reference's generic kernels, on a copy."""
+    out = f32(data).copy()
+    fp = _p(np.ascontiguousarray(flip, np.uint8)) if flip is not None else None
+    lib().orc_fht_primitive(which, fp, _p(out), u64(out.shape[0]), C.c_float(val))
+    return out
+
+
+def fht_kac_transform(flip, x, inverse=False):
+    """FhtKacRotator::Transform / InverseTransform of every row of x with the sign bits `flip` (4 x ceil(d / 8) bytes)."""
+    x = f32(np.atleast_2d(x))
+    flip = np.ascontiguousarray(flip, np.uint8)
+    out = np.empty_like(x)
+    for i in range(x.shape[0]):
+        lib().orc_fht_kac_transform(_p(flip), u64(x.shape[1]), 1 if inverse else 0, _p(x[i]), _p(out[i]))
+    return out
+
+
 def rabitq_bits(qbits, base_bits=1):
     """The `qbits` argument of every rabitq function here: query bits (4 | 32) plus 256 * base bits for multi-bit base
     codes (rabitq_bits_per_dim_base 2..8, fp32 queries only)."""
@@ -491,6 +509,10 @@ _REF_SYMBOLS = {
     "RaBitQFloatSplitCodeIP": "_ZN4vsag7generic22RaBitQFloatSplitCodeIPEPKfPKhS4_mj",
     "NormalizeWithCentroid": "_ZN4vsag7generic21NormalizeWithCentroidEPKfS2_Pfm",
     "InverseNormalizeWithCentroid": "_ZN4vsag7generic28InverseNormalizeWithCentroidEPKfS2_Pfmf",
+    "FlipSign": "_ZN4vsag7generic8FlipSignEPKhPfm",
+    "VecRescale": "_ZN4vsag7generic10VecRescaleEPfmf",
+    "FHTRotate": "_ZN4vsag7generic9FHTRotateEPfm",
+    "KacsWalk": "_ZN4vsag7generic8KacsWalkEPfm",
     "Normalize": "_ZN4vsag7generic9NormalizeEPKfPfm",
 }
 

@@ -70,3 +70,29 @@ def test_no_device_is_a_loud_error_not_a_fallback():
         capi.init(0)
     # compute entry points refuse as well
     assert lib.vsag_amd_kmeans_assign(None, 1, 1, None, 1, None, None, None, None, 0, None) == -2
+
+
+@pytest.mark.parametrize("d", [1, 2, 7, 8, 33, 64, 100, 128, 200, 256])
+def test_fht_rotator_matrix_is_the_rotator(d):
+    """vsag_amd_fht_kac_matrix (host work only): the matrix times a vector equals FhtKacRotator::Transform
+    (fht_kac_rotate_transformer.cpp:64-96) of that vector as the checker restates it, and R^T undoes it
+    (InverseTransform, :97-120)."""
+    import ctypes as C
+
+    import numpy as np
+
+    import oracle as orc
+    lib = capi.load_library()
+    rng = np.random.default_rng(500 + d)
+    flip = rng.integers(0, 256, 4 * ((d + 7) // 8)).astype(np.uint8)
+    rot = np.empty((d, d), np.float32)
+    capi.check(lib.vsag_amd_fht_kac_matrix(flip.ctypes.data_as(C.c_void_p), d, rot.ctypes.data_as(C.c_void_p)))
+    x = rng.standard_normal((5, d)).astype(np.float32)
+    want = orc.fht_kac_transform(flip, x)
+    tol = 4e-6 * np.sqrt(d) * (1 + np.abs(x).max())
+    np.testing.assert_allclose(x.astype(np.float64) @ rot.astype(np.float64).T, want, rtol=0, atol=tol)
+    np.testing.assert_allclose(want.astype(np.float64) @ rot.astype(np.float64), orc.fht_kac_transform(flip, want, inverse=True),
+                               rtol=0, atol=tol)
+    # the images of the basis vectors, entry for entry
+    cols = orc.fht_kac_transform(flip, np.eye(d, dtype=np.float32))
+    np.testing.assert_allclose(rot.T, cols, rtol=0, atol=1e-6)

@@ -46,6 +46,49 @@ def make(name, dim, metric, **index_param):
                                          "index_param": index_param}))
 
 
+@pytest.mark.parametrize("name,d", [("ivf", 128), ("ivf", 100), ("brute_force", 96)])
+def test_rabitq_with_the_fht_rotator(lib, tmp_path, name, d):
+    """rabitq_use_fht (rabitq_quantizer.cpp:81-86): FhtKacRotator's rotation instead of the random orthogonal matrix,
+    for a power-of-two dimension and for others (the Kac walk branch).  An orthogonal map either way: the recall floor of
+    tests/test_ivf.cpp:1212-1230 holds; the file carries the rotator's sign bits (FhtKacRotator::Serialize) and
+    use_fht in its parameters, loads to the same answers, and is refused by an index built without the flag."""
+    n, nq, k = 3000, 50, 10
+    x = vectors(n, d)
+    q = vectors(nq, d, seed=165)
+    labels = np.arange(n, dtype=np.int64)
+    params = dict(base_quantization_type="rabitq")
+    if name == "ivf":
+        params.update(buckets_count=10, train_sample_count=3000, use_reorder=True, precise_quantization_type="fp32")
+    search = json.dumps({"ivf": {"scan_buckets_count": 10, "factor": 20.0}}) if name == "ivf" else "{}"
+    idx = make(name, d, "l2", rabitq_use_fht=True, **params)
+    idx.build(x, labels, n, d)
+    gt, _ = ground_truth(x, q, k, "l2")
+    ids, dists = idx.knn_search_batch(q, k, search)
+    path = tmp_path / "fht.index"
+    idx.serialize(path)
+    plain = make(name, d, "l2", **params)
+    plain.build(x, labels, n, d)
+    if name == "ivf":
+        assert recall(ids, gt, labels) >= 0.85
+    else:
+        # no rerank here: the 1-bit estimate alone, as good with one rotation as with the other
+        assert abs(recall(ids, gt, labels) - recall(plain.knn_search_batch(q, k, search)[0], gt, labels)) <= 0.08
+    plain_path = tmp_path / "plain.index"
+    plain.serialize(plain_path)
+    rot_bytes = d * d * 4 - 4 * ((d + 7) // 8)
+    assert plain_path.stat().st_size - path.stat().st_size >= rot_bytes - 64  # sign bits instead of the matrix
+    assert b'\\"use_fht\\":true' in path.read_bytes() or b'"use_fht":true' in path.read_bytes()
+    again = make(name, d, "l2", rabitq_use_fht=True, **params)
+    again.deserialize(path)
+    ids2, dists2 = again.knn_search_batch(q, k, search)
+    assert np.array_equal(ids, ids2) and np.array_equal(dists, dists2)
+    other = make(name, d, "l2", **params)
+    with pytest.raises(pyvsag.VsagError):
+        other.deserialize(path)
+    for i in (idx, plain, again, other):
+        i.close()
+
+
 @pytest.mark.parametrize("metric", ["l2", "ip", "cosine"])
 @pytest.mark.parametrize("quant,floor", [("fp32", 0.99), ("sq8", 0.84), ("sq4_uniform", 0.5), ("sq8_uniform", 0.84)])
 def test_brute_force_build_and_search(lib, metric, quant, floor):

@@ -439,6 +439,63 @@ def test_rabitq_decode_is_the_sign_point_rotated_back(d):
     assert orc.rabitq_decode(x4, d, rot, cen, orc.L2, qbits=orc.rabitq_bits(32, 4)) is None
 
 
+FHT_DIMS = [1, 2, 7, 8, 33, 64, 100, 128, 200, 256, 960]
+
+
+def test_fht_primitives_match_compiled_reference_kernels():
+    """FlipSign, VecRescale, FHTRotate and KacsWalk (generic.cpp:953-985, butterfly.h) against the reference's own
+    compiled generic kernels: sums and differences only, so bit for bit."""
+    ref = orc.ref()
+    if ref is None:
+        pytest.skip("oracle/_ref is not built (reference sources not mounted)")
+    rng = np.random.default_rng(953)
+    for d in FHT_DIMS:
+        v = rng.standard_normal(d).astype(np.float32)
+        flip = rng.integers(0, 256, (d + 7) // 8).astype(np.uint8)
+        for which, name in enumerate(["FlipSign", "VecRescale", "FHTRotate", "KacsWalk"]):
+            if name == "FHTRotate" and d & (d - 1):
+                continue  # a power-of-two block only
+            want = v.copy()
+            fn = ref[name]
+            fn.restype = None
+            if name == "FlipSign":
+                fn(_p(flip), _p(want), C.c_uint64(d))
+            elif name == "VecRescale":
+                fn(_p(want), C.c_uint64(d), C.c_float(0.37))
+            else:
+                fn(_p(want), C.c_uint64(d))
+            got = orc.fht_primitive(which, v, flip=flip, val=0.37)
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (name, d)
+
+
+@pytest.mark.parametrize("d", FHT_DIMS)
+def test_fht_kac_rotator_is_orthogonal_and_inverts(d):
+    """FhtKacRotator::Transform (fht_kac_rotate_transformer.cpp:64-96) by the reference test's own properties
+    (fht_kac_rotate_transformer_test.cpp:64-86: lengths kept, the inverse returns the input within 1e-4), by
+    orthogonality of the whole map, and -- a power of two without flips -- by the closed form (H / sqrt(d))^4 = I."""
+    rng = np.random.default_rng(64 + d)
+    flip = rng.integers(0, 256, 4 * ((d + 7) // 8)).astype(np.uint8)
+    x = rng.standard_normal((6, d)).astype(np.float32)
+    y = orc.fht_kac_transform(flip, x)
+    back = orc.fht_kac_transform(flip, y, inverse=True)
+    assert np.max(np.abs(back - x)) < 1e-4
+    np.testing.assert_allclose((y.astype(np.float64) ** 2).sum(1), (x.astype(np.float64) ** 2).sum(1), rtol=1e-5)
+    m = orc.fht_kac_transform(flip, np.eye(d, dtype=np.float32)).T.astype(np.float64)  # column j = the image of e_j
+    np.testing.assert_allclose(m @ m.T, np.eye(d), atol=2e-6 * max(8, d) ** 0.5)
+    if d > 2:
+        assert np.abs(m - np.eye(d)).max() > 0.05  # and it does mix
+    if d & (d - 1) == 0:
+        none = np.zeros_like(flip)
+        np.testing.assert_allclose(orc.fht_kac_transform(none, x), x, rtol=0, atol=1e-5)
+        # one round with known flips: H diag(s) x / sqrt(d), H the Sylvester matrix
+        h = np.array([[1.0]])
+        while h.shape[0] < d:
+            h = np.block([[h, h], [h, -h]])
+        s = 1.0 - 2.0 * np.unpackbits(flip[:(d + 7) // 8], bitorder="little")[:d]
+        one = orc.fht_primitive(1, orc.fht_primitive(2, orc.fht_primitive(0, x[0], flip=flip)), val=1.0 / np.sqrt(np.float32(d)))
+        np.testing.assert_allclose(one, h @ (s * x[0]) / np.sqrt(d), rtol=0, atol=1e-5 * (1 + np.abs(x[0]).max()) * np.sqrt(d))
+
+
 def _rabitq_dist(qcode, code, d, metric, qbits):
     L = orc.lib()
     return float(L.orc_rabitq_dist(_p(np.ascontiguousarray(qcode)), _p(np.ascontiguousarray(code)), C.c_uint64(d), metric,

@@ -70,6 +70,7 @@ PROTOTYPES = {
     "vsag_amd_squ_encode": (C.c_int, [_vp, _u64, _u32, _i32, _i32, _vp, _vp, _vp]),
     "vsag_amd_rabitq_train": (C.c_int, [_vp, _u64, _u32, _vp, _vp, _vp]),
     "vsag_amd_rabitq_encode": (C.c_int, [_vp, _u64, _u32, _vp, _vp, _i32, _i32, _vp, _vp]),
+    "vsag_amd_fht_kac_matrix": (C.c_int, [_vp, _u32, _vp]),
     "vsag_amd_rabitq_decode": (C.c_int, [_vp, _u64, _u32, _vp, _vp, _i32, _i32, _vp, _vp]),
     "vsag_amd_rabitq_encode_multibit": (C.c_int, [_vp, _u64, _u32, _vp, _vp, _i32, _i32, _i32, _u32, _vp, _vp]),
     "vsag_amd_rabitq_query_code_size": (_u64, [_u32, _i32, _i32]),

@@ -1296,6 +1296,92 @@ vsag_amd_rabitq_encode(const float* x_dev, uint64_t n, uint32_t dim, const float
     });
 }
 
+// FhtKacRotator (impl/transform/fht_kac_rotate_transformer.cpp:64-96, rabitq_use_fht) as the dense matrix the rabitq
+// entry points take: y = R x with R[i][j] = Transform(e_j)[i].  The rotator is a product of sign flips, Hadamard
+// butterflies on a power-of-two block, Kac walks and scalings, all of them row operations on the matrix of the
+// transformed basis vectors (one column per basis vector), which starts as the identity.  Host memory on both sides.
+extern "C" int
+vsag_amd_fht_kac_matrix(const uint8_t* flip, uint32_t dim, float* rotation) {
+    VA_CHECK_ARG(flip != nullptr && rotation != nullptr, "null pointer");
+    VA_CHECK_ARG(dim >= 1 && dim <= 65536, "dim must be in [1, 65536], got %u", dim);
+    const size_t d = dim;
+    const size_t flip_bytes = (d + 7) / 8;
+    size_t block = 1;  // the largest power of two within dim
+    while (block * 2 <= d) {
+        block *= 2;
+    }
+    const float scale = 1.0F / std::sqrt(static_cast<float>(block));
+    std::fill(rotation, rotation + d * d, 0.0F);
+    for (size_t i = 0; i < d; ++i) {
+        rotation[i * d + i] = 1.0F;
+    }
+    auto row = [&](size_t i) { return rotation + i * d; };
+    auto flip_rows = [&](int round) {
+        const uint8_t* f = flip + static_cast<size_t>(round) * flip_bytes;
+        for (size_t i = 0; i < d; ++i) {
+            if ((f[i >> 3] >> (i & 7)) & 1) {
+                float* r = row(i);
+                for (size_t j = 0; j < d; ++j) {
+                    r[j] = -r[j];
+                }
+            }
+        }
+    };
+    auto pair_rows = [&](size_t a, size_t b) {  // (a, b) <- (a + b, a - b)
+        float* ra = row(a);
+        float* rb = row(b);
+        for (size_t j = 0; j < d; ++j) {
+            const float x = ra[j], y = rb[j];
+            ra[j] = x + y;
+            rb[j] = x - y;
+        }
+    };
+    auto scale_rows = [&](size_t first, size_t count, float v) {
+        for (size_t i = first; i < first + count; ++i) {
+            float* r = row(i);
+            for (size_t j = 0; j < d; ++j) {
+                r[j] *= v;
+            }
+        }
+    };
+    auto hadamard = [&](size_t first) {
+        for (size_t step = 1; step < block; step *= 2) {
+            for (size_t i = 0; i < block; i += 2 * step) {
+                for (size_t j = 0; j < step; ++j) {
+                    pair_rows(first + i + j, first + i + j + step);
+                }
+            }
+        }
+        scale_rows(first, block, scale);
+    };
+    auto kac_walk = [&]() {
+        const size_t half = d / 2, offset = half + d % 2;
+        for (size_t i = 0; i < half; ++i) {
+            pair_rows(i, i + offset);
+        }
+        if (d % 2 != 0) {
+            scale_rows(half, 1, std::sqrt(2.0F));
+        }
+    };
+    if (block == d) {
+        for (int round = 0; round < 4; ++round) {
+            flip_rows(round);
+            hadamard(0);
+        }
+        return 0;
+    }
+    for (int round = 0; round < 4; round += 2) {
+        flip_rows(round);
+        hadamard(0);
+        kac_walk();
+        flip_rows(round + 1);
+        hadamard(d - block);
+        kac_walk();
+    }
+    scale_rows(0, d, 0.25F);  // four Kac walks, each of which doubles the squared length
+    return 0;
+}
+
 // RaBitQuantizer::DecodeOneImpl (rabitq_quantizer.cpp:871-899), 1-bit codes: y = (+-1 / sqrt(d)) * norm + centroid
 // per dimension (InverseNormalizeWithCentroid, simd/kernels/normalize.h:88-119), x = R^T y.  A workgroup per code, a
 // thread per output dimension, the rows of R summed in order.

@@ -541,6 +541,10 @@ struct Quantizer {
     bool rabitq_fast_encode = true;
     uint32_t rabitq_fast_rounds = 6;
     uint32_t pq_dim = 1;  // pqfs: subspaces (PQFastScanQuantizerParameter::pq_dim_, default 1)
+    // rabitq_use_fht: the rotation is FhtKacRotator's (fht_kac_rotate_transformer.cpp), kept as its sign bits (what
+    // the reference serializes) and handed to the device as the dense matrix it stands for.
+    bool rabitq_use_fht = false;
+    std::vector<uint8_t> fht_flip;
     bool trained = false;
     DevBuf lb, diff, bounds, rotation, centroid, codebooks;
 
@@ -590,6 +594,13 @@ struct Quantizer {
         return std::vector<float>(m.begin(), m.end());
     }
 
+    std::vector<float>
+    fht_matrix() const {
+        std::vector<float> rot(static_cast<size_t>(dim) * dim);
+        dev(vsag_amd_fht_kac_matrix(fht_flip.data(), dim, rot.data()));
+        return rot;
+    }
+
     void
     train(const float* x_dev, uint64_t n) {
         if (trained || n == 0) {
@@ -625,7 +636,20 @@ struct Quantizer {
                 break;
             }
             case VSAG_AMD_KIND_RABITQ: {
-                std::vector<float> rot = random_rotation(dim, 20240229U);
+                std::vector<float> rot;
+                if (rabitq_use_fht) {
+                    // FhtKacRotator::Train (fht_kac_rotate_transformer.cpp:50-57): uniform bytes; seeded here, from
+                    // std::random_device there
+                    std::mt19937 gen(20240229U);
+                    std::uniform_int_distribution<int> byte(0, 255);
+                    fht_flip.resize(4 * ((static_cast<size_t>(dim) + 7) / 8));
+                    for (auto& b : fht_flip) {
+                        b = static_cast<uint8_t>(byte(gen));
+                    }
+                    rot = fht_matrix();
+                } else {
+                    rot = random_rotation(dim, 20240229U);
+                }
                 rotation.reserve(rot.size() * 4);
                 centroid.reserve(dim * 4);
                 dev(vsag_amd_memcpy_h2d(rotation.p, rot.data(), rot.size() * 4, nullptr));
@@ -697,11 +721,13 @@ struct Quantizer {
         q.rabitq_fast_encode = rabitq_fast_encode;
         q.rabitq_fast_rounds = rabitq_fast_rounds;
         q.pq_dim = pq_dim;
+        q.rabitq_use_fht = rabitq_use_fht;
         return q;
     }
     void
     take(Quantizer& other) {
         trained = other.trained;
+        std::swap(fht_flip, other.fht_flip);
         for (auto pair : {std::make_pair(&lb, &other.lb), std::make_pair(&diff, &other.diff),
                           std::make_pair(&bounds, &other.bounds), std::make_pair(&rotation, &other.rotation),
                           std::make_pair(&centroid, &other.centroid), std::make_pair(&codebooks, &other.codebooks)}) {
@@ -771,7 +797,14 @@ struct Quantizer {
             }
             case VSAG_AMD_KIND_RABITQ:
                 w.vec(floats(centroid, dim));
-                w.vec(floats(rotation, static_cast<size_t>(dim) * dim));
+                if (rabitq_use_fht) {
+                    // FhtKacRotator::Serialize (fht_kac_rotate_transformer.cpp:122-125): the sign bits
+                    std::vector<uint8_t> flip = fht_flip;
+                    flip.resize(4 * ((static_cast<size_t>(dim) + 7) / 8), 0);
+                    w.vec(flip);
+                } else {
+                    w.vec(floats(rotation, static_cast<size_t>(dim) * dim));
+                }
                 break;
             case VSAG_AMD_KIND_PQFS:
                 // PQFastScanQuantizer::SerializeImpl (pq_fastscan_quantizer.cpp:201-207)
@@ -823,8 +856,19 @@ struct Quantizer {
             }
             case VSAG_AMD_KIND_RABITQ:
                 r.vec(a);
-                r.vec(b);
                 upload(centroid, a, dim);
+                if (rabitq_use_fht) {
+                    r.vec(fht_flip);
+                    if (fht_flip.size() != 4 * ((static_cast<size_t>(dim) + 7) / 8)) {
+                        throw VsagException(ErrorType::INVALID_ARGUMENT, "the serialized rotator has " +
+                                                                             std::to_string(fht_flip.size()) +
+                                                                             " sign bytes, this dimension takes " +
+                                                                             std::to_string(4 * ((dim + 7) / 8)));
+                    }
+                    b = fht_matrix();
+                } else {
+                    r.vec(b);
+                }
                 upload(rotation, b, static_cast<size_t>(dim) * dim);
                 break;
             case VSAG_AMD_KIND_PQFS: {
@@ -1076,7 +1120,8 @@ quantization_params_json(const Quantizer& q) {
     } else if (q.kind == VSAG_AMD_KIND_RABITQ) {
         s += ",\"pca_dim\":0,\"rabitq_version\":\"standard\",\"rabitq_bits_per_dim_query\":" +
              std::to_string(q.rabitq_query_bits) + ",\"rabitq_bits_per_dim_base\":" + std::to_string(q.rabitq_base_bits) +
-             ",\"rabitq_bits_per_dim_filter\":1,\"rabitq_error_rate\":1.9,\"use_fht\":false,\"fast_encode_rabitq\":" +
+             ",\"rabitq_bits_per_dim_filter\":1,\"rabitq_error_rate\":1.9,\"use_fht\":" +
+             (q.rabitq_use_fht ? "true" : "false") + ",\"fast_encode_rabitq\":" +
              (q.rabitq_fast_encode ? "true" : "false") +
              ",\"fast_encode_rabitq_rounds\":" + std::to_string(q.rabitq_fast_rounds);
     }
@@ -1130,7 +1175,7 @@ quantization_params_compatible(const Json& file, const Quantizer& q) {
         if (file.Contains("rabitq_version") && file["rabitq_version"].GetString() != "standard") {
             return false;
         }
-        if (file.Contains("use_fht") && file["use_fht"].GetBool()) {
+        if (file.Contains("use_fht") && file["use_fht"].GetBool() != q.rabitq_use_fht) {
             return false;
         }
     }
@@ -1881,7 +1926,7 @@ read_rabitq_params(const Json& index_param, Quantizer& q) {
             q.rabitq_fast_rounds = static_cast<uint32_t>(rounds);
         }
         if (index_param.Contains("rabitq_use_fht")) {
-            CHECK_ARGUMENT(!index_param["rabitq_use_fht"].GetBool(), "rabitq_use_fht is not supported");
+            q.rabitq_use_fht = index_param["rabitq_use_fht"].GetBool();
         }
     }
 }
