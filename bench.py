@@ -30,6 +30,7 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F32_PEAK_TFLOPS = 157.3
 MFMA_I8_PEAK_TOPS = 5000.0  # dense int8, published
 MFMA_F6F4_PEAK_TFLOPS = 10100.0  # dense fp6 / fp4, published
+MFMA_F16_PEAK_TFLOPS = 2500.0  # dense fp16 / bf16, published
 # HBM/fabric bytes of the last-level launch of prefilter_i8_kernel<l2> on configs[1] (profiles/prefilter_i8_sq8_c2.md)
 PROFILE_TRAFFIC_I8_C2 = 235670.3 * 2.00 * 1024 + 60099.9 * 1024
 
@@ -388,13 +389,16 @@ def run_c2(env):
         # of the launch = 2 d operations per (query, code) pair; the int8 kernel executes twice that (two int8 planes
         # per query), reported beside it.  The same launch by the memory figure: passes x code bytes.
         i8 = r["tile"] == 256
+        # (beyond 128 dimensions the fp16 matrix cores take the code bytes and one fp16 part of the scaled query)
+        h16 = not i8 and d > 128 and args.contraction != 2
         codes = r["bytes_per_pass"] / float(-(-d // 16) * 16)
         ops = 2.0 * codes * d * nq
         rate = ops / (r["kernel_ms"] * 1e-3) / 1e12
-        peak = MFMA_I8_PEAK_TOPS if i8 else MFMA_F32_PEAK_TFLOPS
+        peak = MFMA_I8_PEAK_TOPS if i8 else MFMA_F16_PEAK_TFLOPS if h16 else MFMA_F32_PEAK_TFLOPS
         roof = {"bound": "mfma", "achieved": rate, "peak": peak, "unit": "TOP/s" if i8 else "TFLOP/s",
                 "frac": rate / peak, "traffic": traffic, "traffic_source": traffic_source,
-                "kernel": "prefilter_i8_kernel<l2> (int8 MFMA, last level)" if i8 else "prefilter_kernel<sq8> (fp32 MFMA)",
+                "kernel": "prefilter_i8_kernel<l2> (int8 MFMA, last level)" if i8 else
+                          "prefilter_h16_kernel (fp16 MFMA, last level)" if h16 else "prefilter_kernel<sq8> (fp32 MFMA)",
                 "kernel_ms": r["kernel_ms"], "ops_per_launch": ops, "codes_per_launch": codes,
                 "mfma_frac": rate / peak,
                 "executed_ops_per_launch": (2.0 if i8 else 1.0) * 2.0 * codes * (-(-d // 32) * 32) * nq,
@@ -967,8 +971,8 @@ def main():
     ap.add_argument("--k", type=int, default=10)
     ap.add_argument("--tile", type=int, default=0, help="query tile override (0 = library default)")
     ap.add_argument("--chunks", type=int, default=0, help="base chunk override (0 = library default)")
-    ap.add_argument("--contraction", type=int, default=0, choices=[-1, 0, 1],
-                    help="matrix-core path of the flat scans: -1 never, 0 library default, 1 whenever supported")
+    ap.add_argument("--contraction", type=int, default=0, choices=[-1, 0, 1, 2],
+                    help="matrix-core path of the flat scans: -1 never, 0 library default, 1 whenever supported, 2 the fp32 matrix cores only")
     ap.add_argument("--list-codes", default="sq4_uniform", choices=["sq4_uniform", "sq8_uniform", "sq8", "rabitq", "pqfs", "fp32"],
                     help="c4 only: the quantizer of the posting lists (configs[3] names sq4_uniform)")
     ap.add_argument("--pq-dim", type=int, default=0, help="c4 with --list-codes pqfs: subspaces (default: the dimension)")

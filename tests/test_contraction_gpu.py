@@ -55,6 +55,43 @@ def test_sq8_contraction_equals_streaming(lib, modes, metric, n, d, nq, k):
 
 
 @pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
+@pytest.mark.parametrize("n,d,nq,k", [(30000, 129, 600, 10), (20000, 200, 520, 100), (12000, 960, 512, 10),
+                                      (9000, 1000, 130, 7)])
+def test_sq8_beyond_128_dimensions_on_the_fp16_matrix_cores(lib, modes, metric, n, d, nq, k):
+    """sq8 stores of more than 128 dimensions: the code bytes and the two fp16 parts of the scaled query on
+    v_mfma_f32_32x32x16_f16 (prefilter_h16.hip), rescored exactly.  Awkward queries as for the int8 planes: zeros,
+    tiny and huge magnitudes, one dominant dimension, copies of stored vectors, far outside the trained range, NaN."""
+    rng = np.random.default_rng(n + d + k + metric)
+    x, means = gaussian_mixture(rng, n, d, 20, 0.05)
+    q, _ = gaussian_mixture(rng, nq, d, 20, 0.05, means=means)
+    if metric != orc.COSINE:  # no direction to normalise
+        q[0] = 0.0
+        q[1] = 1e-20
+        q[6] = np.nan
+        q[7, 3] = np.inf
+    q[2] *= 1e6
+    q[3] *= 1e-6
+    q[4] = 0.0
+    q[4, d // 2] = 1e4
+    q[5] = 1e-30
+    q[5, 1] = 3e37 if metric != orc.COSINE else 3.0
+    q[8:40] = x[8:40]
+    q[40:60] = -q[40:60]
+    q[60:80] += 100.0
+    lb, diff = orc.sq_train(x, 8, metric)
+    codes = orc.sq_encode(x, 8, lb, diff, metric)
+    st = Store(capi.KIND_SQ8, metric, d, lb=lb, diff=diff)
+    st.append(codes[:n // 2])
+    st.append(codes[n // 2:])
+    plain, fast, tile = modes(st, q, k, 1)
+    assert tile == 128, "the contraction path did not run"
+    assert same(plain, fast)
+    plain, fp32, tile = modes(st, q, k, 2)  # the fp32 matrix cores: the same again
+    assert tile == 128 and same(plain, fp32)
+    st.destroy()
+
+
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
 @pytest.mark.parametrize("d", [16, 100, 128])
 def test_sq8_int8_planes_hold_for_awkward_queries(lib, modes, metric, d):
     """Queries the two int8 planes represent badly or trivially: one dominant dimension, tiny and huge magnitudes,

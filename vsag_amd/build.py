@@ -21,7 +21,7 @@ HIP_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
 ]
-KERNEL_SOURCES = ["runtime.hip", "store.hip", "quantize.hip", "prepare.hip", "scan.hip", "prefilter.hip", "prefilter_i8.hip", "prefilter_rb.hip", "ivf.hip", "ivf_i8.hip", "ivf_pq.hip",
+KERNEL_SOURCES = ["runtime.hip", "store.hip", "quantize.hip", "prepare.hip", "scan.hip", "prefilter.hip", "prefilter_i8.hip", "prefilter_rb.hip", "prefilter_h16.hip", "ivf.hip", "ivf_i8.hip", "ivf_pq.hip",
                   "kmeans.hip", "lookup.hip", "export.hip", "scan_one.hip", "pq.hip"]
 
 

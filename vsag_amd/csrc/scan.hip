@@ -807,6 +807,7 @@ struct CallPlan {
     uint64_t level_begin[kMaxLevels + 1] = {};
     bool int8 = false;         // the int8 matrix cores pre-select (sq8, at most 128 dimensions)
     bool rb = false;           // RaBitQ store: 1-bit codes x 4-bit queries on the int8 matrix cores
+    size_t h16_scratch = 0;    // sq8 beyond 128 dimensions: bytes of the fp16 query planes (0: the fp32 matrix cores)
     uint32_t cap = 0;          // candidates per query and level
     uint32_t sub_lists[kMaxLevels] = {};  // int8: private candidate lists per query ...
     uint32_t sub_cap[kMaxLevels] = {};    // ... of this many slots
@@ -846,6 +847,8 @@ size_t prefilter_i8_scalar_floats(uint64_t nq);
 uint32_t prefilter_i8_sub_lists(uint64_t nq, uint64_t span);
 bool prefilter_rb_supports(const vsag_amd_store* s);
 size_t prefilter_rb_scratch_bytes(const vsag_amd_store* s, uint64_t nq);
+bool prefilter_h16_supports(const vsag_amd_store* s);
+size_t prefilter_h16_scratch_bytes(const vsag_amd_store* s, uint64_t nq);
 uint32_t prefilter_rb_sub_lists(uint64_t nq, uint64_t span);
 
 // Whether a call goes through the table of approximate distances (see CallPlan::table).
@@ -935,6 +938,10 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
                                            s->kind == VSAG_AMD_KIND_SQ4_UNIFORM || s->kind == VSAG_AMD_KIND_SQ4);
     c->rb = rb;
     c->rb_scratch = rb ? prefilter_rb_scratch_bytes(s, nq) : 0;
+    // (mode 2 keeps the fp32 matrix cores)
+    c->h16_scratch = !c->int8 && !rb && prefilter_mode(s) != 2 && prefilter_h16_supports(s)
+                         ? prefilter_h16_scratch_bytes(s, nq)
+                         : 0;
     c->prefix_tiles = prefix;
     c->cap = static_cast<uint32_t>(cap);
     c->levels = nb - 1;
@@ -1008,8 +1015,8 @@ carve_scan(Carver& c, const CallPlan& cp, uint64_t nq, uint32_t k, ScanBuffers* 
     const uint64_t nq_pad8 = prefilter_i8_query_bytes(nq) / 256;  // whole workgroups of the int8 prefilter
     b->tau = c.take<float>(cp.contraction ? nq_pad8 : 0);
     b->q8_u = c.take<float>(cp.int8 ? prefilter_i8_scalar_floats(nq) : 0);
-    b->q8 = c.take<uint8_t>(cp.int8 ? prefilter_i8_query_bytes(nq) : (cp.rb ? cp.rb_scratch : 0));
-    if (!cp.int8 && !cp.rb) {
+    b->q8 = c.take<uint8_t>(cp.int8 ? prefilter_i8_query_bytes(nq) : (cp.rb ? cp.rb_scratch : cp.h16_scratch));
+    if (!cp.int8 && !cp.rb && cp.h16_scratch == 0) {
         b->q8 = nullptr;
     }
     b->cand_cnt = c.take<uint32_t>(cp.contraction ? nq * std::max<uint32_t>(1, cp.max_lists) : 0);
