@@ -1149,7 +1149,8 @@ int launch_prefilter_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq,
 bool prefilter_i8_supports(const vsag_amd_store* s);
 bool prefilter_h16_supports(const vsag_amd_store* s);
 int launch_prefilter_h16(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint64_t tile_begin, uint64_t tile_end,
-                         float* tau, uint8_t* scratch, uint32_t* cand, uint32_t* cand_cnt, uint32_t cap, hipStream_t st);
+                         const uint32_t* bound, float* tau, uint8_t* scratch, uint32_t* cand, uint32_t* cand_cnt,
+                         uint32_t cap, hipStream_t st);
 
 bool
 prefilter_supports(const vsag_amd_store* s) {
@@ -1278,10 +1279,7 @@ launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32
     }
     if (q8 != nullptr && prefilter_h16_supports(s)) {
         // sq8 beyond 128 dimensions: the fp16 matrix cores pre-select (prefilter_h16.hip); q8 is its scratch.
-        hipLaunchKernelGGL(prefilter_tau_kernel, dim3(static_cast<uint32_t>(nq)), dim3(kWave), 0, st,
-                           reinterpret_cast<const float*>(a.qtab), a.qstride, s->dpad, !l2 ? a.qmeta : nullptr,
-                           a.qmeta_stride, l2 ? 1 : 0, bound, s->pf_ymax, nq, tau);
-        VA_TRY(launch_prefilter_h16(s, a, nq, tile_begin, tile_end, tau, q8, cand, cand_cnt, cap, st));
+        VA_TRY(launch_prefilter_h16(s, a, nq, tile_begin, tile_end, bound, tau, q8, cand, cand_cnt, cap, st));
         return launch_rescore(s, a, nq, k, S, bound, cand, cand_cnt, cap, 0, 0, partial, partial_cnt, nslots, first_slot,
                               out_slot, gate, st);
     }

@@ -3,22 +3,23 @@
 // The int8 pass (prefilter_i8.hip) keeps a query's operands in registers, which ends at 128 dimensions; beyond that
 // sq8 stores used the fp32 matrix cores (prefilter.hip, prefilter_kernel).  The contraction <b, c> of a code c (bytes
 // 0..255) with the query b folded with the per-dimension scale (l2: b_d = (q_d - lb_d) scale_d, ip: b_d = q_d scale_d)
-// does not need fp32 operands: a byte is exact in fp16, and b splits, after a power-of-two scaling per query, into two
-// fp16 parts,
+// does not need fp32 operands: a byte is exact in fp16, and b is taken, after a power-of-two scaling per query, as
+// its nearest fp16 value, hi_d = fp16(2^E b_d).  The products hi_d c_d are exact in the fp32 accumulator of
+// v_mfma_f32_32x32x16_f16, which runs at sixteen times the rate of the fp32 instruction.  A pair is lost only if the
+// matrix cores' product comes out too small (it comes off the distance, and the codes are not negative): what the
+// fp16 values fall short of their b_d is summed per query in double precision, times the largest code value, and the
+// accumulation is allowed two roundings per instruction of the absolute sum.  Both go onto the query's threshold
+// (h16_split_kernel), next to what the streaming kernel's own fp32 arithmetic can be off by -- a multiple of the
+// distance, not of |q| |y|, since no fp32 contraction stands between the test and the truth here.  (A second fp16
+// part of the query would carry the 2^-12 the first misses; it doubles the matrix work and the LDS reads and saves
+// less in rescoring than it costs.)  Everything kept is rescored exactly, so the result equals the streaming scan's
+// bit for bit.
 //
-//      2^E b_d = hi_d + lo_d + r_d,     hi_d = fp16(2^E b_d),   lo_d = fp16(2^E b_d - hi_d),   |r_d| <= 2^-22 |2^E b_d|,
-//
-// whose products with a byte are exact in the fp32 accumulator of v_mfma_f32_32x32x16_f16, which runs at sixteen
-// times the rate of the fp32 instruction: two of them per block of dimensions.  What the two parts miss (r_d, the
-// rounding of b_d itself) is measured per query in double precision against the real product, times the largest code
-// value; the accumulation of the matrix cores is allowed two roundings per instruction of the absolute sum.  Both go
-// onto the query's threshold (h16_split_kernel), on top of the margin the fp32 pass already allows for the streaming
-// kernel's own arithmetic (prefilter_tau_kernel).  Everything kept is rescored exactly, so the result equals the
-// streaming scan's bit for bit.
-//
-// Work split as in prefilter_kernel: a workgroup of four waves multiplies 128 codes (two storage tiles) by 128 queries
-// in stages of 64 dimensions; the stage sits in LDS as 16-byte slots of eight fp16 values, [block of eight dimensions]
-// [row], the operand order of the instruction (lane % 32 = row, lane / 32 = which eight of sixteen dimensions).
+// Work split: a workgroup of four waves multiplies 256 codes (four storage tiles) by 128 queries in stages of 64
+// dimensions, a wave 128 codes by 64 queries; the stage sits in LDS as 16-byte slots of eight fp16 values, [block of
+// eight dimensions][row], the operand order of the instruction (lane % 32 = row, lane / 32 = which eight of sixteen
+// dimensions).  The queries' fp16 values come from a table in the same slot-major order, so global loads and LDS writes
+// are both contiguous.
 #include "distance.h"
 #include "store.h"
 #include "topk.h"
@@ -31,12 +32,11 @@ void timing_end(hipStream_t st);
 typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr uint32_t kH16M = 128;      // codes per workgroup tile
+constexpr uint32_t kH16M = 256;      // codes per workgroup tile (= threads of a workgroup)
 constexpr uint32_t kH16N = 128;      // queries per workgroup tile
 constexpr uint32_t kH16Stage = 64;   // dimensions per stage: eight slots per row
 constexpr uint32_t kH16Slots = kH16Stage / 8;
-// fp16 parts of the query the matrix cores see: with one, what the second would carry goes onto the threshold instead
-constexpr uint32_t kH16Planes = 1;
+
 
 bool
 prefilter_h16_supports(const vsag_amd_store* s) {
@@ -52,11 +52,11 @@ h16_slots_per_row(const vsag_amd_store* s) {
     return round_up(s->dpad, kH16Stage) / 8;
 }
 
-// Scratch of the pass: the two planes, [plane][block of eight dimensions][query] of 16-byte slots, then a factor per query.
+// Scratch of the pass: the queries' fp16 values, [block of eight dimensions][query] of 16-byte slots, then a factor per query.
 size_t
 prefilter_h16_scratch_bytes(const vsag_amd_store* s, uint64_t nq) {
     const uint64_t rows = h16_query_rows(nq);
-    return 2ull * h16_slots_per_row(s) * rows * 16 + rows * sizeof(float);
+    return static_cast<size_t>(h16_slots_per_row(s)) * rows * 16 + rows * sizeof(float);
 }
 
 struct H16SplitArgs {
@@ -68,8 +68,13 @@ struct H16SplitArgs {
     uint32_t slots;      // blocks of eight dimensions per row
     uint4* planes;
     float* factor;       // per query: dot_factor * 2^-E
-    float* tau;          // per query, raised by the error of the split
+    float* tau;          // per query: keep a pair when term_factor |y|^2 + factor <hi, c> <= tau
     float dot_factor;
+    int is_l2;
+    const float* qmeta;  // ip: sum q_d lb_d per query
+    uint32_t qmeta_stride;
+    const uint32_t* bound;      // per query, ordered-float bits; 0xFFFFFFFF = none yet
+    const uint32_t* ymax_bits;  // largest |y| of the store (l2: scaled codes, ip: raw codes)
 };
 
 // One wave per query row (rows at or beyond nq: zeros).
@@ -79,18 +84,24 @@ h16_split_kernel(H16SplitArgs p) {
     const uint32_t lane = threadIdx.x;
     const bool real = q < p.nq;
     const float* row = p.qtab + q * p.qstride;
-    // the largest |b_d| and whether every entry is finite
+    // the largest |b_d|, whether every entry is finite, and the query's |a|^2 and sum |a_d|
     float amax = 0.0F;
     bool finite = true;
+    double a2 = 0.0, a1 = 0.0;
     if (real) {
         for (uint32_t d = lane; d < p.kdim; d += kWave) {
-            const float b = static_cast<float>(static_cast<double>(row[d]) * (p.scale != nullptr ? static_cast<double>(p.scale[d]) : 1.0));
+            const double a = static_cast<double>(row[d]);
+            const float b = static_cast<float>(a * (p.scale != nullptr ? static_cast<double>(p.scale[d]) : 1.0));
             finite = finite && b - b == 0.0F;
             amax = fmaxf(amax, fabsf(b));
+            a2 += a * a;
+            a1 += fabs(a);
         }
     }
     for (int off = 32; off > 0; off >>= 1) {
         amax = fmaxf(amax, __shfl_xor(amax, off));
+        a2 += __shfl_xor(a2, off);
+        a1 += __shfl_xor(a1, off);
     }
     finite = __ballot(!finite) == 0;
     const bool usable = real && finite && amax > 0.0F;
@@ -104,7 +115,7 @@ h16_split_kernel(H16SplitArgs p) {
     const float up = ldexpf(1.0F, e), down = ldexpf(1.0F, -e);
     double miss = 0.0, sum_abs = 0.0;
     for (uint32_t s = lane; s < p.slots; s += kWave) {
-        halfx8 hi, lo;
+        halfx8 hi;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const uint32_t d = 8 * s + i;
@@ -114,16 +125,15 @@ h16_split_kernel(H16SplitArgs p) {
             }
             const float b = static_cast<float>(exact) * up;  // a power of two: exact
             const _Float16 h = static_cast<_Float16>(b);
-            const _Float16 l = kH16Planes == 2 ? static_cast<_Float16>(b - static_cast<float>(h)) : static_cast<_Float16>(0.0F);
+
             hi[i] = h;
-            lo[i] = l;
-            const double kept = (static_cast<double>(static_cast<float>(h)) + static_cast<double>(static_cast<float>(l))) *
-                                static_cast<double>(down);
-            miss += fabs(kept - exact);
+            const double kept = static_cast<double>(static_cast<float>(h)) * static_cast<double>(down);
+            // Only what makes the matrix cores' product too small can lose a pair (the codes are not negative, the
+            // product comes off the distance): the parts of b_d the fp16 value falls short of.
+            miss += exact > kept ? exact - kept : 0.0;
             sum_abs += fabs(kept);
         }
-        p.planes[(0ull * p.slots + s) * p.rows + q] = __builtin_bit_cast(uint4, hi);
-        p.planes[(1ull * p.slots + s) * p.rows + q] = __builtin_bit_cast(uint4, lo);
+        p.planes[static_cast<uint64_t>(s) * p.rows + q] = __builtin_bit_cast(uint4, hi);
     }
     for (int off = 32; off > 0; off >>= 1) {
         miss += __shfl_xor(miss, off);
@@ -136,20 +146,44 @@ h16_split_kernel(H16SplitArgs p) {
     if (!real) {
         return;
     }
-    if (!usable) {
-        // NaN or infinite entries, or an all-zero query: every code is a candidate (the query overflows and streams)
-        if (!finite) {
-            p.tau[q] = 3.0e38F;
-        }
+    const uint32_t bbits = p.bound[q];
+    if (!finite || bbits == 0xFFFFFFFFU) {
+        // no bound yet, or NaN / infinite entries: every code is a candidate (the query overflows and streams)
+        p.tau[q] = 3.0e38F;
         return;
     }
-    // every code value lies in [0, 255]; two roundings of the running absolute sum per matrix instruction (sixteen
-    // dimensions each, two instructions per block) and four for the closing operations
-    const double roundings = 2.0 * (p.kdim / 8.0 + 4.0) * 5.9604644775390625e-8;
+    constexpr double kU = 5.9604644775390625e-8;  // 2^-24, the unit roundoff of fp32
+    const double bd = static_cast<double>(ordered_to_float(bbits));
+    const double ymax = static_cast<double>(__uint_as_float(*p.ymax_bits)) * (1.0 + 1.0e-6);
+    const double dots = sqrt(a2) * ymax;  // |<a, y>| of any code
+    double t;
+    if (p.is_l2) {
+        // The streaming kernel sums fl(fl(c s) - a)^2 in fp32: off from the real sum S by at most
+        // 2u sum |y - a| |y| + (n + 2) u S <= 2u sqrt(S) |y| + (n + 2) u S to first order; twice that is allowed for.
+        // |y|^2 per code is accumulated in double and rounded once.
+        const double s_abs = fabs(bd);
+        const double e_stream = 4.0 * kU * sqrt(s_abs) * ymax + 2.0 * (p.kdim + 4) * kU * s_abs;
+        const double e_term = 2.0 * kU * ymax * ymax;
+        // S = |a|^2 + |y|^2 - 2 <b, c>: the pair can matter when |y|^2 - 2 <b, c> <= bd - |a|^2 + errors
+        t = bd - a2 + e_stream + e_term;
+    } else {
+        // dist = 1 - (fl(sum c a) + qmeta): the fp32 sum is off by at most n u sum |c a|, the two closing operations by u
+        // of their results; twice that is allowed for.
+        const double qm = p.qmeta != nullptr ? static_cast<double>(p.qmeta[q * p.qmeta_stride]) : 0.0;
+        const double m = fmin(255.0 * a1, dots);
+        const double e_stream = 2.0 * (p.kdim + 2) * kU * m + 4.0 * kU * (m + fabs(qm) + 1.0 + fabs(bd));
+        t = bd - 1.0 + qm + e_stream;
+    }
+    // every code value lies in [0, 255]: what the fp16 value misses of b_d, and two roundings of the running absolute
+    // sum per matrix instruction (sixteen dimensions each) plus four for the closing operations
+    const double roundings = 2.0 * (p.kdim / 16.0 + 4.0) * kU;
     const double extra = fabs(static_cast<double>(p.dot_factor)) * 255.0 * (miss + roundings * sum_abs);
-    const float t = p.tau[q];
-    const float raised = t + static_cast<float>(extra) * (1.0F + 1.0e-6F);
-    p.tau[q] = raised < 3.0e38F ? raised : 3.0e38F;
+    // the test itself: fl(term + fl(factor acc)) against the threshold rounded to fp32
+    const double e_test = 4.0 * kU * (ymax * ymax + 2.0 * dots + fabs(t) + extra);
+    t += extra + e_test;
+    const float tf = static_cast<float>(t);
+    const float up1 = tf + fabsf(tf) * 1.2e-7F + 1.0e-37F;  // not below t after the rounding to fp32
+    p.tau[q] = up1 < 3.0e38F ? up1 : 3.0e38F;
 }
 
 struct PrefilterH16Args {
@@ -172,40 +206,43 @@ struct PrefilterH16Args {
 
 struct H16Stage {
     uint4 a[kH16Slots][kH16M];
-    uint4 b[kH16Planes][kH16Slots][kH16N];
+    uint4 b[kH16Slots][kH16N];
 };
 
-// Sixteen code bytes as sixteen fp16 values (two slots).
+// Sixteen code bytes as sixteen fp16 values (two slots).  A byte b under the high byte 0x64 is the fp16 value
+// 1024 + b (the spacing of fp16 is one from 1024 to 2048); taking 1024 off is exact.
+typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
+__device__ inline uint32_t
+h16_two_bytes(uint32_t w, uint32_t selector) {
+    const uint32_t biased = __builtin_amdgcn_perm(0x64646464U, w, selector);
+    const halfx2 v = __builtin_bit_cast(halfx2, biased) - halfx2{static_cast<_Float16>(1024.0F), static_cast<_Float16>(1024.0F)};
+    return __builtin_bit_cast(uint32_t, v);
+}
 __device__ inline void
 h16_bytes_to_halves(uint4 g, uint4* lo8, uint4* hi8) {
-    const uint32_t w[4] = {g.x, g.y, g.z, g.w};
-    halfx8 out[2];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            out[h][i] = static_cast<_Float16>(static_cast<float>((w[2 * h + (i >> 2)] >> (8 * (i & 3))) & 0xffU));
-        }
-    }
-    *lo8 = __builtin_bit_cast(uint4, out[0]);
-    *hi8 = __builtin_bit_cast(uint4, out[1]);
+    // selector bytes 0..3 pick from w, 4..7 from the constant: (w.b0, 0x64, w.b1, 0x64) and (w.b2, 0x64, w.b3, 0x64)
+    constexpr uint32_t kLow = 0x04010400U, kHigh = 0x04030402U;
+    *lo8 = make_uint4(h16_two_bytes(g.x, kLow), h16_two_bytes(g.x, kHigh), h16_two_bytes(g.y, kLow), h16_two_bytes(g.y, kHigh));
+    *hi8 = make_uint4(h16_two_bytes(g.z, kLow), h16_two_bytes(g.z, kHigh), h16_two_bytes(g.w, kLow), h16_two_bytes(g.w, kHigh));
 }
 
-__global__ void __launch_bounds__(256, 3)
+// A workgroup: 256 codes (four storage tiles) x 128 queries, a wave 128 codes x 64 queries (4 x 2 blocks of 32 x 32):
+// 48 KiB of operands per stage from L2 for 2 M multiply-adds, 6 LDS reads per 8 matrix instructions.
+__global__ void __launch_bounds__(256, 2)
 prefilter_h16_kernel(PrefilterH16Args p) {
     __shared__ H16Stage stage;
     __shared__ float code_term[kH16M];
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63;
     const uint32_t wave = tid >> 6;
-    const uint32_t wm = wave & 1;   // which 64 codes of the tile
+    const uint32_t wm = wave & 1;   // which 128 codes of the tile
     const uint32_t wn = wave >> 1;  // which 64 queries of the tile
     const uint32_t half = lane >> 5;
     const uint32_t l32 = lane & 31;
     const uint64_t q0 = static_cast<uint64_t>(blockIdx.y) * kH16N;  // below p.rows: the grid covers whole tiles of rows
     const uint32_t stages = p.slots / kH16Slots;
     const uint64_t span = p.tile_end - p.tile_begin;
-    const uint64_t mtiles = (span + 1) / 2;
+    const uint64_t mtiles = (span + 3) / 4;
 
     float tau_n[2], fac_n[2];
 #pragma unroll
@@ -215,71 +252,60 @@ prefilter_h16_kernel(PrefilterH16Args p) {
         fac_n[j] = q < p.nq ? p.factor[q] : 0.0F;
     }
 
-    // Code loader: thread (crow, cpart) takes granules 2 cpart and 2 cpart + 1 of the stage's four, for code crow.
-    const uint32_t crow = tid & 127;
-    const uint32_t cpart = tid >> 7;
+    // Code loader: thread t takes the stage's four granules of code t of the tile (storage tile t / 64, lane t % 64).
     auto code_granule = [&](uint64_t mt, uint32_t j) __attribute__((always_inline)) {
-        const uint64_t tile = p.tile_begin + 2 * mt + (crow >> 6);
+        const uint64_t tile = p.tile_begin + 4 * mt + (tid >> 6);
         if (tile < p.tile_end && j < p.G) {
-            return p.tiles[(tile * p.G + j) * kWave + (crow & 63)];
+            return p.tiles[(tile * p.G + j) * kWave + (tid & 63)];
         }
         return make_uint4(0, 0, 0, 0);
     };
-    // Query loader: 2 planes x 8 slots x 128 rows = 2048 slots per stage, eight per thread, consecutive threads on
-    // consecutive rows (global and LDS alike).
-    // (Separate variables, not an array: the array ended up in scratch memory.)
-    uint4 rc0, rc1, rq0, rq1, rq2, rq3, rq4, rq5, rq6, rq7;
+    // Query loader: 8 slots x 128 rows per stage, four per thread, consecutive threads on consecutive rows (global and
+    // LDS alike).  (Separate variables, not arrays: an array ended up in scratch memory.)
+    uint4 rc0, rc1, rc2, rc3, rq0, rq1, rq2, rq3;
     auto query_slot = [&](uint32_t st, uint32_t r) __attribute__((always_inline)) {
         const uint32_t idx = tid + 256 * r;
-        const uint32_t row = idx & 127, slot = (idx >> 7) & 7, plane = idx >> 10;
-        return p.planes[(static_cast<uint64_t>(plane) * p.slots + st * kH16Slots + slot) * p.rows + q0 + row];
+        const uint32_t row = idx & 127, slot = idx >> 7;
+        return p.planes[(static_cast<uint64_t>(st) * kH16Slots + slot) * p.rows + q0 + row];
     };
     auto fetch = [&](uint64_t mt, uint32_t st) __attribute__((always_inline)) {
-        rc0 = code_granule(mt, 4 * st + 2 * cpart);
-        rc1 = code_granule(mt, 4 * st + 2 * cpart + 1);
+        rc0 = code_granule(mt, 4 * st);
+        rc1 = code_granule(mt, 4 * st + 1);
+        rc2 = code_granule(mt, 4 * st + 2);
+        rc3 = code_granule(mt, 4 * st + 3);
         rq0 = query_slot(st, 0);
         rq1 = query_slot(st, 1);
         rq2 = query_slot(st, 2);
         rq3 = query_slot(st, 3);
-        if constexpr (kH16Planes == 2) {
-            rq4 = query_slot(st, 4);
-            rq5 = query_slot(st, 5);
-            rq6 = query_slot(st, 6);
-            rq7 = query_slot(st, 7);
-        }
     };
     auto park_codes = [&](uint32_t g, uint4 v) __attribute__((always_inline)) {
         uint4 lo8, hi8;
         h16_bytes_to_halves(v, &lo8, &hi8);
-        stage.a[2 * (2 * cpart + g)][crow] = lo8;
-        stage.a[2 * (2 * cpart + g) + 1][crow] = hi8;
+        stage.a[2 * g][tid] = lo8;
+        stage.a[2 * g + 1][tid] = hi8;
     };
     auto park_query = [&](uint32_t r, uint4 v) __attribute__((always_inline)) {
         const uint32_t idx = tid + 256 * r;
-        stage.b[idx >> 10][(idx >> 7) & 7][idx & 127] = v;
+        stage.b[idx >> 7][idx & 127] = v;
     };
     auto park = [&]() __attribute__((always_inline)) {
         park_codes(0, rc0);
         park_codes(1, rc1);
+        park_codes(2, rc2);
+        park_codes(3, rc3);
         park_query(0, rq0);
         park_query(1, rq1);
         park_query(2, rq2);
         park_query(3, rq3);
-        if constexpr (kH16Planes == 2) {
-            park_query(4, rq4);
-            park_query(5, rq5);
-            park_query(6, rq6);
-            park_query(7, rq7);
-        }
     };
 
     if (blockIdx.x < mtiles) {
         fetch(blockIdx.x, 0);
     }
     for (uint64_t mt = blockIdx.x; mt < mtiles; mt += p.groups) {
-        floatx16 acc[2][2];
+        floatx16 acc[4][2];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < 4; ++i) {
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
 #pragma unroll
@@ -288,12 +314,12 @@ prefilter_h16_kernel(PrefilterH16Args p) {
                 }
             }
         }
-        const uint64_t slot0 = (p.tile_begin + 2 * mt) * kWave;
+        const uint64_t slot0 = (p.tile_begin + 4 * mt) * kWave;
         park();  // the stage is free: the previous tile's contraction ended with a barrier
-        float my_term = 0.0F;
-        if (tid < kH16M) {
+        float my_term;
+        {
             const uint64_t slot = slot0 + tid;
-            const bool real = slot < p.n && p.tile_begin + 2 * mt + (tid >> 6) < p.tile_end;
+            const bool real = slot < p.n && p.tile_begin + 4 * mt + (tid >> 6) < p.tile_end;
             my_term = real ? p.term_factor * p.term[slot] : __builtin_inff();
         }
         __syncthreads();
@@ -303,31 +329,27 @@ prefilter_h16_kernel(PrefilterH16Args p) {
             } else if (mt + p.groups < mtiles) {
                 fetch(mt + p.groups, 0);
             }
-#pragma unroll
+#pragma unroll 2
             for (uint32_t ks = 0; ks < kH16Stage / 16; ++ks) {
                 const uint32_t slot = 2 * ks + half;
-                halfx8 a[2], bh[2], bl[2];
+                halfx8 a[4], b[2];
 #pragma unroll
-                for (int i = 0; i < 2; ++i) {
-                    const uint4 va = stage.a[slot][wm * 64 + i * 32 + l32];
-                    const uint4 vh = stage.b[0][slot][wn * 64 + i * 32 + l32];
-                    const uint4 vl = kH16Planes == 2 ? stage.b[1][slot][wn * 64 + i * 32 + l32] : make_uint4(0, 0, 0, 0);
-                    a[i] = __builtin_bit_cast(halfx8, va);
-                    bh[i] = __builtin_bit_cast(halfx8, vh);
-                    bl[i] = __builtin_bit_cast(halfx8, vl);
+                for (int i = 0; i < 4; ++i) {
+                    a[i] = __builtin_bit_cast(halfx8, stage.a[slot][wm * 128 + i * 32 + l32]);
                 }
 #pragma unroll
-                for (int i = 0; i < 2; ++i) {
+                for (int j = 0; j < 2; ++j) {
+                    b[j] = __builtin_bit_cast(halfx8, stage.b[slot][wn * 64 + j * 32 + l32]);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
 #pragma unroll
                     for (int j = 0; j < 2; ++j) {
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], bh[j], acc[i][j], 0, 0, 0);
-                        if constexpr (kH16Planes == 2) {
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], bl[j], acc[i][j], 0, 0, 0);
-                        }
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
                     }
                 }
             }
-            if (st + 1 == stages && tid < kH16M) {
+            if (st + 1 == stages) {
                 // every wave is past this tile's first barrier, hence out of the previous tile's epilogue
                 code_term[tid] = my_term;
             }
@@ -337,26 +359,26 @@ prefilter_h16_kernel(PrefilterH16Args p) {
                 __syncthreads();
             }
         }
-        // Nearly nothing passes: the verdicts of all 64 products of a lane branch-free, then the rare hits append.
+        // Nearly nothing passes: the verdicts of all 128 products of a lane branch-free, then the rare hits append.
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            uint32_t hits = 0;
+            uint64_t hits = 0;
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
+            for (int i = 0; i < 4; ++i) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    const uint32_t ml = wm * 64 + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+                    const uint32_t ml = wm * 128 + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
                     const float v = code_term[ml] + fac_n[j] * acc[i][j][e];
-                    hits |= (v <= tau_n[j] ? 1U : 0U) << (16 * i + e);
+                    hits |= static_cast<uint64_t>(v <= tau_n[j] ? 1U : 0U) << (16 * i + e);
                 }
             }
             if (hits != 0) {
                 const uint64_t q = q0 + wn * 64 + j * 32 + l32;
                 while (hits != 0) {
-                    const uint32_t bit = static_cast<uint32_t>(__builtin_ctz(hits));
+                    const uint32_t bit = static_cast<uint32_t>(__builtin_ctzll(hits));
                     hits &= hits - 1;
                     const uint32_t i = bit >> 4, e = bit & 15;
-                    const uint32_t ml = wm * 64 + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+                    const uint32_t ml = wm * 128 + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
                     const uint32_t pos = atomicAdd(&p.cand_cnt[q], 1U);
                     if (pos < p.cap) {
                         p.cand[q * p.cap + pos] = static_cast<uint32_t>(slot0 + ml);
@@ -367,15 +389,16 @@ prefilter_h16_kernel(PrefilterH16Args p) {
     }
 }
 
-// tau holds the thresholds of prefilter_tau_kernel for the store's bounds; scratch: prefilter_h16_scratch_bytes.
+// tau: nq floats, written here from the queries' bounds; scratch: prefilter_h16_scratch_bytes.
 int
 launch_prefilter_h16(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint64_t tile_begin, uint64_t tile_end,
-                     float* tau, uint8_t* scratch, uint32_t* cand, uint32_t* cand_cnt, uint32_t cap, hipStream_t st) {
+                     const uint32_t* bound, float* tau, uint8_t* scratch, uint32_t* cand, uint32_t* cand_cnt, uint32_t cap,
+                     hipStream_t st) {
     const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
     const uint64_t rows = h16_query_rows(nq);
     const uint32_t slots = h16_slots_per_row(s);
     uint4* planes = reinterpret_cast<uint4*>(scratch);
-    float* factor = reinterpret_cast<float*>(scratch + 2ull * slots * rows * 16);
+    float* factor = reinterpret_cast<float*>(scratch + static_cast<size_t>(slots) * rows * 16);
     H16SplitArgs sp{};
     sp.qtab = reinterpret_cast<const float*>(a.qtab);
     sp.qstride = a.qstride;
@@ -388,6 +411,11 @@ launch_prefilter_h16(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, ui
     sp.factor = factor;
     sp.tau = tau;
     sp.dot_factor = l2 ? -2.0F : -1.0F;
+    sp.is_l2 = l2 ? 1 : 0;
+    sp.qmeta = l2 ? nullptr : a.qmeta;
+    sp.qmeta_stride = a.qmeta_stride;
+    sp.bound = bound;
+    sp.ymax_bits = s->pf_ymax;
     hipLaunchKernelGGL(h16_split_kernel, dim3(static_cast<uint32_t>(rows)), dim3(kWave), 0, st, sp);
     PrefilterH16Args p{};
     p.tiles = s->tiles;
@@ -406,10 +434,11 @@ launch_prefilter_h16(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, ui
     p.cand = cand;
     p.cand_cnt = cand_cnt;
     p.cap = cap;
-    const uint64_t mtiles = (tile_end - tile_begin + 1) / 2;
+    const uint64_t mtiles = (tile_end - tile_begin + 3) / 4;
     const uint64_t qtiles = rows / kH16N;
-    // About six workgroups per compute unit (two rounds of the three that fit); a group walks every groups-th tile.
-    uint64_t groups = div_up(static_cast<uint64_t>(device_cu_count()) * 6, qtiles);
+    // At most four workgroups per compute unit -- two rounds of the two that fit, and not one workgroup more: a few left
+    // over for a third round would run it alone.  A group walks every groups-th tile.
+    uint64_t groups = static_cast<uint64_t>(device_cu_count()) * 4 / qtiles;
     groups = std::max<uint64_t>(1, std::min<uint64_t>(groups, mtiles));
     p.groups = static_cast<uint32_t>(groups);
     timing_begin(st);

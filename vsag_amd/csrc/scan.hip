@@ -911,7 +911,9 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
         // (1M codes, 10 000 queries: 2.86 ms per call against 2.98 ms at a factor 16 and 3.00 ms at a factor 4).
         r = std::min<uint64_t>(r, 6);
     }
-    const uint64_t min_prefix = forced ? 2 : (i8 ? std::max<uint64_t>(8, div_up(4ull * k, kWave)) : 64);
+    // (The fp16 pass of sq8 stores beyond 128 dimensions is ten times the streaming kernel: a short prefix there too.)
+    const bool h16 = !i8 && !rb && prefilter_mode(s) != 2 && prefilter_h16_supports(s);
+    const uint64_t min_prefix = forced ? 2 : (i8 || h16 ? std::max<uint64_t>(8, div_up(4ull * k, kWave)) : 64);
     uint64_t bounds[CallPlan::kMaxLevels + 1];
     int nb = 0;
     bounds[nb++] = s->ntiles;
@@ -939,9 +941,7 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
     c->rb = rb;
     c->rb_scratch = rb ? prefilter_rb_scratch_bytes(s, nq) : 0;
     // (mode 2 keeps the fp32 matrix cores)
-    c->h16_scratch = !c->int8 && !rb && prefilter_mode(s) != 2 && prefilter_h16_supports(s)
-                         ? prefilter_h16_scratch_bytes(s, nq)
-                         : 0;
+    c->h16_scratch = h16 && !c->int8 ? prefilter_h16_scratch_bytes(s, nq) : 0;
     c->prefix_tiles = prefix;
     c->cap = static_cast<uint32_t>(cap);
     c->levels = nb - 1;
