@@ -1314,9 +1314,9 @@ launch_prefilter(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32
     p.cap = cap;
     const uint64_t mtiles = (tile_end - tile_begin + 1) / 2;
     const uint64_t qtiles = div_up(nq, static_cast<uint64_t>(PN));
-    // About six workgroups per compute unit (two rounds of the three that fit); a group walks every groups-th
-    // code tile.
-    uint64_t groups = div_up(static_cast<uint64_t>(device_cu_count()) * 6, qtiles);
+    // At most six workgroups per compute unit (two rounds of the three that fit) and not one more: a few left over
+    // would run a third round alone.  A group walks every groups-th code tile.
+    uint64_t groups = static_cast<uint64_t>(device_cu_count()) * 6 / qtiles;
     groups = std::max<uint64_t>(1, std::min<uint64_t>(groups, mtiles));
     p.groups = static_cast<uint32_t>(groups);
     dim3 grid(p.groups, static_cast<uint32_t>(qtiles));
