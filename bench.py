@@ -803,18 +803,22 @@ def run_c4(env):
         # (pqfs: a pair is a contraction of the one-hot centroid indices with the byte table, 16 products per subspace)
         ops = 2.0 * (16 * (-(-pq_dim // 32) * 32) if pqfs else -(-d // 32) * 32) * float(rest)
         tops = ops / (kms * 1e-3) / 1e12
-        peak = (MFMA_F32_PEAK_TFLOPS if raw32 or (per_dim and d > 128) else
+        # (sq8 lists beyond 128 dimensions: the fp16 matrix cores, unless --contraction 2 keeps the fp32 ones)
+        h16 = per_dim and d > 128 and bits == 8 and args.contraction != 2
+        peak = (MFMA_F16_PEAK_TFLOPS if h16 else MFMA_F32_PEAK_TFLOPS if raw32 or (per_dim and d > 128) else
                 MFMA_F6F4_PEAK_TFLOPS if one_bit else MFMA_I8_PEAK_TOPS)
         roof = {"bound": "mfma", "achieved": tops, "peak": peak, "unit": "TOP/s" if peak == MFMA_I8_PEAK_TOPS else "TFLOP/s",
                 "frac": tops / peak,
                 # rocprofv3 --pmc FETCH_SIZE (x 2.00) + WRITE_SIZE of this launch: profiles/ivf_i8_sq4u_c4.md
                 "traffic": 491061.0 * 2.00 * 1024 + 73550.7 * 1024
                 if (n, d, nq, k, nlist, bits) == (10000000, 128, 10000, 10, 4096, 4) else None,
-                "kernel": "%s<%s> (%s MFMA, probe columns 1..%d)" % ("ivf_f32_kernel" if peak == MFMA_F32_PEAK_TFLOPS else
+                "kernel": "%s<%s> (%s MFMA, probe columns 1..%d)" % ("ivf_h16_kernel" if h16 else
+                                                                        "ivf_f32_kernel" if peak == MFMA_F32_PEAK_TFLOPS else
                                                                         "ivf_pq_kernel" if pqfs else
                                                                         "prefilter_rb_kernel<lists>" if one_bit else
                                                                         "ivf_sq8_i8_kernel" if per_dim else "ivf_i8_kernel",
-                                                                        kind_name, "fp32" if peak == MFMA_F32_PEAK_TFLOPS else
+                                                                        kind_name, "fp16" if h16 else
+                                                                        "fp32" if peak == MFMA_F32_PEAK_TFLOPS else
                                                                         "fp4 x fp6" if one_bit else "int8",
                                                                         nprobe - 1), "kernel_ms": kms,
                 "ops_per_launch": ops, "distance_evaluations_per_launch": float(rest),

@@ -35,6 +35,7 @@ struct ScanPlanIvf {
     bool planes;              // ... with sq8 codes: two int8 planes per query, records rescored (prefilter_i8.hip)
     bool bits1;               // ... with rabitq codes: expanded bits, records rescored (prefilter_rb.hip)
     bool pq;                  // ... with pqfs codes: one-hot centroid indices against the byte tables (ivf_pq.hip)
+    bool h16;                 // ... sq8 codes beyond 128 dimensions: the fp16 matrix cores, records rescored
     bool f32;                 // ... with fp32 codes (sq8 beyond 128 dimensions): the fp32 matrix cores, records rescored
                               // (prefilter.hip)
 };
@@ -70,6 +71,12 @@ int launch_ivf_rb(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint3
                   uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st);
 int launch_ivf_clear_gated(uint32_t* gate, uint64_t nq, uint32_t nprobe, uint32_t p0, uint32_t* partial_cnt,
                            const int32_t* buckets, uint32_t* gpairs, uint32_t gpairs_cap, uint32_t k, hipStream_t st);
+bool ivf_h16_supports(const vsag_amd_store* s);
+uint32_t ivf_h16_pairs_per_item();
+size_t ivf_h16_scratch_bytes(const vsag_amd_store* s, uint64_t nq);
+int launch_ivf_h16(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, const uint32_t* pair_off,
+                   const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound, uint32_t kcand, float* tau,
+                   uint8_t* scratch, uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st);
 bool ivf_f32_supports(const vsag_amd_store* s);
 uint32_t ivf_f32_pairs_per_item();
 int launch_ivf_f32(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, const uint32_t* pair_off,
@@ -987,11 +994,15 @@ plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, 
     p->pq = !p->mfma && !p->planes && !p->bits1 && !p->chunked && nprobe > 1 && scan_contraction_mode(s) >= 0 &&
             ivf_pq_supports(s) && s->residual_centroids_dev == nullptr &&
             npairs * ivf_i8_lists_per_pair() * kcand * 8 <= (8ull << 30);
-    // fp32 lists, sq8 lists of more than 128 dimensions: the fp32 matrix cores pre-select, the same exact rescoring.
-    p->f32 = !p->mfma && !p->planes && !p->bits1 && !p->pq && !p->chunked && nprobe > 1 && scan_contraction_mode(s) >= 0 &&
+    // sq8 lists of more than 128 dimensions: the fp16 matrix cores (mode 2 keeps the fp32 ones; residual lists too).
+    p->h16 = !p->mfma && !p->planes && !p->bits1 && !p->pq && !p->chunked && nprobe > 1 && scan_contraction_mode(s) >= 0 &&
+             scan_contraction_mode(s) != 2 && ivf_h16_supports(s) && kcand <= ivf_rescore_capacity() &&
+             npairs * ivf_i8_lists_per_pair() * kcand * 8 <= (8ull << 30);
+    // fp32 lists, sq8 lists the fp16 pass does not take: the fp32 matrix cores pre-select, the same exact rescoring.
+    p->f32 = !p->h16 && !p->mfma && !p->planes && !p->bits1 && !p->pq && !p->chunked && nprobe > 1 && scan_contraction_mode(s) >= 0 &&
              ivf_f32_supports(s) && kcand <= ivf_rescore_capacity() &&
              npairs * ivf_i8_lists_per_pair() * kcand * 8 <= (8ull << 30);
-    p->mfma = p->mfma || p->planes || p->bits1 || p->pq || p->f32;
+    p->mfma = p->mfma || p->planes || p->bits1 || p->pq || p->h16 || p->f32;
     if (p->mfma) {
         p->chunks_max = ivf_i8_lists_per_pair();
     }
@@ -1022,7 +1033,8 @@ carve_ivf(Carver& c, const vsag_amd_store* s, const ScanPlanIvf& p, uint64_t nq,
     b->gate = c.take<uint32_t>(p.mfma ? nq + 3 : 0);
     b->gpairs = c.take<uint32_t>(p.mfma ? kGatedPairsCap : 0);
     b->tq = c.take<int32_t>(p.mfma ? 2 * (nq + 1) : 0);  // thresholds, then (sq8_uniform) the sums of the query values
-    b->q8 = c.take<uint8_t>(p.planes ? ivf_sq8_i8_query_bytes(nq) : p.bits1 ? ivf_rb_scratch_bytes(s, nq) : 0);
+    b->q8 = c.take<uint8_t>(p.planes ? ivf_sq8_i8_query_bytes(nq) : p.bits1 ? ivf_rb_scratch_bytes(s, nq)
+                            : p.h16  ? ivf_h16_scratch_bytes(s, nq) : 0);
     b->q8_u = c.take<float>(p.planes ? ivf_sq8_i8_scalar_floats(nq) : 0);
     b->q8_tau = c.take<uint32_t>(p.planes ? ivf_sq8_i8_tau_words(nq) : 0);
     b->res_term = c.take<float>(s->residual_centroids_dev != nullptr ? p.npairs : 0);
@@ -1186,9 +1198,17 @@ vsag_amd_ivf_scan_topk_ex(const vsag_amd_store_t* s, const float* queries_dev, u
             // lists overflowed -- the streaming kernel's items over the same grouping.
             // ivf_i8.hip: items of 256 pairs, kIvfI8ChunkTiles, kIvfI8Chunks
             regroup(p0, p1, pairs,
-                    p.bits1 ? ivf_rb_pairs_per_item() : p.pq ? ivf_pq_pairs_per_item() : p.f32 ? ivf_f32_pairs_per_item() : 256U,
+                    p.bits1 ? ivf_rb_pairs_per_item() : p.pq ? ivf_pq_pairs_per_item() : p.h16 ? ivf_h16_pairs_per_item()
+                    : p.f32 ? ivf_f32_pairs_per_item() : 256U,
                     p.bits1 ? ivf_rb_chunk_tiles() : 32U, 4U);
-            if (p.f32) {
+            if (p.h16) {
+                VA_TRY(launch_ivf_h16(s, a, nq, nprobe, p0, b.pair_off, b.item_off, b.sorted_pair, b.bound, kcand,
+                                      reinterpret_cast<float*>(b.tq), b.q8, b.partial, b.partial_cnt, b.gate, st));
+                VA_TRY(launch_ivf_clear_gated(b.gate, nq, nprobe, p0, b.partial_cnt, buckets_dev, b.gpairs,
+                                              kGatedPairsCap, kcand, st));
+                VA_TRY(launch_ivf_rescore(s, a, nq, nprobe, p0, kcand, p.chunks_max, b.partial, b.partial_cnt, b.bound,
+                                          nullptr, st));
+            } else if (p.f32) {
                 VA_TRY(launch_ivf_f32(s, a, nq, nprobe, p0, b.pair_off, b.item_off, b.sorted_pair, b.bound, kcand,
                                       reinterpret_cast<float*>(b.tq), b.partial, b.partial_cnt, b.gate, v.res_term, st));
                 VA_TRY(launch_ivf_clear_gated(b.gate, nq, nprobe, p0, b.partial_cnt, buckets_dev, b.gpairs,

@@ -448,4 +448,306 @@ launch_prefilter_h16(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, ui
     return 0;
 }
 
+// ---- posting lists -----------------------------------------------------------------------------------------------
+// sq8 lists of more than 128 dimensions (no residual): the probe columns behind the first, grouped by list, as in
+// ivf_f32_kernel (prefilter.hip) -- a work item is a chunk of a list's tiles x up to 128 of the pairs that probe it --
+// with this file's contraction: the rows of the query side are fetched through the pair table.
+constexpr uint32_t kIvfH16Pairs = kH16N;
+constexpr uint32_t kIvfH16ChunkTiles = 32;  // as ivf_i8.hip: kIvfI8ChunkTiles, kIvfI8Chunks
+constexpr uint32_t kIvfH16Chunks = 4;
+
+bool
+ivf_h16_supports(const vsag_amd_store* s) {
+    return s->kind == VSAG_AMD_KIND_SQ8 && s->nlist > 0 && s->dpad > 128 && s->pf_term != nullptr && s->pf_ymax != nullptr &&
+           s->ids_dev != nullptr && s->residual_centroids_dev == nullptr;
+}
+uint32_t
+ivf_h16_pairs_per_item() {
+    return kIvfH16Pairs;
+}
+// (one more row than queries: the row of a pair that does not exist is a row of zeros)
+size_t
+ivf_h16_scratch_bytes(const vsag_amd_store* s, uint64_t nq) {
+    return prefilter_h16_scratch_bytes(s, nq + 1);
+}
+
+struct IvfH16Args {
+    const uint4* tiles;
+    uint32_t G;
+    const uint4* planes;
+    const float* factor;
+    uint64_t nq, rows;
+    uint32_t slots;
+    const float* term;
+    float term_factor;
+    const float* tau;
+    const uint32_t* ids;            // per slot; the padding behind a list's last code holds no id and never passes
+    const uint32_t* list_tile;      // per list: first tile, end tile
+    const uint32_t* pair_off;       // pairs of list b: sorted_pair[pair_off[b] .. pair_off[b + 1])
+    const uint32_t* item_off;       // items of list b: item_off[b] .. item_off[b + 1]
+    const uint32_t* sorted_pair;    // query * nprobe + column
+    uint32_t nlist, nprobe;
+    uint32_t k;                     // records per private list
+    uint64_t* partial;
+    uint32_t* partial_cnt;          // zero before the launch; may end above k (overflow: the pair is scanned again)
+    uint32_t* gate;                 // nq + 2 words as in ivf_i8.hip
+};
+
+__global__ void __launch_bounds__(256, 2)
+ivf_h16_kernel(IvfH16Args p) {
+    __shared__ H16Stage stage;
+    __shared__ float code_term[kH16M];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63;
+    const uint32_t wave = tid >> 6;
+    const uint32_t wm = wave & 1;
+    const uint32_t wn = wave >> 1;
+    const uint32_t half = lane >> 5;
+    const uint32_t l32 = lane & 31;
+    const uint32_t item = blockIdx.x;
+    const cu32_p ioff = as_const(p.item_off);
+    if (item >= ioff[p.nlist]) {
+        return;  // the whole workgroup
+    }
+    uint32_t lo_b = 0, hi_b = p.nlist;
+    while (hi_b - lo_b > 1) {
+        const uint32_t mid = (lo_b + hi_b) >> 1;
+        if (ioff[mid] <= item) {
+            lo_b = mid;
+        } else {
+            hi_b = mid;
+        }
+    }
+    const uint32_t b = lo_b;
+    const uint32_t list_begin = as_const(p.list_tile)[2 * b], list_end = as_const(p.list_tile)[2 * b + 1];
+    uint32_t chunks = (list_end - list_begin + kIvfH16ChunkTiles - 1) / kIvfH16ChunkTiles;
+    chunks = chunks < kIvfH16Chunks ? chunks : kIvfH16Chunks;
+    if (chunks == 0) {
+        return;
+    }
+    const uint32_t per = (list_end - list_begin + chunks - 1) / chunks;
+    const uint32_t chunk = (item - ioff[b]) % chunks;
+    const uint32_t group = (item - ioff[b]) / chunks;
+    uint32_t tile_begin = list_begin + chunk * per;
+    tile_begin = tile_begin < list_end ? tile_begin : list_end;
+    const uint32_t tile_end = tile_begin + per < list_end ? tile_begin + per : list_end;
+    const uint32_t pbeg = as_const(p.pair_off)[b] + group * kIvfH16Pairs;
+    const uint32_t pend = as_const(p.pair_off)[b + 1];
+    const uint32_t mtiles = (tile_end - tile_begin + 3) / 4;
+    if (mtiles == 0 || pbeg >= pend) {
+        return;
+    }
+    const uint32_t stages = p.slots / kH16Slots;
+
+    // The query rows of this item: thread t stages row t % 128 (slots t / 128 + 2 r), the query of pair pbeg + t % 128.
+    uint64_t qsrc;
+    {
+        const uint32_t at = pbeg + (tid & 127);
+        qsrc = at < pend ? as_const(p.sorted_pair)[at] / p.nprobe : p.nq;  // p.nq: no such pair, a row of zeros
+    }
+    float tau_n[2], fac_n[2];
+    uint32_t pair_n[2], query_n[2];
+    bool live[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint32_t at = pbeg + wn * 64 + j * 32 + l32;
+        live[j] = at < pend;
+        pair_n[j] = live[j] ? as_const(p.sorted_pair)[at] : 0U;
+        query_n[j] = pair_n[j] / p.nprobe;
+        tau_n[j] = live[j] ? p.tau[query_n[j]] : -__builtin_inff();
+        fac_n[j] = live[j] ? p.factor[query_n[j]] : 0.0F;
+    }
+
+    auto code_granule = [&](uint32_t mt, uint32_t j) __attribute__((always_inline)) {
+        const uint32_t tile = tile_begin + 4 * mt + (tid >> 6);
+        if (tile < tile_end && j < p.G) {
+            return p.tiles[(static_cast<uint64_t>(tile) * p.G + j) * kWave + (tid & 63)];
+        }
+        return make_uint4(0, 0, 0, 0);
+    };
+    uint4 rc0, rc1, rc2, rc3, rq0, rq1, rq2, rq3;
+    auto query_slot = [&](uint32_t st, uint32_t r) __attribute__((always_inline)) {
+        const uint32_t slot = (tid >> 7) + 2 * r;
+        return p.planes[(static_cast<uint64_t>(st) * kH16Slots + slot) * p.rows + qsrc];
+    };
+    auto fetch = [&](uint32_t mt, uint32_t st) __attribute__((always_inline)) {
+        rc0 = code_granule(mt, 4 * st);
+        rc1 = code_granule(mt, 4 * st + 1);
+        rc2 = code_granule(mt, 4 * st + 2);
+        rc3 = code_granule(mt, 4 * st + 3);
+        rq0 = query_slot(st, 0);
+        rq1 = query_slot(st, 1);
+        rq2 = query_slot(st, 2);
+        rq3 = query_slot(st, 3);
+    };
+    auto park_codes = [&](uint32_t g, uint4 v) __attribute__((always_inline)) {
+        uint4 lo8, hi8;
+        h16_bytes_to_halves(v, &lo8, &hi8);
+        stage.a[2 * g][tid] = lo8;
+        stage.a[2 * g + 1][tid] = hi8;
+    };
+    auto park = [&]() __attribute__((always_inline)) {
+        park_codes(0, rc0);
+        park_codes(1, rc1);
+        park_codes(2, rc2);
+        park_codes(3, rc3);
+        stage.b[(tid >> 7) + 0][tid & 127] = rq0;
+        stage.b[(tid >> 7) + 2][tid & 127] = rq1;
+        stage.b[(tid >> 7) + 4][tid & 127] = rq2;
+        stage.b[(tid >> 7) + 6][tid & 127] = rq3;
+    };
+
+    fetch(0, 0);
+    for (uint32_t mt = 0; mt < mtiles; ++mt) {
+        floatx16 acc[4][2];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    acc[i][j][e] = 0.0F;
+                }
+            }
+        }
+        const uint64_t slot0 = (static_cast<uint64_t>(tile_begin) + 4 * mt) * kWave;
+        park();
+        float my_term;
+        {
+            // (a padding slot is all zeros: under inner product that is a good distance)
+            const bool real = tile_begin + 4 * mt + (tid >> 6) < tile_end && p.ids[slot0 + tid] != VSAG_AMD_INVALID_ID;
+            my_term = real ? p.term_factor * p.term[slot0 + tid] : __builtin_inff();
+        }
+        __syncthreads();
+        for (uint32_t st = 0; st < stages; ++st) {
+            if (st + 1 < stages) {
+                fetch(mt, st + 1);
+            } else if (mt + 1 < mtiles) {
+                fetch(mt + 1, 0);
+            }
+#pragma unroll 2
+            for (uint32_t ks = 0; ks < kH16Stage / 16; ++ks) {
+                const uint32_t slot = 2 * ks + half;
+                halfx8 a[4], bq[2];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    a[i] = __builtin_bit_cast(halfx8, stage.a[slot][wm * 128 + i * 32 + l32]);
+                }
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    bq[j] = __builtin_bit_cast(halfx8, stage.b[slot][wn * 64 + j * 32 + l32]);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], bq[j], acc[i][j], 0, 0, 0);
+                    }
+                }
+            }
+            if (st + 1 == stages) {
+                code_term[tid] = my_term;
+            }
+            __syncthreads();
+            if (st + 1 < stages) {
+                park();
+                __syncthreads();
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            uint64_t hits = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const uint32_t ml = wm * 128 + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+                    const float v = code_term[ml] + fac_n[j] * acc[i][j][e];
+                    hits |= static_cast<uint64_t>(v <= tau_n[j] ? 1U : 0U) << (16 * i + e);
+                }
+            }
+            if (hits != 0 && live[j]) {
+                const uint64_t list = (static_cast<uint64_t>(pair_n[j]) * kIvfH16Chunks + chunk) * 2 + wm;
+                while (hits != 0) {
+                    const uint32_t bit = static_cast<uint32_t>(__builtin_ctzll(hits));
+                    hits &= hits - 1;
+                    const uint32_t i = bit >> 4, e = bit & 15;
+                    const uint32_t ml = wm * 128 + i * 32 + 8 * (e >> 2) + 4 * half + (e & 3);
+                    const uint32_t pos = atomicAdd(&p.partial_cnt[list], 1U);
+                    if (pos < p.k) {
+                        p.partial[list * p.k + pos] = slot0 + ml;
+                    } else if (pos == p.k) {
+                        if (atomicExch(&p.gate[query_n[j]], 1U) == 0U) {
+                            atomicAdd(&p.gate[p.nq], 1U);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Thresholds and fp16 query values from the bounds (tau: nq floats; scratch: ivf_h16_scratch_bytes), then the
+// candidates of probe columns [p0, nprobe) grouped by list (pair_off, sorted_pair; item_off counted with
+// ivf_h16_pairs_per_item() pairs per item) into the private lists (pair * 8 + chunk * 2 + half of the code tile) of
+// kcand records in `partial`; partial_cnt zero before.  gate: nq + 2 words.
+int
+launch_ivf_h16(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t nprobe, uint32_t p0, const uint32_t* pair_off,
+               const uint32_t* item_off, const uint32_t* sorted_pair, const uint32_t* bound, uint32_t kcand, float* tau,
+               uint8_t* scratch, uint64_t* partial, uint32_t* partial_cnt, uint32_t* gate, hipStream_t st) {
+    const bool l2 = s->metric == VSAG_AMD_METRIC_L2;
+    const uint64_t rows = h16_query_rows(nq + 1);
+    const uint32_t slots = h16_slots_per_row(s);
+    uint4* planes = reinterpret_cast<uint4*>(scratch);
+    float* factor = reinterpret_cast<float*>(scratch + static_cast<size_t>(slots) * rows * 16);
+    H16SplitArgs sp{};
+    sp.qtab = reinterpret_cast<const float*>(a.qtab);
+    sp.qstride = a.qstride;
+    sp.kdim = s->dpad;
+    sp.scale = l2 ? s->scale_dev : nullptr;
+    sp.nq = nq;
+    sp.rows = rows;
+    sp.slots = slots;
+    sp.planes = planes;
+    sp.factor = factor;
+    sp.tau = tau;
+    sp.dot_factor = l2 ? -2.0F : -1.0F;
+    sp.is_l2 = l2 ? 1 : 0;
+    sp.qmeta = l2 ? nullptr : a.qmeta;
+    sp.qmeta_stride = a.qmeta_stride;
+    sp.bound = bound;
+    sp.ymax_bits = s->pf_ymax;
+    hipLaunchKernelGGL(h16_split_kernel, dim3(static_cast<uint32_t>(rows)), dim3(kWave), 0, st, sp);
+    IvfH16Args p{};
+    p.tiles = s->tiles;
+    p.G = s->G;
+    p.planes = planes;
+    p.factor = factor;
+    p.nq = nq;
+    p.rows = rows;
+    p.slots = slots;
+    p.term = s->pf_term;
+    p.term_factor = l2 ? 1.0F : 0.0F;
+    p.tau = tau;
+    p.ids = s->ids_dev;
+    p.list_tile = s->list_tile_dev;
+    p.pair_off = pair_off;
+    p.item_off = item_off;
+    p.sorted_pair = sorted_pair;
+    p.nlist = s->nlist;
+    p.nprobe = nprobe;
+    p.k = kcand;
+    p.partial = partial;
+    p.partial_cnt = partial_cnt;
+    p.gate = gate;
+    const uint64_t pairs = nq * (nprobe - p0);
+    const uint64_t max_items =
+        (div_up(pairs, static_cast<uint64_t>(kIvfH16Pairs)) + std::min<uint64_t>(s->nlist, pairs)) * kIvfH16Chunks;
+    timing_begin(st);
+    hipLaunchKernelGGL(ivf_h16_kernel, dim3(static_cast<uint32_t>(max_items)), dim3(256), 0, st, p);
+    timing_end(st);
+    VA_HIP(hipGetLastError());
+    return 0;
+}
+
 }  // namespace vsag_amd
