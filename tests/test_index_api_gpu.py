@@ -507,6 +507,31 @@ def test_large_batch_equals_one_by_one(lib, quant):
     idx.close()
 
 
+@pytest.mark.parametrize("name,metric", [("brute_force", "l2"), ("brute_force", "cosine"), ("ivf", "l2"), ("ivf", "ip")])
+def test_sq8_beyond_128_dimensions_large_batch_equals_one_by_one(lib, name, metric):
+    """sq8 codes of 200 dimensions: a batch large enough for the fp16 matrix cores (flat store: prefilter_h16_kernel,
+    posting lists: ivf_h16_kernel) returns what single queries (streaming scan) return, ids and distance bits."""
+    n, d, k = 70000, 200, 10
+    nq = 600 if name == "brute_force" else 2200
+    x = vectors(n, d, normalize=False)
+    q = vectors(nq, d, seed=165, normalize=False)
+    labels = np.arange(n, dtype=np.int64) * 3 + 2
+    params = dict(base_quantization_type="sq8")
+    search = "{}"
+    if name == "ivf":
+        params.update(buckets_count=64, train_sample_count=20000)
+        search = json.dumps({"ivf": {"scan_buckets_count": 16}})
+    idx = make(name, d, metric, **params)
+    assert idx.build(x, labels, n, d) == 0
+    ids, dists = idx.knn_search_batch(q, k, search)
+    for i in range(0, nq, 53):
+        si, sd = idx.knn_search(q[i], k, search)
+        assert np.array_equal(si, ids[i]) and np.array_equal(sd.view(np.uint32), dists[i].view(np.uint32)), i
+    gt, _ = ground_truth(x, q[:40], k, metric)
+    assert recall(ids[:40], gt, labels) >= (0.95 if name == "brute_force" else 0.3)  # (16 of 64 lists of unclustered rows)
+    idx.close()
+
+
 def test_ivf_with_a_thousand_buckets_routes_large_batches_through_the_table(lib):
     """1024 buckets: Add classifies 65 536 rows a call and a search batch of 1100 queries routes through the table of
     approximate centroid distances; both must give what single queries give (exact routing either way)."""
