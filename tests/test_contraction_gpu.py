@@ -92,6 +92,41 @@ def test_sq8_beyond_128_dimensions_on_the_fp16_matrix_cores(lib, modes, metric, 
 
 
 @pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
+@pytest.mark.parametrize("n,d,nq,k", [(30000, 160, 600, 10), (12000, 960, 512, 10), (9000, 1000, 130, 100)])
+def test_sq4_beyond_128_dimensions_on_the_fp16_matrix_cores(lib, modes, metric, n, d, nq, k):
+    """sq4 stores of more than 128 dimensions take the fp16 pass as well (the nibbles are exact in fp16), in mode 2 too:
+    sq4 has no route on the fp32 matrix cores."""
+    rng = np.random.default_rng(n + d + k + metric)
+    x, means = gaussian_mixture(rng, n, d, 20, 0.05)
+    q, _ = gaussian_mixture(rng, nq, d, 20, 0.05, means=means)
+    if metric != orc.COSINE:
+        q[0] = 0.0
+        q[1] = 1e-20
+        q[6] = np.nan
+    q[2] *= 1e6
+    q[3] *= 1e-6
+    q[4] = 0.0
+    q[4, d // 2] = 1e4
+    q[8:40] = x[8:40]
+    q[60:80] += 100.0
+    lb, diff = orc.sq_train(x, 4, metric)
+    codes = orc.sq_encode(x, 4, lb, diff, metric)
+    st = Store(capi.KIND_SQ4, metric, d, lb=lb, diff=diff)
+    st.append(codes[:n // 2])
+    st.append(codes[n // 2:])
+    for mode in (1, 2):
+        plain, fast, tile = modes(st, q, k, mode)
+        assert tile == 128, "the contraction path did not run"
+        assert same(plain, fast)
+    qs, om = q[8:24], metric
+    if metric == orc.COSINE:  # inner product of the unit query with the codes of the unit rows
+        qs, om = (qs / np.linalg.norm(qs, axis=1, keepdims=True)).astype(np.float32), orc.IP
+    ri, rd = orc.flat_scan_topk(orc.SQ4, om, d, codes, qs, k, lb=lb, diff=diff)
+    assert_topk_close(fast[0][8:24], fast[1][8:24], ri, rd, label="sq4 beyond 128 dimensions")
+    st.destroy()
+
+
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
 @pytest.mark.parametrize("d", [16, 100, 128])
 def test_sq8_int8_planes_hold_for_awkward_queries(lib, modes, metric, d):
     """Queries the two int8 planes represent badly or trivially: one dominant dimension, tiny and huge magnitudes,

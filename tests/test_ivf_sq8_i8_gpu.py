@@ -159,3 +159,26 @@ def test_one_long_list_among_short_and_empty_ones(lib, bits):
     plain, fast = _both(lib, st, q, buckets, kcand)
     assert _same(plain, fast)
     st.destroy()
+
+
+@pytest.mark.parametrize("metric", [orc.L2, orc.IP, orc.COSINE])
+@pytest.mark.parametrize("n,d,nlist,nq,nprobe,kcand", [(20000, 200, 20, 7000, 6, 10), (12000, 960, 16, 9000, 4, 32)])
+def test_sq4_lists_beyond_128_dimensions_on_the_fp16_matrix_cores(lib, metric, n, d, nlist, nq, nprobe, kcand):
+    """sq4 posting lists of more than 128 dimensions: the nibbles and the fp16 value of the scaled query on
+    v_mfma_f32_32x32x16_f16 (ivf_h16_kernel), records rescored with the streaming arithmetic: ids and distance bits equal
+    the streaming scan's."""
+    x, q, cent, labels, codes, (lb, diff), st = _case(n + d + metric, n, d, nlist, nq, metric=metric, bits=4)
+    buckets, _ = orc.ivf_route(cent, q, nprobe)
+    buckets = buckets.copy()
+    buckets[70:73, 0] = -1
+    buckets[80, 0] = buckets[80, nprobe - 1]
+    plain, fast = _both(lib, st, q, buckets, kcand)
+    assert _same(plain, fast)
+    offsets, order = orc.ivf_build_lists(labels, nlist)
+    qs, om = q[:32], metric
+    if metric == orc.COSINE:
+        qs, om = (qs / np.linalg.norm(qs, axis=1, keepdims=True)).astype(np.float32), orc.IP
+    rids, rds = orc.ivf_scan(orc.SQ4, om, d, codes[order], offsets, order, qs, buckets[:32], kcand, lb=lb, diff=diff)
+    assert_topk_close(fast[0][:32], fast[1][:32], rids, rds, rtol=2e-5, atol=1e-5, tie_rtol=2e-5,
+                      label="ivf sq4 beyond 128 dimensions on the matrix cores")
+    st.destroy()

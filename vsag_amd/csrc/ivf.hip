@@ -996,7 +996,8 @@ plan_ivf(const vsag_amd_store* s, uint64_t nq, uint32_t nprobe, uint32_t kcand, 
             npairs * ivf_i8_lists_per_pair() * kcand * 8 <= (8ull << 30);
     // sq8 lists of more than 128 dimensions: the fp16 matrix cores (mode 2 keeps the fp32 ones; residual lists too).
     p->h16 = !p->mfma && !p->planes && !p->bits1 && !p->pq && !p->chunked && nprobe > 1 && scan_contraction_mode(s) >= 0 &&
-             scan_contraction_mode(s) != 2 && ivf_h16_supports(s) && kcand <= ivf_rescore_capacity() &&
+             (scan_contraction_mode(s) != 2 || s->kind == VSAG_AMD_KIND_SQ4) && ivf_h16_supports(s) &&
+             kcand <= ivf_rescore_capacity() &&
              npairs * ivf_i8_lists_per_pair() * kcand * 8 <= (8ull << 30);
     // fp32 lists, sq8 lists the fp16 pass does not take: the fp32 matrix cores pre-select, the same exact rescoring.
     p->f32 = !p->h16 && !p->mfma && !p->planes && !p->bits1 && !p->pq && !p->chunked && nprobe > 1 && scan_contraction_mode(s) >= 0 &&

@@ -1157,7 +1157,10 @@ prefilter_supports(const vsag_amd_store* s) {
     if (prefilter_rb_supports(s)) {
         return true;
     }
-    if (s->kind == VSAG_AMD_KIND_SQ8_UNIFORM || s->kind == VSAG_AMD_KIND_SQ4_UNIFORM || s->kind == VSAG_AMD_KIND_SQ4) {
+    if (s->kind == VSAG_AMD_KIND_SQ4) {
+        return prefilter_i8_supports(s) || prefilter_h16_supports(s);  // int8 up to 128 dimensions, fp16 beyond
+    }
+    if (s->kind == VSAG_AMD_KIND_SQ8_UNIFORM || s->kind == VSAG_AMD_KIND_SQ4_UNIFORM) {
         return prefilter_i8_supports(s);  // the int8 matrix cores or nothing
     }
     return s->nlist == 0 && (s->kind == VSAG_AMD_KIND_FP32 || s->kind == VSAG_AMD_KIND_SQ8) && s->pf_term != nullptr;

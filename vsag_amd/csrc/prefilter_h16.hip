@@ -40,7 +40,8 @@ constexpr uint32_t kH16Slots = kH16Stage / 8;
 
 bool
 prefilter_h16_supports(const vsag_amd_store* s) {
-    return s->kind == VSAG_AMD_KIND_SQ8 && s->nlist == 0 && s->dpad > 128 && s->pf_term != nullptr && s->pf_ymax != nullptr;
+    return (s->kind == VSAG_AMD_KIND_SQ8 || s->kind == VSAG_AMD_KIND_SQ4) && s->nlist == 0 && s->dpad > 128 &&
+           s->pf_term != nullptr && s->pf_ymax != nullptr;
 }
 
 static uint64_t
@@ -70,6 +71,7 @@ struct H16SplitArgs {
     float* factor;       // per query: dot_factor * 2^-E
     float* tau;          // per query: keep a pair when term_factor |y|^2 + factor <hi, c> <= tau
     float dot_factor;
+    float cmax;          // largest code value: 255 (sq8) or 15 (sq4)
     int is_l2;
     const float* qmeta;  // ip: sum q_d lb_d per query
     uint32_t qmeta_stride;
@@ -170,14 +172,14 @@ h16_split_kernel(H16SplitArgs p) {
         // dist = 1 - (fl(sum c a) + qmeta): the fp32 sum is off by at most n u sum |c a|, the two closing operations by u
         // of their results; twice that is allowed for.
         const double qm = p.qmeta != nullptr ? static_cast<double>(p.qmeta[q * p.qmeta_stride]) : 0.0;
-        const double m = fmin(255.0 * a1, dots);
+        const double m = fmin(static_cast<double>(p.cmax) * a1, dots);
         const double e_stream = 2.0 * (p.kdim + 2) * kU * m + 4.0 * kU * (m + fabs(qm) + 1.0 + fabs(bd));
         t = bd - 1.0 + qm + e_stream;
     }
-    // every code value lies in [0, 255]: what the fp16 value misses of b_d, and two roundings of the running absolute
+    // every code value lies in [0, cmax]: what the fp16 value misses of b_d, and two roundings of the running absolute
     // sum per matrix instruction (sixteen dimensions each) plus four for the closing operations
     const double roundings = 2.0 * (p.kdim / 16.0 + 4.0) * kU;
-    const double extra = fabs(static_cast<double>(p.dot_factor)) * 255.0 * (miss + roundings * sum_abs);
+    const double extra = fabs(static_cast<double>(p.dot_factor)) * static_cast<double>(p.cmax) * (miss + roundings * sum_abs);
     // the test itself: fl(term + fl(factor acc)) against the threshold rounded to fp32
     const double e_test = 4.0 * kU * (ymax * ymax + 2.0 * dots + fabs(t) + extra);
     t += extra + e_test;
@@ -226,8 +228,25 @@ h16_bytes_to_halves(uint4 g, uint4* lo8, uint4* hi8) {
     *hi8 = make_uint4(h16_two_bytes(g.z, kLow), h16_two_bytes(g.z, kHigh), h16_two_bytes(g.w, kLow), h16_two_bytes(g.w, kHigh));
 }
 
+// An sq4 granule (32 dimensions: byte b holds dimension 2 b in its low and 2 b + 1 in its high nibble) as 32 fp16
+// values: word w of the granule is the slot of dimensions 8 w .. 8 w + 7.
+__device__ inline uint4
+h16_nibbles_to_halves(uint32_t w) {
+    const uint32_t lo = w & 0x0F0F0F0FU, hi = (w >> 4) & 0x0F0F0F0FU;
+    const halfx2 bias = halfx2{static_cast<_Float16>(1024.0F), static_cast<_Float16>(1024.0F)};
+    uint32_t out[4];
+#pragma unroll
+    for (uint32_t b = 0; b < 4; ++b) {
+        // (low nibble of byte b, zero, high nibble of byte b, zero) under 0x64 in the high bytes
+        const uint32_t pair = __builtin_amdgcn_perm(hi, lo, 0x0c040c00U + b * 0x00010001U) | 0x64006400U;
+        out[b] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(halfx2, pair) - bias);
+    }
+    return make_uint4(out[0], out[1], out[2], out[3]);
+}
+
 // A workgroup: 256 codes (four storage tiles) x 128 queries, a wave 128 codes x 64 queries (4 x 2 blocks of 32 x 32):
 // 48 KiB of operands per stage from L2 for 2 M multiply-adds, 6 LDS reads per 8 matrix instructions.
+template <int KIND>
 __global__ void __launch_bounds__(256, 2)
 prefilter_h16_kernel(PrefilterH16Args p) {
     __shared__ H16Stage stage;
@@ -269,10 +288,15 @@ prefilter_h16_kernel(PrefilterH16Args p) {
         return p.planes[(static_cast<uint64_t>(st) * kH16Slots + slot) * p.rows + q0 + row];
     };
     auto fetch = [&](uint64_t mt, uint32_t st) __attribute__((always_inline)) {
-        rc0 = code_granule(mt, 4 * st);
-        rc1 = code_granule(mt, 4 * st + 1);
-        rc2 = code_granule(mt, 4 * st + 2);
-        rc3 = code_granule(mt, 4 * st + 3);
+        if constexpr (KIND == VSAG_AMD_KIND_SQ4) {
+            rc0 = code_granule(mt, 2 * st);
+            rc1 = code_granule(mt, 2 * st + 1);
+        } else {
+            rc0 = code_granule(mt, 4 * st);
+            rc1 = code_granule(mt, 4 * st + 1);
+            rc2 = code_granule(mt, 4 * st + 2);
+            rc3 = code_granule(mt, 4 * st + 3);
+        }
         rq0 = query_slot(st, 0);
         rq1 = query_slot(st, 1);
         rq2 = query_slot(st, 2);
@@ -289,10 +313,21 @@ prefilter_h16_kernel(PrefilterH16Args p) {
         stage.b[idx >> 7][idx & 127] = v;
     };
     auto park = [&]() __attribute__((always_inline)) {
-        park_codes(0, rc0);
-        park_codes(1, rc1);
-        park_codes(2, rc2);
-        park_codes(3, rc3);
+        if constexpr (KIND == VSAG_AMD_KIND_SQ4) {
+            stage.a[0][tid] = h16_nibbles_to_halves(rc0.x);
+            stage.a[1][tid] = h16_nibbles_to_halves(rc0.y);
+            stage.a[2][tid] = h16_nibbles_to_halves(rc0.z);
+            stage.a[3][tid] = h16_nibbles_to_halves(rc0.w);
+            stage.a[4][tid] = h16_nibbles_to_halves(rc1.x);
+            stage.a[5][tid] = h16_nibbles_to_halves(rc1.y);
+            stage.a[6][tid] = h16_nibbles_to_halves(rc1.z);
+            stage.a[7][tid] = h16_nibbles_to_halves(rc1.w);
+        } else {
+            park_codes(0, rc0);
+            park_codes(1, rc1);
+            park_codes(2, rc2);
+            park_codes(3, rc3);
+        }
         park_query(0, rq0);
         park_query(1, rq1);
         park_query(2, rq2);
@@ -411,6 +446,7 @@ launch_prefilter_h16(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, ui
     sp.factor = factor;
     sp.tau = tau;
     sp.dot_factor = l2 ? -2.0F : -1.0F;
+    sp.cmax = s->kind == VSAG_AMD_KIND_SQ4 ? 15.0F : 255.0F;
     sp.is_l2 = l2 ? 1 : 0;
     sp.qmeta = l2 ? nullptr : a.qmeta;
     sp.qmeta_stride = a.qmeta_stride;
@@ -442,7 +478,13 @@ launch_prefilter_h16(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, ui
     groups = std::max<uint64_t>(1, std::min<uint64_t>(groups, mtiles));
     p.groups = static_cast<uint32_t>(groups);
     timing_begin(st);
-    hipLaunchKernelGGL(prefilter_h16_kernel, dim3(p.groups, static_cast<uint32_t>(qtiles)), dim3(256), 0, st, p);
+    if (s->kind == VSAG_AMD_KIND_SQ4) {
+        hipLaunchKernelGGL(prefilter_h16_kernel<VSAG_AMD_KIND_SQ4>, dim3(p.groups, static_cast<uint32_t>(qtiles)), dim3(256), 0,
+                           st, p);
+    } else {
+        hipLaunchKernelGGL(prefilter_h16_kernel<VSAG_AMD_KIND_SQ8>, dim3(p.groups, static_cast<uint32_t>(qtiles)), dim3(256), 0,
+                           st, p);
+    }
     timing_end(st);
     VA_HIP(hipGetLastError());
     return 0;
@@ -458,7 +500,8 @@ constexpr uint32_t kIvfH16Chunks = 4;
 
 bool
 ivf_h16_supports(const vsag_amd_store* s) {
-    return s->kind == VSAG_AMD_KIND_SQ8 && s->nlist > 0 && s->dpad > 128 && s->pf_term != nullptr && s->pf_ymax != nullptr &&
+    return (s->kind == VSAG_AMD_KIND_SQ8 || s->kind == VSAG_AMD_KIND_SQ4) && s->nlist > 0 && s->dpad > 128 &&
+           s->pf_term != nullptr && s->pf_ymax != nullptr &&
            s->ids_dev != nullptr && s->residual_centroids_dev == nullptr;
 }
 uint32_t
@@ -493,6 +536,7 @@ struct IvfH16Args {
     uint32_t* gate;                 // nq + 2 words as in ivf_i8.hip
 };
 
+template <int KIND>
 __global__ void __launch_bounds__(256, 2)
 ivf_h16_kernel(IvfH16Args p) {
     __shared__ H16Stage stage;
@@ -571,10 +615,15 @@ ivf_h16_kernel(IvfH16Args p) {
         return p.planes[(static_cast<uint64_t>(st) * kH16Slots + slot) * p.rows + qsrc];
     };
     auto fetch = [&](uint32_t mt, uint32_t st) __attribute__((always_inline)) {
-        rc0 = code_granule(mt, 4 * st);
-        rc1 = code_granule(mt, 4 * st + 1);
-        rc2 = code_granule(mt, 4 * st + 2);
-        rc3 = code_granule(mt, 4 * st + 3);
+        if constexpr (KIND == VSAG_AMD_KIND_SQ4) {
+            rc0 = code_granule(mt, 2 * st);
+            rc1 = code_granule(mt, 2 * st + 1);
+        } else {
+            rc0 = code_granule(mt, 4 * st);
+            rc1 = code_granule(mt, 4 * st + 1);
+            rc2 = code_granule(mt, 4 * st + 2);
+            rc3 = code_granule(mt, 4 * st + 3);
+        }
         rq0 = query_slot(st, 0);
         rq1 = query_slot(st, 1);
         rq2 = query_slot(st, 2);
@@ -587,10 +636,21 @@ ivf_h16_kernel(IvfH16Args p) {
         stage.a[2 * g + 1][tid] = hi8;
     };
     auto park = [&]() __attribute__((always_inline)) {
-        park_codes(0, rc0);
-        park_codes(1, rc1);
-        park_codes(2, rc2);
-        park_codes(3, rc3);
+        if constexpr (KIND == VSAG_AMD_KIND_SQ4) {
+            stage.a[0][tid] = h16_nibbles_to_halves(rc0.x);
+            stage.a[1][tid] = h16_nibbles_to_halves(rc0.y);
+            stage.a[2][tid] = h16_nibbles_to_halves(rc0.z);
+            stage.a[3][tid] = h16_nibbles_to_halves(rc0.w);
+            stage.a[4][tid] = h16_nibbles_to_halves(rc1.x);
+            stage.a[5][tid] = h16_nibbles_to_halves(rc1.y);
+            stage.a[6][tid] = h16_nibbles_to_halves(rc1.z);
+            stage.a[7][tid] = h16_nibbles_to_halves(rc1.w);
+        } else {
+            park_codes(0, rc0);
+            park_codes(1, rc1);
+            park_codes(2, rc2);
+            park_codes(3, rc3);
+        }
         stage.b[(tid >> 7) + 0][tid & 127] = rq0;
         stage.b[(tid >> 7) + 2][tid & 127] = rq1;
         stage.b[(tid >> 7) + 4][tid & 127] = rq2;
@@ -712,6 +772,7 @@ launch_ivf_h16(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t
     sp.factor = factor;
     sp.tau = tau;
     sp.dot_factor = l2 ? -2.0F : -1.0F;
+    sp.cmax = s->kind == VSAG_AMD_KIND_SQ4 ? 15.0F : 255.0F;
     sp.is_l2 = l2 ? 1 : 0;
     sp.qmeta = l2 ? nullptr : a.qmeta;
     sp.qmeta_stride = a.qmeta_stride;
@@ -744,7 +805,11 @@ launch_ivf_h16(const vsag_amd_store* s, const ScanArgs& a, uint64_t nq, uint32_t
     const uint64_t max_items =
         (div_up(pairs, static_cast<uint64_t>(kIvfH16Pairs)) + std::min<uint64_t>(s->nlist, pairs)) * kIvfH16Chunks;
     timing_begin(st);
-    hipLaunchKernelGGL(ivf_h16_kernel, dim3(static_cast<uint32_t>(max_items)), dim3(256), 0, st, p);
+    if (s->kind == VSAG_AMD_KIND_SQ4) {
+        hipLaunchKernelGGL(ivf_h16_kernel<VSAG_AMD_KIND_SQ4>, dim3(static_cast<uint32_t>(max_items)), dim3(256), 0, st, p);
+    } else {
+        hipLaunchKernelGGL(ivf_h16_kernel<VSAG_AMD_KIND_SQ8>, dim3(static_cast<uint32_t>(max_items)), dim3(256), 0, st, p);
+    }
     timing_end(st);
     VA_HIP(hipGetLastError());
     return 0;

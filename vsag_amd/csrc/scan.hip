@@ -912,7 +912,8 @@ make_call_plan(const vsag_amd_store* s, uint64_t nq, uint32_t k, CallPlan* c) {
         r = std::min<uint64_t>(r, 6);
     }
     // (The fp16 pass of sq8 stores beyond 128 dimensions is ten times the streaming kernel: a short prefix there too.)
-    const bool h16 = !i8 && !rb && prefilter_mode(s) != 2 && prefilter_h16_supports(s);
+    // (Mode 2 asks for the fp32 matrix cores, which sq4 has no route for.)
+    const bool h16 = !i8 && !rb && (prefilter_mode(s) != 2 || s->kind == VSAG_AMD_KIND_SQ4) && prefilter_h16_supports(s);
     const uint64_t min_prefix = forced ? 2 : (i8 || h16 ? std::max<uint64_t>(8, div_up(4ull * k, kWave)) : 64);
     uint64_t bounds[CallPlan::kMaxLevels + 1];
     int nb = 0;

@@ -691,9 +691,8 @@ vsag_amd_store_create(const vsag_amd_store_params_t* p, vsag_amd_store_t** out) 
         }
     }
     // Stores the matrix cores can pre-select on keep a per-code term (and the largest norm, where a threshold needs it).
-    if (p->kind == VSAG_AMD_KIND_FP32 || p->kind == VSAG_AMD_KIND_SQ8 ||
-        ((p->kind == VSAG_AMD_KIND_SQ8_UNIFORM || p->kind == VSAG_AMD_KIND_SQ4_UNIFORM || p->kind == VSAG_AMD_KIND_SQ4) &&
-         s->dpad <= 128)) {
+    if (p->kind == VSAG_AMD_KIND_FP32 || p->kind == VSAG_AMD_KIND_SQ8 || p->kind == VSAG_AMD_KIND_SQ4 ||
+        ((p->kind == VSAG_AMD_KIND_SQ8_UNIFORM || p->kind == VSAG_AMD_KIND_SQ4_UNIFORM) && s->dpad <= 128)) {
         if (hipMalloc(&s->pf_ymax, 4) != hipSuccess || hipMemset(s->pf_ymax, 0, 4) != hipSuccess) {
             return fail_free(fail(VSAG_AMD_NO_ENOUGH_MEMORY, "hipMalloc of the norm scalar failed"));
         }
@@ -1006,8 +1005,7 @@ append_to_lists(vsag_amd_store* s, const uint8_t* codes_dev, const int32_t* labe
     // The per-slot terms of the matrix-core passes over sq8 / sq4 lists (prefilter_i8.hip) and over fp32 and longer sq8
     // lists (prefilter.hip): recomputed over the whole buffer, which costs a pass over the codes (0.4 ms for ten million
     // sq8 codes) against the classification and encoding an append has behind it already.
-    const bool list_terms = s->kind == VSAG_AMD_KIND_FP32 || s->kind == VSAG_AMD_KIND_SQ8 ||
-                            (s->kind == VSAG_AMD_KIND_SQ4 && s->dpad <= 128);
+    const bool list_terms = s->kind == VSAG_AMD_KIND_FP32 || s->kind == VSAG_AMD_KIND_SQ8 || s->kind == VSAG_AMD_KIND_SQ4;
     // (Residual lists: fp32 and sq8 under l2 / inner product go through the fp32 matrix cores, the int8 passes do not take
     // them.)
     const bool residual_ok = s->residual_centroids_dev == nullptr ||
