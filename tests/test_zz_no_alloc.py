@@ -22,7 +22,7 @@ def memory_marks(lib, reset):
     return free.value, high.value
 
 
-def noalloc_scan(lib, store, queries, k, opt=None):
+def noalloc_scan(lib, store, queries, k, opt=None, count_memory=True):
     q = np.ascontiguousarray(queries, np.float32)
     nq = q.shape[0]
     qb = dev(q)
@@ -40,7 +40,8 @@ def noalloc_scan(lib, store, queries, k, opt=None):
     capi.synchronize()
     free2, high2 = memory_marks(lib, False)
     assert (high1, high2) == (0, 0), "the stream-ordered allocator was used: %d / %d bytes" % (high1, high2)
-    assert free1 >= free0 and free2 >= free0, "device memory was taken: %d -> %d -> %d" % (free0, free1, free2)
+    if count_memory:
+        assert free1 >= free0 and free2 >= free0, "device memory was taken: %d -> %d -> %d" % (free0, free1, free2)
     out = ids.to_numpy(np.uint32, (nq, k)), ds.to_numpy(np.float32, (nq, k))
     for b in (qb, ids, ds):
         b.free()
@@ -63,8 +64,13 @@ def test_noalloc_flat_scan_equals_workspace_scan(lib):
     store.append(codes)
     q1, _ = gaussian_mixture(rng, 96, d, 50, 0.05, means=means)
     q2, _ = gaussian_mixture(rng, 5, d, 50, 0.05, means=means)
+    # The first launch of a kernel in a process lets the HIP runtime take memory of its own (2 MiB here: kernel objects,
+    # kernel-argument pools), whoever launches it: one call before the free bytes are counted, as a caller that cannot
+    # allocate makes one before it starts capturing or serving.  (The stream-ordered allocator is watched even here.)
+    a0 = noalloc_scan(l, store, q1, k, count_memory=False)
     # two calls in a row on the shared array, the second with a smaller input (and another k)
     a1 = noalloc_scan(l, store, q1, k)
+    assert same(a0, a1)
     a2 = noalloc_scan(l, store, q2, 7)
     assert same(a1, store.flat_scan(q1, k))
     assert same(a2, store.flat_scan(q2, 7))
@@ -116,6 +122,7 @@ def test_noalloc_rabitq_store(lib, metric, qbits):
     store.append(codes)
     q1 = rng.standard_normal((40, d)).astype(np.float32)
     q2 = rng.standard_normal((3, d)).astype(np.float32)
+    noalloc_scan(l, store, q1, k, count_memory=False)  # first launches of these kernels in the process: see above
     a1 = noalloc_scan(l, store, q1, k)
     a2 = noalloc_scan(l, store, q2, 5)
     assert same(a1, store.flat_scan(q1, k))
@@ -140,6 +147,7 @@ def test_noalloc_uniform_store_under_cosine(lib, bits):
     store.append(codes)
     q1 = rng.random((33, d), dtype=np.float32)
     q2 = rng.random((2, d), dtype=np.float32)
+    noalloc_scan(l, store, q1, k, count_memory=False)  # first launches of these kernels in the process: see above
     a1 = noalloc_scan(l, store, q1, k)
     a2 = noalloc_scan(l, store, q2, 4)
     assert same(a1, store.flat_scan(q1, k))
