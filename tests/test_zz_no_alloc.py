@@ -64,9 +64,9 @@ def test_noalloc_flat_scan_equals_workspace_scan(lib):
     store.append(codes)
     q1, _ = gaussian_mixture(rng, 96, d, 50, 0.05, means=means)
     q2, _ = gaussian_mixture(rng, 5, d, 50, 0.05, means=means)
-    # The first launch of a kernel in a process lets the HIP runtime take memory of its own (2 MiB here: kernel objects,
-    # kernel-argument pools), whoever launches it: one call before the free bytes are counted, as a caller that cannot
-    # allocate makes one before it starts capturing or serving.  (The stream-ordered allocator is watched even here.)
+    # The first scan of a process lets the HIP runtime take memory of its own (2 MiB here: what it sets up on first use
+    # of kernels and pools, whichever entry point launches them): one call before the free bytes are counted, as a
+    # caller that cannot allocate makes one before it starts capturing or serving.  (The stream-ordered allocator is watched even here.)
     a0 = noalloc_scan(l, store, q1, k, count_memory=False)
     # two calls in a row on the shared array, the second with a smaller input (and another k)
     a1 = noalloc_scan(l, store, q1, k)
