@@ -144,3 +144,56 @@ def test_random_uniform_configuration(lib, seed):
         capi.check(L.vsag_amd_set_scan_contraction(0))
     assert _same(res[-1], res[1]), (bits, n, d, nq, k, metric)
     st.destroy()
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_fp16_configuration(lib, seed):
+    """sq8 and sq4 codes of more than 128 dimensions, flat stores and posting lists, on the fp16 matrix cores
+    (prefilter_h16.hip): random sizes, dimensions (ragged ones too), k, metric and data spread against the streaming scan."""
+    L = lib.load_library()
+    rng = np.random.default_rng(7000 + seed)
+    bits = [8, 4][seed % 2]
+    lists = (seed // 2) % 2 == 1
+    d = int(rng.choice([129, 136, 160, 200, 257, 384, 500, 777, 960, 1024]))
+    n = int(rng.integers(8000, 60000))
+    nq = int(rng.integers(512, 1500))
+    k = int(rng.choice([1, 5, 10, 32, 100]))
+    metric = int(rng.choice([orc.L2, orc.IP, orc.COSINE]))
+    comps = int(rng.choice([1, 5, 50]))
+    sigma = float(rng.choice([0.01, 0.05, 0.3]))
+    x, means = gaussian_mixture(rng, n, d, comps, sigma)
+    q, _ = gaussian_mixture(rng, nq, d, comps, sigma, means=means)
+    if rng.random() < 0.4:
+        q[: nq // 4] = x[rng.integers(0, n, nq // 4)]
+    if rng.random() < 0.5:
+        q[nq // 2:] *= np.float32(10.0 ** rng.integers(-4, 5))
+    lb, diff = orc.sq_train(x, bits, metric)
+    codes = orc.sq_encode(x, bits, lb, diff, metric)
+    st = Store(capi.KIND_SQ8 if bits == 8 else capi.KIND_SQ4, metric, d, lb=lb, diff=diff)
+    buckets = None
+    if lists:
+        nlist = int(rng.choice([16, 40]))
+        nprobe = int(rng.choice([4, 8]))
+        nq = 8192 * 4 // (nprobe - 1) + 64
+        q = np.tile(q, (nq // q.shape[0] + 1, 1))[:nq] + 1e-3 * rng.standard_normal((nq, d)).astype(np.float32)
+        cent = x[rng.choice(n, nlist, replace=False)].copy()
+        labels, _, _ = orc.kmeans_assign(x, cent)
+        st.set_lists(codes, labels, nlist)
+        buckets, _ = orc.ivf_route(cent, q, nprobe)
+    else:
+        st.append(codes[: n // 3])
+        st.append(codes[n // 3:])
+    res = {}
+    try:
+        for mode in ((-1, 0) if lists else (-1, 1)):
+            capi.check(L.vsag_amd_set_scan_contraction(mode))
+            res[mode] = st.ivf_scan(q, buckets, max(k, 10)) if lists else st.flat_scan(q, k)
+            if mode != -1:
+                tile = capi.C.c_int()
+                L.vsag_amd_last_scan_info(capi.C.byref(tile), None, None)
+                assert tile.value >= 128, "the matrix-core route did not run"
+    finally:
+        capi.check(L.vsag_amd_set_scan_contraction(0))
+    for mode, r in res.items():
+        assert _same(res[-1], r), (bits, lists, n, d, nq, k, metric, mode)
+    st.destroy()
